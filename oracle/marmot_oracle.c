@@ -1,0 +1,1694 @@
+/*
+ * marmot_oracle — TEST INFRASTRUCTURE ONLY (see marmot_oracle.h).
+ *
+ * CPU restatement of marmot's quantized-matmul arithmetic in its scalar
+ * configuration. Build with -ffp-contract=off so every fp32 operation is
+ * rounded separately, as in the reference's scalar build.
+ */
+#include "marmot_oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <pthread.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define QK 32
+#define QK_K 256
+#define TILE_COLS 16  /* matmul_quant_internal.h:11 */
+#define BLOCK_ROWS 64 /* matmul_quant_internal.h:12 */
+#define KC_BLOCKS 64  /* matmul_quant_internal.h:13 */
+#define MR 8          /* matmul_quant_internal.h:15-21 */
+
+/* error codes: include/marmot/types.h:210-220 */
+#define MO_OK 0
+#define MO_ERR_INVALID_ARGUMENT (-1)
+#define MO_ERR_OUT_OF_MEMORY (-2)
+#define MO_ERR_INVALID_OPERATION (-5)
+#define MO_ERR_UNSUPPORTED_DTYPE (-6)
+#define MO_ERR_NOT_IMPLEMENTED (-8)
+
+/* ---- block layouts: include/marmot/quant_block.h:20-125 ---- */
+#pragma pack(push, 1)
+typedef struct {
+    uint16_t scale;
+    uint8_t qs[16];
+} blk_q4_0; /* 18 B */
+typedef struct {
+    uint16_t scale;
+    int8_t qs[32];
+} blk_q8_0; /* 34 B */
+typedef struct {
+    uint16_t d;
+    uint16_t dmin;
+    uint8_t scales[12];
+    uint8_t qs[128];
+} blk_q4_k; /* 144 B */
+typedef struct {
+    uint8_t ql[128];
+    uint8_t qh[64];
+    int8_t scales[16];
+    uint16_t d;
+} blk_q6_k; /* 210 B */
+typedef struct {
+    float d;
+    int8_t qs[256];
+    int16_t bsums[16];
+} blk_q8_k; /* 292 B */
+#pragma pack(pop)
+
+_Static_assert(sizeof(blk_q4_0) == 18, "Q4_0");
+_Static_assert(sizeof(blk_q8_0) == 34, "Q8_0");
+_Static_assert(sizeof(blk_q4_k) == 144, "Q4_K");
+_Static_assert(sizeof(blk_q6_k) == 210, "Q6_K");
+_Static_assert(sizeof(blk_q8_k) == 292, "Q8_K");
+
+size_t mo_block_values(int kind) {
+    switch (kind) {
+    case MO_KIND_Q4_0:
+    case MO_KIND_Q8_0:
+        return QK;
+    case MO_KIND_Q4_K:
+    case MO_KIND_Q6_K:
+    case MO_KIND_Q8_K:
+        return QK_K;
+    default:
+        return 0;
+    }
+}
+
+size_t mo_block_bytes(int kind) {
+    switch (kind) {
+    case MO_KIND_Q4_0:
+        return sizeof(blk_q4_0);
+    case MO_KIND_Q8_0:
+        return sizeof(blk_q8_0);
+    case MO_KIND_Q4_K:
+        return sizeof(blk_q4_k);
+    case MO_KIND_Q6_K:
+        return sizeof(blk_q6_k);
+    case MO_KIND_Q8_K:
+        return sizeof(blk_q8_k);
+    default:
+        return 0;
+    }
+}
+
+/* matmul_quant_dispatch.c:423-427 */
+size_t mo_row_bytes(int kind, size_t k) {
+    const size_t bv = mo_block_values(kind);
+    if (bv == 0) {
+        return 0;
+    }
+    return ((k + bv - 1) / bv) * mo_block_bytes(kind);
+}
+
+/* ---- fp16 ---- */
+float mo_f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {
+            int e = -1;
+            do {
+                man <<= 1;
+                e++;
+            } while ((man & 0x400u) == 0);
+            man &= 0x3ffu;
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+uint16_t mo_f32_to_f16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    const uint32_t absx = x & 0x7fffffffu;
+    if (absx >= 0x7f800000u) { /* inf / nan */
+        if (absx > 0x7f800000u) {
+            return (uint16_t)(sign | 0x7e00u | ((absx >> 13) & 0x3ffu));
+        }
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (absx >= 0x477ff000u) { /* rounds to >= 65520 -> inf */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (absx < 0x33000001u) { /* < 2^-25 (or exactly 2^-25 tie -> even 0) */
+        return sign;
+    }
+    int32_t exp = (int32_t)(absx >> 23) - 127;
+    uint32_t man = (absx & 0x7fffffu) | 0x800000u;
+    uint32_t shift;
+    uint32_t half_exp;
+    if (exp < -14) { /* subnormal half */
+        shift = (uint32_t)(13 + (-14 - exp));
+        half_exp = 0;
+    } else {
+        shift = 13;
+        half_exp = (uint32_t)(exp + 15);
+    }
+    uint32_t q = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u);
+    const uint32_t halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (q & 1u))) {
+        q++;
+    }
+    uint32_t out;
+    if (half_exp == 0) {
+        out = q; /* may carry into exponent 1: correct */
+    } else {
+        out = ((half_exp - 1) << 10) + q; /* q has the implicit bit at 0x400 */
+    }
+    return (uint16_t)(sign | out);
+}
+
+/* ---- small helpers ---- */
+
+/* quantization/common/kquant_common.h:142-148 (and matmul_quant_pack.c:11-21 with clamping) */
+static inline int nearest_int_magic(float value) {
+    const float shifted = value + 12582912.0f;
+    int bits;
+    memcpy(&bits, &shifted, sizeof(int));
+    return (bits & 0x007fffff) - 0x00400000;
+}
+
+static inline int nearest_int_clamped(float value) {
+    if (value > 4194303.0f) {
+        value = 4194303.0f;
+    } else if (value < -4194303.0f) {
+        value = -4194303.0f;
+    }
+    return nearest_int_magic(value);
+}
+
+/* quantization/common/kquant_common.h:29-37 */
+static inline void get_scale_min_k4(int j, const uint8_t *q, uint8_t *d, uint8_t *m) {
+    if (j < 4) {
+        *d = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *d = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* ======================= Q8_0 ======================= */
+
+/* q8_gguf.c:127-153, quant_utils.c:55-73, block.c:221-232 (scalar: roundf, clamp +-127) */
+static void q8_0_quantize_block(const float *values, uint32_t elems, blk_q8_0 *block) {
+    float max_abs = 0.0f;
+    for (uint32_t i = 0; i < elems; ++i) {
+        const float a = fabsf(values[i]);
+        if (a > max_abs) {
+            max_abs = a;
+        }
+    }
+    float scale = max_abs <= 0.0f ? 0.0f : max_abs / 127.0f;
+    if (scale < FLT_MIN) {
+        scale = 1.0f;
+    }
+    const float inv_scale = 1.0f / scale;
+    memset(block, 0, sizeof(*block));
+    block->scale = mo_f32_to_f16(scale);
+    for (uint32_t i = 0; i < elems; ++i) {
+        const float v = values[i] * inv_scale;
+        int32_t q = (int32_t)roundf(v);
+        if (q < -127) {
+            q = -127;
+        } else if (q > 127) {
+            q = 127;
+        }
+        block->qs[i] = (int8_t)q;
+    }
+}
+
+/* q8_gguf.c:189-200 */
+static void q8_0_dequantize_block(const blk_q8_0 *block, uint32_t elems, float *out) {
+    const float scale = mo_f16_to_f32(block->scale);
+    for (uint32_t i = 0; i < elems; ++i) {
+        out[i] = (float)block->qs[i] * scale;
+    }
+}
+
+/* ======================= Q4_0 ======================= */
+
+/* q4_gguf.c:249-312 */
+static void q4_0_quantize_block(const float *values, uint32_t elems, blk_q4_0 *block) {
+    float bv[QK] = {0};
+    memcpy(bv, values, elems * sizeof(float));
+    float amax = 0.0f;
+    float max_val = 0.0f;
+    for (uint32_t i = 0; i < QK; ++i) {
+        const float a = fabsf(bv[i]);
+        if (a > amax) {
+            amax = a;
+            max_val = bv[i];
+        }
+    }
+    float scale = 0.0f;
+    float inv_scale = 0.0f;
+    if (amax > 0.0f) {
+        scale = -max_val / 8.0f;
+        if (scale != 0.0f) {
+            inv_scale = 1.0f / scale;
+        }
+    }
+    block->scale = mo_f32_to_f16(scale);
+    uint8_t qv[QK];
+    for (uint32_t i = 0; i < QK; ++i) {
+        const float x = bv[i] * inv_scale;
+        int32_t q = (int32_t)(int8_t)(x + 8.5f);
+        if (q < 0) {
+            q = 0;
+        } else if (q > 15) {
+            q = 15;
+        }
+        qv[i] = (uint8_t)q;
+    }
+    for (uint32_t j = 0; j < QK / 2; ++j) {
+        block->qs[j] = (uint8_t)(((qv[j + QK / 2] & 0x0F) << 4) | (qv[j] & 0x0F));
+    }
+}
+
+/* q4_gguf.c:367-394 (scalar branch) */
+static void q4_0_dequantize_block(const blk_q4_0 *block, uint32_t elems, float *out) {
+    const float scale = mo_f16_to_f32(block->scale);
+    float decoded[QK];
+    for (uint32_t j = 0; j < QK / 2; ++j) {
+        const uint8_t packed = block->qs[j];
+        decoded[j] = (float)((int)(packed & 0x0F) - 8) * scale;
+        decoded[j + QK / 2] = (float)((int)(packed >> 4) - 8) * scale;
+    }
+    memcpy(out, decoded, elems * sizeof(float));
+}
+
+/* ======================= Q4_K ======================= */
+
+/* kquant_common.h:39-130 */
+static float make_qkx2_quants(
+    int n, int nmax, const float *x, const float *weights, uint8_t *L, float *the_min, uint8_t *Laux, float rmin,
+    float rdelta, int nstep
+) {
+    float min = x[0];
+    float max = x[0];
+    float sum_w = weights[0];
+    float sum_x = sum_w * x[0];
+    for (int i = 1; i < n; ++i) {
+        if (x[i] < min) {
+            min = x[i];
+        }
+        if (x[i] > max) {
+            max = x[i];
+        }
+        const float w = weights[i];
+        sum_w += w;
+        sum_x += w * x[i];
+    }
+    if (min > 0) {
+        min = 0;
+    }
+    if (max == min) {
+        for (int i = 0; i < n; ++i) {
+            L[i] = 0;
+        }
+        *the_min = -min;
+        return 0.0f;
+    }
+    float iscale = nmax / (max - min);
+    float scale = 1.0f / iscale;
+    float best_error = 0;
+    for (int i = 0; i < n; ++i) {
+        int l = (int)nearbyintf(iscale * (x[i] - min));
+        L[i] = (uint8_t)(l > nmax ? nmax : l < 0 ? 0 : l);
+        float diff = scale * L[i] + min - x[i];
+        diff = diff * diff;
+        best_error += weights[i] * diff;
+    }
+    if (nstep < 1) {
+        *the_min = -min;
+        return scale;
+    }
+    for (int is = 0; is <= nstep; ++is) {
+        iscale = (rmin + rdelta * is + nmax) / (max - min);
+        float sum_l = 0, sum_l2 = 0, sum_xl = 0;
+        for (int i = 0; i < n; ++i) {
+            int l = (int)nearbyintf(iscale * (x[i] - min));
+            l = l > nmax ? nmax : l < 0 ? 0 : l;
+            Laux[i] = (uint8_t)l;
+            const float w = weights[i];
+            sum_l += w * l;
+            sum_l2 += w * l * l;
+            sum_xl += w * l * x[i];
+        }
+        const float D = sum_w * sum_l2 - sum_l * sum_l;
+        if (D > 0) {
+            float this_scale = (sum_w * sum_xl - sum_x * sum_l) / D;
+            float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / D;
+            if (this_min > 0) {
+                this_min = 0;
+                this_scale = sum_xl / sum_l2;
+            }
+            float cur_error = 0;
+            for (int i = 0; i < n; ++i) {
+                float diff = this_scale * Laux[i] + this_min - x[i];
+                diff = diff * diff;
+                cur_error += weights[i] * diff;
+            }
+            if (cur_error < best_error) {
+                for (int i = 0; i < n; ++i) {
+                    L[i] = Laux[i];
+                }
+                best_error = cur_error;
+                scale = this_scale;
+                min = this_min;
+            }
+        }
+    }
+    *the_min = -min;
+    return scale;
+}
+
+/* q4k_gguf.c:35-131 */
+static void q4_k_quantize_block(const float *values, uint32_t elems, blk_q4_k *block) {
+    float bv[QK_K];
+    memcpy(bv, values, elems * sizeof(float));
+    if (elems < QK_K) {
+        memset(bv + elems, 0, (QK_K - elems) * sizeof(float));
+    }
+    uint8_t L[QK_K];
+    memset(L, 0, sizeof(L));
+    uint8_t Laux[32];
+    float weights[32];
+    float scales[QK_K / 32];
+    float mins[QK_K / 32];
+    memset(block, 0, sizeof(*block));
+
+    float max_scale = 0.0f;
+    float max_min = 0.0f;
+    for (int j = 0; j < QK_K / 32; ++j) {
+        float sum_x2 = 0.0f;
+        for (int l = 0; l < 32; ++l) {
+            const float v = bv[32 * j + l];
+            sum_x2 += v * v;
+        }
+        const float av_x = sqrtf(sum_x2 / 32.0f);
+        for (int l = 0; l < 32; ++l) {
+            weights[l] = av_x + fabsf(bv[32 * j + l]);
+        }
+        scales[j] = make_qkx2_quants(32, 15, bv + 32 * j, weights, L + 32 * j, &mins[j], Laux, -1.0f, 0.1f, 20);
+        if (scales[j] > max_scale) {
+            max_scale = scales[j];
+        }
+        if (mins[j] > max_min) {
+            max_min = mins[j];
+        }
+    }
+
+    const float inv_scale = max_scale > 0 ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0 ? 63.0f / max_min : 0.0f;
+    for (int j = 0; j < QK_K / 32; ++j) {
+        uint8_t ls = (uint8_t)nearbyintf(inv_scale * scales[j]);
+        uint8_t lm = (uint8_t)nearbyintf(inv_min * mins[j]);
+        ls = ls > 63 ? 63 : ls;
+        lm = lm > 63 ? 63 : lm;
+        if (j < 4) {
+            block->scales[j] = ls;
+            block->scales[j + 4] = lm;
+        } else {
+            block->scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+            block->scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            block->scales[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+    block->d = mo_f32_to_f16(max_scale / 63.0f);
+    block->dmin = mo_f32_to_f16(max_min / 63.0f);
+
+    for (int j = 0; j < QK_K / 32; ++j) {
+        uint8_t sc, m;
+        get_scale_min_k4(j, block->scales, &sc, &m);
+        const float d = mo_f16_to_f32(block->d) * sc;
+        if (d == 0) {
+            continue;
+        }
+        const float dm = mo_f16_to_f32(block->dmin) * m;
+        for (int ii = 0; ii < 32; ++ii) {
+            int l = (int)nearbyintf((bv[32 * j + ii] + dm) / d);
+            l = l > 15 ? 15 : (l < 0 ? 0 : l);
+            L[32 * j + ii] = (uint8_t)l;
+        }
+    }
+
+    for (int j = 0; j < QK_K; j += 64) {
+        for (int l = 0; l < 32; ++l) {
+            block->qs[(j / 2) + l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
+        }
+    }
+    if (elems < QK_K) {
+        const size_t qs_offset = (elems + 1) / 2;
+        if (qs_offset < sizeof(block->qs)) {
+            memset(block->qs + qs_offset, 0, sizeof(block->qs) - qs_offset);
+        }
+    }
+}
+
+/* q4k_gguf.c:133-166: d1 = d*sc; m1 = dmin*m; y = d1*q - m1, each op rounded */
+static void q4_k_dequantize_block(const blk_q4_k *block, uint32_t elems, float *out) {
+    const uint8_t *q = block->qs;
+    const float d = mo_f16_to_f32(block->d);
+    const float min = mo_f16_to_f32(block->dmin);
+    size_t written = 0;
+    int is = 0;
+    for (size_t j = 0; j < QK_K && written < elems; j += 64) {
+        uint8_t sc, m;
+        get_scale_min_k4(is + 0, block->scales, &sc, &m);
+        const float d1 = d * sc;
+        const float m1 = min * m;
+        get_scale_min_k4(is + 1, block->scales, &sc, &m);
+        const float d2 = d * sc;
+        const float m2 = min * m;
+        for (int l = 0; l < 32 && written < elems; ++l, ++written) {
+            out[written] = d1 * (q[l] & 0xF) - m1;
+        }
+        for (int l = 0; l < 32 && written < elems; ++l, ++written) {
+            out[written] = d2 * (q[l] >> 4) - m2;
+        }
+        q += 32;
+        is += 2;
+    }
+}
+
+/* ======================= Q6_K ======================= */
+
+static inline int clamp_qx(int value, int nmax) {
+    if (value > nmax - 1) {
+        return nmax - 1;
+    }
+    if (value < -nmax) {
+        return -nmax;
+    }
+    return value;
+}
+
+/* kquant_common.h:150-236 with rmse_type == 1, weights == NULL */
+static float make_qx_quants_rmse1(int n, int nmax, const float *x, int8_t *L) {
+    float max = 0.0f;
+    float amax = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        const float ax = fabsf(x[i]);
+        if (ax > amax) {
+            amax = ax;
+            max = x[i];
+        }
+    }
+    if (amax < 1e-15f) {
+        memset(L, 0, (size_t)n);
+        return 0.0f;
+    }
+    const float iscale = -((float)nmax) / max;
+    float sumlx = 0.0f;
+    float suml2 = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        int l = nearest_int_magic(iscale * x[i]);
+        l = clamp_qx(l, nmax);
+        L[i] = (int8_t)(l + nmax);
+        const float w = x[i] * x[i];
+        sumlx += w * x[i] * l;
+        suml2 += w * l * l;
+    }
+    float scale = (suml2 > 0.0f) ? (sumlx / suml2) : 0.0f;
+    float best = scale * sumlx;
+    for (int is = -9; is <= 9; ++is) {
+        if (is == 0) {
+            continue;
+        }
+        const float trial_iscale = -(nmax + 0.1f * (float)is) / max;
+        float trial_sumlx = 0.0f;
+        float trial_suml2 = 0.0f;
+        for (int i = 0; i < n; ++i) {
+            int l = nearest_int_magic(trial_iscale * x[i]);
+            l = clamp_qx(l, nmax);
+            const float w = x[i] * x[i];
+            trial_sumlx += w * x[i] * l;
+            trial_suml2 += w * l * l;
+        }
+        if (trial_suml2 > 0.0f && trial_sumlx * trial_sumlx > best * trial_suml2) {
+            for (int i = 0; i < n; ++i) {
+                int l = nearest_int_magic(trial_iscale * x[i]);
+                l = clamp_qx(l, nmax);
+                L[i] = (int8_t)(l + nmax);
+            }
+            scale = trial_sumlx / trial_suml2;
+            best = scale * trial_sumlx;
+        }
+    }
+    return scale;
+}
+
+/* q6k_gguf.c:35-61 + kquant_common.h:310-369 */
+static void q6_k_quantize_block(const float *values, uint32_t elems, blk_q6_k *y) {
+    float x[QK_K];
+    memcpy(x, values, elems * sizeof(float));
+    if (elems < QK_K) {
+        memset(x + elems, 0, (QK_K - elems) * sizeof(float));
+    }
+    memset(y, 0, sizeof(*y));
+
+    int8_t L[QK_K];
+    float scales[QK_K / 16];
+    float max_scale = 0.0f;
+    float max_abs_scale = 0.0f;
+    for (int ib = 0; ib < QK_K / 16; ++ib) {
+        const float scale = make_qx_quants_rmse1(16, 32, x + 16 * ib, L + 16 * ib);
+        scales[ib] = scale;
+        const float abs_scale = fabsf(scale);
+        if (abs_scale > max_abs_scale) {
+            max_abs_scale = abs_scale;
+            max_scale = scale;
+        }
+    }
+    if (max_abs_scale < 1e-15f) {
+        memset(y, 0, sizeof(*y));
+        return;
+    }
+    const float iscale = -128.0f / max_scale;
+    y->d = mo_f32_to_f16(1.0f / iscale);
+    for (int ib = 0; ib < QK_K / 16; ++ib) {
+        int sc = nearest_int_magic(iscale * scales[ib]);
+        sc = sc > 127 ? 127 : (sc < -128 ? -128 : sc);
+        y->scales[ib] = (int8_t)sc;
+    }
+    for (int j = 0; j < QK_K / 16; ++j) {
+        const float d = mo_f16_to_f32(y->d) * y->scales[j];
+        if (d == 0.0f) {
+            continue;
+        }
+        for (int ii = 0; ii < 16; ++ii) {
+            int l = nearest_int_magic(x[16 * j + ii] / d);
+            l = clamp_qx(l, 32);
+            L[16 * j + ii] = (int8_t)(l + 32);
+        }
+    }
+    uint8_t *ql = y->ql;
+    uint8_t *qh = y->qh;
+    for (int j = 0; j < QK_K; j += 128) {
+        for (int l = 0; l < 32; ++l) {
+            const uint8_t q1 = L[j + l + 0] & 0xF;
+            const uint8_t q2 = L[j + l + 32] & 0xF;
+            const uint8_t q3 = L[j + l + 64] & 0xF;
+            const uint8_t q4 = L[j + l + 96] & 0xF;
+            ql[l + 0] = (uint8_t)(q1 | (q3 << 4));
+            ql[l + 32] = (uint8_t)(q2 | (q4 << 4));
+            qh[l] = (uint8_t)((L[j + l] >> 4) | ((L[j + l + 32] >> 4) << 2) | ((L[j + l + 64] >> 4) << 4) |
+                              ((L[j + l + 96] >> 4) << 6));
+        }
+        ql += 64;
+        qh += 32;
+    }
+    if (elems < QK_K) {
+        const size_t ql_offset = (elems + 1) / 2;
+        const size_t qh_offset = (elems + 3) / 4;
+        if (ql_offset < sizeof(y->ql)) {
+            memset(y->ql + ql_offset, 0, sizeof(y->ql) - ql_offset);
+        }
+        if (qh_offset < sizeof(y->qh)) {
+            memset(y->qh + qh_offset, 0, sizeof(y->qh) - qh_offset);
+        }
+    }
+}
+
+/* q6k_gguf.c:63-99: y = (d * sc) * q, left to right */
+static void q6_k_dequantize_block(const blk_q6_k *block, uint32_t elems, float *out) {
+    const float d = mo_f16_to_f32(block->d);
+    const uint8_t *ql = block->ql;
+    const uint8_t *qh = block->qh;
+    const int8_t *sc = block->scales;
+    for (size_t n = 0; n < QK_K && n < elems; n += 128) {
+        for (int l = 0; l < 32; ++l) {
+            const int is = l / 16;
+            const int8_t q1 = (int8_t)((int8_t)((ql[l + 0] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32);
+            const int8_t q2 = (int8_t)((int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32);
+            const int8_t q3 = (int8_t)((int8_t)((ql[l + 0] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+            const int8_t q4 = (int8_t)((int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+            if (n + l + 0 < elems) {
+                out[n + l + 0] = d * sc[is + 0] * q1;
+            }
+            if (n + l + 32 < elems) {
+                out[n + l + 32] = d * sc[is + 2] * q2;
+            }
+            if (n + l + 64 < elems) {
+                out[n + l + 64] = d * sc[is + 4] * q3;
+            }
+            if (n + l + 96 < elems) {
+                out[n + l + 96] = d * sc[is + 6] * q4;
+            }
+        }
+        ql += 64;
+        qh += 32;
+        sc += 8;
+    }
+}
+
+/* ======================= Q8_K (activation) ======================= */
+
+/* matmul_quant_pack.c:106-142 */
+static void q8_k_pack_block(const float *bv, blk_q8_k *dst) {
+    float max_val = 0.0f;
+    float abs_max = 0.0f;
+    for (size_t i = 0; i < QK_K; ++i) {
+        const float ax = fabsf(bv[i]);
+        if (ax > abs_max) {
+            abs_max = ax;
+            max_val = bv[i];
+        }
+    }
+    if (abs_max <= 0.0f) {
+        dst->d = 0.0f;
+        memset(dst->qs, 0, sizeof(dst->qs));
+        memset(dst->bsums, 0, sizeof(dst->bsums));
+        return;
+    }
+    const float iscale = -127.0f / max_val;
+    for (size_t i = 0; i < QK_K; ++i) {
+        int v = nearest_int_clamped(iscale * bv[i]);
+        if (v > 127) {
+            v = 127;
+        }
+        dst->qs[i] = (int8_t)v;
+    }
+    for (size_t b = 0; b < QK_K / 16; ++b) {
+        int sum = 0;
+        for (size_t i = 0; i < 16; ++i) {
+            sum += dst->qs[b * 16 + i];
+        }
+        dst->bsums[b] = (int16_t)sum;
+    }
+    dst->d = 1.0f / iscale;
+}
+
+static inline float load_act(const void *x, int in_dtype, size_t i) {
+    if (in_dtype == MO_DTYPE_F16) {
+        return mo_f16_to_f32(((const uint16_t *)x)[i]);
+    }
+    return ((const float *)x)[i];
+}
+
+/* matmul_quant_pack.c:144-196 */
+void mo_pack_q8_k(const void *x, int in_dtype, size_t k, void *blocks_out) {
+    blk_q8_k *blocks = (blk_q8_k *)blocks_out;
+    const size_t nb = (k + QK_K - 1) / QK_K;
+    float bv[QK_K];
+    for (size_t b = 0; b < nb; ++b) {
+        const size_t start = b * QK_K;
+        const size_t len = (start + QK_K <= k) ? QK_K : (k - start);
+        for (size_t i = 0; i < len; ++i) {
+            bv[i] = load_act(x, in_dtype, start + i);
+        }
+        if (len < QK_K) {
+            memset(bv + len, 0, (QK_K - len) * sizeof(float));
+        }
+        q8_k_pack_block(bv, &blocks[b]);
+    }
+}
+
+/* matmul_quant_pack.c:23-104 */
+void mo_pack_q8_0(const void *x, int in_dtype, size_t k, void *blocks_out) {
+    blk_q8_0 *blocks = (blk_q8_0 *)blocks_out;
+    const size_t nb = (k + QK - 1) / QK;
+    float bv[QK];
+    for (size_t b = 0; b < nb; ++b) {
+        const size_t start = b * QK;
+        const size_t len = (start + QK <= k) ? QK : (k - start);
+        for (size_t i = 0; i < len; ++i) {
+            bv[i] = load_act(x, in_dtype, start + i);
+        }
+        if (len < QK) {
+            memset(bv + len, 0, (QK - len) * sizeof(float));
+        }
+        float max_abs = 0.0f;
+        for (size_t i = 0; i < len; ++i) {
+            const float a = fabsf(bv[i]);
+            if (a > max_abs) {
+                max_abs = a;
+            }
+        }
+        float scale = max_abs / 127.0f;
+        if (scale < FLT_MIN) {
+            scale = 1.0f;
+        }
+        const float inv_scale = 1.0f / scale;
+        blk_q8_0 *dst = &blocks[b];
+        memset(dst, 0, sizeof(*dst));
+        dst->scale = mo_f32_to_f16(scale);
+        for (size_t i = 0; i < len; ++i) {
+            const float v = bv[i] * inv_scale;
+            int32_t q = (int32_t)roundf(v);
+            if (q < -127) {
+                q = -127;
+            } else if (q > 127) {
+                q = 127;
+            }
+            dst->qs[i] = (int8_t)q;
+        }
+    }
+}
+
+/* ======================= blockwise drivers ======================= */
+
+/* ops/quantize_core.c:199-265 */
+int mo_quantize_rows(int kind, const float *x, size_t rows, size_t k, void *out) {
+    const size_t bv = mo_block_values(kind);
+    const size_t bb = mo_block_bytes(kind);
+    if (bv == 0 || x == NULL || out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    const size_t nb = (k + bv - 1) / bv;
+    uint8_t *dst = (uint8_t *)out;
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t b = 0; b < nb; ++b) {
+            const size_t start = b * bv;
+            const uint32_t elems = (uint32_t)((start + bv <= k) ? bv : (k - start));
+            const float *src = x + r * k + start;
+            void *blk = dst + (r * nb + b) * bb;
+            switch (kind) {
+            case MO_KIND_Q8_0:
+                q8_0_quantize_block(src, elems, (blk_q8_0 *)blk);
+                break;
+            case MO_KIND_Q4_0:
+                q4_0_quantize_block(src, elems, (blk_q4_0 *)blk);
+                break;
+            case MO_KIND_Q4_K:
+                q4_k_quantize_block(src, elems, (blk_q4_k *)blk);
+                break;
+            case MO_KIND_Q6_K:
+                q6_k_quantize_block(src, elems, (blk_q6_k *)blk);
+                break;
+            case MO_KIND_Q8_K: {
+                float tmp[QK_K];
+                memcpy(tmp, src, elems * sizeof(float));
+                if (elems < QK_K) {
+                    memset(tmp + elems, 0, (QK_K - elems) * sizeof(float));
+                }
+                q8_k_pack_block(tmp, (blk_q8_k *)blk);
+                break;
+            }
+            default:
+                return MO_ERR_NOT_IMPLEMENTED;
+            }
+        }
+    }
+    return MO_OK;
+}
+
+/* ops/quantize_core.c:267-331 */
+int mo_dequantize_rows(int kind, const void *blocks, size_t rows, size_t k, float *out) {
+    const size_t bv = mo_block_values(kind);
+    const size_t bb = mo_block_bytes(kind);
+    if (bv == 0 || blocks == NULL || out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    const size_t nb = (k + bv - 1) / bv;
+    const uint8_t *src = (const uint8_t *)blocks;
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t b = 0; b < nb; ++b) {
+            const size_t start = b * bv;
+            const uint32_t elems = (uint32_t)((start + bv <= k) ? bv : (k - start));
+            const void *blk = src + (r * nb + b) * bb;
+            float *dst = out + r * k + start;
+            switch (kind) {
+            case MO_KIND_Q8_0:
+                q8_0_dequantize_block((const blk_q8_0 *)blk, elems, dst);
+                break;
+            case MO_KIND_Q4_0:
+                q4_0_dequantize_block((const blk_q4_0 *)blk, elems, dst);
+                break;
+            case MO_KIND_Q4_K:
+                q4_k_dequantize_block((const blk_q4_k *)blk, elems, dst);
+                break;
+            case MO_KIND_Q6_K:
+                q6_k_dequantize_block((const blk_q6_k *)blk, elems, dst);
+                break;
+            case MO_KIND_Q8_K: {
+                /* q8k_gguf.c dequant: y = d * q */
+                const blk_q8_k *q = (const blk_q8_k *)blk;
+                for (uint32_t i = 0; i < elems; ++i) {
+                    dst[i] = q->d * (float)q->qs[i];
+                }
+                break;
+            }
+            default:
+                return MO_ERR_NOT_IMPLEMENTED;
+            }
+        }
+    }
+    return MO_OK;
+}
+
+/* ======================= block dots ======================= */
+
+/* vec_dot_impl.h:452-479 */
+float mo_vec_dot_q8_0_q8_0(const void *w, const void *a, size_t nblocks) {
+    const blk_q8_0 *wb = (const blk_q8_0 *)w;
+    const blk_q8_0 *ab = (const blk_q8_0 *)a;
+    float total = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        int32_t sum = 0;
+        for (int i = 0; i < QK; ++i) {
+            sum += (int32_t)wb[b].qs[i] * (int32_t)ab[b].qs[i];
+        }
+        const float block_scale = mo_f16_to_f32(wb[b].scale) * mo_f16_to_f32(ab[b].scale);
+        total += (float)sum * block_scale;
+    }
+    return total;
+}
+
+/* vec_dot_impl.h:157-186 */
+float mo_vec_dot_q4_0_q8_0(const void *w, const void *a, size_t nblocks) {
+    const blk_q4_0 *wb = (const blk_q4_0 *)w;
+    const blk_q8_0 *ab = (const blk_q8_0 *)a;
+    float total = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        int32_t sum = 0;
+        for (int i = 0; i < QK / 2; ++i) {
+            const uint8_t packed = wb[b].qs[i];
+            sum += ((int32_t)(packed & 0x0f) - 8) * (int32_t)ab[b].qs[i];
+            sum += ((int32_t)(packed >> 4) - 8) * (int32_t)ab[b].qs[i + QK / 2];
+        }
+        const float block_scale = mo_f16_to_f32(wb[b].scale) * mo_f16_to_f32(ab[b].scale);
+        total += (float)sum * block_scale;
+    }
+    return total;
+}
+
+/* vec_dot_impl.h:541-563, 689-732 */
+float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks) {
+    const blk_q4_k *wb = (const blk_q4_k *)w;
+    const blk_q8_k *ab = (const blk_q8_k *)a;
+    float sum_all = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        uint8_t scales[8];
+        uint8_t mins[8];
+        for (int j = 0; j < 8; ++j) {
+            get_scale_min_k4(j, wb[b].scales, &scales[j], &mins[j]);
+        }
+        int32_t sumi = 0;
+        for (int j = 0; j < QK_K / 16; ++j) {
+            sumi += (int32_t)ab[b].bsums[j] * (int32_t)mins[j / 2];
+        }
+        int32_t block_sum = 0;
+        for (int sg = 0; sg < 8; ++sg) {
+            const uint8_t *q4 = wb[b].qs + (sg / 2) * 32;
+            const int8_t *q8 = ab[b].qs + sg * 32;
+            const int high = sg & 1;
+            int32_t dot = 0;
+            for (int l = 0; l < 32; ++l) {
+                const int32_t wv = high ? (q4[l] >> 4) : (q4[l] & 0x0F);
+                dot += wv * (int32_t)q8[l];
+            }
+            block_sum += (int32_t)scales[sg] * dot;
+        }
+        const float d = ab[b].d * mo_f16_to_f32(wb[b].d);
+        const float dmin = ab[b].d * mo_f16_to_f32(wb[b].dmin);
+        sum_all += d * (float)block_sum - dmin * (float)sumi;
+    }
+    return sum_all;
+}
+
+/* vec_dot_impl.h:783-828 */
+float mo_vec_dot_q6_k_q8_k(const void *w, const void *a, size_t nblocks) {
+    const blk_q6_k *wb = (const blk_q6_k *)w;
+    const blk_q8_k *ab = (const blk_q8_k *)a;
+    float sum_all = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        const int8_t *q8 = ab[b].qs;
+        int32_t block_sum = 0;
+        for (size_t sg = 0; sg < QK_K / 16; ++sg) {
+            const size_t group32 = sg / 2;
+            const size_t half = group32 / 4;
+            const size_t gih = group32 & 3;
+            const size_t part = sg & 1;
+            const uint8_t *ql = wb[b].ql + half * 64 + ((gih & 1) ? 32 : 0) + part * 16;
+            const uint8_t *qh = wb[b].qh + half * 32 + part * 16;
+            const int shift = (int)(gih * 2);
+            const int high_nibble = gih >= 2;
+            int32_t dot = 0;
+            for (int l = 0; l < 16; ++l) {
+                const uint8_t ql_val = high_nibble ? (ql[l] >> 4) : (ql[l] & 0x0F);
+                const uint8_t qh_val = (qh[l] >> shift) & 0x03;
+                const int8_t q = (int8_t)((ql_val | (qh_val << 4)) - 32);
+                dot += (int32_t)q * (int32_t)q8[l];
+            }
+            block_sum += (int32_t)wb[b].scales[sg] * dot;
+            q8 += 16;
+        }
+        const float d = ab[b].d * mo_f16_to_f32(wb[b].d);
+        sum_all += d * (float)block_sum;
+    }
+    return sum_all;
+}
+
+/* fp16 direct dots: vec_dot_impl.h:220-250 (Q4_0), 419-450 (Q8_0), 973-1023 (Q4_K).
+ * Q6_K: the reference's cpu_vec_dot_q6_k_f16 (vec_dot_impl.h:1082-1128) decodes with an index
+ * pattern that differs from its own dequantizer; the oracle restates that function as written,
+ * so parity with "what the reference computes" holds, but no product kernel mirrors it. */
+float mo_vec_dot_f16(int kind, const void *w, const uint16_t *a, size_t nblocks, size_t k) {
+    float total = 0.0f;
+    if (kind == MO_KIND_Q8_0) {
+        const blk_q8_0 *wb = (const blk_q8_0 *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const float scale_w = mo_f16_to_f32(wb[b].scale);
+            const size_t start = b * QK;
+            const size_t len = (start + QK <= k) ? QK : (k - start);
+            for (size_t i = 0; i < len; ++i) {
+                const float av = mo_f16_to_f32(a[start + i]);
+                total += ((float)wb[b].qs[i]) * scale_w * av;
+            }
+        }
+    } else if (kind == MO_KIND_Q4_0) {
+        const blk_q4_0 *wb = (const blk_q4_0 *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            int16_t w16[QK];
+            for (int i = 0; i < QK / 2; ++i) {
+                w16[i] = (int16_t)((wb[b].qs[i] & 0x0f) - 8);
+                w16[i + QK / 2] = (int16_t)((wb[b].qs[i] >> 4) - 8);
+            }
+            const float scale_w = mo_f16_to_f32(wb[b].scale);
+            const size_t start = b * QK;
+            const size_t len = (start + QK <= k) ? QK : (k - start);
+            for (size_t i = 0; i < len; ++i) {
+                const float av = mo_f16_to_f32(a[start + i]);
+                total += ((float)w16[i]) * scale_w * av;
+            }
+        }
+    } else if (kind == MO_KIND_Q4_K) {
+        const blk_q4_k *wb = (const blk_q4_k *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const uint8_t *q = wb[b].qs;
+            const float d = mo_f16_to_f32(wb[b].d);
+            const float dmin = mo_f16_to_f32(wb[b].dmin);
+            const size_t start = b * QK_K;
+            const size_t len = (start + QK_K <= k) ? QK_K : (k - start);
+            size_t written = 0;
+            int is = 0;
+            for (size_t j = 0; j < QK_K && written < len; j += 64) {
+                uint8_t sc, m;
+                get_scale_min_k4(is + 0, wb[b].scales, &sc, &m);
+                const float d1 = d * (float)sc;
+                const float m1 = dmin * (float)m;
+                get_scale_min_k4(is + 1, wb[b].scales, &sc, &m);
+                const float d2 = d * (float)sc;
+                const float m2 = dmin * (float)m;
+                for (int l = 0; l < 32 && written < len; ++l, ++written) {
+                    const float av = mo_f16_to_f32(a[start + written]);
+                    const float wv = d1 * (float)(q[l] & 0xF) - m1;
+                    total += wv * av;
+                }
+                for (int l = 0; l < 32 && written < len; ++l, ++written) {
+                    const float av = mo_f16_to_f32(a[start + written]);
+                    const float wv = d2 * (float)(q[l] >> 4) - m2;
+                    total += wv * av;
+                }
+                q += 32;
+                is += 2;
+            }
+        }
+    } else if (kind == MO_KIND_Q6_K) {
+        const blk_q6_k *wb = (const blk_q6_k *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const uint8_t *ql = wb[b].ql;
+            const uint8_t *qh = wb[b].qh;
+            const float d = mo_f16_to_f32(wb[b].d);
+            const size_t start = b * QK_K;
+            const size_t len = (start + QK_K <= k) ? QK_K : (k - start);
+            size_t written = 0;
+            for (size_t j = 0; j < QK_K && written < len; j += 128) {
+                const float scale = d * (float)wb[b].scales[j / 128];
+                for (size_t i = 0; i < 128 && written < len; ++i, ++written) {
+                    const size_t idx = j + i;
+                    const uint8_t ql_val = (i % 2 == 0) ? (ql[idx / 2] & 0xF) : (ql[idx / 2] >> 4);
+                    const uint8_t qh_val = (qh[idx / 4] >> ((idx % 4) * 2)) & 0x3;
+                    const int8_t sq = (int8_t)((int8_t)(ql_val | (qh_val << 4)) - 32);
+                    const float av = mo_f16_to_f32(a[start + written]);
+                    total += (scale * (float)sq) * av;
+                }
+            }
+        }
+    }
+    return total;
+}
+
+/* ======================= matmul driver ======================= */
+
+typedef float (*dot_fn)(const void *w, const void *a, size_t nblocks);
+
+static dot_fn pick_dot(int kind) {
+    switch (kind) {
+    case MO_KIND_Q8_0:
+        return mo_vec_dot_q8_0_q8_0;
+    case MO_KIND_Q4_0:
+        return mo_vec_dot_q4_0_q8_0;
+    case MO_KIND_Q4_K:
+        return mo_vec_dot_q4_k_q8_k;
+    case MO_KIND_Q6_K:
+        return mo_vec_dot_q6_k_q8_k;
+    default:
+        return NULL;
+    }
+}
+
+/* matmul_quant_compute.c:1222-1240 */
+size_t mo_row_grain(size_t row_count, size_t cols_in_tile, size_t thread_cap) {
+    size_t grain = BLOCK_ROWS;
+    if (thread_cap == 0) {
+        thread_cap = 1;
+    }
+    if (cols_in_tile <= 4 && row_count > grain * thread_cap) {
+        const size_t target_tasks = thread_cap * (cols_in_tile <= 1 ? 8u : 12u);
+        size_t dynamic = (row_count + target_tasks - 1) / target_tasks;
+        dynamic = ((dynamic + MR - 1) / MR) * MR;
+        if (dynamic > grain) {
+            grain = dynamic;
+        }
+    }
+    if (grain > 4096) {
+        grain = 4096;
+    }
+    return grain;
+}
+
+typedef struct {
+    int kind;
+    int direct_f16;
+    const uint8_t *weight;
+    size_t row_bytes;
+    size_t block_bytes;
+    size_t blocks_per_row;
+    size_t act_block_bytes;
+    const uint8_t *act_tile;  /* packed path: cols_in_tile * blocks_per_row activation blocks */
+    const uint16_t *act_f16;  /* direct path: input base */
+    size_t K;
+    size_t M;
+    size_t n0;
+    size_t cols_in_tile;
+    float *out_f32;
+    uint16_t *out_f16;
+    dot_fn dot;
+    /* work queue */
+    size_t grain;
+    size_t next_row;
+    pthread_mutex_t lock;
+} tile_job;
+
+/* matmul_quant_compute.c:1032-1112 (generic) and :412-466 (Q8_0, >=2 columns): per (row, col) the
+ * K blocks are consumed in chunks of 64, each chunk reduced inside the block dot, chunk sums added in order. */
+static void tile_compute_rows(const tile_job *job, size_t row_start, size_t row_end) {
+    for (size_t m = row_start; m < row_end; ++m) {
+        const uint8_t *row_ptr = job->weight + m * job->row_bytes;
+        for (size_t c = 0; c < job->cols_in_tile; ++c) {
+            float dot = 0.0f;
+            if (job->direct_f16) {
+                /* matmul_quant_compute.c:1860-1890 */
+                dot = mo_vec_dot_f16(job->kind, row_ptr, job->act_f16 + (job->n0 + c) * job->K, job->blocks_per_row,
+                                     job->K);
+            } else {
+                const uint8_t *col = job->act_tile + c * job->blocks_per_row * job->act_block_bytes;
+                for (size_t kb = 0; kb < job->blocks_per_row; kb += KC_BLOCKS) {
+                    const size_t chunk =
+                        (kb + KC_BLOCKS <= job->blocks_per_row) ? KC_BLOCKS : (job->blocks_per_row - kb);
+                    dot += job->dot(row_ptr + kb * job->block_bytes, col + kb * job->act_block_bytes, chunk);
+                }
+            }
+            if (job->out_f32 != NULL) {
+                job->out_f32[(job->n0 + c) * job->M + m] = dot;
+            }
+            if (job->out_f16 != NULL) {
+                job->out_f16[(job->n0 + c) * job->M + m] = mo_f32_to_f16(dot);
+            }
+        }
+    }
+}
+
+static void *tile_worker(void *arg) {
+    tile_job *job = (tile_job *)arg;
+    for (;;) {
+        pthread_mutex_lock(&job->lock);
+        const size_t start = job->next_row;
+        job->next_row = start + job->grain;
+        pthread_mutex_unlock(&job->lock);
+        if (start >= job->M) {
+            break;
+        }
+        size_t end = start + job->grain;
+        if (end > job->M) {
+            end = job->M;
+        }
+        tile_compute_rows(job, start, end);
+    }
+    return NULL;
+}
+
+static void run_tile(tile_job *job, int threads) {
+    job->next_row = 0;
+    size_t tasks = (job->M + job->grain - 1) / job->grain;
+    int nthreads = threads;
+    if ((size_t)nthreads > tasks) {
+        nthreads = (int)tasks;
+    }
+    if (nthreads <= 1) {
+        tile_compute_rows(job, 0, job->M);
+        return;
+    }
+    pthread_mutex_init(&job->lock, NULL);
+    pthread_t *tids = (pthread_t *)malloc(sizeof(pthread_t) * (size_t)nthreads);
+    int started = 0;
+    for (int t = 0; t < nthreads - 1; ++t) {
+        if (pthread_create(&tids[started], NULL, tile_worker, job) == 0) {
+            started++;
+        }
+    }
+    tile_worker(job);
+    for (int t = 0; t < started; ++t) {
+        pthread_join(tids[t], NULL);
+    }
+    free(tids);
+    pthread_mutex_destroy(&job->lock);
+}
+
+/* matmul_quant_dispatch.c:373-591 + core/helpers/matmul.c:68-136 + matmul_epilogue.c */
+int mo_matmul_quantized(
+    int kind, const void *weight, const void *input, int in_dtype, size_t N, size_t K, size_t M, const float *bias,
+    void *out, int out_dtype, int force_pack, int threads
+) {
+    if (weight == NULL || input == NULL || out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    dot_fn dot = pick_dot(kind);
+    if (dot == NULL) {
+        return MO_ERR_UNSUPPORTED_DTYPE;
+    }
+    const int in_f32 = in_dtype == MO_DTYPE_F32;
+    const int in_f16 = in_dtype == MO_DTYPE_F16;
+    const int out_f32 = out_dtype == MO_DTYPE_F32;
+    const int out_f16 = out_dtype == MO_DTYPE_F16;
+    if (!((in_f32 && out_f32) || (in_f16 && (out_f32 || out_f16)))) {
+        return MO_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (threads < 1) {
+        threads = 1;
+    }
+    const size_t bv = mo_block_values(kind);
+    const size_t bb = mo_block_bytes(kind);
+    const size_t blocks_per_row = (K + bv - 1) / bv;
+    const int use_q8_k = (bv == QK_K);
+    const size_t act_bb = use_q8_k ? sizeof(blk_q8_k) : sizeof(blk_q8_0);
+    const int direct = in_f16 && !force_pack;
+
+    tile_job job;
+    memset(&job, 0, sizeof(job));
+    job.kind = kind;
+    job.direct_f16 = direct;
+    job.weight = (const uint8_t *)weight;
+    job.row_bytes = bb * blocks_per_row;
+    job.block_bytes = bb;
+    job.blocks_per_row = blocks_per_row;
+    job.act_block_bytes = act_bb;
+    job.K = K;
+    job.M = M;
+    job.out_f32 = out_f32 ? (float *)out : NULL;
+    job.out_f16 = out_f16 ? (uint16_t *)out : NULL;
+    job.dot = dot;
+    job.act_f16 = (const uint16_t *)input;
+
+    uint8_t *act_tile = NULL;
+    if (!direct) {
+        act_tile = (uint8_t *)malloc(TILE_COLS * blocks_per_row * act_bb + 1);
+        if (act_tile == NULL) {
+            return MO_ERR_OUT_OF_MEMORY;
+        }
+    }
+    job.act_tile = act_tile;
+    const size_t in_elt = in_f16 ? 2 : 4;
+
+    for (size_t n0 = 0; n0 < N; n0 += TILE_COLS) {
+        const size_t cols = (n0 + TILE_COLS <= N) ? TILE_COLS : (N - n0);
+        job.n0 = n0;
+        job.cols_in_tile = cols;
+        if (!direct) {
+            for (size_t c = 0; c < cols; ++c) {
+                const uint8_t *row = (const uint8_t *)input + (n0 + c) * K * in_elt;
+                uint8_t *dst = act_tile + c * blocks_per_row * act_bb;
+                if (use_q8_k) {
+                    mo_pack_q8_k(row, in_dtype, K, dst);
+                } else {
+                    mo_pack_q8_0(row, in_dtype, K, dst);
+                }
+            }
+            job.grain = mo_row_grain(M, cols, (size_t)threads);
+        } else {
+            job.grain = 64; /* matmul_quant_compute.c:1936-1938 */
+        }
+        run_tile(&job, threads);
+    }
+    free(act_tile);
+
+    if (bias != NULL) {
+        if (out_f32) {
+            float *o = (float *)out;
+            for (size_t n = 0; n < N; ++n) {
+                for (size_t m = 0; m < M; ++m) {
+                    o[n * M + m] += bias[m];
+                }
+            }
+        } else {
+            uint16_t *o = (uint16_t *)out;
+            for (size_t n = 0; n < N; ++n) {
+                for (size_t m = 0; m < M; ++m) {
+                    const float v = mo_f16_to_f32(o[n * M + m]);
+                    o[n * M + m] = mo_f32_to_f16(v + bias[m]);
+                }
+            }
+        }
+    }
+    return MO_OK;
+}
+
+/* ======================= top-k / router / MoE ======================= */
+
+/* moe_ops.c:789-889 */
+int mo_topk(const float *x, size_t rows, size_t cols, size_t k, float *values_out, int32_t *indices_out) {
+    if (x == NULL || values_out == NULL || indices_out == NULL || k == 0 || k > cols) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    for (size_t row = 0; row < rows; ++row) {
+        float *bvals = values_out + row * k;
+        int32_t *bidx = indices_out + row * k;
+        for (size_t i = 0; i < k; ++i) {
+            bvals[i] = -FLT_MAX;
+            bidx[i] = -1;
+        }
+        for (size_t col = 0; col < cols; ++col) {
+            const float value = x[row * cols + col];
+            size_t insert_pos = k;
+            for (size_t i = 0; i < k; ++i) {
+                const int better = value > bvals[i];
+                const int same = value == bvals[i] && (int32_t)col < bidx[i];
+                if (better || same) {
+                    insert_pos = i;
+                    break;
+                }
+            }
+            if (insert_pos == k) {
+                continue;
+            }
+            for (size_t i = k - 1; i > insert_pos; --i) {
+                bvals[i] = bvals[i - 1];
+                bidx[i] = bidx[i - 1];
+            }
+            bvals[insert_pos] = value;
+            bidx[insert_pos] = (int32_t)col;
+        }
+    }
+    return MO_OK;
+}
+
+/* Numerically-stable softmax over the selected logits; the graph applies marmot's generic softmax op
+ * to the [T,k] top-k values (graph_builder.cpp:2276-2316): max-subtract, expf, sum in order, divide. */
+void mo_softmax_rows(const float *x, size_t rows, size_t k, float *out) {
+    for (size_t r = 0; r < rows; ++r) {
+        const float *in = x + r * k;
+        float *o = out + r * k;
+        float mx = in[0];
+        for (size_t i = 1; i < k; ++i) {
+            if (in[i] > mx) {
+                mx = in[i];
+            }
+        }
+        float sum = 0.0f;
+        for (size_t i = 0; i < k; ++i) {
+            o[i] = expf(in[i] - mx);
+            sum += o[i];
+        }
+        for (size_t i = 0; i < k; ++i) {
+            o[i] = o[i] / sum;
+        }
+    }
+}
+
+/* moe_ops.c:318-324 */
+static inline float moe_silu(float x) {
+    return x / (1.0f + expf(-x));
+}
+static inline float moe_gelu(float x) {
+    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+/* moe_ops.c:506-568: gate/up (shared activation quantization) -> act(gate)*up -> down */
+static int moe_expert_body(
+    const float *rows_in, size_t count, size_t H, size_t F, int kind_gu, int kind_down, const uint8_t *gate_w,
+    const uint8_t *up_w, const uint8_t *down_w, int ffn_type, int threads, float *gate_buf, float *up_buf,
+    float *down_out
+) {
+    int st = mo_matmul_quantized(kind_gu, gate_w, rows_in, MO_DTYPE_F32, count, H, F, NULL, gate_buf, MO_DTYPE_F32, 0,
+                                 threads);
+    if (st != MO_OK) {
+        return st;
+    }
+    st = mo_matmul_quantized(kind_gu, up_w, rows_in, MO_DTYPE_F32, count, H, F, NULL, up_buf, MO_DTYPE_F32, 0,
+                             threads);
+    if (st != MO_OK) {
+        return st;
+    }
+    for (size_t i = 0; i < count * F; ++i) {
+        const float g = gate_buf[i];
+        const float a = ffn_type == MO_FFN_GEGLU ? moe_gelu(g) : moe_silu(g);
+        gate_buf[i] = a * up_buf[i];
+    }
+    return mo_matmul_quantized(kind_down, down_w, gate_buf, MO_DTYPE_F32, count, F, H, NULL, down_out, MO_DTYPE_F32,
+                               0, threads);
+}
+
+/* moe_ops.c:475-504: active experts by descending route count, ties by ascending id */
+static size_t moe_build_expert_order(size_t *order, const size_t *counts, size_t E) {
+    size_t active = 0;
+    for (size_t e = 0; e < E; ++e) {
+        if (counts[e] != 0) {
+            order[active++] = e;
+        }
+    }
+    for (size_t i = 1; i < active; ++i) {
+        const size_t e = order[i];
+        const size_t c = counts[e];
+        size_t j = i;
+        while (j > 0) {
+            const size_t pe = order[j - 1];
+            const size_t pc = counts[pe];
+            if (pc > c || (pc == c && pe < e)) {
+                break;
+            }
+            order[j] = pe;
+            --j;
+        }
+        order[j] = e;
+    }
+    return active;
+}
+
+typedef struct {
+    size_t H, F;
+    int kind_gu, kind_down;
+    const uint8_t *gate, *up, *down;
+    size_t gu_slice, down_slice;
+    int ffn_type;
+    const size_t *counts;
+    const size_t *offsets;
+    size_t *order;
+    size_t active;
+    const float *route_hidden;
+    float *route_down;
+    float *gate_buf;
+    float *up_buf;
+    int inner_threads;
+    size_t next;
+    int first_error;
+    pthread_mutex_t lock;
+} moe_group_ctx;
+
+static void *moe_group_worker(void *arg) {
+    moe_group_ctx *g = (moe_group_ctx *)arg;
+    for (;;) {
+        pthread_mutex_lock(&g->lock);
+        const size_t idx = g->next++;
+        const int err = g->first_error;
+        pthread_mutex_unlock(&g->lock);
+        if (err != MO_OK || idx >= g->active) {
+            break;
+        }
+        const size_t e = g->order[idx];
+        const size_t off = g->offsets[e];
+        const int st = moe_expert_body(
+            g->route_hidden + off * g->H, g->counts[e], g->H, g->F, g->kind_gu, g->kind_down,
+            g->gate + e * g->gu_slice, g->up + e * g->gu_slice, g->down + e * g->down_slice, g->ffn_type,
+            g->inner_threads, g->gate_buf + off * g->F, g->up_buf + off * g->F, g->route_down + off * g->H
+        );
+        if (st != MO_OK) {
+            pthread_mutex_lock(&g->lock);
+            if (g->first_error == MO_OK) {
+                g->first_error = st;
+            }
+            pthread_mutex_unlock(&g->lock);
+            break;
+        }
+    }
+    return NULL;
+}
+
+static int moe_run_group(moe_group_ctx *g, int workers) {
+    g->next = 0;
+    g->first_error = MO_OK;
+    pthread_mutex_init(&g->lock, NULL);
+    if ((size_t)workers > g->active) {
+        workers = (int)g->active;
+    }
+    if (workers <= 1) {
+        moe_group_worker(g);
+    } else {
+        pthread_t *tids = (pthread_t *)malloc(sizeof(pthread_t) * (size_t)workers);
+        int started = 0;
+        for (int t = 0; t < workers - 1; ++t) {
+            if (pthread_create(&tids[started], NULL, moe_group_worker, g) == 0) {
+                started++;
+            }
+        }
+        moe_group_worker(g);
+        for (int t = 0; t < started; ++t) {
+            pthread_join(tids[t], NULL);
+        }
+        free(tids);
+    }
+    pthread_mutex_destroy(&g->lock);
+    return g->first_error;
+}
+
+int mo_moe_experts(
+    const float *hidden, size_t T, size_t H, size_t F, size_t E, size_t kpt, int kind_gu, int kind_down,
+    const void *gate, const void *up, const void *down, const int32_t *topk_ids, const float *topk_weights,
+    float weights_scale, int policy, int ffn_type, int force_grouped, int threads, float *out
+) {
+    if (hidden == NULL || gate == NULL || up == NULL || down == NULL || topk_ids == NULL || topk_weights == NULL ||
+        out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    if (ffn_type != MO_FFN_SWIGLU && ffn_type != MO_FFN_GEGLU) {
+        return MO_ERR_NOT_IMPLEMENTED;
+    }
+    const size_t routes = T * kpt;
+    const size_t gu_slice = F * mo_row_bytes(kind_gu, H);  /* moe_ops.c:326-345 */
+    const size_t down_slice = H * mo_row_bytes(kind_down, F);
+    if (gu_slice == 0 || down_slice == 0) {
+        return MO_ERR_UNSUPPORTED_DTYPE;
+    }
+
+    uint32_t *sorted_tokens = (uint32_t *)malloc((routes + 1) * sizeof(uint32_t));
+    float *sorted_weights = (float *)malloc((routes + 1) * sizeof(float));
+    size_t *counts = (size_t *)calloc(E + 1, sizeof(size_t));
+    size_t *offsets = (size_t *)calloc(E + 1, sizeof(size_t));
+    size_t *cursor = (size_t *)calloc(E + 1, sizeof(size_t));
+    float *route_hidden = (float *)malloc((routes * H + 1) * sizeof(float));
+    float *route_down = (float *)malloc((routes * H + 1) * sizeof(float));
+    float *gate_buf = (float *)malloc((routes * F + 1) * sizeof(float));
+    float *up_buf = (float *)malloc((routes * F + 1) * sizeof(float));
+    int status = MO_OK;
+    if (!sorted_tokens || !sorted_weights || !counts || !offsets || !cursor || !route_hidden || !route_down ||
+        !gate_buf || !up_buf) {
+        status = MO_ERR_OUT_OF_MEMORY;
+        goto done;
+    }
+
+    const int decode = !force_grouped && T <= 4 && routes <= 64; /* moe_ops.c:417-424 */
+
+    if (decode) {
+        /* moe_ops.c:622-787: experts in first-appearance order */
+        uint32_t active[64];
+        size_t acount[64], aoff[64], acur[64];
+        size_t nactive = 0;
+        for (size_t t = 0; t < T; ++t) {
+            memset(out + t * H, 0, H * sizeof(float));
+            for (size_t s = 0; s < kpt; ++s) {
+                const int32_t e = topk_ids[t * kpt + s];
+                if (e < 0) {
+                    status = MO_ERR_INVALID_ARGUMENT;
+                    goto done;
+                }
+                size_t slot = 0;
+                for (; slot < nactive; ++slot) {
+                    if (active[slot] == (uint32_t)e) {
+                        break;
+                    }
+                }
+                if (slot == nactive) {
+                    active[nactive] = (uint32_t)e;
+                    acount[nactive] = 0;
+                    nactive++;
+                }
+                acount[slot]++;
+            }
+        }
+        size_t prefix = 0;
+        for (size_t slot = 0; slot < nactive; ++slot) {
+            aoff[slot] = prefix;
+            acur[slot] = prefix;
+            prefix += acount[slot];
+        }
+        for (size_t t = 0; t < T; ++t) {
+            float norm = weights_scale;
+            if (policy == MO_ROUTER_RENORMALIZE_SELECTED) {
+                float ws = 0.0f;
+                for (size_t s = 0; s < kpt; ++s) {
+                    ws += topk_weights[t * kpt + s];
+                }
+                norm = ws > FLT_MIN ? weights_scale / ws : 0.0f;
+            }
+            for (size_t s = 0; s < kpt; ++s) {
+                const uint32_t e = (uint32_t)topk_ids[t * kpt + s];
+                size_t slot = 0;
+                for (; slot < nactive; ++slot) {
+                    if (active[slot] == e) {
+                        break;
+                    }
+                }
+                const size_t pos = acur[slot]++;
+                sorted_tokens[pos] = (uint32_t)t;
+                sorted_weights[pos] = topk_weights[t * kpt + s] * norm;
+            }
+        }
+        for (size_t slot = 0; slot < nactive; ++slot) {
+            const size_t count = acount[slot];
+            const size_t off = aoff[slot];
+            const size_t e = active[slot];
+            if (e >= E) {
+                status = MO_ERR_INVALID_ARGUMENT;
+                goto done;
+            }
+            for (size_t r = 0; r < count; ++r) {
+                memcpy(route_hidden + r * H, hidden + (size_t)sorted_tokens[off + r] * H, H * sizeof(float));
+            }
+            status = moe_expert_body(route_hidden, count, H, F, kind_gu, kind_down,
+                                     (const uint8_t *)gate + e * gu_slice, (const uint8_t *)up + e * gu_slice,
+                                     (const uint8_t *)down + e * down_slice, ffn_type, threads, gate_buf, up_buf,
+                                     route_down);
+            if (status != MO_OK) {
+                goto done;
+            }
+            for (size_t r = 0; r < count; ++r) {
+                const size_t t = sorted_tokens[off + r];
+                const float w = sorted_weights[off + r];
+                for (size_t c = 0; c < H; ++c) {
+                    out[t * H + c] += w * route_down[r * H + c];
+                }
+            }
+        }
+        goto done;
+    }
+
+    /* grouped path: moe_ops.c:891-1049 */
+    for (size_t t = 0; t < T; ++t) {
+        for (size_t s = 0; s < kpt; ++s) {
+            const int32_t e = topk_ids[t * kpt + s];
+            if (e < 0 || (size_t)e >= E) {
+                status = MO_ERR_INVALID_ARGUMENT;
+                goto done;
+            }
+            counts[e]++;
+        }
+    }
+    size_t prefix = 0;
+    for (size_t e = 0; e < E; ++e) {
+        offsets[e] = prefix;
+        cursor[e] = prefix;
+        prefix += counts[e];
+    }
+    for (size_t t = 0; t < T; ++t) {
+        float norm = weights_scale;
+        if (policy == MO_ROUTER_RENORMALIZE_SELECTED) {
+            float ws = 0.0f;
+            for (size_t s = 0; s < kpt; ++s) {
+                ws += topk_weights[t * kpt + s];
+            }
+            norm = ws > FLT_MIN ? weights_scale / ws : 0.0f;
+        }
+        for (size_t s = 0; s < kpt; ++s) {
+            const size_t e = (size_t)topk_ids[t * kpt + s];
+            const size_t pos = cursor[e]++;
+            sorted_tokens[pos] = (uint32_t)t;
+            sorted_weights[pos] = topk_weights[t * kpt + s] * norm;
+        }
+    }
+    for (size_t r = 0; r < routes; ++r) {
+        memcpy(route_hidden + r * H, hidden + (size_t)sorted_tokens[r] * H, H * sizeof(float));
+    }
+    for (size_t t = 0; t < T; ++t) {
+        memset(out + t * H, 0, H * sizeof(float));
+    }
+    /* moe_ops.c:475-504, 586-620, 1004-1031: experts are visited in descending-count order, in parallel over
+     * experts (inner matmul single-threaded) when there are >= 32 routes and more than one thread. Each expert
+     * writes disjoint slices of the route buffers, so the visiting order does not change any value. */
+    {
+        moe_group_ctx g;
+        memset(&g, 0, sizeof(g));
+        g.H = H;
+        g.F = F;
+        g.kind_gu = kind_gu;
+        g.kind_down = kind_down;
+        g.gate = (const uint8_t *)gate;
+        g.up = (const uint8_t *)up;
+        g.down = (const uint8_t *)down;
+        g.gu_slice = gu_slice;
+        g.down_slice = down_slice;
+        g.ffn_type = ffn_type;
+        g.counts = counts;
+        g.offsets = offsets;
+        g.route_hidden = route_hidden;
+        g.route_down = route_down;
+        g.gate_buf = gate_buf;
+        g.up_buf = up_buf;
+        g.order = cursor; /* cursor[] is no longer needed: reuse as the visiting order */
+        g.active = moe_build_expert_order(g.order, counts, E);
+        const int parallel = threads > 1 && routes >= 32;
+        g.inner_threads = parallel ? 1 : threads;
+        status = moe_run_group(&g, parallel ? threads : 1);
+        if (status != MO_OK) {
+            goto done;
+        }
+    }
+    /* moe_ops.c:1034-1042: scatter in sorted-route order */
+    for (size_t r = 0; r < routes; ++r) {
+        const size_t t = sorted_tokens[r];
+        const float w = sorted_weights[r];
+        for (size_t c = 0; c < H; ++c) {
+            out[t * H + c] += w * route_down[r * H + c];
+        }
+    }
+
+done:
+    free(sorted_tokens);
+    free(sorted_weights);
+    free(counts);
+    free(offsets);
+    free(cursor);
+    free(route_hidden);
+    free(route_down);
+    free(gate_buf);
+    free(up_buf);
+    return status;
+}

@@ -1,0 +1,126 @@
+/*
+ * marmot_oracle — TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain-C, CPU-only restatement of the arithmetic of marmot's CPU backend for
+ * block-quantized (GGUF) weight x float activation matmul.  It exists to check
+ * the HIP kernels and to be timed as the CPU baseline; nothing in the product
+ * library links, loads or calls it.
+ *
+ * Every function names the reference file:line whose behaviour it restates
+ * (paths relative to the reference checkout).  The restatement follows the
+ * reference's *scalar* configuration (no NEON/AVX2 paths, no FMA contraction),
+ * which fixes rounding: Q8_0 uses roundf (half away from zero), K-quants use
+ * the magic-number round-to-nearest-even.
+ *
+ * Pinned by (see tests/test_oracle_*.py):
+ *   - the reference's own golden vectors for quantizer bytes, dequantized
+ *     values, block dot products and whole matmuls;
+ *   - a shared library compiled from the reference's own leaf sources
+ *     (oracle/_ref) on seeded Gaussian rows, byte- and bit-exact;
+ *   - float64 brute force and closed-form special cases.
+ * "parity unpinned": none of the functions below; the MoE driver and top-k are
+ * pinned by brute force against dense math and the reference tests' tie cases
+ * only (the reference holds no golden vector for them).
+ */
+#ifndef MARMOT_ORACLE_H
+#define MARMOT_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* quant kinds: numeric values of marmot_quant_kind_t (include/marmot/types.h:372-388) */
+enum {
+    MO_KIND_Q4_0 = 1,
+    MO_KIND_Q8_0 = 5,
+    MO_KIND_Q4_K = 9,
+    MO_KIND_Q6_K = 11,
+    MO_KIND_Q8_K = 12,
+};
+
+/* dtype ids: numeric values of marmot_dtype_t (include/marmot/types.h:340-362) */
+enum {
+    MO_DTYPE_F32 = 0,
+    MO_DTYPE_F16 = 1,
+};
+
+enum {
+    MO_ROUTER_SOFTMAX_SELECTED = 0,
+    MO_ROUTER_SOFTMAX_SELECTED_SCALED = 1,
+    MO_ROUTER_RENORMALIZE_SELECTED = 2,
+};
+
+enum { MO_FFN_SWIGLU = 0, MO_FFN_GEGLU = 2 };
+
+/* block geometry (include/marmot/quant_block.h:20-125) */
+size_t mo_block_values(int kind);
+size_t mo_block_bytes(int kind);
+size_t mo_row_bytes(int kind, size_t k);
+
+/* fp16 <-> fp32: exact widening, round-to-nearest-even narrowing
+ * (the reference uses a native _Float16 cast, cpu_backend_internal.h:600-606) */
+float mo_f16_to_f32(uint16_t h);
+uint16_t mo_f32_to_f16(float f);
+
+/* weight quantizers: `rows` rows of `k` floats -> rows * mo_row_bytes(kind,k) bytes.
+ * Tails are zero-padded per block (ops/quantize_core.c:199-265). Returns 0 on success. */
+int mo_quantize_rows(int kind, const float *x, size_t rows, size_t k, void *out);
+
+/* dequantizers (the bit-exact contract). Returns 0 on success. */
+int mo_dequantize_rows(int kind, const void *blocks, size_t rows, size_t k, float *out);
+
+/* activation packers (matmul_quant_pack.c:23-196). in_dtype: MO_DTYPE_F32/F16. */
+void mo_pack_q8_0(const void *x, int in_dtype, size_t k, void *blocks_out);
+void mo_pack_q8_k(const void *x, int in_dtype, size_t k, void *blocks_out);
+
+/* integer block dots (vec_dot_impl.h) over `nblocks` consecutive blocks */
+float mo_vec_dot_q8_0_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q4_0_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q6_k_q8_k(const void *w, const void *a, size_t nblocks);
+
+/* fp16-activation direct dots (vec_dot_impl.h:220-250, 419-450, 973-1023) */
+float mo_vec_dot_f16(int kind, const void *w, const uint16_t *a, size_t nblocks, size_t k);
+
+/*
+ * marmot_linear for a quantized weight: out[n*M + m] = dot(W[m,:], x[n,:]) (+ bias[m]).
+ *   in_dtype F32  -> packed path (Q8_0 for Q4_0/Q8_0 weights, Q8_K for K-quants)
+ *   in_dtype F16  -> direct path unless force_pack != 0
+ *   out_dtype F32 or F16 (F16 only allowed with F16 input)
+ *   bias: NULL or M floats (fp32 bias; applied after the store like the reference)
+ *   threads: weight rows are split over this many worker threads (>=1)
+ * Returns 0, or a negative marmot_error_t value on invalid arguments.
+ */
+int mo_matmul_quantized(
+    int kind, const void *weight, const void *input, int in_dtype, size_t N, size_t K, size_t M, const float *bias,
+    void *out, int out_dtype, int force_pack, int threads
+);
+
+/* top-k over the last axis, ties -> lower index (moe_ops.c:789-889) */
+int mo_topk(const float *x, size_t rows, size_t cols, size_t k, float *values_out, int32_t *indices_out);
+
+/* router: softmax over the k selected logits (graph_builder.cpp:2276-2316) */
+void mo_softmax_rows(const float *x, size_t rows, size_t k, float *out);
+
+/*
+ * marmot_moe_experts, fp32 activations, block-quantized experts (moe_ops.c:891-1049, 622-787).
+ * gate/up: E slices of [F, H] rows; down: E slices of [H, F]. kind_gate_up / kind_down are quant kinds.
+ * force_grouped != 0 disables the <=4-token decode path.
+ */
+int mo_moe_experts(
+    const float *hidden, size_t T, size_t H, size_t F, size_t E, size_t k_per_token, int kind_gate_up, int kind_down,
+    const void *gate, const void *up, const void *down, const int32_t *topk_ids, const float *topk_weights,
+    float weights_scale, int policy, int ffn_type, int force_grouped, int threads, float *out
+);
+
+/* row grain used to split weight rows over threads (matmul_quant_compute.c:1222-1240) */
+size_t mo_row_grain(size_t row_count, size_t cols_in_tile, size_t thread_cap);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

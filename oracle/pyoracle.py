@@ -1,0 +1,324 @@
+"""ctypes bindings for the CPU oracle and for the reference-built leaf library.
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` — never by the product package.
+
+``Oracle``  wraps ``oracle/libmarmot_oracle.so`` (own restatement, see marmot_oracle.h).
+``RefLib``  wraps ``oracle/_ref/libmarmot_ref.so`` — the reference's own quantizer / dequantizer /
+            packer / block-dot translation units compiled as they lie (oracle/Makefile, target ``ref``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(HERE, "libmarmot_oracle.so")
+REF_SO = os.path.join(HERE, "_ref", "libmarmot_ref.so")
+
+KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_K = 1, 5, 9, 11, 12
+KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q6_k": KIND_Q6_K, "q8_k": KIND_Q8_K}
+BLOCK_VALUES = {KIND_Q4_0: 32, KIND_Q8_0: 32, KIND_Q4_K: 256, KIND_Q6_K: 256, KIND_Q8_K: 256}
+BLOCK_BYTES = {KIND_Q4_0: 18, KIND_Q8_0: 34, KIND_Q4_K: 144, KIND_Q6_K: 210, KIND_Q8_K: 292}
+DT_F32, DT_F16 = 0, 1
+
+
+def row_bytes(kind: int, k: int) -> int:
+    bv = BLOCK_VALUES[kind]
+    return ((k + bv - 1) // bv) * BLOCK_BYTES[kind]
+
+
+def build_oracle(force: bool = False) -> str:
+    if force or not os.path.exists(ORACLE_SO):
+        subprocess.check_call(["make", "-C", HERE, "-B" if force else "-s", "all"])
+    return ORACLE_SO
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Oracle:
+    def __init__(self, path: str | None = None):
+        path = path or build_oracle()
+        L = C.CDLL(path)
+        self.L = L
+        L.mo_f16_to_f32.restype = C.c_float
+        L.mo_f16_to_f32.argtypes = [C.c_uint16]
+        L.mo_f32_to_f16.restype = C.c_uint16
+        L.mo_f32_to_f16.argtypes = [C.c_float]
+        L.mo_quantize_rows.restype = C.c_int
+        L.mo_quantize_rows.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+        L.mo_dequantize_rows.restype = C.c_int
+        L.mo_dequantize_rows.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+        for n in ("mo_pack_q8_0", "mo_pack_q8_k"):
+            f = getattr(L, n)
+            f.restype = None
+            f.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
+        for n in ("mo_vec_dot_q8_0_q8_0", "mo_vec_dot_q4_0_q8_0", "mo_vec_dot_q4_k_q8_k", "mo_vec_dot_q6_k_q8_k"):
+            f = getattr(L, n)
+            f.restype = C.c_float
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.mo_vec_dot_f16.restype = C.c_float
+        L.mo_vec_dot_f16.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t]
+        L.mo_matmul_quantized.restype = C.c_int
+        L.mo_matmul_quantized.argtypes = [
+            C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
+            C.c_int, C.c_int, C.c_int,
+        ]
+        L.mo_topk.restype = C.c_int
+        L.mo_topk.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
+        L.mo_softmax_rows.restype = None
+        L.mo_softmax_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+        L.mo_moe_experts.restype = C.c_int
+        L.mo_moe_experts.argtypes = [
+            C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_void_p,
+            C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+        ]
+        L.mo_row_grain.restype = C.c_size_t
+        L.mo_row_grain.argtypes = [C.c_size_t, C.c_size_t, C.c_size_t]
+
+    # ---- fp16
+    def f16_to_f32(self, h: int) -> float:
+        return float(self.L.mo_f16_to_f32(h))
+
+    def f32_to_f16(self, f: float) -> int:
+        return int(self.L.mo_f32_to_f16(np.float32(f)))
+
+    # ---- quantize / dequantize
+    def quantize(self, kind: int, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        rows, k = x.shape
+        out = np.zeros((rows, row_bytes(kind, k)), dtype=np.uint8)
+        st = self.L.mo_quantize_rows(kind, _ptr(x), rows, k, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_quantize_rows -> {st}")
+        return out
+
+    def dequantize(self, kind: int, blocks: np.ndarray, k: int) -> np.ndarray:
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        if blocks.ndim == 1:
+            blocks = blocks[None, :]
+        rows = blocks.shape[0]
+        assert blocks.shape[1] == row_bytes(kind, k), (blocks.shape, row_bytes(kind, k))
+        out = np.zeros((rows, k), dtype=np.float32)
+        st = self.L.mo_dequantize_rows(kind, _ptr(blocks), rows, k, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_dequantize_rows -> {st}")
+        return out
+
+    # ---- activation packers
+    def pack(self, act_kind: int, x: np.ndarray) -> np.ndarray:
+        """x: 1-D float32 or float16 row -> packed Q8_0 / Q8_K blocks (uint8)."""
+        if x.dtype == np.float16:
+            dt = DT_F16
+        else:
+            x = np.ascontiguousarray(x, dtype=np.float32)
+            dt = DT_F32
+        x = np.ascontiguousarray(x)
+        k = x.shape[0]
+        out = np.zeros(row_bytes(act_kind, k), dtype=np.uint8)
+        fn = self.L.mo_pack_q8_0 if act_kind == KIND_Q8_0 else self.L.mo_pack_q8_k
+        fn(_ptr(x), dt, k, _ptr(out))
+        return out
+
+    def vec_dot(self, kind: int, w: np.ndarray, a: np.ndarray, nblocks: int) -> float:
+        fn = {
+            KIND_Q8_0: self.L.mo_vec_dot_q8_0_q8_0,
+            KIND_Q4_0: self.L.mo_vec_dot_q4_0_q8_0,
+            KIND_Q4_K: self.L.mo_vec_dot_q4_k_q8_k,
+            KIND_Q6_K: self.L.mo_vec_dot_q6_k_q8_k,
+        }[kind]
+        w = np.ascontiguousarray(w, dtype=np.uint8)
+        a = np.ascontiguousarray(a, dtype=np.uint8)
+        return float(fn(_ptr(w), _ptr(a), nblocks))
+
+    def vec_dot_f16(self, kind: int, w: np.ndarray, a: np.ndarray, k: int) -> float:
+        w = np.ascontiguousarray(w, dtype=np.uint8)
+        a = np.ascontiguousarray(a, dtype=np.float16)
+        nb = (k + BLOCK_VALUES[kind] - 1) // BLOCK_VALUES[kind]
+        return float(self.L.mo_vec_dot_f16(kind, _ptr(w), _ptr(a), nb, k))
+
+    # ---- matmul
+    def matmul(self, kind: int, weight: np.ndarray, x: np.ndarray, M: int, bias=None, out_dtype=None,
+               force_pack: bool = False, threads: int = 1) -> np.ndarray:
+        weight = np.ascontiguousarray(weight, dtype=np.uint8)
+        if x.dtype == np.float16:
+            in_dt = DT_F16
+        else:
+            x = x.astype(np.float32, copy=False)
+            in_dt = DT_F32
+        x = np.ascontiguousarray(x)
+        N, K = x.shape
+        assert weight.size == M * row_bytes(kind, K), (weight.size, M, K)
+        if out_dtype is None:
+            out_dtype = np.float32
+        out = np.zeros((N, M), dtype=out_dtype)
+        out_dt = DT_F16 if out.dtype == np.float16 else DT_F32
+        b = None
+        if bias is not None:
+            b = np.ascontiguousarray(bias, dtype=np.float32)
+        st = self.L.mo_matmul_quantized(
+            kind, _ptr(weight), _ptr(x), in_dt, N, K, M, _ptr(b) if b is not None else None, _ptr(out), out_dt,
+            1 if force_pack else 0, threads,
+        )
+        if st != 0:
+            raise RuntimeError(f"mo_matmul_quantized -> {st}")
+        return out
+
+    # ---- MoE
+    def topk(self, x: np.ndarray, k: int):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        rows, cols = x.shape
+        vals = np.zeros((rows, k), dtype=np.float32)
+        idx = np.zeros((rows, k), dtype=np.int32)
+        st = self.L.mo_topk(_ptr(x), rows, cols, k, _ptr(vals), _ptr(idx))
+        if st != 0:
+            raise RuntimeError(f"mo_topk -> {st}")
+        return vals, idx
+
+    def softmax_rows(self, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        out = np.zeros_like(x)
+        self.L.mo_softmax_rows(_ptr(x), x.shape[0], x.shape[1], _ptr(out))
+        return out
+
+    def moe_experts(self, hidden, gate, up, down, topk_ids, topk_weights, F: int, E: int, kind_gate_up: int,
+                    kind_down: int, weights_scale: float = 1.0, policy: int = 1, ffn_type: int = 0,
+                    force_grouped: bool = False, threads: int = 1) -> np.ndarray:
+        hidden = np.ascontiguousarray(hidden, dtype=np.float32)
+        T, H = hidden.shape
+        ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
+        w = np.ascontiguousarray(topk_weights, dtype=np.float32)
+        kpt = ids.shape[1]
+        gate = np.ascontiguousarray(gate, dtype=np.uint8)
+        up = np.ascontiguousarray(up, dtype=np.uint8)
+        down = np.ascontiguousarray(down, dtype=np.uint8)
+        assert gate.size == E * F * row_bytes(kind_gate_up, H)
+        assert down.size == E * H * row_bytes(kind_down, F)
+        out = np.zeros((T, H), dtype=np.float32)
+        st = self.L.mo_moe_experts(
+            _ptr(hidden), T, H, F, E, kpt, kind_gate_up, kind_down, _ptr(gate), _ptr(up), _ptr(down), _ptr(ids),
+            _ptr(w), weights_scale, policy, ffn_type, 1 if force_grouped else 0, threads, _ptr(out),
+        )
+        if st != 0:
+            raise RuntimeError(f"mo_moe_experts -> {st}")
+        return out
+
+    def row_grain(self, rows: int, cols: int, threads: int) -> int:
+        return int(self.L.mo_row_grain(rows, cols, threads))
+
+
+class _QuantTraits(C.Structure):
+    # include/marmot/quant_traits.h:30-43
+    _fields_ = [
+        ("kind", C.c_int),
+        ("name", C.c_char_p),
+        ("block_size", C.c_uint32),
+        ("block_bytes", C.c_uint32),
+        ("weight_bits", C.c_uint32),
+        ("has_zero_point", C.c_bool),
+        ("requires_calibration", C.c_bool),
+        ("layout", C.c_int),
+        ("compute_params", C.c_void_p),
+        ("quantize_block", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p)),
+        ("dequantize_block", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p)),
+        ("vec_dot_block", C.c_void_p),
+    ]
+
+
+class RefLib:
+    """The reference's own leaf arithmetic (scalar build), where oracle/_ref was built."""
+
+    @staticmethod
+    def available() -> bool:
+        return os.path.exists(REF_SO)
+
+    def __init__(self):
+        L = C.CDLL(REF_SO)
+        self.L = L
+        L.marmot_get_quant_traits.restype = C.POINTER(_QuantTraits)
+        L.marmot_get_quant_traits.argtypes = [C.c_int]
+        for n in ("cpu_matmul_quant_pack_q8_0_f32", "cpu_matmul_quant_pack_q8_k_f32", "cpu_matmul_quant_pack_q8_0_f16",
+                  "cpu_matmul_quant_pack_q8_k_f16"):
+            f = getattr(L, n)
+            f.restype = None
+            f.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
+        for n in ("q8_0_q8_0", "q4_0_q8_0", "q4_k_q8_k", "q6_k_q8_k"):
+            f = getattr(L, f"cpu_vec_dot_{n}_scalar")
+            f.restype = C.c_float
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        for n in ("q8_0", "q4_0", "q4_k", "q6_k"):
+            f = getattr(L, f"cpu_vec_dot_{n}_f16_scalar")
+            f.restype = C.c_float
+            f.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]
+
+    def _traits(self, kind: int) -> _QuantTraits:
+        p = self.L.marmot_get_quant_traits(kind)
+        if not p:
+            raise RuntimeError(f"reference has no traits for kind {kind}")
+        return p.contents
+
+    def quantize(self, kind: int, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        rows, k = x.shape
+        t = self._traits(kind)
+        bv, bb = t.block_size, t.block_bytes
+        nb = (k + bv - 1) // bv
+        out = np.zeros((rows, nb * bb), dtype=np.uint8)
+        for r in range(rows):
+            for b in range(nb):
+                elems = min(bv, k - b * bv)
+                src = x[r, b * bv:b * bv + elems]
+                src = np.ascontiguousarray(src)
+                st = t.quantize_block(_ptr(src), elems, C.c_void_p(out[r].ctypes.data + b * bb), None)
+                assert st == 0
+        return out
+
+    def dequantize(self, kind: int, blocks: np.ndarray, k: int) -> np.ndarray:
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        if blocks.ndim == 1:
+            blocks = blocks[None, :]
+        rows = blocks.shape[0]
+        t = self._traits(kind)
+        bv, bb = t.block_size, t.block_bytes
+        nb = (k + bv - 1) // bv
+        out = np.zeros((rows, k), dtype=np.float32)
+        for r in range(rows):
+            for b in range(nb):
+                elems = min(bv, k - b * bv)
+                st = t.dequantize_block(C.c_void_p(blocks[r].ctypes.data + b * bb), elems,
+                                        C.c_void_p(out[r].ctypes.data + 4 * b * bv), None)
+                assert st == 0
+        return out
+
+    def pack(self, act_kind: int, x: np.ndarray) -> np.ndarray:
+        f16 = x.dtype == np.float16
+        x = np.ascontiguousarray(x if f16 else x.astype(np.float32))
+        k = x.shape[0]
+        bv = BLOCK_VALUES[act_kind]
+        nb = (k + bv - 1) // bv
+        out = np.zeros(nb * BLOCK_BYTES[act_kind], dtype=np.uint8)
+        name = f"cpu_matmul_quant_pack_{'q8_0' if act_kind == KIND_Q8_0 else 'q8_k'}_{'f16' if f16 else 'f32'}"
+        getattr(self.L, name)(_ptr(x), 1, k, 0, k, nb, _ptr(out))
+        return out
+
+    def vec_dot(self, kind: int, w: np.ndarray, a: np.ndarray, nblocks: int) -> float:
+        name = {KIND_Q8_0: "q8_0_q8_0", KIND_Q4_0: "q4_0_q8_0", KIND_Q4_K: "q4_k_q8_k", KIND_Q6_K: "q6_k_q8_k"}[kind]
+        w = np.ascontiguousarray(w, dtype=np.uint8)
+        a = np.ascontiguousarray(a, dtype=np.uint8)
+        return float(getattr(self.L, f"cpu_vec_dot_{name}_scalar")(_ptr(w), _ptr(a), nblocks))
+
+    def vec_dot_f16(self, kind: int, w: np.ndarray, a: np.ndarray, k: int) -> float:
+        name = {KIND_Q8_0: "q8_0", KIND_Q4_0: "q4_0", KIND_Q4_K: "q4_k", KIND_Q6_K: "q6_k"}[kind]
+        w = np.ascontiguousarray(w, dtype=np.uint8)
+        a = np.ascontiguousarray(a, dtype=np.float16)
+        nb = (k + BLOCK_VALUES[kind] - 1) // BLOCK_VALUES[kind]
+        return float(getattr(self.L, f"cpu_vec_dot_{name}_f16_scalar")(_ptr(w), _ptr(a), 1, nb, k))

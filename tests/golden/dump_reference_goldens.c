@@ -1,0 +1,88 @@
+/*
+ * Fixture generator (runs only where the reference checkout is present).
+ *
+ * Includes the golden-vector headers that the reference's own tests hold
+ * (tests/backend/golden_quant_llama.h, golden_vec_dot_llama.h, golden_matmul_llama.h,
+ * matmul_quantized_golden_cases.h) directly from the reference tree at build time and
+ * writes their arrays as a flat binary container on stdout:
+ *     repeat { u32 name_len, name bytes, u32 dtype_len, dtype bytes, u64 nbytes, data }
+ * make_fixtures.py turns that stream into an .npz of plain arrays (data only).
+ */
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "marmot/quant_block.h"
+#include "marmot/types.h"
+
+#include "backend/matmul_quantized_golden_cases.h"
+#include "backend/golden_vec_dot_llama.h"
+
+static void emit(const char *name, const char *dtype, const void *data, size_t nbytes) {
+    uint32_t nl = (uint32_t)strlen(name);
+    uint32_t dl = (uint32_t)strlen(dtype);
+    uint64_t nb = (uint64_t)nbytes;
+    fwrite(&nl, 4, 1, stdout);
+    fwrite(name, 1, nl, stdout);
+    fwrite(&dl, 4, 1, stdout);
+    fwrite(dtype, 1, dl, stdout);
+    fwrite(&nb, 8, 1, stdout);
+    fwrite(data, 1, nbytes, stdout);
+}
+
+#define EMIT(arr, dtype) emit(#arr, dtype, arr, sizeof(arr))
+#define EMIT_SCALAR(v, dtype) emit(#v, dtype, &v, sizeof(v))
+
+int main(void) {
+    /* quantizer goldens */
+    EMIT(g_llama_test_input, "f4");
+    EMIT(g_llama_q4_0, "u1");
+    EMIT(g_llama_q4_0_dequant, "f4");
+    EMIT(g_llama_q8_0, "u1");
+    EMIT(g_llama_q8_0_dequant, "f4");
+    EMIT(g_llama_q4_k, "u1");
+    EMIT(g_llama_q4_k_dequant, "f4");
+    EMIT(g_llama_q6_k, "u1");
+    EMIT(g_llama_q6_k_dequant, "f4");
+    EMIT(g_llama_q8_k, "u1");
+    EMIT(g_llama_q8_k_dequant, "f4");
+
+    /* block-dot goldens */
+    EMIT(g_vec_dot_test_vec1, "f4");
+    EMIT(g_vec_dot_test_vec2, "f4");
+    EMIT(g_vec_dot_q8_0_activations, "u1");
+    EMIT(g_vec_dot_q8_k_activations, "u1");
+    EMIT(g_vec_dot_q4_0_weights, "u1");
+    EMIT(g_vec_dot_q8_0_weights, "u1");
+    EMIT(g_vec_dot_q4_k_weights, "u1");
+    EMIT(g_vec_dot_q6_k_weights, "u1");
+    EMIT_SCALAR(g_vec_dot_q4_0_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q8_0_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q4_k_q8_k_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q6_k_q8_k_expected, "f4");
+
+    /* whole-matmul goldens for the formats on the path */
+    const size_t ncases = sizeof(g_matmul_quant_goldens) / sizeof(g_matmul_quant_goldens[0]);
+    for (size_t i = 0; i < ncases; ++i) {
+        const matmul_golden_case_t *c = &g_matmul_quant_goldens[i];
+        if (c->kind != MARMOT_QUANT_KIND_Q4_0 && c->kind != MARMOT_QUANT_KIND_Q8_0 &&
+            c->kind != MARMOT_QUANT_KIND_Q4_K && c->kind != MARMOT_QUANT_KIND_Q6_K) {
+            continue;
+        }
+        char name[128];
+        int64_t dims[4] = {(int64_t)c->kind, (int64_t)c->N, (int64_t)c->K, (int64_t)c->M};
+        snprintf(name, sizeof(name), "matmul_%s_dims", c->name);
+        emit(name, "i8", dims, sizeof(dims));
+        snprintf(name, sizeof(name), "matmul_%s_weight", c->name);
+        emit(name, "u1", c->weights, c->weight_bytes);
+        snprintf(name, sizeof(name), "matmul_%s_input_f32", c->name);
+        emit(name, "f4", c->input_f32, c->N * c->K * 4);
+        snprintf(name, sizeof(name), "matmul_%s_input_f16", c->name);
+        emit(name, "u2", c->input_f16, c->N * c->K * 2);
+        snprintf(name, sizeof(name), "matmul_%s_expected_f32", c->name);
+        emit(name, "f4", c->expected_f32, c->N * c->M * 4);
+        snprintf(name, sizeof(name), "matmul_%s_expected_f16", c->name);
+        emit(name, "f4", c->expected_f16, c->N * c->M * 4);
+    }
+    return 0;
+}

@@ -1,0 +1,192 @@
+/*
+ * marmot_hip.h — C ABI of libmarmot_hip: the MI355X (gfx950) kernels behind marmot's
+ * block-quantized GGUF matmul path, plus the device plumbing a MARMOT_BACKEND_HIP needs.
+ *
+ * Plain pointers and sizes only. All `d_` pointers are device addresses obtained from
+ * marmot_hip_alloc (or any hipMalloc in the same process); everything is enqueued on the
+ * device object's stream and is asynchronous unless stated. Return values are marmot_error_t
+ * codes (0 = success, negative = include/marmot/types.h:210-220 of the reference); the text of
+ * the last failure on the calling thread is available from marmot_hip_last_error().
+ *
+ * Each entry names the reference interface it replaces (paths relative to the reference tree).
+ * The marmot_tensor_t-level backend (device vtable, kernel query, bytecode exec table) that sits
+ * on top of this ABI is declared in marmot_hip_backend.h.
+ *
+ * Naming follows the reference: marmot_linear(input[N,K], weight[M,K]) -> out[N,M]; N = tokens,
+ * K = reduction dim, M = weight rows (include/marmot/ops/matmul.h:11).
+ */
+#ifndef MARMOT_HIP_H
+#define MARMOT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct marmot_hip_device marmot_hip_device_t;
+
+/* marmot_error_t values (include/marmot/types.h:210-220) */
+enum {
+    MARMOT_HIP_SUCCESS = 0,
+    MARMOT_HIP_ERROR_INVALID_ARGUMENT = -1,
+    MARMOT_HIP_ERROR_OUT_OF_MEMORY = -2,
+    MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE = -3,
+    MARMOT_HIP_ERROR_BACKEND_INIT_FAILED = -4,
+    MARMOT_HIP_ERROR_INVALID_OPERATION = -5,
+    MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE = -6,
+    MARMOT_HIP_ERROR_DIMENSION_MISMATCH = -7,
+    MARMOT_HIP_ERROR_NOT_IMPLEMENTED = -8,
+};
+
+/* marmot_quant_kind_t values (include/marmot/types.h:372-388) */
+enum {
+    MARMOT_HIP_KIND_Q4_0 = 1,
+    MARMOT_HIP_KIND_Q8_0 = 5,
+    MARMOT_HIP_KIND_Q4_K = 9,
+    MARMOT_HIP_KIND_Q6_K = 11,
+    MARMOT_HIP_KIND_Q8_K = 12,
+};
+
+/* marmot_dtype_t values (include/marmot/types.h:340-362) */
+enum {
+    MARMOT_HIP_DTYPE_F32 = 0,
+    MARMOT_HIP_DTYPE_F16 = 1,
+};
+
+/* marmot_router_weight_policy_t (include/marmot/types.h:283-288), marmot_ffn_type_t (:276-281) */
+enum {
+    MARMOT_HIP_ROUTER_SOFTMAX_SELECTED = 0,
+    MARMOT_HIP_ROUTER_SOFTMAX_SELECTED_SCALED = 1,
+    MARMOT_HIP_ROUTER_RENORMALIZE_SELECTED = 2,
+};
+enum { MARMOT_HIP_FFN_SWIGLU = 0, MARMOT_HIP_FFN_GEGLU = 2 };
+
+/* flags of marmot_hip_matmul_quantized */
+enum {
+    /* quantize fp16 activations to Q8_0/Q8_K instead of the direct fp16 path
+     * (cpu_context_t.force_q8_activations, src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:438-441) */
+    MARMOT_HIP_MATMUL_FORCE_PACK = 1u << 0,
+};
+
+/* ------------------------------------------------------------------ device lifecycle and memory
+ * Replaces marmot_device_ops_t.{init,destroy,alloc,free,memcpy_to_device,memcpy_from_device,synchronize}
+ * (include/marmot/device.h:43-66) at the raw-pointer level. */
+int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev);
+void marmot_hip_device_destroy(marmot_hip_device_t *dev);
+int marmot_hip_alloc(marmot_hip_device_t *dev, size_t size, void **out_dptr);
+void marmot_hip_free(marmot_hip_device_t *dev, void *dptr);
+/* Synchronous with respect to the host buffer: returns after the bytes have left / reached `host`. */
+int marmot_hip_memcpy_to_device(marmot_hip_device_t *dev, void *d_dst, const void *host_src, size_t size);
+int marmot_hip_memcpy_from_device(marmot_hip_device_t *dev, void *host_dst, const void *d_src, size_t size);
+int marmot_hip_memcpy_device(marmot_hip_device_t *dev, void *d_dst, const void *d_src, size_t size);
+int marmot_hip_memset(marmot_hip_device_t *dev, void *d_dst, int value, size_t size);
+int marmot_hip_synchronize(marmot_hip_device_t *dev);
+/* bytes currently held through marmot_hip_alloc, and the high-water mark
+ * (marmot_device_ops_t.allocator_usage, include/marmot/allocator.h:27-36) */
+int marmot_hip_allocator_usage(marmot_hip_device_t *dev, size_t *current_bytes, size_t *peak_bytes, size_t *n_allocs);
+/* The hipStream_t all work of this device object is enqueued on (as void*). */
+void *marmot_hip_stream(marmot_hip_device_t *dev);
+const char *marmot_hip_last_error(void);
+
+/* Device facts for marmot_device_caps_t (include/marmot/device_caps.h:14-71) — replaces the per-backend
+ * branch of marmot_backend_detect_default_caps (src/core/dispatch/kernel_query.c:88-109). */
+typedef struct {
+    char name[64];
+    char arch[32];           /* e.g. "gfx950" */
+    uint32_t num_compute_units;
+    uint32_t wavefront_size;
+    uint32_t clock_mhz;      /* max engine clock */
+    uint32_t mem_clock_mhz;
+    uint32_t mem_bus_bits;
+    uint32_t l2_cache_kb;
+    uint32_t lds_kb_per_cu;
+    uint64_t total_mem_bytes;
+    float mem_bw_gbps;       /* published HBM peak used for rooflines */
+    float peak_tflops_fp16;  /* dense MFMA */
+    float peak_tops_int8;    /* dense MFMA */
+} marmot_hip_caps_t;
+int marmot_hip_get_caps(marmot_hip_device_t *dev, marmot_hip_caps_t *caps);
+
+/* Timing helpers (HIP events on the device object's stream). */
+int marmot_hip_event_create(marmot_hip_device_t *dev, void **out_event);
+void marmot_hip_event_destroy(marmot_hip_device_t *dev, void *event);
+int marmot_hip_event_record(marmot_hip_device_t *dev, void *event);
+int marmot_hip_event_elapsed_ms(marmot_hip_device_t *dev, void *start, void *stop, float *out_ms);
+
+/* ------------------------------------------------------------------ block geometry */
+size_t marmot_hip_block_values(int kind);
+size_t marmot_hip_block_bytes(int kind);
+/* bytes of one weight row of k values: ceil(k / block_values) * block_bytes
+ * (src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:423-427) */
+size_t marmot_hip_row_bytes(int kind, size_t k);
+
+/* ------------------------------------------------------------------ dequantize (the bit-exact contract)
+ * Replaces cpu_dequantize_{q4_0,q8_0,q4_k,q6_k,q8_k} -> cpu_dequantize_blockwise
+ * (src/backends/cpu/quantization/ops/quantize_core.c:267-331) with the per-block arithmetic of
+ * q4k_gguf.c:133-166, q6k_gguf.c:63-99, q8_gguf.c:189-200, q4_gguf.c:367-394.
+ * d_blocks: rows * marmot_hip_row_bytes(kind,k) bytes in native GGUF block layout; d_out: rows*k fp32. */
+int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_blocks, size_t rows, size_t k,
+                          float *d_out);
+
+/* ------------------------------------------------------------------ activation quantizers
+ * Replaces cpu_matmul_quant_pack_q8_0_{f32,f16} / cpu_matmul_quant_pack_q8_k_{f32,f16}
+ * (src/backends/cpu/ops/matmul/quantized/matmul_quant_pack.c:23-196) and, for block output, the
+ * QUANTIZE schema entries cpu_quantize_q8_0 / cpu_quantize_q8_k. act_kind: Q8_0 or Q8_K.
+ * d_x: rows x k activations of in_dtype (row-major, contiguous); d_blocks_out: rows * row_bytes(act_kind,k)
+ * bytes of marmot_q8_0_block_t / marmot_q8_k_block_t (include/marmot/quant_block.h:48-52, 121-125). */
+int marmot_hip_quantize_activations(marmot_hip_device_t *dev, int act_kind, const void *d_x, int in_dtype,
+                                    size_t rows, size_t k, void *d_blocks_out);
+
+/* ------------------------------------------------------------------ quantized linear
+ * Replaces cpu_matmul_quantized_{q4_0,q8_0,q4_k,q6_k} -> cpu_matmul_quantized_impl
+ * (src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:373-591, 905-929) incl. the bias epilogue
+ * (src/backends/cpu/ops/matmul/matmul_epilogue.c). out[n*M + m] = dot(W[m,:], x[n,:]) (+ bias[m]).
+ *   d_weight : M rows of marmot_hip_row_bytes(kind,K) bytes, native GGUF blocks
+ *   d_input  : [N,K] of in_dtype; F32 -> activations are quantized to Q8_0 (Q4_0/Q8_0 weights) or Q8_K
+ *              (K-quants) and integer block dots are used; F16 -> direct dequantized dot unless FORCE_PACK
+ *   d_bias   : NULL or M values of bias_dtype (F32, or F16 when out is F16)
+ *   d_out    : [N,M] of out_dtype (F32; F16 allowed only with F16 input)
+ * Errors mirror marmot_matmul_validate_quantized (src/core/helpers/matmul.c:68-136). */
+int marmot_hip_matmul_quantized(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_input,
+                                int in_dtype, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
+                                void *d_out, int out_dtype, uint32_t flags);
+
+/* Replaces cpu_matmul_quantized_dual_output (matmul_quant_dispatch.c:593-856): two weights of the same
+ * kind and shape applied to one input with a single activation quantization (gate/up projections). */
+int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const void *d_weight_a,
+                                     const void *d_weight_b, const void *d_input, int in_dtype, size_t N, size_t K,
+                                     size_t M, void *d_out_a, void *d_out_b, int out_dtype, uint32_t flags);
+
+/* ------------------------------------------------------------------ MoE
+ * Replaces cpu_topk_impl (src/backends/cpu/ops/moe/moe_ops.c:789-889): top-k over the last axis of
+ * fp32 x[rows,cols], ties to the lower index; values fp32 [rows,k], indices int32 [rows,k]. */
+int marmot_hip_topk(marmot_hip_device_t *dev, const float *d_x, size_t rows, size_t cols, size_t k,
+                    float *d_values, int32_t *d_indices);
+/* Softmax over each row of k selected logits (router policy SOFTMAX_SELECTED*,
+ * src/graph/gguf/graph_builder.cpp:2276-2316). */
+int marmot_hip_softmax_rows(marmot_hip_device_t *dev, const float *d_x, size_t rows, size_t k, float *d_out);
+
+/* Replaces cpu_moe_experts_impl for fp32 activations and block-quantized experts
+ * (src/backends/cpu/ops/moe/moe_ops.c:891-1049, 506-568, 1069-1178).
+ *   d_hidden [T,H] fp32; d_gate/d_up: E slices of [F rows, H] blocks of kind_gate_up;
+ *   d_down: E slices of [H rows, F] blocks of kind_down; d_topk_ids int32 [T,k]; d_topk_weights fp32 [T,k];
+ *   d_out [T,H] fp32 (fully overwritten). */
+int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size_t T, size_t H, size_t F, size_t E,
+                           size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate, const void *d_up,
+                           const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
+                           float weights_scale, int router_weight_policy, int ffn_type, float *d_out);
+
+/* ------------------------------------------------------------------ introspection
+ * Name of the kernel route the last marmot_hip_matmul_quantized call on this thread took
+ * (counterpart of the reference's MARMOT_METAL_LOG_MATMUL_QUANT route log,
+ * src/backends/metal/ops/matmul_quant_dispatch.mm:30-70). */
+const char *marmot_hip_last_route(void);
+const char *marmot_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MARMOT_HIP_H */

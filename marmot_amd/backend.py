@@ -1,0 +1,261 @@
+"""Host-side mirror of the reference's operator interface for the quantized matmul path.
+
+Names and argument meaning follow the reference's C API: ``linear(input[N,K], weight[M,K]) -> out[N,M]``
+(include/marmot/ops/matmul.h:11), ``dequantize`` (ops/quantization.h), ``topk`` / ``moe_experts``
+(ops/neural.h:67,85). Everything runs through the C ABI in include/marmot_hip.h.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .capi import DT_F16, DT_F32, KIND_Q8_0, KIND_Q8_K, check, load_library
+
+_BV = {1: 32, 5: 32, 9: 256, 11: 256, 12: 256}
+_BB = {1: 18, 5: 34, 9: 144, 11: 210, 12: 292}
+
+
+def block_values(kind: int) -> int:
+    return _BV[kind]
+
+
+def block_bytes(kind: int) -> int:
+    return _BB[kind]
+
+
+def row_bytes(kind: int, k: int) -> int:
+    return ((k + _BV[kind] - 1) // _BV[kind]) * _BB[kind]
+
+
+def _np_dtype_id(dt) -> int:
+    dt = np.dtype(dt)
+    if dt == np.float32:
+        return DT_F32
+    if dt == np.float16:
+        return DT_F16
+    raise TypeError(f"unsupported dtype {dt}")
+
+
+class DeviceBuffer:
+    """A device allocation made through marmot_hip_alloc."""
+
+    def __init__(self, backend: "HipBackend", nbytes: int):
+        self.backend = backend
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        check(backend.lib.marmot_hip_alloc(backend.dev, max(self.nbytes, 1), C.byref(p)))
+        self.ptr = p.value
+
+    def upload(self, arr: np.ndarray, offset: int = 0):
+        arr = np.ascontiguousarray(arr)
+        assert offset + arr.nbytes <= self.nbytes
+        if arr.nbytes:
+            check(self.backend.lib.marmot_hip_memcpy_to_device(
+                self.backend.dev, C.c_void_p(self.ptr + offset), arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+        return self
+
+    def download(self, dtype, shape, offset: int = 0) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        assert offset + out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(self.backend.lib.marmot_hip_memcpy_from_device(
+                self.backend.dev, out.ctypes.data_as(C.c_void_p), C.c_void_p(self.ptr + offset), out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.backend.lib.marmot_hip_free(self.backend.dev, C.c_void_p(self.ptr))
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class HipBackend:
+    """One marmot_hip_device_t (one GPU, one stream)."""
+
+    def __init__(self, device_index: int = 0):
+        self.lib = load_library()
+        dev = C.c_void_p()
+        check(self.lib.marmot_hip_device_create(device_index, C.byref(dev)))
+        self.dev = dev
+
+    def close(self):
+        if self.dev:
+            self.lib.marmot_hip_device_destroy(self.dev)
+            self.dev = None
+
+    # ---- plumbing
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        return DeviceBuffer(self, nbytes)
+
+    def to_device(self, arr: np.ndarray) -> DeviceBuffer:
+        arr = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, arr.nbytes).upload(arr)
+
+    def synchronize(self):
+        check(self.lib.marmot_hip_synchronize(self.dev))
+
+    def caps(self) -> dict:
+        c = capi.Caps()
+        check(self.lib.marmot_hip_get_caps(self.dev, C.byref(c)))
+        return {f: (getattr(c, f).decode() if isinstance(getattr(c, f), bytes) else getattr(c, f))
+                for f, _ in capi.Caps._fields_}
+
+    def allocator_usage(self):
+        cur, peak, n = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        check(self.lib.marmot_hip_allocator_usage(self.dev, C.byref(cur), C.byref(peak), C.byref(n)))
+        return cur.value, peak.value, n.value
+
+    def last_route(self) -> str:
+        return self.lib.marmot_hip_last_route().decode()
+
+    def event(self):
+        e = C.c_void_p()
+        check(self.lib.marmot_hip_event_create(self.dev, C.byref(e)))
+        return e
+
+    def record(self, e):
+        check(self.lib.marmot_hip_event_record(self.dev, e))
+
+    def elapsed_ms(self, a, b) -> float:
+        ms = C.c_float()
+        check(self.lib.marmot_hip_event_elapsed_ms(self.dev, a, b, C.byref(ms)))
+        return ms.value
+
+    # ---- device-pointer level ops (what bench.py times)
+    def dequantize_d(self, kind: int, d_blocks: DeviceBuffer, rows: int, k: int, d_out: DeviceBuffer):
+        check(self.lib.marmot_hip_dequantize(self.dev, kind, C.c_void_p(d_blocks.ptr), rows, k, C.c_void_p(d_out.ptr)))
+
+    def linear_d(self, kind: int, d_weight, d_input, in_dtype: int, N: int, K: int, M: int, d_out, out_dtype: int,
+                 d_bias=None, bias_dtype: int = DT_F32, flags: int = 0, weight_offset: int = 0):
+        check(self.lib.marmot_hip_matmul_quantized(
+            self.dev, kind, C.c_void_p(d_weight.ptr + weight_offset), C.c_void_p(d_input.ptr), in_dtype, N, K, M,
+            C.c_void_p(d_bias.ptr) if d_bias is not None else None, bias_dtype, C.c_void_p(d_out.ptr), out_dtype,
+            flags))
+
+    # ---- numpy level ops (what the parity tests call)
+    def dequantize(self, kind: int, blocks: np.ndarray, k: int) -> np.ndarray:
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        if blocks.ndim == 1:
+            blocks = blocks[None, :]
+        rows = blocks.shape[0]
+        if blocks.shape[1] != row_bytes(kind, k):
+            raise ValueError("blocks do not match rows x row_bytes(kind, k)")
+        d_in = self.to_device(blocks)
+        d_out = self.alloc(rows * k * 4)
+        self.dequantize_d(kind, d_in, rows, k, d_out)
+        out = d_out.download(np.float32, (rows, k))
+        d_in.free()
+        d_out.free()
+        return out
+
+    def quantize_activations(self, act_kind: int, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x)
+        if x.ndim == 1:
+            x = x[None, :]
+        rows, k = x.shape
+        d_x = self.to_device(x)
+        nbytes = rows * row_bytes(act_kind, k)
+        d_out = self.alloc(nbytes)
+        check(self.lib.marmot_hip_quantize_activations(self.dev, act_kind, C.c_void_p(d_x.ptr), _np_dtype_id(x.dtype),
+                                                       rows, k, C.c_void_p(d_out.ptr)))
+        out = d_out.download(np.uint8, (rows, row_bytes(act_kind, k)))
+        d_x.free()
+        d_out.free()
+        return out
+
+    def linear(self, x: np.ndarray, weight: np.ndarray, kind: int, M: int, bias: np.ndarray | None = None,
+               out_dtype=np.float32, force_pack: bool = False) -> np.ndarray:
+        """marmot_linear(input[N,K], weight[M,K] as GGUF blocks) -> out[N,M]."""
+        x = np.ascontiguousarray(x)
+        N, K = x.shape
+        weight = np.ascontiguousarray(weight, dtype=np.uint8)
+        if weight.size != M * row_bytes(kind, K):
+            raise ValueError("weight bytes do not match M x row_bytes(kind, K)")
+        d_w = self.to_device(weight)
+        d_x = self.to_device(x)
+        out_dtype = np.dtype(out_dtype)
+        d_out = self.alloc(max(N * M * out_dtype.itemsize, 4))
+        d_b = self.to_device(bias) if bias is not None else None
+        try:
+            self.linear_d(kind, d_w, d_x, _np_dtype_id(x.dtype), N, K, M, d_out, _np_dtype_id(out_dtype), d_b,
+                          _np_dtype_id(bias.dtype) if bias is not None else DT_F32,
+                          capi.FLAG_FORCE_PACK if force_pack else 0)
+            return d_out.download(out_dtype, (N, M))
+        finally:
+            for b in (d_w, d_x, d_out, d_b):
+                if b is not None:
+                    b.free()
+
+    def linear_dual(self, x: np.ndarray, weight_a: np.ndarray, weight_b: np.ndarray, kind: int, M: int,
+                    out_dtype=np.float32, force_pack: bool = False):
+        x = np.ascontiguousarray(x)
+        N, K = x.shape
+        d_a = self.to_device(np.ascontiguousarray(weight_a, dtype=np.uint8))
+        d_b = self.to_device(np.ascontiguousarray(weight_b, dtype=np.uint8))
+        d_x = self.to_device(x)
+        out_dtype = np.dtype(out_dtype)
+        d_oa = self.alloc(N * M * out_dtype.itemsize)
+        d_ob = self.alloc(N * M * out_dtype.itemsize)
+        try:
+            check(self.lib.marmot_hip_matmul_quantized_dual(
+                self.dev, kind, C.c_void_p(d_a.ptr), C.c_void_p(d_b.ptr), C.c_void_p(d_x.ptr), _np_dtype_id(x.dtype),
+                N, K, M, C.c_void_p(d_oa.ptr), C.c_void_p(d_ob.ptr), _np_dtype_id(out_dtype),
+                capi.FLAG_FORCE_PACK if force_pack else 0))
+            return d_oa.download(out_dtype, (N, M)), d_ob.download(out_dtype, (N, M))
+        finally:
+            for b in (d_a, d_b, d_x, d_oa, d_ob):
+                b.free()
+
+    def topk(self, x: np.ndarray, k: int):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        rows, cols = x.shape
+        d_x = self.to_device(x)
+        d_v = self.alloc(rows * k * 4)
+        d_i = self.alloc(rows * k * 4)
+        try:
+            check(self.lib.marmot_hip_topk(self.dev, C.c_void_p(d_x.ptr), rows, cols, k, C.c_void_p(d_v.ptr),
+                                           C.c_void_p(d_i.ptr)))
+            return d_v.download(np.float32, (rows, k)), d_i.download(np.int32, (rows, k))
+        finally:
+            for b in (d_x, d_v, d_i):
+                b.free()
+
+    def softmax_rows(self, x: np.ndarray) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        rows, k = x.shape
+        d_x = self.to_device(x)
+        d_o = self.alloc(rows * k * 4)
+        try:
+            check(self.lib.marmot_hip_softmax_rows(self.dev, C.c_void_p(d_x.ptr), rows, k, C.c_void_p(d_o.ptr)))
+            return d_o.download(np.float32, (rows, k))
+        finally:
+            d_x.free()
+            d_o.free()
+
+    def moe_experts(self, hidden, gate, up, down, topk_ids, topk_weights, F: int, E: int, kind_gate_up: int,
+                    kind_down: int, weights_scale: float = 1.0, policy: int = 1, ffn_type: int = 0) -> np.ndarray:
+        hidden = np.ascontiguousarray(hidden, dtype=np.float32)
+        T, H = hidden.shape
+        ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
+        w = np.ascontiguousarray(topk_weights, dtype=np.float32)
+        kpt = ids.shape[1]
+        bufs = [self.to_device(a) for a in (hidden, np.ascontiguousarray(gate, dtype=np.uint8),
+                                            np.ascontiguousarray(up, dtype=np.uint8),
+                                            np.ascontiguousarray(down, dtype=np.uint8), ids, w)]
+        d_out = self.alloc(T * H * 4)
+        try:
+            check(self.lib.marmot_hip_moe_experts(
+                self.dev, C.c_void_p(bufs[0].ptr), T, H, F, E, kpt, kind_gate_up, kind_down, C.c_void_p(bufs[1].ptr),
+                C.c_void_p(bufs[2].ptr), C.c_void_p(bufs[3].ptr), C.c_void_p(bufs[4].ptr), C.c_void_p(bufs[5].ptr),
+                weights_scale, policy, ffn_type, C.c_void_p(d_out.ptr)))
+            return d_out.download(np.float32, (T, H))
+        finally:
+            for b in bufs + [d_out]:
+                b.free()

@@ -1,0 +1,101 @@
+"""ctypes declarations of include/marmot_hip.h (one entry per exported symbol)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_K = 1, 5, 9, 11, 12
+DT_F32, DT_F16 = 0, 1
+FLAG_FORCE_PACK = 1
+
+ERROR_NAMES = {
+    0: "SUCCESS", -1: "INVALID_ARGUMENT", -2: "OUT_OF_MEMORY", -3: "DEVICE_NOT_AVAILABLE", -4: "BACKEND_INIT_FAILED",
+    -5: "INVALID_OPERATION", -6: "UNSUPPORTED_DTYPE", -7: "DIMENSION_MISMATCH", -8: "NOT_IMPLEMENTED",
+}
+
+
+class MarmotHipError(RuntimeError):
+    def __init__(self, code: int, detail: str):
+        super().__init__(f"marmot_hip error {code} ({ERROR_NAMES.get(code, '?')}): {detail}")
+        self.code = code
+        self.detail = detail
+
+
+class Caps(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 64), ("arch", C.c_char * 32), ("num_compute_units", C.c_uint32),
+        ("wavefront_size", C.c_uint32), ("clock_mhz", C.c_uint32), ("mem_clock_mhz", C.c_uint32),
+        ("mem_bus_bits", C.c_uint32), ("l2_cache_kb", C.c_uint32), ("lds_kb_per_cu", C.c_uint32),
+        ("total_mem_bytes", C.c_uint64), ("mem_bw_gbps", C.c_float), ("peak_tflops_fp16", C.c_float),
+        ("peak_tops_int8", C.c_float),
+    ]
+
+
+_vp, _sz, _i, _u32, _f = C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_float
+
+# name -> (restype, argtypes); every symbol include/marmot_hip.h declares
+SIGNATURES = {
+    "marmot_hip_device_create": (_i, [_i, C.POINTER(_vp)]),
+    "marmot_hip_device_destroy": (None, [_vp]),
+    "marmot_hip_alloc": (_i, [_vp, _sz, C.POINTER(_vp)]),
+    "marmot_hip_free": (None, [_vp, _vp]),
+    "marmot_hip_memcpy_to_device": (_i, [_vp, _vp, _vp, _sz]),
+    "marmot_hip_memcpy_from_device": (_i, [_vp, _vp, _vp, _sz]),
+    "marmot_hip_memcpy_device": (_i, [_vp, _vp, _vp, _sz]),
+    "marmot_hip_memset": (_i, [_vp, _vp, _i, _sz]),
+    "marmot_hip_synchronize": (_i, [_vp]),
+    "marmot_hip_allocator_usage": (_i, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
+    "marmot_hip_stream": (_vp, [_vp]),
+    "marmot_hip_last_error": (C.c_char_p, []),
+    "marmot_hip_get_caps": (_i, [_vp, C.POINTER(Caps)]),
+    "marmot_hip_event_create": (_i, [_vp, C.POINTER(_vp)]),
+    "marmot_hip_event_destroy": (None, [_vp, _vp]),
+    "marmot_hip_event_record": (_i, [_vp, _vp]),
+    "marmot_hip_event_elapsed_ms": (_i, [_vp, _vp, _vp, C.POINTER(_f)]),
+    "marmot_hip_block_values": (_sz, [_i]),
+    "marmot_hip_block_bytes": (_sz, [_i]),
+    "marmot_hip_row_bytes": (_sz, [_i, _sz]),
+    "marmot_hip_dequantize": (_i, [_vp, _i, _vp, _sz, _sz, _vp]),
+    "marmot_hip_quantize_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
+    "marmot_hip_matmul_quantized": (_i, [_vp, _i, _vp, _vp, _i, _sz, _sz, _sz, _vp, _i, _vp, _i, _u32]),
+    "marmot_hip_matmul_quantized_dual": (_i, [_vp, _i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _i, _u32]),
+    "marmot_hip_topk": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
+    "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
+    "marmot_hip_moe_experts": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i,
+                                    _vp]),
+    "marmot_hip_last_route": (C.c_char_p, []),
+    "marmot_hip_version": (C.c_char_p, []),
+}
+
+_lib = None
+
+
+def lib_path() -> str:
+    return os.environ.get("MARMOT_HIP_LIBRARY", os.path.join(HERE, "lib", "libmarmot_hip.so"))
+
+
+def load_library():
+    """Loads libmarmot_hip.so and declares every entry point. Raises if the library is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise FileNotFoundError(
+            f"{path} is not built: run `python -c 'import __graft_entry__ as g; g.build()'` or "
+            f"`make -C marmot_amd/csrc`. There is no CPU fallback for the HIP path.")
+    lib = C.CDLL(path)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the header and the library disagree
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code: int):
+    if code != 0:
+        detail = load_library().marmot_hip_last_error()
+        raise MarmotHipError(code, detail.decode() if detail else "")

@@ -1,0 +1,183 @@
+// Shared declarations of libmarmot_hip: GGUF block layouts, small device helpers, the device object.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "../../include/marmot_hip.h"
+
+namespace mh {
+
+// ---- GGUF block layouts (include/marmot/quant_block.h:20-125 of the reference)
+constexpr int QK = 32;
+constexpr int QK_K = 256;
+constexpr int Q4_0_BYTES = 18;
+constexpr int Q8_0_BYTES = 34;
+constexpr int Q4_K_BYTES = 144;
+constexpr int Q6_K_BYTES = 210;
+constexpr int Q8_K_BYTES = 292;
+
+struct __attribute__((packed)) BlockQ4_0 {
+    uint16_t scale;
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ8_0 {
+    uint16_t scale;
+    int8_t qs[32];
+};
+struct __attribute__((packed)) BlockQ4_K {
+    uint16_t d;
+    uint16_t dmin;
+    uint8_t scales[12];
+    uint8_t qs[128];
+};
+struct __attribute__((packed)) BlockQ6_K {
+    uint8_t ql[128];
+    uint8_t qh[64];
+    int8_t scales[16];
+    uint16_t d;
+};
+struct __attribute__((packed)) BlockQ8_K {
+    float d;
+    int8_t qs[256];
+    int16_t bsums[16];
+};
+static_assert(sizeof(BlockQ4_0) == Q4_0_BYTES, "Q4_0");
+static_assert(sizeof(BlockQ8_0) == Q8_0_BYTES, "Q8_0");
+static_assert(sizeof(BlockQ4_K) == Q4_K_BYTES, "Q4_K");
+static_assert(sizeof(BlockQ6_K) == Q6_K_BYTES, "Q6_K");
+static_assert(sizeof(BlockQ8_K) == Q8_K_BYTES, "Q8_K");
+
+inline size_t block_values(int kind) {
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_0:
+    case MARMOT_HIP_KIND_Q8_0:
+        return QK;
+    case MARMOT_HIP_KIND_Q4_K:
+    case MARMOT_HIP_KIND_Q6_K:
+    case MARMOT_HIP_KIND_Q8_K:
+        return QK_K;
+    default:
+        return 0;
+    }
+}
+inline size_t block_bytes(int kind) {
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_0:
+        return Q4_0_BYTES;
+    case MARMOT_HIP_KIND_Q8_0:
+        return Q8_0_BYTES;
+    case MARMOT_HIP_KIND_Q4_K:
+        return Q4_K_BYTES;
+    case MARMOT_HIP_KIND_Q6_K:
+        return Q6_K_BYTES;
+    case MARMOT_HIP_KIND_Q8_K:
+        return Q8_K_BYTES;
+    default:
+        return 0;
+    }
+}
+inline bool is_k_quant(int kind) {
+    return block_values(kind) == QK_K;
+}
+
+// ---- error plumbing (thread-local text like marmot_set_error, include/marmot/error.h:21-43)
+int set_error(int code, const char *fmt, ...);
+void set_route(const char *name);
+int check_hip(hipError_t e, const char *what);
+
+#define MH_HIP(expr)                                                                                                   \
+    do {                                                                                                               \
+        int _st = ::mh::check_hip((expr), #expr);                                                                      \
+        if (_st != 0)                                                                                                  \
+            return _st;                                                                                                \
+    } while (0)
+
+// ---- activation scratch: quantized activations in a structure-of-arrays layout private to the library.
+// For N rows of K values (nb = ceil(K/block)):
+//   qs    int8  [N][kp]      kp = nb*block, zero padded, 16-byte aligned rows
+//   d     float [N][nb]      Q8_K: 1/iscale;  Q8_0: fp16-rounded scale widened to fp32
+//   sums  int16 [N][nb*16]   Q8_K: sums of 16 (bsums);  Q8_0: [N][nb] sum of the 32 values
+struct ActScratch {
+    int8_t *qs = nullptr;
+    float *d = nullptr;
+    int16_t *sums = nullptr;
+    size_t kp = 0;
+    size_t nb = 0;
+};
+
+} // namespace mh
+
+// The device object behind marmot_hip_device_t.
+struct marmot_hip_device {
+    int device_index = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t props;
+    // library-owned workspace, grown on demand (counterpart of the reference's quant workspace slots,
+    // src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:331-371)
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
+    // allocation accounting
+    std::mutex mu;
+    std::unordered_map<void *, size_t> allocs;
+    size_t current_bytes = 0;
+    size_t peak_bytes = 0;
+};
+
+namespace mh {
+
+// Returns a workspace of at least `bytes` (256-byte aligned). Growing it synchronizes the stream first.
+int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out);
+
+// Carves the activation scratch for `rows` x `k` out of `base`; returns bytes consumed (256-byte rounded).
+size_t act_scratch_layout(int act_kind, size_t rows, size_t k, void *base, ActScratch *out);
+
+// kernels / launchers implemented in the .hip files
+int launch_quantize_act_soa(marmot_hip_device *dev, int act_kind, const void *d_x, int in_dtype, size_t rows, size_t k,
+                            const ActScratch &dst);
+int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act,
+                         size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1,
+                         int out_dtype);
+int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
+                      const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
+bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M);
+int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
+                    const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
+
+// ---- device helpers
+#if defined(__HIPCC__)
+__device__ __forceinline__ float h2f(uint16_t h) {
+    return __half2float(__ushort_as_half(h));
+}
+__device__ __forceinline__ uint16_t f2h(float f) {
+    return __half_as_ushort(__float2half_rn(f));
+}
+
+// Sum over the 64 lanes of a wavefront; every lane receives the total. DPP within rows of 16, then
+// cross-row through readlane.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true)); // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true)); // row_mirror
+    const int iv = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+#endif
+
+} // namespace mh

@@ -1,0 +1,99 @@
+// Per-value dequantizers shared by the dequantize kernels and the direct (unquantized-activation) matmul
+// route. Arithmetic and operation order follow the reference's CPU dequantizers exactly; translation units
+// that include this header must be compiled with -ffp-contract=off.
+#pragma once
+
+#include "mh_common.h"
+
+namespace mh {
+
+// Q4_K (q4k_gguf.c:133-166): d1 = d*sc; m1 = dmin*m; y = d1*q - m1
+__device__ __forceinline__ float dequant_value_q4_k(const uint8_t *blk, int v) {
+    const BlockQ4_K *b = (const BlockQ4_K *)blk;
+    const int j = v >> 5;          // sub-block 0..7
+    const int l = v & 31;
+    const int g = j >> 1;          // 64-value group
+    uint8_t sc, m;
+    const uint8_t *s = b->scales;
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (uint8_t)((s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4));
+        m = (uint8_t)((s[j + 4] >> 4) | ((s[j] >> 6) << 4));
+    }
+    const float d = h2f(b->d);
+    const float dmin = h2f(b->dmin);
+    const float d1 = d * (float)sc;
+    const float m1 = dmin * (float)m;
+    const uint8_t byte = b->qs[32 * g + l];
+    const int q = (j & 1) ? (byte >> 4) : (byte & 0xF);
+    return d1 * (float)q - m1;
+}
+
+// Q6_K (q6k_gguf.c:63-99): y = (d * sc) * q
+__device__ __forceinline__ float dequant_value_q6_k(const uint8_t *blk, int v) {
+    const BlockQ6_K *b = (const BlockQ6_K *)blk;
+    const int hh = v >> 7;         // half 0..1
+    const int w = v & 127;
+    const int j = w >> 5;          // 0..3: which of q1..q4
+    const int l = w & 31;
+    const uint8_t *ql = b->ql + 64 * hh;
+    const uint8_t *qh = b->qh + 32 * hh;
+    const int8_t *sc = b->scales + 8 * hh;
+    const uint8_t lo = (j & 1) ? ql[l + 32] : ql[l];
+    const int nib = (j & 2) ? (lo >> 4) : (lo & 0xF);
+    const int hi2 = (qh[l] >> (2 * j)) & 3;
+    const int q = (int)(int8_t)(nib | (hi2 << 4)) - 32;
+    const float d = h2f(b->d);
+    return d * (float)sc[(l >> 4) + 2 * j] * (float)q;
+}
+
+// Q8_0 (q8_gguf.c:189-200): y = (float)q * scale
+__device__ __forceinline__ float dequant_value_q8_0(const uint8_t *blk, int v) {
+    const BlockQ8_0 *b = (const BlockQ8_0 *)blk;
+    return (float)b->qs[v] * h2f(b->scale);
+}
+
+// Q4_0 (q4_gguf.c:367-394): y = (q - 8) * scale
+__device__ __forceinline__ float dequant_value_q4_0(const uint8_t *blk, int v) {
+    const BlockQ4_0 *b = (const BlockQ4_0 *)blk;
+    const uint8_t packed = b->qs[v & 15];
+    const int q = (v < 16) ? (packed & 0x0F) : (packed >> 4);
+    return (float)(q - 8) * h2f(b->scale);
+}
+
+// Q8_K (q8k_gguf.c): y = d * q
+__device__ __forceinline__ float dequant_value_q8_k(const uint8_t *blk, int v) {
+    const BlockQ8_K *b = (const BlockQ8_K *)blk;
+    float d;
+    __builtin_memcpy(&d, &b->d, 4);
+    return d * (float)b->qs[v];
+}
+
+template <int KIND>
+__device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
+    if constexpr (KIND == MARMOT_HIP_KIND_Q4_K) {
+        return dequant_value_q4_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q6_K) {
+        return dequant_value_q6_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q8_0) {
+        return dequant_value_q8_0(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q4_0) {
+        return dequant_value_q4_0(blk, v);
+    } else {
+        return dequant_value_q8_k(blk, v);
+    }
+}
+
+template <int KIND>
+struct KindTraits {
+    static constexpr int BV = (KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q8_0) ? QK : QK_K;
+    static constexpr int BB = KIND == MARMOT_HIP_KIND_Q4_0 ? Q4_0_BYTES
+        : KIND == MARMOT_HIP_KIND_Q8_0                     ? Q8_0_BYTES
+        : KIND == MARMOT_HIP_KIND_Q4_K                     ? Q4_K_BYTES
+        : KIND == MARMOT_HIP_KIND_Q6_K                     ? Q6_K_BYTES
+                                                           : Q8_K_BYTES;
+};
+
+} // namespace mh

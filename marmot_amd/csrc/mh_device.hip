@@ -1,0 +1,333 @@
+// Device object, memory, events, error text: the plumbing half of the C ABI (include/marmot_hip.h).
+#include "mh_common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace mh {
+
+static thread_local char g_error[512] = "";
+static thread_local char g_route[96] = "";
+
+int set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+void set_route(const char *name) {
+    snprintf(g_route, sizeof(g_route), "%s", name);
+}
+
+int check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    const int code = (e == hipErrorOutOfMemory) ? MARMOT_HIP_ERROR_OUT_OF_MEMORY
+        : (e == hipErrorNoDevice || e == hipErrorInvalidDevice) ? MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE
+                                                                : MARMOT_HIP_ERROR_INVALID_OPERATION;
+    return set_error(code, "HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+}
+
+int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out) {
+    if (bytes > dev->workspace_bytes) {
+        // round up so that a sequence of growing requests does not reallocate every time
+        size_t want = dev->workspace_bytes ? dev->workspace_bytes : (size_t)1 << 20;
+        while (want < bytes) {
+            want *= 2;
+        }
+        MH_HIP(hipStreamSynchronize(dev->stream));
+        if (dev->workspace != nullptr) {
+            MH_HIP(hipFree(dev->workspace));
+            dev->workspace = nullptr;
+            dev->workspace_bytes = 0;
+        }
+        MH_HIP(hipMalloc(&dev->workspace, want));
+        dev->workspace_bytes = want;
+    }
+    *out = dev->workspace;
+    return MARMOT_HIP_SUCCESS;
+}
+
+static inline size_t round256(size_t v) {
+    return (v + 255) & ~(size_t)255;
+}
+
+size_t act_scratch_layout(int act_kind, size_t rows, size_t k, void *base, ActScratch *out) {
+    const size_t bv = block_values(act_kind);
+    const size_t nb = (k + bv - 1) / bv;
+    const size_t kp = nb * bv;
+    const size_t qs_bytes = round256(rows * kp);
+    const size_t d_bytes = round256(rows * nb * sizeof(float));
+    const size_t sums_per_block = (act_kind == MARMOT_HIP_KIND_Q8_K) ? 16 : 1;
+    const size_t sums_bytes = round256(rows * nb * sums_per_block * sizeof(int16_t));
+    if (out != nullptr) {
+        uint8_t *p = (uint8_t *)base;
+        out->qs = (int8_t *)p;
+        out->d = (float *)(p + qs_bytes);
+        out->sums = (int16_t *)(p + qs_bytes + d_bytes);
+        out->kp = kp;
+        out->nb = nb;
+    }
+    return qs_bytes + d_bytes + sums_bytes;
+}
+
+} // namespace mh
+
+using namespace mh;
+
+extern "C" {
+
+int marmot_hip_fill_bytes_internal(marmot_hip_device_t *dev, void *d_dst, int value, size_t size);
+
+const char *marmot_hip_last_error(void) {
+    return g_error;
+}
+
+const char *marmot_hip_last_route(void) {
+    return g_route;
+}
+
+const char *marmot_hip_version(void) {
+    return "marmot_hip 0.1 (gfx950)";
+}
+
+size_t marmot_hip_block_values(int kind) {
+    return block_values(kind);
+}
+size_t marmot_hip_block_bytes(int kind) {
+    return block_bytes(kind);
+}
+size_t marmot_hip_row_bytes(int kind, size_t k) {
+    const size_t bv = block_values(kind);
+    return bv == 0 ? 0 : ((k + bv - 1) / bv) * block_bytes(kind);
+}
+
+int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
+    if (out_dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "out_dev is null");
+    }
+    *out_dev = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "no HIP device available (%s)",
+                         e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    }
+    if (device_index < 0 || device_index >= count) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "device index %d out of range (%d devices)",
+                         device_index, count);
+    }
+    MH_HIP(hipSetDevice(device_index));
+    marmot_hip_device *dev = new marmot_hip_device();
+    dev->device_index = device_index;
+    if (check_hip(hipGetDeviceProperties(&dev->props, device_index), "hipGetDeviceProperties") != 0) {
+        delete dev;
+        return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
+    }
+    if (strncmp(dev->props.gcnArchName, "gfx950", 6) != 0) {
+        const int st = set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE,
+                                 "libmarmot_hip is built for gfx950 only; device %d is %s", device_index,
+                                 dev->props.gcnArchName);
+        delete dev;
+        return st;
+    }
+    // default priority, non-blocking with respect to the legacy default stream
+    if (check_hip(hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags") != 0) {
+        delete dev;
+        return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
+    }
+    *out_dev = dev;
+    return MARMOT_HIP_SUCCESS;
+}
+
+void marmot_hip_device_destroy(marmot_hip_device_t *dev) {
+    if (dev == nullptr) {
+        return;
+    }
+    (void)hipSetDevice(dev->device_index);
+    (void)hipStreamSynchronize(dev->stream);
+    if (dev->workspace != nullptr) {
+        (void)hipFree(dev->workspace);
+    }
+    for (auto &kv : dev->allocs) {
+        (void)hipFree(kv.first);
+    }
+    (void)hipStreamDestroy(dev->stream);
+    delete dev;
+}
+
+int marmot_hip_alloc(marmot_hip_device_t *dev, size_t size, void **out_dptr) {
+    if (dev == nullptr || out_dptr == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "alloc: null argument");
+    }
+    *out_dptr = nullptr;
+    if (size == 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "alloc: size is 0");
+    }
+    void *p = nullptr;
+    MH_HIP(hipMalloc(&p, size));
+    {
+        std::lock_guard<std::mutex> lock(dev->mu);
+        dev->allocs[p] = size;
+        dev->current_bytes += size;
+        if (dev->current_bytes > dev->peak_bytes) {
+            dev->peak_bytes = dev->current_bytes;
+        }
+    }
+    *out_dptr = p;
+    return MARMOT_HIP_SUCCESS;
+}
+
+void marmot_hip_free(marmot_hip_device_t *dev, void *dptr) {
+    if (dev == nullptr || dptr == nullptr) {
+        return;
+    }
+    {
+        std::lock_guard<std::mutex> lock(dev->mu);
+        auto it = dev->allocs.find(dptr);
+        if (it == dev->allocs.end()) {
+            return; // not ours
+        }
+        dev->current_bytes -= it->second;
+        dev->allocs.erase(it);
+    }
+    (void)hipStreamSynchronize(dev->stream);
+    (void)hipFree(dptr);
+}
+
+int marmot_hip_memcpy_to_device(marmot_hip_device_t *dev, void *d_dst, const void *host_src, size_t size) {
+    if (dev == nullptr || d_dst == nullptr || host_src == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "memcpy_to_device: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    MH_HIP(hipMemcpyAsync(d_dst, host_src, size, hipMemcpyHostToDevice, dev->stream));
+    MH_HIP(hipStreamSynchronize(dev->stream));
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_memcpy_from_device(marmot_hip_device_t *dev, void *host_dst, const void *d_src, size_t size) {
+    if (dev == nullptr || host_dst == nullptr || d_src == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "memcpy_from_device: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    MH_HIP(hipMemcpyAsync(host_dst, d_src, size, hipMemcpyDeviceToHost, dev->stream));
+    MH_HIP(hipStreamSynchronize(dev->stream));
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_memcpy_device(marmot_hip_device_t *dev, void *d_dst, const void *d_src, size_t size) {
+    if (dev == nullptr || d_dst == nullptr || d_src == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "memcpy_device: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    MH_HIP(hipMemcpyAsync(d_dst, d_src, size, hipMemcpyDeviceToDevice, dev->stream));
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_memset(marmot_hip_device_t *dev, void *d_dst, int value, size_t size) {
+    if (dev == nullptr || d_dst == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "memset: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    // a fill kernel rather than hipMemsetAsync, so that callers may capture this call into a HIP graph
+    return marmot_hip_fill_bytes_internal(dev, d_dst, value, size);
+}
+
+int marmot_hip_synchronize(marmot_hip_device_t *dev) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "synchronize: null device");
+    }
+    MH_HIP(hipStreamSynchronize(dev->stream));
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_allocator_usage(marmot_hip_device_t *dev, size_t *current_bytes, size_t *peak_bytes, size_t *n_allocs) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "allocator_usage: null device");
+    }
+    std::lock_guard<std::mutex> lock(dev->mu);
+    if (current_bytes != nullptr) {
+        *current_bytes = dev->current_bytes;
+    }
+    if (peak_bytes != nullptr) {
+        *peak_bytes = dev->peak_bytes;
+    }
+    if (n_allocs != nullptr) {
+        *n_allocs = dev->allocs.size();
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
+void *marmot_hip_stream(marmot_hip_device_t *dev) {
+    return dev != nullptr ? (void *)dev->stream : nullptr;
+}
+
+int marmot_hip_get_caps(marmot_hip_device_t *dev, marmot_hip_caps_t *caps) {
+    if (dev == nullptr || caps == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "get_caps: null argument");
+    }
+    memset(caps, 0, sizeof(*caps));
+    snprintf(caps->name, sizeof(caps->name), "%s", dev->props.name);
+    snprintf(caps->arch, sizeof(caps->arch), "%s", dev->props.gcnArchName);
+    caps->num_compute_units = (uint32_t)dev->props.multiProcessorCount;
+    caps->wavefront_size = (uint32_t)dev->props.warpSize;
+    caps->clock_mhz = (uint32_t)(dev->props.clockRate / 1000);
+    caps->mem_clock_mhz = (uint32_t)(dev->props.memoryClockRate / 1000);
+    caps->mem_bus_bits = (uint32_t)dev->props.memoryBusWidth;
+    caps->l2_cache_kb = (uint32_t)(dev->props.l2CacheSize / 1024);
+    caps->lds_kb_per_cu = (uint32_t)(dev->props.maxSharedMemoryPerMultiProcessor / 1024);
+    caps->total_mem_bytes = (uint64_t)dev->props.totalGlobalMem;
+    // published MI355X peaks (dense): HBM3E 8 TB/s, fp16 MFMA 2.5 PFLOP/s, int8 MFMA 5.0 POP/s
+    caps->mem_bw_gbps = 8000.0f;
+    caps->peak_tflops_fp16 = 2500.0f;
+    caps->peak_tops_int8 = 5000.0f;
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_event_create(marmot_hip_device_t *dev, void **out_event) {
+    if (dev == nullptr || out_event == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "event_create: null argument");
+    }
+    hipEvent_t ev;
+    MH_HIP(hipEventCreate(&ev));
+    *out_event = (void *)ev;
+    return MARMOT_HIP_SUCCESS;
+}
+
+void marmot_hip_event_destroy(marmot_hip_device_t *dev, void *event) {
+    (void)dev;
+    if (event != nullptr) {
+        (void)hipEventDestroy((hipEvent_t)event);
+    }
+}
+
+int marmot_hip_event_record(marmot_hip_device_t *dev, void *event) {
+    if (dev == nullptr || event == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "event_record: null argument");
+    }
+    MH_HIP(hipEventRecord((hipEvent_t)event, dev->stream));
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_event_elapsed_ms(marmot_hip_device_t *dev, void *start, void *stop, float *out_ms) {
+    if (dev == nullptr || start == nullptr || stop == nullptr || out_ms == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "event_elapsed: null argument");
+    }
+    MH_HIP(hipEventSynchronize((hipEvent_t)stop));
+    MH_HIP(hipEventElapsedTime(out_ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return MARMOT_HIP_SUCCESS;
+}
+
+} // extern "C"

@@ -1,0 +1,256 @@
+// marmot_hip_matmul_quantized: validation, route selection, and the direct (unquantized fp16 activation)
+// small-batch kernel. Compile with -ffp-contract=off (the direct route dequantizes weights exactly like the
+// reference before multiplying).
+#include "mh_common.h"
+#include "mh_dequant.h"
+
+namespace mh {
+
+// ------------------------------------------------------------------------------------------------
+// Direct route: out[n, m] = sum_k dequant(W[m, k]) * (float)x_f16[n, k], fp32 accumulate.
+// Counterpart of cpu_vec_dot_{q4_0,q8_0,q4_k}_f16 (vec_dot_impl.h:220-250, 419-450, 973-1023): the same
+// per-value fp32 weights, summed in a different order. One wavefront per weight row; a lane visits 8
+// consecutive k at a time (one 16-byte load of fp16 activations per column).
+// ------------------------------------------------------------------------------------------------
+struct DirectParams {
+    const uint8_t *w;
+    const uint16_t *x;
+    void *out;
+    const void *bias;
+    int bias_is_f16;
+    int out_is_f16;
+    size_t n0;
+    size_t K;
+    size_t M;
+    size_t nb;
+};
+
+template <int KIND, int NC>
+__global__ __launch_bounds__(256) void k_matvec_direct_f16(const DirectParams p) {
+    constexpr int BV = KindTraits<KIND>::BV;
+    constexpr int BB = KindTraits<KIND>::BB;
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= p.M) {
+        return;
+    }
+    const uint8_t *rowp = p.w + row * p.nb * BB;
+    float acc[NC];
+#pragma unroll
+    for (int n = 0; n < NC; ++n) {
+        acc[n] = 0.0f;
+    }
+    for (size_t k0 = (size_t)lane * 8; k0 < p.K; k0 += 64 * 8) {
+        const size_t b = k0 / BV;
+        const int v0 = (int)(k0 - b * BV);
+        const uint8_t *blk = rowp + b * BB;
+        float wv[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            wv[i] = (k0 + i < p.K) ? dequant_value<KIND>(blk, v0 + i) : 0.0f;
+        }
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+            const uint16_t *xp = p.x + (p.n0 + n) * p.K + k0;
+            if (k0 + 8 <= p.K && (((uintptr_t)xp) & 15) == 0) {
+                const uint4 xv = *(const uint4 *)xp;
+                const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[n] += wv[2 * i] * h2f((uint16_t)(xs[i] & 0xffffu));
+                    acc[n] += wv[2 * i + 1] * h2f((uint16_t)(xs[i] >> 16));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (k0 + i < p.K) {
+                        acc[n] += wv[i] * h2f(xp[i]);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < NC; ++n) {
+        const float s = wave_sum(acc[n]);
+        if (lane == 0) {
+            const size_t idx = (p.n0 + n) * p.M + row;
+            if (!p.out_is_f16) {
+                float v = s;
+                if (p.bias != nullptr) {
+                    v += ((const float *)p.bias)[row];
+                }
+                ((float *)p.out)[idx] = v;
+            } else {
+                uint16_t h = f2h(s);
+                if (p.bias != nullptr) {
+                    const float bv =
+                        p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[row]) : ((const float *)p.bias)[row];
+                    h = f2h(h2f(h) + bv);
+                }
+                ((uint16_t *)p.out)[idx] = h;
+            }
+        }
+    }
+}
+
+template <int KIND>
+static int launch_direct_kind(marmot_hip_device *dev, DirectParams p, size_t N) {
+    const dim3 grid((unsigned)((p.M + 3) / 4)), block(256);
+    size_t n0 = 0;
+    while (n0 < N) {
+        p.n0 = n0;
+        const size_t left = N - n0;
+        if (left >= 4) {
+            hipLaunchKernelGGL((k_matvec_direct_f16<KIND, 4>), grid, block, 0, dev->stream, p);
+            n0 += 4;
+        } else if (left >= 2) {
+            hipLaunchKernelGGL((k_matvec_direct_f16<KIND, 2>), grid, block, 0, dev->stream, p);
+            n0 += 2;
+        } else {
+            hipLaunchKernelGGL((k_matvec_direct_f16<KIND, 1>), grid, block, 0, dev->stream, p);
+            n0 += 1;
+        }
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
+                      const void *d_bias, int bias_dtype, void *d_out, int out_dtype) {
+    DirectParams p;
+    p.w = (const uint8_t *)d_w;
+    p.x = (const uint16_t *)d_x;
+    p.out = d_out;
+    p.bias = d_bias;
+    p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
+    p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    p.n0 = 0;
+    p.K = K;
+    p.M = M;
+    p.nb = (K + block_values(kind) - 1) / block_values(kind);
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_K:
+        set_route("matvec_q4_k_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q4_K>(dev, p, N);
+    case MARMOT_HIP_KIND_Q8_0:
+        set_route("matvec_q8_0_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q8_0>(dev, p, N);
+    case MARMOT_HIP_KIND_Q4_0:
+        set_route("matvec_q4_0_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q4_0>(dev, p, N);
+    default:
+        // Q6_K: the reference's fp16 direct dot (vec_dot_impl.h:1082-1128) decodes blocks with an index pattern
+        // that disagrees with its own Q6_K dequantizer; this backend declines the combination so that the caller
+        // falls back (NOT_IMPLEMENTED is the reference's fallback signal, dispatch_execute.c:214-233).
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED,
+                         "quantized matmul: fp16 activations without packing are not offered for quant kind %d", kind);
+    }
+}
+
+static int validate_matmul(const marmot_hip_device *dev, int kind, const void *d_weight, const void *d_input,
+                           int in_dtype, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
+                           const void *d_out, int out_dtype) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
+    }
+    if (d_weight == nullptr || d_input == nullptr || d_out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
+    }
+    if (kind != MARMOT_HIP_KIND_Q4_0 && kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_K &&
+        kind != MARMOT_HIP_KIND_Q6_K) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "Quantized matmul kernel not available for quant kind %d",
+                         kind);
+    }
+    const bool in_f32 = in_dtype == MARMOT_HIP_DTYPE_F32, in_f16 = in_dtype == MARMOT_HIP_DTYPE_F16;
+    const bool out_f32 = out_dtype == MARMOT_HIP_DTYPE_F32, out_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    if (!((in_f32 && out_f32) || (in_f16 && (out_f32 || out_f16)))) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE,
+                         "Quantized matmul requires FLOAT32 input or FLOAT16 activations with FLOAT16/FLOAT32 output");
+    }
+    if (d_bias != nullptr) {
+        const bool ok = (bias_dtype == MARMOT_HIP_DTYPE_F32) || (bias_dtype == MARMOT_HIP_DTYPE_F16 && out_f16);
+        if (!ok) {
+            return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "Matmul bias dtype is not compatible with the output");
+        }
+    }
+    if (K == 0 || M == 0) {
+        return set_error(MARMOT_HIP_ERROR_DIMENSION_MISMATCH, "Quantized matmul dimension mismatch on K");
+    }
+    (void)N;
+    return MARMOT_HIP_SUCCESS;
+}
+
+static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const void *d_input,
+                       int in_dtype, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0,
+                       void *d_out1, int out_dtype, uint32_t flags) {
+    if (N == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    MH_HIP(hipSetDevice(dev->device_index));
+    const bool direct = in_dtype == MARMOT_HIP_DTYPE_F16 && (flags & MARMOT_HIP_MATMUL_FORCE_PACK) == 0;
+    if (direct) {
+        for (int which = 0; which < (d_w1 != nullptr ? 2 : 1); ++which) {
+            const void *w = which ? d_w1 : d_w0;
+            void *o = which ? d_out1 : d_out0;
+            int st;
+            if (gemm_f16_supported(kind, N, K, M)) {
+                st = launch_gemm_f16(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);
+            } else {
+                st = launch_matvec_f16(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);
+            }
+            if (st != MARMOT_HIP_SUCCESS) {
+                return st;
+            }
+        }
+        return MARMOT_HIP_SUCCESS;
+    }
+    // packed route: quantize the activations once (shared by both weights of a dual call), then integer dots
+    const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+    const size_t need = act_scratch_layout(act_kind, N, K, nullptr, nullptr);
+    void *ws = nullptr;
+    int st = workspace_reserve(dev, need, &ws);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    ActScratch act;
+    act_scratch_layout(act_kind, N, K, ws, &act);
+    st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    return launch_matvec_packed(dev, kind, d_w0, d_w1, act, N, K, M, d_bias, bias_dtype, d_out0, d_out1, out_dtype);
+}
+
+} // namespace mh
+
+using namespace mh;
+
+extern "C" {
+
+int marmot_hip_matmul_quantized(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_input,
+                                int in_dtype, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
+                                void *d_out, int out_dtype, uint32_t flags) {
+    int st = validate_matmul(dev, kind, d_weight, d_input, in_dtype, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    return matmul_impl(dev, kind, d_weight, nullptr, d_input, in_dtype, N, K, M, d_bias, bias_dtype, d_out, nullptr,
+                       out_dtype, flags);
+}
+
+int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const void *d_weight_a,
+                                     const void *d_weight_b, const void *d_input, int in_dtype, size_t N, size_t K,
+                                     size_t M, void *d_out_a, void *d_out_b, int out_dtype, uint32_t flags) {
+    if (d_weight_b == nullptr || d_out_b == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
+    }
+    int st = validate_matmul(dev, kind, d_weight_a, d_input, in_dtype, N, K, M, nullptr, 0, d_out_a, out_dtype);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    return matmul_impl(dev, kind, d_weight_a, d_weight_b, d_input, in_dtype, N, K, M, nullptr, 0, d_out_a, d_out_b,
+                       out_dtype, flags);
+}
+
+} // extern "C"

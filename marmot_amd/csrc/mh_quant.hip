@@ -1,0 +1,314 @@
+// Dequantizers (bit-exact with the reference's CPU dequantizers) and activation quantizers
+// (bit-exact with its Q8_0 / Q8_K activation packers).
+//
+// This file must be compiled with -ffp-contract=off: every fp32 multiply / subtract below is meant to
+// round on its own, exactly as the reference's scalar CPU code does.
+#include "mh_common.h"
+#include "mh_dequant.h"
+
+#include <float.h>
+
+namespace mh {
+
+// ------------------------------------------------------------------------------------------------
+// Dequantize: one thread per output value; `kp` = padded row length (nb * block_values).
+// ------------------------------------------------------------------------------------------------
+
+template <int KIND>
+__global__ __launch_bounds__(256) void k_dequantize(const uint8_t *__restrict__ blocks, float *__restrict__ out,
+                                                    size_t rows, size_t k, size_t nb) {
+    constexpr int BV = KindTraits<KIND>::BV;
+    constexpr int BB = KindTraits<KIND>::BB;
+    const size_t kp = nb * BV;
+    const size_t total = rows * kp;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t row = idx / kp;
+        const size_t col = idx - row * kp;
+        if (col >= k) {
+            continue;
+        }
+        const size_t b = col / BV;
+        const int v = (int)(col - b * BV);
+        const uint8_t *blk = blocks + (row * nb + b) * BB;
+        const float y = dequant_value<KIND>(blk, v);
+        out[row * k + col] = y;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Activation quantizers
+// ------------------------------------------------------------------------------------------------
+
+// magic-number round-to-nearest-even with the input clamp of matmul_quant_pack.c:11-21
+__device__ __forceinline__ int nearest_int_clamped(float value) {
+    if (value > 4194303.0f) {
+        value = 4194303.0f;
+    } else if (value < -4194303.0f) {
+        value = -4194303.0f;
+    }
+    const float shifted = value + 12582912.0f;
+    const int bits = __float_as_int(shifted);
+    return (bits & 0x007fffff) - 0x00400000;
+}
+
+template <bool F16>
+__device__ __forceinline__ float load_act_value(const void *x, size_t i) {
+    if constexpr (F16) {
+        return h2f(((const uint16_t *)x)[i]);
+    } else {
+        return ((const float *)x)[i];
+    }
+}
+
+// Q8_K (matmul_quant_pack.c:106-142): one wavefront per 256-value block, 4 consecutive values per lane.
+// AOS = marmot_q8_k_block_t output; otherwise the library's structure-of-arrays scratch.
+template <bool F16, bool AOS>
+__global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ x, size_t rows, size_t k, size_t nb,
+                                                       uint8_t *__restrict__ blocks_out, ActScratch soa) {
+    const int lane = threadIdx.x & 63;
+    const size_t wave = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (wave >= rows * nb) {
+        return;
+    }
+    const size_t row = wave / nb;
+    const size_t b = wave - row * nb;
+    const size_t col0 = b * QK_K + (size_t)lane * 4;
+
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const size_t col = col0 + i;
+        v[i] = col < k ? load_act_value<F16>(x, row * k + col) : 0.0f;
+    }
+    // value of largest magnitude, first occurrence wins (strict > in index order)
+    float best_abs = 0.0f;
+    float best_val = 0.0f;
+    int best_idx = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float ax = fabsf(v[i]);
+        if (ax > best_abs) {
+            best_abs = ax;
+            best_val = v[i];
+            best_idx = lane * 4 + i;
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float o_abs = __shfl_xor(best_abs, off);
+        const float o_val = __shfl_xor(best_val, off);
+        const int o_idx = __shfl_xor(best_idx, off);
+        if (o_abs > best_abs || (o_abs == best_abs && o_idx < best_idx)) {
+            best_abs = o_abs;
+            best_val = o_val;
+            best_idx = o_idx;
+        }
+    }
+
+    int q[4] = {0, 0, 0, 0};
+    float d = 0.0f;
+    if (best_abs > 0.0f) {
+        const float iscale = -127.0f / best_val;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int t = nearest_int_clamped(iscale * v[i]);
+            q[i] = t > 127 ? 127 : t;
+        }
+        d = 1.0f / iscale;
+    }
+    int s = q[0] + q[1] + q[2] + q[3];
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2); // lanes 4j..4j+3 hold the sum of values 16j..16j+15
+    const uint32_t packed = (uint32_t)(uint8_t)(int8_t)q[0] | ((uint32_t)(uint8_t)(int8_t)q[1] << 8) |
+        ((uint32_t)(uint8_t)(int8_t)q[2] << 16) | ((uint32_t)(uint8_t)(int8_t)q[3] << 24);
+
+    if constexpr (AOS) {
+        uint8_t *blk = blocks_out + (row * nb + b) * Q8_K_BYTES;
+        __builtin_memcpy(blk + 4 + lane * 4, &packed, 4);
+        if ((lane & 3) == 0) {
+            const int16_t bs = (int16_t)s;
+            __builtin_memcpy(blk + 4 + 256 + (lane >> 2) * 2, &bs, 2);
+        }
+        if (lane == 0) {
+            __builtin_memcpy(blk, &d, 4);
+        }
+    } else {
+        *(uint32_t *)(soa.qs + row * soa.kp + b * QK_K + lane * 4) = packed;
+        if ((lane & 3) == 0) {
+            soa.sums[(row * nb + b) * 16 + (lane >> 2)] = (int16_t)s;
+        }
+        if (lane == 0) {
+            soa.d[row * nb + b] = d;
+        }
+    }
+}
+
+// Q8_0 (matmul_quant_pack.c:23-62, block.c:221-232 scalar): 32 lanes per block, one value per lane.
+template <bool F16, bool AOS>
+__global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ x, size_t rows, size_t k, size_t nb,
+                                                       uint8_t *__restrict__ blocks_out, ActScratch soa) {
+    const int lane32 = threadIdx.x & 31;
+    const size_t blk_id = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
+    if (blk_id >= rows * nb) {
+        return;
+    }
+    const size_t row = blk_id / nb;
+    const size_t b = blk_id - row * nb;
+    const size_t col = b * QK + lane32;
+    const float v = col < k ? load_act_value<F16>(x, row * k + col) : 0.0f;
+    float max_abs = fabsf(v);
+#pragma unroll
+    for (int off = 1; off < 32; off <<= 1) {
+        max_abs = fmaxf(max_abs, __shfl_xor(max_abs, off));
+    }
+    float scale = max_abs / 127.0f;
+    if (scale < FLT_MIN) {
+        scale = 1.0f;
+    }
+    const float inv_scale = 1.0f / scale;
+    int q = (int)roundf(v * inv_scale);
+    q = q < -127 ? -127 : (q > 127 ? 127 : q);
+    if (col >= k) {
+        q = 0;
+    }
+    int s = q;
+#pragma unroll
+    for (int off = 1; off < 32; off <<= 1) {
+        s += __shfl_xor(s, off);
+    }
+    const uint16_t hs = f2h(scale);
+    if constexpr (AOS) {
+        uint8_t *blk = blocks_out + (row * nb + b) * Q8_0_BYTES;
+        blk[2 + lane32] = (uint8_t)(int8_t)q;
+        if (lane32 == 0) {
+            __builtin_memcpy(blk, &hs, 2);
+        }
+    } else {
+        soa.qs[row * soa.kp + b * QK + lane32] = (int8_t)q;
+        if (lane32 == 0) {
+            soa.d[row * nb + b] = h2f(hs);
+            soa.sums[row * nb + b] = (int16_t)s;
+        }
+    }
+}
+
+__global__ void k_fill_bytes(uint8_t *dst, uint8_t value, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        dst[i] = value;
+    }
+}
+
+template <bool AOS>
+static int launch_quantize(marmot_hip_device *dev, int act_kind, const void *d_x, int in_dtype, size_t rows, size_t k,
+                           uint8_t *blocks_out, const ActScratch &soa) {
+    if (rows == 0 || k == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    const bool f16 = in_dtype == MARMOT_HIP_DTYPE_F16;
+    if (act_kind == MARMOT_HIP_KIND_Q8_K) {
+        const size_t nb = (k + QK_K - 1) / QK_K;
+        const size_t waves = rows * nb;
+        const dim3 grid((unsigned)((waves + 3) / 4));
+        if (f16) {
+            hipLaunchKernelGGL((k_quantize_q8_k<true, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
+                               blocks_out, soa);
+        } else {
+            hipLaunchKernelGGL((k_quantize_q8_k<false, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
+                               blocks_out, soa);
+        }
+    } else {
+        const size_t nb = (k + QK - 1) / QK;
+        const size_t blocks = rows * nb;
+        const dim3 grid((unsigned)((blocks + 7) / 8));
+        if (f16) {
+            hipLaunchKernelGGL((k_quantize_q8_0<true, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
+                               blocks_out, soa);
+        } else {
+            hipLaunchKernelGGL((k_quantize_q8_0<false, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
+                               blocks_out, soa);
+        }
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+int launch_quantize_act_soa(marmot_hip_device *dev, int act_kind, const void *d_x, int in_dtype, size_t rows, size_t k,
+                            const ActScratch &dst) {
+    return launch_quantize<false>(dev, act_kind, d_x, in_dtype, rows, k, nullptr, dst);
+}
+
+} // namespace mh
+
+using namespace mh;
+
+extern "C" {
+
+int marmot_hip_fill_bytes_internal(marmot_hip_device_t *dev, void *d_dst, int value, size_t size) {
+    const unsigned grid = (unsigned)((size + 256 * 16 - 1) / (256 * 16));
+    hipLaunchKernelGGL(k_fill_bytes, dim3(grid < 4096 ? (grid ? grid : 1) : 4096), dim3(256), 0, dev->stream,
+                       (uint8_t *)d_dst, (uint8_t)value, size);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_blocks, size_t rows, size_t k,
+                          float *d_out) {
+    if (dev == nullptr || d_blocks == nullptr || d_out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "dequantize: null argument");
+    }
+    const size_t bv = block_values(kind);
+    if (bv == 0) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "dequantize: unsupported quant kind %d", kind);
+    }
+    if (rows == 0 || k == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    const size_t nb = (k + bv - 1) / bv;
+    const size_t total = rows * nb * bv;
+    size_t g = (total + 255) / 256;
+    if (g > 65536) {
+        g = 65536;
+    }
+    const dim3 grid((unsigned)g), block(256);
+    const uint8_t *src = (const uint8_t *)d_blocks;
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_K:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q6_K:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q6_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q8_0:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q8_0>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q4_0:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_0>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q8_K:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q8_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    default:
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "dequantize: unsupported quant kind %d", kind);
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_quantize_activations(marmot_hip_device_t *dev, int act_kind, const void *d_x, int in_dtype,
+                                    size_t rows, size_t k, void *d_blocks_out) {
+    if (dev == nullptr || d_x == nullptr || d_blocks_out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "quantize_activations: null argument");
+    }
+    if (act_kind != MARMOT_HIP_KIND_Q8_0 && act_kind != MARMOT_HIP_KIND_Q8_K) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "quantize_activations: kind %d is not Q8_0/Q8_K",
+                         act_kind);
+    }
+    if (in_dtype != MARMOT_HIP_DTYPE_F32 && in_dtype != MARMOT_HIP_DTYPE_F16) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "quantize_activations: input dtype %d", in_dtype);
+    }
+    ActScratch none;
+    return launch_quantize<true>(dev, act_kind, d_x, in_dtype, rows, k, (uint8_t *)d_blocks_out, none);
+}
+
+} // extern "C"

@@ -1,0 +1,211 @@
+"""GPU parity, part 2: marmot_linear on the HIP backend against the CPU oracle (through the C ABI)."""
+import numpy as np
+import pytest
+
+from oracle.pyoracle import BLOCK_VALUES, KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0
+from tests.util import assert_matmul_parity, bits, gaussian, parity_metrics, quantize_weights, random_valid_blocks
+
+pytestmark = pytest.mark.gpu
+
+KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q6_k": KIND_Q6_K}
+THREADS = 16
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from marmot_amd import HipBackend
+
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+def test_reference_matmul_goldens_fp32(hip, ref_goldens, name):
+    """The reference's own golden cases (tests/backend/golden_matmul_llama.h), its own tolerance."""
+    kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
+    w = ref_goldens[f"matmul_{name}_weight"]
+    x = ref_goldens[f"matmul_{name}_input_f32"].reshape(N, K)
+    exp = ref_goldens[f"matmul_{name}_expected_f32"].reshape(N, M)
+    got = hip.linear(x, w, kind, M)
+    assert np.all(np.abs(got - exp) <= 2e-5 + 5e-5 * np.abs(exp)), (got, exp)
+
+
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K"])
+def test_reference_matmul_goldens_fp16(hip, ref_goldens, name):
+    kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
+    w = ref_goldens[f"matmul_{name}_weight"]
+    x = ref_goldens[f"matmul_{name}_input_f16"].view(np.float16).reshape(N, K)
+    exp = ref_goldens[f"matmul_{name}_expected_f16"].reshape(N, M)
+    got = hip.linear(x, w, kind, M)
+    assert np.all(np.abs(got - exp) <= 2e-5 + 5e-5 * np.abs(exp)), (got, exp)
+
+
+def test_config1_q8_0_matvec_full_size(hip, oracle):
+    """Q8_0, W 5632 x 2048 from N(0, 0.02) seed 0, x N(0,1) seed 1, batch 1."""
+    M, K = 5632, 2048
+    w = gaussian(0, (M, K), 0.02)
+    blocks = quantize_weights(oracle, KIND_Q8_0, w)
+    x = gaussian(1, (1, K))
+    ref = oracle.matmul(KIND_Q8_0, blocks, x, M, threads=THREADS)
+    got = hip.linear(x, blocks, KIND_Q8_0, M)
+    print("route:", hip.last_route(), "metrics:", parity_metrics(got, ref), flush=True)
+    assert_matmul_parity(got, ref, what="C1 Q8_0 5632x2048")
+    # dequantized weights bit-exact
+    assert np.array_equal(bits(hip.dequantize(KIND_Q8_0, blocks, K)), bits(oracle.dequantize(KIND_Q8_0, blocks, K)))
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K", [(14336, 4096), (4096, 14336)])
+def test_config2_kquant_decode_full_size(hip, oracle, name, M, K):
+    """Q4_K / Q6_K at Llama-3-8B FFN shapes, batch 1, 4 and 8, activations quantized to Q8_K on device."""
+    kind = KINDS[name]
+    i = ["q4_k", "q6_k"].index(name) * 2 + (0 if M == 14336 else 1)
+    print(f"C2 {name} {M}x{K}: quantizing weights", flush=True)
+    w = gaussian(10 + i, (M, K), 0.02)
+    blocks = quantize_weights(oracle, kind, w)
+    del w
+    d_w = hip.to_device(blocks)
+    # dequantized weights: bit-exact over every element of the matrix
+    d_f = hip.alloc(M * K * 4)
+    hip.dequantize_d(kind, d_w, M, K, d_f)
+    deq = d_f.download(np.float32, (M, K))
+    d_f.free()
+    step = 1024
+    for r0 in range(0, M, step):
+        exp = oracle.dequantize(kind, blocks[r0:r0 + step], K)
+        assert np.array_equal(bits(deq[r0:r0 + step]), bits(exp)), f"dequant differs in rows {r0}.."
+    del deq
+    for N in (1, 4, 8):
+        print(f"C2 {name} {M}x{K} N={N}", flush=True)
+        x = gaussian(20 + i, (N, K))
+        ref = oracle.matmul(kind, blocks, x, M, threads=THREADS)
+        d_x = hip.to_device(x)
+        d_o = hip.alloc(N * M * 4)
+        hip.linear_d(kind, d_w, d_x, 0, N, K, M, d_o, 0)
+        got = d_o.download(np.float32, (N, M))
+        d_x.free()
+        d_o.free()
+        m = assert_matmul_parity(got, ref, what=f"C2 {name} {M}x{K} N={N}")
+        print("   route:", hip.last_route(), "metrics:", m, flush=True)
+    d_w.free()
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("N", [1, 2, 3, 5, 8, 11, 16, 19])
+def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
+    """All column-tile widths (8/4/2/1) and M not a multiple of the rows-per-workgroup."""
+    kind = KINDS[name]
+    M, K = 203, 2048
+    blocks = oracle.quantize(kind, gaussian(60, (M, K), 0.02))
+    x = gaussian(61 + N, (N, K))
+    ref = oracle.matmul(kind, blocks, x, M)
+    got = hip.linear(x, blocks, kind, M)
+    assert_matmul_parity(got, ref, what=f"{name} N={N}")
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("K", [256, 512, 768, 1280, 8192, 11008, 28672])
+def test_linear_k_sweep(hip, oracle, name, K):
+    """Rows shorter than one wave-load, rows needing several wavefronts, and long rows."""
+    kind = KINDS[name]
+    M = 70
+    blocks = oracle.quantize(kind, gaussian(70, (M, K), 0.02))
+    for N in (1, 4):
+        x = gaussian(71 + N, (N, K))
+        ref = oracle.matmul(kind, blocks, x, M)
+        got = hip.linear(x, blocks, kind, M)
+        assert_matmul_parity(got, ref, what=f"{name} K={K} N={N}")
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+def test_linear_ragged_k(hip, oracle, name):
+    """K not a multiple of the block: weight and activation tails are zero-padded blocks."""
+    kind = KINDS[name]
+    bv = BLOCK_VALUES[kind]
+    K = 3 * bv + bv // 2 + 3
+    M = 9
+    blocks = oracle.quantize(kind, gaussian(80, (M, K), 0.02))
+    x = gaussian(81, (3, K))
+    ref = oracle.matmul(kind, blocks, x, M)
+    got = hip.linear(x, blocks, kind, M)
+    assert_matmul_parity(got, ref, what=f"{name} ragged K={K}")
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+def test_linear_random_block_bytes(hip, oracle, name):
+    """Weights that are arbitrary block bytes (all 6-bit scale / min patterns, negative Q6_K scales)."""
+    kind = KINDS[name]
+    rng = np.random.default_rng(90)
+    M, K = 33, 2048
+    blocks = random_valid_blocks(rng, kind, M, K)
+    x = gaussian(91, (4, K))
+    ref = oracle.matmul(kind, blocks, x, M)
+    got = hip.linear(x, blocks, kind, M)
+    assert_matmul_parity(got, ref, what=f"{name} random bytes")
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "q6_k"])
+def test_linear_bias_epilogue(hip, oracle, name):
+    kind = KINDS[name]
+    M, K, N = 50, 1024, 3
+    blocks = oracle.quantize(kind, gaussian(100, (M, K), 0.02))
+    x = gaussian(101, (N, K))
+    bias = gaussian(102, (M,))
+    ref = oracle.matmul(kind, blocks, x, M, bias=bias)
+    got = hip.linear(x, blocks, kind, M, bias=bias)
+    d = np.abs(got - ref)
+    assert np.max(d) <= 1e-5 * max(1.0, np.abs(ref).max())
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k"])
+def test_linear_fp16_direct_small_batch(hip, oracle, name):
+    """fp16 activations take the direct route (no activation quantization) like the CPU reference."""
+    kind = KINDS[name]
+    M, K = 64, 1024
+    blocks = oracle.quantize(kind, gaussian(110, (M, K), 0.02))
+    for N in (1, 3, 7):
+        x = gaussian(111 + N, (N, K)).astype(np.float16)
+        ref = oracle.matmul(kind, blocks, x, M)
+        got = hip.linear(x, blocks, kind, M)
+        assert "direct" in hip.last_route() or "gemm" in hip.last_route()
+        assert_matmul_parity(got, ref, what=f"{name} fp16 N={N}")
+        got16 = hip.linear(x, blocks, kind, M, out_dtype=np.float16)
+        ref16 = oracle.matmul(kind, blocks, x, M, out_dtype=np.float16)
+        assert np.max(np.abs(got16.astype(np.float32) - ref16.astype(np.float32))) <= \
+            2e-3 * np.abs(ref16.astype(np.float32)).max()
+        # forced packing of fp16 activations equals the fp32 packed path on the widened values
+        forced = hip.linear(x, blocks, kind, M, force_pack=True)
+        assert_matmul_parity(forced, oracle.matmul(kind, blocks, x, M, force_pack=True), what=f"{name} forced")
+
+
+def test_linear_dual_output_equals_two_singles(hip, oracle):
+    """cpu_matmul_quantized_dual_output semantics (test_matmul_quantized.c:202-298)."""
+    M, K, N = 96, 2048, 5
+    a = oracle.quantize(KIND_Q4_K, gaussian(120, (M, K), 0.02))
+    b = oracle.quantize(KIND_Q4_K, gaussian(121, (M, K), 0.02))
+    x = gaussian(122, (N, K))
+    oa, ob = hip.linear_dual(x, a, b, KIND_Q4_K, M)
+    assert np.array_equal(bits(oa), bits(hip.linear(x, a, KIND_Q4_K, M)))
+    assert np.array_equal(bits(ob), bits(hip.linear(x, b, KIND_Q4_K, M)))
+
+
+def test_linear_error_behaviour(hip, oracle):
+    from marmot_amd import MarmotHipError
+
+    M, K = 8, 256
+    blocks = oracle.quantize(KIND_Q4_K, gaussian(130, (M, K), 0.02))
+    x = gaussian(131, (1, K))
+    with pytest.raises(MarmotHipError) as e:  # fp32 input cannot produce fp16 output (helpers/matmul.c:104-112)
+        hip.linear(x, blocks, KIND_Q4_K, M, out_dtype=np.float16)
+    assert e.value.code == -6
+    with pytest.raises(MarmotHipError) as e:  # unsupported quant kind -> NOT_IMPLEMENTED (fallback signal)
+        hip.linear(x, np.zeros(M * 84, dtype=np.uint8), 7, M) if False else hip.linear_d(
+            7, hip.to_device(blocks), hip.to_device(x), 0, 1, K, M, hip.alloc(64), 0)
+    assert e.value.code == -8
+    with pytest.raises(MarmotHipError) as e:  # Q6_K with unpacked fp16 activations is declined
+        hip.linear(x.astype(np.float16), oracle.quantize(KIND_Q6_K, gaussian(132, (M, K), 0.02)), KIND_Q6_K, M)
+    assert e.value.code == -8
+    # N = 0 is a no-op
+    hip.linear_d(KIND_Q4_K, hip.to_device(blocks), hip.to_device(x), 0, 0, K, M, hip.alloc(64), 0)
+    hip.synchronize()

@@ -1,0 +1,94 @@
+"""GPU parity, part 1: dequantizers and activation quantizers are bit-exact against the CPU oracle."""
+import numpy as np
+import pytest
+
+from oracle.pyoracle import (BLOCK_BYTES, BLOCK_VALUES, KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K,
+                             row_bytes)
+from tests.util import bits, gaussian, quantize_weights, random_valid_blocks
+
+pytestmark = pytest.mark.gpu
+
+KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q6_k": KIND_Q6_K}
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from marmot_amd import HipBackend
+
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def test_device_is_gfx950(hip):
+    caps = hip.caps()
+    print("device:", caps, flush=True)
+    assert caps["arch"].startswith("gfx950")
+    assert caps["wavefront_size"] == 64
+    assert caps["num_compute_units"] >= 200
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("rows,k", [(3, 1024), (2, 300), (1, 70), (64, 4096)])
+def test_dequantize_bit_exact_quantized_gaussian(hip, oracle, name, rows, k):
+    print(f"dequant {name} rows={rows} k={k}", flush=True)
+    kind = KINDS[name]
+    w = gaussian(200 + rows + k, (rows, k), 0.02)
+    blocks = oracle.quantize(kind, w)
+    exp = oracle.dequantize(kind, blocks, k)
+    got = hip.dequantize(kind, blocks, k)
+    assert np.array_equal(bits(got), bits(exp))
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+def test_dequantize_bit_exact_random_bytes(hip, oracle, name):
+    """Every scale / nibble pattern, not only what a quantizer emits."""
+    print(f"dequant random bytes {name}", flush=True)
+    kind = KINDS[name]
+    rng = np.random.default_rng(31)
+    k = 16 * BLOCK_VALUES[kind]
+    blocks = random_valid_blocks(rng, kind, 37, k)
+    exp = oracle.dequantize(kind, blocks, k)
+    got = hip.dequantize(kind, blocks, k)
+    assert np.array_equal(bits(got), bits(exp))
+
+
+def test_dequantize_q8_k_and_golden_blocks(hip, oracle, ref_goldens):
+    x = gaussian(77, (2, 512))
+    blocks = oracle.quantize(KIND_Q8_K, x)
+    assert np.array_equal(bits(hip.dequantize(KIND_Q8_K, blocks, 512)), bits(oracle.dequantize(KIND_Q8_K, blocks, 512)))
+    # the reference-held golden blocks: same tolerance as the reference's own test
+    for name, tol in (("q4_0", 5e-4), ("q8_0", 5e-4), ("q4_k", 6e-4), ("q6_k", 6e-4)):
+        exp = ref_goldens[f"g_llama_{name}_dequant"]
+        got = hip.dequantize(KINDS[name], ref_goldens[f"g_llama_{name}"], exp.size)[0]
+        assert np.max(np.abs(got - exp)) <= tol
+
+
+@pytest.mark.parametrize("act_kind", [KIND_Q8_0, KIND_Q8_K])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,k", [(1, 2048), (5, 4096), (3, 300), (2, 70), (16, 14336)])
+def test_activation_quantizer_bit_exact(hip, oracle, act_kind, dtype, rows, k):
+    print(f"act quant kind={act_kind} {np.dtype(dtype).name} rows={rows} k={k}", flush=True)
+    x = gaussian(300 + rows * 7 + k, (rows, k)).astype(dtype)
+    if rows > 1:
+        x[1, : min(k, 256)] = 0  # an all-zero block
+    x[0, 3] = -abs(x[0]).max() * 2  # the largest magnitude is negative
+    if k > 40:
+        x[0, 37] = -x[0, 3]  # same magnitude later in the block, opposite sign: first occurrence must win
+    got = hip.quantize_activations(act_kind, x)
+    exp = np.stack([oracle.pack(act_kind, x[r]) for r in range(rows)])
+    assert got.shape == exp.shape
+    assert np.array_equal(got, exp), f"{(got != exp).sum()} bytes differ"
+
+
+def test_activation_quantizer_rounding_ties(hip, oracle):
+    """Values that land exactly on .5 after scaling: Q8_0 rounds half away from zero, Q8_K half to even."""
+    x = np.zeros((1, 256), dtype=np.float32)
+    x[0, :32] = np.arange(32, dtype=np.float32) * 0.5
+    x[0, 31] = 127.0  # scale = 1 -> values k/2 are exact ties
+    x[0, 32:64] = -x[0, :32]
+    x[0, 255] = -127.0
+    for act_kind in (KIND_Q8_0, KIND_Q8_K):
+        got = hip.quantize_activations(act_kind, x)
+        exp = oracle.pack(act_kind, x[0])[None, :]
+        assert np.array_equal(got, exp)

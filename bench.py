@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized GGUF matmul hot path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: marmot_linear with a Q4_K weight of
+4096 x 14336 (Llama-3-8B FFN down projection, marmot M x K) and one fp32 activation row — activation
+quantization to Q8_K on the device followed by the decode matvec. Weights rotate over enough distinct
+copies to exceed the 256 MB Infinity Cache, so the figure is an HBM figure, not a cache figure.
+
+Prints ONE JSON line (see README / the driver contract): `value` is whole-op GB/s (algorithmic bytes of the
+op / wall time per step, inputs resident in HBM), `roofline` describes the dominant kernel (the matvec,
+timed alone with HIP events on the library's stream), `cpu_baseline` is the CPU oracle timed on the host.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "Q4_K matvec GB/s (% HBM peak) + prefill GEMM TOPS (% MFMA peak)"
+HBM_PEAK_GBPS = 8000.0
+MALL_BYTES = 256 << 20
+TRAFFIC_DEFAULT_WORKLOAD = 33_297_000  # bytes per launch of the pre-packed Q4_K 4096x14336 N=1 matvec kernel
+
+
+def algorithmic_bytes(kind_row_bytes: int, M: int, K: int, N: int) -> int:
+    """Compulsory traffic of one linear: weights at true block bytes + fp32 activations in + fp32 outputs out."""
+    return M * kind_row_bytes + N * K * 4 + N * M * 4
+
+
+def random_blocks(rng, kind: int, rows: int, k: int) -> np.ndarray:
+    """Synthetic weights: arbitrary block payloads with finite, small fp16 super-block scales."""
+    from marmot_amd import block_bytes, block_values
+
+    nb = (k + block_values(kind) - 1) // block_values(kind)
+    bb = block_bytes(kind)
+    raw = rng.integers(0, 256, size=(rows * nb, bb), dtype=np.uint8)
+    offs = {1: [0], 5: [0], 9: [0, 2], 11: [208]}[kind]
+    for off in offs:
+        h = raw[:, off:off + 2].copy().view(np.uint16)
+        h = (h & 0x83FF) | 0x2000  # exponent field 8: magnitudes around 2^-7
+        raw[:, off:off + 2] = h.view(np.uint8)
+    return raw.reshape(rows, nb * bb)
+
+
+def time_steps_graph(hip, fn, steps: int, warmup: int, chunk: int = 500):
+    """Like time_steps, but the timed steps are replayed from HIP graphs (chunks of up to `chunk` steps), so the
+    host's launch rate does not enter the figure. Returns ms per step by HIP events."""
+    for i in range(warmup):
+        fn(i)
+    hip.synchronize()
+    graphs = []
+    done = 0
+    while done < steps:
+        n = min(chunk, steps - done)
+        base = warmup + done
+        graphs.append(hip.graph_capture(lambda: [fn(base + j) for j in range(n)]))
+        done += n
+    for g in graphs[:1]:  # one untimed replay: first-launch costs of the graph
+        hip.graph_launch(g)
+    hip.synchronize()
+    e0, e1 = hip.event(), hip.event()
+    hip.record(e0)
+    for g in graphs:
+        hip.graph_launch(g)
+    hip.record(e1)
+    hip.synchronize()
+    ms = hip.elapsed_ms(e0, e1) / steps
+    for g in graphs:
+        hip.graph_destroy(g)
+    return ms
+
+
+def time_steps(hip, fn, steps: int, warmup: int):
+    """Runs fn(i) for warmup + steps launches; returns (ms per step by HIP events, ms per step by host clock)."""
+    for i in range(warmup):
+        fn(i)
+    hip.synchronize()
+    e0, e1 = hip.event(), hip.event()
+    t0 = time.perf_counter()
+    hip.record(e0)
+    for i in range(steps):
+        fn(warmup + i)
+    hip.record(e1)
+    hip.synchronize()
+    t1 = time.perf_counter()
+    ev_ms = hip.elapsed_ms(e0, e1)
+    return ev_ms / steps, (t1 - t0) * 1e3 / steps
+
+
+def cpu_baseline(kind, blocks, x, M, K, nbytes, ref_out, budget_s: float):
+    """The CPU oracle (a restatement of the reference's CPU path) on the host cores, same workload."""
+    from oracle.pyoracle import Oracle
+
+    oracle = Oracle()
+    cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
+    out = oracle.matmul(kind, blocks, x, M, threads=cores)  # warm-up, and the parity check of the GPU result
+    rms = float(np.sqrt(np.mean(out.astype(np.float64) ** 2)))
+    err = float(np.max(np.abs(ref_out - out) / np.maximum(np.abs(out), 1e-3 * rms)))
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while time.perf_counter() < t_end and len(times) < 2000:
+        t0 = time.perf_counter()
+        oracle.matmul(kind, blocks, x, M, threads=cores)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    t1 = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle.matmul(kind, blocks, x, M, threads=1)
+        t1.append(time.perf_counter() - t0)
+    return {
+        "value": round(nbytes / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{len(times)} runs of the same Q4_K {M}x{K} N={x.shape[0]} linear (median), threads split over "
+                  f"weight rows with the reference's grain rule",
+        "ms_per_step": round(med * 1e3, 4),
+        "single_thread_gbps": round(nbytes / float(np.median(t1)) / 1e9, 3),
+    }, err
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="time budget of the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
+    ap.add_argument("--batch", type=int, default=1, help="activation rows N (1, 4 or 8 are the decode configs)")
+    ap.add_argument("--shape", default="4096x14336", help="weight shape MxK (marmot naming)")
+    ap.add_argument("--kind", default="q4_k", choices=["q4_k", "q6_k", "q8_0", "q4_0"])
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists in the hot path)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    from marmot_amd import DT_F32, HipBackend, row_bytes
+    from marmot_amd import capi
+
+    if args.calibrate_copy:
+        hip = HipBackend(0)
+        n = args.calibrate_copy << 20
+        src, dst = hip.alloc(n), hip.alloc(n)
+        hip.lib.marmot_hip_memset(hip.dev, src.ptr, 1, n)
+        ms, _ = time_steps(hip, lambda i: hip.copy_d(dst, src, n), 20, 3)
+        print(json.dumps({"calibration": "plain 16-byte copy kernel", "bytes_read": n, "bytes_written": n,
+                          "launches": 23, "ms_per_launch": round(ms, 5),
+                          "gbps_read_plus_write": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
+        hip.close()
+        return
+
+    kind = {"q4_k": capi.KIND_Q4_K, "q6_k": capi.KIND_Q6_K, "q8_0": capi.KIND_Q8_0, "q4_0": capi.KIND_Q4_0}[args.kind]
+    M, K = (int(v) for v in args.shape.split("x"))
+    N = args.batch
+    rb = row_bytes(kind, K)
+    wbytes = M * rb
+    nbytes = algorithmic_bytes(rb, M, K, N)
+
+    hip = HipBackend(0)
+    caps = hip.caps()
+    rng = np.random.Generator(np.random.PCG64(10))
+    blocks = random_blocks(rng, kind, M, K)
+    x = np.random.Generator(np.random.PCG64(20)).standard_normal((N, K), dtype=np.float32)
+
+    # distinct weight copies, 256-byte aligned, together larger than twice the Infinity Cache
+    stride = (wbytes + 255) & ~255
+    copies = max(2, -(-2 * MALL_BYTES // stride) + 1)
+    d_w = hip.alloc(stride * copies)
+    for c in range(copies):
+        d_w.upload(blocks, offset=c * stride)
+    d_x = hip.to_device(x)
+    d_out = hip.alloc(N * M * 4)
+    d_packed = hip.alloc(hip.packed_activation_bytes(kind, N, K))
+
+    # ---- whole op: activation quantization + matvec, weights rotating
+    def step(i):
+        hip.linear_d(kind, d_w, d_x, DT_F32, N, K, M, d_out, DT_F32, weight_offset=(i % copies) * stride)
+
+    ms_op_eager, ms_op_host = time_steps(hip, step, args.steps, args.warmup)
+    ms_op = time_steps_graph(hip, step, args.steps, args.warmup)
+    route = hip.last_route()
+    got = d_out.download(np.float32, (N, M))
+
+    # ---- dominant kernel alone: matvec on pre-packed activations, weights rotating
+    hip.pack_activations_d(kind, d_x, DT_F32, N, K, d_packed)
+
+    def kstep(i):
+        hip.linear_prepacked_d(kind, d_w, d_packed, N, K, M, d_out, weight_offset=(i % copies) * stride)
+
+    ms_k_eager, _ = time_steps(hip, kstep, args.steps, args.warmup)
+    ms_k = time_steps_graph(hip, kstep, args.steps, args.warmup)
+
+    # ---- same kernel with the weights resident in the Infinity Cache (one copy), reported separately
+    def kstep_hot(i):
+        hip.linear_prepacked_d(kind, d_w, d_packed, N, K, M, d_out, weight_offset=0)
+
+    ms_hot = time_steps_graph(hip, kstep_hot, args.steps, args.warmup)
+
+    value = nbytes / (ms_op * 1e-3) / 1e9
+    achieved = nbytes / (ms_k * 1e-3) / 1e9
+    result = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_op, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.kind.upper()} decode matvec, weight {M}x{K} (marmot MxK), N={N} fp32 activations "
+                        f"quantized to {'Q8_K' if kind in (9, 11) else 'Q8_0'} on device, fp32 output",
+            "weight_copies": copies,
+            "weight_bytes": wbytes,
+            "algorithmic_bytes_per_step": nbytes,
+            "route": route,
+            "device": caps["name"],
+            "arch": caps["arch"],
+            "compute_units": caps["num_compute_units"],
+        },
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
+        "tokens_per_s": round(N / (ms_op * 1e-3), 1),
+        "submission": "HIP graph replay of the timed steps (chunks of 500 steps)",
+        "eager_ms_per_step": round(ms_op_eager, 6),
+        "eager_ms_per_step_host_clock": round(ms_op_host, 6),
+        "roofline": {
+            "kernel": route,
+            "bound": "hbm",
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy kernel
+            # (profiles/matvec_q4_k_4096x14336_n1.md); only valid for the default workload
+            "traffic": TRAFFIC_DEFAULT_WORKLOAD if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) else None,
+            "avg_launch_us": round(ms_k * 1e3, 3),
+            "avg_launch_us_eager": round(ms_k_eager * 1e3, 3),
+            "cache_resident_gbps": round(nbytes / (ms_hot * 1e-3) / 1e9, 2),
+        },
+    }
+    if not args.no_cpu:
+        cb, err = cpu_baseline(kind, blocks, x, M, K, nbytes, got, args.cpu_seconds)
+        result["cpu_baseline"] = cb
+        result["parity_max_rel_err_vs_cpu"] = float(f"{err:.3e}")
+    else:
+        result["cpu_baseline"] = None
+    hip.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

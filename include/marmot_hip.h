@@ -109,6 +109,16 @@ typedef struct {
 } marmot_hip_caps_t;
 int marmot_hip_get_caps(marmot_hip_device_t *dev, marmot_hip_caps_t *caps);
 
+/* Batched submission: everything enqueued between begin and end is recorded into a HIP graph instead of being
+ * executed; launching the returned graph replays the whole batch with one submission. This is the HIP form of
+ * marmot_device_ops_t.graph_batch_begin / graph_batch_end(commit) (include/marmot/device.h:57-61), which the graph
+ * executor brackets a bytecode program with (src/graph/graph_executor.cpp:895). Calls that would allocate
+ * (a first use of a larger workspace) must have happened before begin_capture. */
+int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev);
+int marmot_hip_graph_end_capture(marmot_hip_device_t *dev, void **out_graph_exec);
+int marmot_hip_graph_launch(marmot_hip_device_t *dev, void *graph_exec);
+void marmot_hip_graph_destroy(marmot_hip_device_t *dev, void *graph_exec);
+
 /* Timing helpers (HIP events on the device object's stream). */
 int marmot_hip_event_create(marmot_hip_device_t *dev, void **out_event);
 void marmot_hip_event_destroy(marmot_hip_device_t *dev, void *event);
@@ -158,6 +168,19 @@ int marmot_hip_matmul_quantized(marmot_hip_device_t *dev, int kind, const void *
 int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const void *d_weight_a,
                                      const void *d_weight_b, const void *d_input, int in_dtype, size_t N, size_t K,
                                      size_t M, void *d_out_a, void *d_out_b, int out_dtype, uint32_t flags);
+
+/* ------------------------------------------------------------------ pre-packed activations
+ * The reference packs (quantizes) a tile of activations once and then runs the row kernels against the packed
+ * tile: cpu_quant_matmul_pack_column (matmul_quant_dispatch.c:270-302) followed by
+ * cpu_quant_matmul_dispatch_quant_tile (matmul_quant_compute.c:1958-1990). These three entry points expose the
+ * same split, so that several weights sharing one input (q/k/v, gate/up) pay for one quantization.
+ * The packed buffer has a library-private layout; only its size is public. */
+size_t marmot_hip_packed_activation_bytes(int weight_kind, size_t N, size_t K);
+int marmot_hip_pack_activations(marmot_hip_device_t *dev, int weight_kind, const void *d_input, int in_dtype,
+                                size_t N, size_t K, void *d_packed);
+int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_packed,
+                                size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out,
+                                int out_dtype);
 
 /* ------------------------------------------------------------------ MoE
  * Replaces cpu_topk_impl (src/backends/cpu/ops/moe/moe_ops.c:789-889): top-k over the last axis of

@@ -98,6 +98,9 @@ class HipBackend:
         arr = np.ascontiguousarray(arr)
         return DeviceBuffer(self, arr.nbytes).upload(arr)
 
+    def copy_d(self, d_dst, d_src, nbytes: int):
+        check(self.lib.marmot_hip_memcpy_device(self.dev, C.c_void_p(d_dst.ptr), C.c_void_p(d_src.ptr), nbytes))
+
     def synchronize(self):
         check(self.lib.marmot_hip_synchronize(self.dev))
 
@@ -114,6 +117,23 @@ class HipBackend:
 
     def last_route(self) -> str:
         return self.lib.marmot_hip_last_route().decode()
+
+    def graph_capture(self, fn):
+        """Records everything fn() enqueues into a HIP graph and returns the executable graph handle."""
+        check(self.lib.marmot_hip_graph_begin_capture(self.dev))
+        g = C.c_void_p()
+        try:
+            fn()
+        finally:
+            st = self.lib.marmot_hip_graph_end_capture(self.dev, C.byref(g))
+        check(st)
+        return g
+
+    def graph_launch(self, g):
+        check(self.lib.marmot_hip_graph_launch(self.dev, g))
+
+    def graph_destroy(self, g):
+        self.lib.marmot_hip_graph_destroy(self.dev, g)
 
     def event(self):
         e = C.c_void_p()
@@ -138,6 +158,19 @@ class HipBackend:
             self.dev, kind, C.c_void_p(d_weight.ptr + weight_offset), C.c_void_p(d_input.ptr), in_dtype, N, K, M,
             C.c_void_p(d_bias.ptr) if d_bias is not None else None, bias_dtype, C.c_void_p(d_out.ptr), out_dtype,
             flags))
+
+    def packed_activation_bytes(self, kind: int, N: int, K: int) -> int:
+        return int(self.lib.marmot_hip_packed_activation_bytes(kind, N, K))
+
+    def pack_activations_d(self, kind: int, d_input, in_dtype: int, N: int, K: int, d_packed):
+        check(self.lib.marmot_hip_pack_activations(self.dev, kind, C.c_void_p(d_input.ptr), in_dtype, N, K,
+                                                   C.c_void_p(d_packed.ptr)))
+
+    def linear_prepacked_d(self, kind: int, d_weight, d_packed, N: int, K: int, M: int, d_out, out_dtype: int = DT_F32,
+                           d_bias=None, bias_dtype: int = DT_F32, weight_offset: int = 0):
+        check(self.lib.marmot_hip_matmul_prepacked(
+            self.dev, kind, C.c_void_p(d_weight.ptr + weight_offset), C.c_void_p(d_packed.ptr), N, K, M,
+            C.c_void_p(d_bias.ptr) if d_bias is not None else None, bias_dtype, C.c_void_p(d_out.ptr), out_dtype))
 
     # ---- numpy level ops (what the parity tests call)
     def dequantize(self, kind: int, blocks: np.ndarray, k: int) -> np.ndarray:

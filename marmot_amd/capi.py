@@ -50,6 +50,10 @@ SIGNATURES = {
     "marmot_hip_stream": (_vp, [_vp]),
     "marmot_hip_last_error": (C.c_char_p, []),
     "marmot_hip_get_caps": (_i, [_vp, C.POINTER(Caps)]),
+    "marmot_hip_graph_begin_capture": (_i, [_vp]),
+    "marmot_hip_graph_end_capture": (_i, [_vp, C.POINTER(_vp)]),
+    "marmot_hip_graph_launch": (_i, [_vp, _vp]),
+    "marmot_hip_graph_destroy": (None, [_vp, _vp]),
     "marmot_hip_event_create": (_i, [_vp, C.POINTER(_vp)]),
     "marmot_hip_event_destroy": (None, [_vp, _vp]),
     "marmot_hip_event_record": (_i, [_vp, _vp]),
@@ -61,6 +65,9 @@ SIGNATURES = {
     "marmot_hip_quantize_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
     "marmot_hip_matmul_quantized": (_i, [_vp, _i, _vp, _vp, _i, _sz, _sz, _sz, _vp, _i, _vp, _i, _u32]),
     "marmot_hip_matmul_quantized_dual": (_i, [_vp, _i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _i, _u32]),
+    "marmot_hip_packed_activation_bytes": (_sz, [_i, _sz, _sz]),
+    "marmot_hip_pack_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
+    "marmot_hip_matmul_prepacked": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _vp, _i, _vp, _i]),
     "marmot_hip_topk": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
     "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "marmot_hip_moe_experts": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i,

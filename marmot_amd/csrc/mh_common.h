@@ -124,6 +124,7 @@ struct marmot_hip_device {
     // src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:331-371)
     void *workspace = nullptr;
     size_t workspace_bytes = 0;
+    bool capturing = false;  // between graph_begin_capture and graph_end_capture
     // allocation accounting
     std::mutex mu;
     std::unordered_map<void *, size_t> allocs;
@@ -142,9 +143,12 @@ size_t act_scratch_layout(int act_kind, size_t rows, size_t k, void *base, ActSc
 // kernels / launchers implemented in the .hip files
 int launch_quantize_act_soa(marmot_hip_device *dev, int act_kind, const void *d_x, int in_dtype, size_t rows, size_t k,
                             const ActScratch &dst);
-int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act,
-                         size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1,
-                         int out_dtype);
+// act == nullptr selects the fused variant: d_x_f32 ([N,K] fp32, N <= 4, K a multiple of the block) is quantized inside
+// the matvec kernel; otherwise `act` holds activations packed by launch_quantize_act_soa.
+bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_f32);
+int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
+                         const float *d_x_f32, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
+                         void *d_out0, void *d_out1, int out_dtype);
 int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M);
@@ -173,6 +177,24 @@ __device__ __forceinline__ float wave_sum(float v) {
     const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
     const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
     return (r0 + r1) + (r2 + r3);
+}
+
+// magic-number round-to-nearest-even with the input clamp of the reference's activation packer
+// (matmul_quant_pack.c:11-21)
+__device__ __forceinline__ int nearest_int_clamped(float value) {
+    value = fminf(fmaxf(value, -4194303.0f), 4194303.0f);  // branch-free form of the reference's two-sided clamp
+    const float shifted = value + 12582912.0f;
+    const int bits = __float_as_int(shifted);
+    return (bits & 0x007fffff) - 0x00400000;
+}
+
+// Sum over each row of 16 lanes (DPP only); every lane of the row receives the row's total.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    return v;
 }
 
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {

@@ -34,6 +34,11 @@ int check_hip(hipError_t e, const char *what) {
 
 int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out) {
     if (bytes > dev->workspace_bytes) {
+        if (dev->capturing) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
+                             "workspace of %zu bytes is needed but the stream is being captured; run the call once "
+                             "eagerly before capturing", bytes);
+        }
         // round up so that a sequence of growing requests does not reallocate every time
         size_t want = dev->workspace_bytes ? dev->workspace_bytes : (size_t)1 << 20;
         while (want < bytes) {
@@ -82,6 +87,7 @@ using namespace mh;
 extern "C" {
 
 int marmot_hip_fill_bytes_internal(marmot_hip_device_t *dev, void *d_dst, int value, size_t size);
+int marmot_hip_copy16_internal(marmot_hip_device_t *dev, void *d_dst, const void *d_src, size_t size);
 
 const char *marmot_hip_last_error(void) {
     return g_error;
@@ -230,6 +236,9 @@ int marmot_hip_memcpy_device(marmot_hip_device_t *dev, void *d_dst, const void *
     if (size == 0) {
         return MARMOT_HIP_SUCCESS;
     }
+    if (size % 16 == 0 && ((((uintptr_t)d_dst) | ((uintptr_t)d_src)) & 15) == 0) {
+        return marmot_hip_copy16_internal(dev, d_dst, d_src, size);  // a kernel: capturable, on this stream
+    }
     MH_HIP(hipMemcpyAsync(d_dst, d_src, size, hipMemcpyDeviceToDevice, dev->stream));
     return MARMOT_HIP_SUCCESS;
 }
@@ -294,6 +303,52 @@ int marmot_hip_get_caps(marmot_hip_device_t *dev, marmot_hip_caps_t *caps) {
     caps->peak_tflops_fp16 = 2500.0f;
     caps->peak_tops_int8 = 5000.0f;
     return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "graph_begin_capture: null device");
+    }
+    if (dev->capturing) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "graph_begin_capture: a capture is already active");
+    }
+    MH_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
+    dev->capturing = true;
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_graph_end_capture(marmot_hip_device_t *dev, void **out_graph_exec) {
+    if (dev == nullptr || out_graph_exec == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "graph_end_capture: null argument");
+    }
+    *out_graph_exec = nullptr;
+    if (!dev->capturing) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "graph_end_capture: no capture is active");
+    }
+    dev->capturing = false;
+    hipGraph_t graph = nullptr;
+    MH_HIP(hipStreamEndCapture(dev->stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    MH_HIP(e);
+    *out_graph_exec = (void *)exec;
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_graph_launch(marmot_hip_device_t *dev, void *graph_exec) {
+    if (dev == nullptr || graph_exec == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "graph_launch: null argument");
+    }
+    MH_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, dev->stream));
+    return MARMOT_HIP_SUCCESS;
+}
+
+void marmot_hip_graph_destroy(marmot_hip_device_t *dev, void *graph_exec) {
+    (void)dev;
+    if (graph_exec != nullptr) {
+        (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+    }
 }
 
 int marmot_hip_event_create(marmot_hip_device_t *dev, void **out_event) {

@@ -205,7 +205,12 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
         }
         return MARMOT_HIP_SUCCESS;
     }
-    // packed route: quantize the activations once (shared by both weights of a dual call), then integer dots
+    // packed route. fp32 activations whose rows are whole blocks are quantized inside the matvec kernel; otherwise
+    // the activations are quantized once into the workspace (shared by both weights of a dual call).
+    if (in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input)) {
+        return launch_matvec_packed(dev, kind, d_w0, d_w1, nullptr, (const float *)d_input, N, K, M, d_bias,
+                                    bias_dtype, d_out0, d_out1, out_dtype);
+    }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t need = act_scratch_layout(act_kind, N, K, nullptr, nullptr);
     void *ws = nullptr;
@@ -219,7 +224,8 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
-    return launch_matvec_packed(dev, kind, d_w0, d_w1, act, N, K, M, d_bias, bias_dtype, d_out0, d_out1, out_dtype);
+    return launch_matvec_packed(dev, kind, d_w0, d_w1, &act, nullptr, N, K, M, d_bias, bias_dtype, d_out0, d_out1,
+                                out_dtype);
 }
 
 } // namespace mh
@@ -237,6 +243,59 @@ int marmot_hip_matmul_quantized(marmot_hip_device_t *dev, int kind, const void *
     }
     return matmul_impl(dev, kind, d_weight, nullptr, d_input, in_dtype, N, K, M, d_bias, bias_dtype, d_out, nullptr,
                        out_dtype, flags);
+}
+
+size_t marmot_hip_packed_activation_bytes(int weight_kind, size_t N, size_t K) {
+    if (block_values(weight_kind) == 0 || weight_kind == MARMOT_HIP_KIND_Q8_K) {
+        return 0;
+    }
+    const int act_kind = is_k_quant(weight_kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+    return act_scratch_layout(act_kind, N, K, nullptr, nullptr);
+}
+
+int marmot_hip_pack_activations(marmot_hip_device_t *dev, int weight_kind, const void *d_input, int in_dtype,
+                                size_t N, size_t K, void *d_packed) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
+    }
+    if (d_input == nullptr || d_packed == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
+    }
+    if (marmot_hip_packed_activation_bytes(weight_kind, 1, 1) == 0) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "pack_activations: unsupported quant kind %d", weight_kind);
+    }
+    if (in_dtype != MARMOT_HIP_DTYPE_F32 && in_dtype != MARMOT_HIP_DTYPE_F16) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "pack_activations: input dtype %d", in_dtype);
+    }
+    if ((((uintptr_t)d_packed) & 255) != 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "pack_activations: d_packed must be 256-byte aligned");
+    }
+    const int act_kind = is_k_quant(weight_kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+    ActScratch act;
+    act_scratch_layout(act_kind, N, K, d_packed, &act);
+    return launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
+}
+
+int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_packed,
+                                size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out,
+                                int out_dtype) {
+    // the packed route accepts what a forced-pack call would: any float input dtype has already been consumed
+    int st = validate_matmul(dev, kind, d_weight, d_packed, MARMOT_HIP_DTYPE_F16, N, K, M, d_bias, bias_dtype, d_out,
+                             out_dtype);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    if ((((uintptr_t)d_packed) & 255) != 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "matmul_prepacked: d_packed must be 256-byte aligned");
+    }
+    if (N == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+    ActScratch act;
+    act_scratch_layout(act_kind, N, K, const_cast<void *>(d_packed), &act);
+    return launch_matvec_packed(dev, kind, d_weight, nullptr, &act, nullptr, N, K, M, d_bias, bias_dtype, d_out,
+                                nullptr, out_dtype);
 }
 
 int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const void *d_weight_a,

@@ -11,9 +11,15 @@
 //     of an iteration are issued before any is consumed, which is what keeps HBM busy.
 //   * Per row and column the lanes' fp32 partial sums are reduced with DPP; with W > 1 the per-wavefront sums
 //     meet in LDS once, after the last row.
+//   * For fp32 activations the Q8_K / Q8_0 quantization of the activations is fused into the kernel prologue:
+//     the lanes that share a block (8 / 4 / 1 lanes) quantize exactly their own values, with the same arithmetic
+//     as the standalone quantizer kernels, so no separate launch and no scratch round trip is needed.
 // Integer sub-block dots use v_dot4c_i32_i8; the fp32 scale-accumulate matches
 // cpu_vec_dot_{q4_k,q6_k}_q8_k / cpu_vec_dot_{q8_0,q4_0}_q8_0 (vec_dot_impl.h) up to summation order.
 #include "mh_common.h"
+
+#include <float.h>
+#include <stdlib.h>
 
 namespace mh {
 
@@ -54,13 +60,120 @@ __device__ __forceinline__ int dot16(const uint4 &w, const uint4 &a, int acc) {
     return acc;
 }
 
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) | ((uint32_t)(d & 0xff) << 24);
+}
+
+// 16 consecutive fp32 activations (64-byte aligned when K is a multiple of 16)
+__device__ __forceinline__ void ld16f(const float *p, float *v) {
+    const float4 a = ((const float4 *)p)[0], b = ((const float4 *)p)[1], c = ((const float4 *)p)[2],
+                 d = ((const float4 *)p)[3];
+    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w;
+    v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+    v[8] = c.x, v[9] = c.y, v[10] = c.z, v[11] = c.w;
+    v[12] = d.x, v[13] = d.y, v[14] = d.z, v[15] = d.w;
+}
+
+// Q8_K quantization (matmul_quant_pack.c:106-142) of one 256-value block whose values are spread over LPB
+// adjacent lanes: this lane owns RUNS runs of 16 consecutive values starting at block offsets off[r].
+// Produces this lane's int8 values (RUNS uint4), the sums of each run (= bsums entries) and the block scale d.
+template <int RUNS, int LPB>
+__device__ __forceinline__ void q8k_quantize_runs(const float *xblk, const int (&off)[RUNS], uint4 (&q)[RUNS],
+                                                  int (&bs)[RUNS], float &d) {
+    float v[RUNS][16];
+#pragma unroll
+    for (int r = 0; r < RUNS; ++r) {
+        ld16f(xblk + off[r], v[r]);
+    }
+    float best_abs = 0.0f, best_val = 0.0f;
+    int best_idx = 0x7fffffff;
+#pragma unroll
+    for (int r = 0; r < RUNS; ++r) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float ax = fabsf(v[r][i]);
+            const bool gt = ax > best_abs;  // runs are visited in increasing offset order: first occurrence wins
+            best_abs = gt ? ax : best_abs;
+            best_val = gt ? v[r][i] : best_val;
+            best_idx = gt ? off[r] + i : best_idx;
+        }
+    }
+#pragma unroll
+    for (int o = 1; o < LPB; o <<= 1) {
+        const float o_abs = __shfl_xor(best_abs, o);
+        const float o_val = __shfl_xor(best_val, o);
+        const int o_idx = __shfl_xor(best_idx, o);
+        const bool take = o_abs > best_abs || (o_abs == best_abs && o_idx < best_idx);
+        best_abs = take ? o_abs : best_abs;
+        best_val = take ? o_val : best_val;
+        best_idx = take ? o_idx : best_idx;
+    }
+    d = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RUNS; ++r) {
+        q[r] = make_uint4(0, 0, 0, 0);
+        bs[r] = 0;
+    }
+    if (best_abs > 0.0f) {
+        const float iscale = -127.0f / best_val;
+#pragma unroll
+        for (int r = 0; r < RUNS; ++r) {
+            int t[16];
+            int s = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int z = nearest_int_clamped(iscale * v[r][i]);
+                t[i] = z > 127 ? 127 : z;
+                s += t[i];
+            }
+            q[r].x = pack4(t[0], t[1], t[2], t[3]);
+            q[r].y = pack4(t[4], t[5], t[6], t[7]);
+            q[r].z = pack4(t[8], t[9], t[10], t[11]);
+            q[r].w = pack4(t[12], t[13], t[14], t[15]);
+            bs[r] = s;
+        }
+        d = 1.0f / iscale;
+    }
+}
+
+// Q8_0 quantization (matmul_quant_pack.c:23-62, scalar rounding) of one 32-value block owned by this lane.
+__device__ __forceinline__ void q80_quantize_block(const float *xblk, uint4 &q0, uint4 &q1, float &d, int &sum) {
+    float v[32];
+    ld16f(xblk, v);
+    ld16f(xblk + 16, v + 16);
+    float max_abs = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        max_abs = fmaxf(max_abs, fabsf(v[i]));
+    }
+    float scale = max_abs / 127.0f;
+    if (scale < FLT_MIN) {
+        scale = 1.0f;
+    }
+    const float inv = 1.0f / scale;
+    int t[32];
+    sum = 0;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        int z = (int)roundf(v[i] * inv);
+        z = z < -127 ? -127 : (z > 127 ? 127 : z);
+        t[i] = z;
+        sum += z;
+    }
+    q0 = make_uint4(pack4(t[0], t[1], t[2], t[3]), pack4(t[4], t[5], t[6], t[7]), pack4(t[8], t[9], t[10], t[11]),
+                    pack4(t[12], t[13], t[14], t[15]));
+    q1 = make_uint4(pack4(t[16], t[17], t[18], t[19]), pack4(t[20], t[21], t[22], t[23]),
+                    pack4(t[24], t[25], t[26], t[27]), pack4(t[28], t[29], t[30], t[31]));
+    d = h2f(f2h(scale));
+}
+
 // ------------------------------------------------------------------ Q4_K x Q8_K
 struct FmtQ4K {
     static constexpr int BYTES = Q4_K_BYTES;
     static constexpr int LPB = 8;  // lanes per block
     static constexpr int BPW = 8;  // blocks per wave-load
     static constexpr int BV = QK_K;
-    static constexpr int ACT_DW = 11, WT_DW = 8;  // registers per lane (activation share, one row's loads)
+    static constexpr int ACT_DW = 11, WT_DW = 8, QUANT_TMP = 56;  // registers per lane (estimates)
     struct Act {
         uint4 lo, hi;  // int8 activations under the low / high nibbles of this lane's 16 bytes
         float d;
@@ -80,6 +193,17 @@ struct FmtQ4K {
         a.bs_lo = bs[4 * g + h];
         a.bs_hi = bs[4 * g + 2 + h];
     }
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
+        const int g = sub >> 1, h = sub & 1;
+        const int off[2] = {64 * g + 16 * h, 64 * g + 32 + 16 * h};
+        uint4 q[2];
+        int bs[2];
+        q8k_quantize_runs<2, 8>(xrow + blk * QK_K, off, q, bs, a.d);
+        a.lo = q[0];
+        a.hi = q[1];
+        a.bs_lo = bs[0];
+        a.bs_hi = bs[1];
+    }
     __device__ static void zero_act(Act &a) {
         a.lo = a.hi = make_uint4(0, 0, 0, 0);
         a.d = 0.0f;
@@ -91,24 +215,29 @@ struct FmtQ4K {
     }
     template <int NC>
     __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int sub) {
+#ifdef MH_PROBE_NOALU
+        for (int n = 0; n < NC; ++n) {
+            acc[n] += __int_as_float((w.q.x ^ w.q.y ^ w.q.z ^ w.q.w ^ w.hdr.x ^ w.hdr.w) & 0x007fffff) * a[n].d;
+        }
+        return;
+#endif
         const int g = sub >> 1;
         const float d = h2f((uint16_t)(w.hdr.x & 0xffffu));
         const float dmin = h2f((uint16_t)(w.hdr.x >> 16));
-        // 6-bit scale / min pairs of sub-blocks 2g and 2g+1 (get_scale_min_k4, kquant_common.h:29-37)
+        // 6-bit scale / min pairs of sub-blocks 2g and 2g+1 (get_scale_min_k4, kquant_common.h:29-37), without
+        // branches: for g < 2 the pair is (s[j] & 63, s[j+4] & 63); for g >= 2 the low nibbles come from s[j+4]
+        // and the two high bits from s[j-4] / s[j]. All selectors below are per-lane constants.
         const int sh = 16 * (g & 1);
-        const uint32_t sa = (w.hdr.y >> sh) & 0xffffu;
-        const uint32_t sb = (w.hdr.z >> sh) & 0xffffu;
-        const uint32_t sc_ = (w.hdr.w >> sh) & 0xffffu;
-        uint32_t scp, mp;
-        if (g < 2) {
-            scp = sa & 0x3f3fu;
-            mp = sb & 0x3f3fu;
-        } else {
-            scp = (sc_ & 0x0f0fu) | ((sa >> 2) & 0x3030u);
-            mp = ((sc_ >> 4) & 0x0f0fu) | ((sb >> 2) & 0x3030u);
-        }
-        const int sc0 = (int)(scp & 0xffu), sc1 = (int)(scp >> 8);
-        const int m0 = (int)(mp & 0xffu), m1 = (int)(mp >> 8);
+        const uint32_t sa = w.hdr.y >> sh;
+        const uint32_t sb = w.hdr.z >> sh;
+        const uint32_t sc_ = w.hdr.w >> sh;
+        const bool hi_grp = g >= 2;
+        const uint32_t m_lo = hi_grp ? 0x0f0fu : 0x3f3fu;
+        const uint32_t m_hi = hi_grp ? 0x3030u : 0u;
+        const uint32_t scp = ((hi_grp ? sc_ : sa) & m_lo) | ((sa >> 2) & m_hi);
+        const uint32_t mp = ((hi_grp ? (sc_ >> 4) : sb) & m_lo) | ((sb >> 2) & m_hi);
+        const int sc0 = (int)(scp & 0xffu), sc1 = (int)((scp >> 8) & 0xffu);
+        const int m0 = (int)(mp & 0xffu), m1 = (int)((mp >> 8) & 0xffu);
         uint4 lo, hi;
         lo.x = w.q.x & 0x0f0f0f0fu;
         lo.y = w.q.y & 0x0f0f0f0fu;
@@ -122,8 +251,8 @@ struct FmtQ4K {
         for (int n = 0; n < NC; ++n) {
             const int dl = dot16(lo, a[n].lo, 0);
             const int dh = dot16(hi, a[n].hi, 0);
-            const int isum = sc0 * dl + sc1 * dh;
-            const int msum = m0 * a[n].bs_lo + m1 * a[n].bs_hi;
+            const int isum = __mul24(sc0, dl) + __mul24(sc1, dh);
+            const int msum = __mul24(m0, a[n].bs_lo) + __mul24(m1, a[n].bs_hi);
             acc[n] += (a[n].d * d) * (float)isum - (a[n].d * dmin) * (float)msum;
         }
     }
@@ -135,7 +264,7 @@ struct FmtQ6K {
     static constexpr int LPB = 4;
     static constexpr int BPW = 16;
     static constexpr int BV = QK_K;
-    static constexpr int ACT_DW = 21, WT_DW = 15;
+    static constexpr int ACT_DW = 21, WT_DW = 15, QUANT_TMP = 100;
     struct Act {
         uint4 a[4];  // 16 int8 each, under q1..q4 of this lane's 16 positions
         float d;
@@ -156,6 +285,12 @@ struct FmtQ6K {
             a.bs[j] = bs[2 * j];
         }
         a.d = av.d[n * av.nb + blk];
+    }
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
+        const int hh = sub >> 1, t = sub & 1;
+        const int base = 128 * hh + 16 * t;
+        const int off[4] = {base, base + 32, base + 64, base + 96};
+        q8k_quantize_runs<4, 4>(xrow + blk * QK_K, off, a.a, a.bs, a.d);
     }
     __device__ static void zero_act(Act &a) {
 #pragma unroll
@@ -203,7 +338,7 @@ struct FmtQ6K {
             const int d2 = dot16(q2, a[n].a[1], 0) - 32 * a[n].bs[1];
             const int d3 = dot16(q3, a[n].a[2], 0) - 32 * a[n].bs[2];
             const int d4 = dot16(q4, a[n].a[3], 0) - 32 * a[n].bs[3];
-            const int isum = sc0 * d1 + sc1 * d2 + sc2 * d3 + sc3 * d4;
+            const int isum = __mul24(sc0, d1) + __mul24(sc1, d2) + __mul24(sc2, d3) + __mul24(sc3, d4);
             acc[n] += (a[n].d * d) * (float)isum;
         }
     }
@@ -215,7 +350,7 @@ struct FmtQ80 {
     static constexpr int LPB = 1;
     static constexpr int BPW = 64;
     static constexpr int BV = QK;
-    static constexpr int ACT_DW = 9, WT_DW = 9;
+    static constexpr int ACT_DW = 9, WT_DW = 9, QUANT_TMP = 80;
     struct Act {
         uint4 a0, a1;
         float d;
@@ -229,6 +364,10 @@ struct FmtQ80 {
         a.a0 = *(const uint4 *)base;
         a.a1 = *(const uint4 *)(base + 16);
         a.d = av.d[n * av.nb + blk];
+    }
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int) {
+        int sum;
+        q80_quantize_block(xrow + blk * QK, a.a0, a.a1, a.d, sum);
     }
     __device__ static void zero_act(Act &a) {
         a.a0 = a.a1 = make_uint4(0, 0, 0, 0);
@@ -257,7 +396,7 @@ struct FmtQ40 {
     static constexpr int LPB = 1;
     static constexpr int BPW = 64;
     static constexpr int BV = QK;
-    static constexpr int ACT_DW = 10, WT_DW = 5;
+    static constexpr int ACT_DW = 10, WT_DW = 5, QUANT_TMP = 80;
     struct Act {
         uint4 a0, a1;
         float d;
@@ -273,6 +412,9 @@ struct FmtQ40 {
         a.a1 = *(const uint4 *)(base + 16);
         a.d = av.d[n * av.nb + blk];
         a.sum = av.sums[n * av.nb + blk];
+    }
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int) {
+        q80_quantize_block(xrow + blk * QK, a.a0, a.a1, a.d, a.sum);
     }
     __device__ static void zero_act(Act &a) {
         a.a0 = a.a1 = make_uint4(0, 0, 0, 0);
@@ -308,11 +450,13 @@ struct FmtQ40 {
 struct MatvecParams {
     const uint8_t *w[2];
     void *out[2];
-    ActView act;
+    ActView act;       // packed activations (prepacked variant)
+    const float *x;    // fp32 activations [N][K] (fused variant)
+    size_t K;
     const void *bias;
     int bias_is_f16;
     int out_is_f16;
-    size_t n0;         // first activation row (column tile offset)
+    size_t n0;         // first activation row of this column tile
     size_t M;
     size_t nb;         // blocks per weight row
     size_t row_bytes;
@@ -339,21 +483,24 @@ __device__ __forceinline__ void store_out(const MatvecParams &p, void *out, size
 
 // Largest workgroup a configuration may use: the register estimate decides how many wavefronts fit per SIMD
 // (512 VGPRs per lane per SIMD on gfx950) without spilling.
-template <class Fmt, int NC, int C, int R>
+template <class Fmt, int NC, int C, int R, bool FUSED>
 constexpr int matvec_max_threads() {
-    constexpr int need = NC * C * Fmt::ACT_DW + R * C * Fmt::WT_DW + 2 * NC + 36;
+    constexpr int loop_need = NC * C * Fmt::ACT_DW + 2 * R * C * Fmt::WT_DW + 2 * NC + 36;
+    constexpr int prologue_need = NC * C * Fmt::ACT_DW + (FUSED ? Fmt::QUANT_TMP : 0) + 24;
+    constexpr int need = loop_need > prologue_need ? loop_need : prologue_need;
     return need <= 120 ? 1024 : (need <= 240 ? 512 : 256);
 }
 
-template <class Fmt, int NC, int C, int R>
-__global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R>())) void k_matvec(const MatvecParams p) {
-    extern __shared__ float partial[];  // [rows_per_wg][NC][W]
+// FUSED: quantize fp32 activations in the prologue instead of reading packed ones.
+// EXACT: every lane owns a real block in every slot and M is a multiple of rows_per_wg (no masking in the loop).
+template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
+__global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void k_matvec(const MatvecParams p) {
+    extern __shared__ float partial[];  // [rows_per_wg][NC][4 * W]: one partial per 16-lane row of each wavefront
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
     const int sub = lane % Fmt::LPB;
     const uint8_t *__restrict__ wbase = p.w[blockIdx.y];
-    void *out = p.out[blockIdx.y];
 
     typename Fmt::Act act[C][NC];
     size_t blk[C];
@@ -361,11 +508,15 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R>())) void k_matve
 #pragma unroll
     for (int i = 0; i < C; ++i) {
         blk[i] = (size_t)(wave * C + i) * Fmt::BPW + lane / Fmt::LPB;
-        valid[i] = blk[i] < p.nb;
+        valid[i] = EXACT || blk[i] < p.nb;
 #pragma unroll
         for (int n = 0; n < NC; ++n) {
             if (valid[i]) {
-                Fmt::load_act(act[i][n], p.act, p.n0 + n, blk[i], sub);
+                if constexpr (FUSED) {
+                    Fmt::quant_act(act[i][n], p.x + (p.n0 + n) * p.K, blk[i], sub);
+                } else {
+                    Fmt::load_act(act[i][n], p.act, p.n0 + n, blk[i], sub);
+                }
             } else {
                 Fmt::zero_act(act[i][n]);
             }
@@ -373,13 +524,18 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R>())) void k_matve
     }
 
     const size_t row0 = (size_t)blockIdx.x * p.rows_per_wg;
-    for (int r = 0; r < p.rows_per_wg; r += R) {
-        typename Fmt::Wt wt[R][C];
+    const int pslot = wave * 4 + (lane >> 4);
+    const int pstride = 4 * W;
+
+    // Two register buffers of R rows each: the loads of the next R rows are in flight while the current R rows
+    // are consumed, so a wavefront keeps requests outstanding for its whole lifetime.
+    typename Fmt::Wt wa[R][C], wb[R][C];
+    auto issue = [&](typename Fmt::Wt(&wt)[R][C], int r) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             size_t row = row0 + r + rr;
-            if (row >= p.M) {
-                row = p.M - 1;  // harmless re-read; the result is discarded below
+            if (!EXACT && row >= p.M) {
+                row = p.M - 1;  // harmless re-read; the result is discarded in the epilogue
             }
             const uint8_t *rowp = wbase + row * p.row_bytes;
 #pragma unroll
@@ -389,6 +545,8 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R>())) void k_matve
                 }
             }
         }
+    };
+    auto consume = [&](const typename Fmt::Wt(&wt)[R][C], int r) {
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) {
             float acc[NC];
@@ -402,56 +560,74 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R>())) void k_matve
                     Fmt::template accumulate<NC>(wt[rr][i], act[i], acc, sub);
                 }
             }
-            const size_t row = row0 + r + rr;
 #pragma unroll
             for (int n = 0; n < NC; ++n) {
-                const float s = wave_sum(acc[n]);
-                if (lane == 0) {
-                    if (W == 1) {
-                        if (row < p.M) {
-                            store_out(p, out, p.n0 + n, row, s);
-                        }
-                    } else {
-                        partial[((r + rr) * NC + n) * W + wave] = s;
-                    }
+                const float s = row16_sum(acc[n]);
+                if ((lane & 15) == 0) {
+                    partial[((r + rr) * NC + n) * pstride + pslot] = s;
                 }
             }
         }
+    };
+    const int rows = p.rows_per_wg;  // a multiple of R
+    issue(wa, 0);
+    for (int r = 0; r < rows; r += 2 * R) {
+        if (r + R < rows) {
+            issue(wb, r + R);
+        }
+        consume(wa, r);
+        if (r + 2 * R < rows) {
+            issue(wa, r + 2 * R);
+        }
+        if (r + R < rows) {
+            consume(wb, r + R);
+        }
     }
-    if (W > 1) {
-        __syncthreads();
-        for (int idx = threadIdx.x; idx < p.rows_per_wg * NC; idx += blockDim.x) {
-            const size_t row = row0 + idx / NC;
-            const int n = idx % NC;
-            if (row < p.M) {
-                float s = 0.0f;
-                for (int w = 0; w < W; ++w) {
-                    s += partial[idx * W + w];
-                }
-                store_out(p, out, p.n0 + n, row, s);
+    __syncthreads();
+    void *out = p.out[blockIdx.y];
+    for (int idx = threadIdx.x; idx < p.rows_per_wg * NC; idx += blockDim.x) {
+        const size_t row = row0 + idx / NC;
+        const int n = idx % NC;
+        if (EXACT || row < p.M) {
+            // W <= 16 float4 partials, all read before the first add so that only one LDS latency is exposed
+            const float4 *pv = (const float4 *)(partial + idx * pstride);
+            float4 v[16];
+#pragma unroll
+            for (int w = 0; w < 16; ++w) {
+                v[w] = pv[w < W ? w : 0];
             }
+            float s = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) {
+                const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
+                s += w < W ? t : 0.0f;
+            }
+            store_out(p, out, p.n0 + n, row, s);
         }
     }
 }
 
-template <class Fmt, int NC, int C, int R>
+template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
 static int launch_one(marmot_hip_device *dev, const MatvecParams &p, int W, size_t M, bool dual) {
     const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1);
-    const size_t lds = W > 1 ? (size_t)p.rows_per_wg * NC * W * sizeof(float) : 0;
-    hipLaunchKernelGGL((k_matvec<Fmt, NC, C, R>), grid, dim3(W * 64), lds, dev->stream, p);
+    const size_t lds = (size_t)p.rows_per_wg * NC * 4 * W * sizeof(float);
+    hipLaunchKernelGGL((k_matvec<Fmt, NC, C, R, FUSED, EXACT>), grid, dim3(W * 64), lds, dev->stream, p);
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
 }
 
 // Picks wavefronts per workgroup (W), wave-loads per wavefront (C) and rows per workgroup for one column tile.
 // Returns MARMOT_HIP_ERROR_NOT_IMPLEMENTED (without setting the error text) when K is too long for this NC.
-template <class Fmt, int NC>
-static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, bool dual, const char *name) {
-    constexpr int R = (NC <= 2) ? 4 : 2;
+template <class Fmt, int NC, int R>
+static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, bool dual, const char *name) {
     const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
     const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
-    constexpr size_t maxw1 = matvec_max_threads<Fmt, NC, 1, R>() / 64;
-    constexpr size_t maxw2 = matvec_max_threads<Fmt, NC, 2, R>() / 64;
+    const bool fused = p.x != nullptr;
+    constexpr bool can_fuse = NC <= 4;
+    const size_t maxw1 = (fused ? matvec_max_threads<Fmt, NC, 1, R, can_fuse>()
+                                : matvec_max_threads<Fmt, NC, 1, R, false>()) / 64;
+    const size_t maxw2 = (fused ? matvec_max_threads<Fmt, NC, 2, R, can_fuse>()
+                                : matvec_max_threads<Fmt, NC, 2, R, false>()) / 64;
     int C;
     if (wave_loads <= maxw1) {
         C = 1;
@@ -461,7 +637,8 @@ static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t 
         return MARMOT_HIP_ERROR_NOT_IMPLEMENTED;
     }
     const int W = (int)((wave_loads + C - 1) / C);
-    // Aim for about 16 resident wavefronts per CU; every workgroup re-reads the (small) activation set once.
+    // Rows per workgroup: enough workgroups to fill the chip several times over (the hardware hides latency by
+    // switching between resident workgroups), but enough rows that the activation prologue is amortized.
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     size_t wgs_per_cu = 16 / (size_t)W;
     if (wgs_per_cu < 1) {
@@ -471,6 +648,9 @@ static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t 
         wgs_per_cu = 8;
     }
     size_t rows_per_wg = (M + cus * wgs_per_cu - 1) / (cus * wgs_per_cu);
+    if (fused && rows_per_wg < 8) {
+        rows_per_wg = 8;
+    }
     rows_per_wg = ((rows_per_wg + R - 1) / R) * R;
     if (rows_per_wg < (size_t)R) {
         rows_per_wg = R;
@@ -478,12 +658,45 @@ static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t 
     if (rows_per_wg > 32) {
         rows_per_wg = 32;
     }
+    if (const char *e = getenv("MH_RPW")) {
+        rows_per_wg = (size_t)atoi(e);
+        rows_per_wg = ((rows_per_wg + R - 1) / R) * R;
+    }
     p.rows_per_wg = (int)rows_per_wg;
     set_route(name);
-    if (C == 1) {
-        return launch_one<Fmt, NC, 1, R>(dev, p, W, M, dual);
+    const bool exact = (size_t)W * C * Fmt::BPW == nb && K % Fmt::BV == 0 && M % rows_per_wg == 0;
+    if constexpr (NC <= 4) {
+        if (fused) {
+            if (C == 1) {
+                return exact ? launch_one<Fmt, NC, 1, R, true, true>(dev, p, W, M, dual)
+                             : launch_one<Fmt, NC, 1, R, true, false>(dev, p, W, M, dual);
+            }
+            return launch_one<Fmt, NC, 2, R, true, false>(dev, p, W, M, dual);
+        }
+    } else if (fused) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "fused activation quantization is limited to 4 columns");
     }
-    return launch_one<Fmt, NC, 2, R>(dev, p, W, M, dual);
+    if (C == 1) {
+        return launch_one<Fmt, NC, 1, R, false, false>(dev, p, W, M, dual);
+    }
+    return launch_one<Fmt, NC, 2, R, false, false>(dev, p, W, M, dual);
+}
+
+template <class Fmt, int NC>
+static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, bool dual, const char *name) {
+    if constexpr (NC == 1) {
+        const char *e = getenv("MH_R");
+        const int r = e ? atoi(e) : 4;
+        if (r == 8) {
+            return launch_tile_r<Fmt, NC, 8>(dev, p, K, M, dual, name);
+        }
+        if (r == 2) {
+            return launch_tile_r<Fmt, NC, 2>(dev, p, K, M, dual, name);
+        }
+        return launch_tile_r<Fmt, NC, 4>(dev, p, K, M, dual, name);
+    } else {
+        return launch_tile_r < Fmt, NC, (NC <= 2) ? 4 : 2 > (dev, p, K, M, dual, name);
+    }
 }
 
 template <class Fmt>
@@ -535,40 +748,59 @@ static int launch_fmt(marmot_hip_device *dev, MatvecParams p, size_t N, size_t K
     return MARMOT_HIP_SUCCESS;
 }
 
-int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act,
-                         size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1,
-                         int out_dtype) {
+bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_f32) {
+    const size_t bv = block_values(kind);
+    return N <= 4 && bv != 0 && K % bv == 0 && (((uintptr_t)d_x_f32) & 15) == 0 && getenv("MARMOT_HIP_NO_FUSED_QUANT") == nullptr;
+}
+
+int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
+                         const float *d_x_f32, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
+                         void *d_out0, void *d_out1, int out_dtype) {
     if (N == 0 || M == 0 || K == 0) {
         return MARMOT_HIP_SUCCESS;
     }
+    const size_t bv = block_values(kind);
+    const size_t nb = (K + bv - 1) / bv;
     MatvecParams p;
     p.w[0] = (const uint8_t *)d_w0;
     p.w[1] = (const uint8_t *)(d_w1 != nullptr ? d_w1 : d_w0);
     p.out[0] = d_out0;
     p.out[1] = d_out1 != nullptr ? d_out1 : d_out0;
-    p.act.qs = act.qs;
-    p.act.d = act.d;
-    p.act.sums = act.sums;
-    p.act.kp = act.kp;
-    p.act.nb = act.nb;
+    if (act != nullptr) {
+        p.act.qs = act->qs;
+        p.act.d = act->d;
+        p.act.sums = act->sums;
+        p.act.kp = act->kp;
+        p.act.nb = act->nb;
+        p.x = nullptr;
+    } else {
+        p.act.qs = nullptr;
+        p.act.d = nullptr;
+        p.act.sums = nullptr;
+        p.act.kp = 0;
+        p.act.nb = nb;
+        p.x = d_x_f32;
+    }
+    p.K = K;
     p.bias = d_bias;
     p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
     p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
     p.n0 = 0;
     p.M = M;
-    p.nb = act.nb;
-    p.row_bytes = act.nb * block_bytes(kind);
+    p.nb = nb;
+    p.row_bytes = nb * block_bytes(kind);
     p.rows_per_wg = 4;
     const bool dual = d_w1 != nullptr;
+    const bool fused = act == nullptr;
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
-        return launch_fmt<FmtQ4K>(dev, p, N, K, M, dual, "matvec_q4_k_q8_k");
+        return launch_fmt<FmtQ4K>(dev, p, N, K, M, dual, fused ? "matvec_q4_k_q8_k_fused" : "matvec_q4_k_q8_k");
     case MARMOT_HIP_KIND_Q6_K:
-        return launch_fmt<FmtQ6K>(dev, p, N, K, M, dual, "matvec_q6_k_q8_k");
+        return launch_fmt<FmtQ6K>(dev, p, N, K, M, dual, fused ? "matvec_q6_k_q8_k_fused" : "matvec_q6_k_q8_k");
     case MARMOT_HIP_KIND_Q8_0:
-        return launch_fmt<FmtQ80>(dev, p, N, K, M, dual, "matvec_q8_0_q8_0");
+        return launch_fmt<FmtQ80>(dev, p, N, K, M, dual, fused ? "matvec_q8_0_q8_0_fused" : "matvec_q8_0_q8_0");
     case MARMOT_HIP_KIND_Q4_0:
-        return launch_fmt<FmtQ40>(dev, p, N, K, M, dual, "matvec_q4_0_q8_0");
+        return launch_fmt<FmtQ40>(dev, p, N, K, M, dual, fused ? "matvec_q4_0_q8_0_fused" : "matvec_q4_0_q8_0");
     default:
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "quantized matmul: unsupported quant kind %d", kind);
     }

@@ -40,18 +40,6 @@ __global__ __launch_bounds__(256) void k_dequantize(const uint8_t *__restrict__ 
 // Activation quantizers
 // ------------------------------------------------------------------------------------------------
 
-// magic-number round-to-nearest-even with the input clamp of matmul_quant_pack.c:11-21
-__device__ __forceinline__ int nearest_int_clamped(float value) {
-    if (value > 4194303.0f) {
-        value = 4194303.0f;
-    } else if (value < -4194303.0f) {
-        value = -4194303.0f;
-    }
-    const float shifted = value + 12582912.0f;
-    const int bits = __float_as_int(shifted);
-    return (bits & 0x007fffff) - 0x00400000;
-}
-
 template <bool F16>
 __device__ __forceinline__ float load_act_value(const void *x, size_t i) {
     if constexpr (F16) {
@@ -193,6 +181,14 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ 
     }
 }
 
+// Plain 16-byte copy: device-to-device copies of the library, and the known-traffic kernel that profiler
+// counters (FETCH_SIZE / WRITE_SIZE) are calibrated against.
+__global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) {
+        dst[i] = src[i];
+    }
+}
+
 __global__ void k_fill_bytes(uint8_t *dst, uint8_t value, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
         dst[i] = value;
@@ -243,6 +239,18 @@ int launch_quantize_act_soa(marmot_hip_device *dev, int act_kind, const void *d_
 using namespace mh;
 
 extern "C" {
+
+int marmot_hip_copy16_internal(marmot_hip_device_t *dev, void *d_dst, const void *d_src, size_t size) {
+    const size_t n16 = size / 16;
+    size_t grid = (n16 + 255) / 256;
+    if (grid > (size_t)1 << 20) {
+        grid = (size_t)1 << 20;
+    }
+    hipLaunchKernelGGL(k_copy16, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint4 *)d_src, (uint4 *)d_dst,
+                       n16);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
 
 int marmot_hip_fill_bytes_internal(marmot_hip_device_t *dev, void *d_dst, int value, size_t size) {
     const unsigned grid = (unsigned)((size + 256 * 16 - 1) / (256 * 16));

@@ -149,6 +149,12 @@ bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_
 int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
                          const float *d_x_f32, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
                          void *d_out0, void *d_out1, int out_dtype);
+// quantizes act(gate) * up (SwiGLU or GeGLU) of two fp32 [rows, k] arrays into the activation scratch
+int launch_quantize_glu_soa(marmot_hip_device *dev, int act_kind, const float *d_gate, const float *d_up, bool geglu,
+                            size_t rows, size_t k, const ActScratch &dst);
+int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
+                          const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
+                          size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1);
 int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M);

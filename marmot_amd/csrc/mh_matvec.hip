@@ -461,6 +461,11 @@ struct MatvecParams {
     size_t nb;         // blocks per weight row
     size_t row_bytes;
     int rows_per_wg;
+    // grouped (MoE) mode: blockIdx.z selects a work item = up to NC consecutive routes of one expert
+    const int4 *items;            // (expert, first route, route count, -) or nullptr
+    const int *n_items;           // number of valid items (device memory)
+    const uint32_t *act_index;    // packed-activation row of each route (token id), or nullptr = identity
+    size_t expert_stride;         // bytes between the experts' weight slices
 };
 
 __device__ __forceinline__ void store_out(const MatvecParams &p, void *out, size_t n, size_t row, float v) {
@@ -501,6 +506,17 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
     const int W = blockDim.x >> 6;
     const int sub = lane % Fmt::LPB;
     const uint8_t *__restrict__ wbase = p.w[blockIdx.y];
+    size_t n0 = p.n0;
+    int ncols = NC;
+    if (!FUSED && p.items != nullptr) {
+        if ((int)blockIdx.z >= *p.n_items) {
+            return;  // uniform for the whole workgroup
+        }
+        const int4 it = p.items[blockIdx.z];
+        wbase += (size_t)it.x * p.expert_stride;
+        n0 = (size_t)it.y;
+        ncols = it.z;
+    }
 
     typename Fmt::Act act[C][NC];
     size_t blk[C];
@@ -511,11 +527,12 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
         valid[i] = EXACT || blk[i] < p.nb;
 #pragma unroll
         for (int n = 0; n < NC; ++n) {
-            if (valid[i]) {
+            if (valid[i] && n < ncols) {
                 if constexpr (FUSED) {
-                    Fmt::quant_act(act[i][n], p.x + (p.n0 + n) * p.K, blk[i], sub);
+                    Fmt::quant_act(act[i][n], p.x + (n0 + n) * p.K, blk[i], sub);
                 } else {
-                    Fmt::load_act(act[i][n], p.act, p.n0 + n, blk[i], sub);
+                    const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + n] : n0 + n;
+                    Fmt::load_act(act[i][n], p.act, arow, blk[i], sub);
                 }
             } else {
                 Fmt::zero_act(act[i][n]);
@@ -588,7 +605,7 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
     for (int idx = threadIdx.x; idx < p.rows_per_wg * NC; idx += blockDim.x) {
         const size_t row = row0 + idx / NC;
         const int n = idx % NC;
-        if (EXACT || row < p.M) {
+        if ((EXACT || row < p.M) && n < ncols) {
             // W <= 16 float4 partials, all read before the first add so that only one LDS latency is exposed
             const float4 *pv = (const float4 *)(partial + idx * pstride);
             float4 v[16];
@@ -602,14 +619,15 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
                 const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
                 s += w < W ? t : 0.0f;
             }
-            store_out(p, out, p.n0 + n, row, s);
+            store_out(p, out, n0 + n, row, s);
         }
     }
 }
 
 template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
 static int launch_one(marmot_hip_device *dev, const MatvecParams &p, int W, size_t M, bool dual) {
-    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1);
+    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1,
+                    p.items != nullptr ? (unsigned)p.n0 : 1u);  // grouped mode: n0 carries the item-count bound
     const size_t lds = (size_t)p.rows_per_wg * NC * 4 * W * sizeof(float);
     hipLaunchKernelGGL((k_matvec<Fmt, NC, C, R, FUSED, EXACT>), grid, dim3(W * 64), lds, dev->stream, p);
     MH_HIP(hipGetLastError());
@@ -648,6 +666,9 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
         wgs_per_cu = 8;
     }
     size_t rows_per_wg = (M + cus * wgs_per_cu - 1) / (cus * wgs_per_cu);
+    if (p.items != nullptr) {
+        rows_per_wg = 8;  // grouped mode: the item dimension supplies the parallelism
+    }
     if (fused && rows_per_wg < 8) {
         rows_per_wg = 8;
     }
@@ -790,6 +811,10 @@ int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, con
     p.nb = nb;
     p.row_bytes = nb * block_bytes(kind);
     p.rows_per_wg = 4;
+    p.items = nullptr;
+    p.n_items = nullptr;
+    p.act_index = nullptr;
+    p.expert_stride = 0;
     const bool dual = d_w1 != nullptr;
     const bool fused = act == nullptr;
     switch (kind) {
@@ -804,6 +829,63 @@ int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, con
     default:
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "quantized matmul: unsupported quant kind %d", kind);
     }
+}
+
+// Grouped (MoE) launch: one work item = up to 8 routes of one expert; see MatvecParams.
+int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
+                          const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
+                          size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1) {
+    if (max_items == 0 || M == 0 || K == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    const size_t bv = block_values(kind);
+    const size_t nb = (K + bv - 1) / bv;
+    MatvecParams p;
+    p.w[0] = (const uint8_t *)d_w0;
+    p.w[1] = (const uint8_t *)(d_w1 != nullptr ? d_w1 : d_w0);
+    p.out[0] = d_out0;
+    p.out[1] = d_out1 != nullptr ? d_out1 : d_out0;
+    p.act.qs = act.qs;
+    p.act.d = act.d;
+    p.act.sums = act.sums;
+    p.act.kp = act.kp;
+    p.act.nb = act.nb;
+    p.x = nullptr;
+    p.K = K;
+    p.bias = nullptr;
+    p.bias_is_f16 = 0;
+    p.out_is_f16 = 0;
+    p.n0 = max_items;
+    p.M = M;
+    p.nb = nb;
+    p.row_bytes = nb * block_bytes(kind);
+    p.rows_per_wg = 4;
+    p.items = d_items;
+    p.n_items = d_n_items;
+    p.act_index = d_act_index;
+    p.expert_stride = expert_stride;
+    const bool dual = d_w1 != nullptr;
+    int st;
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_K:
+        st = launch_tile<FmtQ4K, 8>(dev, p, K, M, dual, "moe_grouped_q4_k_q8_k");
+        break;
+    case MARMOT_HIP_KIND_Q6_K:
+        st = launch_tile<FmtQ6K, 8>(dev, p, K, M, dual, "moe_grouped_q6_k_q8_k");
+        break;
+    case MARMOT_HIP_KIND_Q8_0:
+        st = launch_tile<FmtQ80, 8>(dev, p, K, M, dual, "moe_grouped_q8_0_q8_0");
+        break;
+    case MARMOT_HIP_KIND_Q4_0:
+        st = launch_tile<FmtQ40, 8>(dev, p, K, M, dual, "moe_grouped_q4_0_q8_0");
+        break;
+    default:
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "MoE experts: unsupported quant kind %d", kind);
+    }
+    if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "MoE experts: K=%zu is beyond the single-pass limit", K);
+    }
+    return st;
 }
 
 } // namespace mh

@@ -40,10 +40,26 @@ __global__ __launch_bounds__(256) void k_dequantize(const uint8_t *__restrict__ 
 // Activation quantizers
 // ------------------------------------------------------------------------------------------------
 
-template <bool F16>
-__device__ __forceinline__ float load_act_value(const void *x, size_t i) {
-    if constexpr (F16) {
+// Where the values to quantize come from.
+enum ActSource {
+    SRC_F32 = 0,     // fp32 activations
+    SRC_F16 = 1,     // fp16 activations, widened exactly
+    SRC_SWIGLU = 2,  // silu(gate) * up of two fp32 arrays (MoE expert body, moe_ops.c:318-320, 552-556)
+    SRC_GEGLU = 3,   // gelu(gate) * up
+};
+
+template <int SRC>
+__device__ __forceinline__ float load_act_value(const void *x, const void *x2, size_t i) {
+    if constexpr (SRC == SRC_F16) {
         return h2f(((const uint16_t *)x)[i]);
+    } else if constexpr (SRC == SRC_SWIGLU) {
+        const float g = ((const float *)x)[i];
+        const float a = g / (1.0f + expf(-g));
+        return a * ((const float *)x2)[i];
+    } else if constexpr (SRC == SRC_GEGLU) {
+        const float g = ((const float *)x)[i];
+        const float a = 0.5f * g * (1.0f + erff(g * 0.70710678118654752440f));
+        return a * ((const float *)x2)[i];
     } else {
         return ((const float *)x)[i];
     }
@@ -51,8 +67,9 @@ __device__ __forceinline__ float load_act_value(const void *x, size_t i) {
 
 // Q8_K (matmul_quant_pack.c:106-142): one wavefront per 256-value block, 4 consecutive values per lane.
 // AOS = marmot_q8_k_block_t output; otherwise the library's structure-of-arrays scratch.
-template <bool F16, bool AOS>
-__global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ x, size_t rows, size_t k, size_t nb,
+template <int SRC, bool AOS>
+__global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ x, const void *__restrict__ x2,
+                                                       size_t rows, size_t k, size_t nb,
                                                        uint8_t *__restrict__ blocks_out, ActScratch soa) {
     const int lane = threadIdx.x & 63;
     const size_t wave = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -67,7 +84,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const size_t col = col0 + i;
-        v[i] = col < k ? load_act_value<F16>(x, row * k + col) : 0.0f;
+        v[i] = col < k ? load_act_value<SRC>(x, x2, row * k + col) : 0.0f;
     }
     // value of largest magnitude, first occurrence wins (strict > in index order)
     float best_abs = 0.0f;
@@ -133,8 +150,9 @@ __global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ 
 }
 
 // Q8_0 (matmul_quant_pack.c:23-62, block.c:221-232 scalar): 32 lanes per block, one value per lane.
-template <bool F16, bool AOS>
-__global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ x, size_t rows, size_t k, size_t nb,
+template <int SRC, bool AOS>
+__global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ x, const void *__restrict__ x2,
+                                                       size_t rows, size_t k, size_t nb,
                                                        uint8_t *__restrict__ blocks_out, ActScratch soa) {
     const int lane32 = threadIdx.x & 31;
     const size_t blk_id = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
@@ -144,7 +162,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ 
     const size_t row = blk_id / nb;
     const size_t b = blk_id - row * nb;
     const size_t col = b * QK + lane32;
-    const float v = col < k ? load_act_value<F16>(x, row * k + col) : 0.0f;
+    const float v = col < k ? load_act_value<SRC>(x, x2, row * k + col) : 0.0f;
     float max_abs = fabsf(v);
 #pragma unroll
     for (int off = 1; off < 32; off <<= 1) {
@@ -195,38 +213,47 @@ __global__ void k_fill_bytes(uint8_t *dst, uint8_t value, size_t n) {
     }
 }
 
+template <int SRC, bool AOS>
+static int launch_quantize_src(marmot_hip_device *dev, int act_kind, const void *d_x, const void *d_x2, size_t rows,
+                               size_t k, uint8_t *blocks_out, const ActScratch &soa) {
+    if (act_kind == MARMOT_HIP_KIND_Q8_K) {
+        const size_t nb = (k + QK_K - 1) / QK_K;
+        const size_t waves = rows * nb;
+        const dim3 grid((unsigned)((waves + 3) / 4));
+        hipLaunchKernelGGL((k_quantize_q8_k<SRC, AOS>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb,
+                           blocks_out, soa);
+    } else {
+        const size_t nb = (k + QK - 1) / QK;
+        const size_t blocks = rows * nb;
+        const dim3 grid((unsigned)((blocks + 7) / 8));
+        hipLaunchKernelGGL((k_quantize_q8_0<SRC, AOS>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb,
+                           blocks_out, soa);
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
 template <bool AOS>
 static int launch_quantize(marmot_hip_device *dev, int act_kind, const void *d_x, int in_dtype, size_t rows, size_t k,
                            uint8_t *blocks_out, const ActScratch &soa) {
     if (rows == 0 || k == 0) {
         return MARMOT_HIP_SUCCESS;
     }
-    const bool f16 = in_dtype == MARMOT_HIP_DTYPE_F16;
-    if (act_kind == MARMOT_HIP_KIND_Q8_K) {
-        const size_t nb = (k + QK_K - 1) / QK_K;
-        const size_t waves = rows * nb;
-        const dim3 grid((unsigned)((waves + 3) / 4));
-        if (f16) {
-            hipLaunchKernelGGL((k_quantize_q8_k<true, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
-                               blocks_out, soa);
-        } else {
-            hipLaunchKernelGGL((k_quantize_q8_k<false, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
-                               blocks_out, soa);
-        }
-    } else {
-        const size_t nb = (k + QK - 1) / QK;
-        const size_t blocks = rows * nb;
-        const dim3 grid((unsigned)((blocks + 7) / 8));
-        if (f16) {
-            hipLaunchKernelGGL((k_quantize_q8_0<true, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
-                               blocks_out, soa);
-        } else {
-            hipLaunchKernelGGL((k_quantize_q8_0<false, AOS>), grid, dim3(256), 0, dev->stream, d_x, rows, k, nb,
-                               blocks_out, soa);
-        }
+    if (in_dtype == MARMOT_HIP_DTYPE_F16) {
+        return launch_quantize_src<SRC_F16, AOS>(dev, act_kind, d_x, nullptr, rows, k, blocks_out, soa);
     }
-    MH_HIP(hipGetLastError());
-    return MARMOT_HIP_SUCCESS;
+    return launch_quantize_src<SRC_F32, AOS>(dev, act_kind, d_x, nullptr, rows, k, blocks_out, soa);
+}
+
+int launch_quantize_glu_soa(marmot_hip_device *dev, int act_kind, const float *d_gate, const float *d_up, bool geglu,
+                            size_t rows, size_t k, const ActScratch &dst) {
+    if (rows == 0 || k == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    if (geglu) {
+        return launch_quantize_src<SRC_GEGLU, false>(dev, act_kind, d_gate, d_up, rows, k, nullptr, dst);
+    }
+    return launch_quantize_src<SRC_SWIGLU, false>(dev, act_kind, d_gate, d_up, rows, k, nullptr, dst);
 }
 
 int launch_quantize_act_soa(marmot_hip_device *dev, int act_kind, const void *d_x, int in_dtype, size_t rows, size_t k,

@@ -55,6 +55,17 @@ def assert_matmul_parity(y, r, tol=1e-3, what=""):
     return m1, m2, m3
 
 
+def assert_moe_parity(y, r, tol=1e-3, what=""):
+    """MoE re-quantizes silu(gate)*up to Q8 before the down projection, so a last-ulp difference upstream (fp32
+    summation order, expf) can move one int8 value by one step; that shifts individual outputs by ~1/127 of one of F
+    terms. The bound is therefore taken against the output scale: max|d| / max|r| and sum|d| / sum|r| <= 1e-3
+    (the reference's own MoE tests allow 3e-2..9e-2 against dense math, tests/backend/test_backend_moe.c:620-1081)."""
+    m1, m2, m3 = parity_metrics(y, r)
+    assert np.all(np.isfinite(np.asarray(y, dtype=np.float64))), f"{what}: non-finite output"
+    assert m3 <= tol and m2 <= tol, f"{what}: max-norm error {m3:.3e}, sum-rel {m2:.3e} (floored-relative {m1:.3e})"
+    return m1, m2, m3
+
+
 def random_valid_blocks(rng, kind: int, rows: int, k: int) -> np.ndarray:
     """Arbitrary block bytes with finite, moderate fp16 scale fields (exercises every nibble / scale pattern)."""
     from oracle.pyoracle import BLOCK_BYTES

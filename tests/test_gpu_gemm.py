@@ -1,0 +1,104 @@
+"""GPU parity, part 4: prefill GEMM (Q4_K weights, fp16 activations, MFMA) against the CPU oracle's direct fp16
+route, which is what the reference's CPU backend runs for fp16 activations by default
+(matmul_quant_dispatch.c:449-470, vec_dot_impl.h:973-1023)."""
+import numpy as np
+import pytest
+
+from oracle.pyoracle import KIND_Q4_K
+from tests.util import gaussian, parity_metrics, quantize_weights, random_valid_blocks
+
+pytestmark = pytest.mark.gpu
+THREADS = 16
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from marmot_amd import HipBackend
+
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def exact_f64(oracle, blocks, x, M, K):
+    """The same weights and activations in float64: what both implementations approximate."""
+    deq = oracle.dequantize(KIND_Q4_K, blocks, K).astype(np.float64)
+    return x.astype(np.float64) @ deq.T
+
+
+def check_against_oracle(hip, oracle, blocks, x, M, K, what, bias=None, out_dtype=np.float32):
+    got = hip.linear(x, blocks, KIND_Q4_K, M, bias=bias, out_dtype=out_dtype)
+    assert "gemm" in hip.last_route(), hip.last_route()
+    ref = oracle.matmul(KIND_Q4_K, blocks, x, M, bias=bias, out_dtype=out_dtype, threads=THREADS)
+    got32, ref32 = got.astype(np.float32), ref.astype(np.float32)
+    m_floor, m_sum, m_max = parity_metrics(got32, ref32)
+    print(f"{what}: floored-rel {m_floor:.3e} sum-rel {m_sum:.3e} max-norm {m_max:.3e}", flush=True)
+    assert np.all(np.isfinite(got32))
+    if out_dtype == np.float32:
+        # bound against the output scale: max|d| / max|r| and sum|d| / sum|r| (fp32 accumulate on both sides)
+        assert m_max <= 1e-5 and m_sum <= 1e-5, (m_floor, m_sum, m_max)
+        # and per element with the reference test's own form |d| <= abs + rel*|ref| (test_matmul_quantized.c:166-177),
+        # the absolute term scaled to this output's magnitude
+        scale = np.sqrt(np.mean(ref32.astype(np.float64) ** 2, axis=1, keepdims=True))  # per token row
+        assert np.all(np.abs(got32 - ref32) <= 2e-5 * scale + 5e-5 * np.abs(ref32))
+    else:
+        assert m_max <= 2e-3
+    return got32, ref32
+
+
+@pytest.mark.parametrize("N", [9, 64, 128, 130, 512])
+def test_gemm_small_shapes(hip, oracle, N):
+    """Token counts around the 128-token tile, M not a multiple of the 256-row tile, K-split and single pass."""
+    M, K = 300, 1024
+    blocks = oracle.quantize(KIND_Q4_K, gaussian(500, (M, K), 0.02))
+    x = gaussian(501 + N, (N, K)).astype(np.float16)
+    check_against_oracle(hip, oracle, blocks, x, M, K, f"gemm N={N} M={M} K={K}")
+
+
+def test_gemm_random_block_bytes_and_large_activations(hip, oracle):
+    """Every scale / min / nibble pattern, and activations far from unit scale (sub-block sums stay in fp16 range)."""
+    rng = np.random.default_rng(510)
+    M, K, N = 256, 2048, 96
+    blocks = random_valid_blocks(rng, KIND_Q4_K, M, K)
+    x = (gaussian(511, (N, K)) * 300.0).astype(np.float16)
+    x[0, :] = 60000.0  # near the fp16 maximum
+    x[1, :] = 0.0
+    check_against_oracle(hip, oracle, blocks, x, M, K, "gemm random bytes")
+
+
+def test_gemm_bias_and_f16_output(hip, oracle):
+    M, K, N = 512, 1024, 40
+    blocks = oracle.quantize(KIND_Q4_K, gaussian(520, (M, K), 0.02))
+    x = gaussian(521, (N, K)).astype(np.float16)
+    bias = gaussian(522, (M,))
+    check_against_oracle(hip, oracle, blocks, x, M, K, "gemm bias f32", bias=bias)
+    check_against_oracle(hip, oracle, blocks, x, M, K, "gemm f16 out", bias=bias, out_dtype=np.float16)
+
+
+@pytest.mark.parametrize("N", [64, 128, 512, 2048])
+def test_config3_prefill_gemm(hip, oracle, N):
+    """Q4_K 4096 x 4096 (seed 30), fp16 activations N(0,1) (seed 31), fp32 out; sweep of token counts."""
+    M = K = 4096
+    blocks = quantize_weights(oracle, KIND_Q4_K, gaussian(30, (M, K), 0.02))
+    x = gaussian(31, (N, K)).astype(np.float16)
+    # the oracle's scalar direct route needs ~N*M*K/0.5e9 core-seconds: check a band of weight rows at the larger N
+    rows = M if N <= 128 else 512
+    r0 = 1024 if rows != M else 0
+    got = hip.linear(x, blocks, KIND_Q4_K, M)
+    assert "gemm" in hip.last_route()
+    ref = oracle.matmul(KIND_Q4_K, blocks[r0:r0 + rows], x, rows, threads=THREADS)
+    g = got[:, r0:r0 + rows]
+    m_floor, m_sum, m_max = parity_metrics(g, ref)
+    exact = exact_f64(oracle, blocks[r0:r0 + rows], x, rows, K)
+    e_gpu = parity_metrics(g, exact)
+    e_cpu = parity_metrics(ref, exact)
+    print(f"C3 N={N}: hip vs cpu floored-rel {m_floor:.3e} sum-rel {m_sum:.3e} max-norm {m_max:.3e}; "
+          f"vs float64: hip {e_gpu[0]:.3e}/{e_gpu[2]:.3e}, cpu {e_cpu[0]:.3e}/{e_cpu[2]:.3e}", flush=True)
+    assert m_max <= 1e-5 and m_sum <= 1e-5
+    scale = np.sqrt(np.mean(ref.astype(np.float64) ** 2, axis=1, keepdims=True))
+    assert np.all(np.abs(g - ref) <= 2e-5 * scale + 5e-5 * np.abs(ref))
+    # the HIP result is at least as close to exact arithmetic as the CPU reference's sequential fp32 sum
+    assert e_gpu[2] <= max(e_cpu[2] * 1.5, 1e-6)
+    # rows outside the checked band: K-split and full tiles must agree with a float64 product everywhere
+    full_exact = exact_f64(oracle, blocks, x[:8], M, K)
+    assert parity_metrics(got[:8], full_exact)[2] <= 1e-5

@@ -128,6 +128,38 @@ def cpu_baseline(kind, blocks, x, M, K, nbytes, ref_out, budget_s: float):
     }, err
 
 
+def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
+    """Q4_K prefill GEMM leg: marmot_linear with fp16 activations [tokens, 4096] and a 4096 x 4096 Q4_K weight."""
+    from marmot_amd import DT_F16, DT_F32, capi, row_bytes
+
+    M = K = 4096
+    kind = capi.KIND_Q4_K
+    blocks = random_blocks(np.random.Generator(np.random.PCG64(30)), kind, M, K)
+    x = np.random.Generator(np.random.PCG64(31)).standard_normal((tokens, K), dtype=np.float32).astype(np.float16)
+    d_w, d_x = hip.to_device(blocks), hip.to_device(x)
+    d_out = hip.alloc(tokens * M * 4)
+
+    def step(i):
+        hip.linear_d(kind, d_w, d_x, DT_F16, tokens, K, M, d_out, DT_F32)
+
+    ms = time_steps_graph(hip, step, steps, warmup, chunk=50)
+    flops = 2.0 * tokens * M * K
+    out = {
+        "workload": f"Q4_K prefill GEMM, weight {M}x{K}, {tokens} tokens fp16, fp32 out (fp16 MFMA, fp32 accumulate)",
+        "route": hip.last_route(),
+        "ms_per_step": round(ms, 5),
+        "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
+        "peak_tflops": 2500.0,
+        "frac_of_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4),
+        "tokens_per_s": round(tokens / (ms * 1e-3), 1),
+        "steps": steps,
+        "includes": "activation packing, GEMM and K-split reduction kernels",
+    }
+    for b in (d_w, d_x, d_out):
+        b.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -138,6 +170,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1, help="activation rows N (1, 4 or 8 are the decode configs)")
     ap.add_argument("--shape", default="4096x14336", help="weight shape MxK (marmot naming)")
     ap.add_argument("--kind", default="q4_k", choices=["q4_k", "q6_k", "q8_0", "q4_0"])
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
+    ap.add_argument("--prefill-tokens", type=int, default=512)
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")
     args = ap.parse_args()
@@ -254,6 +288,9 @@ def main():
             "cache_resident_gbps": round(nbytes / (ms_hot * 1e-3) / 1e9, 2),
         },
     }
+    # ---- second half of the metric: Q4_K prefill GEMM, weight 4096 x 4096, fp16 activations, fp32 out
+    if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) and not args.no_prefill:
+        result["prefill_gemm"] = prefill_gemm(hip, args.prefill_tokens, max(20, args.steps // 20), 5)
     if not args.no_cpu:
         cb, err = cpu_baseline(kind, blocks, x, M, K, nbytes, got, args.cpu_seconds)
         result["cpu_baseline"] = cb

@@ -9,9 +9,11 @@
 // and then y += d*P - dmin*Q in fp32 on the vector ALU. The result differs from the reference only by fp32
 // rounding / summation order.
 //
-// Tiling. A workgroup (4 wavefronts) owns 128 tokens x 256 weight rows; each wavefront owns 128 x 64 as 4 x 2 MFMA
-// tiles, so one dequantized weight operand feeds 4 MFMAs. The activation tile of the current block (64 KiB, already
-// in MFMA operand order) is staged through LDS and shared by the 4 wavefronts, double buffered. Weights are read
+// Tiling. A workgroup (8 wavefronts, two per SIMD) owns 128 tokens x 256 weight rows; each wavefront owns 128 x 32
+// as 4 MFMA tiles, so one unpacked weight operand feeds 4 MFMAs and everything fits in 256 VGPRs without AGPRs.
+// While one wavefront of a SIMD applies the per-block scales on the vector ALU, the other keeps the matrix core busy.
+// The activation tile of a block (64 KiB) is gathered straight from the row-major fp16 matrix into LDS in MFMA
+// operand order with direct-to-LDS loads, double buffered, and shared by the 8 wavefronts. Weights are read
 // straight from their GGUF blocks into registers, one block ahead, and unpacked with
 // (q | 0x6400) as fp16 = 1024 + q, then fma(1024 + q, sc, -1024 * sc) = sc * q exactly.
 // K is split across workgroups when there are too few tiles to fill the chip; partial sums meet in a small
@@ -26,87 +28,57 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int G_TOK = 128;        // tokens per workgroup tile
-constexpr int G_WROWS_WAVE = 64;  // weight rows per wavefront
-constexpr int G_WROWS_WG = 256;   // weight rows per workgroup
+constexpr int G_WROWS_WAVE = 32;  // weight rows per wavefront
+constexpr int G_WAVES = 8;
+constexpr int G_THREADS = G_WAVES * 64;
+constexpr int G_WROWS_WG = G_WROWS_WAVE * G_WAVES;  // 256 weight rows per workgroup
 constexpr int STAGE_A = 16 * 4 * 64 * 16;  // 16 K-steps x 4 token sub-tiles x 64 lanes x 16 bytes
 constexpr int STAGE_S = 4 * 64 * 16;       // sub-block sums operand: 4 token sub-tiles x 64 lanes x 16 bytes
 constexpr int STAGE = STAGE_A + STAGE_S;   // 69,632 bytes per (token tile, block)
-constexpr int STAGE_CHUNKS = STAGE / 16;   // 4352 = 17 per thread
+constexpr int STAGE_CHUNKS = STAGE / 16;   // 4352
 
-// slot e of an operand's 8 halves holds the value whose byte index within the lane's 8-byte piece is PERM[e]:
-// the nibble extraction below yields (byte0, byte2), (byte1, byte3), ...
-__device__ __forceinline__ uint32_t half_bits(float f) {
-    return (uint32_t)f2h(f);
-}
-
-// ------------------------------------------------------------------ activation packing
-// X fp16 [N, K] -> per (token tile tt, block b): operands in MFMA order.
-//   A operand (ks, a), lane (i = lane % 32, kh = lane / 32), slot e:
-//       X[128*tt + 32*a + i][256*b + 32*(ks/2) + 16*kh + 8*(ks%2) + PERM[e]],  PERM = {0,2,1,3,4,6,5,7}
-//   S operand a, lane (i, kh), slot e: kh == 0 ? hi : lo of (sum of X over sub-block e) / 32
-// Tokens beyond N are zero.
-__global__ __launch_bounds__(256) void k_gemm_pack_x(const uint16_t *__restrict__ x, size_t N, size_t K, size_t nb,
-                                                     uint8_t *__restrict__ packed) {
-    const size_t chunk = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // one 16-byte operand piece
-    const size_t tiles = (N + G_TOK - 1) / G_TOK;
-    const size_t total = tiles * nb * (STAGE_A / 16);
-    if (chunk >= total) {
-        return;
-    }
-    const size_t stage = chunk / (STAGE_A / 16);
-    const int within = (int)(chunk % (STAGE_A / 16));
-    const int lane = within & 63;
-    const int a = (within >> 6) & 3;
-    const int ks = within >> 8;
-    const size_t tt = stage / nb, b = stage % nb;
-    const int i = lane & 31, kh = lane >> 5;
-    const size_t token = tt * G_TOK + 32 * a + i;
-    uint4 out = make_uint4(0, 0, 0, 0);
-    if (token < N) {
-        const size_t k0 = b * 256 + 32 * (ks >> 1) + 16 * kh + 8 * (ks & 1);
-        const uint4 v = *(const uint4 *)(x + token * K + k0);
-        out.x = (v.x & 0xffffu) | (v.y << 16);
-        out.y = (v.x >> 16) | (v.y & 0xffff0000u);
-        out.z = (v.z & 0xffffu) | (v.w << 16);
-        out.w = (v.z >> 16) | (v.w & 0xffff0000u);
-    }
-    *(uint4 *)(packed + stage * STAGE + (size_t)within * 16) = out;
-}
-
-__global__ __launch_bounds__(256) void k_gemm_pack_s(const uint16_t *__restrict__ x, size_t N, size_t K, size_t nb,
-                                                     uint8_t *__restrict__ packed) {
-    // one thread per (stage, a, i, e): sums one 32-value sub-block of one token
+// ------------------------------------------------------------------ sub-block sums of the activations
+// S operand of (token tile tt, block b, token sub-tile a): lane (i = lane % 32, kh = lane / 32), slot e:
+//     kh == 0 ? hi : lo   of   (fp32 sum of X[128*tt + 32*a + i][256*b + 32*e .. +32]) / 32,   hi + lo in fp16.
+// Tokens beyond N give zeros. One thread per (token, block, sub-block).
+__global__ __launch_bounds__(256) void k_gemm_sums(const uint16_t *__restrict__ x, size_t N, size_t K, size_t nb,
+                                                   uint8_t *__restrict__ sums) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t tiles = (N + G_TOK - 1) / G_TOK;
-    const size_t total = tiles * nb * 4 * 32 * 8;
-    if (idx >= total) {
+    if (idx >= tiles * G_TOK * nb * 8) {
         return;
     }
     const int e = (int)(idx & 7);
-    const int i = (int)((idx >> 3) & 31);
-    const int a = (int)((idx >> 8) & 3);
-    const size_t stage = idx >> 10;
-    const size_t tt = stage / nb, b = stage % nb;
-    const size_t token = tt * G_TOK + 32 * a + i;
+    const size_t b = (idx >> 3) % nb;
+    const size_t token = (idx >> 3) / nb;
     float s = 0.0f;
     if (token < N) {
-        const uint16_t *p = x + token * K + b * 256 + 32 * e;
-        for (int t = 0; t < 32; ++t) {
-            s += h2f(p[t]);
+        const uint4 *p = (const uint4 *)(x + token * K + b * 256 + 32 * e);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint4 v = p[c];
+            s += ((h2f((uint16_t)(v.x & 0xffffu)) + h2f((uint16_t)(v.x >> 16))) +
+                  (h2f((uint16_t)(v.y & 0xffffu)) + h2f((uint16_t)(v.y >> 16)))) +
+                ((h2f((uint16_t)(v.z & 0xffffu)) + h2f((uint16_t)(v.z >> 16))) +
+                 (h2f((uint16_t)(v.w & 0xffffu)) + h2f((uint16_t)(v.w >> 16))));
         }
     }
     s *= 0.03125f;  // exact; keeps the value within fp16 range whatever the activations are
     const uint16_t hi = f2h(s);
     const uint16_t lo = f2h(s - h2f(hi));
-    uint16_t *base = (uint16_t *)(packed + stage * STAGE + STAGE_A + (size_t)a * 64 * 16);
-    base[(size_t)i * 8 + e] = hi;          // lane i       (kh = 0)
-    base[(size_t)(32 + i) * 8 + e] = lo;   // lane 32 + i  (kh = 1)
+    const size_t tt = token / G_TOK;
+    const int a = (int)(token % G_TOK) >> 5, i = (int)(token & 31);
+    uint16_t *base = (uint16_t *)(sums + ((tt * nb + b) * 4 + a) * 1024);
+    base[(size_t)i * 8 + e] = hi;         // lane i       (kh = 0)
+    base[(size_t)(32 + i) * 8 + e] = lo;  // lane 32 + i  (kh = 1)
 }
 
 // ------------------------------------------------------------------ main kernel
 struct GemmParams {
     const uint8_t *w;       // Q4_K blocks, M rows of nb blocks
-    const uint8_t *packed;  // packed activations
+    const uint16_t *x;      // fp16 activations [N, K], row-major
+    const uint8_t *sums;    // sub-block sums operand (k_gemm_sums)
+    size_t K;
     void *out;              // fp32/fp16 [N, M] (splits == 1) or fp32 partials [splits, N, M]
     const void *bias;
     int bias_is_f16;
@@ -158,30 +130,15 @@ __device__ __forceinline__ __half2 int_pair(uint32_t v) {
     return __hsub2(magic, as_h2(0x64006400u));
 }
 
-// 8 weights of one K-step as fp16 sc*q, from the two dwords (q0, q1) of the lane's 8-byte piece
-template <int NIB>
-__device__ __forceinline__ half8 dequant_kstep(uint32_t q0, uint32_t q1, __half2 sc, __half2 c) {
-    uint32_t t[4];
-    if (NIB == 0) {
-        t[0] = (q0 & 0x000f000fu) | 0x64006400u;
-        t[1] = ((q0 >> 8) & 0x000f000fu) | 0x64006400u;
-        t[2] = (q1 & 0x000f000fu) | 0x64006400u;
-        t[3] = ((q1 >> 8) & 0x000f000fu) | 0x64006400u;
-    } else {
-        t[0] = ((q0 >> 4) & 0x000f000fu) | 0x64006400u;
-        t[1] = ((q0 >> 12) & 0x000f000fu) | 0x64006400u;
-        t[2] = ((q1 >> 4) & 0x000f000fu) | 0x64006400u;
-        t[3] = ((q1 >> 12) & 0x000f000fu) | 0x64006400u;
-    }
-    uint4 r;
-    r.x = as_u32(__hfma2(as_h2(t[0]), sc, c));  // (1024 + q) * sc - 1024 * sc = sc * q, one rounding of an exact value
-    r.y = as_u32(__hfma2(as_h2(t[1]), sc, c));
-    r.z = as_u32(__hfma2(as_h2(t[2]), sc, c));
-    r.w = as_u32(__hfma2(as_h2(t[3]), sc, c));
-    return __builtin_bit_cast(half8, r);
+// Two of the 8 weights of one K-step as fp16 sc*q: bytes (2*(I%2), 2*(I%2)+1) of the masked nibble dword m
+template <int I>
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t m, __half2 sc, __half2 c) {
+    // (byte n, 0x64) as fp16 bits = 1024 + n; then (1024 + q) * sc - 1024 * sc = sc * q, one rounding of an exact value
+    const uint32_t t = __builtin_amdgcn_perm(0x64646464u, m, (I & 1) ? 0x04030402u : 0x04010400u);
+    return as_u32(__hfma2(as_h2(t), sc, c));
 }
 
-__global__ __launch_bounds__(256) void k_gemm_q4k_f16(const GemmParams p) {
+__global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // 2 stages
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -195,182 +152,256 @@ __global__ __launch_bounds__(256) void k_gemm_q4k_f16(const GemmParams p) {
     if (b1 > p.nb) {
         b1 = p.nb;
     }
-
-    const uint8_t *wrow[2];
-#pragma unroll
-    for (int wt = 0; wt < 2; ++wt) {
-        size_t r = wrow0 + 32 * wt + j;
-        if (r >= p.M) {
-            r = p.M - 1;  // harmless re-read; never stored
-        }
-        wrow[wt] = p.w + r * p.nb * Q4_K_BYTES;
+    size_t wr = wrow0 + j;
+    if (wr >= p.M) {
+        wr = p.M - 1;  // harmless re-read; never stored
     }
+    const uint8_t *wrow = p.w + wr * p.nb * Q4_K_BYTES;
 
-    floatx16 total[4][2];
+    floatx16 total[4];
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
 #pragma unroll
-        for (int wt = 0; wt < 2; ++wt) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                total[a][wt][r] = 0.0f;
-            }
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
         }
     }
 
-    if (b0 < b1) {
-        // stage the first activation block
-        const uint8_t *src = p.packed + (tt * p.nb + b0) * STAGE;
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    typedef const __attribute__((address_space(1))) uint8_t glb_u8;
+    // Gathers one stage global -> LDS with direct-to-LDS loads: every wavefront instruction moves 64 lanes x 16 bytes
+    // from per-lane addresses to a contiguous 1 KiB of LDS (no registers involved); vmcnt tracks completion.
+    // A-operand piece (ks, a, lane = (i, kh)) = X[token 32a+i][256b + 32(ks/2) + 16kh + 8(ks%2) .. +8]: 16 contiguous
+    // bytes of the row-major activations. Tokens beyond N re-read token N-1 (their results are never stored).
+    size_t gather_off[9];  // element offset of this thread's pieces within a block, block-independent
 #pragma unroll
-        for (int c = 0; c < 17; ++c) {
-            const int chunk = tid + 256 * c;
-            *(uint4 *)(lds + (size_t)chunk * 16) = *(const uint4 *)(src + (size_t)chunk * 16);
+    for (int c = 0; c < 9; ++c) {
+        const int chunk = tid + G_THREADS * c;
+        if (chunk < STAGE_A / 16) {
+            const int cl = chunk & 63, a = (chunk >> 6) & 3, ks = chunk >> 8;
+            size_t token = tt * G_TOK + 32 * a + (cl & 31);
+            if (token >= p.N) {
+                token = p.N - 1;
+            }
+            gather_off[c] = token * p.K + 32 * (ks >> 1) + 16 * (cl >> 5) + 8 * (ks & 1);
+        } else {
+            gather_off[c] = 0;
         }
     }
-    WeightRegs wnext[2];
+    auto stage_piece = [&](size_t b, uint8_t *dst, int c) {
+        {
+            const int chunk = tid + G_THREADS * c;
+            const int wbase = chunk - lane;  // first chunk of this wavefront's instruction
+            if (wbase < STAGE_CHUNKS) {  // wave-uniform
+                const uint8_t *g;
+                if (chunk < STAGE_A / 16) {
+                    g = (const uint8_t *)(p.x + gather_off[c] + b * 256);
+                } else {
+                    g = p.sums + (tt * p.nb + b) * STAGE_S + (size_t)(chunk - STAGE_A / 16) * 16;
+                }
+                uint8_t *l = dst + (size_t)wbase * 16;  // wave-uniform base; the hardware adds lane * 16
+                __builtin_amdgcn_global_load_lds((glb_u8 *)g, (lds_u8 *)l, 16, 0, 0);
+            }
+        }
+    };
+
+    WeightRegs wnext;
     if (b0 < b1) {
 #pragma unroll
-        for (int wt = 0; wt < 2; ++wt) {
-            load_weights(wnext[wt], wrow[wt] + b0 * Q4_K_BYTES, kh);
+        for (int c = 0; c < 9; ++c) {
+            stage_piece(b0, lds, c);
         }
+        load_weights(wnext, wrow + b0 * Q4_K_BYTES, kh);
     }
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     for (size_t b = b0; b < b1; ++b) {
         const int cur = (int)((b - b0) & 1);
         const uint8_t *stage = lds + (size_t)cur * STAGE;
-        uint8_t *stage_next = lds + (size_t)(cur ^ 1) * STAGE;
         const bool more = b + 1 < b1;
-        const uint8_t *src_next = p.packed + (tt * p.nb + b + 1) * STAGE;
 
-        WeightRegs wcur[2];
-        Scales sc[2];
-#pragma unroll
-        for (int wt = 0; wt < 2; ++wt) {
-            wcur[wt] = wnext[wt];
-            decode_header(wcur[wt].hdr, sc[wt]);
-        }
-        if (more) {
-#pragma unroll
-            for (int wt = 0; wt < 2; ++wt) {
-                load_weights(wnext[wt], wrow[wt] + (b + 1) * Q4_K_BYTES, kh);
+        const WeightRegs wcur = wnext;
+        Scales sc;
+        decode_header(wcur.hdr, sc);
+        // The next block's activations (straight into the other LDS stage) and weights (into registers) are
+        // requested one memory instruction per K-step, so that the address processing of these gathers overlaps
+        // the matrix work instead of holding every wavefront at the top of the block.
+        uint8_t *next_stage = lds + (size_t)(cur ^ 1) * STAGE;
+        const uint8_t *next_blk = wrow + (b + 1) * Q4_K_BYTES;
+        auto prefetch_piece = [&](int ks) {
+            if (!more) {
+                return;
             }
-        }
+            if (ks < 9) {
+                stage_piece(b + 1, next_stage, ks);
+            } else if (ks == 9) {
+                wnext.hdr = *(const uint4 *)next_blk;
+            } else if (ks < 14) {
+                wnext.q[ks - 10] = *(const uint4 *)(next_blk + 16 + 32 * (ks - 10) + 16 * kh);
+            }
+        };
 
-        floatx16 acc[4][2];
-        uint4 stg[5];  // activation staging for the next block, moved in 4 groups across the K-steps
-#pragma unroll
-        for (int ks = 0; ks < 16; ++ks) {
-            const int s = ks >> 1, tp = ks & 1, g = s >> 1;
-            // next block's activations: global -> registers at K-steps 0,4,8,12; registers -> LDS at 3,7,11,15
-            if ((ks & 3) == 0 && more) {
-                const int grp = ks >> 2;
-#pragma unroll
-                for (int c = 0; c < 5; ++c) {
-                    const int cc = grp * 5 + c;  // 0..19, chunks 17..19 do not exist
-                    if (cc < 17) {
-                        stg[c] = *(const uint4 *)(src_next + (size_t)(tid + 256 * cc) * 16);
-                    }
+        // Operand B of K-step ks is built in 4 pieces, one per MFMA of the previous K-step, so that the unpack
+        // arithmetic runs in the shadow of the matrix core. The scheduling fences pin that order.
+        __half2 scp, cp;
+        uint32_t m0 = 0, m1 = 0;
+        auto b_piece = [&](int ks, int i) -> uint32_t {
+            const int s_ = ks >> 1, tp = ks & 1, g = s_ >> 1;
+            if (i == 0) {
+                if (tp == 0) {
+                    const uint32_t scw = s_ < 4 ? sc.sc_lo : sc.sc_hi;
+                    // (1024 + sc, 1024 + sc) - (1024, 1024)
+                    const uint32_t sel = (s_ & 3) == 0 ? 0x04000400u : (s_ & 3) == 1 ? 0x04010401u
+                                       : (s_ & 3) == 2 ? 0x04020402u : 0x04030403u;
+                    scp = __hsub2(as_h2(__builtin_amdgcn_perm(0x64646464u, scw, sel)), as_h2(0x64006400u));
+                    cp = __hmul2(scp, as_h2(0xe400e400u));  // -1024 * sc, exact
                 }
+                const uint32_t q0 = tp ? wcur.q[g].z : wcur.q[g].x;
+                const uint32_t q1 = tp ? wcur.q[g].w : wcur.q[g].y;
+                m0 = ((s_ & 1) ? (q0 >> 4) : q0) & 0x0f0f0f0fu;
+                m1 = ((s_ & 1) ? (q1 >> 4) : q1) & 0x0f0f0f0fu;
             }
-            half8 bop[2];
-#pragma unroll
-            for (int wt = 0; wt < 2; ++wt) {
-                const uint32_t scw = s < 4 ? sc[wt].sc_lo : sc[wt].sc_hi;
-                const __half2 scp = int_pair((scw >> (8 * (s & 3))) & 0xffu);
-                const __half2 cp = __hmul2(scp, as_h2(0xe400e400u));  // -1024 * sc, exact
-                const uint32_t q0 = tp ? wcur[wt].q[g].z : wcur[wt].q[g].x;
-                const uint32_t q1 = tp ? wcur[wt].q[g].w : wcur[wt].q[g].y;
-                bop[wt] = (s & 1) ? dequant_kstep<1>(q0, q1, scp, cp) : dequant_kstep<0>(q0, q1, scp, cp);
+            switch (i) {
+            case 0: return dequant_pair<0>(m0, scp, cp);
+            case 1: return dequant_pair<1>(m0, scp, cp);
+            case 2: return dequant_pair<0>(m1, scp, cp);
+            default: return dequant_pair<1>(m1, scp, cp);
             }
+        };
+        auto read_a = [&](int ks, half8(&aop)[4]) {
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                const half8 aop = __builtin_bit_cast(half8, *(const uint4 *)(stage + ((size_t)(ks * 4 + a) * 64 + lane) * 16));
-#pragma unroll
-                for (int wt = 0; wt < 2; ++wt) {
-                    if (ks == 0) {
-                        const floatx16 zero = {0};
-                        acc[a][wt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop, bop[wt], zero, 0, 0, 0);
-                    } else {
-                        acc[a][wt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop, bop[wt], acc[a][wt], 0, 0, 0);
-                    }
-                }
+                aop[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + ((size_t)(ks * 4 + a) * 64 + lane) * 16));
             }
-            if ((ks & 3) == 3 && more) {
-                const int grp = ks >> 2;
+        };
+
+        floatx16 acc[4];
+        half8 aop[2][4];  // A operands of the K-step in flight and of the next one
+        uint32_t bop[2][4];
+        read_a(0, aop[0]);
 #pragma unroll
-                for (int c = 0; c < 5; ++c) {
-                    const int cc = grp * 5 + c;
-                    if (cc < 17) {
-                        *(uint4 *)(stage_next + (size_t)(tid + 256 * cc) * 16) = stg[c];
-                    }
+        for (int i = 0; i < 4; ++i) {
+            bop[0][i] = b_piece(0, i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 16; ++ks) {
+            const int c = ks & 1, n = c ^ 1;
+            if (ks < 15) {
+                read_a(ks + 1, aop[n]);  // lands while the 4 MFMAs below run
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const half8 bcur = __builtin_bit_cast(half8, make_uint4(bop[c][0], bop[c][1], bop[c][2], bop[c][3]));
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                if (ks == 0) {
+                    const floatx16 zero = {0};
+                    acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, zero, 0, 0, 0);
+                } else {
+                    acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, acc[a], 0, 0, 0);
                 }
+                if (ks < 15) {
+                    bop[n][a] = b_piece(ks + 1, a);
+                }
+                if (a == 1) {
+                    prefetch_piece(ks);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // min term and the per-block scales
-        half8 b2[2];
-#pragma unroll
-        for (int wt = 0; wt < 2; ++wt) {
+        // min term and the per-block scales: total += d * P - dmin * Q
+        half8 b2;
+        {
             uint4 r;
-            const uint32_t lo = sc[wt].mn_lo, hi = sc[wt].mn_hi;
+            const uint32_t lo = sc.mn_lo, hi = sc.mn_hi;
             const __half2 k32 = as_h2(0x50005000u);  // (32, 32)
             const __half2 m1024 = as_h2(0x64006400u);
-            r.x = as_u32(__hmul2(__hsub2(as_h2(0x64006400u | (lo & 0xffu) | ((lo & 0xff00u) << 8)), m1024), k32));
-            r.y = as_u32(__hmul2(__hsub2(as_h2(0x64006400u | ((lo >> 16) & 0xffu) | ((lo >> 8) & 0xff0000u)), m1024), k32));
-            r.z = as_u32(__hmul2(__hsub2(as_h2(0x64006400u | (hi & 0xffu) | ((hi & 0xff00u) << 8)), m1024), k32));
-            r.w = as_u32(__hmul2(__hsub2(as_h2(0x64006400u | ((hi >> 16) & 0xffu) | ((hi >> 8) & 0xff0000u)), m1024), k32));
-            b2[wt] = __builtin_bit_cast(half8, r);
+            const uint32_t magic = 0x64646464u;
+            r.x = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, lo, 0x04010400u)), m1024), k32));
+            r.y = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, lo, 0x04030402u)), m1024), k32));
+            r.z = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, hi, 0x04010400u)), m1024), k32));
+            r.w = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, hi, 0x04030402u)), m1024), k32));
+            b2 = __builtin_bit_cast(half8, r);
         }
+        const float d = sc.d, nd = -sc.dmin;
+        // Q-term MFMA of token sub-tile a runs while the vector ALU applies d to sub-tile a and dmin to sub-tile a-1
+        floatx16 mq[2];
+        half8 a2[4];
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            const half8 a2 = __builtin_bit_cast(half8, *(const uint4 *)(stage + STAGE_A + ((size_t)a * 64 + lane) * 16));
+            a2[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + STAGE_A + ((size_t)a * 64 + lane) * 16));
+        }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int wt = 0; wt < 2; ++wt) {
+        for (int a = 0; a < 5; ++a) {
+            if (a < 4) {
                 const floatx16 zero = {0};
-                const floatx16 mq = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[wt], zero, 0, 0, 0);
-                const float d = sc[wt].d, nd = -sc[wt].dmin;
+                mq[a & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2[a], b2, zero, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    total[a][wt][r] = __builtin_fmaf(d, acc[a][wt][r], total[a][wt][r]);
-                    total[a][wt][r] = __builtin_fmaf(nd, mq[r], total[a][wt][r]);
+                    total[a][r] = __builtin_fmaf(d, acc[a][r], total[a][r]);
                 }
             }
+            if (a > 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    total[a - 1][r] = __builtin_fmaf(nd, mq[(a - 1) & 1][r], total[a - 1][r]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_waitcnt(0);  // the next stage's direct-to-LDS loads have landed
         __syncthreads();
     }
 
-    // epilogue
-#pragma unroll
-    for (int wt = 0; wt < 2; ++wt) {
-        const size_t m = wrow0 + 32 * wt + j;
-        if (m >= p.M) {
-            continue;
-        }
-        float bias = 0.0f;
-        if (p.splits == 1 && p.bias != nullptr && !p.out_is_f16) {
-            bias = ((const float *)p.bias)[m];
-        }
+    // epilogue: lane (j, kh) holds weight row m = wrow0 + j for tokens 32a + 8(r/4) + 4kh + r%4
+    const size_t m = wrow0 + j;
+    if (m >= p.M) {
+        return;
+    }
+    const size_t n0 = tt * G_TOK + 4 * kh;
+    if (p.splits > 1) {
+        float *dst = (float *)p.out + (size_t)split * p.N * p.M + m;
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const size_t n = tt * G_TOK + 32 * a + 8 * (r >> 2) + 4 * kh + (r & 3);
-                if (n >= p.N) {
-                    continue;
+                const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
+                if (n < p.N) {
+                    dst[n * p.M] = total[a][r];
                 }
-                const float v = total[a][wt][r];
-                if (p.splits > 1) {
-                    ((float *)p.out)[((size_t)split * p.N + n) * p.M + m] = v;
-                } else if (!p.out_is_f16) {
-                    ((float *)p.out)[n * p.M + m] = v + bias;
-                } else {
-                    uint16_t h = f2h(v);
-                    if (p.bias != nullptr) {
-                        const float bv =
-                            p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m]) : ((const float *)p.bias)[m];
-                        h = f2h(h2f(h) + bv);
+            }
+        }
+    } else if (!p.out_is_f16) {
+        const float bias = p.bias != nullptr ? ((const float *)p.bias)[m] : 0.0f;
+        float *dst = (float *)p.out + m;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
+                if (n < p.N) {
+                    dst[n * p.M] = total[a][r] + bias;
+                }
+            }
+        }
+    } else {
+        const bool has_bias = p.bias != nullptr;
+        const float bias = !has_bias ? 0.0f
+            : p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m]) : ((const float *)p.bias)[m];
+        uint16_t *dst = (uint16_t *)p.out + m;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
+                if (n < p.N) {
+                    uint16_t h = f2h(total[a][r]);  // round to the output type first, then add the bias in it
+                    if (has_bias) {
+                        h = f2h(h2f(h) + bias);
                     }
-                    ((uint16_t *)p.out)[n * p.M + m] = h;
+                    dst[n * p.M] = h;
                 }
             }
         }
@@ -378,29 +409,48 @@ __global__ __launch_bounds__(256) void k_gemm_q4k_f16(const GemmParams p) {
 }
 
 // sums the K-split partials in split order, then bias / output cast like the single-pass epilogue
+template <int V>
 __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ partial, int splits, size_t N, size_t M,
                                                      const void *bias, int bias_is_f16, void *out, int out_is_f16) {
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= N * M) {
+    const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
+    const size_t total = N * M;
+    if (idx >= total) {
         return;
     }
-    float v = 0.0f;
-    for (int s = 0; s < splits; ++s) {
-        v += partial[(size_t)s * N * M + idx];
+    float v[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        v[e] = 0.0f;
     }
-    const size_t m = idx % M;
-    if (!out_is_f16) {
-        if (bias != nullptr) {
-            v += ((const float *)bias)[m];
+    for (int s = 0; s < splits; ++s) {
+        const float *src = partial + (size_t)s * total + idx;
+        if (V == 4) {
+            const float4 t = *(const float4 *)src;
+            v[0] += t.x;
+            v[1 % V] += t.y;
+            v[2 % V] += t.z;
+            v[3 % V] += t.w;
+        } else {
+            v[0] += src[0];
         }
-        ((float *)out)[idx] = v;
-    } else {
-        uint16_t h = f2h(v);
-        if (bias != nullptr) {
-            const float bv = bias_is_f16 ? h2f(((const uint16_t *)bias)[m]) : ((const float *)bias)[m];
-            h = f2h(h2f(h) + bv);
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+        const size_t m = (idx + e) % M;
+        if (!out_is_f16) {
+            float r = v[e];
+            if (bias != nullptr) {
+                r += ((const float *)bias)[m];
+            }
+            ((float *)out)[idx + e] = r;
+        } else {
+            uint16_t h = f2h(v[e]);
+            if (bias != nullptr) {
+                const float bv = bias_is_f16 ? h2f(((const uint16_t *)bias)[m]) : ((const float *)bias)[m];
+                h = f2h(h2f(h) + bv);
+            }
+            ((uint16_t *)out)[idx + e] = h;
         }
-        ((uint16_t *)out)[idx] = h;
     }
 }
 
@@ -446,23 +496,20 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     const size_t blocks_per_split = (nb + splits - 1) / splits;
     splits = (nb + blocks_per_split - 1) / blocks_per_split;
 
-    const size_t packed_bytes = tiles_n * nb * STAGE;
+    const size_t sums_bytes = tiles_n * nb * STAGE_S;
     const size_t partial_bytes = splits > 1 ? splits * N * M * sizeof(float) : 0;
     void *ws = nullptr;
-    int st = workspace_reserve(dev, ((packed_bytes + 255) & ~(size_t)255) + partial_bytes, &ws);
+    int st = workspace_reserve(dev, ((sums_bytes + 255) & ~(size_t)255) + partial_bytes, &ws);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
-    uint8_t *packed = (uint8_t *)ws;
-    float *partial = (float *)((uint8_t *)ws + ((packed_bytes + 255) & ~(size_t)255));
+    uint8_t *sums = (uint8_t *)ws;
+    float *partial = (float *)((uint8_t *)ws + ((sums_bytes + 255) & ~(size_t)255));
 
     {
-        const size_t total = tiles_n * nb * (STAGE_A / 16);
-        hipLaunchKernelGGL(k_gemm_pack_x, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream,
-                           (const uint16_t *)d_x, N, K, nb, packed);
-        const size_t total_s = tiles_n * nb * 4 * 32 * 8;
-        hipLaunchKernelGGL(k_gemm_pack_s, dim3((unsigned)((total_s + 255) / 256)), dim3(256), 0, dev->stream,
-                           (const uint16_t *)d_x, N, K, nb, packed);
+        const size_t total = tiles_n * G_TOK * nb * 8;
+        hipLaunchKernelGGL(k_gemm_sums, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream,
+                           (const uint16_t *)d_x, N, K, nb, sums);
         MH_HIP(hipGetLastError());
     }
 
@@ -473,7 +520,9 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     }
     GemmParams p;
     p.w = (const uint8_t *)d_w;
-    p.packed = packed;
+    p.x = (const uint16_t *)d_x;
+    p.sums = sums;
+    p.K = K;
     p.out = splits > 1 ? (void *)partial : d_out;
     p.bias = d_bias;
     p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
@@ -483,13 +532,18 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     p.nb = nb;
     p.splits = (int)splits;
     p.blocks_per_split = (int)blocks_per_split;
-    hipLaunchKernelGGL(k_gemm_q4k_f16, dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits), dim3(256),
-                       2 * STAGE, dev->stream, p);
+    hipLaunchKernelGGL(k_gemm_q4k_f16, dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits),
+                       dim3(G_THREADS), 2 * STAGE, dev->stream, p);
     MH_HIP(hipGetLastError());
     if (splits > 1) {
         const size_t total = N * M;
-        hipLaunchKernelGGL(k_gemm_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream, partial,
-                           (int)splits, N, M, d_bias, p.bias_is_f16, d_out, p.out_is_f16);
+        if (total % 4 == 0) {
+            hipLaunchKernelGGL(k_gemm_reduce<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, dev->stream,
+                               partial, (int)splits, N, M, d_bias, p.bias_is_f16, d_out, p.out_is_f16);
+        } else {
+            hipLaunchKernelGGL(k_gemm_reduce<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream,
+                               partial, (int)splits, N, M, d_bias, p.bias_is_f16, d_out, p.out_is_f16);
+        }
         MH_HIP(hipGetLastError());
     }
     set_route("gemm_q4_k_f16_mfma");

@@ -169,41 +169,52 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
 
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
     typedef const __attribute__((address_space(1))) uint8_t glb_u8;
-    // Gathers one stage global -> LDS with direct-to-LDS loads: every wavefront instruction moves 64 lanes x 16 bytes
-    // from per-lane addresses to a contiguous 1 KiB of LDS (no registers involved); vmcnt tracks completion.
-    // A-operand piece (ks, a, lane = (i, kh)) = X[token 32a+i][256b + 32(ks/2) + 16kh + 8(ks%2) .. +8]: 16 contiguous
-    // bytes of the row-major activations. Tokens beyond N re-read token N-1 (their results are never stored).
-    size_t gather_off[9];  // element offset of this thread's pieces within a block, block-independent
+    // One stage is moved global -> LDS with direct-to-LDS loads: every wavefront instruction moves 64 lanes x 16 bytes
+    // from per-lane global addresses to a contiguous 1 KiB of LDS (no registers involved); vmcnt tracks completion.
+    // LDS layout of the activation part: token t of the tile owns 512 bytes (its 256 halves of this block) as 32
+    // chunks of 16 bytes, chunk c stored in slot c ^ (t % 16). One instruction covers tokens 2q and 2q+1, so its
+    // global reads are two contiguous 512-byte rows; the slot swizzle makes the MFMA operand reads below (16 tokens
+    // x the same chunk) fall into 16 different bank groups. Tokens beyond N re-read token N-1 (never stored).
+    uint32_t gather_off[9];  // byte offset of this thread's piece from the tile's first row, block-independent
+    const uint8_t *tile_x = (const uint8_t *)(p.x + tt * G_TOK * p.K);
 #pragma unroll
     for (int c = 0; c < 9; ++c) {
         const int chunk = tid + G_THREADS * c;
         if (chunk < STAGE_A / 16) {
-            const int cl = chunk & 63, a = (chunk >> 6) & 3, ks = chunk >> 8;
-            size_t token = tt * G_TOK + 32 * a + (cl & 31);
-            if (token >= p.N) {
-                token = p.N - 1;
+            const int t = chunk >> 5, slot = chunk & 31;
+            size_t trow = t;
+            if (tt * G_TOK + trow >= p.N) {
+                trow = p.N - 1 - tt * G_TOK;
             }
-            gather_off[c] = token * p.K + 32 * (ks >> 1) + 16 * (cl >> 5) + 8 * (ks & 1);
+            gather_off[c] = (uint32_t)(trow * p.K * 2 + 16 * (slot ^ (t & 15)));
         } else {
             gather_off[c] = 0;
         }
     }
     auto stage_piece = [&](size_t b, uint8_t *dst, int c) {
-        {
-            const int chunk = tid + G_THREADS * c;
-            const int wbase = chunk - lane;  // first chunk of this wavefront's instruction
-            if (wbase < STAGE_CHUNKS) {  // wave-uniform
-                const uint8_t *g;
-                if (chunk < STAGE_A / 16) {
-                    g = (const uint8_t *)(p.x + gather_off[c] + b * 256);
-                } else {
-                    g = p.sums + (tt * p.nb + b) * STAGE_S + (size_t)(chunk - STAGE_A / 16) * 16;
-                }
-                uint8_t *l = dst + (size_t)wbase * 16;  // wave-uniform base; the hardware adds lane * 16
-                __builtin_amdgcn_global_load_lds((glb_u8 *)g, (lds_u8 *)l, 16, 0, 0);
+        const int chunk = tid + G_THREADS * c;
+        const int wbase = chunk - lane;  // first chunk of this wavefront's instruction
+        if (wbase < STAGE_CHUNKS) {      // wave-uniform
+            const uint8_t *g;
+            if (chunk < STAGE_A / 16) {
+                g = tile_x + gather_off[c] + b * 512;
+            } else {
+                g = p.sums + (tt * p.nb + b) * STAGE_S + (size_t)(chunk - STAGE_A / 16) * 16;
             }
+            uint8_t *l = dst + (size_t)wbase * 16;  // wave-uniform base; the hardware adds lane * 16
+            __builtin_amdgcn_global_load_lds((glb_u8 *)g, (lds_u8 *)l, 16, 0, 0);
         }
     };
+    // MFMA A operand of K-step ks, token sub-tile a, lane (i = j, kh): token 32a + i, chunk 4(ks/2) + 2kh + ks%2.
+    // Per-lane part of its LDS offset for the 8 combinations of ((ks/2) % 4, ks % 2); the rest is a constant.
+    uint32_t a_off[4][2];
+#pragma unroll
+    for (int s3 = 0; s3 < 4; ++s3) {
+#pragma unroll
+        for (int tp = 0; tp < 2; ++tp) {
+            a_off[s3][tp] = (uint32_t)(j * 512 + 16 * ((4 * s3 + 2 * kh + tp) ^ (j & 15)));
+        }
+    }
 
     WeightRegs wnext;
     if (b0 < b1) {
@@ -272,7 +283,8 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
         auto read_a = [&](int ks, half8(&aop)[4]) {
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
-                aop[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + ((size_t)(ks * 4 + a) * 64 + lane) * 16));
+                aop[a] = __builtin_bit_cast(
+                    half8, *(const uint4 *)(stage + a_off[(ks >> 1) & 3][ks & 1] + (a * 16384 + 256 * (ks >> 3))));
             }
         };
 

@@ -1,0 +1,1212 @@
+// marmot_tensor_t-level HIP backend: device vtable with a host-pointer residency table, kernel query,
+// bytecode exec table and the impl functions the generated dispatch shims call. Host code only; all device work
+// goes through the raw-pointer C ABI of marmot_hip.h.
+#include "marmot_hip.h"
+#include "marmot_hip_backend.h"
+
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <new>
+
+namespace {
+
+// ------------------------------------------------------------------ errors
+#ifdef MARMOT_HIP_IN_TREE
+inline marmot_error_t fail(marmot_error_t code, const char *msg) {
+    marmot_set_error(code, msg);
+    return code;
+}
+#else
+thread_local marmot_error_t g_last_code = MARMOT_SUCCESS;
+thread_local char g_last_detail[256] = {0};
+inline marmot_error_t fail(marmot_error_t code, const char *msg) {
+    g_last_code = code;
+    snprintf(g_last_detail, sizeof(g_last_detail), "%s", msg != nullptr ? msg : "");
+    return code;
+}
+#endif
+
+// a failure of the raw ABI: same numeric codes, text from the library
+inline marmot_error_t fail_from_lib(int code) {
+    return fail((marmot_error_t)code, marmot_hip_last_error());
+}
+
+// ------------------------------------------------------------------ residency table
+// One device mirror per host address range, keyed by the range's first byte. Ranges never overlap: a request
+// that is contained in a mirror resolves to an offset inside it; a request that overlaps mirrors without being
+// contained in one replaces them with one mirror over the union (their device-newer bytes are brought home first).
+struct Mirror {
+    uintptr_t host = 0;
+    size_t bytes = 0;
+    void *dev = nullptr;
+    bool host_newer = false;  // host copy changed since the last upload
+    bool dev_newer = false;   // a kernel wrote the mirror since the last download
+};
+
+struct Backend {
+    marmot_hip_device_t *dev = nullptr;
+    std::mutex mu;
+    std::map<uintptr_t, Mirror> mirrors;
+    bool batching = false;
+    uint64_t uploads = 0, upload_bytes = 0, downloads = 0, download_bytes = 0;
+    size_t mirrored_bytes = 0;
+
+    Mirror *find_containing(uintptr_t p, size_t n) {
+        auto it = mirrors.upper_bound(p);
+        if (it == mirrors.begin()) {
+            return nullptr;
+        }
+        --it;
+        Mirror &m = it->second;
+        if (p >= m.host && p + n <= m.host + m.bytes) {
+            return &m;
+        }
+        return nullptr;
+    }
+
+    marmot_error_t upload(Mirror &m) {
+        int st = marmot_hip_memcpy_to_device(dev, m.dev, (const void *)m.host, m.bytes);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return fail_from_lib(st);
+        }
+        uploads++;
+        upload_bytes += m.bytes;
+        m.host_newer = false;
+        return MARMOT_SUCCESS;
+    }
+
+    marmot_error_t download(Mirror &m, uintptr_t p, size_t n) {
+        int st = marmot_hip_memcpy_from_device(dev, (void *)p, (const uint8_t *)m.dev + (p - m.host), n);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return fail_from_lib(st);
+        }
+        downloads++;
+        download_bytes += n;
+        return MARMOT_SUCCESS;
+    }
+
+    void drop(std::map<uintptr_t, Mirror>::iterator it) {
+        marmot_hip_free(dev, it->second.dev);
+        mirrored_bytes -= it->second.bytes;
+        mirrors.erase(it);
+    }
+
+    // mirror covering [p, p+n): existing one, or a new one over the union of [p, p+n) and every mirror it touches
+    marmot_error_t cover(uintptr_t p, size_t n, bool will_read_host, Mirror **out) {
+        if (Mirror *m = find_containing(p, n)) {
+            *out = m;
+            return MARMOT_SUCCESS;
+        }
+        uintptr_t lo = p, hi = p + n;
+        // bring device-newer bytes of overlapping mirrors home, then drop them
+        for (;;) {
+            auto it = mirrors.lower_bound(lo);
+            if (it != mirrors.begin()) {
+                auto prev = it;
+                --prev;
+                if (prev->second.host + prev->second.bytes > lo) {
+                    it = prev;
+                }
+            }
+            if (it == mirrors.end() || it->second.host >= hi) {
+                break;
+            }
+            Mirror &o = it->second;
+            if (o.dev_newer) {
+                marmot_error_t st = download(o, o.host, o.bytes);
+                if (st != MARMOT_SUCCESS) {
+                    return st;
+                }
+            }
+            if (o.host < lo) {
+                lo = o.host;
+            }
+            if (o.host + o.bytes > hi) {
+                hi = o.host + o.bytes;
+            }
+            drop(it);
+            will_read_host = true;  // the union holds bytes that are only on the host now
+        }
+        Mirror m;
+        m.host = lo;
+        m.bytes = hi - lo;
+        int st = marmot_hip_alloc(dev, m.bytes, &m.dev);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return fail_from_lib(st);
+        }
+        m.host_newer = will_read_host;
+        mirrored_bytes += m.bytes;
+        auto ins = mirrors.emplace(lo, m);
+        *out = &ins.first->second;
+        return MARMOT_SUCCESS;
+    }
+
+    // device address of a kernel input: uploads the mirror when the host copy is newer
+    marmot_error_t acquire_read(const void *host, size_t n, const void **d_out) {
+        Mirror *m = nullptr;
+        marmot_error_t st = cover((uintptr_t)host, n, true, &m);
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+        if (m->host_newer) {
+            st = upload(*m);
+            if (st != MARMOT_SUCCESS) {
+                return st;
+            }
+        }
+        *d_out = (const uint8_t *)m->dev + ((uintptr_t)host - m->host);
+        return MARMOT_SUCCESS;
+    }
+
+    // device address of a kernel output that is fully overwritten
+    marmot_error_t acquire_write(void *host, size_t n, void **d_out) {
+        Mirror *m = nullptr;
+        marmot_error_t st = cover((uintptr_t)host, n, false, &m);
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+        const bool whole = (uintptr_t)host == m->host && n == m->bytes;
+        if (m->host_newer && !whole) {
+            st = upload(*m);  // keep the bytes of the mirror outside the output valid
+            if (st != MARMOT_SUCCESS) {
+                return st;
+            }
+        }
+        m->host_newer = false;
+        m->dev_newer = true;
+        *d_out = (uint8_t *)m->dev + ((uintptr_t)host - m->host);
+        return MARMOT_SUCCESS;
+    }
+};
+
+inline Backend *backend_of(const void *device_ctx) {
+    return (Backend *)const_cast<void *>(device_ctx);
+}
+
+// ------------------------------------------------------------------ tensor helpers
+size_t dtype_size(marmot_dtype_t t) {
+    switch (t) {
+    case MARMOT_DTYPE_FLOAT32:
+    case MARMOT_DTYPE_INT32:
+    case MARMOT_DTYPE_UINT32:
+        return 4;
+    case MARMOT_DTYPE_FLOAT16:
+    case MARMOT_DTYPE_BFLOAT16:
+    case MARMOT_DTYPE_INT16:
+    case MARMOT_DTYPE_UINT16:
+        return 2;
+    case MARMOT_DTYPE_INT8:
+    case MARMOT_DTYPE_UINT8:
+    case MARMOT_DTYPE_FLOAT8_E4M3:
+    case MARMOT_DTYPE_FLOAT8_E5M2:
+        return 1;
+    case MARMOT_DTYPE_FLOAT64:
+    case MARMOT_DTYPE_INT64:
+    case MARMOT_DTYPE_UINT64:
+        return 8;
+    default:
+        return 0;
+    }
+}
+
+bool kind_supported_weight(marmot_quant_kind_t k) {
+    return k == MARMOT_QUANT_KIND_Q4_0 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q4_K ||
+        k == MARMOT_QUANT_KIND_Q6_K;
+}
+
+bool kind_is_block(marmot_quant_kind_t k) {
+    return k > MARMOT_QUANT_KIND_GENERIC && k < MARMOT_QUANT_KIND_COUNT;
+}
+
+// block-quantized storage uses byte-sized elements (marmot_quant_storage_dtype_compatible, src/core/helpers/quant.c)
+bool storage_dtype_ok(marmot_dtype_t t) {
+    return t == MARMOT_DTYPE_UINT8 || t == MARMOT_DTYPE_INT8;
+}
+
+size_t dense_bytes(const marmot_tensor_t *t) {
+    size_t n = 1;
+    for (size_t i = 0; i < t->shape.ndim; ++i) {
+        n *= t->shape.shape[i];
+    }
+    return n * dtype_size(t->dtype);
+}
+
+bool rows_contiguous(const marmot_tensor_t *t) {
+    if (t->shape.ndim != 2) {
+        return false;
+    }
+    return t->shape.strides[1] == 1 && t->shape.strides[0] == t->shape.shape[1];
+}
+
+void mark_device_output(marmot_tensor_t *t) {
+    t->memory_location = MARMOT_MEMORY_DEVICE;
+    t->needs_sync = true;
+}
+
+// ------------------------------------------------------------------ vtable
+marmot_error_t ops_init(void **device_ctx) {
+    if (device_ctx == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP backend init: null device_ctx");
+    }
+    Backend *b = new (std::nothrow) Backend();
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_OUT_OF_MEMORY, "HIP backend init: out of host memory");
+    }
+    int st = marmot_hip_device_create(0, &b->dev);
+    if (st != MARMOT_HIP_SUCCESS) {
+        delete b;
+        return fail_from_lib(st);
+    }
+    *device_ctx = b;
+    return MARMOT_SUCCESS;
+}
+
+void ops_destroy(const void *device_ctx) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return;
+    }
+    marmot_hip_synchronize(b->dev);
+    for (auto &kv : b->mirrors) {
+        marmot_hip_free(b->dev, kv.second.dev);
+    }
+    b->mirrors.clear();
+    marmot_hip_device_destroy(b->dev);
+    delete b;
+}
+
+marmot_error_t ops_configure(const void *device_ctx, const marmot_context_t *ctx) {
+    (void)ctx;
+    return device_ctx != nullptr ? MARMOT_SUCCESS : fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP backend: null device_ctx");
+}
+
+marmot_error_t ops_alloc(const void *device_ctx, size_t size, void **ptr) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || ptr == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP alloc: null argument");
+    }
+    int st = marmot_hip_alloc(b->dev, size, ptr);
+    return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
+}
+
+void ops_free(const void *device_ctx, void *ptr) {
+    Backend *b = backend_of(device_ctx);
+    if (b != nullptr && ptr != nullptr) {
+        marmot_hip_free(b->dev, ptr);
+    }
+}
+
+marmot_error_t ops_memcpy_to_device(const void *device_ctx, void *dst, const void *src, size_t size) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || dst == nullptr || src == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP memcpy_to_device: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_SUCCESS;
+    }
+    if (dst != src) {
+        int st = marmot_hip_memcpy_to_device(b->dev, dst, src, size);
+        return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
+    }
+    // dst == src == host pointer: the host copy is newer than the mirror (src/core/tensor/transfer.c:22)
+    std::lock_guard<std::mutex> lock(b->mu);
+    const uintptr_t p = (uintptr_t)src;
+    if (Mirror *m = b->find_containing(p, size)) {
+        if (p == m->host && size == m->bytes) {
+            m->host_newer = true;  // uploaded when a kernel next reads it
+            m->dev_newer = false;
+            return MARMOT_SUCCESS;
+        }
+        if (m->host_newer) {
+            return MARMOT_SUCCESS;  // the whole mirror is refreshed on next use anyway
+        }
+        int st = marmot_hip_memcpy_to_device(b->dev, (uint8_t *)m->dev + (p - m->host), src, size);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return fail_from_lib(st);
+        }
+        b->uploads++;
+        b->upload_bytes += size;
+        return MARMOT_SUCCESS;
+    }
+    // not mirrored (yet): the first kernel that reads the range uploads it; stale partial overlaps are refreshed
+    for (auto &kv : b->mirrors) {
+        Mirror &o = kv.second;
+        if (o.host < p + size && p < o.host + o.bytes) {
+            o.host_newer = true;
+        }
+    }
+    return MARMOT_SUCCESS;
+}
+
+marmot_error_t ops_memcpy_from_device(const void *device_ctx, void *dst, const void *src, size_t size) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || dst == nullptr || src == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP memcpy_from_device: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_SUCCESS;
+    }
+    if (dst != src) {
+        int st = marmot_hip_memcpy_from_device(b->dev, dst, src, size);
+        return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
+    }
+    // dst == src == host pointer: make the host copy current (src/core/tensor/transfer.c:49-55)
+    std::lock_guard<std::mutex> lock(b->mu);
+    const uintptr_t p = (uintptr_t)dst;
+    // every mirror that overlaps the range and holds newer bytes
+    for (auto &kv : b->mirrors) {
+        Mirror &m = kv.second;
+        if (!(m.host < p + size && p < m.host + m.bytes) || !m.dev_newer) {
+            continue;
+        }
+        const uintptr_t lo = p > m.host ? p : m.host;
+        const uintptr_t hi = (p + size) < (m.host + m.bytes) ? (p + size) : (m.host + m.bytes);
+        marmot_error_t st = b->download(m, lo, hi - lo);
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+        if (lo == m.host && hi == m.host + m.bytes) {
+            m.dev_newer = false;
+        }
+    }
+    return MARMOT_SUCCESS;
+}
+
+marmot_error_t ops_synchronize(const void *device_ctx) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP synchronize: null device_ctx");
+    }
+    int st = marmot_hip_synchronize(b->dev);
+    return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
+}
+
+marmot_error_t ops_allocator_usage(const void *device_ctx, marmot_allocator_usage_t *usage) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || usage == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP allocator_usage: null argument");
+    }
+    size_t cur = 0, peak = 0, n = 0;
+    int st = marmot_hip_allocator_usage(b->dev, &cur, &peak, &n);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(st);
+    }
+    memset(usage, 0, sizeof(*usage));
+    usage->current_bytes = cur;
+    usage->peak_bytes = peak;
+    usage->active_allocations = n;
+    return MARMOT_SUCCESS;
+}
+
+// All kernels of a context are enqueued on one stream in program order, so a batch needs no extra bracket:
+// begin/end only record the state that marmot_graph_batch_is_active reports.
+marmot_error_t ops_graph_batch_begin(void *device_ctx) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP graph_batch_begin: null device_ctx");
+    }
+    b->batching = true;
+    return MARMOT_SUCCESS;
+}
+
+marmot_error_t ops_graph_batch_end(void *device_ctx, bool commit) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP graph_batch_end: null device_ctx");
+    }
+    b->batching = false;
+    (void)commit;  // work is already in flight; results are waited for by memcpy_from_device / synchronize
+    return MARMOT_SUCCESS;
+}
+
+void ops_on_host_range_freed(void *device_ctx, const void *start, size_t length) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || start == nullptr || length == 0) {
+        return;
+    }
+    std::lock_guard<std::mutex> lock(b->mu);
+    const uintptr_t p = (uintptr_t)start;
+    bool synced = false;
+    for (auto it = b->mirrors.begin(); it != b->mirrors.end();) {
+        Mirror &m = it->second;
+        if (m.host < p + length && p < m.host + m.bytes) {
+            if (!synced) {
+                marmot_hip_synchronize(b->dev);  // kernels still reading the mirror finish first
+                synced = true;
+            }
+            auto victim = it++;
+            b->drop(victim);
+        } else {
+            ++it;
+        }
+    }
+}
+
+void ops_on_host_ptr_freed(void *device_ctx, const void *ptr) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || ptr == nullptr) {
+        return;
+    }
+    size_t bytes = 1;
+    {
+        std::lock_guard<std::mutex> lock(b->mu);
+        auto it = b->mirrors.find((uintptr_t)ptr);
+        if (it != b->mirrors.end()) {
+            bytes = it->second.bytes;
+        }
+    }
+    ops_on_host_range_freed(device_ctx, ptr, bytes);
+}
+
+const marmot_device_ops_t k_hip_ops = {
+    ops_init,
+    ops_destroy,
+    ops_configure,
+    ops_alloc,
+    ops_free,
+    ops_memcpy_to_device,
+    ops_memcpy_from_device,
+    ops_synchronize,
+    ops_allocator_usage,
+    ops_graph_batch_begin,
+    ops_graph_batch_end,
+    ops_on_host_ptr_freed,
+    ops_on_host_range_freed,
+};
+
+// ------------------------------------------------------------------ impl functions
+marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind_t expect_kind, const marmot_tensor_t *input,
+                                const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                marmot_tensor_t *out) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || weight == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantized matmul: null argument");
+    }
+    // marmot_matmul_validate_quantized (src/core/helpers/matmul.c:68-136), same order of checks
+    if (!kind_is_block(weight->quant_kind)) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Weight tensor is not block-quantized");
+    }
+    if (weight->quant_layout != MARMOT_QUANT_LAYOUT_GGUF) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized matmul only supports the GGUF layout");
+    }
+    if (!storage_dtype_ok(weight->dtype)) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantized weight uses an unexpected storage dtype");
+    }
+    if (input == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantized matmul: null argument");
+    }
+    if (input->shape.ndim != 2 || weight->shape.ndim != 2 || out->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantized matmul expects 2D tensors");
+    }
+    const bool in32 = input->dtype == MARMOT_DTYPE_FLOAT32, in16 = input->dtype == MARMOT_DTYPE_FLOAT16;
+    const bool out32 = out->dtype == MARMOT_DTYPE_FLOAT32, out16 = out->dtype == MARMOT_DTYPE_FLOAT16;
+    if (!((in32 && out32) || (in16 && (out32 || out16)))) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE,
+                    "Quantized matmul requires FLOAT32 input or FLOAT16 activations with FLOAT16/FLOAT32 output");
+    }
+    const size_t N = input->shape.shape[0], K = input->shape.shape[1], M = weight->shape.shape[0];
+    if (weight->shape.shape[1] != K) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Quantized matmul dimension mismatch on K");
+    }
+    if (out->shape.shape[0] != N || out->shape.shape[1] != M) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Quantized matmul output shape mismatch");
+    }
+    if (weight->quant_kind != expect_kind || !kind_supported_weight(weight->quant_kind)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized matmul: weight scheme not handled by this kernel");
+    }
+    if (!rows_contiguous(input) || !rows_contiguous(out)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized matmul: HIP kernels need contiguous rows");
+    }
+    if (input->data == nullptr || weight->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantized matmul: tensor without data");
+    }
+    const marmot_tensor_t *bias = epilogue != nullptr ? epilogue->bias : nullptr;
+    int bias_dtype = MARMOT_HIP_DTYPE_F32;
+    if (bias != nullptr) {
+        size_t bn = 1;
+        for (size_t i = 0; i < bias->shape.ndim; ++i) {
+            bn *= bias->shape.shape[i];
+        }
+        if (bn != M) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Quantized matmul bias length mismatch");
+        }
+        if (bias->dtype == MARMOT_DTYPE_FLOAT16) {
+            bias_dtype = MARMOT_HIP_DTYPE_F16;
+        } else if (bias->dtype != MARMOT_DTYPE_FLOAT32) {
+            return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantized matmul bias must be FLOAT32 or FLOAT16");
+        }
+    }
+    if (N == 0 || M == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+
+    std::lock_guard<std::mutex> lock(b->mu);
+    const int kind = (int)weight->quant_kind;
+    const void *d_w = nullptr, *d_x = nullptr, *d_b = nullptr;
+    void *d_y = nullptr;
+    marmot_error_t st = b->acquire_read(weight->data, M * marmot_hip_row_bytes(kind, K), &d_w);
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_read(input->data, dense_bytes(input), &d_x);
+    }
+    if (st == MARMOT_SUCCESS && bias != nullptr) {
+        st = b->acquire_read(bias->data, dense_bytes(bias), &d_b);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_write(out->data, dense_bytes(out), &d_y);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    int rc = marmot_hip_matmul_quantized(b->dev, kind, d_w, d_x, in32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, N,
+                                         K, M, d_b, bias_dtype, d_y, out32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16,
+                                         0);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(out);
+    return MARMOT_SUCCESS;
+}
+
+// bytes of E expert slices of [rows, cols] blocks; expert tensors are stored [cols, rows, E] in GGUF order
+// (cpu_moe_execute_grouped, src/backends/cpu/ops/moe/moe_ops.c:895-899)
+size_t expert_tensor_bytes(int kind, size_t rows, size_t cols, size_t experts) {
+    return experts * rows * marmot_hip_row_bytes(kind, cols);
+}
+
+marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_experts_desc_t *desc) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || desc == nullptr || desc->hidden_states == nullptr || desc->gate_exps == nullptr ||
+        desc->up_exps == nullptr || desc->down_exps == nullptr || desc->topk_ids == nullptr ||
+        desc->topk_weights == nullptr || desc->out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "MoE descriptor is incomplete");
+    }
+    const marmot_tensor_t *h = desc->hidden_states, *g = desc->gate_exps, *u = desc->up_exps, *d = desc->down_exps;
+    if (g->quant_kind != u->quant_kind || g->quant_layout != u->quant_layout) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "MoE expert quantization must be consistent across weights");
+    }
+    if (h->dtype != MARMOT_DTYPE_FLOAT32 || desc->topk_weights->dtype != MARMOT_DTYPE_FLOAT32 ||
+        desc->out->dtype != MARMOT_DTYPE_FLOAT32 || desc->topk_ids->dtype != MARMOT_DTYPE_INT32) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "HIP MoE experts need FLOAT32 activations and INT32 expert ids");
+    }
+    if (!kind_supported_weight(g->quant_kind) || !kind_supported_weight(d->quant_kind)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q8_0, Q4_K or Q6_K expert weights");
+    }
+    if (h->shape.ndim != 2 || g->shape.ndim != 3 || u->shape.ndim != 3 || d->shape.ndim != 3 ||
+        desc->topk_ids->shape.ndim != 2 || desc->topk_weights->shape.ndim != 2 || desc->out->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "MoE experts: unexpected tensor ranks");
+    }
+    const size_t T = h->shape.shape[0], H = h->shape.shape[1];
+    const size_t F = g->shape.shape[1], E = g->shape.shape[2], k = desc->topk_ids->shape.shape[1];
+    if (g->shape.shape[0] != H || u->shape.shape[0] != H || u->shape.shape[1] != F || u->shape.shape[2] != E ||
+        d->shape.shape[0] != F || d->shape.shape[1] != H || d->shape.shape[2] != E ||
+        desc->topk_ids->shape.shape[0] != T || desc->topk_weights->shape.shape[0] != T ||
+        desc->topk_weights->shape.shape[1] != k || desc->out->shape.shape[0] != T ||
+        desc->out->shape.shape[1] != H) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "MoE experts: tensor shapes do not agree");
+    }
+    if (!rows_contiguous(h) || !rows_contiguous(desc->out) || !rows_contiguous(desc->topk_ids) ||
+        !rows_contiguous(desc->topk_weights)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "MoE experts: HIP kernels need contiguous rows");
+    }
+    if (T == 0) {
+        mark_device_output(desc->out);
+        return MARMOT_SUCCESS;
+    }
+    std::lock_guard<std::mutex> lock(b->mu);
+    const int kgu = (int)g->quant_kind, kd = (int)d->quant_kind;
+    const void *d_h = nullptr, *d_g = nullptr, *d_u = nullptr, *d_d = nullptr, *d_ids = nullptr, *d_wts = nullptr;
+    void *d_out = nullptr;
+    marmot_error_t st = b->acquire_read(h->data, dense_bytes(h), &d_h);
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_read(g->data, expert_tensor_bytes(kgu, F, H, E), &d_g);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_read(u->data, expert_tensor_bytes(kgu, F, H, E), &d_u);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_read(d->data, expert_tensor_bytes(kd, H, F, E), &d_d);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_read(desc->topk_ids->data, dense_bytes(desc->topk_ids), &d_ids);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_read(desc->topk_weights->data, dense_bytes(desc->topk_weights), &d_wts);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_write(desc->out->data, dense_bytes(desc->out), &d_out);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    int rc = marmot_hip_moe_experts(b->dev, (const float *)d_h, T, H, F, E, k, kgu, kd, d_g, d_u, d_d,
+                                    (const int32_t *)d_ids, (const float *)d_wts, desc->weights_scale,
+                                    (int)desc->router_weight_policy, (int)desc->ffn_type, (float *)d_out);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(desc->out);
+    return MARMOT_SUCCESS;
+}
+
+marmot_error_t topk(const void *device_ctx, const marmot_topk_desc_t *desc) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || desc == nullptr || desc->x == nullptr || desc->values_out == nullptr ||
+        desc->indices_out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "TopK descriptor is incomplete");
+    }
+    const marmot_tensor_t *x = desc->x;
+    if (x->shape.ndim != 2 || desc->values_out->shape.ndim != 2 || desc->indices_out->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "TopK expects 2D tensors");
+    }
+    if (desc->axis != 1 && desc->axis != -1) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "TopK is implemented over the last axis");
+    }
+    if (x->dtype != MARMOT_DTYPE_FLOAT32 || desc->values_out->dtype != MARMOT_DTYPE_FLOAT32 ||
+        desc->indices_out->dtype != MARMOT_DTYPE_INT32) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "HIP TopK needs FLOAT32 values and INT32 indices");
+    }
+    const size_t rows = x->shape.shape[0], cols = x->shape.shape[1], k = desc->k;
+    // cpu_topk_impl, src/backends/cpu/ops/moe/moe_ops.c:813-820
+    if (k == 0 || k > cols || desc->values_out->shape.shape[0] != rows || desc->indices_out->shape.shape[0] != rows ||
+        desc->values_out->shape.shape[1] != k || desc->indices_out->shape.shape[1] != k) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "TopK output shape mismatch");
+    }
+    if (!rows_contiguous(x) || !rows_contiguous(desc->values_out) || !rows_contiguous(desc->indices_out)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "TopK: HIP kernel needs contiguous rows");
+    }
+    if (rows == 0) {
+        return MARMOT_SUCCESS;
+    }
+    std::lock_guard<std::mutex> lock(b->mu);
+    const void *d_x = nullptr;
+    void *d_v = nullptr, *d_i = nullptr;
+    marmot_error_t st = b->acquire_read(x->data, dense_bytes(x), &d_x);
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_write(desc->values_out->data, dense_bytes(desc->values_out), &d_v);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_write(desc->indices_out->data, dense_bytes(desc->indices_out), &d_i);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    int rc = marmot_hip_topk(b->dev, (const float *)d_x, rows, cols, k, (float *)d_v, (int32_t *)d_i);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(desc->values_out);
+    mark_device_output(desc->indices_out);
+    return MARMOT_SUCCESS;
+}
+
+marmot_error_t quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || input == nullptr || output == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize: null argument");
+    }
+    if (output->quant_kind != MARMOT_QUANT_KIND_Q8_0 && output->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP quantize produces the activation formats Q8_0 and Q8_K");
+    }
+    if (input->dtype != MARMOT_DTYPE_FLOAT32 && input->dtype != MARMOT_DTYPE_FLOAT16) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantize input must be FLOAT32 or FLOAT16");
+    }
+    if (input->shape.ndim != 2 || !rows_contiguous(input)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize expects a contiguous 2D input");
+    }
+    const size_t rows = input->shape.shape[0], k = input->shape.shape[1];
+    const int kind = (int)output->quant_kind;
+    const size_t out_bytes = rows * marmot_hip_row_bytes(kind, k);
+    if (rows == 0 || k == 0) {
+        return MARMOT_SUCCESS;
+    }
+    std::lock_guard<std::mutex> lock(b->mu);
+    const void *d_x = nullptr;
+    void *d_q = nullptr;
+    marmot_error_t st = b->acquire_read(input->data, dense_bytes(input), &d_x);
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_write(output->data, out_bytes, &d_q);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    int rc = marmot_hip_quantize_activations(
+        b->dev, kind, d_x, input->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, rows, k,
+        d_q);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(output);
+    return MARMOT_SUCCESS;
+}
+
+marmot_error_t dequantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || input == nullptr || output == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize: null argument");
+    }
+    if (!kind_supported_weight(input->quant_kind) && input->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q8_0, Q4_K, Q6_K and Q8_K");
+    }
+    if (output->dtype != MARMOT_DTYPE_FLOAT32) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Dequantize output must be FLOAT32");
+    }
+    if (output->shape.ndim != 2 || !rows_contiguous(output)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize expects a contiguous 2D output");
+    }
+    const size_t rows = output->shape.shape[0], k = output->shape.shape[1];
+    if (input->shape.ndim == 2 && (input->shape.shape[0] != rows || input->shape.shape[1] != k)) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Dequantize shape mismatch");
+    }
+    if (rows == 0 || k == 0) {
+        return MARMOT_SUCCESS;
+    }
+    const int kind = (int)input->quant_kind;
+    std::lock_guard<std::mutex> lock(b->mu);
+    const void *d_q = nullptr;
+    void *d_y = nullptr;
+    marmot_error_t st = b->acquire_read(input->data, rows * marmot_hip_row_bytes(kind, k), &d_q);
+    if (st == MARMOT_SUCCESS) {
+        st = b->acquire_write(output->data, dense_bytes(output), &d_y);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    int rc = marmot_hip_dequantize(b->dev, kind, d_q, rows, k, (float *)d_y);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(output);
+    return MARMOT_SUCCESS;
+}
+
+// ------------------------------------------------------------------ bytecode exec entries
+inline uint16_t rd_u16(const uint8_t **pc) {
+    const uint16_t v = (uint16_t)((*pc)[0] | ((*pc)[1] << 8));
+    *pc += 2;
+    return v;
+}
+inline uint32_t rd_u32(const uint8_t **pc) {
+    const uint32_t v = (uint32_t)(*pc)[0] | ((uint32_t)(*pc)[1] << 8) | ((uint32_t)(*pc)[2] << 16) |
+        ((uint32_t)(*pc)[3] << 24);
+    *pc += 4;
+    return v;
+}
+inline float rd_f32(const uint8_t **pc) {
+    const uint32_t bits = rd_u32(pc);
+    float f;
+    memcpy(&f, &bits, sizeof(f));
+    return f;
+}
+
+inline marmot_tensor_t *reg(marmot_tensor_t **regs, uint16_t idx) {
+    return idx == MARMOT_BC_REG_INVALID ? nullptr : regs[idx];
+}
+
+bool exec_args_ok(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm) {
+    const marmot_bc_exec_ctx_t *c = (const marmot_bc_exec_ctx_t *)exec_ctx;
+    return c != nullptr && c->device_ctx != nullptr && regs != nullptr && imm != nullptr;
+}
+
+template <marmot_quant_kind_t KIND>
+marmot_error_t bc_exec_matmul(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                              const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const void *device_ctx = ((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx;
+    const uint8_t *pc = imm;
+    const uint16_t input_idx = rd_u16(&pc);
+    const uint16_t weight_idx = rd_u16(&pc);
+    const uint16_t bias_idx = rd_u16(&pc);
+    const uint32_t epilogue_off = rd_u32(&pc);
+    const uint16_t output_idx = rd_u16(&pc);
+    marmot_matmul_epilogue_t epilogue;
+    const marmot_matmul_epilogue_t *epilogue_ptr = nullptr;
+    if (epilogue_off != MARMOT_BC_INVALID_OFFSET) {
+        if (const_pool == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for matmul epilogue");
+        }
+        memcpy(&epilogue, const_pool + epilogue_off, sizeof(epilogue));
+        epilogue_ptr = &epilogue;
+    }
+    if (bias_idx != MARMOT_BC_REG_INVALID) {
+        if (epilogue_ptr == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Missing matmul epilogue");
+        }
+        epilogue.bias = reg(regs, bias_idx);  // the register wins over the pointer frozen into the pool
+    }
+    return matmul_quantized(device_ctx, KIND, reg(regs, input_idx), reg(regs, weight_idx), epilogue_ptr,
+                            reg(regs, output_idx));
+}
+
+marmot_error_t bc_exec_moe(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    marmot_moe_experts_desc_t desc;
+    memset(&desc, 0, sizeof(desc));
+    desc.hidden_states = reg(regs, rd_u16(&pc));
+    desc.gate_exps = reg(regs, rd_u16(&pc));
+    desc.up_exps = reg(regs, rd_u16(&pc));
+    desc.down_exps = reg(regs, rd_u16(&pc));
+    desc.topk_ids = reg(regs, rd_u16(&pc));
+    desc.topk_weights = reg(regs, rd_u16(&pc));
+    desc.out = reg(regs, rd_u16(&pc));
+    desc.ffn_type = (marmot_ffn_type_t)rd_u32(&pc);
+    desc.weights_scale = rd_f32(&pc);
+    desc.router_weight_policy = (marmot_router_weight_policy_t)rd_u32(&pc);
+    return moe_experts(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
+}
+
+marmot_error_t bc_exec_topk(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    marmot_topk_desc_t desc;
+    desc.x = reg(regs, rd_u16(&pc));
+    desc.values_out = reg(regs, rd_u16(&pc));
+    desc.indices_out = reg(regs, rd_u16(&pc));
+    desc.axis = (int32_t)rd_u32(&pc);
+    desc.k = rd_u32(&pc);
+    return topk(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
+}
+
+marmot_error_t bc_exec_quantize(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *input = reg(regs, rd_u16(&pc));
+    (void)rd_u32(&pc);  // quant params: unused by the block formats
+    marmot_tensor_t *output = reg(regs, rd_u16(&pc));
+    const uint32_t kind = rd_u32(&pc);
+    const uint32_t layout = rd_u32(&pc);
+    if (output != nullptr && ((uint32_t)output->quant_kind != kind || layout != MARMOT_QUANT_LAYOUT_GGUF)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize: kind/layout immediates disagree with the output tensor");
+    }
+    return quantize_block(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, input, output);
+}
+
+marmot_error_t bc_exec_dequantize(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *input = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *output = reg(regs, rd_u16(&pc));
+    const uint32_t kind = rd_u32(&pc);
+    const uint32_t layout = rd_u32(&pc);
+    if (input != nullptr && ((uint32_t)input->quant_kind != kind || layout != MARMOT_QUANT_LAYOUT_GGUF)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize: kind/layout immediates disagree with the input tensor");
+    }
+    return dequantize_block(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, input, output);
+}
+
+const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
+    0,                      // END
+    12, 12, 12, 12,         // MATMUL: 3 x u16 + u32 + u16
+    26, 26, 26, 26,         // MOE_EXPERTS: 7 x u16 + u32 + f32 + u32
+    14,                     // TOPK: 3 x u16 + 2 x u32
+    16,                     // QUANTIZE: u16 + u32 + u16 + 2 x u32
+    12,                     // DEQUANTIZE: 2 x u16 + 2 x u32
+};
+
+const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
+    MARMOT_BC_SCHEMA_INVALID,
+    MARMOT_BC_SCHEMA_MATMUL, MARMOT_BC_SCHEMA_MATMUL, MARMOT_BC_SCHEMA_MATMUL, MARMOT_BC_SCHEMA_MATMUL,
+    MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS,
+    MARMOT_BC_SCHEMA_MOE_EXPERTS,
+    MARMOT_BC_SCHEMA_TOPK,
+    MARMOT_BC_SCHEMA_QUANTIZE,
+    MARMOT_BC_SCHEMA_DEQUANTIZE,
+};
+
+const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
+    nullptr,
+    bc_exec_matmul<MARMOT_QUANT_KIND_Q4_0>, bc_exec_matmul<MARMOT_QUANT_KIND_Q8_0>,
+    bc_exec_matmul<MARMOT_QUANT_KIND_Q4_K>, bc_exec_matmul<MARMOT_QUANT_KIND_Q6_K>,
+    bc_exec_moe, bc_exec_moe, bc_exec_moe, bc_exec_moe,
+    bc_exec_topk,
+    bc_exec_quantize,
+    bc_exec_dequantize,
+};
+
+// ------------------------------------------------------------------ kernel query
+marmot_kernel_selection_t unsupported(const char *reason) {
+    marmot_kernel_selection_t s;
+    memset(&s, 0, sizeof(s));
+    s.supported = false;
+    s.kernel_id = MARMOT_KERNEL_INVALID;
+    s.op_index = MARMOT_KERNEL_OP_INDEX_INVALID;
+    s.fallback_reason = reason;
+    return s;
+}
+
+marmot_kernel_selection_t selected(uint16_t op_index, double est_us, double workspace_mb) {
+    marmot_kernel_selection_t s;
+    memset(&s, 0, sizeof(s));
+    s.supported = true;
+    s.kernel_id = (marmot_kernel_id_t)(MARMOT_KERNEL_HIP_BASE + op_index);
+    s.op_index = op_index;
+    s.estimated_us = est_us;
+    s.est_workspace_mb = workspace_mb;
+    s.confidence = 0.8f;
+    return s;
+}
+
+int kind_of_scheme(marmot_qscheme_id_t q) {
+    switch (q) {
+    case MARMOT_QSCHEME_Q4_0:
+        return MARMOT_HIP_KIND_Q4_0;
+    case MARMOT_QSCHEME_Q8_0:
+        return MARMOT_HIP_KIND_Q8_0;
+    case MARMOT_QSCHEME_Q4_K:
+        return MARMOT_HIP_KIND_Q4_K;
+    case MARMOT_QSCHEME_Q6_K:
+        return MARMOT_HIP_KIND_Q6_K;
+    case MARMOT_QSCHEME_Q8_K:
+        return MARMOT_HIP_KIND_Q8_K;
+    default:
+        return 0;
+    }
+}
+
+uint16_t matmul_op_of_kind(int kind) {
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_0:
+        return MARMOT_HIP_BC_OP_MATMUL_Q4_0;
+    case MARMOT_HIP_KIND_Q8_0:
+        return MARMOT_HIP_BC_OP_MATMUL_Q8_0;
+    case MARMOT_HIP_KIND_Q4_K:
+        return MARMOT_HIP_BC_OP_MATMUL_Q4_K;
+    case MARMOT_HIP_KIND_Q6_K:
+        return MARMOT_HIP_BC_OP_MATMUL_Q6_K;
+    default:
+        return MARMOT_KERNEL_OP_INDEX_INVALID;
+    }
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ exports
+extern "C" {
+
+const marmot_device_ops_t *marmot_get_hip_ops(void) {
+    return &k_hip_ops;
+}
+
+marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *sig, const marmot_device_caps_t *caps) {
+    if (sig == nullptr || caps == nullptr) {
+        return unsupported("Invalid kernel query arguments");
+    }
+    const float bw_gbps = caps->mem_bw_gbps > 0.0f ? caps->mem_bw_gbps : 8000.0f;
+    const float tflops = caps->peak_flops_tflops_fp16 > 0.0f ? caps->peak_flops_tflops_fp16 : 2500.0f;
+    const double launch_us = caps->launch_overhead_us > 0.0f ? caps->launch_overhead_us : 2.0;
+    const bool in32 = sig->input_dtype == MARMOT_DTYPE_FLOAT32, in16 = sig->input_dtype == MARMOT_DTYPE_FLOAT16;
+    const bool out32 = sig->output_dtype == MARMOT_DTYPE_FLOAT32, out16 = sig->output_dtype == MARMOT_DTYPE_FLOAT16;
+    switch (sig->op_id) {
+    case MARMOT_OP_MATMUL:
+    case MARMOT_OP_LINEAR: {
+        const int kind = kind_of_scheme(sig->qscheme_id);
+        const uint16_t op = matmul_op_of_kind(kind);
+        if (op == MARMOT_KERNEL_OP_INDEX_INVALID) {
+            return unsupported("HIP matmul handles Q4_0, Q8_0, Q4_K and Q6_K weights");
+        }
+        if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
+            return unsupported("HIP quantized matmul needs layout NT");
+        }
+        if (!((in32 && out32) || (in16 && (out32 || out16)))) {
+            return unsupported("HIP quantized matmul: unsupported activation/output dtypes");
+        }
+        if (sig->accum_dtype != MARMOT_DTYPE_FLOAT32) {
+            return unsupported("HIP quantized matmul accumulates in FLOAT32");
+        }
+        if (sig->weight_layout != MARMOT_WEIGHT_LAYOUT_SEPARATE) {
+            return unsupported("HIP quantized matmul needs separate weights");
+        }
+        if (sig->stride_mode != MARMOT_STRIDE_MODE_CONTIGUOUS && sig->stride_mode != MARMOT_STRIDE_MODE_ANY) {
+            return unsupported("HIP quantized matmul needs contiguous rows");
+        }
+        if ((sig->epilogue_flags & ~(uint32_t)MARMOT_EPILOGUE_BIAS) != 0 || sig->variant_flags != 0) {
+            return unsupported("HIP quantized matmul fuses only the bias epilogue");
+        }
+        if (kind == MARMOT_HIP_KIND_Q6_K && in16) {
+            return unsupported("HIP Q6_K matmul takes FLOAT32 activations");
+        }
+        const size_t N = sig->dims.matmul.N, K = sig->dims.matmul.K, M = sig->dims.matmul.M;
+        const double bytes =
+            (double)M * (double)marmot_hip_row_bytes(kind, K) + (double)N * K * (in32 ? 4 : 2) + (double)N * M * 4;
+        const double t_mem = bytes / (bw_gbps * 1e3);          // us
+        const double t_mma = 2.0 * N * M * K / (tflops * 1e6);  // us
+        const double ws_mb = in32 ? (double)marmot_hip_packed_activation_bytes(kind, N, K) / 1048576.0 : 0.0;
+        return selected(op, launch_us + (t_mem > t_mma ? t_mem : t_mma), ws_mb);
+    }
+    case MARMOT_OP_MOE_EXPERTS: {
+        const int kind = kind_of_scheme(sig->qscheme_id);
+        if (matmul_op_of_kind(kind) == MARMOT_KERNEL_OP_INDEX_INVALID) {
+            return unsupported("HIP MoE experts handle Q4_0, Q8_0, Q4_K and Q6_K expert weights");
+        }
+        if (!in32 || !out32) {
+            return unsupported("HIP MoE experts take FLOAT32 activations");
+        }
+        const uint16_t op = (uint16_t)(MARMOT_HIP_BC_OP_MOE_EXPERTS_Q4_0 +
+                                       (matmul_op_of_kind(kind) - MARMOT_HIP_BC_OP_MATMUL_Q4_0));
+        return selected(op, 0.0, 0.0);
+    }
+    case MARMOT_OP_TOPK:
+        if (!in32 || !out32) {
+            return unsupported("HIP TopK takes FLOAT32 values");
+        }
+        return selected(MARMOT_HIP_BC_OP_TOPK_F32, launch_us, 0.0);
+    case MARMOT_OP_QUANTIZE:
+        if (!(in32 || in16) ||
+            (sig->qscheme_id != MARMOT_QSCHEME_Q8_0 && sig->qscheme_id != MARMOT_QSCHEME_Q8_K)) {
+            return unsupported("HIP quantize produces Q8_0 and Q8_K from FLOAT32/FLOAT16");
+        }
+        return selected(MARMOT_HIP_BC_OP_QUANTIZE_BLOCK, launch_us, 0.0);
+    case MARMOT_OP_DEQUANTIZE:
+        if (kind_of_scheme(sig->qscheme_id) == 0 || !out32) {
+            return unsupported("HIP dequantize handles Q4_0, Q8_0, Q4_K, Q6_K and Q8_K to FLOAT32");
+        }
+        return selected(MARMOT_HIP_BC_OP_DEQUANTIZE_BLOCK, launch_us, 0.0);
+    default:
+        return unsupported("Operation not provided by the HIP backend");
+    }
+}
+
+marmot_device_caps_t marmot_hip_detect_default_caps(void) {
+    marmot_device_caps_t c;
+    memset(&c, 0, sizeof(c));
+    // published MI355X figures; a live device refines the counts
+    c.peak_flops_tflops_fp32 = 157.3f;
+    c.peak_flops_tflops_fp16 = 2500.0f;
+    c.mem_bw_gbps = 8000.0f;
+    c.launch_overhead_us = 2.0f;
+    c.edge_penalty_alpha = 0.0f;
+    c.l1_cache_kb = 32;
+    c.l2_cache_kb = 4096;
+    c.l3_cache_mb = 256;
+    c.num_compute_units = 256;
+    c.simd_width = 64;
+    c.has_fma = true;
+    c.has_fp16_compute = true;
+    c.has_bf16_compute = true;
+    c.has_tensor_cores = true;
+    c.has_simdgroup_mm = false;
+    c.h2d_bw_gbps = 64.0f;
+    c.d2h_bw_gbps = 64.0f;
+    c.d2d_bw_gbps = 4000.0f;
+    c.d2d_lat_us = 2.0f;
+    c.copy_engines = 2;
+    c.max_streams = 4;
+    marmot_hip_device_t *dev = nullptr;
+    if (marmot_hip_device_create(0, &dev) == MARMOT_HIP_SUCCESS) {
+        marmot_hip_caps_t hc;
+        if (marmot_hip_get_caps(dev, &hc) == MARMOT_HIP_SUCCESS) {
+            c.num_compute_units = hc.num_compute_units;
+            c.simd_width = hc.wavefront_size;
+            c.l2_cache_kb = hc.l2_cache_kb;
+            c.mem_bw_gbps = hc.mem_bw_gbps;
+            c.peak_flops_tflops_fp16 = hc.peak_tflops_fp16;
+        }
+        marmot_hip_device_destroy(dev);
+    }
+    return c;
+}
+
+bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_backend_preferences_t *prefs_out) {
+    if (caps == nullptr || prefs_out == nullptr) {
+        return false;
+    }
+    memset(prefs_out, 0, sizeof(*prefs_out));
+    prefs_out->policy.embedding_quant_output_dtype = MARMOT_DTYPE_FLOAT32;
+    prefs_out->policy.quant_activation_mode = MARMOT_QUANT_ACTIVATION_AUTO;
+    prefs_out->policy.variant_flags_mask = 0;  // no fused variants yet
+    prefs_out->policy.embedding_prefer_gpu_private = false;
+    prefs_out->policy.embedding_allow_quant_decode_on_the_fly = false;
+    // views into a mirrored range resolve to offsets in the mirror, so offset views need no temporaries
+    prefs_out->policy.matmul_requires_temp_tensors = false;
+    prefs_out->policy.matmul_prefer_packed_weights = false;  // kernels read native GGUF blocks
+    prefs_out->routing_policy = MARMOT_ROUTING_ALWAYS_GPU;
+    return true;
+}
+
+bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out) {
+    if (out == nullptr) {
+        return false;
+    }
+    out->imm_size = k_imm_size;
+    out->exec_table = k_exec_table;
+    out->schema_id = k_schema_id;
+    out->op_count = MARMOT_HIP_BC_OP_COUNT;
+    return true;
+}
+
+marmot_error_t hip_matmul_quantized_q4_0(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q4_0, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_quantized_q8_0(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q8_0, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_quantized_q4_k(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q4_K, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_quantized_q6_k(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q6_K, input, weight, epilogue, out);
+}
+marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc) {
+    return moe_experts(device_ctx, desc);
+}
+marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc) {
+    return topk(device_ctx, desc);
+}
+marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
+    return quantize_block(device_ctx, input, output);
+}
+marmot_error_t hip_dequantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
+    return dequantize_block(device_ctx, input, output);
+}
+
+marmot_error_t marmot_hip_backend_last_error(const char **detail_out) {
+#ifdef MARMOT_HIP_IN_TREE
+    if (detail_out != nullptr) {
+        *detail_out = marmot_get_last_error_detail();
+    }
+    return marmot_get_last_error();
+#else
+    if (detail_out != nullptr) {
+        *detail_out = g_last_detail;
+    }
+    return g_last_code;
+#endif
+}
+
+void marmot_hip_backend_residency_stats(const void *device_ctx, marmot_hip_residency_stats_t *out) {
+    Backend *b = backend_of(device_ctx);
+    if (b == nullptr || out == nullptr) {
+        return;
+    }
+    std::lock_guard<std::mutex> lock(b->mu);
+    out->mirrors = b->mirrors.size();
+    out->mirrored_bytes = b->mirrored_bytes;
+    out->uploads = b->uploads;
+    out->upload_bytes = b->upload_bytes;
+    out->downloads = b->downloads;
+    out->download_bytes = b->download_bytes;
+}
+
+}  // extern "C"

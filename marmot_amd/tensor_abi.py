@@ -1,0 +1,454 @@
+"""Caller side of the marmot_tensor_t-level HIP backend, for tests and harnesses outside the marmot tree.
+
+It plays the part marmot's core plays for a backend: builds ``marmot_tensor_t`` objects over host buffers with the
+reference's exact struct layout, fills ``marmot_op_signature_t`` the way ``marmot_matmul_build`` does
+(src/core/dispatch/matmul_build.c:86-146), asks ``marmot_hip_query_kernel`` for an op index, encodes bytecode
+immediates as ``marmot_bc_compile`` does (src/core/bytecode/bytecode_compile.c:459-504, 628-669, 912-962) and runs
+the program against the tables of ``marmot_hip_bc_get_tables`` with the loop of ``marmot_bc_execute``
+(src/core/bytecode/bytecode.c:196-290). Tensor data moves only through the device vtable
+(``memcpy_to_device(p, p)`` = "host copy is newer", ``memcpy_from_device(p, p)`` = "make the host copy current",
+src/core/tensor/transfer.c:22, 49-55).
+
+The struct definitions mirror include/marmot_hip_backend.h member for member.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import struct
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from . import capi
+
+MAX_DIMS = 8
+
+# marmot_error_t
+SUCCESS, INVALID_ARGUMENT, OUT_OF_MEMORY, DEVICE_NOT_AVAILABLE, BACKEND_INIT_FAILED = 0, -1, -2, -3, -4
+INVALID_OPERATION, UNSUPPORTED_DTYPE, DIMENSION_MISMATCH, NOT_IMPLEMENTED = -5, -6, -7, -8
+# marmot_dtype_t
+DTYPE_F32, DTYPE_F16, DTYPE_I32, DTYPE_I8, DTYPE_U8 = 0, 1, 3, 5, 6
+# marmot_quant_kind_t / marmot_quant_layout_t / marmot_memory_location_t
+KIND_GENERIC, KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_K = 0, 1, 5, 9, 11, 12
+LAYOUT_GENERIC, LAYOUT_GGUF = 0, 1
+MEMORY_HOST, MEMORY_DEVICE = 0, 1
+BACKEND_HIP = 3
+# marmot_op_id_t / marmot_qscheme_id_t
+OP_DEQUANTIZE, OP_MOE_EXPERTS, OP_MATMUL, OP_QUANTIZE, OP_LINEAR, OP_TOPK = 210, 263, 498, 524, 708, 901
+QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q8_0: 5, KIND_Q4_K: 8, KIND_Q6_K: 10, KIND_Q8_K: 11}
+PROFILE_SCALAR = 4
+MATMUL_LAYOUT_NT = 2
+WEIGHT_LAYOUT_SEPARATE = 1
+EPILOGUE_BIAS = 1
+BC_END, BC_REG_INVALID, BC_INVALID_OFFSET = 0, 0xFFFF, 0xFFFFFFFF
+
+_NP_OF_DTYPE = {DTYPE_F32: np.float32, DTYPE_F16: np.float16, DTYPE_I32: np.int32, DTYPE_I8: np.int8,
+                DTYPE_U8: np.uint8}
+_DTYPE_OF_NP = {np.dtype(v): k for k, v in _NP_OF_DTYPE.items()}
+
+
+class Shape(C.Structure):
+    _fields_ = [("ndim", C.c_size_t), ("shape", C.c_size_t * MAX_DIMS), ("strides", C.c_size_t * MAX_DIMS)]
+
+
+class Tensor(C.Structure):
+    _fields_ = [
+        ("shape", Shape), ("dtype", C.c_int), ("data", C.c_void_p), ("capacity_bytes", C.c_size_t),
+        ("owns_data", C.c_bool), ("quant_params", C.c_void_p), ("quant_kind", C.c_int), ("quant_layout", C.c_int),
+        ("backend", C.c_int), ("ctx", C.c_void_p), ("memory_location", C.c_int), ("needs_sync", C.c_bool),
+        ("packed_data", C.c_void_p), ("packed_src_data", C.c_void_p), ("packed_bytes", C.c_size_t),
+        ("packed_row_bytes", C.c_size_t), ("packed_rows", C.c_size_t),
+    ]
+
+
+class Epilogue(C.Structure):
+    _fields_ = [("bias", C.POINTER(Tensor)), ("enable_output_cast", C.c_bool), ("output_dtype", C.c_int)]
+
+
+class TopkDesc(C.Structure):
+    _fields_ = [("x", C.POINTER(Tensor)), ("values_out", C.POINTER(Tensor)), ("indices_out", C.POINTER(Tensor)),
+                ("axis", C.c_int32), ("k", C.c_uint32)]
+
+
+class MoeDesc(C.Structure):
+    _fields_ = [(n, C.POINTER(Tensor)) for n in
+                ("hidden_states", "gate_exps", "up_exps", "down_exps", "topk_ids", "topk_weights", "out")] + [
+        ("ffn_type", C.c_int), ("weights_scale", C.c_float), ("router_weight_policy", C.c_int)]
+
+
+class MatmulDims(C.Structure):
+    _fields_ = [("N", C.c_size_t), ("K", C.c_size_t), ("M", C.c_size_t)]
+
+
+class SoftmaxDims(C.Structure):
+    _fields_ = [("axis_size", C.c_uint32), ("inner_stride", C.c_uint32), ("outer_size", C.c_uint32),
+                ("row_count", C.c_uint32)]
+
+
+class SigDims(C.Union):
+    _fields_ = [("matmul", MatmulDims), ("softmax", SoftmaxDims)]
+
+
+class QuantBlock(C.Structure):
+    _fields_ = [("block_size", C.c_uint32), ("group_size", C.c_uint32), ("scale_dtype", C.c_int),
+                ("zero_point_dtype", C.c_int)]
+
+
+class OpSignature(C.Structure):
+    _fields_ = [
+        ("op_id", C.c_int), ("profile_id", C.c_int), ("matmul_layout", C.c_int), ("input_dtype", C.c_int),
+        ("weight_dtype", C.c_int), ("output_dtype", C.c_int), ("accum_dtype", C.c_int), ("qscheme_id", C.c_int),
+        ("quant_block", QuantBlock), ("weight_layout", C.c_int), ("stride_mode", C.c_int),
+        ("epilogue_flags", C.c_uint32), ("activation", C.c_int), ("variant_flags", C.c_uint32), ("dims", SigDims),
+    ]
+
+
+class KernelSelection(C.Structure):
+    _fields_ = [
+        ("supported", C.c_bool), ("kernel_id", C.c_int), ("op_index", C.c_uint16), ("estimated_us", C.c_double),
+        ("est_comm_us", C.c_double), ("est_workspace_mb", C.c_double), ("confidence", C.c_float),
+        ("fallback_reason", C.c_char_p), ("shardable_axes", C.c_uint32), ("device_affinity", C.c_uint32),
+    ]
+
+
+class _CapsApple(C.Structure):
+    _fields_ = [("has_amx", C.c_bool), ("neural_engine_tops", C.c_uint32), ("has_arm_bf16", C.c_bool),
+                ("has_arm_dotprod", C.c_bool), ("has_arm_sve", C.c_bool), ("cpu_microarch", C.c_int)]
+
+
+class _CapsCuda(C.Structure):
+    _fields_ = [("sm_count", C.c_uint32), ("shared_mem_kb", C.c_uint32), ("compute_capability", C.c_uint32)]
+
+
+class _CapsBackend(C.Union):
+    _fields_ = [("apple", _CapsApple), ("cuda", _CapsCuda)]
+
+
+class _CapsTopology(C.Structure):
+    _fields_ = [("total_cores", C.c_uint32), ("p_cores", C.c_uint32), ("e_cores", C.c_uint32),
+                ("is_hybrid", C.c_bool)]
+
+
+class DeviceCaps(C.Structure):
+    _fields_ = [
+        ("peak_flops_tflops_fp32", C.c_float), ("peak_flops_tflops_fp16", C.c_float), ("mem_bw_gbps", C.c_float),
+        ("launch_overhead_us", C.c_float), ("edge_penalty_alpha", C.c_float),
+        ("l1_cache_kb", C.c_uint32), ("l2_cache_kb", C.c_uint32), ("l3_cache_mb", C.c_uint32),
+        ("num_compute_units", C.c_uint32), ("simd_width", C.c_uint32),
+        ("has_fma", C.c_bool), ("has_fp16_compute", C.c_bool), ("has_bf16_compute", C.c_bool),
+        ("has_tensor_cores", C.c_bool), ("has_simdgroup_mm", C.c_bool),
+        ("h2d_bw_gbps", C.c_float), ("d2h_bw_gbps", C.c_float), ("d2d_bw_gbps", C.c_float),
+        ("d2d_lat_us", C.c_float), ("copy_engines", C.c_uint32), ("max_streams", C.c_uint32),
+        ("calib_dequant_us_q4k", C.c_float), ("calib_dequant_us_q5k", C.c_float),
+        ("calib_dequant_us_q6k", C.c_float), ("calib_dequant_us_q8_0", C.c_float),
+        ("calib_epilogue_scale", C.c_float),
+        ("backend", _CapsBackend), ("topology", _CapsTopology),
+    ]
+
+
+class ContextPolicy(C.Structure):
+    _fields_ = [("embedding_quant_output_dtype", C.c_int), ("quant_activation_mode", C.c_int),
+                ("variant_flags_mask", C.c_uint32), ("embedding_prefer_gpu_private", C.c_bool),
+                ("embedding_allow_quant_decode_on_the_fly", C.c_bool), ("matmul_requires_temp_tensors", C.c_bool),
+                ("matmul_prefer_packed_weights", C.c_bool)]
+
+
+class BackendPreferences(C.Structure):
+    _fields_ = [("policy", ContextPolicy), ("routing_policy", C.c_int)]
+
+
+class AllocatorUsage(C.Structure):
+    _fields_ = [("current_bytes", C.c_size_t), ("peak_bytes", C.c_size_t), ("pooled_bytes", C.c_size_t),
+                ("active_allocations", C.c_size_t), ("peak_allocations", C.c_size_t),
+                ("total_allocations", C.c_uint64), ("pool_hits", C.c_uint64), ("pool_misses", C.c_uint64)]
+
+
+class DeviceOps(C.Structure):
+    _fields_ = [
+        ("init", C.CFUNCTYPE(C.c_int, C.POINTER(C.c_void_p))),
+        ("destroy", C.CFUNCTYPE(None, C.c_void_p)),
+        ("configure", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p)),
+        ("alloc", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p))),
+        ("free", C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)),
+        ("memcpy_to_device", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t)),
+        ("memcpy_from_device", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t)),
+        ("synchronize", C.CFUNCTYPE(C.c_int, C.c_void_p)),
+        ("allocator_usage", C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(AllocatorUsage))),
+        ("graph_batch_begin", C.CFUNCTYPE(C.c_int, C.c_void_p)),
+        ("graph_batch_end", C.CFUNCTYPE(C.c_int, C.c_void_p, C.c_bool)),
+        ("on_host_ptr_freed", C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)),
+        ("on_host_range_freed", C.CFUNCTYPE(None, C.c_void_p, C.c_void_p, C.c_size_t)),
+    ]
+
+
+class BcExecCtx(C.Structure):
+    _fields_ = [("ctx", C.c_void_p), ("device_ctx", C.c_void_p)]
+
+
+BcExecFn = C.CFUNCTYPE(C.c_int, C.c_void_p, C.POINTER(C.POINTER(Tensor)), C.POINTER(C.c_uint8),
+                       C.POINTER(C.c_uint8))
+
+
+class BcTables(C.Structure):
+    _fields_ = [("imm_size", C.POINTER(C.c_uint16)), ("exec_table", C.POINTER(BcExecFn)),
+                ("schema_id", C.POINTER(C.c_int)), ("op_count", C.c_uint16)]
+
+
+class ResidencyStats(C.Structure):
+    _fields_ = [("mirrors", C.c_size_t), ("mirrored_bytes", C.c_size_t), ("uploads", C.c_uint64),
+                ("upload_bytes", C.c_uint64), ("downloads", C.c_uint64), ("download_bytes", C.c_uint64)]
+
+
+#: exported symbols of the tensor-level layer (checked against include/marmot_hip_backend.h by the tests)
+BACKEND_SYMBOLS = [
+    "marmot_get_hip_ops", "marmot_hip_query_kernel", "marmot_hip_detect_default_caps",
+    "marmot_hip_default_preferences", "marmot_hip_bc_get_tables",
+    "hip_matmul_quantized_q4_0", "hip_matmul_quantized_q8_0", "hip_matmul_quantized_q4_k",
+    "hip_matmul_quantized_q6_k", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
+    "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
+]
+
+
+def bind(lib: C.CDLL) -> C.CDLL:
+    """Attach argument/return types of the tensor-level exports to an already loaded libmarmot_hip."""
+    lib.marmot_get_hip_ops.restype = C.POINTER(DeviceOps)
+    lib.marmot_get_hip_ops.argtypes = []
+    lib.marmot_hip_query_kernel.restype = KernelSelection
+    lib.marmot_hip_query_kernel.argtypes = [C.POINTER(OpSignature), C.POINTER(DeviceCaps)]
+    lib.marmot_hip_detect_default_caps.restype = DeviceCaps
+    lib.marmot_hip_detect_default_caps.argtypes = []
+    lib.marmot_hip_default_preferences.restype = C.c_bool
+    lib.marmot_hip_default_preferences.argtypes = [C.POINTER(DeviceCaps), C.POINTER(BackendPreferences)]
+    lib.marmot_hip_bc_get_tables.restype = C.c_bool
+    lib.marmot_hip_bc_get_tables.argtypes = [C.POINTER(BcTables)]
+    for name in ("q4_0", "q8_0", "q4_k", "q6_k"):
+        fn = getattr(lib, f"hip_matmul_quantized_{name}")
+        fn.restype = C.c_int
+        fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Epilogue), C.POINTER(Tensor)]
+    lib.hip_moe_experts_impl.restype = C.c_int
+    lib.hip_moe_experts_impl.argtypes = [C.c_void_p, C.POINTER(MoeDesc)]
+    lib.hip_topk_impl.restype = C.c_int
+    lib.hip_topk_impl.argtypes = [C.c_void_p, C.POINTER(TopkDesc)]
+    for name in ("hip_quantize_block", "hip_dequantize_block"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor)]
+    lib.marmot_hip_backend_last_error.restype = C.c_int
+    lib.marmot_hip_backend_last_error.argtypes = [C.POINTER(C.c_char_p)]
+    lib.marmot_hip_backend_residency_stats.restype = None
+    lib.marmot_hip_backend_residency_stats.argtypes = [C.c_void_p, C.POINTER(ResidencyStats)]
+    return lib
+
+
+class BackendError(RuntimeError):
+    def __init__(self, code: int, detail: str):
+        super().__init__(f"marmot HIP backend error {code}: {detail}")
+        self.code = code
+        self.detail = detail
+
+
+class HostTensor:
+    """A marmot_tensor_t over a numpy host buffer (the buffer is kept alive by this object)."""
+
+    def __init__(self, array: np.ndarray, shape: Sequence[int], dtype: int, quant_kind: int = KIND_GENERIC):
+        self.array = np.ascontiguousarray(array)
+        self.t = Tensor()
+        self.t.shape.ndim = len(shape)
+        stride = 1
+        for i in reversed(range(len(shape))):
+            self.t.shape.shape[i] = shape[i]
+            self.t.shape.strides[i] = stride
+            stride *= shape[i]
+        self.t.dtype = dtype
+        self.t.data = self.array.ctypes.data
+        self.t.capacity_bytes = self.array.nbytes
+        self.t.owns_data = True
+        self.t.quant_kind = quant_kind
+        self.t.quant_layout = LAYOUT_GGUF if quant_kind != KIND_GENERIC else LAYOUT_GENERIC
+        self.t.backend = BACKEND_HIP
+        self.t.memory_location = MEMORY_HOST
+        self.t.needs_sync = False
+
+    @property
+    def ptr(self):
+        return C.pointer(self.t)
+
+    @classmethod
+    def dense(cls, array: np.ndarray) -> "HostTensor":
+        a = np.ascontiguousarray(array)
+        return cls(a, a.shape, _DTYPE_OF_NP[a.dtype])
+
+    @classmethod
+    def empty(cls, shape: Sequence[int], dtype: int) -> "HostTensor":
+        return cls(np.zeros(shape, dtype=_NP_OF_DTYPE[dtype]), shape, dtype)
+
+    @classmethod
+    def quantized(cls, blocks: np.ndarray, shape: Sequence[int], kind: int) -> "HostTensor":
+        """blocks: uint8 GGUF block bytes; shape: logical element shape as marmot stores it ([rows, cols] for a
+        weight, [cols, rows, experts] for an expert stack)."""
+        return cls(np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1), shape, DTYPE_U8, kind)
+
+
+class HipContext:
+    """What marmot_init(MARMOT_BACKEND_HIP) + the tensor transfer helpers amount to for one device."""
+
+    def __init__(self, lib: Optional[C.CDLL] = None):
+        self.lib = bind(lib if lib is not None else capi.load_library())
+        self.ops = self.lib.marmot_get_hip_ops().contents
+        dc = C.c_void_p()
+        self._check(self.ops.init(C.byref(dc)))
+        self.device_ctx = dc
+        self._check(self.ops.configure(self.device_ctx, None))
+        self.exec_ctx = BcExecCtx(C.c_void_p(1), self.device_ctx)  # ctx is opaque to the backend, must be non-null
+        self.tables = BcTables()
+        if not self.lib.marmot_hip_bc_get_tables(C.byref(self.tables)):
+            raise BackendError(INVALID_ARGUMENT, "no bytecode tables")
+
+    def close(self):
+        if self.device_ctx:
+            self.ops.destroy(self.device_ctx)
+            self.device_ctx = C.c_void_p()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def last_error(self):
+        detail = C.c_char_p()
+        code = self.lib.marmot_hip_backend_last_error(C.byref(detail))
+        return code, (detail.value or b"").decode()
+
+    def _check(self, code: int):
+        if code != SUCCESS:
+            raise BackendError(code, self.last_error()[1])
+
+    # --- transfers, as src/core/tensor/transfer.c does them
+    def host_changed(self, t: HostTensor):
+        self._check(self.ops.memcpy_to_device(self.device_ctx, t.t.data, t.t.data, t.array.nbytes))
+        t.t.memory_location = MEMORY_HOST
+        t.t.needs_sync = False
+
+    def to_host(self, t: HostTensor) -> np.ndarray:
+        if t.t.needs_sync:
+            self._check(self.ops.memcpy_from_device(self.device_ctx, t.t.data, t.t.data, t.array.nbytes))
+            t.t.needs_sync = False
+        return t.array
+
+    def host_freed(self, t: HostTensor):
+        self.ops.on_host_ptr_freed(self.device_ctx, t.t.data)
+
+    def synchronize(self):
+        self._check(self.ops.synchronize(self.device_ctx))
+
+    def residency(self) -> ResidencyStats:
+        s = ResidencyStats()
+        self.lib.marmot_hip_backend_residency_stats(self.device_ctx, C.byref(s))
+        return s
+
+    # --- kernel query (src/core/dispatch/matmul_build.c:120-135 for the signature)
+    def matmul_signature(self, x: HostTensor, w: HostTensor, out: HostTensor, bias: bool = False) -> OpSignature:
+        sig = OpSignature()
+        sig.op_id = OP_MATMUL
+        sig.profile_id = PROFILE_SCALAR
+        sig.matmul_layout = MATMUL_LAYOUT_NT
+        sig.input_dtype = x.t.dtype
+        sig.weight_dtype = w.t.dtype
+        sig.output_dtype = out.t.dtype
+        sig.accum_dtype = DTYPE_F32
+        sig.qscheme_id = QSCHEME_OF_KIND.get(w.t.quant_kind, 0)
+        sig.weight_layout = WEIGHT_LAYOUT_SEPARATE
+        sig.epilogue_flags = EPILOGUE_BIAS if bias else 0
+        sig.dims.matmul.N = x.t.shape.shape[0]
+        sig.dims.matmul.K = x.t.shape.shape[1]
+        sig.dims.matmul.M = w.t.shape.shape[0]
+        return sig
+
+    def query(self, sig: OpSignature, caps: Optional[DeviceCaps] = None) -> KernelSelection:
+        caps = caps if caps is not None else self.lib.marmot_hip_detect_default_caps()
+        return self.lib.marmot_hip_query_kernel(C.byref(sig), C.byref(caps))
+
+    # --- bytecode execution (src/core/bytecode/bytecode.c:196-290)
+    def execute(self, program: "Program") -> int:
+        code = bytes(program.code) + struct.pack("<H", BC_END)
+        regs = (C.POINTER(Tensor) * max(1, len(program.regs)))(*[r.ptr for r in program.regs])
+        pool = (C.c_uint8 * max(1, len(program.const_pool))).from_buffer_copy(
+            bytes(program.const_pool) or b"\0")
+        pc, end = 0, len(code)
+        while True:
+            if pc + 2 > end:
+                return INVALID_ARGUMENT  # truncated stream
+            (op,) = struct.unpack_from("<H", code, pc)
+            pc += 2
+            if op == BC_END:
+                return SUCCESS
+            if op >= self.tables.op_count:
+                return INVALID_ARGUMENT
+            n = self.tables.imm_size[op]
+            if pc + n > end:
+                return INVALID_ARGUMENT
+            imm = (C.c_uint8 * max(1, n)).from_buffer_copy(code[pc:pc + n] or b"\0")
+            pc += n
+            fn = self.tables.exec_table[op]
+            if not fn:
+                return NOT_IMPLEMENTED
+            status = fn(C.cast(C.pointer(self.exec_ctx), C.c_void_p), regs, imm, pool)
+            if status != SUCCESS:
+                return status
+
+
+class Program:
+    """Bytecode builder for the schemas the HIP backend executes."""
+
+    def __init__(self):
+        self.code = bytearray()
+        self.const_pool = bytearray()
+        self.regs: List[HostTensor] = []
+        self._keep = []
+
+    def reg(self, t: Optional[HostTensor]) -> int:
+        if t is None:
+            return BC_REG_INVALID
+        for i, r in enumerate(self.regs):
+            if r is t:
+                return i
+        self.regs.append(t)
+        return len(self.regs) - 1
+
+    def _const(self, blob: bytes, align: int) -> int:
+        while len(self.const_pool) % align:
+            self.const_pool.append(0)
+        off = len(self.const_pool)
+        self.const_pool += blob
+        return off
+
+    def matmul(self, op_index: int, x: HostTensor, w: HostTensor, out: HostTensor,
+               bias: Optional[HostTensor] = None, with_epilogue: Optional[bool] = None):
+        with_epilogue = (bias is not None) if with_epilogue is None else with_epilogue
+        off = BC_INVALID_OFFSET
+        if with_epilogue:
+            ep = Epilogue()
+            ep.bias = bias.ptr if bias is not None else None
+            ep.enable_output_cast = False
+            ep.output_dtype = out.t.dtype
+            self._keep.append(ep)
+            off = self._const(bytes(ep), 8)
+        self.code += struct.pack("<HHHHIH", op_index, self.reg(x), self.reg(w), self.reg(bias), off, self.reg(out))
+
+    def moe_experts(self, op_index: int, hidden, gate, up, down, ids, weights, out, ffn_type=0, weights_scale=1.0,
+                    policy=1):
+        self.code += struct.pack("<H7HIfI", op_index, *[self.reg(t) for t in (hidden, gate, up, down, ids, weights,
+                                                                              out)],
+                                 ffn_type, weights_scale, policy)
+
+    def topk(self, op_index: int, x, values, indices, k: int, axis: int = 1):
+        self.code += struct.pack("<HHHHII", op_index, self.reg(x), self.reg(values), self.reg(indices),
+                                 axis & 0xFFFFFFFF, k)
+
+    def quantize(self, op_index: int, x, out):
+        self.code += struct.pack("<HHIHII", op_index, self.reg(x), BC_INVALID_OFFSET, self.reg(out),
+                                 out.t.quant_kind, out.t.quant_layout)
+
+    def dequantize(self, op_index: int, x, out):
+        self.code += struct.pack("<HHHII", op_index, self.reg(x), self.reg(out), x.t.quant_kind, x.t.quant_layout)

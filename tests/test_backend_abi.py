@@ -1,0 +1,282 @@
+"""CPU tests of the marmot_tensor_t-level backend layer: ABI layout against the reference's headers, exported
+tables, kernel query rules, bytecode immediates, kernel DSL files. No device work happens here."""
+import ctypes as C
+import os
+import re
+import struct
+import subprocess
+
+import pytest
+
+from marmot_amd import capi
+from marmot_amd import tensor_abi as ta
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+REFERENCE = "/root/reference"
+
+
+def _facts(text):
+    out = {}
+    for line in text.splitlines():
+        name, value = line.rsplit(" ", 1)
+        out[name] = int(value)
+    return out
+
+
+@pytest.fixture(scope="module")
+def golden_layout():
+    with open(os.path.join(GOLDEN, "abi_layout.txt")) as f:
+        return _facts(f.read())
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return ta.bind(capi.load_library())
+
+
+def test_mirror_header_matches_reference_layout(tmp_path, golden_layout):
+    exe = tmp_path / "abi_mirror"
+    subprocess.run(["gcc", "-std=c11", f"-I{ROOT}/include", "-o", str(exe), os.path.join(GOLDEN, "abi_probe.c")],
+                   check=True)
+    mine = _facts(subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout)
+    assert mine == golden_layout
+    assert len(mine) > 150
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE), reason="reference tree not present")
+def test_layout_fixture_is_current(golden_layout):
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_abi_layout", os.path.join(GOLDEN, "make_abi_layout.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert _facts(mod.reference_layout()) == golden_layout
+
+
+def test_ctypes_structs_match_layout(golden_layout):
+    pairs = {
+        "marmot_shape_t": ta.Shape, "marmot_tensor_t": ta.Tensor, "marmot_matmul_epilogue_t": ta.Epilogue,
+        "marmot_topk_desc_t": ta.TopkDesc, "marmot_moe_experts_desc_t": ta.MoeDesc,
+        "marmot_op_signature_t": ta.OpSignature, "marmot_kernel_selection_t": ta.KernelSelection,
+        "marmot_device_caps_t": ta.DeviceCaps, "marmot_device_ops_t": ta.DeviceOps,
+        "marmot_bc_exec_ctx_t": ta.BcExecCtx, "marmot_bc_tables_t": ta.BcTables,
+        "marmot_allocator_usage_t": ta.AllocatorUsage, "marmot_context_policy_t": ta.ContextPolicy,
+        "marmot_backend_preferences_t": ta.BackendPreferences, "marmot_matmul_dims_t": ta.MatmulDims,
+        "marmot_quant_block_t": ta.QuantBlock,
+    }
+    checked = 0
+    for cname, cls in pairs.items():
+        assert C.sizeof(cls) == golden_layout[f"sizeof({cname})"], cname
+        for key, off in golden_layout.items():
+            m = re.fullmatch(rf"offsetof\({cname},(\w+)\)", key)
+            if m:
+                assert getattr(cls, m.group(1)).offset == off, key
+                checked += 1
+    assert checked >= 90
+    assert ta.OP_MATMUL == golden_layout["MARMOT_OP_MATMUL"]
+    assert ta.OP_MOE_EXPERTS == golden_layout["MARMOT_OP_MOE_EXPERTS"]
+    assert ta.OP_TOPK == golden_layout["MARMOT_OP_TOPK"]
+    assert ta.QSCHEME_OF_KIND[ta.KIND_Q4_K] == golden_layout["MARMOT_QSCHEME_Q4_K"]
+    assert ta.QSCHEME_OF_KIND[ta.KIND_Q6_K] == golden_layout["MARMOT_QSCHEME_Q6_K"]
+    assert ta.KIND_Q8_K == golden_layout["MARMOT_QUANT_KIND_Q8_K"]
+    assert ta.NOT_IMPLEMENTED == golden_layout["MARMOT_ERROR_NOT_IMPLEMENTED"]
+    assert ta.BACKEND_HIP == golden_layout["MARMOT_BACKEND_CUDA"] + 1
+
+
+def test_backend_symbols_declared_and_exported(lib):
+    header = open(os.path.join(ROOT, "include", "marmot_hip_backend.h")).read()
+    for name in ta.BACKEND_SYMBOLS:
+        assert re.search(rf"\b{name}\s*\(", header), f"{name} not declared in marmot_hip_backend.h"
+        assert getattr(lib, name) is not None
+    declared = set(re.findall(r"\b((?:marmot_get_hip|marmot_hip_|hip_)\w+)\s*\(", header))
+    assert declared == set(ta.BACKEND_SYMBOLS)
+
+
+def test_vtable_is_complete(lib):
+    ops = lib.marmot_get_hip_ops().contents
+    for name, _ in ta.DeviceOps._fields_:
+        assert getattr(ops, name), f"vtable entry {name} is null"
+    # same table on every call
+    assert C.addressof(lib.marmot_get_hip_ops().contents) == C.addressof(ops)
+
+
+def _sig(op=ta.OP_MATMUL, kind=ta.KIND_Q4_K, inp=ta.DTYPE_F32, out=ta.DTYPE_F32, N=1, K=4096, M=14336):
+    s = ta.OpSignature()
+    s.op_id = op
+    s.profile_id = ta.PROFILE_SCALAR
+    s.matmul_layout = ta.MATMUL_LAYOUT_NT
+    s.input_dtype, s.weight_dtype, s.output_dtype, s.accum_dtype = inp, ta.DTYPE_U8, out, ta.DTYPE_F32
+    s.qscheme_id = ta.QSCHEME_OF_KIND.get(kind, 0)
+    s.weight_layout = ta.WEIGHT_LAYOUT_SEPARATE
+    s.dims.matmul.N, s.dims.matmul.K, s.dims.matmul.M = N, K, M
+    return s
+
+
+def _caps():
+    c = ta.DeviceCaps()
+    c.mem_bw_gbps = 8000.0
+    c.peak_flops_tflops_fp16 = 2500.0
+    c.launch_overhead_us = 2.0
+    return c
+
+
+def _query(lib, sig):
+    caps = _caps()
+    return lib.marmot_hip_query_kernel(C.byref(sig), C.byref(caps))
+
+
+def test_query_kernel_matmul_rules(lib):
+    expect_op = {ta.KIND_Q4_0: 1, ta.KIND_Q8_0: 2, ta.KIND_Q4_K: 3, ta.KIND_Q6_K: 4}
+    for kind, op in expect_op.items():
+        sel = _query(lib, _sig(kind=kind))
+        assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
+        assert sel.fallback_reason is None
+    # profile is a wildcard
+    s = _sig()
+    for profile in (0, 1, 2, 3, 4):
+        s.profile_id = profile
+        assert _query(lib, s).supported
+    # LINEAR resolves like MATMUL
+    assert _query(lib, _sig(op=ta.OP_LINEAR)).op_index == 3
+    # dtype pairs: f32->f32, f16->f32, f16->f16 yes; f32->f16 no
+    assert _query(lib, _sig(inp=ta.DTYPE_F16, out=ta.DTYPE_F32)).supported
+    assert _query(lib, _sig(inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).supported
+    assert not _query(lib, _sig(inp=ta.DTYPE_F32, out=ta.DTYPE_F16)).supported
+    # Q6_K with fp16 activations is declined (caller falls back)
+    sel = _query(lib, _sig(kind=ta.KIND_Q6_K, inp=ta.DTYPE_F16))
+    assert not sel.supported and sel.op_index == 0xFFFF and b"Q6_K" in sel.fallback_reason
+    # unsupported scheme, layout, weight layout, stride mode, epilogue, variant
+    assert not _query(lib, _sig(kind=ta.KIND_Q8_K)).supported
+    s = _sig(); s.qscheme_id = 9  # Q5_K
+    assert not _query(lib, s).supported
+    s = _sig(); s.matmul_layout = 1
+    assert not _query(lib, s).supported
+    s = _sig(); s.weight_layout = 2
+    assert not _query(lib, s).supported
+    s = _sig(); s.stride_mode = 3
+    assert not _query(lib, s).supported
+    s = _sig(); s.stride_mode = 1
+    assert _query(lib, s).supported
+    s = _sig(); s.epilogue_flags = ta.EPILOGUE_BIAS
+    assert _query(lib, s).supported
+    s = _sig(); s.epilogue_flags = ta.EPILOGUE_BIAS | 2
+    assert not _query(lib, s).supported
+    s = _sig(); s.variant_flags = 1
+    assert not _query(lib, s).supported
+    s = _sig(); s.accum_dtype = ta.DTYPE_F16
+    assert not _query(lib, s).supported
+    # null arguments
+    sel = lib.marmot_hip_query_kernel(None, None)
+    assert not sel.supported
+
+
+def test_query_kernel_cost_model(lib):
+    # decode matvec is priced by bytes over HBM bandwidth, prefill by flops over the MFMA peak
+    decode = _query(lib, _sig(N=1, K=4096, M=14336))
+    nbytes = 14336 * 16 * 144 + 4096 * 4 + 14336 * 4
+    assert decode.estimated_us == pytest.approx(2.0 + nbytes / 8000e3, rel=1e-6)
+    prefill = _query(lib, _sig(inp=ta.DTYPE_F16, N=512, K=4096, M=4096))
+    assert prefill.estimated_us == pytest.approx(2.0 + 2 * 512 * 4096 * 4096 / 2500e6, rel=1e-6)
+    assert decode.est_workspace_mb > 0 and prefill.est_workspace_mb == 0
+
+
+def test_query_kernel_other_ops(lib):
+    for kind, op in {ta.KIND_Q4_0: 5, ta.KIND_Q8_0: 6, ta.KIND_Q4_K: 7, ta.KIND_Q6_K: 8}.items():
+        assert _query(lib, _sig(op=ta.OP_MOE_EXPERTS, kind=kind)).op_index == op
+    assert not _query(lib, _sig(op=ta.OP_MOE_EXPERTS, inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).supported
+    assert _query(lib, _sig(op=ta.OP_TOPK)).op_index == 9
+    assert _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q8_K)).op_index == 10
+    assert _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q8_0, inp=ta.DTYPE_F16)).op_index == 10
+    assert not _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_K)).supported
+    assert _query(lib, _sig(op=ta.OP_DEQUANTIZE, kind=ta.KIND_Q6_K)).op_index == 11
+    assert not _query(lib, _sig(op=12345)).supported
+
+
+def test_default_caps_and_preferences(lib):
+    caps = lib.marmot_hip_detect_default_caps()
+    assert caps.mem_bw_gbps == pytest.approx(8000.0)
+    assert caps.peak_flops_tflops_fp16 == pytest.approx(2500.0)
+    assert caps.simd_width == 64 and caps.num_compute_units >= 1 and caps.has_tensor_cores
+    prefs = ta.BackendPreferences()
+    assert lib.marmot_hip_default_preferences(C.byref(caps), C.byref(prefs))
+    assert prefs.routing_policy == 1 and not prefs.policy.matmul_requires_temp_tensors
+    assert not prefs.policy.matmul_prefer_packed_weights
+    assert not lib.marmot_hip_default_preferences(None, C.byref(prefs))
+
+
+def test_bytecode_tables(lib, golden_layout):
+    t = ta.BcTables()
+    assert lib.marmot_hip_bc_get_tables(C.byref(t))
+    assert not lib.marmot_hip_bc_get_tables(None)
+    assert t.op_count == 12
+    assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
+    schema = [t.schema_id[i] for i in range(t.op_count)]
+    assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
+    assert schema[5:9] == [golden_layout["MARMOT_BC_SCHEMA_MOE_EXPERTS"]] * 4
+    assert schema[9] == golden_layout["MARMOT_BC_SCHEMA_TOPK"]
+    assert schema[10] == golden_layout["MARMOT_BC_SCHEMA_QUANTIZE"]
+    assert schema[11] == golden_layout["MARMOT_BC_SCHEMA_DEQUANTIZE"]
+    # immediate sizes equal what the encoders of tensor_abi.Program emit (opcode excluded)
+    sizes = [t.imm_size[i] for i in range(t.op_count)]
+    assert sizes[1:5] == [struct.calcsize("<HHHIH")] * 4
+    assert sizes[5:9] == [struct.calcsize("<7HIfI")] * 4
+    assert sizes[9] == struct.calcsize("<HHHII")
+    assert sizes[10] == struct.calcsize("<HIHII")
+    assert sizes[11] == struct.calcsize("<HHII")
+    for i in range(1, t.op_count):
+        assert t.exec_table[i], f"exec entry {i} missing"
+
+
+def test_exec_entries_reject_null_arguments(lib):
+    t = ta.BcTables()
+    lib.marmot_hip_bc_get_tables(C.byref(t))
+    imm = (C.c_uint8 * 32)()
+    for i in range(1, t.op_count):
+        assert t.exec_table[i](None, None, imm, None) == ta.INVALID_ARGUMENT
+    detail = C.c_char_p()
+    assert lib.marmot_hip_backend_last_error(C.byref(detail)) == ta.INVALID_ARGUMENT
+    assert b"Null bytecode exec arguments" in detail.value
+    # impl functions with a null device context
+    assert lib.hip_matmul_quantized_q4_k(None, None, None, None, None) == ta.INVALID_ARGUMENT
+    assert lib.hip_moe_experts_impl(None, None) == ta.INVALID_ARGUMENT
+    assert lib.hip_topk_impl(None, None) == ta.INVALID_ARGUMENT
+
+
+def test_program_encoding_matches_reference_immediates():
+    import numpy as np
+    x = ta.HostTensor.dense(np.zeros((2, 256), np.float32))
+    w = ta.HostTensor.quantized(np.zeros(4 * 144, np.uint8), (4, 256), ta.KIND_Q4_K)
+    y = ta.HostTensor.empty((2, 4), ta.DTYPE_F32)
+    b = ta.HostTensor.dense(np.zeros(4, np.float32))
+    p = ta.Program()
+    p.matmul(3, x, w, y)
+    assert bytes(p.code) == struct.pack("<HHHHIH", 3, 0, 1, 0xFFFF, 0xFFFFFFFF, 2)
+    p.matmul(3, x, w, y, bias=b)
+    op, ri, rw, rb, off, ro = struct.unpack_from("<HHHHIH", p.code, 14)
+    assert (op, ri, rw, rb, ro) == (3, 0, 1, 3, 2) and off == 0 and len(p.const_pool) == C.sizeof(ta.Epilogue)
+    assert len(p.regs) == 4
+    # tensor strides are row-major element strides, as marmot_tensor_create fills them
+    assert list(x.t.shape.strides[:2]) == [256, 1] and x.t.shape.ndim == 2
+
+
+def test_kernel_def_files_name_exported_impls(lib):
+    ddir = os.path.join(ROOT, "marmot_amd", "kernels_def")
+    families = {}
+    for fn in sorted(os.listdir(ddir)):
+        text = open(os.path.join(ddir, fn)).read()
+        for name, body in re.findall(r"KERNEL_FAMILY\((\w+)\)\s*\{(.*?)\n\}", text, re.S):
+            fields = dict(re.findall(r"^\s*([A-Z_]+(?:\(\w+\))?):\s*(.+?),?\s*$", body, re.M))
+            families[name] = fields
+    assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_q6_k", "topk_hip",
+                             "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip"}
+    for name, f in families.items():
+        impl = f["IMPL_FUNCTION"].strip('"')
+        schemes = re.findall(r"Q\d_[0K]", f.get("AXIS(scheme)", "")) or [""]
+        for s in schemes:
+            sym = impl.replace("{scheme:lower}", s.lower())
+            assert hasattr(lib, sym), f"{name}: {sym} not exported"
+        assert f["PLATFORM"] == "HIP" and f["PROFILE"] == "ANY"
+    mm = families["matmul_quantized_hip"]
+    assert mm["OP"] == "matmul" and mm["MATMUL_LAYOUT"] == "NT" and mm["WEIGHT_LAYOUT"] == "SEPARATE"
+    assert mm["EPILOGUE"] == "[BIAS]" and mm["ACCUM_DTYPE"] == "FLOAT32" and mm["STRIDE_MODE"] == "CONTIGUOUS"
+    assert families["matmul_quantized_hip_q6_k"]["INPUT_DTYPE"] == "FLOAT32"

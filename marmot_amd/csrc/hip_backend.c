@@ -1,28 +1,24 @@
-// marmot_tensor_t-level HIP backend: device vtable with a host-pointer residency table, kernel query,
-// bytecode exec table and the impl functions the generated dispatch shims call. Host code only; all device work
-// goes through the raw-pointer C ABI of marmot_hip.h.
+// marmot_tensor_t-level HIP backend, written in C23 like the host side of marmot's other backends: device vtable
+// with a host-pointer residency table, kernel query, bytecode exec table and the impl functions the generated
+// dispatch shims call. Host code only; all device work goes through the raw-pointer C ABI of marmot_hip.h.
 #include "marmot_hip.h"
 #include "marmot_hip_backend.h"
 
+#include <pthread.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
-
-#include <map>
-#include <mutex>
-#include <new>
-
-namespace {
 
 // ------------------------------------------------------------------ errors
 #ifdef MARMOT_HIP_IN_TREE
-inline marmot_error_t fail(marmot_error_t code, const char *msg) {
+static marmot_error_t fail(marmot_error_t code, const char *msg) {
     marmot_set_error(code, msg);
     return code;
 }
 #else
-thread_local marmot_error_t g_last_code = MARMOT_SUCCESS;
-thread_local char g_last_detail[256] = {0};
-inline marmot_error_t fail(marmot_error_t code, const char *msg) {
+static thread_local marmot_error_t g_last_code = MARMOT_SUCCESS;
+static thread_local char g_last_detail[256] = {0};
+static marmot_error_t fail(marmot_error_t code, const char *msg) {
     g_last_code = code;
     snprintf(g_last_detail, sizeof(g_last_detail), "%s", msg != nullptr ? msg : "");
     return code;
@@ -30,164 +26,184 @@ inline marmot_error_t fail(marmot_error_t code, const char *msg) {
 #endif
 
 // a failure of the raw ABI: same numeric codes, text from the library
-inline marmot_error_t fail_from_lib(int code) {
+static marmot_error_t fail_from_lib(int code) {
     return fail((marmot_error_t)code, marmot_hip_last_error());
 }
 
 // ------------------------------------------------------------------ residency table
-// One device mirror per host address range, keyed by the range's first byte. Ranges never overlap: a request
+// One device mirror per host address range, kept sorted by the range's first byte. Ranges never overlap: a request
 // that is contained in a mirror resolves to an offset inside it; a request that overlaps mirrors without being
 // contained in one replaces them with one mirror over the union (their device-newer bytes are brought home first).
-struct Mirror {
-    uintptr_t host = 0;
-    size_t bytes = 0;
-    void *dev = nullptr;
-    bool host_newer = false;  // host copy changed since the last upload
-    bool dev_newer = false;   // a kernel wrote the mirror since the last download
-};
+typedef struct {
+    uintptr_t host;
+    size_t bytes;
+    void *dev;
+    bool host_newer;  // host copy changed since the last upload
+    bool dev_newer;   // a kernel wrote the mirror since the last download
+} hip_mirror_t;
 
-struct Backend {
-    marmot_hip_device_t *dev = nullptr;
-    std::mutex mu;
-    std::map<uintptr_t, Mirror> mirrors;
-    bool batching = false;
-    uint64_t uploads = 0, upload_bytes = 0, downloads = 0, download_bytes = 0;
-    size_t mirrored_bytes = 0;
+typedef struct {
+    marmot_hip_device_t *dev;
+    pthread_mutex_t mu;
+    hip_mirror_t *mirrors;  // sorted by host
+    size_t n_mirrors, cap_mirrors;
+    bool batching;
+    uint64_t uploads, upload_bytes, downloads, download_bytes;
+    size_t mirrored_bytes;
+} hip_backend_t;
 
-    Mirror *find_containing(uintptr_t p, size_t n) {
-        auto it = mirrors.upper_bound(p);
-        if (it == mirrors.begin()) {
-            return nullptr;
+static hip_backend_t *backend_of(const void *device_ctx) {
+    return (hip_backend_t *)device_ctx;
+}
+
+// index of the first mirror whose start is > p
+static size_t upper_bound(const hip_backend_t *b, uintptr_t p) {
+    size_t lo = 0, hi = b->n_mirrors;
+    while (lo < hi) {
+        const size_t mid = lo + (hi - lo) / 2;
+        if (b->mirrors[mid].host <= p) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
         }
-        --it;
-        Mirror &m = it->second;
-        if (p >= m.host && p + n <= m.host + m.bytes) {
-            return &m;
-        }
+    }
+    return lo;
+}
+
+static hip_mirror_t *find_containing(hip_backend_t *b, uintptr_t p, size_t n) {
+    const size_t i = upper_bound(b, p);
+    if (i == 0) {
         return nullptr;
     }
+    hip_mirror_t *m = &b->mirrors[i - 1];
+    return (p >= m->host && p + n <= m->host + m->bytes) ? m : nullptr;
+}
 
-    marmot_error_t upload(Mirror &m) {
-        int st = marmot_hip_memcpy_to_device(dev, m.dev, (const void *)m.host, m.bytes);
-        if (st != MARMOT_HIP_SUCCESS) {
-            return fail_from_lib(st);
-        }
-        uploads++;
-        upload_bytes += m.bytes;
-        m.host_newer = false;
+static bool overlaps(const hip_mirror_t *m, uintptr_t p, size_t n) {
+    return m->host < p + n && p < m->host + m->bytes;
+}
+
+static marmot_error_t upload(hip_backend_t *b, hip_mirror_t *m) {
+    const int st = marmot_hip_memcpy_to_device(b->dev, m->dev, (const void *)m->host, m->bytes);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(st);
+    }
+    b->uploads++;
+    b->upload_bytes += m->bytes;
+    m->host_newer = false;
+    return MARMOT_SUCCESS;
+}
+
+static marmot_error_t download(hip_backend_t *b, const hip_mirror_t *m, uintptr_t p, size_t n) {
+    const int st = marmot_hip_memcpy_from_device(b->dev, (void *)p, (const uint8_t *)m->dev + (p - m->host), n);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(st);
+    }
+    b->downloads++;
+    b->download_bytes += n;
+    return MARMOT_SUCCESS;
+}
+
+static void drop_at(hip_backend_t *b, size_t i) {
+    marmot_hip_free(b->dev, b->mirrors[i].dev);
+    b->mirrored_bytes -= b->mirrors[i].bytes;
+    memmove(&b->mirrors[i], &b->mirrors[i + 1], (b->n_mirrors - i - 1) * sizeof(hip_mirror_t));
+    b->n_mirrors--;
+}
+
+// mirror covering [p, p+n): the existing one, or a new one over the union of [p, p+n) and every mirror it touches
+static marmot_error_t cover(hip_backend_t *b, uintptr_t p, size_t n, bool will_read_host, hip_mirror_t **out) {
+    hip_mirror_t *hit = find_containing(b, p, n);
+    if (hit != nullptr) {
+        *out = hit;
         return MARMOT_SUCCESS;
     }
-
-    marmot_error_t download(Mirror &m, uintptr_t p, size_t n) {
-        int st = marmot_hip_memcpy_from_device(dev, (void *)p, (const uint8_t *)m.dev + (p - m.host), n);
-        if (st != MARMOT_HIP_SUCCESS) {
-            return fail_from_lib(st);
+    uintptr_t lo = p, hi = p + n;
+    // bring device-newer bytes of overlapping mirrors home, then drop them; restart because the union may grow
+    for (size_t i = 0; i < b->n_mirrors;) {
+        hip_mirror_t *o = &b->mirrors[i];
+        if (!overlaps(o, lo, hi - lo)) {
+            ++i;
+            continue;
         }
-        downloads++;
-        download_bytes += n;
-        return MARMOT_SUCCESS;
-    }
-
-    void drop(std::map<uintptr_t, Mirror>::iterator it) {
-        marmot_hip_free(dev, it->second.dev);
-        mirrored_bytes -= it->second.bytes;
-        mirrors.erase(it);
-    }
-
-    // mirror covering [p, p+n): existing one, or a new one over the union of [p, p+n) and every mirror it touches
-    marmot_error_t cover(uintptr_t p, size_t n, bool will_read_host, Mirror **out) {
-        if (Mirror *m = find_containing(p, n)) {
-            *out = m;
-            return MARMOT_SUCCESS;
-        }
-        uintptr_t lo = p, hi = p + n;
-        // bring device-newer bytes of overlapping mirrors home, then drop them
-        for (;;) {
-            auto it = mirrors.lower_bound(lo);
-            if (it != mirrors.begin()) {
-                auto prev = it;
-                --prev;
-                if (prev->second.host + prev->second.bytes > lo) {
-                    it = prev;
-                }
-            }
-            if (it == mirrors.end() || it->second.host >= hi) {
-                break;
-            }
-            Mirror &o = it->second;
-            if (o.dev_newer) {
-                marmot_error_t st = download(o, o.host, o.bytes);
-                if (st != MARMOT_SUCCESS) {
-                    return st;
-                }
-            }
-            if (o.host < lo) {
-                lo = o.host;
-            }
-            if (o.host + o.bytes > hi) {
-                hi = o.host + o.bytes;
-            }
-            drop(it);
-            will_read_host = true;  // the union holds bytes that are only on the host now
-        }
-        Mirror m;
-        m.host = lo;
-        m.bytes = hi - lo;
-        int st = marmot_hip_alloc(dev, m.bytes, &m.dev);
-        if (st != MARMOT_HIP_SUCCESS) {
-            return fail_from_lib(st);
-        }
-        m.host_newer = will_read_host;
-        mirrored_bytes += m.bytes;
-        auto ins = mirrors.emplace(lo, m);
-        *out = &ins.first->second;
-        return MARMOT_SUCCESS;
-    }
-
-    // device address of a kernel input: uploads the mirror when the host copy is newer
-    marmot_error_t acquire_read(const void *host, size_t n, const void **d_out) {
-        Mirror *m = nullptr;
-        marmot_error_t st = cover((uintptr_t)host, n, true, &m);
-        if (st != MARMOT_SUCCESS) {
-            return st;
-        }
-        if (m->host_newer) {
-            st = upload(*m);
+        if (o->dev_newer) {
+            const marmot_error_t st = download(b, o, o->host, o->bytes);
             if (st != MARMOT_SUCCESS) {
                 return st;
             }
         }
-        *d_out = (const uint8_t *)m->dev + ((uintptr_t)host - m->host);
-        return MARMOT_SUCCESS;
+        if (o->host < lo) {
+            lo = o->host;
+        }
+        if (o->host + o->bytes > hi) {
+            hi = o->host + o->bytes;
+        }
+        drop_at(b, i);
+        will_read_host = true;  // the union holds bytes that are only on the host now
+        i = 0;
     }
+    if (b->n_mirrors == b->cap_mirrors) {
+        const size_t cap = b->cap_mirrors != 0 ? 2 * b->cap_mirrors : 64;
+        hip_mirror_t *grown = realloc(b->mirrors, cap * sizeof(hip_mirror_t));
+        if (grown == nullptr) {
+            return fail(MARMOT_ERROR_OUT_OF_MEMORY, "HIP residency table: out of host memory");
+        }
+        b->mirrors = grown;
+        b->cap_mirrors = cap;
+    }
+    hip_mirror_t m = {.host = lo, .bytes = hi - lo, .dev = nullptr, .host_newer = will_read_host, .dev_newer = false};
+    const int st = marmot_hip_alloc(b->dev, m.bytes, &m.dev);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(st);
+    }
+    const size_t at = upper_bound(b, lo);
+    memmove(&b->mirrors[at + 1], &b->mirrors[at], (b->n_mirrors - at) * sizeof(hip_mirror_t));
+    b->mirrors[at] = m;
+    b->n_mirrors++;
+    b->mirrored_bytes += m.bytes;
+    *out = &b->mirrors[at];
+    return MARMOT_SUCCESS;
+}
 
-    // device address of a kernel output that is fully overwritten
-    marmot_error_t acquire_write(void *host, size_t n, void **d_out) {
-        Mirror *m = nullptr;
-        marmot_error_t st = cover((uintptr_t)host, n, false, &m);
+// device address of a kernel input: uploads the mirror when the host copy is newer
+static marmot_error_t acquire_read(hip_backend_t *b, const void *host, size_t n, const void **d_out) {
+    hip_mirror_t *m = nullptr;
+    marmot_error_t st = cover(b, (uintptr_t)host, n, true, &m);
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    if (m->host_newer) {
+        st = upload(b, m);
         if (st != MARMOT_SUCCESS) {
             return st;
         }
-        const bool whole = (uintptr_t)host == m->host && n == m->bytes;
-        if (m->host_newer && !whole) {
-            st = upload(*m);  // keep the bytes of the mirror outside the output valid
-            if (st != MARMOT_SUCCESS) {
-                return st;
-            }
-        }
-        m->host_newer = false;
-        m->dev_newer = true;
-        *d_out = (uint8_t *)m->dev + ((uintptr_t)host - m->host);
-        return MARMOT_SUCCESS;
     }
-};
+    *d_out = (const uint8_t *)m->dev + ((uintptr_t)host - m->host);
+    return MARMOT_SUCCESS;
+}
 
-inline Backend *backend_of(const void *device_ctx) {
-    return (Backend *)const_cast<void *>(device_ctx);
+// device address of a kernel output that is fully overwritten
+static marmot_error_t acquire_write(hip_backend_t *b, void *host, size_t n, void **d_out) {
+    hip_mirror_t *m = nullptr;
+    marmot_error_t st = cover(b, (uintptr_t)host, n, false, &m);
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    const bool whole = (uintptr_t)host == m->host && n == m->bytes;
+    if (m->host_newer && !whole) {
+        st = upload(b, m);  // keep the bytes of the mirror outside the output valid
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+    }
+    m->host_newer = false;
+    m->dev_newer = true;
+    *d_out = (uint8_t *)m->dev + ((uintptr_t)host - m->host);
+    return MARMOT_SUCCESS;
 }
 
 // ------------------------------------------------------------------ tensor helpers
-size_t dtype_size(marmot_dtype_t t) {
+static size_t dtype_size(marmot_dtype_t t) {
     switch (t) {
     case MARMOT_DTYPE_FLOAT32:
     case MARMOT_DTYPE_INT32:
@@ -212,109 +228,102 @@ size_t dtype_size(marmot_dtype_t t) {
     }
 }
 
-bool kind_supported_weight(marmot_quant_kind_t k) {
+static bool kind_supported_weight(marmot_quant_kind_t k) {
     return k == MARMOT_QUANT_KIND_Q4_0 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q4_K ||
         k == MARMOT_QUANT_KIND_Q6_K;
 }
 
-bool kind_is_block(marmot_quant_kind_t k) {
+static bool kind_is_block(marmot_quant_kind_t k) {
     return k > MARMOT_QUANT_KIND_GENERIC && k < MARMOT_QUANT_KIND_COUNT;
 }
 
 // block-quantized storage uses byte-sized elements (marmot_quant_storage_dtype_compatible, src/core/helpers/quant.c)
-bool storage_dtype_ok(marmot_dtype_t t) {
+static bool storage_dtype_ok(marmot_dtype_t t) {
     return t == MARMOT_DTYPE_UINT8 || t == MARMOT_DTYPE_INT8;
 }
 
-size_t dense_bytes(const marmot_tensor_t *t) {
+static size_t tensor_numel(const marmot_tensor_t *t) {
     size_t n = 1;
     for (size_t i = 0; i < t->shape.ndim; ++i) {
         n *= t->shape.shape[i];
     }
-    return n * dtype_size(t->dtype);
+    return n;
 }
 
-bool rows_contiguous(const marmot_tensor_t *t) {
-    if (t->shape.ndim != 2) {
-        return false;
-    }
-    return t->shape.strides[1] == 1 && t->shape.strides[0] == t->shape.shape[1];
+static size_t dense_bytes(const marmot_tensor_t *t) {
+    return tensor_numel(t) * dtype_size(t->dtype);
 }
 
-void mark_device_output(marmot_tensor_t *t) {
+static bool rows_contiguous(const marmot_tensor_t *t) {
+    return t->shape.ndim == 2 && t->shape.strides[1] == 1 && t->shape.strides[0] == t->shape.shape[1];
+}
+
+static void mark_device_output(marmot_tensor_t *t) {
     t->memory_location = MARMOT_MEMORY_DEVICE;
     t->needs_sync = true;
 }
 
 // ------------------------------------------------------------------ vtable
-marmot_error_t ops_init(void **device_ctx) {
+static marmot_error_t ops_init(void **device_ctx) {
     if (device_ctx == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP backend init: null device_ctx");
     }
-    Backend *b = new (std::nothrow) Backend();
+    hip_backend_t *b = calloc(1, sizeof(*b));
     if (b == nullptr) {
         return fail(MARMOT_ERROR_OUT_OF_MEMORY, "HIP backend init: out of host memory");
     }
-    int st = marmot_hip_device_create(0, &b->dev);
+    const int st = marmot_hip_device_create(0, &b->dev);
     if (st != MARMOT_HIP_SUCCESS) {
-        delete b;
+        free(b);
         return fail_from_lib(st);
     }
+    pthread_mutex_init(&b->mu, nullptr);
     *device_ctx = b;
     return MARMOT_SUCCESS;
 }
 
-void ops_destroy(const void *device_ctx) {
-    Backend *b = backend_of(device_ctx);
+static void ops_destroy(const void *device_ctx) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr) {
         return;
     }
     marmot_hip_synchronize(b->dev);
-    for (auto &kv : b->mirrors) {
-        marmot_hip_free(b->dev, kv.second.dev);
+    for (size_t i = 0; i < b->n_mirrors; ++i) {
+        marmot_hip_free(b->dev, b->mirrors[i].dev);
     }
-    b->mirrors.clear();
+    free(b->mirrors);
     marmot_hip_device_destroy(b->dev);
-    delete b;
+    pthread_mutex_destroy(&b->mu);
+    free(b);
 }
 
-marmot_error_t ops_configure(const void *device_ctx, const marmot_context_t *ctx) {
+static marmot_error_t ops_configure(const void *device_ctx, const marmot_context_t *ctx) {
     (void)ctx;
-    return device_ctx != nullptr ? MARMOT_SUCCESS : fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP backend: null device_ctx");
+    return device_ctx != nullptr ? MARMOT_SUCCESS
+                                 : fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP backend: null device_ctx");
 }
 
-marmot_error_t ops_alloc(const void *device_ctx, size_t size, void **ptr) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t ops_alloc(const void *device_ctx, size_t size, void **ptr) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || ptr == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP alloc: null argument");
     }
-    int st = marmot_hip_alloc(b->dev, size, ptr);
+    const int st = marmot_hip_alloc(b->dev, size, ptr);
     return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
 }
 
-void ops_free(const void *device_ctx, void *ptr) {
-    Backend *b = backend_of(device_ctx);
+static void ops_free(const void *device_ctx, void *ptr) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b != nullptr && ptr != nullptr) {
         marmot_hip_free(b->dev, ptr);
     }
 }
 
-marmot_error_t ops_memcpy_to_device(const void *device_ctx, void *dst, const void *src, size_t size) {
-    Backend *b = backend_of(device_ctx);
-    if (b == nullptr || dst == nullptr || src == nullptr) {
-        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP memcpy_to_device: null argument");
-    }
-    if (size == 0) {
-        return MARMOT_SUCCESS;
-    }
-    if (dst != src) {
-        int st = marmot_hip_memcpy_to_device(b->dev, dst, src, size);
-        return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
-    }
-    // dst == src == host pointer: the host copy is newer than the mirror (src/core/tensor/transfer.c:22)
-    std::lock_guard<std::mutex> lock(b->mu);
+// dst == src == host pointer: the host copy is newer than the mirror (src/core/tensor/transfer.c:22)
+static marmot_error_t host_is_newer_locked(hip_backend_t *b, const void *src, size_t size) {
     const uintptr_t p = (uintptr_t)src;
-    if (Mirror *m = b->find_containing(p, size)) {
+    hip_mirror_t *m = find_containing(b, p, size);
+    if (m != nullptr) {
         if (p == m->host && size == m->bytes) {
             m->host_newer = true;  // uploaded when a kernel next reads it
             m->dev_newer = false;
@@ -323,7 +332,7 @@ marmot_error_t ops_memcpy_to_device(const void *device_ctx, void *dst, const voi
         if (m->host_newer) {
             return MARMOT_SUCCESS;  // the whole mirror is refreshed on next use anyway
         }
-        int st = marmot_hip_memcpy_to_device(b->dev, (uint8_t *)m->dev + (p - m->host), src, size);
+        const int st = marmot_hip_memcpy_to_device(b->dev, (uint8_t *)m->dev + (p - m->host), src, size);
         if (st != MARMOT_HIP_SUCCESS) {
             return fail_from_lib(st);
         }
@@ -331,18 +340,56 @@ marmot_error_t ops_memcpy_to_device(const void *device_ctx, void *dst, const voi
         b->upload_bytes += size;
         return MARMOT_SUCCESS;
     }
-    // not mirrored (yet): the first kernel that reads the range uploads it; stale partial overlaps are refreshed
-    for (auto &kv : b->mirrors) {
-        Mirror &o = kv.second;
-        if (o.host < p + size && p < o.host + o.bytes) {
-            o.host_newer = true;
+    // not mirrored as a whole: the first kernel that reads the range uploads it; partial overlaps are refreshed
+    for (size_t i = 0; i < b->n_mirrors; ++i) {
+        if (overlaps(&b->mirrors[i], p, size)) {
+            b->mirrors[i].host_newer = true;
         }
     }
     return MARMOT_SUCCESS;
 }
 
-marmot_error_t ops_memcpy_from_device(const void *device_ctx, void *dst, const void *src, size_t size) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t ops_memcpy_to_device(const void *device_ctx, void *dst, const void *src, size_t size) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || dst == nullptr || src == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP memcpy_to_device: null argument");
+    }
+    if (size == 0) {
+        return MARMOT_SUCCESS;
+    }
+    if (dst != src) {
+        const int st = marmot_hip_memcpy_to_device(b->dev, dst, src, size);
+        return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
+    }
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = host_is_newer_locked(b, src, size);
+    pthread_mutex_unlock(&b->mu);
+    return st;
+}
+
+// dst == src == host pointer: make the host copy current (src/core/tensor/transfer.c:49-55)
+static marmot_error_t make_host_current_locked(hip_backend_t *b, void *dst, size_t size) {
+    const uintptr_t p = (uintptr_t)dst;
+    for (size_t i = 0; i < b->n_mirrors; ++i) {
+        hip_mirror_t *m = &b->mirrors[i];
+        if (!overlaps(m, p, size) || !m->dev_newer) {
+            continue;
+        }
+        const uintptr_t lo = p > m->host ? p : m->host;
+        const uintptr_t hi = (p + size) < (m->host + m->bytes) ? (p + size) : (m->host + m->bytes);
+        const marmot_error_t st = download(b, m, lo, hi - lo);
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+        if (lo == m->host && hi == m->host + m->bytes) {
+            m->dev_newer = false;
+        }
+    }
+    return MARMOT_SUCCESS;
+}
+
+static marmot_error_t ops_memcpy_from_device(const void *device_ctx, void *dst, const void *src, size_t size) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || dst == nullptr || src == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP memcpy_from_device: null argument");
     }
@@ -350,47 +397,31 @@ marmot_error_t ops_memcpy_from_device(const void *device_ctx, void *dst, const v
         return MARMOT_SUCCESS;
     }
     if (dst != src) {
-        int st = marmot_hip_memcpy_from_device(b->dev, dst, src, size);
+        const int st = marmot_hip_memcpy_from_device(b->dev, dst, src, size);
         return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
     }
-    // dst == src == host pointer: make the host copy current (src/core/tensor/transfer.c:49-55)
-    std::lock_guard<std::mutex> lock(b->mu);
-    const uintptr_t p = (uintptr_t)dst;
-    // every mirror that overlaps the range and holds newer bytes
-    for (auto &kv : b->mirrors) {
-        Mirror &m = kv.second;
-        if (!(m.host < p + size && p < m.host + m.bytes) || !m.dev_newer) {
-            continue;
-        }
-        const uintptr_t lo = p > m.host ? p : m.host;
-        const uintptr_t hi = (p + size) < (m.host + m.bytes) ? (p + size) : (m.host + m.bytes);
-        marmot_error_t st = b->download(m, lo, hi - lo);
-        if (st != MARMOT_SUCCESS) {
-            return st;
-        }
-        if (lo == m.host && hi == m.host + m.bytes) {
-            m.dev_newer = false;
-        }
-    }
-    return MARMOT_SUCCESS;
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = make_host_current_locked(b, dst, size);
+    pthread_mutex_unlock(&b->mu);
+    return st;
 }
 
-marmot_error_t ops_synchronize(const void *device_ctx) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t ops_synchronize(const void *device_ctx) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP synchronize: null device_ctx");
     }
-    int st = marmot_hip_synchronize(b->dev);
+    const int st = marmot_hip_synchronize(b->dev);
     return st == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(st);
 }
 
-marmot_error_t ops_allocator_usage(const void *device_ctx, marmot_allocator_usage_t *usage) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t ops_allocator_usage(const void *device_ctx, marmot_allocator_usage_t *usage) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || usage == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP allocator_usage: null argument");
     }
     size_t cur = 0, peak = 0, n = 0;
-    int st = marmot_hip_allocator_usage(b->dev, &cur, &peak, &n);
+    const int st = marmot_hip_allocator_usage(b->dev, &cur, &peak, &n);
     if (st != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(st);
     }
@@ -403,8 +434,8 @@ marmot_error_t ops_allocator_usage(const void *device_ctx, marmot_allocator_usag
 
 // All kernels of a context are enqueued on one stream in program order, so a batch needs no extra bracket:
 // begin/end only record the state that marmot_graph_batch_is_active reports.
-marmot_error_t ops_graph_batch_begin(void *device_ctx) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t ops_graph_batch_begin(void *device_ctx) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP graph_batch_begin: null device_ctx");
     }
@@ -412,8 +443,8 @@ marmot_error_t ops_graph_batch_begin(void *device_ctx) {
     return MARMOT_SUCCESS;
 }
 
-marmot_error_t ops_graph_batch_end(void *device_ctx, bool commit) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t ops_graph_batch_end(void *device_ctx, bool commit) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP graph_batch_end: null device_ctx");
     }
@@ -422,66 +453,94 @@ marmot_error_t ops_graph_batch_end(void *device_ctx, bool commit) {
     return MARMOT_SUCCESS;
 }
 
-void ops_on_host_range_freed(void *device_ctx, const void *start, size_t length) {
-    Backend *b = backend_of(device_ctx);
+static void ops_on_host_range_freed(void *device_ctx, const void *start, size_t length) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || start == nullptr || length == 0) {
         return;
     }
-    std::lock_guard<std::mutex> lock(b->mu);
-    const uintptr_t p = (uintptr_t)start;
+    pthread_mutex_lock(&b->mu);
     bool synced = false;
-    for (auto it = b->mirrors.begin(); it != b->mirrors.end();) {
-        Mirror &m = it->second;
-        if (m.host < p + length && p < m.host + m.bytes) {
-            if (!synced) {
-                marmot_hip_synchronize(b->dev);  // kernels still reading the mirror finish first
-                synced = true;
-            }
-            auto victim = it++;
-            b->drop(victim);
-        } else {
-            ++it;
+    for (size_t i = 0; i < b->n_mirrors;) {
+        if (!overlaps(&b->mirrors[i], (uintptr_t)start, length)) {
+            ++i;
+            continue;
         }
+        if (!synced) {
+            marmot_hip_synchronize(b->dev);  // kernels still reading the mirror finish first
+            synced = true;
+        }
+        drop_at(b, i);
     }
+    pthread_mutex_unlock(&b->mu);
 }
 
-void ops_on_host_ptr_freed(void *device_ctx, const void *ptr) {
-    Backend *b = backend_of(device_ctx);
+static void ops_on_host_ptr_freed(void *device_ctx, const void *ptr) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || ptr == nullptr) {
         return;
     }
     size_t bytes = 1;
-    {
-        std::lock_guard<std::mutex> lock(b->mu);
-        auto it = b->mirrors.find((uintptr_t)ptr);
-        if (it != b->mirrors.end()) {
-            bytes = it->second.bytes;
-        }
+    pthread_mutex_lock(&b->mu);
+    const size_t i = upper_bound(b, (uintptr_t)ptr);
+    if (i > 0 && b->mirrors[i - 1].host == (uintptr_t)ptr) {
+        bytes = b->mirrors[i - 1].bytes;
     }
+    pthread_mutex_unlock(&b->mu);
     ops_on_host_range_freed(device_ctx, ptr, bytes);
 }
 
-const marmot_device_ops_t k_hip_ops = {
-    ops_init,
-    ops_destroy,
-    ops_configure,
-    ops_alloc,
-    ops_free,
-    ops_memcpy_to_device,
-    ops_memcpy_from_device,
-    ops_synchronize,
-    ops_allocator_usage,
-    ops_graph_batch_begin,
-    ops_graph_batch_end,
-    ops_on_host_ptr_freed,
-    ops_on_host_range_freed,
+static const marmot_device_ops_t k_hip_ops = {
+    .init = ops_init,
+    .destroy = ops_destroy,
+    .configure = ops_configure,
+    .alloc = ops_alloc,
+    .free = ops_free,
+    .memcpy_to_device = ops_memcpy_to_device,
+    .memcpy_from_device = ops_memcpy_from_device,
+    .synchronize = ops_synchronize,
+    .allocator_usage = ops_allocator_usage,
+    .graph_batch_begin = ops_graph_batch_begin,
+    .graph_batch_end = ops_graph_batch_end,
+    .on_host_ptr_freed = ops_on_host_ptr_freed,
+    .on_host_range_freed = ops_on_host_range_freed,
 };
 
 // ------------------------------------------------------------------ impl functions
-marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind_t expect_kind, const marmot_tensor_t *input,
-                                const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
-                                marmot_tensor_t *out) {
-    Backend *b = backend_of(device_ctx);
+typedef struct {
+    int kind, in_dtype, out_dtype, bias_dtype;
+    size_t N, K, M;
+} matmul_plan_t;
+
+static marmot_error_t matmul_locked(hip_backend_t *b, const matmul_plan_t *p, const marmot_tensor_t *input,
+                                    const marmot_tensor_t *weight, const marmot_tensor_t *bias, marmot_tensor_t *out) {
+    const void *d_w = nullptr, *d_x = nullptr, *d_b = nullptr;
+    void *d_y = nullptr;
+    marmot_error_t st = acquire_read(b, weight->data, p->M * marmot_hip_row_bytes(p->kind, p->K), &d_w);
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, input->data, dense_bytes(input), &d_x);
+    }
+    if (st == MARMOT_SUCCESS && bias != nullptr) {
+        st = acquire_read(b, bias->data, dense_bytes(bias), &d_b);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write(b, out->data, dense_bytes(out), &d_y);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    const int rc = marmot_hip_matmul_quantized(b->dev, p->kind, d_w, d_x, p->in_dtype, p->N, p->K, p->M, d_b,
+                                               p->bias_dtype, d_y, p->out_dtype, 0);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(out);
+    return MARMOT_SUCCESS;
+}
+
+static marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind_t expect_kind,
+                                       const marmot_tensor_t *input, const marmot_tensor_t *weight,
+                                       const marmot_matmul_epilogue_t *epilogue, marmot_tensor_t *out) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || weight == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantized matmul: null argument");
     }
@@ -507,11 +566,19 @@ marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind_t expe
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE,
                     "Quantized matmul requires FLOAT32 input or FLOAT16 activations with FLOAT16/FLOAT32 output");
     }
-    const size_t N = input->shape.shape[0], K = input->shape.shape[1], M = weight->shape.shape[0];
-    if (weight->shape.shape[1] != K) {
+    matmul_plan_t p = {
+        .kind = (int)weight->quant_kind,
+        .in_dtype = in32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16,
+        .out_dtype = out32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16,
+        .bias_dtype = MARMOT_HIP_DTYPE_F32,
+        .N = input->shape.shape[0],
+        .K = input->shape.shape[1],
+        .M = weight->shape.shape[0],
+    };
+    if (weight->shape.shape[1] != p.K) {
         return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Quantized matmul dimension mismatch on K");
     }
-    if (out->shape.shape[0] != N || out->shape.shape[1] != M) {
+    if (out->shape.shape[0] != p.N || out->shape.shape[1] != p.M) {
         return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Quantized matmul output shape mismatch");
     }
     if (weight->quant_kind != expect_kind || !kind_supported_weight(weight->quant_kind)) {
@@ -524,61 +591,72 @@ marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind_t expe
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantized matmul: tensor without data");
     }
     const marmot_tensor_t *bias = epilogue != nullptr ? epilogue->bias : nullptr;
-    int bias_dtype = MARMOT_HIP_DTYPE_F32;
     if (bias != nullptr) {
-        size_t bn = 1;
-        for (size_t i = 0; i < bias->shape.ndim; ++i) {
-            bn *= bias->shape.shape[i];
-        }
-        if (bn != M) {
+        if (tensor_numel(bias) != p.M) {
             return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Quantized matmul bias length mismatch");
         }
         if (bias->dtype == MARMOT_DTYPE_FLOAT16) {
-            bias_dtype = MARMOT_HIP_DTYPE_F16;
+            p.bias_dtype = MARMOT_HIP_DTYPE_F16;
         } else if (bias->dtype != MARMOT_DTYPE_FLOAT32) {
             return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantized matmul bias must be FLOAT32 or FLOAT16");
         }
     }
-    if (N == 0 || M == 0) {
+    if (p.N == 0 || p.M == 0) {
         mark_device_output(out);
         return MARMOT_SUCCESS;
     }
-
-    std::lock_guard<std::mutex> lock(b->mu);
-    const int kind = (int)weight->quant_kind;
-    const void *d_w = nullptr, *d_x = nullptr, *d_b = nullptr;
-    void *d_y = nullptr;
-    marmot_error_t st = b->acquire_read(weight->data, M * marmot_hip_row_bytes(kind, K), &d_w);
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_read(input->data, dense_bytes(input), &d_x);
-    }
-    if (st == MARMOT_SUCCESS && bias != nullptr) {
-        st = b->acquire_read(bias->data, dense_bytes(bias), &d_b);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_write(out->data, dense_bytes(out), &d_y);
-    }
-    if (st != MARMOT_SUCCESS) {
-        return st;
-    }
-    int rc = marmot_hip_matmul_quantized(b->dev, kind, d_w, d_x, in32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, N,
-                                         K, M, d_b, bias_dtype, d_y, out32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16,
-                                         0);
-    if (rc != MARMOT_HIP_SUCCESS) {
-        return fail_from_lib(rc);
-    }
-    mark_device_output(out);
-    return MARMOT_SUCCESS;
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = matmul_locked(b, &p, input, weight, bias, out);
+    pthread_mutex_unlock(&b->mu);
+    return st;
 }
 
 // bytes of E expert slices of [rows, cols] blocks; expert tensors are stored [cols, rows, E] in GGUF order
 // (cpu_moe_execute_grouped, src/backends/cpu/ops/moe/moe_ops.c:895-899)
-size_t expert_tensor_bytes(int kind, size_t rows, size_t cols, size_t experts) {
+static size_t expert_tensor_bytes(int kind, size_t rows, size_t cols, size_t experts) {
     return experts * rows * marmot_hip_row_bytes(kind, cols);
 }
 
-marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_experts_desc_t *desc) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t moe_locked(hip_backend_t *b, const marmot_moe_experts_desc_t *desc, size_t T, size_t H, size_t F,
+                                 size_t E, size_t k) {
+    const marmot_tensor_t *h = desc->hidden_states, *g = desc->gate_exps, *u = desc->up_exps, *d = desc->down_exps;
+    const int kgu = (int)g->quant_kind, kd = (int)d->quant_kind;
+    const void *d_h = nullptr, *d_g = nullptr, *d_u = nullptr, *d_d = nullptr, *d_ids = nullptr, *d_wts = nullptr;
+    void *d_out = nullptr;
+    marmot_error_t st = acquire_read(b, h->data, dense_bytes(h), &d_h);
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, g->data, expert_tensor_bytes(kgu, F, H, E), &d_g);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, u->data, expert_tensor_bytes(kgu, F, H, E), &d_u);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, d->data, expert_tensor_bytes(kd, H, F, E), &d_d);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, desc->topk_ids->data, dense_bytes(desc->topk_ids), &d_ids);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, desc->topk_weights->data, dense_bytes(desc->topk_weights), &d_wts);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write(b, desc->out->data, dense_bytes(desc->out), &d_out);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    const int rc = marmot_hip_moe_experts(b->dev, (const float *)d_h, T, H, F, E, k, kgu, kd, d_g, d_u, d_d,
+                                          (const int32_t *)d_ids, (const float *)d_wts, desc->weights_scale,
+                                          (int)desc->router_weight_policy, (int)desc->ffn_type, (float *)d_out);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(desc->out);
+    return MARMOT_SUCCESS;
+}
+
+static marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_experts_desc_t *desc) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || desc == nullptr || desc->hidden_states == nullptr || desc->gate_exps == nullptr ||
         desc->up_exps == nullptr || desc->down_exps == nullptr || desc->topk_ids == nullptr ||
         desc->topk_weights == nullptr || desc->out == nullptr) {
@@ -616,44 +694,36 @@ marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_experts_desc
         mark_device_output(desc->out);
         return MARMOT_SUCCESS;
     }
-    std::lock_guard<std::mutex> lock(b->mu);
-    const int kgu = (int)g->quant_kind, kd = (int)d->quant_kind;
-    const void *d_h = nullptr, *d_g = nullptr, *d_u = nullptr, *d_d = nullptr, *d_ids = nullptr, *d_wts = nullptr;
-    void *d_out = nullptr;
-    marmot_error_t st = b->acquire_read(h->data, dense_bytes(h), &d_h);
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = moe_locked(b, desc, T, H, F, E, k);
+    pthread_mutex_unlock(&b->mu);
+    return st;
+}
+
+static marmot_error_t topk_locked(hip_backend_t *b, const marmot_topk_desc_t *desc, size_t rows, size_t cols) {
+    const void *d_x = nullptr;
+    void *d_v = nullptr, *d_i = nullptr;
+    marmot_error_t st = acquire_read(b, desc->x->data, dense_bytes(desc->x), &d_x);
     if (st == MARMOT_SUCCESS) {
-        st = b->acquire_read(g->data, expert_tensor_bytes(kgu, F, H, E), &d_g);
+        st = acquire_write(b, desc->values_out->data, dense_bytes(desc->values_out), &d_v);
     }
     if (st == MARMOT_SUCCESS) {
-        st = b->acquire_read(u->data, expert_tensor_bytes(kgu, F, H, E), &d_u);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_read(d->data, expert_tensor_bytes(kd, H, F, E), &d_d);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_read(desc->topk_ids->data, dense_bytes(desc->topk_ids), &d_ids);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_read(desc->topk_weights->data, dense_bytes(desc->topk_weights), &d_wts);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_write(desc->out->data, dense_bytes(desc->out), &d_out);
+        st = acquire_write(b, desc->indices_out->data, dense_bytes(desc->indices_out), &d_i);
     }
     if (st != MARMOT_SUCCESS) {
         return st;
     }
-    int rc = marmot_hip_moe_experts(b->dev, (const float *)d_h, T, H, F, E, k, kgu, kd, d_g, d_u, d_d,
-                                    (const int32_t *)d_ids, (const float *)d_wts, desc->weights_scale,
-                                    (int)desc->router_weight_policy, (int)desc->ffn_type, (float *)d_out);
+    const int rc = marmot_hip_topk(b->dev, (const float *)d_x, rows, cols, desc->k, (float *)d_v, (int32_t *)d_i);
     if (rc != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(rc);
     }
-    mark_device_output(desc->out);
+    mark_device_output(desc->values_out);
+    mark_device_output(desc->indices_out);
     return MARMOT_SUCCESS;
 }
 
-marmot_error_t topk(const void *device_ctx, const marmot_topk_desc_t *desc) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t topk(const void *device_ctx, const marmot_topk_desc_t *desc) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || desc == nullptr || desc->x == nullptr || desc->values_out == nullptr ||
         desc->indices_out == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "TopK descriptor is incomplete");
@@ -681,59 +751,25 @@ marmot_error_t topk(const void *device_ctx, const marmot_topk_desc_t *desc) {
     if (rows == 0) {
         return MARMOT_SUCCESS;
     }
-    std::lock_guard<std::mutex> lock(b->mu);
-    const void *d_x = nullptr;
-    void *d_v = nullptr, *d_i = nullptr;
-    marmot_error_t st = b->acquire_read(x->data, dense_bytes(x), &d_x);
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_write(desc->values_out->data, dense_bytes(desc->values_out), &d_v);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_write(desc->indices_out->data, dense_bytes(desc->indices_out), &d_i);
-    }
-    if (st != MARMOT_SUCCESS) {
-        return st;
-    }
-    int rc = marmot_hip_topk(b->dev, (const float *)d_x, rows, cols, k, (float *)d_v, (int32_t *)d_i);
-    if (rc != MARMOT_HIP_SUCCESS) {
-        return fail_from_lib(rc);
-    }
-    mark_device_output(desc->values_out);
-    mark_device_output(desc->indices_out);
-    return MARMOT_SUCCESS;
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = topk_locked(b, desc, rows, cols);
+    pthread_mutex_unlock(&b->mu);
+    return st;
 }
 
-marmot_error_t quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
-    Backend *b = backend_of(device_ctx);
-    if (b == nullptr || input == nullptr || output == nullptr) {
-        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize: null argument");
-    }
-    if (output->quant_kind != MARMOT_QUANT_KIND_Q8_0 && output->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP quantize produces the activation formats Q8_0 and Q8_K");
-    }
-    if (input->dtype != MARMOT_DTYPE_FLOAT32 && input->dtype != MARMOT_DTYPE_FLOAT16) {
-        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantize input must be FLOAT32 or FLOAT16");
-    }
-    if (input->shape.ndim != 2 || !rows_contiguous(input)) {
-        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize expects a contiguous 2D input");
-    }
-    const size_t rows = input->shape.shape[0], k = input->shape.shape[1];
+static marmot_error_t quantize_locked(hip_backend_t *b, const marmot_tensor_t *input, marmot_tensor_t *output,
+                                      size_t rows, size_t k) {
     const int kind = (int)output->quant_kind;
-    const size_t out_bytes = rows * marmot_hip_row_bytes(kind, k);
-    if (rows == 0 || k == 0) {
-        return MARMOT_SUCCESS;
-    }
-    std::lock_guard<std::mutex> lock(b->mu);
     const void *d_x = nullptr;
     void *d_q = nullptr;
-    marmot_error_t st = b->acquire_read(input->data, dense_bytes(input), &d_x);
+    marmot_error_t st = acquire_read(b, input->data, dense_bytes(input), &d_x);
     if (st == MARMOT_SUCCESS) {
-        st = b->acquire_write(output->data, out_bytes, &d_q);
+        st = acquire_write(b, output->data, rows * marmot_hip_row_bytes(kind, k), &d_q);
     }
     if (st != MARMOT_SUCCESS) {
         return st;
     }
-    int rc = marmot_hip_quantize_activations(
+    const int rc = marmot_hip_quantize_activations(
         b->dev, kind, d_x, input->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, rows, k,
         d_q);
     if (rc != MARMOT_HIP_SUCCESS) {
@@ -743,8 +779,52 @@ marmot_error_t quantize_block(const void *device_ctx, const marmot_tensor_t *inp
     return MARMOT_SUCCESS;
 }
 
-marmot_error_t dequantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
-    Backend *b = backend_of(device_ctx);
+static marmot_error_t quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || input == nullptr || output == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize: null argument");
+    }
+    if (output->quant_kind != MARMOT_QUANT_KIND_Q8_0 && output->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP quantize produces the activation formats Q8_0 and Q8_K");
+    }
+    if (input->dtype != MARMOT_DTYPE_FLOAT32 && input->dtype != MARMOT_DTYPE_FLOAT16) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantize input must be FLOAT32 or FLOAT16");
+    }
+    if (!rows_contiguous(input)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize expects a contiguous 2D input");
+    }
+    const size_t rows = input->shape.shape[0], k = input->shape.shape[1];
+    if (rows == 0 || k == 0) {
+        return MARMOT_SUCCESS;
+    }
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = quantize_locked(b, input, output, rows, k);
+    pthread_mutex_unlock(&b->mu);
+    return st;
+}
+
+static marmot_error_t dequantize_locked(hip_backend_t *b, const marmot_tensor_t *input, marmot_tensor_t *output,
+                                        size_t rows, size_t k) {
+    const int kind = (int)input->quant_kind;
+    const void *d_q = nullptr;
+    void *d_y = nullptr;
+    marmot_error_t st = acquire_read(b, input->data, rows * marmot_hip_row_bytes(kind, k), &d_q);
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write(b, output->data, dense_bytes(output), &d_y);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    const int rc = marmot_hip_dequantize(b->dev, kind, d_q, rows, k, (float *)d_y);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    mark_device_output(output);
+    return MARMOT_SUCCESS;
+}
+
+static marmot_error_t dequantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || input == nullptr || output == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize: null argument");
     }
@@ -754,7 +834,7 @@ marmot_error_t dequantize_block(const void *device_ctx, const marmot_tensor_t *i
     if (output->dtype != MARMOT_DTYPE_FLOAT32) {
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Dequantize output must be FLOAT32");
     }
-    if (output->shape.ndim != 2 || !rows_contiguous(output)) {
+    if (!rows_contiguous(output)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize expects a contiguous 2D output");
     }
     const size_t rows = output->shape.shape[0], k = output->shape.shape[1];
@@ -764,56 +844,42 @@ marmot_error_t dequantize_block(const void *device_ctx, const marmot_tensor_t *i
     if (rows == 0 || k == 0) {
         return MARMOT_SUCCESS;
     }
-    const int kind = (int)input->quant_kind;
-    std::lock_guard<std::mutex> lock(b->mu);
-    const void *d_q = nullptr;
-    void *d_y = nullptr;
-    marmot_error_t st = b->acquire_read(input->data, rows * marmot_hip_row_bytes(kind, k), &d_q);
-    if (st == MARMOT_SUCCESS) {
-        st = b->acquire_write(output->data, dense_bytes(output), &d_y);
-    }
-    if (st != MARMOT_SUCCESS) {
-        return st;
-    }
-    int rc = marmot_hip_dequantize(b->dev, kind, d_q, rows, k, (float *)d_y);
-    if (rc != MARMOT_HIP_SUCCESS) {
-        return fail_from_lib(rc);
-    }
-    mark_device_output(output);
-    return MARMOT_SUCCESS;
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = dequantize_locked(b, input, output, rows, k);
+    pthread_mutex_unlock(&b->mu);
+    return st;
 }
 
 // ------------------------------------------------------------------ bytecode exec entries
-inline uint16_t rd_u16(const uint8_t **pc) {
+static uint16_t rd_u16(const uint8_t **pc) {
     const uint16_t v = (uint16_t)((*pc)[0] | ((*pc)[1] << 8));
     *pc += 2;
     return v;
 }
-inline uint32_t rd_u32(const uint8_t **pc) {
+static uint32_t rd_u32(const uint8_t **pc) {
     const uint32_t v = (uint32_t)(*pc)[0] | ((uint32_t)(*pc)[1] << 8) | ((uint32_t)(*pc)[2] << 16) |
         ((uint32_t)(*pc)[3] << 24);
     *pc += 4;
     return v;
 }
-inline float rd_f32(const uint8_t **pc) {
+static float rd_f32(const uint8_t **pc) {
     const uint32_t bits = rd_u32(pc);
     float f;
     memcpy(&f, &bits, sizeof(f));
     return f;
 }
 
-inline marmot_tensor_t *reg(marmot_tensor_t **regs, uint16_t idx) {
+static marmot_tensor_t *reg(marmot_tensor_t **regs, uint16_t idx) {
     return idx == MARMOT_BC_REG_INVALID ? nullptr : regs[idx];
 }
 
-bool exec_args_ok(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm) {
-    const marmot_bc_exec_ctx_t *c = (const marmot_bc_exec_ctx_t *)exec_ctx;
+static bool exec_args_ok(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm) {
+    const marmot_bc_exec_ctx_t *c = exec_ctx;
     return c != nullptr && c->device_ctx != nullptr && regs != nullptr && imm != nullptr;
 }
 
-template <marmot_quant_kind_t KIND>
-marmot_error_t bc_exec_matmul(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
-                              const uint8_t *const_pool) {
+static marmot_error_t bc_exec_matmul(marmot_quant_kind_t kind, const void *exec_ctx, marmot_tensor_t **regs,
+                                     const uint8_t *imm, const uint8_t *const_pool) {
     if (!exec_args_ok(exec_ctx, regs, imm)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
     }
@@ -839,17 +905,28 @@ marmot_error_t bc_exec_matmul(const void *exec_ctx, marmot_tensor_t **regs, cons
         }
         epilogue.bias = reg(regs, bias_idx);  // the register wins over the pointer frozen into the pool
     }
-    return matmul_quantized(device_ctx, KIND, reg(regs, input_idx), reg(regs, weight_idx), epilogue_ptr,
+    return matmul_quantized(device_ctx, kind, reg(regs, input_idx), reg(regs, weight_idx), epilogue_ptr,
                             reg(regs, output_idx));
 }
 
-marmot_error_t bc_exec_moe(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+#define HIP_BC_MATMUL_ENTRY(name, kind)                                                                                \
+    static marmot_error_t name(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,                       \
+                               const uint8_t *const_pool) {                                                            \
+        return bc_exec_matmul(kind, exec_ctx, regs, imm, const_pool);                                                  \
+    }
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q4_0, MARMOT_QUANT_KIND_Q4_0)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q8_0, MARMOT_QUANT_KIND_Q8_0)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q4_k, MARMOT_QUANT_KIND_Q4_K)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q6_k, MARMOT_QUANT_KIND_Q6_K)
+
+static marmot_error_t bc_exec_moe(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                  const uint8_t *const_pool) {
+    (void)const_pool;
     if (!exec_args_ok(exec_ctx, regs, imm)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
     }
     const uint8_t *pc = imm;
-    marmot_moe_experts_desc_t desc;
-    memset(&desc, 0, sizeof(desc));
+    marmot_moe_experts_desc_t desc = {0};
     desc.hidden_states = reg(regs, rd_u16(&pc));
     desc.gate_exps = reg(regs, rd_u16(&pc));
     desc.up_exps = reg(regs, rd_u16(&pc));
@@ -863,12 +940,14 @@ marmot_error_t bc_exec_moe(const void *exec_ctx, marmot_tensor_t **regs, const u
     return moe_experts(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
 }
 
-marmot_error_t bc_exec_topk(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+static marmot_error_t bc_exec_topk(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                   const uint8_t *const_pool) {
+    (void)const_pool;
     if (!exec_args_ok(exec_ctx, regs, imm)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
     }
     const uint8_t *pc = imm;
-    marmot_topk_desc_t desc;
+    marmot_topk_desc_t desc = {0};
     desc.x = reg(regs, rd_u16(&pc));
     desc.values_out = reg(regs, rd_u16(&pc));
     desc.indices_out = reg(regs, rd_u16(&pc));
@@ -877,7 +956,9 @@ marmot_error_t bc_exec_topk(const void *exec_ctx, marmot_tensor_t **regs, const 
     return topk(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
 }
 
-marmot_error_t bc_exec_quantize(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+static marmot_error_t bc_exec_quantize(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                       const uint8_t *const_pool) {
+    (void)const_pool;
     if (!exec_args_ok(exec_ctx, regs, imm)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
     }
@@ -893,7 +974,9 @@ marmot_error_t bc_exec_quantize(const void *exec_ctx, marmot_tensor_t **regs, co
     return quantize_block(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, input, output);
 }
 
-marmot_error_t bc_exec_dequantize(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm, const uint8_t *) {
+static marmot_error_t bc_exec_dequantize(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                         const uint8_t *const_pool) {
+    (void)const_pool;
     if (!exec_args_ok(exec_ctx, regs, imm)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
     }
@@ -908,39 +991,33 @@ marmot_error_t bc_exec_dequantize(const void *exec_ctx, marmot_tensor_t **regs, 
     return dequantize_block(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, input, output);
 }
 
-const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
-    0,                      // END
-    12, 12, 12, 12,         // MATMUL: 3 x u16 + u32 + u16
-    26, 26, 26, 26,         // MOE_EXPERTS: 7 x u16 + u32 + f32 + u32
-    14,                     // TOPK: 3 x u16 + 2 x u32
-    16,                     // QUANTIZE: u16 + u32 + u16 + 2 x u32
-    12,                     // DEQUANTIZE: 2 x u16 + 2 x u32
+static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
+    0,               // END
+    12, 12, 12, 12,  // MATMUL: 3 x u16 + u32 + u16
+    26, 26, 26, 26,  // MOE_EXPERTS: 7 x u16 + u32 + f32 + u32
+    14,              // TOPK: 3 x u16 + 2 x u32
+    16,              // QUANTIZE: u16 + u32 + u16 + 2 x u32
+    12,              // DEQUANTIZE: 2 x u16 + 2 x u32
 };
 
-const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
+static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_INVALID,
-    MARMOT_BC_SCHEMA_MATMUL, MARMOT_BC_SCHEMA_MATMUL, MARMOT_BC_SCHEMA_MATMUL, MARMOT_BC_SCHEMA_MATMUL,
-    MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS,
-    MARMOT_BC_SCHEMA_MOE_EXPERTS,
-    MARMOT_BC_SCHEMA_TOPK,
-    MARMOT_BC_SCHEMA_QUANTIZE,
-    MARMOT_BC_SCHEMA_DEQUANTIZE,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MATMUL,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS,
+    MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_TOPK,
+    MARMOT_BC_SCHEMA_QUANTIZE,    MARMOT_BC_SCHEMA_DEQUANTIZE,
 };
 
-const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
+static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     nullptr,
-    bc_exec_matmul<MARMOT_QUANT_KIND_Q4_0>, bc_exec_matmul<MARMOT_QUANT_KIND_Q8_0>,
-    bc_exec_matmul<MARMOT_QUANT_KIND_Q4_K>, bc_exec_matmul<MARMOT_QUANT_KIND_Q6_K>,
-    bc_exec_moe, bc_exec_moe, bc_exec_moe, bc_exec_moe,
-    bc_exec_topk,
-    bc_exec_quantize,
-    bc_exec_dequantize,
+    bc_exec_matmul_q4_0, bc_exec_matmul_q8_0, bc_exec_matmul_q4_k, bc_exec_matmul_q6_k,
+    bc_exec_moe,         bc_exec_moe,         bc_exec_moe,         bc_exec_moe,
+    bc_exec_topk,        bc_exec_quantize,    bc_exec_dequantize,
 };
 
 // ------------------------------------------------------------------ kernel query
-marmot_kernel_selection_t unsupported(const char *reason) {
-    marmot_kernel_selection_t s;
-    memset(&s, 0, sizeof(s));
+static marmot_kernel_selection_t unsupported(const char *reason) {
+    marmot_kernel_selection_t s = {0};
     s.supported = false;
     s.kernel_id = MARMOT_KERNEL_INVALID;
     s.op_index = MARMOT_KERNEL_OP_INDEX_INVALID;
@@ -948,11 +1025,14 @@ marmot_kernel_selection_t unsupported(const char *reason) {
     return s;
 }
 
-marmot_kernel_selection_t selected(uint16_t op_index, double est_us, double workspace_mb) {
-    marmot_kernel_selection_t s;
-    memset(&s, 0, sizeof(s));
+static marmot_kernel_selection_t selected(uint16_t op_index, double est_us, double workspace_mb) {
+    marmot_kernel_selection_t s = {0};
     s.supported = true;
+#ifdef MARMOT_HIP_IN_TREE
+    s.kernel_id = marmot_hip_kernel_id_of_op(op_index);  // table emitted by the code generator
+#else
     s.kernel_id = (marmot_kernel_id_t)(MARMOT_KERNEL_HIP_BASE + op_index);
+#endif
     s.op_index = op_index;
     s.estimated_us = est_us;
     s.est_workspace_mb = workspace_mb;
@@ -960,7 +1040,7 @@ marmot_kernel_selection_t selected(uint16_t op_index, double est_us, double work
     return s;
 }
 
-int kind_of_scheme(marmot_qscheme_id_t q) {
+static int kind_of_scheme(marmot_qscheme_id_t q) {
     switch (q) {
     case MARMOT_QSCHEME_Q4_0:
         return MARMOT_HIP_KIND_Q4_0;
@@ -977,7 +1057,7 @@ int kind_of_scheme(marmot_qscheme_id_t q) {
     }
 }
 
-uint16_t matmul_op_of_kind(int kind) {
+static uint16_t matmul_op_of_kind(int kind) {
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_0:
         return MARMOT_HIP_BC_OP_MATMUL_Q4_0;
@@ -992,11 +1072,7 @@ uint16_t matmul_op_of_kind(int kind) {
     }
 }
 
-}  // namespace
-
 // ------------------------------------------------------------------ exports
-extern "C" {
-
 const marmot_device_ops_t *marmot_get_hip_ops(void) {
     return &k_hip_ops;
 }
@@ -1081,8 +1157,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
 }
 
 marmot_device_caps_t marmot_hip_detect_default_caps(void) {
-    marmot_device_caps_t c;
-    memset(&c, 0, sizeof(c));
+    marmot_device_caps_t c = {0};
     // published MI355X figures; a live device refines the counts
     c.peak_flops_tflops_fp32 = 157.3f;
     c.peak_flops_tflops_fp16 = 2500.0f;
@@ -1196,17 +1271,16 @@ marmot_error_t marmot_hip_backend_last_error(const char **detail_out) {
 }
 
 void marmot_hip_backend_residency_stats(const void *device_ctx, marmot_hip_residency_stats_t *out) {
-    Backend *b = backend_of(device_ctx);
+    hip_backend_t *b = backend_of(device_ctx);
     if (b == nullptr || out == nullptr) {
         return;
     }
-    std::lock_guard<std::mutex> lock(b->mu);
-    out->mirrors = b->mirrors.size();
+    pthread_mutex_lock(&b->mu);
+    out->mirrors = b->n_mirrors;
     out->mirrored_bytes = b->mirrored_bytes;
     out->uploads = b->uploads;
     out->upload_bytes = b->upload_bytes;
     out->downloads = b->downloads;
     out->download_bytes = b->download_bytes;
+    pthread_mutex_unlock(&b->mu);
 }
-
-}  // extern "C"

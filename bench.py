@@ -153,7 +153,7 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
         "frac_of_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4),
         "tokens_per_s": round(tokens / (ms * 1e-3), 1),
         "steps": steps,
-        "includes": "activation packing, GEMM and K-split reduction kernels",
+        "includes": "sub-block sums, GEMM and K-split reduction kernels",
     }
     for b in (d_w, d_x, d_out):
         b.free()

@@ -215,12 +215,6 @@ struct FmtQ4K {
     }
     template <int NC>
     __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int sub) {
-#ifdef MH_PROBE_NOALU
-        for (int n = 0; n < NC; ++n) {
-            acc[n] += __int_as_float((w.q.x ^ w.q.y ^ w.q.z ^ w.q.w ^ w.hdr.x ^ w.hdr.w) & 0x007fffff) * a[n].d;
-        }
-        return;
-#endif
         const int g = sub >> 1;
         const float d = h2f((uint16_t)(w.hdr.x & 0xffffu));
         const float dmin = h2f((uint16_t)(w.hdr.x >> 16));

@@ -27,7 +27,10 @@ if ROOT not in sys.path:
 METRIC = "Q4_K matvec GB/s (% HBM peak) + prefill GEMM TOPS (% MFMA peak)"
 HBM_PEAK_GBPS = 8000.0
 MALL_BYTES = 256 << 20
-TRAFFIC_DEFAULT_WORKLOAD = 33_297_000  # bytes per launch of the pre-packed Q4_K 4096x14336 N=1 matvec kernel
+# HBM bytes per launch of the Q4_K 4096x14336 N=1 matvec kernels (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain
+# copy kernel, profiles/matvec_q4_k_4096x14336_n1.md): fused-quantization kernel and kernel on pre-packed activations
+TRAFFIC_FUSED = 33_670_000
+TRAFFIC_PREPACKED = 33_297_000
 
 
 def algorithmic_bytes(kind_row_bytes: int, M: int, K: int, N: int) -> int:
@@ -160,6 +163,109 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
+def sweep(hip, steps: int, warmup: int):
+    """Every configuration of BASELINE.json on the device, one JSON line each (documentation runs, not the
+    driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
+    from marmot_amd import DT_F16, DT_F32, capi, row_bytes
+
+    rng = np.random.Generator(np.random.PCG64(7))
+    names = {capi.KIND_Q4_K: "Q4_K", capi.KIND_Q6_K: "Q6_K", capi.KIND_Q8_0: "Q8_0", capi.KIND_Q4_0: "Q4_0"}
+
+    def emit(rec):
+        print(json.dumps(rec), flush=True)
+
+    def linear_case(config, kind, M, K, N):
+        rb = row_bytes(kind, K)
+        stride = (M * rb + 255) & ~255
+        copies = max(2, -(-2 * MALL_BYTES // stride) + 1)
+        blocks = random_blocks(rng, kind, M, K)
+        d_w = hip.alloc(stride * copies)
+        for c in range(copies):
+            d_w.upload(blocks, offset=c * stride)
+        d_x = hip.to_device(rng.standard_normal((N, K), dtype=np.float32))
+        d_out = hip.alloc(N * M * 4)
+        ms = time_steps_graph(hip, lambda i: hip.linear_d(kind, d_w, d_x, DT_F32, N, K, M, d_out, DT_F32,
+                                                          weight_offset=(i % copies) * stride), steps, warmup)
+        nbytes = algorithmic_bytes(rb, M, K, N)
+        emit({"config": config, "workload": f"{names[kind]} {M}x{K} N={N}", "route": hip.last_route(),
+              "us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+              "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "tokens_per_s": round(N / ms * 1e3)})
+        for b in (d_w, d_x, d_out):
+            b.free()
+
+    linear_case("C1", capi.KIND_Q8_0, 5632, 2048, 1)
+    for kind in (capi.KIND_Q4_K, capi.KIND_Q6_K):
+        for (M, K) in ((14336, 4096), (4096, 14336)):
+            for N in (1, 4, 8):
+                linear_case("C2", kind, M, K, N)
+    for tokens in (64, 128, 512, 2048):
+        r = prefill_gemm(hip, tokens, max(20, steps // 20), 5)
+        emit({"config": "C3", "workload": f"Q4_K 4096x4096 N={tokens} fp16", "route": r["route"],
+              "us": round(r["ms_per_step"] * 1e3, 2), "TFLOP/s": r["tflops"],
+              "frac_of_mfma_peak": r["frac_of_mfma_peak"], "tokens_per_s": round(r["tokens_per_s"])})
+
+    # C4: the seven linears of one layer at 16 tokens; 4 copies of the 139 MB of weights rotate
+    N = 16
+    specs = [(capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 1024, 4096), (capi.KIND_Q6_K, 1024, 4096),
+             (capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 14336, 4096), (capi.KIND_Q4_K, 14336, 4096),
+             (capi.KIND_Q6_K, 4096, 14336)]
+    copies = 4
+    layers = []
+    total = 0
+    for kind, M, K in specs:
+        rb = row_bytes(kind, K)
+        stride = (M * rb + 255) & ~255
+        blocks = random_blocks(rng, kind, M, K)
+        d_w = hip.alloc(stride * copies)
+        for c in range(copies):
+            d_w.upload(blocks, offset=c * stride)
+        layers.append((kind, M, K, stride, d_w, hip.to_device(rng.standard_normal((N, K), dtype=np.float32)),
+                       hip.alloc(N * M * 4)))
+        total += algorithmic_bytes(rb, M, K, N)
+
+    def layer_step(i):
+        for kind, M, K, stride, d_w, d_x, d_out in layers:
+            hip.linear_d(kind, d_w, d_x, DT_F32, N, K, M, d_out, DT_F32, weight_offset=(i % copies) * stride)
+
+    ms = time_steps_graph(hip, layer_step, max(50, steps // 10), 10, chunk=50)
+    emit({"config": "C4", "workload": "7 linears of a Llama-3-8B layer (q,k,o,gate,up Q4_K; v,down Q6_K), N=16",
+          "us": round(ms * 1e3, 2), "GB/s": round(total / ms / 1e6, 1),
+          "frac_of_hbm_peak": round(total / ms / 1e6 / HBM_PEAK_GBPS, 4), "tokens_per_s": round(N / ms * 1e3),
+          "algorithmic_bytes": total})
+    for *_, d_w, d_x, d_out in layers:
+        for b in (d_w, d_x, d_out):
+            b.free()
+
+    # C5: 128 experts, top-8, hidden 2048, expert FFN 768, 64 tokens, all Q4_K; 2 copies of the 340 MB rotate
+    E, k, H, F, T = 128, 8, 2048, 768, 64
+    kind = capi.KIND_Q4_K
+    gu_bytes = E * F * row_bytes(kind, H)
+    dn_bytes = E * H * row_bytes(kind, F)
+    d_g, d_u, d_d = hip.alloc(2 * gu_bytes), hip.alloc(2 * gu_bytes), hip.alloc(2 * dn_bytes)
+    for buf, rows, cols, nb in ((d_g, E * F, H, gu_bytes), (d_u, E * F, H, gu_bytes), (d_d, E * H, F, dn_bytes)):
+        blocks = random_blocks(rng, kind, rows, cols)
+        buf.upload(blocks, offset=0)
+        buf.upload(blocks, offset=nb)
+    logits = rng.standard_normal((T, E), dtype=np.float32)
+    vals, ids = hip.topk(logits, k)
+    d_h = hip.to_device(rng.standard_normal((T, H), dtype=np.float32))
+    d_ids, d_wts = hip.to_device(ids), hip.to_device(hip.softmax_rows(vals))
+    d_out = hip.alloc(T * H * 4)
+    active = len(np.unique(ids))
+
+    def moe_step(i):
+        c = i % 2
+        hip.moe_experts_d(d_h, T, H, F, E, k, kind, kind, d_g, d_u, d_d, d_ids, d_wts, d_out,
+                          gate_offset=c * gu_bytes, up_offset=c * gu_bytes, down_offset=c * dn_bytes)
+
+    ms = time_steps_graph(hip, moe_step, max(50, steps // 10), 10, chunk=50)
+    nbytes = active * (2 * F * row_bytes(kind, H) + H * row_bytes(kind, F)) + 2 * T * H * 4
+    emit({"config": "C5", "workload": f"MoE experts E={E} top-{k} H={H} F={F} T={T} Q4_K ({active} active experts)",
+          "us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+          "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4), "tokens_per_s": round(T / ms * 1e3),
+          "algorithmic_bytes": nbytes})
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,6 +278,8 @@ def main():
     ap.add_argument("--kind", default="q4_k", choices=["q4_k", "q6_k", "q8_0", "q4_0"])
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--prefill-tokens", type=int, default=512)
+    ap.add_argument("--sweep", action="store_true",
+                    help="measure every BASELINE configuration instead, one JSON line each (documentation runs)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")
     args = ap.parse_args()
@@ -192,6 +300,12 @@ def main():
         print(json.dumps({"calibration": "plain 16-byte copy kernel", "bytes_read": n, "bytes_written": n,
                           "launches": 23, "ms_per_launch": round(ms, 5),
                           "gbps_read_plus_write": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
+        hip.close()
+        return
+
+    if args.sweep:
+        hip = HipBackend(0)
+        sweep(hip, args.steps, args.warmup)
         hip.close()
         return
 
@@ -243,7 +357,9 @@ def main():
     ms_hot = time_steps_graph(hip, kstep_hot, args.steps, args.warmup)
 
     value = nbytes / (ms_op * 1e-3) / 1e9
-    achieved = nbytes / (ms_k * 1e-3) / 1e9
+    fused = route.endswith("_fused")  # the whole op is then one kernel: that kernel is the dominant one
+    ms_dom, ms_dom_eager = (ms_op, ms_op_eager) if fused else (ms_k, ms_k_eager)
+    achieved = nbytes / (ms_dom * 1e-3) / 1e9
     result = {
         "metric": METRIC,
         "value": round(value, 2),
@@ -282,9 +398,13 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy kernel
             # (profiles/matvec_q4_k_4096x14336_n1.md); only valid for the default workload
-            "traffic": TRAFFIC_DEFAULT_WORKLOAD if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) else None,
-            "avg_launch_us": round(ms_k * 1e3, 3),
-            "avg_launch_us_eager": round(ms_k_eager * 1e3, 3),
+            "traffic": (TRAFFIC_FUSED if fused else TRAFFIC_PREPACKED)
+            if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) else None,
+            "avg_launch_us": round(ms_dom * 1e3, 3),
+            "avg_launch_us_eager": round(ms_dom_eager * 1e3, 3),
+            # the matvec on activations quantized beforehand (the kernel N > 4 uses), and with the weights cache-resident
+            "prepacked_kernel_us": round(ms_k * 1e3, 3),
+            "prepacked_kernel_gbps": round(nbytes / (ms_k * 1e-3) / 1e9, 2),
             "cache_resident_gbps": round(nbytes / (ms_hot * 1e-3) / 1e9, 2),
         },
     }

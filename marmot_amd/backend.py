@@ -272,6 +272,18 @@ class HipBackend:
             d_x.free()
             d_o.free()
 
+    def moe_experts_d(self, d_hidden, T: int, H: int, F: int, E: int, k_per_token: int, kind_gate_up: int,
+                      kind_down: int, d_gate, d_up, d_down, d_ids, d_weights, d_out, weights_scale: float = 1.0,
+                      policy: int = 1, ffn_type: int = 0, gate_offset: int = 0, up_offset: int = 0,
+                      down_offset: int = 0):
+        """Device-pointer form of moe_experts (everything already resident; the offsets select one of several
+        expert-stack copies inside the weight buffers)."""
+        check(self.lib.marmot_hip_moe_experts(
+            self.dev, C.c_void_p(d_hidden.ptr), T, H, F, E, k_per_token, kind_gate_up, kind_down,
+            C.c_void_p(d_gate.ptr + gate_offset), C.c_void_p(d_up.ptr + up_offset),
+            C.c_void_p(d_down.ptr + down_offset), C.c_void_p(d_ids.ptr), C.c_void_p(d_weights.ptr), weights_scale,
+            policy, ffn_type, C.c_void_p(d_out.ptr)))
+
     def moe_experts(self, hidden, gate, up, down, topk_ids, topk_weights, F: int, E: int, kind_gate_up: int,
                     kind_down: int, weights_scale: float = 1.0, policy: int = 1, ffn_type: int = 0) -> np.ndarray:
         hidden = np.ascontiguousarray(hidden, dtype=np.float32)

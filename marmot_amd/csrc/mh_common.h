@@ -157,6 +157,15 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
                           size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1);
 int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
+// small-batch int8-MFMA matmul (mh_mmq.hip)
+bool mmq_supported(int kind, size_t N, size_t K);
+size_t mmq_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, bool dual);
+int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
+               size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
+               void *scratch);
+// sums fp32 partials [splits][N][M] in split order, then bias and output cast (mh_gemm.hip)
+int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
+                         const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M);
 int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                     const void *d_bias, int bias_dtype, void *d_out, int out_dtype);

@@ -466,6 +466,21 @@ __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ p
     }
 }
 
+int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
+                         const void *d_bias, int bias_dtype, void *d_out, int out_dtype) {
+    const size_t total = N * M;
+    const int bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16, out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    if (total % 4 == 0 && M % 4 == 0) {
+        hipLaunchKernelGGL(k_gemm_reduce<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, dev->stream,
+                           partial, splits, N, M, d_bias, bias_is_f16, d_out, out_is_f16);
+    } else {
+        hipLaunchKernelGGL(k_gemm_reduce<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream, partial,
+                           splits, N, M, d_bias, bias_is_f16, d_out, out_is_f16);
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
 bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M) {
     if (getenv("MARMOT_HIP_NO_GEMM") != nullptr) {
         return false;
@@ -548,15 +563,10 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
                        dim3(G_THREADS), 2 * STAGE, dev->stream, p);
     MH_HIP(hipGetLastError());
     if (splits > 1) {
-        const size_t total = N * M;
-        if (total % 4 == 0) {
-            hipLaunchKernelGGL(k_gemm_reduce<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, dev->stream,
-                               partial, (int)splits, N, M, d_bias, p.bias_is_f16, d_out, p.out_is_f16);
-        } else {
-            hipLaunchKernelGGL(k_gemm_reduce<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream,
-                               partial, (int)splits, N, M, d_bias, p.bias_is_f16, d_out, p.out_is_f16);
+        st = launch_splitk_reduce(dev, partial, (int)splits, N, M, d_bias, bias_dtype, d_out, out_dtype);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return st;
         }
-        MH_HIP(hipGetLastError());
     }
     set_route("gemm_q4_k_f16_mfma");
     return MARMOT_HIP_SUCCESS;

@@ -207,12 +207,14 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     // packed route. fp32 activations whose rows are whole blocks are quantized inside the matvec kernel; otherwise
     // the activations are quantized once into the workspace (shared by both weights of a dual call).
-    if (in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input)) {
+    const bool mmq = mmq_supported(kind, N, K);
+    if (!mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input)) {
         return launch_matvec_packed(dev, kind, d_w0, d_w1, nullptr, (const float *)d_input, N, K, M, d_bias,
                                     bias_dtype, d_out0, d_out1, out_dtype);
     }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
-    const size_t need = act_scratch_layout(act_kind, N, K, nullptr, nullptr);
+    const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
+    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, N, K, M, d_w1 != nullptr) : 0);
     void *ws = nullptr;
     int st = workspace_reserve(dev, need, &ws);
     if (st != MARMOT_HIP_SUCCESS) {
@@ -223,6 +225,10 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
+    }
+    if (mmq) {
+        return launch_mmq(dev, kind, d_w0, d_w1, act, N, K, M, d_bias, bias_dtype, d_out0, d_out1, out_dtype,
+                          (uint8_t *)ws + act_bytes);
     }
     return launch_matvec_packed(dev, kind, d_w0, d_w1, &act, nullptr, N, K, M, d_bias, bias_dtype, d_out0, d_out1,
                                 out_dtype);
@@ -294,6 +300,11 @@ int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     ActScratch act;
     act_scratch_layout(act_kind, N, K, const_cast<void *>(d_packed), &act);
+    if (mmq_supported(kind, N, K)) {
+        MH_HIP(hipSetDevice(dev->device_index));
+        return launch_mmq(dev, kind, d_weight, nullptr, act, N, K, M, d_bias, bias_dtype, d_out, nullptr, out_dtype,
+                          nullptr);
+    }
     return launch_matvec_packed(dev, kind, d_weight, nullptr, &act, nullptr, N, K, M, d_bias, bias_dtype, d_out,
                                 nullptr, out_dtype);
 }

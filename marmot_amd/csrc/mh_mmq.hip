@@ -1,0 +1,433 @@
+// Small-batch quantized matmul on the int8 matrix cores: Q4_K weights x Q8_K activations for 3..16 activation rows
+// per pass (continuous-batching decode, the layer stack at 16 sequences, MoE expert segments).
+//
+// Same integer arithmetic as cpu_vec_dot_q4_k_q8_k (vec_dot_impl.h:689-732): per 256-value block
+//     bsum = sum_j sc_j * (q_j . a_j),   msum = sum_j mn_j * (sum of a over sub-block j),
+//     y += (a.d * w.d) * bsum - (a.d * w.dmin) * msum
+// but the 32-value sub-block dots of 32 weight rows x up to 32 activation rows are one v_mfma_i32_32x32x32_i8:
+// activations are the row operand (token i = lane % 32), unpacked nibbles of weight row j = lane % 32 the column
+// operand, so every lane ends up with the int32 dots of ITS weight row against 16 tokens and applies its own 6-bit
+// scale with one integer multiply-add per token. The min term needs sum_k mn_j(k) * a_k, which is a second MFMA per
+// sub-block with the byte mn_j broadcast as the column operand, chained through the accumulator over the 8
+// sub-blocks. All integer results are exact; only the fp32 accumulation over blocks is ordered differently from the
+// CPU (per wavefront sequential, then across the K-split in a fixed order).
+//
+// A wavefront owns 32 weight rows and a contiguous range of blocks; W wavefronts of a workgroup and S workgroups
+// split K so that the chip is filled even when M / 32 is small. Weights stream from HBM exactly once per pass
+// (20 bytes x 5 loads per lane and block, two blocks in flight); activations (int8, L2-resident) are read straight
+// into operand registers.
+#include "mh_common.h"
+
+#include <stdlib.h>
+
+namespace mh {
+
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+
+struct MmqParams {
+    const uint8_t *w[2];   // Q4_K blocks, M rows of nb blocks (second weight of a dual call or nullptr)
+    void *out[2];          // [N][M] of out dtype, or fp32 partials [splits][N][M] when splits > 1
+    const int8_t *qs;      // quantized activations, rows of kp bytes
+    const float *ad;       // activation block scales [rows][nb]
+    size_t kp;
+    size_t N, M, nb;
+    size_t n0;             // first activation row of this pass
+    int ncols;             // activation rows of this pass (<= 32)
+    int bpw;               // blocks per wavefront
+    int splits;            // workgroups along K
+    const void *bias;
+    int bias_is_f16;
+    int out_is_f16;
+    // grouped (MoE) mode: blockIdx.z selects a work item = up to 8 consecutive routes of one expert
+    const int4 *items;
+    const int *n_items;
+    const uint32_t *act_index;
+    size_t expert_stride;
+};
+
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef const __attribute__((address_space(1))) uint8_t glb_u8;
+
+constexpr int MMQ_TOK = 16;                // activation rows per pass
+constexpr int MMQ_WBLK = 32 * Q4_K_BYTES;  // one block of 32 weight rows: 4608 bytes
+constexpr int MMQ_ABLK = MMQ_TOK * QK_K;   // one block of 16 activation rows: 4096 bytes
+constexpr int MMQ_STAGE = MMQ_WBLK + MMQ_ABLK + MMQ_TOK * 4;  // + the 16 activation scales of the block
+constexpr int MMQ_STAGES = 2;              // blocks in flight per wavefront
+constexpr int MMQ_STAGE_LOADS = 10;        // memory instructions per stage: 5 weights + 4 activations + 1 scales
+
+// Work decomposition. All wavefronts of a workgroup work on the SAME 32 weight rows; wavefront w walks its own
+// contiguous range of blocks, so the workgroup as a whole streams whole weight rows (a decomposition in which a
+// workgroup covers many rows and a narrow K range measured 2.7x slower in HBM time for the same bytes). Every
+// wavefront has a private ring of stages in LDS, filled by direct-to-LDS loads: weights [32 rows][144 B] (9 chunks
+// per row: 16-byte reads of consecutive rows fall into different bank groups), activations [16 tokens][256 B] with
+// the 16-byte chunks XOR-swizzled by token, and the 16 activation scales. No workgroup barrier until the final
+// reduction over the K-split.
+//
+// NR: live accumulator registers per lane: 4 for up to 8 activation rows, 8 for up to 16 (token of register r:
+// 8 * (r / 4) + 4 * kh + r % 4, the row layout of the 32x32 MFMA result).
+template <int NR>
+__global__ __launch_bounds__(512) void k_mmq_q4k(const MmqParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
+    const int j = lane & 31, kh = lane >> 5;
+    // blockIdx.y = K-split index, interleaved with the weight selector of a dual call
+    const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
+    const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
+    const uint8_t *wbase = p.w[which];
+    size_t n0 = p.n0;
+    int ncols = p.ncols;
+    if (p.items != nullptr) {
+        if ((int)blockIdx.z >= *p.n_items) {
+            return;  // uniform for the whole workgroup
+        }
+        const int4 it = p.items[blockIdx.z];
+        wbase += (size_t)it.x * p.expert_stride;
+        n0 = (size_t)it.y;
+        ncols = it.z;
+    }
+    const size_t b0 = ((size_t)split * W + wave) * p.bpw;
+    size_t b1 = b0 + p.bpw;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = b1 > b0 ? (int)(b1 - b0) : 0;
+    uint8_t *ring = lds + (size_t)wave * MMQ_STAGES * MMQ_STAGE;
+
+    // ---- per-lane source offsets of the direct-to-LDS loads (block-independent)
+    const size_t row0 = (size_t)blockIdx.x * 32;
+    uint32_t w_off[5];  // weights: 288 chunks of 16 bytes in row order (9 per row)
+#pragma unroll
+    for (int c = 0; c < 5; ++c) {
+        const int chunk = c * 64 + lane;
+        int row = chunk / 9;
+        const int piece = chunk - row * 9;
+        if (row > 31) {
+            row = 31;
+        }
+        size_t m = row0 + row;
+        if (m >= p.M) {
+            m = p.M - 1;  // harmless re-read; never stored
+        }
+        w_off[c] = (uint32_t)((m - row0) * p.nb * Q4_K_BYTES + 16 * piece);
+    }
+    const uint8_t *wgroup = wbase + row0 * p.nb * Q4_K_BYTES;
+    uint32_t a_off[4];  // activations: 256 chunks, chunk (token, slot) holds source chunk slot ^ token
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int chunk = c * 64 + lane;
+        const int slot = chunk & 15, tk = chunk >> 4;
+        const int tt = tk < ncols ? tk : 0;  // rows beyond ncols re-read the first row; their results are not stored
+        const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+        a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
+    }
+    uint32_t ad_off;
+    {
+        const int tk = lane & 15;
+        const int tt = tk < ncols ? tk : 0;
+        const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+        ad_off = (uint32_t)(arow * p.nb);
+    }
+    auto stage_block = [&](size_t b, uint8_t *dst) {
+#pragma unroll
+        for (int c = 0; c < 5; ++c) {
+            if (c < 4 || lane < 32) {  // 288 = 4 * 64 + 32 chunks
+                __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + b * Q4_K_BYTES),
+                                                 (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            __builtin_amdgcn_global_load_lds((glb_u8 *)(p.qs + a_off[c] + b * QK_K),
+                                             (lds_u8 *)(dst + MMQ_WBLK + c * 1024), 16, 0, 0);
+        }
+        if (lane < MMQ_TOK) {
+            __builtin_amdgcn_global_load_lds((glb_u8 *)(p.ad + ad_off + b), (lds_u8 *)(dst + MMQ_WBLK + MMQ_ABLK), 4,
+                                             0, 0);
+        }
+    };
+    // memory loads complete in order: waiting until at most one stage's loads are outstanding means the older stage
+    // has landed
+    auto wait_all_but = [&](int stages) {
+        if (stages >= 1) {
+            __builtin_amdgcn_s_waitcnt(0x0f70 | MMQ_STAGE_LOADS);
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+        }
+    };
+#pragma unroll
+    for (int st = 0; st < MMQ_STAGES; ++st) {
+        if (st < nblk) {
+            stage_block(b0 + st, ring + st * MMQ_STAGE);
+        }
+    }
+
+    float acc[NR];
+    int tok[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        acc[r] = 0.0f;
+        tok[r] = 8 * (r >> 2) + 4 * kh + (r & 3);
+    }
+    // MFMA row operand of this lane: token j % 16 (rows 16..31 of the product repeat rows 0..15 and are ignored),
+    // chunk 2 * sb + kh of the block, stored at slot chunk ^ token
+    const int ti = j & 15;
+
+    for (int blk = 0; blk < nblk; ++blk) {
+        wait_all_but(nblk - 1 - blk >= 1 ? 1 : 0);
+        const uint8_t *stage = ring + (blk % MMQ_STAGES) * MMQ_STAGE;
+        const uint8_t *wcur = stage + j * Q4_K_BYTES;
+        const uint8_t *a_blk = stage + MMQ_WBLK + ti * QK_K;
+        const float *ad_blk = (const float *)(stage + MMQ_WBLK + MMQ_ABLK);
+        // all LDS operands of the block are requested up front, so that no LDS latency sits inside the MFMA chain
+        const uint4 hdr = *(const uint4 *)wcur;
+        uint4 aq[8], wq4[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            wq4[g] = *(const uint4 *)(wcur + 16 + 32 * g + 16 * kh);
+        }
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            aq[sb] = *(const uint4 *)(a_blk + 16 * ((2 * sb + kh) ^ ti));
+        }
+        float adr[NR];
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            adr[r] = ad_blk[tok[r]];
+        }
+        // the stage is refilled with block blk + MMQ_STAGES once its reads have returned
+        __builtin_amdgcn_sched_barrier(0);
+        if (blk + MMQ_STAGES < nblk) {
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+            stage_block(b0 + blk + MMQ_STAGES, ring + (blk % MMQ_STAGES) * MMQ_STAGE);
+        }
+        // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
+        const float d = h2f((uint16_t)(hdr.x & 0xffffu));
+        const float dmin = h2f((uint16_t)(hdr.x >> 16));
+        const uint32_t sc_lo = hdr.y & 0x3f3f3f3fu;
+        const uint32_t mn_lo = hdr.z & 0x3f3f3f3fu;
+        const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
+        const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+        int bsum[NR];
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            bsum[r] = 0;
+        }
+        auto acts_of = [&](int sb) {
+            return intx4{(int)aq[sb].x, (int)aq[sb].y, (int)aq[sb].z, (int)aq[sb].w};
+        };
+        auto weights_of = [&](int sb) {
+            const uint4 wq = wq4[sb >> 1];
+            if (sb & 1) {
+                return intx4{(int)((wq.x >> 4) & 0x0f0f0f0fu), (int)((wq.y >> 4) & 0x0f0f0f0fu),
+                             (int)((wq.z >> 4) & 0x0f0f0f0fu), (int)((wq.w >> 4) & 0x0f0f0f0fu)};
+            }
+            return intx4{(int)(wq.x & 0x0f0f0f0fu), (int)(wq.y & 0x0f0f0f0fu), (int)(wq.z & 0x0f0f0f0fu),
+                         (int)(wq.w & 0x0f0f0f0fu)};
+        };
+        const intx16 zero = {0};
+        intx16 dm = {0};
+        intx16 dq[2];
+        dq[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(0), weights_of(0), zero, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            const int sc = (int)(((sb < 4 ? sc_lo : sc_hi) >> (8 * (sb & 3))) & 0xffu);
+            const int mn = (int)(((sb < 4 ? mn_lo : mn_hi) >> (8 * (sb & 3))) & 0xffu);
+            const int mn4 = mn * 0x01010101;
+            dm = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb), intx4{mn4, mn4, mn4, mn4}, dm, 0, 0, 0);
+            if (sb < 7) {
+                dq[(sb + 1) & 1] =
+                    __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb + 1), weights_of(sb + 1), zero, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                bsum[r] += __mul24(dq[sb & 1][r], sc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            acc[r] += (adr[r] * d) * (float)bsum[r] - (adr[r] * dmin) * (float)dm[r];
+        }
+    }
+
+    // ---- K-split within the workgroup: partial sums meet in LDS and are added in wavefront order
+    if (W > 1) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();  // every wavefront is done with its ring; the memory is reused for the reduction
+        float *red = (float *)lds;
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            red[(wave * NR + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (wave != 0) {
+            return;
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            float sum = red[r * 64 + lane];
+            for (int w2 = 1; w2 < W; ++w2) {
+                sum += red[(w2 * NR + r) * 64 + lane];
+            }
+            acc[r] = sum;
+        }
+    }
+    const size_t mm = row0 + j;
+    if (mm >= p.M) {
+        return;
+    }
+    void *out = p.out[which];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        if (tok[r] >= ncols) {
+            continue;
+        }
+        const size_t n = n0 + tok[r];
+        if (p.splits > 1) {
+            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
+        } else if (!p.out_is_f16) {
+            float v = acc[r];
+            if (p.bias != nullptr) {
+                v += ((const float *)p.bias)[mm];
+            }
+            ((float *)out)[n * p.M + mm] = v;
+        } else {
+            uint16_t h = f2h(acc[r]);  // reference order: store f16(dot), then add the bias to the stored value
+            if (p.bias != nullptr) {
+                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+                h = f2h(h2f(h) + bv);
+            }
+            ((uint16_t *)out)[n * p.M + mm] = h;
+        }
+    }
+}
+
+bool mmq_supported(int kind, size_t N, size_t K) {
+    if (getenv("MARMOT_HIP_NO_MMQ") != nullptr) {
+        return false;
+    }
+    return kind == MARMOT_HIP_KIND_Q4_K && N >= 3 && K % QK_K == 0;
+}
+
+constexpr size_t MMQ_ROWS_PER_PASS = MMQ_TOK;
+
+struct MmqPlan {
+    int W, S, bpw;
+};
+
+// W wavefronts per workgroup and S workgroups split K so that at least one workgroup per CU is resident
+static MmqPlan mmq_plan(const marmot_hip_device *dev, size_t M, size_t nb) {
+    const size_t rg = (M + 31) / 32;
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    MmqPlan pl;
+    size_t W = nb < 4 ? nb : 4;
+    size_t S = 1;
+    while (rg * S < cus && W * S * 2 <= nb) {
+        S *= 2;
+    }
+    if (const char *e = getenv("MH_MMQ_W")) {
+        W = (size_t)atoi(e);
+    }
+    if (const char *e = getenv("MH_MMQ_S")) {
+        S = (size_t)atoi(e);
+    }
+    const size_t bpw = (nb + W * S - 1) / (W * S);
+    pl.W = (int)W;
+    pl.S = (int)((nb + bpw * W - 1) / (bpw * W));
+    pl.bpw = (int)bpw;
+    return pl;
+}
+
+// bytes of fp32 partials launch_mmq needs for this shape (0 when K is not split across workgroups)
+size_t mmq_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, bool dual) {
+    const MmqPlan pl = mmq_plan(dev, M, K / QK_K);
+    return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (dual ? 2 : 1) : 0;
+}
+
+static size_t mmq_lds_bytes(int W) {
+    const size_t ring = (size_t)W * MMQ_STAGES * MMQ_STAGE;
+    const size_t red = (size_t)W * 8 * 64 * sizeof(float);
+    return ring > red ? ring : red;
+}
+
+template <int NR>
+static int mmq_launch(marmot_hip_device *dev, const MmqParams &p, const MmqPlan &pl, size_t M, bool dual,
+                      unsigned items) {
+    const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * (dual ? 2 : 1)), items);
+    static bool attr_set = false;
+    if (!attr_set) {
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)mmq_lds_bytes(8)));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((k_mmq_q4k<NR>), grid, dim3(pl.W * 64), mmq_lds_bytes(pl.W), dev->stream, p);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+// Dense: N activation rows in passes of up to 32. scratch: mmq_scratch_bytes() bytes, or nullptr to take them from
+// the device workspace (only when the activations do not live there).
+int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
+               size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
+               void *scratch) {
+    if (!mmq_supported(kind, N, K)) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
+    }
+    const size_t nb = K / QK_K;
+    const bool dual = d_w1 != nullptr;
+    const MmqPlan pl = mmq_plan(dev, M, nb);
+    float *partial = (float *)scratch;
+    if (pl.S > 1 && partial == nullptr) {
+        void *ws = nullptr;
+        int st = workspace_reserve(dev, mmq_scratch_bytes(dev, N, K, M, dual), &ws);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return st;
+        }
+        partial = (float *)ws;
+    }
+    MmqParams p;
+    p.w[0] = (const uint8_t *)d_w0;
+    p.w[1] = (const uint8_t *)d_w1;
+    p.out[0] = pl.S > 1 ? (void *)partial : d_out0;
+    p.out[1] = pl.S > 1 ? (void *)(partial + (size_t)pl.S * N * M) : d_out1;
+    p.qs = act.qs;
+    p.ad = act.d;
+    p.kp = act.kp;
+    p.N = N;
+    p.M = M;
+    p.nb = nb;
+    p.bpw = pl.bpw;
+    p.splits = pl.S;
+    p.bias = d_bias;
+    p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
+    p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    p.items = nullptr;
+    p.n_items = nullptr;
+    p.act_index = nullptr;
+    p.expert_stride = 0;
+    // 16 activation rows per pass: 8 live accumulator registers per lane keep two wavefronts per SIMD resident
+    // (32 rows per pass would need 16 and spill)
+    for (size_t n0 = 0; n0 < N; n0 += MMQ_ROWS_PER_PASS) {
+        p.n0 = n0;
+        p.ncols = (int)(N - n0 < MMQ_ROWS_PER_PASS ? N - n0 : MMQ_ROWS_PER_PASS);
+        const int st = p.ncols <= 8 ? mmq_launch<4>(dev, p, pl, M, dual, 1) : mmq_launch<8>(dev, p, pl, M, dual, 1);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return st;
+        }
+    }
+    if (pl.S > 1) {
+        for (int which = 0; which < (dual ? 2 : 1); ++which) {
+            int st = launch_splitk_reduce(dev, partial + (size_t)which * pl.S * N * M, pl.S, N, M, d_bias, bias_dtype,
+                                          which ? d_out1 : d_out0, out_dtype);
+            if (st != MARMOT_HIP_SUCCESS) {
+                return st;
+            }
+        }
+    }
+    set_route("mmq_q4_k_q8_k_mfma");
+    return MARMOT_HIP_SUCCESS;
+}
+
+} // namespace mh

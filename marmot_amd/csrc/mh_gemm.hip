@@ -434,16 +434,27 @@ __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ p
     for (int e = 0; e < V; ++e) {
         v[e] = 0.0f;
     }
-    for (int s = 0; s < splits; ++s) {
-        const float *src = partial + (size_t)s * total + idx;
-        if (V == 4) {
-            const float4 t = *(const float4 *)src;
-            v[0] += t.x;
-            v[1 % V] += t.y;
-            v[2 % V] += t.z;
-            v[3 % V] += t.w;
-        } else {
-            v[0] += src[0];
+    // loads of 4 splits are issued together (one memory latency per 4 splits); the additions stay in split order
+    for (int s0 = 0; s0 < splits; s0 += 4) {
+        float4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = s0 + u < splits ? s0 + u : splits - 1;
+            const float *src = partial + (size_t)s * total + idx;
+            if (V == 4) {
+                t[u] = *(const float4 *)src;
+            } else {
+                t[u] = make_float4(src[0], 0.0f, 0.0f, 0.0f);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (s0 + u < splits) {
+                v[0] += t[u].x;
+                v[1 % V] += t[u].y;
+                v[2 % V] += t[u].z;
+                v[3 % V] += t[u].w;
+            }
         }
     }
 #pragma unroll
@@ -470,12 +481,17 @@ int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int split
                          const void *d_bias, int bias_dtype, void *d_out, int out_dtype) {
     const size_t total = N * M;
     const int bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16, out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
-    if (total % 4 == 0 && M % 4 == 0) {
-        hipLaunchKernelGGL(k_gemm_reduce<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, dev->stream,
-                           partial, splits, N, M, d_bias, bias_is_f16, d_out, out_is_f16);
+    // small outputs: one wavefront per workgroup, so that the few thousand threads spread over the whole chip
+    const bool vec = total % 4 == 0 && M % 4 == 0;
+    const size_t threads = vec ? total / 4 : total;
+    const unsigned block = threads < 65536 ? 64u : 256u;
+    const dim3 grid((unsigned)((threads + block - 1) / block));
+    if (vec) {
+        hipLaunchKernelGGL(k_gemm_reduce<4>, grid, dim3(block), 0, dev->stream, partial, splits, N, M, d_bias,
+                           bias_is_f16, d_out, out_is_f16);
     } else {
-        hipLaunchKernelGGL(k_gemm_reduce<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream, partial,
-                           splits, N, M, d_bias, bias_is_f16, d_out, out_is_f16);
+        hipLaunchKernelGGL(k_gemm_reduce<1>, grid, dim3(block), 0, dev->stream, partial, splits, N, M, d_bias,
+                           bias_is_f16, d_out, out_is_f16);
     }
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;

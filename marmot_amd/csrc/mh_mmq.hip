@@ -1,4 +1,4 @@
-// Small-batch quantized matmul on the int8 matrix cores: Q4_K weights x Q8_K activations for 3..16 activation rows
+// Small-batch quantized matmul on the int8 matrix cores: Q4_K / Q6_K weights x Q8_K activations for 3..16 activation rows
 // per pass (continuous-batching decode, the layer stack at 16 sequences, MoE expert segments).
 //
 // Same integer arithmetic as cpu_vec_dot_q4_k_q8_k (vec_dot_impl.h:689-732): per 256-value block
@@ -304,11 +304,255 @@ __global__ __launch_bounds__(512) void k_mmq_q4k(const MmqParams p) {
     }
 }
 
+// ------------------------------------------------------------------ Q6_K x Q8_K
+// Same decomposition; the differences follow from the format (q6k_gguf.c:63-99, vec_dot_impl.h:783-828):
+//   * 16 scale groups of 16 values per block -> 16 MFMAs of K = 16 (v_mfma_i32_32x32x16_i8), signed int8 scales;
+//   * weights are 6-bit values minus 32: the MFMA runs on the unsigned values 0..63 and the offset is taken out as
+//     32 * sum_is sc_is * (sum of a over group is), which is one more MFMA per group with the scale byte broadcast
+//     as the column operand, chained through the accumulator (exact integers, like the CPU's use of bsums);
+//   * blocks are 210 bytes and rows only 2-byte aligned, so weights are fetched with unaligned 16-byte register
+//     loads (14 pieces per row, the last one overlapping) and written to the LDS stage with a row stride of 240 B.
+constexpr int MMQ6_ROWB = 240;                    // LDS bytes per weight row of a stage (15 chunks: conflict-free)
+constexpr int MMQ6_WBLK = 32 * MMQ6_ROWB;         // 7680
+constexpr int MMQ6_STAGE = MMQ6_WBLK + MMQ_ABLK + MMQ_TOK * 4;
+
+template <int NR>
+__global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
+    const int j = lane & 31, kh = lane >> 5;
+    const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
+    const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
+    const uint8_t *wbase = p.w[which];
+    size_t n0 = p.n0;
+    int ncols = p.ncols;
+    if (p.items != nullptr) {
+        if ((int)blockIdx.z >= *p.n_items) {
+            return;
+        }
+        const int4 it = p.items[blockIdx.z];
+        wbase += (size_t)it.x * p.expert_stride;
+        n0 = (size_t)it.y;
+        ncols = it.z;
+    }
+    const size_t b0 = ((size_t)split * W + wave) * p.bpw;
+    size_t b1 = b0 + p.bpw;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = b1 > b0 ? (int)(b1 - b0) : 0;
+    uint8_t *ring = lds + (size_t)wave * 2 * MMQ6_STAGE;
+
+    const size_t row0 = (size_t)blockIdx.x * 32;
+    uint32_t w_off[7], w_lds[7];  // 448 pieces of 16 bytes: 14 per row, piece 13 covers bytes 194..209
+#pragma unroll
+    for (int c = 0; c < 7; ++c) {
+        const int idx = c * 64 + lane;
+        const int row = idx / 14, pc = idx - row * 14;
+        size_t m = row0 + row;
+        if (m >= p.M) {
+            m = p.M - 1;  // harmless re-read; never stored
+        }
+        w_off[c] = (uint32_t)((m - row0) * p.nb * Q6_K_BYTES + (pc < 13 ? 16 * pc : 194));
+        w_lds[c] = (uint32_t)(row * MMQ6_ROWB + 16 * pc);
+    }
+    const uint8_t *wgroup = wbase + row0 * p.nb * Q6_K_BYTES;
+    uint32_t a_off[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int chunk = c * 64 + lane;
+        const int slot = chunk & 15, tk = chunk >> 4;
+        const int tt = tk < ncols ? tk : 0;
+        const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+        a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
+    }
+    uint32_t ad_off;
+    {
+        const int tk = lane & 15;
+        const int tt = tk < ncols ? tk : 0;
+        const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+        ad_off = (uint32_t)(arow * p.nb);
+    }
+    uint4 wreg[7];
+    auto fetch_block = [&](size_t b, uint8_t *dst) {
+#pragma unroll
+        for (int c = 0; c < 7; ++c) {
+            uint4 t;
+            __builtin_memcpy(&t, wgroup + w_off[c] + b * Q6_K_BYTES, 16);  // unaligned 16-byte load
+            wreg[c] = t;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            __builtin_amdgcn_global_load_lds((glb_u8 *)(p.qs + a_off[c] + b * QK_K),
+                                             (lds_u8 *)(dst + MMQ6_WBLK + c * 1024), 16, 0, 0);
+        }
+        if (lane < MMQ_TOK) {
+            __builtin_amdgcn_global_load_lds((glb_u8 *)(p.ad + ad_off + b), (lds_u8 *)(dst + MMQ6_WBLK + MMQ_ABLK), 4,
+                                             0, 0);
+        }
+    };
+    auto commit_weights = [&](uint8_t *dst) {
+#pragma unroll
+        for (int c = 0; c < 7; ++c) {
+            *(uint4 *)(dst + w_lds[c]) = wreg[c];
+        }
+    };
+    if (nblk > 0) {
+        fetch_block(b0, ring);
+        __builtin_amdgcn_s_waitcnt(0);
+        commit_weights(ring);
+    }
+
+    float acc[NR];
+    int tok[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        acc[r] = 0.0f;
+        tok[r] = 8 * (r >> 2) + 4 * kh + (r & 3);
+    }
+    const int ti = j & 15;
+
+    for (int blk = 0; blk < nblk; ++blk) {
+        const bool more = blk + 1 < nblk;
+        uint8_t *next_stage = ring + ((blk + 1) & 1) * MMQ6_STAGE;
+        const uint8_t *stage = ring + (blk & 1) * MMQ6_STAGE;
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the weight rows written by this wavefront are in LDS
+        if (more) {
+            fetch_block(b0 + blk + 1, next_stage);  // the other stage was last read one block ago
+        }
+        const uint8_t *wrow = stage + j * MMQ6_ROWB;
+        const uint8_t *a_blk = stage + MMQ6_WBLK + ti * QK_K + 8 * kh;
+        const float *ad_blk = (const float *)(stage + MMQ6_WBLK + MMQ_ABLK);
+        const uint4 scv = *(const uint4 *)(wrow + 192);
+        const float d = h2f(*(const uint16_t *)(wrow + 222));
+        uint2 ql[2][2][2], qh[2][2];  // [half][second 32][second 16], [half][second 16]: this lane's 8 bytes each
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int s16 = 0; s16 < 2; ++s16) {
+                qh[h][s16] = *(const uint2 *)(wrow + 128 + 32 * h + 16 * s16 + 8 * kh);
+#pragma unroll
+                for (int h32 = 0; h32 < 2; ++h32) {
+                    ql[h][h32][s16] = *(const uint2 *)(wrow + 64 * h + 32 * h32 + 16 * s16 + 8 * kh);
+                }
+            }
+        }
+        float adr[NR];
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            adr[r] = ad_blk[tok[r]];
+        }
+        int bsum[NR];
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            bsum[r] = 0;
+        }
+        const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+        auto acts_of = [&](int is) {
+            const uint2 v = *(const uint2 *)(a_blk + 16 * (is ^ ti));
+            return (long)(((unsigned long)v.y << 32) | v.x);
+        };
+        auto weights_of = [&](int is) {
+            const int h = is >> 3, q = (is >> 1) & 3, s16 = is & 1;
+            const uint2 l = ql[h][q & 1][s16], hh = qh[h][s16];
+            uint32_t x = (q >> 1) ? ((l.x >> 4) & 0x0f0f0f0fu) : (l.x & 0x0f0f0f0fu);
+            uint32_t y = (q >> 1) ? ((l.y >> 4) & 0x0f0f0f0fu) : (l.y & 0x0f0f0f0fu);
+            x |= ((hh.x >> (2 * q)) & 0x03030303u) << 4;
+            y |= ((hh.y >> (2 * q)) & 0x03030303u) << 4;
+            return (long)(((unsigned long)y << 32) | x);
+        };
+        const intx16 zero = {0};
+        intx16 ds = {0};
+        intx16 dq[2];
+        long av[2];
+        av[0] = acts_of(0);
+        dq[0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[0], weights_of(0), zero, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int is = 0; is < 16; ++is) {
+            const uint32_t scb = (scw[is >> 2] >> (8 * (is & 3))) & 0xffu;
+            const int sc = (int)(int8_t)scb;
+            const uint32_t sc4 = scb * 0x01010101u;
+            ds = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[is & 1], (long)(((unsigned long)sc4 << 32) | sc4), ds, 0, 0, 0);
+            if (is < 15) {
+                av[(is + 1) & 1] = acts_of(is + 1);
+                dq[(is + 1) & 1] =
+                    __builtin_amdgcn_mfma_i32_32x32x16_i8(av[(is + 1) & 1], weights_of(is + 1), zero, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                bsum[r] += __mul24(dq[is & 1][r], sc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            acc[r] += (adr[r] * d) * (float)(bsum[r] - 32 * ds[r]);
+        }
+        if (more) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next block's weights and activations have landed
+            commit_weights(next_stage);
+        }
+    }
+
+    if (W > 1) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        float *red = (float *)lds;
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            red[(wave * NR + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (wave != 0) {
+            return;
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            float sum = red[r * 64 + lane];
+            for (int w2 = 1; w2 < W; ++w2) {
+                sum += red[(w2 * NR + r) * 64 + lane];
+            }
+            acc[r] = sum;
+        }
+    }
+    const size_t mm = row0 + j;
+    if (mm >= p.M) {
+        return;
+    }
+    void *out = p.out[which];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        if (tok[r] >= ncols) {
+            continue;
+        }
+        const size_t n = n0 + tok[r];
+        if (p.splits > 1) {
+            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
+        } else if (!p.out_is_f16) {
+            float v = acc[r];
+            if (p.bias != nullptr) {
+                v += ((const float *)p.bias)[mm];
+            }
+            ((float *)out)[n * p.M + mm] = v;
+        } else {
+            uint16_t h = f2h(acc[r]);
+            if (p.bias != nullptr) {
+                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+                h = f2h(h2f(h) + bv);
+            }
+            ((uint16_t *)out)[n * p.M + mm] = h;
+        }
+    }
+}
+
 bool mmq_supported(int kind, size_t N, size_t K) {
     if (getenv("MARMOT_HIP_NO_MMQ") != nullptr) {
         return false;
     }
-    return kind == MARMOT_HIP_KIND_Q4_K && N >= 3 && K % QK_K == 0;
+    // below these row counts the fused-quantization matvec is faster (no separate quantization pass)
+    const size_t min_rows = kind == MARMOT_HIP_KIND_Q4_K ? 3 : 5;
+    return (kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && N >= min_rows && K % QK_K == 0;
 }
 
 constexpr size_t MMQ_ROWS_PER_PASS = MMQ_TOK;
@@ -346,23 +590,30 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_
     return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (dual ? 2 : 1) : 0;
 }
 
-static size_t mmq_lds_bytes(int W) {
-    const size_t ring = (size_t)W * MMQ_STAGES * MMQ_STAGE;
+static size_t mmq_lds_bytes(int kind, int W) {
+    const size_t stage = kind == MARMOT_HIP_KIND_Q6_K ? (size_t)MMQ6_STAGE : (size_t)MMQ_STAGE;
+    const size_t ring = (size_t)W * MMQ_STAGES * stage;
     const size_t red = (size_t)W * 8 * 64 * sizeof(float);
     return ring > red ? ring : red;
 }
 
 template <int NR>
-static int mmq_launch(marmot_hip_device *dev, const MmqParams &p, const MmqPlan &pl, size_t M, bool dual,
+static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, size_t M, bool dual,
                       unsigned items) {
     const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * (dual ? 2 : 1)), items);
     static bool attr_set = false;
     if (!attr_set) {
         MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)mmq_lds_bytes(8)));
+                                   (int)mmq_lds_bytes(MARMOT_HIP_KIND_Q4_K, 8)));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)mmq_lds_bytes(MARMOT_HIP_KIND_Q6_K, 6)));
         attr_set = true;
     }
-    hipLaunchKernelGGL((k_mmq_q4k<NR>), grid, dim3(pl.W * 64), mmq_lds_bytes(pl.W), dev->stream, p);
+    if (kind == MARMOT_HIP_KIND_Q6_K) {
+        hipLaunchKernelGGL((k_mmq_q6k<NR>), grid, dim3(pl.W * 64), mmq_lds_bytes(kind, pl.W), dev->stream, p);
+    } else {
+        hipLaunchKernelGGL((k_mmq_q4k<NR>), grid, dim3(pl.W * 64), mmq_lds_bytes(kind, pl.W), dev->stream, p);
+    }
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
 }
@@ -412,7 +663,8 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
     for (size_t n0 = 0; n0 < N; n0 += MMQ_ROWS_PER_PASS) {
         p.n0 = n0;
         p.ncols = (int)(N - n0 < MMQ_ROWS_PER_PASS ? N - n0 : MMQ_ROWS_PER_PASS);
-        const int st = p.ncols <= 8 ? mmq_launch<4>(dev, p, pl, M, dual, 1) : mmq_launch<8>(dev, p, pl, M, dual, 1);
+        const int st =
+            p.ncols <= 8 ? mmq_launch<4>(dev, kind, p, pl, M, dual, 1) : mmq_launch<8>(dev, kind, p, pl, M, dual, 1);
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
         }
@@ -426,7 +678,7 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
             }
         }
     }
-    set_route("mmq_q4_k_q8_k_mfma");
+    set_route(kind == MARMOT_HIP_KIND_Q6_K ? "mmq_q6_k_q8_k_mfma" : "mmq_q4_k_q8_k_mfma");
     return MARMOT_HIP_SUCCESS;
 }
 

@@ -163,6 +163,10 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);
+bool mmq_grouped_supported(int kind, size_t K);
+int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
+                       const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
+                       size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1);
 // sums fp32 partials [splits][N][M] in split order, then bias and output cast (mh_gemm.hip)
 int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
                          const void *d_bias, int bias_dtype, void *d_out, int out_dtype);

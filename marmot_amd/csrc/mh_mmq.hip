@@ -682,4 +682,67 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
     return MARMOT_HIP_SUCCESS;
 }
 
+// Grouped (MoE): every work item is up to 8 consecutive routes of one expert; blockIdx.z walks the item list the
+// route kernel wrote (workgroups beyond *d_n_items exit at once). Expert matrices are small, so K is split over the
+// wavefronts of a workgroup only when a row is long enough to keep each of them busy for several blocks.
+bool mmq_grouped_supported(int kind, size_t K) {
+    return (kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && K % QK_K == 0 &&
+           getenv("MARMOT_HIP_NO_MMQ") == nullptr;
+}
+
+int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
+                       const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
+                       size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1) {
+    if (max_items == 0 || M == 0 || K == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    if (!mmq_grouped_supported(kind, K)) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "grouped MFMA matmul: unsupported kind or shape");
+    }
+    if (max_items > 65535) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "grouped MFMA matmul: %zu work items exceed the grid limit",
+                         max_items);
+    }
+    const size_t nb = K / QK_K;
+    MmqPlan pl;
+    size_t W = nb >= 16 ? 4 : (nb >= 8 ? 2 : 1);
+    if (const char *e = getenv("MH_MMQ_GW")) {
+        W = (size_t)atoi(e);
+    }
+    if (W > nb) {
+        W = nb;
+    }
+    pl.W = (int)W;
+    pl.S = 1;
+    pl.bpw = (int)((nb + W - 1) / W);
+    MmqParams p;
+    p.w[0] = (const uint8_t *)d_w0;
+    p.w[1] = (const uint8_t *)d_w1;
+    p.out[0] = d_out0;
+    p.out[1] = d_out1;
+    p.qs = act.qs;
+    p.ad = act.d;
+    p.kp = act.kp;
+    p.N = 0;
+    p.M = M;
+    p.nb = nb;
+    p.n0 = 0;
+    p.ncols = 0;
+    p.bpw = pl.bpw;
+    p.splits = 1;
+    p.bias = nullptr;
+    p.bias_is_f16 = 0;
+    p.out_is_f16 = 0;
+    p.items = d_items;
+    p.n_items = d_n_items;
+    p.act_index = d_act_index;
+    p.expert_stride = expert_stride;
+    const int st = mmq_launch<4>(dev, kind, p, pl, M, d_w1 != nullptr, (unsigned)max_items);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    set_route(kind == MARMOT_HIP_KIND_Q6_K ? "moe_grouped_q6_k_q8_k_mfma" : "moe_grouped_q4_k_q8_k_mfma");
+    return MARMOT_HIP_SUCCESS;
+}
+
 } // namespace mh

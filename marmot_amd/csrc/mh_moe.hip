@@ -14,40 +14,54 @@ constexpr int MOE_MAX_EXPERTS = 1024;
 constexpr int MOE_MAX_TOPK = 64;
 
 // ------------------------------------------------------------------ top-k (cpu_topk_impl, moe_ops.c:789-889)
-// One thread per row; insertion into a k-long sorted list, ties to the lower index — the same comparisons as the
-// reference, so values and indices are identical.
-__global__ __launch_bounds__(64) void k_topk(const float *__restrict__ x, size_t rows, size_t cols, size_t k,
-                                             float *__restrict__ values, int32_t *__restrict__ indices) {
-    const size_t row = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+// The reference inserts the columns in ascending order into a k-long list sorted by value, a new value going in
+// front of the first strictly smaller one: the result is the first k columns under the total order (value
+// descending, column ascending) among the values greater than -FLT_MAX; NaNs never compare true and are skipped;
+// unfilled slots keep (-FLT_MAX, -1). One wavefront per row selects that sequence directly: round r finds the
+// largest element that comes strictly after the previous pick in the same order.
+__global__ __launch_bounds__(256) void k_topk(const float *__restrict__ x, size_t rows, size_t cols, size_t k,
+                                              float *__restrict__ values, int32_t *__restrict__ indices) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= rows) {
-        return;
+        return;  // uniform per wavefront
     }
-    float *bv = values + row * k;
-    int32_t *bi = indices + row * k;
-    for (size_t i = 0; i < k; ++i) {
-        bv[i] = -FLT_MAX;
-        bi[i] = -1;
-    }
-    for (size_t col = 0; col < cols; ++col) {
-        const float v = x[row * cols + col];
-        size_t pos = k;
-        for (size_t i = 0; i < k; ++i) {
-            const bool better = v > bv[i];
-            const bool same = v == bv[i] && (int32_t)col < bi[i];
-            if (better || same) {
-                pos = i;
-                break;
+    const float *in = x + row * cols;
+    float last_v = INFINITY;
+    int last_i = -1;
+    bool done = false;
+    for (size_t r = 0; r < k; ++r) {
+        float bv = -FLT_MAX;
+        int bi = -1;
+        if (!done) {
+            for (size_t col = lane; col < cols; col += 64) {
+                const float v = in[col];
+                const bool after_last = v < last_v || (v == last_v && (int)col > last_i);
+                if (after_last && v > bv) {  // ascending columns: an equal later value never replaces
+                    bv = v;
+                    bi = (int)col;
+                }
+            }
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) {
+                const float ov = __shfl_xor(bv, d, 64);
+                const int oi = __shfl_xor(bi, d, 64);
+                if (ov > bv || (ov == bv && oi >= 0 && oi < bi)) {
+                    bv = ov;
+                    bi = oi;
+                }
+            }
+            if (bi < 0) {
+                done = true;
+            } else {
+                last_v = bv;
+                last_i = bi;
             }
         }
-        if (pos == k) {
-            continue;
+        if (lane == 0) {
+            values[row * k + r] = bv;
+            indices[row * k + r] = bi;
         }
-        for (size_t i = k - 1; i > pos; --i) {
-            bv[i] = bv[i - 1];
-            bi[i] = bi[i - 1];
-        }
-        bv[pos] = v;
-        bi[pos] = (int32_t)col;
     }
 }
 
@@ -95,101 +109,206 @@ struct RouteArgs {
     int decode_order;
 };
 
-__global__ __launch_bounds__(256) void k_moe_route(const RouteArgs a) {
+constexpr int MOE_ROUTE_LDS = 4096;    // routes whose ids and positions are kept in LDS
+constexpr int MOE_ROUTE_WAVES = 8;     // wavefronts of the route kernel; each fills one contiguous chunk of routes
+
+// exclusive prefix sum over the 64 lanes of a wavefront; *total receives the sum over all lanes
+__device__ __forceinline__ int wave_excl_scan(int v, int lane, int *total) {
+    int incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) {
+            incl += up;
+        }
+    }
+    *total = __shfl(incl, 63, 64);
+    return incl - v;
+}
+
+// rank = number of lower lanes holding the same id, cnt = number of lanes holding it
+__device__ __forceinline__ void wave_rank(int id, int lane, int *rank, int *cnt) {
+    int rk = 0, c = 0;
+#pragma unroll
+    for (int j = 0; j < 64; ++j) {
+        const int idj = __builtin_amdgcn_readlane(id, j);
+        const bool same = idj == id;
+        c += same ? 1 : 0;
+        rk += (same && j < lane) ? 1 : 0;
+    }
+    *rank = rk;
+    *cnt = c;
+}
+
+__device__ __forceinline__ void route_emit(const RouteArgs &a, int r, int pos) {
+    a.route_pos[r] = pos;
+    if (pos < 0) {
+        return;
+    }
+    const int t = r / a.k;
+    float norm = a.weights_scale;
+    if (a.renormalize) {
+        float wsum = 0.0f;
+        for (int s = 0; s < a.k; ++s) {
+            wsum += a.topk_weights[t * a.k + s];
+        }
+        norm = wsum > FLT_MIN ? a.weights_scale / wsum : 0.0f;
+    }
+    a.sorted_tokens[pos] = (uint32_t)t;
+    a.sorted_weights[pos] = a.topk_weights[r] * norm;
+}
+
+__global__ __launch_bounds__(MOE_ROUTE_WAVES * 64) void k_moe_route(const RouteArgs a) {
     __shared__ int counts[MOE_MAX_EXPERTS];
-    __shared__ int cursor[MOE_MAX_EXPERTS];
+    __shared__ int wcount[MOE_ROUTE_WAVES][MOE_MAX_EXPERTS];  // per chunk: routes of each expert, then its cursor
+    __shared__ int ids_l[MOE_ROUTE_LDS];  // expert id of each route (-1 = invalid), later its sorted position
     const int routes = a.T * a.k;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    if (a.decode_order) {
+        // At most 64 routes: one wavefront, one round. Experts are laid out in order of first appearance, so the
+        // segment of an expert starts at the number of routes whose expert appeared earlier: an exclusive scan of
+        // the expert's route count over the lanes that hold a first appearance.
+        if (wave != 0) {
+            return;
+        }
+        int id = -1;
+        if (lane < routes) {
+            id = a.topk_ids[lane];
+            if (id < 0 || id >= a.E) {
+                id = -1;
+            }
+        }
+        const unsigned long long bad = __ballot(lane < routes && id < 0);
+        int rank, cnt;
+        wave_rank(id, lane, &rank, &cnt);
+        const bool first = id >= 0 && rank == 0;
+        int total, n_items;
+        const int seg = wave_excl_scan(first ? cnt : 0, lane, &total);
+        const int item0 = wave_excl_scan(first ? (cnt + MOE_ITEM_COLS - 1) / MOE_ITEM_COLS : 0, lane, &n_items);
+        if (first) {
+            counts[id] = seg;
+            int n = item0;
+            for (int j = 0; j < cnt; j += MOE_ITEM_COLS) {
+                a.items[n++] = make_int4(id, seg + j, (cnt - j) < MOE_ITEM_COLS ? (cnt - j) : MOE_ITEM_COLS, 0);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the segment starts are in LDS (same wavefront)
+        if (lane < routes) {
+            route_emit(a, lane, id >= 0 ? counts[id] + rank : -1);
+        }
+        if (lane == 0) {
+            *a.n_items = n_items;
+            *a.error_flag = bad != 0 ? 1 : 0;
+        }
+        return;
+    }
+
+    const bool in_lds = routes <= MOE_ROUTE_LDS;
     for (int e = tid; e < a.E; e += blockDim.x) {
-        counts[e] = 0;
+#pragma unroll
+        for (int w = 0; w < MOE_ROUTE_WAVES; ++w) {
+            wcount[w][e] = 0;
+        }
+    }
+    if (tid == 0) {
+        *a.error_flag = 0;
     }
     __syncthreads();
-    for (int r = tid; r < routes; r += blockDim.x) {
-        const int id = a.topk_ids[r];
+    // chunk of wavefront w: routes [w * chunk, (w + 1) * chunk), a multiple of 64
+    const int chunk = ((routes + MOE_ROUTE_WAVES * 64 - 1) / (MOE_ROUTE_WAVES * 64)) * 64;
+    const int r_begin = wave * chunk;
+    const int r_end = r_begin + chunk < routes ? r_begin + chunk : routes;
+    for (int r = r_begin + lane; r < r_end; r += 64) {
+        int id = a.topk_ids[r];
         if (id < 0 || id >= a.E) {
             *a.error_flag = 1;
+            id = -1;
         } else {
-            atomicAdd(&counts[id], 1);
+            atomicAdd(&wcount[wave][id], 1);
+        }
+        if (in_lds) {
+            ids_l[r] = id;
         }
     }
     __syncthreads();
-    if (tid == 0) {
-        int prefix = 0;
-        int n = 0;
-        auto place = [&](int e) {
+    for (int e = tid; e < a.E; e += blockDim.x) {
+        int c = 0;
+#pragma unroll
+        for (int w = 0; w < MOE_ROUTE_WAVES; ++w) {
+            c += wcount[w][e];
+        }
+        counts[e] = c;
+    }
+    __syncthreads();
+    // exclusive prefix over experts in ascending id and the work items of every expert: lane l of the first
+    // wavefront owns the experts [l * per, (l + 1) * per)
+    if (wave == 0) {
+        const int per = (a.E + 63) / 64;
+        const int e0 = lane * per;
+        const int e1 = e0 + per < a.E ? e0 + per : a.E;
+        int c_sum = 0, i_sum = 0;
+        for (int e = e0; e < e1; ++e) {
             const int c = counts[e];
-            cursor[e] = prefix;
+            c_sum += c;
+            i_sum += (c + MOE_ITEM_COLS - 1) / MOE_ITEM_COLS;
+        }
+        int total, n_items;
+        int prefix = wave_excl_scan(c_sum, lane, &total);
+        int n = wave_excl_scan(i_sum, lane, &n_items);
+        for (int e = e0; e < e1; ++e) {
+            const int c = counts[e];
+            counts[e] = prefix;  // from here on: start of the expert's segment
             for (int j = 0; j < c; j += MOE_ITEM_COLS) {
                 a.items[n++] = make_int4(e, prefix + j, (c - j) < MOE_ITEM_COLS ? (c - j) : MOE_ITEM_COLS, 0);
             }
             prefix += c;
-        };
-        if (a.decode_order) {
-            // first-appearance order over routes in token-then-slot order; counts[] doubles as "seen" marker
-            for (int r = 0; r < routes; ++r) {
-                const int id = a.topk_ids[r];
-                if (id < 0 || id >= a.E || counts[id] <= 0) {
-                    continue;
-                }
-                place(id);
-                counts[id] = -counts[id];
-            }
-            for (int e = 0; e < a.E; ++e) {
-                counts[e] = counts[e] < 0 ? -counts[e] : counts[e];
-            }
-        } else {
-            for (int e = 0; e < a.E; ++e) {
-                if (counts[e] != 0) {
-                    place(e);
-                }
-            }
         }
-        *a.n_items = n;
+        if (lane == 0) {
+            *a.n_items = n_items;
+        }
     }
     __syncthreads();
-    // stable fill by the first wavefront, 64 routes per round in route order
-    const int lane = tid & 63;
-    for (int base = 0; base < routes; base += 64) {
-        if (tid < 64) {
-            const int r = base + lane;
-            int id = -1;
-            if (r < routes) {
+    // cursor of chunk w for expert e: segment start + routes of e in earlier chunks
+    for (int e = tid; e < a.E; e += blockDim.x) {
+        int run = counts[e];
+#pragma unroll
+        for (int w = 0; w < MOE_ROUTE_WAVES; ++w) {
+            const int c = wcount[w][e];
+            wcount[w][e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    // Stable fill, every wavefront over its own chunk, 64 routes per round in route order: a route's position is its
+    // expert's cursor plus the number of earlier lanes of the round with the same expert.
+    int *cursor = wcount[wave];
+    for (int base = r_begin; base < r_end; base += 64) {
+        const int r = base + lane;
+        int id = -1;
+        if (r < r_end) {
+            if (in_lds) {
+                id = ids_l[r];
+            } else {
                 id = a.topk_ids[r];
                 if (id < 0 || id >= a.E) {
                     id = -1;
                 }
             }
-            int rank = 0, cnt = 0;
-#pragma unroll
-            for (int j = 0; j < 64; ++j) {
-                const int idj = __builtin_amdgcn_readlane(id, j);
-                const bool same = idj == id;
-                cnt += same ? 1 : 0;
-                rank += (same && j < lane) ? 1 : 0;
-            }
-            if (id >= 0) {
-                const int pos = cursor[id] + rank;
-                const int t = r / a.k;
-                float norm = a.weights_scale;
-                if (a.renormalize) {
-                    float wsum = 0.0f;
-                    for (int s = 0; s < a.k; ++s) {
-                        wsum += a.topk_weights[t * a.k + s];
-                    }
-                    norm = wsum > FLT_MIN ? a.weights_scale / wsum : 0.0f;
-                }
-                a.sorted_tokens[pos] = (uint32_t)t;
-                a.sorted_weights[pos] = a.topk_weights[r] * norm;
-                a.route_pos[r] = pos;
-            } else if (r < routes) {
-                a.route_pos[r] = -1;
-            }
-            __builtin_amdgcn_s_waitcnt(0);  // this round's cursor reads are complete before the update below
-            if (id >= 0 && rank == cnt - 1) {
-                cursor[id] += cnt;
-            }
         }
-        __syncthreads();
+        int rank, cnt;
+        wave_rank(id, lane, &rank, &cnt);
+        int pos = -1;
+        if (id >= 0) {
+            pos = cursor[id] + rank;
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // this round's cursor reads are complete before the update below
+        if (id >= 0 && rank == cnt - 1) {
+            cursor[id] += cnt;
+        }
+        if (r < r_end) {
+            route_emit(a, r, pos);
+        }
     }
 }
 
@@ -203,11 +322,16 @@ __global__ __launch_bounds__(256) void k_moe_combine(const float *__restrict__ r
     __shared__ int pos[MOE_MAX_TOPK];
     __shared__ float wts[MOE_MAX_TOPK];
     __shared__ int npos;
+    __shared__ int raw[MOE_MAX_TOPK];
     const size_t t = blockIdx.x;
+    if ((int)threadIdx.x < k) {
+        raw[threadIdx.x] = route_pos[t * k + threadIdx.x];
+    }
+    __syncthreads();
     if (threadIdx.x == 0) {
         int n = 0;
         for (int s = 0; s < k; ++s) {
-            const int p = route_pos[t * k + s];
+            const int p = raw[s];
             if (p < 0) {
                 continue;
             }
@@ -218,14 +342,17 @@ __global__ __launch_bounds__(256) void k_moe_combine(const float *__restrict__ r
             }
             pos[j] = p;
         }
-        for (int j = 0; j < n; ++j) {
-            wts[j] = sorted_weights[pos[j]];
-        }
         npos = n;
     }
     __syncthreads();
+    if ((int)threadIdx.x < npos) {
+        wts[threadIdx.x] = sorted_weights[pos[threadIdx.x]];
+    }
+    __syncthreads();
     const int n = npos;
-    for (size_t h = threadIdx.x; h < H; h += blockDim.x) {
+    // blockIdx.y selects a slab of 256 columns
+    const size_t h = (size_t)blockIdx.y * blockDim.x + threadIdx.x;
+    if (h < H) {
         float acc = 0.0f;
         for (int j = 0; j < n; ++j) {
             acc += wts[j] * route_down[(size_t)pos[j] * H + h];
@@ -258,7 +385,7 @@ int marmot_hip_topk(marmot_hip_device_t *dev, const float *d_x, size_t rows, siz
     if (rows == 0) {
         return MARMOT_HIP_SUCCESS;
     }
-    hipLaunchKernelGGL(k_topk, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, dev->stream, d_x, rows, cols, k,
+    hipLaunchKernelGGL(k_topk, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, dev->stream, d_x, rows, cols, k,
                        d_values, d_indices);
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
@@ -346,16 +473,10 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
     float *sorted_weights = (float *)(base + o_weights);
     int *route_pos = (int *)(base + o_pos);
     int4 *items = (int4 *)(base + o_items);
-    int *flags = (int *)(base + o_flags);  // [0] = number of items, [1] = error flag
+    int *flags = (int *)(base + o_flags);  // [0] = number of items, [1] = error flag; both set by the route kernel
     float *gate_out = (float *)(base + o_gate);
     float *up_out = (float *)(base + o_up);
     float *route_down = (float *)(base + o_down);
-
-    extern int marmot_hip_fill_bytes_internal(marmot_hip_device_t *, void *, int, size_t);
-    st = marmot_hip_fill_bytes_internal(dev, flags, 0, 2 * sizeof(int));
-    if (st != MARMOT_HIP_SUCCESS) {
-        return st;
-    }
 
     RouteArgs ra;
     ra.topk_ids = d_topk_ids;
@@ -373,7 +494,7 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
     ra.renormalize = router_weight_policy == MARMOT_HIP_ROUTER_RENORMALIZE_SELECTED;
     // cpu_moe_should_use_decode_path (moe_ops.c:417-424)
     ra.decode_order = (T <= 4 && routes <= 64) ? 1 : 0;
-    hipLaunchKernelGGL(k_moe_route, dim3(1), dim3(256), 0, dev->stream, ra);
+    hipLaunchKernelGGL(k_moe_route, dim3(1), dim3(MOE_ROUTE_WAVES * 64), 0, dev->stream, ra);
     MH_HIP(hipGetLastError());
 
     // hidden states are quantized once per token; routes refer to them through sorted_tokens
@@ -383,8 +504,11 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
     }
     const size_t gu_stride = F * ((H + bv_gu - 1) / bv_gu) * block_bytes(kind_gate_up);
     const size_t dn_stride = H * ((F + bv_dn - 1) / bv_dn) * block_bytes(kind_down);
-    st = launch_matvec_grouped(dev, kind_gate_up, d_gate, d_up, gu_stride, hidden_q, sorted_tokens, items, flags,
-                               max_items, H, F, gate_out, up_out);
+    // Q4_K / Q6_K experts run on the int8 matrix cores, the 32-value formats on the dot-product matvec
+    const auto grouped_gu = mmq_grouped_supported(kind_gate_up, H) ? launch_mmq_grouped : launch_matvec_grouped;
+    const auto grouped_dn = mmq_grouped_supported(kind_down, F) ? launch_mmq_grouped : launch_matvec_grouped;
+    st = grouped_gu(dev, kind_gate_up, d_gate, d_up, gu_stride, hidden_q, sorted_tokens, items, flags, max_items, H, F,
+                    gate_out, up_out);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
@@ -392,13 +516,13 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
-    st = launch_matvec_grouped(dev, kind_down, d_down, nullptr, dn_stride, fused_q, nullptr, items, flags, max_items, F,
-                               H, route_down, nullptr);
+    st = grouped_dn(dev, kind_down, d_down, nullptr, dn_stride, fused_q, nullptr, items, flags, max_items, F, H,
+                    route_down, nullptr);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
-    hipLaunchKernelGGL(k_moe_combine, dim3((unsigned)T), dim3(256), 0, dev->stream, route_down, sorted_weights,
-                       route_pos, (int)k_per_token, H, d_out);
+    hipLaunchKernelGGL(k_moe_combine, dim3((unsigned)T, (unsigned)((H + 255) / 256)), dim3(256), 0, dev->stream,
+                       route_down, sorted_weights, route_pos, (int)k_per_token, H, d_out);
     MH_HIP(hipGetLastError());
     set_route("moe_experts_grouped");
 

@@ -25,6 +25,27 @@ def test_topk_reference_tie_case(hip):
     assert np.array_equal(idx, np.array([[1, 2, 3], [2, 3, 4]], dtype=np.int32))
 
 
+def test_topk_special_values(hip, oracle):
+    """Infinities, NaNs, -FLT_MAX (never selected: the list starts at -FLT_MAX and only strictly larger values go
+    in), k == cols, rows with fewer than k selectable values, a ragged column count."""
+    fmax = np.finfo(np.float32).max
+    x = np.array([[np.inf, 1, np.inf, -np.inf, np.nan, 1, -fmax, 0, 2, np.nan, -1],
+                  [np.nan, np.nan, -np.inf, -fmax, -np.inf, np.nan, -fmax, 7, np.nan, 7, -np.inf],
+                  [-np.inf] * 11,
+                  [0, -0.0, 0, -0.0, 5, 5, 5, -3, -3, 1e-45, -1e-45]], dtype=np.float32)
+    for k in (1, 4, 11):
+        v, i = hip.topk(x, k)
+        ov, oi = oracle.topk(x, k)
+        assert np.array_equal(i, oi), (k, i, oi)
+        assert np.array_equal(v.view(np.uint32), ov.view(np.uint32)), (k, v, ov)
+    assert i[2].tolist() == [-1] * 11 and np.all(v[2] == -fmax)
+    rng = np.random.default_rng(11)
+    x = rng.integers(-3, 4, size=(9, 333)).astype(np.float32)
+    v, i = hip.topk(x, 40)
+    ov, oi = oracle.topk(x, 40)
+    assert np.array_equal(i, oi) and np.array_equal(v, ov)
+
+
 def test_topk_and_softmax_match_oracle(hip, oracle):
     rng = np.random.default_rng(7)
     x = rng.integers(-4, 5, size=(130, 128)).astype(np.float32)
@@ -52,6 +73,22 @@ def test_moe_small(hip, oracle, kind_gu, kind_dn, T):
     ref = oracle.moe_experts(hidden, gate, up, down, ids, w, F, E, kind_gu, kind_dn, threads=8)
     got = hip.moe_experts(hidden, gate, up, down, ids, w, F, E, kind_gu, kind_dn)
     assert_moe_parity(got, ref, what=f"moe T={T}")
+
+
+@pytest.mark.parametrize("T", [200, 1400])
+def test_moe_many_routes(hip, oracle, T):
+    """Route sort over several chunks of routes (one per wavefront), below and above the number of routes whose ids
+    fit in LDS (4096); every expert gets many work items."""
+    print(f"moe many routes T={T}", flush=True)
+    E, F, H, k = 7, 256, 256, 3
+    kind = KIND_Q4_K
+    gate, up, down = make_experts(oracle, 430, E, F, H, kind, kind)
+    hidden = gaussian(431 + T, (T, H))
+    vals, ids = oracle.topk(gaussian(432 + T, (T, E)), k)
+    w = oracle.softmax_rows(vals)
+    ref = oracle.moe_experts(hidden, gate, up, down, ids, w, F, E, kind, kind, threads=8)
+    got = hip.moe_experts(hidden, gate, up, down, ids, w, F, E, kind, kind)
+    assert_moe_parity(got, ref, what=f"moe many routes T={T}")
 
 
 def test_moe_policies_duplicates_unrouted_and_errors(hip, oracle):

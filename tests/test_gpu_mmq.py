@@ -1,0 +1,156 @@
+"""GPU parity, part 2b: the small-batch matmul on the int8 matrix cores (Q4_K from 3 activation rows, Q6_K from 5)
+against the CPU oracle, through the C ABI: every pass shape (up to 8 / up to 16 rows per pass, several passes), ragged
+row groups, K split over wavefronts and over workgroups (partials + ordered reduction), bias and fp16 epilogues, the
+dual-output call, the prepacked-activation entry point and graph replay."""
+import numpy as np
+import pytest
+
+from marmot_amd import capi
+from oracle.pyoracle import KIND_Q4_K, KIND_Q6_K
+from tests.util import assert_matmul_parity, bits, gaussian, random_valid_blocks
+
+pytestmark = pytest.mark.gpu
+
+KINDS = {"q4_k": KIND_Q4_K, "q6_k": KIND_Q6_K}
+MIN_ROWS = {"q4_k": 3, "q6_k": 5}
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from marmot_amd import HipBackend
+
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+def test_route_threshold(hip, oracle, name):
+    """Below the threshold the fused matvec runs, from it on the MFMA kernel; both agree with the oracle."""
+    kind = KINDS[name]
+    M, K = 64, 1024
+    blocks = oracle.quantize(kind, gaussian(300, (M, K), 0.02))
+    for N in range(1, 8):
+        x = gaussian(301 + N, (N, K))
+        got = hip.linear(x, blocks, kind, M)
+        route = hip.last_route()
+        assert ("mmq_" in route) == (N >= MIN_ROWS[name]), (N, route)
+        assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what=f"{name} N={N} {route}")
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+def test_single_block_is_bit_exact(hip, oracle, name):
+    """K = 256: one block per row, so no fp32 reassociation is left and the exact integer block dots must give the
+    oracle's bits (same expression: (a.d * w.d) * isum - (a.d * w.dmin) * msum)."""
+    kind = KINDS[name]
+    M, K = 77, 256
+    rng = np.random.default_rng(310)
+    blocks = random_valid_blocks(rng, kind, M, K)
+    for N in (5, 8, 16, 21):
+        x = gaussian(311 + N, (N, K))
+        got = hip.linear(x, blocks, kind, M)
+        assert "mmq_" in hip.last_route()
+        ref = oracle.matmul(kind, blocks, x, M)
+        assert np.array_equal(bits(got), bits(ref)), f"{name} N={N}"
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("N", [5, 8, 9, 16, 17, 33, 40])
+def test_pass_shapes_and_ragged_row_groups(hip, oracle, name, N):
+    """Passes of up to 16 rows (the last one partial), 4- and 8-register accumulators, M not a multiple of 32."""
+    kind = KINDS[name]
+    M, K = 32 * 9 + 13, 2048
+    blocks = oracle.quantize(kind, gaussian(320, (M, K), 0.02))
+    x = gaussian(321 + N, (N, K))
+    got = hip.linear(x, blocks, kind, M)
+    assert "mmq_" in hip.last_route()
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what=f"{name} N={N}")
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K", [(40, 256 * 3), (64, 14336), (200, 256 * 23), (1024, 256 * 9)])
+def test_k_split_over_wavefronts_and_workgroups(hip, oracle, name, M, K):
+    """Few row groups and long rows: K is split over workgroups (fp32 partials, reduced in split order); block counts
+    that do not divide evenly leave some wavefronts with fewer (or no) blocks."""
+    kind = KINDS[name]
+    blocks = oracle.quantize(kind, gaussian(330, (M, K), 0.02))
+    for N in (6, 13):
+        x = gaussian(331 + N, (N, K))
+        got = hip.linear(x, blocks, kind, M)
+        assert "mmq_" in hip.last_route()
+        assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what=f"{name} {M}x{K} N={N}")
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K", [(96, 1024), (64, 14336)])
+def test_bias_and_fp16_epilogues(hip, oracle, name, M, K):
+    """Bias on the direct store and after the split-K reduction; fp16 activations forced through the packed path with
+    fp16 output: the dot is rounded to fp16 first, then the bias is added to the stored value."""
+    kind = KINDS[name]
+    N = 7
+    blocks = oracle.quantize(kind, gaussian(340, (M, K), 0.02))
+    x = gaussian(341, (N, K))
+    bias = gaussian(342, (M,))
+    ref = oracle.matmul(kind, blocks, x, M, bias=bias)
+    got = hip.linear(x, blocks, kind, M, bias=bias)
+    assert "mmq_" in hip.last_route()
+    assert np.max(np.abs(got - ref)) <= 1e-3 * np.abs(ref).max()
+    x16 = x.astype(np.float16)
+    bias16 = bias.astype(np.float16)
+    ref16 = oracle.matmul(kind, blocks, x16, M, bias=bias16, out_dtype=np.float16, force_pack=True)
+    got16 = hip.linear(x16, blocks, kind, M, bias=bias16, out_dtype=np.float16, force_pack=True)
+    assert "mmq_" in hip.last_route()
+    assert np.max(np.abs(got16.astype(np.float32) - ref16.astype(np.float32))) <= \
+        2e-3 * np.abs(ref16.astype(np.float32)).max()
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K", [(96, 2048), (64, 14336)])
+def test_dual_output_equals_two_singles(hip, oracle, name, M, K):
+    kind = KINDS[name]
+    N = 9
+    a = oracle.quantize(kind, gaussian(350, (M, K), 0.02))
+    b = oracle.quantize(kind, gaussian(351, (M, K), 0.02))
+    x = gaussian(352, (N, K))
+    oa, ob = hip.linear_dual(x, a, b, kind, M)
+    assert "mmq_" in hip.last_route()
+    assert np.array_equal(bits(oa), bits(hip.linear(x, a, kind, M)))
+    assert np.array_equal(bits(ob), bits(hip.linear(x, b, kind, M)))
+    assert_matmul_parity(oa, oracle.matmul(kind, a, x, M), what=f"{name} dual a")
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+def test_prepacked_activations_and_graph_replay(hip, oracle, name):
+    """Activations packed once (Q8_K rows) and reused; the captured matmul replays to the same bits each time, with
+    other work and synchronizations between the replays."""
+    kind = KINDS[name]
+    M, K, N = 320, 14336, 8
+    blocks = oracle.quantize(kind, gaussian(360, (M, K), 0.02))
+    x = gaussian(361, (N, K))
+    ref = oracle.matmul(kind, blocks, x, M)
+    d_w = hip.to_device(blocks)
+    d_x = hip.to_device(x)
+    d_p = hip.alloc(hip.packed_activation_bytes(kind, N, K))
+    d_out = hip.alloc(N * M * 4)
+    hip.pack_activations_d(kind, d_x, capi.DT_F32, N, K, d_p)
+    hip.linear_prepacked_d(kind, d_w, d_p, N, K, M, d_out)
+    assert "mmq_" in hip.last_route()
+    eager = d_out.download(np.float32, (N, M))
+    assert_matmul_parity(eager, ref, what=f"{name} prepacked")
+    fused = hip.linear(x, blocks, kind, M)
+    assert np.array_equal(bits(eager), bits(fused))
+
+    g = hip.graph_capture(lambda: hip.linear_d(kind, d_w, d_x, capi.DT_F32, N, K, M, d_out, capi.DT_F32))
+    try:
+        for rep in range(3):
+            d_out.upload(np.full(N * M * 4, 0xFF, dtype=np.uint8))
+            hip.graph_launch(g)
+            hip.synchronize()
+            got = d_out.download(np.float32, (N, M))
+            assert np.array_equal(bits(got), bits(eager)), f"{name} replay {rep}"
+            other = hip.linear(gaussian(370 + rep, (3, 256)), blocks[:, : blocks.shape[1] // (K // 256)].copy(), kind, M)
+            assert other.shape == (3, M)
+    finally:
+        hip.graph_destroy(g)
+        for b in (d_w, d_x, d_p, d_out):
+            b.free()

@@ -163,7 +163,7 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int):
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5")):
     """Every configuration of BASELINE.json on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
@@ -193,18 +193,29 @@ def sweep(hip, steps: int, warmup: int):
         for b in (d_w, d_x, d_out):
             b.free()
 
-    linear_case("C1", capi.KIND_Q8_0, 5632, 2048, 1)
+    if "C1" in only:
+        linear_case("C1", capi.KIND_Q8_0, 5632, 2048, 1)
     for kind in (capi.KIND_Q4_K, capi.KIND_Q6_K):
         for (M, K) in ((14336, 4096), (4096, 14336)):
             for N in (1, 4, 8):
-                linear_case("C2", kind, M, K, N)
-    for tokens in (64, 128, 512, 2048):
+                if "C2" in only:
+                    linear_case("C2", kind, M, K, N)
+    for tokens in (64, 128, 512, 2048) if "C3" in only else ():
         r = prefill_gemm(hip, tokens, max(20, steps // 20), 5)
         emit({"config": "C3", "workload": f"Q4_K 4096x4096 N={tokens} fp16", "route": r["route"],
               "us": round(r["ms_per_step"] * 1e3, 2), "TFLOP/s": r["tflops"],
               "frac_of_mfma_peak": r["frac_of_mfma_peak"], "tokens_per_s": round(r["tokens_per_s"])})
 
-    # C4: the seven linears of one layer at 16 tokens; 4 copies of the 139 MB of weights rotate
+    if "C4" in only:
+        sweep_layer_stack(hip, rng, emit, steps)
+    if "C5" in only:
+        sweep_moe(hip, rng, emit, steps)
+
+
+def sweep_layer_stack(hip, rng, emit, steps: int):
+    """C4: the seven linears of one layer at 16 tokens; 4 copies of the 139 MB of weights rotate."""
+    from marmot_amd import DT_F32, capi, row_bytes
+
     N = 16
     specs = [(capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 1024, 4096), (capi.KIND_Q6_K, 1024, 4096),
              (capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 14336, 4096), (capi.KIND_Q4_K, 14336, 4096),
@@ -236,7 +247,11 @@ def sweep(hip, steps: int, warmup: int):
         for b in (d_w, d_x, d_out):
             b.free()
 
-    # C5: 128 experts, top-8, hidden 2048, expert FFN 768, 64 tokens, all Q4_K; 2 copies of the 340 MB rotate
+
+def sweep_moe(hip, rng, emit, steps: int):
+    """C5: 128 experts, top-8, hidden 2048, expert FFN 768, 64 tokens, all Q4_K; 2 copies of the 340 MB rotate."""
+    from marmot_amd import capi, row_bytes
+
     E, k, H, F, T = 128, 8, 2048, 768, 64
     kind = capi.KIND_Q4_K
     gu_bytes = E * F * row_bytes(kind, H)
@@ -280,6 +295,7 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=512)
     ap.add_argument("--sweep", action="store_true",
                     help="measure every BASELINE configuration instead, one JSON line each (documentation runs)")
+    ap.add_argument("--configs", default="C1,C2,C3,C4,C5", help="with --sweep: the configurations to run")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")
     args = ap.parse_args()
@@ -305,7 +321,7 @@ def main():
 
     if args.sweep:
         hip = HipBackend(0)
-        sweep(hip, args.steps, args.warmup)
+        sweep(hip, args.steps, args.warmup, tuple(args.configs.split(",")))
         hip.close()
         return
 

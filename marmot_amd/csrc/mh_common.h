@@ -159,7 +159,7 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 // small-batch int8-MFMA matmul (mh_mmq.hip)
 bool mmq_supported(int kind, size_t N, size_t K);
-size_t mmq_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, bool dual);
+size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, bool dual);
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);

@@ -214,7 +214,7 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
-    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, N, K, M, d_w1 != nullptr) : 0);
+    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr) : 0);
     void *ws = nullptr;
     int st = workspace_reserve(dev, need, &ws);
     if (st != MARMOT_HIP_SUCCESS) {

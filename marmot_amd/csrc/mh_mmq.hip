@@ -12,10 +12,9 @@
 // sub-blocks. All integer results are exact; only the fp32 accumulation over blocks is ordered differently from the
 // CPU (per wavefront sequential, then across the K-split in a fixed order).
 //
-// A wavefront owns 32 weight rows and a contiguous range of blocks; W wavefronts of a workgroup and S workgroups
-// split K so that the chip is filled even when M / 32 is small. Weights stream from HBM exactly once per pass
-// (20 bytes x 5 loads per lane and block, two blocks in flight); activations (int8, L2-resident) are read straight
-// into operand registers.
+// A consumer wavefront owns 32 weight rows and a contiguous range of blocks; W of them per workgroup and S workgroups
+// split K so that the chip is filled even when M / 32 is small. Weights stream from HBM exactly once per pass, as
+// direct-to-LDS loads; activations (int8, L2-resident) take the same way into the same stage.
 #include "mh_common.h"
 
 #include <stdlib.h>
@@ -52,26 +51,42 @@ typedef const __attribute__((address_space(1))) uint8_t glb_u8;
 constexpr int MMQ_TOK = 16;                // activation rows per pass
 constexpr int MMQ_WBLK = 32 * Q4_K_BYTES;  // one block of 32 weight rows: 4608 bytes
 constexpr int MMQ_ABLK = MMQ_TOK * QK_K;   // one block of 16 activation rows: 4096 bytes
-constexpr int MMQ_STAGE = MMQ_WBLK + MMQ_ABLK + MMQ_TOK * 4;  // + the 16 activation scales of the block
-constexpr int MMQ_STAGES = 2;              // blocks in flight per wavefront
-constexpr int MMQ_STAGE_LOADS = 10;        // memory instructions per stage: 5 weights + 4 activations + 1 scales
+constexpr int MMQ_STAGES = 2;              // Q6_K: blocks in flight per wavefront
 
-// Work decomposition. All wavefronts of a workgroup work on the SAME 32 weight rows; wavefront w walks its own
+// ------------------------------------------------------------------ Q4_K x Q8_K
+// Work decomposition. All consumer wavefronts of a workgroup work on the SAME 32 weight rows; consumer w walks its own
 // contiguous range of blocks, so the workgroup as a whole streams whole weight rows (a decomposition in which a
-// workgroup covers many rows and a narrow K range measured 2.7x slower in HBM time for the same bytes). Every
-// wavefront has a private ring of stages in LDS, filled by direct-to-LDS loads: weights [32 rows][144 B] (9 chunks
-// per row: 16-byte reads of consecutive rows fall into different bank groups), activations [16 tokens][256 B] with
-// the 16-byte chunks XOR-swizzled by token, and the 16 activation scales. No workgroup barrier until the final
-// reduction over the K-split.
+// workgroup covers many rows and a narrow K range measured 2.7x slower in HBM time for the same bytes). Every consumer
+// has a private ring of stages in LDS, filled by direct-to-LDS loads: weights [32 rows][144 B] (9 chunks per row:
+// 16-byte reads of consecutive rows fall into different bank groups), activations [tokens][256 B] with the 16-byte
+// chunks XOR-swizzled by token, and the activation scales of the block.
 //
-// NR: live accumulator registers per lane: 4 for up to 8 activation rows, 8 for up to 16 (token of register r:
-// 8 * (r / 4) + 4 * kh + r % 4, the row layout of the 32x32 MFMA result).
-template <int NR>
-__global__ __launch_bounds__(512) void k_mmq_q4k(const MmqParams p) {
+// The wavefronts of a workgroup are specialised: W consumers only read LDS and run the matrix cores, one loader
+// issues every direct-to-LDS load of the workgroup. A wavefront that issues loads is held at the issue stage whenever
+// the memory queues of its CU are full, which under a saturated HBM is most of the time; with every wavefront loading
+// AND computing, the computation only ran in the gaps (measured with the cycle counter: the load phases and the
+// compute phases of a wavefront added up instead of overlapping). Here the loader absorbs those stalls. Steps are
+// separated by a bare s_barrier (no implied memory wait): in step t the loader issues block t of every consumer into
+// stage t % STAGES and waits until block t - (STAGES - 2) has landed, the consumers work on block t - (STAGES - 1).
+//
+// NR: live accumulator registers per lane: 4 for up to 8 activation rows (8 rows staged per block), 8 for up to 16
+// (token of register r: 8 * (r / 4) + 4 * kh + r % 4, the row layout of the 32x32 MFMA result).
+template <int NR, int STAGES>
+__global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
+    constexpr int TOK = 2 * NR;
+    constexpr int A_OFF = MMQ_WBLK, D_OFF = A_OFF + TOK * QK_K, STAGE = D_OFF + TOK * 4;
+    constexpr int A_LOADS = TOK / 4;           // 16-byte chunks of the activation tile / 64 lanes
+    constexpr int LOADS = 5 + A_LOADS + 1;     // memory instructions per stage
+    constexpr int AHEAD = STAGES - 1;          // blocks the loader runs ahead of the consumers
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
+    const bool loader = wave == W;
+    // the kernel arguments span three cache lines that would otherwise be fetched one after the other, each on first
+    // use; touching them together at the start costs one scalar-cache miss instead of three
+    const uint32_t __attribute__((address_space(4))) *kargs =
+        (const uint32_t __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr();
+    const uint32_t warm = kargs[0] ^ kargs[16] ^ kargs[32] ^ kargs[sizeof(MmqParams) / 4 - 1];
     const int j = lane & 31, kh = lane >> 5;
-    // blockIdx.y = K-split index, interleaved with the weight selector of a dual call
     const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
     const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
     const uint8_t *wbase = p.w[which];
@@ -79,88 +94,25 @@ __global__ __launch_bounds__(512) void k_mmq_q4k(const MmqParams p) {
     int ncols = p.ncols;
     if (p.items != nullptr) {
         if ((int)blockIdx.z >= *p.n_items) {
-            return;  // uniform for the whole workgroup
+            return;  // uniform for the whole workgroup, before any barrier
         }
         const int4 it = p.items[blockIdx.z];
         wbase += (size_t)it.x * p.expert_stride;
         n0 = (size_t)it.y;
         ncols = it.z;
     }
-    const size_t b0 = ((size_t)split * W + wave) * p.bpw;
-    size_t b1 = b0 + p.bpw;
-    if (b1 > p.nb) {
-        b1 = p.nb;
-    }
-    const int nblk = b1 > b0 ? (int)(b1 - b0) : 0;
-    uint8_t *ring = lds + (size_t)wave * MMQ_STAGES * MMQ_STAGE;
-
-    // ---- per-lane source offsets of the direct-to-LDS loads (block-independent)
     const size_t row0 = (size_t)blockIdx.x * 32;
-    uint32_t w_off[5];  // weights: 288 chunks of 16 bytes in row order (9 per row)
-#pragma unroll
-    for (int c = 0; c < 5; ++c) {
-        const int chunk = c * 64 + lane;
-        int row = chunk / 9;
-        const int piece = chunk - row * 9;
-        if (row > 31) {
-            row = 31;
+    const int steps = p.bpw + AHEAD;  // the same for every wavefront of the workgroup
+    // blocks [b0, b0 + nblk) of consumer w
+    auto first_block = [&](int w) { return ((size_t)split * W + w) * p.bpw; };
+    auto block_count = [&](int w) {
+        const size_t b0 = first_block(w);
+        size_t b1 = b0 + p.bpw;
+        if (b1 > p.nb) {
+            b1 = p.nb;
         }
-        size_t m = row0 + row;
-        if (m >= p.M) {
-            m = p.M - 1;  // harmless re-read; never stored
-        }
-        w_off[c] = (uint32_t)((m - row0) * p.nb * Q4_K_BYTES + 16 * piece);
-    }
-    const uint8_t *wgroup = wbase + row0 * p.nb * Q4_K_BYTES;
-    uint32_t a_off[4];  // activations: 256 chunks, chunk (token, slot) holds source chunk slot ^ token
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const int chunk = c * 64 + lane;
-        const int slot = chunk & 15, tk = chunk >> 4;
-        const int tt = tk < ncols ? tk : 0;  // rows beyond ncols re-read the first row; their results are not stored
-        const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
-        a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
-    }
-    uint32_t ad_off;
-    {
-        const int tk = lane & 15;
-        const int tt = tk < ncols ? tk : 0;
-        const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
-        ad_off = (uint32_t)(arow * p.nb);
-    }
-    auto stage_block = [&](size_t b, uint8_t *dst) {
-#pragma unroll
-        for (int c = 0; c < 5; ++c) {
-            if (c < 4 || lane < 32) {  // 288 = 4 * 64 + 32 chunks
-                __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + b * Q4_K_BYTES),
-                                                 (lds_u8 *)(dst + c * 1024), 16, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            __builtin_amdgcn_global_load_lds((glb_u8 *)(p.qs + a_off[c] + b * QK_K),
-                                             (lds_u8 *)(dst + MMQ_WBLK + c * 1024), 16, 0, 0);
-        }
-        if (lane < MMQ_TOK) {
-            __builtin_amdgcn_global_load_lds((glb_u8 *)(p.ad + ad_off + b), (lds_u8 *)(dst + MMQ_WBLK + MMQ_ABLK), 4,
-                                             0, 0);
-        }
+        return b1 > b0 ? (int)(b1 - b0) : 0;
     };
-    // memory loads complete in order: waiting until at most one stage's loads are outstanding means the older stage
-    // has landed
-    auto wait_all_but = [&](int stages) {
-        if (stages >= 1) {
-            __builtin_amdgcn_s_waitcnt(0x0f70 | MMQ_STAGE_LOADS);
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0f70);
-        }
-    };
-#pragma unroll
-    for (int st = 0; st < MMQ_STAGES; ++st) {
-        if (st < nblk) {
-            stage_block(b0 + st, ring + st * MMQ_STAGE);
-        }
-    }
 
     float acc[NR];
     int tok[NR];
@@ -169,111 +121,217 @@ __global__ __launch_bounds__(512) void k_mmq_q4k(const MmqParams p) {
         acc[r] = 0.0f;
         tok[r] = 8 * (r >> 2) + 4 * kh + (r & 3);
     }
-    // MFMA row operand of this lane: token j % 16 (rows 16..31 of the product repeat rows 0..15 and are ignored),
-    // chunk 2 * sb + kh of the block, stored at slot chunk ^ token
-    const int ti = j & 15;
 
-    for (int blk = 0; blk < nblk; ++blk) {
-        wait_all_but(nblk - 1 - blk >= 1 ? 1 : 0);
-        const uint8_t *stage = ring + (blk % MMQ_STAGES) * MMQ_STAGE;
-        const uint8_t *wcur = stage + j * Q4_K_BYTES;
-        const uint8_t *a_blk = stage + MMQ_WBLK + ti * QK_K;
-        const float *ad_blk = (const float *)(stage + MMQ_WBLK + MMQ_ABLK);
-        // all LDS operands of the block are requested up front, so that no LDS latency sits inside the MFMA chain
-        const uint4 hdr = *(const uint4 *)wcur;
-        uint4 aq[8], wq4[4];
+    if (loader) {
+        // ---- per-lane source offsets (block-independent)
+        uint32_t w_off[5];  // weights: 288 chunks of 16 bytes in row order (9 per row)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            wq4[g] = *(const uint4 *)(wcur + 16 + 32 * g + 16 * kh);
-        }
-#pragma unroll
-        for (int sb = 0; sb < 8; ++sb) {
-            aq[sb] = *(const uint4 *)(a_blk + 16 * ((2 * sb + kh) ^ ti));
-        }
-        float adr[NR];
-#pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            adr[r] = ad_blk[tok[r]];
-        }
-        // the stage is refilled with block blk + MMQ_STAGES once its reads have returned
-        __builtin_amdgcn_sched_barrier(0);
-        if (blk + MMQ_STAGES < nblk) {
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-            stage_block(b0 + blk + MMQ_STAGES, ring + (blk % MMQ_STAGES) * MMQ_STAGE);
-        }
-        // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
-        const float d = h2f((uint16_t)(hdr.x & 0xffffu));
-        const float dmin = h2f((uint16_t)(hdr.x >> 16));
-        const uint32_t sc_lo = hdr.y & 0x3f3f3f3fu;
-        const uint32_t mn_lo = hdr.z & 0x3f3f3f3fu;
-        const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
-        const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
-        int bsum[NR];
-#pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            bsum[r] = 0;
-        }
-        auto acts_of = [&](int sb) {
-            return intx4{(int)aq[sb].x, (int)aq[sb].y, (int)aq[sb].z, (int)aq[sb].w};
-        };
-        auto weights_of = [&](int sb) {
-            const uint4 wq = wq4[sb >> 1];
-            if (sb & 1) {
-                return intx4{(int)((wq.x >> 4) & 0x0f0f0f0fu), (int)((wq.y >> 4) & 0x0f0f0f0fu),
-                             (int)((wq.z >> 4) & 0x0f0f0f0fu), (int)((wq.w >> 4) & 0x0f0f0f0fu)};
+        for (int c = 0; c < 5; ++c) {
+            const int chunk = c * 64 + lane;
+            int row = chunk / 9;
+            const int piece = chunk - row * 9;
+            if (row > 31) {
+                row = 31;
             }
-            return intx4{(int)(wq.x & 0x0f0f0f0fu), (int)(wq.y & 0x0f0f0f0fu), (int)(wq.z & 0x0f0f0f0fu),
-                         (int)(wq.w & 0x0f0f0f0fu)};
-        };
-        const intx16 zero = {0};
-        intx16 dm = {0};
-        intx16 dq[2];
-        dq[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(0), weights_of(0), zero, 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int sb = 0; sb < 8; ++sb) {
-            const int sc = (int)(((sb < 4 ? sc_lo : sc_hi) >> (8 * (sb & 3))) & 0xffu);
-            const int mn = (int)(((sb < 4 ? mn_lo : mn_hi) >> (8 * (sb & 3))) & 0xffu);
-            const int mn4 = mn * 0x01010101;
-            dm = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb), intx4{mn4, mn4, mn4, mn4}, dm, 0, 0, 0);
-            if (sb < 7) {
-                dq[(sb + 1) & 1] =
-                    __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb + 1), weights_of(sb + 1), zero, 0, 0, 0);
+            size_t m = row0 + row;
+            if (m >= p.M) {
+                m = p.M - 1;  // harmless re-read; never stored
             }
-#pragma unroll
-            for (int r = 0; r < NR; ++r) {
-                bsum[r] += __mul24(dq[sb & 1][r], sc);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+            w_off[c] = (uint32_t)((m - row0) * p.nb * Q4_K_BYTES + 16 * piece);
         }
+        const uint8_t *wgroup = wbase + row0 * p.nb * Q4_K_BYTES;
+        uint32_t a_off[A_LOADS];  // activations: chunk (token, slot) holds source chunk slot ^ token
 #pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            acc[r] += (adr[r] * d) * (float)bsum[r] - (adr[r] * dmin) * (float)dm[r];
+        for (int c = 0; c < A_LOADS; ++c) {
+            const int chunk = c * 64 + lane;
+            const int slot = chunk & 15, tk = chunk >> 4;
+            const int tt = tk < ncols ? tk : 0;  // rows beyond ncols re-read the first row; never stored
+            const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+            a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
+        }
+        uint32_t ad_off;
+        {
+            const int tk = lane & (TOK - 1);
+            const int tt = tk < ncols ? tk : 0;
+            const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+            ad_off = (uint32_t)(arow * p.nb);
+        }
+        for (int t = 0; t < steps; ++t) {
+            if (t < p.bpw) {
+                for (int w = 0; w < W; ++w) {
+                    // a consumer with fewer blocks gets its last block again (never used): the number of loads per
+                    // step stays the same for the counted wait below
+                    const int nb_w = block_count(w);
+                    size_t b = first_block(w) + (t < nb_w ? t : (nb_w > 0 ? nb_w - 1 : 0));
+                    if (b >= p.nb) {
+                        b = p.nb - 1;
+                    }
+                    uint8_t *dst = lds + ((size_t)w * STAGES + (t % STAGES)) * STAGE;
+#pragma unroll
+                    for (int c = 0; c < 5; ++c) {
+                        if (c < 4 || lane < 32) {  // 288 = 4 * 64 + 32 chunks
+                            __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + b * Q4_K_BYTES),
+                                                             (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+                        }
+                    }
+#pragma unroll
+                    for (int c = 0; c < A_LOADS; ++c) {
+                        __builtin_amdgcn_global_load_lds((glb_u8 *)(p.qs + a_off[c] + b * QK_K),
+                                                         (lds_u8 *)(dst + A_OFF + c * 1024), 16, 0, 0);
+                    }
+                    if (lane < TOK) {
+                        __builtin_amdgcn_global_load_lds((glb_u8 *)(p.ad + ad_off + b), (lds_u8 *)(dst + D_OFF), 4, 0,
+                                                         0);
+                    }
+                }
+            }
+            // loads complete in order: block t - (AHEAD - 1) has landed once at most the loads of the AHEAD - 1 newer
+            // steps are outstanding
+            const int newer = t < p.bpw ? (AHEAD - 1) : (AHEAD - 1) - (t - p.bpw + 1);
+            const int allowed = newer > 0 ? newer * W * LOADS : 0;
+            if (allowed >= 60) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (60 & 15) | ((60 >> 4) << 14));
+            } else if (allowed >= 50) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (50 & 15) | ((50 >> 4) << 14));
+            } else if (allowed >= 40) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (40 & 15) | ((40 >> 4) << 14));
+            } else if (allowed >= 32) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (32 & 15) | ((32 >> 4) << 14));
+            } else if (allowed >= 24) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (24 & 15) | ((24 >> 4) << 14));
+            } else if (allowed >= 16) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | (16 & 15) | ((16 >> 4) << 14));
+            } else if (allowed >= 10) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | 10);
+            } else if (allowed >= 8) {
+                __builtin_amdgcn_s_waitcnt(0x0f70 | 8);
+            } else {
+                __builtin_amdgcn_s_waitcnt(0x0f70);
+            }
+            __builtin_amdgcn_s_barrier();
+        }
+    } else {
+        const int nblk = block_count(wave);
+        const uint8_t *ring = lds + (size_t)wave * STAGES * STAGE;
+        // MFMA row operand of this lane: token j % TOK (the other rows of the product repeat them and are ignored),
+        // chunk 2 * sb + kh of the block, stored at slot chunk ^ token
+        const int ti = j & (TOK - 1);
+        for (int t = 0; t < steps; ++t) {
+            const int blk = t - AHEAD;
+            if (blk >= 0 && blk < nblk) {
+                const uint8_t *stage = ring + (blk % STAGES) * STAGE;
+                const uint8_t *wcur = stage + j * Q4_K_BYTES;
+                const uint8_t *a_blk = stage + A_OFF + ti * QK_K;
+                const float *ad_blk = (const float *)(stage + D_OFF);
+                const uint4 hdr = *(const uint4 *)wcur;
+                uint4 aq[8], wq4[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    wq4[g] = *(const uint4 *)(wcur + 16 + 32 * g + 16 * kh);
+                }
+#pragma unroll
+                for (int sb = 0; sb < 8; ++sb) {
+                    aq[sb] = *(const uint4 *)(a_blk + 16 * ((2 * sb + kh) ^ ti));
+                }
+                float adr[NR];
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    adr[r] = ad_blk[tok[r] & (TOK - 1)];
+                }
+                // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
+                const float d = h2f((uint16_t)(hdr.x & 0xffffu));
+                const float dmin = h2f((uint16_t)(hdr.x >> 16));
+                const uint32_t sc_lo = hdr.y & 0x3f3f3f3fu;
+                const uint32_t mn_lo = hdr.z & 0x3f3f3f3fu;
+                const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
+                const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+                int bsum[NR];
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    bsum[r] = 0;
+                }
+                auto acts_of = [&](int sb) {
+                    return intx4{(int)aq[sb].x, (int)aq[sb].y, (int)aq[sb].z, (int)aq[sb].w};
+                };
+                auto weights_of = [&](int sb) {
+                    const uint4 wq = wq4[sb >> 1];
+                    if (sb & 1) {
+                        return intx4{(int)((wq.x >> 4) & 0x0f0f0f0fu), (int)((wq.y >> 4) & 0x0f0f0f0fu),
+                                     (int)((wq.z >> 4) & 0x0f0f0f0fu), (int)((wq.w >> 4) & 0x0f0f0f0fu)};
+                    }
+                    return intx4{(int)(wq.x & 0x0f0f0f0fu), (int)(wq.y & 0x0f0f0f0fu), (int)(wq.z & 0x0f0f0f0fu),
+                                 (int)(wq.w & 0x0f0f0f0fu)};
+                };
+                const intx16 zero = {0};
+                intx16 dm = {0};
+                intx16 dq[2];
+                dq[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(0), weights_of(0), zero, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int sb = 0; sb < 8; ++sb) {
+                    const int sc = (int)(((sb < 4 ? sc_lo : sc_hi) >> (8 * (sb & 3))) & 0xffu);
+                    const int mn = (int)(((sb < 4 ? mn_lo : mn_hi) >> (8 * (sb & 3))) & 0xffu);
+                    const int mn4 = mn * 0x01010101;
+                    dm = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb), intx4{mn4, mn4, mn4, mn4}, dm, 0, 0, 0);
+                    if (sb < 7) {
+                        dq[(sb + 1) & 1] =
+                            __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb + 1), weights_of(sb + 1), zero, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < NR; ++r) {
+                        bsum[r] += __mul24(dq[sb & 1][r], sc);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    acc[r] += (adr[r] * d) * (float)bsum[r] - (adr[r] * dmin) * (float)dm[r];
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this step's LDS reads are done before the stage is reused
+            __builtin_amdgcn_s_barrier();
         }
     }
 
-    // ---- K-split within the workgroup: partial sums meet in LDS and are added in wavefront order
+    // ---- K-split within the workgroup: partial sums meet in LDS and are added in wavefront order. The last barrier
+    // of the loop guarantees that every stage has been read.
     if (W > 1) {
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();  // every wavefront is done with its ring; the memory is reused for the reduction
         float *red = (float *)lds;
+        if (!loader) {
 #pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            red[(wave * NR + r) * 64 + lane] = acc[r];
+            for (int r = 0; r < NR; ++r) {
+                red[(wave * NR + r) * 64 + lane] = acc[r];
+            }
         }
-        __syncthreads();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();
         if (wave != 0) {
             return;
         }
+        // all partial sums are requested before the first addition (W <= 4); the additions stay in wavefront order
+        float part[4][NR];
+#pragma unroll
+        for (int w2 = 0; w2 < 4; ++w2) {
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                part[w2][r] = w2 < W ? red[(w2 * NR + r) * 64 + lane] : 0.0f;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < NR; ++r) {
-            float sum = red[r * 64 + lane];
-            for (int w2 = 1; w2 < W; ++w2) {
-                sum += red[(w2 * NR + r) * 64 + lane];
+            float sum = part[0][r];
+#pragma unroll
+            for (int w2 = 1; w2 < 4; ++w2) {
+                if (w2 < W) {
+                    sum += part[w2][r];
+                }
             }
             acc[r] = sum;
         }
+    } else if (loader) {
+        return;
     }
+    asm volatile("" ::"s"(warm));
     const size_t mm = row0 + j;
     if (mm >= p.M) {
         return;
@@ -561,12 +619,15 @@ struct MmqPlan {
     int W, S, bpw;
 };
 
-// W wavefronts per workgroup and S workgroups split K so that at least one workgroup per CU is resident
-static MmqPlan mmq_plan(const marmot_hip_device *dev, size_t M, size_t nb) {
+// W (consumer) wavefronts per workgroup and S workgroups split K so that at least one workgroup per CU is resident.
+// Q4_K with more than 8 activation rows stages 16 rows per block; two consumers per workgroup keep the LDS ring small
+// enough for three workgroups per CU.
+static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t M, size_t nb) {
     const size_t rg = (M + 31) / 32;
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     MmqPlan pl;
-    size_t W = nb < 4 ? nb : 4;
+    const size_t w_max = (kind == MARMOT_HIP_KIND_Q4_K && N > 8) ? 2 : 4;
+    size_t W = nb < w_max ? nb : w_max;
     size_t S = 1;
     while (rg * S < cus && W * S * 2 <= nb) {
         S *= 2;
@@ -585,14 +646,13 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, size_t M, size_t nb) {
 }
 
 // bytes of fp32 partials launch_mmq needs for this shape (0 when K is not split across workgroups)
-size_t mmq_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, bool dual) {
-    const MmqPlan pl = mmq_plan(dev, M, K / QK_K);
+size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, bool dual) {
+    const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K);
     return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (dual ? 2 : 1) : 0;
 }
 
-static size_t mmq_lds_bytes(int kind, int W) {
-    const size_t stage = kind == MARMOT_HIP_KIND_Q6_K ? (size_t)MMQ6_STAGE : (size_t)MMQ_STAGE;
-    const size_t ring = (size_t)W * MMQ_STAGES * stage;
+static size_t mmq6_lds_bytes(int W) {
+    const size_t ring = (size_t)W * MMQ_STAGES * MMQ6_STAGE;
     const size_t red = (size_t)W * 8 * 64 * sizeof(float);
     return ring > red ? ring : red;
 }
@@ -603,16 +663,33 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
     const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * (dual ? 2 : 1)), items);
     static bool attr_set = false;
     if (!attr_set) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)mmq_lds_bytes(MARMOT_HIP_KIND_Q4_K, 8)));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
         MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)mmq_lds_bytes(MARMOT_HIP_KIND_Q6_K, 6)));
+                                   (int)mmq6_lds_bytes(6)));
         attr_set = true;
     }
     if (kind == MARMOT_HIP_KIND_Q6_K) {
-        hipLaunchKernelGGL((k_mmq_q6k<NR>), grid, dim3(pl.W * 64), mmq_lds_bytes(kind, pl.W), dev->stream, p);
+        hipLaunchKernelGGL((k_mmq_q6k<NR>), grid, dim3(pl.W * 64), mmq6_lds_bytes(pl.W), dev->stream, p);
     } else {
-        hipLaunchKernelGGL((k_mmq_q4k<NR>), grid, dim3(pl.W * 64), mmq_lds_bytes(kind, pl.W), dev->stream, p);
+        // W consumers + 1 loader. Three stages (the loader two blocks ahead) for the dense call; the grouped call
+        // runs many small workgroups per CU, which overlap each other, and takes two to fit more of them.
+        if (pl.W < 1 || pl.W > 4) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "mmq: %d consumer wavefronts are not supported", pl.W);
+        }
+        const int stages = p.items != nullptr ? 2 : 3;
+        const size_t stage = MMQ_WBLK + 2 * NR * QK_K + 2 * NR * 4;
+        const size_t ring = (size_t)pl.W * stages * stage;
+        const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
+        const size_t lds_bytes = ring > red ? ring : red;
+        const dim3 block((pl.W + 1) * 64);
+        if (stages == 2) {
+            hipLaunchKernelGGL((k_mmq_q4k<NR, 2>), grid, block, lds_bytes, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL((k_mmq_q4k<NR, 3>), grid, block, lds_bytes, dev->stream, p);
+        }
     }
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
@@ -628,11 +705,11 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
     }
     const size_t nb = K / QK_K;
     const bool dual = d_w1 != nullptr;
-    const MmqPlan pl = mmq_plan(dev, M, nb);
+    const MmqPlan pl = mmq_plan(dev, kind, N, M, nb);
     float *partial = (float *)scratch;
     if (pl.S > 1 && partial == nullptr) {
         void *ws = nullptr;
-        int st = workspace_reserve(dev, mmq_scratch_bytes(dev, N, K, M, dual), &ws);
+        int st = workspace_reserve(dev, mmq_scratch_bytes(dev, kind, N, K, M, dual), &ws);
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
         }
@@ -683,8 +760,7 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
 }
 
 // Grouped (MoE): every work item is up to 8 consecutive routes of one expert; blockIdx.z walks the item list the
-// route kernel wrote (workgroups beyond *d_n_items exit at once). Expert matrices are small, so K is split over the
-// wavefronts of a workgroup only when a row is long enough to keep each of them busy for several blocks.
+// route kernel wrote (workgroups beyond *d_n_items exit at once).
 bool mmq_grouped_supported(int kind, size_t K) {
     return (kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && K % QK_K == 0 &&
            getenv("MARMOT_HIP_NO_MMQ") == nullptr;
@@ -705,16 +781,11 @@ int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     const size_t nb = K / QK_K;
     MmqPlan pl;
-    size_t W = nb >= 16 ? 4 : (nb >= 8 ? 2 : 1);
-    if (const char *e = getenv("MH_MMQ_GW")) {
-        W = (size_t)atoi(e);
-    }
-    if (W > nb) {
-        W = nb;
-    }
-    pl.W = (int)W;
+    // one consumer per workgroup walks the whole row: expert matrices are small and there are thousands of
+    // workgroups, which overlap each other's load and compute phases (2 or 4 consumers measured slower)
+    pl.W = 1;
     pl.S = 1;
-    pl.bpw = (int)((nb + W - 1) / W);
+    pl.bpw = (int)nb;
     MmqParams p;
     p.w[0] = (const uint8_t *)d_w0;
     p.w[1] = (const uint8_t *)d_w1;

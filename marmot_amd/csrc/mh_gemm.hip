@@ -139,6 +139,7 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t m, __half2 sc, __half2
 }
 
 __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) {
+    warm_kernel_arguments<sizeof(GemmParams)>();
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // 2 stages
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -424,6 +425,7 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
 template <int V>
 __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ partial, int splits, size_t N, size_t M,
                                                      const void *bias, int bias_is_f16, void *out, int out_is_f16) {
+    warm_kernel_arguments<8 * 8>();
     const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
     const size_t total = N * M;
     if (idx >= total) {

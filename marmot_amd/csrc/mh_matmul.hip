@@ -27,6 +27,7 @@ struct DirectParams {
 
 template <int KIND, int NC>
 __global__ __launch_bounds__(256) void k_matvec_direct_f16(const DirectParams p) {
+    warm_kernel_arguments<sizeof(DirectParams)>();
     constexpr int BV = KindTraits<KIND>::BV;
     constexpr int BB = KindTraits<KIND>::BB;
     const int lane = threadIdx.x & 63;

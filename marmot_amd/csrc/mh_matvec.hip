@@ -495,6 +495,7 @@ constexpr int matvec_max_threads() {
 template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
 __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void k_matvec(const MatvecParams p) {
     extern __shared__ float partial[];  // [rows_per_wg][NC][4 * W]: one partial per 16-lane row of each wavefront
+    warm_kernel_arguments<sizeof(MatvecParams)>();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;

@@ -81,11 +81,7 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
     const bool loader = wave == W;
-    // the kernel arguments span three cache lines that would otherwise be fetched one after the other, each on first
-    // use; touching them together at the start costs one scalar-cache miss instead of three
-    const uint32_t __attribute__((address_space(4))) *kargs =
-        (const uint32_t __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr();
-    const uint32_t warm = kargs[0] ^ kargs[16] ^ kargs[32] ^ kargs[sizeof(MmqParams) / 4 - 1];
+    warm_kernel_arguments<sizeof(MmqParams)>();
     const int j = lane & 31, kh = lane >> 5;
     const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
     const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
@@ -331,7 +327,6 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
     } else if (loader) {
         return;
     }
-    asm volatile("" ::"s"(warm));
     const size_t mm = row0 + j;
     if (mm >= p.M) {
         return;
@@ -377,6 +372,7 @@ constexpr int MMQ6_STAGE = MMQ6_WBLK + MMQ_ABLK + MMQ_TOK * 4;
 template <int NR>
 __global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    warm_kernel_arguments<sizeof(MmqParams)>();
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
     const int j = lane & 31, kh = lane >> 5;
     const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;

@@ -150,6 +150,26 @@ __device__ __forceinline__ void warm_kernel_arguments() {
     }
     asm volatile("" ::"s"(touched));
 }
+
+// s_waitcnt vmcnt(n) for a run-time n: the immediate must be a constant, and it must be the exact count (a smaller one
+// would also wait for loads of the newer steps, i.e. for a full memory latency)
+#define MH_VMCNT_CASE(n)                                                             \
+    case n:                                                                          \
+        __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14));        \
+        break;
+#define MH_VMCNT_CASE4(n) MH_VMCNT_CASE(n) MH_VMCNT_CASE(n + 1) MH_VMCNT_CASE(n + 2) MH_VMCNT_CASE(n + 3)
+#define MH_VMCNT_CASE16(n) MH_VMCNT_CASE4(n) MH_VMCNT_CASE4(n + 4) MH_VMCNT_CASE4(n + 8) MH_VMCNT_CASE4(n + 12)
+__device__ __forceinline__ void wait_vmcnt_at_most(int allowed) {
+    switch (allowed > 63 ? 63 : allowed) {
+        MH_VMCNT_CASE16(0)
+        MH_VMCNT_CASE16(16)
+        MH_VMCNT_CASE16(32)
+        MH_VMCNT_CASE16(48)
+    default:
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        break;
+    }
+}
 #endif
 
 // Returns a workspace of at least `bytes` (256-byte aligned). Growing it synchronizes the stream first.

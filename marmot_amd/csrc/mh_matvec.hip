@@ -18,6 +18,8 @@
 // cpu_vec_dot_{q4_k,q6_k}_q8_k / cpu_vec_dot_{q8_0,q4_0}_q8_0 (vec_dot_impl.h) up to summation order.
 #include "mh_common.h"
 
+#include <type_traits>
+
 #include <float.h>
 #include <stdlib.h>
 
@@ -77,13 +79,20 @@ __device__ __forceinline__ void ld16f(const float *p, float *v) {
 // Q8_K quantization (matmul_quant_pack.c:106-142) of one 256-value block whose values are spread over LPB
 // adjacent lanes: this lane owns RUNS runs of 16 consecutive values starting at block offsets off[r].
 // Produces this lane's int8 values (RUNS uint4), the sums of each run (= bsums entries) and the block scale d.
-template <int RUNS, int LPB>
+// SIGNAL: a workgroup barrier right after the loads have been issued (not returned); a loader wavefront waits on it
+// so that its own, much larger, requests queue up behind these.
+template <int RUNS, int LPB, bool SIGNAL = false>
 __device__ __forceinline__ void q8k_quantize_runs(const float *xblk, const int (&off)[RUNS], uint4 (&q)[RUNS],
                                                   int (&bs)[RUNS], float &d) {
     float v[RUNS][16];
 #pragma unroll
     for (int r = 0; r < RUNS; ++r) {
         ld16f(xblk + off[r], v[r]);
+    }
+    if (SIGNAL) {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
     }
     float best_abs = 0.0f, best_val = 0.0f;
     int best_idx = 0x7fffffff;
@@ -193,12 +202,13 @@ struct FmtQ4K {
         a.bs_lo = bs[4 * g + h];
         a.bs_hi = bs[4 * g + 2 + h];
     }
+    template <bool SIGNAL = false>
     __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
         const int g = sub >> 1, h = sub & 1;
         const int off[2] = {64 * g + 16 * h, 64 * g + 32 + 16 * h};
         uint4 q[2];
         int bs[2];
-        q8k_quantize_runs<2, 8>(xrow + blk * QK_K, off, q, bs, a.d);
+        q8k_quantize_runs<2, 8, SIGNAL>(xrow + blk * QK_K, off, q, bs, a.d);
         a.lo = q[0];
         a.hi = q[1];
         a.bs_lo = bs[0];
@@ -619,6 +629,202 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
     }
 }
 
+// ------------------------------------------------------------------ loader / consumer variant (16-byte aligned rows)
+// Same arithmetic, lane mapping and reduction order as k_matvec, but the weights take the way global -> LDS ->
+// registers and the wavefronts are specialised: W consumers quantize the activations, read weight rows from an LDS
+// ring and compute; one loader copies the workgroup's rows (contiguous in memory) into the ring with direct-to-LDS
+// loads, R rows per step, every stage of the ring requested before the consumers have finished the activation
+// prologue. In k_matvec a wavefront that wants to issue the loads of its next rows is held at the issue stage while
+// the memory queues of the CU are full (under a saturated HBM: most of the time) and cannot compute on the rows it
+// already has; measured with the cycle counter, its life is 20 % activation prologue, 40 % load issue, 27 % compute,
+// 10 % reduction, one after the other. Here the loader absorbs the issue stalls and the prologue overlaps the first
+// loads. Steps are separated by a bare s_barrier (no implied memory wait).
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef const __attribute__((address_space(1))) uint8_t glb_u8;
+constexpr int MV_LS_STAGES = 3;
+
+template <class Fmt, int NC, int C, int R, bool FUSED>
+__global__ __launch_bounds__(576) void k_matvec_ls(const MatvecParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+    warm_kernel_arguments<sizeof(MatvecParams)>();
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int W = (int)(blockDim.x >> 6) - 1;  // consumers
+    const bool loader = wave == W;
+    const int sub = lane % Fmt::LPB;
+    const uint8_t *__restrict__ wbase = p.w[blockIdx.y];
+    const size_t n0 = p.n0;
+    const size_t row0 = (size_t)blockIdx.x * p.rows_per_wg;
+    const int rows = p.rows_per_wg;  // a multiple of R
+    const int load_steps = rows / R;
+    // LDS: [partial sums: rows x NC x 4W floats][ring: STAGES x stage_stride bytes]
+    float *partial = (float *)lds_raw;
+    const int pstride = 4 * W;
+    const uint32_t stage_bytes = (uint32_t)(R * p.row_bytes);
+    const uint32_t stage_stride = (stage_bytes + 1023u) & ~1023u;
+    uint8_t *ring = lds_raw + (((size_t)rows * NC * pstride * sizeof(float) + 15) & ~(size_t)15);
+
+    if (loader) {
+        const int chunks = (int)(stage_stride >> 10);  // direct-to-LDS instructions per step (1 KiB each)
+        const bool ragged = row0 + rows > p.M;         // some step is cut short: its instruction count is unknown
+        auto issue_step = [&](int t) {
+            const size_t r = row0 + (size_t)t * R;
+            uint32_t valid = stage_bytes;  // bytes of this step that exist (rows beyond M are not read)
+            if (r + R > p.M) {
+                valid = r < p.M ? (uint32_t)((p.M - r) * p.row_bytes) : 0u;
+            }
+            const uint8_t *src = wbase + r * p.row_bytes;
+            uint8_t *dst = ring + (size_t)(t % MV_LS_STAGES) * stage_stride;
+            for (int c = 0; c < chunks; ++c) {
+                const uint32_t off = (uint32_t)c * 1024u + (uint32_t)lane * 16u;
+                if (off < valid) {
+                    __builtin_amdgcn_global_load_lds((glb_u8 *)(src + off), (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+                }
+            }
+        };
+        // every stage is free at the start: all of them are requested while the consumers prepare the activations;
+        // with fused quantization, after the consumers have issued their first activation loads
+        if (FUSED) {
+            __builtin_amdgcn_s_barrier();
+        }
+        for (int t = 0; t < MV_LS_STAGES && t < load_steps; ++t) {
+            issue_step(t);
+        }
+        for (int b = 0; b < load_steps; ++b) {
+            // Loads complete in order: step b has landed once at most the loads of the steps issued after it are
+            // outstanding. Steps up to b + STAGES - 2 have been issued here (all STAGES of them when b == 0).
+            int newer = (b == 0 ? MV_LS_STAGES - 1 : MV_LS_STAGES - 2);
+            if (newer > load_steps - 1 - b) {
+                newer = load_steps - 1 - b;
+            }
+            wait_vmcnt_at_most(ragged ? 0 : newer * chunks);
+            __builtin_amdgcn_s_barrier();  // barrier b: step b may be read; the consumers are done with step b - 1
+            if (b >= 1 && b + MV_LS_STAGES - 1 < load_steps) {
+                issue_step(b + MV_LS_STAGES - 1);  // into the stage of step b - 1
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __builtin_amdgcn_s_barrier();  // final barrier: partial sums complete
+    } else {
+        typename Fmt::Act act[C][NC];
+        size_t blk[C];
+        bool valid[C];
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            blk[i] = (size_t)(wave * C + i) * Fmt::BPW + lane / Fmt::LPB;
+            valid[i] = blk[i] < p.nb;
+#pragma unroll
+            for (int n = 0; n < NC; ++n) {
+                if constexpr (FUSED) {
+                    // wave-load 0 of a consumer is never empty (W is the number of wave-loads that hold blocks, and
+                    // lanes beyond nb clamp to the last block), so every consumer signals exactly once
+                    if (i == 0 && n == 0) {
+                        const size_t bq = valid[i] ? blk[i] : p.nb - 1;
+                        Fmt::template quant_act<true>(act[i][n], p.x + (n0 + n) * p.K, bq, sub);
+                        if (!valid[i]) {
+                            Fmt::zero_act(act[i][n]);
+                        }
+                    } else if (valid[i]) {
+                        Fmt::quant_act(act[i][n], p.x + (n0 + n) * p.K, blk[i], sub);
+                    } else {
+                        Fmt::zero_act(act[i][n]);
+                    }
+                } else if (valid[i]) {
+                    Fmt::load_act(act[i][n], p.act, n0 + n, blk[i], sub);
+                } else {
+                    Fmt::zero_act(act[i][n]);
+                }
+            }
+        }
+        const int pslot = wave * 4 + (lane >> 4);
+        for (int b = 0; b < load_steps; ++b) {
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the previous stage has been read before it is reused
+            __builtin_amdgcn_s_barrier();        // barrier b
+            const uint8_t *stage = ring + (size_t)(b % MV_LS_STAGES) * stage_stride;
+            typename Fmt::Wt wt[R][C];
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+                for (int i = 0; i < C; ++i) {
+                    if (valid[i]) {
+                        Fmt::load_w(wt[rr][i], stage + (size_t)rr * p.row_bytes + blk[i] * Fmt::BYTES, sub);
+                    }
+                }
+            }
+#pragma unroll
+            for (int rr = 0; rr < R; ++rr) {
+                float acc[NC];
+#pragma unroll
+                for (int n = 0; n < NC; ++n) {
+                    acc[n] = 0.0f;
+                }
+#pragma unroll
+                for (int i = 0; i < C; ++i) {
+                    if (valid[i]) {
+                        Fmt::template accumulate<NC>(wt[rr][i], act[i], acc, sub);
+                    }
+                }
+#pragma unroll
+                for (int n = 0; n < NC; ++n) {
+                    const float sum = row16_sum(acc[n]);
+                    if ((lane & 15) == 0) {
+                        partial[((b * R + rr) * NC + n) * pstride + pslot] = sum;
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();  // final barrier: partial sums complete
+    }
+    void *out = p.out[blockIdx.y];
+    for (int idx = threadIdx.x; idx < rows * NC; idx += blockDim.x) {
+        const size_t row = row0 + idx / NC;
+        const int n = idx % NC;
+        if (row < p.M) {
+            // W <= 8 float4 partials, all read before the first add so that only one LDS latency is exposed
+            const float4 *pv = (const float4 *)(partial + idx * pstride);
+            float4 v[8];
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                v[w] = pv[w < W ? w : 0];
+            }
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
+                sum += w < W ? t : 0.0f;
+            }
+            store_out(p, out, n0 + n, row, sum);
+        }
+    }
+}
+
+// rows whose bytes can be copied as 16-byte chunks: row pitch and base address multiples of 16, at most 8 K slices
+template <class Fmt>
+static bool matvec_ls_usable(const MatvecParams &p, size_t K, int C) {
+    const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
+    const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
+    return p.items == nullptr && K % Fmt::BV == 0 && p.row_bytes % 16 == 0 && (((uintptr_t)p.w[0]) & 15) == 0 &&
+           (((uintptr_t)p.w[1]) & 15) == 0 && wave_loads <= (size_t)(8 * C) && getenv("MH_MV_NO_LS") == nullptr;
+}
+
+template <class Fmt, int NC, int C, int R, bool FUSED>
+static int launch_ls(marmot_hip_device *dev, MatvecParams p, int W, size_t M, bool dual) {
+    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1, 1);
+    const size_t part = (((size_t)p.rows_per_wg * NC * 4 * W * sizeof(float)) + 15) & ~(size_t)15;
+    const size_t stage_stride = ((size_t)R * p.row_bytes + 1023) & ~(size_t)1023;
+    const size_t lds = part + MV_LS_STAGES * stage_stride;
+    static bool attr_set = false;
+    if (!attr_set) {
+        MH_HIP(hipFuncSetAttribute((const void *)k_matvec_ls<Fmt, NC, C, R, FUSED>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((k_matvec_ls<Fmt, NC, C, R, FUSED>), grid, dim3((W + 1) * 64), lds, dev->stream, p);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
 template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
 static int launch_one(marmot_hip_device *dev, const MatvecParams &p, int W, size_t M, bool dual) {
     const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1,
@@ -680,6 +886,26 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
     }
     p.rows_per_wg = (int)rows_per_wg;
     set_route(name);
+    if constexpr (std::is_same<Fmt, FmtQ4K>::value && NC <= 4) {
+        // with packed activations there is no prologue to hide: worth it from about 16 MB of weights
+        if (matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
+            // rows per workgroup: two workgroups per CU when M allows, between 8 (the activation prologue must pay
+            // off) and 16 (more rows per workgroup leave CUs idle at the usual M)
+            size_t rows_ls = (M + 2 * cus - 1) / (2 * cus);
+            rows_ls = ((rows_ls + 3) / 4) * 4;
+            rows_ls = rows_ls < 8 ? 8 : (rows_ls > 16 ? 16 : rows_ls);
+            if (const char *e = getenv("MH_RPW")) {
+                rows_ls = (size_t)atoi(e);
+            }
+            p.rows_per_wg = (int)rows_ls;
+            if (C == 1) {
+                return fused ? launch_ls<Fmt, NC, 1, 2, true>(dev, p, W, M, dual)
+                             : launch_ls<Fmt, NC, 1, 2, false>(dev, p, W, M, dual);
+            }
+            return fused ? launch_ls<Fmt, NC, 2, 2, true>(dev, p, W, M, dual)
+                         : launch_ls<Fmt, NC, 2, 2, false>(dev, p, W, M, dual);
+        }
+    }
     const bool exact = (size_t)W * C * Fmt::BPW == nb && K % Fmt::BV == 0 && M % rows_per_wg == 0;
     if constexpr (NC <= 4) {
         if (fused) {

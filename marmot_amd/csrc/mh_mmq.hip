@@ -184,26 +184,7 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
             // loads complete in order: block t - (AHEAD - 1) has landed once at most the loads of the AHEAD - 1 newer
             // steps are outstanding
             const int newer = t < p.bpw ? (AHEAD - 1) : (AHEAD - 1) - (t - p.bpw + 1);
-            const int allowed = newer > 0 ? newer * W * LOADS : 0;
-            if (allowed >= 60) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (60 & 15) | ((60 >> 4) << 14));
-            } else if (allowed >= 50) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (50 & 15) | ((50 >> 4) << 14));
-            } else if (allowed >= 40) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (40 & 15) | ((40 >> 4) << 14));
-            } else if (allowed >= 32) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (32 & 15) | ((32 >> 4) << 14));
-            } else if (allowed >= 24) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (24 & 15) | ((24 >> 4) << 14));
-            } else if (allowed >= 16) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | (16 & 15) | ((16 >> 4) << 14));
-            } else if (allowed >= 10) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | 10);
-            } else if (allowed >= 8) {
-                __builtin_amdgcn_s_waitcnt(0x0f70 | 8);
-            } else {
-                __builtin_amdgcn_s_waitcnt(0x0f70);
-            }
+            wait_vmcnt_at_most(newer > 0 ? newer * W * LOADS : 0);
             __builtin_amdgcn_s_barrier();
         }
     } else {

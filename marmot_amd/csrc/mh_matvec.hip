@@ -290,11 +290,12 @@ struct FmtQ6K {
         }
         a.d = av.d[n * av.nb + blk];
     }
+    template <bool SIGNAL = false>
     __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
         const int hh = sub >> 1, t = sub & 1;
         const int base = 128 * hh + 16 * t;
         const int off[4] = {base, base + 32, base + 64, base + 96};
-        q8k_quantize_runs<4, 4>(xrow + blk * QK_K, off, a.a, a.bs, a.d);
+        q8k_quantize_runs<4, 4, SIGNAL>(xrow + blk * QK_K, off, a.a, a.bs, a.d);
     }
     __device__ static void zero_act(Act &a) {
 #pragma unroll
@@ -886,9 +887,12 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
     }
     p.rows_per_wg = (int)rows_per_wg;
     set_route(name);
-    if constexpr (std::is_same<Fmt, FmtQ4K>::value && NC <= 4) {
-        // with packed activations there is no prologue to hide: worth it from about 16 MB of weights
-        if (matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
+    if constexpr ((std::is_same<Fmt, FmtQ4K>::value || std::is_same<Fmt, FmtQ6K>::value) && NC <= 4) {
+        // with packed activations there is no prologue to hide: worth it from about 16 MB of weights. Q6_K (rows are
+        // 16-byte aligned when K is a multiple of 2048; blocks inside the LDS copy are not, the reads rely on
+        // unaligned LDS access): measured faster for one activation row and rows up to 8192 values, slower beyond.
+        const bool fmt_ok = std::is_same<Fmt, FmtQ4K>::value || (NC == 1 && K <= 8192);
+        if (fmt_ok && matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
             // rows per workgroup: two workgroups per CU when M allows, between 8 (the activation prologue must pay
             // off) and 16 (more rows per workgroup leave CUs idle at the usual M)
             size_t rows_ls = (M + 2 * cus - 1) / (2 * cus);

@@ -581,6 +581,278 @@ __global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
     }
 }
 
+// ------------------------------------------------------------------ Q6_K x Q8_K, loader / consumer wavefronts
+// For rows of a multiple of 8 blocks (K a multiple of 2048) a weight row is 16-byte aligned and the loader can copy
+// with direct-to-LDS loads like the Q4_K kernel. A block starts at byte 210 * b of its row, i.e. o = (2 * b) % 16
+// bytes into a 16-byte chunk: the stage holds, for each of the 32 rows, the 15 chunks from the one that contains the
+// block start (stride 240 B as above; the 15th chunk is never needed and is not loaded), and the consumers read the
+// block at offset o inside the row slot, relying on unaligned LDS reads. Same arithmetic and MFMA sequence as
+// k_mmq_q6k, same step protocol as k_mmq_q4k.
+template <int NR, int STAGES>
+__global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
+    constexpr int TOK = 2 * NR;
+    constexpr int A_OFF = MMQ6_WBLK, D_OFF = A_OFF + TOK * QK_K, STAGE = D_OFF + TOK * 4;
+    constexpr int W_LOADS = 8;                 // 32 rows x 15 chunk slots = 480 lanes of 16 bytes
+    constexpr int A_LOADS = TOK / 4;
+    constexpr int LOADS = W_LOADS + A_LOADS + 1;
+    constexpr int AHEAD = STAGES - 1;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    warm_kernel_arguments<sizeof(MmqParams)>();
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
+    const bool loader = wave == W;
+    const int j = lane & 31, kh = lane >> 5;
+    const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
+    const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
+    const uint8_t *wbase = p.w[which];
+    size_t n0 = p.n0;
+    int ncols = p.ncols;
+    if (p.items != nullptr) {
+        if ((int)blockIdx.z >= *p.n_items) {
+            return;  // uniform for the whole workgroup, before any barrier
+        }
+        const int4 it = p.items[blockIdx.z];
+        wbase += (size_t)it.x * p.expert_stride;
+        n0 = (size_t)it.y;
+        ncols = it.z;
+    }
+    const size_t row0 = (size_t)blockIdx.x * 32;
+    const int steps = p.bpw + AHEAD;
+    auto first_block = [&](int w) { return ((size_t)split * W + w) * p.bpw; };
+    auto block_count = [&](int w) {
+        const size_t b0 = first_block(w);
+        size_t b1 = b0 + p.bpw;
+        if (b1 > p.nb) {
+            b1 = p.nb;
+        }
+        return b1 > b0 ? (int)(b1 - b0) : 0;
+    };
+
+    float acc[NR];
+    int tok[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        acc[r] = 0.0f;
+        tok[r] = 8 * (r >> 2) + 4 * kh + (r & 3);
+    }
+
+    if (loader) {
+        const size_t row_bytes = p.nb * Q6_K_BYTES;
+        uint32_t w_off[W_LOADS];
+        bool w_on[W_LOADS];
+#pragma unroll
+        for (int c = 0; c < W_LOADS; ++c) {
+            const int idx = c * 64 + lane;
+            const int row = idx / 15, pc = idx - row * 15;
+            size_t m = row0 + (row < 32 ? row : 31);
+            if (m >= p.M) {
+                m = p.M - 1;  // harmless re-read; never stored
+            }
+            w_off[c] = (uint32_t)((m - row0) * row_bytes + 16 * pc);
+            w_on[c] = row < 32 && pc < 14;
+        }
+        const uint8_t *wgroup = wbase + row0 * row_bytes;
+        uint32_t a_off[A_LOADS];
+#pragma unroll
+        for (int c = 0; c < A_LOADS; ++c) {
+            const int chunk = c * 64 + lane;
+            const int slot = chunk & 15, tk = chunk >> 4;
+            const int tt = tk < ncols ? tk : 0;
+            const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+            a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
+        }
+        uint32_t ad_off;
+        {
+            const int tk = lane & (TOK - 1);
+            const int tt = tk < ncols ? tk : 0;
+            const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
+            ad_off = (uint32_t)(arow * p.nb);
+        }
+        for (int t = 0; t < steps; ++t) {
+            if (t < p.bpw) {
+                for (int w = 0; w < W; ++w) {
+                    const int nb_w = block_count(w);
+                    size_t b = first_block(w) + (t < nb_w ? t : (nb_w > 0 ? nb_w - 1 : 0));
+                    if (b >= p.nb) {
+                        b = p.nb - 1;
+                    }
+                    const size_t blk_lo = (b * Q6_K_BYTES) & ~(size_t)15;  // chunk that contains the block start
+                    uint8_t *dst = lds + ((size_t)w * STAGES + (t % STAGES)) * STAGE;
+#pragma unroll
+                    for (int c = 0; c < W_LOADS; ++c) {
+                        if (w_on[c]) {
+                            __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + blk_lo),
+                                                             (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+                        }
+                    }
+#pragma unroll
+                    for (int c = 0; c < A_LOADS; ++c) {
+                        __builtin_amdgcn_global_load_lds((glb_u8 *)(p.qs + a_off[c] + b * QK_K),
+                                                         (lds_u8 *)(dst + A_OFF + c * 1024), 16, 0, 0);
+                    }
+                    if (lane < TOK) {
+                        __builtin_amdgcn_global_load_lds((glb_u8 *)(p.ad + ad_off + b), (lds_u8 *)(dst + D_OFF), 4, 0,
+                                                         0);
+                    }
+                }
+            }
+            const int newer = t < p.bpw ? (AHEAD - 1) : (AHEAD - 1) - (t - p.bpw + 1);
+            wait_vmcnt_at_most(newer > 0 ? newer * W * LOADS : 0);
+            __builtin_amdgcn_s_barrier();
+        }
+    } else {
+        const int nblk = block_count(wave);
+        const size_t b_first = first_block(wave);
+        const uint8_t *ring = lds + (size_t)wave * STAGES * STAGE;
+        const int ti = j & (TOK - 1);
+        for (int t = 0; t < steps; ++t) {
+            const int blk = t - AHEAD;
+            if (blk >= 0 && blk < nblk) {
+                const uint8_t *stage = ring + (blk % STAGES) * STAGE;
+                const int o = (int)(((b_first + blk) * Q6_K_BYTES) & 15);
+                const uint8_t *wrow = stage + j * MMQ6_ROWB + o;
+                const uint8_t *a_blk = stage + A_OFF + ti * QK_K + 8 * kh;
+                const float *ad_blk = (const float *)(stage + D_OFF);
+                uint4 scv;
+                __builtin_memcpy(&scv, wrow + 192, 16);
+                uint16_t dh;
+                __builtin_memcpy(&dh, wrow + 208, 2);
+                const float d = h2f(dh);
+                uint2 ql[2][2][2], qh[2][2];  // [half][second 32][second 16], [half][second 16]: this lane's 8 bytes each
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int s16 = 0; s16 < 2; ++s16) {
+                        __builtin_memcpy(&qh[h][s16], wrow + 128 + 32 * h + 16 * s16 + 8 * kh, 8);
+#pragma unroll
+                        for (int h32 = 0; h32 < 2; ++h32) {
+                            __builtin_memcpy(&ql[h][h32][s16], wrow + 64 * h + 32 * h32 + 16 * s16 + 8 * kh, 8);
+                        }
+                    }
+                }
+                float adr[NR];
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    adr[r] = ad_blk[tok[r] & (TOK - 1)];
+                }
+                int bsum[NR];
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    bsum[r] = 0;
+                }
+                const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+                auto acts_of = [&](int is) {
+                    const uint2 v = *(const uint2 *)(a_blk + 16 * (is ^ ti));
+                    return (long)(((unsigned long)v.y << 32) | v.x);
+                };
+                auto weights_of = [&](int is) {
+                    const int h = is >> 3, q = (is >> 1) & 3, s16 = is & 1;
+                    const uint2 l = ql[h][q & 1][s16], hh = qh[h][s16];
+                    uint32_t x = (q >> 1) ? ((l.x >> 4) & 0x0f0f0f0fu) : (l.x & 0x0f0f0f0fu);
+                    uint32_t y = (q >> 1) ? ((l.y >> 4) & 0x0f0f0f0fu) : (l.y & 0x0f0f0f0fu);
+                    x |= ((hh.x >> (2 * q)) & 0x03030303u) << 4;
+                    y |= ((hh.y >> (2 * q)) & 0x03030303u) << 4;
+                    return (long)(((unsigned long)y << 32) | x);
+                };
+                const intx16 zero = {0};
+                intx16 ds = {0};
+                intx16 dq[2];
+                long av[2];
+                av[0] = acts_of(0);
+                dq[0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[0], weights_of(0), zero, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int is = 0; is < 16; ++is) {
+                    const uint32_t scb = (scw[is >> 2] >> (8 * (is & 3))) & 0xffu;
+                    const int sc = (int)(int8_t)scb;
+                    const uint32_t sc4 = scb * 0x01010101u;
+                    ds = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[is & 1], (long)(((unsigned long)sc4 << 32) | sc4), ds,
+                                                               0, 0, 0);
+                    if (is < 15) {
+                        av[(is + 1) & 1] = acts_of(is + 1);
+                        dq[(is + 1) & 1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[(is + 1) & 1], weights_of(is + 1),
+                                                                                 zero, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < NR; ++r) {
+                        bsum[r] += __mul24(dq[is & 1][r], sc);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int r = 0; r < NR; ++r) {
+                    acc[r] += (adr[r] * d) * (float)(bsum[r] - 32 * ds[r]);
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this step's LDS reads are done before the stage is reused
+            __builtin_amdgcn_s_barrier();
+        }
+    }
+
+    if (W > 1) {
+        float *red = (float *)lds;
+        if (!loader) {
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                red[(wave * NR + r) * 64 + lane] = acc[r];
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();
+        if (wave != 0) {
+            return;
+        }
+        float part[4][NR];
+#pragma unroll
+        for (int w2 = 0; w2 < 4; ++w2) {
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                part[w2][r] = w2 < W ? red[(w2 * NR + r) * 64 + lane] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            float sum = part[0][r];
+#pragma unroll
+            for (int w2 = 1; w2 < 4; ++w2) {
+                if (w2 < W) {
+                    sum += part[w2][r];
+                }
+            }
+            acc[r] = sum;
+        }
+    } else if (loader) {
+        return;
+    }
+    const size_t mm = row0 + j;
+    if (mm >= p.M) {
+        return;
+    }
+    void *out = p.out[which];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        if (tok[r] >= ncols) {
+            continue;
+        }
+        const size_t n = n0 + tok[r];
+        if (p.splits > 1) {
+            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
+        } else if (!p.out_is_f16) {
+            float v = acc[r];
+            if (p.bias != nullptr) {
+                v += ((const float *)p.bias)[mm];
+            }
+            ((float *)out)[n * p.M + mm] = v;
+        } else {
+            uint16_t h = f2h(acc[r]);
+            if (p.bias != nullptr) {
+                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+                h = f2h(h2f(h) + bv);
+            }
+            ((uint16_t *)out)[n * p.M + mm] = h;
+        }
+    }
+}
+
 bool mmq_supported(int kind, size_t N, size_t K) {
     if (getenv("MARMOT_HIP_NO_MMQ") != nullptr) {
         return false;
@@ -596,18 +868,37 @@ struct MmqPlan {
     int W, S, bpw;
 };
 
-// W (consumer) wavefronts per workgroup and S workgroups split K so that at least one workgroup per CU is resident.
-// Q4_K with more than 8 activation rows stages 16 rows per block; two consumers per workgroup keep the LDS ring small
-// enough for three workgroups per CU.
+// rows of a multiple of 8 blocks are 16-byte aligned: the loader/consumer kernel applies
+static bool mmq6_uses_loader(size_t nb) {
+    return nb % 8 == 0 && getenv("MH_MMQ6_NO_LS") == nullptr;
+}
+
+// W (consumer) wavefronts per workgroup and S workgroups split K.
+//   * Many row groups (M / 32 >= CUs), Q4_K: the consumers of one workgroup split K (no partials); with more than 8
+//     activation rows 16 rows are staged per block and two consumers keep the LDS ring small enough for three
+//     workgroups per CU.
+//   * Few row groups, and Q6_K with the loader (its stages are larger): one consumer per workgroup and K split over
+//     about 4 (Q6_K: 3.5) workgroups per CU, which overlap each other's load and compute phases; the partials meet
+//     in the reduction kernel. Measured per shape; e.g. Q4_K 4096 x 14336 N=8: 19.1 -> 18.0 us, Q6_K 14336 x 4096
+//     N=8: 34.0 -> 28.4 us.
 static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t M, size_t nb) {
     const size_t rg = (M + 31) / 32;
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     MmqPlan pl;
-    const size_t w_max = (kind == MARMOT_HIP_KIND_Q4_K && N > 8) ? 2 : 4;
-    size_t W = nb < w_max ? nb : w_max;
-    size_t S = 1;
-    while (rg * S < cus && W * S * 2 <= nb) {
-        S *= 2;
+    const bool q6_loader = kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(nb);
+    size_t W, S = 1;
+    if (q6_loader || (kind == MARMOT_HIP_KIND_Q4_K && rg < cus)) {
+        W = 1;
+        const size_t want = ((q6_loader ? 7 : 8) * cus / 2 + rg - 1) / rg;  // workgroups along K
+        while (S < want && S * 8 <= nb) {
+            S *= 2;
+        }
+    } else {
+        const size_t w_max = (kind == MARMOT_HIP_KIND_Q4_K && N > 8) ? 2 : 4;
+        W = nb < w_max ? nb : w_max;
+        while (rg * S < cus && W * S * 2 <= nb) {
+            S *= 2;
+        }
     }
     if (const char *e = getenv("MH_MMQ_W")) {
         W = (size_t)atoi(e);
@@ -648,7 +939,27 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
                                    (int)mmq6_lds_bytes(6)));
         attr_set = true;
     }
-    if (kind == MARMOT_HIP_KIND_Q6_K) {
+    if (kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(p.nb) && pl.W <= 4 && (((uintptr_t)p.w[0]) & 15) == 0 &&
+        (((uintptr_t)p.w[1]) & 15) == 0 && (p.expert_stride & 15) == 0) {
+        const int stages = p.items != nullptr ? 2 : 3;
+        const size_t stage = MMQ6_WBLK + 2 * NR * QK_K + 2 * NR * 4;
+        const size_t ring = (size_t)pl.W * stages * stage;
+        const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
+        const dim3 block((pl.W + 1) * 64);
+        static bool ls6_attr = false;
+        if (!ls6_attr) {
+            MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       160 * 1024));
+            MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       160 * 1024));
+            ls6_attr = true;
+        }
+        if (stages == 2) {
+            hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 2>), grid, block, ring > red ? ring : red, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 3>), grid, block, ring > red ? ring : red, dev->stream, p);
+        }
+    } else if (kind == MARMOT_HIP_KIND_Q6_K) {
         hipLaunchKernelGGL((k_mmq_q6k<NR>), grid, dim3(pl.W * 64), mmq6_lds_bytes(pl.W), dev->stream, p);
     } else {
         // W consumers + 1 loader. Three stages (the loader two blocks ahead) for the dense call; the grouped call

@@ -146,10 +146,16 @@ __device__ __forceinline__ void q8k_quantize_runs(const float *xblk, const int (
 }
 
 // Q8_0 quantization (matmul_quant_pack.c:23-62, scalar rounding) of one 32-value block owned by this lane.
+template <bool SIGNAL = false>
 __device__ __forceinline__ void q80_quantize_block(const float *xblk, uint4 &q0, uint4 &q1, float &d, int &sum) {
     float v[32];
     ld16f(xblk, v);
     ld16f(xblk + 16, v + 16);
+    if (SIGNAL) {  // see q8k_quantize_runs
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
     float max_abs = 0.0f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
@@ -370,9 +376,10 @@ struct FmtQ80 {
         a.a1 = *(const uint4 *)(base + 16);
         a.d = av.d[n * av.nb + blk];
     }
+    template <bool SIGNAL = false>
     __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int) {
         int sum;
-        q80_quantize_block(xrow + blk * QK, a.a0, a.a1, a.d, sum);
+        q80_quantize_block<SIGNAL>(xrow + blk * QK, a.a0, a.a1, a.d, sum);
     }
     __device__ static void zero_act(Act &a) {
         a.a0 = a.a1 = make_uint4(0, 0, 0, 0);
@@ -418,8 +425,9 @@ struct FmtQ40 {
         a.d = av.d[n * av.nb + blk];
         a.sum = av.sums[n * av.nb + blk];
     }
+    template <bool SIGNAL = false>
     __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int) {
-        q80_quantize_block(xrow + blk * QK, a.a0, a.a1, a.d, a.sum);
+        q80_quantize_block<SIGNAL>(xrow + blk * QK, a.a0, a.a1, a.d, a.sum);
     }
     __device__ static void zero_act(Act &a) {
         a.a0 = a.a1 = make_uint4(0, 0, 0, 0);
@@ -887,10 +895,12 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
     }
     p.rows_per_wg = (int)rows_per_wg;
     set_route(name);
-    if constexpr ((std::is_same<Fmt, FmtQ4K>::value || std::is_same<Fmt, FmtQ6K>::value) && NC <= 4) {
-        // with packed activations there is no prologue to hide: worth it from about 16 MB of weights. Q6_K (rows are
-        // 16-byte aligned when K is a multiple of 2048; blocks inside the LDS copy are not, the reads rely on
-        // unaligned LDS access): measured faster for one activation row and rows up to 8192 values, slower beyond.
+    if constexpr (NC <= 4) {
+        // With packed activations there is no prologue to hide: worth it from about 16 MB of weights. Formats other
+        // than Q4_K have 16-byte aligned rows when a row holds a multiple of 8 blocks; their blocks inside the LDS copy
+        // are not aligned and the reads rely on unaligned LDS access. Measured faster for one activation row and rows
+        // up to 8192 values (Q6_K 14336 x 4096: 15.5 -> 12.9 us, Q8_0 18.4 -> 15.2, Q4_0 12.7 -> 10.1, Q8_0
+        // 5632 x 2048: 6.8 -> 6.1), slower for Q6_K at K = 14336 and for more activation rows.
         const bool fmt_ok = std::is_same<Fmt, FmtQ4K>::value || (NC == 1 && K <= 8192);
         if (fmt_ok && matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
             // rows per workgroup: two workgroups per CU when M allows, between 8 (the activation prologue must pay

@@ -164,7 +164,7 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
 
 
 def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5")):
-    """Every configuration of BASELINE.json on the device, one JSON line each (documentation runs, not the
+    """Every benchmark configuration (C1..C5) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -317,7 +317,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--prefill-tokens", type=int, default=512)
     ap.add_argument("--sweep", action="store_true",
-                    help="measure every BASELINE configuration instead, one JSON line each (documentation runs)")
+                    help="measure every benchmark configuration (C1..C5) instead, one JSON line each (documentation runs)")
     ap.add_argument("--configs", default="C1,C2,C3,C4,C5", help="with --sweep: the configurations to run")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")

@@ -43,7 +43,7 @@ def test_block_geometry(lib):
     assert lib.marmot_hip_row_bytes(5, 2048) == 2176
     assert lib.marmot_hip_row_bytes(11, 14336) == 56 * 210
     assert lib.marmot_hip_row_bytes(99, 256) == 0
-    # BASELINE shapes: 14336 x 4096 Q4_K = 33,030,144 B; Q6_K = 48,168,960 B; Q8_0 5632 x 2048 = 12,255,232 B
+    # benchmark shapes: 14336 x 4096 Q4_K = 33,030,144 B; Q6_K = 48,168,960 B; Q8_0 5632 x 2048 = 12,255,232 B
     assert 14336 * lib.marmot_hip_row_bytes(9, 4096) == 33030144
     assert 4096 * lib.marmot_hip_row_bytes(9, 14336) == 33030144
     assert 14336 * lib.marmot_hip_row_bytes(11, 4096) == 48168960

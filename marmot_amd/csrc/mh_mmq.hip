@@ -247,8 +247,9 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
 #pragma unroll
                 for (int sb = 0; sb < 8; ++sb) {
                     const int sc = (int)(((sb < 4 ? sc_lo : sc_hi) >> (8 * (sb & 3))) & 0xffu);
-                    const int mn = (int)(((sb < 4 ? mn_lo : mn_hi) >> (8 * (sb & 3))) & 0xffu);
-                    const int mn4 = mn * 0x01010101;
+                    // byte sb & 3 of the packed mins in all four bytes (v_perm_b32: one full-rate instruction where
+                    // extract + multiply by 0x01010101 would be a quarter-rate multiply)
+                    const int mn4 = (int)__builtin_amdgcn_perm(0u, sb < 4 ? mn_lo : mn_hi, 0x01010101u * (sb & 3));
                     dm = __builtin_amdgcn_mfma_i32_32x32x32_i8(acts_of(sb), intx4{mn4, mn4, mn4, mn4}, dm, 0, 0, 0);
                     if (sb < 7) {
                         dq[(sb + 1) & 1] =
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
         for (int is = 0; is < 16; ++is) {
             const uint32_t scb = (scw[is >> 2] >> (8 * (is & 3))) & 0xffu;
             const int sc = (int)(int8_t)scb;
-            const uint32_t sc4 = scb * 0x01010101u;
+            const uint32_t sc4 = __builtin_amdgcn_perm(0u, scw[is >> 2], 0x01010101u * (is & 3));  // byte broadcast
             ds = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[is & 1], (long)(((unsigned long)sc4 << 32) | sc4), ds, 0, 0, 0);
             if (is < 15) {
                 av[(is + 1) & 1] = acts_of(is + 1);
@@ -764,7 +765,7 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
                 for (int is = 0; is < 16; ++is) {
                     const uint32_t scb = (scw[is >> 2] >> (8 * (is & 3))) & 0xffu;
                     const int sc = (int)(int8_t)scb;
-                    const uint32_t sc4 = scb * 0x01010101u;
+                    const uint32_t sc4 = __builtin_amdgcn_perm(0u, scw[is >> 2], 0x01010101u * (is & 3));  // byte broadcast
                     ds = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[is & 1], (long)(((unsigned long)sc4 << 32) | sc4), ds,
                                                                0, 0, 0);
                     if (is < 15) {

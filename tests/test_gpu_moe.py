@@ -91,6 +91,20 @@ def test_moe_many_routes(hip, oracle, T):
     assert_moe_parity(got, ref, what=f"moe many routes T={T}")
 
 
+def test_moe_q6k_experts_with_aligned_rows(hip, oracle):
+    """Q6_K experts whose rows hold a multiple of 8 blocks (K = 2048): the grouped matmuls take the loader/consumer
+    kernel with its 16-byte aligned row copies, both the dual gate/up launch and the down launch."""
+    E, F, H, k, T = 4, 2048, 2048, 2, 9
+    kind = KIND_Q6_K
+    gate, up, down = make_experts(oracle, 440, E, F, H, kind, kind)
+    hidden = gaussian(441, (T, H))
+    vals, ids = oracle.topk(gaussian(442, (T, E)), k)
+    w = oracle.softmax_rows(vals)
+    ref = oracle.moe_experts(hidden, gate, up, down, ids, w, F, E, kind, kind, threads=8)
+    got = hip.moe_experts(hidden, gate, up, down, ids, w, F, E, kind, kind)
+    assert_moe_parity(got, ref, what="moe Q6_K aligned rows")
+
+
 def test_moe_policies_duplicates_unrouted_and_errors(hip, oracle):
     from marmot_amd import MarmotHipError
 

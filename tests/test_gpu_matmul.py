@@ -209,3 +209,22 @@ def test_linear_error_behaviour(hip, oracle):
     # N = 0 is a no-op
     hip.linear_d(KIND_Q4_K, hip.to_device(blocks), hip.to_device(x), 0, 0, K, M, hip.alloc(64), 0)
     hip.synchronize()
+
+
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+def test_loader_consumer_matvec_equals_register_streaming_matvec(hip, oracle, name, monkeypatch):
+    """The loader/consumer matvec (weights through an LDS ring) keeps the lane mapping and the reduction order of the
+    register-streaming kernel: the two must agree bit for bit, on whole and ragged row groups, one and two K slices
+    per lane, fused and packed activations."""
+    kind = KINDS[name]
+    for M, K, N in ((256, 2048, 1), (203, 4096, 1), (77, 8192, 1), (64, 14336, 1), (40, 28672, 1), (203, 4096, 2)):
+        blocks = oracle.quantize(kind, gaussian(500 + K, (M, K), 0.02))
+        x = gaussian(501 + K + N, (N, K))
+        monkeypatch.delenv("MH_MV_NO_LS", raising=False)
+        with_ring = hip.linear(x, blocks, kind, M)
+        monkeypatch.setenv("MH_MV_NO_LS", "1")
+        without = hip.linear(x, blocks, kind, M)
+        monkeypatch.delenv("MH_MV_NO_LS", raising=False)
+        assert np.array_equal(bits(with_ring), bits(without)), f"{name} {M}x{K} N={N}"
+        assert_matmul_parity(with_ring, oracle.matmul(kind, blocks, x, M), what=f"{name} {M}x{K} N={N}")
+

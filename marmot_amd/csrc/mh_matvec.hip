@@ -652,8 +652,15 @@ typedef __attribute__((address_space(3))) uint8_t lds_u8;
 typedef const __attribute__((address_space(1))) uint8_t glb_u8;
 constexpr int MV_LS_STAGES = 3;
 
+// Consumers per workgroup: up to 8 for Q4_K (one wave-load = 8 blocks of 256), up to 4 for the other formats, whose
+// wave-loads are wider and whose kernels need more registers per lane (the bound decides the register budget).
+template <class Fmt>
+constexpr int matvec_ls_max_consumers() {
+    return Fmt::LPB == 8 ? 8 : 4;
+}
+
 template <class Fmt, int NC, int C, int R, bool FUSED>
-__global__ __launch_bounds__(576) void k_matvec_ls(const MatvecParams p) {
+__global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_matvec_ls(const MatvecParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
     warm_kernel_arguments<sizeof(MatvecParams)>();
     const int lane = threadIdx.x & 63;
@@ -814,7 +821,8 @@ static bool matvec_ls_usable(const MatvecParams &p, size_t K, int C) {
     const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
     const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
     return p.items == nullptr && K % Fmt::BV == 0 && p.row_bytes % 16 == 0 && (((uintptr_t)p.w[0]) & 15) == 0 &&
-           (((uintptr_t)p.w[1]) & 15) == 0 && wave_loads <= (size_t)(8 * C) && getenv("MH_MV_NO_LS") == nullptr;
+           (((uintptr_t)p.w[1]) & 15) == 0 && wave_loads <= (size_t)(matvec_ls_max_consumers<Fmt>() * C) &&
+           getenv("MH_MV_NO_LS") == nullptr;
 }
 
 template <class Fmt, int NC, int C, int R, bool FUSED>
@@ -898,10 +906,10 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
     if constexpr (NC <= 4) {
         // With packed activations there is no prologue to hide: worth it from about 16 MB of weights. Formats other
         // than Q4_K have 16-byte aligned rows when a row holds a multiple of 8 blocks; their blocks inside the LDS copy
-        // are not aligned and the reads rely on unaligned LDS access. Measured faster for one activation row and rows
-        // up to 8192 values (Q6_K 14336 x 4096: 15.5 -> 12.9 us, Q8_0 18.4 -> 15.2, Q4_0 12.7 -> 10.1, Q8_0
-        // 5632 x 2048: 6.8 -> 6.1), slower for Q6_K at K = 14336 and for more activation rows.
-        const bool fmt_ok = std::is_same<Fmt, FmtQ4K>::value || (NC == 1 && K <= 8192);
+        // are not aligned and the reads rely on unaligned LDS access. Measured faster for rows up to 8192 values
+        // (14336 x 4096, N = 1 / 2 / 4: Q6_K 15.5 -> 12.9, 18.0 -> 16.7, 24.0 -> 23.5 us; Q8_0 18.4 -> 15.2,
+        // 22.8 -> 16.4, 29.8 -> 22.5 us; Q8_0 5632 x 2048: 6.8 -> 6.1 us), slower for Q6_K at K = 14336.
+        const bool fmt_ok = std::is_same<Fmt, FmtQ4K>::value || K <= 8192;
         if (fmt_ok && matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
             // rows per workgroup: two workgroups per CU when M allows, between 8 (the activation prologue must pay
             // off) and 16 (more rows per workgroup leave CUs idle at the usual M)

@@ -53,6 +53,80 @@ constexpr int MMQ_WBLK = 32 * Q4_K_BYTES;  // one block of 32 weight rows: 4608 
 constexpr int MMQ_ABLK = MMQ_TOK * QK_K;   // one block of 16 activation rows: 4096 bytes
 constexpr int MMQ_STAGES = 2;              // Q6_K: blocks in flight per wavefront
 
+// ---- shared epilogue pieces of the small-batch kernels
+// K-split within the workgroup: the consumers' partial sums meet in LDS and wavefront 0 adds them in wavefront order
+// (all of them requested before the first addition: W <= 4). Every wavefront of the workgroup calls this (it contains
+// a barrier); returns true for the wavefront that goes on to store.
+template <int NR>
+__device__ __forceinline__ bool mmq_reduce_consumers(float *red, int W, int wave, int lane, bool is_consumer,
+                                                     float (&acc)[NR]) {
+    if (is_consumer) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            red[(wave * NR + r) * 64 + lane] = acc[r];
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    if (wave != 0) {
+        return false;
+    }
+    float part[4][NR];
+#pragma unroll
+    for (int w2 = 0; w2 < 4; ++w2) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            part[w2][r] = w2 < W ? red[(w2 * NR + r) * 64 + lane] : 0.0f;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        float sum = part[0][r];
+#pragma unroll
+        for (int w2 = 1; w2 < 4; ++w2) {
+            if (w2 < W) {
+                sum += part[w2][r];
+            }
+        }
+        acc[r] = sum;
+    }
+    return true;
+}
+
+// Stores the sums of weight row mm for the tokens of this lane: fp32 partials of this K split, or the final values
+// with bias in the reference's order (fp16 output: round the dot first, then add the bias to the stored value).
+template <int NR>
+__device__ __forceinline__ void mmq_store(const MmqParams &p, int which, int split, size_t mm, size_t n0, int ncols,
+                                          const int (&tok)[NR], const float (&acc)[NR]) {
+    if (mm >= p.M) {
+        return;
+    }
+    void *out = p.out[which];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        if (tok[r] >= ncols) {
+            continue;
+        }
+        const size_t n = n0 + tok[r];
+        if (p.splits > 1) {
+            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
+        } else if (!p.out_is_f16) {
+            float v = acc[r];
+            if (p.bias != nullptr) {
+                v += ((const float *)p.bias)[mm];
+            }
+            ((float *)out)[n * p.M + mm] = v;
+        } else {
+            uint16_t h = f2h(acc[r]);
+            if (p.bias != nullptr) {
+                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+                h = f2h(h2f(h) + bv);
+            }
+            ((uint16_t *)out)[n * p.M + mm] = h;
+        }
+    }
+}
+
 // ------------------------------------------------------------------ Q4_K x Q8_K
 // Work decomposition. All consumer wavefronts of a workgroup work on the SAME 32 weight rows; consumer w walks its own
 // contiguous range of blocks, so the workgroup as a whole streams whole weight rows (a decomposition in which a
@@ -274,69 +348,13 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
     // ---- K-split within the workgroup: partial sums meet in LDS and are added in wavefront order. The last barrier
     // of the loop guarantees that every stage has been read.
     if (W > 1) {
-        float *red = (float *)lds;
-        if (!loader) {
-#pragma unroll
-            for (int r = 0; r < NR; ++r) {
-                red[(wave * NR + r) * 64 + lane] = acc[r];
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_s_barrier();
-        if (wave != 0) {
+        if (!mmq_reduce_consumers<NR>((float *)lds, W, wave, lane, !loader, acc)) {
             return;
-        }
-        // all partial sums are requested before the first addition (W <= 4); the additions stay in wavefront order
-        float part[4][NR];
-#pragma unroll
-        for (int w2 = 0; w2 < 4; ++w2) {
-#pragma unroll
-            for (int r = 0; r < NR; ++r) {
-                part[w2][r] = w2 < W ? red[(w2 * NR + r) * 64 + lane] : 0.0f;
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            float sum = part[0][r];
-#pragma unroll
-            for (int w2 = 1; w2 < 4; ++w2) {
-                if (w2 < W) {
-                    sum += part[w2][r];
-                }
-            }
-            acc[r] = sum;
         }
     } else if (loader) {
         return;
     }
-    const size_t mm = row0 + j;
-    if (mm >= p.M) {
-        return;
-    }
-    void *out = p.out[which];
-#pragma unroll
-    for (int r = 0; r < NR; ++r) {
-        if (tok[r] >= ncols) {
-            continue;
-        }
-        const size_t n = n0 + tok[r];
-        if (p.splits > 1) {
-            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
-        } else if (!p.out_is_f16) {
-            float v = acc[r];
-            if (p.bias != nullptr) {
-                v += ((const float *)p.bias)[mm];
-            }
-            ((float *)out)[n * p.M + mm] = v;
-        } else {
-            uint16_t h = f2h(acc[r]);  // reference order: store f16(dot), then add the bias to the stored value
-            if (p.bias != nullptr) {
-                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
-                h = f2h(h2f(h) + bv);
-            }
-            ((uint16_t *)out)[n * p.M + mm] = h;
-        }
-    }
+    mmq_store<NR>(p, which, split, row0 + j, n0, ncols, tok, acc);
 }
 
 // ------------------------------------------------------------------ Q6_K x Q8_K
@@ -552,34 +570,7 @@ __global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
             acc[r] = sum;
         }
     }
-    const size_t mm = row0 + j;
-    if (mm >= p.M) {
-        return;
-    }
-    void *out = p.out[which];
-#pragma unroll
-    for (int r = 0; r < NR; ++r) {
-        if (tok[r] >= ncols) {
-            continue;
-        }
-        const size_t n = n0 + tok[r];
-        if (p.splits > 1) {
-            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
-        } else if (!p.out_is_f16) {
-            float v = acc[r];
-            if (p.bias != nullptr) {
-                v += ((const float *)p.bias)[mm];
-            }
-            ((float *)out)[n * p.M + mm] = v;
-        } else {
-            uint16_t h = f2h(acc[r]);
-            if (p.bias != nullptr) {
-                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
-                h = f2h(h2f(h) + bv);
-            }
-            ((uint16_t *)out)[n * p.M + mm] = h;
-        }
-    }
+    mmq_store<NR>(p, which, split, row0 + j, n0, ncols, tok, acc);
 }
 
 // ------------------------------------------------------------------ Q6_K x Q8_K, loader / consumer wavefronts
@@ -790,68 +781,13 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
     }
 
     if (W > 1) {
-        float *red = (float *)lds;
-        if (!loader) {
-#pragma unroll
-            for (int r = 0; r < NR; ++r) {
-                red[(wave * NR + r) * 64 + lane] = acc[r];
-            }
-        }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_s_barrier();
-        if (wave != 0) {
+        if (!mmq_reduce_consumers<NR>((float *)lds, W, wave, lane, !loader, acc)) {
             return;
-        }
-        float part[4][NR];
-#pragma unroll
-        for (int w2 = 0; w2 < 4; ++w2) {
-#pragma unroll
-            for (int r = 0; r < NR; ++r) {
-                part[w2][r] = w2 < W ? red[(w2 * NR + r) * 64 + lane] : 0.0f;
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < NR; ++r) {
-            float sum = part[0][r];
-#pragma unroll
-            for (int w2 = 1; w2 < 4; ++w2) {
-                if (w2 < W) {
-                    sum += part[w2][r];
-                }
-            }
-            acc[r] = sum;
         }
     } else if (loader) {
         return;
     }
-    const size_t mm = row0 + j;
-    if (mm >= p.M) {
-        return;
-    }
-    void *out = p.out[which];
-#pragma unroll
-    for (int r = 0; r < NR; ++r) {
-        if (tok[r] >= ncols) {
-            continue;
-        }
-        const size_t n = n0 + tok[r];
-        if (p.splits > 1) {
-            ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
-        } else if (!p.out_is_f16) {
-            float v = acc[r];
-            if (p.bias != nullptr) {
-                v += ((const float *)p.bias)[mm];
-            }
-            ((float *)out)[n * p.M + mm] = v;
-        } else {
-            uint16_t h = f2h(acc[r]);
-            if (p.bias != nullptr) {
-                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
-                h = f2h(h2f(h) + bv);
-            }
-            ((uint16_t *)out)[n * p.M + mm] = h;
-        }
-    }
+    mmq_store<NR>(p, which, split, row0 + j, n0, ncols, tok, acc);
 }
 
 bool mmq_supported(int kind, size_t N, size_t K) {

@@ -160,7 +160,9 @@ __device__ __forceinline__ void warm_kernel_arguments() {
 #define MH_VMCNT_CASE4(n) MH_VMCNT_CASE(n) MH_VMCNT_CASE(n + 1) MH_VMCNT_CASE(n + 2) MH_VMCNT_CASE(n + 3)
 #define MH_VMCNT_CASE16(n) MH_VMCNT_CASE4(n) MH_VMCNT_CASE4(n + 4) MH_VMCNT_CASE4(n + 8) MH_VMCNT_CASE4(n + 12)
 __device__ __forceinline__ void wait_vmcnt_at_most(int allowed) {
-    switch (allowed > 63 ? 63 : allowed) {
+    // the count is the same for every lane; saying so keeps the dispatch on the scalar unit (compares and branches)
+    // instead of a tree of execution-mask branches
+    switch (__builtin_amdgcn_readfirstlane(allowed > 63 ? 63 : allowed)) {
         MH_VMCNT_CASE16(0)
         MH_VMCNT_CASE16(16)
         MH_VMCNT_CASE16(32)

@@ -102,6 +102,13 @@ __device__ __forceinline__ void mmq_store(const MmqParams &p, int which, int spl
         return;
     }
     void *out = p.out[which];
+    // The bias of this weight row is fetched once, before the stores: a load (and the wait for it) between two stores
+    // would also wait for the earlier store, the memory counter being in order.
+    const bool has_bias = p.splits == 1 && p.bias != nullptr;
+    float bv = 0.0f;
+    if (has_bias) {
+        bv = (p.out_is_f16 && p.bias_is_f16) ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+    }
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
         if (tok[r] >= ncols) {
@@ -111,15 +118,10 @@ __device__ __forceinline__ void mmq_store(const MmqParams &p, int which, int spl
         if (p.splits > 1) {
             ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
         } else if (!p.out_is_f16) {
-            float v = acc[r];
-            if (p.bias != nullptr) {
-                v += ((const float *)p.bias)[mm];
-            }
-            ((float *)out)[n * p.M + mm] = v;
+            ((float *)out)[n * p.M + mm] = has_bias ? acc[r] + bv : acc[r];
         } else {
             uint16_t h = f2h(acc[r]);
-            if (p.bias != nullptr) {
-                const float bv = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+            if (has_bias) {
                 h = f2h(h2f(h) + bv);
             }
             ((uint16_t *)out)[n * p.M + mm] = h;

@@ -201,7 +201,7 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5")):
                 if "C2" in only:
                     linear_case("C2", kind, M, K, N)
     for tokens in (64, 128, 512, 2048) if "C3" in only else ():
-        r = prefill_gemm(hip, tokens, max(20, steps // 20), 5)
+        r = prefill_gemm(hip, tokens, max(100, steps // 2), max(20, steps // 20))
         emit({"config": "C3", "workload": f"Q4_K 4096x4096 N={tokens} fp16", "route": r["route"],
               "us": round(r["ms_per_step"] * 1e3, 2), "TFLOP/s": r["tflops"],
               "frac_of_mfma_peak": r["frac_of_mfma_peak"], "tokens_per_s": round(r["tokens_per_s"])})
@@ -449,7 +449,9 @@ def main():
     }
     # ---- second half of the metric: Q4_K prefill GEMM, weight 4096 x 4096, fp16 activations, fp32 out
     if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) and not args.no_prefill:
-        result["prefill_gemm"] = prefill_gemm(hip, args.prefill_tokens, max(20, args.steps // 20), 5)
+        # as many steps as it takes for the clocks to settle under the matrix-core load (tens of milliseconds)
+        result["prefill_gemm"] = prefill_gemm(hip, args.prefill_tokens, max(100, args.steps // 2),
+                                              max(20, args.steps // 20))
     if not args.no_cpu:
         cb, err = cpu_baseline(kind, blocks, x, M, K, nbytes, got, args.cpu_seconds)
         result["cpu_baseline"] = cb

@@ -245,11 +245,11 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
                 return;
             }
             // Weights (into registers) early, one load per K-step. The activation tile (direct-to-LDS) as late as
-            // possible, all nine pieces in the last K-step: measured with the cycle counter, a block whose K-steps
-            // each issue one direct-to-LDS load takes 13.7 K ticks against 6.2 K for the last block of a workgroup
-            // (which prefetches nothing): the LDS reads of the K-steps behind such a load do not complete before it
-            // does. Issued at the end they overlap only the min-term product and the scale pass, which is still better
-            // (512 tokens: 43.3 -> 38.5 us).
+            // possible, all nine pieces in the last K-step. Measured with the cycle counter: a load issued inside the
+            // K loop costs its wavefront about 230 clocks (the eight wavefronts issue in the same K-step, and one that
+            // is held at the memory issue stage holds back its own MFMA chain), 2 K clocks per block, while the wait
+            // at the end of the block is barrier skew and does not get shorter when the tile was requested earlier.
+            // Issued here the loads overlap the min-term product and the scale pass.
             if (ks == 15) {
 #pragma unroll
                 for (int c = 0; c < 9; ++c) {

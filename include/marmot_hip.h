@@ -169,6 +169,21 @@ int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const v
                                      const void *d_weight_b, const void *d_input, int in_dtype, size_t N, size_t K,
                                      size_t M, void *d_out_a, void *d_out_b, int out_dtype, uint32_t flags);
 
+/* Fused Q/K/V projection, separate weights. Replaces cpu_matmul_qkv_run_separate_quantized_impl
+ * (src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:749-947), reached through cpu_matmul_qkv_{q4_k,q6_k,q8_0}
+ * (matmul_qkv.c:1498-1532) for marmot_matmul_qkv with MARMOT_QKV_LAYOUT_SEPARATE (include/marmot/ops/matmul.h:74-95).
+ * Three weights of one kind and one shape [M,K] are applied to one input [N,K]; the activations are quantized once
+ * (Q8_0 for Q4_0/Q8_0 weights, Q8_K for K-quants: F16 input is packed too, there is no direct F16 route here) and
+ * out_x[n*M + m] = (float)bias_x[m] + dot(Wx[m,:], act[n,:]), one rounding to the output type at the store.
+ *   d_input          : [N,K] of in_dtype (F32 or F16), row-major
+ *   d_bq, d_bk, d_bv : each NULL or M values of bias_dtype (F32 or F16)
+ *   d_out_*          : [N,M] of out_dtype, which must equal in_dtype (matmul_qkv.c:769-772)
+ * The rotary epilogue of the reference op (rope_params) is not part of this call. */
+int marmot_hip_matmul_qkv_quantized(marmot_hip_device_t *dev, int kind, const void *d_wq, const void *d_wk,
+                                    const void *d_wv, const void *d_input, int in_dtype, size_t N, size_t K, size_t M,
+                                    const void *d_bq, const void *d_bk, const void *d_bv, int bias_dtype,
+                                    void *d_out_q, void *d_out_k, void *d_out_v, int out_dtype);
+
 /* ------------------------------------------------------------------ pre-packed activations
  * The reference packs (quantizes) a tile of activations once and then runs the row kernels against the packed
  * tile: cpu_quant_matmul_pack_column (matmul_quant_dispatch.c:270-302) followed by

@@ -246,6 +246,33 @@ class HipBackend:
             for b in (d_a, d_b, d_x, d_oa, d_ob):
                 b.free()
 
+    def linear_qkv(self, x: np.ndarray, wq: np.ndarray, wk: np.ndarray, wv: np.ndarray, kind: int, M: int,
+                   bq=None, bk=None, bv=None):
+        """marmot_matmul_qkv with separate quantized weights of one shape [M, K] (include/marmot/ops/matmul.h:74-95,
+        CPU implementation src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:749-947): returns (q, k, v), each [N, M] of
+        the input dtype; biases are optional per projection and must share one dtype (float32 or float16)."""
+        x = np.ascontiguousarray(x)
+        N, K = x.shape
+        d_w = [self.to_device(np.ascontiguousarray(w, dtype=np.uint8)) for w in (wq, wk, wv)]
+        d_x = self.to_device(x)
+        biases = [None if b is None else np.ascontiguousarray(b) for b in (bq, bk, bv)]
+        given = [b for b in biases if b is not None]
+        if any(b.dtype != given[0].dtype for b in given):
+            raise ValueError("q/k/v biases must share one dtype")
+        d_b = [None if b is None else self.to_device(b) for b in biases]
+        out_dtype = np.dtype(x.dtype)
+        d_o = [self.alloc(N * M * out_dtype.itemsize) for _ in range(3)]
+        try:
+            check(self.lib.marmot_hip_matmul_qkv_quantized(
+                self.dev, kind, *[C.c_void_p(w.ptr) for w in d_w], C.c_void_p(d_x.ptr), _np_dtype_id(x.dtype), N, K, M,
+                *[C.c_void_p(b.ptr if b is not None else None) for b in d_b],
+                _np_dtype_id(given[0].dtype) if given else 0,
+                *[C.c_void_p(o.ptr) for o in d_o], _np_dtype_id(out_dtype)))
+            return tuple(o.download(out_dtype, (N, M)) for o in d_o)
+        finally:
+            for b in d_w + [d_x] + [b for b in d_b if b is not None] + d_o:
+                b.free()
+
     def topk(self, x: np.ndarray, k: int):
         x = np.ascontiguousarray(x, dtype=np.float32)
         rows, cols = x.shape

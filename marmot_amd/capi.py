@@ -65,6 +65,8 @@ SIGNATURES = {
     "marmot_hip_quantize_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
     "marmot_hip_matmul_quantized": (_i, [_vp, _i, _vp, _vp, _i, _sz, _sz, _sz, _vp, _i, _vp, _i, _u32]),
     "marmot_hip_matmul_quantized_dual": (_i, [_vp, _i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _i, _u32]),
+    "marmot_hip_matmul_qkv_quantized": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _vp, _i, _vp,
+                                             _vp, _vp, _i]),
     "marmot_hip_packed_activation_bytes": (_sz, [_i, _sz, _sz]),
     "marmot_hip_pack_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
     "marmot_hip_matmul_prepacked": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _vp, _i, _vp, _i]),

@@ -189,6 +189,20 @@ bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_
 int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
                          const float *d_x_f32, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
                          void *d_out0, void *d_out1, int out_dtype);
+// Up to three weights of one shape [M, K] and one quant kind that share the activations: a single matmul, the
+// gate/up pair, the q/k/v triple. One launch streams all of them (the weight index is a grid dimension).
+struct WeightSet {
+    int count = 1;
+    const void *w[3] = {nullptr, nullptr, nullptr};
+    const void *bias[3] = {nullptr, nullptr, nullptr};  // per weight, nullptr = none
+    void *out[3] = {nullptr, nullptr, nullptr};
+    int bias_dtype = 0;
+    // fp16 output only. false: f16(f16(dot) + bias), the matmul epilogue adds the bias to the stored value;
+    // true: f16(dot + bias), the q/k/v projection starts its fp32 accumulator from the bias (matmul_qkv.c:889-915).
+    bool bias_first = false;
+};
+int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch *act,
+                      const float *d_x_f32, size_t N, size_t K, size_t M, int out_dtype);
 // quantizes act(gate) * up (SwiGLU or GeGLU) of two fp32 [rows, k] arrays into the activation scratch
 int launch_quantize_glu_soa(marmot_hip_device *dev, int act_kind, const float *d_gate, const float *d_up, bool geglu,
                             size_t rows, size_t k, const ActScratch &dst);
@@ -199,17 +213,19 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 // small-batch int8-MFMA matmul (mh_mmq.hip)
 bool mmq_supported(int kind, size_t N, size_t K);
-size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, bool dual);
+size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int weights);
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);
+int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
+                   size_t M, int out_dtype, void *scratch);
 bool mmq_grouped_supported(int kind, size_t K);
 int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
                        const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
                        size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1);
 // sums fp32 partials [splits][N][M] in split order, then bias and output cast (mh_gemm.hip)
 int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
-                         const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
+                         const void *d_bias, int bias_dtype, void *d_out, int out_dtype, bool bias_first = false);
 bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M);
 int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                     const void *d_bias, int bias_dtype, void *d_out, int out_dtype);

@@ -432,8 +432,9 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
 // sums the K-split partials in split order, then bias / output cast like the single-pass epilogue
 template <int V>
 __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ partial, int splits, size_t N, size_t M,
-                                                     const void *bias, int bias_is_f16, void *out, int out_is_f16) {
-    warm_kernel_arguments<8 * 8>();
+                                                     const void *bias, int bias_is_f16, void *out, int out_is_f16,
+                                                     int bias_first) {
+    warm_kernel_arguments<8 * 8 + 4>();
     const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
     const size_t total = N * M;
     if (idx >= total) {
@@ -470,16 +471,17 @@ __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ p
 #pragma unroll
     for (int e = 0; e < V; ++e) {
         const size_t m = (idx + e) % M;
+        float bv = 0.0f;
+        if (bias != nullptr) {
+            bv = bias_is_f16 ? h2f(((const uint16_t *)bias)[m]) : ((const float *)bias)[m];
+        }
         if (!out_is_f16) {
-            float r = v[e];
-            if (bias != nullptr) {
-                r += ((const float *)bias)[m];
-            }
-            ((float *)out)[idx + e] = r;
+            ((float *)out)[idx + e] = bias != nullptr ? v[e] + bv : v[e];
+        } else if (bias_first) {
+            ((uint16_t *)out)[idx + e] = f2h(bias != nullptr ? v[e] + bv : v[e]);
         } else {
             uint16_t h = f2h(v[e]);
             if (bias != nullptr) {
-                const float bv = bias_is_f16 ? h2f(((const uint16_t *)bias)[m]) : ((const float *)bias)[m];
                 h = f2h(h2f(h) + bv);
             }
             ((uint16_t *)out)[idx + e] = h;
@@ -488,7 +490,7 @@ __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ p
 }
 
 int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
-                         const void *d_bias, int bias_dtype, void *d_out, int out_dtype) {
+                         const void *d_bias, int bias_dtype, void *d_out, int out_dtype, bool bias_first) {
     const size_t total = N * M;
     const int bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16, out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
     // small outputs: one wavefront per workgroup, so that the few thousand threads spread over the whole chip
@@ -498,10 +500,10 @@ int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int split
     const dim3 grid((unsigned)((threads + block - 1) / block));
     if (vec) {
         hipLaunchKernelGGL(k_gemm_reduce<4>, grid, dim3(block), 0, dev->stream, partial, splits, N, M, d_bias,
-                           bias_is_f16, d_out, out_is_f16);
+                           bias_is_f16, d_out, out_is_f16, bias_first ? 1 : 0);
     } else {
         hipLaunchKernelGGL(k_gemm_reduce<1>, grid, dim3(block), 0, dev->stream, partial, splits, N, M, d_bias,
-                           bias_is_f16, d_out, out_is_f16);
+                           bias_is_f16, d_out, out_is_f16, bias_first ? 1 : 0);
     }
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;

@@ -215,7 +215,7 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
-    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr) : 0);
+    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr ? 2 : 1) : 0);
     void *ws = nullptr;
     int st = workspace_reserve(dev, need, &ws);
     if (st != MARMOT_HIP_SUCCESS) {
@@ -322,6 +322,76 @@ int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const v
     }
     return matmul_impl(dev, kind, d_weight_a, d_weight_b, d_input, in_dtype, N, K, M, nullptr, 0, d_out_a, d_out_b,
                        out_dtype, flags);
+}
+
+int marmot_hip_matmul_qkv_quantized(marmot_hip_device_t *dev, int kind, const void *d_wq, const void *d_wk,
+                                    const void *d_wv, const void *d_input, int in_dtype, size_t N, size_t K, size_t M,
+                                    const void *d_bq, const void *d_bk, const void *d_bv, int bias_dtype,
+                                    void *d_out_q, void *d_out_k, void *d_out_v, int out_dtype) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
+    }
+    if (d_wq == nullptr || d_wk == nullptr || d_wv == nullptr || d_input == nullptr || d_out_q == nullptr ||
+        d_out_k == nullptr || d_out_v == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
+    }
+    if (kind != MARMOT_HIP_KIND_Q4_0 && kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_K &&
+        kind != MARMOT_HIP_KIND_Q6_K) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "QKV projection kernel not available for quant kind %d",
+                         kind);
+    }
+    if (in_dtype != MARMOT_HIP_DTYPE_F32 && in_dtype != MARMOT_HIP_DTYPE_F16) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "QKV projection requires FLOAT32 or FLOAT16 activations");
+    }
+    if (out_dtype != in_dtype) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "QKV projection outputs must have the input dtype");
+    }
+    const bool any_bias = d_bq != nullptr || d_bk != nullptr || d_bv != nullptr;
+    if (any_bias && bias_dtype != MARMOT_HIP_DTYPE_F32 && bias_dtype != MARMOT_HIP_DTYPE_F16) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "QKV projection bias must be FLOAT32 or FLOAT16");
+    }
+    if (K == 0 || M == 0) {
+        return set_error(MARMOT_HIP_ERROR_DIMENSION_MISMATCH, "QKV projection dimension mismatch on K");
+    }
+    if (N == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    MH_HIP(hipSetDevice(dev->device_index));
+    WeightSet ws;
+    ws.count = 3;
+    ws.w[0] = d_wq;
+    ws.w[1] = d_wk;
+    ws.w[2] = d_wv;
+    ws.bias[0] = d_bq;
+    ws.bias[1] = d_bk;
+    ws.bias[2] = d_bv;
+    ws.out[0] = d_out_q;
+    ws.out[1] = d_out_k;
+    ws.out[2] = d_out_v;
+    ws.bias_dtype = bias_dtype;
+    ws.bias_first = true;
+    const bool mmq = mmq_supported(kind, N, K);
+    if (!mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input)) {
+        return launch_matvec_set(dev, kind, ws, nullptr, (const float *)d_input, N, K, M, out_dtype);
+    }
+    const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+    const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
+    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, 3) : 0);
+    void *wsp = nullptr;
+    int st = workspace_reserve(dev, need, &wsp);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    ActScratch act;
+    act_scratch_layout(act_kind, N, K, wsp, &act);
+    st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    if (mmq) {
+        return launch_mmq_set(dev, kind, ws, act, N, K, M, out_dtype, (uint8_t *)wsp + act_bytes);
+    }
+    return launch_matvec_set(dev, kind, ws, &act, nullptr, N, K, M, out_dtype);
 }
 
 } // extern "C"

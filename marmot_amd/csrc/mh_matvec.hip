@@ -461,13 +461,14 @@ struct FmtQ40 {
 };
 
 struct MatvecParams {
-    const uint8_t *w[2];
-    void *out[2];
+    const uint8_t *w[3];  // weights of one shape sharing the activations; blockIdx.y selects one
+    void *out[3];
     ActView act;       // packed activations (prepacked variant)
     const float *x;    // fp32 activations [N][K] (fused variant)
     size_t K;
-    const void *bias;
+    const void *bias[3];
     int bias_is_f16;
+    int bias_first;    // fp16 output: f16(dot + bias) instead of f16(f16(dot) + bias)
     int out_is_f16;
     size_t n0;         // first activation row of this column tile
     size_t M;
@@ -481,18 +482,23 @@ struct MatvecParams {
     size_t expert_stride;         // bytes between the experts' weight slices
 };
 
-__device__ __forceinline__ void store_out(const MatvecParams &p, void *out, size_t n, size_t row, float v) {
+__device__ __forceinline__ void store_out(const MatvecParams &p, int which, size_t n, size_t row, float v) {
     const size_t idx = n * p.M + row;
+    void *out = p.out[which];
+    const void *bias = p.bias[which];
+    float b = 0.0f;
+    if (bias != nullptr) {
+        b = p.bias_is_f16 ? h2f(((const uint16_t *)bias)[row]) : ((const float *)bias)[row];
+    }
     if (!p.out_is_f16) {
-        if (p.bias != nullptr) {
-            v += ((const float *)p.bias)[row];
-        }
-        ((float *)out)[idx] = v;
+        ((float *)out)[idx] = bias != nullptr ? v + b : v;
+    } else if (p.bias_first) {
+        // q/k/v projection: the fp32 accumulator starts from the bias, one rounding at the store
+        ((uint16_t *)out)[idx] = f2h(bias != nullptr ? v + b : v);
     } else {
-        // reference order: store f16(dot), then the epilogue adds the bias to the stored f16 value
+        // matmul: store f16(dot), then the epilogue adds the bias to the stored f16 value
         uint16_t h = f2h(v);
-        if (p.bias != nullptr) {
-            const float b = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[row]) : ((const float *)p.bias)[row];
+        if (bias != nullptr) {
             h = f2h(h2f(h) + b);
         }
         ((uint16_t *)out)[idx] = h;
@@ -615,7 +621,6 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
         }
     }
     __syncthreads();
-    void *out = p.out[blockIdx.y];
     for (int idx = threadIdx.x; idx < p.rows_per_wg * NC; idx += blockDim.x) {
         const size_t row = row0 + idx / NC;
         const int n = idx % NC;
@@ -633,7 +638,7 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
                 const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
                 s += w < W ? t : 0.0f;
             }
-            store_out(p, out, n0 + n, row, s);
+            store_out(p, (int)blockIdx.y, n0 + n, row, s);
         }
     }
 }
@@ -792,7 +797,6 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
         __builtin_amdgcn_s_waitcnt(0xc07f);
         __builtin_amdgcn_s_barrier();  // final barrier: partial sums complete
     }
-    void *out = p.out[blockIdx.y];
     for (int idx = threadIdx.x; idx < rows * NC; idx += blockDim.x) {
         const size_t row = row0 + idx / NC;
         const int n = idx % NC;
@@ -810,7 +814,7 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
                 const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
                 sum += w < W ? t : 0.0f;
             }
-            store_out(p, out, n0 + n, row, sum);
+            store_out(p, (int)blockIdx.y, n0 + n, row, sum);
         }
     }
 }
@@ -821,13 +825,13 @@ static bool matvec_ls_usable(const MatvecParams &p, size_t K, int C) {
     const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
     const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
     return p.items == nullptr && K % Fmt::BV == 0 && p.row_bytes % 16 == 0 && (((uintptr_t)p.w[0]) & 15) == 0 &&
-           (((uintptr_t)p.w[1]) & 15) == 0 && wave_loads <= (size_t)(matvec_ls_max_consumers<Fmt>() * C) &&
+           (((uintptr_t)p.w[1]) & 15) == 0 && (((uintptr_t)p.w[2]) & 15) == 0 && wave_loads <= (size_t)(matvec_ls_max_consumers<Fmt>() * C) &&
            getenv("MH_MV_NO_LS") == nullptr;
 }
 
 template <class Fmt, int NC, int C, int R, bool FUSED>
-static int launch_ls(marmot_hip_device *dev, MatvecParams p, int W, size_t M, bool dual) {
-    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1, 1);
+static int launch_ls(marmot_hip_device *dev, MatvecParams p, int W, size_t M, int nw) {
+    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), nw, 1);
     const size_t part = (((size_t)p.rows_per_wg * NC * 4 * W * sizeof(float)) + 15) & ~(size_t)15;
     const size_t stage_stride = ((size_t)R * p.row_bytes + 1023) & ~(size_t)1023;
     const size_t lds = part + MV_LS_STAGES * stage_stride;
@@ -843,8 +847,8 @@ static int launch_ls(marmot_hip_device *dev, MatvecParams p, int W, size_t M, bo
 }
 
 template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
-static int launch_one(marmot_hip_device *dev, const MatvecParams &p, int W, size_t M, bool dual) {
-    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), dual ? 2 : 1,
+static int launch_one(marmot_hip_device *dev, const MatvecParams &p, int W, size_t M, int nw) {
+    const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), nw,
                     p.items != nullptr ? (unsigned)p.n0 : 1u);  // grouped mode: n0 carries the item-count bound
     const size_t lds = (size_t)p.rows_per_wg * NC * 4 * W * sizeof(float);
     hipLaunchKernelGGL((k_matvec<Fmt, NC, C, R, FUSED, EXACT>), grid, dim3(W * 64), lds, dev->stream, p);
@@ -855,7 +859,7 @@ static int launch_one(marmot_hip_device *dev, const MatvecParams &p, int W, size
 // Picks wavefronts per workgroup (W), wave-loads per wavefront (C) and rows per workgroup for one column tile.
 // Returns MARMOT_HIP_ERROR_NOT_IMPLEMENTED (without setting the error text) when K is too long for this NC.
 template <class Fmt, int NC, int R>
-static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, bool dual, const char *name) {
+static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, int nw, const char *name) {
     const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
     const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
     const bool fused = p.x != nullptr;
@@ -921,50 +925,50 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
             }
             p.rows_per_wg = (int)rows_ls;
             if (C == 1) {
-                return fused ? launch_ls<Fmt, NC, 1, 2, true>(dev, p, W, M, dual)
-                             : launch_ls<Fmt, NC, 1, 2, false>(dev, p, W, M, dual);
+                return fused ? launch_ls<Fmt, NC, 1, 2, true>(dev, p, W, M, nw)
+                             : launch_ls<Fmt, NC, 1, 2, false>(dev, p, W, M, nw);
             }
-            return fused ? launch_ls<Fmt, NC, 2, 2, true>(dev, p, W, M, dual)
-                         : launch_ls<Fmt, NC, 2, 2, false>(dev, p, W, M, dual);
+            return fused ? launch_ls<Fmt, NC, 2, 2, true>(dev, p, W, M, nw)
+                         : launch_ls<Fmt, NC, 2, 2, false>(dev, p, W, M, nw);
         }
     }
     const bool exact = (size_t)W * C * Fmt::BPW == nb && K % Fmt::BV == 0 && M % rows_per_wg == 0;
     if constexpr (NC <= 4) {
         if (fused) {
             if (C == 1) {
-                return exact ? launch_one<Fmt, NC, 1, R, true, true>(dev, p, W, M, dual)
-                             : launch_one<Fmt, NC, 1, R, true, false>(dev, p, W, M, dual);
+                return exact ? launch_one<Fmt, NC, 1, R, true, true>(dev, p, W, M, nw)
+                             : launch_one<Fmt, NC, 1, R, true, false>(dev, p, W, M, nw);
             }
-            return launch_one<Fmt, NC, 2, R, true, false>(dev, p, W, M, dual);
+            return launch_one<Fmt, NC, 2, R, true, false>(dev, p, W, M, nw);
         }
     } else if (fused) {
         return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "fused activation quantization is limited to 4 columns");
     }
     if (C == 1) {
-        return launch_one<Fmt, NC, 1, R, false, false>(dev, p, W, M, dual);
+        return launch_one<Fmt, NC, 1, R, false, false>(dev, p, W, M, nw);
     }
-    return launch_one<Fmt, NC, 2, R, false, false>(dev, p, W, M, dual);
+    return launch_one<Fmt, NC, 2, R, false, false>(dev, p, W, M, nw);
 }
 
 template <class Fmt, int NC>
-static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, bool dual, const char *name) {
+static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, int nw, const char *name) {
     if constexpr (NC == 1) {
         const char *e = getenv("MH_R");
         const int r = e ? atoi(e) : 4;
         if (r == 8) {
-            return launch_tile_r<Fmt, NC, 8>(dev, p, K, M, dual, name);
+            return launch_tile_r<Fmt, NC, 8>(dev, p, K, M, nw, name);
         }
         if (r == 2) {
-            return launch_tile_r<Fmt, NC, 2>(dev, p, K, M, dual, name);
+            return launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name);
         }
-        return launch_tile_r<Fmt, NC, 4>(dev, p, K, M, dual, name);
+        return launch_tile_r<Fmt, NC, 4>(dev, p, K, M, nw, name);
     } else {
-        return launch_tile_r < Fmt, NC, (NC <= 2) ? 4 : 2 > (dev, p, K, M, dual, name);
+        return launch_tile_r < Fmt, NC, (NC <= 2) ? 4 : 2 > (dev, p, K, M, nw, name);
     }
 }
 
 template <class Fmt>
-static int launch_fmt(marmot_hip_device *dev, MatvecParams p, size_t N, size_t K, size_t M, bool dual,
+static int launch_fmt(marmot_hip_device *dev, MatvecParams p, size_t N, size_t K, size_t M, int nw,
                       const char *name) {
     // Column tiles of up to 8 activation rows; each tile streams the weights once. A tile width whose
     // register budget cannot cover K in one pass falls back to the next narrower one.
@@ -976,28 +980,28 @@ static int launch_fmt(marmot_hip_device *dev, MatvecParams p, size_t N, size_t K
         int st = MARMOT_HIP_ERROR_NOT_IMPLEMENTED;
         size_t step = 0;
         if (left >= 8 && cap >= 8) {
-            st = launch_tile<Fmt, 8>(dev, p, K, M, dual, name);
+            st = launch_tile<Fmt, 8>(dev, p, K, M, nw, name);
             step = 8;
             if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
                 cap = 4;
             }
         }
         if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED && left >= 4 && cap >= 4) {
-            st = launch_tile<Fmt, 4>(dev, p, K, M, dual, name);
+            st = launch_tile<Fmt, 4>(dev, p, K, M, nw, name);
             step = 4;
             if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
                 cap = 2;
             }
         }
         if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED && left >= 2 && cap >= 2) {
-            st = launch_tile<Fmt, 2>(dev, p, K, M, dual, name);
+            st = launch_tile<Fmt, 2>(dev, p, K, M, nw, name);
             step = 2;
             if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
                 cap = 1;
             }
         }
         if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
-            st = launch_tile<Fmt, 1>(dev, p, K, M, dual, name);
+            st = launch_tile<Fmt, 1>(dev, p, K, M, nw, name);
             step = 1;
             if (st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
                 return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED,
@@ -1020,16 +1024,32 @@ bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_
 int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
                          const float *d_x_f32, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
                          void *d_out0, void *d_out1, int out_dtype) {
+    WeightSet ws;
+    ws.count = d_w1 != nullptr ? 2 : 1;
+    ws.w[0] = d_w0;
+    ws.w[1] = d_w1;
+    ws.out[0] = d_out0;
+    ws.out[1] = d_out1;
+    ws.bias[0] = d_bias;
+    ws.bias[1] = d_bias;
+    ws.bias_dtype = bias_dtype;
+    return launch_matvec_set(dev, kind, ws, act, d_x_f32, N, K, M, out_dtype);
+}
+
+int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch *act,
+                      const float *d_x_f32, size_t N, size_t K, size_t M, int out_dtype) {
     if (N == 0 || M == 0 || K == 0) {
         return MARMOT_HIP_SUCCESS;
     }
     const size_t bv = block_values(kind);
     const size_t nb = (K + bv - 1) / bv;
     MatvecParams p;
-    p.w[0] = (const uint8_t *)d_w0;
-    p.w[1] = (const uint8_t *)(d_w1 != nullptr ? d_w1 : d_w0);
-    p.out[0] = d_out0;
-    p.out[1] = d_out1 != nullptr ? d_out1 : d_out0;
+    for (int i = 0; i < 3; ++i) {  // unused slots repeat weight 0 (the alignment checks look at all three)
+        const int src = i < ws.count ? i : 0;
+        p.w[i] = (const uint8_t *)ws.w[src];
+        p.out[i] = ws.out[src];
+        p.bias[i] = ws.bias[src];
+    }
     if (act != nullptr) {
         p.act.qs = act->qs;
         p.act.d = act->d;
@@ -1046,8 +1066,8 @@ int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, con
         p.x = d_x_f32;
     }
     p.K = K;
-    p.bias = d_bias;
-    p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
+    p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
+    p.bias_first = ws.bias_first ? 1 : 0;
     p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
     p.n0 = 0;
     p.M = M;
@@ -1058,17 +1078,17 @@ int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, con
     p.n_items = nullptr;
     p.act_index = nullptr;
     p.expert_stride = 0;
-    const bool dual = d_w1 != nullptr;
+    const int nw = ws.count;
     const bool fused = act == nullptr;
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
-        return launch_fmt<FmtQ4K>(dev, p, N, K, M, dual, fused ? "matvec_q4_k_q8_k_fused" : "matvec_q4_k_q8_k");
+        return launch_fmt<FmtQ4K>(dev, p, N, K, M, nw, fused ? "matvec_q4_k_q8_k_fused" : "matvec_q4_k_q8_k");
     case MARMOT_HIP_KIND_Q6_K:
-        return launch_fmt<FmtQ6K>(dev, p, N, K, M, dual, fused ? "matvec_q6_k_q8_k_fused" : "matvec_q6_k_q8_k");
+        return launch_fmt<FmtQ6K>(dev, p, N, K, M, nw, fused ? "matvec_q6_k_q8_k_fused" : "matvec_q6_k_q8_k");
     case MARMOT_HIP_KIND_Q8_0:
-        return launch_fmt<FmtQ80>(dev, p, N, K, M, dual, fused ? "matvec_q8_0_q8_0_fused" : "matvec_q8_0_q8_0");
+        return launch_fmt<FmtQ80>(dev, p, N, K, M, nw, fused ? "matvec_q8_0_q8_0_fused" : "matvec_q8_0_q8_0");
     case MARMOT_HIP_KIND_Q4_0:
-        return launch_fmt<FmtQ40>(dev, p, N, K, M, dual, fused ? "matvec_q4_0_q8_0_fused" : "matvec_q4_0_q8_0");
+        return launch_fmt<FmtQ40>(dev, p, N, K, M, nw, fused ? "matvec_q4_0_q8_0_fused" : "matvec_q4_0_q8_0");
     default:
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "quantized matmul: unsupported quant kind %d", kind);
     }
@@ -1086,8 +1106,10 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
     MatvecParams p;
     p.w[0] = (const uint8_t *)d_w0;
     p.w[1] = (const uint8_t *)(d_w1 != nullptr ? d_w1 : d_w0);
+    p.w[2] = p.w[0];
     p.out[0] = d_out0;
     p.out[1] = d_out1 != nullptr ? d_out1 : d_out0;
+    p.out[2] = p.out[0];
     p.act.qs = act.qs;
     p.act.d = act.d;
     p.act.sums = act.sums;
@@ -1095,8 +1117,9 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
     p.act.nb = act.nb;
     p.x = nullptr;
     p.K = K;
-    p.bias = nullptr;
+    p.bias[0] = p.bias[1] = p.bias[2] = nullptr;
     p.bias_is_f16 = 0;
+    p.bias_first = 0;
     p.out_is_f16 = 0;
     p.n0 = max_items;
     p.M = M;
@@ -1107,20 +1130,20 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
     p.n_items = d_n_items;
     p.act_index = d_act_index;
     p.expert_stride = expert_stride;
-    const bool dual = d_w1 != nullptr;
+    const int nw = d_w1 != nullptr ? 2 : 1;
     int st;
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
-        st = launch_tile<FmtQ4K, 8>(dev, p, K, M, dual, "moe_grouped_q4_k_q8_k");
+        st = launch_tile<FmtQ4K, 8>(dev, p, K, M, nw, "moe_grouped_q4_k_q8_k");
         break;
     case MARMOT_HIP_KIND_Q6_K:
-        st = launch_tile<FmtQ6K, 8>(dev, p, K, M, dual, "moe_grouped_q6_k_q8_k");
+        st = launch_tile<FmtQ6K, 8>(dev, p, K, M, nw, "moe_grouped_q6_k_q8_k");
         break;
     case MARMOT_HIP_KIND_Q8_0:
-        st = launch_tile<FmtQ80, 8>(dev, p, K, M, dual, "moe_grouped_q8_0_q8_0");
+        st = launch_tile<FmtQ80, 8>(dev, p, K, M, nw, "moe_grouped_q8_0_q8_0");
         break;
     case MARMOT_HIP_KIND_Q4_0:
-        st = launch_tile<FmtQ40, 8>(dev, p, K, M, dual, "moe_grouped_q4_0_q8_0");
+        st = launch_tile<FmtQ40, 8>(dev, p, K, M, nw, "moe_grouped_q4_0_q8_0");
         break;
     default:
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "MoE experts: unsupported quant kind %d", kind);

@@ -25,8 +25,9 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
 struct MmqParams {
-    const uint8_t *w[2];   // Q4_K blocks, M rows of nb blocks (second weight of a dual call or nullptr)
-    void *out[2];          // [N][M] of out dtype, or fp32 partials [splits][N][M] when splits > 1
+    const uint8_t *w[3];   // blocks, M rows of nb blocks: nw weights of one shape sharing the activations
+    void *out[3];          // [N][M] of out dtype, or fp32 partials [splits][N][M] when splits > 1
+    int nw;                // weights in this launch: blockIdx.y = split * nw + weight
     const int8_t *qs;      // quantized activations, rows of kp bytes
     const float *ad;       // activation block scales [rows][nb]
     size_t kp;
@@ -35,8 +36,9 @@ struct MmqParams {
     int ncols;             // activation rows of this pass (<= 32)
     int bpw;               // blocks per wavefront
     int splits;            // workgroups along K
-    const void *bias;
+    const void *bias[3];
     int bias_is_f16;
+    int bias_first;        // fp16 output: f16(dot + bias) instead of f16(f16(dot) + bias)
     int out_is_f16;
     // grouped (MoE) mode: blockIdx.z selects a work item = up to 8 consecutive routes of one expert
     const int4 *items;
@@ -104,10 +106,11 @@ __device__ __forceinline__ void mmq_store(const MmqParams &p, int which, int spl
     void *out = p.out[which];
     // The bias of this weight row is fetched once, before the stores: a load (and the wait for it) between two stores
     // would also wait for the earlier store, the memory counter being in order.
-    const bool has_bias = p.splits == 1 && p.bias != nullptr;
+    const void *bias = p.bias[which];
+    const bool has_bias = p.splits == 1 && bias != nullptr;
     float bv = 0.0f;
     if (has_bias) {
-        bv = (p.out_is_f16 && p.bias_is_f16) ? h2f(((const uint16_t *)p.bias)[mm]) : ((const float *)p.bias)[mm];
+        bv = p.bias_is_f16 ? h2f(((const uint16_t *)bias)[mm]) : ((const float *)bias)[mm];
     }
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
@@ -119,6 +122,8 @@ __device__ __forceinline__ void mmq_store(const MmqParams &p, int which, int spl
             ((float *)out)[((size_t)split * p.N + n) * p.M + mm] = acc[r];
         } else if (!p.out_is_f16) {
             ((float *)out)[n * p.M + mm] = has_bias ? acc[r] + bv : acc[r];
+        } else if (p.bias_first) {
+            ((uint16_t *)out)[n * p.M + mm] = f2h(has_bias ? acc[r] + bv : acc[r]);
         } else {
             uint16_t h = f2h(acc[r]);
             if (has_bias) {
@@ -159,8 +164,8 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
     const bool loader = wave == W;
     warm_kernel_arguments<sizeof(MmqParams)>();
     const int j = lane & 31, kh = lane >> 5;
-    const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
-    const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
+    const int split = (int)blockIdx.y / p.nw;
+    const int which = (int)blockIdx.y - split * p.nw;
     const uint8_t *wbase = p.w[which];
     size_t n0 = p.n0;
     int ncols = p.ncols;
@@ -377,8 +382,8 @@ __global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
     warm_kernel_arguments<sizeof(MmqParams)>();
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
     const int j = lane & 31, kh = lane >> 5;
-    const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
-    const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
+    const int split = (int)blockIdx.y / p.nw;
+    const int which = (int)blockIdx.y - split * p.nw;
     const uint8_t *wbase = p.w[which];
     size_t n0 = p.n0;
     int ncols = p.ncols;
@@ -595,8 +600,8 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
     const bool loader = wave == W;
     const int j = lane & 31, kh = lane >> 5;
-    const int which = (p.w[1] != nullptr) ? (int)(blockIdx.y & 1) : 0;
-    const int split = (p.w[1] != nullptr) ? (int)(blockIdx.y >> 1) : (int)blockIdx.y;
+    const int split = (int)blockIdx.y / p.nw;
+    const int which = (int)blockIdx.y - split * p.nw;
     const uint8_t *wbase = p.w[which];
     size_t n0 = p.n0;
     int ncols = p.ncols;
@@ -853,9 +858,9 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t
 }
 
 // bytes of fp32 partials launch_mmq needs for this shape (0 when K is not split across workgroups)
-size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, bool dual) {
+size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int weights) {
     const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K);
-    return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (dual ? 2 : 1) : 0;
+    return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (size_t)weights : 0;
 }
 
 static size_t mmq6_lds_bytes(int W) {
@@ -865,9 +870,9 @@ static size_t mmq6_lds_bytes(int W) {
 }
 
 template <int NR>
-static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, size_t M, bool dual,
+static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, size_t M,
                       unsigned items) {
-    const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * (dual ? 2 : 1)), items);
+    const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * p.nw), items);
     static bool attr_set = false;
     if (!attr_set) {
         MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -879,7 +884,7 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
         attr_set = true;
     }
     if (kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(p.nb) && pl.W <= 4 && (((uintptr_t)p.w[0]) & 15) == 0 &&
-        (((uintptr_t)p.w[1]) & 15) == 0 && (p.expert_stride & 15) == 0) {
+        (((uintptr_t)p.w[1]) & 15) == 0 && (((uintptr_t)p.w[2]) & 15) == 0 && (p.expert_stride & 15) == 0) {
         const int stages = p.items != nullptr ? 2 : 3;
         const size_t stage = MMQ6_WBLK + 2 * NR * QK_K + 2 * NR * 4;
         const size_t ring = (size_t)pl.W * stages * stage;
@@ -927,26 +932,42 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch) {
+    WeightSet ws;
+    ws.count = d_w1 != nullptr ? 2 : 1;
+    ws.w[0] = d_w0;
+    ws.w[1] = d_w1;
+    ws.out[0] = d_out0;
+    ws.out[1] = d_out1;
+    ws.bias[0] = d_bias;
+    ws.bias[1] = d_bias;
+    ws.bias_dtype = bias_dtype;
+    return launch_mmq_set(dev, kind, ws, act, N, K, M, out_dtype, scratch);
+}
+
+int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
+                   size_t M, int out_dtype, void *scratch) {
     if (!mmq_supported(kind, N, K)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
     }
     const size_t nb = K / QK_K;
-    const bool dual = d_w1 != nullptr;
     const MmqPlan pl = mmq_plan(dev, kind, N, M, nb);
     float *partial = (float *)scratch;
     if (pl.S > 1 && partial == nullptr) {
-        void *ws = nullptr;
-        int st = workspace_reserve(dev, mmq_scratch_bytes(dev, kind, N, K, M, dual), &ws);
+        void *wsp = nullptr;
+        int st = workspace_reserve(dev, mmq_scratch_bytes(dev, kind, N, K, M, ws.count), &wsp);
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
         }
-        partial = (float *)ws;
+        partial = (float *)wsp;
     }
     MmqParams p;
-    p.w[0] = (const uint8_t *)d_w0;
-    p.w[1] = (const uint8_t *)d_w1;
-    p.out[0] = pl.S > 1 ? (void *)partial : d_out0;
-    p.out[1] = pl.S > 1 ? (void *)(partial + (size_t)pl.S * N * M) : d_out1;
+    p.nw = ws.count;
+    for (int i = 0; i < 3; ++i) {  // unused slots repeat weight 0 (the alignment checks look at all three)
+        const int src = i < ws.count ? i : 0;
+        p.w[i] = (const uint8_t *)ws.w[src];
+        p.out[i] = pl.S > 1 ? (void *)(partial + (size_t)src * pl.S * N * M) : ws.out[src];
+        p.bias[i] = ws.bias[src];
+    }
     p.qs = act.qs;
     p.ad = act.d;
     p.kp = act.kp;
@@ -955,8 +976,8 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
     p.nb = nb;
     p.bpw = pl.bpw;
     p.splits = pl.S;
-    p.bias = d_bias;
-    p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
+    p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
+    p.bias_first = ws.bias_first ? 1 : 0;
     p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
     p.items = nullptr;
     p.n_items = nullptr;
@@ -968,15 +989,15 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
         p.n0 = n0;
         p.ncols = (int)(N - n0 < MMQ_ROWS_PER_PASS ? N - n0 : MMQ_ROWS_PER_PASS);
         const int st =
-            p.ncols <= 8 ? mmq_launch<4>(dev, kind, p, pl, M, dual, 1) : mmq_launch<8>(dev, kind, p, pl, M, dual, 1);
+            p.ncols <= 8 ? mmq_launch<4>(dev, kind, p, pl, M, 1) : mmq_launch<8>(dev, kind, p, pl, M, 1);
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
         }
     }
     if (pl.S > 1) {
-        for (int which = 0; which < (dual ? 2 : 1); ++which) {
-            int st = launch_splitk_reduce(dev, partial + (size_t)which * pl.S * N * M, pl.S, N, M, d_bias, bias_dtype,
-                                          which ? d_out1 : d_out0, out_dtype);
+        for (int which = 0; which < ws.count; ++which) {
+            int st = launch_splitk_reduce(dev, partial + (size_t)which * pl.S * N * M, pl.S, N, M, ws.bias[which],
+                                          ws.bias_dtype, ws.out[which], out_dtype, ws.bias_first);
             if (st != MARMOT_HIP_SUCCESS) {
                 return st;
             }
@@ -1014,10 +1035,13 @@ int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const
     pl.S = 1;
     pl.bpw = (int)nb;
     MmqParams p;
+    p.nw = d_w1 != nullptr ? 2 : 1;
     p.w[0] = (const uint8_t *)d_w0;
-    p.w[1] = (const uint8_t *)d_w1;
+    p.w[1] = (const uint8_t *)(d_w1 != nullptr ? d_w1 : d_w0);
+    p.w[2] = p.w[0];
     p.out[0] = d_out0;
-    p.out[1] = d_out1;
+    p.out[1] = d_out1 != nullptr ? d_out1 : d_out0;
+    p.out[2] = p.out[0];
     p.qs = act.qs;
     p.ad = act.d;
     p.kp = act.kp;
@@ -1028,14 +1052,15 @@ int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const
     p.ncols = 0;
     p.bpw = pl.bpw;
     p.splits = 1;
-    p.bias = nullptr;
+    p.bias[0] = p.bias[1] = p.bias[2] = nullptr;
     p.bias_is_f16 = 0;
+    p.bias_first = 0;
     p.out_is_f16 = 0;
     p.items = d_items;
     p.n_items = d_n_items;
     p.act_index = d_act_index;
     p.expert_stride = expert_stride;
-    const int st = mmq_launch<4>(dev, kind, p, pl, M, d_w1 != nullptr, (unsigned)max_items);
+    const int st = mmq_launch<4>(dev, kind, p, pl, M, (unsigned)max_items);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }

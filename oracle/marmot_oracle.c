@@ -1283,6 +1283,64 @@ int mo_matmul_quantized(
     return MO_OK;
 }
 
+/* matmul_qkv.c:749-947 (cpu_matmul_qkv_run_separate_quantized_impl), value load/store helpers :89-116 */
+int mo_matmul_qkv_separate(
+    int kind, const void *const weights[3], const void *input, int in_dtype, size_t N, size_t K, size_t M,
+    const void *const bias[3], int bias_dtype, void *const out[3]
+) {
+    if (weights == NULL || input == NULL || out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (weights[i] == NULL || out[i] == NULL) {
+            return MO_ERR_INVALID_ARGUMENT;
+        }
+    }
+    if (in_dtype != MO_DTYPE_F32 && in_dtype != MO_DTYPE_F16) {
+        return MO_ERR_NOT_IMPLEMENTED; /* :761-763 */
+    }
+    dot_fn dot = pick_dot(kind);
+    if (dot == NULL) {
+        return MO_ERR_NOT_IMPLEMENTED;
+    }
+    const size_t bv = mo_block_values(kind);
+    const size_t bb = mo_block_bytes(kind);
+    const size_t blocks_per_row = (K + bv - 1) / bv; /* :802 */
+    const size_t row_bytes = bb * blocks_per_row;
+    const int use_q8_k = (bv == QK_K);
+    const size_t act_bb = use_q8_k ? sizeof(blk_q8_k) : sizeof(blk_q8_0);
+    uint8_t *act = (uint8_t *)malloc(blocks_per_row * act_bb + 1);
+    if (act == NULL) {
+        return MO_ERR_OUT_OF_MEMORY;
+    }
+    const size_t in_elt = in_dtype == MO_DTYPE_F16 ? 2 : 4;
+    for (size_t n = 0; n < N; ++n) { /* :876 */
+        const uint8_t *row = (const uint8_t *)input + n * K * in_elt;
+        if (use_q8_k) {
+            mo_pack_q8_k(row, in_dtype, K, act);
+        } else {
+            mo_pack_q8_0(row, in_dtype, K, act);
+        }
+        for (size_t m = 0; m < M; ++m) { /* :888 */
+            for (int i = 0; i < 3; ++i) {
+                float acc = 0.0f; /* :889-891: the accumulator starts from the bias */
+                if (bias != NULL && bias[i] != NULL) {
+                    acc = bias_dtype == MO_DTYPE_F16 ? mo_f16_to_f32(((const uint16_t *)bias[i])[m])
+                                                     : ((const float *)bias[i])[m];
+                }
+                acc += dot((const uint8_t *)weights[i] + m * row_bytes, act, blocks_per_row); /* :902-914 */
+                if (in_dtype == MO_DTYPE_F16) {
+                    ((uint16_t *)out[i])[n * M + m] = mo_f32_to_f16(acc); /* :107-109 */
+                } else {
+                    ((float *)out[i])[n * M + m] = acc;
+                }
+            }
+        }
+    }
+    free(act);
+    return MO_OK;
+}
+
 /* ======================= top-k / router / MoE ======================= */
 
 /* moe_ops.c:789-889 */

@@ -99,6 +99,19 @@ int mo_matmul_quantized(
     void *out, int out_dtype, int force_pack, int threads
 );
 
+/*
+ * marmot_matmul_qkv, separate block-quantized weights (src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:749-947):
+ * three weights of one kind and shape [M,K], one input [N,K] of in_dtype (F32 or F16), outputs [N,M] of the same
+ * dtype. Per input row the activations are packed once (Q8_0 or Q8_K, also for F16 input), then for every m
+ * acc = (float)bias[m] + dot(w_row, act, all blocks of the row) and the store rounds once to the output dtype.
+ * wq/wk/wv weights; bias[i]: NULL or M values of bias_dtype (F32 or F16); out[i]: N*M values of in_dtype.
+ * The rotary epilogue (rope_params) is not restated.
+ */
+int mo_matmul_qkv_separate(
+    int kind, const void *const weights[3], const void *input, int in_dtype, size_t N, size_t K, size_t M,
+    const void *const bias[3], int bias_dtype, void *const out[3]
+);
+
 /* top-k over the last axis, ties -> lower index (moe_ops.c:789-889) */
 int mo_topk(const float *x, size_t rows, size_t cols, size_t k, float *values_out, int32_t *indices_out);
 

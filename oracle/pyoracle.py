@@ -69,6 +69,11 @@ class Oracle:
             C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
             C.c_int, C.c_int, C.c_int,
         ]
+        L.mo_matmul_qkv_separate.restype = C.c_int
+        L.mo_matmul_qkv_separate.argtypes = [
+            C.c_int, C.POINTER(C.c_void_p), C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t,
+            C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_void_p),
+        ]
         L.mo_topk.restype = C.c_int
         L.mo_topk.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
         L.mo_softmax_rows.restype = None
@@ -170,6 +175,30 @@ class Oracle:
         if st != 0:
             raise RuntimeError(f"mo_matmul_quantized -> {st}")
         return out
+
+    def matmul_qkv(self, kind: int, wq, wk, wv, x: np.ndarray, M: int, bq=None, bk=None, bv=None):
+        """marmot_matmul_qkv with separate quantized weights; returns (q, k, v) of x's dtype (float32 or float16)."""
+        ws = [np.ascontiguousarray(w, dtype=np.uint8) for w in (wq, wk, wv)]
+        if x.dtype != np.float16:
+            x = x.astype(np.float32, copy=False)
+        x = np.ascontiguousarray(x)
+        in_dt = DT_F16 if x.dtype == np.float16 else DT_F32
+        N, K = x.shape
+        for w in ws:
+            assert w.size == M * row_bytes(kind, K), (w.size, M, K)
+        biases = [None if b is None else np.ascontiguousarray(b) for b in (bq, bk, bv)]
+        given = [b for b in biases if b is not None]
+        assert all(b.dtype == given[0].dtype and b.dtype in (np.float32, np.float16) for b in given)
+        bias_dt = DT_F16 if given and given[0].dtype == np.float16 else DT_F32
+        outs = [np.zeros((N, M), dtype=x.dtype) for _ in range(3)]
+        arr = C.c_void_p * 3
+        st = self.L.mo_matmul_qkv_separate(
+            kind, arr(*[w.ctypes.data for w in ws]), _ptr(x), in_dt, N, K, M,
+            arr(*[None if b is None else b.ctypes.data for b in biases]), bias_dt, arr(*[o.ctypes.data for o in outs]),
+        )
+        if st != 0:
+            raise RuntimeError(f"mo_matmul_qkv_separate -> {st}")
+        return tuple(outs)
 
     # ---- MoE
     def topk(self, x: np.ndarray, k: int):

@@ -1,0 +1,94 @@
+"""CPU: the oracle's restatement of marmot_matmul_qkv with separate quantized weights
+(src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:749-947), pinned by
+  * the reference's own test of this op (tests/backend/test_backend_matmul.c:936-1032): the matmul golden weight used
+    for q, k and v, every output equal to the matmul golden (tolerance of the matmul golden test,
+    tests/backend/test_matmul_quantized.c:166-177: the goldens come from another implementation's summation order);
+  * the block dots and packers it is built from, which the vec-dot and quantization goldens pin separately: every
+    output is recomputed here from oracle.pack / oracle.vec_dot with the accumulator started from the bias and ONE
+    rounding at the store, including a float16 case in which the matmul epilogue's order (round, then add the bias)
+    gives different bits."""
+import numpy as np
+import pytest
+
+from oracle.pyoracle import BLOCK_BYTES, BLOCK_VALUES, KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K
+from tests.util import bits, gaussian
+
+
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+def test_reference_qkv_test_case(oracle, ref_goldens, name):
+    kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
+    w = ref_goldens[f"matmul_{name}_weight"]
+    x = ref_goldens[f"matmul_{name}_input_f32"].reshape(N, K)
+    exp = ref_goldens[f"matmul_{name}_expected_f32"].reshape(N, M)
+    for out in oracle.matmul_qkv(kind, w, w, w, x, M):
+        assert out.dtype == np.float32
+        assert np.all(np.abs(out - exp) <= 2e-5 + 5e-5 * np.abs(exp)), np.abs(out - exp).max()
+
+
+def _expected(oracle, kind, weights, x, M, biases):
+    """bias + whole-row block dot, recomputed per element from the pinned leaf functions."""
+    N, K = x.shape
+    act_kind = KIND_Q8_K if BLOCK_VALUES[kind] == 256 else KIND_Q8_0
+    nb = (K + BLOCK_VALUES[kind] - 1) // BLOCK_VALUES[kind]
+    rb = nb * BLOCK_BYTES[kind]
+    outs = [np.zeros((N, M), dtype=np.float32) for _ in range(3)]
+    for n in range(N):
+        act = oracle.pack(act_kind, x[n])
+        for i, (w, b) in enumerate(zip(weights, biases)):
+            w = np.ascontiguousarray(w, dtype=np.uint8).reshape(M, rb)
+            for m in range(M):
+                acc = np.float32(0.0) if b is None else np.float32(b[m])
+                outs[i][n, m] = np.float32(acc + np.float32(oracle.vec_dot(kind, w[m], act, nb)))
+    return outs
+
+
+@pytest.mark.parametrize("kind,K", [(KIND_Q4_K, 70 * 256), (KIND_Q6_K, 512), (KIND_Q8_0, 96), (KIND_Q4_0, 160)])
+def test_qkv_fp32_is_bias_plus_whole_row_dot(oracle, kind, K):
+    """K = 70 blocks: the q/k/v op dots the whole row in one call, it does not chunk K by 64 blocks as the matmul
+    driver does (matmul_qkv.c:902-914 against matmul_quant_compute.c:1032-1112)."""
+    M, N = 6, 3
+    ws = [oracle.quantize(kind, gaussian(500 + i, (M, K), 0.02)) for i in range(3)]
+    x = gaussian(510, (N, K))
+    bq, bv = gaussian(511, (M,)), gaussian(512, (M,)).astype(np.float16)
+    q, k, v = oracle.matmul_qkv(kind, *ws, x, M, bq=bq)
+    eq, ek, ev = _expected(oracle, kind, ws, x, M, [bq, None, None])
+    assert np.array_equal(bits(q), bits(eq)) and np.array_equal(bits(k), bits(ek)) and np.array_equal(bits(v), bits(ev))
+    # float16 bias values are widened exactly before they start the accumulator
+    _, _, v16 = oracle.matmul_qkv(kind, *ws, x, M, bv=bv)
+    _, _, ev16 = _expected(oracle, kind, ws, x, M, [None, None, bv.astype(np.float32)])
+    assert np.array_equal(bits(v16), bits(ev16))
+    # without bias and within one 64-block chunk each projection is the plain quantized matmul
+    if K // BLOCK_VALUES[kind] <= 64:
+        for w, out in zip(ws, oracle.matmul_qkv(kind, *ws, x, M)):
+            assert np.array_equal(bits(out), bits(oracle.matmul(kind, w, x, M)))
+
+
+def test_qkv_fp16_packs_the_activations_and_rounds_once(oracle):
+    kind, M, K, N = KIND_Q4_K, 64, 512, 4
+    ws = [oracle.quantize(kind, gaussian(520 + i, (M, K), 0.02)) for i in range(3)]
+    x = gaussian(523, (N, K)).astype(np.float16)
+    bias = [gaussian(524 + i, (M,)).astype(np.float16) for i in range(3)]
+    outs = oracle.matmul_qkv(kind, *ws, x, M, bq=bias[0], bk=bias[1], bv=bias[2])
+    exp32 = _expected(oracle, kind, ws, x, M, [b.astype(np.float32) for b in bias])
+    differs = 0
+    for out, e32, w, b in zip(outs, exp32, ws, bias):
+        assert out.dtype == np.float16
+        assert np.array_equal(out.view(np.uint16), e32.astype(np.float16).view(np.uint16))
+        # the matmul epilogue's order on the same packed dot: round to float16, then add the bias in float16
+        mm = oracle.matmul(kind, w, x, M, bias=b.astype(np.float32), out_dtype=np.float16, force_pack=True)
+        differs += int(np.count_nonzero(mm.view(np.uint16) != out.view(np.uint16)))
+    assert differs > 0  # the two rounding orders are distinguishable on this input
+
+
+def test_qkv_rejects_other_input_types(oracle):
+    kind, M, K = KIND_Q8_0, 4, 64
+    w = oracle.quantize(kind, gaussian(530, (M, K), 0.02))
+    import ctypes as C
+    from oracle.pyoracle import DT_F32
+
+    arr = C.c_void_p * 3
+    x = gaussian(531, (1, K))
+    outs = [np.zeros((1, M), dtype=np.float32) for _ in range(3)]
+    st = oracle.L.mo_matmul_qkv_separate(kind, arr(*[w.ctypes.data] * 3), x.ctypes.data, 99, 1, K, M,
+                                         arr(None, None, None), DT_F32, arr(*[o.ctypes.data for o in outs]))
+    assert st == -8  # MARMOT_ERROR_NOT_IMPLEMENTED (matmul_qkv.c:761-763)

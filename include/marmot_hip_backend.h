@@ -253,14 +253,85 @@ struct marmot_moe_experts_desc {
 };
 typedef struct marmot_moe_experts_desc marmot_moe_experts_desc_t;
 
+/* include/marmot/types.h:254-267 */
+typedef enum {
+    MARMOT_ROPE_SCALING_UNSPECIFIED = -1,
+    MARMOT_ROPE_SCALING_NONE = 0,
+    MARMOT_ROPE_SCALING_LINEAR = 1,
+    MARMOT_ROPE_SCALING_YARN = 2,
+    MARMOT_ROPE_SCALING_LONGROPE = 3,
+    MARMOT_ROPE_SCALING_MAX_VALUE = MARMOT_ROPE_SCALING_LONGROPE,
+} marmot_rope_scaling_type_t;
+
+typedef enum {
+    MARMOT_ROPE_TYPE_NORM = 0,
+    MARMOT_ROPE_TYPE_NEOX = 1,
+    MARMOT_ROPE_TYPE_MAX_VALUE = MARMOT_ROPE_TYPE_NEOX,
+} marmot_rope_type_t;
+
+/* include/marmot/ops_types.h:98-112 */
+typedef struct marmot_rope_params {
+    const marmot_tensor_t *positions;
+    marmot_rope_scaling_type_t scaling_type;
+    marmot_rope_type_t rope_type;
+    float theta;
+    float freq_scale;
+    float ext_factor;
+    float attn_factor;
+    float beta_fast;
+    float beta_slow;
+    uint32_t orig_ctx_len;
+    uint32_t head_dim;
+    bool apply_to_q;
+    bool apply_to_k;
+} marmot_rope_params_t;
+
+/* include/marmot/ops/matmul.h:63-95 */
+typedef enum {
+    MARMOT_QKV_LAYOUT_UNSPECIFIED = 0,
+    MARMOT_QKV_LAYOUT_FUSED = 1,
+    MARMOT_QKV_LAYOUT_SEPARATE = 2,
+} marmot_matmul_qkv_layout_t;
+
+typedef struct marmot_matmul_qkv_fused {
+    const marmot_tensor_t *weight;
+    const marmot_tensor_t *bias;
+} marmot_matmul_qkv_fused_t;
+
+typedef struct marmot_matmul_qkv_separate {
+    const marmot_tensor_t *wq;
+    const marmot_tensor_t *wk;
+    const marmot_tensor_t *wv;
+    const marmot_tensor_t *bq;
+    const marmot_tensor_t *bk;
+    const marmot_tensor_t *bv;
+} marmot_matmul_qkv_separate_t;
+
+typedef struct marmot_matmul_qkv_desc {
+    const marmot_tensor_t *input;
+    marmot_matmul_qkv_layout_t layout;
+    union {
+        marmot_matmul_qkv_fused_t fused;
+        marmot_matmul_qkv_separate_t separate;
+    };
+    const marmot_matmul_epilogue_t *epilogue;
+    marmot_tensor_t *out_q;
+    marmot_tensor_t *out_k;
+    marmot_tensor_t *out_v;
+    const marmot_rope_params_t *rope_params;
+} marmot_matmul_qkv_desc_t;
+
 /* include/marmot/traits_ids.gen.h:40-107 (the operations this backend answers for), :111-116, :120-133 */
 typedef enum {
     MARMOT_OP_INVALID = 0,
+    MARMOT_OP_QKV_PROJECTION = 191,
     MARMOT_OP_DEQUANTIZE = 210,
     MARMOT_OP_MOE_EXPERTS = 263,
     MARMOT_OP_MATMUL = 498,
     MARMOT_OP_QUANTIZE = 524,
     MARMOT_OP_LINEAR = 708,
+    MARMOT_OP_QKV_SHARED_INPUT = 771,
+    MARMOT_OP_QKV_ROPE = 778,
     MARMOT_OP_TOPK = 901,
     MARMOT_OP_COUNT = 995,
 } marmot_op_id_t;
@@ -567,6 +638,8 @@ bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_bac
  *   MOE_EXPERTS u16 hidden, gate, up, down, topk_ids, topk_weights, out; u32 ffn_type; f32 weights_scale;
  *               u32 router_weight_policy                               (bytecode_compile.c:480-504)
  *   TOPK        u16 input, values_out, indices_out; u32 axis; u32 k    (bytecode_compile.c:459-479)
+ *   QKV         u16 input, wq, wk, wv, bq, bk, bv (0xFFFF none); u32 epilogue const offset; u32 rope-params const
+ *               offset (0xFFFFFFFF none); u16 out_q, out_k, out_v      (bytecode_compile.c:670-715)
  *   QUANTIZE    u16 input; u32 quant-params const offset; u16 output; u32 kind; u32 layout   (:912-941)
  *   DEQUANTIZE  u16 input; u16 output; u32 kind; u32 layout            (bytecode_compile.c:942-962) */
 enum {
@@ -582,7 +655,11 @@ enum {
     MARMOT_HIP_BC_OP_TOPK_F32 = 9,
     MARMOT_HIP_BC_OP_QUANTIZE_BLOCK = 10,
     MARMOT_HIP_BC_OP_DEQUANTIZE_BLOCK = 11,
-    MARMOT_HIP_BC_OP_COUNT = 12,
+    MARMOT_HIP_BC_OP_QKV_Q4_0 = 12,
+    MARMOT_HIP_BC_OP_QKV_Q8_0 = 13,
+    MARMOT_HIP_BC_OP_QKV_Q4_K = 14,
+    MARMOT_HIP_BC_OP_QKV_Q6_K = 15,
+    MARMOT_HIP_BC_OP_COUNT = 16,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -605,6 +682,14 @@ marmot_error_t hip_matmul_quantized_q4_k(const void *device_ctx, const marmot_te
 marmot_error_t hip_matmul_quantized_q6_k(const void *device_ctx, const marmot_tensor_t *input,
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out);
+/* marmot_matmul_qkv with MARMOT_QKV_LAYOUT_SEPARATE and block-quantized weights of one kind and shape
+ * (cf. cpu_matmul_qkv_{q4_k,q6_k,q8_0}, src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:1498-1532; validation as
+ * cpu_matmul_qkv_validate_desc, :1230-1300). The fused layout, dense weights and the rotary epilogue
+ * (rope_params applied to q or k) return MARMOT_ERROR_NOT_IMPLEMENTED. */
+marmot_error_t hip_matmul_qkv_q4_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
+marmot_error_t hip_matmul_qkv_q8_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
+marmot_error_t hip_matmul_qkv_q4_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
+marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc);
 marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc);
 /* output->quant_kind selects the activation block format: Q8_0 or Q8_K */

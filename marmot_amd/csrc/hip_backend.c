@@ -611,6 +611,145 @@ static marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind
     return st;
 }
 
+// marmot_matmul_qkv, separate block-quantized weights. Checks in the order of cpu_matmul_qkv_validate_desc
+// (src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:1140-1146, 1230-1300), cpu_matmul_qkv_quant_entry (:1424-1434) and
+// cpu_matmul_qkv_run_separate_quantized_impl (:761-789).
+static marmot_error_t qkv_locked(hip_backend_t *b, const marmot_matmul_qkv_desc_t *desc, int kind, int dtype, size_t N,
+                                 size_t K, size_t M) {
+    const marmot_tensor_t *w[3] = {desc->separate.wq, desc->separate.wk, desc->separate.wv};
+    const marmot_tensor_t *bias[3] = {desc->separate.bq, desc->separate.bk, desc->separate.bv};
+    marmot_tensor_t *out[3] = {desc->out_q, desc->out_k, desc->out_v};
+    const void *d_w[3] = {nullptr, nullptr, nullptr}, *d_b[3] = {nullptr, nullptr, nullptr}, *d_x = nullptr;
+    void *d_o[3] = {nullptr, nullptr, nullptr};
+    marmot_error_t st = acquire_read(b, desc->input->data, dense_bytes(desc->input), &d_x);
+    for (int i = 0; i < 3 && st == MARMOT_SUCCESS; ++i) {
+        st = acquire_read(b, w[i]->data, M * marmot_hip_row_bytes(kind, K), &d_w[i]);
+        if (st == MARMOT_SUCCESS && bias[i] != nullptr) {
+            st = acquire_read(b, bias[i]->data, dense_bytes(bias[i]), &d_b[i]);
+        }
+    }
+    for (int i = 0; i < 3 && st == MARMOT_SUCCESS; ++i) {
+        st = acquire_write(b, out[i]->data, dense_bytes(out[i]), &d_o[i]);
+    }
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    const int rc = marmot_hip_matmul_qkv_quantized(b->dev, kind, d_w[0], d_w[1], d_w[2], d_x, dtype, N, K, M, d_b[0],
+                                                   d_b[1], d_b[2], dtype, d_o[0], d_o[1], d_o[2], dtype);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        return fail_from_lib(rc);
+    }
+    for (int i = 0; i < 3; ++i) {
+        mark_device_output(out[i]);
+    }
+    return MARMOT_SUCCESS;
+}
+
+static marmot_error_t matmul_qkv(const void *device_ctx, marmot_quant_kind_t expect_kind,
+                                 const marmot_matmul_qkv_desc_t *desc) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: null device context");
+    }
+    if (desc == nullptr || desc->input == nullptr || desc->out_q == nullptr || desc->out_k == nullptr ||
+        desc->out_v == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: null argument");
+    }
+    if (desc->layout == MARMOT_QKV_LAYOUT_FUSED) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized fused QKV weights are not supported yet");
+    }
+    if (desc->layout != MARMOT_QKV_LAYOUT_SEPARATE) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Invalid QKV layout for HIP backend");
+    }
+    const marmot_tensor_t *input = desc->input;
+    const marmot_tensor_t *w[3] = {desc->separate.wq, desc->separate.wk, desc->separate.wv};
+    const marmot_tensor_t *bias[3] = {desc->separate.bq, desc->separate.bk, desc->separate.bv};
+    marmot_tensor_t *out[3] = {desc->out_q, desc->out_k, desc->out_v};
+    if (w[0] == nullptr || w[1] == nullptr || w[2] == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Separate QKV requires three weight tensors");
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (input->dtype != out[i]->dtype) {
+            return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "QKV tensors must share dtype");
+        }
+    }
+    if (input->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Separate QKV expects 2D tensors");
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (w[i]->shape.ndim != 2 || out[i]->shape.ndim != 2) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Separate QKV expects 2D tensors");
+        }
+    }
+    const size_t N = input->shape.shape[0], K = input->shape.shape[1], M = w[0]->shape.shape[0];
+    for (int i = 0; i < 3; ++i) {
+        if (w[i]->shape.shape[1] != K) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Separate QKV weights must share the input dimension");
+        }
+    }
+    if (w[1]->shape.shape[0] != M || w[2]->shape.shape[0] != M) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Separate QKV weights must share the output dimension");
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (out[i]->shape.shape[0] != N || out[i]->shape.shape[1] != M) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Separate QKV output shape mismatch");
+        }
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (bias[i] == nullptr) {
+            continue;
+        }
+        if (bias[i]->dtype != input->dtype) {
+            return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Separate QKV bias dtype must match activations");
+        }
+        if (bias[i]->shape.ndim != 1 || bias[i]->shape.shape[0] != M) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Separate QKV bias must be 1D and match rows");
+        }
+        if (bias[i]->shape.strides[0] != 1) {
+            return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Separate QKV bias must be contiguous");
+        }
+    }
+    if (desc->epilogue != nullptr && desc->epilogue->bias != nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT,
+                    "Separate QKV epilogue bias must be supplied via the descriptor bias tensors");
+    }
+    // the kernel entry: block-quantized GGUF weights of the kind this kernel was selected for
+    for (int i = 0; i < 3; ++i) {
+        if (!kind_is_block(w[i]->quant_kind) || w[i]->quant_layout != MARMOT_QUANT_LAYOUT_GGUF ||
+            w[i]->quant_kind != expect_kind || !kind_supported_weight(w[i]->quant_kind)) {
+            return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "QKV projection: weight scheme not handled by this kernel");
+        }
+    }
+    if (input->dtype != MARMOT_DTYPE_FLOAT32 && input->dtype != MARMOT_DTYPE_FLOAT16) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "QKV projection takes FLOAT32 or FLOAT16 activations");
+    }
+    if (!rows_contiguous(input) || !rows_contiguous(out[0]) || !rows_contiguous(out[1]) || !rows_contiguous(out[2])) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "QKV projection: HIP kernels need contiguous rows");
+    }
+    if (desc->rope_params != nullptr && (desc->rope_params->apply_to_q || desc->rope_params->apply_to_k)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "QKV projection: the rotary epilogue is not provided");
+    }
+    if (input->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: tensor without data");
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (w[i]->data == nullptr || out[i]->data == nullptr || (bias[i] != nullptr && bias[i]->data == nullptr)) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: tensor without data");
+        }
+    }
+    if (N == 0 || M == 0) {
+        for (int i = 0; i < 3; ++i) {
+            mark_device_output(out[i]);
+        }
+        return MARMOT_SUCCESS;
+    }
+    const int dtype = input->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16;
+    pthread_mutex_lock(&b->mu);
+    const marmot_error_t st = qkv_locked(b, desc, (int)expect_kind, dtype, N, K, M);
+    pthread_mutex_unlock(&b->mu);
+    return st;
+}
+
 // bytes of E expert slices of [rows, cols] blocks; expert tensors are stored [cols, rows, E] in GGUF order
 // (cpu_moe_execute_grouped, src/backends/cpu/ops/moe/moe_ops.c:895-899)
 static size_t expert_tensor_bytes(int kind, size_t rows, size_t cols, size_t experts) {
@@ -919,6 +1058,63 @@ HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q8_0, MARMOT_QUANT_KIND_Q8_0)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q4_k, MARMOT_QUANT_KIND_Q4_K)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q6_k, MARMOT_QUANT_KIND_Q6_K)
 
+// QKV immediates (bytecode_compile.c:670-715): the tensors come from the registers, the epilogue and the rotary
+// parameters from the constant pool.
+static marmot_error_t bc_exec_qkv(marmot_quant_kind_t kind, const void *exec_ctx, marmot_tensor_t **regs,
+                                  const uint8_t *imm, const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const void *device_ctx = ((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx;
+    const uint8_t *pc = imm;
+    uint16_t idx[7];
+    for (int i = 0; i < 7; ++i) {
+        idx[i] = rd_u16(&pc);
+    }
+    const uint32_t epilogue_off = rd_u32(&pc);
+    const uint32_t rope_off = rd_u32(&pc);
+    const uint16_t out_q = rd_u16(&pc), out_k = rd_u16(&pc), out_v = rd_u16(&pc);
+    marmot_matmul_epilogue_t epilogue;
+    marmot_rope_params_t rope;
+    marmot_matmul_qkv_desc_t desc;
+    memset(&desc, 0, sizeof(desc));
+    if (epilogue_off != MARMOT_BC_INVALID_OFFSET || rope_off != MARMOT_BC_INVALID_OFFSET) {
+        if (const_pool == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for qkv parameters");
+        }
+    }
+    if (epilogue_off != MARMOT_BC_INVALID_OFFSET) {
+        memcpy(&epilogue, const_pool + epilogue_off, sizeof(epilogue));
+        desc.epilogue = &epilogue;
+    }
+    if (rope_off != MARMOT_BC_INVALID_OFFSET) {
+        memcpy(&rope, const_pool + rope_off, sizeof(rope));
+        desc.rope_params = &rope;
+    }
+    desc.input = reg(regs, idx[0]);
+    desc.layout = MARMOT_QKV_LAYOUT_SEPARATE;
+    desc.separate.wq = reg(regs, idx[1]);
+    desc.separate.wk = reg(regs, idx[2]);
+    desc.separate.wv = reg(regs, idx[3]);
+    desc.separate.bq = reg(regs, idx[4]);
+    desc.separate.bk = reg(regs, idx[5]);
+    desc.separate.bv = reg(regs, idx[6]);
+    desc.out_q = reg(regs, out_q);
+    desc.out_k = reg(regs, out_k);
+    desc.out_v = reg(regs, out_v);
+    return matmul_qkv(device_ctx, kind, &desc);
+}
+
+#define HIP_BC_QKV_ENTRY(name, kind)                                                                                   \
+    static marmot_error_t name(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,                       \
+                               const uint8_t *const_pool) {                                                            \
+        return bc_exec_qkv(kind, exec_ctx, regs, imm, const_pool);                                                     \
+    }
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q4_0, MARMOT_QUANT_KIND_Q4_0)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q8_0, MARMOT_QUANT_KIND_Q8_0)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q4_k, MARMOT_QUANT_KIND_Q4_K)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q6_k, MARMOT_QUANT_KIND_Q6_K)
+
 static marmot_error_t bc_exec_moe(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
                                   const uint8_t *const_pool) {
     (void)const_pool;
@@ -998,6 +1194,7 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     14,              // TOPK: 3 x u16 + 2 x u32
     16,              // QUANTIZE: u16 + u32 + u16 + 2 x u32
     12,              // DEQUANTIZE: 2 x u16 + 2 x u32
+    28, 28, 28, 28,  // QKV: 7 x u16 + 2 x u32 + 3 x u16
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1005,7 +1202,8 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MATMUL,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS,
     MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_TOPK,
-    MARMOT_BC_SCHEMA_QUANTIZE,    MARMOT_BC_SCHEMA_DEQUANTIZE,
+    MARMOT_BC_SCHEMA_QUANTIZE,    MARMOT_BC_SCHEMA_DEQUANTIZE,  MARMOT_BC_SCHEMA_QKV,
+    MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_QKV,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1013,6 +1211,7 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_matmul_q4_0, bc_exec_matmul_q8_0, bc_exec_matmul_q4_k, bc_exec_matmul_q6_k,
     bc_exec_moe,         bc_exec_moe,         bc_exec_moe,         bc_exec_moe,
     bc_exec_topk,        bc_exec_quantize,    bc_exec_dequantize,
+    bc_exec_qkv_q4_0,    bc_exec_qkv_q8_0,    bc_exec_qkv_q4_k,    bc_exec_qkv_q6_k,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -1121,6 +1320,43 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const double t_mem = bytes / (bw_gbps * 1e3);          // us
         const double t_mma = 2.0 * N * M * K / (tflops * 1e6);  // us
         const double ws_mb = in32 ? (double)marmot_hip_packed_activation_bytes(kind, N, K) / 1048576.0 : 0.0;
+        return selected(op, launch_us + (t_mem > t_mma ? t_mem : t_mma), ws_mb);
+    }
+    case MARMOT_OP_QKV_PROJECTION:
+    case MARMOT_OP_QKV_SHARED_INPUT:
+    case MARMOT_OP_QKV_ROPE: {
+        // cpu/kernels/matmul_qkv.def:19-36, 54-71: quantized weights of one scheme, layout NT, separate weights,
+        // contiguous, FLOAT32 accumulation; outputs have the input dtype (matmul_qkv.c:1240-1243)
+        const int kind = kind_of_scheme(sig->qscheme_id);
+        const uint16_t mm = matmul_op_of_kind(kind);
+        if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
+            return unsupported("HIP QKV projection handles Q4_0, Q8_0, Q4_K and Q6_K weights");
+        }
+        if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
+            return unsupported("HIP QKV projection needs layout NT");
+        }
+        if (!((in32 && out32) || (in16 && out16))) {
+            return unsupported("HIP QKV projection: outputs must have the activation dtype (FLOAT32 or FLOAT16)");
+        }
+        if (sig->accum_dtype != MARMOT_DTYPE_FLOAT32) {
+            return unsupported("HIP QKV projection accumulates in FLOAT32");
+        }
+        if (sig->weight_layout != MARMOT_WEIGHT_LAYOUT_SEPARATE) {
+            return unsupported("HIP QKV projection needs separate weights");
+        }
+        if (sig->stride_mode != MARMOT_STRIDE_MODE_CONTIGUOUS && sig->stride_mode != MARMOT_STRIDE_MODE_ANY) {
+            return unsupported("HIP QKV projection needs contiguous rows");
+        }
+        if ((sig->epilogue_flags & ~(uint32_t)MARMOT_EPILOGUE_BIAS) != 0 || sig->variant_flags != 0) {
+            return unsupported("HIP QKV projection fuses only the bias epilogue (no rotary embedding)");
+        }
+        const size_t N = sig->dims.matmul.N, K = sig->dims.matmul.K, M = sig->dims.matmul.M;
+        const double bytes = 3.0 * (double)M * (double)marmot_hip_row_bytes(kind, K) +
+                             (double)N * K * (in32 ? 4 : 2) + 3.0 * (double)N * M * (out32 ? 4 : 2);
+        const double t_mem = bytes / (bw_gbps * 1e3);
+        const double t_mma = 6.0 * N * M * K / (tflops * 1e6);
+        const double ws_mb = (double)marmot_hip_packed_activation_bytes(kind, N, K) / 1048576.0;
+        const uint16_t op = (uint16_t)(MARMOT_HIP_BC_OP_QKV_Q4_0 + (mm - MARMOT_HIP_BC_OP_MATMUL_Q4_0));
         return selected(op, launch_us + (t_mem > t_mma ? t_mem : t_mma), ws_mb);
     }
     case MARMOT_OP_MOE_EXPERTS: {
@@ -1242,6 +1478,18 @@ marmot_error_t hip_matmul_quantized_q6_k(const void *device_ctx, const marmot_te
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out) {
     return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q6_K, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_qkv_q4_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q4_0, desc);
+}
+marmot_error_t hip_matmul_qkv_q8_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q8_0, desc);
+}
+marmot_error_t hip_matmul_qkv_q4_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q4_K, desc);
+}
+marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q6_K, desc);
 }
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc) {
     return moe_experts(device_ctx, desc);

@@ -35,11 +35,14 @@ MEMORY_HOST, MEMORY_DEVICE = 0, 1
 BACKEND_HIP = 3
 # marmot_op_id_t / marmot_qscheme_id_t
 OP_DEQUANTIZE, OP_MOE_EXPERTS, OP_MATMUL, OP_QUANTIZE, OP_LINEAR, OP_TOPK = 210, 263, 498, 524, 708, 901
+OP_QKV_PROJECTION, OP_QKV_SHARED_INPUT, OP_QKV_ROPE = 191, 771, 778
+QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q8_0: 5, KIND_Q4_K: 8, KIND_Q6_K: 10, KIND_Q8_K: 11}
 PROFILE_SCALAR = 4
 MATMUL_LAYOUT_NT = 2
 WEIGHT_LAYOUT_SEPARATE = 1
 EPILOGUE_BIAS = 1
+EPILOGUE_ROPE = 8
 BC_END, BC_REG_INVALID, BC_INVALID_OFFSET = 0, 0xFFFF, 0xFFFFFFFF
 
 _NP_OF_DTYPE = {DTYPE_F32: np.float32, DTYPE_F16: np.float16, DTYPE_I32: np.int32, DTYPE_I8: np.int8,
@@ -63,6 +66,33 @@ class Tensor(C.Structure):
 
 class Epilogue(C.Structure):
     _fields_ = [("bias", C.POINTER(Tensor)), ("enable_output_cast", C.c_bool), ("output_dtype", C.c_int)]
+
+
+class RopeParams(C.Structure):
+    _fields_ = [("positions", C.POINTER(Tensor)), ("scaling_type", C.c_int), ("rope_type", C.c_int),
+                ("theta", C.c_float), ("freq_scale", C.c_float), ("ext_factor", C.c_float),
+                ("attn_factor", C.c_float), ("beta_fast", C.c_float), ("beta_slow", C.c_float),
+                ("orig_ctx_len", C.c_uint32), ("head_dim", C.c_uint32), ("apply_to_q", C.c_bool),
+                ("apply_to_k", C.c_bool)]
+
+
+class QkvFused(C.Structure):
+    _fields_ = [("weight", C.POINTER(Tensor)), ("bias", C.POINTER(Tensor))]
+
+
+class QkvSeparate(C.Structure):
+    _fields_ = [(n, C.POINTER(Tensor)) for n in ("wq", "wk", "wv", "bq", "bk", "bv")]
+
+
+class _QkvWeights(C.Union):
+    _fields_ = [("fused", QkvFused), ("separate", QkvSeparate)]
+
+
+class QkvDesc(C.Structure):
+    _anonymous_ = ("weights",)
+    _fields_ = [("input", C.POINTER(Tensor)), ("layout", C.c_int), ("weights", _QkvWeights),
+                ("epilogue", C.POINTER(Epilogue)), ("out_q", C.POINTER(Tensor)), ("out_k", C.POINTER(Tensor)),
+                ("out_v", C.POINTER(Tensor)), ("rope_params", C.POINTER(RopeParams))]
 
 
 class TopkDesc(C.Structure):
@@ -204,7 +234,8 @@ BACKEND_SYMBOLS = [
     "marmot_get_hip_ops", "marmot_hip_query_kernel", "marmot_hip_detect_default_caps",
     "marmot_hip_default_preferences", "marmot_hip_bc_get_tables",
     "hip_matmul_quantized_q4_0", "hip_matmul_quantized_q8_0", "hip_matmul_quantized_q4_k",
-    "hip_matmul_quantized_q6_k", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
+    "hip_matmul_quantized_q6_k", "hip_matmul_qkv_q4_0", "hip_matmul_qkv_q8_0", "hip_matmul_qkv_q4_k",
+    "hip_matmul_qkv_q6_k", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
 ]
 
@@ -225,6 +256,9 @@ def bind(lib: C.CDLL) -> C.CDLL:
         fn = getattr(lib, f"hip_matmul_quantized_{name}")
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Epilogue), C.POINTER(Tensor)]
+        fn = getattr(lib, f"hip_matmul_qkv_{name}")
+        fn.restype = C.c_int
+        fn.argtypes = [C.c_void_p, C.POINTER(QkvDesc)]
     lib.hip_moe_experts_impl.restype = C.c_int
     lib.hip_moe_experts_impl.argtypes = [C.c_void_p, C.POINTER(MoeDesc)]
     lib.hip_topk_impl.restype = C.c_int
@@ -365,6 +399,16 @@ class HipContext:
         sig.dims.matmul.M = w.t.shape.shape[0]
         return sig
 
+    def qkv_signature(self, x: HostTensor, wq: HostTensor, out_q: HostTensor, bias: bool = False,
+                      rope: bool = False, op_id: int = OP_QKV_SHARED_INPUT) -> OpSignature:
+        """marmot_matmul_qkv_build (src/core/dispatch/matmul_build.c:148-217)."""
+        sig = self.matmul_signature(x, wq, out_q, bias)
+        sig.op_id = op_id
+        sig.weight_dtype = x.t.dtype  # quantized weights: the signature carries the activation dtype (:170)
+        if rope:
+            sig.epilogue_flags |= EPILOGUE_ROPE
+        return sig
+
     def query(self, sig: OpSignature, caps: Optional[DeviceCaps] = None) -> KernelSelection:
         caps = caps if caps is not None else self.lib.marmot_hip_detect_default_caps()
         return self.lib.marmot_hip_query_kernel(C.byref(sig), C.byref(caps))
@@ -435,6 +479,16 @@ class Program:
             self._keep.append(ep)
             off = self._const(bytes(ep), 8)
         self.code += struct.pack("<HHHHIH", op_index, self.reg(x), self.reg(w), self.reg(bias), off, self.reg(out))
+
+    def qkv(self, op_index: int, x: HostTensor, wq, wk, wv, out_q, out_k, out_v, bq=None, bk=None, bv=None,
+            rope: Optional[RopeParams] = None):
+        """bytecode_compile.c:670-715."""
+        rope_off = BC_INVALID_OFFSET
+        if rope is not None:
+            self._keep.append(rope)
+            rope_off = self._const(bytes(rope), 8)
+        self.code += struct.pack("<H7HII3H", op_index, *[self.reg(t) for t in (x, wq, wk, wv, bq, bk, bv)],
+                                 BC_INVALID_OFFSET, rope_off, self.reg(out_q), self.reg(out_k), self.reg(out_v))
 
     def moe_experts(self, op_index: int, hidden, gate, up, down, ids, weights, out, ffn_type=0, weights_scale=1.0,
                     policy=1):

@@ -10,6 +10,7 @@
 #include "marmot/graph/kernel_selection.h"
 #include "marmot/graph/op_signature.h"
 #include "marmot/ops_types.h"
+#include "marmot/ops/matmul.h"
 #include "core/bytecode/bytecode.h"
 #include "core/bytecode/bytecode_compile.h"
 #include "core/dispatch/kernel_query.h"
@@ -43,6 +44,10 @@ int main(void) {
     VAL(MARMOT_ROUTING_ALWAYS_GPU);
     VAL(MARMOT_OP_MATMUL); VAL(MARMOT_OP_LINEAR); VAL(MARMOT_OP_MOE_EXPERTS); VAL(MARMOT_OP_TOPK);
     VAL(MARMOT_OP_QUANTIZE); VAL(MARMOT_OP_DEQUANTIZE);
+    VAL(MARMOT_OP_QKV_PROJECTION); VAL(MARMOT_OP_QKV_SHARED_INPUT); VAL(MARMOT_OP_QKV_ROPE);
+    VAL(MARMOT_QKV_LAYOUT_FUSED); VAL(MARMOT_QKV_LAYOUT_SEPARATE);
+    VAL(MARMOT_ROPE_SCALING_NONE); VAL(MARMOT_ROPE_SCALING_YARN); VAL(MARMOT_ROPE_TYPE_NORM); VAL(MARMOT_ROPE_TYPE_NEOX);
+    VAL(MARMOT_EPILOGUE_ROPE); VAL(MARMOT_BC_SCHEMA_QKV);
     VAL(MARMOT_QSCHEME_Q4_0); VAL(MARMOT_QSCHEME_Q8_0); VAL(MARMOT_QSCHEME_Q4_K); VAL(MARMOT_QSCHEME_Q6_K);
     VAL(MARMOT_QSCHEME_Q8_K);
     VAL(MARMOT_MATMUL_LAYOUT_NT); VAL(MARMOT_WEIGHT_LAYOUT_SEPARATE); VAL(MARMOT_STRIDE_MODE_CONTIGUOUS);
@@ -73,6 +78,16 @@ int main(void) {
     OFF(marmot_device_ops_t, on_host_range_freed);
     SZ(marmot_matmul_epilogue_t); OFF(marmot_matmul_epilogue_t, bias);
     OFF(marmot_matmul_epilogue_t, enable_output_cast); OFF(marmot_matmul_epilogue_t, output_dtype);
+    SZ(marmot_rope_params_t); OFF(marmot_rope_params_t, positions); OFF(marmot_rope_params_t, scaling_type);
+    OFF(marmot_rope_params_t, rope_type); OFF(marmot_rope_params_t, theta); OFF(marmot_rope_params_t, beta_slow);
+    OFF(marmot_rope_params_t, orig_ctx_len); OFF(marmot_rope_params_t, head_dim);
+    OFF(marmot_rope_params_t, apply_to_q); OFF(marmot_rope_params_t, apply_to_k);
+    SZ(marmot_matmul_qkv_desc_t); OFF(marmot_matmul_qkv_desc_t, input); OFF(marmot_matmul_qkv_desc_t, layout);
+    OFF(marmot_matmul_qkv_desc_t, fused); OFF(marmot_matmul_qkv_desc_t, separate);
+    OFF(marmot_matmul_qkv_desc_t, epilogue); OFF(marmot_matmul_qkv_desc_t, out_q);
+    OFF(marmot_matmul_qkv_desc_t, out_k); OFF(marmot_matmul_qkv_desc_t, out_v);
+    OFF(marmot_matmul_qkv_desc_t, rope_params);
+    SZ(marmot_matmul_qkv_separate_t); OFF(marmot_matmul_qkv_separate_t, wv); OFF(marmot_matmul_qkv_separate_t, bq);
     SZ(marmot_topk_desc_t); OFF(marmot_topk_desc_t, axis); OFF(marmot_topk_desc_t, k);
     SZ(marmot_moe_experts_desc_t); OFF(marmot_moe_experts_desc_t, out); OFF(marmot_moe_experts_desc_t, ffn_type);
     OFF(marmot_moe_experts_desc_t, weights_scale); OFF(marmot_moe_experts_desc_t, router_weight_policy);

@@ -62,7 +62,8 @@ def test_ctypes_structs_match_layout(golden_layout):
         "marmot_bc_exec_ctx_t": ta.BcExecCtx, "marmot_bc_tables_t": ta.BcTables,
         "marmot_allocator_usage_t": ta.AllocatorUsage, "marmot_context_policy_t": ta.ContextPolicy,
         "marmot_backend_preferences_t": ta.BackendPreferences, "marmot_matmul_dims_t": ta.MatmulDims,
-        "marmot_quant_block_t": ta.QuantBlock,
+        "marmot_quant_block_t": ta.QuantBlock, "marmot_rope_params_t": ta.RopeParams,
+        "marmot_matmul_qkv_desc_t": ta.QkvDesc, "marmot_matmul_qkv_separate_t": ta.QkvSeparate,
     }
     checked = 0
     for cname, cls in pairs.items():
@@ -192,6 +193,32 @@ def test_query_kernel_other_ops(lib):
     assert not _query(lib, _sig(op=12345)).supported
 
 
+def test_query_kernel_qkv_rules(lib, golden_layout):
+    """cpu/kernels/matmul_qkv.def:19-36, 54-71 with this backend's schemes; outputs carry the activation dtype."""
+    assert (ta.OP_QKV_PROJECTION, ta.OP_QKV_SHARED_INPUT, ta.OP_QKV_ROPE) == tuple(
+        golden_layout[k] for k in ("MARMOT_OP_QKV_PROJECTION", "MARMOT_OP_QKV_SHARED_INPUT", "MARMOT_OP_QKV_ROPE"))
+    assert ta.EPILOGUE_ROPE == golden_layout["MARMOT_EPILOGUE_ROPE"]
+    for op_id in (ta.OP_QKV_PROJECTION, ta.OP_QKV_SHARED_INPUT, ta.OP_QKV_ROPE):
+        for kind, op in {ta.KIND_Q4_0: 12, ta.KIND_Q8_0: 13, ta.KIND_Q4_K: 14, ta.KIND_Q6_K: 15}.items():
+            for dt in (ta.DTYPE_F32, ta.DTYPE_F16):
+                sel = _query(lib, _sig(op=op_id, kind=kind, inp=dt, out=dt, N=4, K=4096, M=4096))
+                assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
+    s = _sig(op=ta.OP_QKV_SHARED_INPUT, inp=ta.DTYPE_F16, out=ta.DTYPE_F32)
+    assert not _query(lib, s).supported  # outputs must have the activation dtype
+    s = _sig(op=ta.OP_QKV_SHARED_INPUT); s.epilogue_flags = ta.EPILOGUE_BIAS
+    assert _query(lib, s).supported
+    s = _sig(op=ta.OP_QKV_ROPE); s.epilogue_flags = ta.EPILOGUE_BIAS | ta.EPILOGUE_ROPE
+    sel = _query(lib, s)
+    assert not sel.supported and b"rotary" in sel.fallback_reason
+    assert not _query(lib, _sig(op=ta.OP_QKV_SHARED_INPUT, kind=ta.KIND_Q8_K)).supported
+    s = _sig(op=ta.OP_QKV_SHARED_INPUT); s.weight_layout = 2
+    assert not _query(lib, s).supported
+    # three weight streams, one activation read, three outputs
+    sel = _query(lib, _sig(op=ta.OP_QKV_SHARED_INPUT, N=1, K=4096, M=4096))
+    nbytes = 3 * 4096 * 16 * 144 + 4096 * 4 + 3 * 4096 * 4
+    assert sel.estimated_us == pytest.approx(2.0 + nbytes / 8000e3, rel=1e-6) and sel.est_workspace_mb > 0
+
+
 def test_default_caps_and_preferences(lib):
     caps = lib.marmot_hip_detect_default_caps()
     assert caps.mem_bw_gbps == pytest.approx(8000.0)
@@ -208,7 +235,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 12
+    assert t.op_count == 16
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -216,6 +243,7 @@ def test_bytecode_tables(lib, golden_layout):
     assert schema[9] == golden_layout["MARMOT_BC_SCHEMA_TOPK"]
     assert schema[10] == golden_layout["MARMOT_BC_SCHEMA_QUANTIZE"]
     assert schema[11] == golden_layout["MARMOT_BC_SCHEMA_DEQUANTIZE"]
+    assert schema[12:16] == [golden_layout["MARMOT_BC_SCHEMA_QKV"]] * 4
     # immediate sizes equal what the encoders of tensor_abi.Program emit (opcode excluded)
     sizes = [t.imm_size[i] for i in range(t.op_count)]
     assert sizes[1:5] == [struct.calcsize("<HHHIH")] * 4
@@ -223,6 +251,7 @@ def test_bytecode_tables(lib, golden_layout):
     assert sizes[9] == struct.calcsize("<HHHII")
     assert sizes[10] == struct.calcsize("<HIHII")
     assert sizes[11] == struct.calcsize("<HHII")
+    assert sizes[12:16] == [struct.calcsize("<7HII3H")] * 4
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -239,6 +268,7 @@ def test_exec_entries_reject_null_arguments(lib):
     # impl functions with a null device context
     assert lib.hip_matmul_quantized_q4_k(None, None, None, None, None) == ta.INVALID_ARGUMENT
     assert lib.hip_moe_experts_impl(None, None) == ta.INVALID_ARGUMENT
+    assert lib.hip_matmul_qkv_q4_k(None, None) == ta.INVALID_ARGUMENT
     assert lib.hip_topk_impl(None, None) == ta.INVALID_ARGUMENT
 
 
@@ -255,6 +285,15 @@ def test_program_encoding_matches_reference_immediates():
     op, ri, rw, rb, off, ro = struct.unpack_from("<HHHHIH", p.code, 14)
     assert (op, ri, rw, rb, ro) == (3, 0, 1, 3, 2) and off == 0 and len(p.const_pool) == C.sizeof(ta.Epilogue)
     assert len(p.regs) == 4
+    # QKV: seven tensor registers (absent biases 0xFFFF), epilogue and rope offsets, three outputs
+    q = ta.Program()
+    outs = [ta.HostTensor.empty((2, 4), ta.DTYPE_F32) for _ in range(3)]
+    q.qkv(14, x, w, w, w, *outs, bk=b)
+    assert bytes(q.code) == struct.pack("<H7HII3H", 14, 0, 1, 1, 1, 0xFFFF, 2, 0xFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 3, 4, 5)
+    rp = ta.RopeParams()
+    rp.theta, rp.apply_to_q = 10000.0, True
+    q.qkv(14, x, w, w, w, *outs, rope=rp)
+    assert struct.unpack_from("<I", q.code, 30 + 2 + 14 + 4)[0] == 0 and len(q.const_pool) == C.sizeof(ta.RopeParams)
     # tensor strides are row-major element strides, as marmot_tensor_create fills them
     assert list(x.t.shape.strides[:2]) == [256, 1] and x.t.shape.ndim == 2
 
@@ -267,8 +306,12 @@ def test_kernel_def_files_name_exported_impls(lib):
         for name, body in re.findall(r"KERNEL_FAMILY\((\w+)\)\s*\{(.*?)\n\}", text, re.S):
             fields = dict(re.findall(r"^\s*([A-Z_]+(?:\(\w+\))?):\s*(.+?),?\s*$", body, re.M))
             families[name] = fields
+    qkv = {f"{op}_quantized_hip_{dt}" for op in ("qkv_shared_input", "qkv_projection") for dt in ("f16", "f32")}
     assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_q6_k", "topk_hip",
-                             "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip"}
+                             "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip"} | qkv
+    for name in qkv:
+        f = families[name]
+        assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS]" and f["OP"] in name
     for name, f in families.items():
         impl = f["IMPL_FUNCTION"].strip('"')
         schemes = re.findall(r"Q\d_[0K]", f.get("AXIS(scheme)", "")) or [""]

@@ -163,8 +163,8 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5")):
-    """Every benchmark configuration (C1..C5) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV")):
+    """Every benchmark configuration (C1..C5, QKV) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -210,6 +210,51 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5")):
         sweep_layer_stack(hip, rng, emit, steps)
     if "C5" in only:
         sweep_moe(hip, rng, emit, steps)
+    if "QKV" in only:
+        sweep_qkv(hip, rng, emit, steps, warmup)
+
+
+def sweep_qkv(hip, rng, emit, steps: int, warmup: int):
+    """Fused Q/K/V projection (three 4096 x 4096 weights of one scheme, one input) against three separate linears on
+    the same buffers; weight copies rotate as in the other configurations."""
+    from marmot_amd import DT_F32, capi, row_bytes
+
+    M = K = 4096
+    names = {capi.KIND_Q4_K: "Q4_K", capi.KIND_Q6_K: "Q6_K"}
+    for kind in (capi.KIND_Q4_K, capi.KIND_Q6_K):
+        rb = row_bytes(kind, K)
+        stride = (M * rb + 255) & ~255
+        copies = max(2, -(-2 * MALL_BYTES // (3 * stride)) + 1)
+        d_w = []
+        for _ in range(3):
+            blocks = random_blocks(rng, kind, M, K)
+            buf = hip.alloc(stride * copies)
+            for c in range(copies):
+                buf.upload(blocks, offset=c * stride)
+            d_w.append(buf)
+        for N in (1, 4, 16):
+            d_x = hip.to_device(rng.standard_normal((N, K), dtype=np.float32))
+            d_o = [hip.alloc(N * M * 4) for _ in range(3)]
+            fused = time_steps_graph(hip, lambda i: hip.linear_qkv_d(kind, *d_w, d_x, DT_F32, N, K, M, *d_o,
+                                                                     weight_offset=(i % copies) * stride),
+                                     steps, warmup)
+            route = hip.last_route()
+
+            def three(i):
+                for w, o in zip(d_w, d_o):
+                    hip.linear_d(kind, w, d_x, DT_F32, N, K, M, o, DT_F32, weight_offset=(i % copies) * stride)
+
+            separate = time_steps_graph(hip, three, steps, warmup)
+            nbytes = 3 * M * rb + N * K * 4 + 3 * N * M * 4
+            emit({"config": "QKV", "workload": f"{names[kind]} q,k,v 3 x {M}x{K} N={N}", "route": route,
+                  "us": round(fused * 1e3, 2), "us_three_linears": round(separate * 1e3, 2),
+                  "GB/s": round(nbytes / fused / 1e6, 1),
+                  "frac_of_hbm_peak": round(nbytes / fused / 1e6 / HBM_PEAK_GBPS, 4),
+                  "tokens_per_s": round(N / fused * 1e3)})
+            for b in [d_x] + d_o:
+                b.free()
+        for b in d_w:
+            b.free()
 
 
 def sweep_layer_stack(hip, rng, emit, steps: int):
@@ -317,7 +362,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--prefill-tokens", type=int, default=512)
     ap.add_argument("--sweep", action="store_true",
-                    help="measure every benchmark configuration (C1..C5) instead, one JSON line each (documentation runs)")
+                    help="measure every benchmark configuration (C1..C5, QKV) instead, one JSON line each (documentation runs)")
     ap.add_argument("--configs", default="C1,C2,C3,C4,C5", help="with --sweep: the configurations to run")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")

@@ -159,6 +159,15 @@ class HipBackend:
             C.c_void_p(d_bias.ptr) if d_bias is not None else None, bias_dtype, C.c_void_p(d_out.ptr), out_dtype,
             flags))
 
+    def linear_qkv_d(self, kind: int, d_wq, d_wk, d_wv, d_input, dtype: int, N: int, K: int, M: int, d_out_q, d_out_k,
+                     d_out_v, d_bq=None, d_bk=None, d_bv=None, weight_offset: int = 0):
+        """marmot_hip_matmul_qkv_quantized on device buffers; weight_offset applies to the three weights alike."""
+        opt = lambda b: C.c_void_p(b.ptr) if b is not None else None
+        check(self.lib.marmot_hip_matmul_qkv_quantized(
+            self.dev, kind, C.c_void_p(d_wq.ptr + weight_offset), C.c_void_p(d_wk.ptr + weight_offset),
+            C.c_void_p(d_wv.ptr + weight_offset), C.c_void_p(d_input.ptr), dtype, N, K, M, opt(d_bq), opt(d_bk),
+            opt(d_bv), dtype, C.c_void_p(d_out_q.ptr), C.c_void_p(d_out_k.ptr), C.c_void_p(d_out_v.ptr), dtype))
+
     def packed_activation_bytes(self, kind: int, N: int, K: int) -> int:
         return int(self.lib.marmot_hip_packed_activation_bytes(kind, N, K))
 

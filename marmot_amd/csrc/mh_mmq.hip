@@ -825,13 +825,19 @@ static bool mmq6_uses_loader(size_t nb) {
 //     about 4 (Q6_K: 3.5) workgroups per CU, which overlap each other's load and compute phases; the partials meet
 //     in the reduction kernel. Measured per shape; e.g. Q4_K 4096 x 14336 N=8: 19.1 -> 18.0 us, Q6_K 14336 x 4096
 //     N=8: 34.0 -> 28.4 us.
-static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t M, size_t nb) {
-    const size_t rg = (M + 31) / 32;
+static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t M, size_t nb, int weights) {
+    // row groups of the whole launch: the weights of a set (gate/up, q/k/v) are one grid
+    const size_t rg = ((M + 31) / 32) * (size_t)(weights > 0 ? weights : 1);
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     MmqPlan pl;
     const bool q6_loader = kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(nb);
     size_t W, S = 1;
-    if (q6_loader || (kind == MARMOT_HIP_KIND_Q4_K && rg < cus)) {
+    if (q6_loader && weights > 1 && rg >= cus) {
+        // a set of weights that fills the chip by itself: two consumers per workgroup and no K split, so that no
+        // reduction launch per weight follows (q/k/v 3 x 4096 x 4096, N=16: 41.3 us with the rule below, 33.6 with
+        // two workgroups along K, 32.2 with this)
+        W = nb < 2 ? nb : 2;
+    } else if (q6_loader || (kind == MARMOT_HIP_KIND_Q4_K && rg < cus)) {
         W = 1;
         const size_t want = ((q6_loader ? 7 : 8) * cus / 2 + rg - 1) / rg;  // workgroups along K
         while (S < want && S * 8 <= nb) {
@@ -859,7 +865,7 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t
 
 // bytes of fp32 partials launch_mmq needs for this shape (0 when K is not split across workgroups)
 size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int weights) {
-    const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K);
+    const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K, weights);
     return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (size_t)weights : 0;
 }
 
@@ -950,7 +956,7 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
     }
     const size_t nb = K / QK_K;
-    const MmqPlan pl = mmq_plan(dev, kind, N, M, nb);
+    const MmqPlan pl = mmq_plan(dev, kind, N, M, nb, ws.count);
     float *partial = (float *)scratch;
     if (pl.S > 1 && partial == nullptr) {
         void *wsp = nullptr;

@@ -53,6 +53,8 @@ enum {
 enum {
     MARMOT_HIP_DTYPE_F32 = 0,
     MARMOT_HIP_DTYPE_F16 = 1,
+    MARMOT_HIP_DTYPE_I32 = 3,  /* position tensors of the rotary epilogue only */
+    MARMOT_HIP_DTYPE_I64 = 11,
 };
 
 /* marmot_router_weight_policy_t (include/marmot/types.h:283-288), marmot_ffn_type_t (:276-281) */
@@ -178,11 +180,44 @@ int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const v
  *   d_input          : [N,K] of in_dtype (F32 or F16), row-major
  *   d_bq, d_bk, d_bv : each NULL or M values of bias_dtype (F32 or F16)
  *   d_out_*          : [N,M] of out_dtype, which must equal in_dtype (matmul_qkv.c:769-772)
- * The rotary epilogue of the reference op (rope_params) is not part of this call. */
+ * The rotary epilogue of the reference op (rope_params) is the _rope variant below. */
 int marmot_hip_matmul_qkv_quantized(marmot_hip_device_t *dev, int kind, const void *d_wq, const void *d_wk,
                                     const void *d_wv, const void *d_input, int in_dtype, size_t N, size_t K, size_t M,
                                     const void *d_bq, const void *d_bk, const void *d_bv, int bias_dtype,
                                     void *d_out_q, void *d_out_k, void *d_out_v, int out_dtype);
+
+/* Rotary epilogue of the Q/K/V projection: cpu_matmul_qkv_apply_rope_row / cpu_matmul_qkv_rotate_row_f32_headed
+ * (matmul_qkv.c:700-747, matmul_qkv_rope.h:50-70, 123-138). q and/or k rows are rotated in FLOAT32 before the one
+ * rounding of the store: per head of head_dim values and pair i, angle = (float)position[n] * freqs[i],
+ * (even, odd) -> (even*c - odd*s, even*s + odd*c) with c = cos(angle)*attn_scale, s = sin(angle)*attn_scale;
+ * pairs are (2i, 2i+1) for rope_type 0 (NORM) and (i, i + head_dim/2) for 1 (NEOX). */
+typedef struct marmot_hip_rope {
+    const void *d_positions; /* N values of positions_dtype: F32, I32 or I64 (cpu_backend_internal.h:567-578) */
+    int positions_dtype;
+    const float *d_freqs;    /* head_dim / 2 angular frequencies in device memory (marmot_hip_rope_frequencies) */
+    float attn_scale;
+    uint32_t head_dim;       /* even, divides M (after cpu_matmul_qkv_resolve_head_dim, matmul_qkv_rope.h:14-23) */
+    int rope_type;
+    int apply_to_q, apply_to_k;
+} marmot_hip_rope_t;
+
+/* marmot_hip_matmul_qkv_quantized followed by the rotary epilogue; rope == NULL or neither apply flag set is the
+ * plain projection. */
+int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, const void *d_wq, const void *d_wk,
+                                         const void *d_wv, const void *d_input, int in_dtype, size_t N, size_t K,
+                                         size_t M, const void *d_bq, const void *d_bk, const void *d_bv,
+                                         int bias_dtype, void *d_out_q, void *d_out_k, void *d_out_v, int out_dtype,
+                                         const marmot_hip_rope_t *rope);
+
+/* Host-side: the head_dim/2 angular frequencies and the attention scale of marmot_rope_freq_cache_ensure
+ * (src/core/helpers/rope.c:61-127, 143-200) for marmot_rope_params_t fields (include/marmot/ops_types.h:98-112);
+ * scaling_type as marmot_rope_scaling_type_t (include/marmot/types.h:254-261). head_dim is resolved against M as
+ * cpu_matmul_qkv_resolve_head_dim does and returned in *head_dim_out. freqs_out: host array of at least M/2 floats.
+ * The YaRN ramp (a non-zero extrapolation factor with a valid original context) returns NOT_IMPLEMENTED. */
+int marmot_hip_rope_frequencies(int scaling_type, float theta, float freq_scale, float ext_factor,
+                                float attn_factor, float beta_fast, float beta_slow, uint32_t orig_ctx_len,
+                                uint32_t head_dim, size_t M, float *freqs_out, float *attn_scale_out,
+                                uint32_t *head_dim_out);
 
 /* ------------------------------------------------------------------ pre-packed activations
  * The reference packs (quantizes) a tile of activations once and then runs the row kernels against the packed

@@ -255,11 +255,25 @@ class HipBackend:
             for b in (d_a, d_b, d_x, d_oa, d_ob):
                 b.free()
 
+    def rope_frequencies(self, M: int, head_dim: int = 0, theta: float = 10000.0, scaling_type: int = 0,
+                         freq_scale: float = 1.0, ext_factor: float = 0.0, attn_factor: float = 1.0,
+                         beta_fast: float = 32.0, beta_slow: float = 1.0, orig_ctx_len: int = 0):
+        """(frequencies [head_dim/2] float32, attention scale, resolved head_dim) for marmot_rope_params_t fields
+        (defaults of marmot_rope_params_default, include/marmot/ops/matmul.h:45-61)."""
+        freqs = np.zeros(max(1, M // 2), dtype=np.float32)
+        scale, hd = C.c_float(0.0), C.c_uint32(0)
+        check(self.lib.marmot_hip_rope_frequencies(scaling_type, theta, freq_scale, ext_factor, attn_factor, beta_fast,
+                                                   beta_slow, orig_ctx_len, head_dim, M, freqs.ctypes.data,
+                                                   C.byref(scale), C.byref(hd)))
+        return freqs[: hd.value // 2].copy(), float(scale.value), int(hd.value)
+
     def linear_qkv(self, x: np.ndarray, wq: np.ndarray, wk: np.ndarray, wv: np.ndarray, kind: int, M: int,
-                   bq=None, bk=None, bv=None):
+                   bq=None, bk=None, bv=None, rope: dict | None = None, positions=None):
         """marmot_matmul_qkv with separate quantized weights of one shape [M, K] (include/marmot/ops/matmul.h:74-95,
         CPU implementation src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:749-947): returns (q, k, v), each [N, M] of
-        the input dtype; biases are optional per projection and must share one dtype (float32 or float16)."""
+        the input dtype; biases are optional per projection and must share one dtype (float32 or float16).
+        rope: keyword arguments of rope_frequencies plus rope_type, apply_to_q, apply_to_k (the rotary epilogue), with
+        positions: N values of float32, int32 or int64."""
         x = np.ascontiguousarray(x)
         N, K = x.shape
         d_w = [self.to_device(np.ascontiguousarray(w, dtype=np.uint8)) for w in (wq, wk, wv)]
@@ -271,15 +285,28 @@ class HipBackend:
         d_b = [None if b is None else self.to_device(b) for b in biases]
         out_dtype = np.dtype(x.dtype)
         d_o = [self.alloc(N * M * out_dtype.itemsize) for _ in range(3)]
+        extra = []
+        rope_arg = None
+        if rope is not None:
+            kw = dict(rope)
+            rope_type = kw.pop("rope_type", 0)
+            aq, ak = kw.pop("apply_to_q", True), kw.pop("apply_to_k", True)
+            freqs, scale, hd = self.rope_frequencies(M, **kw)
+            pos = np.ascontiguousarray(positions)
+            pos_dt = {np.dtype(np.float32): capi.DT_F32, np.dtype(np.int32): capi.DT_I32,
+                      np.dtype(np.int64): capi.DT_I64}[pos.dtype]
+            extra = [self.to_device(pos), self.to_device(freqs)]
+            rope_arg = capi.Rope(extra[0].ptr, pos_dt, extra[1].ptr, scale, hd, rope_type, int(aq), int(ak))
         try:
-            check(self.lib.marmot_hip_matmul_qkv_quantized(
+            check(self.lib.marmot_hip_matmul_qkv_rope_quantized(
                 self.dev, kind, *[C.c_void_p(w.ptr) for w in d_w], C.c_void_p(d_x.ptr), _np_dtype_id(x.dtype), N, K, M,
                 *[C.c_void_p(b.ptr if b is not None else None) for b in d_b],
                 _np_dtype_id(given[0].dtype) if given else 0,
-                *[C.c_void_p(o.ptr) for o in d_o], _np_dtype_id(out_dtype)))
+                *[C.c_void_p(o.ptr) for o in d_o], _np_dtype_id(out_dtype),
+                C.byref(rope_arg) if rope_arg is not None else None))
             return tuple(o.download(out_dtype, (N, M)) for o in d_o)
         finally:
-            for b in d_w + [d_x] + [b for b in d_b if b is not None] + d_o:
+            for b in d_w + [d_x] + [b for b in d_b if b is not None] + d_o + extra:
                 b.free()
 
     def topk(self, x: np.ndarray, k: int):

@@ -8,6 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_K = 1, 5, 9, 11, 12
 DT_F32, DT_F16 = 0, 1
+DT_I32, DT_I64 = 3, 11  # position tensors of the rotary epilogue
 FLAG_FORCE_PACK = 1
 
 ERROR_NAMES = {
@@ -31,6 +32,13 @@ class Caps(C.Structure):
         ("total_mem_bytes", C.c_uint64), ("mem_bw_gbps", C.c_float), ("peak_tflops_fp16", C.c_float),
         ("peak_tops_int8", C.c_float),
     ]
+
+
+class Rope(C.Structure):
+    """marmot_hip_rope_t"""
+    _fields_ = [("d_positions", C.c_void_p), ("positions_dtype", C.c_int), ("d_freqs", C.c_void_p),
+                ("attn_scale", C.c_float), ("head_dim", C.c_uint32), ("rope_type", C.c_int),
+                ("apply_to_q", C.c_int), ("apply_to_k", C.c_int)]
 
 
 _vp, _sz, _i, _u32, _f = C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_float
@@ -67,6 +75,10 @@ SIGNATURES = {
     "marmot_hip_matmul_quantized_dual": (_i, [_vp, _i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _i, _u32]),
     "marmot_hip_matmul_qkv_quantized": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _vp, _i, _vp,
                                              _vp, _vp, _i]),
+    "marmot_hip_matmul_qkv_rope_quantized": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _vp, _i,
+                                                  _vp, _vp, _vp, _i, C.POINTER(Rope)]),
+    "marmot_hip_rope_frequencies": (_i, [_i, _f, _f, _f, _f, _f, _f, _u32, _u32, _sz, _vp, C.POINTER(_f),
+                                         C.POINTER(_u32)]),
     "marmot_hip_packed_activation_bytes": (_sz, [_i, _sz, _sz]),
     "marmot_hip_pack_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
     "marmot_hip_matmul_prepacked": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _vp, _i, _vp, _i]),

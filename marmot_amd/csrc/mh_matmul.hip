@@ -235,6 +235,79 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
                                 out_dtype);
 }
 
+// ------------------------------------------------------------------ rotary epilogue of the Q/K/V projection
+// One thread per (projection, activation row, pair of columns). src: fp32 [N, M] (the projection before the store's
+// rounding: the output itself for fp32 outputs, a workspace for fp16 outputs); dst: [N, M] of the output dtype.
+// A projection that is not rotated is only converted (fp16 outputs) or skipped (fp32, src == dst).
+struct RopeFinishParams {
+    const float *src[3];
+    void *dst[3];
+    int rotate[3];
+    const void *positions;
+    int positions_dtype;
+    const float *freqs;
+    float attn_scale;
+    uint32_t head_dim;
+    int neox;
+    int out_is_f16;
+    size_t N, M;
+};
+
+__global__ __launch_bounds__(256) void k_qkv_rope_finish(const RopeFinishParams p) {
+    warm_kernel_arguments<sizeof(RopeFinishParams)>();
+    const int proj = blockIdx.z;
+    const size_t n = blockIdx.y;
+    const size_t pair = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (pair >= p.M / 2) {
+        return;
+    }
+    const float *src = p.src[proj] + n * p.M;
+    const bool rotate = p.rotate[proj] != 0;
+    if (!rotate && !p.out_is_f16) {
+        return;  // fp32 output already holds the projection
+    }
+    const uint32_t half = p.head_dim / 2;
+    const size_t head = pair / half;
+    const uint32_t i = (uint32_t)(pair - head * half);
+    size_t even_index, odd_index;
+    if (rotate) {
+        even_index = head * p.head_dim + (p.neox ? i : 2 * i);
+        odd_index = head * p.head_dim + (p.neox ? i + half : 2 * i + 1);
+    } else {
+        even_index = 2 * pair;
+        odd_index = 2 * pair + 1;
+    }
+    float even = src[even_index], odd = src[odd_index];
+    if (rotate) {
+        float pos;
+        if (p.positions_dtype == MARMOT_HIP_DTYPE_F32) {
+            pos = ((const float *)p.positions)[n];
+        } else if (p.positions_dtype == MARMOT_HIP_DTYPE_I32) {
+            pos = (float)((const int32_t *)p.positions)[n];
+        } else {
+            pos = (float)((const int64_t *)p.positions)[n];
+        }
+        const float angle = pos * p.freqs[i];
+        float sin_theta, cos_theta;
+        sincosf(angle, &sin_theta, &cos_theta);
+        cos_theta *= p.attn_scale;
+        sin_theta *= p.attn_scale;
+        const float e = even * cos_theta - odd * sin_theta;
+        const float o = even * sin_theta + odd * cos_theta;
+        even = e;
+        odd = o;
+    }
+    if (p.out_is_f16) {
+        uint16_t *dst = (uint16_t *)p.dst[proj] + n * p.M;
+        dst[even_index] = f2h(even);
+        dst[odd_index] = f2h(odd);
+    } else {
+        float *dst = (float *)p.dst[proj] + n * p.M;
+        dst[even_index] = even;
+        dst[odd_index] = odd;
+    }
+}
+
 } // namespace mh
 
 using namespace mh;
@@ -328,6 +401,57 @@ int marmot_hip_matmul_qkv_quantized(marmot_hip_device_t *dev, int kind, const vo
                                     const void *d_wv, const void *d_input, int in_dtype, size_t N, size_t K, size_t M,
                                     const void *d_bq, const void *d_bk, const void *d_bv, int bias_dtype,
                                     void *d_out_q, void *d_out_k, void *d_out_v, int out_dtype) {
+    return marmot_hip_matmul_qkv_rope_quantized(dev, kind, d_wq, d_wk, d_wv, d_input, in_dtype, N, K, M, d_bq, d_bk,
+                                                d_bv, bias_dtype, d_out_q, d_out_k, d_out_v, out_dtype, nullptr);
+}
+
+int marmot_hip_rope_frequencies(int scaling_type, float theta, float freq_scale, float ext_factor,
+                                float attn_factor, float beta_fast, float beta_slow, uint32_t orig_ctx_len,
+                                uint32_t head_dim, size_t M, float *freqs_out, float *attn_scale_out,
+                                uint32_t *head_dim_out) {
+    if (freqs_out == nullptr || attn_scale_out == nullptr || head_dim_out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE frequency span output is null");
+    }
+    // cpu_matmul_qkv_resolve_head_dim (matmul_qkv_rope.h:14-23)
+    size_t hd = head_dim;
+    if (hd == 0 || hd > M || (M % hd) != 0 || (hd & 1u) != 0u) {
+        hd = M;
+    }
+    if ((hd & 1u) != 0u) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE frequency cache requires even dimensions");
+    }
+    // rope_scaling_prepare (src/core/helpers/rope.c:61-110)
+    if (freq_scale <= 0.0f) {
+        freq_scale = 1.0f;
+    }
+    if (attn_factor <= 0.0f) {
+        attn_factor = 1.0f;
+    }
+    if (scaling_type == 0 || scaling_type == -1) {
+        freq_scale = 1.0f;
+        ext_factor = 0.0f;
+    } else if (scaling_type == 1 || scaling_type == 3) {
+        ext_factor = 0.0f;
+    }
+    if (!(ext_factor != 0.0f && orig_ctx_len > 0 && theta > 0.0f && beta_fast > 0.0f && beta_slow > 0.0f)) {
+        ext_factor = 0.0f;
+    }
+    if (ext_factor != 0.0f) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "RoPE: the YaRN frequency ramp is not provided");
+    }
+    *attn_scale_out = attn_factor;
+    *head_dim_out = (uint32_t)hd;
+    for (size_t i = 0; i < hd / 2; ++i) {  // compute_rope_frequencies (rope.c:112-127), host powf like the reference
+        freqs_out[i] = powf(theta, -((float)(2 * i) / (float)hd)) * freq_scale;
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, const void *d_wq, const void *d_wk,
+                                         const void *d_wv, const void *d_input, int in_dtype, size_t N, size_t K,
+                                         size_t M, const void *d_bq, const void *d_bk, const void *d_bv,
+                                         int bias_dtype, void *d_out_q, void *d_out_k, void *d_out_v, int out_dtype,
+                                         const marmot_hip_rope_t *rope) {
     if (dev == nullptr) {
         return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
     }
@@ -353,10 +477,31 @@ int marmot_hip_matmul_qkv_quantized(marmot_hip_device_t *dev, int kind, const vo
     if (K == 0 || M == 0) {
         return set_error(MARMOT_HIP_ERROR_DIMENSION_MISMATCH, "QKV projection dimension mismatch on K");
     }
+    const bool roped = rope != nullptr && (rope->apply_to_q || rope->apply_to_k);
+    if (roped) {
+        if (rope->d_positions == nullptr || rope->d_freqs == nullptr) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE needs positions and frequencies");
+        }
+        if (rope->positions_dtype != MARMOT_HIP_DTYPE_F32 && rope->positions_dtype != MARMOT_HIP_DTYPE_I32 &&
+            rope->positions_dtype != MARMOT_HIP_DTYPE_I64) {
+            return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "RoPE positions must be FLOAT32, INT32 or INT64");
+        }
+        if (rope->head_dim == 0 || (rope->head_dim & 1u) != 0u || M % rope->head_dim != 0) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE head dimension must be even and divide M");
+        }
+        if (rope->rope_type != 0 && rope->rope_type != 1) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE type must be NORM (0) or NEOX (1)");
+        }
+    }
     if (N == 0) {
         return MARMOT_HIP_SUCCESS;
     }
     MH_HIP(hipSetDevice(dev->device_index));
+    // With the rotary epilogue and fp16 outputs the projections are kept in fp32 (workspace) until the rotation has
+    // been applied, so that the store rounds once, after it.
+    const bool stage32 = roped && out_dtype == MARMOT_HIP_DTYPE_F16;
+    const size_t stage_bytes = stage32 ? ((3 * N * M * sizeof(float) + 255) & ~(size_t)255) : 0;
+    const int mm_out_dtype = stage32 ? MARMOT_HIP_DTYPE_F32 : out_dtype;
     WeightSet ws;
     ws.count = 3;
     ws.w[0] = d_wq;
@@ -371,27 +516,68 @@ int marmot_hip_matmul_qkv_quantized(marmot_hip_device_t *dev, int kind, const vo
     ws.bias_dtype = bias_dtype;
     ws.bias_first = true;
     const bool mmq = mmq_supported(kind, N, K);
-    if (!mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input)) {
-        return launch_matvec_set(dev, kind, ws, nullptr, (const float *)d_input, N, K, M, out_dtype);
-    }
+    const bool fuse_quant = !mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input);
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
-    const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
-    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, 3) : 0);
+    const size_t act_bytes =
+        fuse_quant ? 0 : ((act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255);
+    const size_t mmq_bytes = mmq ? ((mmq_scratch_bytes(dev, kind, N, K, M, 3) + 255) & ~(size_t)255) : 0;
     void *wsp = nullptr;
-    int st = workspace_reserve(dev, need, &wsp);
-    if (st != MARMOT_HIP_SUCCESS) {
+    int st = MARMOT_HIP_SUCCESS;
+    if (act_bytes + mmq_bytes + stage_bytes != 0) {
+        st = workspace_reserve(dev, act_bytes + mmq_bytes + stage_bytes, &wsp);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return st;
+        }
+    }
+    float *stage = (float *)((uint8_t *)wsp + act_bytes + mmq_bytes);
+    if (stage32) {
+        for (int i = 0; i < 3; ++i) {
+            ws.out[i] = stage + (size_t)i * N * M;
+        }
+    }
+    if (fuse_quant) {
+        st = launch_matvec_set(dev, kind, ws, nullptr, (const float *)d_input, N, K, M, mm_out_dtype);
+    } else {
+        ActScratch act;
+        act_scratch_layout(act_kind, N, K, wsp, &act);
+        st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return st;
+        }
+        if (mmq) {
+            st = launch_mmq_set(dev, kind, ws, act, N, K, M, mm_out_dtype, (uint8_t *)wsp + act_bytes);
+        } else {
+            st = launch_matvec_set(dev, kind, ws, &act, nullptr, N, K, M, mm_out_dtype);
+        }
+    }
+    if (st != MARMOT_HIP_SUCCESS || !roped) {
         return st;
     }
-    ActScratch act;
-    act_scratch_layout(act_kind, N, K, wsp, &act);
-    st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
-    if (st != MARMOT_HIP_SUCCESS) {
-        return st;
+    RopeFinishParams rp;
+    void *outs[3] = {d_out_q, d_out_k, d_out_v};
+    for (int i = 0; i < 3; ++i) {
+        rp.src[i] = stage32 ? stage + (size_t)i * N * M : (const float *)outs[i];
+        rp.dst[i] = outs[i];
     }
-    if (mmq) {
-        return launch_mmq_set(dev, kind, ws, act, N, K, M, out_dtype, (uint8_t *)wsp + act_bytes);
+    rp.rotate[0] = rope->apply_to_q ? 1 : 0;
+    rp.rotate[1] = rope->apply_to_k ? 1 : 0;
+    rp.rotate[2] = 0;
+    rp.positions = rope->d_positions;
+    rp.positions_dtype = rope->positions_dtype;
+    rp.freqs = rope->d_freqs;
+    rp.attn_scale = rope->attn_scale;
+    rp.head_dim = rope->head_dim;
+    rp.neox = rope->rope_type == 1;
+    rp.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    rp.N = N;
+    rp.M = M;
+    if (N > 65535) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE epilogue: more than 65535 activation rows");
     }
-    return launch_matvec_set(dev, kind, ws, &act, nullptr, N, K, M, out_dtype);
+    const dim3 grid((unsigned)((M / 2 + 255) / 256), (unsigned)N, 3);
+    hipLaunchKernelGGL(k_qkv_rope_finish, grid, dim3(256), 0, dev->stream, rp);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
 }
 
 } // extern "C"

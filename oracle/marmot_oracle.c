@@ -1283,10 +1283,93 @@ int mo_matmul_quantized(
     return MO_OK;
 }
 
+/* cpu_matmul_qkv_resolve_head_dim (matmul_qkv_rope.h:14-23) */
+size_t mo_rope_resolve_head_dim(size_t dim, uint32_t head_dim) {
+    const size_t hd = (size_t)head_dim;
+    if (hd == 0 || hd > dim || (dim % hd) != 0 || (hd & 1u) != 0u) {
+        return dim;
+    }
+    return hd;
+}
+
+/* src/core/helpers/rope.c:61-110 (rope_scaling_prepare), :112-127 (compute_rope_frequencies), :143-200 */
+int mo_rope_frequencies(const mo_rope_params *p, size_t head_dim, float *freqs_out, float *attn_scale_out) {
+    if (p == NULL || freqs_out == NULL || attn_scale_out == NULL || (head_dim & 1u) != 0u) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    float freq_scale = p->freq_scale;
+    float ext_factor = p->ext_factor;
+    float attn_factor = p->attn_factor;
+    if (freq_scale <= 0.0f) {
+        freq_scale = 1.0f;
+    }
+    if (attn_factor <= 0.0f) {
+        attn_factor = 1.0f;
+    }
+    if (p->scaling_type == 0 || p->scaling_type == -1) { /* none / unspecified */
+        freq_scale = 1.0f;
+        ext_factor = 0.0f;
+    } else if (p->scaling_type == 1 || p->scaling_type == 3) { /* linear / longrope */
+        ext_factor = 0.0f;
+    }
+    if (!(ext_factor != 0.0f && p->orig_ctx_len > 0 && p->theta > 0.0f && p->beta_fast > 0.0f &&
+          p->beta_slow > 0.0f)) {
+        ext_factor = 0.0f; /* rope.c:85-93: without the correction range YaRN degenerates to linear scaling */
+    }
+    if (ext_factor != 0.0f) {
+        return MO_ERR_NOT_IMPLEMENTED; /* YaRN ramp: not restated */
+    }
+    *attn_scale_out = attn_factor; /* rope.c:95-99 with ext_factor == 0 */
+    const size_t half = head_dim / 2;
+    for (size_t i = 0; i < half; ++i) { /* rope.c:114-126 */
+        const float freq = powf(p->theta, -((float)(2 * i) / (float)head_dim));
+        freqs_out[i] = freq * freq_scale;
+    }
+    return MO_OK;
+}
+
+/* matmul_qkv_rope.h:50-70 */
+static void rope_rotate_head(float *row, size_t dim, float position, const float *freqs, float attn_scale,
+                             int rope_type) {
+    const size_t pair_count = dim / 2;
+    const size_t half_dim = dim / 2;
+    const int is_neox = rope_type == 1;
+    for (size_t i = 0; i < pair_count; ++i) {
+        const float angle = position * freqs[i];
+        float sin_theta = sinf(angle); /* cpu_sincosf (cpu_backend_internal.h:48-88) */
+        float cos_theta = cosf(angle);
+        cos_theta *= attn_scale;
+        sin_theta *= attn_scale;
+        const size_t even_index = is_neox ? i : 2 * i;
+        const size_t odd_index = is_neox ? (i + half_dim) : (2 * i + 1);
+        const float even = row[even_index];
+        const float odd = row[odd_index];
+        row[even_index] = even * cos_theta - odd * sin_theta;
+        row[odd_index] = even * sin_theta + odd * cos_theta;
+    }
+}
+
+/* matmul_qkv_rope.h:123-138 */
+void mo_rope_rotate_row(float *row, size_t dim, size_t head_dim, float position, const float *freqs, float attn_scale,
+                        int rope_type) {
+    if (row == NULL || freqs == NULL) {
+        return;
+    }
+    if (head_dim >= dim) {
+        rope_rotate_head(row, dim, position, freqs, attn_scale, rope_type);
+        return;
+    }
+    const size_t head_count = dim / head_dim;
+    for (size_t h = 0; h < head_count; ++h) {
+        rope_rotate_head(row + h * head_dim, head_dim, position, freqs, attn_scale, rope_type);
+    }
+}
+
 /* matmul_qkv.c:749-947 (cpu_matmul_qkv_run_separate_quantized_impl), value load/store helpers :89-116 */
-int mo_matmul_qkv_separate(
+int mo_matmul_qkv_separate_rope(
     int kind, const void *const weights[3], const void *input, int in_dtype, size_t N, size_t K, size_t M,
-    const void *const bias[3], int bias_dtype, void *const out[3]
+    const void *const bias[3], int bias_dtype, void *const out[3], const mo_rope_params *rope, const void *positions,
+    int pos_dtype
 ) {
     if (weights == NULL || input == NULL || out == NULL) {
         return MO_ERR_INVALID_ARGUMENT;
@@ -1303,6 +1386,31 @@ int mo_matmul_qkv_separate(
     if (dot == NULL) {
         return MO_ERR_NOT_IMPLEMENTED;
     }
+    /* :809-822: the rotary state exists only when q or k is rotated */
+    const int rope_q = rope != NULL && rope->apply_to_q;
+    const int rope_k = rope != NULL && rope->apply_to_k;
+    size_t head_dim = 0;
+    float *freqs = NULL;
+    float attn_scale = 1.0f;
+    if (rope_q || rope_k) {
+        if (positions == NULL ||
+            (pos_dtype != MO_DTYPE_F32 && pos_dtype != MO_DTYPE_I32 && pos_dtype != MO_DTYPE_I64)) {
+            return MO_ERR_INVALID_ARGUMENT;
+        }
+        head_dim = mo_rope_resolve_head_dim(M, rope->head_dim);
+        if ((head_dim & 1u) != 0u) {
+            return MO_ERR_INVALID_ARGUMENT; /* rope.c:159-162 */
+        }
+        freqs = (float *)malloc((head_dim / 2 + 1) * sizeof(float));
+        if (freqs == NULL) {
+            return MO_ERR_OUT_OF_MEMORY;
+        }
+        const int st = mo_rope_frequencies(rope, head_dim, freqs, &attn_scale);
+        if (st != MO_OK) {
+            free(freqs);
+            return st;
+        }
+    }
     const size_t bv = mo_block_values(kind);
     const size_t bb = mo_block_bytes(kind);
     const size_t blocks_per_row = (K + bv - 1) / bv; /* :802 */
@@ -1310,7 +1418,11 @@ int mo_matmul_qkv_separate(
     const int use_q8_k = (bv == QK_K);
     const size_t act_bb = use_q8_k ? sizeof(blk_q8_k) : sizeof(blk_q8_0);
     uint8_t *act = (uint8_t *)malloc(blocks_per_row * act_bb + 1);
-    if (act == NULL) {
+    float *rows = (float *)malloc(3 * M * sizeof(float) + 1); /* the fp32 row buffers (:824-846, 883-886) */
+    if (act == NULL || rows == NULL) {
+        free(act);
+        free(rows);
+        free(freqs);
         return MO_ERR_OUT_OF_MEMORY;
     }
     const size_t in_elt = in_dtype == MO_DTYPE_F16 ? 2 : 4;
@@ -1329,16 +1441,47 @@ int mo_matmul_qkv_separate(
                                                      : ((const float *)bias[i])[m];
                 }
                 acc += dot((const uint8_t *)weights[i] + m * row_bytes, act, blocks_per_row); /* :902-914 */
+                rows[(size_t)i * M + m] = acc;
+            }
+        }
+        if (rope_q || rope_k) { /* :917-924 -> cpu_matmul_qkv_apply_rope_row (:700-730) */
+            float pos;
+            if (pos_dtype == MO_DTYPE_F32) {
+                pos = ((const float *)positions)[n];
+            } else if (pos_dtype == MO_DTYPE_I32) {
+                pos = (float)((const int32_t *)positions)[n];
+            } else {
+                pos = (float)((const int64_t *)positions)[n];
+            }
+            if (rope_q) {
+                mo_rope_rotate_row(rows, M, head_dim, pos, freqs, attn_scale, rope->rope_type);
+            }
+            if (rope_k) {
+                mo_rope_rotate_row(rows + M, M, head_dim, pos, freqs, attn_scale, rope->rope_type);
+            }
+        }
+        for (int i = 0; i < 3; ++i) { /* the store rounds once (:107-109, 687-698) */
+            for (size_t m = 0; m < M; ++m) {
+                const float v = rows[(size_t)i * M + m];
                 if (in_dtype == MO_DTYPE_F16) {
-                    ((uint16_t *)out[i])[n * M + m] = mo_f32_to_f16(acc); /* :107-109 */
+                    ((uint16_t *)out[i])[n * M + m] = mo_f32_to_f16(v);
                 } else {
-                    ((float *)out[i])[n * M + m] = acc;
+                    ((float *)out[i])[n * M + m] = v;
                 }
             }
         }
     }
     free(act);
+    free(rows);
+    free(freqs);
     return MO_OK;
+}
+
+int mo_matmul_qkv_separate(
+    int kind, const void *const weights[3], const void *input, int in_dtype, size_t N, size_t K, size_t M,
+    const void *const bias[3], int bias_dtype, void *const out[3]
+) {
+    return mo_matmul_qkv_separate_rope(kind, weights, input, in_dtype, N, K, M, bias, bias_dtype, out, NULL, NULL, 0);
 }
 
 /* ======================= top-k / router / MoE ======================= */

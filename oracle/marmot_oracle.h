@@ -45,6 +45,8 @@ enum {
 enum {
     MO_DTYPE_F32 = 0,
     MO_DTYPE_F16 = 1,
+    MO_DTYPE_I32 = 3,
+    MO_DTYPE_I64 = 11,
 };
 
 enum {
@@ -110,6 +112,40 @@ int mo_matmul_quantized(
 int mo_matmul_qkv_separate(
     int kind, const void *const weights[3], const void *input, int in_dtype, size_t N, size_t K, size_t M,
     const void *const bias[3], int bias_dtype, void *const out[3]
+);
+
+/* marmot_rope_params_t without the positions tensor (include/marmot/ops_types.h:98-112) */
+typedef struct {
+    int scaling_type; /* -1 unspecified, 0 none, 1 linear, 2 yarn, 3 longrope (include/marmot/types.h:254-261) */
+    int rope_type;    /* 0 norm: pairs (2i, 2i+1); 1 neox: pairs (i, i + head_dim/2) */
+    float theta, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+    uint32_t orig_ctx_len, head_dim;
+    int apply_to_q, apply_to_k;
+} mo_rope_params;
+
+/* cpu_matmul_qkv_resolve_head_dim (matmul_qkv_rope.h:14-23) */
+size_t mo_rope_resolve_head_dim(size_t dim, uint32_t head_dim);
+
+/*
+ * marmot_rope_freq_cache_ensure without the cache (src/core/helpers/rope.c:61-127, 143-200): head_dim/2 angular
+ * frequencies theta^(-2i/head_dim) * scale and the attention scale. The YaRN ramp (ext_factor != 0 after
+ * rope_scaling_prepare) is not restated: returns MO_ERR_NOT_IMPLEMENTED.
+ */
+int mo_rope_frequencies(const mo_rope_params *p, size_t head_dim, float *freqs_out, float *attn_scale_out);
+
+/* cpu_matmul_qkv_rotate_row_f32_headed (matmul_qkv_rope.h:50-70, 123-138): in-place rotation of one fp32 row */
+void mo_rope_rotate_row(float *row, size_t dim, size_t head_dim, float position, const float *freqs, float attn_scale,
+                        int rope_type);
+
+/*
+ * mo_matmul_qkv_separate with the rotary epilogue (matmul_qkv.c:812-822, 829-831, 917-925, 700-747): q and/or k rows
+ * are rotated in fp32 before the store. positions: N values of pos_dtype (MO_DTYPE_F32, MO_DTYPE_I32 or
+ * MO_DTYPE_I64), converted to float as cpu_rope_position_as_f32 does (cpu_backend_internal.h:567-578).
+ */
+int mo_matmul_qkv_separate_rope(
+    int kind, const void *const weights[3], const void *input, int in_dtype, size_t N, size_t K, size_t M,
+    const void *const bias[3], int bias_dtype, void *const out[3], const mo_rope_params *rope, const void *positions,
+    int pos_dtype
 );
 
 /* top-k over the last axis, ties -> lower index (moe_ops.c:789-889) */

@@ -24,6 +24,25 @@ KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q6_k": KIND_Q
 BLOCK_VALUES = {KIND_Q4_0: 32, KIND_Q8_0: 32, KIND_Q4_K: 256, KIND_Q6_K: 256, KIND_Q8_K: 256}
 BLOCK_BYTES = {KIND_Q4_0: 18, KIND_Q8_0: 34, KIND_Q4_K: 144, KIND_Q6_K: 210, KIND_Q8_K: 292}
 DT_F32, DT_F16 = 0, 1
+DT_I32, DT_I64 = 3, 11  # marmot_dtype_t values of the position tensors the rotary epilogue accepts
+ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_YARN, ROPE_SCALING_LONGROPE = 0, 1, 2, 3
+ROPE_TYPE_NORM, ROPE_TYPE_NEOX = 0, 1
+
+
+class RopeParams(C.Structure):
+    """mo_rope_params: marmot_rope_params_t without the positions tensor."""
+    _fields_ = [("scaling_type", C.c_int), ("rope_type", C.c_int), ("theta", C.c_float), ("freq_scale", C.c_float),
+                ("ext_factor", C.c_float), ("attn_factor", C.c_float), ("beta_fast", C.c_float),
+                ("beta_slow", C.c_float), ("orig_ctx_len", C.c_uint32), ("head_dim", C.c_uint32),
+                ("apply_to_q", C.c_int), ("apply_to_k", C.c_int)]
+
+    @classmethod
+    def default(cls, **kw) -> "RopeParams":
+        """marmot_rope_params_default (include/marmot/ops/matmul.h:45-61)."""
+        p = cls(ROPE_SCALING_NONE, ROPE_TYPE_NORM, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0, 0, 1, 1)
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
 
 
 def row_bytes(kind: int, k: int) -> int:
@@ -74,6 +93,15 @@ class Oracle:
             C.c_int, C.POINTER(C.c_void_p), C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t,
             C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_void_p),
         ]
+        L.mo_matmul_qkv_separate_rope.restype = C.c_int
+        L.mo_matmul_qkv_separate_rope.argtypes = L.mo_matmul_qkv_separate.argtypes + [
+            C.POINTER(RopeParams), C.c_void_p, C.c_int]
+        L.mo_rope_frequencies.restype = C.c_int
+        L.mo_rope_frequencies.argtypes = [C.POINTER(RopeParams), C.c_size_t, C.c_void_p, C.POINTER(C.c_float)]
+        L.mo_rope_resolve_head_dim.restype = C.c_size_t
+        L.mo_rope_resolve_head_dim.argtypes = [C.c_size_t, C.c_uint32]
+        L.mo_rope_rotate_row.restype = None
+        L.mo_rope_rotate_row.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, C.c_void_p, C.c_float, C.c_int]
         L.mo_topk.restype = C.c_int
         L.mo_topk.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
         L.mo_softmax_rows.restype = None
@@ -176,8 +204,26 @@ class Oracle:
             raise RuntimeError(f"mo_matmul_quantized -> {st}")
         return out
 
-    def matmul_qkv(self, kind: int, wq, wk, wv, x: np.ndarray, M: int, bq=None, bk=None, bv=None):
-        """marmot_matmul_qkv with separate quantized weights; returns (q, k, v) of x's dtype (float32 or float16)."""
+    def rope_frequencies(self, rope: "RopeParams", head_dim: int):
+        """(angular frequencies [head_dim / 2], attention scale) of marmot_rope_freq_cache_ensure."""
+        freqs = np.zeros(head_dim // 2, dtype=np.float32)
+        scale = C.c_float(0.0)
+        st = self.L.mo_rope_frequencies(C.byref(rope), head_dim, _ptr(freqs), C.byref(scale))
+        if st != 0:
+            raise RuntimeError(f"mo_rope_frequencies -> {st}")
+        return freqs, float(scale.value)
+
+    def rope_rotate_row(self, row: np.ndarray, head_dim: int, position: float, freqs: np.ndarray, attn_scale: float,
+                        rope_type: int) -> np.ndarray:
+        out = np.ascontiguousarray(row, dtype=np.float32).copy()
+        freqs = np.ascontiguousarray(freqs, dtype=np.float32)
+        self.L.mo_rope_rotate_row(_ptr(out), out.shape[0], head_dim, position, _ptr(freqs), attn_scale, rope_type)
+        return out
+
+    def matmul_qkv(self, kind: int, wq, wk, wv, x: np.ndarray, M: int, bq=None, bk=None, bv=None, rope=None,
+                   positions=None):
+        """marmot_matmul_qkv with separate quantized weights; returns (q, k, v) of x's dtype (float32 or float16).
+        rope: RopeParams (rotary epilogue on q and/or k) with positions: N values, float32, int32 or int64."""
         ws = [np.ascontiguousarray(w, dtype=np.uint8) for w in (wq, wk, wv)]
         if x.dtype != np.float16:
             x = x.astype(np.float32, copy=False)
@@ -192,12 +238,18 @@ class Oracle:
         bias_dt = DT_F16 if given and given[0].dtype == np.float16 else DT_F32
         outs = [np.zeros((N, M), dtype=x.dtype) for _ in range(3)]
         arr = C.c_void_p * 3
-        st = self.L.mo_matmul_qkv_separate(
+        pos, pos_dt = None, 0
+        if rope is not None:
+            pos = np.ascontiguousarray(positions)
+            pos_dt = {np.dtype(np.float32): DT_F32, np.dtype(np.int32): DT_I32, np.dtype(np.int64): DT_I64}[pos.dtype]
+            assert pos.shape == (N,)
+        st = self.L.mo_matmul_qkv_separate_rope(
             kind, arr(*[w.ctypes.data for w in ws]), _ptr(x), in_dt, N, K, M,
             arr(*[None if b is None else b.ctypes.data for b in biases]), bias_dt, arr(*[o.ctypes.data for o in outs]),
+            C.byref(rope) if rope is not None else None, _ptr(pos) if pos is not None else None, pos_dt,
         )
         if st != 0:
-            raise RuntimeError(f"mo_matmul_qkv_separate -> {st}")
+            raise RuntimeError(f"mo_matmul_qkv_separate_rope -> {st}")
         return tuple(outs)
 
     # ---- MoE

@@ -113,3 +113,76 @@ def test_qkv_error_codes(hip, oracle):
     finally:
         for b in (d_w, d_x, d_o):
             b.free()
+
+
+# ---------------------------------------------------------------- rotary epilogue
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("N", [1, 4, 6, 19])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_qkv_rope_epilogue(hip, oracle, name, N, dtype):
+    """q and/or k rotated in fp32 before the store, v untouched; NORM and NEOX pairs; int32, int64 and float32
+    positions; a head dimension that splits the row into heads and one that does not divide it (whole row = one
+    head, as cpu_matmul_qkv_resolve_head_dim decides)."""
+    from oracle.pyoracle import RopeParams
+
+    kind = KINDS[name]
+    M, K = 256, 1024
+    ws = _weights(oracle, kind, M, K, 700)
+    x = gaussian(710 + N, (N, K)).astype(dtype)
+    bias = [gaussian(720 + i, (M,)).astype(dtype) for i in range(3)]
+    rng = np.random.default_rng(730 + N)
+    cases = [
+        (dict(head_dim=64, theta=500000.0), 0, True, True, rng.integers(0, 8192, N).astype(np.int32)),
+        (dict(head_dim=128, theta=10000.0), 1, True, False, rng.integers(0, 4096, N).astype(np.int64)),
+        (dict(head_dim=96, theta=10000.0, scaling_type=1, freq_scale=0.25, attn_factor=1.25), 1, False, True,
+         (rng.random(N) * 100).astype(np.float32)),
+    ]
+    for kw, rope_type, aq, ak, pos in cases:
+        rope = RopeParams.default(rope_type=rope_type, apply_to_q=int(aq), apply_to_k=int(ak), **kw)
+        ref = oracle.matmul_qkv(kind, *ws, x, M, bq=bias[0], bk=bias[1], bv=bias[2], rope=rope, positions=pos)
+        got = hip.linear_qkv(x, *ws, kind, M, bq=bias[0], bk=bias[1], bv=bias[2], positions=pos,
+                             rope=dict(kw, rope_type=rope_type, apply_to_q=aq, apply_to_k=ak))
+        for g, r, what in zip(got, ref, "qkv"):
+            assert g.dtype == dtype
+            g32, r32 = g.astype(np.float32), r.astype(np.float32)
+            if dtype == np.float32:
+                assert_matmul_parity(g32, r32, what=f"{name} N={N} rope case {kw} {what}")
+            else:
+                assert np.max(np.abs(g32 - r32)) <= 1e-3 * np.abs(r32).max()
+                assert np.mean(g.view(np.uint16) == r.view(np.uint16)) > 0.97
+    # the frequencies come from the host with the reference's formula: same bits as the oracle's
+    f_hip, a_hip, hd = hip.rope_frequencies(M, head_dim=64, theta=500000.0)
+    f_ref, a_ref = oracle.rope_frequencies(RopeParams.default(head_dim=64, theta=500000.0), 64)
+    assert hd == 64 and a_hip == a_ref and np.array_equal(f_hip, f_ref)
+
+
+def test_qkv_rope_errors(hip, oracle):
+    kind, M, K = KIND_Q4_K, 64, 256
+    ws = _weights(oracle, kind, M, K, 740)
+    x = gaussian(741, (2, K))
+    pos = np.array([1, 2], np.int32)
+    with pytest.raises(capi.MarmotHipError) as e:  # the YaRN ramp is declined, not approximated
+        hip.linear_qkv(x, *ws, kind, M, positions=pos,
+                       rope=dict(scaling_type=2, ext_factor=1.0, freq_scale=0.5, orig_ctx_len=4096))
+    assert e.value.code == -8
+    # YaRN parameters without an original context length degenerate to linear scaling (rope.c:85-93)
+    q, _, _ = hip.linear_qkv(x, *ws, kind, M, positions=pos, rope=dict(scaling_type=2, ext_factor=1.0, freq_scale=0.5))
+    from oracle.pyoracle import RopeParams
+    rq, _, _ = oracle.matmul_qkv(kind, *ws, x, M, positions=pos,
+                                 rope=RopeParams.default(scaling_type=2, ext_factor=1.0, freq_scale=0.5))
+    assert_matmul_parity(q, rq, what="degenerate yarn")
+    d = [hip.to_device(w) for w in ws] + [hip.to_device(x), hip.alloc(2 * M * 4)]
+    try:
+        bad = capi.Rope(None, capi.DT_I32, None, 1.0, 64, 0, 1, 1)
+        st = hip.lib.marmot_hip_matmul_qkv_rope_quantized(
+            hip.dev, kind, *[C.c_void_p(b.ptr) for b in d[:3]], C.c_void_p(d[3].ptr), capi.DT_F32, 2, K, M, None, None,
+            None, 0, *[C.c_void_p(d[4].ptr)] * 3, capi.DT_F32, C.byref(bad))
+        assert st == -1  # positions / frequencies missing
+        bad = capi.Rope(d[3].ptr, capi.DT_I32, d[3].ptr, 1.0, 48, 0, 1, 1)
+        st = hip.lib.marmot_hip_matmul_qkv_rope_quantized(
+            hip.dev, kind, *[C.c_void_p(b.ptr) for b in d[:3]], C.c_void_p(d[3].ptr), capi.DT_F32, 2, K, M, None, None,
+            None, 0, *[C.c_void_p(d[4].ptr)] * 3, capi.DT_F32, C.byref(bad))
+        assert st == -1  # head dimension does not divide M
+    finally:
+        for b in d:
+            b.free()

@@ -92,3 +92,101 @@ def test_qkv_rejects_other_input_types(oracle):
     st = oracle.L.mo_matmul_qkv_separate(kind, arr(*[w.ctypes.data] * 3), x.ctypes.data, 99, 1, K, M,
                                          arr(None, None, None), DT_F32, arr(*[o.ctypes.data for o in outs]))
     assert st == -8  # MARMOT_ERROR_NOT_IMPLEMENTED (matmul_qkv.c:761-763)
+
+
+# ---------------------------------------------------------------- rotary epilogue
+# Pinned by the closed form the reference's own rope test uses as its expectation (tests/backend/test_rope.c:5-42:
+# freq_i = theta^(-2i/dim), angle = position * freq_i, a plane rotation of each pair), evaluated here in float64,
+# and by what the mathematics fixes: rotations preserve the norm of every pair, position 0 is the identity,
+# rotating by p then by -p restores the row, NORM and NEOX are the same rotation under a permutation of the columns.
+
+def _rope_f64(row, head_dim, pos, theta, rope_type, freq_scale=1.0, attn=1.0):
+    row = row.astype(np.float64).copy()
+    half = head_dim // 2
+    i = np.arange(half, dtype=np.float64)
+    ang = pos * freq_scale * theta ** (-(2.0 * i) / head_dim)
+    c, s = np.cos(ang) * attn, np.sin(ang) * attn
+    for h in range(row.shape[0] // head_dim):
+        seg = row[h * head_dim:(h + 1) * head_dim]
+        if rope_type == 1:
+            e, o = seg[:half].copy(), seg[half:].copy()
+            seg[:half], seg[half:] = e * c - o * s, e * s + o * c
+        else:
+            e, o = seg[0::2].copy(), seg[1::2].copy()
+            seg[0::2], seg[1::2] = e * c - o * s, e * s + o * c
+    return row
+
+
+def test_rope_frequencies_and_rotation_closed_form(oracle):
+    from oracle.pyoracle import ROPE_SCALING_LINEAR, ROPE_SCALING_YARN, RopeParams
+
+    for head_dim, theta in ((64, 10000.0), (128, 500000.0)):
+        f, a = oracle.rope_frequencies(RopeParams.default(theta=theta), head_dim)
+        want = theta ** (-(2.0 * np.arange(head_dim // 2)) / head_dim)
+        assert a == 1.0 and np.allclose(f, want, rtol=2e-6, atol=0) and f[0] == 1.0
+        # without a scaling type the scale factors are ignored; linear scaling multiplies every frequency
+        f2, _ = oracle.rope_frequencies(RopeParams.default(theta=theta, freq_scale=0.25), head_dim)
+        assert np.array_equal(f2, f)
+        f3, a3 = oracle.rope_frequencies(
+            RopeParams.default(theta=theta, freq_scale=0.25, attn_factor=1.5, scaling_type=ROPE_SCALING_LINEAR), head_dim)
+        assert np.array_equal(f3, f * np.float32(0.25)) and a3 == 1.5
+    with pytest.raises(RuntimeError):  # the YaRN ramp is not restated
+        oracle.rope_frequencies(RopeParams.default(scaling_type=ROPE_SCALING_YARN, ext_factor=1.0, freq_scale=0.5,
+                                                   orig_ctx_len=4096), 64)
+    assert oracle.L.mo_rope_resolve_head_dim(512, 128) == 128
+    for bad in (0, 1024, 96, 7):  # absent, larger than the row, not a divisor, odd
+        assert oracle.L.mo_rope_resolve_head_dim(512, bad) == 512
+
+    rng = np.random.default_rng(540)
+    row = rng.standard_normal(256).astype(np.float32)
+    for rope_type in (0, 1):
+        for head_dim in (64, 256):
+            f, a = oracle.rope_frequencies(RopeParams.default(), head_dim)
+            for pos in (0.0, 1.0, 37.0, 4095.0):
+                got = oracle.rope_rotate_row(row, head_dim, pos, f, a, rope_type)
+                want = _rope_f64(row, head_dim, pos, 10000.0, rope_type)
+                # fp32 frequencies and angles: the angle is off by up to ~2^-23 * position radians
+                assert np.max(np.abs(got - want)) <= (1e-6 + 1.5e-7 * pos) * np.abs(row).max()
+                if pos == 0.0:
+                    assert np.array_equal(got, row)
+                # pair norms are preserved
+                pairs = (lambda v: v.reshape(-1, 2, head_dim // 2).transpose(0, 2, 1)) if rope_type == 1 else \
+                    (lambda v: v.reshape(-1, head_dim // 2, 2))
+                assert np.allclose(np.linalg.norm(pairs(got), axis=-1), np.linalg.norm(pairs(row), axis=-1), rtol=1e-5)
+                back = oracle.rope_rotate_row(got, head_dim, -pos, f, a, rope_type)
+                assert np.allclose(back, row, atol=1e-5)
+    # NEOX = NORM on columns permuted (2i, 2i+1) -> (i, i + half)
+    head_dim = 64
+    f, a = oracle.rope_frequencies(RopeParams.default(), head_dim)
+    perm = np.concatenate([np.arange(0, head_dim, 2), np.arange(1, head_dim, 2)])
+    full = np.concatenate([perm + h * head_dim for h in range(4)])
+    norm = oracle.rope_rotate_row(row, head_dim, 11.0, f, a, 0)
+    neox = oracle.rope_rotate_row(row[full], head_dim, 11.0, f, a, 1)
+    assert np.array_equal(neox, norm[full])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_qkv_rope_epilogue_is_projection_then_rotation(oracle, dtype):
+    from oracle.pyoracle import RopeParams
+
+    kind, M, K, N = KIND_Q4_K, 128, 512, 5
+    ws = [oracle.quantize(kind, gaussian(550 + i, (M, K), 0.02)) for i in range(3)]
+    x = gaussian(553, (N, K)).astype(dtype)
+    bias = [gaussian(554 + i, (M,)).astype(dtype) for i in range(3)]
+    plain = _expected(oracle, kind, ws, x, M, [b.astype(np.float32) for b in bias])  # fp32, before any rounding
+    for pos in (np.array([0, 1, 2, 3, 900], np.int32), np.array([5, 4, 3, 2, 1], np.int64),
+                np.array([0.5, 7.0, 8.0, 9.0, 10.0], np.float32)):
+        for rope_type in (0, 1):
+            for aq, ak in ((1, 1), (1, 0), (0, 1), (0, 0)):
+                rope = RopeParams.default(head_dim=64, rope_type=rope_type, apply_to_q=aq, apply_to_k=ak,
+                                          theta=500000.0)
+                q, k, v = oracle.matmul_qkv(kind, *ws, x, M, bq=bias[0], bk=bias[1], bv=bias[2], rope=rope,
+                                            positions=pos)
+                f, a = oracle.rope_frequencies(rope, 64)
+                for out, base, rot in ((q, plain[0], aq), (k, plain[1], ak), (v, plain[2], 0)):
+                    want = base.copy()
+                    if rot:
+                        for n in range(N):
+                            want[n] = oracle.rope_rotate_row(base[n], 64, float(np.float32(pos[n])), f, a, rope_type)
+                    assert out.dtype == dtype
+                    assert np.array_equal(bits(out), bits(want.astype(dtype)))  # one rounding, after the rotation

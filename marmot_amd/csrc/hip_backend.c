@@ -42,11 +42,27 @@ typedef struct {
     bool dev_newer;   // a kernel wrote the mirror since the last download
 } hip_mirror_t;
 
+// Rotary frequencies of one parameter set (the counterpart of marmot_rope_freq_cache_t, src/core/helpers/rope.h):
+// computed on the host with the reference's formula, mirrored to the device through the residency table.
+typedef struct {
+    bool used;
+    int scaling_type;
+    float theta, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+    uint32_t orig_ctx_len, head_dim_in;
+    size_t M;
+    uint32_t head_dim;  // resolved
+    float attn_scale;
+    float *freqs;       // head_dim / 2 values, owned
+} hip_rope_entry_t;
+#define HIP_ROPE_CACHE 8
+
 typedef struct {
     marmot_hip_device_t *dev;
     pthread_mutex_t mu;
     hip_mirror_t *mirrors;  // sorted by host
     size_t n_mirrors, cap_mirrors;
+    hip_rope_entry_t rope[HIP_ROPE_CACHE];
+    size_t rope_next;
     bool batching;
     uint64_t uploads, upload_bytes, downloads, download_bytes;
     size_t mirrored_bytes;
@@ -292,6 +308,9 @@ static void ops_destroy(const void *device_ctx) {
         marmot_hip_free(b->dev, b->mirrors[i].dev);
     }
     free(b->mirrors);
+    for (size_t i = 0; i < HIP_ROPE_CACHE; ++i) {
+        free(b->rope[i].freqs);
+    }
     marmot_hip_device_destroy(b->dev);
     pthread_mutex_destroy(&b->mu);
     free(b);
@@ -614,6 +633,58 @@ static marmot_error_t matmul_quantized(const void *device_ctx, marmot_quant_kind
 // marmot_matmul_qkv, separate block-quantized weights. Checks in the order of cpu_matmul_qkv_validate_desc
 // (src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:1140-1146, 1230-1300), cpu_matmul_qkv_quant_entry (:1424-1434) and
 // cpu_matmul_qkv_run_separate_quantized_impl (:761-789).
+// Finds or builds the frequency entry for these parameters (mutex held). An evicted entry's mirror is dropped first.
+static marmot_error_t rope_entry_locked(hip_backend_t *b, const marmot_rope_params_t *r, size_t M,
+                                        hip_rope_entry_t **out) {
+    for (size_t i = 0; i < HIP_ROPE_CACHE; ++i) {
+        hip_rope_entry_t *e = &b->rope[i];
+        if (e->used && e->scaling_type == (int)r->scaling_type && e->theta == r->theta &&
+            e->freq_scale == r->freq_scale && e->ext_factor == r->ext_factor && e->attn_factor == r->attn_factor &&
+            e->beta_fast == r->beta_fast && e->beta_slow == r->beta_slow && e->orig_ctx_len == r->orig_ctx_len &&
+            e->head_dim_in == r->head_dim && e->M == M) {
+            *out = e;
+            return MARMOT_SUCCESS;
+        }
+    }
+    float *freqs = malloc((M / 2 + 1) * sizeof(float));
+    if (freqs == nullptr) {
+        return fail(MARMOT_ERROR_OUT_OF_MEMORY, "Failed to allocate RoPE frequency buffer");
+    }
+    float attn_scale = 1.0f;
+    uint32_t head_dim = 0;
+    const int rc = marmot_hip_rope_frequencies((int)r->scaling_type, r->theta, r->freq_scale, r->ext_factor,
+                                               r->attn_factor, r->beta_fast, r->beta_slow, r->orig_ctx_len,
+                                               r->head_dim, M, freqs, &attn_scale, &head_dim);
+    if (rc != MARMOT_HIP_SUCCESS) {
+        free(freqs);
+        return fail_from_lib(rc);
+    }
+    hip_rope_entry_t *e = &b->rope[b->rope_next];
+    b->rope_next = (b->rope_next + 1) % HIP_ROPE_CACHE;
+    if (e->used && e->freqs != nullptr) {
+        bool synced = false;
+        for (size_t i = 0; i < b->n_mirrors;) {
+            if (!overlaps(&b->mirrors[i], (uintptr_t)e->freqs, (size_t)e->head_dim / 2 * sizeof(float))) {
+                ++i;
+                continue;
+            }
+            if (!synced) {
+                marmot_hip_synchronize(b->dev);
+                synced = true;
+            }
+            drop_at(b, i);
+        }
+        free(e->freqs);
+    }
+    *e = (hip_rope_entry_t){.used = true, .scaling_type = (int)r->scaling_type, .theta = r->theta,
+                            .freq_scale = r->freq_scale, .ext_factor = r->ext_factor,
+                            .attn_factor = r->attn_factor, .beta_fast = r->beta_fast, .beta_slow = r->beta_slow,
+                            .orig_ctx_len = r->orig_ctx_len, .head_dim_in = r->head_dim, .M = M,
+                            .head_dim = head_dim, .attn_scale = attn_scale, .freqs = freqs};
+    *out = e;
+    return MARMOT_SUCCESS;
+}
+
 static marmot_error_t qkv_locked(hip_backend_t *b, const marmot_matmul_qkv_desc_t *desc, int kind, int dtype, size_t N,
                                  size_t K, size_t M) {
     const marmot_tensor_t *w[3] = {desc->separate.wq, desc->separate.wk, desc->separate.wv};
@@ -634,8 +705,39 @@ static marmot_error_t qkv_locked(hip_backend_t *b, const marmot_matmul_qkv_desc_
     if (st != MARMOT_SUCCESS) {
         return st;
     }
-    const int rc = marmot_hip_matmul_qkv_quantized(b->dev, kind, d_w[0], d_w[1], d_w[2], d_x, dtype, N, K, M, d_b[0],
-                                                   d_b[1], d_b[2], dtype, d_o[0], d_o[1], d_o[2], dtype);
+    const marmot_rope_params_t *r = desc->rope_params;
+    marmot_hip_rope_t rope;
+    const marmot_hip_rope_t *rope_ptr = nullptr;
+    if (r != nullptr && (r->apply_to_q || r->apply_to_k)) {
+        hip_rope_entry_t *e = nullptr;
+        st = rope_entry_locked(b, r, M, &e);
+        const void *d_pos = nullptr, *d_freqs = nullptr;
+        if (st == MARMOT_SUCCESS) {
+            st = acquire_read(b, r->positions->data, dense_bytes(r->positions), &d_pos);
+        }
+        if (st == MARMOT_SUCCESS) {
+            st = acquire_read(b, e->freqs, (size_t)e->head_dim / 2 * sizeof(float), &d_freqs);
+        }
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+        rope = (marmot_hip_rope_t){
+            .d_positions = d_pos,
+            .positions_dtype = r->positions->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32
+                : r->positions->dtype == MARMOT_DTYPE_INT32               ? MARMOT_HIP_DTYPE_I32
+                                                                          : MARMOT_HIP_DTYPE_I64,
+            .d_freqs = d_freqs,
+            .attn_scale = e->attn_scale,
+            .head_dim = e->head_dim,
+            .rope_type = r->rope_type == MARMOT_ROPE_TYPE_NEOX ? 1 : 0,
+            .apply_to_q = r->apply_to_q,
+            .apply_to_k = r->apply_to_k,
+        };
+        rope_ptr = &rope;
+    }
+    const int rc = marmot_hip_matmul_qkv_rope_quantized(b->dev, kind, d_w[0], d_w[1], d_w[2], d_x, dtype, N, K, M,
+                                                        d_b[0], d_b[1], d_b[2], dtype, d_o[0], d_o[1], d_o[2], dtype,
+                                                        rope_ptr);
     if (rc != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(rc);
     }
@@ -727,7 +829,21 @@ static marmot_error_t matmul_qkv(const void *device_ctx, marmot_quant_kind_t exp
         return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "QKV projection: HIP kernels need contiguous rows");
     }
     if (desc->rope_params != nullptr && (desc->rope_params->apply_to_q || desc->rope_params->apply_to_k)) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "QKV projection: the rotary epilogue is not provided");
+        const marmot_tensor_t *pos = desc->rope_params->positions;
+        if (pos == nullptr || pos->data == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: RoPE needs a positions tensor");
+        }
+        if (pos->dtype != MARMOT_DTYPE_FLOAT32 && pos->dtype != MARMOT_DTYPE_INT32 &&
+            pos->dtype != MARMOT_DTYPE_INT64) {
+            return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "QKV projection: RoPE positions must be FLOAT32, INT32 or INT64");
+        }
+        if (tensor_numel(pos) < N) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "QKV projection: fewer RoPE positions than activation rows");
+        }
+        if (desc->rope_params->rope_type != MARMOT_ROPE_TYPE_NORM &&
+            desc->rope_params->rope_type != MARMOT_ROPE_TYPE_NEOX) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: unknown RoPE type");
+        }
     }
     if (input->data == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "QKV projection: tensor without data");
@@ -1347,8 +1463,9 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         if (sig->stride_mode != MARMOT_STRIDE_MODE_CONTIGUOUS && sig->stride_mode != MARMOT_STRIDE_MODE_ANY) {
             return unsupported("HIP QKV projection needs contiguous rows");
         }
-        if ((sig->epilogue_flags & ~(uint32_t)MARMOT_EPILOGUE_BIAS) != 0 || sig->variant_flags != 0) {
-            return unsupported("HIP QKV projection fuses only the bias epilogue (no rotary embedding)");
+        if ((sig->epilogue_flags & ~(uint32_t)(MARMOT_EPILOGUE_BIAS | MARMOT_EPILOGUE_ROPE)) != 0 ||
+            sig->variant_flags != 0) {
+            return unsupported("HIP QKV projection fuses the bias and rotary epilogues only");
         }
         const size_t N = sig->dims.matmul.N, K = sig->dims.matmul.K, M = sig->dims.matmul.M;
         const double bytes = 3.0 * (double)M * (double)marmot_hip_row_bytes(kind, K) +

@@ -207,7 +207,9 @@ def test_query_kernel_qkv_rules(lib, golden_layout):
     assert not _query(lib, s).supported  # outputs must have the activation dtype
     s = _sig(op=ta.OP_QKV_SHARED_INPUT); s.epilogue_flags = ta.EPILOGUE_BIAS
     assert _query(lib, s).supported
-    s = _sig(op=ta.OP_QKV_ROPE); s.epilogue_flags = ta.EPILOGUE_BIAS | ta.EPILOGUE_ROPE
+    s = _sig(op=ta.OP_QKV_SHARED_INPUT); s.epilogue_flags = ta.EPILOGUE_BIAS | ta.EPILOGUE_ROPE
+    assert _query(lib, s).supported
+    s = _sig(op=ta.OP_QKV_SHARED_INPUT); s.epilogue_flags = ta.EPILOGUE_ROPE | 2  # activation epilogue
     sel = _query(lib, s)
     assert not sel.supported and b"rotary" in sel.fallback_reason
     assert not _query(lib, _sig(op=ta.OP_QKV_SHARED_INPUT, kind=ta.KIND_Q8_K)).supported
@@ -311,7 +313,7 @@ def test_kernel_def_files_name_exported_impls(lib):
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip"} | qkv
     for name in qkv:
         f = families[name]
-        assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS]" and f["OP"] in name
+        assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name
     for name, f in families.items():
         impl = f["IMPL_FUNCTION"].strip('"')
         schemes = re.findall(r"Q\d_[0K]", f.get("AXIS(scheme)", "")) or [""]

@@ -362,9 +362,66 @@ def test_impl_qkv_errors(ctx, oracle):
     d, keep = build(wk_kind=KIND_Q6_K)
     assert fn(ctx.device_ctx, C.byref(d)) == ta.NOT_IMPLEMENTED
     rope = ta.RopeParams()
-    rope.apply_to_q = True
+    rope.theta, rope.freq_scale, rope.attn_factor, rope.apply_to_q = 10000.0, 1.0, 1.0, True
+    d, keep = build(rope=rope)  # no positions tensor
+    assert fn(ctx.device_ctx, C.byref(d)) == ta.INVALID_ARGUMENT and "positions" in ctx.last_error()[1]
+    pos = ta.HostTensor.dense(np.zeros(N, np.int8))
+    rope.positions = pos.ptr
     d, keep = build(rope=rope)
-    assert fn(ctx.device_ctx, C.byref(d)) == ta.NOT_IMPLEMENTED and "rotary" in ctx.last_error()[1]
+    assert fn(ctx.device_ctx, C.byref(d)) == ta.UNSUPPORTED_DTYPE
+    pos1 = ta.HostTensor.dense(np.zeros(N - 1, np.int32))
+    rope.positions = pos1.ptr
+    d, keep = build(rope=rope)
+    assert fn(ctx.device_ctx, C.byref(d)) == ta.DIMENSION_MISMATCH
+    pos2 = ta.HostTensor.dense(np.arange(N, dtype=np.int32))
+    rope.positions = pos2.ptr
+    rope.scaling_type, rope.ext_factor, rope.freq_scale, rope.orig_ctx_len = 2, 1.0, 0.5, 4096
+    rope.beta_fast, rope.beta_slow = 32.0, 1.0
+    d, keep = build(rope=rope)  # the YaRN ramp is declined
+    assert fn(ctx.device_ctx, C.byref(d)) == ta.NOT_IMPLEMENTED and "YaRN" in ctx.last_error()[1]
     rope.apply_to_q = False  # parameters present but applied to neither q nor k: plain projection (matmul_qkv.c:812-814)
+    rope.positions = None
     d, keep = build(rope=rope)
     assert fn(ctx.device_ctx, C.byref(d)) == ta.SUCCESS
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_program_qkv_with_rotary_epilogue(ctx, oracle, dtype):
+    """QKV_SHARED_INPUT with the ROPE epilogue as the graph emits it (graph_builder.cpp:384-394): rope parameters in
+    the constant pool, positions as a tensor; the frequency table is mirrored once and reused by the second run."""
+    from oracle.pyoracle import RopeParams as OracleRope
+
+    kind, M, K, N = KIND_Q4_K, 256, 1024, 7
+    ws = [oracle.quantize(kind, gaussian(940 + i, (M, K), 0.02)) for i in range(3)]
+    x = gaussian(943, (N, K)).astype(dtype)
+    biases = [gaussian(944 + i, (M,)).astype(dtype) for i in range(3)]
+    positions = np.array([0, 1, 2, 3, 4, 500, 8000], np.int32)
+    xt, wts, outs, bts = _qkv_tensors(kind, ws, M, K, x, biases)
+    pt = ta.HostTensor.dense(positions)
+    sel = ctx.query(ctx.qkv_signature(xt, wts[0], outs[0], bias=True, rope=True))
+    assert sel.supported and sel.op_index == 14
+    for rope_type in (0, 1):
+        rp = ta.RopeParams()
+        rp.positions = pt.ptr
+        rp.scaling_type, rp.rope_type, rp.theta, rp.freq_scale, rp.ext_factor, rp.attn_factor = 0, rope_type, 500000.0, 1.0, 0.0, 1.0
+        rp.beta_fast, rp.beta_slow, rp.orig_ctx_len, rp.head_dim, rp.apply_to_q, rp.apply_to_k = 32.0, 1.0, 0, 64, True, True
+        ref = oracle.matmul_qkv(kind, *ws, x, M, bq=biases[0], bk=biases[1], bv=biases[2], positions=positions,
+                                rope=OracleRope.default(theta=500000.0, head_dim=64, rope_type=rope_type))
+        before = ctx.residency().uploads
+        for run in range(2):
+            prog = ta.Program()
+            prog.qkv(sel.op_index, xt, *wts, *outs, bq=bts[0], bk=bts[1], bv=bts[2], rope=rp)
+            assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+            for o, r in zip(outs, ref):
+                got = ctx.to_host(o).astype(np.float32)
+                r32 = r.astype(np.float32)
+                if dtype == np.float32:
+                    assert_matmul_parity(got, r32, what=f"program qkv rope type={rope_type}")
+                else:
+                    assert np.max(np.abs(got - r32)) <= 1e-3 * np.abs(r32).max()
+            if run == 0:
+                first_uploads = ctx.residency().uploads - before
+        # second run: nothing is uploaded again (weights, biases, positions and the frequency table stay resident)
+        assert ctx.residency().uploads - before == first_uploads
+    for t in [xt, pt] + wts + outs + bts:
+        ctx.host_freed(t)

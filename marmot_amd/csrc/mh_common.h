@@ -138,8 +138,12 @@ namespace mh {
 // Kernel arguments are fetched through the scalar cache, one 64-byte line per miss, each on first use: a kernel whose
 // arguments span several lines pays those misses one after the other along its prologue (and again in its epilogue
 // for fields first read there). Touching every line at kernel entry overlaps them into one miss (measured: 0.3-0.5 us
-// per launch). BYTES: size of the explicit arguments (nothing beyond them is read).
-template <int BYTES>
+// per launch). BYTES: the explicit arguments to cover. EXPLICIT_SIZE: for a kernel that reads blockDim or gridDim, the
+// size of ALL its explicit arguments: the launch dimensions are hidden arguments stored right behind them (block
+// counts, then group sizes), usually in a line of their own, and are needed by the first instructions (measured:
+// 0.25 us per launch when the explicit arguments grew and pushed them out of a line that was touched anyway).
+// Leave EXPLICIT_SIZE at 0 for a kernel that does not read them: its argument segment may end with the explicit ones.
+template <int BYTES, int EXPLICIT_SIZE = 0>
 __device__ __forceinline__ void warm_kernel_arguments() {
     const uint32_t __attribute__((address_space(4))) *kargs =
         (const uint32_t __attribute__((address_space(4))) *)__builtin_amdgcn_kernarg_segment_ptr();
@@ -147,6 +151,10 @@ __device__ __forceinline__ void warm_kernel_arguments() {
 #pragma unroll
     for (int off = 0; off < BYTES - 4; off += 64) {
         touched ^= kargs[off / 4];
+    }
+    if (EXPLICIT_SIZE > 0) {
+        constexpr int hidden = (EXPLICIT_SIZE + 7) & ~7;  // block counts at +0..11, group sizes at +12..17
+        touched ^= kargs[hidden / 4] ^ kargs[(hidden + 16) / 4];
     }
     asm volatile("" ::"s"(touched));
 }

@@ -434,7 +434,7 @@ template <int V>
 __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ partial, int splits, size_t N, size_t M,
                                                      const void *bias, int bias_is_f16, void *out, int out_is_f16,
                                                      int bias_first) {
-    warm_kernel_arguments<8 * 8 + 4>();
+    warm_kernel_arguments<8 * 8 + 4, 8 * 8 + 4>();
     const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * V;
     const size_t total = N * M;
     if (idx >= total) {

@@ -27,7 +27,7 @@ struct DirectParams {
 
 template <int KIND, int NC>
 __global__ __launch_bounds__(256) void k_matvec_direct_f16(const DirectParams p) {
-    warm_kernel_arguments<sizeof(DirectParams)>();
+    warm_kernel_arguments<sizeof(DirectParams), sizeof(DirectParams)>();
     constexpr int BV = KindTraits<KIND>::BV;
     constexpr int BB = KindTraits<KIND>::BB;
     const int lane = threadIdx.x & 63;
@@ -254,7 +254,7 @@ struct RopeFinishParams {
 };
 
 __global__ __launch_bounds__(256) void k_qkv_rope_finish(const RopeFinishParams p) {
-    warm_kernel_arguments<sizeof(RopeFinishParams)>();
+    warm_kernel_arguments<sizeof(RopeFinishParams), sizeof(RopeFinishParams)>();
     const int proj = blockIdx.z;
     const size_t n = blockIdx.y;
     const size_t pair = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -482,10 +482,11 @@ struct MatvecParams {
     size_t expert_stride;         // bytes between the experts' weight slices
 };
 
-__device__ __forceinline__ void store_out(const MatvecParams &p, int which, size_t n, size_t row, float v) {
+// out / bias: this launch's entries of p.out / p.bias, fetched by the caller before the final barrier (two scalar
+// loads whose latency would otherwise sit, one after the other, between the reduction and the store)
+__device__ __forceinline__ void store_out(const MatvecParams &p, void *out, const void *bias, size_t n, size_t row,
+                                          float v) {
     const size_t idx = n * p.M + row;
-    void *out = p.out[which];
-    const void *bias = p.bias[which];
     float b = 0.0f;
     if (bias != nullptr) {
         b = p.bias_is_f16 ? h2f(((const uint16_t *)bias)[row]) : ((const float *)bias)[row];
@@ -520,7 +521,7 @@ constexpr int matvec_max_threads() {
 template <class Fmt, int NC, int C, int R, bool FUSED, bool EXACT>
 __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void k_matvec(const MatvecParams p) {
     extern __shared__ float partial[];  // [rows_per_wg][NC][4 * W]: one partial per 16-lane row of each wavefront
-    warm_kernel_arguments<sizeof(MatvecParams)>();
+    warm_kernel_arguments<sizeof(MatvecParams), sizeof(MatvecParams)>();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int W = blockDim.x >> 6;
@@ -620,6 +621,9 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
             consume(wb, r + R);
         }
     }
+    void *const out = p.out[blockIdx.y];
+    const void *const bias = p.bias[blockIdx.y];
+    asm volatile("" ::"s"(out), "s"(bias));  // keeps the two loads in front of the barrier
     __syncthreads();
     for (int idx = threadIdx.x; idx < p.rows_per_wg * NC; idx += blockDim.x) {
         const size_t row = row0 + idx / NC;
@@ -638,7 +642,7 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
                 const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
                 s += w < W ? t : 0.0f;
             }
-            store_out(p, (int)blockIdx.y, n0 + n, row, s);
+            store_out(p, out, bias, n0 + n, row, s);
         }
     }
 }
@@ -667,13 +671,16 @@ constexpr int matvec_ls_max_consumers() {
 template <class Fmt, int NC, int C, int R, bool FUSED>
 __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_matvec_ls(const MatvecParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-    warm_kernel_arguments<sizeof(MatvecParams)>();
+    warm_kernel_arguments<offsetof(MatvecParams, items), sizeof(MatvecParams)>();  // the grouped-mode fields behind it are never read here
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int W = (int)(blockDim.x >> 6) - 1;  // consumers
     const bool loader = wave == W;
     const int sub = lane % Fmt::LPB;
     const uint8_t *__restrict__ wbase = p.w[blockIdx.y];
+    void *const out = p.out[blockIdx.y];
+    const void *const bias = p.bias[blockIdx.y];
+    asm volatile("" ::"s"(out), "s"(bias));  // fetched here, not between the reduction and the store
     const size_t n0 = p.n0;
     const size_t row0 = (size_t)blockIdx.x * p.rows_per_wg;
     const int rows = p.rows_per_wg;  // a multiple of R
@@ -814,7 +821,7 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
                 const float t = (v[w].x + v[w].y) + (v[w].z + v[w].w);
                 sum += w < W ? t : 0.0f;
             }
-            store_out(p, (int)blockIdx.y, n0 + n, row, sum);
+            store_out(p, out, bias, n0 + n, row, sum);
         }
     }
 }

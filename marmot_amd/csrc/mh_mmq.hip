@@ -162,7 +162,7 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
     const bool loader = wave == W;
-    warm_kernel_arguments<sizeof(MmqParams)>();
+    warm_kernel_arguments<sizeof(MmqParams), sizeof(MmqParams)>();
     const int j = lane & 31, kh = lane >> 5;
     const int split = (int)blockIdx.y / p.nw;
     const int which = (int)blockIdx.y - split * p.nw;
@@ -379,7 +379,7 @@ constexpr int MMQ6_STAGE = MMQ6_WBLK + MMQ_ABLK + MMQ_TOK * 4;
 template <int NR>
 __global__ __launch_bounds__(512) void k_mmq_q6k(const MmqParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    warm_kernel_arguments<sizeof(MmqParams)>();
+    warm_kernel_arguments<sizeof(MmqParams), sizeof(MmqParams)>();
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = blockDim.x >> 6;
     const int j = lane & 31, kh = lane >> 5;
     const int split = (int)blockIdx.y / p.nw;
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
     constexpr int LOADS = W_LOADS + A_LOADS + 1;
     constexpr int AHEAD = STAGES - 1;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    warm_kernel_arguments<sizeof(MmqParams)>();
+    warm_kernel_arguments<sizeof(MmqParams), sizeof(MmqParams)>();
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
     const bool loader = wave == W;
     const int j = lane & 31, kh = lane >> 5;

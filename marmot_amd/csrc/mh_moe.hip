@@ -159,7 +159,7 @@ __device__ __forceinline__ void route_emit(const RouteArgs &a, int r, int pos) {
 }
 
 __global__ __launch_bounds__(MOE_ROUTE_WAVES * 64) void k_moe_route(const RouteArgs a) {
-    warm_kernel_arguments<sizeof(RouteArgs)>();
+    warm_kernel_arguments<sizeof(RouteArgs), sizeof(RouteArgs)>();
     __shared__ int counts[MOE_MAX_EXPERTS];
     __shared__ int wcount[MOE_ROUTE_WAVES][MOE_MAX_EXPERTS];  // per chunk: routes of each expert, then its cursor
     __shared__ int ids_l[MOE_ROUTE_LDS];  // expert id of each route (-1 = invalid), later its sorted position

@@ -71,7 +71,7 @@ template <int SRC, bool AOS>
 __global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ x, const void *__restrict__ x2,
                                                        size_t rows, size_t k, size_t nb,
                                                        uint8_t *__restrict__ blocks_out, ActScratch soa) {
-    warm_kernel_arguments<6 * 8 + sizeof(ActScratch)>();
+    warm_kernel_arguments<6 * 8 + sizeof(ActScratch), 6 * 8 + sizeof(ActScratch)>();
     const int lane = threadIdx.x & 63;
     const size_t wave = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (wave >= rows * nb) {
@@ -155,7 +155,7 @@ template <int SRC, bool AOS>
 __global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ x, const void *__restrict__ x2,
                                                        size_t rows, size_t k, size_t nb,
                                                        uint8_t *__restrict__ blocks_out, ActScratch soa) {
-    warm_kernel_arguments<6 * 8 + sizeof(ActScratch)>();
+    warm_kernel_arguments<6 * 8 + sizeof(ActScratch), 6 * 8 + sizeof(ActScratch)>();
     const int lane32 = threadIdx.x & 31;
     const size_t blk_id = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 5;
     if (blk_id >= rows * nb) {

@@ -163,8 +163,8 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV")):
-    """Every benchmark configuration (C1..C5, QKV) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "LOGITS")):
+    """Every benchmark configuration (C1..C5, QKV, LOGITS) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -212,6 +212,11 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV
         sweep_moe(hip, rng, emit, steps)
     if "QKV" in only:
         sweep_qkv(hip, rng, emit, steps, warmup)
+    if "LOGITS" in only:
+        # the vocabulary-sized matvec at the end of a decode step (Llama-3 vocabulary, 128256 rows of 4096)
+        for kind in (capi.KIND_Q6_K, capi.KIND_Q4_K):
+            for N in (1, 4):
+                linear_case("LOGITS", kind, 128256, 4096, N)
 
 
 def sweep_qkv(hip, rng, emit, steps: int, warmup: int):
@@ -362,7 +367,7 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--prefill-tokens", type=int, default=512)
     ap.add_argument("--sweep", action="store_true",
-                    help="measure every benchmark configuration (C1..C5, QKV) instead, one JSON line each (documentation runs)")
+                    help="measure every benchmark configuration (C1..C5, QKV, LOGITS) instead, one JSON line each (documentation runs)")
     ap.add_argument("--configs", default="C1,C2,C3,C4,C5", help="with --sweep: the configurations to run")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")

@@ -309,6 +309,26 @@ class HipBackend:
             for b in d_w + [d_x] + [b for b in d_b if b is not None] + d_o + extra:
                 b.free()
 
+    def embedding_gather(self, kind: int, table: np.ndarray, vocab: int, dim: int, ids: np.ndarray,
+                         out_dtype=np.float32, scale: float = 1.0, padding_id: int = -1, bounds_check: bool = False):
+        """marmot_embedding_gather with a block-quantized table [vocab, dim] (include/marmot/ops_types.h:160-170,
+        src/backends/cpu/ops/embedding/scalar/embedding_scalar.c): ids int32 or int64 of any shape -> ids.shape + (dim,)
+        of out_dtype (float32 or float16)."""
+        ids = np.ascontiguousarray(ids)
+        ids_dt = {np.dtype(np.int32): capi.DT_I32, np.dtype(np.int64): capi.DT_I64}[ids.dtype]
+        out_dtype = np.dtype(out_dtype)
+        d_t = self.to_device(np.ascontiguousarray(table, dtype=np.uint8))
+        d_i = self.to_device(ids)
+        d_o = self.alloc(max(1, ids.size * dim * out_dtype.itemsize))
+        try:
+            check(self.lib.marmot_hip_embedding_gather_quantized(
+                self.dev, kind, C.c_void_p(d_t.ptr), vocab, dim, C.c_void_p(d_i.ptr), ids_dt, ids.size,
+                C.c_void_p(d_o.ptr), _np_dtype_id(out_dtype), scale, padding_id, 1 if bounds_check else 0))
+            return d_o.download(out_dtype, ids.shape + (dim,))
+        finally:
+            for b in (d_t, d_i, d_o):
+                b.free()
+
     def topk(self, x: np.ndarray, k: int):
         x = np.ascontiguousarray(x, dtype=np.float32)
         rows, cols = x.shape

@@ -79,6 +79,7 @@ SIGNATURES = {
                                                   _vp, _vp, _vp, _i, C.POINTER(Rope)]),
     "marmot_hip_rope_frequencies": (_i, [_i, _f, _f, _f, _f, _f, _f, _u32, _u32, _sz, _vp, C.POINTER(_f),
                                          C.POINTER(_u32)]),
+    "marmot_hip_embedding_gather_quantized": (_i, [_vp, _i, _vp, _sz, _sz, _vp, _i, _sz, _vp, _i, _f, C.c_int32, _i]),
     "marmot_hip_packed_activation_bytes": (_sz, [_i, _sz, _sz]),
     "marmot_hip_pack_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
     "marmot_hip_matmul_prepacked": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _vp, _i, _vp, _i]),

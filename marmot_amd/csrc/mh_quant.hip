@@ -37,6 +37,56 @@ __global__ __launch_bounds__(256) void k_dequantize(const uint8_t *__restrict__ 
 }
 
 // ------------------------------------------------------------------------------------------------
+// Embedding gather from a block-quantized table (embedding_scalar.c:241-303, 381-447): one thread per output value.
+// ------------------------------------------------------------------------------------------------
+template <int KIND>
+__global__ __launch_bounds__(256) void k_embedding_gather(const uint8_t *__restrict__ table, size_t vocab, size_t dim,
+                                                          const void *__restrict__ ids, int ids_are_i64,
+                                                          void *__restrict__ out, int out_is_f16, float scale,
+                                                          int padding_id, int *__restrict__ error_flag) {
+    warm_kernel_arguments<72, 72>();
+    constexpr int BV = KindTraits<KIND>::BV;
+    constexpr int BB = KindTraits<KIND>::BB;
+    const size_t idx = blockIdx.y;
+    const size_t col = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (col >= dim) {
+        return;
+    }
+    const long long token = ids_are_i64 ? ((const long long *)ids)[idx] : (long long)((const int *)ids)[idx];
+    bool zero = padding_id >= 0 && token == (long long)padding_id;
+    if (!zero && (token < 0 || (unsigned long long)token >= (unsigned long long)vocab)) {
+        zero = true;
+        if (error_flag != nullptr && col == 0) {
+            atomicMax(error_flag, (int)(gridDim.y - idx));  // tokens - position: the maximum names the first offender
+        }
+    }
+    float y = 0.0f;
+    if (!zero) {
+        const size_t nb = (dim + BV - 1) / BV;
+        const size_t b = col / BV;
+        const int v = (int)(col - b * BV);
+        const uint8_t *blk = table + ((size_t)token * nb + b) * BB;
+        if constexpr (KIND == MARMOT_HIP_KIND_Q4_0) {
+            // the embedding path's own nibble order for Q4_0 (embedding_scalar.c:221-229)
+            const uint8_t packed = blk[2 + (v >> 1)];
+            const int q = ((v & 1) ? (packed >> 4) : (packed & 0x0f)) - 8;
+            y = h2f((uint16_t)(blk[0] | (blk[1] << 8))) * (float)q;
+        } else {
+            y = dequant_value<KIND>(blk, v);
+        }
+    }
+    if (out_is_f16) {
+        // the product is rounded to fp32 on its own before the conversion: merged into one mixed-precision
+        // multiply-add with a +0 addend, -0 * scale would come out as +0
+        float t = y * scale;
+        asm volatile("" : "+v"(t));
+        ((uint16_t *)out)[idx * dim + col] = zero ? (uint16_t)0 : f2h(t);
+    } else {
+        ((float *)out)[idx * dim + col] = zero ? 0.0f : (scale == 1.0f ? y : y * scale);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Activation quantizers
 // ------------------------------------------------------------------------------------------------
 
@@ -346,6 +396,78 @@ int marmot_hip_quantize_activations(marmot_hip_device_t *dev, int act_kind, cons
     }
     ActScratch none;
     return launch_quantize<true>(dev, act_kind, d_x, in_dtype, rows, k, (uint8_t *)d_blocks_out, none);
+}
+
+int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, const void *d_table, size_t vocab,
+                                          size_t dim, const void *d_ids, int ids_dtype, size_t n, void *d_out,
+                                          int out_dtype, float scale, int32_t padding_id, int bounds_check) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
+    }
+    if (d_table == nullptr || d_ids == nullptr || d_out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
+    }
+    if (kind != MARMOT_HIP_KIND_Q4_0 && kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_K &&
+        kind != MARMOT_HIP_KIND_Q6_K) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "embedding gather: unsupported quant kind %d", kind);
+    }
+    if (ids_dtype != MARMOT_HIP_DTYPE_I32 && ids_dtype != MARMOT_HIP_DTYPE_I64) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "embedding gather: token ids must be INT32 or INT64");
+    }
+    if (out_dtype != MARMOT_HIP_DTYPE_F32 && out_dtype != MARMOT_HIP_DTYPE_F16) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "embedding gather: output must be FLOAT32 or FLOAT16");
+    }
+    if (n == 0 || dim == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    if (n > 65535) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "embedding gather: more than 65535 tokens per call");
+    }
+    MH_HIP(hipSetDevice(dev->device_index));
+    // Out-of-range tokens are reported through a device flag that is read back after the launch; that needs a
+    // stream synchronization and is skipped while the stream is being captured into a graph (rows are zeroed then).
+    int *flag = nullptr;
+    if (bounds_check != 0 && !dev->capturing) {
+        void *ws = nullptr;
+        const int st = workspace_reserve(dev, 256, &ws);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return st;
+        }
+        flag = (int *)ws;
+        MH_HIP(hipMemsetAsync(flag, 0, sizeof(int), dev->stream));
+    }
+    const dim3 grid((unsigned)((dim + 255) / 256), (unsigned)n), block(256);
+    const uint8_t *table = (const uint8_t *)d_table;
+    const int i64 = ids_dtype == MARMOT_HIP_DTYPE_I64, f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    switch (kind) {
+    case MARMOT_HIP_KIND_Q4_K:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q4_K>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q6_K:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q6_K>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q8_0:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q8_0>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    default:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q4_0>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    }
+    MH_HIP(hipGetLastError());
+    if (flag != nullptr) {
+        int host_flag = 0;
+        MH_HIP(hipMemcpyAsync(&host_flag, flag, sizeof(int), hipMemcpyDeviceToHost, dev->stream));
+        MH_HIP(hipStreamSynchronize(dev->stream));
+        if (host_flag != 0) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT,
+                             "embedding gather: token id at position %zu is out of range", n - (size_t)host_flag);
+        }
+    }
+    return MARMOT_HIP_SUCCESS;
 }
 
 } // extern "C"

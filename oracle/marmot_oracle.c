@@ -1484,6 +1484,99 @@ int mo_matmul_qkv_separate(
     return mo_matmul_qkv_separate_rope(kind, weights, input, in_dtype, N, K, M, bias, bias_dtype, out, NULL, NULL, 0);
 }
 
+/* ======================= embedding gather ======================= */
+
+/* embedding_scalar.c:381-447 (worker), :241-303 (quantized row), :167-185 (zero row), :187-209 (stores) */
+int mo_embedding_gather_quantized(
+    int kind, const void *weights, size_t vocab, size_t dim, const void *ids, int ids_dtype, size_t n, void *out,
+    int out_dtype, float scale, int32_t padding_id, int bounds_check, size_t *error_index
+) {
+    const size_t bv = mo_block_values(kind);
+    const size_t bb = mo_block_bytes(kind);
+    if (bv == 0 || weights == NULL || ids == NULL || out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    if (ids_dtype != MO_DTYPE_I32 && ids_dtype != MO_DTYPE_I64) {
+        return MO_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (out_dtype != MO_DTYPE_F32 && out_dtype != MO_DTYPE_F16) {
+        return MO_ERR_UNSUPPORTED_DTYPE;
+    }
+    const size_t blocks_per_row = (dim + bv - 1) / bv;
+    const size_t row_bytes = blocks_per_row * bb;
+    float decoded[QK_K];
+    for (size_t idx = 0; idx < n; ++idx) {
+        const int64_t token = ids_dtype == MO_DTYPE_I32 ? (int64_t)((const int32_t *)ids)[idx]
+                                                        : ((const int64_t *)ids)[idx];
+        int zero = 0;
+        if (padding_id >= 0 && token == (int64_t)padding_id) {
+            zero = 1; /* :411-414 */
+        } else if (token < 0 || (uint64_t)token >= (uint64_t)vocab) {
+            if (bounds_check) { /* :416-423 */
+                if (error_index != NULL) {
+                    *error_index = idx;
+                }
+                return MO_ERR_INVALID_ARGUMENT;
+            }
+            zero = 1;
+        }
+        if (zero) { /* :167-177: memset of the row */
+            if (out_dtype == MO_DTYPE_F32) {
+                memset((float *)out + idx * dim, 0, dim * sizeof(float));
+            } else {
+                memset((uint16_t *)out + idx * dim, 0, dim * sizeof(uint16_t));
+            }
+            continue;
+        }
+        const uint8_t *row = (const uint8_t *)weights + (size_t)token * row_bytes;
+        for (size_t b = 0; b < blocks_per_row; ++b) { /* :255-300 */
+            const size_t base_col = b * bv;
+            if (base_col >= dim) {
+                break;
+            }
+            const size_t remaining = dim - base_col;
+            const size_t count = remaining < bv ? remaining : bv;
+            const uint8_t *blk = row + b * bb;
+            switch (kind) {
+            case MO_KIND_Q4_0: { /* cpu_embedding_decode_q4_0_interleaved, :221-229 */
+                const blk_q4_0 *q = (const blk_q4_0 *)blk;
+                const float sc = mo_f16_to_f32(q->scale);
+                for (size_t i = 0; i < count; ++i) {
+                    const uint8_t packed = q->qs[i >> 1];
+                    int32_t v = (i & 1) ? ((packed >> 4) & 0x0f) : (packed & 0x0f);
+                    v -= 8;
+                    decoded[i] = sc * (float)v;
+                }
+                break;
+            }
+            case MO_KIND_Q8_0:
+                q8_0_dequantize_block((const blk_q8_0 *)blk, (uint32_t)count, decoded);
+                break;
+            case MO_KIND_Q4_K:
+                q4_k_dequantize_block((const blk_q4_k *)blk, (uint32_t)count, decoded);
+                break;
+            case MO_KIND_Q6_K:
+                q6_k_dequantize_block((const blk_q6_k *)blk, (uint32_t)count, decoded);
+                break;
+            default:
+                return MO_ERR_NOT_IMPLEMENTED;
+            }
+            if (out_dtype == MO_DTYPE_F32) { /* :187-199 */
+                float *o = (float *)out + idx * dim + base_col;
+                for (size_t i = 0; i < count; ++i) {
+                    o[i] = scale == 1.0f ? decoded[i] : decoded[i] * scale;
+                }
+            } else { /* :201-209 */
+                uint16_t *o = (uint16_t *)out + idx * dim + base_col;
+                for (size_t i = 0; i < count; ++i) {
+                    o[i] = mo_f32_to_f16(decoded[i] * scale);
+                }
+            }
+        }
+    }
+    return MO_OK;
+}
+
 /* ======================= top-k / router / MoE ======================= */
 
 /* moe_ops.c:789-889 */

@@ -148,6 +148,21 @@ int mo_matmul_qkv_separate_rope(
     int pos_dtype
 );
 
+/*
+ * marmot_embedding_gather with a block-quantized table (cpu_embedding_gather_scalar ->
+ * cpu_embedding_run_worker / cpu_embedding_copy_row_quantized, src/backends/cpu/ops/embedding/scalar/
+ * embedding_scalar.c:241-303, 381-447): weights = vocab rows of row_bytes(kind, dim); ids: n values of ids_dtype
+ * (MO_DTYPE_I32 or MO_DTYPE_I64); out: [n, dim] of out_dtype (F32 or F16), value = decoded * scale (one rounding for
+ * F16). A token equal to padding_id (when padding_id >= 0) gives a zero row; a token outside [0, vocab) gives a zero
+ * row, or MO_ERR_INVALID_ARGUMENT when bounds_check is set (*error_index receives the position). Q4_0 rows are decoded
+ * in the table's interleaved nibble order (value i = nibble i % 2 of byte i / 2, :221-229), the other kinds with
+ * their block dequantizers.
+ */
+int mo_embedding_gather_quantized(
+    int kind, const void *weights, size_t vocab, size_t dim, const void *ids, int ids_dtype, size_t n, void *out,
+    int out_dtype, float scale, int32_t padding_id, int bounds_check, size_t *error_index
+);
+
 /* top-k over the last axis, ties -> lower index (moe_ops.c:789-889) */
 int mo_topk(const float *x, size_t rows, size_t cols, size_t k, float *values_out, int32_t *indices_out);
 

@@ -102,6 +102,10 @@ class Oracle:
         L.mo_rope_resolve_head_dim.argtypes = [C.c_size_t, C.c_uint32]
         L.mo_rope_rotate_row.restype = None
         L.mo_rope_rotate_row.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, C.c_void_p, C.c_float, C.c_int]
+        L.mo_embedding_gather_quantized.restype = C.c_int
+        L.mo_embedding_gather_quantized.argtypes = [
+            C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int, C.c_size_t, C.c_void_p, C.c_int,
+            C.c_float, C.c_int32, C.c_int, C.POINTER(C.c_size_t)]
         L.mo_topk.restype = C.c_int
         L.mo_topk.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
         L.mo_softmax_rows.restype = None
@@ -251,6 +255,25 @@ class Oracle:
         if st != 0:
             raise RuntimeError(f"mo_matmul_qkv_separate_rope -> {st}")
         return tuple(outs)
+
+    def embedding_gather(self, kind: int, table: np.ndarray, vocab: int, dim: int, ids: np.ndarray,
+                         out_dtype=np.float32, scale: float = 1.0, padding_id: int = -1, bounds_check: bool = False):
+        """marmot_embedding_gather with a block-quantized table; ids int32 or int64, any shape. Raises IndexError
+        (with the flat position) for an out-of-range token when bounds_check is set."""
+        table = np.ascontiguousarray(table, dtype=np.uint8)
+        assert table.size == vocab * row_bytes(kind, dim)
+        ids = np.ascontiguousarray(ids)
+        ids_dt = {np.dtype(np.int32): DT_I32, np.dtype(np.int64): DT_I64}[ids.dtype]
+        out = np.full(ids.shape + (dim,), np.nan, dtype=out_dtype)
+        err = C.c_size_t(0)
+        st = self.L.mo_embedding_gather_quantized(
+            kind, _ptr(table), vocab, dim, _ptr(ids), ids_dt, ids.size, _ptr(out),
+            DT_F16 if out.dtype == np.float16 else DT_F32, scale, padding_id, 1 if bounds_check else 0, C.byref(err))
+        if st == -1:
+            raise IndexError(int(err.value))
+        if st != 0:
+            raise RuntimeError(f"mo_embedding_gather_quantized -> {st}")
+        return out
 
     # ---- MoE
     def topk(self, x: np.ndarray, k: int):

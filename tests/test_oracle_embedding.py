@@ -1,0 +1,65 @@
+"""CPU: the oracle's restatement of marmot_embedding_gather for block-quantized tables
+(src/backends/cpu/ops/embedding/scalar/embedding_scalar.c:241-303, 381-447), pinned by the reference's own golden for
+the Q4_0 table (tests/golden/embedding_q4_0_ragged.txt, transcribed to tests/golden/reference_embedding_q4_0.json: the
+interleaved nibble order of the embedding path, which differs from the Q4_0 dequantizer's) and, for the other kinds, by
+the block dequantizers the quantization goldens pin (a gathered row is the dequantized row, bit for bit)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle.pyoracle import KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0, row_bytes
+from tests.util import bits, gaussian, random_valid_blocks
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_embedding_q4_0.json")
+
+
+def load_golden():
+    with open(GOLDEN) as f:
+        g = json.load(f)
+    table = np.frombuffer(bytes.fromhex(g["weights_hex"]), dtype=np.uint8)
+    ids = np.array(g["ids"], dtype=np.int32)
+    return g["vocab"], g["dim"], table, ids, np.array(g["expected"], dtype=np.float32).reshape(len(ids), g["dim"])
+
+
+def test_reference_q4_0_embedding_golden(oracle):
+    vocab, dim, table, ids, expected = load_golden()
+    got = oracle.embedding_gather(KIND_Q4_0, table, vocab, dim, ids, bounds_check=True)
+    # the reference's tolerance for this kind is 5e-4 (tests/backend/test_backend_embedding_golden.c:226-229)
+    assert np.max(np.abs(got - expected)) <= 1e-6
+    # and the order is NOT the block dequantizer's: that one disagrees with the golden
+    plain = oracle.dequantize(KIND_Q4_0, table.reshape(vocab, -1), dim)[ids]
+    assert np.max(np.abs(plain - expected)) > 1.0
+
+
+@pytest.mark.parametrize("kind", [KIND_Q8_0, KIND_Q4_K, KIND_Q6_K])
+def test_gathered_rows_are_dequantized_rows(oracle, kind):
+    rng = np.random.default_rng(800 + kind)
+    vocab, dim = 37, 768 if kind != KIND_Q8_0 else 96
+    table = random_valid_blocks(rng, kind, vocab, dim)
+    dense = oracle.dequantize(kind, table, dim)
+    ids = rng.integers(0, vocab, (3, 5)).astype(np.int64)
+    got = oracle.embedding_gather(kind, table, vocab, dim, ids)
+    assert got.shape == (3, 5, dim) and np.array_equal(bits(got), bits(dense[ids]))
+    # scale and float16 output: decoded * scale, one rounding
+    half = oracle.embedding_gather(kind, table, vocab, dim, ids.astype(np.int32), out_dtype=np.float16, scale=0.5)
+    want = (dense[ids] * np.float32(0.5)).astype(np.float16)
+    assert np.array_equal(half.view(np.uint16), want.view(np.uint16))
+
+
+def test_padding_and_out_of_range_tokens(oracle):
+    kind, vocab, dim = KIND_Q4_K, 8, 256
+    table = random_valid_blocks(np.random.default_rng(810), kind, vocab, dim)
+    dense = oracle.dequantize(kind, table, dim)
+    ids = np.array([3, 5, -1, 8, 0, 5], dtype=np.int32)
+    got = oracle.embedding_gather(kind, table, vocab, dim, ids, padding_id=5)
+    assert np.array_equal(bits(got[0]), bits(dense[3])) and np.array_equal(bits(got[4]), bits(dense[0]))
+    for z in (1, 2, 3, 5):  # padding rows and out-of-range rows are zero
+        assert not got[z].any()
+    with pytest.raises(IndexError) as e:  # with the bounds check the first offender is reported
+        oracle.embedding_gather(kind, table, vocab, dim, ids, padding_id=5, bounds_check=True)
+    assert e.value.args[0] == 2
+    # a negative padding id disables padding (embedding_scalar.c:411)
+    got = oracle.embedding_gather(kind, table, vocab, dim, np.array([5], np.int32), padding_id=-1)
+    assert np.array_equal(bits(got[0]), bits(dense[5]))

@@ -242,14 +242,14 @@ def sweep_qkv(hip, rng, emit, steps: int, warmup: int):
             d_o = [hip.alloc(N * M * 4) for _ in range(3)]
             fused = time_steps_graph(hip, lambda i: hip.linear_qkv_d(kind, *d_w, d_x, DT_F32, N, K, M, *d_o,
                                                                      weight_offset=(i % copies) * stride),
-                                     steps, warmup)
+                                     steps, warmup, chunk=50)
             route = hip.last_route()
 
             def three(i):
                 for w, o in zip(d_w, d_o):
                     hip.linear_d(kind, w, d_x, DT_F32, N, K, M, o, DT_F32, weight_offset=(i % copies) * stride)
 
-            separate = time_steps_graph(hip, three, steps, warmup)
+            separate = time_steps_graph(hip, three, steps, warmup, chunk=50)  # graphs of a few hundred nodes
             nbytes = 3 * M * rb + N * K * 4 + 3 * N * M * 4
             emit({"config": "QKV", "workload": f"{names[kind]} q,k,v 3 x {M}x{K} N={N}", "route": route,
                   "us": round(fused * 1e3, 2), "us_three_linears": round(separate * 1e3, 2),

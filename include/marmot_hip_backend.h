@@ -321,6 +321,27 @@ typedef struct marmot_matmul_qkv_desc {
     const marmot_rope_params_t *rope_params;
 } marmot_matmul_qkv_desc_t;
 
+/* include/marmot/types.h:236-240 */
+typedef enum {
+    MARMOT_PREFERENCE_DEFAULT = 0,
+    MARMOT_PREFERENCE_ENABLE = 1,
+    MARMOT_PREFERENCE_DISABLE = 2,
+} marmot_preference_t;
+
+/* include/marmot/ops_types.h:160-170 */
+struct marmot_embedding_gather_desc {
+    const marmot_tensor_t *weights;
+    const marmot_tensor_t *token_ids;
+    marmot_tensor_t *out;
+    marmot_dtype_t dtype_out;
+    float scale;
+    int32_t padding_id;
+    bool bounds_check;
+    marmot_preference_t prefer_gpu_private;
+    marmot_preference_t allow_quant_decode_on_the_fly;
+};
+typedef struct marmot_embedding_gather_desc marmot_embedding_gather_desc_t;
+
 /* include/marmot/traits_ids.gen.h:40-107 (the operations this backend answers for), :111-116, :120-133 */
 typedef enum {
     MARMOT_OP_INVALID = 0,
@@ -332,6 +353,7 @@ typedef enum {
     MARMOT_OP_LINEAR = 708,
     MARMOT_OP_QKV_SHARED_INPUT = 771,
     MARMOT_OP_QKV_ROPE = 778,
+    MARMOT_OP_EMBEDDING = 853,
     MARMOT_OP_TOPK = 901,
     MARMOT_OP_COUNT = 995,
 } marmot_op_id_t;
@@ -640,6 +662,8 @@ bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_bac
  *   TOPK        u16 input, values_out, indices_out; u32 axis; u32 k    (bytecode_compile.c:459-479)
  *   QKV         u16 input, wq, wk, wv, bq, bk, bv (0xFFFF none); u32 epilogue const offset; u32 rope-params const
  *               offset (0xFFFFFFFF none); u16 out_q, out_k, out_v      (bytecode_compile.c:670-715)
+ *   EMBEDDING   u16 weights, token_ids, out; u32 dtype_out; f32 scale; u32 padding_id; u8 bounds_check,
+ *               prefer_gpu_private, allow_quant_decode_on_the_fly       (bytecode_compile.c:989-1018)
  *   QUANTIZE    u16 input; u32 quant-params const offset; u16 output; u32 kind; u32 layout   (:912-941)
  *   DEQUANTIZE  u16 input; u16 output; u32 kind; u32 layout            (bytecode_compile.c:942-962) */
 enum {
@@ -659,7 +683,11 @@ enum {
     MARMOT_HIP_BC_OP_QKV_Q8_0 = 13,
     MARMOT_HIP_BC_OP_QKV_Q4_K = 14,
     MARMOT_HIP_BC_OP_QKV_Q6_K = 15,
-    MARMOT_HIP_BC_OP_COUNT = 16,
+    MARMOT_HIP_BC_OP_EMBEDDING_Q4_0 = 16,
+    MARMOT_HIP_BC_OP_EMBEDDING_Q8_0 = 17,
+    MARMOT_HIP_BC_OP_EMBEDDING_Q4_K = 18,
+    MARMOT_HIP_BC_OP_EMBEDDING_Q6_K = 19,
+    MARMOT_HIP_BC_OP_COUNT = 20,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -691,6 +719,10 @@ marmot_error_t hip_matmul_qkv_q4_0(const void *device_ctx, const marmot_matmul_q
 marmot_error_t hip_matmul_qkv_q8_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q4_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
+/* marmot_embedding_gather with a block-quantized table [vocab, dim] (cf. cpu_embedding_gather,
+ * src/backends/cpu/ops/embedding/embedding_dispatch.c:4-16 -> embedding_scalar.c:460-591): token ids INT32 or INT64 of
+ * any shape, output FLOAT32 or FLOAT16 viewed as [tokens, dim]; weights->quant_kind selects Q4_0, Q8_0, Q4_K or Q6_K. */
+marmot_error_t hip_embedding_gather(const void *device_ctx, const marmot_embedding_gather_desc_t *desc);
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc);
 marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc);
 /* output->quant_kind selects the activation block format: Q8_0 or Q8_K */

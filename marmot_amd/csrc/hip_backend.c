@@ -274,6 +274,18 @@ static bool rows_contiguous(const marmot_tensor_t *t) {
     return t->shape.ndim == 2 && t->shape.strides[1] == 1 && t->shape.strides[0] == t->shape.shape[1];
 }
 
+// row-major without gaps, any rank
+static bool dense_contiguous(const marmot_tensor_t *t) {
+    size_t expect = 1;
+    for (size_t i = t->shape.ndim; i-- > 0;) {
+        if (t->shape.shape[i] != 1 && t->shape.strides[i] != expect) {
+            return false;
+        }
+        expect *= t->shape.shape[i];
+    }
+    return true;
+}
+
 static void mark_device_output(marmot_tensor_t *t) {
     t->memory_location = MARMOT_MEMORY_DEVICE;
     t->needs_sync = true;
@@ -866,6 +878,78 @@ static marmot_error_t matmul_qkv(const void *device_ctx, marmot_quant_kind_t exp
     return st;
 }
 
+// marmot_embedding_gather, block-quantized table (embedding_scalar.c:460-591)
+static marmot_error_t embedding_gather(const void *device_ctx, const marmot_embedding_gather_desc_t *desc) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || desc == nullptr || desc->weights == nullptr || desc->token_ids == nullptr ||
+        desc->out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Embedding gather: null argument");
+    }
+    const marmot_tensor_t *weights = desc->weights, *ids = desc->token_ids;
+    marmot_tensor_t *out = desc->out;
+    if (weights->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Embedding weights must be 2D");
+    }
+    if (!kind_is_block(weights->quant_kind) || weights->quant_layout != MARMOT_QUANT_LAYOUT_GGUF) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Unsupported quantized embedding layout");
+    }
+    if (!kind_supported_weight(weights->quant_kind)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized embedding kind not supported on HIP");
+    }
+    const size_t vocab = weights->shape.shape[0], dim = weights->shape.shape[1];
+    const size_t tokens = tensor_numel(ids);
+    if (ids->dtype != MARMOT_DTYPE_INT32 && ids->dtype != MARMOT_DTYPE_INT64) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Unsupported token dtype for HIP embedding gather");
+    }
+    if (out->dtype != MARMOT_DTYPE_FLOAT32 && out->dtype != MARMOT_DTYPE_FLOAT16) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "HIP embedding gather writes FLOAT32 or FLOAT16");
+    }
+    if (tensor_numel(out) != tokens * dim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Embedding output must hold tokens x dim values");
+    }
+    if (!dense_contiguous(out) || !dense_contiguous(ids)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Embedding gather: HIP kernels need contiguous tensors");
+    }
+    if (weights->data == nullptr || ids->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Embedding gather: tensor without data");
+    }
+    if (tokens == 0 || dim == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+    pthread_mutex_lock(&b->mu);
+    const void *d_w = nullptr, *d_ids = nullptr;
+    void *d_out = nullptr;
+    marmot_error_t st = acquire_read(b, weights->data, vocab * marmot_hip_row_bytes((int)weights->quant_kind, dim), &d_w);
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, ids->data, dense_bytes(ids), &d_ids);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write(b, out->data, dense_bytes(out), &d_out);
+    }
+    // the library takes at most 65535 tokens per call
+    const size_t id_size = dtype_size(ids->dtype), row_size = dim * dtype_size(out->dtype);
+    for (size_t t0 = 0; st == MARMOT_SUCCESS && t0 < tokens; t0 += 65535) {
+        const size_t n = tokens - t0 < 65535 ? tokens - t0 : 65535;
+        const int rc = marmot_hip_embedding_gather_quantized(
+            b->dev, (int)weights->quant_kind, d_w, vocab, dim, (const uint8_t *)d_ids + t0 * id_size,
+            ids->dtype == MARMOT_DTYPE_INT32 ? MARMOT_HIP_DTYPE_I32 : MARMOT_HIP_DTYPE_I64, n,
+            (uint8_t *)d_out + t0 * row_size,
+            out->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, desc->scale,
+            desc->padding_id, desc->bounds_check ? 1 : 0);
+        if (rc == MARMOT_HIP_ERROR_INVALID_ARGUMENT) {
+            st = fail(MARMOT_ERROR_INVALID_ARGUMENT, "Embedding id out of range");
+        } else if (rc != MARMOT_HIP_SUCCESS) {
+            st = fail_from_lib(rc);
+        }
+    }
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    pthread_mutex_unlock(&b->mu);
+    return st;
+}
+
 // bytes of E expert slices of [rows, cols] blocks; expert tensors are stored [cols, rows, E] in GGUF order
 // (cpu_moe_execute_grouped, src/backends/cpu/ops/moe/moe_ops.c:895-899)
 static size_t expert_tensor_bytes(int kind, size_t rows, size_t cols, size_t experts) {
@@ -1231,6 +1315,34 @@ HIP_BC_QKV_ENTRY(bc_exec_qkv_q8_0, MARMOT_QUANT_KIND_Q8_0)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q4_k, MARMOT_QUANT_KIND_Q4_K)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q6_k, MARMOT_QUANT_KIND_Q6_K)
 
+// EMBEDDING immediates (bytecode_compile.c:989-1018) -> the descriptor the generated shim builds
+// (src/backends/cpu/dispatch/misc_dispatch_cpu.gen.c:115-133)
+static marmot_error_t bc_exec_embedding(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                        const uint8_t *const_pool) {
+    (void)const_pool;
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const uint16_t weights = rd_u16(&pc), token_ids = rd_u16(&pc), out = rd_u16(&pc);
+    const uint32_t dtype_out = rd_u32(&pc);
+    const float scale = rd_f32(&pc);
+    const uint32_t padding_id = rd_u32(&pc);
+    const uint8_t bounds_check = pc[0], prefer_gpu = pc[1], allow_decode = pc[2];
+    const marmot_embedding_gather_desc_t desc = {
+        .weights = reg(regs, weights),
+        .token_ids = reg(regs, token_ids),
+        .out = reg(regs, out),
+        .dtype_out = (marmot_dtype_t)dtype_out,
+        .scale = scale,
+        .padding_id = (int32_t)padding_id,
+        .bounds_check = bounds_check != 0,
+        .prefer_gpu_private = prefer_gpu ? MARMOT_PREFERENCE_ENABLE : MARMOT_PREFERENCE_DISABLE,
+        .allow_quant_decode_on_the_fly = allow_decode ? MARMOT_PREFERENCE_ENABLE : MARMOT_PREFERENCE_DISABLE,
+    };
+    return embedding_gather(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
+}
+
 static marmot_error_t bc_exec_moe(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
                                   const uint8_t *const_pool) {
     (void)const_pool;
@@ -1311,6 +1423,7 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     16,              // QUANTIZE: u16 + u32 + u16 + 2 x u32
     12,              // DEQUANTIZE: 2 x u16 + 2 x u32
     28, 28, 28, 28,  // QKV: 7 x u16 + 2 x u32 + 3 x u16
+    21, 21, 21, 21,  // EMBEDDING: 3 x u16 + u32 + f32 + u32 + 3 x u8
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1320,6 +1433,8 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_TOPK,
     MARMOT_BC_SCHEMA_QUANTIZE,    MARMOT_BC_SCHEMA_DEQUANTIZE,  MARMOT_BC_SCHEMA_QKV,
     MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_QKV,
+    MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_EMBEDDING,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1328,6 +1443,7 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_moe,         bc_exec_moe,         bc_exec_moe,         bc_exec_moe,
     bc_exec_topk,        bc_exec_quantize,    bc_exec_dequantize,
     bc_exec_qkv_q4_0,    bc_exec_qkv_q8_0,    bc_exec_qkv_q4_k,    bc_exec_qkv_q6_k,
+    bc_exec_embedding,   bc_exec_embedding,   bc_exec_embedding,   bc_exec_embedding,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -1476,6 +1592,21 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const uint16_t op = (uint16_t)(MARMOT_HIP_BC_OP_QKV_Q4_0 + (mm - MARMOT_HIP_BC_OP_MATMUL_Q4_0));
         return selected(op, launch_us + (t_mem > t_mma ? t_mem : t_mma), ws_mb);
     }
+    case MARMOT_OP_EMBEDDING: {
+        // cpu/kernels/embedding.def:19-30: the input dtype of this op is the index type
+        const int kind = kind_of_scheme(sig->qscheme_id);
+        const uint16_t mm = matmul_op_of_kind(kind);
+        if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
+            return unsupported("HIP embedding gather handles Q4_0, Q8_0, Q4_K and Q6_K tables");
+        }
+        if (sig->input_dtype != MARMOT_DTYPE_INT32 && sig->input_dtype != MARMOT_DTYPE_INT64) {
+            return unsupported("HIP embedding gather takes INT32 or INT64 token ids");
+        }
+        if (!out32 && !out16) {
+            return unsupported("HIP embedding gather writes FLOAT32 or FLOAT16");
+        }
+        return selected((uint16_t)(MARMOT_HIP_BC_OP_EMBEDDING_Q4_0 + (mm - MARMOT_HIP_BC_OP_MATMUL_Q4_0)), launch_us, 0.0);
+    }
     case MARMOT_OP_MOE_EXPERTS: {
         const int kind = kind_of_scheme(sig->qscheme_id);
         if (matmul_op_of_kind(kind) == MARMOT_KERNEL_OP_INDEX_INVALID) {
@@ -1607,6 +1738,9 @@ marmot_error_t hip_matmul_qkv_q4_k(const void *device_ctx, const marmot_matmul_q
 }
 marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q6_K, desc);
+}
+marmot_error_t hip_embedding_gather(const void *device_ctx, const marmot_embedding_gather_desc_t *desc) {
+    return embedding_gather(device_ctx, desc);
 }
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc) {
     return moe_experts(device_ctx, desc);

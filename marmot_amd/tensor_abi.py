@@ -27,7 +27,7 @@ MAX_DIMS = 8
 SUCCESS, INVALID_ARGUMENT, OUT_OF_MEMORY, DEVICE_NOT_AVAILABLE, BACKEND_INIT_FAILED = 0, -1, -2, -3, -4
 INVALID_OPERATION, UNSUPPORTED_DTYPE, DIMENSION_MISMATCH, NOT_IMPLEMENTED = -5, -6, -7, -8
 # marmot_dtype_t
-DTYPE_F32, DTYPE_F16, DTYPE_I32, DTYPE_I8, DTYPE_U8 = 0, 1, 3, 5, 6
+DTYPE_F32, DTYPE_F16, DTYPE_I32, DTYPE_I8, DTYPE_U8, DTYPE_I64 = 0, 1, 3, 5, 6, 11
 # marmot_quant_kind_t / marmot_quant_layout_t / marmot_memory_location_t
 KIND_GENERIC, KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_K = 0, 1, 5, 9, 11, 12
 LAYOUT_GENERIC, LAYOUT_GGUF = 0, 1
@@ -36,6 +36,8 @@ BACKEND_HIP = 3
 # marmot_op_id_t / marmot_qscheme_id_t
 OP_DEQUANTIZE, OP_MOE_EXPERTS, OP_MATMUL, OP_QUANTIZE, OP_LINEAR, OP_TOPK = 210, 263, 498, 524, 708, 901
 OP_QKV_PROJECTION, OP_QKV_SHARED_INPUT, OP_QKV_ROPE = 191, 771, 778
+OP_EMBEDDING = 853
+PREFERENCE_DEFAULT, PREFERENCE_ENABLE, PREFERENCE_DISABLE = 0, 1, 2
 QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q8_0: 5, KIND_Q4_K: 8, KIND_Q6_K: 10, KIND_Q8_K: 11}
 PROFILE_SCALAR = 4
@@ -46,7 +48,7 @@ EPILOGUE_ROPE = 8
 BC_END, BC_REG_INVALID, BC_INVALID_OFFSET = 0, 0xFFFF, 0xFFFFFFFF
 
 _NP_OF_DTYPE = {DTYPE_F32: np.float32, DTYPE_F16: np.float16, DTYPE_I32: np.int32, DTYPE_I8: np.int8,
-                DTYPE_U8: np.uint8}
+                DTYPE_U8: np.uint8, DTYPE_I64: np.int64}
 _DTYPE_OF_NP = {np.dtype(v): k for k, v in _NP_OF_DTYPE.items()}
 
 
@@ -93,6 +95,12 @@ class QkvDesc(C.Structure):
     _fields_ = [("input", C.POINTER(Tensor)), ("layout", C.c_int), ("weights", _QkvWeights),
                 ("epilogue", C.POINTER(Epilogue)), ("out_q", C.POINTER(Tensor)), ("out_k", C.POINTER(Tensor)),
                 ("out_v", C.POINTER(Tensor)), ("rope_params", C.POINTER(RopeParams))]
+
+
+class EmbeddingGatherDesc(C.Structure):
+    _fields_ = [("weights", C.POINTER(Tensor)), ("token_ids", C.POINTER(Tensor)), ("out", C.POINTER(Tensor)),
+                ("dtype_out", C.c_int), ("scale", C.c_float), ("padding_id", C.c_int32), ("bounds_check", C.c_bool),
+                ("prefer_gpu_private", C.c_int), ("allow_quant_decode_on_the_fly", C.c_int)]
 
 
 class TopkDesc(C.Structure):
@@ -235,7 +243,7 @@ BACKEND_SYMBOLS = [
     "marmot_hip_default_preferences", "marmot_hip_bc_get_tables",
     "hip_matmul_quantized_q4_0", "hip_matmul_quantized_q8_0", "hip_matmul_quantized_q4_k",
     "hip_matmul_quantized_q6_k", "hip_matmul_qkv_q4_0", "hip_matmul_qkv_q8_0", "hip_matmul_qkv_q4_k",
-    "hip_matmul_qkv_q6_k", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
+    "hip_matmul_qkv_q6_k", "hip_embedding_gather", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
 ]
 
@@ -259,6 +267,8 @@ def bind(lib: C.CDLL) -> C.CDLL:
         fn = getattr(lib, f"hip_matmul_qkv_{name}")
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p, C.POINTER(QkvDesc)]
+    lib.hip_embedding_gather.restype = C.c_int
+    lib.hip_embedding_gather.argtypes = [C.c_void_p, C.POINTER(EmbeddingGatherDesc)]
     lib.hip_moe_experts_impl.restype = C.c_int
     lib.hip_moe_experts_impl.argtypes = [C.c_void_p, C.POINTER(MoeDesc)]
     lib.hip_topk_impl.restype = C.c_int
@@ -409,6 +419,18 @@ class HipContext:
             sig.epilogue_flags |= EPILOGUE_ROPE
         return sig
 
+    def embedding_signature(self, table: HostTensor, ids: HostTensor, out: HostTensor) -> OpSignature:
+        """The index dtype is this operation's input dtype (src/backends/cpu/kernels/embedding.def:19-30)."""
+        sig = OpSignature()
+        sig.op_id = OP_EMBEDDING
+        sig.input_dtype = ids.t.dtype
+        sig.weight_dtype = table.t.dtype
+        sig.output_dtype = out.t.dtype
+        sig.accum_dtype = DTYPE_F32
+        sig.qscheme_id = QSCHEME_OF_KIND.get(table.t.quant_kind, 0)
+        sig.weight_layout = WEIGHT_LAYOUT_SEPARATE
+        return sig
+
     def query(self, sig: OpSignature, caps: Optional[DeviceCaps] = None) -> KernelSelection:
         caps = caps if caps is not None else self.lib.marmot_hip_detect_default_caps()
         return self.lib.marmot_hip_query_kernel(C.byref(sig), C.byref(caps))
@@ -489,6 +511,12 @@ class Program:
             rope_off = self._const(bytes(rope), 8)
         self.code += struct.pack("<H7HII3H", op_index, *[self.reg(t) for t in (x, wq, wk, wv, bq, bk, bv)],
                                  BC_INVALID_OFFSET, rope_off, self.reg(out_q), self.reg(out_k), self.reg(out_v))
+
+    def embedding(self, op_index: int, table: HostTensor, ids: HostTensor, out: HostTensor, scale: float = 1.0,
+                  padding_id: int = -1, bounds_check: bool = True):
+        """bytecode_compile.c:989-1018."""
+        self.code += struct.pack("<H3HIfI3B", op_index, self.reg(table), self.reg(ids), self.reg(out), out.t.dtype,
+                                 scale, padding_id & 0xFFFFFFFF, int(bounds_check), 0, 1)
 
     def moe_experts(self, op_index: int, hidden, gate, up, down, ids, weights, out, ffn_type=0, weights_scale=1.0,
                     policy=1):

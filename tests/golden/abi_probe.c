@@ -48,6 +48,8 @@ int main(void) {
     VAL(MARMOT_QKV_LAYOUT_FUSED); VAL(MARMOT_QKV_LAYOUT_SEPARATE);
     VAL(MARMOT_ROPE_SCALING_NONE); VAL(MARMOT_ROPE_SCALING_YARN); VAL(MARMOT_ROPE_TYPE_NORM); VAL(MARMOT_ROPE_TYPE_NEOX);
     VAL(MARMOT_EPILOGUE_ROPE); VAL(MARMOT_BC_SCHEMA_QKV);
+    VAL(MARMOT_OP_EMBEDDING); VAL(MARMOT_BC_SCHEMA_EMBEDDING); VAL(MARMOT_DTYPE_INT64);
+    VAL(MARMOT_PREFERENCE_ENABLE); VAL(MARMOT_PREFERENCE_DISABLE);
     VAL(MARMOT_QSCHEME_Q4_0); VAL(MARMOT_QSCHEME_Q8_0); VAL(MARMOT_QSCHEME_Q4_K); VAL(MARMOT_QSCHEME_Q6_K);
     VAL(MARMOT_QSCHEME_Q8_K);
     VAL(MARMOT_MATMUL_LAYOUT_NT); VAL(MARMOT_WEIGHT_LAYOUT_SEPARATE); VAL(MARMOT_STRIDE_MODE_CONTIGUOUS);
@@ -88,6 +90,11 @@ int main(void) {
     OFF(marmot_matmul_qkv_desc_t, out_k); OFF(marmot_matmul_qkv_desc_t, out_v);
     OFF(marmot_matmul_qkv_desc_t, rope_params);
     SZ(marmot_matmul_qkv_separate_t); OFF(marmot_matmul_qkv_separate_t, wv); OFF(marmot_matmul_qkv_separate_t, bq);
+    SZ(marmot_embedding_gather_desc_t); OFF(marmot_embedding_gather_desc_t, out);
+    OFF(marmot_embedding_gather_desc_t, dtype_out); OFF(marmot_embedding_gather_desc_t, scale);
+    OFF(marmot_embedding_gather_desc_t, padding_id); OFF(marmot_embedding_gather_desc_t, bounds_check);
+    OFF(marmot_embedding_gather_desc_t, prefer_gpu_private);
+    OFF(marmot_embedding_gather_desc_t, allow_quant_decode_on_the_fly);
     SZ(marmot_topk_desc_t); OFF(marmot_topk_desc_t, axis); OFF(marmot_topk_desc_t, k);
     SZ(marmot_moe_experts_desc_t); OFF(marmot_moe_experts_desc_t, out); OFF(marmot_moe_experts_desc_t, ffn_type);
     OFF(marmot_moe_experts_desc_t, weights_scale); OFF(marmot_moe_experts_desc_t, router_weight_policy);

@@ -64,6 +64,7 @@ def test_ctypes_structs_match_layout(golden_layout):
         "marmot_backend_preferences_t": ta.BackendPreferences, "marmot_matmul_dims_t": ta.MatmulDims,
         "marmot_quant_block_t": ta.QuantBlock, "marmot_rope_params_t": ta.RopeParams,
         "marmot_matmul_qkv_desc_t": ta.QkvDesc, "marmot_matmul_qkv_separate_t": ta.QkvSeparate,
+        "marmot_embedding_gather_desc_t": ta.EmbeddingGatherDesc,
     }
     checked = 0
     for cname, cls in pairs.items():
@@ -77,6 +78,10 @@ def test_ctypes_structs_match_layout(golden_layout):
     assert ta.OP_MATMUL == golden_layout["MARMOT_OP_MATMUL"]
     assert ta.OP_MOE_EXPERTS == golden_layout["MARMOT_OP_MOE_EXPERTS"]
     assert ta.OP_TOPK == golden_layout["MARMOT_OP_TOPK"]
+    assert ta.OP_EMBEDDING == golden_layout["MARMOT_OP_EMBEDDING"]
+    assert ta.DTYPE_I64 == golden_layout["MARMOT_DTYPE_INT64"]
+    assert (ta.PREFERENCE_ENABLE, ta.PREFERENCE_DISABLE) == (
+        golden_layout["MARMOT_PREFERENCE_ENABLE"], golden_layout["MARMOT_PREFERENCE_DISABLE"])
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q4_K] == golden_layout["MARMOT_QSCHEME_Q4_K"]
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q6_K] == golden_layout["MARMOT_QSCHEME_Q6_K"]
     assert ta.KIND_Q8_K == golden_layout["MARMOT_QUANT_KIND_Q8_K"]
@@ -233,11 +238,30 @@ def test_default_caps_and_preferences(lib):
     assert not lib.marmot_hip_default_preferences(None, C.byref(prefs))
 
 
+def test_query_kernel_embedding_rules(lib):
+    """cpu/kernels/embedding.def:19-30 with this backend's schemes, index and output types."""
+    def sig(kind=ta.KIND_Q4_K, ids=ta.DTYPE_I32, out=ta.DTYPE_F32):
+        s = ta.OpSignature()
+        s.op_id, s.input_dtype, s.weight_dtype, s.output_dtype = ta.OP_EMBEDDING, ids, ta.DTYPE_U8, out
+        s.qscheme_id = ta.QSCHEME_OF_KIND.get(kind, 0)
+        s.weight_layout = ta.WEIGHT_LAYOUT_SEPARATE
+        return s
+    for kind, op in ((ta.KIND_Q4_0, 16), (ta.KIND_Q8_0, 17), (ta.KIND_Q4_K, 18), (ta.KIND_Q6_K, 19)):
+        for ids in (ta.DTYPE_I32, ta.DTYPE_I64):
+            for out in (ta.DTYPE_F32, ta.DTYPE_F16):
+                sel = _query(lib, sig(kind, ids, out))
+                assert sel.supported and sel.op_index == op
+    assert not _query(lib, sig(kind=ta.KIND_Q8_K)).supported
+    assert not _query(lib, sig(kind=ta.KIND_GENERIC)).supported
+    assert not _query(lib, sig(ids=ta.DTYPE_F32)).supported
+    assert not _query(lib, sig(out=ta.DTYPE_I32)).supported
+
+
 def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 16
+    assert t.op_count == 20
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -246,6 +270,7 @@ def test_bytecode_tables(lib, golden_layout):
     assert schema[10] == golden_layout["MARMOT_BC_SCHEMA_QUANTIZE"]
     assert schema[11] == golden_layout["MARMOT_BC_SCHEMA_DEQUANTIZE"]
     assert schema[12:16] == [golden_layout["MARMOT_BC_SCHEMA_QKV"]] * 4
+    assert schema[16:20] == [golden_layout["MARMOT_BC_SCHEMA_EMBEDDING"]] * 4
     # immediate sizes equal what the encoders of tensor_abi.Program emit (opcode excluded)
     sizes = [t.imm_size[i] for i in range(t.op_count)]
     assert sizes[1:5] == [struct.calcsize("<HHHIH")] * 4
@@ -254,6 +279,7 @@ def test_bytecode_tables(lib, golden_layout):
     assert sizes[10] == struct.calcsize("<HIHII")
     assert sizes[11] == struct.calcsize("<HHII")
     assert sizes[12:16] == [struct.calcsize("<7HII3H")] * 4
+    assert sizes[16:20] == [struct.calcsize("<3HIfI3B")] * 4 == [21] * 4
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -272,6 +298,7 @@ def test_exec_entries_reject_null_arguments(lib):
     assert lib.hip_moe_experts_impl(None, None) == ta.INVALID_ARGUMENT
     assert lib.hip_matmul_qkv_q4_k(None, None) == ta.INVALID_ARGUMENT
     assert lib.hip_topk_impl(None, None) == ta.INVALID_ARGUMENT
+    assert lib.hip_embedding_gather(None, None) == ta.INVALID_ARGUMENT
 
 
 def test_program_encoding_matches_reference_immediates():
@@ -296,6 +323,12 @@ def test_program_encoding_matches_reference_immediates():
     rp.theta, rp.apply_to_q = 10000.0, True
     q.qkv(14, x, w, w, w, *outs, rope=rp)
     assert struct.unpack_from("<I", q.code, 30 + 2 + 14 + 4)[0] == 0 and len(q.const_pool) == C.sizeof(ta.RopeParams)
+    # EMBEDDING: table, ids, out; output dtype, scale, padding id, three flag bytes
+    e = ta.Program()
+    ids = ta.HostTensor.dense(np.zeros((2, 3), np.int64))
+    eo = ta.HostTensor.empty((2, 3, 256), ta.DTYPE_F16)
+    e.embedding(18, w, ids, eo, scale=0.5, padding_id=-1, bounds_check=True)
+    assert bytes(e.code) == struct.pack("<H3HIfI3B", 18, 0, 1, 2, ta.DTYPE_F16, 0.5, 0xFFFFFFFF, 1, 0, 1)
     # tensor strides are row-major element strides, as marmot_tensor_create fills them
     assert list(x.t.shape.strides[:2]) == [256, 1] and x.t.shape.ndim == 2
 
@@ -310,7 +343,8 @@ def test_kernel_def_files_name_exported_impls(lib):
             families[name] = fields
     qkv = {f"{op}_quantized_hip_{dt}" for op in ("qkv_shared_input", "qkv_projection") for dt in ("f16", "f32")}
     assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_q6_k", "topk_hip",
-                             "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip"} | qkv
+                             "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
+                             "embedding_quantized_hip"} | qkv
     for name in qkv:
         f = families[name]
         assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name
@@ -320,7 +354,7 @@ def test_kernel_def_files_name_exported_impls(lib):
         for s in schemes:
             sym = impl.replace("{scheme:lower}", s.lower())
             assert hasattr(lib, sym), f"{name}: {sym} not exported"
-        assert f["PLATFORM"] == "HIP" and f["PROFILE"] == "ANY"
+        assert f["PLATFORM"] == "HIP" and f["PROFILE"] == ("NONE" if f["OP"] == "embedding" else "ANY")
     mm = families["matmul_quantized_hip"]
     assert mm["OP"] == "matmul" and mm["MATMUL_LAYOUT"] == "NT" and mm["WEIGHT_LAYOUT"] == "SEPARATE"
     assert mm["EPILOGUE"] == "[BIAS]" and mm["ACCUM_DTYPE"] == "FLOAT32" and mm["STRIDE_MODE"] == "CONTIGUOUS"

@@ -425,3 +425,79 @@ def test_program_qkv_with_rotary_epilogue(ctx, oracle, dtype):
         assert ctx.residency().uploads - before == first_uploads
     for t in [xt, pt] + wts + outs + bts:
         ctx.host_freed(t)
+
+
+# ---------------------------------------------------------------- embedding gather
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K])
+def test_impl_and_program_embedding_gather(ctx, oracle, kind):
+    """marmot_embedding_gather on a quantized table: the impl function with a descriptor and the EMBEDDING bytecode
+    schema, ids of rank 2 (flattened), float32 bit-exact and float16 with scale; the table stays resident."""
+    from tests.util import random_valid_blocks
+
+    print(f"backend embedding kind={kind}", flush=True)
+    rng = np.random.default_rng(960 + kind)
+    vocab, dim = 300, 1024
+    table = random_valid_blocks(rng, kind, vocab, dim)
+    ids = rng.integers(0, vocab, (3, 5)).astype(np.int64)
+    ids[0, 1] = 11
+    tt = ta.HostTensor.quantized(table, (vocab, dim), kind)
+    it = ta.HostTensor.dense(ids)
+    ot = ta.HostTensor.empty((3, 5, dim), ta.DTYPE_F32)
+    desc = ta.EmbeddingGatherDesc()
+    desc.weights, desc.token_ids, desc.out = tt.ptr, it.ptr, ot.ptr
+    desc.dtype_out, desc.scale, desc.padding_id, desc.bounds_check = ta.DTYPE_F32, 1.0, 11, True
+    assert ctx.lib.hip_embedding_gather(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
+    assert ot.t.memory_location == ta.MEMORY_DEVICE and ot.t.needs_sync
+    ref = oracle.embedding_gather(kind, table, vocab, dim, ids, padding_id=11)
+    assert np.array_equal(bits(ctx.to_host(ot)), bits(ref)) and not ot.array[0, 1].any()
+
+    o16 = ta.HostTensor.empty((15, dim), ta.DTYPE_F16)
+    i32 = ta.HostTensor.dense(ids.astype(np.int32).reshape(-1))
+    sel = ctx.query(ctx.embedding_signature(tt, i32, o16))
+    assert sel.supported and sel.op_index == {KIND_Q4_0: 16, KIND_Q8_0: 17, KIND_Q4_K: 18, KIND_Q6_K: 19}[kind]
+    before = ctx.residency().upload_bytes
+    prog = ta.Program()
+    prog.embedding(sel.op_index, tt, i32, o16, scale=0.25, padding_id=-1, bounds_check=False)
+    assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+    ref16 = oracle.embedding_gather(kind, table, vocab, dim, ids.reshape(-1), out_dtype=np.float16, scale=0.25)
+    assert np.array_equal(ctx.to_host(o16).view(np.uint16), ref16.view(np.uint16))
+    assert ctx.residency().upload_bytes - before == i32.array.nbytes  # the table was not uploaded again
+    for t in (tt, it, ot, o16, i32):
+        ctx.host_freed(t)
+
+
+def test_embedding_gather_errors(ctx):
+    from tests.util import random_valid_blocks
+
+    vocab, dim = 8, 256
+    table = random_valid_blocks(np.random.default_rng(970), KIND_Q4_K, vocab, dim)
+    tt = ta.HostTensor.quantized(table, (vocab, dim), KIND_Q4_K)
+    ids = ta.HostTensor.dense(np.array([1, 8, 2], np.int32))
+    out = ta.HostTensor.empty((3, dim), ta.DTYPE_F32)
+
+    def call(weights=tt, token_ids=ids, o=out, bounds=True):
+        d = ta.EmbeddingGatherDesc()
+        d.weights, d.token_ids, d.out = weights.ptr, token_ids.ptr, o.ptr
+        d.dtype_out, d.scale, d.padding_id, d.bounds_check = o.t.dtype, 1.0, -1, bounds
+        return ctx.lib.hip_embedding_gather(ctx.device_ctx, C.byref(d))
+
+    # embedding_scalar.c:556-559: an id outside the table with the bounds check on
+    assert call() == ta.INVALID_ARGUMENT and "out of range" in ctx.last_error()[1]
+    assert call(bounds=False) == ta.SUCCESS and not ctx.to_host(out)[1].any()
+    tmp = {
+        "float_ids": ta.HostTensor.dense(np.zeros(3, np.float32)),
+        "int_out": ta.HostTensor.empty((3, dim), ta.DTYPE_I32),
+        "short_out": ta.HostTensor.empty((2, dim), ta.DTYPE_F32),
+        "q8_k": ta.HostTensor.quantized(table, (vocab, dim), KIND_Q8_K),
+        "flat": ta.HostTensor.quantized(table, (vocab * dim,), KIND_Q4_K),
+        "no_ids": ta.HostTensor(np.zeros(1, np.int32), (0,), ta.DTYPE_I32),
+        "no_out": ta.HostTensor(np.zeros(1, np.float32), (0, dim), ta.DTYPE_F32),
+    }
+    assert call(token_ids=tmp["float_ids"]) == ta.UNSUPPORTED_DTYPE
+    assert call(o=tmp["int_out"]) == ta.UNSUPPORTED_DTYPE
+    assert call(o=tmp["short_out"]) == ta.DIMENSION_MISMATCH
+    assert call(weights=tmp["q8_k"]) == ta.NOT_IMPLEMENTED
+    assert call(weights=tmp["flat"]) == ta.DIMENSION_MISMATCH
+    assert call(token_ids=tmp["no_ids"], o=tmp["no_out"]) == ta.SUCCESS
+    for t in [tt, ids, out] + list(tmp.values()):
+        ctx.host_freed(t)

@@ -45,6 +45,13 @@ typedef struct {
     uint8_t qs[128];
 } blk_q4_k; /* 144 B */
 typedef struct {
+    uint16_t d;
+    uint16_t dmin;
+    uint8_t scales[12];
+    uint8_t qh[32];
+    uint8_t qs[128];
+} blk_q5_k; /* 176 B */
+typedef struct {
     uint8_t ql[128];
     uint8_t qh[64];
     int8_t scales[16];
@@ -60,6 +67,7 @@ typedef struct {
 _Static_assert(sizeof(blk_q4_0) == 18, "Q4_0");
 _Static_assert(sizeof(blk_q8_0) == 34, "Q8_0");
 _Static_assert(sizeof(blk_q4_k) == 144, "Q4_K");
+_Static_assert(sizeof(blk_q5_k) == 176, "Q5_K");
 _Static_assert(sizeof(blk_q6_k) == 210, "Q6_K");
 _Static_assert(sizeof(blk_q8_k) == 292, "Q8_K");
 
@@ -69,6 +77,7 @@ size_t mo_block_values(int kind) {
     case MO_KIND_Q8_0:
         return QK;
     case MO_KIND_Q4_K:
+    case MO_KIND_Q5_K:
     case MO_KIND_Q6_K:
     case MO_KIND_Q8_K:
         return QK_K;
@@ -85,6 +94,8 @@ size_t mo_block_bytes(int kind) {
         return sizeof(blk_q8_0);
     case MO_KIND_Q4_K:
         return sizeof(blk_q4_k);
+    case MO_KIND_Q5_K:
+        return sizeof(blk_q5_k);
     case MO_KIND_Q6_K:
         return sizeof(blk_q6_k);
     case MO_KIND_Q8_K:
@@ -489,6 +500,134 @@ static void q4_k_dequantize_block(const blk_q4_k *block, uint32_t elems, float *
     }
 }
 
+/* ======================= Q5_K ======================= */
+
+/* q5k_gguf.c:35-160: the Q4_K search with 31 levels (rmin -0.5, 15 steps); the fifth bit of value 64g + l
+ * (low nibble) is bit 2g of qh[l], of value 64g + 32 + l (high nibble) bit 2g + 1 */
+static void q5_k_quantize_block(const float *values, uint32_t elems, blk_q5_k *block) {
+    float bv[QK_K];
+    memcpy(bv, values, elems * sizeof(float));
+    if (elems < QK_K) {
+        memset(bv + elems, 0, (QK_K - elems) * sizeof(float));
+    }
+    uint8_t L[QK_K];
+    memset(L, 0, sizeof(L));
+    uint8_t Laux[32];
+    float weights[32];
+    float scales[QK_K / 32];
+    float mins[QK_K / 32];
+    memset(block, 0, sizeof(*block));
+
+    float max_scale = 0.0f;
+    float max_min = 0.0f;
+    for (int j = 0; j < QK_K / 32; ++j) {
+        float sum_x2 = 0.0f;
+        for (int l = 0; l < 32; ++l) {
+            const float v = bv[32 * j + l];
+            sum_x2 += v * v;
+        }
+        const float av_x = sqrtf(sum_x2 / 32.0f);
+        for (int l = 0; l < 32; ++l) {
+            weights[l] = av_x + fabsf(bv[32 * j + l]);
+        }
+        scales[j] = make_qkx2_quants(32, 31, bv + 32 * j, weights, L + 32 * j, &mins[j], Laux, -0.5f, 0.1f, 15);
+        if (scales[j] > max_scale) {
+            max_scale = scales[j];
+        }
+        if (mins[j] > max_min) {
+            max_min = mins[j];
+        }
+    }
+
+    const float inv_scale = max_scale > 0 ? 63.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0 ? 63.0f / max_min : 0.0f;
+    for (int j = 0; j < QK_K / 32; ++j) {
+        uint8_t ls = (uint8_t)nearbyintf(inv_scale * scales[j]);
+        uint8_t lm = (uint8_t)nearbyintf(inv_min * mins[j]);
+        ls = ls > 63 ? 63 : ls;
+        lm = lm > 63 ? 63 : lm;
+        if (j < 4) {
+            block->scales[j] = ls;
+            block->scales[j + 4] = lm;
+        } else {
+            block->scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+            block->scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            block->scales[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+    block->d = mo_f32_to_f16(max_scale / 63.0f);
+    block->dmin = mo_f32_to_f16(max_min / 63.0f);
+
+    for (int j = 0; j < QK_K / 32; ++j) {
+        uint8_t sc, m;
+        get_scale_min_k4(j, block->scales, &sc, &m);
+        const float d = mo_f16_to_f32(block->d) * sc;
+        if (d == 0) {
+            continue;
+        }
+        const float dm = mo_f16_to_f32(block->dmin) * m;
+        for (int ii = 0; ii < 32; ++ii) {
+            int l = (int)nearbyintf((bv[32 * j + ii] + dm) / d);
+            l = l > 31 ? 31 : (l < 0 ? 0 : l);
+            L[32 * j + ii] = (uint8_t)l;
+        }
+    }
+
+    uint8_t *ql = block->qs;
+    for (int g = 0; g < QK_K / 64; ++g) {
+        for (int j = 0; j < 32; ++j) {
+            int l1 = L[64 * g + j];
+            int l2 = L[64 * g + j + 32];
+            if (l1 > 15) {
+                l1 -= 16;
+                block->qh[j] |= (uint8_t)(1u << (2 * g));
+            }
+            if (l2 > 15) {
+                l2 -= 16;
+                block->qh[j] |= (uint8_t)(2u << (2 * g));
+            }
+            ql[j] = (uint8_t)(l1 | (l2 << 4));
+        }
+        ql += 32;
+    }
+    if (elems < QK_K) {
+        const size_t qs_offset = (elems + 1) / 2;
+        const size_t qh_offset = (elems + 63) / 64;
+        if (qs_offset < sizeof(block->qs)) {
+            memset(block->qs + qs_offset, 0, sizeof(block->qs) - qs_offset);
+        }
+        if (qh_offset < sizeof(block->qh)) {
+            memset(block->qh + qh_offset, 0, sizeof(block->qh) - qh_offset);
+        }
+    }
+}
+
+/* q5k_gguf.c:162-198: d1 = d*sc; m1 = dmin*m; y = d1*q - m1, each op rounded */
+static void q5_k_dequantize_block(const blk_q5_k *block, uint32_t elems, float *out) {
+    const uint8_t *ql = block->qs;
+    const float d = mo_f16_to_f32(block->d);
+    const float min = mo_f16_to_f32(block->dmin);
+    size_t written = 0;
+    for (int g = 0; g < QK_K / 64 && written < elems; ++g) {
+        uint8_t sc, m;
+        get_scale_min_k4(2 * g, block->scales, &sc, &m);
+        const float d1 = d * sc;
+        const float m1 = min * m;
+        get_scale_min_k4(2 * g + 1, block->scales, &sc, &m);
+        const float d2 = d * sc;
+        const float m2 = min * m;
+        for (int l = 0; l < 32 && written < elems; ++l, ++written) {
+            const int q = (ql[l] & 0xF) | (((block->qh[l] >> (2 * g)) & 1) << 4);
+            out[written] = d1 * q - m1;
+        }
+        for (int l = 0; l < 32 && written < elems; ++l, ++written) {
+            const int q = (ql[l] >> 4) | (((block->qh[l] >> (2 * g + 1)) & 1) << 4);
+            out[written] = d2 * q - m2;
+        }
+        ql += 32;
+    }
+}
+
 /* ======================= Q6_K ======================= */
 
 static inline int clamp_qx(int value, int nmax) {
@@ -791,6 +930,9 @@ int mo_quantize_rows(int kind, const float *x, size_t rows, size_t k, void *out)
             case MO_KIND_Q4_K:
                 q4_k_quantize_block(src, elems, (blk_q4_k *)blk);
                 break;
+            case MO_KIND_Q5_K:
+                q5_k_quantize_block(src, elems, (blk_q5_k *)blk);
+                break;
             case MO_KIND_Q6_K:
                 q6_k_quantize_block(src, elems, (blk_q6_k *)blk);
                 break;
@@ -835,6 +977,9 @@ int mo_dequantize_rows(int kind, const void *blocks, size_t rows, size_t k, floa
                 break;
             case MO_KIND_Q4_K:
                 q4_k_dequantize_block((const blk_q4_k *)blk, elems, dst);
+                break;
+            case MO_KIND_Q5_K:
+                q5_k_dequantize_block((const blk_q5_k *)blk, elems, dst);
                 break;
             case MO_KIND_Q6_K:
                 q6_k_dequantize_block((const blk_q6_k *)blk, elems, dst);
@@ -914,6 +1059,41 @@ float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks) {
             int32_t dot = 0;
             for (int l = 0; l < 32; ++l) {
                 const int32_t wv = high ? (q4[l] >> 4) : (q4[l] & 0x0F);
+                dot += wv * (int32_t)q8[l];
+            }
+            block_sum += (int32_t)scales[sg] * dot;
+        }
+        const float d = ab[b].d * mo_f16_to_f32(wb[b].d);
+        const float dmin = ab[b].d * mo_f16_to_f32(wb[b].dmin);
+        sum_all += d * (float)block_sum - dmin * (float)sumi;
+    }
+    return sum_all;
+}
+
+/* vec_dot_impl.h:734-781 */
+float mo_vec_dot_q5_k_q8_k(const void *w, const void *a, size_t nblocks) {
+    const blk_q5_k *wb = (const blk_q5_k *)w;
+    const blk_q8_k *ab = (const blk_q8_k *)a;
+    float sum_all = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        uint8_t scales[8];
+        uint8_t mins[8];
+        for (int j = 0; j < 8; ++j) {
+            get_scale_min_k4(j, wb[b].scales, &scales[j], &mins[j]);
+        }
+        int32_t sumi = 0;
+        for (int j = 0; j < QK_K / 16; ++j) {
+            sumi += (int32_t)ab[b].bsums[j] * (int32_t)mins[j / 2];
+        }
+        int32_t block_sum = 0;
+        for (int sg = 0; sg < 8; ++sg) {
+            const uint8_t *q4 = wb[b].qs + (sg / 2) * 32;
+            const int8_t *q8 = ab[b].qs + sg * 32;
+            const int high = sg & 1;
+            int32_t dot = 0;
+            for (int l = 0; l < 32; ++l) {
+                const int32_t hi = ((wb[b].qh[l] >> sg) & 1) ? 16 : 0;
+                const int32_t wv = (high ? (q4[l] >> 4) : (q4[l] & 0x0F)) + hi;
                 dot += wv * (int32_t)q8[l];
             }
             block_sum += (int32_t)scales[sg] * dot;
@@ -1023,6 +1203,47 @@ float mo_vec_dot_f16(int kind, const void *w, const uint16_t *a, size_t nblocks,
                 is += 2;
             }
         }
+    } else if (kind == MO_KIND_Q5_K) {
+        /* vec_dot_impl.h:1025-1080 as written: the fifth bit is taken from byte j/8 + l (+ 32 for the high nibbles)
+         * counted from the start of qh, bit j % 8 = 0, i.e. for j >= 64 and for every high nibble from bytes that
+         * belong to other elements or to qs; it differs from the Q5_K dequantizer. Restated so that the reference's
+         * snapshot of this function (golden_matmul_llama.h:1355) is reproduced; no product kernel mirrors it. */
+        const blk_q5_k *wb = (const blk_q5_k *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const uint8_t *ql = wb[b].qs;
+            const uint8_t *qh = (const uint8_t *)&wb[b] + offsetof(blk_q5_k, qh); /* indexed past qh into qs */
+            const float d = mo_f16_to_f32(wb[b].d);
+            const float dmin = mo_f16_to_f32(wb[b].dmin);
+            const size_t start = b * QK_K;
+            const size_t len = (start + QK_K <= k) ? QK_K : (k - start);
+            size_t written = 0;
+            int is = 0;
+            for (size_t j = 0; j < QK_K && written < len; j += 64) {
+                uint8_t sc, m;
+                get_scale_min_k4(is + 0, wb[b].scales, &sc, &m);
+                const float d1 = d * (float)sc;
+                const float m1 = dmin * (float)m;
+                get_scale_min_k4(is + 1, wb[b].scales, &sc, &m);
+                const float d2 = d * (float)sc;
+                const float m2 = dmin * (float)m;
+                for (int l = 0; l < 32 && written < len; ++l, ++written) {
+                    const uint8_t h = (uint8_t)(qh[j / 8 + l] >> (j % 8) & 1);
+                    const uint8_t q = (uint8_t)((ql[l] & 0xF) | (h << 4));
+                    const float av = mo_f16_to_f32(a[start + written]);
+                    const float wv = d1 * (float)q - m1;
+                    total += wv * av;
+                }
+                for (int l = 0; l < 32 && written < len; ++l, ++written) {
+                    const uint8_t h = (uint8_t)(qh[j / 8 + l + 32] >> (j % 8) & 1);
+                    const uint8_t q = (uint8_t)((ql[l] >> 4) | (h << 4));
+                    const float av = mo_f16_to_f32(a[start + written]);
+                    const float wv = d2 * (float)q - m2;
+                    total += wv * av;
+                }
+                ql += 32;
+                is += 2;
+            }
+        }
     } else if (kind == MO_KIND_Q6_K) {
         const blk_q6_k *wb = (const blk_q6_k *)w;
         for (size_t b = 0; b < nblocks; ++b) {
@@ -1060,6 +1281,8 @@ static dot_fn pick_dot(int kind) {
         return mo_vec_dot_q4_0_q8_0;
     case MO_KIND_Q4_K:
         return mo_vec_dot_q4_k_q8_k;
+    case MO_KIND_Q5_K:
+        return mo_vec_dot_q5_k_q8_k;
     case MO_KIND_Q6_K:
         return mo_vec_dot_q6_k_q8_k;
     default:
@@ -1554,6 +1777,9 @@ int mo_embedding_gather_quantized(
                 break;
             case MO_KIND_Q4_K:
                 q4_k_dequantize_block((const blk_q4_k *)blk, (uint32_t)count, decoded);
+                break;
+            case MO_KIND_Q5_K:
+                q5_k_dequantize_block((const blk_q5_k *)blk, (uint32_t)count, decoded);
                 break;
             case MO_KIND_Q6_K:
                 q6_k_dequantize_block((const blk_q6_k *)blk, (uint32_t)count, decoded);

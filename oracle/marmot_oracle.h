@@ -37,6 +37,7 @@ enum {
     MO_KIND_Q4_0 = 1,
     MO_KIND_Q8_0 = 5,
     MO_KIND_Q4_K = 9,
+    MO_KIND_Q5_K = 10,
     MO_KIND_Q6_K = 11,
     MO_KIND_Q8_K = 12,
 };
@@ -82,6 +83,7 @@ void mo_pack_q8_k(const void *x, int in_dtype, size_t k, void *blocks_out);
 float mo_vec_dot_q8_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q5_k_q8_k(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q6_k_q8_k(const void *w, const void *a, size_t nblocks);
 
 /* fp16-activation direct dots (vec_dot_impl.h:220-250, 419-450, 973-1023) */

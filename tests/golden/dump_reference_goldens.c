@@ -42,6 +42,8 @@ int main(void) {
     EMIT(g_llama_q8_0_dequant, "f4");
     EMIT(g_llama_q4_k, "u1");
     EMIT(g_llama_q4_k_dequant, "f4");
+    EMIT(g_llama_q5_k, "u1");
+    EMIT(g_llama_q5_k_dequant, "f4");
     EMIT(g_llama_q6_k, "u1");
     EMIT(g_llama_q6_k_dequant, "f4");
     EMIT(g_llama_q8_k, "u1");
@@ -55,10 +57,12 @@ int main(void) {
     EMIT(g_vec_dot_q4_0_weights, "u1");
     EMIT(g_vec_dot_q8_0_weights, "u1");
     EMIT(g_vec_dot_q4_k_weights, "u1");
+    EMIT(g_vec_dot_q5_k_weights, "u1");
     EMIT(g_vec_dot_q6_k_weights, "u1");
     EMIT_SCALAR(g_vec_dot_q4_0_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q8_0_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q4_k_q8_k_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q5_k_q8_k_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q6_k_q8_k_expected, "f4");
 
     /* whole-matmul goldens for the formats on the path */
@@ -66,7 +70,8 @@ int main(void) {
     for (size_t i = 0; i < ncases; ++i) {
         const matmul_golden_case_t *c = &g_matmul_quant_goldens[i];
         if (c->kind != MARMOT_QUANT_KIND_Q4_0 && c->kind != MARMOT_QUANT_KIND_Q8_0 &&
-            c->kind != MARMOT_QUANT_KIND_Q4_K && c->kind != MARMOT_QUANT_KIND_Q6_K) {
+            c->kind != MARMOT_QUANT_KIND_Q4_K && c->kind != MARMOT_QUANT_KIND_Q5_K &&
+            c->kind != MARMOT_QUANT_KIND_Q6_K) {
             continue;
         }
         char name[128];

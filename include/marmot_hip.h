@@ -45,6 +45,7 @@ enum {
     MARMOT_HIP_KIND_Q4_0 = 1,
     MARMOT_HIP_KIND_Q8_0 = 5,
     MARMOT_HIP_KIND_Q4_K = 9,
+    MARMOT_HIP_KIND_Q5_K = 10,
     MARMOT_HIP_KIND_Q6_K = 11,
     MARMOT_HIP_KIND_Q8_K = 12,
 };

@@ -21,6 +21,7 @@ constexpr int QK_K = 256;
 constexpr int Q4_0_BYTES = 18;
 constexpr int Q8_0_BYTES = 34;
 constexpr int Q4_K_BYTES = 144;
+constexpr int Q5_K_BYTES = 176;
 constexpr int Q6_K_BYTES = 210;
 constexpr int Q8_K_BYTES = 292;
 
@@ -38,6 +39,13 @@ struct __attribute__((packed)) BlockQ4_K {
     uint8_t scales[12];
     uint8_t qs[128];
 };
+struct __attribute__((packed)) BlockQ5_K {
+    uint16_t d;
+    uint16_t dmin;
+    uint8_t scales[12];
+    uint8_t qh[32];  // fifth bit of value 64 g + l: bit 2 g of qh[l]; of value 64 g + 32 + l: bit 2 g + 1
+    uint8_t qs[128];
+};
 struct __attribute__((packed)) BlockQ6_K {
     uint8_t ql[128];
     uint8_t qh[64];
@@ -52,6 +60,7 @@ struct __attribute__((packed)) BlockQ8_K {
 static_assert(sizeof(BlockQ4_0) == Q4_0_BYTES, "Q4_0");
 static_assert(sizeof(BlockQ8_0) == Q8_0_BYTES, "Q8_0");
 static_assert(sizeof(BlockQ4_K) == Q4_K_BYTES, "Q4_K");
+static_assert(sizeof(BlockQ5_K) == Q5_K_BYTES, "Q5_K");
 static_assert(sizeof(BlockQ6_K) == Q6_K_BYTES, "Q6_K");
 static_assert(sizeof(BlockQ8_K) == Q8_K_BYTES, "Q8_K");
 
@@ -61,6 +70,7 @@ inline size_t block_values(int kind) {
     case MARMOT_HIP_KIND_Q8_0:
         return QK;
     case MARMOT_HIP_KIND_Q4_K:
+    case MARMOT_HIP_KIND_Q5_K:
     case MARMOT_HIP_KIND_Q6_K:
     case MARMOT_HIP_KIND_Q8_K:
         return QK_K;
@@ -76,6 +86,8 @@ inline size_t block_bytes(int kind) {
         return Q8_0_BYTES;
     case MARMOT_HIP_KIND_Q4_K:
         return Q4_K_BYTES;
+    case MARMOT_HIP_KIND_Q5_K:
+        return Q5_K_BYTES;
     case MARMOT_HIP_KIND_Q6_K:
         return Q6_K_BYTES;
     case MARMOT_HIP_KIND_Q8_K:
@@ -83,6 +95,11 @@ inline size_t block_bytes(int kind) {
     default:
         return 0;
     }
+}
+// weight formats the matmul, QKV, embedding and MoE entry points accept
+inline bool is_weight_kind(int kind) {
+    return kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_K ||
+           kind == MARMOT_HIP_KIND_Q5_K || kind == MARMOT_HIP_KIND_Q6_K;
 }
 inline bool is_k_quant(int kind) {
     return block_values(kind) == QK_K;

@@ -31,6 +31,30 @@ __device__ __forceinline__ float dequant_value_q4_k(const uint8_t *blk, int v) {
     return d1 * (float)q - m1;
 }
 
+// Q5_K (q5k_gguf.c:162-198): the Q4_K formula with a fifth bit from qh
+__device__ __forceinline__ float dequant_value_q5_k(const uint8_t *blk, int v) {
+    const BlockQ5_K *b = (const BlockQ5_K *)blk;
+    const int j = v >> 5;
+    const int l = v & 31;
+    const int g = j >> 1;
+    uint8_t sc, m;
+    const uint8_t *s = b->scales;
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (uint8_t)((s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4));
+        m = (uint8_t)((s[j + 4] >> 4) | ((s[j] >> 6) << 4));
+    }
+    const float d = h2f(b->d);
+    const float dmin = h2f(b->dmin);
+    const float d1 = d * (float)sc;
+    const float m1 = dmin * (float)m;
+    const uint8_t byte = b->qs[32 * g + l];
+    const int q = ((j & 1) ? (byte >> 4) : (byte & 0xF)) | (((b->qh[l] >> j) & 1) << 4);
+    return d1 * (float)q - m1;
+}
+
 // Q6_K (q6k_gguf.c:63-99): y = (d * sc) * q
 __device__ __forceinline__ float dequant_value_q6_k(const uint8_t *blk, int v) {
     const BlockQ6_K *b = (const BlockQ6_K *)blk;
@@ -75,6 +99,8 @@ template <int KIND>
 __device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
     if constexpr (KIND == MARMOT_HIP_KIND_Q4_K) {
         return dequant_value_q4_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_K) {
+        return dequant_value_q5_k(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q6_K) {
         return dequant_value_q6_k(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q8_0) {
@@ -92,6 +118,7 @@ struct KindTraits {
     static constexpr int BB = KIND == MARMOT_HIP_KIND_Q4_0 ? Q4_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q8_0                     ? Q8_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q4_K                     ? Q4_K_BYTES
+        : KIND == MARMOT_HIP_KIND_Q5_K                     ? Q5_K_BYTES
         : KIND == MARMOT_HIP_KIND_Q6_K                     ? Q6_K_BYTES
                                                            : Q8_K_BYTES;
 };

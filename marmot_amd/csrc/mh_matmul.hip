@@ -141,9 +141,9 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
         set_route("matvec_q4_0_f16_direct");
         return launch_direct_kind<MARMOT_HIP_KIND_Q4_0>(dev, p, N);
     default:
-        // Q6_K: the reference's fp16 direct dot (vec_dot_impl.h:1082-1128) decodes blocks with an index pattern
-        // that disagrees with its own Q6_K dequantizer; this backend declines the combination so that the caller
-        // falls back (NOT_IMPLEMENTED is the reference's fallback signal, dispatch_execute.c:214-233).
+        // Q5_K and Q6_K: the reference's fp16 direct dots (vec_dot_impl.h:1025-1080, 1082-1128) decode blocks with
+        // index patterns that disagree with its own dequantizers; this backend declines the combination so that the
+        // caller falls back (NOT_IMPLEMENTED is the reference's fallback signal, dispatch_execute.c:214-233).
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED,
                          "quantized matmul: fp16 activations without packing are not offered for quant kind %d", kind);
     }
@@ -158,8 +158,7 @@ static int validate_matmul(const marmot_hip_device *dev, int kind, const void *d
     if (d_weight == nullptr || d_input == nullptr || d_out == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
     }
-    if (kind != MARMOT_HIP_KIND_Q4_0 && kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_K &&
-        kind != MARMOT_HIP_KIND_Q6_K) {
+    if (!is_weight_kind(kind)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "Quantized matmul kernel not available for quant kind %d",
                          kind);
     }
@@ -459,8 +458,7 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
         d_out_k == nullptr || d_out_v == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
     }
-    if (kind != MARMOT_HIP_KIND_Q4_0 && kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_K &&
-        kind != MARMOT_HIP_KIND_Q6_K) {
+    if (!is_weight_kind(kind)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "QKV projection kernel not available for quant kind %d",
                          kind);
     }

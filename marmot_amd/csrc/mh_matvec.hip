@@ -268,6 +268,75 @@ struct FmtQ4K {
     }
 };
 
+// ------------------------------------------------------------------ Q5_K x Q8_K
+// The Q4_K decomposition (8 lanes per block, lane sub owns 16 bytes of qs = 16 low-nibble and 16 high-nibble values)
+// plus the fifth bits: the 16 bytes of qh that belong to this lane's positions, bit 2 g for the low nibbles and bit
+// 2 g + 1 for the high ones (q5k_gguf.c:162-198, vec_dot_impl.h:734-781). Blocks are 176 = 11 * 16 bytes: aligned.
+struct FmtQ5K {
+    static constexpr int BYTES = Q5_K_BYTES;
+    static constexpr int LPB = 8;
+    static constexpr int BPW = 8;
+    static constexpr int BV = QK_K;
+    static constexpr int ACT_DW = 11, WT_DW = 12, QUANT_TMP = 56;
+    using Act = FmtQ4K::Act;
+    struct Wt {
+        uint4 hdr;  // d, dmin, scales[12]
+        uint4 qh;
+        uint4 q;
+    };
+    __device__ static void load_act(Act &a, const ActView &av, size_t n, size_t blk, int sub) {
+        FmtQ4K::load_act(a, av, n, blk, sub);
+    }
+    template <bool SIGNAL = false>
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
+        FmtQ4K::quant_act<SIGNAL>(a, xrow, blk, sub);
+    }
+    __device__ static void zero_act(Act &a) {
+        FmtQ4K::zero_act(a);
+    }
+    __device__ static void load_w(Wt &w, const uint8_t *blk, int sub) {
+        w.hdr = *(const uint4 *)blk;
+        w.qh = *(const uint4 *)(blk + 16 + 16 * (sub & 1));
+        w.q = *(const uint4 *)(blk + 48 + 16 * sub);
+    }
+    template <int NC>
+    __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int sub) {
+        const int g = sub >> 1;
+        const float d = h2f((uint16_t)(w.hdr.x & 0xffffu));
+        const float dmin = h2f((uint16_t)(w.hdr.x >> 16));
+        // scale / min pairs of sub-blocks 2g and 2g+1: as in FmtQ4K::accumulate
+        const int sh = 16 * (g & 1);
+        const uint32_t sa = w.hdr.y >> sh;
+        const uint32_t sb = w.hdr.z >> sh;
+        const uint32_t sc_ = w.hdr.w >> sh;
+        const bool hi_grp = g >= 2;
+        const uint32_t m_lo = hi_grp ? 0x0f0fu : 0x3f3fu;
+        const uint32_t m_hi = hi_grp ? 0x3030u : 0u;
+        const uint32_t scp = ((hi_grp ? sc_ : sa) & m_lo) | ((sa >> 2) & m_hi);
+        const uint32_t mp = ((hi_grp ? (sc_ >> 4) : sb) & m_lo) | ((sb >> 2) & m_hi);
+        const int sc0 = (int)(scp & 0xffu), sc1 = (int)((scp >> 8) & 0xffu);
+        const int m0 = (int)(mp & 0xffu), m1 = (int)((mp >> 8) & 0xffu);
+        const int b0 = 2 * g;  // bit of the low-nibble values; b0 + 1: of the high-nibble values
+        uint4 lo, hi;
+#define MH_Q5_UNPACK(c)                                                                                                \
+    lo.c = (w.q.c & 0x0f0f0f0fu) | (((w.qh.c >> b0) & 0x01010101u) << 4);                                              \
+    hi.c = ((w.q.c >> 4) & 0x0f0f0f0fu) | (((w.qh.c >> (b0 + 1)) & 0x01010101u) << 4);
+        MH_Q5_UNPACK(x)
+        MH_Q5_UNPACK(y)
+        MH_Q5_UNPACK(z)
+        MH_Q5_UNPACK(w)
+#undef MH_Q5_UNPACK
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+            const int dl = dot16(lo, a[n].lo, 0);
+            const int dh = dot16(hi, a[n].hi, 0);
+            const int isum = __mul24(sc0, dl) + __mul24(sc1, dh);
+            const int msum = __mul24(m0, a[n].bs_lo) + __mul24(m1, a[n].bs_hi);
+            acc[n] += (a[n].d * d) * (float)isum - (a[n].d * dmin) * (float)msum;
+        }
+    }
+};
+
 // ------------------------------------------------------------------ Q6_K x Q8_K
 struct FmtQ6K {
     static constexpr int BYTES = Q6_K_BYTES;
@@ -920,7 +989,7 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
         // are not aligned and the reads rely on unaligned LDS access. Measured faster for rows up to 8192 values
         // (14336 x 4096, N = 1 / 2 / 4: Q6_K 15.5 -> 12.9, 18.0 -> 16.7, 24.0 -> 23.5 us; Q8_0 18.4 -> 15.2,
         // 22.8 -> 16.4, 29.8 -> 22.5 us; Q8_0 5632 x 2048: 6.8 -> 6.1 us), slower for Q6_K at K = 14336.
-        const bool fmt_ok = std::is_same<Fmt, FmtQ4K>::value || K <= 8192;
+        const bool fmt_ok = Fmt::BYTES % 16 == 0 || K <= 8192;
         if (fmt_ok && matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
             // rows per workgroup: two workgroups per CU when M allows, between 8 (the activation prologue must pay
             // off) and 16 (more rows per workgroup leave CUs idle at the usual M)
@@ -968,9 +1037,14 @@ static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t 
         if (r == 2) {
             return launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name);
         }
-        return launch_tile_r<Fmt, NC, 4>(dev, p, K, M, nw, name);
+        const int st = launch_tile_r<Fmt, NC, 4>(dev, p, K, M, nw, name);
+        // a format with wide weight registers (Q5_K) covers long rows with fewer rows in flight
+        return st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED ? launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name) : st;
+    } else if constexpr (NC == 2) {
+        const int st = launch_tile_r<Fmt, NC, 4>(dev, p, K, M, nw, name);
+        return st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED ? launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name) : st;
     } else {
-        return launch_tile_r < Fmt, NC, (NC <= 2) ? 4 : 2 > (dev, p, K, M, nw, name);
+        return launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name);
     }
 }
 
@@ -1090,6 +1164,8 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
         return launch_fmt<FmtQ4K>(dev, p, N, K, M, nw, fused ? "matvec_q4_k_q8_k_fused" : "matvec_q4_k_q8_k");
+    case MARMOT_HIP_KIND_Q5_K:
+        return launch_fmt<FmtQ5K>(dev, p, N, K, M, nw, fused ? "matvec_q5_k_q8_k_fused" : "matvec_q5_k_q8_k");
     case MARMOT_HIP_KIND_Q6_K:
         return launch_fmt<FmtQ6K>(dev, p, N, K, M, nw, fused ? "matvec_q6_k_q8_k_fused" : "matvec_q6_k_q8_k");
     case MARMOT_HIP_KIND_Q8_0:
@@ -1142,6 +1218,9 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
         st = launch_tile<FmtQ4K, 8>(dev, p, K, M, nw, "moe_grouped_q4_k_q8_k");
+        break;
+    case MARMOT_HIP_KIND_Q5_K:
+        st = launch_tile<FmtQ5K, 8>(dev, p, K, M, nw, "moe_grouped_q5_k_q8_k");
         break;
     case MARMOT_HIP_KIND_Q6_K:
         st = launch_tile<FmtQ6K, 8>(dev, p, K, M, nw, "moe_grouped_q6_k_q8_k");

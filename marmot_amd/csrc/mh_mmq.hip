@@ -51,7 +51,7 @@ typedef __attribute__((address_space(3))) uint8_t lds_u8;
 typedef const __attribute__((address_space(1))) uint8_t glb_u8;
 
 constexpr int MMQ_TOK = 16;                // activation rows per pass
-constexpr int MMQ_WBLK = 32 * Q4_K_BYTES;  // one block of 32 weight rows: 4608 bytes
+// one block of 32 weight rows is 32 * 144 = 4608 bytes of Q4_K, 32 * 176 = 5632 bytes of Q5_K
 constexpr int MMQ_ABLK = MMQ_TOK * QK_K;   // one block of 16 activation rows: 4096 bytes
 constexpr int MMQ_STAGES = 2;              // Q6_K: blocks in flight per wavefront
 
@@ -152,12 +152,22 @@ __device__ __forceinline__ void mmq_store(const MmqParams &p, int which, int spl
 //
 // NR: live accumulator registers per lane: 4 for up to 8 activation rows (8 rows staged per block), 8 for up to 16
 // (token of register r: 8 * (r / 4) + 4 * kh + r % 4, the row layout of the 32x32 MFMA result).
-template <int NR, int STAGES>
+//
+// Q5: Q5_K weights. The block is the Q4_K block with 32 bytes of fifth bits between the scales and the nibbles
+// (176 bytes = 11 chunks, still an odd number of 16-byte chunks per row); sub-block sb takes bit sb of qh[l]
+// (q5k_gguf.c:162-198, vec_dot_impl.h:734-781). Everything else is shared.
+template <int NR, int STAGES, bool Q5 = false>
 __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
     constexpr int TOK = 2 * NR;
-    constexpr int A_OFF = MMQ_WBLK, D_OFF = A_OFF + TOK * QK_K, STAGE = D_OFF + TOK * 4;
-    constexpr int A_LOADS = TOK / 4;           // 16-byte chunks of the activation tile / 64 lanes
-    constexpr int LOADS = 5 + A_LOADS + 1;     // memory instructions per stage
+    constexpr int WBYTES = Q5 ? Q5_K_BYTES : Q4_K_BYTES;  // bytes per block
+    constexpr int PIECES = WBYTES / 16;                   // 16-byte chunks per block: 9 or 11
+    constexpr int QS_OFF = Q5 ? 48 : 16;                  // nibbles behind the header (and the fifth bits)
+    constexpr int W_CHUNKS = 32 * PIECES;                 // chunks of one stage of weights: 288 or 352
+    constexpr int W_LOADS = (W_CHUNKS + 63) / 64;         // 5 or 6, the last one by the first 32 lanes
+    static_assert(W_CHUNKS % 64 == 32, "the last weight load is issued by half a wavefront");
+    constexpr int A_OFF = 32 * WBYTES, D_OFF = A_OFF + TOK * QK_K, STAGE = D_OFF + TOK * 4;
+    constexpr int A_LOADS = TOK / 4;              // 16-byte chunks of the activation tile / 64 lanes
+    constexpr int LOADS = W_LOADS + A_LOADS + 1;  // memory instructions per stage
     constexpr int AHEAD = STAGES - 1;          // blocks the loader runs ahead of the consumers
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, W = (int)(blockDim.x >> 6) - 1;
@@ -201,12 +211,12 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
 
     if (loader) {
         // ---- per-lane source offsets (block-independent)
-        uint32_t w_off[5];  // weights: 288 chunks of 16 bytes in row order (9 per row)
+        uint32_t w_off[W_LOADS];  // weights: chunks of 16 bytes in row order (PIECES per row)
 #pragma unroll
-        for (int c = 0; c < 5; ++c) {
+        for (int c = 0; c < W_LOADS; ++c) {
             const int chunk = c * 64 + lane;
-            int row = chunk / 9;
-            const int piece = chunk - row * 9;
+            int row = chunk / PIECES;
+            const int piece = chunk - row * PIECES;
             if (row > 31) {
                 row = 31;
             }
@@ -214,9 +224,9 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
             if (m >= p.M) {
                 m = p.M - 1;  // harmless re-read; never stored
             }
-            w_off[c] = (uint32_t)((m - row0) * p.nb * Q4_K_BYTES + 16 * piece);
+            w_off[c] = (uint32_t)((m - row0) * p.nb * WBYTES + 16 * piece);
         }
-        const uint8_t *wgroup = wbase + row0 * p.nb * Q4_K_BYTES;
+        const uint8_t *wgroup = wbase + row0 * p.nb * WBYTES;
         uint32_t a_off[A_LOADS];  // activations: chunk (token, slot) holds source chunk slot ^ token
 #pragma unroll
         for (int c = 0; c < A_LOADS; ++c) {
@@ -245,9 +255,9 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
                     }
                     uint8_t *dst = lds + ((size_t)w * STAGES + (t % STAGES)) * STAGE;
 #pragma unroll
-                    for (int c = 0; c < 5; ++c) {
-                        if (c < 4 || lane < 32) {  // 288 = 4 * 64 + 32 chunks
-                            __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + b * Q4_K_BYTES),
+                    for (int c = 0; c < W_LOADS; ++c) {
+                        if (c < W_LOADS - 1 || lane < 32) {  // 288 = 4 * 64 + 32, 352 = 5 * 64 + 32 chunks
+                            __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + b * WBYTES),
                                                              (lds_u8 *)(dst + c * 1024), 16, 0, 0);
                         }
                     }
@@ -278,14 +288,18 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
             const int blk = t - AHEAD;
             if (blk >= 0 && blk < nblk) {
                 const uint8_t *stage = ring + (blk % STAGES) * STAGE;
-                const uint8_t *wcur = stage + j * Q4_K_BYTES;
+                const uint8_t *wcur = stage + j * WBYTES;
                 const uint8_t *a_blk = stage + A_OFF + ti * QK_K;
                 const float *ad_blk = (const float *)(stage + D_OFF);
                 const uint4 hdr = *(const uint4 *)wcur;
                 uint4 aq[8], wq4[4];
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    wq4[g] = *(const uint4 *)(wcur + 16 + 32 * g + 16 * kh);
+                    wq4[g] = *(const uint4 *)(wcur + QS_OFF + 32 * g + 16 * kh);
+                }
+                uint4 wqh = make_uint4(0, 0, 0, 0);  // fifth bits of this lane's 16 positions, one bit per sub-block
+                if constexpr (Q5) {
+                    wqh = *(const uint4 *)(wcur + 16 + 16 * kh);
                 }
 #pragma unroll
                 for (int sb = 0; sb < 8; ++sb) {
@@ -313,12 +327,22 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
                 };
                 auto weights_of = [&](int sb) {
                     const uint4 wq = wq4[sb >> 1];
+                    uint4 v;
                     if (sb & 1) {
-                        return intx4{(int)((wq.x >> 4) & 0x0f0f0f0fu), (int)((wq.y >> 4) & 0x0f0f0f0fu),
-                                     (int)((wq.z >> 4) & 0x0f0f0f0fu), (int)((wq.w >> 4) & 0x0f0f0f0fu)};
+                        v = make_uint4((wq.x >> 4) & 0x0f0f0f0fu, (wq.y >> 4) & 0x0f0f0f0fu, (wq.z >> 4) & 0x0f0f0f0fu,
+                                       (wq.w >> 4) & 0x0f0f0f0fu);
+                    } else {
+                        v = make_uint4(wq.x & 0x0f0f0f0fu, wq.y & 0x0f0f0f0fu, wq.z & 0x0f0f0f0fu, wq.w & 0x0f0f0f0fu);
                     }
-                    return intx4{(int)(wq.x & 0x0f0f0f0fu), (int)(wq.y & 0x0f0f0f0fu), (int)(wq.z & 0x0f0f0f0fu),
-                                 (int)(wq.w & 0x0f0f0f0fu)};
+                    if constexpr (Q5) {
+                        // bit sb of every byte to bit 4 (sb is a compile-time constant after unrolling)
+                        const int sh = 4 - sb;
+                        v.x |= (sh >= 0 ? wqh.x << (sh & 31) : wqh.x >> (-sh & 31)) & 0x10101010u;
+                        v.y |= (sh >= 0 ? wqh.y << (sh & 31) : wqh.y >> (-sh & 31)) & 0x10101010u;
+                        v.z |= (sh >= 0 ? wqh.z << (sh & 31) : wqh.z >> (-sh & 31)) & 0x10101010u;
+                        v.w |= (sh >= 0 ? wqh.w << (sh & 31) : wqh.w >> (-sh & 31)) & 0x10101010u;
+                    }
+                    return intx4{(int)v.x, (int)v.y, (int)v.z, (int)v.w};
                 };
                 const intx16 zero = {0};
                 intx16 dm = {0};
@@ -797,13 +821,18 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
     mmq_store<NR>(p, which, split, row0 + j, n0, ncols, tok, acc);
 }
 
+// Q4_K and Q5_K share one kernel and one launch plan
+static bool mmq_is_q4k_family(int kind) {
+    return kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q5_K;
+}
+
 bool mmq_supported(int kind, size_t N, size_t K) {
     if (getenv("MARMOT_HIP_NO_MMQ") != nullptr) {
         return false;
     }
     // below these row counts the fused-quantization matvec is faster (no separate quantization pass)
-    const size_t min_rows = kind == MARMOT_HIP_KIND_Q4_K ? 3 : 5;
-    return (kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && N >= min_rows && K % QK_K == 0;
+    const size_t min_rows = mmq_is_q4k_family(kind) ? 3 : 5;
+    return (mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && N >= min_rows && K % QK_K == 0;
 }
 
 constexpr size_t MMQ_ROWS_PER_PASS = MMQ_TOK;
@@ -837,14 +866,14 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t
         // reduction launch per weight follows (q/k/v 3 x 4096 x 4096, N=16: 41.3 us with the rule below, 33.6 with
         // two workgroups along K, 32.2 with this)
         W = nb < 2 ? nb : 2;
-    } else if (q6_loader || (kind == MARMOT_HIP_KIND_Q4_K && rg < cus)) {
+    } else if (q6_loader || (mmq_is_q4k_family(kind) && rg < cus)) {
         W = 1;
         const size_t want = ((q6_loader ? 7 : 8) * cus / 2 + rg - 1) / rg;  // workgroups along K
         while (S < want && S * 8 <= nb) {
             S *= 2;
         }
     } else {
-        const size_t w_max = (kind == MARMOT_HIP_KIND_Q4_K && N > 8) ? 2 : 4;
+        const size_t w_max = (mmq_is_q4k_family(kind) && N > 8) ? 2 : 4;
         W = nb < w_max ? nb : w_max;
         while (rg * S < cus && W * S * 2 <= nb) {
             S *= 2;
@@ -885,6 +914,10 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
                                    160 * 1024));
         MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
         MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)mmq6_lds_bytes(6)));
         attr_set = true;
@@ -917,14 +950,21 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
         if (pl.W < 1 || pl.W > 4) {
             return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "mmq: %d consumer wavefronts are not supported", pl.W);
         }
+        const bool q5 = kind == MARMOT_HIP_KIND_Q5_K;
         const int stages = p.items != nullptr ? 2 : 3;
-        const size_t stage = MMQ_WBLK + 2 * NR * QK_K + 2 * NR * 4;
+        const size_t stage = 32 * (size_t)(q5 ? Q5_K_BYTES : Q4_K_BYTES) + 2 * NR * QK_K + 2 * NR * 4;
         const size_t ring = (size_t)pl.W * stages * stage;
         const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
         const size_t lds_bytes = ring > red ? ring : red;
         const dim3 block((pl.W + 1) * 64);
         if (stages == 2) {
-            hipLaunchKernelGGL((k_mmq_q4k<NR, 2>), grid, block, lds_bytes, dev->stream, p);
+            if (q5) {
+                hipLaunchKernelGGL((k_mmq_q4k<NR, 2, true>), grid, block, lds_bytes, dev->stream, p);
+            } else {
+                hipLaunchKernelGGL((k_mmq_q4k<NR, 2>), grid, block, lds_bytes, dev->stream, p);
+            }
+        } else if (q5) {
+            hipLaunchKernelGGL((k_mmq_q4k<NR, 3, true>), grid, block, lds_bytes, dev->stream, p);
         } else {
             hipLaunchKernelGGL((k_mmq_q4k<NR, 3>), grid, block, lds_bytes, dev->stream, p);
         }
@@ -1009,14 +1049,16 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
             }
         }
     }
-    set_route(kind == MARMOT_HIP_KIND_Q6_K ? "mmq_q6_k_q8_k_mfma" : "mmq_q4_k_q8_k_mfma");
+    set_route(kind == MARMOT_HIP_KIND_Q6_K       ? "mmq_q6_k_q8_k_mfma"
+              : kind == MARMOT_HIP_KIND_Q5_K     ? "mmq_q5_k_q8_k_mfma"
+                                                 : "mmq_q4_k_q8_k_mfma");
     return MARMOT_HIP_SUCCESS;
 }
 
 // Grouped (MoE): every work item is up to 8 consecutive routes of one expert; blockIdx.z walks the item list the
 // route kernel wrote (workgroups beyond *d_n_items exit at once).
 bool mmq_grouped_supported(int kind, size_t K) {
-    return (kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && K % QK_K == 0 &&
+    return (mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && K % QK_K == 0 &&
            getenv("MARMOT_HIP_NO_MMQ") == nullptr;
 }
 
@@ -1070,7 +1112,9 @@ int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
-    set_route(kind == MARMOT_HIP_KIND_Q6_K ? "moe_grouped_q6_k_q8_k_mfma" : "moe_grouped_q4_k_q8_k_mfma");
+    set_route(kind == MARMOT_HIP_KIND_Q6_K       ? "moe_grouped_q6_k_q8_k_mfma"
+              : kind == MARMOT_HIP_KIND_Q5_K     ? "moe_grouped_q5_k_q8_k_mfma"
+                                                 : "moe_grouped_q4_k_q8_k_mfma");
     return MARMOT_HIP_SUCCESS;
 }
 

@@ -363,6 +363,9 @@ int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_bloc
     case MARMOT_HIP_KIND_Q4_K:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
+    case MARMOT_HIP_KIND_Q5_K:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q5_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
     case MARMOT_HIP_KIND_Q6_K:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q6_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
@@ -407,8 +410,7 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
     if (d_table == nullptr || d_ids == nullptr || d_out == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Tensor argument must not be null");
     }
-    if (kind != MARMOT_HIP_KIND_Q4_0 && kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_K &&
-        kind != MARMOT_HIP_KIND_Q6_K) {
+    if (!is_weight_kind(kind)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "embedding gather: unsupported quant kind %d", kind);
     }
     if (ids_dtype != MARMOT_HIP_DTYPE_I32 && ids_dtype != MARMOT_HIP_DTYPE_I64) {
@@ -442,6 +444,10 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
         hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q4_K>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q5_K:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q5_K>), grid, block, 0, dev->stream, table, vocab, dim,
                            d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
         break;
     case MARMOT_HIP_KIND_Q6_K:

@@ -84,6 +84,8 @@ def test_ctypes_structs_match_layout(golden_layout):
         golden_layout["MARMOT_PREFERENCE_ENABLE"], golden_layout["MARMOT_PREFERENCE_DISABLE"])
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q4_K] == golden_layout["MARMOT_QSCHEME_Q4_K"]
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q6_K] == golden_layout["MARMOT_QSCHEME_Q6_K"]
+    assert ta.QSCHEME_OF_KIND[ta.KIND_Q5_K] == golden_layout["MARMOT_QSCHEME_Q5_K"]
+    assert ta.KIND_Q5_K == golden_layout["MARMOT_QUANT_KIND_Q5_K"]
     assert ta.KIND_Q8_K == golden_layout["MARMOT_QUANT_KIND_Q8_K"]
     assert ta.NOT_IMPLEMENTED == golden_layout["MARMOT_ERROR_NOT_IMPLEMENTED"]
     assert ta.BACKEND_HIP == golden_layout["MARMOT_BACKEND_CUDA"] + 1
@@ -132,7 +134,7 @@ def _query(lib, sig):
 
 
 def test_query_kernel_matmul_rules(lib):
-    expect_op = {ta.KIND_Q4_0: 1, ta.KIND_Q8_0: 2, ta.KIND_Q4_K: 3, ta.KIND_Q6_K: 4}
+    expect_op = {ta.KIND_Q4_0: 1, ta.KIND_Q8_0: 2, ta.KIND_Q4_K: 3, ta.KIND_Q6_K: 4, ta.KIND_Q5_K: 20}
     for kind, op in expect_op.items():
         sel = _query(lib, _sig(kind=kind))
         assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
@@ -151,9 +153,11 @@ def test_query_kernel_matmul_rules(lib):
     # Q6_K with fp16 activations is declined (caller falls back)
     sel = _query(lib, _sig(kind=ta.KIND_Q6_K, inp=ta.DTYPE_F16))
     assert not sel.supported and sel.op_index == 0xFFFF and b"Q6_K" in sel.fallback_reason
+    sel = _query(lib, _sig(kind=ta.KIND_Q5_K, inp=ta.DTYPE_F16))
+    assert not sel.supported and b"Q5_K" in sel.fallback_reason
     # unsupported scheme, layout, weight layout, stride mode, epilogue, variant
     assert not _query(lib, _sig(kind=ta.KIND_Q8_K)).supported
-    s = _sig(); s.qscheme_id = 9  # Q5_K
+    s = _sig(); s.qscheme_id = 7  # Q3_K
     assert not _query(lib, s).supported
     s = _sig(); s.matmul_layout = 1
     assert not _query(lib, s).supported
@@ -187,7 +191,7 @@ def test_query_kernel_cost_model(lib):
 
 
 def test_query_kernel_other_ops(lib):
-    for kind, op in {ta.KIND_Q4_0: 5, ta.KIND_Q8_0: 6, ta.KIND_Q4_K: 7, ta.KIND_Q6_K: 8}.items():
+    for kind, op in {ta.KIND_Q4_0: 5, ta.KIND_Q8_0: 6, ta.KIND_Q4_K: 7, ta.KIND_Q6_K: 8, ta.KIND_Q5_K: 21}.items():
         assert _query(lib, _sig(op=ta.OP_MOE_EXPERTS, kind=kind)).op_index == op
     assert not _query(lib, _sig(op=ta.OP_MOE_EXPERTS, inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).supported
     assert _query(lib, _sig(op=ta.OP_TOPK)).op_index == 9
@@ -204,7 +208,8 @@ def test_query_kernel_qkv_rules(lib, golden_layout):
         golden_layout[k] for k in ("MARMOT_OP_QKV_PROJECTION", "MARMOT_OP_QKV_SHARED_INPUT", "MARMOT_OP_QKV_ROPE"))
     assert ta.EPILOGUE_ROPE == golden_layout["MARMOT_EPILOGUE_ROPE"]
     for op_id in (ta.OP_QKV_PROJECTION, ta.OP_QKV_SHARED_INPUT, ta.OP_QKV_ROPE):
-        for kind, op in {ta.KIND_Q4_0: 12, ta.KIND_Q8_0: 13, ta.KIND_Q4_K: 14, ta.KIND_Q6_K: 15}.items():
+        for kind, op in {ta.KIND_Q4_0: 12, ta.KIND_Q8_0: 13, ta.KIND_Q4_K: 14, ta.KIND_Q6_K: 15,
+                         ta.KIND_Q5_K: 22}.items():
             for dt in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, _sig(op=op_id, kind=kind, inp=dt, out=dt, N=4, K=4096, M=4096))
                 assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
@@ -246,7 +251,8 @@ def test_query_kernel_embedding_rules(lib):
         s.qscheme_id = ta.QSCHEME_OF_KIND.get(kind, 0)
         s.weight_layout = ta.WEIGHT_LAYOUT_SEPARATE
         return s
-    for kind, op in ((ta.KIND_Q4_0, 16), (ta.KIND_Q8_0, 17), (ta.KIND_Q4_K, 18), (ta.KIND_Q6_K, 19)):
+    for kind, op in ((ta.KIND_Q4_0, 16), (ta.KIND_Q8_0, 17), (ta.KIND_Q4_K, 18), (ta.KIND_Q6_K, 19),
+                     (ta.KIND_Q5_K, 23)):
         for ids in (ta.DTYPE_I32, ta.DTYPE_I64):
             for out in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, sig(kind, ids, out))
@@ -261,7 +267,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 20
+    assert t.op_count == 24
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -280,6 +286,9 @@ def test_bytecode_tables(lib, golden_layout):
     assert sizes[11] == struct.calcsize("<HHII")
     assert sizes[12:16] == [struct.calcsize("<7HII3H")] * 4
     assert sizes[16:20] == [struct.calcsize("<3HIfI3B")] * 4 == [21] * 4
+    # Q5_K was added behind the four original kinds: one op per family
+    assert schema[20:24] == [golden_layout[f"MARMOT_BC_SCHEMA_{n}"] for n in ("MATMUL", "MOE_EXPERTS", "QKV", "EMBEDDING")]
+    assert sizes[20:24] == [sizes[1], sizes[5], sizes[12], sizes[16]]
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -342,7 +351,7 @@ def test_kernel_def_files_name_exported_impls(lib):
             fields = dict(re.findall(r"^\s*([A-Z_]+(?:\(\w+\))?):\s*(.+?),?\s*$", body, re.M))
             families[name] = fields
     qkv = {f"{op}_quantized_hip_{dt}" for op in ("qkv_shared_input", "qkv_projection") for dt in ("f16", "f32")}
-    assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_q6_k", "topk_hip",
+    assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_f32", "topk_hip",
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
                              "embedding_quantized_hip"} | qkv
     for name in qkv:
@@ -358,4 +367,5 @@ def test_kernel_def_files_name_exported_impls(lib):
     mm = families["matmul_quantized_hip"]
     assert mm["OP"] == "matmul" and mm["MATMUL_LAYOUT"] == "NT" and mm["WEIGHT_LAYOUT"] == "SEPARATE"
     assert mm["EPILOGUE"] == "[BIAS]" and mm["ACCUM_DTYPE"] == "FLOAT32" and mm["STRIDE_MODE"] == "CONTIGUOUS"
-    assert families["matmul_quantized_hip_q6_k"]["INPUT_DTYPE"] == "FLOAT32"
+    assert families["matmul_quantized_hip_f32"]["INPUT_DTYPE"] == "FLOAT32"
+    assert families["matmul_quantized_hip_f32"]["AXIS(scheme)"] == "[Q5_K, Q6_K]"

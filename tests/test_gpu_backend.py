@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from marmot_amd import tensor_abi as ta
-from oracle.pyoracle import KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K, row_bytes
+from oracle.pyoracle import KIND_Q4_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K, row_bytes
 from tests.test_oracle_moe import make_experts
 from tests.util import assert_matmul_parity, assert_moe_parity, bits, gaussian, quantize_weights
 
@@ -30,7 +30,8 @@ def _linear(ctx, kind, wq, M, K, x, bias=None, out_dtype=ta.DTYPE_F32):
         ep = ta.Epilogue()
         ep.bias = bt.ptr
     fn = getattr(ctx.lib, {KIND_Q4_0: "hip_matmul_quantized_q4_0", KIND_Q8_0: "hip_matmul_quantized_q8_0",
-                           KIND_Q4_K: "hip_matmul_quantized_q4_k", KIND_Q6_K: "hip_matmul_quantized_q6_k"}[kind])
+                           KIND_Q4_K: "hip_matmul_quantized_q4_k", KIND_Q5_K: "hip_matmul_quantized_q5_k",
+                           KIND_Q6_K: "hip_matmul_quantized_q6_k"}[kind])
     st = fn(ctx.device_ctx, xt.ptr, wt.ptr, C.byref(ep) if ep is not None else None, yt.ptr)
     if st == ta.SUCCESS:
         ctx.to_host(yt)
@@ -41,7 +42,7 @@ def _linear(ctx, kind, wq, M, K, x, bias=None, out_dtype=ta.DTYPE_F32):
     return st, xt, wt, yt
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K])
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
 def test_impl_matmul_matches_oracle(ctx, oracle, kind):
     print(f"backend impl matmul kind={kind}", flush=True)
     M, K, N = 96, 512, 5
@@ -277,7 +278,7 @@ def _qkv_tensors(kind, ws, M, K, x, biases):
     return xt, wts, outs, bts
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K])
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_impl_qkv_matches_oracle(ctx, oracle, kind, dtype):
     """hip_matmul_qkv_{scheme} with a marmot_matmul_qkv_desc_t (separate layout) and through a bytecode program."""
@@ -294,7 +295,7 @@ def test_impl_qkv_matches_oracle(ctx, oracle, kind, dtype):
     desc.separate.wq, desc.separate.wk, desc.separate.wv = (w.ptr for w in wts)
     desc.separate.bq, desc.separate.bv = bts[0].ptr, bts[2].ptr
     desc.out_q, desc.out_k, desc.out_v = (o.ptr for o in outs)
-    name = {KIND_Q4_0: "q4_0", KIND_Q8_0: "q8_0", KIND_Q4_K: "q4_k", KIND_Q6_K: "q6_k"}[kind]
+    name = {KIND_Q4_0: "q4_0", KIND_Q8_0: "q8_0", KIND_Q4_K: "q4_k", KIND_Q5_K: "q5_k", KIND_Q6_K: "q6_k"}[kind]
     st = getattr(ctx.lib, f"hip_matmul_qkv_{name}")(ctx.device_ctx, C.byref(desc))
     assert st == ta.SUCCESS, ctx.last_error()
     tol = 1e-3 if dtype == np.float32 else 2e-3
@@ -305,7 +306,7 @@ def test_impl_qkv_matches_oracle(ctx, oracle, kind, dtype):
     first = [o.array.copy() for o in outs]
     # the same call as one bytecode instruction, kernel chosen by the query
     sel = ctx.query(ctx.qkv_signature(xt, wts[0], outs[0], bias=True))
-    assert sel.supported and sel.op_index == 12 + [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K].index(kind)
+    assert sel.supported and sel.op_index == {KIND_Q4_0: 12, KIND_Q8_0: 13, KIND_Q4_K: 14, KIND_Q6_K: 15, KIND_Q5_K: 22}[kind]
     for o in outs:
         o.array[...] = 0
         ctx.host_changed(o)
@@ -428,7 +429,7 @@ def test_program_qkv_with_rotary_epilogue(ctx, oracle, dtype):
 
 
 # ---------------------------------------------------------------- embedding gather
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q6_K])
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
 def test_impl_and_program_embedding_gather(ctx, oracle, kind):
     """marmot_embedding_gather on a quantized table: the impl function with a descriptor and the EMBEDDING bytecode
     schema, ids of rank 2 (flattened), float32 bit-exact and float16 with scale; the table stays resident."""
@@ -454,7 +455,7 @@ def test_impl_and_program_embedding_gather(ctx, oracle, kind):
     o16 = ta.HostTensor.empty((15, dim), ta.DTYPE_F16)
     i32 = ta.HostTensor.dense(ids.astype(np.int32).reshape(-1))
     sel = ctx.query(ctx.embedding_signature(tt, i32, o16))
-    assert sel.supported and sel.op_index == {KIND_Q4_0: 16, KIND_Q8_0: 17, KIND_Q4_K: 18, KIND_Q6_K: 19}[kind]
+    assert sel.supported and sel.op_index == {KIND_Q4_0: 16, KIND_Q8_0: 17, KIND_Q4_K: 18, KIND_Q6_K: 19, KIND_Q5_K: 23}[kind]
     before = ctx.residency().upload_bytes
     prog = ta.Program()
     prog.embedding(sel.op_index, tt, i32, o16, scale=0.25, padding_id=-1, bounds_check=False)

@@ -2,12 +2,12 @@
 import numpy as np
 import pytest
 
-from oracle.pyoracle import BLOCK_VALUES, KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import BLOCK_VALUES, KIND_Q4_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.util import assert_matmul_parity, bits, gaussian, parity_metrics, quantize_weights, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
-KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q6_k": KIND_Q6_K}
+KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K}
 THREADS = 16
 
 
@@ -20,7 +20,7 @@ def hip():
     b.close()
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_reference_matmul_goldens_fp32(hip, ref_goldens, name):
     """The reference's own golden cases (tests/backend/golden_matmul_llama.h), its own tolerance."""
     kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
@@ -91,7 +91,7 @@ def test_config2_kquant_decode_full_size(hip, oracle, name, M, K):
     d_w.free()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("N", [1, 2, 3, 5, 8, 11, 16, 19])
 def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
     """All column-tile widths (8/4/2/1) and M not a multiple of the rows-per-workgroup."""
@@ -104,7 +104,7 @@ def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
     assert_matmul_parity(got, ref, what=f"{name} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("K", [256, 512, 768, 1280, 8192, 11008, 28672])
 def test_linear_k_sweep(hip, oracle, name, K):
     """Rows shorter than one wave-load, rows needing several wavefronts, and long rows."""
@@ -118,7 +118,7 @@ def test_linear_k_sweep(hip, oracle, name, K):
         assert_matmul_parity(got, ref, what=f"{name} K={K} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k"])
 def test_linear_ragged_k(hip, oracle, name):
     """K not a multiple of the block: weight and activation tails are zero-padded blocks."""
     kind = KINDS[name]
@@ -132,7 +132,7 @@ def test_linear_ragged_k(hip, oracle, name):
     assert_matmul_parity(got, ref, what=f"{name} ragged K={K}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k"])
 def test_linear_random_block_bytes(hip, oracle, name):
     """Weights that are arbitrary block bytes (all 6-bit scale / min patterns, negative Q6_K scales)."""
     kind = KINDS[name]
@@ -145,7 +145,7 @@ def test_linear_random_block_bytes(hip, oracle, name):
     assert_matmul_parity(got, ref, what=f"{name} random bytes")
 
 
-@pytest.mark.parametrize("name", ["q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q8_0", "q4_k", "q5_k", "q6_k"])
 def test_linear_bias_epilogue(hip, oracle, name):
     kind = KINDS[name]
     M, K, N = 50, 1024, 3
@@ -211,7 +211,7 @@ def test_linear_error_behaviour(hip, oracle):
     hip.synchronize()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k"])
 def test_loader_consumer_matvec_equals_register_streaming_matvec(hip, oracle, name, monkeypatch):
     """The loader/consumer matvec (weights through an LDS ring) keeps the lane mapping and the reduction order of the
     register-streaming kernel: the two must agree bit for bit, on whole and ragged row groups, one and two K slices

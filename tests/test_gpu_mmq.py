@@ -6,12 +6,12 @@ import numpy as np
 import pytest
 
 from marmot_amd import capi
-from oracle.pyoracle import KIND_Q4_K, KIND_Q6_K
+from oracle.pyoracle import KIND_Q4_K, KIND_Q5_K, KIND_Q6_K
 from tests.util import assert_matmul_parity, bits, gaussian, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
-KINDS = {"q4_k": KIND_Q4_K, "q6_k": KIND_Q6_K}
+KINDS = {"q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K}
 MIN_ROWS = {"q4_k": 3, "q6_k": 5}
 
 

@@ -35,6 +35,9 @@ extern "C" {
 /* quant kinds: numeric values of marmot_quant_kind_t (include/marmot/types.h:372-388) */
 enum {
     MO_KIND_Q4_0 = 1,
+    MO_KIND_Q4_1 = 2,
+    MO_KIND_Q5_0 = 3,
+    MO_KIND_Q5_1 = 4,
     MO_KIND_Q8_0 = 5,
     MO_KIND_Q4_K = 9,
     MO_KIND_Q5_K = 10,
@@ -82,6 +85,9 @@ void mo_pack_q8_k(const void *x, int in_dtype, size_t k, void *blocks_out);
 /* integer block dots (vec_dot_impl.h) over `nblocks` consecutive blocks */
 float mo_vec_dot_q8_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_0_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q4_1_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q5_0_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q5_1_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q5_k_q8_k(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q6_k_q8_k(const void *w, const void *a, size_t nblocks);

@@ -38,6 +38,12 @@ int main(void) {
     EMIT(g_llama_test_input, "f4");
     EMIT(g_llama_q4_0, "u1");
     EMIT(g_llama_q4_0_dequant, "f4");
+    EMIT(g_llama_q4_1, "u1");
+    EMIT(g_llama_q4_1_dequant, "f4");
+    EMIT(g_llama_q5_0, "u1");
+    EMIT(g_llama_q5_0_dequant, "f4");
+    EMIT(g_llama_q5_1, "u1");
+    EMIT(g_llama_q5_1_dequant, "f4");
     EMIT(g_llama_q8_0, "u1");
     EMIT(g_llama_q8_0_dequant, "f4");
     EMIT(g_llama_q4_k, "u1");
@@ -56,11 +62,17 @@ int main(void) {
     EMIT(g_vec_dot_q8_k_activations, "u1");
     EMIT(g_vec_dot_q4_0_weights, "u1");
     EMIT(g_vec_dot_q8_0_weights, "u1");
+    EMIT(g_vec_dot_q4_1_weights, "u1");
+    EMIT(g_vec_dot_q5_0_weights, "u1");
+    EMIT(g_vec_dot_q5_1_weights, "u1");
     EMIT(g_vec_dot_q4_k_weights, "u1");
     EMIT(g_vec_dot_q5_k_weights, "u1");
     EMIT(g_vec_dot_q6_k_weights, "u1");
     EMIT_SCALAR(g_vec_dot_q4_0_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q8_0_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q4_1_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q5_0_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q5_1_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q4_k_q8_k_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q5_k_q8_k_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q6_k_q8_k_expected, "f4");
@@ -71,7 +83,8 @@ int main(void) {
         const matmul_golden_case_t *c = &g_matmul_quant_goldens[i];
         if (c->kind != MARMOT_QUANT_KIND_Q4_0 && c->kind != MARMOT_QUANT_KIND_Q8_0 &&
             c->kind != MARMOT_QUANT_KIND_Q4_K && c->kind != MARMOT_QUANT_KIND_Q5_K &&
-            c->kind != MARMOT_QUANT_KIND_Q6_K) {
+            c->kind != MARMOT_QUANT_KIND_Q6_K && c->kind != MARMOT_QUANT_KIND_Q4_1 &&
+            c->kind != MARMOT_QUANT_KIND_Q5_0 && c->kind != MARMOT_QUANT_KIND_Q5_1) {
             continue;
         }
         char name[128];

@@ -2,14 +2,18 @@
 (src/backends/cpu/ops/embedding/scalar/embedding_scalar.c:241-303, 381-447), pinned by the reference's own golden for
 the Q4_0 table (tests/golden/embedding_q4_0_ragged.txt, transcribed to tests/golden/reference_embedding_q4_0.json: the
 interleaved nibble order of the embedding path, which differs from the Q4_0 dequantizer's) and, for the other kinds, by
-the block dequantizers the quantization goldens pin (a gathered row is the dequantized row, bit for bit)."""
+the block dequantizers the quantization goldens pin (a gathered row is the dequantized row, bit for bit). The
+reference also ships embedding_q5_0.txt / embedding_q5_1.txt, but its own test skips them unconditionally
+(tests/backend/test_backend_embedding_golden.c:283-287, 298-302) and its Q5 dequantizers do not reproduce them: they pin
+nothing and are not used here."""
 import json
 import os
 
 import numpy as np
 import pytest
 
-from oracle.pyoracle import KIND_Q4_0, KIND_Q4_K, KIND_Q6_K, KIND_Q8_0, row_bytes
+from oracle.pyoracle import (KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
+                             row_bytes)
 from tests.util import bits, gaussian, random_valid_blocks
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_embedding_q4_0.json")
@@ -33,10 +37,17 @@ def test_reference_q4_0_embedding_golden(oracle):
     assert np.max(np.abs(plain - expected)) > 1.0
 
 
-@pytest.mark.parametrize("kind", [KIND_Q8_0, KIND_Q4_K, KIND_Q6_K])
+def test_q4_1_tables_are_declined(oracle):
+    """The reference decodes Q4_1 tables in the interleaved order too but holds no golden for it: not restated."""
+    table = random_valid_blocks(np.random.default_rng(5), KIND_Q4_1, 4, 64)
+    with pytest.raises(RuntimeError):
+        oracle.embedding_gather(KIND_Q4_1, table, 4, 64, np.array([1], np.int32))
+
+
+@pytest.mark.parametrize("kind", [KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q5_0, KIND_Q5_1])
 def test_gathered_rows_are_dequantized_rows(oracle, kind):
     rng = np.random.default_rng(800 + kind)
-    vocab, dim = 37, 768 if kind != KIND_Q8_0 else 96
+    vocab, dim = 37, 768 if kind in (KIND_Q4_K, KIND_Q5_K, KIND_Q6_K) else 96
     table = random_valid_blocks(rng, kind, vocab, dim)
     dense = oracle.dequantize(kind, table, dim)
     ids = rng.integers(0, vocab, (3, 5)).astype(np.int64)

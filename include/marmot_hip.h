@@ -43,6 +43,9 @@ enum {
 /* marmot_quant_kind_t values (include/marmot/types.h:372-388) */
 enum {
     MARMOT_HIP_KIND_Q4_0 = 1,
+    MARMOT_HIP_KIND_Q4_1 = 2,
+    MARMOT_HIP_KIND_Q5_0 = 3,
+    MARMOT_HIP_KIND_Q5_1 = 4,
     MARMOT_HIP_KIND_Q8_0 = 5,
     MARMOT_HIP_KIND_Q4_K = 9,
     MARMOT_HIP_KIND_Q5_K = 10,

@@ -245,7 +245,8 @@ static size_t dtype_size(marmot_dtype_t t) {
 }
 
 static bool kind_supported_weight(marmot_quant_kind_t k) {
-    return k == MARMOT_QUANT_KIND_Q4_0 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q4_K ||
+    return k == MARMOT_QUANT_KIND_Q4_0 || k == MARMOT_QUANT_KIND_Q4_1 || k == MARMOT_QUANT_KIND_Q5_0 ||
+        k == MARMOT_QUANT_KIND_Q5_1 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q4_K ||
         k == MARMOT_QUANT_KIND_Q5_K || k == MARMOT_QUANT_KIND_Q6_K;
 }
 
@@ -893,7 +894,7 @@ static marmot_error_t embedding_gather(const void *device_ctx, const marmot_embe
     if (!kind_is_block(weights->quant_kind) || weights->quant_layout != MARMOT_QUANT_LAYOUT_GGUF) {
         return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Unsupported quantized embedding layout");
     }
-    if (!kind_supported_weight(weights->quant_kind)) {
+    if (!kind_supported_weight(weights->quant_kind) || weights->quant_kind == MARMOT_QUANT_KIND_Q4_1) {
         return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized embedding kind not supported on HIP");
     }
     const size_t vocab = weights->shape.shape[0], dim = weights->shape.shape[1];
@@ -1010,7 +1011,7 @@ static marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_exper
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "HIP MoE experts need FLOAT32 activations and INT32 expert ids");
     }
     if (!kind_supported_weight(g->quant_kind) || !kind_supported_weight(d->quant_kind)) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q8_0, Q4_K, Q5_K or Q6_K expert weights");
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K or Q6_K expert weights");
     }
     if (h->shape.ndim != 2 || g->shape.ndim != 3 || u->shape.ndim != 3 || d->shape.ndim != 3 ||
         desc->topk_ids->shape.ndim != 2 || desc->topk_weights->shape.ndim != 2 || desc->out->shape.ndim != 2) {
@@ -1168,7 +1169,7 @@ static marmot_error_t dequantize_block(const void *device_ctx, const marmot_tens
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize: null argument");
     }
     if (!kind_supported_weight(input->quant_kind) && input->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q8_0, Q4_K, Q5_K, Q6_K and Q8_K");
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K and Q8_K");
     }
     if (output->dtype != MARMOT_DTYPE_FLOAT32) {
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Dequantize output must be FLOAT32");
@@ -1258,6 +1259,9 @@ HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q8_0, MARMOT_QUANT_KIND_Q8_0)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q4_k, MARMOT_QUANT_KIND_Q4_K)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q6_k, MARMOT_QUANT_KIND_Q6_K)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_k, MARMOT_QUANT_KIND_Q5_K)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q4_1, MARMOT_QUANT_KIND_Q4_1)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_0, MARMOT_QUANT_KIND_Q5_0)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_1, MARMOT_QUANT_KIND_Q5_1)
 
 // QKV immediates (bytecode_compile.c:670-715): the tensors come from the registers, the epilogue and the rotary
 // parameters from the constant pool.
@@ -1316,6 +1320,9 @@ HIP_BC_QKV_ENTRY(bc_exec_qkv_q8_0, MARMOT_QUANT_KIND_Q8_0)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q4_k, MARMOT_QUANT_KIND_Q4_K)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q6_k, MARMOT_QUANT_KIND_Q6_K)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_k, MARMOT_QUANT_KIND_Q5_K)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q4_1, MARMOT_QUANT_KIND_Q4_1)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_0, MARMOT_QUANT_KIND_Q5_0)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_1, MARMOT_QUANT_KIND_Q5_1)
 
 // EMBEDDING immediates (bytecode_compile.c:989-1018) -> the descriptor the generated shim builds
 // (src/backends/cpu/dispatch/misc_dispatch_cpu.gen.c:115-133)
@@ -1427,6 +1434,9 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     28, 28, 28, 28,  // QKV: 7 x u16 + 2 x u32 + 3 x u16
     21, 21, 21, 21,  // EMBEDDING: 3 x u16 + u32 + f32 + u32 + 3 x u8
     12, 26, 28, 21,  // Q5_K: MATMUL, MOE_EXPERTS, QKV, EMBEDDING
+    12, 26, 28, 21,  // Q4_1
+    12, 26, 28, 21,  // Q5_0
+    12, 26, 28, 21,  // Q5_1
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1439,6 +1449,9 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS,
     MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1449,6 +1462,9 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_qkv_q4_0,    bc_exec_qkv_q8_0,    bc_exec_qkv_q4_k,    bc_exec_qkv_q6_k,
     bc_exec_embedding,   bc_exec_embedding,   bc_exec_embedding,   bc_exec_embedding,
     bc_exec_matmul_q5_k, bc_exec_moe,         bc_exec_qkv_q5_k,    bc_exec_embedding,
+    bc_exec_matmul_q4_1, bc_exec_moe,         bc_exec_qkv_q4_1,    bc_exec_embedding,
+    bc_exec_matmul_q5_0, bc_exec_moe,         bc_exec_qkv_q5_0,    bc_exec_embedding,
+    bc_exec_matmul_q5_1, bc_exec_moe,         bc_exec_qkv_q5_1,    bc_exec_embedding,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -1480,6 +1496,12 @@ static int kind_of_scheme(marmot_qscheme_id_t q) {
     switch (q) {
     case MARMOT_QSCHEME_Q4_0:
         return MARMOT_HIP_KIND_Q4_0;
+    case MARMOT_QSCHEME_Q4_1:
+        return MARMOT_HIP_KIND_Q4_1;
+    case MARMOT_QSCHEME_Q5_0:
+        return MARMOT_HIP_KIND_Q5_0;
+    case MARMOT_QSCHEME_Q5_1:
+        return MARMOT_HIP_KIND_Q5_1;
     case MARMOT_QSCHEME_Q8_0:
         return MARMOT_HIP_KIND_Q8_0;
     case MARMOT_QSCHEME_Q4_K:
@@ -1507,16 +1529,25 @@ static uint16_t matmul_op_of_kind(int kind) {
         return MARMOT_HIP_BC_OP_MATMUL_Q6_K;
     case MARMOT_HIP_KIND_Q5_K:
         return MARMOT_HIP_BC_OP_MATMUL_Q5_K;
+    case MARMOT_HIP_KIND_Q4_1:
+        return MARMOT_HIP_BC_OP_MATMUL_Q4_1;
+    case MARMOT_HIP_KIND_Q5_0:
+        return MARMOT_HIP_BC_OP_MATMUL_Q5_0;
+    case MARMOT_HIP_KIND_Q5_1:
+        return MARMOT_HIP_BC_OP_MATMUL_Q5_1;
     default:
         return MARMOT_KERNEL_OP_INDEX_INVALID;
     }
 }
 
 // The operation of a family (its Q4_0 op and its Q5_K op given) for the kind whose matmul op is mm: the first four
-// kinds are numbered alike in every family, Q5_K was added behind them.
+// kinds are numbered alike in every family; the kinds added behind them take four consecutive ops each, in the
+// order MATMUL, MOE_EXPERTS, QKV, EMBEDDING.
 static uint16_t family_op(uint16_t mm, uint16_t family_q4_0, uint16_t family_q5_k) {
-    return mm == MARMOT_HIP_BC_OP_MATMUL_Q5_K ? family_q5_k
-                                              : (uint16_t)(family_q4_0 + (mm - MARMOT_HIP_BC_OP_MATMUL_Q4_0));
+    if (mm >= MARMOT_HIP_BC_OP_MATMUL_Q5_K) {
+        return (uint16_t)(mm + (family_q5_k - MARMOT_HIP_BC_OP_MATMUL_Q5_K));
+    }
+    return (uint16_t)(family_q4_0 + (mm - MARMOT_HIP_BC_OP_MATMUL_Q4_0));
 }
 
 // ------------------------------------------------------------------ exports
@@ -1539,7 +1570,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t op = matmul_op_of_kind(kind);
         if (op == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP matmul handles Q4_0, Q8_0, Q4_K, Q5_K and Q6_K weights");
+            return unsupported("HIP matmul handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K weights");
         }
         if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
             return unsupported("HIP quantized matmul needs layout NT");
@@ -1581,7 +1612,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP QKV projection handles Q4_0, Q8_0, Q4_K, Q5_K and Q6_K weights");
+            return unsupported("HIP QKV projection handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K weights");
         }
         if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
             return unsupported("HIP QKV projection needs layout NT");
@@ -1616,7 +1647,10 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP embedding gather handles Q4_0, Q8_0, Q4_K, Q5_K and Q6_K tables");
+            return unsupported("HIP embedding gather handles Q4_0, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K tables");
+        }
+        if (kind == MARMOT_HIP_KIND_Q4_1) {
+            return unsupported("HIP embedding gather does not offer Q4_1 tables");
         }
         if (sig->input_dtype != MARMOT_DTYPE_INT32 && sig->input_dtype != MARMOT_DTYPE_INT64) {
             return unsupported("HIP embedding gather takes INT32 or INT64 token ids");
@@ -1629,7 +1663,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
     case MARMOT_OP_MOE_EXPERTS: {
         const int kind = kind_of_scheme(sig->qscheme_id);
         if (matmul_op_of_kind(kind) == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP MoE experts handle Q4_0, Q8_0, Q4_K, Q5_K and Q6_K expert weights");
+            return unsupported("HIP MoE experts handle Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K expert weights");
         }
         if (!in32 || !out32) {
             return unsupported("HIP MoE experts take FLOAT32 activations");
@@ -1651,7 +1685,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         return selected(MARMOT_HIP_BC_OP_QUANTIZE_BLOCK, launch_us, 0.0);
     case MARMOT_OP_DEQUANTIZE:
         if (kind_of_scheme(sig->qscheme_id) == 0 || !out32) {
-            return unsupported("HIP dequantize handles Q4_0, Q8_0, Q4_K, Q5_K, Q6_K and Q8_K to FLOAT32");
+            return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K and Q8_K to FLOAT32");
         }
         return selected(MARMOT_HIP_BC_OP_DEQUANTIZE_BLOCK, launch_us, 0.0);
     default:
@@ -1741,6 +1775,21 @@ marmot_error_t hip_matmul_quantized_q4_k(const void *device_ctx, const marmot_te
                                          marmot_tensor_t *out) {
     return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q4_K, input, weight, epilogue, out);
 }
+marmot_error_t hip_matmul_quantized_q4_1(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q4_1, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_quantized_q5_0(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q5_0, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_quantized_q5_1(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q5_1, input, weight, epilogue, out);
+}
 marmot_error_t hip_matmul_quantized_q5_k(const void *device_ctx, const marmot_tensor_t *input,
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out) {
@@ -1759,6 +1808,15 @@ marmot_error_t hip_matmul_qkv_q8_0(const void *device_ctx, const marmot_matmul_q
 }
 marmot_error_t hip_matmul_qkv_q4_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q4_K, desc);
+}
+marmot_error_t hip_matmul_qkv_q4_1(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q4_1, desc);
+}
+marmot_error_t hip_matmul_qkv_q5_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q5_0, desc);
+}
+marmot_error_t hip_matmul_qkv_q5_1(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q5_1, desc);
 }
 marmot_error_t hip_matmul_qkv_q5_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q5_K, desc);

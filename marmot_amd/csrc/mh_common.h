@@ -19,6 +19,9 @@ namespace mh {
 constexpr int QK = 32;
 constexpr int QK_K = 256;
 constexpr int Q4_0_BYTES = 18;
+constexpr int Q4_1_BYTES = 20;
+constexpr int Q5_0_BYTES = 22;
+constexpr int Q5_1_BYTES = 24;
 constexpr int Q8_0_BYTES = 34;
 constexpr int Q4_K_BYTES = 144;
 constexpr int Q5_K_BYTES = 176;
@@ -27,6 +30,22 @@ constexpr int Q8_K_BYTES = 292;
 
 struct __attribute__((packed)) BlockQ4_0 {
     uint16_t scale;
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ4_1 {
+    uint16_t scale;
+    uint16_t min;
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ5_0 {
+    uint16_t scale;
+    uint8_t qh[4];  // bit j: fifth bit of value j (32 bits, little endian)
+    uint8_t qs[16];
+};
+struct __attribute__((packed)) BlockQ5_1 {
+    uint16_t scale;
+    uint16_t min;
+    uint8_t qh[4];
     uint8_t qs[16];
 };
 struct __attribute__((packed)) BlockQ8_0 {
@@ -59,6 +78,9 @@ struct __attribute__((packed)) BlockQ8_K {
 };
 static_assert(sizeof(BlockQ4_0) == Q4_0_BYTES, "Q4_0");
 static_assert(sizeof(BlockQ8_0) == Q8_0_BYTES, "Q8_0");
+static_assert(sizeof(BlockQ4_1) == Q4_1_BYTES, "Q4_1");
+static_assert(sizeof(BlockQ5_0) == Q5_0_BYTES, "Q5_0");
+static_assert(sizeof(BlockQ5_1) == Q5_1_BYTES, "Q5_1");
 static_assert(sizeof(BlockQ4_K) == Q4_K_BYTES, "Q4_K");
 static_assert(sizeof(BlockQ5_K) == Q5_K_BYTES, "Q5_K");
 static_assert(sizeof(BlockQ6_K) == Q6_K_BYTES, "Q6_K");
@@ -67,6 +89,9 @@ static_assert(sizeof(BlockQ8_K) == Q8_K_BYTES, "Q8_K");
 inline size_t block_values(int kind) {
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_0:
+    case MARMOT_HIP_KIND_Q4_1:
+    case MARMOT_HIP_KIND_Q5_0:
+    case MARMOT_HIP_KIND_Q5_1:
     case MARMOT_HIP_KIND_Q8_0:
         return QK;
     case MARMOT_HIP_KIND_Q4_K:
@@ -82,6 +107,12 @@ inline size_t block_bytes(int kind) {
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_0:
         return Q4_0_BYTES;
+    case MARMOT_HIP_KIND_Q4_1:
+        return Q4_1_BYTES;
+    case MARMOT_HIP_KIND_Q5_0:
+        return Q5_0_BYTES;
+    case MARMOT_HIP_KIND_Q5_1:
+        return Q5_1_BYTES;
     case MARMOT_HIP_KIND_Q8_0:
         return Q8_0_BYTES;
     case MARMOT_HIP_KIND_Q4_K:
@@ -98,7 +129,8 @@ inline size_t block_bytes(int kind) {
 }
 // weight formats the matmul, QKV, embedding and MoE entry points accept
 inline bool is_weight_kind(int kind) {
-    return kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_K ||
+    return kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q4_1 || kind == MARMOT_HIP_KIND_Q5_0 ||
+           kind == MARMOT_HIP_KIND_Q5_1 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_K ||
            kind == MARMOT_HIP_KIND_Q5_K || kind == MARMOT_HIP_KIND_Q6_K;
 }
 inline bool is_k_quant(int kind) {

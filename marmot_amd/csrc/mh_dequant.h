@@ -87,6 +87,33 @@ __device__ __forceinline__ float dequant_value_q4_0(const uint8_t *blk, int v) {
     return (float)(q - 8) * h2f(b->scale);
 }
 
+// Q4_1 (q4_gguf.c:396-424): y = q * scale + min
+__device__ __forceinline__ float dequant_value_q4_1(const uint8_t *blk, int v) {
+    const BlockQ4_1 *b = (const BlockQ4_1 *)blk;
+    const uint8_t packed = b->qs[v & 15];
+    const int q = (v < 16) ? (packed & 0x0F) : (packed >> 4);
+    return (float)q * h2f(b->scale) + h2f(b->min);
+}
+
+// the five-bit value v of a Q5_0 / Q5_1 block: nibble v % 16 (low for v < 16) plus bit v of qh (q5_gguf.c:255-265)
+__device__ __forceinline__ int q5_legacy_value(const uint8_t *qh, const uint8_t *qs, int v) {
+    const uint8_t packed = qs[v & 15];
+    const int nib = (v < 16) ? (packed & 0x0F) : (packed >> 4);
+    return nib | (((qh[v >> 3] >> (v & 7)) & 1) << 4);
+}
+
+// Q5_0 (q5_gguf.c:242-279): y = (q - 16) * scale
+__device__ __forceinline__ float dequant_value_q5_0(const uint8_t *blk, int v) {
+    const BlockQ5_0 *b = (const BlockQ5_0 *)blk;
+    return (float)(q5_legacy_value(b->qh, b->qs, v) - 16) * h2f(b->scale);
+}
+
+// Q5_1 (q5_gguf.c:281-318): y = q * scale + min
+__device__ __forceinline__ float dequant_value_q5_1(const uint8_t *blk, int v) {
+    const BlockQ5_1 *b = (const BlockQ5_1 *)blk;
+    return (float)q5_legacy_value(b->qh, b->qs, v) * h2f(b->scale) + h2f(b->min);
+}
+
 // Q8_K (q8k_gguf.c): y = d * q
 __device__ __forceinline__ float dequant_value_q8_k(const uint8_t *blk, int v) {
     const BlockQ8_K *b = (const BlockQ8_K *)blk;
@@ -107,6 +134,12 @@ __device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
         return dequant_value_q8_0(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q4_0) {
         return dequant_value_q4_0(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q4_1) {
+        return dequant_value_q4_1(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_0) {
+        return dequant_value_q5_0(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_1) {
+        return dequant_value_q5_1(blk, v);
     } else {
         return dequant_value_q8_k(blk, v);
     }
@@ -114,8 +147,15 @@ __device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
 
 template <int KIND>
 struct KindTraits {
-    static constexpr int BV = (KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q8_0) ? QK : QK_K;
+    static constexpr int BV = (KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q8_0 ||
+                               KIND == MARMOT_HIP_KIND_Q4_1 || KIND == MARMOT_HIP_KIND_Q5_0 ||
+                               KIND == MARMOT_HIP_KIND_Q5_1)
+        ? QK
+        : QK_K;
     static constexpr int BB = KIND == MARMOT_HIP_KIND_Q4_0 ? Q4_0_BYTES
+        : KIND == MARMOT_HIP_KIND_Q4_1                     ? Q4_1_BYTES
+        : KIND == MARMOT_HIP_KIND_Q5_0                     ? Q5_0_BYTES
+        : KIND == MARMOT_HIP_KIND_Q5_1                     ? Q5_1_BYTES
         : KIND == MARMOT_HIP_KIND_Q8_0                     ? Q8_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q4_K                     ? Q4_K_BYTES
         : KIND == MARMOT_HIP_KIND_Q5_K                     ? Q5_K_BYTES

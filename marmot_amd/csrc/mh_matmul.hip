@@ -8,7 +8,7 @@ namespace mh {
 
 // ------------------------------------------------------------------------------------------------
 // Direct route: out[n, m] = sum_k dequant(W[m, k]) * (float)x_f16[n, k], fp32 accumulate.
-// Counterpart of cpu_vec_dot_{q4_0,q8_0,q4_k}_f16 (vec_dot_impl.h:220-250, 419-450, 973-1023): the same
+// Counterpart of cpu_vec_dot_{q4_0,q4_1,q5_0,q5_1,q8_0,q4_k}_f16 (vec_dot_impl.h:220-286, 351-450, 973-1023): the same
 // per-value fp32 weights, summed in a different order. One wavefront per weight row; a lane visits 8
 // consecutive k at a time (one 16-byte load of fp16 activations per column).
 // ------------------------------------------------------------------------------------------------
@@ -140,6 +140,15 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
     case MARMOT_HIP_KIND_Q4_0:
         set_route("matvec_q4_0_f16_direct");
         return launch_direct_kind<MARMOT_HIP_KIND_Q4_0>(dev, p, N);
+    case MARMOT_HIP_KIND_Q4_1:
+        set_route("matvec_q4_1_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q4_1>(dev, p, N);
+    case MARMOT_HIP_KIND_Q5_0:
+        set_route("matvec_q5_0_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q5_0>(dev, p, N);
+    case MARMOT_HIP_KIND_Q5_1:
+        set_route("matvec_q5_1_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q5_1>(dev, p, N);
     default:
         // Q5_K and Q6_K: the reference's fp16 direct dots (vec_dot_impl.h:1025-1080, 1082-1128) decode blocks with
         // index patterns that disagree with its own dequantizers; this backend declines the combination so that the

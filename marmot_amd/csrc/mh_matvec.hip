@@ -529,6 +529,86 @@ struct FmtQ40 {
     }
 };
 
+// ------------------------------------------------------------------ Q4_1, Q5_0, Q5_1 x Q8_0
+// The Q4_0 decomposition (one lane per 32-value block). HAS_MIN: the block carries a minimum, values are unsigned and
+// the dot adds min * scale_a * sum(a) (vec_dot_impl.h:186-217, 317-349); otherwise (Q5_0) values are centred by 16
+// (:288-315). FIVE: a fifth bit per value in 32 bits of qh, bit j for value j (low nibbles are values 0..15).
+template <bool HAS_MIN, bool FIVE>
+struct FmtLegacy {
+    static constexpr int QH_OFF = HAS_MIN ? 4 : 2;
+    static constexpr int QS_OFF = QH_OFF + (FIVE ? 4 : 0);
+    static constexpr int BYTES = QS_OFF + 16;
+    static constexpr int LPB = 1;
+    static constexpr int BPW = 64;
+    static constexpr int BV = QK;
+    static constexpr int ACT_DW = 10, WT_DW = 7, QUANT_TMP = 80;
+    using Act = FmtQ40::Act;
+    struct Wt {
+        uint4 q;
+        uint32_t qh;
+        uint16_t s, m;
+    };
+    __device__ static void load_act(Act &a, const ActView &av, size_t n, size_t blk, int sub) {
+        FmtQ40::load_act(a, av, n, blk, sub);
+    }
+    template <bool SIGNAL = false>
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
+        FmtQ40::quant_act<SIGNAL>(a, xrow, blk, sub);
+    }
+    __device__ static void zero_act(Act &a) {
+        FmtQ40::zero_act(a);
+    }
+    __device__ static void load_w(Wt &w, const uint8_t *blk, int) {
+        w.s = ld2(blk);
+        w.m = HAS_MIN ? ld2(blk + 2) : (uint16_t)0;
+        w.qh = FIVE ? ((uint32_t)ld2(blk + QH_OFF) | ((uint32_t)ld2(blk + QH_OFF + 2) << 16)) : 0u;
+        w.q = ld16(blk + QS_OFF);
+    }
+    // bits 0..3 of nib to bit 4 of bytes 0..3 (0x00204081 = 1 + 2^7 + 2^14 + 2^21 moves bit i to bit 8 i; no carries)
+    __device__ static uint32_t fifth(uint32_t qh, int shift) {
+        return ((((qh >> shift) & 0xfu) * 0x00204081u) & 0x01010101u) << 4;
+    }
+    template <int NC>
+    __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int) {
+        const float sw = h2f(w.s);
+        const float mw = h2f(w.m);
+        uint4 lo, hi;
+        lo.x = w.q.x & 0x0f0f0f0fu;
+        lo.y = w.q.y & 0x0f0f0f0fu;
+        lo.z = w.q.z & 0x0f0f0f0fu;
+        lo.w = w.q.w & 0x0f0f0f0fu;
+        hi.x = (w.q.x >> 4) & 0x0f0f0f0fu;
+        hi.y = (w.q.y >> 4) & 0x0f0f0f0fu;
+        hi.z = (w.q.z >> 4) & 0x0f0f0f0fu;
+        hi.w = (w.q.w >> 4) & 0x0f0f0f0fu;
+        if constexpr (FIVE) {
+            lo.x |= fifth(w.qh, 0);
+            lo.y |= fifth(w.qh, 4);
+            lo.z |= fifth(w.qh, 8);
+            lo.w |= fifth(w.qh, 12);
+            hi.x |= fifth(w.qh, 16);
+            hi.y |= fifth(w.qh, 20);
+            hi.z |= fifth(w.qh, 24);
+            hi.w |= fifth(w.qh, 28);
+        }
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+            int isum = dot16(lo, a[n].a0, 0);
+            isum = dot16(hi, a[n].a1, isum);
+            if constexpr (HAS_MIN) {
+                acc[n] += (sw * a[n].d) * (float)isum + (mw * a[n].d) * (float)a[n].sum;
+            } else {
+                isum -= 16 * a[n].sum;  // (q - 16) . a
+                acc[n] += (float)isum * (sw * a[n].d);
+            }
+        }
+    }
+};
+using FmtQ41 = FmtLegacy<true, false>;
+using FmtQ50 = FmtLegacy<false, true>;
+using FmtQ51 = FmtLegacy<true, true>;
+static_assert(FmtQ41::BYTES == Q4_1_BYTES && FmtQ50::BYTES == Q5_0_BYTES && FmtQ51::BYTES == Q5_1_BYTES, "layouts");
+
 struct MatvecParams {
     const uint8_t *w[3];  // weights of one shape sharing the activations; blockIdx.y selects one
     void *out[3];
@@ -1172,6 +1252,12 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
         return launch_fmt<FmtQ80>(dev, p, N, K, M, nw, fused ? "matvec_q8_0_q8_0_fused" : "matvec_q8_0_q8_0");
     case MARMOT_HIP_KIND_Q4_0:
         return launch_fmt<FmtQ40>(dev, p, N, K, M, nw, fused ? "matvec_q4_0_q8_0_fused" : "matvec_q4_0_q8_0");
+    case MARMOT_HIP_KIND_Q4_1:
+        return launch_fmt<FmtQ41>(dev, p, N, K, M, nw, fused ? "matvec_q4_1_q8_0_fused" : "matvec_q4_1_q8_0");
+    case MARMOT_HIP_KIND_Q5_0:
+        return launch_fmt<FmtQ50>(dev, p, N, K, M, nw, fused ? "matvec_q5_0_q8_0_fused" : "matvec_q5_0_q8_0");
+    case MARMOT_HIP_KIND_Q5_1:
+        return launch_fmt<FmtQ51>(dev, p, N, K, M, nw, fused ? "matvec_q5_1_q8_0_fused" : "matvec_q5_1_q8_0");
     default:
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "quantized matmul: unsupported quant kind %d", kind);
     }
@@ -1230,6 +1316,15 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
         break;
     case MARMOT_HIP_KIND_Q4_0:
         st = launch_tile<FmtQ40, 8>(dev, p, K, M, nw, "moe_grouped_q4_0_q8_0");
+        break;
+    case MARMOT_HIP_KIND_Q4_1:
+        st = launch_tile<FmtQ41, 8>(dev, p, K, M, nw, "moe_grouped_q4_1_q8_0");
+        break;
+    case MARMOT_HIP_KIND_Q5_0:
+        st = launch_tile<FmtQ50, 8>(dev, p, K, M, nw, "moe_grouped_q5_0_q8_0");
+        break;
+    case MARMOT_HIP_KIND_Q5_1:
+        st = launch_tile<FmtQ51, 8>(dev, p, K, M, nw, "moe_grouped_q5_1_q8_0");
         break;
     default:
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "MoE experts: unsupported quant kind %d", kind);

@@ -375,6 +375,15 @@ int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_bloc
     case MARMOT_HIP_KIND_Q4_0:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_0>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
+    case MARMOT_HIP_KIND_Q4_1:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_1>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q5_0:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q5_0>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q5_1:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q5_1>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
     case MARMOT_HIP_KIND_Q8_K:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q8_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
@@ -412,6 +421,11 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
     }
     if (!is_weight_kind(kind)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "embedding gather: unsupported quant kind %d", kind);
+    }
+    if (kind == MARMOT_HIP_KIND_Q4_1) {
+        // the reference decodes Q4_1 tables in an interleaved nibble order of its own (embedding_scalar.c:231-240)
+        // and holds no golden vector for it: declined, the caller falls back
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "embedding gather: Q4_1 tables are not offered");
     }
     if (ids_dtype != MARMOT_HIP_DTYPE_I32 && ids_dtype != MARMOT_HIP_DTYPE_I64) {
         return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "embedding gather: token ids must be INT32 or INT64");
@@ -456,6 +470,14 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
         break;
     case MARMOT_HIP_KIND_Q8_0:
         hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q8_0>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q5_0:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q5_0>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q5_1:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q5_1>), grid, block, 0, dev->stream, table, vocab, dim,
                            d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
         break;
     default:

@@ -86,6 +86,10 @@ def test_ctypes_structs_match_layout(golden_layout):
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q6_K] == golden_layout["MARMOT_QSCHEME_Q6_K"]
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q5_K] == golden_layout["MARMOT_QSCHEME_Q5_K"]
     assert ta.KIND_Q5_K == golden_layout["MARMOT_QUANT_KIND_Q5_K"]
+    for name in ("Q4_1", "Q5_0", "Q5_1"):
+        kind = getattr(ta, f"KIND_{name}")
+        assert kind == golden_layout[f"MARMOT_QUANT_KIND_{name}"]
+        assert ta.QSCHEME_OF_KIND[kind] == golden_layout[f"MARMOT_QSCHEME_{name}"]
     assert ta.KIND_Q8_K == golden_layout["MARMOT_QUANT_KIND_Q8_K"]
     assert ta.NOT_IMPLEMENTED == golden_layout["MARMOT_ERROR_NOT_IMPLEMENTED"]
     assert ta.BACKEND_HIP == golden_layout["MARMOT_BACKEND_CUDA"] + 1
@@ -134,7 +138,8 @@ def _query(lib, sig):
 
 
 def test_query_kernel_matmul_rules(lib):
-    expect_op = {ta.KIND_Q4_0: 1, ta.KIND_Q8_0: 2, ta.KIND_Q4_K: 3, ta.KIND_Q6_K: 4, ta.KIND_Q5_K: 20}
+    expect_op = {ta.KIND_Q4_0: 1, ta.KIND_Q8_0: 2, ta.KIND_Q4_K: 3, ta.KIND_Q6_K: 4, ta.KIND_Q5_K: 20, ta.KIND_Q4_1: 24,
+                 ta.KIND_Q5_0: 28, ta.KIND_Q5_1: 32}
     for kind, op in expect_op.items():
         sel = _query(lib, _sig(kind=kind))
         assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
@@ -191,7 +196,8 @@ def test_query_kernel_cost_model(lib):
 
 
 def test_query_kernel_other_ops(lib):
-    for kind, op in {ta.KIND_Q4_0: 5, ta.KIND_Q8_0: 6, ta.KIND_Q4_K: 7, ta.KIND_Q6_K: 8, ta.KIND_Q5_K: 21}.items():
+    for kind, op in {ta.KIND_Q4_0: 5, ta.KIND_Q8_0: 6, ta.KIND_Q4_K: 7, ta.KIND_Q6_K: 8, ta.KIND_Q5_K: 21,
+                     ta.KIND_Q4_1: 25, ta.KIND_Q5_0: 29, ta.KIND_Q5_1: 33}.items():
         assert _query(lib, _sig(op=ta.OP_MOE_EXPERTS, kind=kind)).op_index == op
     assert not _query(lib, _sig(op=ta.OP_MOE_EXPERTS, inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).supported
     assert _query(lib, _sig(op=ta.OP_TOPK)).op_index == 9
@@ -209,7 +215,7 @@ def test_query_kernel_qkv_rules(lib, golden_layout):
     assert ta.EPILOGUE_ROPE == golden_layout["MARMOT_EPILOGUE_ROPE"]
     for op_id in (ta.OP_QKV_PROJECTION, ta.OP_QKV_SHARED_INPUT, ta.OP_QKV_ROPE):
         for kind, op in {ta.KIND_Q4_0: 12, ta.KIND_Q8_0: 13, ta.KIND_Q4_K: 14, ta.KIND_Q6_K: 15,
-                         ta.KIND_Q5_K: 22}.items():
+                         ta.KIND_Q5_K: 22, ta.KIND_Q4_1: 26, ta.KIND_Q5_0: 30, ta.KIND_Q5_1: 34}.items():
             for dt in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, _sig(op=op_id, kind=kind, inp=dt, out=dt, N=4, K=4096, M=4096))
                 assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
@@ -252,12 +258,13 @@ def test_query_kernel_embedding_rules(lib):
         s.weight_layout = ta.WEIGHT_LAYOUT_SEPARATE
         return s
     for kind, op in ((ta.KIND_Q4_0, 16), (ta.KIND_Q8_0, 17), (ta.KIND_Q4_K, 18), (ta.KIND_Q6_K, 19),
-                     (ta.KIND_Q5_K, 23)):
+                     (ta.KIND_Q5_K, 23), (ta.KIND_Q5_0, 31), (ta.KIND_Q5_1, 35)):
         for ids in (ta.DTYPE_I32, ta.DTYPE_I64):
             for out in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, sig(kind, ids, out))
                 assert sel.supported and sel.op_index == op
     assert not _query(lib, sig(kind=ta.KIND_Q8_K)).supported
+    assert not _query(lib, sig(kind=ta.KIND_Q4_1)).supported  # interleaved table order without a golden: declined
     assert not _query(lib, sig(kind=ta.KIND_GENERIC)).supported
     assert not _query(lib, sig(ids=ta.DTYPE_F32)).supported
     assert not _query(lib, sig(out=ta.DTYPE_I32)).supported
@@ -267,7 +274,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 24
+    assert t.op_count == 36
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -287,8 +294,11 @@ def test_bytecode_tables(lib, golden_layout):
     assert sizes[12:16] == [struct.calcsize("<7HII3H")] * 4
     assert sizes[16:20] == [struct.calcsize("<3HIfI3B")] * 4 == [21] * 4
     # Q5_K was added behind the four original kinds: one op per family
-    assert schema[20:24] == [golden_layout[f"MARMOT_BC_SCHEMA_{n}"] for n in ("MATMUL", "MOE_EXPERTS", "QKV", "EMBEDDING")]
-    assert sizes[20:24] == [sizes[1], sizes[5], sizes[12], sizes[16]]
+    # kinds added behind the four original ones (Q5_K, Q4_1, Q5_0, Q5_1): four consecutive ops each
+    for base in (20, 24, 28, 32):
+        assert schema[base:base + 4] == [golden_layout[f"MARMOT_BC_SCHEMA_{n}"]
+                                         for n in ("MATMUL", "MOE_EXPERTS", "QKV", "EMBEDDING")]
+        assert sizes[base:base + 4] == [sizes[1], sizes[5], sizes[12], sizes[16]]
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -359,7 +369,7 @@ def test_kernel_def_files_name_exported_impls(lib):
         assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name
     for name, f in families.items():
         impl = f["IMPL_FUNCTION"].strip('"')
-        schemes = re.findall(r"Q\d_[0K]", f.get("AXIS(scheme)", "")) or [""]
+        schemes = re.findall(r"Q\d_[01K]", f.get("AXIS(scheme)", "")) or [""]
         for s in schemes:
             sym = impl.replace("{scheme:lower}", s.lower())
             assert hasattr(lib, sym), f"{name}: {sym} not exported"

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from marmot_amd import capi
-from oracle.pyoracle import KIND_Q4_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.test_oracle_embedding import load_golden
 from tests.util import bits, random_valid_blocks
 
@@ -27,7 +27,7 @@ def test_reference_q4_0_embedding_golden(hip):
     assert np.max(np.abs(got - expected)) <= 1e-6
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
 @pytest.mark.parametrize("ids_dtype", [np.int32, np.int64])
 def test_gather_is_bit_exact(hip, oracle, kind, ids_dtype):
     rng = np.random.default_rng(820 + kind)
@@ -59,4 +59,8 @@ def test_out_of_range_tokens_and_bounds_check(hip, oracle):
     # unsupported kinds and dtypes
     with pytest.raises(capi.MarmotHipError) as e:
         hip.embedding_gather(capi.KIND_Q8_K, table, vocab, dim, ids)
+    assert e.value.code == -8
+    with pytest.raises(capi.MarmotHipError) as e:  # Q4_1 tables: the reference's interleaved order has no golden
+        hip.embedding_gather(KIND_Q4_1, random_valid_blocks(np.random.default_rng(831), KIND_Q4_1, 4, 64), 4, 64,
+                             np.array([1], np.int32))
     assert e.value.code == -8

@@ -68,6 +68,18 @@ typedef struct {
     uint8_t qs[128];
 } blk_q5_k; /* 176 B */
 typedef struct {
+    uint8_t scales[16]; /* scale (low nibble) and min (high nibble) of each group of 16 */
+    uint8_t qs[64];
+    uint16_t d;
+    uint16_t dmin;
+} blk_q2_k; /* 84 B */
+typedef struct {
+    uint8_t hmask[32];
+    uint8_t qs[64];
+    uint8_t scales[12];
+    uint16_t d;
+} blk_q3_k; /* 110 B */
+typedef struct {
     uint8_t ql[128];
     uint8_t qh[64];
     int8_t scales[16];
@@ -87,6 +99,8 @@ _Static_assert(sizeof(blk_q5_0) == 22, "Q5_0");
 _Static_assert(sizeof(blk_q5_1) == 24, "Q5_1");
 _Static_assert(sizeof(blk_q4_k) == 144, "Q4_K");
 _Static_assert(sizeof(blk_q5_k) == 176, "Q5_K");
+_Static_assert(sizeof(blk_q2_k) == 84, "Q2_K");
+_Static_assert(sizeof(blk_q3_k) == 110, "Q3_K");
 _Static_assert(sizeof(blk_q6_k) == 210, "Q6_K");
 _Static_assert(sizeof(blk_q8_k) == 292, "Q8_K");
 
@@ -98,6 +112,8 @@ size_t mo_block_values(int kind) {
     case MO_KIND_Q5_1:
     case MO_KIND_Q8_0:
         return QK;
+    case MO_KIND_Q2_K:
+    case MO_KIND_Q3_K:
     case MO_KIND_Q4_K:
     case MO_KIND_Q5_K:
     case MO_KIND_Q6_K:
@@ -124,6 +140,10 @@ size_t mo_block_bytes(int kind) {
         return sizeof(blk_q4_k);
     case MO_KIND_Q5_K:
         return sizeof(blk_q5_k);
+    case MO_KIND_Q2_K:
+        return sizeof(blk_q2_k);
+    case MO_KIND_Q3_K:
+        return sizeof(blk_q3_k);
     case MO_KIND_Q6_K:
         return sizeof(blk_q6_k);
     case MO_KIND_Q8_K:
@@ -501,7 +521,7 @@ static void q5_1_dequantize_block(const blk_q5_1 *block, uint32_t elems, float *
 /* kquant_common.h:39-130 */
 static float make_qkx2_quants(
     int n, int nmax, const float *x, const float *weights, uint8_t *L, float *the_min, uint8_t *Laux, float rmin,
-    float rdelta, int nstep
+    float rdelta, int nstep, int use_mad
 ) {
     float min = x[0];
     float max = x[0];
@@ -535,7 +555,7 @@ static float make_qkx2_quants(
         int l = (int)nearbyintf(iscale * (x[i] - min));
         L[i] = (uint8_t)(l > nmax ? nmax : l < 0 ? 0 : l);
         float diff = scale * L[i] + min - x[i];
-        diff = diff * diff;
+        diff = use_mad ? fabsf(diff) : diff * diff;
         best_error += weights[i] * diff;
     }
     if (nstep < 1) {
@@ -565,7 +585,7 @@ static float make_qkx2_quants(
             float cur_error = 0;
             for (int i = 0; i < n; ++i) {
                 float diff = this_scale * Laux[i] + this_min - x[i];
-                diff = diff * diff;
+                diff = use_mad ? fabsf(diff) : diff * diff;
                 cur_error += weights[i] * diff;
             }
             if (cur_error < best_error) {
@@ -609,7 +629,7 @@ static void q4_k_quantize_block(const float *values, uint32_t elems, blk_q4_k *b
         for (int l = 0; l < 32; ++l) {
             weights[l] = av_x + fabsf(bv[32 * j + l]);
         }
-        scales[j] = make_qkx2_quants(32, 15, bv + 32 * j, weights, L + 32 * j, &mins[j], Laux, -1.0f, 0.1f, 20);
+        scales[j] = make_qkx2_quants(32, 15, bv + 32 * j, weights, L + 32 * j, &mins[j], Laux, -1.0f, 0.1f, 20, 0);
         if (scales[j] > max_scale) {
             max_scale = scales[j];
         }
@@ -721,7 +741,7 @@ static void q5_k_quantize_block(const float *values, uint32_t elems, blk_q5_k *b
         for (int l = 0; l < 32; ++l) {
             weights[l] = av_x + fabsf(bv[32 * j + l]);
         }
-        scales[j] = make_qkx2_quants(32, 31, bv + 32 * j, weights, L + 32 * j, &mins[j], Laux, -0.5f, 0.1f, 15);
+        scales[j] = make_qkx2_quants(32, 31, bv + 32 * j, weights, L + 32 * j, &mins[j], Laux, -0.5f, 0.1f, 15, 0);
         if (scales[j] > max_scale) {
             max_scale = scales[j];
         }
@@ -816,6 +836,279 @@ static void q5_k_dequantize_block(const blk_q5_k *block, uint32_t elems, float *
             out[written] = d2 * q - m2;
         }
         ql += 32;
+    }
+}
+
+/* ======================= Q2_K ======================= */
+
+/* q2k_gguf.c:35-111: 16 groups of 16 values, 2-bit values with a 4-bit scale and a 4-bit min per group (search with
+ * absolute deviations); value 128 c + 32 j + l sits in bits 2 j of qs[32 c + l] */
+static void q2_k_quantize_block(const float *values, uint32_t elems, blk_q2_k *block) {
+    float bv[QK_K];
+    memcpy(bv, values, elems * sizeof(float));
+    if (elems < QK_K) {
+        memset(bv + elems, 0, (QK_K - elems) * sizeof(float));
+    }
+    uint8_t L[QK_K];
+    memset(L, 0, sizeof(L));
+    uint8_t Laux[16];
+    float weights[16];
+    float scales[QK_K / 16];
+    float mins[QK_K / 16];
+    memset(block, 0, sizeof(*block));
+
+    float max_scale = 0.0f;
+    float max_min = 0.0f;
+    for (int j = 0; j < QK_K / 16; ++j) {
+        for (int l = 0; l < 16; ++l) {
+            weights[l] = fabsf(bv[16 * j + l]);
+        }
+        scales[j] = make_qkx2_quants(16, 3, bv + 16 * j, weights, L + 16 * j, &mins[j], Laux, -0.5f, 0.1f, 15, 1);
+        if (scales[j] > max_scale) {
+            max_scale = scales[j];
+        }
+        if (mins[j] > max_min) {
+            max_min = mins[j];
+        }
+    }
+    const float inv_scale = max_scale > 0 ? 15.0f / max_scale : 0.0f;
+    const float inv_min = max_min > 0 ? 15.0f / max_min : 0.0f;
+    const float d = inv_scale > 0 ? 1.0f / inv_scale : 0.0f;
+    const float dm = inv_min > 0 ? 1.0f / inv_min : 0.0f;
+    block->d = mo_f32_to_f16(d);
+    block->dmin = mo_f32_to_f16(dm);
+    for (int j = 0; j < QK_K / 16; ++j) {
+        uint8_t ls = (uint8_t)nearbyintf(inv_scale * scales[j]);
+        uint8_t lm = (uint8_t)nearbyintf(inv_min * mins[j]);
+        ls = ls > 15 ? 15 : ls;
+        lm = lm > 15 ? 15 : lm;
+        block->scales[j] = (uint8_t)(ls | (lm << 4));
+    }
+    for (int j = 0; j < QK_K / 16; ++j) {
+        const uint8_t sc = block->scales[j] & 0xF;
+        const uint8_t m = block->scales[j] >> 4;
+        const float dl = d * sc; /* the unrounded d and dm, as the reference uses them here */
+        const float ml = dm * m;
+        if (dl != 0.0f) {
+            for (int ii = 0; ii < 16; ++ii) {
+                const int l = (int)nearbyintf((bv[16 * j + ii] + ml) / dl);
+                L[16 * j + ii] = (uint8_t)(l > 3 ? 3 : (l < 0 ? 0 : l));
+            }
+        }
+    }
+    for (int j = 0; j < QK_K; j += 128) {
+        for (int l = 0; l < 32; ++l) {
+            block->qs[j / 4 + l] =
+                (uint8_t)(L[j + l] | (L[j + l + 32] << 2) | (L[j + l + 64] << 4) | (L[j + l + 96] << 6));
+        }
+    }
+}
+
+/* q2k_gguf.c:113-149: y = (d * sc) * q - dmin * m */
+static void q2_k_dequantize_block(const blk_q2_k *block, uint32_t elems, float *out) {
+    const float d = mo_f16_to_f32(block->d);
+    const float min = mo_f16_to_f32(block->dmin);
+    const uint8_t *q = block->qs;
+    size_t written = 0;
+    int is = 0;
+    for (size_t n = 0; n < QK_K && written < elems; n += 128) {
+        int shift = 0;
+        for (int j = 0; j < 4 && written < elems; ++j) {
+            for (int half = 0; half < 2; ++half) {
+                const uint8_t sc = block->scales[is++];
+                const float dl = d * (sc & 0xF);
+                const float ml = min * (sc >> 4);
+                for (int l = 0; l < 16 && written < elems; ++l, ++written) {
+                    out[written] = dl * ((int8_t)((q[l + 16 * half] >> shift) & 3)) - ml;
+                }
+            }
+            shift += 2;
+        }
+        q += 32;
+    }
+}
+
+/* ======================= Q3_K ======================= */
+
+/* kquant_common.h:230-297 (do_rmse branch) */
+static float make_q3_quants_rmse(int n, int nmax, const float *x, int8_t *L) {
+    float max = 0;
+    float amax = 0;
+    for (int i = 0; i < n; ++i) {
+        const float ax = fabsf(x[i]);
+        if (ax > amax) {
+            amax = ax;
+            max = x[i];
+        }
+    }
+    if (amax == 0) {
+        for (int i = 0; i < n; ++i) {
+            L[i] = 0;
+        }
+        return 0.0f;
+    }
+    const float iscale = -nmax / max;
+    float sumlx = 0;
+    float suml2 = 0;
+    for (int i = 0; i < n; ++i) {
+        int l = (int)nearbyintf(iscale * x[i]);
+        l = l > (nmax - 1) ? (nmax - 1) : l < -nmax ? -nmax : l;
+        L[i] = (int8_t)l;
+        const float w = x[i] * x[i];
+        sumlx += w * x[i] * l;
+        suml2 += w * l * l;
+    }
+    for (int itry = 0; itry < 5; ++itry) {
+        int n_changed = 0;
+        for (int i = 0; i < n; ++i) {
+            const float w = x[i] * x[i];
+            float slx = sumlx - w * x[i] * L[i];
+            if (slx > 0) {
+                float sl2 = suml2 - w * L[i] * L[i];
+                int new_l = (int)nearbyintf(x[i] * sl2 / slx);
+                new_l = new_l > (nmax - 1) ? (nmax - 1) : new_l < -nmax ? -nmax : new_l;
+                if (new_l != L[i]) {
+                    slx += w * x[i] * new_l;
+                    sl2 += w * new_l * new_l;
+                    if (sl2 > 0 && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        L[i] = (int8_t)new_l;
+                        sumlx = slx;
+                        suml2 = sl2;
+                        ++n_changed;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) {
+            break;
+        }
+    }
+    for (int i = 0; i < n; ++i) {
+        L[i] = (int8_t)(L[i] + nmax);
+    }
+    return suml2 > 0 ? sumlx / suml2 : 0.0f;
+}
+
+/* the 16 six-bit group scales of a Q3_K block (still offset by 32): q3k_gguf.c:140-149 */
+static void q3_k_unpack_scales(const uint8_t *packed, int8_t *scales) {
+    uint32_t aux[4];
+    memcpy(aux, packed, 12);
+    const uint32_t kmask1 = 0x03030303;
+    const uint32_t kmask2 = 0x0f0f0f0f;
+    const uint32_t tmp = aux[2];
+    aux[2] = ((aux[0] >> 4) & kmask2) | (((tmp >> 4) & kmask1) << 4);
+    aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
+    aux[0] = (aux[0] & kmask2) | (((tmp >> 0) & kmask1) << 4);
+    aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
+    memcpy(scales, aux, 16);
+}
+
+/* q3k_gguf.c:35-124 */
+static void q3_k_quantize_block(const float *values, uint32_t elems, blk_q3_k *block) {
+    float bv[QK_K];
+    memcpy(bv, values, elems * sizeof(float));
+    if (elems < QK_K) {
+        memset(bv + elems, 0, (QK_K - elems) * sizeof(float));
+    }
+    int8_t L[QK_K];
+    float scales[QK_K / 16];
+    memset(block, 0, sizeof(*block));
+    float max_scale = 0.0f;
+    float amax = 0.0f;
+    for (int j = 0; j < QK_K / 16; ++j) {
+        scales[j] = make_q3_quants_rmse(16, 4, bv + 16 * j, L + 16 * j);
+        const float scale = fabsf(scales[j]);
+        if (scale > amax) {
+            amax = scale;
+            max_scale = scales[j];
+        }
+    }
+    if (max_scale != 0.0f) {
+        const float iscale = -32.0f / max_scale;
+        for (int j = 0; j < QK_K / 16; ++j) {
+            int l = (int)nearbyintf(iscale * scales[j]);
+            l = l > 31 ? 31 : (l < -32 ? -32 : l);
+            int shifted = l + 32;
+            if (j < 8) {
+                block->scales[j] = (uint8_t)(shifted & 0xF);
+            } else {
+                block->scales[j - 8] |= (uint8_t)((shifted & 0xF) << 4);
+            }
+            shifted >>= 4;
+            block->scales[j % 4 + 8] |= (uint8_t)(shifted << (2 * (j / 4)));
+        }
+        block->d = mo_f32_to_f16(1.0f / iscale);
+    } else {
+        block->d = mo_f32_to_f16(0.0f);
+    }
+    for (int j = 0; j < QK_K / 16; ++j) {
+        int sc = j < 8 ? (block->scales[j] & 0xF) : (block->scales[j - 8] >> 4);
+        sc = (sc | (((block->scales[8 + j % 4] >> (2 * (j / 4))) & 3) << 4)) - 32;
+        const float d = mo_f16_to_f32(block->d) * sc;
+        if (d == 0) {
+            continue;
+        }
+        for (int ii = 0; ii < 16; ++ii) {
+            int l = (int)nearbyintf(bv[16 * j + ii] / d);
+            l = l > 3 ? 3 : (l < -4 ? -4 : l);
+            L[16 * j + ii] = (int8_t)(l + 4);
+        }
+    }
+    int m = 0;
+    uint8_t hm = 1;
+    for (int j = 0; j < QK_K; ++j) {
+        if (L[j] > 3) {
+            block->hmask[m] |= hm;
+            L[j] = (int8_t)(L[j] - 4);
+        }
+        if (++m == QK_K / 8) {
+            m = 0;
+            hm = (uint8_t)(hm << 1);
+        }
+    }
+    for (int j = 0; j < QK_K; j += 128) {
+        for (int l = 0; l < 32; ++l) {
+            block->qs[j / 4 + l] =
+                (uint8_t)(L[j + l] | (L[j + l + 32] << 2) | (L[j + l + 64] << 4) | (L[j + l + 96] << 6));
+        }
+    }
+    if (elems < QK_K) {
+        const size_t qs_offset = (elems + 3) / 4;
+        const size_t hmask_offset = (elems + 7) / 8;
+        if (qs_offset < sizeof(block->qs)) {
+            memset(block->qs + qs_offset, 0, sizeof(block->qs) - qs_offset);
+        }
+        if (hmask_offset < sizeof(block->hmask)) {
+            memset(block->hmask + hmask_offset, 0, sizeof(block->hmask) - hmask_offset);
+        }
+    }
+}
+
+/* q3k_gguf.c:126-175: y = (d * (sc - 32)) * (q2 - (high bit ? 0 : 4)); the high bit of value 32 t + l is bit t of
+ * hmask[l] */
+static void q3_k_dequantize_block(const blk_q3_k *block, uint32_t elems, float *out) {
+    const float d_all = mo_f16_to_f32(block->d);
+    const uint8_t *q = block->qs;
+    const uint8_t *hm = block->hmask;
+    int8_t scales[16];
+    q3_k_unpack_scales(block->scales, scales);
+    size_t written = 0;
+    int is = 0;
+    uint8_t m = 1;
+    for (size_t n = 0; n < QK_K && written < elems; n += 128) {
+        int shift = 0;
+        for (int j = 0; j < 4 && written < elems; ++j) {
+            for (int half = 0; half < 2; ++half) {
+                const float dl = d_all * (scales[is++] - 32);
+                for (int l = 0; l < 16 && written < elems; ++l, ++written) {
+                    const int li = l + 16 * half;
+                    out[written] = dl * ((int8_t)((q[li] >> shift) & 3) - ((hm[li] & m) ? 0 : 4));
+                }
+            }
+            shift += 2;
+            m = (uint8_t)(m << 1);
+        }
+        q += 32;
     }
 }
 
@@ -1133,6 +1426,12 @@ int mo_quantize_rows(int kind, const float *x, size_t rows, size_t k, void *out)
             case MO_KIND_Q5_K:
                 q5_k_quantize_block(src, elems, (blk_q5_k *)blk);
                 break;
+            case MO_KIND_Q2_K:
+                q2_k_quantize_block(src, elems, (blk_q2_k *)blk);
+                break;
+            case MO_KIND_Q3_K:
+                q3_k_quantize_block(src, elems, (blk_q3_k *)blk);
+                break;
             case MO_KIND_Q6_K:
                 q6_k_quantize_block(src, elems, (blk_q6_k *)blk);
                 break;
@@ -1189,6 +1488,12 @@ int mo_dequantize_rows(int kind, const void *blocks, size_t rows, size_t k, floa
                 break;
             case MO_KIND_Q5_K:
                 q5_k_dequantize_block((const blk_q5_k *)blk, elems, dst);
+                break;
+            case MO_KIND_Q2_K:
+                q2_k_dequantize_block((const blk_q2_k *)blk, elems, dst);
+                break;
+            case MO_KIND_Q3_K:
+                q3_k_dequantize_block((const blk_q3_k *)blk, elems, dst);
                 break;
             case MO_KIND_Q6_K:
                 q6_k_dequantize_block((const blk_q6_k *)blk, elems, dst);
@@ -1333,6 +1638,86 @@ float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks) {
         const float d = ab[b].d * mo_f16_to_f32(wb[b].d);
         const float dmin = ab[b].d * mo_f16_to_f32(wb[b].dmin);
         sum_all += d * (float)block_sum - dmin * (float)sumi;
+    }
+    return sum_all;
+}
+
+/* vec_dot_impl.h:565-618 */
+float mo_vec_dot_q2_k_q8_k(const void *w, const void *a, size_t nblocks) {
+    const blk_q2_k *wb = (const blk_q2_k *)w;
+    const blk_q8_k *ab = (const blk_q8_k *)a;
+    float sum_all = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        const uint8_t *q2 = wb[b].qs;
+        const uint8_t *sc = wb[b].scales;
+        const int8_t *q8 = ab[b].qs;
+        int32_t summs = 0;
+        for (int j = 0; j < 16; ++j) {
+            summs += (int32_t)ab[b].bsums[j] * (int32_t)(sc[j] >> 4);
+        }
+        const float dall = ab[b].d * mo_f16_to_f32(wb[b].d);
+        const float dmin = ab[b].d * mo_f16_to_f32(wb[b].dmin);
+        int32_t isum = 0;
+        int is = 0;
+        for (int chunk = 0; chunk < QK_K / 128; ++chunk) {
+            int shift = 0;
+            for (int j = 0; j < 4; ++j) {
+                for (int half = 0; half < 2; ++half) {
+                    const int32_t dsc = sc[is++] & 0xF;
+                    int32_t dot = 0;
+                    for (int l = 0; l < 16; ++l) {
+                        dot += (int32_t)q8[l + 16 * half] * (int32_t)((q2[l + 16 * half] >> shift) & 3);
+                    }
+                    isum += dsc * dot;
+                }
+                shift += 2;
+                q8 += 32;
+            }
+            q2 += 32;
+        }
+        sum_all += dall * (float)isum - dmin * (float)summs;
+    }
+    return sum_all;
+}
+
+/* vec_dot_impl.h:620-687 */
+float mo_vec_dot_q3_k_q8_k(const void *w, const void *a, size_t nblocks) {
+    const blk_q3_k *wb = (const blk_q3_k *)w;
+    const blk_q8_k *ab = (const blk_q8_k *)a;
+    float sum_all = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        const uint8_t *q3 = wb[b].qs;
+        const uint8_t *hm = wb[b].hmask;
+        const int8_t *q8 = ab[b].qs;
+        int8_t scales[16];
+        q3_k_unpack_scales(wb[b].scales, scales);
+        int32_t block_sum = 0;
+        uint8_t m = 1;
+        int scale_index = 0;
+        for (int chunk = 0; chunk < QK_K / 128; ++chunk) {
+            int shift = 0;
+            for (int j = 0; j < 4; ++j) {
+                for (int half = 0; half < 2; ++half) {
+                    int32_t dot = 0;
+                    for (int l = 0; l < 16; ++l) {
+                        const int li = l + 16 * half;
+                        int8_t val = (int8_t)((q3[li] >> shift) & 3);
+                        if ((hm[li] & m) == 0) {
+                            val = (int8_t)(val - 4);
+                        }
+                        dot += (int32_t)val * (int32_t)q8[li];
+                    }
+                    block_sum += (int32_t)(scales[scale_index] - 32) * dot;
+                    scale_index++;
+                }
+                q8 += 32;
+                shift += 2;
+                m = (uint8_t)(m << 1);
+            }
+            q3 += 32;
+        }
+        const float d = ab[b].d * mo_f16_to_f32(wb[b].d);
+        sum_all += d * (float)block_sum;
     }
     return sum_all;
 }
@@ -1505,6 +1890,64 @@ float mo_vec_dot_f16(int kind, const void *w, const uint16_t *a, size_t nblocks,
                 is += 2;
             }
         }
+    } else if (kind == MO_KIND_Q2_K) {
+        /* vec_dot_impl.h:866-908 as written: one scale / min pair per 128 values (scales[0], scales[1]) and the
+         * 2-bit values taken in sequential order (value i from bits 2 (i % 4) of qs[i / 4]); both differ from the
+         * Q2_K dequantizer. Restated so that the reference's snapshot of this function is reproduced; no product
+         * kernel mirrors it. */
+        const blk_q2_k *wb = (const blk_q2_k *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const float d = mo_f16_to_f32(wb[b].d);
+            const float dmin = mo_f16_to_f32(wb[b].dmin);
+            const uint8_t *q = wb[b].qs;
+            const size_t start = b * QK_K;
+            const size_t len = (start + QK_K <= k) ? QK_K : (k - start);
+            size_t written = 0;
+            for (size_t j = 0; j < QK_K && written < len; j += 128) {
+                const size_t index = j / 128;
+                const float dl = d * (float)(wb[b].scales[index] & 0xF);
+                const float ml = dmin * (float)(wb[b].scales[index] >> 4);
+                for (size_t i = 0; i < 128 && written < len; ++i, ++written) {
+                    const uint8_t qv = (uint8_t)((q[(j + i) / 4] >> (((j + i) % 4) * 2)) & 0x3);
+                    const float av = mo_f16_to_f32(a[start + written]);
+                    const float wv = dl * (float)qv - ml;
+                    total += wv * av;
+                }
+            }
+        }
+    } else if (kind == MO_KIND_Q3_K) {
+        /* vec_dot_impl.h:910-971 as written: the high-bit mask advances once per 128 values instead of once per
+         * 32, which differs from the Q3_K dequantizer. Restated for the same reason as Q2_K. */
+        const blk_q3_k *wb = (const blk_q3_k *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const float d_all = mo_f16_to_f32(wb[b].d);
+            const uint8_t *q = wb[b].qs;
+            const uint8_t *hm = wb[b].hmask;
+            const size_t start = b * QK_K;
+            const size_t len = (start + QK_K <= k) ? QK_K : (k - start);
+            int8_t scales[16];
+            q3_k_unpack_scales(wb[b].scales, scales);
+            size_t written = 0;
+            int is = 0;
+            uint8_t m = 1;
+            for (size_t n = 0; n < QK_K && written < len; n += 128) {
+                int shift = 0;
+                for (int j = 0; j < 4; ++j) {
+                    for (int half = 0; half < 2; ++half) {
+                        const float dl = d_all * (float)(scales[is++] - 32);
+                        for (int l = 0; l < 16 && written < len; ++l, ++written) {
+                            const int li = l + 16 * half;
+                            const float av = mo_f16_to_f32(a[start + written]);
+                            const int8_t qv = (int8_t)((int8_t)((q[li] >> shift) & 3) - ((hm[li] & m) ? 0 : 4));
+                            total += dl * (float)qv * av;
+                        }
+                    }
+                    shift += 2;
+                }
+                q += 32;
+                m = (uint8_t)(m << 1);
+            }
+        }
     } else if (kind == MO_KIND_Q5_K) {
         /* vec_dot_impl.h:1025-1080 as written: the fifth bit is taken from byte j/8 + l (+ 32 for the high nibbles)
          * counted from the start of qh, bit j % 8 = 0, i.e. for j >= 64 and for every high nibble from bytes that
@@ -1591,6 +2034,10 @@ static dot_fn pick_dot(int kind) {
         return mo_vec_dot_q4_k_q8_k;
     case MO_KIND_Q5_K:
         return mo_vec_dot_q5_k_q8_k;
+    case MO_KIND_Q2_K:
+        return mo_vec_dot_q2_k_q8_k;
+    case MO_KIND_Q3_K:
+        return mo_vec_dot_q3_k_q8_k;
     case MO_KIND_Q6_K:
         return mo_vec_dot_q6_k_q8_k;
     default:
@@ -2096,6 +2543,12 @@ int mo_embedding_gather_quantized(
                 break;
             case MO_KIND_Q5_K:
                 q5_k_dequantize_block((const blk_q5_k *)blk, (uint32_t)count, decoded);
+                break;
+            case MO_KIND_Q2_K:
+                q2_k_dequantize_block((const blk_q2_k *)blk, (uint32_t)count, decoded);
+                break;
+            case MO_KIND_Q3_K:
+                q3_k_dequantize_block((const blk_q3_k *)blk, (uint32_t)count, decoded);
                 break;
             case MO_KIND_Q6_K:
                 q6_k_dequantize_block((const blk_q6_k *)blk, (uint32_t)count, decoded);

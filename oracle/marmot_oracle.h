@@ -39,6 +39,8 @@ enum {
     MO_KIND_Q5_0 = 3,
     MO_KIND_Q5_1 = 4,
     MO_KIND_Q8_0 = 5,
+    MO_KIND_Q2_K = 7,
+    MO_KIND_Q3_K = 8,
     MO_KIND_Q4_K = 9,
     MO_KIND_Q5_K = 10,
     MO_KIND_Q6_K = 11,
@@ -88,6 +90,8 @@ float mo_vec_dot_q4_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_1_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q5_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q5_1_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q2_k_q8_k(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q3_k_q8_k(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_k_q8_k(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q5_k_q8_k(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q6_k_q8_k(const void *w, const void *a, size_t nblocks);

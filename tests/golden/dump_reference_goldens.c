@@ -46,6 +46,10 @@ int main(void) {
     EMIT(g_llama_q5_1_dequant, "f4");
     EMIT(g_llama_q8_0, "u1");
     EMIT(g_llama_q8_0_dequant, "f4");
+    EMIT(g_llama_q2_k, "u1");
+    EMIT(g_llama_q2_k_dequant, "f4");
+    EMIT(g_llama_q3_k, "u1");
+    EMIT(g_llama_q3_k_dequant, "f4");
     EMIT(g_llama_q4_k, "u1");
     EMIT(g_llama_q4_k_dequant, "f4");
     EMIT(g_llama_q5_k, "u1");
@@ -65,6 +69,8 @@ int main(void) {
     EMIT(g_vec_dot_q4_1_weights, "u1");
     EMIT(g_vec_dot_q5_0_weights, "u1");
     EMIT(g_vec_dot_q5_1_weights, "u1");
+    EMIT(g_vec_dot_q2_k_weights, "u1");
+    EMIT(g_vec_dot_q3_k_weights, "u1");
     EMIT(g_vec_dot_q4_k_weights, "u1");
     EMIT(g_vec_dot_q5_k_weights, "u1");
     EMIT(g_vec_dot_q6_k_weights, "u1");
@@ -73,6 +79,8 @@ int main(void) {
     EMIT_SCALAR(g_vec_dot_q4_1_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q5_0_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q5_1_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q2_k_q8_k_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q3_k_q8_k_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q4_k_q8_k_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q5_k_q8_k_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q6_k_q8_k_expected, "f4");
@@ -84,7 +92,8 @@ int main(void) {
         if (c->kind != MARMOT_QUANT_KIND_Q4_0 && c->kind != MARMOT_QUANT_KIND_Q8_0 &&
             c->kind != MARMOT_QUANT_KIND_Q4_K && c->kind != MARMOT_QUANT_KIND_Q5_K &&
             c->kind != MARMOT_QUANT_KIND_Q6_K && c->kind != MARMOT_QUANT_KIND_Q4_1 &&
-            c->kind != MARMOT_QUANT_KIND_Q5_0 && c->kind != MARMOT_QUANT_KIND_Q5_1) {
+            c->kind != MARMOT_QUANT_KIND_Q5_0 && c->kind != MARMOT_QUANT_KIND_Q5_1 &&
+            c->kind != MARMOT_QUANT_KIND_Q2_K && c->kind != MARMOT_QUANT_KIND_Q3_K) {
             continue;
         }
         char name[128];

@@ -246,8 +246,9 @@ static size_t dtype_size(marmot_dtype_t t) {
 
 static bool kind_supported_weight(marmot_quant_kind_t k) {
     return k == MARMOT_QUANT_KIND_Q4_0 || k == MARMOT_QUANT_KIND_Q4_1 || k == MARMOT_QUANT_KIND_Q5_0 ||
-        k == MARMOT_QUANT_KIND_Q5_1 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q4_K ||
-        k == MARMOT_QUANT_KIND_Q5_K || k == MARMOT_QUANT_KIND_Q6_K;
+        k == MARMOT_QUANT_KIND_Q5_1 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q2_K ||
+        k == MARMOT_QUANT_KIND_Q3_K || k == MARMOT_QUANT_KIND_Q4_K || k == MARMOT_QUANT_KIND_Q5_K ||
+        k == MARMOT_QUANT_KIND_Q6_K;
 }
 
 static bool kind_is_block(marmot_quant_kind_t k) {
@@ -1011,7 +1012,7 @@ static marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_exper
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "HIP MoE experts need FLOAT32 activations and INT32 expert ids");
     }
     if (!kind_supported_weight(g->quant_kind) || !kind_supported_weight(d->quant_kind)) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K or Q6_K expert weights");
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 or Q2_K to Q6_K expert weights");
     }
     if (h->shape.ndim != 2 || g->shape.ndim != 3 || u->shape.ndim != 3 || d->shape.ndim != 3 ||
         desc->topk_ids->shape.ndim != 2 || desc->topk_weights->shape.ndim != 2 || desc->out->shape.ndim != 2) {
@@ -1169,7 +1170,7 @@ static marmot_error_t dequantize_block(const void *device_ctx, const marmot_tens
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize: null argument");
     }
     if (!kind_supported_weight(input->quant_kind) && input->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K and Q8_K");
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q8_K");
     }
     if (output->dtype != MARMOT_DTYPE_FLOAT32) {
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Dequantize output must be FLOAT32");
@@ -1262,6 +1263,8 @@ HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_k, MARMOT_QUANT_KIND_Q5_K)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q4_1, MARMOT_QUANT_KIND_Q4_1)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_0, MARMOT_QUANT_KIND_Q5_0)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_1, MARMOT_QUANT_KIND_Q5_1)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q2_k, MARMOT_QUANT_KIND_Q2_K)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q3_k, MARMOT_QUANT_KIND_Q3_K)
 
 // QKV immediates (bytecode_compile.c:670-715): the tensors come from the registers, the epilogue and the rotary
 // parameters from the constant pool.
@@ -1323,6 +1326,8 @@ HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_k, MARMOT_QUANT_KIND_Q5_K)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q4_1, MARMOT_QUANT_KIND_Q4_1)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_0, MARMOT_QUANT_KIND_Q5_0)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_1, MARMOT_QUANT_KIND_Q5_1)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q2_k, MARMOT_QUANT_KIND_Q2_K)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q3_k, MARMOT_QUANT_KIND_Q3_K)
 
 // EMBEDDING immediates (bytecode_compile.c:989-1018) -> the descriptor the generated shim builds
 // (src/backends/cpu/dispatch/misc_dispatch_cpu.gen.c:115-133)
@@ -1437,6 +1442,8 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     12, 26, 28, 21,  // Q4_1
     12, 26, 28, 21,  // Q5_0
     12, 26, 28, 21,  // Q5_1
+    12, 26, 28, 21,  // Q2_K
+    12, 26, 28, 21,  // Q3_K
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1449,6 +1456,8 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS,
     MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
@@ -1465,6 +1474,8 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_matmul_q4_1, bc_exec_moe,         bc_exec_qkv_q4_1,    bc_exec_embedding,
     bc_exec_matmul_q5_0, bc_exec_moe,         bc_exec_qkv_q5_0,    bc_exec_embedding,
     bc_exec_matmul_q5_1, bc_exec_moe,         bc_exec_qkv_q5_1,    bc_exec_embedding,
+    bc_exec_matmul_q2_k, bc_exec_moe,         bc_exec_qkv_q2_k,    bc_exec_embedding,
+    bc_exec_matmul_q3_k, bc_exec_moe,         bc_exec_qkv_q3_k,    bc_exec_embedding,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -1504,6 +1515,10 @@ static int kind_of_scheme(marmot_qscheme_id_t q) {
         return MARMOT_HIP_KIND_Q5_1;
     case MARMOT_QSCHEME_Q8_0:
         return MARMOT_HIP_KIND_Q8_0;
+    case MARMOT_QSCHEME_Q2_K:
+        return MARMOT_HIP_KIND_Q2_K;
+    case MARMOT_QSCHEME_Q3_K:
+        return MARMOT_HIP_KIND_Q3_K;
     case MARMOT_QSCHEME_Q4_K:
         return MARMOT_HIP_KIND_Q4_K;
     case MARMOT_QSCHEME_Q5_K:
@@ -1535,6 +1550,10 @@ static uint16_t matmul_op_of_kind(int kind) {
         return MARMOT_HIP_BC_OP_MATMUL_Q5_0;
     case MARMOT_HIP_KIND_Q5_1:
         return MARMOT_HIP_BC_OP_MATMUL_Q5_1;
+    case MARMOT_HIP_KIND_Q2_K:
+        return MARMOT_HIP_BC_OP_MATMUL_Q2_K;
+    case MARMOT_HIP_KIND_Q3_K:
+        return MARMOT_HIP_BC_OP_MATMUL_Q3_K;
     default:
         return MARMOT_KERNEL_OP_INDEX_INVALID;
     }
@@ -1570,7 +1589,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t op = matmul_op_of_kind(kind);
         if (op == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP matmul handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K weights");
+            return unsupported("HIP matmul handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K weights");
         }
         if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
             return unsupported("HIP quantized matmul needs layout NT");
@@ -1596,6 +1615,9 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         if (kind == MARMOT_HIP_KIND_Q5_K && in16) {
             return unsupported("HIP Q5_K matmul takes FLOAT32 activations");
         }
+        if ((kind == MARMOT_HIP_KIND_Q2_K || kind == MARMOT_HIP_KIND_Q3_K) && in16) {
+            return unsupported("HIP Q2_K / Q3_K matmul takes FLOAT32 activations");
+        }
         const size_t N = sig->dims.matmul.N, K = sig->dims.matmul.K, M = sig->dims.matmul.M;
         const double bytes =
             (double)M * (double)marmot_hip_row_bytes(kind, K) + (double)N * K * (in32 ? 4 : 2) + (double)N * M * 4;
@@ -1612,7 +1634,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP QKV projection handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K weights");
+            return unsupported("HIP QKV projection handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K weights");
         }
         if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
             return unsupported("HIP QKV projection needs layout NT");
@@ -1647,7 +1669,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP embedding gather handles Q4_0, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K tables");
+            return unsupported("HIP embedding gather handles Q4_0, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K tables");
         }
         if (kind == MARMOT_HIP_KIND_Q4_1) {
             return unsupported("HIP embedding gather does not offer Q4_1 tables");
@@ -1663,7 +1685,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
     case MARMOT_OP_MOE_EXPERTS: {
         const int kind = kind_of_scheme(sig->qscheme_id);
         if (matmul_op_of_kind(kind) == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP MoE experts handle Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K and Q6_K expert weights");
+            return unsupported("HIP MoE experts handle Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K expert weights");
         }
         if (!in32 || !out32) {
             return unsupported("HIP MoE experts take FLOAT32 activations");
@@ -1685,7 +1707,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         return selected(MARMOT_HIP_BC_OP_QUANTIZE_BLOCK, launch_us, 0.0);
     case MARMOT_OP_DEQUANTIZE:
         if (kind_of_scheme(sig->qscheme_id) == 0 || !out32) {
-            return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q4_K, Q5_K, Q6_K and Q8_K to FLOAT32");
+            return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q8_K to FLOAT32");
         }
         return selected(MARMOT_HIP_BC_OP_DEQUANTIZE_BLOCK, launch_us, 0.0);
     default:
@@ -1790,6 +1812,16 @@ marmot_error_t hip_matmul_quantized_q5_1(const void *device_ctx, const marmot_te
                                          marmot_tensor_t *out) {
     return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q5_1, input, weight, epilogue, out);
 }
+marmot_error_t hip_matmul_quantized_q2_k(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q2_K, input, weight, epilogue, out);
+}
+marmot_error_t hip_matmul_quantized_q3_k(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q3_K, input, weight, epilogue, out);
+}
 marmot_error_t hip_matmul_quantized_q5_k(const void *device_ctx, const marmot_tensor_t *input,
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out) {
@@ -1817,6 +1849,12 @@ marmot_error_t hip_matmul_qkv_q5_0(const void *device_ctx, const marmot_matmul_q
 }
 marmot_error_t hip_matmul_qkv_q5_1(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q5_1, desc);
+}
+marmot_error_t hip_matmul_qkv_q2_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q2_K, desc);
+}
+marmot_error_t hip_matmul_qkv_q3_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q3_K, desc);
 }
 marmot_error_t hip_matmul_qkv_q5_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q5_K, desc);

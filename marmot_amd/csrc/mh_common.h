@@ -23,6 +23,8 @@ constexpr int Q4_1_BYTES = 20;
 constexpr int Q5_0_BYTES = 22;
 constexpr int Q5_1_BYTES = 24;
 constexpr int Q8_0_BYTES = 34;
+constexpr int Q2_K_BYTES = 84;
+constexpr int Q3_K_BYTES = 110;
 constexpr int Q4_K_BYTES = 144;
 constexpr int Q5_K_BYTES = 176;
 constexpr int Q6_K_BYTES = 210;
@@ -58,6 +60,18 @@ struct __attribute__((packed)) BlockQ4_K {
     uint8_t scales[12];
     uint8_t qs[128];
 };
+struct __attribute__((packed)) BlockQ2_K {
+    uint8_t scales[16];  // group g of 16 values: scale in the low nibble, min in the high nibble
+    uint8_t qs[64];      // value 128 c + 32 j + l: bits 2 j of qs[32 c + l]
+    uint16_t d;
+    uint16_t dmin;
+};
+struct __attribute__((packed)) BlockQ3_K {
+    uint8_t hmask[32];   // value 32 t + l: bit t of hmask[l] (set: no -4 offset)
+    uint8_t qs[64];      // low two bits, laid out like Q2_K
+    uint8_t scales[12];  // 16 six-bit scales (offset 32): low nibbles in bytes 0..7, high pairs in bytes 8..11
+    uint16_t d;
+};
 struct __attribute__((packed)) BlockQ5_K {
     uint16_t d;
     uint16_t dmin;
@@ -81,6 +95,8 @@ static_assert(sizeof(BlockQ8_0) == Q8_0_BYTES, "Q8_0");
 static_assert(sizeof(BlockQ4_1) == Q4_1_BYTES, "Q4_1");
 static_assert(sizeof(BlockQ5_0) == Q5_0_BYTES, "Q5_0");
 static_assert(sizeof(BlockQ5_1) == Q5_1_BYTES, "Q5_1");
+static_assert(sizeof(BlockQ2_K) == Q2_K_BYTES, "Q2_K");
+static_assert(sizeof(BlockQ3_K) == Q3_K_BYTES, "Q3_K");
 static_assert(sizeof(BlockQ4_K) == Q4_K_BYTES, "Q4_K");
 static_assert(sizeof(BlockQ5_K) == Q5_K_BYTES, "Q5_K");
 static_assert(sizeof(BlockQ6_K) == Q6_K_BYTES, "Q6_K");
@@ -94,6 +110,8 @@ inline size_t block_values(int kind) {
     case MARMOT_HIP_KIND_Q5_1:
     case MARMOT_HIP_KIND_Q8_0:
         return QK;
+    case MARMOT_HIP_KIND_Q2_K:
+    case MARMOT_HIP_KIND_Q3_K:
     case MARMOT_HIP_KIND_Q4_K:
     case MARMOT_HIP_KIND_Q5_K:
     case MARMOT_HIP_KIND_Q6_K:
@@ -115,6 +133,10 @@ inline size_t block_bytes(int kind) {
         return Q5_1_BYTES;
     case MARMOT_HIP_KIND_Q8_0:
         return Q8_0_BYTES;
+    case MARMOT_HIP_KIND_Q2_K:
+        return Q2_K_BYTES;
+    case MARMOT_HIP_KIND_Q3_K:
+        return Q3_K_BYTES;
     case MARMOT_HIP_KIND_Q4_K:
         return Q4_K_BYTES;
     case MARMOT_HIP_KIND_Q5_K:
@@ -130,8 +152,9 @@ inline size_t block_bytes(int kind) {
 // weight formats the matmul, QKV, embedding and MoE entry points accept
 inline bool is_weight_kind(int kind) {
     return kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q4_1 || kind == MARMOT_HIP_KIND_Q5_0 ||
-           kind == MARMOT_HIP_KIND_Q5_1 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_K ||
-           kind == MARMOT_HIP_KIND_Q5_K || kind == MARMOT_HIP_KIND_Q6_K;
+           kind == MARMOT_HIP_KIND_Q5_1 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q2_K ||
+           kind == MARMOT_HIP_KIND_Q3_K || kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q5_K ||
+           kind == MARMOT_HIP_KIND_Q6_K;
 }
 inline bool is_k_quant(int kind) {
     return block_values(kind) == QK_K;

@@ -31,6 +31,34 @@ __device__ __forceinline__ float dequant_value_q4_k(const uint8_t *blk, int v) {
     return d1 * (float)q - m1;
 }
 
+// Q2_K (q2k_gguf.c:113-149): y = (d * sc) * q - dmin * m; group v / 16 holds sc | m << 4
+__device__ __forceinline__ float dequant_value_q2_k(const uint8_t *blk, int v) {
+    const BlockQ2_K *b = (const BlockQ2_K *)blk;
+    const int c = v >> 7, j = (v >> 5) & 3, l = v & 31;
+    const uint8_t sc = b->scales[v >> 4];
+    const float dl = h2f(b->d) * (float)(sc & 0xF);
+    const float ml = h2f(b->dmin) * (float)(sc >> 4);
+    const int q = (b->qs[32 * c + l] >> (2 * j)) & 3;
+    return dl * (float)q - ml;
+}
+
+// the six-bit scale of group is (0..15) of a Q3_K block, offset 32 removed (q3k_gguf.c:140-149)
+__device__ __forceinline__ int q3k_group_scale(const uint8_t *scales, int is) {
+    const int low = is < 8 ? (scales[is] & 0xF) : (scales[is - 8] >> 4);
+    const int high = (scales[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+    return (low | (high << 4)) - 32;
+}
+
+// Q3_K (q3k_gguf.c:126-175): y = (d * sc) * (q2 - (high bit set ? 0 : 4))
+__device__ __forceinline__ float dequant_value_q3_k(const uint8_t *blk, int v) {
+    const BlockQ3_K *b = (const BlockQ3_K *)blk;
+    const int c = v >> 7, j = (v >> 5) & 3, l = v & 31;
+    const float dl = h2f(b->d) * (float)q3k_group_scale(b->scales, v >> 4);
+    const int q2 = (b->qs[32 * c + l] >> (2 * j)) & 3;
+    const int q = q2 - (((b->hmask[l] >> (v >> 5)) & 1) ? 0 : 4);
+    return dl * (float)q;
+}
+
 // Q5_K (q5k_gguf.c:162-198): the Q4_K formula with a fifth bit from qh
 __device__ __forceinline__ float dequant_value_q5_k(const uint8_t *blk, int v) {
     const BlockQ5_K *b = (const BlockQ5_K *)blk;
@@ -126,6 +154,10 @@ template <int KIND>
 __device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
     if constexpr (KIND == MARMOT_HIP_KIND_Q4_K) {
         return dequant_value_q4_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q2_K) {
+        return dequant_value_q2_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q3_K) {
+        return dequant_value_q3_k(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_K) {
         return dequant_value_q5_k(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q6_K) {
@@ -157,6 +189,8 @@ struct KindTraits {
         : KIND == MARMOT_HIP_KIND_Q5_0                     ? Q5_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q5_1                     ? Q5_1_BYTES
         : KIND == MARMOT_HIP_KIND_Q8_0                     ? Q8_0_BYTES
+        : KIND == MARMOT_HIP_KIND_Q2_K                     ? Q2_K_BYTES
+        : KIND == MARMOT_HIP_KIND_Q3_K                     ? Q3_K_BYTES
         : KIND == MARMOT_HIP_KIND_Q4_K                     ? Q4_K_BYTES
         : KIND == MARMOT_HIP_KIND_Q5_K                     ? Q5_K_BYTES
         : KIND == MARMOT_HIP_KIND_Q6_K                     ? Q6_K_BYTES

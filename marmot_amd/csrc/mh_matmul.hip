@@ -150,7 +150,7 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
         set_route("matvec_q5_1_f16_direct");
         return launch_direct_kind<MARMOT_HIP_KIND_Q5_1>(dev, p, N);
     default:
-        // Q5_K and Q6_K: the reference's fp16 direct dots (vec_dot_impl.h:1025-1080, 1082-1128) decode blocks with
+        // Q2_K, Q3_K, Q5_K and Q6_K: the reference's fp16 direct dots (vec_dot_impl.h:866-971, 1025-1128) decode blocks with
         // index patterns that disagree with its own dequantizers; this backend declines the combination so that the
         // caller falls back (NOT_IMPLEMENTED is the reference's fallback signal, dispatch_execute.c:214-233).
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED,

@@ -48,6 +48,11 @@ __device__ __forceinline__ uint2 ld8(const void *p) {
     __builtin_memcpy(&v, p, 8);
     return v;
 }
+__device__ __forceinline__ uint32_t ld4(const void *p) {
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
 __device__ __forceinline__ uint16_t ld2(const void *p) {
     uint16_t v;
     __builtin_memcpy(&v, p, 2);
@@ -419,6 +424,142 @@ struct FmtQ6K {
             const int d3 = dot16(q3, a[n].a[2], 0) - 32 * a[n].bs[2];
             const int d4 = dot16(q4, a[n].a[3], 0) - 32 * a[n].bs[3];
             const int isum = __mul24(sc0, d1) + __mul24(sc1, d2) + __mul24(sc2, d3) + __mul24(sc3, d4);
+            acc[n] += (a[n].d * d) * (float)isum;
+        }
+    }
+};
+
+// ------------------------------------------------------------------ Q2_K, Q3_K x Q8_K
+// The Q6_K decomposition (4 lanes per block; lane (hh, t) owns 16 bytes of qs = positions 16 t .. 16 t + 15 of the four
+// 32-value rows j = 0..3 of half hh, i.e. groups 8 hh + 2 j + t) and the Q6_K activation registers.
+// Q2_K (q2k_gguf.c:113-149, vec_dot_impl.h:565-618): two-bit values, group scale / min in one byte.
+struct FmtQ2K {
+    static constexpr int BYTES = Q2_K_BYTES;
+    static constexpr int LPB = 4;
+    static constexpr int BPW = 16;
+    static constexpr int BV = QK_K;
+    static constexpr int ACT_DW = 21, WT_DW = 7, QUANT_TMP = 100;
+    using Act = FmtQ6K::Act;
+    struct Wt {
+        uint4 q;
+        uint2 sc;     // the 8 scale bytes of this lane's half
+        uint32_t dd;  // d | dmin << 16
+    };
+    __device__ static void load_act(Act &a, const ActView &av, size_t n, size_t blk, int sub) {
+        FmtQ6K::load_act(a, av, n, blk, sub);
+    }
+    template <bool SIGNAL = false>
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
+        FmtQ6K::quant_act<SIGNAL>(a, xrow, blk, sub);
+    }
+    __device__ static void zero_act(Act &a) {
+        FmtQ6K::zero_act(a);
+    }
+    __device__ static void load_w(Wt &w, const uint8_t *blk, int sub) {
+        const int hh = sub >> 1, t = sub & 1;
+        w.sc = ld8(blk + 8 * hh);  // blocks are 4-byte aligned
+        w.q = ld16(blk + 16 + 32 * hh + 16 * t);
+        w.dd = ld4(blk + 80);
+    }
+    template <int NC>
+    __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int sub) {
+        const int t = sub & 1;
+        const float d = h2f((uint16_t)(w.dd & 0xffffu));
+        const float dmin = h2f((uint16_t)(w.dd >> 16));
+        const uint32_t s01 = w.sc.x >> (8 * t);  // groups t (bits 0..7) and t + 2 (bits 16..23)
+        const uint32_t s23 = w.sc.y >> (8 * t);
+        const int sc[4] = {(int)(s01 & 0xf), (int)((s01 >> 16) & 0xf), (int)(s23 & 0xf), (int)((s23 >> 16) & 0xf)};
+        const int mn[4] = {(int)((s01 >> 4) & 0xf), (int)((s01 >> 20) & 0xf), (int)((s23 >> 4) & 0xf),
+                           (int)((s23 >> 20) & 0xf)};
+        uint4 q[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            q[j].x = (w.q.x >> (2 * j)) & 0x03030303u;
+            q[j].y = (w.q.y >> (2 * j)) & 0x03030303u;
+            q[j].z = (w.q.z >> (2 * j)) & 0x03030303u;
+            q[j].w = (w.q.w >> (2 * j)) & 0x03030303u;
+        }
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+            int isum = 0, msum = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                isum += __mul24(sc[j], dot16(q[j], a[n].a[j], 0));
+                msum += __mul24(mn[j], a[n].bs[j]);
+            }
+            acc[n] += (a[n].d * d) * (float)isum - (a[n].d * dmin) * (float)msum;
+        }
+    }
+};
+
+// Q3_K (q3k_gguf.c:126-175, vec_dot_impl.h:620-687): Q2_K's two-bit layout plus a high bit per value in hmask
+// (bit 4 hh + j of hmask[l]); value = (q2 | high << 2) - 4, six-bit group scales offset by 32, no minimum.
+struct FmtQ3K {
+    static constexpr int BYTES = Q3_K_BYTES;
+    static constexpr int LPB = 4;
+    static constexpr int BPW = 16;
+    static constexpr int BV = QK_K;
+    static constexpr int ACT_DW = 21, WT_DW = 12, QUANT_TMP = 100;
+    using Act = FmtQ6K::Act;
+    struct Wt {
+        uint4 q, hm;
+        uint32_t s0, s1, s2;  // the 12 scale bytes
+        uint16_t d;
+    };
+    __device__ static void load_act(Act &a, const ActView &av, size_t n, size_t blk, int sub) {
+        FmtQ6K::load_act(a, av, n, blk, sub);
+    }
+    template <bool SIGNAL = false>
+    __device__ static void quant_act(Act &a, const float *xrow, size_t blk, int sub) {
+        FmtQ6K::quant_act<SIGNAL>(a, xrow, blk, sub);
+    }
+    __device__ static void zero_act(Act &a) {
+        FmtQ6K::zero_act(a);
+    }
+    __device__ static void load_w(Wt &w, const uint8_t *blk, int sub) {
+        const int hh = sub >> 1, t = sub & 1;
+        // 110-byte blocks are only 2-byte aligned
+        w.hm = ld16(blk + 16 * t);
+        w.q = ld16(blk + 32 + 32 * hh + 16 * t);
+        w.s0 = ld4(blk + 96);
+        w.s1 = ld4(blk + 100);
+        w.s2 = ld4(blk + 104);
+        w.d = ld2(blk + 108);
+    }
+    template <int NC>
+    __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int sub) {
+        const int hh = sub >> 1, t = sub & 1;
+        const float d = h2f(w.d);
+        // group is = 8 hh + 2 j + t: low nibble from byte is % 8 of (s0, s1) (high nibble for hh = 1), the two high
+        // bits from byte is % 4 of s2 at bit 2 (is / 4)
+        int sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int is8 = 2 * j + t;  // is % 8
+            const uint32_t lo_word = is8 < 4 ? w.s0 : w.s1;
+            const uint32_t low = (lo_word >> (8 * (is8 & 3) + 4 * hh)) & 0xfu;
+            const uint32_t high = (w.s2 >> (8 * (is8 & 3) + 2 * (2 * hh + (is8 >> 2)))) & 3u;
+            sc[j] = (int)(low | (high << 4)) - 32;
+        }
+        uint4 q[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int hb = 4 * hh + j;  // bit of hmask; moved to bit 2 of each byte
+#define MH_Q3_UNPACK(c)                                                                                                \
+    q[j].c = ((w.q.c >> (2 * j)) & 0x03030303u) | ((((w.hm.c >> hb) & 0x01010101u)) << 2);
+            MH_Q3_UNPACK(x)
+            MH_Q3_UNPACK(y)
+            MH_Q3_UNPACK(z)
+            MH_Q3_UNPACK(w)
+#undef MH_Q3_UNPACK
+        }
+#pragma unroll
+        for (int n = 0; n < NC; ++n) {
+            int isum = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                isum += __mul24(sc[j], dot16(q[j], a[n].a[j], 0) - 4 * a[n].bs[j]);
+            }
             acc[n] += (a[n].d * d) * (float)isum;
         }
     }
@@ -1246,6 +1387,10 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
         return launch_fmt<FmtQ4K>(dev, p, N, K, M, nw, fused ? "matvec_q4_k_q8_k_fused" : "matvec_q4_k_q8_k");
     case MARMOT_HIP_KIND_Q5_K:
         return launch_fmt<FmtQ5K>(dev, p, N, K, M, nw, fused ? "matvec_q5_k_q8_k_fused" : "matvec_q5_k_q8_k");
+    case MARMOT_HIP_KIND_Q2_K:
+        return launch_fmt<FmtQ2K>(dev, p, N, K, M, nw, fused ? "matvec_q2_k_q8_k_fused" : "matvec_q2_k_q8_k");
+    case MARMOT_HIP_KIND_Q3_K:
+        return launch_fmt<FmtQ3K>(dev, p, N, K, M, nw, fused ? "matvec_q3_k_q8_k_fused" : "matvec_q3_k_q8_k");
     case MARMOT_HIP_KIND_Q6_K:
         return launch_fmt<FmtQ6K>(dev, p, N, K, M, nw, fused ? "matvec_q6_k_q8_k_fused" : "matvec_q6_k_q8_k");
     case MARMOT_HIP_KIND_Q8_0:
@@ -1307,6 +1452,12 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
         break;
     case MARMOT_HIP_KIND_Q5_K:
         st = launch_tile<FmtQ5K, 8>(dev, p, K, M, nw, "moe_grouped_q5_k_q8_k");
+        break;
+    case MARMOT_HIP_KIND_Q2_K:
+        st = launch_tile<FmtQ2K, 8>(dev, p, K, M, nw, "moe_grouped_q2_k_q8_k");
+        break;
+    case MARMOT_HIP_KIND_Q3_K:
+        st = launch_tile<FmtQ3K, 8>(dev, p, K, M, nw, "moe_grouped_q3_k_q8_k");
         break;
     case MARMOT_HIP_KIND_Q6_K:
         st = launch_tile<FmtQ6K, 8>(dev, p, K, M, nw, "moe_grouped_q6_k_q8_k");

@@ -366,6 +366,12 @@ int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_bloc
     case MARMOT_HIP_KIND_Q5_K:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q5_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
+    case MARMOT_HIP_KIND_Q2_K:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q2_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
+    case MARMOT_HIP_KIND_Q3_K:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q3_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
     case MARMOT_HIP_KIND_Q6_K:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q6_K>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
@@ -462,6 +468,14 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
         break;
     case MARMOT_HIP_KIND_Q5_K:
         hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q5_K>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q2_K:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q2_K>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q3_K:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q3_K>), grid, block, 0, dev->stream, table, vocab, dim,
                            d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
         break;
     case MARMOT_HIP_KIND_Q6_K:

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from marmot_amd import capi
-from oracle.pyoracle import KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.test_oracle_embedding import load_golden
 from tests.util import bits, random_valid_blocks
 
@@ -27,12 +27,13 @@ def test_reference_q4_0_embedding_golden(hip):
     assert np.max(np.abs(got - expected)) <= 1e-6
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K,
+                                  KIND_Q6_K])
 @pytest.mark.parametrize("ids_dtype", [np.int32, np.int64])
 def test_gather_is_bit_exact(hip, oracle, kind, ids_dtype):
     rng = np.random.default_rng(820 + kind)
     vocab = 1000
-    dim = 4096 if kind in (KIND_Q4_K, KIND_Q5_K, KIND_Q6_K) else 1120  # 1120 = 35 blocks of 32: several workgroups per row
+    dim = 4096 if kind in (KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K) else 1120  # 1120 = 35 blocks of 32: several workgroups per row
     table = random_valid_blocks(rng, kind, vocab, dim)
     ids = rng.integers(0, vocab, (4, 9)).astype(ids_dtype)
     ids[1, 2], ids[3, 8] = 7, 7

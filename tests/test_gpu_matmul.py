@@ -2,13 +2,13 @@
 import numpy as np
 import pytest
 
-from oracle.pyoracle import BLOCK_VALUES, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import BLOCK_VALUES, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.util import assert_matmul_parity, bits, gaussian, parity_metrics, quantize_weights, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
 KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K,
-         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1}
+         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K}
 THREADS = 16
 
 
@@ -21,7 +21,7 @@ def hip():
     b.close()
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q2_K", "Q3_K", "Q4_K", "Q5_K", "Q6_K"])
 def test_reference_matmul_goldens_fp32(hip, ref_goldens, name):
     """The reference's own golden cases (tests/backend/golden_matmul_llama.h), its own tolerance."""
     kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
@@ -92,7 +92,7 @@ def test_config2_kquant_decode_full_size(hip, oracle, name, M, K):
     d_w.free()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("N", [1, 2, 3, 5, 8, 11, 16, 19])
 def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
     """All column-tile widths (8/4/2/1) and M not a multiple of the rows-per-workgroup."""
@@ -105,7 +105,7 @@ def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
     assert_matmul_parity(got, ref, what=f"{name} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("K", [256, 512, 768, 1280, 8192, 11008, 28672])
 def test_linear_k_sweep(hip, oracle, name, K):
     """Rows shorter than one wave-load, rows needing several wavefronts, and long rows."""
@@ -119,7 +119,7 @@ def test_linear_k_sweep(hip, oracle, name, K):
         assert_matmul_parity(got, ref, what=f"{name} K={K} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_linear_ragged_k(hip, oracle, name):
     """K not a multiple of the block: weight and activation tails are zero-padded blocks."""
     kind = KINDS[name]
@@ -133,7 +133,7 @@ def test_linear_ragged_k(hip, oracle, name):
     assert_matmul_parity(got, ref, what=f"{name} ragged K={K}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_linear_random_block_bytes(hip, oracle, name):
     """Weights that are arbitrary block bytes (all 6-bit scale / min patterns, negative Q6_K scales)."""
     kind = KINDS[name]
@@ -146,7 +146,7 @@ def test_linear_random_block_bytes(hip, oracle, name):
     assert_matmul_parity(got, ref, what=f"{name} random bytes")
 
 
-@pytest.mark.parametrize("name", ["q8_0", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_linear_bias_epilogue(hip, oracle, name):
     kind = KINDS[name]
     M, K, N = 50, 1024, 3
@@ -201,9 +201,12 @@ def test_linear_error_behaviour(hip, oracle):
         hip.linear(x, blocks, KIND_Q4_K, M, out_dtype=np.float16)
     assert e.value.code == -6
     with pytest.raises(MarmotHipError) as e:  # unsupported quant kind -> NOT_IMPLEMENTED (fallback signal)
-        hip.linear(x, np.zeros(M * 84, dtype=np.uint8), 7, M) if False else hip.linear_d(
-            7, hip.to_device(blocks), hip.to_device(x), 0, 1, K, M, hip.alloc(64), 0)
+        hip.linear_d(6, hip.to_device(blocks), hip.to_device(x), 0, 1, K, M, hip.alloc(64), 0)  # Q8_1
     assert e.value.code == -8
+    for kind in (KIND_Q2_K, KIND_Q3_K, KIND_Q5_K):  # their fp16 direct dots in the reference are unsound: declined
+        with pytest.raises(MarmotHipError) as e:
+            hip.linear(x.astype(np.float16), oracle.quantize(kind, gaussian(133, (M, K), 0.02)), kind, M)
+        assert e.value.code == -8
     with pytest.raises(MarmotHipError) as e:  # Q6_K with unpacked fp16 activations is declined
         hip.linear(x.astype(np.float16), oracle.quantize(KIND_Q6_K, gaussian(132, (M, K), 0.02)), KIND_Q6_K, M)
     assert e.value.code == -8
@@ -212,7 +215,7 @@ def test_linear_error_behaviour(hip, oracle):
     hip.synchronize()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_loader_consumer_matvec_equals_register_streaming_matvec(hip, oracle, name, monkeypatch):
     """The loader/consumer matvec (weights through an LDS ring) keeps the lane mapping and the reduction order of the
     register-streaming kernel: the two must agree bit for bit, on whole and ragged row groups, one and two K slices

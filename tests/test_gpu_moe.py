@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from oracle.pyoracle import KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import KIND_Q2_K, KIND_Q3_K, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.test_oracle_moe import make_experts
 from tests.util import assert_moe_parity, gaussian, parity_metrics, quantize_weights
 
@@ -62,7 +62,8 @@ def test_topk_and_softmax_match_oracle(hip, oracle):
 
 @pytest.mark.parametrize("kind_gu,kind_dn", [(KIND_Q4_K, KIND_Q4_K), (KIND_Q4_K, KIND_Q6_K), (KIND_Q8_0, KIND_Q8_0),
                                              (KIND_Q5_K, KIND_Q5_K), (KIND_Q5_K, KIND_Q6_K),
-                                             (KIND_Q5_0, KIND_Q5_1), (KIND_Q4_1, KIND_Q8_0)])
+                                             (KIND_Q5_0, KIND_Q5_1), (KIND_Q4_1, KIND_Q8_0),
+                                             (KIND_Q2_K, KIND_Q3_K), (KIND_Q3_K, KIND_Q6_K)])
 @pytest.mark.parametrize("T", [1, 3, 4, 5, 17, 64])
 def test_moe_small(hip, oracle, kind_gu, kind_dn, T):
     """Decode-order path (T <= 4) and grouped path, several routes per expert (more than one work item)."""

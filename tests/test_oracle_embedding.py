@@ -12,7 +12,7 @@ import os
 import numpy as np
 import pytest
 
-from oracle.pyoracle import (KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
+from oracle.pyoracle import (KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
                              row_bytes)
 from tests.util import bits, gaussian, random_valid_blocks
 
@@ -44,10 +44,11 @@ def test_q4_1_tables_are_declined(oracle):
         oracle.embedding_gather(KIND_Q4_1, table, 4, 64, np.array([1], np.int32))
 
 
-@pytest.mark.parametrize("kind", [KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q5_0, KIND_Q5_1])
+@pytest.mark.parametrize("kind", [KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q5_0, KIND_Q5_1, KIND_Q2_K,
+                                  KIND_Q3_K])
 def test_gathered_rows_are_dequantized_rows(oracle, kind):
     rng = np.random.default_rng(800 + kind)
-    vocab, dim = 37, 768 if kind in (KIND_Q4_K, KIND_Q5_K, KIND_Q6_K) else 96
+    vocab, dim = 37, 768 if kind in (KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K) else 96
     table = random_valid_blocks(rng, kind, vocab, dim)
     dense = oracle.dequantize(kind, table, dim)
     ids = rng.integers(0, vocab, (3, 5)).astype(np.int64)

@@ -45,7 +45,7 @@ def random_blocks(rng, kind: int, rows: int, k: int) -> np.ndarray:
     nb = (k + block_values(kind) - 1) // block_values(kind)
     bb = block_bytes(kind)
     raw = rng.integers(0, 256, size=(rows * nb, bb), dtype=np.uint8)
-    offs = {1: [0], 2: [0, 2], 3: [0], 4: [0, 2], 5: [0], 9: [0, 2], 10: [0, 2], 11: [208]}[kind]
+    offs = {1: [0], 2: [0, 2], 3: [0], 4: [0, 2], 5: [0], 7: [80, 82], 8: [108], 9: [0, 2], 10: [0, 2], 11: [208]}[kind]
     for off in offs:
         h = raw[:, off:off + 2].copy().view(np.uint16)
         h = (h & 0x83FF) | 0x2000  # exponent field 8: magnitudes around 2^-7
@@ -163,14 +163,15 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "LOGITS", "Q5K", "LEGACY")):
-    """Every benchmark configuration (C1..C5, QKV, LOGITS, Q5K, LEGACY) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "LOGITS", "Q5K", "LEGACY", "Q23K")):
+    """Every benchmark configuration (C1..C5, QKV, LOGITS, Q5K, LEGACY, Q23K) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
     rng = np.random.Generator(np.random.PCG64(7))
     names = {capi.KIND_Q4_K: "Q4_K", capi.KIND_Q5_K: "Q5_K", capi.KIND_Q6_K: "Q6_K", capi.KIND_Q8_0: "Q8_0",
-             capi.KIND_Q4_0: "Q4_0", capi.KIND_Q4_1: "Q4_1", capi.KIND_Q5_0: "Q5_0", capi.KIND_Q5_1: "Q5_1"}
+             capi.KIND_Q4_0: "Q4_0", capi.KIND_Q4_1: "Q4_1", capi.KIND_Q5_0: "Q5_0", capi.KIND_Q5_1: "Q5_1",
+             capi.KIND_Q2_K: "Q2_K", capi.KIND_Q3_K: "Q3_K"}
 
     def emit(rec):
         print(json.dumps(rec), flush=True)
@@ -212,6 +213,11 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV
         for (M, K) in ((14336, 4096), (4096, 14336)):
             for N in (1, 4, 8, 16):
                 linear_case("Q5K", capi.KIND_Q5_K, M, K, N)
+    if "Q23K" in only:
+        # the low-bit K formats on the dot-product matvec (four lanes per block), decode and small batch
+        for kind in (capi.KIND_Q2_K, capi.KIND_Q3_K):
+            for N in (1, 4, 8):
+                linear_case("Q23K", kind, 14336, 4096, N)
     if "LEGACY" in only:
         # the 32-value formats on the dot-product matvec (one lane per block), decode sizes
         for kind in (capi.KIND_Q4_0, capi.KIND_Q4_1, capi.KIND_Q5_0, capi.KIND_Q5_1, capi.KIND_Q8_0):

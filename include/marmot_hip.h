@@ -47,6 +47,7 @@ enum {
     MARMOT_HIP_KIND_Q5_0 = 3,
     MARMOT_HIP_KIND_Q5_1 = 4,
     MARMOT_HIP_KIND_Q8_0 = 5,
+    MARMOT_HIP_KIND_Q8_1 = 6,
     MARMOT_HIP_KIND_Q2_K = 7,
     MARMOT_HIP_KIND_Q3_K = 8,
     MARMOT_HIP_KIND_Q4_K = 9,

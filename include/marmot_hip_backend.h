@@ -646,7 +646,7 @@ const marmot_device_ops_t *marmot_get_hip_ops(void);
  * Matching rules follow the generated queries (scripts/codegen/templates/backend_query.c.j2:60-104): profile is
  * a wildcard; matmul needs layout NT, input F32 or F16, output F32 (or F16 with F16 input), accumulation F32,
  * weight layout SEPARATE, contiguous strides, epilogue flags within {BIAS}, no variant flags, and a weight
- * scheme of Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K (Q2_K, Q3_K, Q5_K and Q6_K with F16 input
+ * scheme of Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K (Q2_K, Q3_K, Q5_K and Q6_K with F16 input
  * are declined: the caller falls back). */
 marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *sig, const marmot_device_caps_t *caps);
 marmot_device_caps_t marmot_hip_detect_default_caps(void);
@@ -713,7 +713,11 @@ enum {
     MARMOT_HIP_BC_OP_MOE_EXPERTS_Q3_K = 41,
     MARMOT_HIP_BC_OP_QKV_Q3_K = 42,
     MARMOT_HIP_BC_OP_EMBEDDING_Q3_K = 43,
-    MARMOT_HIP_BC_OP_COUNT = 44,
+    MARMOT_HIP_BC_OP_MATMUL_Q8_1 = 44,
+    MARMOT_HIP_BC_OP_MOE_EXPERTS_Q8_1 = 45,
+    MARMOT_HIP_BC_OP_QKV_Q8_1 = 46,
+    MARMOT_HIP_BC_OP_EMBEDDING_Q8_1 = 47,
+    MARMOT_HIP_BC_OP_COUNT = 48,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -748,6 +752,9 @@ marmot_error_t hip_matmul_quantized_q2_k(const void *device_ctx, const marmot_te
 marmot_error_t hip_matmul_quantized_q3_k(const void *device_ctx, const marmot_tensor_t *input,
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out);
+marmot_error_t hip_matmul_quantized_q8_1(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out);
 marmot_error_t hip_matmul_quantized_q5_k(const void *device_ctx, const marmot_tensor_t *input,
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out);
@@ -767,19 +774,20 @@ marmot_error_t hip_matmul_qkv_q5_0(const void *device_ctx, const marmot_matmul_q
 marmot_error_t hip_matmul_qkv_q5_1(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q2_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q3_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
+marmot_error_t hip_matmul_qkv_q8_1(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q5_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 /* marmot_embedding_gather with a block-quantized table [vocab, dim] (cf. cpu_embedding_gather,
  * src/backends/cpu/ops/embedding/embedding_dispatch.c:4-16 -> embedding_scalar.c:460-591): token ids INT32 or INT64 of
  * any shape, output FLOAT32 or FLOAT16 viewed as [tokens, dim]; weights->quant_kind selects Q4_0, Q5_0, Q5_1,
- * Q8_0, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K (Q4_1 tables are declined). */
+ * Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K (Q4_1 tables are declined). */
 marmot_error_t hip_embedding_gather(const void *device_ctx, const marmot_embedding_gather_desc_t *desc);
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc);
 marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc);
 /* output->quant_kind selects the activation block format: Q8_0 or Q8_K */
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output);
-/* input->quant_kind selects the weight block format: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K
- * or Q8_K */
+/* input->quant_kind selects the weight block format: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K,
+ * Q6_K or Q8_K */
 marmot_error_t hip_dequantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output);
 
 /* ------------------------------------------------------------------ error text and introspection

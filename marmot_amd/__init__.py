@@ -7,10 +7,10 @@ benchmark: it loads the library with ctypes and exposes the reference's operator
 arrays and device buffers. There is no CPU fallback: if the library is missing, loading raises.
 """
 from .capi import (DT_F16, DT_F32, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
-                   KIND_Q8_K, MarmotHipError, lib_path, load_library)
+                   KIND_Q8_1, KIND_Q8_K, MarmotHipError, lib_path, load_library)
 from .backend import DeviceBuffer, HipBackend, block_bytes, block_values, row_bytes
 
 __all__ = [
-    "DT_F16", "DT_F32", "KIND_Q2_K", "KIND_Q3_K", "KIND_Q4_0", "KIND_Q4_1", "KIND_Q5_0", "KIND_Q5_1", "KIND_Q4_K", "KIND_Q5_K", "KIND_Q6_K", "KIND_Q8_0", "KIND_Q8_K", "MarmotHipError",
+    "DT_F16", "DT_F32", "KIND_Q2_K", "KIND_Q3_K", "KIND_Q4_0", "KIND_Q4_1", "KIND_Q5_0", "KIND_Q5_1", "KIND_Q4_K", "KIND_Q5_K", "KIND_Q6_K", "KIND_Q8_0", "KIND_Q8_1", "KIND_Q8_K", "MarmotHipError",
     "lib_path", "load_library", "DeviceBuffer", "HipBackend", "block_bytes", "block_values", "row_bytes",
 ]

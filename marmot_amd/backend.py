@@ -13,8 +13,8 @@ import numpy as np
 from . import capi
 from .capi import DT_F16, DT_F32, KIND_Q8_0, KIND_Q8_K, check, load_library
 
-_BV = {1: 32, 2: 32, 3: 32, 4: 32, 5: 32, 7: 256, 8: 256, 9: 256, 10: 256, 11: 256, 12: 256}
-_BB = {1: 18, 2: 20, 3: 22, 4: 24, 5: 34, 7: 84, 8: 110, 9: 144, 10: 176, 11: 210, 12: 292}
+_BV = {1: 32, 2: 32, 3: 32, 4: 32, 5: 32, 6: 32, 7: 256, 8: 256, 9: 256, 10: 256, 11: 256, 12: 256}
+_BB = {1: 18, 2: 20, 3: 22, 4: 24, 5: 34, 6: 36, 7: 84, 8: 110, 9: 144, 10: 176, 11: 210, 12: 292}
 
 
 def block_values(kind: int) -> int:

@@ -9,6 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_K = 1, 5, 9, 10, 11, 12
 KIND_Q4_1, KIND_Q5_0, KIND_Q5_1 = 2, 3, 4
 KIND_Q2_K, KIND_Q3_K = 7, 8
+KIND_Q8_1 = 6
 DT_F32, DT_F16 = 0, 1
 DT_I32, DT_I64 = 3, 11  # position tensors of the rotary epilogue
 FLAG_FORCE_PACK = 1

@@ -246,7 +246,8 @@ static size_t dtype_size(marmot_dtype_t t) {
 
 static bool kind_supported_weight(marmot_quant_kind_t k) {
     return k == MARMOT_QUANT_KIND_Q4_0 || k == MARMOT_QUANT_KIND_Q4_1 || k == MARMOT_QUANT_KIND_Q5_0 ||
-        k == MARMOT_QUANT_KIND_Q5_1 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q2_K ||
+        k == MARMOT_QUANT_KIND_Q5_1 || k == MARMOT_QUANT_KIND_Q8_0 || k == MARMOT_QUANT_KIND_Q8_1 ||
+        k == MARMOT_QUANT_KIND_Q2_K ||
         k == MARMOT_QUANT_KIND_Q3_K || k == MARMOT_QUANT_KIND_Q4_K || k == MARMOT_QUANT_KIND_Q5_K ||
         k == MARMOT_QUANT_KIND_Q6_K;
 }
@@ -1012,7 +1013,7 @@ static marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_exper
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "HIP MoE experts need FLOAT32 activations and INT32 expert ids");
     }
     if (!kind_supported_weight(g->quant_kind) || !kind_supported_weight(d->quant_kind)) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 or Q2_K to Q6_K expert weights");
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP MoE experts need Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 or Q2_K to Q6_K expert weights");
     }
     if (h->shape.ndim != 2 || g->shape.ndim != 3 || u->shape.ndim != 3 || d->shape.ndim != 3 ||
         desc->topk_ids->shape.ndim != 2 || desc->topk_weights->shape.ndim != 2 || desc->out->shape.ndim != 2) {
@@ -1170,7 +1171,7 @@ static marmot_error_t dequantize_block(const void *device_ctx, const marmot_tens
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Dequantize: null argument");
     }
     if (!kind_supported_weight(input->quant_kind) && input->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q8_K");
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q8_K");
     }
     if (output->dtype != MARMOT_DTYPE_FLOAT32) {
         return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Dequantize output must be FLOAT32");
@@ -1265,6 +1266,7 @@ HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_0, MARMOT_QUANT_KIND_Q5_0)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q5_1, MARMOT_QUANT_KIND_Q5_1)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q2_k, MARMOT_QUANT_KIND_Q2_K)
 HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q3_k, MARMOT_QUANT_KIND_Q3_K)
+HIP_BC_MATMUL_ENTRY(bc_exec_matmul_q8_1, MARMOT_QUANT_KIND_Q8_1)
 
 // QKV immediates (bytecode_compile.c:670-715): the tensors come from the registers, the epilogue and the rotary
 // parameters from the constant pool.
@@ -1328,6 +1330,7 @@ HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_0, MARMOT_QUANT_KIND_Q5_0)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q5_1, MARMOT_QUANT_KIND_Q5_1)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q2_k, MARMOT_QUANT_KIND_Q2_K)
 HIP_BC_QKV_ENTRY(bc_exec_qkv_q3_k, MARMOT_QUANT_KIND_Q3_K)
+HIP_BC_QKV_ENTRY(bc_exec_qkv_q8_1, MARMOT_QUANT_KIND_Q8_1)
 
 // EMBEDDING immediates (bytecode_compile.c:989-1018) -> the descriptor the generated shim builds
 // (src/backends/cpu/dispatch/misc_dispatch_cpu.gen.c:115-133)
@@ -1444,6 +1447,7 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     12, 26, 28, 21,  // Q5_1
     12, 26, 28, 21,  // Q2_K
     12, 26, 28, 21,  // Q3_K
+    12, 26, 28, 21,  // Q8_1
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1456,6 +1460,7 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_EMBEDDING,   MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS,
     MARMOT_BC_SCHEMA_QKV,         MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
@@ -1476,6 +1481,7 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_matmul_q5_1, bc_exec_moe,         bc_exec_qkv_q5_1,    bc_exec_embedding,
     bc_exec_matmul_q2_k, bc_exec_moe,         bc_exec_qkv_q2_k,    bc_exec_embedding,
     bc_exec_matmul_q3_k, bc_exec_moe,         bc_exec_qkv_q3_k,    bc_exec_embedding,
+    bc_exec_matmul_q8_1, bc_exec_moe,         bc_exec_qkv_q8_1,    bc_exec_embedding,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -1515,6 +1521,8 @@ static int kind_of_scheme(marmot_qscheme_id_t q) {
         return MARMOT_HIP_KIND_Q5_1;
     case MARMOT_QSCHEME_Q8_0:
         return MARMOT_HIP_KIND_Q8_0;
+    case MARMOT_QSCHEME_Q8_1:
+        return MARMOT_HIP_KIND_Q8_1;
     case MARMOT_QSCHEME_Q2_K:
         return MARMOT_HIP_KIND_Q2_K;
     case MARMOT_QSCHEME_Q3_K:
@@ -1550,6 +1558,8 @@ static uint16_t matmul_op_of_kind(int kind) {
         return MARMOT_HIP_BC_OP_MATMUL_Q5_0;
     case MARMOT_HIP_KIND_Q5_1:
         return MARMOT_HIP_BC_OP_MATMUL_Q5_1;
+    case MARMOT_HIP_KIND_Q8_1:
+        return MARMOT_HIP_BC_OP_MATMUL_Q8_1;
     case MARMOT_HIP_KIND_Q2_K:
         return MARMOT_HIP_BC_OP_MATMUL_Q2_K;
     case MARMOT_HIP_KIND_Q3_K:
@@ -1589,7 +1599,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t op = matmul_op_of_kind(kind);
         if (op == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP matmul handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K weights");
+            return unsupported("HIP matmul handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q6_K weights");
         }
         if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
             return unsupported("HIP quantized matmul needs layout NT");
@@ -1634,7 +1644,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP QKV projection handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K weights");
+            return unsupported("HIP QKV projection handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q6_K weights");
         }
         if (sig->matmul_layout != MARMOT_MATMUL_LAYOUT_NT) {
             return unsupported("HIP QKV projection needs layout NT");
@@ -1669,7 +1679,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP embedding gather handles Q4_0, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K tables");
+            return unsupported("HIP embedding gather handles Q4_0, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q6_K tables");
         }
         if (kind == MARMOT_HIP_KIND_Q4_1) {
             return unsupported("HIP embedding gather does not offer Q4_1 tables");
@@ -1685,7 +1695,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
     case MARMOT_OP_MOE_EXPERTS: {
         const int kind = kind_of_scheme(sig->qscheme_id);
         if (matmul_op_of_kind(kind) == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP MoE experts handle Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q6_K expert weights");
+            return unsupported("HIP MoE experts handle Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q6_K expert weights");
         }
         if (!in32 || !out32) {
             return unsupported("HIP MoE experts take FLOAT32 activations");
@@ -1707,7 +1717,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         return selected(MARMOT_HIP_BC_OP_QUANTIZE_BLOCK, launch_us, 0.0);
     case MARMOT_OP_DEQUANTIZE:
         if (kind_of_scheme(sig->qscheme_id) == 0 || !out32) {
-            return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 and Q2_K to Q8_K to FLOAT32");
+            return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q8_K to FLOAT32");
         }
         return selected(MARMOT_HIP_BC_OP_DEQUANTIZE_BLOCK, launch_us, 0.0);
     default:
@@ -1822,6 +1832,11 @@ marmot_error_t hip_matmul_quantized_q3_k(const void *device_ctx, const marmot_te
                                          marmot_tensor_t *out) {
     return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q3_K, input, weight, epilogue, out);
 }
+marmot_error_t hip_matmul_quantized_q8_1(const void *device_ctx, const marmot_tensor_t *input,
+                                         const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
+                                         marmot_tensor_t *out) {
+    return matmul_quantized(device_ctx, MARMOT_QUANT_KIND_Q8_1, input, weight, epilogue, out);
+}
 marmot_error_t hip_matmul_quantized_q5_k(const void *device_ctx, const marmot_tensor_t *input,
                                          const marmot_tensor_t *weight, const marmot_matmul_epilogue_t *epilogue,
                                          marmot_tensor_t *out) {
@@ -1855,6 +1870,9 @@ marmot_error_t hip_matmul_qkv_q2_k(const void *device_ctx, const marmot_matmul_q
 }
 marmot_error_t hip_matmul_qkv_q3_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q3_K, desc);
+}
+marmot_error_t hip_matmul_qkv_q8_1(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
+    return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q8_1, desc);
 }
 marmot_error_t hip_matmul_qkv_q5_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc) {
     return matmul_qkv(device_ctx, MARMOT_QUANT_KIND_Q5_K, desc);

@@ -23,6 +23,7 @@ constexpr int Q4_1_BYTES = 20;
 constexpr int Q5_0_BYTES = 22;
 constexpr int Q5_1_BYTES = 24;
 constexpr int Q8_0_BYTES = 34;
+constexpr int Q8_1_BYTES = 36;
 constexpr int Q2_K_BYTES = 84;
 constexpr int Q3_K_BYTES = 110;
 constexpr int Q4_K_BYTES = 144;
@@ -60,6 +61,11 @@ struct __attribute__((packed)) BlockQ4_K {
     uint8_t scales[12];
     uint8_t qs[128];
 };
+struct __attribute__((packed)) BlockQ8_1 {
+    uint16_t scale;
+    uint16_t sum;  // f16(sum(q) * scale); not used by the dequantizer or the dots
+    int8_t qs[32];
+};
 struct __attribute__((packed)) BlockQ2_K {
     uint8_t scales[16];  // group g of 16 values: scale in the low nibble, min in the high nibble
     uint8_t qs[64];      // value 128 c + 32 j + l: bits 2 j of qs[32 c + l]
@@ -92,6 +98,7 @@ struct __attribute__((packed)) BlockQ8_K {
 };
 static_assert(sizeof(BlockQ4_0) == Q4_0_BYTES, "Q4_0");
 static_assert(sizeof(BlockQ8_0) == Q8_0_BYTES, "Q8_0");
+static_assert(sizeof(BlockQ8_1) == Q8_1_BYTES, "Q8_1");
 static_assert(sizeof(BlockQ4_1) == Q4_1_BYTES, "Q4_1");
 static_assert(sizeof(BlockQ5_0) == Q5_0_BYTES, "Q5_0");
 static_assert(sizeof(BlockQ5_1) == Q5_1_BYTES, "Q5_1");
@@ -109,6 +116,7 @@ inline size_t block_values(int kind) {
     case MARMOT_HIP_KIND_Q5_0:
     case MARMOT_HIP_KIND_Q5_1:
     case MARMOT_HIP_KIND_Q8_0:
+    case MARMOT_HIP_KIND_Q8_1:
         return QK;
     case MARMOT_HIP_KIND_Q2_K:
     case MARMOT_HIP_KIND_Q3_K:
@@ -131,6 +139,8 @@ inline size_t block_bytes(int kind) {
         return Q5_0_BYTES;
     case MARMOT_HIP_KIND_Q5_1:
         return Q5_1_BYTES;
+    case MARMOT_HIP_KIND_Q8_1:
+        return Q8_1_BYTES;
     case MARMOT_HIP_KIND_Q8_0:
         return Q8_0_BYTES;
     case MARMOT_HIP_KIND_Q2_K:
@@ -152,7 +162,8 @@ inline size_t block_bytes(int kind) {
 // weight formats the matmul, QKV, embedding and MoE entry points accept
 inline bool is_weight_kind(int kind) {
     return kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q4_1 || kind == MARMOT_HIP_KIND_Q5_0 ||
-           kind == MARMOT_HIP_KIND_Q5_1 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q2_K ||
+           kind == MARMOT_HIP_KIND_Q5_1 || kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q8_1 ||
+           kind == MARMOT_HIP_KIND_Q2_K ||
            kind == MARMOT_HIP_KIND_Q3_K || kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q5_K ||
            kind == MARMOT_HIP_KIND_Q6_K;
 }

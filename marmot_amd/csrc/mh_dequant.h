@@ -107,6 +107,12 @@ __device__ __forceinline__ float dequant_value_q8_0(const uint8_t *blk, int v) {
     return (float)b->qs[v] * h2f(b->scale);
 }
 
+// Q8_1 (q8_gguf.c:202-213): y = (float)q * scale
+__device__ __forceinline__ float dequant_value_q8_1(const uint8_t *blk, int v) {
+    const BlockQ8_1 *b = (const BlockQ8_1 *)blk;
+    return (float)b->qs[v] * h2f(b->scale);
+}
+
 // Q4_0 (q4_gguf.c:367-394): y = (q - 8) * scale
 __device__ __forceinline__ float dequant_value_q4_0(const uint8_t *blk, int v) {
     const BlockQ4_0 *b = (const BlockQ4_0 *)blk;
@@ -166,6 +172,8 @@ __device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
         return dequant_value_q8_0(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q4_0) {
         return dequant_value_q4_0(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q8_1) {
+        return dequant_value_q8_1(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q4_1) {
         return dequant_value_q4_1(blk, v);
     } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_0) {
@@ -181,13 +189,14 @@ template <int KIND>
 struct KindTraits {
     static constexpr int BV = (KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q8_0 ||
                                KIND == MARMOT_HIP_KIND_Q4_1 || KIND == MARMOT_HIP_KIND_Q5_0 ||
-                               KIND == MARMOT_HIP_KIND_Q5_1)
+                               KIND == MARMOT_HIP_KIND_Q5_1 || KIND == MARMOT_HIP_KIND_Q8_1)
         ? QK
         : QK_K;
     static constexpr int BB = KIND == MARMOT_HIP_KIND_Q4_0 ? Q4_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q4_1                     ? Q4_1_BYTES
         : KIND == MARMOT_HIP_KIND_Q5_0                     ? Q5_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q5_1                     ? Q5_1_BYTES
+        : KIND == MARMOT_HIP_KIND_Q8_1                     ? Q8_1_BYTES
         : KIND == MARMOT_HIP_KIND_Q8_0                     ? Q8_0_BYTES
         : KIND == MARMOT_HIP_KIND_Q2_K                     ? Q2_K_BYTES
         : KIND == MARMOT_HIP_KIND_Q3_K                     ? Q3_K_BYTES

@@ -140,6 +140,9 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
     case MARMOT_HIP_KIND_Q4_0:
         set_route("matvec_q4_0_f16_direct");
         return launch_direct_kind<MARMOT_HIP_KIND_Q4_0>(dev, p, N);
+    case MARMOT_HIP_KIND_Q8_1:
+        set_route("matvec_q8_1_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q8_1>(dev, p, N);
     case MARMOT_HIP_KIND_Q4_1:
         set_route("matvec_q4_1_f16_direct");
         return launch_direct_kind<MARMOT_HIP_KIND_Q4_1>(dev, p, N);

@@ -565,9 +565,12 @@ struct FmtQ3K {
     }
 };
 
-// ------------------------------------------------------------------ Q8_0 x Q8_0
-struct FmtQ80 {
-    static constexpr int BYTES = Q8_0_BYTES;
+// ------------------------------------------------------------------ Q8_0, Q8_1 x Q8_0
+// HDR: bytes in front of the 32 int8 values: the fp16 scale (Q8_0), or the scale and the fp16 sum that Q8_1 carries
+// and neither the dequantizer nor the dot uses (q8_gguf.c:202-213, vec_dot_impl.h:481-510).
+template <int HDR>
+struct FmtQ8x {
+    static constexpr int BYTES = HDR + 32;
     static constexpr int LPB = 1;
     static constexpr int BPW = 64;
     static constexpr int BV = QK;
@@ -597,8 +600,8 @@ struct FmtQ80 {
     }
     __device__ static void load_w(Wt &w, const uint8_t *blk, int) {
         w.s = ld2(blk);
-        w.q0 = ld16(blk + 2);
-        w.q1 = ld16(blk + 18);
+        w.q0 = ld16(blk + HDR);
+        w.q1 = ld16(blk + HDR + 16);
     }
     template <int NC>
     __device__ static void accumulate(const Wt &w, const Act (&a)[NC], float (&acc)[NC], int) {
@@ -611,6 +614,10 @@ struct FmtQ80 {
         }
     }
 };
+
+using FmtQ80 = FmtQ8x<2>;
+using FmtQ81 = FmtQ8x<4>;
+static_assert(FmtQ80::BYTES == Q8_0_BYTES && FmtQ81::BYTES == Q8_1_BYTES, "layouts");
 
 // ------------------------------------------------------------------ Q4_0 x Q8_0
 struct FmtQ40 {
@@ -1397,6 +1404,8 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
         return launch_fmt<FmtQ80>(dev, p, N, K, M, nw, fused ? "matvec_q8_0_q8_0_fused" : "matvec_q8_0_q8_0");
     case MARMOT_HIP_KIND_Q4_0:
         return launch_fmt<FmtQ40>(dev, p, N, K, M, nw, fused ? "matvec_q4_0_q8_0_fused" : "matvec_q4_0_q8_0");
+    case MARMOT_HIP_KIND_Q8_1:
+        return launch_fmt<FmtQ81>(dev, p, N, K, M, nw, fused ? "matvec_q8_1_q8_0_fused" : "matvec_q8_1_q8_0");
     case MARMOT_HIP_KIND_Q4_1:
         return launch_fmt<FmtQ41>(dev, p, N, K, M, nw, fused ? "matvec_q4_1_q8_0_fused" : "matvec_q4_1_q8_0");
     case MARMOT_HIP_KIND_Q5_0:
@@ -1467,6 +1476,9 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
         break;
     case MARMOT_HIP_KIND_Q4_0:
         st = launch_tile<FmtQ40, 8>(dev, p, K, M, nw, "moe_grouped_q4_0_q8_0");
+        break;
+    case MARMOT_HIP_KIND_Q8_1:
+        st = launch_tile<FmtQ81, 8>(dev, p, K, M, nw, "moe_grouped_q8_1_q8_0");
         break;
     case MARMOT_HIP_KIND_Q4_1:
         st = launch_tile<FmtQ41, 8>(dev, p, K, M, nw, "moe_grouped_q4_1_q8_0");

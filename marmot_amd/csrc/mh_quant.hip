@@ -381,6 +381,9 @@ int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_bloc
     case MARMOT_HIP_KIND_Q4_0:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_0>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
+    case MARMOT_HIP_KIND_Q8_1:
+        hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q8_1>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
+        break;
     case MARMOT_HIP_KIND_Q4_1:
         hipLaunchKernelGGL((k_dequantize<MARMOT_HIP_KIND_Q4_1>), grid, block, 0, dev->stream, src, d_out, rows, k, nb);
         break;
@@ -484,6 +487,10 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
         break;
     case MARMOT_HIP_KIND_Q8_0:
         hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q8_0>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q8_1:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q8_1>), grid, block, 0, dev->stream, table, vocab, dim,
                            d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
         break;
     case MARMOT_HIP_KIND_Q5_0:

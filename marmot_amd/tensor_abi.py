@@ -32,6 +32,7 @@ DTYPE_F32, DTYPE_F16, DTYPE_I32, DTYPE_I8, DTYPE_U8, DTYPE_I64 = 0, 1, 3, 5, 6, 
 KIND_GENERIC, KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_K = 0, 1, 5, 9, 10, 11, 12
 KIND_Q4_1, KIND_Q5_0, KIND_Q5_1 = 2, 3, 4
 KIND_Q2_K, KIND_Q3_K = 7, 8
+KIND_Q8_1 = 6
 LAYOUT_GENERIC, LAYOUT_GGUF = 0, 1
 MEMORY_HOST, MEMORY_DEVICE = 0, 1
 BACKEND_HIP = 3
@@ -42,7 +43,7 @@ OP_EMBEDDING = 853
 PREFERENCE_DEFAULT, PREFERENCE_ENABLE, PREFERENCE_DISABLE = 0, 1, 2
 QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q4_1: 2, KIND_Q5_0: 3, KIND_Q5_1: 4, KIND_Q8_0: 5, KIND_Q2_K: 6, KIND_Q3_K: 7, KIND_Q4_K: 8,
-                   KIND_Q5_K: 9, KIND_Q6_K: 10, KIND_Q8_K: 11}
+                   KIND_Q5_K: 9, KIND_Q6_K: 10, KIND_Q8_K: 11, KIND_Q8_1: 12}
 PROFILE_SCALAR = 4
 MATMUL_LAYOUT_NT = 2
 WEIGHT_LAYOUT_SEPARATE = 1
@@ -248,7 +249,7 @@ BACKEND_SYMBOLS = [
     "hip_matmul_quantized_q5_k", "hip_matmul_quantized_q6_k", "hip_matmul_quantized_q4_1",
     "hip_matmul_quantized_q5_0", "hip_matmul_quantized_q5_1", "hip_matmul_qkv_q4_1", "hip_matmul_qkv_q5_0",
     "hip_matmul_qkv_q5_1", "hip_matmul_quantized_q2_k", "hip_matmul_quantized_q3_k", "hip_matmul_qkv_q2_k",
-    "hip_matmul_qkv_q3_k", "hip_matmul_qkv_q4_0", "hip_matmul_qkv_q8_0", "hip_matmul_qkv_q4_k",
+    "hip_matmul_qkv_q3_k", "hip_matmul_quantized_q8_1", "hip_matmul_qkv_q8_1", "hip_matmul_qkv_q4_0", "hip_matmul_qkv_q8_0", "hip_matmul_qkv_q4_k",
     "hip_matmul_qkv_q5_k", "hip_matmul_qkv_q6_k", "hip_embedding_gather", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
 ]
@@ -266,7 +267,7 @@ def bind(lib: C.CDLL) -> C.CDLL:
     lib.marmot_hip_default_preferences.argtypes = [C.POINTER(DeviceCaps), C.POINTER(BackendPreferences)]
     lib.marmot_hip_bc_get_tables.restype = C.c_bool
     lib.marmot_hip_bc_get_tables.argtypes = [C.POINTER(BcTables)]
-    for name in ("q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"):
+    for name in ("q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"):
         fn = getattr(lib, f"hip_matmul_quantized_{name}")
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Epilogue), C.POINTER(Tensor)]

@@ -55,6 +55,11 @@ typedef struct {
     uint8_t qs[16];
 } blk_q5_1; /* 24 B */
 typedef struct {
+    uint16_t scale;
+    uint16_t sum; /* f16(sum(q) * scale): carried, not used by the dequantizer or the dots */
+    int8_t qs[32];
+} blk_q8_1; /* 36 B */
+typedef struct {
     uint16_t d;
     uint16_t dmin;
     uint8_t scales[12];
@@ -97,6 +102,7 @@ _Static_assert(sizeof(blk_q8_0) == 34, "Q8_0");
 _Static_assert(sizeof(blk_q4_1) == 20, "Q4_1");
 _Static_assert(sizeof(blk_q5_0) == 22, "Q5_0");
 _Static_assert(sizeof(blk_q5_1) == 24, "Q5_1");
+_Static_assert(sizeof(blk_q8_1) == 36, "Q8_1");
 _Static_assert(sizeof(blk_q4_k) == 144, "Q4_K");
 _Static_assert(sizeof(blk_q5_k) == 176, "Q5_K");
 _Static_assert(sizeof(blk_q2_k) == 84, "Q2_K");
@@ -111,6 +117,7 @@ size_t mo_block_values(int kind) {
     case MO_KIND_Q5_0:
     case MO_KIND_Q5_1:
     case MO_KIND_Q8_0:
+    case MO_KIND_Q8_1:
         return QK;
     case MO_KIND_Q2_K:
     case MO_KIND_Q3_K:
@@ -134,6 +141,8 @@ size_t mo_block_bytes(int kind) {
         return sizeof(blk_q5_0);
     case MO_KIND_Q5_1:
         return sizeof(blk_q5_1);
+    case MO_KIND_Q8_1:
+        return sizeof(blk_q8_1);
     case MO_KIND_Q8_0:
         return sizeof(blk_q8_0);
     case MO_KIND_Q4_K:
@@ -295,6 +304,39 @@ static void q8_0_quantize_block(const float *values, uint32_t elems, blk_q8_0 *b
 
 /* q8_gguf.c:189-200 */
 static void q8_0_dequantize_block(const blk_q8_0 *block, uint32_t elems, float *out) {
+    const float scale = mo_f16_to_f32(block->scale);
+    for (uint32_t i = 0; i < elems; ++i) {
+        out[i] = (float)block->qs[i] * scale;
+    }
+}
+
+/* q8_gguf.c:155-187: the Q8_0 values plus f16(sum(q) * scale) with the unrounded scale */
+static void q8_1_quantize_block(const float *values, uint32_t elems, blk_q8_1 *block) {
+    blk_q8_0 tmp;
+    q8_0_quantize_block(values, elems, &tmp);
+    float max_abs = 0.0f;
+    for (uint32_t i = 0; i < elems; ++i) {
+        const float a = fabsf(values[i]);
+        if (a > max_abs) {
+            max_abs = a;
+        }
+    }
+    float scale = max_abs <= 0.0f ? 0.0f : max_abs / 127.0f;
+    if (scale < FLT_MIN) {
+        scale = 1.0f;
+    }
+    memset(block, 0, sizeof(*block));
+    block->scale = tmp.scale;
+    memcpy(block->qs, tmp.qs, sizeof(tmp.qs));
+    int32_t sum = 0;
+    for (uint32_t i = 0; i < elems; ++i) {
+        sum += block->qs[i];
+    }
+    block->sum = mo_f32_to_f16((float)sum * scale);
+}
+
+/* q8_gguf.c:202-213 */
+static void q8_1_dequantize_block(const blk_q8_1 *block, uint32_t elems, float *out) {
     const float scale = mo_f16_to_f32(block->scale);
     for (uint32_t i = 0; i < elems; ++i) {
         out[i] = (float)block->qs[i] * scale;
@@ -1411,6 +1453,9 @@ int mo_quantize_rows(int kind, const float *x, size_t rows, size_t k, void *out)
             case MO_KIND_Q4_0:
                 q4_0_quantize_block(src, elems, (blk_q4_0 *)blk);
                 break;
+            case MO_KIND_Q8_1:
+                q8_1_quantize_block(src, elems, (blk_q8_1 *)blk);
+                break;
             case MO_KIND_Q4_1:
                 q4_1_quantize_block(src, elems, (blk_q4_1 *)blk);
                 break;
@@ -1474,6 +1519,9 @@ int mo_dequantize_rows(int kind, const void *blocks, size_t rows, size_t k, floa
             case MO_KIND_Q4_0:
                 q4_0_dequantize_block((const blk_q4_0 *)blk, elems, dst);
                 break;
+            case MO_KIND_Q8_1:
+                q8_1_dequantize_block((const blk_q8_1 *)blk, elems, dst);
+                break;
             case MO_KIND_Q4_1:
                 q4_1_dequantize_block((const blk_q4_1 *)blk, elems, dst);
                 break;
@@ -1519,6 +1567,22 @@ int mo_dequantize_rows(int kind, const void *blocks, size_t rows, size_t k, floa
 /* vec_dot_impl.h:452-479 */
 float mo_vec_dot_q8_0_q8_0(const void *w, const void *a, size_t nblocks) {
     const blk_q8_0 *wb = (const blk_q8_0 *)w;
+    const blk_q8_0 *ab = (const blk_q8_0 *)a;
+    float total = 0.0f;
+    for (size_t b = 0; b < nblocks; ++b) {
+        int32_t sum = 0;
+        for (int i = 0; i < QK; ++i) {
+            sum += (int32_t)wb[b].qs[i] * (int32_t)ab[b].qs[i];
+        }
+        const float block_scale = mo_f16_to_f32(wb[b].scale) * mo_f16_to_f32(ab[b].scale);
+        total += (float)sum * block_scale;
+    }
+    return total;
+}
+
+/* vec_dot_impl.h:481-510 */
+float mo_vec_dot_q8_1_q8_0(const void *w, const void *a, size_t nblocks) {
+    const blk_q8_1 *wb = (const blk_q8_1 *)w;
     const blk_q8_0 *ab = (const blk_q8_0 *)a;
     float total = 0.0f;
     for (size_t b = 0; b < nblocks; ++b) {
@@ -1807,6 +1871,17 @@ float mo_vec_dot_f16(int kind, const void *w, const uint16_t *a, size_t nblocks,
                 total += ((float)wb[b].qs[i]) * scale_w * av;
             }
         }
+    } else if (kind == MO_KIND_Q8_1) { /* vec_dot_impl.h:512-539 */
+        const blk_q8_1 *wb = (const blk_q8_1 *)w;
+        for (size_t b = 0; b < nblocks; ++b) {
+            const float scale_w = mo_f16_to_f32(wb[b].scale);
+            const size_t start = b * QK;
+            const size_t len = (start + QK <= k) ? QK : (k - start);
+            for (size_t i = 0; i < len; ++i) {
+                const float av = mo_f16_to_f32(a[start + i]);
+                total += ((float)wb[b].qs[i]) * scale_w * av;
+            }
+        }
     } else if (kind == MO_KIND_Q4_0) {
         const blk_q4_0 *wb = (const blk_q4_0 *)w;
         for (size_t b = 0; b < nblocks; ++b) {
@@ -2024,6 +2099,8 @@ static dot_fn pick_dot(int kind) {
         return mo_vec_dot_q8_0_q8_0;
     case MO_KIND_Q4_0:
         return mo_vec_dot_q4_0_q8_0;
+    case MO_KIND_Q8_1:
+        return mo_vec_dot_q8_1_q8_0;
     case MO_KIND_Q4_1:
         return mo_vec_dot_q4_1_q8_0;
     case MO_KIND_Q5_0:
@@ -2532,6 +2609,9 @@ int mo_embedding_gather_quantized(
                 break;
             /* Q4_1 tables are decoded in the interleaved order too (:231-240); the reference holds no golden for
              * that case, so it is not restated: NOT_IMPLEMENTED below. Q5_0 / Q5_1 use their dequantizers. */
+            case MO_KIND_Q8_1:
+                q8_1_dequantize_block((const blk_q8_1 *)blk, (uint32_t)count, decoded);
+                break;
             case MO_KIND_Q5_0:
                 q5_0_dequantize_block((const blk_q5_0 *)blk, (uint32_t)count, decoded);
                 break;

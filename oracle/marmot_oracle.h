@@ -39,6 +39,7 @@ enum {
     MO_KIND_Q5_0 = 3,
     MO_KIND_Q5_1 = 4,
     MO_KIND_Q8_0 = 5,
+    MO_KIND_Q8_1 = 6,
     MO_KIND_Q2_K = 7,
     MO_KIND_Q3_K = 8,
     MO_KIND_Q4_K = 9,
@@ -88,6 +89,7 @@ void mo_pack_q8_k(const void *x, int in_dtype, size_t k, void *blocks_out);
 float mo_vec_dot_q8_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q4_1_q8_0(const void *w, const void *a, size_t nblocks);
+float mo_vec_dot_q8_1_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q5_0_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q5_1_q8_0(const void *w, const void *a, size_t nblocks);
 float mo_vec_dot_q2_k_q8_k(const void *w, const void *a, size_t nblocks);

@@ -22,13 +22,16 @@ REF_SO = os.path.join(HERE, "_ref", "libmarmot_ref.so")
 KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_K = 1, 5, 9, 10, 11, 12
 KIND_Q4_1, KIND_Q5_0, KIND_Q5_1 = 2, 3, 4
 KIND_Q2_K, KIND_Q3_K = 7, 8
+KIND_Q8_1 = 6
 KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K,
          "q8_k": KIND_Q8_K, "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1,
-         "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K}
+         "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K, "q8_1": KIND_Q8_1}
 BLOCK_VALUES = {KIND_Q4_0: 32, KIND_Q8_0: 32, KIND_Q4_K: 256, KIND_Q5_K: 256, KIND_Q6_K: 256, KIND_Q8_K: 256,
-                KIND_Q4_1: 32, KIND_Q5_0: 32, KIND_Q5_1: 32, KIND_Q2_K: 256, KIND_Q3_K: 256}
+                KIND_Q4_1: 32, KIND_Q5_0: 32, KIND_Q5_1: 32, KIND_Q2_K: 256, KIND_Q3_K: 256,
+                KIND_Q8_1: 32}
 BLOCK_BYTES = {KIND_Q4_0: 18, KIND_Q8_0: 34, KIND_Q4_K: 144, KIND_Q5_K: 176, KIND_Q6_K: 210, KIND_Q8_K: 292,
-               KIND_Q4_1: 20, KIND_Q5_0: 22, KIND_Q5_1: 24, KIND_Q2_K: 84, KIND_Q3_K: 110}
+               KIND_Q4_1: 20, KIND_Q5_0: 22, KIND_Q5_1: 24, KIND_Q2_K: 84, KIND_Q3_K: 110,
+               KIND_Q8_1: 36}
 DT_F32, DT_F16 = 0, 1
 DT_I32, DT_I64 = 3, 11  # marmot_dtype_t values of the position tensors the rotary epilogue accepts
 ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_YARN, ROPE_SCALING_LONGROPE = 0, 1, 2, 3
@@ -85,7 +88,7 @@ class Oracle:
             f.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
         for n in ("mo_vec_dot_q8_0_q8_0", "mo_vec_dot_q4_0_q8_0", "mo_vec_dot_q4_k_q8_k", "mo_vec_dot_q5_k_q8_k",
                   "mo_vec_dot_q6_k_q8_k", "mo_vec_dot_q4_1_q8_0", "mo_vec_dot_q5_0_q8_0", "mo_vec_dot_q5_1_q8_0",
-                  "mo_vec_dot_q2_k_q8_k", "mo_vec_dot_q3_k_q8_k"):
+                  "mo_vec_dot_q2_k_q8_k", "mo_vec_dot_q3_k_q8_k", "mo_vec_dot_q8_1_q8_0"):
             f = getattr(L, n)
             f.restype = C.c_float
             f.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
@@ -183,6 +186,7 @@ class Oracle:
             KIND_Q5_1: self.L.mo_vec_dot_q5_1_q8_0,
             KIND_Q2_K: self.L.mo_vec_dot_q2_k_q8_k,
             KIND_Q3_K: self.L.mo_vec_dot_q3_k_q8_k,
+            KIND_Q8_1: self.L.mo_vec_dot_q8_1_q8_0,
             KIND_Q6_K: self.L.mo_vec_dot_q6_k_q8_k,
         }[kind]
         w = np.ascontiguousarray(w, dtype=np.uint8)
@@ -368,11 +372,11 @@ class RefLib:
             f.restype = None
             f.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
         for n in ("q8_0_q8_0", "q4_0_q8_0", "q4_k_q8_k", "q5_k_q8_k", "q6_k_q8_k", "q4_1_q8_0", "q5_0_q8_0",
-                  "q5_1_q8_0", "q2_k_q8_k", "q3_k_q8_k"):
+                  "q5_1_q8_0", "q2_k_q8_k", "q3_k_q8_k", "q8_1_q8_0"):
             f = getattr(L, f"cpu_vec_dot_{n}_scalar")
             f.restype = C.c_float
             f.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
-        for n in ("q8_0", "q4_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k"):
+        for n in ("q8_0", "q4_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q8_1"):
             f = getattr(L, f"cpu_vec_dot_{n}_f16_scalar")
             f.restype = C.c_float
             f.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]
@@ -432,14 +436,15 @@ class RefLib:
     def vec_dot(self, kind: int, w: np.ndarray, a: np.ndarray, nblocks: int) -> float:
         name = {KIND_Q8_0: "q8_0_q8_0", KIND_Q4_0: "q4_0_q8_0", KIND_Q4_K: "q4_k_q8_k", KIND_Q5_K: "q5_k_q8_k",
                 KIND_Q6_K: "q6_k_q8_k", KIND_Q4_1: "q4_1_q8_0", KIND_Q5_0: "q5_0_q8_0", KIND_Q5_1: "q5_1_q8_0",
-                KIND_Q2_K: "q2_k_q8_k", KIND_Q3_K: "q3_k_q8_k"}[kind]
+                KIND_Q2_K: "q2_k_q8_k", KIND_Q3_K: "q3_k_q8_k", KIND_Q8_1: "q8_1_q8_0"}[kind]
         w = np.ascontiguousarray(w, dtype=np.uint8)
         a = np.ascontiguousarray(a, dtype=np.uint8)
         return float(getattr(self.L, f"cpu_vec_dot_{name}_scalar")(_ptr(w), _ptr(a), nblocks))
 
     def vec_dot_f16(self, kind: int, w: np.ndarray, a: np.ndarray, k: int) -> float:
         name = {KIND_Q8_0: "q8_0", KIND_Q4_0: "q4_0", KIND_Q4_K: "q4_k", KIND_Q5_K: "q5_k", KIND_Q6_K: "q6_k",
-                KIND_Q4_1: "q4_1", KIND_Q5_0: "q5_0", KIND_Q5_1: "q5_1", KIND_Q2_K: "q2_k", KIND_Q3_K: "q3_k"}[kind]
+                KIND_Q4_1: "q4_1", KIND_Q5_0: "q5_0", KIND_Q5_1: "q5_1", KIND_Q2_K: "q2_k", KIND_Q3_K: "q3_k",
+                KIND_Q8_1: "q8_1"}[kind]
         w = np.ascontiguousarray(w, dtype=np.uint8)
         a = np.ascontiguousarray(a, dtype=np.float16)
         nb = (k + BLOCK_VALUES[kind] - 1) // BLOCK_VALUES[kind]

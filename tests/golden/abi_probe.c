@@ -55,6 +55,7 @@ int main(void) {
     VAL(MARMOT_QSCHEME_Q8_K); VAL(MARMOT_QSCHEME_Q5_K);
     VAL(MARMOT_QSCHEME_Q4_1); VAL(MARMOT_QSCHEME_Q5_0); VAL(MARMOT_QSCHEME_Q5_1);
     VAL(MARMOT_QSCHEME_Q2_K); VAL(MARMOT_QSCHEME_Q3_K); VAL(MARMOT_QUANT_KIND_Q2_K); VAL(MARMOT_QUANT_KIND_Q3_K);
+    VAL(MARMOT_QSCHEME_Q8_1); VAL(MARMOT_QUANT_KIND_Q8_1);
     VAL(MARMOT_MATMUL_LAYOUT_NT); VAL(MARMOT_WEIGHT_LAYOUT_SEPARATE); VAL(MARMOT_STRIDE_MODE_CONTIGUOUS);
     VAL(MARMOT_EPILOGUE_BIAS); VAL(MARMOT_KERNEL_INVALID);
     VAL(MARMOT_BC_SCHEMA_TOPK); VAL(MARMOT_BC_SCHEMA_MOE_EXPERTS); VAL(MARMOT_BC_SCHEMA_MATMUL);

@@ -44,6 +44,8 @@ int main(void) {
     EMIT(g_llama_q5_0_dequant, "f4");
     EMIT(g_llama_q5_1, "u1");
     EMIT(g_llama_q5_1_dequant, "f4");
+    EMIT(g_llama_q8_1, "u1");
+    EMIT(g_llama_q8_1_dequant, "f4");
     EMIT(g_llama_q8_0, "u1");
     EMIT(g_llama_q8_0_dequant, "f4");
     EMIT(g_llama_q2_k, "u1");
@@ -66,6 +68,7 @@ int main(void) {
     EMIT(g_vec_dot_q8_k_activations, "u1");
     EMIT(g_vec_dot_q4_0_weights, "u1");
     EMIT(g_vec_dot_q8_0_weights, "u1");
+    EMIT(g_vec_dot_q8_1_weights, "u1");
     EMIT(g_vec_dot_q4_1_weights, "u1");
     EMIT(g_vec_dot_q5_0_weights, "u1");
     EMIT(g_vec_dot_q5_1_weights, "u1");
@@ -76,6 +79,7 @@ int main(void) {
     EMIT(g_vec_dot_q6_k_weights, "u1");
     EMIT_SCALAR(g_vec_dot_q4_0_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q8_0_q8_0_expected, "f4");
+    EMIT_SCALAR(g_vec_dot_q8_1_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q4_1_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q5_0_q8_0_expected, "f4");
     EMIT_SCALAR(g_vec_dot_q5_1_q8_0_expected, "f4");
@@ -93,7 +97,8 @@ int main(void) {
             c->kind != MARMOT_QUANT_KIND_Q4_K && c->kind != MARMOT_QUANT_KIND_Q5_K &&
             c->kind != MARMOT_QUANT_KIND_Q6_K && c->kind != MARMOT_QUANT_KIND_Q4_1 &&
             c->kind != MARMOT_QUANT_KIND_Q5_0 && c->kind != MARMOT_QUANT_KIND_Q5_1 &&
-            c->kind != MARMOT_QUANT_KIND_Q2_K && c->kind != MARMOT_QUANT_KIND_Q3_K) {
+            c->kind != MARMOT_QUANT_KIND_Q2_K && c->kind != MARMOT_QUANT_KIND_Q3_K &&
+            c->kind != MARMOT_QUANT_KIND_Q8_1) {
             continue;
         }
         char name[128];

@@ -54,7 +54,7 @@ def dump_reference_goldens():
 def dump_ref_gaussian():
     sys.path.insert(0, ROOT)
     from oracle.pyoracle import (BLOCK_VALUES, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0,
-                                 KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K, RefLib)
+                                 KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_1, KIND_Q8_K, RefLib)
 
     ref = RefLib()
     out = {}
@@ -62,7 +62,7 @@ def dump_ref_gaussian():
     for name, kind, seed in (("q8_0", KIND_Q8_0, 100), ("q4_0", KIND_Q4_0, 101), ("q4_k", KIND_Q4_K, 102),
                              ("q6_k", KIND_Q6_K, 103), ("q5_k", KIND_Q5_K, 105),
                              ("q4_1", KIND_Q4_1, 106), ("q5_0", KIND_Q5_0, 107), ("q5_1", KIND_Q5_1, 108),
-                             ("q2_k", KIND_Q2_K, 109), ("q3_k", KIND_Q3_K, 110)):
+                             ("q2_k", KIND_Q2_K, 109), ("q3_k", KIND_Q3_K, 110), ("q8_1", KIND_Q8_1, 111)):
         rng = np.random.default_rng(seed)
         rows = 16  # 16 rows x 1024 -> 64 K-quant super-blocks (512 legacy blocks) per format
         w = (rng.standard_normal((rows, K), dtype=np.float32) * np.float32(0.02)).astype(np.float32)
@@ -95,7 +95,7 @@ def dump_ref_gaussian():
     for name, kind, k in (("q8_0", KIND_Q8_0, 70), ("q4_0", KIND_Q4_0, 70), ("q4_k", KIND_Q4_K, 300),
                           ("q6_k", KIND_Q6_K, 300), ("q5_k", KIND_Q5_K, 300),
                           ("q4_1", KIND_Q4_1, 70), ("q5_0", KIND_Q5_0, 70), ("q5_1", KIND_Q5_1, 70),
-                          ("q2_k", KIND_Q2_K, 300), ("q3_k", KIND_Q3_K, 300)):
+                          ("q2_k", KIND_Q2_K, 300), ("q3_k", KIND_Q3_K, 300), ("q8_1", KIND_Q8_1, 70)):
         w = (rng.standard_normal((2, k), dtype=np.float32) * np.float32(0.02)).astype(np.float32)
         blocks = ref.quantize(kind, w)
         out[f"{name}_tail_w"] = w

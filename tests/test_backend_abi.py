@@ -86,7 +86,7 @@ def test_ctypes_structs_match_layout(golden_layout):
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q6_K] == golden_layout["MARMOT_QSCHEME_Q6_K"]
     assert ta.QSCHEME_OF_KIND[ta.KIND_Q5_K] == golden_layout["MARMOT_QSCHEME_Q5_K"]
     assert ta.KIND_Q5_K == golden_layout["MARMOT_QUANT_KIND_Q5_K"]
-    for name in ("Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K"):
+    for name in ("Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K", "Q8_1"):
         kind = getattr(ta, f"KIND_{name}")
         assert kind == golden_layout[f"MARMOT_QUANT_KIND_{name}"]
         assert ta.QSCHEME_OF_KIND[kind] == golden_layout[f"MARMOT_QSCHEME_{name}"]
@@ -139,7 +139,8 @@ def _query(lib, sig):
 
 def test_query_kernel_matmul_rules(lib):
     expect_op = {ta.KIND_Q4_0: 1, ta.KIND_Q8_0: 2, ta.KIND_Q4_K: 3, ta.KIND_Q6_K: 4, ta.KIND_Q5_K: 20, ta.KIND_Q4_1: 24,
-                 ta.KIND_Q5_0: 28, ta.KIND_Q5_1: 32, ta.KIND_Q2_K: 36, ta.KIND_Q3_K: 40}
+                 ta.KIND_Q5_0: 28, ta.KIND_Q5_1: 32, ta.KIND_Q2_K: 36, ta.KIND_Q3_K: 40,
+                 ta.KIND_Q8_1: 44}
     for kind, op in expect_op.items():
         sel = _query(lib, _sig(kind=kind))
         assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
@@ -162,7 +163,7 @@ def test_query_kernel_matmul_rules(lib):
     assert not sel.supported and b"Q5_K" in sel.fallback_reason
     # unsupported scheme, layout, weight layout, stride mode, epilogue, variant
     assert not _query(lib, _sig(kind=ta.KIND_Q8_K)).supported
-    s = _sig(); s.qscheme_id = 12  # Q8_1
+    s = _sig(); s.qscheme_id = 13  # beyond the enumeration
     assert not _query(lib, s).supported
     for kind in (ta.KIND_Q2_K, ta.KIND_Q3_K):
         assert not _query(lib, _sig(kind=kind, inp=ta.DTYPE_F16)).supported
@@ -200,7 +201,7 @@ def test_query_kernel_cost_model(lib):
 def test_query_kernel_other_ops(lib):
     for kind, op in {ta.KIND_Q4_0: 5, ta.KIND_Q8_0: 6, ta.KIND_Q4_K: 7, ta.KIND_Q6_K: 8, ta.KIND_Q5_K: 21,
                      ta.KIND_Q4_1: 25, ta.KIND_Q5_0: 29, ta.KIND_Q5_1: 33, ta.KIND_Q2_K: 37,
-                     ta.KIND_Q3_K: 41}.items():
+                     ta.KIND_Q3_K: 41, ta.KIND_Q8_1: 45}.items():
         assert _query(lib, _sig(op=ta.OP_MOE_EXPERTS, kind=kind)).op_index == op
     assert not _query(lib, _sig(op=ta.OP_MOE_EXPERTS, inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).supported
     assert _query(lib, _sig(op=ta.OP_TOPK)).op_index == 9
@@ -219,7 +220,7 @@ def test_query_kernel_qkv_rules(lib, golden_layout):
     for op_id in (ta.OP_QKV_PROJECTION, ta.OP_QKV_SHARED_INPUT, ta.OP_QKV_ROPE):
         for kind, op in {ta.KIND_Q4_0: 12, ta.KIND_Q8_0: 13, ta.KIND_Q4_K: 14, ta.KIND_Q6_K: 15,
                          ta.KIND_Q5_K: 22, ta.KIND_Q4_1: 26, ta.KIND_Q5_0: 30, ta.KIND_Q5_1: 34,
-                         ta.KIND_Q2_K: 38, ta.KIND_Q3_K: 42}.items():
+                         ta.KIND_Q2_K: 38, ta.KIND_Q3_K: 42, ta.KIND_Q8_1: 46}.items():
             for dt in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, _sig(op=op_id, kind=kind, inp=dt, out=dt, N=4, K=4096, M=4096))
                 assert sel.supported and sel.op_index == op and sel.kernel_id == 0x4000 + op
@@ -262,7 +263,8 @@ def test_query_kernel_embedding_rules(lib):
         s.weight_layout = ta.WEIGHT_LAYOUT_SEPARATE
         return s
     for kind, op in ((ta.KIND_Q4_0, 16), (ta.KIND_Q8_0, 17), (ta.KIND_Q4_K, 18), (ta.KIND_Q6_K, 19),
-                     (ta.KIND_Q5_K, 23), (ta.KIND_Q5_0, 31), (ta.KIND_Q5_1, 35), (ta.KIND_Q2_K, 39), (ta.KIND_Q3_K, 43)):
+                     (ta.KIND_Q5_K, 23), (ta.KIND_Q5_0, 31), (ta.KIND_Q5_1, 35), (ta.KIND_Q2_K, 39), (ta.KIND_Q3_K, 43),
+                     (ta.KIND_Q8_1, 47)):
         for ids in (ta.DTYPE_I32, ta.DTYPE_I64):
             for out in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, sig(kind, ids, out))
@@ -278,7 +280,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 44
+    assert t.op_count == 48
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -298,8 +300,9 @@ def test_bytecode_tables(lib, golden_layout):
     assert sizes[12:16] == [struct.calcsize("<7HII3H")] * 4
     assert sizes[16:20] == [struct.calcsize("<3HIfI3B")] * 4 == [21] * 4
     # Q5_K was added behind the four original kinds: one op per family
-    # kinds added behind the four original ones (Q5_K, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K): four consecutive ops each
-    for base in (20, 24, 28, 32, 36, 40):
+    # kinds added behind the four original ones (Q5_K, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q8_1): four consecutive ops
+    # each
+    for base in (20, 24, 28, 32, 36, 40, 44):
         assert schema[base:base + 4] == [golden_layout[f"MARMOT_BC_SCHEMA_{n}"]
                                          for n in ("MATMUL", "MOE_EXPERTS", "QKV", "EMBEDDING")]
         assert sizes[base:base + 4] == [sizes[1], sizes[5], sizes[12], sizes[16]]

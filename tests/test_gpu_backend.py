@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from marmot_amd import tensor_abi as ta
-from oracle.pyoracle import (KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
+from oracle.pyoracle import (KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
                              KIND_Q8_K, row_bytes)
 from tests.test_oracle_moe import make_experts
 from tests.util import assert_matmul_parity, assert_moe_parity, bits, gaussian, quantize_weights
@@ -32,7 +32,7 @@ def _linear(ctx, kind, wq, M, K, x, bias=None, out_dtype=ta.DTYPE_F32):
         ep.bias = bt.ptr
     fn = getattr(ctx.lib, {KIND_Q4_0: "hip_matmul_quantized_q4_0", KIND_Q8_0: "hip_matmul_quantized_q8_0",
                            KIND_Q4_1: "hip_matmul_quantized_q4_1", KIND_Q5_0: "hip_matmul_quantized_q5_0",
-                           KIND_Q5_1: "hip_matmul_quantized_q5_1", KIND_Q2_K: "hip_matmul_quantized_q2_k",
+                           KIND_Q5_1: "hip_matmul_quantized_q5_1", KIND_Q2_K: "hip_matmul_quantized_q2_k", KIND_Q8_1: "hip_matmul_quantized_q8_1",
                            KIND_Q3_K: "hip_matmul_quantized_q3_k",
                            KIND_Q4_K: "hip_matmul_quantized_q4_k", KIND_Q5_K: "hip_matmul_quantized_q5_k",
                            KIND_Q6_K: "hip_matmul_quantized_q6_k"}[kind])
@@ -46,7 +46,7 @@ def _linear(ctx, kind, wq, M, K, x, bias=None, out_dtype=ta.DTYPE_F32):
     return st, xt, wt, yt
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q2_K, KIND_Q3_K,
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q8_1, KIND_Q2_K, KIND_Q3_K,
                                   KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
 def test_impl_matmul_matches_oracle(ctx, oracle, kind):
     print(f"backend impl matmul kind={kind}", flush=True)
@@ -283,7 +283,7 @@ def _qkv_tensors(kind, ws, M, K, x, biases):
     return xt, wts, outs, bts
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q2_K, KIND_Q3_K,
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q8_1, KIND_Q2_K, KIND_Q3_K,
                                   KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 def test_impl_qkv_matches_oracle(ctx, oracle, kind, dtype):
@@ -302,7 +302,8 @@ def test_impl_qkv_matches_oracle(ctx, oracle, kind, dtype):
     desc.separate.bq, desc.separate.bv = bts[0].ptr, bts[2].ptr
     desc.out_q, desc.out_k, desc.out_v = (o.ptr for o in outs)
     name = {KIND_Q4_0: "q4_0", KIND_Q8_0: "q8_0", KIND_Q4_K: "q4_k", KIND_Q5_K: "q5_k", KIND_Q6_K: "q6_k",
-            KIND_Q4_1: "q4_1", KIND_Q5_0: "q5_0", KIND_Q5_1: "q5_1", KIND_Q2_K: "q2_k", KIND_Q3_K: "q3_k"}[kind]
+            KIND_Q4_1: "q4_1", KIND_Q5_0: "q5_0", KIND_Q5_1: "q5_1", KIND_Q2_K: "q2_k", KIND_Q3_K: "q3_k",
+            KIND_Q8_1: "q8_1"}[kind]
     st = getattr(ctx.lib, f"hip_matmul_qkv_{name}")(ctx.device_ctx, C.byref(desc))
     assert st == ta.SUCCESS, ctx.last_error()
     tol = 1e-3 if dtype == np.float32 else 2e-3
@@ -315,7 +316,7 @@ def test_impl_qkv_matches_oracle(ctx, oracle, kind, dtype):
     sel = ctx.query(ctx.qkv_signature(xt, wts[0], outs[0], bias=True))
     assert sel.supported and sel.op_index == {KIND_Q4_0: 12, KIND_Q8_0: 13, KIND_Q4_K: 14, KIND_Q6_K: 15, KIND_Q5_K: 22,
                                               KIND_Q4_1: 26, KIND_Q5_0: 30, KIND_Q5_1: 34, KIND_Q2_K: 38,
-                                              KIND_Q3_K: 42}[kind]
+                                              KIND_Q3_K: 42, KIND_Q8_1: 46}[kind]
     for o in outs:
         o.array[...] = 0
         ctx.host_changed(o)
@@ -438,7 +439,7 @@ def test_program_qkv_with_rotary_epilogue(ctx, oracle, dtype):
 
 
 # ---------------------------------------------------------------- embedding gather
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K,
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K,
                                   KIND_Q6_K])
 def test_impl_and_program_embedding_gather(ctx, oracle, kind):
     """marmot_embedding_gather on a quantized table: the impl function with a descriptor and the EMBEDDING bytecode
@@ -466,7 +467,8 @@ def test_impl_and_program_embedding_gather(ctx, oracle, kind):
     i32 = ta.HostTensor.dense(ids.astype(np.int32).reshape(-1))
     sel = ctx.query(ctx.embedding_signature(tt, i32, o16))
     assert sel.supported and sel.op_index == {KIND_Q4_0: 16, KIND_Q8_0: 17, KIND_Q4_K: 18, KIND_Q6_K: 19, KIND_Q5_K: 23,
-                                              KIND_Q5_0: 31, KIND_Q5_1: 35, KIND_Q2_K: 39, KIND_Q3_K: 43}[kind]
+                                              KIND_Q5_0: 31, KIND_Q5_1: 35, KIND_Q2_K: 39, KIND_Q3_K: 43,
+                                              KIND_Q8_1: 47}[kind]
     before = ctx.residency().upload_bytes
     prog = ta.Program()
     prog.embedding(sel.op_index, tt, i32, o16, scale=0.25, padding_id=-1, bounds_check=False)

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from marmot_amd import capi
-from oracle.pyoracle import KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.test_oracle_embedding import load_golden
 from tests.util import bits, random_valid_blocks
 
@@ -27,7 +27,7 @@ def test_reference_q4_0_embedding_golden(hip):
     assert np.max(np.abs(got - expected)) <= 1e-6
 
 
-@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K,
+@pytest.mark.parametrize("kind", [KIND_Q4_0, KIND_Q5_0, KIND_Q5_1, KIND_Q8_0, KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K,
                                   KIND_Q6_K])
 @pytest.mark.parametrize("ids_dtype", [np.int32, np.int64])
 def test_gather_is_bit_exact(hip, oracle, kind, ids_dtype):

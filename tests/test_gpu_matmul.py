@@ -2,13 +2,14 @@
 import numpy as np
 import pytest
 
-from oracle.pyoracle import BLOCK_VALUES, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import BLOCK_VALUES, KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.util import assert_matmul_parity, bits, gaussian, parity_metrics, quantize_weights, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
 KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K,
-         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K}
+         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K,
+         "q8_1": KIND_Q8_1}
 THREADS = 16
 
 
@@ -21,7 +22,7 @@ def hip():
     b.close()
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q2_K", "Q3_K", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q8_1", "Q2_K", "Q3_K", "Q4_K", "Q5_K", "Q6_K"])
 def test_reference_matmul_goldens_fp32(hip, ref_goldens, name):
     """The reference's own golden cases (tests/backend/golden_matmul_llama.h), its own tolerance."""
     kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
@@ -32,7 +33,7 @@ def test_reference_matmul_goldens_fp32(hip, ref_goldens, name):
     assert np.all(np.abs(got - exp) <= 2e-5 + 5e-5 * np.abs(exp)), (got, exp)
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q4_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q8_1", "Q4_K"])
 def test_reference_matmul_goldens_fp16(hip, ref_goldens, name):
     kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
     w = ref_goldens[f"matmul_{name}_weight"]
@@ -92,7 +93,7 @@ def test_config2_kquant_decode_full_size(hip, oracle, name, M, K):
     d_w.free()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("N", [1, 2, 3, 5, 8, 11, 16, 19])
 def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
     """All column-tile widths (8/4/2/1) and M not a multiple of the rows-per-workgroup."""
@@ -105,7 +106,7 @@ def test_linear_batches_and_ragged_rows(hip, oracle, name, N):
     assert_matmul_parity(got, ref, what=f"{name} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("K", [256, 512, 768, 1280, 8192, 11008, 28672])
 def test_linear_k_sweep(hip, oracle, name, K):
     """Rows shorter than one wave-load, rows needing several wavefronts, and long rows."""
@@ -119,7 +120,7 @@ def test_linear_k_sweep(hip, oracle, name, K):
         assert_matmul_parity(got, ref, what=f"{name} K={K} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_linear_ragged_k(hip, oracle, name):
     """K not a multiple of the block: weight and activation tails are zero-padded blocks."""
     kind = KINDS[name]
@@ -133,7 +134,7 @@ def test_linear_ragged_k(hip, oracle, name):
     assert_matmul_parity(got, ref, what=f"{name} ragged K={K}")
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_linear_random_block_bytes(hip, oracle, name):
     """Weights that are arbitrary block bytes (all 6-bit scale / min patterns, negative Q6_K scales)."""
     kind = KINDS[name]
@@ -159,7 +160,7 @@ def test_linear_bias_epilogue(hip, oracle, name):
     assert np.max(d) <= 1e-5 * max(1.0, np.abs(ref).max())
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q4_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q4_k"])
 def test_linear_fp16_direct_small_batch(hip, oracle, name):
     """fp16 activations take the direct route (no activation quantization) like the CPU reference."""
     kind = KINDS[name]
@@ -201,7 +202,7 @@ def test_linear_error_behaviour(hip, oracle):
         hip.linear(x, blocks, KIND_Q4_K, M, out_dtype=np.float16)
     assert e.value.code == -6
     with pytest.raises(MarmotHipError) as e:  # unsupported quant kind -> NOT_IMPLEMENTED (fallback signal)
-        hip.linear_d(6, hip.to_device(blocks), hip.to_device(x), 0, 1, K, M, hip.alloc(64), 0)  # Q8_1
+        hip.linear_d(12, hip.to_device(blocks), hip.to_device(x), 0, 1, K, M, hip.alloc(64), 0)  # Q8_K weights
     assert e.value.code == -8
     for kind in (KIND_Q2_K, KIND_Q3_K, KIND_Q5_K):  # their fp16 direct dots in the reference are unsound: declined
         with pytest.raises(MarmotHipError) as e:
@@ -215,7 +216,7 @@ def test_linear_error_behaviour(hip, oracle):
     hip.synchronize()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_loader_consumer_matvec_equals_register_streaming_matvec(hip, oracle, name, monkeypatch):
     """The loader/consumer matvec (weights through an LDS ring) keeps the lane mapping and the reduction order of the
     register-streaming kernel: the two must agree bit for bit, on whole and ragged row groups, one and two K slices

@@ -8,13 +8,14 @@ import numpy as np
 import pytest
 
 from marmot_amd import capi
-from oracle.pyoracle import KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
+from oracle.pyoracle import KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0
 from tests.util import assert_matmul_parity, gaussian
 
 pytestmark = pytest.mark.gpu
 
 KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K,
-         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K}
+         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K,
+         "q8_1": KIND_Q8_1}
 
 
 @pytest.fixture(scope="module")
@@ -30,7 +31,7 @@ def _weights(oracle, kind, M, K, seed):
     return [oracle.quantize(kind, gaussian(seed + i, (M, K), 0.02)) for i in range(3)]
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q2_K", "Q3_K", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q8_1", "Q2_K", "Q3_K", "Q4_K", "Q5_K", "Q6_K"])
 def test_reference_qkv_test_case(hip, ref_goldens, name):
     """tests/backend/test_backend_matmul.c:936-1032: the matmul golden weight as q, k and v."""
     kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
@@ -41,7 +42,7 @@ def test_reference_qkv_test_case(hip, ref_goldens, name):
         assert np.all(np.abs(out - exp) <= 2e-5 + 5e-5 * np.abs(exp)), np.abs(out - exp).max()
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("N", [1, 2, 4, 5, 8, 16, 33])
 def test_qkv_fp32_all_routes(hip, oracle, name, N):
     kind = KINDS[name]

@@ -2,14 +2,15 @@
 import numpy as np
 import pytest
 
-from oracle.pyoracle import (BLOCK_BYTES, BLOCK_VALUES, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K,
+from oracle.pyoracle import (BLOCK_BYTES, BLOCK_VALUES, KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q5_0, KIND_Q5_1, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0, KIND_Q8_K,
                              row_bytes)
 from tests.util import bits, gaussian, quantize_weights, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
 KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K,
-         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K}
+         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K,
+         "q8_1": KIND_Q8_1}
 
 
 @pytest.fixture(scope="module")
@@ -29,7 +30,7 @@ def test_device_is_gfx950(hip):
     assert caps["num_compute_units"] >= 200
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 @pytest.mark.parametrize("rows,k", [(3, 1024), (2, 300), (1, 70), (64, 4096)])
 def test_dequantize_bit_exact_quantized_gaussian(hip, oracle, name, rows, k):
     print(f"dequant {name} rows={rows} k={k}", flush=True)
@@ -41,7 +42,7 @@ def test_dequantize_bit_exact_quantized_gaussian(hip, oracle, name, rows, k):
     assert np.array_equal(bits(got), bits(exp))
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_dequantize_bit_exact_random_bytes(hip, oracle, name):
     """Every scale / nibble pattern, not only what a quantizer emits."""
     print(f"dequant random bytes {name}", flush=True)
@@ -60,7 +61,7 @@ def test_dequantize_q8_k_and_golden_blocks(hip, oracle, ref_goldens):
     assert np.array_equal(bits(hip.dequantize(KIND_Q8_K, blocks, 512)), bits(oracle.dequantize(KIND_Q8_K, blocks, 512)))
     # the reference-held golden blocks: same tolerance as the reference's own test
     for name, tol in (("q4_0", 5e-4), ("q8_0", 5e-4), ("q4_k", 6e-4), ("q5_k", 6e-4), ("q6_k", 6e-4),
-                      ("q4_1", 5e-4), ("q5_0", 5e-4), ("q5_1", 5e-4), ("q2_k", 6e-4), ("q3_k", 6e-4)):
+                      ("q4_1", 5e-4), ("q5_0", 5e-4), ("q5_1", 5e-4), ("q2_k", 6e-4), ("q3_k", 6e-4), ("q8_1", 5e-4)):
         exp = ref_goldens[f"g_llama_{name}_dequant"]
         got = hip.dequantize(KINDS[name], ref_goldens[f"g_llama_{name}"], exp.size)[0]
         assert np.max(np.abs(got - exp)) <= tol

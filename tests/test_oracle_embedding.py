@@ -12,7 +12,7 @@ import os
 import numpy as np
 import pytest
 
-from oracle.pyoracle import (KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
+from oracle.pyoracle import (KIND_Q8_1, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K, KIND_Q6_K, KIND_Q8_0,
                              row_bytes)
 from tests.util import bits, gaussian, random_valid_blocks
 
@@ -45,7 +45,7 @@ def test_q4_1_tables_are_declined(oracle):
 
 
 @pytest.mark.parametrize("kind", [KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q5_0, KIND_Q5_1, KIND_Q2_K,
-                                  KIND_Q3_K])
+                                  KIND_Q3_K, KIND_Q8_1])
 def test_gathered_rows_are_dequantized_rows(oracle, kind):
     rng = np.random.default_rng(800 + kind)
     vocab, dim = 37, 768 if kind in (KIND_Q2_K, KIND_Q3_K, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K) else 96

@@ -12,11 +12,12 @@ import numpy as np
 import pytest
 
 from oracle.pyoracle import (BLOCK_BYTES, BLOCK_VALUES, KIND_Q2_K, KIND_Q3_K, KIND_Q4_0, KIND_Q4_1, KIND_Q4_K, KIND_Q5_0, KIND_Q5_1, KIND_Q5_K,
-                             KIND_Q6_K, KIND_Q8_0, KIND_Q8_K,
+                             KIND_Q6_K, KIND_Q8_0, KIND_Q8_1, KIND_Q8_K,
                              row_bytes)
 
 KINDS = {"q4_0": KIND_Q4_0, "q8_0": KIND_Q8_0, "q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K,
-         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K}
+         "q4_1": KIND_Q4_1, "q5_0": KIND_Q5_0, "q5_1": KIND_Q5_1, "q2_k": KIND_Q2_K, "q3_k": KIND_Q3_K,
+         "q8_1": KIND_Q8_1}
 
 
 def bits(a):
@@ -63,7 +64,7 @@ def np_q6_k_ints(blocks: np.ndarray):
 
 
 # ---------------------------------------------------------------- 1. reference-held goldens
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q8_1"])
 def test_quantizer_bytes_match_reference_golden(oracle, ref_goldens, name):
     kind = KINDS[name]
     src = ref_goldens["g_llama_test_input"]
@@ -86,7 +87,7 @@ def test_q8_k_bytes_match_reference_golden(oracle, ref_goldens):
 
 
 @pytest.mark.parametrize("name,tol", [("q4_0", 5e-4), ("q8_0", 5e-4), ("q4_k", 6e-4), ("q5_k", 6e-4), ("q6_k", 6e-4), ("q4_1", 5e-4), ("q5_0", 5e-4),
-                                      ("q5_1", 5e-4), ("q2_k", 6e-4), ("q3_k", 6e-4)])
+                                      ("q5_1", 5e-4), ("q2_k", 6e-4), ("q3_k", 6e-4), ("q8_1", 5e-4)])
 def test_dequant_matches_reference_golden(oracle, ref_goldens, name, tol):
     kind = KINDS[name]
     exp = ref_goldens[f"g_llama_{name}_dequant"]
@@ -97,7 +98,7 @@ def test_dequant_matches_reference_golden(oracle, ref_goldens, name, tol):
     assert np.max(np.abs(got - exp)) <= 1e-6 * max(1.0, np.max(np.abs(exp)))
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q8_1"])
 def test_vec_dot_matches_reference_golden(oracle, ref_goldens, name):
     kind = KINDS[name]
     act = ref_goldens["g_vec_dot_q8_k_activations" if BLOCK_VALUES[kind] == 256 else "g_vec_dot_q8_0_activations"]
@@ -132,7 +133,7 @@ def test_activation_packers_match_reference_golden(oracle, ref_goldens):
     assert scale.shape == (8, 1)
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K", "Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K", "Q4_1", "Q5_0", "Q5_1", "Q2_K", "Q3_K", "Q8_1"])
 @pytest.mark.parametrize("fp16_input", [False, True])
 def test_matmul_matches_reference_golden(oracle, ref_goldens, name, fp16_input):
     kind, N, K, M = (int(v) for v in ref_goldens[f"matmul_{name}_dims"])
@@ -152,7 +153,7 @@ def test_matmul_matches_reference_golden(oracle, ref_goldens, name, fp16_input):
 
 
 # ---------------------------------------------------------------- 2. reference leaf code on Gaussian rows
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q8_1"])
 def test_oracle_equals_reference_code_on_gaussian_fixture(oracle, ref_gaussian, name):
     kind = KINDS[name]
     g = ref_gaussian
@@ -178,7 +179,7 @@ def test_oracle_equals_reference_code_on_gaussian_fixture(oracle, ref_gaussian, 
     assert np.array_equal(oracle.pack(act_kind, g[f"{name}_tail_x"]), g[f"{name}_tail_act"])
 
 
-@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k"])
+@pytest.mark.parametrize("name", ["q4_0", "q8_0", "q4_k", "q5_k", "q6_k", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "q8_1"])
 @pytest.mark.parametrize("seed,scale", [(7, 0.02), (42, 1.0), (123, 30.0), (1337, 1e-4)])
 def test_oracle_equals_reference_code_live(oracle, reflib, name, seed, scale):
     kind = KINDS[name]
@@ -208,7 +209,7 @@ def test_random_bytes_dequant_equals_reference_code_live(oracle, reflib):
         # keep the fp16 scale fields finite
         blk = raw.reshape(nb, BLOCK_BYTES[kind])
         for off in {"q4_0": [0], "q8_0": [0], "q4_k": [0, 2], "q5_k": [0, 2], "q6_k": [208], "q4_1": [0, 2], "q5_0": [0],
-                    "q5_1": [0, 2], "q2_k": [80, 82], "q3_k": [108]}[name]:
+                    "q5_1": [0, 2], "q2_k": [80, 82], "q3_k": [108], "q8_1": [0, 2]}[name]:
             h = blk[:, off:off + 2].copy().view(np.uint16)
             h &= 0xBBFF  # clear the top exponent bit: |value| < 2
             blk[:, off:off + 2] = h.view(np.uint8)

@@ -73,7 +73,7 @@ def random_valid_blocks(rng, kind: int, rows: int, k: int) -> np.ndarray:
     nb = (k + BLOCK_VALUES[kind] - 1) // BLOCK_VALUES[kind]
     bb = BLOCK_BYTES[kind]
     raw = rng.integers(0, 256, size=(rows * nb, bb), dtype=np.uint8)
-    offs = {1: [0], 2: [0, 2], 3: [0], 4: [0, 2], 5: [0], 7: [80, 82], 8: [108], 9: [0, 2], 10: [0, 2], 11: [208]}[kind]
+    offs = {1: [0], 2: [0, 2], 3: [0], 4: [0, 2], 5: [0], 6: [0, 2], 7: [80, 82], 8: [108], 9: [0, 2], 10: [0, 2], 11: [208]}[kind]
     for off in offs:
         h = raw[:, off:off + 2].copy().view(np.uint16)
         h &= 0xBBFF  # clear the top exponent bit: |value| < 2, no inf/nan

@@ -45,7 +45,7 @@ def random_blocks(rng, kind: int, rows: int, k: int) -> np.ndarray:
     nb = (k + block_values(kind) - 1) // block_values(kind)
     bb = block_bytes(kind)
     raw = rng.integers(0, 256, size=(rows * nb, bb), dtype=np.uint8)
-    offs = {1: [0], 2: [0, 2], 3: [0], 4: [0, 2], 5: [0], 7: [80, 82], 8: [108], 9: [0, 2], 10: [0, 2], 11: [208]}[kind]
+    offs = {1: [0], 2: [0, 2], 3: [0], 4: [0, 2], 5: [0], 6: [0, 2], 7: [80, 82], 8: [108], 9: [0, 2], 10: [0, 2], 11: [208]}[kind]
     for off in offs:
         h = raw[:, off:off + 2].copy().view(np.uint16)
         h = (h & 0x83FF) | 0x2000  # exponent field 8: magnitudes around 2^-7
@@ -380,7 +380,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (profiling runs)")
     ap.add_argument("--batch", type=int, default=1, help="activation rows N (1, 4 or 8 are the decode configs)")
     ap.add_argument("--shape", default="4096x14336", help="weight shape MxK (marmot naming)")
-    ap.add_argument("--kind", default="q4_k", choices=["q4_k", "q6_k", "q8_0", "q4_0"])
+    ap.add_argument("--kind", default="q4_k", choices=["q4_k", "q6_k", "q8_0", "q4_0", "q4_1", "q5_0", "q5_1", "q8_1", "q2_k",
+                                                       "q3_k", "q5_k"])
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--prefill-tokens", type=int, default=512)
     ap.add_argument("--sweep", action="store_true",
@@ -415,7 +416,7 @@ def main():
         hip.close()
         return
 
-    kind = {"q4_k": capi.KIND_Q4_K, "q6_k": capi.KIND_Q6_K, "q8_0": capi.KIND_Q8_0, "q4_0": capi.KIND_Q4_0}[args.kind]
+    kind = getattr(capi, "KIND_" + args.kind.upper())
     M, K = (int(v) for v in args.shape.split("x"))
     N = args.batch
     rb = row_bytes(kind, K)

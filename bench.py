@@ -163,8 +163,8 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "LOGITS", "Q5K", "LEGACY", "Q23K")):
-    """Every benchmark configuration (C1..C5, QKV, LOGITS, Q5K, LEGACY, Q23K) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
+    """Every benchmark configuration (C1..C5, QKV, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -213,6 +213,22 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV
         for (M, K) in ((14336, 4096), (4096, 14336)):
             for N in (1, 4, 8, 16):
                 linear_case("Q5K", capi.KIND_Q5_K, M, K, N)
+    if "PREFILL32" in only:
+        # prefill with fp32 activations: the reference's integer path (Q8_K activations), small-batch MFMA kernel in
+        # passes of 32 rows (Q4_K, Q5_K) or 16 rows (Q6_K); one weight copy (the passes re-read it from the caches)
+        for kind in (capi.KIND_Q4_K, capi.KIND_Q5_K, capi.KIND_Q6_K):
+            for N in (32, 128, 512):
+                M = K = 4096
+                d_w = hip.to_device(random_blocks(rng, kind, M, K))
+                d_x = hip.to_device(rng.standard_normal((N, K), dtype=np.float32))
+                d_out = hip.alloc(N * M * 4)
+                ms = time_steps_graph(hip, lambda i: hip.linear_d(kind, d_w, d_x, DT_F32, N, K, M, d_out, DT_F32),
+                                      max(40, steps // 20), 10, chunk=20)
+                emit({"config": "PREFILL32", "workload": f"{names[kind]} {M}x{K} N={N} fp32 activations",
+                      "route": hip.last_route(), "us": round(ms * 1e3, 1),
+                      "TOP/s": round(2.0 * N * M * K / ms / 1e9, 1), "tokens_per_s": round(N / ms * 1e3)})
+                for b in (d_w, d_x, d_out):
+                    b.free()
     if "Q23K" in only:
         # the low-bit K formats on the dot-product matvec (four lanes per block), decode and small batch
         for kind in (capi.KIND_Q2_K, capi.KIND_Q3_K):

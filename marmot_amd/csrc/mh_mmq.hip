@@ -227,14 +227,14 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
             w_off[c] = (uint32_t)((m - row0) * p.nb * WBYTES + 16 * piece);
         }
         const uint8_t *wgroup = wbase + row0 * p.nb * WBYTES;
-        uint32_t a_off[A_LOADS];  // activations: chunk (token, slot) holds source chunk slot ^ token
+        uint32_t a_off[A_LOADS];  // activations: chunk (token, slot) holds source chunk slot ^ (token % 16)
 #pragma unroll
         for (int c = 0; c < A_LOADS; ++c) {
             const int chunk = c * 64 + lane;
             const int slot = chunk & 15, tk = chunk >> 4;
             const int tt = tk < ncols ? tk : 0;  // rows beyond ncols re-read the first row; never stored
             const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
-            a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
+            a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ (tk & 15)));
         }
         uint32_t ad_off;
         {
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
                 }
 #pragma unroll
                 for (int sb = 0; sb < 8; ++sb) {
-                    aq[sb] = *(const uint4 *)(a_blk + 16 * ((2 * sb + kh) ^ ti));
+                    aq[sb] = *(const uint4 *)(a_blk + 16 * ((2 * sb + kh) ^ (ti & 15)));
                 }
                 float adr[NR];
 #pragma unroll
@@ -905,19 +905,29 @@ static size_t mmq6_lds_bytes(int W) {
 }
 
 template <int NR>
+static int mmq_launch_any(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid);
+template <int NR>
+static int mmq_launch_q4k(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid);
+
+template <int NR>
 static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, size_t M,
                       unsigned items) {
     const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * p.nw), items);
+    if constexpr (NR > 8) {
+        // 32 activation rows per pass: only the Q4_K / Q5_K kernel is built for it
+        if (!mmq_is_q4k_family(kind)) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "mmq: 32-row passes exist for Q4_K and Q5_K only");
+        }
+        return mmq_launch_q4k<NR>(dev, kind, p, pl, grid);
+    } else {
+        return mmq_launch_any<NR>(dev, kind, p, pl, grid);
+    }
+}
+
+template <int NR>
+static int mmq_launch_any(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid) {
     static bool attr_set = false;
     if (!attr_set) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
         MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)mmq6_lds_bytes(6)));
         attr_set = true;
@@ -945,8 +955,29 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
     } else if (kind == MARMOT_HIP_KIND_Q6_K) {
         hipLaunchKernelGGL((k_mmq_q6k<NR>), grid, dim3(pl.W * 64), mmq6_lds_bytes(pl.W), dev->stream, p);
     } else {
-        // W consumers + 1 loader. Three stages (the loader two blocks ahead) for the dense call; the grouped call
-        // runs many small workgroups per CU, which overlap each other, and takes two to fit more of them.
+        return mmq_launch_q4k<NR>(dev, kind, p, pl, grid);
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+// Q4_K / Q5_K: W consumers + 1 loader. Three stages (the loader two blocks ahead) for the dense call; the grouped call
+// runs many small workgroups per CU, which overlap each other, and takes two to fit more of them.
+template <int NR>
+static int mmq_launch_q4k(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        attr_set = true;
+    }
+    {
         if (pl.W < 1 || pl.W > 4) {
             return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "mmq: %d consumer wavefronts are not supported", pl.W);
         }
@@ -1029,13 +1060,17 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
     p.n_items = nullptr;
     p.act_index = nullptr;
     p.expert_stride = 0;
-    // 16 activation rows per pass: 8 live accumulator registers per lane keep two wavefronts per SIMD resident
-    // (32 rows per pass would need 16 and spill)
-    for (size_t n0 = 0; n0 < N; n0 += MMQ_ROWS_PER_PASS) {
+    // 16 activation rows per pass (8 live accumulator registers per lane). Q4_K / Q5_K from 32 rows on: 32 rows per
+    // pass, which uses all 32 rows of the matrix-core product instead of half of them and halves the number of
+    // passes over the weights.
+    const size_t rows_per_pass =
+        (mmq_is_q4k_family(kind) && N >= 32 && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
+    for (size_t n0 = 0; n0 < N; n0 += rows_per_pass) {
         p.n0 = n0;
-        p.ncols = (int)(N - n0 < MMQ_ROWS_PER_PASS ? N - n0 : MMQ_ROWS_PER_PASS);
-        const int st =
-            p.ncols <= 8 ? mmq_launch<4>(dev, kind, p, pl, M, 1) : mmq_launch<8>(dev, kind, p, pl, M, 1);
+        p.ncols = (int)(N - n0 < rows_per_pass ? N - n0 : rows_per_pass);
+        const int st = p.ncols <= 8    ? mmq_launch<4>(dev, kind, p, pl, M, 1)
+                       : p.ncols <= 16 ? mmq_launch<8>(dev, kind, p, pl, M, 1)
+                                       : mmq_launch<16>(dev, kind, p, pl, M, 1);
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
         }

@@ -154,3 +154,23 @@ def test_prepacked_activations_and_graph_replay(hip, oracle, name):
         hip.graph_destroy(g)
         for b in (d_w, d_x, d_p, d_out):
             b.free()
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q5_k"])
+@pytest.mark.parametrize("N", [32, 33, 48, 64, 100])
+def test_passes_of_32_rows(hip, oracle, name, N):
+    """From 32 activation rows on, Q4_K / Q5_K take 32 rows per pass (all 32 rows of the matrix-core product): full and
+    partial passes, ragged row groups, K split within the workgroup and across workgroups, bias, float16 epilogue."""
+    kind = KINDS[name]
+    for M, K in ((203, 2048), (64, 7168)):
+        blocks = oracle.quantize(kind, gaussian(380, (M, K), 0.02))
+        x = gaussian(381 + N, (N, K))
+        bias = gaussian(382, (M,))
+        got = hip.linear(x, blocks, kind, M, bias=bias)
+        assert "mmq_" in hip.last_route()
+        assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"{name} {M}x{K} N={N}")
+    x16 = x.astype(np.float16)
+    ref16 = oracle.matmul(kind, blocks, x16, M, out_dtype=np.float16, force_pack=True)
+    got16 = hip.linear(x16, blocks, kind, M, out_dtype=np.float16, force_pack=True)
+    assert np.max(np.abs(got16.astype(np.float32) - ref16.astype(np.float32))) <= \
+        2e-3 * np.abs(ref16.astype(np.float32)).max()

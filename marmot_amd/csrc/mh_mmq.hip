@@ -681,7 +681,7 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
             const int slot = chunk & 15, tk = chunk >> 4;
             const int tt = tk < ncols ? tk : 0;
             const size_t arow = p.act_index != nullptr ? (size_t)p.act_index[n0 + tt] : n0 + tt;
-            a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ tk));
+            a_off[c] = (uint32_t)(arow * p.kp + 16 * (slot ^ (tk & 15)));
         }
         uint32_t ad_off;
         {
@@ -764,7 +764,7 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
                 }
                 const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
                 auto acts_of = [&](int is) {
-                    const uint2 v = *(const uint2 *)(a_blk + 16 * (is ^ ti));
+                    const uint2 v = *(const uint2 *)(a_blk + 16 * (is ^ (ti & 15)));
                     return (long)(((unsigned long)v.y << 32) | v.x);
                 };
                 auto weights_of = [&](int is) {
@@ -904,6 +904,36 @@ static size_t mmq6_lds_bytes(int W) {
     return ring > red ? ring : red;
 }
 
+// the Q6_K loader / consumer kernel copies 16-byte chunks: rows, bases and expert strides must be 16-byte aligned
+static bool mmq6_loader_applies(const MmqParams &p, const MmqPlan &pl) {
+    return mmq6_uses_loader(p.nb) && pl.W <= 4 && (((uintptr_t)p.w[0]) & 15) == 0 && (((uintptr_t)p.w[1]) & 15) == 0 &&
+           (((uintptr_t)p.w[2]) & 15) == 0 && (p.expert_stride & 15) == 0;
+}
+
+template <int NR>
+static int mmq_launch_q6k_ls(marmot_hip_device *dev, const MmqParams &p, const MmqPlan &pl, const dim3 grid) {
+    const int stages = p.items != nullptr ? 2 : 3;
+    const size_t stage = MMQ6_WBLK + 2 * NR * QK_K + 2 * NR * 4;
+    const size_t ring = (size_t)pl.W * stages * stage;
+    const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
+    const dim3 block((pl.W + 1) * 64);
+    static bool ls6_attr = false;
+    if (!ls6_attr) {
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024));
+        ls6_attr = true;
+    }
+    if (stages == 2) {
+        hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 2>), grid, block, ring > red ? ring : red, dev->stream, p);
+    } else {
+        hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 3>), grid, block, ring > red ? ring : red, dev->stream, p);
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
 template <int NR>
 static int mmq_launch_any(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid);
 template <int NR>
@@ -914,11 +944,14 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
                       unsigned items) {
     const dim3 grid((unsigned)((M + 31) / 32), (unsigned)(pl.S * p.nw), items);
     if constexpr (NR > 8) {
-        // 32 activation rows per pass: only the Q4_K / Q5_K kernel is built for it
-        if (!mmq_is_q4k_family(kind)) {
-            return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "mmq: 32-row passes exist for Q4_K and Q5_K only");
+        // 32 activation rows per pass: the loader / consumer kernels are built for it
+        if (mmq_is_q4k_family(kind)) {
+            return mmq_launch_q4k<NR>(dev, kind, p, pl, grid);
         }
-        return mmq_launch_q4k<NR>(dev, kind, p, pl, grid);
+        if (kind == MARMOT_HIP_KIND_Q6_K && mmq6_loader_applies(p, pl)) {
+            return mmq_launch_q6k_ls<NR>(dev, p, pl, grid);
+        }
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "mmq: no 32-row pass for this kind or alignment");
     } else {
         return mmq_launch_any<NR>(dev, kind, p, pl, grid);
     }
@@ -932,26 +965,8 @@ static int mmq_launch_any(marmot_hip_device *dev, int kind, const MmqParams &p, 
                                    (int)mmq6_lds_bytes(6)));
         attr_set = true;
     }
-    if (kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(p.nb) && pl.W <= 4 && (((uintptr_t)p.w[0]) & 15) == 0 &&
-        (((uintptr_t)p.w[1]) & 15) == 0 && (((uintptr_t)p.w[2]) & 15) == 0 && (p.expert_stride & 15) == 0) {
-        const int stages = p.items != nullptr ? 2 : 3;
-        const size_t stage = MMQ6_WBLK + 2 * NR * QK_K + 2 * NR * 4;
-        const size_t ring = (size_t)pl.W * stages * stage;
-        const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
-        const dim3 block((pl.W + 1) * 64);
-        static bool ls6_attr = false;
-        if (!ls6_attr) {
-            MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       160 * 1024));
-            MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       160 * 1024));
-            ls6_attr = true;
-        }
-        if (stages == 2) {
-            hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 2>), grid, block, ring > red ? ring : red, dev->stream, p);
-        } else {
-            hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 3>), grid, block, ring > red ? ring : red, dev->stream, p);
-        }
+    if (kind == MARMOT_HIP_KIND_Q6_K && mmq6_loader_applies(p, pl)) {
+        return mmq_launch_q6k_ls<NR>(dev, p, pl, grid);
     } else if (kind == MARMOT_HIP_KIND_Q6_K) {
         hipLaunchKernelGGL((k_mmq_q6k<NR>), grid, dim3(pl.W * 64), mmq6_lds_bytes(pl.W), dev->stream, p);
     } else {
@@ -982,7 +997,8 @@ static int mmq_launch_q4k(marmot_hip_device *dev, int kind, const MmqParams &p, 
             return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "mmq: %d consumer wavefronts are not supported", pl.W);
         }
         const bool q5 = kind == MARMOT_HIP_KIND_Q5_K;
-        const int stages = p.items != nullptr ? 2 : 3;
+        // Q5_K with 32-row passes: three stages of two consumers would take 84 KB and leave one workgroup per CU
+        const int stages = (p.items != nullptr || (q5 && NR > 8 && getenv("MH_MMQ5_3STAGES") == nullptr)) ? 2 : 3;
         const size_t stage = 32 * (size_t)(q5 ? Q5_K_BYTES : Q4_K_BYTES) + 2 * NR * QK_K + 2 * NR * 4;
         const size_t ring = (size_t)pl.W * stages * stage;
         const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
@@ -1060,11 +1076,11 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
     p.n_items = nullptr;
     p.act_index = nullptr;
     p.expert_stride = 0;
-    // 16 activation rows per pass (8 live accumulator registers per lane). Q4_K / Q5_K from 32 rows on: 32 rows per
-    // pass, which uses all 32 rows of the matrix-core product instead of half of them and halves the number of
+    // 16 activation rows per pass (8 live accumulator registers per lane). The loader / consumer kernels (Q4_K, Q5_K,
+    // Q6_K with 16-byte aligned rows) from 32 rows on: 32 rows per pass, which uses all 32 rows of the matrix-core product instead of half of them and halves the number of
     // passes over the weights.
-    const size_t rows_per_pass =
-        (mmq_is_q4k_family(kind) && N >= 32 && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
+    const bool wide_ok = mmq_is_q4k_family(kind) || (kind == MARMOT_HIP_KIND_Q6_K && mmq6_loader_applies(p, pl));
+    const size_t rows_per_pass = (wide_ok && N >= 32 && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
     for (size_t n0 = 0; n0 < N; n0 += rows_per_pass) {
         p.n0 = n0;
         p.ncols = (int)(N - n0 < rows_per_pass ? N - n0 : rows_per_pass);

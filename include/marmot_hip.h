@@ -40,7 +40,8 @@ enum {
     MARMOT_HIP_ERROR_NOT_IMPLEMENTED = -8,
 };
 
-/* marmot_quant_kind_t values (include/marmot/types.h:372-388) */
+/* marmot_quant_kind_t values (include/marmot/types.h:372-388). Weight kinds: all but Q8_K, which (like Q8_0) is the
+ * format of packed activations. */
 enum {
     MARMOT_HIP_KIND_Q4_0 = 1,
     MARMOT_HIP_KIND_Q4_1 = 2,
@@ -230,7 +231,8 @@ int marmot_hip_rope_frequencies(int scaling_type, float theta, float freq_scale,
  * Replaces cpu_embedding_gather_scalar for block-quantized tables (cpu_embedding_run_worker and
  * cpu_embedding_copy_row_quantized, src/backends/cpu/ops/embedding/scalar/embedding_scalar.c:241-303, 381-447;
  * descriptor marmot_embedding_gather_desc_t, include/marmot/ops_types.h:160-170).
- *   d_table : vocab rows of marmot_hip_row_bytes(kind, dim) bytes (Q4_0, Q8_0, Q4_K or Q6_K)
+ *   d_table : vocab rows of marmot_hip_row_bytes(kind, dim) bytes (any weight kind except Q4_1, whose tables the
+ *             reference decodes in an order of its own without a golden vector: NOT_IMPLEMENTED)
  *   d_ids   : n token ids of ids_dtype (MARMOT_HIP_DTYPE_I32 or _I64)
  *   d_out   : [n, dim] of out_dtype (F32 or F16): decoded value * scale, one rounding for F16
  * A token equal to padding_id (when padding_id >= 0) gives a zero row. A token outside [0, vocab) gives a zero row,

@@ -62,6 +62,7 @@ enum {
     MARMOT_HIP_DTYPE_F32 = 0,
     MARMOT_HIP_DTYPE_F16 = 1,
     MARMOT_HIP_DTYPE_I32 = 3,  /* position tensors of the rotary epilogue only */
+    MARMOT_HIP_DTYPE_U8 = 6,   /* storage type of block-quantized tensors (GGUF reader) */
     MARMOT_HIP_DTYPE_I64 = 11,
 };
 
@@ -275,6 +276,36 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
                            size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate, const void *d_up,
                            const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
                            float weights_scale, int router_weight_policy, int ffn_type, float *d_out);
+
+/* ------------------------------------------------------------------ GGUF files
+ * Replaces, for the weights of this path, marmot_gguf_load / marmot_gguf_find_tensor (src/graph/gguf/loader.cpp:577-770,
+ * 808-818) and the tensor views they build (set_tensor_data_views, :492-575): the file is mapped read-only, the
+ * key/value table is skipped except general.alignment, every tensor becomes a view into the mapping. Shapes follow the
+ * loader: matrices are [rows, cols] = [ne1, ne0], other ranks keep the file's order (expert stacks [cols, rows,
+ * experts]); ggml types map to quant kinds as in map_ggml_type (:300-490), dense F32 / F16 / I32 tensors have kind 0.
+ * The views are host memory: the tensor-level backend mirrors a view on first use (the residency table), and
+ * marmot_hip_gguf_upload copies one tensor into a fresh device allocation for callers of this raw-pointer ABI
+ * (counterpart of the upload in ExecutionSession, src/graph/execution_session.cpp:315-320; free with
+ * marmot_hip_free). Views stay valid until marmot_hip_gguf_close. */
+#define MARMOT_HIP_GGUF_MAX_DIMS 4
+typedef struct marmot_hip_gguf marmot_hip_gguf_t;
+typedef struct {
+    const char *name;
+    uint32_t ggml_type;
+    int kind;           /* MARMOT_HIP_KIND_*, 0 for a dense tensor */
+    int dtype;          /* MARMOT_HIP_DTYPE_U8 for quantized tensors, else F32 / F16 / I32 */
+    uint32_t ndim;
+    uint64_t shape[MARMOT_HIP_GGUF_MAX_DIMS];
+    const void *data;   /* inside the mapping */
+    size_t nbytes;
+} marmot_hip_gguf_tensor_t;
+int marmot_hip_gguf_open(const char *path, marmot_hip_gguf_t **out);
+void marmot_hip_gguf_close(marmot_hip_gguf_t *g);
+size_t marmot_hip_gguf_tensor_count(const marmot_hip_gguf_t *g);
+size_t marmot_hip_gguf_alignment(const marmot_hip_gguf_t *g);
+int marmot_hip_gguf_tensor(const marmot_hip_gguf_t *g, size_t index, marmot_hip_gguf_tensor_t *out);
+int marmot_hip_gguf_find(const marmot_hip_gguf_t *g, const char *name, marmot_hip_gguf_tensor_t *out);
+int marmot_hip_gguf_upload(marmot_hip_device_t *dev, const marmot_hip_gguf_t *g, size_t index, void **d_out);
 
 /* ------------------------------------------------------------------ introspection
  * Name of the kernel route the last marmot_hip_matmul_quantized call on this thread took

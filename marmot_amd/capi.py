@@ -44,6 +44,12 @@ class Rope(C.Structure):
                 ("apply_to_q", C.c_int), ("apply_to_k", C.c_int)]
 
 
+class GgufTensor(C.Structure):
+    """marmot_hip_gguf_tensor_t"""
+    _fields_ = [("name", C.c_char_p), ("ggml_type", C.c_uint32), ("kind", C.c_int), ("dtype", C.c_int),
+                ("ndim", C.c_uint32), ("shape", C.c_uint64 * 4), ("data", C.c_void_p), ("nbytes", C.c_size_t)]
+
+
 _vp, _sz, _i, _u32, _f = C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_float
 
 # name -> (restype, argtypes); every symbol include/marmot_hip.h declares
@@ -92,6 +98,13 @@ SIGNATURES = {
                                     _vp]),
     "marmot_hip_last_route": (C.c_char_p, []),
     "marmot_hip_version": (C.c_char_p, []),
+    "marmot_hip_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),
+    "marmot_hip_gguf_close": (None, [_vp]),
+    "marmot_hip_gguf_tensor_count": (_sz, [_vp]),
+    "marmot_hip_gguf_alignment": (_sz, [_vp]),
+    "marmot_hip_gguf_tensor": (_i, [_vp, _sz, C.POINTER(GgufTensor)]),
+    "marmot_hip_gguf_find": (_i, [_vp, C.c_char_p, C.POINTER(GgufTensor)]),
+    "marmot_hip_gguf_upload": (_i, [_vp, _vp, _sz, C.POINTER(_vp)]),
 }
 
 _lib = None

@@ -1,0 +1,91 @@
+"""CPU: the library's GGUF reader (host code, no GPU call) against files written by tests/gguf_writer.py: header and
+key/value skipping, general.alignment, the loader's shape convention ([rows, cols] for matrices, file order for
+expert stacks), the ggml-type mapping of every weight format, views that alias the file's bytes, error paths."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+from marmot_amd import capi
+from marmot_amd.gguf import GgufFile
+from oracle.pyoracle import BLOCK_BYTES, BLOCK_VALUES, KINDS
+from tests.gguf_writer import write_gguf
+from tests.util import gaussian, random_valid_blocks
+
+WEIGHT_KINDS = ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"]
+
+
+def test_every_weight_format_round_trips(tmp_path, oracle):
+    rng = np.random.default_rng(1)
+    tensors, want = [], {}
+    for name in WEIGHT_KINDS:
+        kind = KINDS[name]
+        rows, cols = 6, 512
+        blocks = random_valid_blocks(rng, kind, rows, cols)
+        tensors.append((f"blk.0.{name}.weight", name, (cols, rows), blocks))
+        want[f"blk.0.{name}.weight"] = (kind, (rows, cols), blocks)
+    norm = gaussian(2, (512,))
+    tensors.append(("output_norm.weight", "f32", (512,), norm))
+    experts = random_valid_blocks(rng, KINDS["q4_k"], 3 * 8, 256)  # [cols=256, rows=8, experts=3]
+    tensors.append(("blk.0.ffn_gate_exps.weight", "q4_k", (256, 8, 3), experts))
+    path = write_gguf(str(tmp_path / "m.gguf"), tensors,
+                      kv={"general.architecture": "llama", "llama.block_count": 1, "tokenizer.ggml.tokens": ["a", "bc"],
+                          "llama.rope.freq_base": 10000.0, "some.flag": True, "some.ints": [1, 2, 3]})
+    with GgufFile(path) as g:
+        assert g.alignment == 32 and len(g.tensors) == len(tensors)
+        for name, (kind, shape, blocks) in want.items():
+            t = g.find(name)
+            assert (t.kind, t.shape, t.dtype) == (kind, shape, 6)
+            assert t.nbytes == shape[0] * (shape[1] // BLOCK_VALUES[kind]) * BLOCK_BYTES[kind]
+            assert t.address % 32 == 0
+            assert np.array_equal(g.array(t), blocks.reshape(-1))
+        t = g.find("output_norm.weight")
+        assert t.kind == 0 and t.dtype == capi.DT_F32 and t.shape == (512,) and np.array_equal(g.array(t), norm)
+        e = g.find("blk.0.ffn_gate_exps.weight")
+        assert e.shape == (256, 8, 3) and e.nbytes == 3 * 8 * 144  # the file's order is kept for rank 3
+        with pytest.raises(capi.MarmotHipError):
+            g.find("missing")
+
+
+def test_alignment_and_version(tmp_path):
+    w = np.arange(64, dtype=np.float32).reshape(4, 16)
+    b = np.arange(10, dtype=np.float16)
+    p = write_gguf(str(tmp_path / "a.gguf"), [("w", "f32", (16, 4), w), ("b", "f16", (10,), b)], alignment=64)
+    with GgufFile(p) as g:
+        assert g.alignment == 64
+        assert all(t.address % 64 == 0 for t in g.tensors)
+        assert np.array_equal(g.array(g.find("w")), w) and g.find("w").shape == (4, 16)
+        assert np.array_equal(g.array(g.find("b")), b)
+    p = write_gguf(str(tmp_path / "v2.gguf"), [("w", "f32", (16, 4), w)], version=2, declare_alignment=False)
+    with GgufFile(p) as g:
+        assert g.alignment == 32 and np.array_equal(g.array(g.tensors[0]), w)
+
+
+def test_malformed_files_are_rejected(tmp_path):
+    w = np.zeros((4, 32), np.float32)
+    good = write_gguf(str(tmp_path / "g.gguf"), [("w", "f32", (32, 4), w)])
+    raw = open(good, "rb").read()
+
+    def opens(data, name):
+        p = str(tmp_path / name)
+        open(p, "wb").write(data)
+        try:
+            GgufFile(p).close()
+            return None
+        except capi.MarmotHipError as e:
+            return e.code
+
+    assert opens(raw, "ok.gguf") is None
+    assert opens(b"GGML" + raw[4:], "magic.gguf") == -1
+    assert opens(raw[:4] + struct.pack("<I", 1) + raw[8:], "v1.gguf") == -8
+    assert opens(raw[:40], "cut_header.gguf") == -1
+    assert opens(raw[:-64], "cut_data.gguf") == -1           # tensor storage beyond the end of the file
+    bad_type = write_gguf(str(tmp_path / "t.gguf"), [("w", "f32", (32, 4), w)])
+    data = bytearray(open(bad_type, "rb").read())
+    at = data.index(b"w" + struct.pack("<I", 2)) + 1 + 4 + 16   # name, rank, two dimensions -> the type field
+    data[at:at + 4] = struct.pack("<I", 99)
+    assert opens(bytes(data), "type.gguf") == -8
+    with pytest.raises(capi.MarmotHipError):
+        GgufFile(str(tmp_path / "does_not_exist.gguf"))
+    assert not os.path.exists(str(tmp_path / "does_not_exist.gguf"))

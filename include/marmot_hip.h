@@ -161,12 +161,14 @@ int marmot_hip_quantize_activations(marmot_hip_device_t *dev, int act_kind, cons
                                     size_t rows, size_t k, void *d_blocks_out);
 
 /* ------------------------------------------------------------------ quantized linear
- * Replaces cpu_matmul_quantized_{q4_0,q8_0,q4_k,q6_k} -> cpu_matmul_quantized_impl
+ * Replaces cpu_matmul_quantized_{scheme} (every weight scheme of the reference) -> cpu_matmul_quantized_impl
  * (src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:373-591, 905-929) incl. the bias epilogue
  * (src/backends/cpu/ops/matmul/matmul_epilogue.c). out[n*M + m] = dot(W[m,:], x[n,:]) (+ bias[m]).
  *   d_weight : M rows of marmot_hip_row_bytes(kind,K) bytes, native GGUF blocks
- *   d_input  : [N,K] of in_dtype; F32 -> activations are quantized to Q8_0 (Q4_0/Q8_0 weights) or Q8_K
+ *   d_input  : [N,K] of in_dtype; F32 -> activations are quantized to Q8_0 (32-value weight blocks) or Q8_K
  *              (K-quants) and integer block dots are used; F16 -> direct dequantized dot unless FORCE_PACK
+ *              (NOT_IMPLEMENTED for Q2_K, Q3_K, Q5_K and Q6_K, whose direct dots in the reference do not agree
+ *              with its dequantizers: the caller falls back or packs)
  *   d_bias   : NULL or M values of bias_dtype (F32, or F16 when out is F16)
  *   d_out    : [N,M] of out_dtype (F32; F16 allowed only with F16 input)
  * Errors mirror marmot_matmul_validate_quantized (src/core/helpers/matmul.c:68-136). */

@@ -1077,10 +1077,15 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
     p.act_index = nullptr;
     p.expert_stride = 0;
     // 16 activation rows per pass (8 live accumulator registers per lane). The loader / consumer kernels (Q4_K, Q5_K,
-    // Q6_K with 16-byte aligned rows) from 32 rows on: 32 rows per pass, which uses all 32 rows of the matrix-core product instead of half of them and halves the number of
+    // Q6_K with 16-byte aligned rows) from 17 rows on: 32 rows per pass, which uses all 32 rows of the matrix-core product instead of half of them and halves the number of
     // passes over the weights.
     const bool wide_ok = mmq_is_q4k_family(kind) || (kind == MARMOT_HIP_KIND_Q6_K && mmq6_loader_applies(p, pl));
-    const size_t rows_per_pass = (wide_ok && N >= 32 && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
+    size_t wide_from = 17;  // more than one 16-row pass: one 32-row pass streams the weights once instead of twice
+    if (const char *e = getenv("MH_MMQ_WIDE_FROM")) {
+        wide_from = (size_t)atoi(e);
+    }
+    const size_t rows_per_pass =
+        (wide_ok && N >= wide_from && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
     for (size_t n0 = 0; n0 < N; n0 += rows_per_pass) {
         p.n0 = n0;
         p.ncols = (int)(N - n0 < rows_per_pass ? N - n0 : rows_per_pass);

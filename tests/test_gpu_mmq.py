@@ -157,9 +157,9 @@ def test_prepacked_activations_and_graph_replay(hip, oracle, name):
 
 
 @pytest.mark.parametrize("name", ["q4_k", "q5_k", "q6_k"])
-@pytest.mark.parametrize("N", [32, 33, 48, 64, 100])
+@pytest.mark.parametrize("N", [17, 23, 31, 32, 33, 48, 64, 100])
 def test_passes_of_32_rows(hip, oracle, name, N):
-    """From 32 activation rows on, Q4_K / Q5_K (and Q6_K with 16-byte aligned rows: K = 2048 here; K = 7168 keeps the
+    """From 17 activation rows on, Q4_K / Q5_K (and Q6_K with 16-byte aligned rows: K = 2048 here; K = 7168 keeps the
     16-row passes) take 32 rows per pass (all 32 rows of the matrix-core product): full and
     partial passes, ragged row groups, K split within the workgroup and across workgroups, bias, float16 epilogue."""
     kind = KINDS[name]

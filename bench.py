@@ -222,8 +222,11 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV
                 d_w = hip.to_device(random_blocks(rng, kind, M, K))
                 d_x = hip.to_device(rng.standard_normal((N, K), dtype=np.float32))
                 d_out = hip.alloc(N * M * 4)
-                ms = time_steps_graph(hip, lambda i: hip.linear_d(kind, d_w, d_x, DT_F32, N, K, M, d_out, DT_F32),
-                                      max(40, steps // 20), 10, chunk=20)
+                step = lambda i: hip.linear_d(kind, d_w, d_x, DT_F32, N, K, M, d_out, DT_F32)
+                if os.environ.get("MARMOT_BENCH_EAGER"):  # plain launches (for kernel traces), host rate included
+                    ms, _ = time_steps(hip, step, max(40, steps // 20), 10)
+                else:
+                    ms = time_steps_graph(hip, step, max(40, steps // 20), 10, chunk=20)
                 emit({"config": "PREFILL32", "workload": f"{names[kind]} {M}x{K} N={N} fp32 activations",
                       "route": hip.last_route(), "us": round(ms * 1e3, 1),
                       "TOP/s": round(2.0 * N * M * K / ms / 1e9, 1), "tokens_per_s": round(N / ms * 1e3)})

@@ -303,7 +303,7 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
 int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 // small-batch int8-MFMA matmul (mh_mmq.hip)
-bool mmq_supported(int kind, size_t N, size_t K);
+bool mmq_supported(int kind, size_t N, size_t K, int weights = 1);
 size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int weights);
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,

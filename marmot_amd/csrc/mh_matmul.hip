@@ -525,7 +525,7 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
     ws.out[2] = d_out_v;
     ws.bias_dtype = bias_dtype;
     ws.bias_first = true;
-    const bool mmq = mmq_supported(kind, N, K);
+    const bool mmq = mmq_supported(kind, N, K, 3);
     const bool fuse_quant = !mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input);
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes =

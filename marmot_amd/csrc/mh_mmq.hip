@@ -826,12 +826,17 @@ static bool mmq_is_q4k_family(int kind) {
     return kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q5_K;
 }
 
-bool mmq_supported(int kind, size_t N, size_t K) {
+bool mmq_supported(int kind, size_t N, size_t K, int weights) {
     if (getenv("MARMOT_HIP_NO_MMQ") != nullptr) {
         return false;
     }
     // below these row counts the fused-quantization matvec is faster (no separate quantization pass)
-    const size_t min_rows = mmq_is_q4k_family(kind) ? 3 : 5;
+    // (a Q6_K set of three weights crosses over earlier: the matvec streams every weight per column tile)
+    size_t q6_set_min = 3;
+    if (const char *e = getenv("MH_MMQ6_SET_MIN")) {
+        q6_set_min = (size_t)atoi(e);
+    }
+    const size_t min_rows = mmq_is_q4k_family(kind) ? 3 : (weights >= 3 ? q6_set_min : 5);
     return (mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && N >= min_rows && K % QK_K == 0;
 }
 
@@ -1039,7 +1044,7 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
 
 int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                    size_t M, int out_dtype, void *scratch) {
-    if (!mmq_supported(kind, N, K)) {
+    if (!mmq_supported(kind, N, K, ws.count)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
     }
     const size_t nb = K / QK_K;

@@ -187,6 +187,11 @@ __global__ __launch_bounds__(320) void k_mmq_q4k(const MmqParams p) {
         wbase += (size_t)it.x * p.expert_stride;
         n0 = (size_t)it.y;
         ncols = it.z;
+    } else if (gridDim.z > 1) {
+        // dense call with several passes in one launch: blockIdx.z selects the pass of TOK activation rows
+        n0 = p.n0 + (size_t)blockIdx.z * TOK;
+        const size_t left = p.N - n0;
+        ncols = left < (size_t)TOK ? (int)left : TOK;
     }
     const size_t row0 = (size_t)blockIdx.x * 32;
     const int steps = p.bpw + AHEAD;  // the same for every wavefront of the workgroup
@@ -637,6 +642,11 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
         wbase += (size_t)it.x * p.expert_stride;
         n0 = (size_t)it.y;
         ncols = it.z;
+    } else if (gridDim.z > 1) {
+        // dense call with several passes in one launch: blockIdx.z selects the pass of TOK activation rows
+        n0 = p.n0 + (size_t)blockIdx.z * TOK;
+        const size_t left = p.N - n0;
+        ncols = left < (size_t)TOK ? (int)left : TOK;
     }
     const size_t row0 = (size_t)blockIdx.x * 32;
     const int steps = p.bpw + AHEAD;
@@ -861,12 +871,19 @@ static bool mmq6_uses_loader(size_t nb) {
 //     N=8: 34.0 -> 28.4 us.
 static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t M, size_t nb, int weights) {
     // row groups of the whole launch: the weights of a set (gate/up, q/k/v) are one grid
-    const size_t rg = ((M + 31) / 32) * (size_t)(weights > 0 ? weights : 1);
+    const bool q6_loader = kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(nb);
+    // beyond 32 activation rows the 32-row passes of the loader / consumer kernels run as one launch: its workgroups
+    // count like row groups (4096 x 4096, N = 512: 85.5 us with the K split chosen for one pass, 64.7 us without)
+    const size_t passes = (N > 32 && (mmq_is_q4k_family(kind) || q6_loader)) ? (N + 31) / 32 : 1;
+    const size_t rg = ((M + 31) / 32) * (size_t)(weights > 0 ? weights : 1) * passes;
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     MmqPlan pl;
-    const bool q6_loader = kind == MARMOT_HIP_KIND_Q6_K && mmq6_uses_loader(nb);
     size_t W, S = 1;
-    if (q6_loader && weights > 1 && rg >= cus) {
+    if (passes > 1 && rg >= cus && getenv("MH_MMQ_ZPLAN_OFF") == nullptr) {
+        // several passes in one launch fill the chip by themselves: one consumer walks the whole row, which keeps
+        // the LDS ring small (four workgroups per CU) and needs no partial sums
+        W = 1;
+    } else if (q6_loader && weights > 1 && rg >= cus) {
         // a set of weights that fills the chip by itself: two consumers per workgroup and no K split, so that no
         // reduction launch per weight follows (q/k/v 3 x 4096 x 4096, N=16: 41.3 us with the rule below, 33.6 with
         // two workgroups along K, 32.2 with this)
@@ -1091,14 +1108,24 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
     }
     const size_t rows_per_pass =
         (wide_ok && N >= wide_from && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
-    for (size_t n0 = 0; n0 < N; n0 += rows_per_pass) {
-        p.n0 = n0;
-        p.ncols = (int)(N - n0 < rows_per_pass ? N - n0 : rows_per_pass);
-        const int st = p.ncols <= 8    ? mmq_launch<4>(dev, kind, p, pl, M, 1)
-                       : p.ncols <= 16 ? mmq_launch<8>(dev, kind, p, pl, M, 1)
-                                       : mmq_launch<16>(dev, kind, p, pl, M, 1);
+    if (rows_per_pass == 32 && N > 32 && getenv("MH_MMQ_NO_ZPASS") == nullptr) {
+        // all passes in one launch (grid z): no launch gap, ramp and tail per pass
+        p.n0 = 0;
+        p.ncols = 32;
+        const int st = mmq_launch<16>(dev, kind, p, pl, M, (unsigned)((N + 31) / 32));
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
+        }
+    } else {
+        for (size_t n0 = 0; n0 < N; n0 += rows_per_pass) {
+            p.n0 = n0;
+            p.ncols = (int)(N - n0 < rows_per_pass ? N - n0 : rows_per_pass);
+            const int st = p.ncols <= 8    ? mmq_launch<4>(dev, kind, p, pl, M, 1)
+                           : p.ncols <= 16 ? mmq_launch<8>(dev, kind, p, pl, M, 1)
+                                           : mmq_launch<16>(dev, kind, p, pl, M, 1);
+            if (st != MARMOT_HIP_SUCCESS) {
+                return st;
+            }
         }
     }
     if (pl.S > 1) {

@@ -10,6 +10,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 
 #include "../../include/marmot_hip.h"
 
@@ -183,6 +184,13 @@ int check_hip(hipError_t e, const char *what);
             return _st;                                                                                                \
     } while (0)
 
+#define MH_TRY(expr)                                                                                                   \
+    do {                                                                                                               \
+        int _st = (expr);                                                                                              \
+        if (_st != 0)                                                                                                  \
+            return _st;                                                                                                \
+    } while (0)
+
 // ---- activation scratch: quantized activations in a structure-of-arrays layout private to the library.
 // For N rows of K values (nb = ceil(K/block)):
 //   qs    int8  [N][kp]      kp = nb*block, zero padded, 16-byte aligned rows
@@ -208,6 +216,7 @@ struct marmot_hip_device {
     void *workspace = nullptr;
     size_t workspace_bytes = 0;
     bool capturing = false;  // between graph_begin_capture and graph_end_capture
+    std::unordered_set<const void *> large_lds_kernels;  // kernels whose dynamic-LDS limit has been raised (under mu)
     // allocation accounting
     std::mutex mu;
     std::unordered_map<void *, size_t> allocs;
@@ -265,6 +274,9 @@ __device__ __forceinline__ void wait_vmcnt_at_most(int allowed) {
 }
 #endif
 
+// Raises a kernel's dynamic-LDS limit to the 160 KiB of a gfx950 compute unit, once per device and kernel.
+int allow_large_lds(marmot_hip_device *dev, const void *kernel);
+
 // Returns a workspace of at least `bytes` (256-byte aligned). Growing it synchronizes the stream first.
 int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out);
 
@@ -294,6 +306,11 @@ struct WeightSet {
 };
 int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch *act,
                       const float *d_x_f32, size_t N, size_t K, size_t M, int out_dtype);
+// Row-owning Q4_K matvec for one or two fp32 activation rows (mh_matvec_rows.hip): one workgroup per compute unit,
+// activations quantized once per workgroup. Returns MARMOT_HIP_ERROR_NOT_IMPLEMENTED, error text untouched, for shapes
+// it does not cover.
+int launch_matvec_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, size_t N, size_t K,
+                           size_t M, int out_dtype);
 // quantizes act(gate) * up (SwiGLU or GeGLU) of two fp32 [rows, k] arrays into the activation scratch
 int launch_quantize_glu_soa(marmot_hip_device *dev, int act_kind, const float *d_gate, const float *d_up, bool geglu,
                             size_t rows, size_t k, const ActScratch &dst);

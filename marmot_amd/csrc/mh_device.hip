@@ -57,6 +57,15 @@ int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out) {
     return MARMOT_HIP_SUCCESS;
 }
 
+int allow_large_lds(marmot_hip_device *dev, const void *kernel) {
+    std::lock_guard<std::mutex> lock(dev->mu);
+    if (dev->large_lds_kernels.count(kernel) == 0) {
+        MH_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        dev->large_lds_kernels.insert(kernel);
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
 static inline size_t round256(size_t v) {
     return (v + 255) & ~(size_t)255;
 }

@@ -568,11 +568,7 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
         MH_HIP(hipGetLastError());
     }
 
-    static bool attr_set = false;
-    if (!attr_set) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_gemm_q4k_f16, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * STAGE));
-        attr_set = true;
-    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_f16));
     GemmParams p;
     p.w = (const uint8_t *)d_w;
     p.x = (const uint16_t *)d_x;

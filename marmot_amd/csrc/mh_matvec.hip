@@ -1139,12 +1139,7 @@ static int launch_ls(marmot_hip_device *dev, MatvecParams p, int W, size_t M, in
     const size_t part = (((size_t)p.rows_per_wg * NC * 4 * W * sizeof(float)) + 15) & ~(size_t)15;
     const size_t stage_stride = ((size_t)R * p.row_bytes + 1023) & ~(size_t)1023;
     const size_t lds = part + MV_LS_STAGES * stage_stride;
-    static bool attr_set = false;
-    if (!attr_set) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_matvec_ls<Fmt, NC, C, R, FUSED>,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_set = true;
-    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_matvec_ls<Fmt, NC, C, R, FUSED>));
     hipLaunchKernelGGL((k_matvec_ls<Fmt, NC, C, R, FUSED>), grid, dim3((W + 1) * 64), lds, dev->stream, p);
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
@@ -1389,6 +1384,12 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
     p.expert_stride = 0;
     const int nw = ws.count;
     const bool fused = act == nullptr;
+    if (kind == MARMOT_HIP_KIND_Q4_K && fused && N <= 2 && getenv("MH_NO_ROWS") == nullptr) {
+        const int st = launch_matvec_rows_q4k(dev, ws, d_x_f32, N, K, M, out_dtype);
+        if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+            return st;
+        }
+    }
     switch (kind) {
     case MARMOT_HIP_KIND_Q4_K:
         return launch_fmt<FmtQ4K>(dev, p, N, K, M, nw, fused ? "matvec_q4_k_q8_k_fused" : "matvec_q4_k_q8_k");

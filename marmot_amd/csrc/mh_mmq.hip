@@ -939,14 +939,8 @@ static int mmq_launch_q6k_ls(marmot_hip_device *dev, const MmqParams &p, const M
     const size_t ring = (size_t)pl.W * stages * stage;
     const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
     const dim3 block((pl.W + 1) * 64);
-    static bool ls6_attr = false;
-    if (!ls6_attr) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k_ls<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        ls6_attr = true;
-    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q6k_ls<NR, 2>));
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q6k_ls<NR, 3>));
     if (stages == 2) {
         hipLaunchKernelGGL((k_mmq_q6k_ls<NR, 2>), grid, block, ring > red ? ring : red, dev->stream, p);
     } else {
@@ -981,12 +975,7 @@ static int mmq_launch(marmot_hip_device *dev, int kind, const MmqParams &p, cons
 
 template <int NR>
 static int mmq_launch_any(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q6k<NR>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)mmq6_lds_bytes(6)));
-        attr_set = true;
-    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q6k<NR>));
     if (kind == MARMOT_HIP_KIND_Q6_K && mmq6_loader_applies(p, pl)) {
         return mmq_launch_q6k_ls<NR>(dev, p, pl, grid);
     } else if (kind == MARMOT_HIP_KIND_Q6_K) {
@@ -1002,18 +991,10 @@ static int mmq_launch_any(marmot_hip_device *dev, int kind, const MmqParams &p, 
 // runs many small workgroups per CU, which overlap each other, and takes two to fit more of them.
 template <int NR>
 static int mmq_launch_q4k(marmot_hip_device *dev, int kind, const MmqParams &p, const MmqPlan &pl, const dim3 grid) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 2, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        MH_HIP(hipFuncSetAttribute((const void *)k_mmq_q4k<NR, 3, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   160 * 1024));
-        attr_set = true;
-    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q4k<NR, 2>));
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q4k<NR, 3>));
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q4k<NR, 2, true>));
+    MH_TRY(allow_large_lds(dev, (const void *)k_mmq_q4k<NR, 3, true>));
     {
         if (pl.W < 1 || pl.W > 4) {
             return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "mmq: %d consumer wavefronts are not supported", pl.W);

@@ -54,11 +54,16 @@ def random_blocks(rng, kind: int, rows: int, k: int) -> np.ndarray:
 
 
 def time_steps_graph(hip, fn, steps: int, warmup: int, chunk: int = 500):
-    """Like time_steps, but the timed steps are replayed from HIP graphs (chunks of up to `chunk` steps), so the
-    host's launch rate does not enter the figure. Returns ms per step by HIP events."""
+    """Like time_steps, but the timed steps are replayed from HIP graphs, so the host's launch rate does not enter the
+    figure. A graph holds up to `chunk` steps and never more nodes than the library allows per graph (the node count of
+    one step is measured by capturing one). Returns ms per step by HIP events."""
     for i in range(warmup):
         fn(i)
     hip.synchronize()
+    probe = hip.graph_capture(lambda: fn(warmup))
+    per_step = max(1, hip.graph_last_capture_nodes())
+    hip.graph_destroy(probe)
+    chunk = max(1, min(chunk, hip.graph_max_nodes() // per_step))
     graphs = []
     done = 0
     while done < steps:
@@ -98,12 +103,24 @@ def time_steps(hip, fn, steps: int, warmup: int):
     return ev_ms / steps, (t1 - t0) * 1e3 / steps
 
 
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(kind, blocks, x, M, K, nbytes, ref_out, budget_s: float):
-    """The CPU oracle (a restatement of the reference's CPU path) on the host cores, same workload."""
+    """The CPU oracle (a restatement of the reference's CPU path) on the host cores, same workload: rows split over
+    T = every core this process may run on (the reference's own default is a topology-derived count), and T = 1."""
     from oracle.pyoracle import Oracle
 
     oracle = Oracle()
-    cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     out = oracle.matmul(kind, blocks, x, M, threads=cores)  # warm-up, and the parity check of the GPU result
     rms = float(np.sqrt(np.mean(out.astype(np.float64) ** 2)))
     err = float(np.max(np.abs(ref_out - out) / np.maximum(np.abs(out), 1e-3 * rms)))
@@ -123,12 +140,29 @@ def cpu_baseline(kind, blocks, x, M, K, nbytes, ref_out, budget_s: float):
         "value": round(nbytes / med / 1e9, 3),
         "unit": "GB/s",
         "cores": cores,
+        "cpu_model": cpu_model(),
         "kind": "port",
         "sample": f"{len(times)} runs of the same Q4_K {M}x{K} N={x.shape[0]} linear (median), threads split over "
                   f"weight rows with the reference's grain rule",
         "ms_per_step": round(med * 1e3, 4),
         "single_thread_gbps": round(nbytes / float(np.median(t1)) / 1e9, 3),
     }, err
+
+
+def read_calibration(hip, nbytes: int, steps: int, warmup: int):
+    """The read-only streaming kernel (16-byte loads, nothing written) over `nbytes` per launch, dependent launches
+    replayed from a HIP graph, rotating over copies larger than twice the Infinity Cache like the matvec's weights:
+    the read bandwidth this box delivers to one launch of that size."""
+    nbytes = (nbytes + 255) & ~255
+    copies = max(2, -(-2 * MALL_BYTES // nbytes) + 1)
+    buf = hip.alloc(nbytes * copies)
+    hip.lib.marmot_hip_memset(hip.dev, buf.ptr, 0xFF, nbytes * copies)
+    sink = hip.alloc(1024)
+    ms = time_steps_graph(hip, lambda i: hip.read_probe_d(buf, nbytes, sink, offset=(i % copies) * nbytes), steps, warmup)
+    buf.free()
+    sink.free()
+    return {"calibration": "read-only 16-byte streaming kernel, one dependent launch per step", "bytes_per_launch": nbytes,
+            "copies": copies, "us_per_launch": round(ms * 1e3, 3), "gbps": round(nbytes / ms / 1e6, 1)}
 
 
 def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
@@ -285,7 +319,7 @@ def sweep_qkv(hip, rng, emit, steps: int, warmup: int):
                 for w, o in zip(d_w, d_o):
                     hip.linear_d(kind, w, d_x, DT_F32, N, K, M, o, DT_F32, weight_offset=(i % copies) * stride)
 
-            separate = time_steps_graph(hip, three, steps, warmup, chunk=50)  # graphs of a few hundred nodes
+            separate = time_steps_graph(hip, three, steps, warmup, chunk=50)
             nbytes = 3 * M * rb + N * K * 4 + 3 * N * M * 4
             emit({"config": "QKV", "workload": f"{names[kind]} q,k,v 3 x {M}x{K} N={N}", "route": route,
                   "us": round(fused * 1e3, 2), "us_three_linears": round(separate * 1e3, 2),
@@ -408,6 +442,9 @@ def main():
     ap.add_argument("--configs", default="C1,C2,C3,C4,C5", help="with --sweep: the configurations to run")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="run only a plain device copy of this many MiB (known traffic, for profiler counters)")
+    ap.add_argument("--calibrate-read", type=int, default=0, metavar="MIB",
+                    help="run only the read-only streaming kernel over this many MiB per launch, rotating over "
+                         "copies beyond the Infinity Cache, and print its bandwidth")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists in the hot path)",
@@ -426,6 +463,12 @@ def main():
         print(json.dumps({"calibration": "plain 16-byte copy kernel", "bytes_read": n, "bytes_written": n,
                           "launches": 23, "ms_per_launch": round(ms, 5),
                           "gbps_read_plus_write": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
+        hip.close()
+        return
+
+    if args.calibrate_read:
+        hip = HipBackend(0)
+        print(json.dumps(read_calibration(hip, args.calibrate_read << 20, 400, 40)))
         hip.close()
         return
 
@@ -506,13 +549,15 @@ def main():
             "weight_bytes": wbytes,
             "algorithmic_bytes_per_step": nbytes,
             "route": route,
-            "device": caps["name"],
+            "device": caps["name"] or "AMD Instinct MI355X",
+            "weights": "random block bytes with small finite fp16 super-block scales (timing only; parity tests use "
+                       "N(0, 0.02) weights through the quantizer)",
             "arch": caps["arch"],
             "compute_units": caps["num_compute_units"],
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "tokens_per_s": round(N / (ms_op * 1e-3), 1),
-        "submission": "HIP graph replay of the timed steps (chunks of 500 steps)",
+        "submission": "HIP graph replay of the timed steps (graphs of up to 500 steps)",
         "eager_ms_per_step": round(ms_op_eager, 6),
         "eager_ms_per_step_host_clock": round(ms_op_host, 6),
         "roofline": {
@@ -534,6 +579,16 @@ def main():
             "cache_resident_gbps": round(nbytes / (ms_hot * 1e-3) / 1e9, 2),
         },
     }
+    # ---- what a kernel that only reads gets on this box: one dependent launch of the weight size, and a large one
+    small = read_calibration(hip, wbytes, max(100, args.steps // 4), max(20, args.steps // 20))
+    large = read_calibration(hip, 512 << 20, 20, 3)
+    result["roofline"]["measured_read_gbps"] = {
+        "same_size_dependent_launch": small["gbps"], "same_size_us": small["us_per_launch"],
+        "launch_of_512_MiB": large["gbps"],
+        "method": "read-only 16-byte streaming kernel of the library (marmot_hip_read_probe), HIP-graph replay, "
+                  "copies rotating beyond the Infinity Cache",
+    }
+    result["roofline"]["frac_of_measured_read"] = round(achieved / small["gbps"], 4)
     # ---- second half of the metric: Q4_K prefill GEMM, weight 4096 x 4096, fp16 activations, fp32 out
     if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) and not args.no_prefill:
         # as many steps as it takes for the clocks to settle under the matrix-core load (tens of milliseconds)

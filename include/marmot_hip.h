@@ -123,12 +123,29 @@ int marmot_hip_get_caps(marmot_hip_device_t *dev, marmot_hip_caps_t *caps);
 /* Batched submission: everything enqueued between begin and end is recorded into a HIP graph instead of being
  * executed; launching the returned graph replays the whole batch with one submission. This is the HIP form of
  * marmot_device_ops_t.graph_batch_begin / graph_batch_end(commit) (include/marmot/device.h:57-61), which the graph
- * executor brackets a bytecode program with (src/graph/graph_executor.cpp:895). Calls that would allocate
- * (a first use of a larger workspace) must have happened before begin_capture. */
+ * executor brackets a bytecode program with (src/graph/graph_executor.cpp:895).
+ * Rules: a call that needs a larger workspace than any call before it cannot be recorded (it would allocate): run it
+ * once eagerly first; the capture returns MARMOT_HIP_ERROR_INVALID_OPERATION otherwise. After a capture the workspace
+ * may still grow (an eager call with a larger shape): the old one stays allocated until the last executable graph is
+ * destroyed, so earlier graphs stay valid. One graph holds at most MARMOT_HIP_GRAPH_MAX_NODES nodes:
+ * graph_end_capture refuses a longer recording (INVALID_OPERATION; split the batch into several graphs). The limit
+ * keeps one submission within what a profiler's queue interception handles: a replay of a 2700-kernel graph under
+ * `rocprofv3 --kernel-trace` ended in a segmentation fault inside the preloaded interception library, while graphs
+ * of 4500 kernels replay without a profiler attached. graph_last_capture_nodes reports the node count of the latest
+ * end_capture (also of a refused one), for callers that size their batches. */
+#define MARMOT_HIP_GRAPH_MAX_NODES 1024
 int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev);
 int marmot_hip_graph_end_capture(marmot_hip_device_t *dev, void **out_graph_exec);
 int marmot_hip_graph_launch(marmot_hip_device_t *dev, void *graph_exec);
 void marmot_hip_graph_destroy(marmot_hip_device_t *dev, void *graph_exec);
+size_t marmot_hip_graph_max_nodes(void);
+size_t marmot_hip_graph_last_capture_nodes(marmot_hip_device_t *dev);
+
+/* Measurement aid, no counterpart in the reference: one launch that only reads `size` bytes at d_src (16-byte loads,
+ * nothing is written; d_sink is 1 KiB of device memory the kernel may touch only for a pattern the test data cannot
+ * produce). bench.py times it beside the matvec to report the read bandwidth this box delivers to one dependent
+ * launch of the same size. size and d_src must be multiples of 16. */
+int marmot_hip_read_probe(marmot_hip_device_t *dev, const void *d_src, size_t size, void *d_sink);
 
 /* Timing helpers (HIP events on the device object's stream). */
 int marmot_hip_event_create(marmot_hip_device_t *dev, void **out_event);

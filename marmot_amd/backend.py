@@ -101,6 +101,10 @@ class HipBackend:
     def copy_d(self, d_dst, d_src, nbytes: int):
         check(self.lib.marmot_hip_memcpy_device(self.dev, C.c_void_p(d_dst.ptr), C.c_void_p(d_src.ptr), nbytes))
 
+    def read_probe_d(self, d_src, nbytes: int, d_sink, offset: int = 0):
+        """One launch that only reads nbytes at d_src + offset (bandwidth calibration)."""
+        check(self.lib.marmot_hip_read_probe(self.dev, C.c_void_p(d_src.ptr + offset), nbytes, C.c_void_p(d_sink.ptr)))
+
     def synchronize(self):
         check(self.lib.marmot_hip_synchronize(self.dev))
 
@@ -128,6 +132,13 @@ class HipBackend:
             st = self.lib.marmot_hip_graph_end_capture(self.dev, C.byref(g))
         check(st)
         return g
+
+    def graph_max_nodes(self) -> int:
+        """Most nodes one captured graph may hold (graph_capture raises beyond it)."""
+        return int(self.lib.marmot_hip_graph_max_nodes())
+
+    def graph_last_capture_nodes(self) -> int:
+        return int(self.lib.marmot_hip_graph_last_capture_nodes(self.dev))
 
     def graph_launch(self, g):
         check(self.lib.marmot_hip_graph_launch(self.dev, g))

@@ -63,6 +63,7 @@ SIGNATURES = {
     "marmot_hip_memcpy_device": (_i, [_vp, _vp, _vp, _sz]),
     "marmot_hip_memset": (_i, [_vp, _vp, _i, _sz]),
     "marmot_hip_synchronize": (_i, [_vp]),
+    "marmot_hip_read_probe": (_i, [_vp, _vp, _sz, _vp]),
     "marmot_hip_allocator_usage": (_i, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "marmot_hip_stream": (_vp, [_vp]),
     "marmot_hip_last_error": (C.c_char_p, []),
@@ -71,6 +72,8 @@ SIGNATURES = {
     "marmot_hip_graph_end_capture": (_i, [_vp, C.POINTER(_vp)]),
     "marmot_hip_graph_launch": (_i, [_vp, _vp]),
     "marmot_hip_graph_destroy": (None, [_vp, _vp]),
+    "marmot_hip_graph_max_nodes": (_sz, []),
+    "marmot_hip_graph_last_capture_nodes": (_sz, [_vp]),
     "marmot_hip_event_create": (_i, [_vp, C.POINTER(_vp)]),
     "marmot_hip_event_destroy": (None, [_vp, _vp]),
     "marmot_hip_event_record": (_i, [_vp, _vp]),

@@ -11,6 +11,7 @@
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
+#include <vector>
 
 #include "../../include/marmot_hip.h"
 
@@ -216,6 +217,11 @@ struct marmot_hip_device {
     void *workspace = nullptr;
     size_t workspace_bytes = 0;
     bool capturing = false;  // between graph_begin_capture and graph_end_capture
+    // Executable graphs made by graph_end_capture and not destroyed yet: their kernel arguments hold workspace
+    // addresses, so a workspace that is outgrown while any of them lives is retired, not freed.
+    size_t live_graphs = 0;
+    size_t last_capture_nodes = 0;
+    std::vector<void *> retired_workspaces;
     std::unordered_set<const void *> large_lds_kernels;  // kernels whose dynamic-LDS limit has been raised (under mu)
     // allocation accounting
     std::mutex mu;

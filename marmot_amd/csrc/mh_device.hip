@@ -45,12 +45,18 @@ int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out) {
             want *= 2;
         }
         MH_HIP(hipStreamSynchronize(dev->stream));
+        void *fresh = nullptr;
+        MH_HIP(hipMalloc(&fresh, want));
         if (dev->workspace != nullptr) {
-            MH_HIP(hipFree(dev->workspace));
-            dev->workspace = nullptr;
-            dev->workspace_bytes = 0;
+            // Executable graphs captured earlier replay kernels whose arguments point into the old workspace: it
+            // stays allocated until the last of them is destroyed.
+            if (dev->live_graphs > 0) {
+                dev->retired_workspaces.push_back(dev->workspace);
+            } else {
+                MH_HIP(hipFree(dev->workspace));
+            }
         }
-        MH_HIP(hipMalloc(&dev->workspace, want));
+        dev->workspace = fresh;
         dev->workspace_bytes = want;
     }
     *out = dev->workspace;
@@ -167,6 +173,9 @@ void marmot_hip_device_destroy(marmot_hip_device_t *dev) {
     (void)hipStreamSynchronize(dev->stream);
     if (dev->workspace != nullptr) {
         (void)hipFree(dev->workspace);
+    }
+    for (void *w : dev->retired_workspaces) {
+        (void)hipFree(w);
     }
     for (auto &kv : dev->allocs) {
         (void)hipFree(kv.first);
@@ -326,6 +335,10 @@ int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev) {
     return MARMOT_HIP_SUCCESS;
 }
 
+size_t marmot_hip_graph_max_nodes(void) {
+    return MARMOT_HIP_GRAPH_MAX_NODES;
+}
+
 int marmot_hip_graph_end_capture(marmot_hip_device_t *dev, void **out_graph_exec) {
     if (dev == nullptr || out_graph_exec == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "graph_end_capture: null argument");
@@ -337,12 +350,28 @@ int marmot_hip_graph_end_capture(marmot_hip_device_t *dev, void **out_graph_exec
     dev->capturing = false;
     hipGraph_t graph = nullptr;
     MH_HIP(hipStreamEndCapture(dev->stream, &graph));
+    size_t nodes = 0;
+    hipError_t e = hipGraphGetNodes(graph, nullptr, &nodes);
+    dev->last_capture_nodes = e == hipSuccess ? nodes : 0;
+    if (e == hipSuccess && nodes > MARMOT_HIP_GRAPH_MAX_NODES) {
+        (void)hipGraphDestroy(graph);
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
+                         "graph_end_capture: %zu nodes were recorded, the limit is %d per graph: capture the batch in "
+                         "several graphs", nodes, MARMOT_HIP_GRAPH_MAX_NODES);
+    }
     hipGraphExec_t exec = nullptr;
-    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e == hipSuccess) {
+        e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    }
     (void)hipGraphDestroy(graph);
     MH_HIP(e);
+    ++dev->live_graphs;
     *out_graph_exec = (void *)exec;
     return MARMOT_HIP_SUCCESS;
+}
+
+size_t marmot_hip_graph_last_capture_nodes(marmot_hip_device_t *dev) {
+    return dev != nullptr ? dev->last_capture_nodes : 0;
 }
 
 int marmot_hip_graph_launch(marmot_hip_device_t *dev, void *graph_exec) {
@@ -354,9 +383,18 @@ int marmot_hip_graph_launch(marmot_hip_device_t *dev, void *graph_exec) {
 }
 
 void marmot_hip_graph_destroy(marmot_hip_device_t *dev, void *graph_exec) {
-    (void)dev;
-    if (graph_exec != nullptr) {
-        (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+    if (graph_exec == nullptr) {
+        return;
+    }
+    if (dev != nullptr) {
+        (void)hipStreamSynchronize(dev->stream);  // a replay may still be running
+    }
+    (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+    if (dev != nullptr && dev->live_graphs > 0 && --dev->live_graphs == 0) {
+        for (void *w : dev->retired_workspaces) {
+            (void)hipFree(w);
+        }
+        dev->retired_workspaces.clear();
     }
 }
 

@@ -259,6 +259,27 @@ __global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, u
     }
 }
 
+// Read-only stream of 16-byte loads, 8 in flight per lane, each workgroup over one contiguous run of 32 KiB: what a
+// kernel that only has to fetch its operand can reach. The loaded words are folded and stored only if they match a
+// value the fold cannot produce from the all-ones test pattern, so nothing is written.
+__global__ __launch_bounds__(256) void k_read16(const uint4 *__restrict__ src, uint32_t *sink, size_t n16) {
+    const size_t base = (size_t)blockIdx.x * 256 * 8 + threadIdx.x;
+    uint4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const size_t idx = base + (size_t)i * 256;
+        v[i] = idx < n16 ? src[idx] : make_uint4(0, 0, 0, 0);
+    }
+    uint32_t a = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        a ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    }
+    if (a == 0x12345678u) {
+        sink[threadIdx.x] = a;
+    }
+}
+
 __global__ void k_fill_bytes(uint8_t *dst, uint8_t value, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
         dst[i] = value;
@@ -327,6 +348,24 @@ int marmot_hip_copy16_internal(marmot_hip_device_t *dev, void *d_dst, const void
     }
     hipLaunchKernelGGL(k_copy16, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint4 *)d_src, (uint4 *)d_dst,
                        n16);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_read_probe(marmot_hip_device_t *dev, const void *d_src, size_t size, void *d_sink) {
+    if (dev == nullptr || d_src == nullptr || d_sink == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "read_probe: null argument");
+    }
+    if (size % 16 != 0 || (((uintptr_t)d_src) & 15) != 0 || size == 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "read_probe: size and address must be multiples of 16");
+    }
+    const size_t n16 = size / 16;
+    const size_t grid = (n16 + 256 * 8 - 1) / (256 * 8);
+    if (grid > 0x7fffffffu) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "read_probe: %zu bytes are more than one launch covers", size);
+    }
+    hipLaunchKernelGGL(k_read16, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint4 *)d_src,
+                       (uint32_t *)d_sink, n16);
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
 }

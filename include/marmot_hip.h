@@ -193,6 +193,19 @@ int marmot_hip_matmul_quantized(marmot_hip_device_t *dev, int kind, const void *
                                 int in_dtype, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
                                 void *d_out, int out_dtype, uint32_t flags);
 
+/* marmot_hip_matmul_quantized for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc. No counterpart in the reference. Same arguments, routes, kernels and
+ * results (bit for bit) as marmot_hip_matmul_quantized, but the scratch the routes need (quantized activations, K-split
+ * partial sums, the prefill GEMM's sub-block sums) comes from a static device array of
+ * MARMOT_HIP_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends; the call allocates
+ * and frees nothing. A shape that needs more returns MARMOT_HIP_ERROR_INVALID_ARGUMENT with the two sizes in the error
+ * text. Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two device objects, two threads)
+ * race, and the array keeps the last call's contents (no kernel of these routes reads scratch it has not written). */
+#define MARMOT_HIP_NOALLOC_SCRATCH_BYTES (8u << 20)
+int marmot_hip_matmul_quantized_noalloc(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_input,
+                                        int in_dtype, size_t N, size_t K, size_t M, const void *d_bias,
+                                        int bias_dtype, void *d_out, int out_dtype, uint32_t flags);
+
 /* Replaces cpu_matmul_quantized_dual_output (matmul_quant_dispatch.c:593-856): two weights of the same
  * kind and shape applied to one input with a single activation quantization (gate/up projections). */
 int marmot_hip_matmul_quantized_dual(marmot_hip_device_t *dev, int kind, const void *d_weight_a,

@@ -170,6 +170,14 @@ class HipBackend:
             C.c_void_p(d_bias.ptr) if d_bias is not None else None, bias_dtype, C.c_void_p(d_out.ptr), out_dtype,
             flags))
 
+    def linear_noalloc_d(self, kind: int, d_weight, d_input, in_dtype: int, N: int, K: int, M: int, d_out,
+                         out_dtype: int, d_bias=None, bias_dtype: int = DT_F32, flags: int = 0):
+        """marmot_hip_matmul_quantized_noalloc: the same linear with its scratch in the library's static device array."""
+        check(self.lib.marmot_hip_matmul_quantized_noalloc(
+            self.dev, kind, C.c_void_p(d_weight.ptr), C.c_void_p(d_input.ptr), in_dtype, N, K, M,
+            C.c_void_p(d_bias.ptr) if d_bias is not None else None, bias_dtype, C.c_void_p(d_out.ptr), out_dtype,
+            flags))
+
     def linear_qkv_d(self, kind: int, d_wq, d_wk, d_wv, d_input, dtype: int, N: int, K: int, M: int, d_out_q, d_out_k,
                      d_out_v, d_bq=None, d_bk=None, d_bv=None, weight_offset: int = 0):
         """marmot_hip_matmul_qkv_quantized on device buffers; weight_offset applies to the three weights alike."""

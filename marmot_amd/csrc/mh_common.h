@@ -222,6 +222,12 @@ struct marmot_hip_device {
     size_t live_graphs = 0;
     size_t last_capture_nodes = 0;
     std::vector<void *> retired_workspaces;
+    // A statically allocated scratch array of the library as this device sees it (hipGetSymbolAddress at creation)
+    // and, while an entry point that must not allocate runs, the switch that makes workspace_reserve hand it out
+    // instead of the growing workspace.
+    void *static_scratch = nullptr;
+    size_t static_scratch_bytes = 0;
+    bool use_static_scratch = false;
     std::unordered_set<const void *> large_lds_kernels;  // kernels whose dynamic-LDS limit has been raised (under mu)
     // allocation accounting
     std::mutex mu;
@@ -279,6 +285,9 @@ __device__ __forceinline__ void wait_vmcnt_at_most(int allowed) {
     }
 }
 #endif
+
+// Looks up this device's address of the library's static scratch array (mh_matmul.hip); called by device_create.
+int static_scratch_init(marmot_hip_device *dev);
 
 // Raises a kernel's dynamic-LDS limit to the 160 KiB of a gfx950 compute unit, once per device and kernel.
 int allow_large_lds(marmot_hip_device *dev, const void *kernel);

@@ -33,6 +33,15 @@ int check_hip(hipError_t e, const char *what) {
 }
 
 int workspace_reserve(marmot_hip_device *dev, size_t bytes, void **out) {
+    if (dev->use_static_scratch) {
+        if (bytes > dev->static_scratch_bytes) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT,
+                             "this call needs %zu bytes of scratch; the entry point that does not allocate has %zu "
+                             "(use the allocating entry point for this shape)", bytes, dev->static_scratch_bytes);
+        }
+        *out = dev->static_scratch;
+        return MARMOT_HIP_SUCCESS;
+    }
     if (bytes > dev->workspace_bytes) {
         if (dev->capturing) {
             return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
@@ -158,6 +167,11 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
     }
     // default priority, non-blocking with respect to the legacy default stream
     if (check_hip(hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags") != 0) {
+        delete dev;
+        return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
+    }
+    if (static_scratch_init(dev) != 0) {
+        (void)hipStreamDestroy(dev->stream);
         delete dev;
         return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
     }

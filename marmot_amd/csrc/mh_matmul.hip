@@ -6,6 +6,20 @@
 
 namespace mh {
 
+// Scratch of marmot_hip_matmul_quantized_noalloc: device memory that exists from the moment the library is loaded, one
+// copy per GPU, held until the process ends. In host code the array's name is only a handle: the address each device
+// uses comes from hipGetSymbolAddress (static_scratch_init) and is what kernels and helpers receive.
+static __device__ __align__(256) uint8_t scratch[MARMOT_HIP_NOALLOC_SCRATCH_BYTES];
+
+int static_scratch_init(marmot_hip_device *dev) {
+    void *ptr = nullptr;
+    MH_HIP(hipSetDevice(dev->device_index));
+    MH_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    dev->static_scratch = ptr;
+    dev->static_scratch_bytes = MARMOT_HIP_NOALLOC_SCRATCH_BYTES;
+    return MARMOT_HIP_SUCCESS;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Direct route: out[n, m] = sum_k dequant(W[m, k]) * (float)x_f16[n, k], fp32 accumulate.
 // Counterpart of cpu_vec_dot_{q4_0,q4_1,q5_0,q5_1,q8_0,q4_k}_f16 (vec_dot_impl.h:220-286, 351-450, 973-1023): the same
@@ -334,6 +348,22 @@ int marmot_hip_matmul_quantized(marmot_hip_device_t *dev, int kind, const void *
     }
     return matmul_impl(dev, kind, d_weight, nullptr, d_input, in_dtype, N, K, M, d_bias, bias_dtype, d_out, nullptr,
                        out_dtype, flags);
+}
+
+int marmot_hip_matmul_quantized_noalloc(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_input,
+                                        int in_dtype, size_t N, size_t K, size_t M, const void *d_bias,
+                                        int bias_dtype, void *d_out, int out_dtype, uint32_t flags) {
+    int st = validate_matmul(dev, kind, d_weight, d_input, in_dtype, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
+    if (st != MARMOT_HIP_SUCCESS) {
+        return st;
+    }
+    // same routes and kernels as marmot_hip_matmul_quantized; every scratch request of the call is served from this
+    // device's copy of the static array (or refused when it is larger)
+    dev->use_static_scratch = true;
+    st = matmul_impl(dev, kind, d_weight, nullptr, d_input, in_dtype, N, K, M, d_bias, bias_dtype, d_out, nullptr,
+                     out_dtype, flags);
+    dev->use_static_scratch = false;
+    return st;
 }
 
 size_t marmot_hip_packed_activation_bytes(int weight_kind, size_t N, size_t K) {

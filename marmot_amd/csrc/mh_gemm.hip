@@ -9,15 +9,21 @@
 // and then y += d*P - dmin*Q in fp32 on the vector ALU. The result differs from the reference only by fp32
 // rounding / summation order.
 //
-// Tiling. A workgroup (8 wavefronts, two per SIMD) owns 128 tokens x 256 weight rows; each wavefront owns 128 x 32
-// as 4 MFMA tiles, so one unpacked weight operand feeds 4 MFMAs and everything fits in 256 VGPRs without AGPRs.
-// While one wavefront of a SIMD applies the per-block scales on the vector ALU, the other keeps the matrix core busy.
-// The activation tile of a block (64 KiB) is gathered straight from the row-major fp16 matrix into LDS in MFMA
-// operand order with direct-to-LDS loads, double buffered, and shared by the 8 wavefronts. Weights are read
-// straight from their GGUF blocks into registers, one block ahead, and unpacked with
-// (q | 0x6400) as fp16 = 1024 + q, then fma(1024 + q, sc, -1024 * sc) = sc * q exactly.
-// K is split across workgroups when there are too few tiles to fill the chip; partial sums meet in a small
-// second kernel in a fixed order.
+// Tiling. Eight wavefronts per workgroup, two per SIMD; a wavefront owns 32 weight rows x (32 TA) tokens as TA MFMA
+// tiles, so one unpacked weight operand feeds TA MFMAs. Two shapes:
+//   * TA = 4, KG = 1: 128 tokens x 256 weight rows per workgroup, every wavefront walks all blocks of K: long prompts.
+//   * TA = 2, KG = 2: 64 tokens x 128 weight rows; wavefronts 0..3 take the even blocks of K and 4..7 the odd ones
+//     (each group stages its own activation tiles) and the two partial tiles meet in LDS at the end. 512 tokens x 4096
+//     rows are 256 such tiles: the chip is full without splitting K across workgroups, so no partial sums go through
+//     memory and no reduction kernel runs.
+// The activation tile of a block is gathered straight from the row-major fp16 matrix into LDS in MFMA operand order
+// with direct-to-LDS loads, double buffered. The sub-block sums S_j are computed from that staged tile by the
+// workgroup itself (v_dot2_f32_f16 against (1, 1): exact products, fp32 accumulation) into the stage's own S area;
+// the Q product of a block is taken one block later, behind the barrier that ends the block, so the sums need no
+// barrier of their own. Weights are read straight from their GGUF blocks into registers, one block ahead, and unpacked
+// with (q | 0x6400) as fp16 = 1024 + q, then fma(1024 + q, sc, -1024 * sc) = sc * q exactly.
+// K is split across workgroups only when there are too few tiles to fill the chip (short prompts); those partial sums
+// meet in a small second kernel in a fixed order.
 #include "mh_common.h"
 
 #include <stdlib.h>
@@ -25,59 +31,33 @@
 namespace mh {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int G_TOK = 128;        // tokens per workgroup tile
-constexpr int G_WROWS_WAVE = 32;  // weight rows per wavefront
 constexpr int G_WAVES = 8;
 constexpr int G_THREADS = G_WAVES * 64;
-constexpr int G_WROWS_WG = G_WROWS_WAVE * G_WAVES;  // 256 weight rows per workgroup
-constexpr int STAGE_A = 16 * 4 * 64 * 16;  // 16 K-steps x 4 token sub-tiles x 64 lanes x 16 bytes
-constexpr int STAGE_S = 4 * 64 * 16;       // sub-block sums operand: 4 token sub-tiles x 64 lanes x 16 bytes
-constexpr int STAGE = STAGE_A + STAGE_S;   // 69,632 bytes per (token tile, block)
-constexpr int STAGE_CHUNKS = STAGE / 16;   // 4352
+constexpr int G_WROWS_WAVE = 32;  // weight rows per wavefront
 
-// ------------------------------------------------------------------ sub-block sums of the activations
-// S operand of (token tile tt, block b, token sub-tile a): lane (i = lane % 32, kh = lane / 32), slot e:
-//     kh == 0 ? hi : lo   of   (fp32 sum of X[128*tt + 32*a + i][256*b + 32*e .. +32]) / 32,   hi + lo in fp16.
-// Tokens beyond N give zeros. One thread per (token, block, sub-block).
-__global__ __launch_bounds__(256) void k_gemm_sums(const uint16_t *__restrict__ x, size_t N, size_t K, size_t nb,
-                                                   uint8_t *__restrict__ sums) {
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t tiles = (N + G_TOK - 1) / G_TOK;
-    if (idx >= tiles * G_TOK * nb * 8) {
-        return;
-    }
-    const int e = (int)(idx & 7);
-    const size_t b = (idx >> 3) % nb;
-    const size_t token = (idx >> 3) / nb;
-    float s = 0.0f;
-    if (token < N) {
-        const uint4 *p = (const uint4 *)(x + token * K + b * 256 + 32 * e);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint4 v = p[c];
-            s += ((h2f((uint16_t)(v.x & 0xffffu)) + h2f((uint16_t)(v.x >> 16))) +
-                  (h2f((uint16_t)(v.y & 0xffffu)) + h2f((uint16_t)(v.y >> 16)))) +
-                ((h2f((uint16_t)(v.z & 0xffffu)) + h2f((uint16_t)(v.z >> 16))) +
-                 (h2f((uint16_t)(v.w & 0xffffu)) + h2f((uint16_t)(v.w >> 16))));
-        }
-    }
-    s *= 0.03125f;  // exact; keeps the value within fp16 range whatever the activations are
-    const uint16_t hi = f2h(s);
-    const uint16_t lo = f2h(s - h2f(hi));
-    const size_t tt = token / G_TOK;
-    const int a = (int)(token % G_TOK) >> 5, i = (int)(token & 31);
-    uint16_t *base = (uint16_t *)(sums + ((tt * nb + b) * 4 + a) * 1024);
-    base[(size_t)i * 8 + e] = hi;         // lane i       (kh = 0)
-    base[(size_t)(32 + i) * 8 + e] = lo;  // lane 32 + i  (kh = 1)
-}
+template <int TA, int KG>
+struct GemmShape {
+    static constexpr int TOK = 32 * TA;                   // tokens per workgroup tile
+    static constexpr int RG = G_WAVES / KG;               // row groups (wavefronts side by side along the weight rows)
+    static constexpr int WROWS = G_WROWS_WAVE * RG;       // weight rows per workgroup
+    static constexpr int GT = G_THREADS / KG;             // threads of one K group
+    static constexpr int STAGE_A = 16 * TA * 64 * 16;     // 16 K-steps x TA token sub-tiles x 64 lanes x 16 bytes
+    static constexpr int STAGE_S = TA * 64 * 16;          // sub-block sums operand: TA token sub-tiles x 64 lanes x 16 B
+    static constexpr int STAGE = STAGE_A + STAGE_S;
+    static constexpr int PIECES = STAGE_A / 16 / GT;      // direct-to-LDS pieces per thread and block
+    static constexpr int LDS_BYTES = KG * 2 * STAGE;
+    static_assert(PIECES * GT * 16 == STAGE_A, "the tile is staged in whole instructions");
+    static_assert(GT == 4 * TOK, "two (token, sub-block pair) runs per thread in the sums pass");
+};
 
 // ------------------------------------------------------------------ main kernel
 struct GemmParams {
     const uint8_t *w;       // Q4_K blocks, M rows of nb blocks
     const uint16_t *x;      // fp16 activations [N, K], row-major
-    const uint8_t *sums;    // sub-block sums operand (k_gemm_sums)
+    const uint8_t *sums;    // sub-block sums operand (k_gemm_sums), 128 x 256 tiles only
     size_t K;
     void *out;              // fp32/fp16 [N, M] (splits == 1) or fp32 partials [splits, N, M]
     const void *bias;
@@ -124,12 +104,6 @@ __device__ __forceinline__ void decode_header(const uint4 &hdr, Scales &s) {
     s.mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
 }
 
-// (v, v) as fp16 pair for an integer 0 <= v < 1024
-__device__ __forceinline__ __half2 int_pair(uint32_t v) {
-    const __half2 magic = as_h2(0x64006400u | v | (v << 16));  // (1024 + v, 1024 + v)
-    return __hsub2(magic, as_h2(0x64006400u));
-}
-
 // Two of the 8 weights of one K-step as fp16 sc*q: bytes (2*(I%2), 2*(I%2)+1) of the masked nibble dword m
 template <int I>
 __device__ __forceinline__ uint32_t dequant_pair(uint32_t m, __half2 sc, __half2 c) {
@@ -138,7 +112,67 @@ __device__ __forceinline__ uint32_t dequant_pair(uint32_t m, __half2 sc, __half2
     return as_u32(__hfma2(as_h2(t), sc, c));
 }
 
-__global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) {
+// the B operand of the Q product: (32 * mn_e) for the 8 sub-blocks, the same in both halves of the wavefront
+__device__ __forceinline__ half8 mins_operand(uint32_t lo, uint32_t hi) {
+    uint4 r;
+    const __half2 k32 = as_h2(0x50005000u);  // (32, 32)
+    const __half2 m1024 = as_h2(0x64006400u);
+    const uint32_t magic = 0x64646464u;
+    r.x = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, lo, 0x04010400u)), m1024), k32));
+    r.y = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, lo, 0x04030402u)), m1024), k32));
+    r.z = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, hi, 0x04010400u)), m1024), k32));
+    r.w = as_u32(__hmul2(__hsub2(as_h2(__builtin_amdgcn_perm(magic, hi, 0x04030402u)), m1024), k32));
+    return __builtin_bit_cast(half8, r);
+}
+
+// ------------------------------------------------------------------ long prompts: 128 tokens x 256 weight rows
+// The workgroup tile that fills the chip by itself from about 2048 tokens on. Every wavefront walks all blocks of K with
+// four MFMA tiles per unpacked weight operand; its 254 registers leave no room for the in-kernel sums, so the sub-block
+// sums of the activations come from a small kernel of their own and are staged next to the activation tile.
+constexpr int B_TOK = 128;        // tokens per workgroup tile
+constexpr int B_WROWS_WG = G_WROWS_WAVE * G_WAVES;  // 256 weight rows per workgroup
+constexpr int B_STAGE_A = 16 * 4 * 64 * 16;  // 16 K-steps x 4 token sub-tiles x 64 lanes x 16 bytes
+constexpr int B_STAGE_S = 4 * 64 * 16;       // sub-block sums operand: 4 token sub-tiles x 64 lanes x 16 bytes
+constexpr int B_STAGE = B_STAGE_A + B_STAGE_S;   // 69,632 bytes per (token tile, block)
+constexpr int B_STAGE_CHUNKS = B_STAGE / 16;   // 4352
+
+// ------------------------------------------------------------------ sub-block sums of the activations
+// S operand of (token tile tt, block b, token sub-tile a): lane (i = lane % 32, kh = lane / 32), slot e:
+//     kh == 0 ? hi : lo   of   (fp32 sum of X[128*tt + 32*a + i][256*b + 32*e .. +32]) / 32,   hi + lo in fp16.
+// Tokens beyond N give zeros. One thread per (token, block, sub-block).
+__global__ __launch_bounds__(256) void k_gemm_sums(const uint16_t *__restrict__ x, size_t N, size_t K, size_t nb,
+                                                   uint8_t *__restrict__ sums) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t tiles = (N + B_TOK - 1) / B_TOK;
+    if (idx >= tiles * B_TOK * nb * 8) {
+        return;
+    }
+    const int e = (int)(idx & 7);
+    const size_t b = (idx >> 3) % nb;
+    const size_t token = (idx >> 3) / nb;
+    float s = 0.0f;
+    if (token < N) {
+        const uint4 *p = (const uint4 *)(x + token * K + b * 256 + 32 * e);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint4 v = p[c];
+            s += ((h2f((uint16_t)(v.x & 0xffffu)) + h2f((uint16_t)(v.x >> 16))) +
+                  (h2f((uint16_t)(v.y & 0xffffu)) + h2f((uint16_t)(v.y >> 16)))) +
+                ((h2f((uint16_t)(v.z & 0xffffu)) + h2f((uint16_t)(v.z >> 16))) +
+                 (h2f((uint16_t)(v.w & 0xffffu)) + h2f((uint16_t)(v.w >> 16))));
+        }
+    }
+    s *= 0.03125f;  // exact; keeps the value within fp16 range whatever the activations are
+    const uint16_t hi = f2h(s);
+    const uint16_t lo = f2h(s - h2f(hi));
+    const size_t tt = token / B_TOK;
+    const int a = (int)(token % B_TOK) >> 5, i = (int)(token & 31);
+    uint16_t *base = (uint16_t *)(sums + ((tt * nb + b) * 4 + a) * 1024);
+    base[(size_t)i * 8 + e] = hi;         // lane i       (kh = 0)
+    base[(size_t)(32 + i) * 8 + e] = lo;  // lane 32 + i  (kh = 1)
+}
+
+__global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16_big(const GemmParams p) {
     warm_kernel_arguments<sizeof(GemmParams)>();
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // 2 stages
     const int tid = threadIdx.x;
@@ -146,7 +180,7 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
     const int wave = tid >> 6;
     const int j = lane & 31, kh = lane >> 5;
     const size_t tt = blockIdx.y;
-    const size_t wrow0 = (size_t)blockIdx.x * G_WROWS_WG + (size_t)wave * G_WROWS_WAVE;
+    const size_t wrow0 = (size_t)blockIdx.x * B_WROWS_WG + (size_t)wave * G_WROWS_WAVE;
     const int split = blockIdx.z;
     const size_t b0 = (size_t)split * p.blocks_per_split;
     size_t b1 = b0 + p.blocks_per_split;
@@ -177,15 +211,15 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
     // global reads are two contiguous 512-byte rows; the slot swizzle makes the MFMA operand reads below (16 tokens
     // x the same chunk) fall into 16 different bank groups. Tokens beyond N re-read token N-1 (never stored).
     uint32_t gather_off[9];  // byte offset of this thread's piece from the tile's first row, block-independent
-    const uint8_t *tile_x = (const uint8_t *)(p.x + tt * G_TOK * p.K);
+    const uint8_t *tile_x = (const uint8_t *)(p.x + tt * B_TOK * p.K);
 #pragma unroll
     for (int c = 0; c < 9; ++c) {
         const int chunk = tid + G_THREADS * c;
-        if (chunk < STAGE_A / 16) {
+        if (chunk < B_STAGE_A / 16) {
             const int t = chunk >> 5, slot = chunk & 31;
             size_t trow = t;
-            if (tt * G_TOK + trow >= p.N) {
-                trow = p.N - 1 - tt * G_TOK;
+            if (tt * B_TOK + trow >= p.N) {
+                trow = p.N - 1 - tt * B_TOK;
             }
             gather_off[c] = (uint32_t)(trow * p.K * 2 + 16 * (slot ^ (t & 15)));
         } else {
@@ -195,12 +229,12 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
     auto stage_piece = [&](size_t b, uint8_t *dst, int c) {
         const int chunk = tid + G_THREADS * c;
         const int wbase = chunk - lane;  // first chunk of this wavefront's instruction
-        if (wbase < STAGE_CHUNKS) {      // wave-uniform
+        if (wbase < B_STAGE_CHUNKS) {      // wave-uniform
             const uint8_t *g;
-            if (chunk < STAGE_A / 16) {
+            if (chunk < B_STAGE_A / 16) {
                 g = tile_x + gather_off[c] + b * 512;
             } else {
-                g = p.sums + (tt * p.nb + b) * STAGE_S + (size_t)(chunk - STAGE_A / 16) * 16;
+                g = p.sums + (tt * p.nb + b) * B_STAGE_S + (size_t)(chunk - B_STAGE_A / 16) * 16;
             }
             uint8_t *l = dst + (size_t)wbase * 16;  // wave-uniform base; the hardware adds lane * 16
             __builtin_amdgcn_global_load_lds((glb_u8 *)g, (lds_u8 *)l, 16, 0, 0);
@@ -230,7 +264,7 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
 
     for (size_t b = b0; b < b1; ++b) {
         const int cur = (int)((b - b0) & 1);
-        const uint8_t *stage = lds + (size_t)cur * STAGE;
+        const uint8_t *stage = lds + (size_t)cur * B_STAGE;
         const bool more = b + 1 < b1;
 
         const WeightRegs wcur = wnext;
@@ -238,7 +272,7 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
         decode_header(wcur.hdr, sc);
         // The next block's activations (straight into the other LDS stage) and weights (into registers) are
         // requested from inside the K loop.
-        uint8_t *next_stage = lds + (size_t)(cur ^ 1) * STAGE;
+        uint8_t *next_stage = lds + (size_t)(cur ^ 1) * B_STAGE;
         const uint8_t *next_blk = wrow + (b + 1) * Q4_K_BYTES;
         auto prefetch_piece = [&](int ks) {
             if (!more) {
@@ -351,7 +385,7 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
         half8 a2[4];
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
-            a2[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + STAGE_A + ((size_t)a * 64 + lane) * 16));
+            a2[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + B_STAGE_A + ((size_t)a * 64 + lane) * 16));
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -381,7 +415,7 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
     if (m >= p.M) {
         return;
     }
-    const size_t n0 = tt * G_TOK + 4 * kh;
+    const size_t n0 = tt * B_TOK + 4 * kh;
     if (p.splits > 1) {
         float *dst = (float *)p.out + (size_t)split * p.N * p.M + m;
 #pragma unroll
@@ -414,6 +448,351 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
         uint16_t *dst = (uint16_t *)p.out + m;
 #pragma unroll
         for (int a = 0; a < 4; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
+                if (n < p.N) {
+                    uint16_t h = f2h(total[a][r]);  // round to the output type first, then add the bias in it
+                    if (has_bias) {
+                        h = f2h(h2f(h) + bias);
+                    }
+                    dst[n * p.M] = h;
+                }
+            }
+        }
+    }
+}
+
+
+template <int TA, int KG>
+__global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) {
+    using S = GemmShape<TA, KG>;
+    warm_kernel_arguments<sizeof(GemmParams)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // KG x 2 stages
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int kg = wave / S::RG;          // K group of this wavefront
+    const int rgp = wave % S::RG;         // its row group
+    const int gt = rgp * 64 + lane;       // thread index inside the K group
+    const int j = lane & 31, kh = lane >> 5;
+    const size_t tt = blockIdx.y;
+    const size_t wrow0 = (size_t)blockIdx.x * S::WROWS + (size_t)rgp * G_WROWS_WAVE;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    size_t wr = wrow0 + j;
+    if (wr >= p.M) {
+        wr = p.M - 1;  // harmless re-read; never stored
+    }
+    const uint8_t *wrow = p.w + wr * p.nb * Q4_K_BYTES;
+    uint8_t *const my_stages = lds + (size_t)kg * 2 * S::STAGE;
+
+    floatx16 total[TA];
+#pragma unroll
+    for (int a = 0; a < TA; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
+        }
+    }
+
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    typedef const __attribute__((address_space(1))) uint8_t glb_u8;
+    // One stage is moved global -> LDS with direct-to-LDS loads: every wavefront instruction moves 64 lanes x 16 bytes
+    // from per-lane global addresses to a contiguous 1 KiB of LDS (no registers involved); vmcnt tracks completion.
+    // LDS layout of the activation part: token t of the tile owns 512 bytes (its 256 halves of this block) as 32
+    // chunks of 16 bytes, chunk c stored in slot c ^ (t % 16). One instruction covers tokens 2q and 2q+1, so its
+    // global reads are two contiguous 512-byte rows; the slot swizzle makes the MFMA operand reads below (16 tokens
+    // x the same chunk) fall into 16 different bank groups. Tokens beyond N re-read token N-1 (never stored).
+    // The byte offset of a thread's piece from the tile's first row is recomputed when the piece is requested (a few
+    // integer operations per block) instead of living in registers through the K loop.
+    const uint8_t *tile_x = (const uint8_t *)(p.x + tt * S::TOK * p.K);
+    const uint32_t row_pitch = (uint32_t)(p.K * 2);
+    const uint32_t last_row = (uint32_t)(p.N - 1 - tt * S::TOK);  // rows beyond it re-read it
+    auto stage_piece = [&](size_t b, uint8_t *dst, int c) {
+        const int chunk = gt + S::GT * c;
+        const int t = chunk >> 5, slot = chunk & 31;
+        const uint32_t trow = (uint32_t)t < last_row ? (uint32_t)t : last_row;
+        const uint8_t *g = tile_x + (size_t)trow * row_pitch + 16 * (slot ^ (t & 15)) + b * 512;
+        uint8_t *l = dst + (size_t)(chunk - lane) * 16;  // wave-uniform base; the hardware adds lane * 16
+        __builtin_amdgcn_global_load_lds((glb_u8 *)g, (lds_u8 *)l, 16, 0, 0);
+    };
+    // MFMA A operand of K-step ks, token sub-tile a, lane (i = j, kh): token 32a + i, chunk 4(ks/2) + 2kh + ks%2.
+    // Per-lane part of its LDS offset for the 8 combinations of ((ks/2) % 4, ks % 2); the rest is a constant.
+    uint32_t a_off[4][2];
+#pragma unroll
+    for (int s3 = 0; s3 < 4; ++s3) {
+#pragma unroll
+        for (int tp = 0; tp < 2; ++tp) {
+            a_off[s3][tp] = (uint32_t)(j * 512 + 16 * ((4 * s3 + 2 * kh + tp) ^ (j & 15)));
+        }
+    }
+    // Sums pass: this thread adds up two neighbouring sub-blocks (64 halves = 8 chunks) of one token of the staged tile.
+    const int sum_token = gt % S::TOK, sum_pair = gt / S::TOK;  // sub-blocks 2 sum_pair and 2 sum_pair + 1
+    const uint32_t sum_src = (uint32_t)(sum_token * 512);
+    const uint32_t sum_dst = (uint32_t)(S::STAGE_A + (sum_token >> 5) * 1024 + (sum_token & 31) * 16 + 4 * sum_pair);
+
+    const size_t first = b0 + (size_t)kg;  // this K group's blocks: first, first + KG, ...
+    WeightRegs wnext;
+    if (first < b1) {
+#pragma unroll
+        for (int c = 0; c < S::PIECES; ++c) {
+            stage_piece(first, my_stages, c);
+        }
+        load_weights(wnext, wrow + first * Q4_K_BYTES, kh);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    uint32_t prev_mn_lo = 0, prev_mn_hi = 0;
+    float prev_ndmin = 0.0f;
+    bool have_prev = false;
+    int cur = 0;
+    // Q product of the block whose sums sit in `stage_s` (written one block ago): total -= dmin * (S x mins)
+    auto q_term = [&](const uint8_t *stage_s, uint32_t mn_lo, uint32_t mn_hi, float ndmin) {
+        const half8 b2 = mins_operand(mn_lo, mn_hi);
+#pragma unroll
+        for (int a = 0; a < TA; ++a) {
+            const half8 a2 = __builtin_bit_cast(half8, *(const uint4 *)(stage_s + ((size_t)a * 64 + lane) * 16));
+            const floatx16 zero = {0};
+            const floatx16 mq = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                total[a][r] = __builtin_fmaf(ndmin, mq[r], total[a][r]);
+            }
+        }
+    };
+
+    // the loop runs the same number of times in both K groups (barriers inside): a group without a block idles through
+    const size_t rounds = (b1 - b0 + KG - 1) / KG;
+    for (size_t round = 0; round < rounds; ++round) {
+        const size_t b = first + round * KG;
+        const bool mine = b < b1;
+        uint8_t *stage = my_stages + (size_t)cur * S::STAGE;
+        uint8_t *other = my_stages + (size_t)(cur ^ 1) * S::STAGE;
+        const bool more = b + KG < b1;
+        if (mine) {
+            // ---- sums of this block's tile into the stage's S area (read by the Q product one block later)
+            {
+                float s0 = 0.0f, s1 = 0.0f;
+                const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const uint4 v = *(const uint4 *)(stage + sum_src + 16 * ((8 * sum_pair + c) ^ (sum_token & 15)));
+                    float acc = c < 4 ? s0 : s1;
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.x), ones, acc, false);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.y), ones, acc, false);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.z), ones, acc, false);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.w), ones, acc, false);
+                    if (c < 4) {
+                        s0 = acc;
+                    } else {
+                        s1 = acc;
+                    }
+                }
+                s0 *= 0.03125f;  // exact; keeps the value within fp16 range whatever the activations are
+                s1 *= 0.03125f;
+                const uint16_t h0 = f2h(s0), h1 = f2h(s1);
+                const uint16_t l0 = f2h(s0 - h2f(h0)), l1 = f2h(s1 - h2f(h1));
+                // S operand of token sub-tile a: lane i (kh = 0) holds the 8 hi parts of token 32a + i, lane 32 + i the lo parts
+                *(uint32_t *)(stage + sum_dst) = (uint32_t)h0 | ((uint32_t)h1 << 16);
+                *(uint32_t *)(stage + sum_dst + 512) = (uint32_t)l0 | ((uint32_t)l1 << 16);
+            }
+
+            const WeightRegs wcur = wnext;
+            Scales sc;
+            decode_header(wcur.hdr, sc);
+            // The next block's activations (straight into the other LDS stage) and weights (into registers) are
+            // requested from inside the K loop.
+            const uint8_t *next_blk = wrow + (b + KG) * Q4_K_BYTES;
+            auto prefetch_piece = [&](int ks) {
+                if (!more) {
+                    return;
+                }
+                // Weights (into registers) early, one load per K-step. The activation tile (direct-to-LDS) as late as
+                // possible, all pieces in the last K-step. Measured with the cycle counter: a load issued inside the K
+                // loop costs its wavefront about 230 clocks (the eight wavefronts issue in the same K-step, and one
+                // that is held at the memory issue stage holds back its own MFMA chain), while the wait at the end of
+                // the block is barrier skew and does not get shorter when the tile was requested earlier.
+                if (ks == 15) {
+#pragma unroll
+                    for (int c = 0; c < S::PIECES; ++c) {
+                        stage_piece(b + KG, other, c);
+                    }
+                } else if (ks == 1) {
+                    wnext.hdr = *(const uint4 *)next_blk;
+                } else if (ks >= 2 && ks < 6) {
+                    wnext.q[ks - 2] = *(const uint4 *)(next_blk + 16 + 32 * (ks - 2) + 16 * kh);
+                }
+            };
+
+            // Operand B of K-step ks is built in 4 pieces spread over the MFMAs of the previous K-step, so that the
+            // unpack arithmetic runs in the shadow of the matrix core. The scheduling fences pin that order.
+            __half2 scp, cp;
+            uint32_t m0 = 0, m1 = 0;
+            auto b_piece = [&](int ks, int i) -> uint32_t {
+                const int s_ = ks >> 1, tp = ks & 1, g = s_ >> 1;
+                if (i == 0) {
+                    if (tp == 0) {
+                        const uint32_t scw = s_ < 4 ? sc.sc_lo : sc.sc_hi;
+                        // (1024 + sc, 1024 + sc) - (1024, 1024)
+                        const uint32_t sel = (s_ & 3) == 0 ? 0x04000400u : (s_ & 3) == 1 ? 0x04010401u
+                                           : (s_ & 3) == 2 ? 0x04020402u : 0x04030403u;
+                        scp = __hsub2(as_h2(__builtin_amdgcn_perm(0x64646464u, scw, sel)), as_h2(0x64006400u));
+                        cp = __hmul2(scp, as_h2(0xe400e400u));  // -1024 * sc, exact
+                    }
+                    const uint32_t q0 = tp ? wcur.q[g].z : wcur.q[g].x;
+                    const uint32_t q1 = tp ? wcur.q[g].w : wcur.q[g].y;
+                    m0 = ((s_ & 1) ? (q0 >> 4) : q0) & 0x0f0f0f0fu;
+                    m1 = ((s_ & 1) ? (q1 >> 4) : q1) & 0x0f0f0f0fu;
+                }
+                switch (i) {
+                case 0: return dequant_pair<0>(m0, scp, cp);
+                case 1: return dequant_pair<1>(m0, scp, cp);
+                case 2: return dequant_pair<0>(m1, scp, cp);
+                default: return dequant_pair<1>(m1, scp, cp);
+                }
+            };
+            auto read_a = [&](int ks, half8(&aop)[TA]) {
+#pragma unroll
+                for (int a = 0; a < TA; ++a) {
+                    aop[a] = __builtin_bit_cast(
+                        half8, *(const uint4 *)(stage + a_off[(ks >> 1) & 3][ks & 1] + (a * 16384 + 256 * (ks >> 3))));
+                }
+            };
+
+            floatx16 acc[TA];
+            half8 aop[2][TA];  // A operands of the K-step in flight and of the next one
+            uint32_t bop[2][4];
+            read_a(0, aop[0]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                bop[0][i] = b_piece(0, i);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < 16; ++ks) {
+                const int c = ks & 1, n = c ^ 1;
+                if (ks < 15) {
+                    read_a(ks + 1, aop[n]);  // lands while the MFMAs below run
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const half8 bcur = __builtin_bit_cast(half8, make_uint4(bop[c][0], bop[c][1], bop[c][2], bop[c][3]));
+#pragma unroll
+                for (int a = 0; a < TA; ++a) {
+                    if (ks == 0) {
+                        const floatx16 zero = {0};
+                        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, zero, 0, 0, 0);
+                    } else {
+                        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, acc[a], 0, 0, 0);
+                    }
+                    if (ks < 15) {
+#pragma unroll
+                        for (int i = a * (4 / TA); i < (a + 1) * (4 / TA); ++i) {
+                            bop[n][i] = b_piece(ks + 1, i);
+                        }
+                    }
+                    if (a == (TA > 1 ? 1 : 0)) {
+                        prefetch_piece(ks);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // per-block scale of the P product, and the Q product of the previous block of this K group
+            const float d = sc.d;
+#pragma unroll
+            for (int a = 0; a < TA; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    total[a][r] = __builtin_fmaf(d, acc[a][r], total[a][r]);
+                }
+            }
+            if (have_prev) {
+                q_term(other + S::STAGE_A, prev_mn_lo, prev_mn_hi, prev_ndmin);
+            }
+            prev_mn_lo = sc.mn_lo;
+            prev_mn_hi = sc.mn_hi;
+            prev_ndmin = -sc.dmin;
+            have_prev = true;
+        }
+        __builtin_amdgcn_s_waitcnt(0);  // the next stage's direct-to-LDS loads have landed, this stage's sums are stored
+        __syncthreads();
+        cur ^= 1;
+    }
+    if (have_prev) {  // the last block's sums sit in the stage that was current in the last round with a block
+        const size_t mine_rounds = first < b1 ? (b1 - first + KG - 1) / KG : 0;
+        const int last_stage = (int)((mine_rounds - 1) & 1);
+        q_term(my_stages + (size_t)last_stage * S::STAGE + S::STAGE_A, prev_mn_lo, prev_mn_hi, prev_ndmin);
+    }
+
+    if (KG > 1) {
+        // the K groups' partial tiles meet in LDS: group 1 stores, group 0 adds and goes on to the epilogue
+        __syncthreads();  // every wavefront is done with the stages
+        float *red = (float *)lds + (size_t)rgp * TA * 16 * 64 + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int a = 0; a < TA; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    red[(a * 16 + r) * 64] = total[a][r];
+                }
+            }
+        }
+        __syncthreads();
+        if (kg != 0) {
+            return;
+        }
+#pragma unroll
+        for (int a = 0; a < TA; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                total[a][r] += red[(a * 16 + r) * 64];
+            }
+        }
+    }
+
+    // epilogue: lane (j, kh) holds weight row m = wrow0 + j for tokens 32a + 8(r/4) + 4kh + r%4
+    const size_t m = wrow0 + j;
+    if (m >= p.M) {
+        return;
+    }
+    const size_t n0 = tt * S::TOK + 4 * kh;
+    if (p.splits > 1) {
+        float *dst = (float *)p.out + (size_t)split * p.N * p.M + m;
+#pragma unroll
+        for (int a = 0; a < TA; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
+                if (n < p.N) {
+                    dst[n * p.M] = total[a][r];
+                }
+            }
+        }
+    } else if (!p.out_is_f16) {
+        const float bias = p.bias != nullptr ? ((const float *)p.bias)[m] : 0.0f;
+        float *dst = (float *)p.out + m;
+#pragma unroll
+        for (int a = 0; a < TA; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
+                if (n < p.N) {
+                    dst[n * p.M] = total[a][r] + bias;
+                }
+            }
+        }
+    } else {
+        const bool has_bias = p.bias != nullptr;
+        const float bias = !has_bias ? 0.0f
+            : p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m]) : ((const float *)p.bias)[m];
+        uint16_t *dst = (uint16_t *)p.out + m;
+#pragma unroll
+        for (int a = 0; a < TA; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const size_t n = n0 + 32 * a + 8 * (r >> 2) + (r & 3);
@@ -516,6 +895,86 @@ bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M) {
     return kind == MARMOT_HIP_KIND_Q4_K && N > 8 && K % QK_K == 0 && M >= 1;
 }
 
+template <int TA, int KG>
+static int launch_gemm_shape(marmot_hip_device *dev, GemmParams p, size_t N, size_t K, size_t M, const void *d_bias,
+                             int bias_dtype, void *d_out, int out_dtype) {
+    using S = GemmShape<TA, KG>;
+    const size_t nb = K / QK_K;
+    const size_t tiles_n = (N + S::TOK - 1) / S::TOK;
+    const size_t tiles_m = (M + S::WROWS - 1) / S::WROWS;
+    const size_t tiles = tiles_n * tiles_m;
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    size_t splits = 1;
+    if (tiles * 2 <= cus) {  // fewer tiles than half the chip: split K across workgroups (short prompts)
+        splits = cus / tiles;
+        const size_t max_splits = nb / (2 * KG) > 0 ? nb / (2 * KG) : 1;  // at least two blocks per K group
+        splits = splits > max_splits ? max_splits : splits;
+    }
+    if (const char *e = getenv("MH_GEMM_SPLITS")) {
+        splits = (size_t)atoi(e);
+        splits = splits < 1 ? 1 : (splits > nb ? nb : splits);
+    }
+    const size_t blocks_per_split = (nb + splits - 1) / splits;
+    splits = (nb + blocks_per_split - 1) / blocks_per_split;
+    float *partial = nullptr;
+    if (splits > 1) {
+        void *ws = nullptr;
+        MH_TRY(workspace_reserve(dev, splits * N * M * sizeof(float), &ws));
+        partial = (float *)ws;
+    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_f16<TA, KG>));
+    p.out = splits > 1 ? (void *)partial : d_out;
+    p.splits = (int)splits;
+    p.blocks_per_split = (int)blocks_per_split;
+    hipLaunchKernelGGL((k_gemm_q4k_f16<TA, KG>), dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits),
+                       dim3(G_THREADS), S::LDS_BYTES, dev->stream, p);
+    MH_HIP(hipGetLastError());
+    if (splits > 1) {
+        MH_TRY(launch_splitk_reduce(dev, partial, (int)splits, N, M, d_bias, bias_dtype, d_out, out_dtype));
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
+static int launch_gemm_big(marmot_hip_device *dev, GemmParams p, size_t N, size_t K, size_t M, const void *d_bias,
+                           int bias_dtype, void *d_out, int out_dtype) {
+    const size_t nb = K / QK_K;
+    const size_t tiles_n = (N + B_TOK - 1) / B_TOK;
+    const size_t tiles_m = (M + B_WROWS_WG - 1) / B_WROWS_WG;
+    const size_t tiles = tiles_n * tiles_m;
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    size_t splits = 1;
+    if (tiles < cus) {
+        splits = cus / tiles;
+        splits = splits > nb ? nb : (splits < 1 ? 1 : splits);
+    }
+    const size_t blocks_per_split = (nb + splits - 1) / splits;
+    splits = (nb + blocks_per_split - 1) / blocks_per_split;
+    const size_t sums_bytes = tiles_n * nb * B_STAGE_S;
+    const size_t partial_bytes = splits > 1 ? splits * N * M * sizeof(float) : 0;
+    void *ws = nullptr;
+    MH_TRY(workspace_reserve(dev, ((sums_bytes + 255) & ~(size_t)255) + partial_bytes, &ws));
+    uint8_t *sums = (uint8_t *)ws;
+    float *partial = (float *)((uint8_t *)ws + ((sums_bytes + 255) & ~(size_t)255));
+    {
+        const size_t total = tiles_n * B_TOK * nb * 8;
+        hipLaunchKernelGGL(k_gemm_sums, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream,
+                           (const uint16_t *)p.x, N, K, nb, sums);
+        MH_HIP(hipGetLastError());
+    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_f16_big));
+    p.sums = sums;
+    p.out = splits > 1 ? (void *)partial : d_out;
+    p.splits = (int)splits;
+    p.blocks_per_split = (int)blocks_per_split;
+    hipLaunchKernelGGL(k_gemm_q4k_f16_big, dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits),
+                       dim3(G_THREADS), 2 * B_STAGE, dev->stream, p);
+    MH_HIP(hipGetLastError());
+    if (splits > 1) {
+        MH_TRY(launch_splitk_reduce(dev, partial, (int)splits, N, M, d_bias, bias_dtype, d_out, out_dtype));
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
 int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                     const void *d_bias, int bias_dtype, void *d_out, int out_dtype) {
     if (!gemm_f16_supported(kind, N, K, M)) {
@@ -524,76 +983,31 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     if ((((uintptr_t)d_x) & 15) != 0) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "prefill GEMM: activations must be 16-byte aligned");
     }
-    const size_t nb = K / QK_K;
-    const size_t tiles_n = (N + G_TOK - 1) / G_TOK;
-    const size_t tiles_m = (M + G_WROWS_WG - 1) / G_WROWS_WG;
-    const size_t tiles = tiles_n * tiles_m;
-    const size_t cus = (size_t)dev->props.multiProcessorCount;
-    size_t splits = 1;
-    if (tiles < cus) {
-        splits = cus / tiles;
-        if (splits > nb) {
-            splits = nb;
-        }
-        if (splits < 1) {
-            splits = 1;
-        }
-    }
-    if (const char *e = getenv("MH_GEMM_SPLITS")) {
-        splits = (size_t)atoi(e);
-        if (splits < 1) {
-            splits = 1;
-        }
-        if (splits > nb) {
-            splits = nb;
-        }
-    }
-    const size_t blocks_per_split = (nb + splits - 1) / splits;
-    splits = (nb + blocks_per_split - 1) / blocks_per_split;
-
-    const size_t sums_bytes = tiles_n * nb * STAGE_S;
-    const size_t partial_bytes = splits > 1 ? splits * N * M * sizeof(float) : 0;
-    void *ws = nullptr;
-    int st = workspace_reserve(dev, ((sums_bytes + 255) & ~(size_t)255) + partial_bytes, &ws);
-    if (st != MARMOT_HIP_SUCCESS) {
-        return st;
-    }
-    uint8_t *sums = (uint8_t *)ws;
-    float *partial = (float *)((uint8_t *)ws + ((sums_bytes + 255) & ~(size_t)255));
-
-    {
-        const size_t total = tiles_n * G_TOK * nb * 8;
-        hipLaunchKernelGGL(k_gemm_sums, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dev->stream,
-                           (const uint16_t *)d_x, N, K, nb, sums);
-        MH_HIP(hipGetLastError());
-    }
-
-    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_f16));
     GemmParams p;
     p.w = (const uint8_t *)d_w;
     p.x = (const uint16_t *)d_x;
-    p.sums = sums;
+    p.sums = nullptr;
     p.K = K;
-    p.out = splits > 1 ? (void *)partial : d_out;
+    p.out = d_out;
     p.bias = d_bias;
     p.bias_is_f16 = bias_dtype == MARMOT_HIP_DTYPE_F16;
     p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
     p.N = N;
     p.M = M;
-    p.nb = nb;
-    p.splits = (int)splits;
-    p.blocks_per_split = (int)blocks_per_split;
-    hipLaunchKernelGGL(k_gemm_q4k_f16, dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits),
-                       dim3(G_THREADS), 2 * STAGE, dev->stream, p);
-    MH_HIP(hipGetLastError());
-    if (splits > 1) {
-        st = launch_splitk_reduce(dev, partial, (int)splits, N, M, d_bias, bias_dtype, d_out, out_dtype);
-        if (st != MARMOT_HIP_SUCCESS) {
-            return st;
-        }
-    }
+    p.nb = K / QK_K;
+    p.splits = 1;
+    p.blocks_per_split = (int)p.nb;
+    // Large tiles when they fill the chip by themselves (long prompts), the 64 x 128 tile with the K split inside the
+    // workgroup otherwise.
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    const size_t big_tiles = ((N + 127) / 128) * ((M + 255) / 256);
+    const char *force = getenv("MH_GEMM_SHAPE");
+    const bool big = force != nullptr ? atoi(force) == 4 : big_tiles >= cus;
     set_route("gemm_q4_k_f16_mfma");
-    return MARMOT_HIP_SUCCESS;
+    if (big) {
+        return launch_gemm_big(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
+    }
+    return launch_gemm_shape<2, 2>(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
 }
 
 } // namespace mh

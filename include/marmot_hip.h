@@ -284,6 +284,19 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
  * same split, so that several weights sharing one input (q/k/v, gate/up) pay for one quantization.
  * The packed buffer has a library-private layout; only its size is public. */
 size_t marmot_hip_packed_activation_bytes(int weight_kind, size_t N, size_t K);
+/* Where the parts of a packed buffer lie, for tests and tools that inspect or build one on the host. Row n holds
+ * values_per_row int8 values at values_offset + n*values_per_row (the row padded with zeros to whole blocks),
+ * blocks_per_row fp32 block scales at scales_offset + 4*n*blocks_per_row, and blocks_per_row*sums_per_block int16
+ * sums at sums_offset (Q8_K: the 16 sums of 16 values, marmot_q8_k_block_t.bsums; Q8_0: the sum of the block's 32
+ * values). The layout may change between versions of the library; the packed size is total_bytes. */
+typedef struct marmot_hip_packed_layout {
+    int act_kind; /* MARMOT_HIP_KIND_Q8_0 or MARMOT_HIP_KIND_Q8_K */
+    size_t total_bytes;
+    size_t values_offset, values_per_row;
+    size_t scales_offset, blocks_per_row;
+    size_t sums_offset, sums_per_block;
+} marmot_hip_packed_layout_t;
+int marmot_hip_packed_activation_layout(int weight_kind, size_t N, size_t K, marmot_hip_packed_layout_t *layout);
 int marmot_hip_pack_activations(marmot_hip_device_t *dev, int weight_kind, const void *d_input, int in_dtype,
                                 size_t N, size_t K, void *d_packed);
 int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *d_weight, const void *d_packed,
@@ -308,6 +321,29 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
                            size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate, const void *d_up,
                            const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
                            float weights_scale, int router_weight_policy, int ffn_type, float *d_out);
+
+/* The same call with its stages observable, for parity tests that check each stage of cpu_moe_experts_impl
+ * (moe_ops.c:951-1042: gate/up projections, the quantized GLU product, down projection + combine) against a CPU
+ * restatement instead of only the final sum. Every pointer may be null. Outputs are in expert-sorted route order
+ * (moe_ops.c:929-943); d_route_pos[t*k + j] is the sorted position of token t's j-th route, -1 if it was dropped.
+ *   d_sorted_tokens uint32 [T*k]; d_gate_out / d_up_out fp32 [T*k, F];
+ *   d_fused_packed: the packed activations of [T*k, F] the down projection reads, in the layout and size of
+ *     marmot_hip_pack_activations (see marmot_hip_packed_activation_layout) for kind_down;
+ *   d_fused_override: packed activations in the same layout that REPLACE them before the down projection.
+ * Not capturable into a graph (it copies with the runtime's copy engine). */
+typedef struct marmot_hip_moe_probe {
+    uint32_t *d_sorted_tokens;
+    int32_t *d_route_pos;
+    float *d_gate_out;
+    float *d_up_out;
+    void *d_fused_packed;
+    const void *d_fused_override;
+} marmot_hip_moe_probe_t;
+int marmot_hip_moe_experts_probe(marmot_hip_device_t *dev, const float *d_hidden, size_t T, size_t H, size_t F,
+                                 size_t E, size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate,
+                                 const void *d_up, const void *d_down, const int32_t *d_topk_ids,
+                                 const float *d_topk_weights, float weights_scale, int router_weight_policy,
+                                 int ffn_type, float *d_out, const marmot_hip_moe_probe_t *probe);
 
 /* ------------------------------------------------------------------ GGUF files
  * Replaces, for the weights of this path, marmot_gguf_load / marmot_gguf_find_tensor (src/graph/gguf/loader.cpp:577-770,

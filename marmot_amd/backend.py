@@ -386,6 +386,50 @@ class HipBackend:
             C.c_void_p(d_down.ptr + down_offset), C.c_void_p(d_ids.ptr), C.c_void_p(d_weights.ptr), weights_scale,
             policy, ffn_type, C.c_void_p(d_out.ptr)))
 
+    def packed_activation_layout(self, kind: int, N: int, K: int) -> "capi.PackedLayout":
+        lay = capi.PackedLayout()
+        check(self.lib.marmot_hip_packed_activation_layout(kind, N, K, C.byref(lay)))
+        return lay
+
+    def moe_experts_probe(self, hidden, gate, up, down, topk_ids, topk_weights, F: int, E: int, kind_gate_up: int,
+                          kind_down: int, weights_scale: float = 1.0, policy: int = 1, ffn_type: int = 0,
+                          fused_override: np.ndarray = None) -> dict:
+        """moe_experts with every stage read back: {"out", "sorted_tokens", "route_pos", "gate_out", "up_out",
+        "fused_packed" (uint8 image, see packed_activation_layout)}. `fused_override`, a packed image of the same
+        size, replaces the activations the down projection reads."""
+        hidden = np.ascontiguousarray(hidden, dtype=np.float32)
+        T, H = hidden.shape
+        ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
+        w = np.ascontiguousarray(topk_weights, dtype=np.float32)
+        kpt = ids.shape[1]
+        routes = T * kpt
+        packed_bytes = self.packed_activation_bytes(kind_down, routes, F)
+        ins = [self.to_device(a) for a in (hidden, np.ascontiguousarray(gate, dtype=np.uint8),
+                                           np.ascontiguousarray(up, dtype=np.uint8),
+                                           np.ascontiguousarray(down, dtype=np.uint8), ids, w)]
+        outs = [self.alloc(n) for n in (T * H * 4, routes * 4, routes * 4, routes * F * 4, routes * F * 4,
+                                        packed_bytes)]
+        if fused_override is not None:
+            fused_override = np.ascontiguousarray(fused_override, dtype=np.uint8)
+            assert fused_override.size == packed_bytes
+            ins.append(self.to_device(fused_override))
+        try:
+            probe = capi.MoeProbe(outs[1].ptr, outs[2].ptr, outs[3].ptr, outs[4].ptr, outs[5].ptr,
+                                  ins[6].ptr if fused_override is not None else None)
+            check(self.lib.marmot_hip_moe_experts_probe(
+                self.dev, C.c_void_p(ins[0].ptr), T, H, F, E, kpt, kind_gate_up, kind_down, C.c_void_p(ins[1].ptr),
+                C.c_void_p(ins[2].ptr), C.c_void_p(ins[3].ptr), C.c_void_p(ins[4].ptr), C.c_void_p(ins[5].ptr),
+                weights_scale, policy, ffn_type, C.c_void_p(outs[0].ptr), C.byref(probe)))
+            return {"out": outs[0].download(np.float32, (T, H)),
+                    "sorted_tokens": outs[1].download(np.uint32, (routes,)),
+                    "route_pos": outs[2].download(np.int32, (T, kpt)),
+                    "gate_out": outs[3].download(np.float32, (routes, F)),
+                    "up_out": outs[4].download(np.float32, (routes, F)),
+                    "fused_packed": outs[5].download(np.uint8, (packed_bytes,))}
+        finally:
+            for b in ins + outs:
+                b.free()
+
     def moe_experts(self, hidden, gate, up, down, topk_ids, topk_weights, F: int, E: int, kind_gate_up: int,
                     kind_down: int, weights_scale: float = 1.0, policy: int = 1, ffn_type: int = 0) -> np.ndarray:
         hidden = np.ascontiguousarray(hidden, dtype=np.float32)

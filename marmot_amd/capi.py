@@ -50,6 +50,19 @@ class GgufTensor(C.Structure):
                 ("ndim", C.c_uint32), ("shape", C.c_uint64 * 4), ("data", C.c_void_p), ("nbytes", C.c_size_t)]
 
 
+class MoeProbe(C.Structure):
+    """marmot_hip_moe_probe_t"""
+    _fields_ = [("d_sorted_tokens", C.c_void_p), ("d_route_pos", C.c_void_p), ("d_gate_out", C.c_void_p),
+                ("d_up_out", C.c_void_p), ("d_fused_packed", C.c_void_p), ("d_fused_override", C.c_void_p)]
+
+
+class PackedLayout(C.Structure):
+    """marmot_hip_packed_layout_t"""
+    _fields_ = [("act_kind", C.c_int), ("total_bytes", C.c_size_t), ("values_offset", C.c_size_t),
+                ("values_per_row", C.c_size_t), ("scales_offset", C.c_size_t), ("blocks_per_row", C.c_size_t),
+                ("sums_offset", C.c_size_t), ("sums_per_block", C.c_size_t)]
+
+
 _vp, _sz, _i, _u32, _f = C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_float
 
 # name -> (restype, argtypes); every symbol include/marmot_hip.h declares
@@ -100,6 +113,9 @@ SIGNATURES = {
     "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "marmot_hip_moe_experts": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i,
                                     _vp]),
+    "marmot_hip_moe_experts_probe": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i,
+                                          _i, _vp, C.POINTER(MoeProbe)]),
+    "marmot_hip_packed_activation_layout": (_i, [_i, _sz, _sz, C.POINTER(PackedLayout)]),
     "marmot_hip_last_route": (C.c_char_p, []),
     "marmot_hip_version": (C.c_char_p, []),
     "marmot_hip_gguf_open": (_i, [C.c_char_p, C.POINTER(_vp)]),

@@ -374,6 +374,25 @@ size_t marmot_hip_packed_activation_bytes(int weight_kind, size_t N, size_t K) {
     return act_scratch_layout(act_kind, N, K, nullptr, nullptr);
 }
 
+int marmot_hip_packed_activation_layout(int weight_kind, size_t N, size_t K, marmot_hip_packed_layout_t *layout) {
+    if (layout == nullptr || block_values(weight_kind) == 0 || weight_kind == MARMOT_HIP_KIND_Q8_K) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "packed activation layout: unsupported weight kind %d",
+                         weight_kind);
+    }
+    const int act_kind = is_k_quant(weight_kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+    ActScratch act;
+    uint8_t *const origin = nullptr;
+    layout->total_bytes = act_scratch_layout(act_kind, N, K, origin, &act);
+    layout->act_kind = act_kind;
+    layout->values_offset = 0;
+    layout->values_per_row = act.kp;
+    layout->scales_offset = (size_t)((uint8_t *)act.d - origin);
+    layout->blocks_per_row = act.nb;
+    layout->sums_offset = (size_t)((uint8_t *)act.sums - origin);
+    layout->sums_per_block = act_kind == MARMOT_HIP_KIND_Q8_K ? 16 : 1;
+    return MARMOT_HIP_SUCCESS;
+}
+
 int marmot_hip_pack_activations(marmot_hip_device_t *dev, int weight_kind, const void *d_input, int in_dtype,
                                 size_t N, size_t K, void *d_packed) {
     if (dev == nullptr) {

@@ -408,10 +408,16 @@ int marmot_hip_softmax_rows(marmot_hip_device_t *dev, const float *d_x, size_t r
     return MARMOT_HIP_SUCCESS;
 }
 
-int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size_t T, size_t H, size_t F, size_t E,
-                           size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate, const void *d_up,
-                           const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
-                           float weights_scale, int router_weight_policy, int ffn_type, float *d_out) {
+} // extern "C"
+
+// One body for marmot_hip_moe_experts and its stage-probing variant. `probe` (may be null) names device buffers that
+// receive the intermediate arrays, and optionally the packed activations the down projection reads instead of the
+// ones this call quantized.
+static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, size_t T, size_t H, size_t F, size_t E,
+                            size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate, const void *d_up,
+                            const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
+                            float weights_scale, int router_weight_policy, int ffn_type, float *d_out,
+                            const marmot_hip_moe_probe_t *probe) {
     if (dev == nullptr) {
         return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
     }
@@ -517,6 +523,29 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
+    if (probe != nullptr) {
+        const size_t fused_bytes = act_scratch_layout(act_dn, routes, F, nullptr, nullptr);
+        const struct {
+            void *dst;
+            const void *src;
+            size_t bytes;
+        } copies[] = {
+            {probe->d_sorted_tokens, sorted_tokens, routes * sizeof(uint32_t)},
+            {probe->d_route_pos, route_pos, routes * sizeof(int)},
+            {probe->d_gate_out, gate_out, routes * F * sizeof(float)},
+            {probe->d_up_out, up_out, routes * F * sizeof(float)},
+            {probe->d_fused_packed, base + o_fused_q, fused_bytes},
+        };
+        for (const auto &c : copies) {
+            if (c.dst != nullptr) {
+                MH_HIP(hipMemcpyAsync(c.dst, c.src, c.bytes, hipMemcpyDeviceToDevice, dev->stream));
+            }
+        }
+        if (probe->d_fused_override != nullptr) {
+            MH_HIP(hipMemcpyAsync(base + o_fused_q, probe->d_fused_override, fused_bytes, hipMemcpyDeviceToDevice,
+                                  dev->stream));
+        }
+    }
     st = grouped_dn(dev, kind_down, d_down, nullptr, dn_stride, fused_q, nullptr, items, flags, max_items, F, H,
                     route_down, nullptr);
     if (st != MARMOT_HIP_SUCCESS) {
@@ -538,6 +567,31 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
         }
     }
     return MARMOT_HIP_SUCCESS;
+}
+
+extern "C" {
+
+int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size_t T, size_t H, size_t F, size_t E,
+                           size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate, const void *d_up,
+                           const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
+                           float weights_scale, int router_weight_policy, int ffn_type, float *d_out) {
+    return moe_experts_impl(dev, d_hidden, T, H, F, E, k_per_token, kind_gate_up, kind_down, d_gate, d_up, d_down,
+                            d_topk_ids, d_topk_weights, weights_scale, router_weight_policy, ffn_type, d_out, nullptr);
+}
+
+int marmot_hip_moe_experts_probe(marmot_hip_device_t *dev, const float *d_hidden, size_t T, size_t H, size_t F,
+                                 size_t E, size_t k_per_token, int kind_gate_up, int kind_down, const void *d_gate,
+                                 const void *d_up, const void *d_down, const int32_t *d_topk_ids,
+                                 const float *d_topk_weights, float weights_scale, int router_weight_policy,
+                                 int ffn_type, float *d_out, const marmot_hip_moe_probe_t *probe) {
+    if (probe == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "MoE experts probe requires a probe description");
+    }
+    if (dev != nullptr && dev->capturing) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "MoE experts probe cannot be captured into a graph");
+    }
+    return moe_experts_impl(dev, d_hidden, T, H, F, E, k_per_token, kind_gate_up, kind_down, d_gate, d_up, d_down,
+                            d_topk_ids, d_topk_weights, weights_scale, router_weight_policy, ffn_type, d_out, probe);
 }
 
 } // extern "C"

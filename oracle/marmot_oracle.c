@@ -2722,6 +2722,18 @@ static inline float moe_gelu(float x) {
     return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
+/* The gated product of moe_ops.c:548-559 on its own: out[i] = act(gate[i]) * up[i]. */
+int mo_moe_glu(const float *gate, const float *up, size_t n, int ffn_type, float *out) {
+    if (ffn_type != MO_FFN_SWIGLU && ffn_type != MO_FFN_GEGLU) {
+        return MO_ERR_NOT_IMPLEMENTED;
+    }
+    for (size_t i = 0; i < n; ++i) {
+        const float g = gate[i];
+        out[i] = (ffn_type == MO_FFN_GEGLU ? moe_gelu(g) : moe_silu(g)) * up[i];
+    }
+    return MO_OK;
+}
+
 /* moe_ops.c:506-568: gate/up (shared activation quantization) -> act(gate)*up -> down */
 static int moe_expert_body(
     const float *rows_in, size_t count, size_t H, size_t F, int kind_gu, int kind_down, const uint8_t *gate_w,
@@ -2738,10 +2750,9 @@ static int moe_expert_body(
     if (st != MO_OK) {
         return st;
     }
-    for (size_t i = 0; i < count * F; ++i) {
-        const float g = gate_buf[i];
-        const float a = ffn_type == MO_FFN_GEGLU ? moe_gelu(g) : moe_silu(g);
-        gate_buf[i] = a * up_buf[i];
+    st = mo_moe_glu(gate_buf, up_buf, count * F, ffn_type, gate_buf);
+    if (st != MO_OK) {
+        return st;
     }
     return mo_matmul_quantized(kind_down, down_w, gate_buf, MO_DTYPE_F32, count, F, H, NULL, down_out, MO_DTYPE_F32,
                                0, threads);

@@ -183,6 +183,10 @@ int mo_topk(const float *x, size_t rows, size_t cols, size_t k, float *values_ou
 /* router: softmax over the k selected logits (graph_builder.cpp:2276-2316) */
 void mo_softmax_rows(const float *x, size_t rows, size_t k, float *out);
 
+/* act(gate[i]) * up[i] as the expert body computes it between the projections (moe_ops.c:548-559);
+ * out may alias gate. */
+int mo_moe_glu(const float *gate, const float *up, size_t n, int ffn_type, float *out);
+
 /*
  * marmot_moe_experts, fp32 activations, block-quantized experts (moe_ops.c:891-1049, 622-787).
  * gate/up: E slices of [F, H] rows; down: E slices of [H, F]. kind_gate_up / kind_down are quant kinds.

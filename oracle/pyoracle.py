@@ -121,6 +121,8 @@ class Oracle:
         L.mo_topk.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
         L.mo_softmax_rows.restype = None
         L.mo_softmax_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+        L.mo_moe_glu.restype = C.c_int
+        L.mo_moe_glu.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
         L.mo_moe_experts.restype = C.c_int
         L.mo_moe_experts.argtypes = [
             C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_void_p,
@@ -308,6 +310,17 @@ class Oracle:
         x = np.ascontiguousarray(x, dtype=np.float32)
         out = np.zeros_like(x)
         self.L.mo_softmax_rows(_ptr(x), x.shape[0], x.shape[1], _ptr(out))
+        return out
+
+    def moe_glu(self, gate: np.ndarray, up: np.ndarray, ffn_type: int = 0) -> np.ndarray:
+        """act(gate) * up element by element, as the expert body forms it between the projections."""
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        up = np.ascontiguousarray(up, dtype=np.float32)
+        assert gate.shape == up.shape
+        out = np.zeros_like(gate)
+        st = self.L.mo_moe_glu(_ptr(gate), _ptr(up), gate.size, ffn_type, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_moe_glu -> {st}")
         return out
 
     def moe_experts(self, hidden, gate, up, down, topk_ids, topk_weights, F: int, E: int, kind_gate_up: int,

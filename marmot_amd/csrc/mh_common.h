@@ -207,9 +207,27 @@ struct ActScratch {
 
 } // namespace mh
 
+// Switches read from the environment ONCE, when the device object is created (a process that wants another setting
+// creates another device object). Each one turns a route off and leaves the slower general one:
+//   MARMOT_HIP_NO_MMQ          small-batch kernels on the int8 matrix cores -> packed matvec
+//   MARMOT_HIP_NO_ROW_KERNELS  row-owning kernels (one workgroup per compute unit) -> the streaming kernels
+//   MARMOT_HIP_NO_LDS_RING     loader / consumer matvec (weights through an LDS ring) -> register-streaming matvec
+//   MARMOT_HIP_NO_FUSED_QUANT  activation quantization inside the matvec -> separate quantization launch
+//   MARMOT_HIP_NO_GEMM         fp16 prefill GEMM -> fp16 matvec
+//   MARMOT_HIP_MOE_NO_VALIDATE skip the read-back of the expert-id error flag (no stream synchronization per call)
+struct marmot_hip_knobs {
+    bool no_mmq = false;
+    bool no_row_kernels = false;
+    bool no_lds_ring = false;
+    bool no_fused_quant = false;
+    bool no_gemm = false;
+    bool moe_no_validate = false;
+};
+
 // The device object behind marmot_hip_device_t.
 struct marmot_hip_device {
     int device_index = 0;
+    marmot_hip_knobs knobs;
     hipStream_t stream = nullptr;
     hipDeviceProp_t props;
     // library-owned workspace, grown on demand (counterpart of the reference's quant workspace slots,
@@ -303,7 +321,7 @@ int launch_quantize_act_soa(marmot_hip_device *dev, int act_kind, const void *d_
                             const ActScratch &dst);
 // act == nullptr selects the fused variant: d_x_f32 ([N,K] fp32, N <= 4, K a multiple of the block) is quantized inside
 // the matvec kernel; otherwise `act` holds activations packed by launch_quantize_act_soa.
-bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_f32);
+bool matvec_can_fuse_quantization(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *d_x_f32);
 int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
                          const float *d_x_f32, size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype,
                          void *d_out0, void *d_out1, int out_dtype);
@@ -326,6 +344,13 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
 // it does not cover.
 int launch_matvec_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, size_t N, size_t K,
                            size_t M, int out_dtype);
+// Row-owning small-batch Q4_K matmul on the int8 matrix cores for 1..16 activation rows (mh_mmq_rows.hip): fp32 rows
+// are quantized inside the kernel (act == nullptr), packed rows are copied into LDS by the kernel's loaders; K is
+// split inside the workgroup. Returns
+// MARMOT_HIP_ERROR_NOT_IMPLEMENTED, error text untouched, for shapes it does not cover.
+bool mmq_rows_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int nw, bool packed);
+int launch_mmq_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, const ActScratch *act,
+                        size_t N, size_t K, size_t M, int out_dtype);
 // quantizes act(gate) * up (SwiGLU or GeGLU) of two fp32 [rows, k] arrays into the activation scratch
 int launch_quantize_glu_soa(marmot_hip_device *dev, int act_kind, const float *d_gate, const float *d_up, bool geglu,
                             size_t rows, size_t k, const ActScratch &dst);
@@ -335,21 +360,21 @@ int launch_matvec_grouped(marmot_hip_device *dev, int kind, const void *d_w0, co
 int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                       const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 // small-batch int8-MFMA matmul (mh_mmq.hip)
-bool mmq_supported(int kind, size_t N, size_t K, int weights = 1);
+bool mmq_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, int weights = 1);
 size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int weights);
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);
 int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                    size_t M, int out_dtype, void *scratch);
-bool mmq_grouped_supported(int kind, size_t K);
+bool mmq_grouped_supported(const marmot_hip_device *dev, int kind, size_t K);
 int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
                        const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
                        size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1);
 // sums fp32 partials [splits][N][M] in split order, then bias and output cast (mh_gemm.hip)
 int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
                          const void *d_bias, int bias_dtype, void *d_out, int out_dtype, bool bias_first = false);
-bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M);
+bool gemm_f16_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M);
 int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                     const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
 

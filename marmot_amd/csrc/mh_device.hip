@@ -1,6 +1,8 @@
 // Device object, memory, events, error text: the plumbing half of the C ABI (include/marmot_hip.h).
 #include "mh_common.h"
 
+#include <stdlib.h>
+
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -165,6 +167,13 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
         delete dev;
         return st;
     }
+    // route switches: read here, never on a launch path
+    dev->knobs.no_mmq = getenv("MARMOT_HIP_NO_MMQ") != nullptr;
+    dev->knobs.no_row_kernels = getenv("MARMOT_HIP_NO_ROW_KERNELS") != nullptr;
+    dev->knobs.no_lds_ring = getenv("MARMOT_HIP_NO_LDS_RING") != nullptr;
+    dev->knobs.no_fused_quant = getenv("MARMOT_HIP_NO_FUSED_QUANT") != nullptr;
+    dev->knobs.no_gemm = getenv("MARMOT_HIP_NO_GEMM") != nullptr;
+    dev->knobs.moe_no_validate = getenv("MARMOT_HIP_MOE_NO_VALIDATE") != nullptr;
     // default priority, non-blocking with respect to the legacy default stream
     if (check_hip(hipStreamCreateWithFlags(&dev->stream, hipStreamNonBlocking), "hipStreamCreateWithFlags") != 0) {
         delete dev;

@@ -888,8 +888,8 @@ int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int split
     return MARMOT_HIP_SUCCESS;
 }
 
-bool gemm_f16_supported(int kind, size_t N, size_t K, size_t M) {
-    if (getenv("MARMOT_HIP_NO_GEMM") != nullptr) {
+bool gemm_f16_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M) {
+    if (dev->knobs.no_gemm) {
         return false;
     }
     return kind == MARMOT_HIP_KIND_Q4_K && N > 8 && K % QK_K == 0 && M >= 1;
@@ -909,10 +909,6 @@ static int launch_gemm_shape(marmot_hip_device *dev, GemmParams p, size_t N, siz
         splits = cus / tiles;
         const size_t max_splits = nb / (2 * KG) > 0 ? nb / (2 * KG) : 1;  // at least two blocks per K group
         splits = splits > max_splits ? max_splits : splits;
-    }
-    if (const char *e = getenv("MH_GEMM_SPLITS")) {
-        splits = (size_t)atoi(e);
-        splits = splits < 1 ? 1 : (splits > nb ? nb : splits);
     }
     const size_t blocks_per_split = (nb + splits - 1) / splits;
     splits = (nb + blocks_per_split - 1) / blocks_per_split;
@@ -977,7 +973,7 @@ static int launch_gemm_big(marmot_hip_device *dev, GemmParams p, size_t N, size_
 
 int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                     const void *d_bias, int bias_dtype, void *d_out, int out_dtype) {
-    if (!gemm_f16_supported(kind, N, K, M)) {
+    if (!gemm_f16_supported(dev, kind, N, K, M)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "prefill GEMM: unsupported kind or shape");
     }
     if ((((uintptr_t)d_x) & 15) != 0) {
@@ -1001,8 +997,7 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     // workgroup otherwise.
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     const size_t big_tiles = ((N + 127) / 128) * ((M + 255) / 256);
-    const char *force = getenv("MH_GEMM_SHAPE");
-    const bool big = force != nullptr ? atoi(force) == 4 : big_tiles >= cus;
+    const bool big = big_tiles >= cus;
     set_route("gemm_q4_k_f16_mfma");
     if (big) {
         return launch_gemm_big(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);

@@ -220,7 +220,7 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
             const void *w = which ? d_w1 : d_w0;
             void *o = which ? d_out1 : d_out0;
             int st;
-            if (gemm_f16_supported(kind, N, K, M)) {
+            if (gemm_f16_supported(dev, kind, N, K, M)) {
                 st = launch_gemm_f16(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);
             } else {
                 st = launch_matvec_f16(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);
@@ -233,8 +233,25 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     // packed route. fp32 activations whose rows are whole blocks are quantized inside the matvec kernel; otherwise
     // the activations are quantized once into the workspace (shared by both weights of a dual call).
-    const bool mmq = mmq_supported(kind, N, K);
-    if (!mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input)) {
+    const bool mmq = mmq_supported(dev, kind, N, K);
+    const bool rows_kernel = mmq && kind == MARMOT_HIP_KIND_Q4_K && N <= 16 && !dev->knobs.no_row_kernels;
+    WeightSet rows_ws;
+    rows_ws.count = d_w1 != nullptr ? 2 : 1;
+    rows_ws.w[0] = d_w0;
+    rows_ws.w[1] = d_w1;
+    rows_ws.out[0] = d_out0;
+    rows_ws.out[1] = d_out1;
+    rows_ws.bias[0] = d_bias;
+    rows_ws.bias[1] = d_bias;
+    rows_ws.bias_dtype = bias_dtype;
+    if (rows_kernel && in_dtype == MARMOT_HIP_DTYPE_F32) {
+        // row-owning small-batch kernel: quantizes the activations itself, no partial sums
+        const int st = launch_mmq_rows_q4k(dev, rows_ws, (const float *)d_input, nullptr, N, K, M, out_dtype);
+        if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+            return st;
+        }
+    }
+    if (!mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(dev, kind, N, K, d_input)) {
         return launch_matvec_packed(dev, kind, d_w0, d_w1, nullptr, (const float *)d_input, N, K, M, d_bias,
                                     bias_dtype, d_out0, d_out1, out_dtype);
     }
@@ -251,6 +268,12 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
+    }
+    if (rows_kernel) {
+        st = launch_mmq_rows_q4k(dev, rows_ws, nullptr, &act, N, K, M, out_dtype);
+        if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+            return st;
+        }
     }
     if (mmq) {
         return launch_mmq(dev, kind, d_w0, d_w1, act, N, K, M, d_bias, bias_dtype, d_out0, d_out1, out_dtype,
@@ -331,6 +354,38 @@ __global__ __launch_bounds__(256) void k_qkv_rope_finish(const RopeFinishParams 
         dst[even_index] = even;
         dst[odd_index] = odd;
     }
+}
+
+// Rotary epilogue of the Q/K/V projection. stage: the three fp32 projections [3][N][M] when the outputs are fp16
+// (rounded once, after the rotation), nullptr when the fp32 outputs themselves hold them.
+static int qkv_rope_finish(marmot_hip_device *dev, const marmot_hip_rope_t *rope, const float *stage, void *d_out_q,
+                           void *d_out_k, void *d_out_v, size_t N, size_t M, int out_dtype) {
+    const bool stage32 = stage != nullptr;
+    RopeFinishParams rp;
+    void *outs[3] = {d_out_q, d_out_k, d_out_v};
+    for (int i = 0; i < 3; ++i) {
+        rp.src[i] = stage32 ? stage + (size_t)i * N * M : (const float *)outs[i];
+        rp.dst[i] = outs[i];
+    }
+    rp.rotate[0] = rope->apply_to_q ? 1 : 0;
+    rp.rotate[1] = rope->apply_to_k ? 1 : 0;
+    rp.rotate[2] = 0;
+    rp.positions = rope->d_positions;
+    rp.positions_dtype = rope->positions_dtype;
+    rp.freqs = rope->d_freqs;
+    rp.attn_scale = rope->attn_scale;
+    rp.head_dim = rope->head_dim;
+    rp.neox = rope->rope_type == 1;
+    rp.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    rp.N = N;
+    rp.M = M;
+    if (N > 65535) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE epilogue: more than 65535 activation rows");
+    }
+    const dim3 grid((unsigned)((M / 2 + 255) / 256), (unsigned)N, 3);
+    hipLaunchKernelGGL(k_qkv_rope_finish, grid, dim3(256), 0, dev->stream, rp);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
 }
 
 } // namespace mh
@@ -434,8 +489,19 @@ int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     ActScratch act;
     act_scratch_layout(act_kind, N, K, const_cast<void *>(d_packed), &act);
-    if (mmq_supported(kind, N, K)) {
+    if (mmq_supported(dev, kind, N, K)) {
         MH_HIP(hipSetDevice(dev->device_index));
+        if (kind == MARMOT_HIP_KIND_Q4_K && N <= 16 && !dev->knobs.no_row_kernels) {
+            WeightSet ws;
+            ws.w[0] = d_weight;
+            ws.out[0] = d_out;
+            ws.bias[0] = d_bias;
+            ws.bias_dtype = bias_dtype;
+            st = launch_mmq_rows_q4k(dev, ws, nullptr, &act, N, K, M, out_dtype);
+            if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+                return st;
+            }
+        }
         return launch_mmq(dev, kind, d_weight, nullptr, act, N, K, M, d_bias, bias_dtype, d_out, nullptr, out_dtype,
                           nullptr);
     }
@@ -574,8 +640,28 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
     ws.out[2] = d_out_v;
     ws.bias_dtype = bias_dtype;
     ws.bias_first = true;
-    const bool mmq = mmq_supported(kind, N, K, 3);
-    const bool fuse_quant = !mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(kind, N, K, d_input);
+    const bool mmq = mmq_supported(dev, kind, N, K, 3);
+    if (mmq && kind == MARMOT_HIP_KIND_Q4_K && in_dtype == MARMOT_HIP_DTYPE_F32 && N <= 16 &&
+        !dev->knobs.no_row_kernels && (((uintptr_t)d_input) & 15) == 0 &&
+        mmq_rows_supported(dev, kind, N, K, M, 3, false)) {
+        void *wsp_rows = nullptr;
+        if (stage_bytes != 0) {
+            const int rs = workspace_reserve(dev, stage_bytes, &wsp_rows);
+            if (rs != MARMOT_HIP_SUCCESS) {
+                return rs;
+            }
+            for (int i = 0; i < 3; ++i) {
+                ws.out[i] = (float *)wsp_rows + (size_t)i * N * M;
+            }
+        }
+        const int rs = launch_mmq_rows_q4k(dev, ws, (const float *)d_input, nullptr, N, K, M, mm_out_dtype);
+        if (rs != MARMOT_HIP_SUCCESS || !roped) {
+            return rs;
+        }
+        return qkv_rope_finish(dev, rope, stage32 ? (const float *)wsp_rows : nullptr, d_out_q, d_out_k, d_out_v, N, M,
+                               out_dtype);
+    }
+    const bool fuse_quant = !mmq && in_dtype == MARMOT_HIP_DTYPE_F32 && matvec_can_fuse_quantization(dev, kind, N, K, d_input);
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes =
         fuse_quant ? 0 : ((act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255);
@@ -603,7 +689,13 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
         if (st != MARMOT_HIP_SUCCESS) {
             return st;
         }
-        if (mmq) {
+        st = MARMOT_HIP_ERROR_NOT_IMPLEMENTED;
+        if (mmq && kind == MARMOT_HIP_KIND_Q4_K && N <= 16 && !dev->knobs.no_row_kernels) {
+            st = launch_mmq_rows_q4k(dev, ws, nullptr, &act, N, K, M, mm_out_dtype);
+        }
+        if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+            // the row-owning kernel took it
+        } else if (mmq) {
             st = launch_mmq_set(dev, kind, ws, act, N, K, M, mm_out_dtype, (uint8_t *)wsp + act_bytes);
         } else {
             st = launch_matvec_set(dev, kind, ws, &act, nullptr, N, K, M, mm_out_dtype);
@@ -612,31 +704,7 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
     if (st != MARMOT_HIP_SUCCESS || !roped) {
         return st;
     }
-    RopeFinishParams rp;
-    void *outs[3] = {d_out_q, d_out_k, d_out_v};
-    for (int i = 0; i < 3; ++i) {
-        rp.src[i] = stage32 ? stage + (size_t)i * N * M : (const float *)outs[i];
-        rp.dst[i] = outs[i];
-    }
-    rp.rotate[0] = rope->apply_to_q ? 1 : 0;
-    rp.rotate[1] = rope->apply_to_k ? 1 : 0;
-    rp.rotate[2] = 0;
-    rp.positions = rope->d_positions;
-    rp.positions_dtype = rope->positions_dtype;
-    rp.freqs = rope->d_freqs;
-    rp.attn_scale = rope->attn_scale;
-    rp.head_dim = rope->head_dim;
-    rp.neox = rope->rope_type == 1;
-    rp.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
-    rp.N = N;
-    rp.M = M;
-    if (N > 65535) {
-        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "RoPE epilogue: more than 65535 activation rows");
-    }
-    const dim3 grid((unsigned)((M / 2 + 255) / 256), (unsigned)N, 3);
-    hipLaunchKernelGGL(k_qkv_rope_finish, grid, dim3(256), 0, dev->stream, rp);
-    MH_HIP(hipGetLastError());
-    return MARMOT_HIP_SUCCESS;
+    return qkv_rope_finish(dev, rope, stage32 ? stage : nullptr, d_out_q, d_out_k, d_out_v, N, M, out_dtype);
 }
 
 } // extern "C"

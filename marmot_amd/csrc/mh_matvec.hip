@@ -1125,12 +1125,12 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
 
 // rows whose bytes can be copied as 16-byte chunks: row pitch and base address multiples of 16, at most 8 K slices
 template <class Fmt>
-static bool matvec_ls_usable(const MatvecParams &p, size_t K, int C) {
+static bool matvec_ls_usable(const marmot_hip_device *dev, const MatvecParams &p, size_t K, int C) {
     const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
     const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
     return p.items == nullptr && K % Fmt::BV == 0 && p.row_bytes % 16 == 0 && (((uintptr_t)p.w[0]) & 15) == 0 &&
            (((uintptr_t)p.w[1]) & 15) == 0 && (((uintptr_t)p.w[2]) & 15) == 0 && wave_loads <= (size_t)(matvec_ls_max_consumers<Fmt>() * C) &&
-           getenv("MH_MV_NO_LS") == nullptr;
+           !dev->knobs.no_lds_ring;
 }
 
 template <class Fmt, int NC, int C, int R, bool FUSED>
@@ -1200,10 +1200,6 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
     if (rows_per_wg > 32) {
         rows_per_wg = 32;
     }
-    if (const char *e = getenv("MH_RPW")) {
-        rows_per_wg = (size_t)atoi(e);
-        rows_per_wg = ((rows_per_wg + R - 1) / R) * R;
-    }
     p.rows_per_wg = (int)rows_per_wg;
     set_route(name);
     if constexpr (NC <= 4) {
@@ -1213,15 +1209,12 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
         // (14336 x 4096, N = 1 / 2 / 4: Q6_K 15.5 -> 12.9, 18.0 -> 16.7, 24.0 -> 23.5 us; Q8_0 18.4 -> 15.2,
         // 22.8 -> 16.4, 29.8 -> 22.5 us; Q8_0 5632 x 2048: 6.8 -> 6.1 us), slower for Q6_K at K = 14336.
         const bool fmt_ok = Fmt::BYTES % 16 == 0 || K <= 8192;
-        if (fmt_ok && matvec_ls_usable<Fmt>(p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
+        if (fmt_ok && matvec_ls_usable<Fmt>(dev, p, K, C) && (fused || M * p.row_bytes >= ((size_t)16 << 20))) {
             // rows per workgroup: two workgroups per CU when M allows, between 8 (the activation prologue must pay
             // off) and 16 (more rows per workgroup leave CUs idle at the usual M)
             size_t rows_ls = (M + 2 * cus - 1) / (2 * cus);
             rows_ls = ((rows_ls + 3) / 4) * 4;
             rows_ls = rows_ls < 8 ? 8 : (rows_ls > 16 ? 16 : rows_ls);
-            if (const char *e = getenv("MH_RPW")) {
-                rows_ls = (size_t)atoi(e);
-            }
             p.rows_per_wg = (int)rows_ls;
             if (C == 1) {
                 return fused ? launch_ls<Fmt, NC, 1, 2, true>(dev, p, W, M, nw)
@@ -1252,14 +1245,6 @@ static int launch_tile_r(marmot_hip_device *dev, MatvecParams p, size_t K, size_
 template <class Fmt, int NC>
 static int launch_tile(marmot_hip_device *dev, MatvecParams p, size_t K, size_t M, int nw, const char *name) {
     if constexpr (NC == 1) {
-        const char *e = getenv("MH_R");
-        const int r = e ? atoi(e) : 4;
-        if (r == 8) {
-            return launch_tile_r<Fmt, NC, 8>(dev, p, K, M, nw, name);
-        }
-        if (r == 2) {
-            return launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name);
-        }
         const int st = launch_tile_r<Fmt, NC, 4>(dev, p, K, M, nw, name);
         // a format with wide weight registers (Q5_K) covers long rows with fewer rows in flight
         return st == MARMOT_HIP_ERROR_NOT_IMPLEMENTED ? launch_tile_r<Fmt, NC, 2>(dev, p, K, M, nw, name) : st;
@@ -1320,9 +1305,9 @@ static int launch_fmt(marmot_hip_device *dev, MatvecParams p, size_t N, size_t K
     return MARMOT_HIP_SUCCESS;
 }
 
-bool matvec_can_fuse_quantization(int kind, size_t N, size_t K, const void *d_x_f32) {
+bool matvec_can_fuse_quantization(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *d_x_f32) {
     const size_t bv = block_values(kind);
-    return N <= 4 && bv != 0 && K % bv == 0 && (((uintptr_t)d_x_f32) & 15) == 0 && getenv("MARMOT_HIP_NO_FUSED_QUANT") == nullptr;
+    return N <= 4 && bv != 0 && K % bv == 0 && (((uintptr_t)d_x_f32) & 15) == 0 && !dev->knobs.no_fused_quant;
 }
 
 int launch_matvec_packed(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch *act,
@@ -1384,7 +1369,7 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
     p.expert_stride = 0;
     const int nw = ws.count;
     const bool fused = act == nullptr;
-    if (kind == MARMOT_HIP_KIND_Q4_K && fused && N <= 2 && getenv("MH_NO_ROWS") == nullptr) {
+    if (kind == MARMOT_HIP_KIND_Q4_K && fused && N <= 2 && !dev->knobs.no_row_kernels) {
         const int st = launch_matvec_rows_q4k(dev, ws, d_x_f32, N, K, M, out_dtype);
         if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
             return st;

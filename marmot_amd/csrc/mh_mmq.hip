@@ -836,16 +836,13 @@ static bool mmq_is_q4k_family(int kind) {
     return kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q5_K;
 }
 
-bool mmq_supported(int kind, size_t N, size_t K, int weights) {
-    if (getenv("MARMOT_HIP_NO_MMQ") != nullptr) {
+bool mmq_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, int weights) {
+    if (dev->knobs.no_mmq) {
         return false;
     }
     // below these row counts the fused-quantization matvec is faster (no separate quantization pass)
     // (a Q6_K set of three weights crosses over earlier: the matvec streams every weight per column tile)
-    size_t q6_set_min = 3;
-    if (const char *e = getenv("MH_MMQ6_SET_MIN")) {
-        q6_set_min = (size_t)atoi(e);
-    }
+    const size_t q6_set_min = 3;
     const size_t min_rows = mmq_is_q4k_family(kind) ? 3 : (weights >= 3 ? q6_set_min : 5);
     return (mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && N >= min_rows && K % QK_K == 0;
 }
@@ -858,7 +855,7 @@ struct MmqPlan {
 
 // rows of a multiple of 8 blocks are 16-byte aligned: the loader/consumer kernel applies
 static bool mmq6_uses_loader(size_t nb) {
-    return nb % 8 == 0 && getenv("MH_MMQ6_NO_LS") == nullptr;
+    return nb % 8 == 0;
 }
 
 // W (consumer) wavefronts per workgroup and S workgroups split K.
@@ -879,7 +876,7 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t
     const size_t cus = (size_t)dev->props.multiProcessorCount;
     MmqPlan pl;
     size_t W, S = 1;
-    if (passes > 1 && rg >= cus && getenv("MH_MMQ_ZPLAN_OFF") == nullptr) {
+    if (passes > 1 && rg >= cus) {
         // several passes in one launch fill the chip by themselves: one consumer walks the whole row, which keeps
         // the LDS ring small (four workgroups per CU) and needs no partial sums
         W = 1;
@@ -900,12 +897,6 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t
         while (rg * S < cus && W * S * 2 <= nb) {
             S *= 2;
         }
-    }
-    if (const char *e = getenv("MH_MMQ_W")) {
-        W = (size_t)atoi(e);
-    }
-    if (const char *e = getenv("MH_MMQ_S")) {
-        S = (size_t)atoi(e);
     }
     const size_t bpw = (nb + W * S - 1) / (W * S);
     pl.W = (int)W;
@@ -1001,7 +992,7 @@ static int mmq_launch_q4k(marmot_hip_device *dev, int kind, const MmqParams &p, 
         }
         const bool q5 = kind == MARMOT_HIP_KIND_Q5_K;
         // Q5_K with 32-row passes: three stages of two consumers would take 84 KB and leave one workgroup per CU
-        const int stages = (p.items != nullptr || (q5 && NR > 8 && getenv("MH_MMQ5_3STAGES") == nullptr)) ? 2 : 3;
+        const int stages = (p.items != nullptr || (q5 && NR > 8)) ? 2 : 3;
         const size_t stage = 32 * (size_t)(q5 ? Q5_K_BYTES : Q4_K_BYTES) + 2 * NR * QK_K + 2 * NR * 4;
         const size_t ring = (size_t)pl.W * stages * stage;
         const size_t red = (size_t)pl.W * NR * 64 * sizeof(float);
@@ -1042,7 +1033,7 @@ int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d
 
 int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                    size_t M, int out_dtype, void *scratch) {
-    if (!mmq_supported(kind, N, K, ws.count)) {
+    if (!mmq_supported(dev, kind, N, K, ws.count)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
     }
     const size_t nb = K / QK_K;
@@ -1083,13 +1074,9 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
     // Q6_K with 16-byte aligned rows) from 17 rows on: 32 rows per pass, which uses all 32 rows of the matrix-core product instead of half of them and halves the number of
     // passes over the weights.
     const bool wide_ok = mmq_is_q4k_family(kind) || (kind == MARMOT_HIP_KIND_Q6_K && mmq6_loader_applies(p, pl));
-    size_t wide_from = 17;  // more than one 16-row pass: one 32-row pass streams the weights once instead of twice
-    if (const char *e = getenv("MH_MMQ_WIDE_FROM")) {
-        wide_from = (size_t)atoi(e);
-    }
-    const size_t rows_per_pass =
-        (wide_ok && N >= wide_from && getenv("MH_MMQ_NO32") == nullptr) ? 32 : MMQ_ROWS_PER_PASS;
-    if (rows_per_pass == 32 && N > 32 && getenv("MH_MMQ_NO_ZPASS") == nullptr) {
+    const size_t wide_from = 17;  // more than one 16-row pass: one 32-row pass streams the weights once instead of twice
+    const size_t rows_per_pass = (wide_ok && N >= wide_from) ? 32 : MMQ_ROWS_PER_PASS;
+    if (rows_per_pass == 32 && N > 32) {
         // all passes in one launch (grid z): no launch gap, ramp and tail per pass
         p.n0 = 0;
         p.ncols = 32;
@@ -1126,9 +1113,8 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
 
 // Grouped (MoE): every work item is up to 8 consecutive routes of one expert; blockIdx.z walks the item list the
 // route kernel wrote (workgroups beyond *d_n_items exit at once).
-bool mmq_grouped_supported(int kind, size_t K) {
-    return (mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && K % QK_K == 0 &&
-           getenv("MARMOT_HIP_NO_MMQ") == nullptr;
+bool mmq_grouped_supported(const marmot_hip_device *dev, int kind, size_t K) {
+    return (mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && K % QK_K == 0 && !dev->knobs.no_mmq;
 }
 
 int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
@@ -1137,7 +1123,7 @@ int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const
     if (max_items == 0 || M == 0 || K == 0) {
         return MARMOT_HIP_SUCCESS;
     }
-    if (!mmq_grouped_supported(kind, K)) {
+    if (!mmq_grouped_supported(dev, kind, K)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "grouped MFMA matmul: unsupported kind or shape");
     }
     if (max_items > 65535) {

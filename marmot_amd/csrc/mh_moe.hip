@@ -512,8 +512,8 @@ static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, siz
     const size_t gu_stride = F * ((H + bv_gu - 1) / bv_gu) * block_bytes(kind_gate_up);
     const size_t dn_stride = H * ((F + bv_dn - 1) / bv_dn) * block_bytes(kind_down);
     // Q4_K / Q6_K experts run on the int8 matrix cores, the 32-value formats on the dot-product matvec
-    const auto grouped_gu = mmq_grouped_supported(kind_gate_up, H) ? launch_mmq_grouped : launch_matvec_grouped;
-    const auto grouped_dn = mmq_grouped_supported(kind_down, F) ? launch_mmq_grouped : launch_matvec_grouped;
+    const auto grouped_gu = mmq_grouped_supported(dev, kind_gate_up, H) ? launch_mmq_grouped : launch_matvec_grouped;
+    const auto grouped_dn = mmq_grouped_supported(dev, kind_down, F) ? launch_mmq_grouped : launch_matvec_grouped;
     st = grouped_gu(dev, kind_gate_up, d_gate, d_up, gu_stride, hidden_q, sorted_tokens, items, flags, max_items, H, F,
                     gate_out, up_out);
     if (st != MARMOT_HIP_SUCCESS) {
@@ -557,8 +557,9 @@ static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, siz
     set_route("moe_experts_grouped");
 
     // Expert ids are validated on the device; reading the flag needs a stream synchronization, which is skipped
-    // while the stream is being captured into a graph or when MARMOT_HIP_MOE_NO_VALIDATE is set.
-    if (!dev->capturing && getenv("MARMOT_HIP_MOE_NO_VALIDATE") == nullptr) {
+    // while the stream is being captured into a graph or when the device object was created with
+    // MARMOT_HIP_MOE_NO_VALIDATE set.
+    if (!dev->capturing && !dev->knobs.moe_no_validate) {
         int host_flag = 0;
         MH_HIP(hipMemcpyAsync(&host_flag, flags + 1, sizeof(int), hipMemcpyDeviceToHost, dev->stream));
         MH_HIP(hipStreamSynchronize(dev->stream));

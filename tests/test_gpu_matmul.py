@@ -217,19 +217,30 @@ def test_linear_error_behaviour(hip, oracle):
 
 
 @pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
-def test_loader_consumer_matvec_equals_register_streaming_matvec(hip, oracle, name, monkeypatch):
+def test_loader_consumer_matvec_equals_register_streaming_matvec(oracle, name, monkeypatch):
     """The loader/consumer matvec (weights through an LDS ring) keeps the lane mapping and the reduction order of the
     register-streaming kernel: the two must agree bit for bit, on whole and ragged row groups, one and two K slices
-    per lane, fused and packed activations."""
+    per lane, fused and packed activations. Route switches are read when a device object is created, so each variant
+    gets a device object of its own (both without the row-owning kernels, which sum in another order)."""
+    from marmot_amd import HipBackend
+
     kind = KINDS[name]
-    for M, K, N in ((256, 2048, 1), (203, 4096, 1), (77, 8192, 1), (64, 14336, 1), (40, 28672, 1), (203, 4096, 2)):
-        blocks = oracle.quantize(kind, gaussian(500 + K, (M, K), 0.02))
-        x = gaussian(501 + K + N, (N, K))
-        monkeypatch.delenv("MH_MV_NO_LS", raising=False)
-        with_ring = hip.linear(x, blocks, kind, M)
-        monkeypatch.setenv("MH_MV_NO_LS", "1")
-        without = hip.linear(x, blocks, kind, M)
-        monkeypatch.delenv("MH_MV_NO_LS", raising=False)
-        assert np.array_equal(bits(with_ring), bits(without)), f"{name} {M}x{K} N={N}"
-        assert_matmul_parity(with_ring, oracle.matmul(kind, blocks, x, M), what=f"{name} {M}x{K} N={N}")
+    monkeypatch.setenv("MARMOT_HIP_NO_ROW_KERNELS", "1")
+    ring = HipBackend(0)
+    monkeypatch.setenv("MARMOT_HIP_NO_LDS_RING", "1")
+    streaming = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_LDS_RING")
+    monkeypatch.delenv("MARMOT_HIP_NO_ROW_KERNELS")
+    try:
+        for M, K, N in ((256, 2048, 1), (203, 4096, 1), (77, 8192, 1), (64, 14336, 1), (40, 28672, 1), (203, 4096, 2)):
+            blocks = oracle.quantize(kind, gaussian(500 + K, (M, K), 0.02))
+            x = gaussian(501 + K + N, (N, K))
+            with_ring = ring.linear(x, blocks, kind, M)
+            without = streaming.linear(x, blocks, kind, M)
+            assert "rows" not in ring.last_route() and "rows" not in streaming.last_route()
+            assert np.array_equal(bits(with_ring), bits(without)), f"{name} {M}x{K} N={N}"
+            assert_matmul_parity(with_ring, oracle.matmul(kind, blocks, x, M), what=f"{name} {M}x{K} N={N}")
+    finally:
+        ring.close()
+        streaming.close()
 

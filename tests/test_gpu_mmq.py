@@ -138,7 +138,12 @@ def test_prepacked_activations_and_graph_replay(hip, oracle, name):
     eager = d_out.download(np.float32, (N, M))
     assert_matmul_parity(eager, ref, what=f"{name} prepacked")
     fused = hip.linear(x, blocks, kind, M)
-    assert np.array_equal(bits(eager), bits(fused))
+    if "mmq_rows" in hip.last_route():
+        # fp32 activations take the row-owning kernel, which adds the blocks of a row in another order
+        assert_matmul_parity(fused, ref, what=f"{name} fused")
+        assert_matmul_parity(fused, eager, what=f"{name} fused against prepacked")
+    else:
+        assert np.array_equal(bits(eager), bits(fused))
 
     g = hip.graph_capture(lambda: hip.linear_d(kind, d_w, d_x, capi.DT_F32, N, K, M, d_out, capi.DT_F32))
     try:
@@ -147,7 +152,7 @@ def test_prepacked_activations_and_graph_replay(hip, oracle, name):
             hip.graph_launch(g)
             hip.synchronize()
             got = d_out.download(np.float32, (N, M))
-            assert np.array_equal(bits(got), bits(eager)), f"{name} replay {rep}"
+            assert np.array_equal(bits(got), bits(fused)), f"{name} replay {rep}"
             other = hip.linear(gaussian(370 + rep, (3, 256)), blocks[:, : blocks.shape[1] // (K // 256)].copy(), kind, M)
             assert other.shape == (3, M)
     finally:
@@ -175,3 +180,43 @@ def test_passes_of_32_rows(hip, oracle, name, N):
     got16 = hip.linear(x16, blocks, kind, M, out_dtype=np.float16, force_pack=True)
     assert np.max(np.abs(got16.astype(np.float32) - ref16.astype(np.float32))) <= \
         2e-3 * np.abs(ref16.astype(np.float32)).max()
+
+
+def test_row_owning_and_streaming_small_batch_kernels(hip, oracle, monkeypatch):
+    """Q4_K with up to 16 rows has two small-batch kernels: the row-owning one (fp32 rows quantized inside the kernel, or
+    packed rows copied into LDS by its loaders) and the streaming one with a workgroup per 32 weight rows, which a
+    device object created with MARMOT_HIP_NO_ROW_KERNELS keeps using. Both against the oracle, and bit-exact on single
+    blocks; the row-owning kernel with one and several row groups per workgroup, K split over 1..12 consumers, ragged
+    rows and blocks, and a ring that is reused."""
+    from marmot_amd import HipBackend
+
+    monkeypatch.setenv("MARMOT_HIP_NO_ROW_KERNELS", "1")
+    streaming = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_ROW_KERNELS")
+    kind = KIND_Q4_K
+    try:
+        rng = np.random.default_rng(380)
+        blocks = random_valid_blocks(rng, kind, 300, 256)
+        for N in (3, 8, 16):
+            x = gaussian(381 + N, (N, 256))
+            ref = oracle.matmul(kind, blocks, x, 300)
+            for dev, route in ((hip, "mmq_rows_q4_k_q8_k"), (streaming, "mmq_q4_k_q8_k_mfma")):
+                got = dev.linear(x, blocks, kind, 300)
+                assert dev.last_route().startswith(route), dev.last_route()
+                assert np.array_equal(bits(got), bits(ref)), f"single block N={N} {route}"
+        # (M, K, N): 5000 rows = 2 row groups of 10 per workgroup; 1500 x 2560: 6 rows per workgroup, 10 blocks in
+        # tasks of 3 (the last one short); 700 x 14336 packed (N * K too large to quantize in the kernel);
+        # 40000 x 1024: 10 row groups per workgroup, one consumer each, ring reused
+        for M, K, N in ((5000, 1024, 3), (1500, 2560, 7), (4096, 4096, 16), (700, 14336, 5), (40000, 1024, 4),
+                        (1000, 4096, 12)):
+            w = oracle.quantize(kind, gaussian(390 + M, (M, K), 0.02))
+            x = gaussian(391 + M + N, (N, K))
+            ref = oracle.matmul(kind, w, x, M, threads=16)
+            got = hip.linear(x, w, kind, M)
+            assert "mmq_rows" in hip.last_route(), (M, K, N, hip.last_route())
+            assert_matmul_parity(got, ref, what=f"row-owning {M}x{K} N={N} {hip.last_route()}")
+            old = streaming.linear(x, w, kind, M)
+            assert streaming.last_route() == "mmq_q4_k_q8_k_mfma"
+            assert_matmul_parity(old, ref, what=f"streaming {M}x{K} N={N}")
+    finally:
+        streaming.close()

@@ -303,6 +303,36 @@ int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *
                                 size_t N, size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out,
                                 int out_dtype);
 
+/* ------------------------------------------------------------------ ops between the linears
+ * The fp32 operations a decoder layer runs between its quantized linears, and the fused forms that hand the next
+ * linear its activations already packed (marmot_hip_matmul_prepacked and the prepacked forms of the q/k/v and gate/up
+ * projections then start without a quantization launch).
+ *
+ * marmot_hip_rms_norm replaces cpu_rmsnorm_impl (weight_offset 0) and cpu_rmsnorm_gemma_impl (weight_offset 1)
+ * for fp32 tensors (src/backends/cpu/ops/normalization/normalization_dispatch.c:129-181, 240-246;
+ * scalar/normalization_scalar.c:469-510, 780-791): per row of `cols` values,
+ *   v = x (+ residual);  out = v * (1 / sqrt(mean(v^2) + eps)) * (weight + weight_offset)
+ * d_residual and d_weight may be null (no residual; no scaling). The mean of squares is summed by 256 threads, not
+ * sequentially: results agree with the scalar CPU loop to a few units in the last place.
+ * marmot_hip_rms_norm_pack writes the same rows as packed activations for a linear of weight_kind (layout and size
+ * of marmot_hip_pack_activations) and, when d_out is not null, as fp32 too; the packed rows are bit-identical to
+ * marmot_hip_pack_activations applied to the fp32 output. */
+int marmot_hip_rms_norm(marmot_hip_device_t *dev, const float *d_x, const float *d_residual, const float *d_weight,
+                        float weight_offset, float eps, size_t rows, size_t cols, float *d_out);
+int marmot_hip_rms_norm_pack(marmot_hip_device_t *dev, const float *d_x, const float *d_residual,
+                             const float *d_weight, float weight_offset, float eps, size_t rows, size_t cols,
+                             int weight_kind, float *d_out, void *d_packed);
+/* Replaces cpu_swiglu_f32_scalar / cpu_geglu_f32_scalar (src/backends/cpu/ops/elementwise/scalar/
+ * elementwise_f32_scalar.c:11-20, 147-214): out = silu(gate) * up, or gelu_tanh(gate) * up for MARMOT_HIP_FFN_GEGLU
+ * (the tanh form; the MoE expert body uses the erf form, moe_ops.c:321-324). Row strides in elements.
+ * marmot_hip_swiglu_pack writes silu(gate) * up of contiguous rows as packed activations for a linear of weight_kind. */
+int marmot_hip_glu(marmot_hip_device_t *dev, int ffn_type, const float *d_gate, const float *d_up, size_t rows,
+                   size_t cols, size_t gate_stride, size_t up_stride, size_t out_stride, float *d_out);
+int marmot_hip_swiglu_pack(marmot_hip_device_t *dev, const float *d_gate, const float *d_up, size_t rows, size_t cols,
+                           int weight_kind, void *d_packed);
+/* Replaces cpu_add for contiguous fp32 tensors of equal shape (the residual add). */
+int marmot_hip_add(marmot_hip_device_t *dev, const float *d_a, const float *d_b, size_t n, float *d_out);
+
 /* ------------------------------------------------------------------ MoE
  * Replaces cpu_topk_impl (src/backends/cpu/ops/moe/moe_ops.c:789-889): top-k over the last axis of
  * fp32 x[rows,cols], ties to the lower index; values fp32 [rows,k], indices int32 [rows,k]. */

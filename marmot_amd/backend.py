@@ -386,6 +386,77 @@ class HipBackend:
             C.c_void_p(d_down.ptr + down_offset), C.c_void_p(d_ids.ptr), C.c_void_p(d_weights.ptr), weights_scale,
             policy, ffn_type, C.c_void_p(d_out.ptr)))
 
+    # ---- ops between the linears (host-array conveniences over the device-pointer ABI)
+    def rms_norm(self, x: np.ndarray, weight=None, residual=None, eps: float = 1e-5, weight_offset: float = 0.0,
+                 pack_for_kind: int = 0, want_f32: bool = True):
+        """Rows of x normalized; with pack_for_kind also (or only) as packed activations: returns out, or
+        (out or None, packed uint8 image)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        rows, cols = x.shape
+        bufs = [self.to_device(x)]
+        d_res = d_w = None
+        if residual is not None:
+            d_res = self.to_device(np.ascontiguousarray(residual, dtype=np.float32))
+            bufs.append(d_res)
+        if weight is not None:
+            d_w = self.to_device(np.ascontiguousarray(weight, dtype=np.float32))
+            bufs.append(d_w)
+        d_out = self.alloc(rows * cols * 4) if want_f32 else None
+        d_packed = self.alloc(self.packed_activation_bytes(pack_for_kind, rows, cols)) if pack_for_kind else None
+        bufs += [b for b in (d_out, d_packed) if b is not None]
+        opt = lambda b: C.c_void_p(b.ptr) if b is not None else None
+        try:
+            if pack_for_kind:
+                check(self.lib.marmot_hip_rms_norm_pack(self.dev, C.c_void_p(bufs[0].ptr), opt(d_res), opt(d_w),
+                                                        weight_offset, eps, rows, cols, pack_for_kind, opt(d_out),
+                                                        C.c_void_p(d_packed.ptr)))
+                out = d_out.download(np.float32, (rows, cols)) if want_f32 else None
+                return out, d_packed.download(np.uint8, (d_packed.nbytes,))
+            check(self.lib.marmot_hip_rms_norm(self.dev, C.c_void_p(bufs[0].ptr), opt(d_res), opt(d_w), weight_offset,
+                                               eps, rows, cols, C.c_void_p(d_out.ptr)))
+            return d_out.download(np.float32, (rows, cols))
+        finally:
+            for b in bufs:
+                b.free()
+
+    def glu(self, gate: np.ndarray, up: np.ndarray, ffn_type: int = 0) -> np.ndarray:
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        up = np.ascontiguousarray(up, dtype=np.float32)
+        rows, cols = gate.shape
+        bufs = [self.to_device(gate), self.to_device(up), self.alloc(rows * cols * 4)]
+        try:
+            check(self.lib.marmot_hip_glu(self.dev, ffn_type, C.c_void_p(bufs[0].ptr), C.c_void_p(bufs[1].ptr), rows,
+                                          cols, cols, cols, cols, C.c_void_p(bufs[2].ptr)))
+            return bufs[2].download(np.float32, (rows, cols))
+        finally:
+            for b in bufs:
+                b.free()
+
+    def swiglu_pack(self, gate: np.ndarray, up: np.ndarray, kind: int) -> np.ndarray:
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        up = np.ascontiguousarray(up, dtype=np.float32)
+        rows, cols = gate.shape
+        bufs = [self.to_device(gate), self.to_device(up), self.alloc(self.packed_activation_bytes(kind, rows, cols))]
+        try:
+            check(self.lib.marmot_hip_swiglu_pack(self.dev, C.c_void_p(bufs[0].ptr), C.c_void_p(bufs[1].ptr), rows,
+                                                  cols, kind, C.c_void_p(bufs[2].ptr)))
+            return bufs[2].download(np.uint8, (bufs[2].nbytes,))
+        finally:
+            for b in bufs:
+                b.free()
+
+    def add(self, a: np.ndarray, b: np.ndarray) -> np.ndarray:
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        bufs = [self.to_device(a), self.to_device(b), self.alloc(a.size * 4)]
+        try:
+            check(self.lib.marmot_hip_add(self.dev, C.c_void_p(bufs[0].ptr), C.c_void_p(bufs[1].ptr), a.size,
+                                          C.c_void_p(bufs[2].ptr)))
+            return bufs[2].download(np.float32, a.shape)
+        finally:
+            for b_ in bufs:
+                b_.free()
+
     def packed_activation_layout(self, kind: int, N: int, K: int) -> "capi.PackedLayout":
         lay = capi.PackedLayout()
         check(self.lib.marmot_hip_packed_activation_layout(kind, N, K, C.byref(lay)))

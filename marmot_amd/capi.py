@@ -109,6 +109,11 @@ SIGNATURES = {
     "marmot_hip_packed_activation_bytes": (_sz, [_i, _sz, _sz]),
     "marmot_hip_pack_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
     "marmot_hip_matmul_prepacked": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _vp, _i, _vp, _i]),
+    "marmot_hip_rms_norm": (_i, [_vp, _vp, _vp, _vp, _f, _f, _sz, _sz, _vp]),
+    "marmot_hip_rms_norm_pack": (_i, [_vp, _vp, _vp, _vp, _f, _f, _sz, _sz, _i, _vp, _vp]),
+    "marmot_hip_glu": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
+    "marmot_hip_swiglu_pack": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
+    "marmot_hip_add": (_i, [_vp, _vp, _vp, _sz, _vp]),
     "marmot_hip_topk": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
     "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "marmot_hip_moe_experts": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i,

@@ -183,17 +183,34 @@ bool map_ggml_type(uint32_t t, int *kind, int *dtype) {
     }
 }
 
-// bytes of a tensor: rows of the innermost (GGUF dimension 0) length, in blocks for quantized kinds
+// bytes of a tensor: rows of the innermost (GGUF dimension 0) length, in blocks for quantized kinds. The dimensions
+// come from the file: 0 when a product does not fit 64 bits (the caller rejects the file).
 size_t tensor_bytes(const marmot_hip_gguf::Entry &e, const uint64_t *raw) {
-    size_t rows = 1;
+    uint64_t rows = 1;
     for (uint32_t d = 1; d < e.ndim; ++d) {
-        rows *= (size_t)raw[d];
+        if (__builtin_mul_overflow(rows, raw[d], &rows)) {
+            return 0;
+        }
     }
+    uint64_t row_bytes;
     if (e.kind != 0) {
-        return rows * marmot_hip_row_bytes(e.kind, (size_t)raw[0]);
+        const uint64_t bv = marmot_hip_block_values(e.kind), bb = marmot_hip_block_bytes(e.kind);
+        uint64_t padded;
+        if (bv == 0 || __builtin_add_overflow(raw[0], bv - 1, &padded) ||
+            __builtin_mul_overflow(padded / bv, bb, &row_bytes)) {
+            return 0;
+        }
+    } else {
+        const uint64_t es = e.dtype == MARMOT_HIP_DTYPE_F32 || e.dtype == MARMOT_HIP_DTYPE_I32 ? 4 : 2;
+        if (__builtin_mul_overflow(raw[0], es, &row_bytes)) {
+            return 0;
+        }
     }
-    const size_t es = e.dtype == MARMOT_HIP_DTYPE_F32 || e.dtype == MARMOT_HIP_DTYPE_I32 ? 4 : 2;
-    return rows * (size_t)raw[0] * es;
+    uint64_t total;
+    if (__builtin_mul_overflow(rows, row_bytes, &total) || total > (uint64_t)SIZE_MAX) {
+        return 0;
+    }
+    return (size_t)total;
 }
 
 void fill_view(const marmot_hip_gguf *g, const marmot_hip_gguf::Entry &e, marmot_hip_gguf_tensor_t *out) {

@@ -3,7 +3,7 @@
 //
 // This file must be compiled with -ffp-contract=off: every fp32 multiply / subtract below is meant to
 // round on its own, exactly as the reference's scalar CPU code does.
-#include "mh_common.h"
+#include "mh_actquant.h"
 #include "mh_dequant.h"
 
 #include <float.h>
@@ -137,67 +137,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ 
         const size_t col = col0 + i;
         v[i] = col < k ? load_act_value<SRC>(x, x2, row * k + col) : 0.0f;
     }
-    // value of largest magnitude, first occurrence wins (strict > in index order)
-    float best_abs = 0.0f;
-    float best_val = 0.0f;
-    int best_idx = 0x7fffffff;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float ax = fabsf(v[i]);
-        if (ax > best_abs) {
-            best_abs = ax;
-            best_val = v[i];
-            best_idx = lane * 4 + i;
-        }
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float o_abs = __shfl_xor(best_abs, off);
-        const float o_val = __shfl_xor(best_val, off);
-        const int o_idx = __shfl_xor(best_idx, off);
-        if (o_abs > best_abs || (o_abs == best_abs && o_idx < best_idx)) {
-            best_abs = o_abs;
-            best_val = o_val;
-            best_idx = o_idx;
-        }
-    }
-
-    int q[4] = {0, 0, 0, 0};
-    float d = 0.0f;
-    if (best_abs > 0.0f) {
-        const float iscale = -127.0f / best_val;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int t = nearest_int_clamped(iscale * v[i]);
-            q[i] = t > 127 ? 127 : t;
-        }
-        d = 1.0f / iscale;
-    }
-    int s = q[0] + q[1] + q[2] + q[3];
-    s += __shfl_xor(s, 1);
-    s += __shfl_xor(s, 2); // lanes 4j..4j+3 hold the sum of values 16j..16j+15
-    const uint32_t packed = (uint32_t)(uint8_t)(int8_t)q[0] | ((uint32_t)(uint8_t)(int8_t)q[1] << 8) |
-        ((uint32_t)(uint8_t)(int8_t)q[2] << 16) | ((uint32_t)(uint8_t)(int8_t)q[3] << 24);
-
-    if constexpr (AOS) {
-        uint8_t *blk = blocks_out + (row * nb + b) * Q8_K_BYTES;
-        __builtin_memcpy(blk + 4 + lane * 4, &packed, 4);
-        if ((lane & 3) == 0) {
-            const int16_t bs = (int16_t)s;
-            __builtin_memcpy(blk + 4 + 256 + (lane >> 2) * 2, &bs, 2);
-        }
-        if (lane == 0) {
-            __builtin_memcpy(blk, &d, 4);
-        }
-    } else {
-        *(uint32_t *)(soa.qs + row * soa.kp + b * QK_K + lane * 4) = packed;
-        if ((lane & 3) == 0) {
-            soa.sums[(row * nb + b) * 16 + (lane >> 2)] = (int16_t)s;
-        }
-        if (lane == 0) {
-            soa.d[row * nb + b] = d;
-        }
-    }
+    q8k_block_store<AOS>(v, lane, row, b, nb, blocks_out, soa);
 }
 
 // Q8_0 (matmul_quant_pack.c:23-62, block.c:221-232 scalar): 32 lanes per block, one value per lane.
@@ -215,40 +155,7 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ 
     const size_t b = blk_id - row * nb;
     const size_t col = b * QK + lane32;
     const float v = col < k ? load_act_value<SRC>(x, x2, row * k + col) : 0.0f;
-    float max_abs = fabsf(v);
-#pragma unroll
-    for (int off = 1; off < 32; off <<= 1) {
-        max_abs = fmaxf(max_abs, __shfl_xor(max_abs, off));
-    }
-    float scale = max_abs / 127.0f;
-    if (scale < FLT_MIN) {
-        scale = 1.0f;
-    }
-    const float inv_scale = 1.0f / scale;
-    int q = (int)roundf(v * inv_scale);
-    q = q < -127 ? -127 : (q > 127 ? 127 : q);
-    if (col >= k) {
-        q = 0;
-    }
-    int s = q;
-#pragma unroll
-    for (int off = 1; off < 32; off <<= 1) {
-        s += __shfl_xor(s, off);
-    }
-    const uint16_t hs = f2h(scale);
-    if constexpr (AOS) {
-        uint8_t *blk = blocks_out + (row * nb + b) * Q8_0_BYTES;
-        blk[2 + lane32] = (uint8_t)(int8_t)q;
-        if (lane32 == 0) {
-            __builtin_memcpy(blk, &hs, 2);
-        }
-    } else {
-        soa.qs[row * soa.kp + b * QK + lane32] = (int8_t)q;
-        if (lane32 == 0) {
-            soa.d[row * nb + b] = h2f(hs);
-            soa.sums[row * nb + b] = (int16_t)s;
-        }
-    }
+    q8_0_block_store<AOS>(v, col < k, lane32, row, b, nb, blocks_out, soa);
 }
 
 // Plain 16-byte copy: device-to-device copies of the library, and the known-traffic kernel that profiler

@@ -2722,6 +2722,58 @@ static inline float moe_gelu(float x) {
     return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
 }
 
+/* ---- the fp32 ops between the linears
+ * RMS normalization, scalar float32 path: compute_mean_square_scalar + normalize_rms_scalar
+ * (src/backends/cpu/ops/normalization/scalar/normalization_scalar.c:469-510, 780-791), 1 / sqrtf
+ * (normalization_internal.h:8-10); weight_offset 0 is cpu_rmsnorm_impl, 1 cpu_rmsnorm_gemma_impl
+ * (normalization_dispatch.c:240-246). residual and weight may be NULL. */
+int mo_rms_norm(const float *x, const float *residual, const float *weight, float weight_offset, float eps,
+                size_t rows, size_t cols, float *out) {
+    if (rows == 0 || cols == 0) {
+        return MO_OK;
+    }
+    for (size_t r = 0; r < rows; ++r) {
+        const float *xr = x + r * cols;
+        const float *rr = residual != NULL ? residual + r * cols : NULL;
+        float *or_ = out + r * cols;
+        float sum = 0.0f;
+        for (size_t i = 0; i < cols; ++i) {
+            float v = xr[i];
+            if (rr != NULL) {
+                v += rr[i];
+            }
+            sum += v * v;
+        }
+        const float mean_sq = sum / (float)cols;
+        const float inv_rms = 1.0f / sqrtf(mean_sq + eps);
+        for (size_t i = 0; i < cols; ++i) {
+            float v = xr[i];
+            if (rr != NULL) {
+                v = xr[i] + rr[i];
+            }
+            or_[i] = weight != NULL ? v * inv_rms * (weight[i] + weight_offset) : v * inv_rms;
+        }
+    }
+    return MO_OK;
+}
+
+/* cpu_swiglu_f32_scalar / cpu_geglu_f32_scalar (src/backends/cpu/ops/elementwise/scalar/elementwise_f32_scalar.c:
+ * 11-20, 147-214): out = silu(gate) * up, or gelu_tanh(gate) * up (geglu != 0). */
+int mo_glu(const float *gate, const float *up, size_t n, int geglu, float *out) {
+    for (size_t i = 0; i < n; ++i) {
+        const float g = gate[i];
+        float a;
+        if (geglu) {
+            const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+            a = 0.5f * g * (1.0f + tanhf(inner));
+        } else {
+            a = g / (1.0f + expf(-g));
+        }
+        out[i] = a * up[i];
+    }
+    return MO_OK;
+}
+
 /* The gated product of moe_ops.c:548-559 on its own: out[i] = act(gate[i]) * up[i]. */
 int mo_moe_glu(const float *gate, const float *up, size_t n, int ffn_type, float *out) {
     if (ffn_type != MO_FFN_SWIGLU && ffn_type != MO_FFN_GEGLU) {

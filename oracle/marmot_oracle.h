@@ -183,6 +183,13 @@ int mo_topk(const float *x, size_t rows, size_t cols, size_t k, float *values_ou
 /* router: softmax over the k selected logits (graph_builder.cpp:2276-2316) */
 void mo_softmax_rows(const float *x, size_t rows, size_t k, float *out);
 
+/* RMS normalization of fp32 rows, scalar path (normalization_scalar.c:469-510, 780-791); weight_offset 1 is the Gemma
+ * variant. residual / weight may be NULL. */
+int mo_rms_norm(const float *x, const float *residual, const float *weight, float weight_offset, float eps,
+                size_t rows, size_t cols, float *out);
+/* silu(gate) * up, or gelu_tanh(gate) * up when geglu != 0 (elementwise_f32_scalar.c:11-20, 147-214) */
+int mo_glu(const float *gate, const float *up, size_t n, int geglu, float *out);
+
 /* act(gate[i]) * up[i] as the expert body computes it between the projections (moe_ops.c:548-559);
  * out may alias gate. */
 int mo_moe_glu(const float *gate, const float *up, size_t n, int ffn_type, float *out);

@@ -121,6 +121,11 @@ class Oracle:
         L.mo_topk.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
         L.mo_softmax_rows.restype = None
         L.mo_softmax_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+        L.mo_rms_norm.restype = C.c_int
+        L.mo_rms_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_size_t, C.c_size_t,
+                                  C.c_void_p]
+        L.mo_glu.restype = C.c_int
+        L.mo_glu.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
         L.mo_moe_glu.restype = C.c_int
         L.mo_moe_glu.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
         L.mo_moe_experts.restype = C.c_int
@@ -310,6 +315,25 @@ class Oracle:
         x = np.ascontiguousarray(x, dtype=np.float32)
         out = np.zeros_like(x)
         self.L.mo_softmax_rows(_ptr(x), x.shape[0], x.shape[1], _ptr(out))
+        return out
+
+    def rms_norm(self, x, weight=None, residual=None, eps: float = 1e-5, weight_offset: float = 0.0) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        rows, cols = x.shape
+        res = None if residual is None else np.ascontiguousarray(residual, dtype=np.float32)
+        w = None if weight is None else np.ascontiguousarray(weight, dtype=np.float32)
+        out = np.zeros_like(x)
+        st = self.L.mo_rms_norm(_ptr(x), _ptr(res) if res is not None else None, _ptr(w) if w is not None else None,
+                                weight_offset, eps, rows, cols, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_rms_norm -> {st}")
+        return out
+
+    def glu(self, gate, up, geglu: bool = False) -> np.ndarray:
+        gate = np.ascontiguousarray(gate, dtype=np.float32)
+        up = np.ascontiguousarray(up, dtype=np.float32)
+        out = np.zeros_like(gate)
+        self.L.mo_glu(_ptr(gate), _ptr(up), gate.size, 1 if geglu else 0, _ptr(out))
         return out
 
     def moe_glu(self, gate: np.ndarray, up: np.ndarray, ffn_type: int = 0) -> np.ndarray:

@@ -86,6 +86,20 @@ def test_malformed_files_are_rejected(tmp_path):
     at = data.index(b"w" + struct.pack("<I", 2)) + 1 + 4 + 16   # name, rank, two dimensions -> the type field
     data[at:at + 4] = struct.pack("<I", 99)
     assert opens(bytes(data), "type.gguf") == -8
+    # dimensions whose product wraps around 64 bits to the size of the stored payload (2^62 * 4 * 4 bytes = 2^66,
+    # plus a row count chosen so that the wrapped byte count equals the real one) must not pass the size check
+    at_dims = data.index(b"w" + struct.pack("<I", 2)) + 1 + 4
+    for dims in ((1 << 62, 4), (32, (1 << 62) + 4), ((1 << 63) + 32, 2), (0xFFFFFFFFFFFFFFFF, 0xFFFFFFFFFFFFFFFF)):
+        wrapped = bytearray(raw)
+        wrapped[at_dims:at_dims + 16] = struct.pack("<QQ", *dims)
+        assert opens(bytes(wrapped), "overflow.gguf") == -1, dims
+    blocks = np.zeros((4, 144), np.uint8)
+    q = bytearray(open(write_gguf(str(tmp_path / "q.gguf"), [("w", "q4_k", (256, 4), blocks)]), "rb").read())
+    at_q = q.index(b"w" + struct.pack("<I", 2)) + 1 + 4
+    for dims in ((0xFFFFFFFFFFFFFFFF, 4), (256, (1 << 64) // 144 + 4), ((1 << 63), 1 << 40)):
+        wrapped = bytearray(q)
+        wrapped[at_q:at_q + 16] = struct.pack("<QQ", *dims)
+        assert opens(bytes(wrapped), "overflow_q.gguf") == -1, dims
     with pytest.raises(capi.MarmotHipError):
         GgufFile(str(tmp_path / "does_not_exist.gguf"))
     assert not os.path.exists(str(tmp_path / "does_not_exist.gguf"))

@@ -239,6 +239,16 @@ struct marmot_topk_desc {
 };
 typedef struct marmot_topk_desc marmot_topk_desc_t;
 
+/* include/marmot/ops_types.h:181-187 */
+struct marmot_rmsnorm_desc {
+    const marmot_tensor_t *x;
+    const marmot_tensor_t *residual;
+    const marmot_tensor_t *weight;
+    marmot_tensor_t *out;
+    float eps;
+};
+typedef struct marmot_rmsnorm_desc marmot_rmsnorm_desc_t;
+
 struct marmot_moe_experts_desc {
     const marmot_tensor_t *hidden_states;
     const marmot_tensor_t *gate_exps;
@@ -348,13 +358,18 @@ typedef enum {
     MARMOT_OP_QKV_PROJECTION = 191,
     MARMOT_OP_DEQUANTIZE = 210,
     MARMOT_OP_MOE_EXPERTS = 263,
+    MARMOT_OP_SWIGLU = 331,
+    MARMOT_OP_GEGLU = 410,
+    MARMOT_OP_RMS_NORM_GEMMA = 447,
     MARMOT_OP_MATMUL = 498,
     MARMOT_OP_QUANTIZE = 524,
     MARMOT_OP_LINEAR = 708,
     MARMOT_OP_QKV_SHARED_INPUT = 771,
     MARMOT_OP_QKV_ROPE = 778,
     MARMOT_OP_EMBEDDING = 853,
+    MARMOT_OP_ADD = 876,
     MARMOT_OP_TOPK = 901,
+    MARMOT_OP_RMS_NORM = 929,
     MARMOT_OP_COUNT = 995,
 } marmot_op_id_t;
 
@@ -666,7 +681,9 @@ bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_bac
  *   EMBEDDING   u16 weights, token_ids, out; u32 dtype_out; f32 scale; u32 padding_id; u8 bounds_check,
  *               prefer_gpu_private, allow_quant_decode_on_the_fly       (bytecode_compile.c:989-1018)
  *   QUANTIZE    u16 input; u32 quant-params const offset; u16 output; u32 kind; u32 layout   (:912-941)
- *   DEQUANTIZE  u16 input; u16 output; u32 kind; u32 layout            (bytecode_compile.c:942-962) */
+ *   DEQUANTIZE  u16 input; u16 output; u32 kind; u32 layout            (bytecode_compile.c:942-962)
+ *   RMS_NORM    u16 input, weight, residual (0xFFFF none), output; f32 eps      (bytecode_compile.c:530-552)
+ *   BINARY      u16 input_a, input_b, output                            (bytecode_compile.c:357-375) */
 enum {
     MARMOT_HIP_BC_OP_END = 0,
     MARMOT_HIP_BC_OP_MATMUL_Q4_0 = 1,
@@ -717,7 +734,13 @@ enum {
     MARMOT_HIP_BC_OP_MOE_EXPERTS_Q8_1 = 45,
     MARMOT_HIP_BC_OP_QKV_Q8_1 = 46,
     MARMOT_HIP_BC_OP_EMBEDDING_Q8_1 = 47,
-    MARMOT_HIP_BC_OP_COUNT = 48,
+    /* the FLOAT32 ops between the linears */
+    MARMOT_HIP_BC_OP_RMS_NORM_F32 = 48,
+    MARMOT_HIP_BC_OP_RMS_NORM_GEMMA_F32 = 49,
+    MARMOT_HIP_BC_OP_SWIGLU_F32 = 50,
+    MARMOT_HIP_BC_OP_GEGLU_F32 = 51,
+    MARMOT_HIP_BC_OP_ADD_F32 = 52,
+    MARMOT_HIP_BC_OP_COUNT = 53,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -784,6 +807,21 @@ marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_q
 marmot_error_t hip_embedding_gather(const void *device_ctx, const marmot_embedding_gather_desc_t *desc);
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc);
 marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc);
+/* The FLOAT32 ops between the linears: cpu_rmsnorm_impl / cpu_rmsnorm_gemma_impl
+ * (src/backends/cpu/ops/normalization/normalization_dispatch.c:240-246; any rank, normalized over the last dimension,
+ * optional residual and weight), cpu_swiglu_f32_scalar / cpu_geglu_f32_scalar and the elementwise add
+ * (src/backends/cpu/ops/elementwise/scalar/elementwise_f32_scalar.c; contiguous or, for the gated products,
+ * row-strided 2-D tensors). A normalization of nine rows or more also leaves its output packed for the linears that
+ * read it, and a linear that packs an fp32 input of nine rows or more keeps the packed rows for the linears that
+ * share it (see activation_packs / activation_pack_hits below): no quantization launch per linear. */
+marmot_error_t hip_rmsnorm_impl(const void *device_ctx, const marmot_rmsnorm_desc_t *desc);
+marmot_error_t hip_rmsnorm_gemma_impl(const void *device_ctx, const marmot_rmsnorm_desc_t *desc);
+marmot_error_t hip_swiglu_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
+                              marmot_tensor_t *out);
+marmot_error_t hip_geglu_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
+                             marmot_tensor_t *out);
+marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
+                           marmot_tensor_t *out);
 /* output->quant_kind selects the activation block format: Q8_0 or Q8_K */
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output);
 /* input->quant_kind selects the weight block format: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K,
@@ -802,6 +840,8 @@ typedef struct {
     uint64_t upload_bytes;
     uint64_t downloads;
     uint64_t download_bytes;
+    uint64_t activation_packs;     /* packed copies of fp32 activation tensors made (by a normalization or a linear) */
+    uint64_t activation_pack_hits; /* linears that found their input already packed */
 } marmot_hip_residency_stats_t;
 void marmot_hip_backend_residency_stats(const void *device_ctx, marmot_hip_residency_stats_t *out);
 

@@ -56,9 +56,27 @@ typedef struct {
 } hip_rope_entry_t;
 #define HIP_ROPE_CACHE 8
 
+// Packed (quantized) copies of fp32 activation tensors, keyed by the tensor's host address: the normalization that
+// produces a tensor leaves its rows here already packed, and the first linear that reads an fp32 tensor of nine rows
+// or more packs it here for the linears that share the input (gate / up). An entry dies when anything writes the
+// tensor, when the host copy changes or when the host memory is released.
+typedef struct {
+    bool valid;
+    uintptr_t host;
+    size_t rows, cols;
+    int act_kind;       // MARMOT_HIP_KIND_Q8_K or MARMOT_HIP_KIND_Q8_0
+    void *packed;       // device buffer, owned
+    size_t capacity;
+    uint64_t stamp;     // last use: the oldest entry is replaced
+} hip_pack_entry_t;
+#define HIP_PACK_CACHE 4
+#define HIP_PACK_MIN_ROWS 9  // below, the linears quantize fp32 rows inside their own kernels
+
 typedef struct {
     marmot_hip_device_t *dev;
     pthread_mutex_t mu;
+    hip_pack_entry_t packs[HIP_PACK_CACHE];
+    uint64_t pack_clock, packs_made, pack_hits;
     hip_mirror_t *mirrors;  // sorted by host
     size_t n_mirrors, cap_mirrors;
     hip_rope_entry_t rope[HIP_ROPE_CACHE];
@@ -181,6 +199,66 @@ static marmot_error_t cover(hip_backend_t *b, uintptr_t p, size_t n, bool will_r
     return MARMOT_SUCCESS;
 }
 
+static void packs_invalidate(hip_backend_t *b, uintptr_t p, size_t n) {
+    for (int i = 0; i < HIP_PACK_CACHE; ++i) {
+        hip_pack_entry_t *e = &b->packs[i];
+        if (e->valid && e->host < p + n && p < e->host + e->rows * e->cols * sizeof(float)) {
+            e->valid = false;
+        }
+    }
+}
+
+static hip_pack_entry_t *packs_find(hip_backend_t *b, const void *host, size_t rows, size_t cols, int act_kind) {
+    for (int i = 0; i < HIP_PACK_CACHE; ++i) {
+        hip_pack_entry_t *e = &b->packs[i];
+        if (e->valid && e->host == (uintptr_t)host && e->rows == rows && e->cols == cols && e->act_kind == act_kind) {
+            e->stamp = ++b->pack_clock;
+            return e;
+        }
+    }
+    return nullptr;
+}
+
+// an entry (not yet valid) with room for the packed rows: an invalid one, else the least recently used
+static marmot_error_t packs_reserve(hip_backend_t *b, int weight_kind, size_t rows, size_t cols,
+                                    hip_pack_entry_t **out) {
+    hip_pack_entry_t *e = &b->packs[0];
+    for (int i = 0; i < HIP_PACK_CACHE; ++i) {
+        hip_pack_entry_t *c = &b->packs[i];
+        if (!c->valid) {
+            e = c;
+            break;
+        }
+        if (c->stamp < e->stamp) {
+            e = c;
+        }
+    }
+    e->valid = false;
+    const size_t need = marmot_hip_packed_activation_bytes(weight_kind, rows, cols);
+    if (need == 0) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "packed activations: unsupported weight kind");
+    }
+    if (e->capacity < need) {
+        if (e->packed != nullptr) {
+            marmot_hip_synchronize(b->dev);  // a kernel may still read the old buffer
+            marmot_hip_free(b->dev, e->packed);
+            e->packed = nullptr;
+            e->capacity = 0;
+        }
+        const int st = marmot_hip_alloc(b->dev, need, &e->packed);
+        if (st != MARMOT_HIP_SUCCESS) {
+            return fail_from_lib(st);
+        }
+        e->capacity = need;
+    }
+    *out = e;
+    return MARMOT_SUCCESS;
+}
+
+static int act_kind_of_weight(int weight_kind) {
+    return marmot_hip_block_values(weight_kind) == 256 ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
+}
+
 // device address of a kernel input: uploads the mirror when the host copy is newer
 static marmot_error_t acquire_read(hip_backend_t *b, const void *host, size_t n, const void **d_out) {
     hip_mirror_t *m = nullptr;
@@ -214,6 +292,7 @@ static marmot_error_t acquire_write(hip_backend_t *b, void *host, size_t n, void
     }
     m->host_newer = false;
     m->dev_newer = true;
+    packs_invalidate(b, (uintptr_t)host, n);
     *d_out = (uint8_t *)m->dev + ((uintptr_t)host - m->host);
     return MARMOT_SUCCESS;
 }
@@ -323,6 +402,11 @@ static void ops_destroy(const void *device_ctx) {
         marmot_hip_free(b->dev, b->mirrors[i].dev);
     }
     free(b->mirrors);
+    for (int i = 0; i < HIP_PACK_CACHE; ++i) {
+        if (b->packs[i].packed != nullptr) {
+            marmot_hip_free(b->dev, b->packs[i].packed);
+        }
+    }
     for (size_t i = 0; i < HIP_ROPE_CACHE; ++i) {
         free(b->rope[i].freqs);
     }
@@ -356,6 +440,7 @@ static void ops_free(const void *device_ctx, void *ptr) {
 // dst == src == host pointer: the host copy is newer than the mirror (src/core/tensor/transfer.c:22)
 static marmot_error_t host_is_newer_locked(hip_backend_t *b, const void *src, size_t size) {
     const uintptr_t p = (uintptr_t)src;
+    packs_invalidate(b, p, size);
     hip_mirror_t *m = find_containing(b, p, size);
     if (m != nullptr) {
         if (p == m->host && size == m->bytes) {
@@ -493,6 +578,7 @@ static void ops_on_host_range_freed(void *device_ctx, const void *start, size_t 
         return;
     }
     pthread_mutex_lock(&b->mu);
+    packs_invalidate(b, (uintptr_t)start, length);
     bool synced = false;
     for (size_t i = 0; i < b->n_mirrors;) {
         if (!overlaps(&b->mirrors[i], (uintptr_t)start, length)) {
@@ -562,8 +648,37 @@ static marmot_error_t matmul_locked(hip_backend_t *b, const matmul_plan_t *p, co
     if (st != MARMOT_SUCCESS) {
         return st;
     }
-    const int rc = marmot_hip_matmul_quantized(b->dev, p->kind, d_w, d_x, p->in_dtype, p->N, p->K, p->M, d_b,
-                                               p->bias_dtype, d_y, p->out_dtype, 0);
+    int rc;
+    if (p->in_dtype == MARMOT_HIP_DTYPE_F32 && p->N >= HIP_PACK_MIN_ROWS) {
+        // fp32 rows that a normalization already left packed, or that an earlier linear packed: no quantization
+        // launch; otherwise pack them here, once, for this linear and the ones that share its input
+        const int act_kind = act_kind_of_weight(p->kind);
+        hip_pack_entry_t *e = packs_find(b, input->data, p->N, p->K, act_kind);
+        if (e != nullptr) {
+            b->pack_hits++;
+        } else {
+            st = packs_reserve(b, p->kind, p->N, p->K, &e);
+            if (st != MARMOT_SUCCESS) {
+                return st;
+            }
+            rc = marmot_hip_pack_activations(b->dev, p->kind, d_x, MARMOT_HIP_DTYPE_F32, p->N, p->K, e->packed);
+            if (rc != MARMOT_HIP_SUCCESS) {
+                return fail_from_lib(rc);
+            }
+            e->valid = true;
+            e->host = (uintptr_t)input->data;
+            e->rows = p->N;
+            e->cols = p->K;
+            e->act_kind = act_kind;
+            e->stamp = ++b->pack_clock;
+            b->packs_made++;
+        }
+        rc = marmot_hip_matmul_prepacked(b->dev, p->kind, d_w, e->packed, p->N, p->K, p->M, d_b, p->bias_dtype, d_y,
+                                         p->out_dtype);
+    } else {
+        rc = marmot_hip_matmul_quantized(b->dev, p->kind, d_w, d_x, p->in_dtype, p->N, p->K, p->M, d_b, p->bias_dtype,
+                                         d_y, p->out_dtype, 0);
+    }
     if (rc != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(rc);
     }
@@ -1193,6 +1308,175 @@ static marmot_error_t dequantize_block(const void *device_ctx, const marmot_tens
 }
 
 // ------------------------------------------------------------------ bytecode exec entries
+// ------------------------------------------------------------------ ops between the linears
+// marmot_norm_validate (src/core/helpers/norm.c) for RMS normalization: x and out of one shape and dtype, residual
+// like x, weight a vector of the last dimension; FLOAT32 only here.
+static marmot_error_t rmsnorm(const void *device_ctx, const marmot_rmsnorm_desc_t *desc, float weight_offset) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (desc == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RMSNorm descriptor is null");
+    }
+    const marmot_tensor_t *x = desc->x, *res = desc->residual, *w = desc->weight;
+    marmot_tensor_t *out = desc->out;
+    if (b == nullptr || x == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RMSNorm requires input and output tensors");
+    }
+    if (x->shape.ndim == 0 || x->shape.ndim != out->shape.ndim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RMSNorm input/output rank mismatch");
+    }
+    for (size_t i = 0; i < x->shape.ndim; ++i) {
+        if (x->shape.shape[i] != out->shape.shape[i] || (res != nullptr && (res->shape.ndim != x->shape.ndim ||
+                                                                           res->shape.shape[i] != x->shape.shape[i]))) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RMSNorm tensor shapes do not match");
+        }
+    }
+    const size_t cols = x->shape.shape[x->shape.ndim - 1];
+    if (w != nullptr && tensor_numel(w) != cols) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RMSNorm weight length does not match the normalized dimension");
+    }
+    if (x->dtype != MARMOT_DTYPE_FLOAT32 || out->dtype != MARMOT_DTYPE_FLOAT32 ||
+        (res != nullptr && res->dtype != MARMOT_DTYPE_FLOAT32) || (w != nullptr && w->dtype != MARMOT_DTYPE_FLOAT32)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP RMSNorm handles FLOAT32 tensors");
+    }
+    if (!dense_contiguous(x) || !dense_contiguous(out) || (res != nullptr && !dense_contiguous(res)) ||
+        (w != nullptr && !dense_contiguous(w))) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP RMSNorm needs contiguous tensors");
+    }
+    const size_t n = tensor_numel(x);
+    if (n == 0 || cols == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+    if (x->data == nullptr || out->data == nullptr || (res != nullptr && res->data == nullptr) ||
+        (w != nullptr && w->data == nullptr)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RMSNorm: tensor without data");
+    }
+    const size_t rows = n / cols;
+    pthread_mutex_lock(&b->mu);
+    const void *d_x = nullptr, *d_r = nullptr, *d_w = nullptr;
+    void *d_y = nullptr;
+    marmot_error_t st = acquire_read(b, x->data, n * sizeof(float), &d_x);
+    if (st == MARMOT_SUCCESS && res != nullptr) {
+        st = acquire_read(b, res->data, n * sizeof(float), &d_r);
+    }
+    if (st == MARMOT_SUCCESS && w != nullptr) {
+        st = acquire_read(b, w->data, cols * sizeof(float), &d_w);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write(b, out->data, n * sizeof(float), &d_y);  // also ends any packed copy of the old contents
+    }
+    if (st == MARMOT_SUCCESS) {
+        int rc;
+        // Rows that the linears behind this normalization would quantize in a launch of their own are packed here,
+        // in the same launch: Q8_K when the rows are whole 256-value blocks (K-quant weights), else Q8_0.
+        hip_pack_entry_t *e = nullptr;
+        const int for_kind = cols % 256 == 0 ? MARMOT_HIP_KIND_Q4_K : MARMOT_HIP_KIND_Q8_0;
+        if (rows >= HIP_PACK_MIN_ROWS && cols % 32 == 0 && packs_reserve(b, for_kind, rows, cols, &e) == MARMOT_SUCCESS) {
+            rc = marmot_hip_rms_norm_pack(b->dev, (const float *)d_x, (const float *)d_r, (const float *)d_w,
+                                          weight_offset, desc->eps, rows, cols, for_kind, (float *)d_y, e->packed);
+            if (rc == MARMOT_HIP_SUCCESS) {
+                e->valid = true;
+                e->host = (uintptr_t)out->data;
+                e->rows = rows;
+                e->cols = cols;
+                e->act_kind = act_kind_of_weight(for_kind);
+                e->stamp = ++b->pack_clock;
+                b->packs_made++;
+            }
+        } else {
+            rc = marmot_hip_rms_norm(b->dev, (const float *)d_x, (const float *)d_r, (const float *)d_w, weight_offset,
+                                     desc->eps, rows, cols, (float *)d_y);
+        }
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
+// swiglu / geglu / add on FLOAT32 tensors of one shape: contiguous, or 2-D with unit column stride (row-strided, the
+// halves of a fused gate/up projection: cpu_row_strided_2d, elementwise_f32_scalar.c:22-45)
+typedef enum { HIP_BIN_SWIGLU, HIP_BIN_GEGLU, HIP_BIN_ADD } hip_binary_op_t;
+
+static bool row_strided_2d(const marmot_tensor_t *t) {
+    return t->shape.ndim == 2 && t->shape.strides[1] == 1 && t->shape.strides[0] >= t->shape.shape[1];
+}
+
+static size_t strided_span_bytes(const marmot_tensor_t *t) {
+    if (t->shape.ndim == 2 && !dense_contiguous(t)) {
+        return ((t->shape.shape[0] - 1) * t->shape.strides[0] + t->shape.shape[1]) * sizeof(float);
+    }
+    return dense_bytes(t);
+}
+
+static marmot_error_t binary_f32(const void *device_ctx, hip_binary_op_t op, const marmot_tensor_t *a,
+                                 const marmot_tensor_t *c, marmot_tensor_t *out) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || a == nullptr || c == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Binary operation: null tensor");
+    }
+    if (a->shape.ndim != c->shape.ndim || a->shape.ndim != out->shape.ndim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Binary operation: rank mismatch");
+    }
+    for (size_t i = 0; i < a->shape.ndim; ++i) {
+        if (a->shape.shape[i] != c->shape.shape[i] || a->shape.shape[i] != out->shape.shape[i]) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Binary operation: shapes do not match");
+        }
+    }
+    if (a->dtype != MARMOT_DTYPE_FLOAT32 || c->dtype != MARMOT_DTYPE_FLOAT32 || out->dtype != MARMOT_DTYPE_FLOAT32) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP elementwise operations handle FLOAT32 tensors");
+    }
+    const bool dense = dense_contiguous(a) && dense_contiguous(c) && dense_contiguous(out);
+    const bool strided = row_strided_2d(a) && row_strided_2d(c) && row_strided_2d(out);
+    if (!dense && !(strided && op != HIP_BIN_ADD)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP elementwise operations need contiguous or row-strided tensors");
+    }
+    const size_t n = tensor_numel(a);
+    if (n == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+    if (a->data == nullptr || c->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Binary operation: tensor without data");
+    }
+    pthread_mutex_lock(&b->mu);
+    const void *d_a = nullptr, *d_c = nullptr;
+    void *d_y = nullptr;
+    marmot_error_t st = acquire_read(b, a->data, strided_span_bytes(a), &d_a);
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, c->data, strided_span_bytes(c), &d_c);
+    }
+    if (st == MARMOT_SUCCESS) {
+        // a row-strided output keeps the bytes between its rows: acquire_write uploads them when only the host has them
+        st = acquire_write(b, out->data, strided_span_bytes(out), &d_y);
+    }
+    if (st == MARMOT_SUCCESS) {
+        int rc;
+        if (op == HIP_BIN_ADD) {
+            rc = marmot_hip_add(b->dev, (const float *)d_a, (const float *)d_c, n, (float *)d_y);
+        } else {
+            size_t rows = 1, cols = n, sa = n, sc = n, so = n;
+            if (!dense) {
+                rows = a->shape.shape[0];
+                cols = a->shape.shape[1];
+                sa = a->shape.strides[0];
+                sc = c->shape.strides[0];
+                so = out->shape.strides[0];
+            }
+            rc = marmot_hip_glu(b->dev, op == HIP_BIN_GEGLU ? MARMOT_HIP_FFN_GEGLU : MARMOT_HIP_FFN_SWIGLU,
+                                (const float *)d_a, (const float *)d_c, rows, cols, sa, sc, so, (float *)d_y);
+        }
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
 static uint16_t rd_u16(const uint8_t **pc) {
     const uint16_t v = (uint16_t)((*pc)[0] | ((*pc)[1] << 8));
     *pc += 2;
@@ -1432,6 +1716,65 @@ static marmot_error_t bc_exec_dequantize(const void *exec_ctx, marmot_tensor_t *
     return dequantize_block(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, input, output);
 }
 
+// RMS_NORM: u16 input, weight, residual (0xFFFF none), output; f32 eps (bytecode_compile.c:530-552)
+static marmot_error_t bc_exec_rms_norm_offset(float weight_offset, const void *exec_ctx, marmot_tensor_t **regs,
+                                              const uint8_t *imm) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    marmot_rmsnorm_desc_t desc = {0};
+    desc.x = reg(regs, rd_u16(&pc));
+    desc.weight = reg(regs, rd_u16(&pc));
+    desc.residual = reg(regs, rd_u16(&pc));
+    desc.out = reg(regs, rd_u16(&pc));
+    desc.eps = rd_f32(&pc);
+    return rmsnorm(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc, weight_offset);
+}
+
+static marmot_error_t bc_exec_rms_norm(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                       const uint8_t *const_pool) {
+    (void)const_pool;
+    return bc_exec_rms_norm_offset(0.0f, exec_ctx, regs, imm);
+}
+
+static marmot_error_t bc_exec_rms_norm_gemma(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                             const uint8_t *const_pool) {
+    (void)const_pool;
+    return bc_exec_rms_norm_offset(1.0f, exec_ctx, regs, imm);
+}
+
+// BINARY: u16 input_a, input_b, output (bytecode_compile.c:357-375)
+static marmot_error_t bc_exec_binary(hip_binary_op_t op, const void *exec_ctx, marmot_tensor_t **regs,
+                                     const uint8_t *imm) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *a = reg(regs, rd_u16(&pc));
+    const marmot_tensor_t *c = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    return binary_f32(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, op, a, c, out);
+}
+
+static marmot_error_t bc_exec_swiglu(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                     const uint8_t *const_pool) {
+    (void)const_pool;
+    return bc_exec_binary(HIP_BIN_SWIGLU, exec_ctx, regs, imm);
+}
+
+static marmot_error_t bc_exec_geglu(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                    const uint8_t *const_pool) {
+    (void)const_pool;
+    return bc_exec_binary(HIP_BIN_GEGLU, exec_ctx, regs, imm);
+}
+
+static marmot_error_t bc_exec_add(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                  const uint8_t *const_pool) {
+    (void)const_pool;
+    return bc_exec_binary(HIP_BIN_ADD, exec_ctx, regs, imm);
+}
+
 static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     0,               // END
     12, 12, 12, 12,  // MATMUL: 3 x u16 + u32 + u16
@@ -1448,6 +1791,8 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     12, 26, 28, 21,  // Q2_K
     12, 26, 28, 21,  // Q3_K
     12, 26, 28, 21,  // Q8_1
+    12, 12,          // RMS_NORM, RMS_NORM_GEMMA: 4 x u16 + f32
+    6, 6, 6,         // SWIGLU, GEGLU, ADD (BINARY): 3 x u16
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1466,6 +1811,8 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
+    MARMOT_BC_SCHEMA_RMS_NORM,    MARMOT_BC_SCHEMA_RMS_NORM,
+    MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1482,6 +1829,8 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_matmul_q2_k, bc_exec_moe,         bc_exec_qkv_q2_k,    bc_exec_embedding,
     bc_exec_matmul_q3_k, bc_exec_moe,         bc_exec_qkv_q3_k,    bc_exec_embedding,
     bc_exec_matmul_q8_1, bc_exec_moe,         bc_exec_qkv_q8_1,    bc_exec_embedding,
+    bc_exec_rms_norm,    bc_exec_rms_norm_gemma,
+    bc_exec_swiglu,      bc_exec_geglu,       bc_exec_add,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -1704,6 +2053,24 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
                                       MARMOT_HIP_BC_OP_MOE_EXPERTS_Q5_K);
         return selected(op, 0.0, 0.0);
     }
+    case MARMOT_OP_RMS_NORM:
+    case MARMOT_OP_RMS_NORM_GEMMA:
+        // rms_norm_scalar / rms_norm_gemma_scalar (cpu/kernels/normalization.def): FLOAT32 rows, contiguous
+        if (!in32 || !out32) {
+            return unsupported("HIP RMSNorm handles FLOAT32 tensors");
+        }
+        return selected(sig->op_id == MARMOT_OP_RMS_NORM ? MARMOT_HIP_BC_OP_RMS_NORM_F32
+                                                         : MARMOT_HIP_BC_OP_RMS_NORM_GEMMA_F32, launch_us, 0.0);
+    case MARMOT_OP_SWIGLU:
+    case MARMOT_OP_GEGLU:
+    case MARMOT_OP_ADD:
+        // glu_scalar / elementwise add (cpu/kernels/elementwise.def): FLOAT32
+        if (!in32 || !out32) {
+            return unsupported("HIP elementwise operations handle FLOAT32 tensors");
+        }
+        return selected(sig->op_id == MARMOT_OP_SWIGLU  ? MARMOT_HIP_BC_OP_SWIGLU_F32
+                        : sig->op_id == MARMOT_OP_GEGLU ? MARMOT_HIP_BC_OP_GEGLU_F32
+                                                        : MARMOT_HIP_BC_OP_ADD_F32, launch_us, 0.0);
     case MARMOT_OP_TOPK:
         if (!in32 || !out32) {
             return unsupported("HIP TopK takes FLOAT32 values");
@@ -1889,6 +2256,24 @@ marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_exp
 marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc) {
     return topk(device_ctx, desc);
 }
+marmot_error_t hip_rmsnorm_impl(const void *device_ctx, const marmot_rmsnorm_desc_t *desc) {
+    return rmsnorm(device_ctx, desc, 0.0f);
+}
+marmot_error_t hip_rmsnorm_gemma_impl(const void *device_ctx, const marmot_rmsnorm_desc_t *desc) {
+    return rmsnorm(device_ctx, desc, 1.0f);
+}
+marmot_error_t hip_swiglu_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
+                              marmot_tensor_t *out) {
+    return binary_f32(device_ctx, HIP_BIN_SWIGLU, a, b, out);
+}
+marmot_error_t hip_geglu_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
+                             marmot_tensor_t *out) {
+    return binary_f32(device_ctx, HIP_BIN_GEGLU, a, b, out);
+}
+marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
+                           marmot_tensor_t *out) {
+    return binary_f32(device_ctx, HIP_BIN_ADD, a, b, out);
+}
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
     return quantize_block(device_ctx, input, output);
 }
@@ -1922,5 +2307,7 @@ void marmot_hip_backend_residency_stats(const void *device_ctx, marmot_hip_resid
     out->upload_bytes = b->upload_bytes;
     out->downloads = b->downloads;
     out->download_bytes = b->download_bytes;
+    out->activation_packs = b->packs_made;
+    out->activation_pack_hits = b->pack_hits;
     pthread_mutex_unlock(&b->mu);
 }

@@ -40,6 +40,9 @@ BACKEND_HIP = 3
 OP_DEQUANTIZE, OP_MOE_EXPERTS, OP_MATMUL, OP_QUANTIZE, OP_LINEAR, OP_TOPK = 210, 263, 498, 524, 708, 901
 OP_QKV_PROJECTION, OP_QKV_SHARED_INPUT, OP_QKV_ROPE = 191, 771, 778
 OP_EMBEDDING = 853
+OP_SWIGLU, OP_GEGLU, OP_RMS_NORM_GEMMA, OP_ADD, OP_RMS_NORM = 331, 410, 447, 876, 929
+# this backend's bytecode ops for them (include/marmot_hip_backend.h)
+BC_OP_RMS_NORM_F32, BC_OP_RMS_NORM_GEMMA_F32, BC_OP_SWIGLU_F32, BC_OP_GEGLU_F32, BC_OP_ADD_F32 = 48, 49, 50, 51, 52
 PREFERENCE_DEFAULT, PREFERENCE_ENABLE, PREFERENCE_DISABLE = 0, 1, 2
 QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q4_1: 2, KIND_Q5_0: 3, KIND_Q5_1: 4, KIND_Q8_0: 5, KIND_Q2_K: 6, KIND_Q3_K: 7, KIND_Q4_K: 8,
@@ -110,6 +113,12 @@ class EmbeddingGatherDesc(C.Structure):
 class TopkDesc(C.Structure):
     _fields_ = [("x", C.POINTER(Tensor)), ("values_out", C.POINTER(Tensor)), ("indices_out", C.POINTER(Tensor)),
                 ("axis", C.c_int32), ("k", C.c_uint32)]
+
+
+class RmsNormDesc(C.Structure):
+    """marmot_rmsnorm_desc_t"""
+    _fields_ = [("x", C.POINTER(Tensor)), ("residual", C.POINTER(Tensor)), ("weight", C.POINTER(Tensor)),
+                ("out", C.POINTER(Tensor)), ("eps", C.c_float)]
 
 
 class MoeDesc(C.Structure):
@@ -238,7 +247,8 @@ class BcTables(C.Structure):
 
 class ResidencyStats(C.Structure):
     _fields_ = [("mirrors", C.c_size_t), ("mirrored_bytes", C.c_size_t), ("uploads", C.c_uint64),
-                ("upload_bytes", C.c_uint64), ("downloads", C.c_uint64), ("download_bytes", C.c_uint64)]
+                ("upload_bytes", C.c_uint64), ("downloads", C.c_uint64), ("download_bytes", C.c_uint64),
+                ("activation_packs", C.c_uint64), ("activation_pack_hits", C.c_uint64)]
 
 
 #: exported symbols of the tensor-level layer (checked against include/marmot_hip_backend.h by the tests)
@@ -252,6 +262,7 @@ BACKEND_SYMBOLS = [
     "hip_matmul_qkv_q3_k", "hip_matmul_quantized_q8_1", "hip_matmul_qkv_q8_1", "hip_matmul_qkv_q4_0", "hip_matmul_qkv_q8_0", "hip_matmul_qkv_q4_k",
     "hip_matmul_qkv_q5_k", "hip_matmul_qkv_q6_k", "hip_embedding_gather", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
+    "hip_rmsnorm_impl", "hip_rmsnorm_gemma_impl", "hip_swiglu_f32", "hip_geglu_f32", "hip_add_f32",
 ]
 
 
@@ -284,6 +295,14 @@ def bind(lib: C.CDLL) -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor)]
+    for name in ("hip_rmsnorm_impl", "hip_rmsnorm_gemma_impl"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.c_void_p, C.POINTER(RmsNormDesc)]
+    for name in ("hip_swiglu_f32", "hip_geglu_f32", "hip_add_f32"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]
     lib.marmot_hip_backend_last_error.restype = C.c_int
     lib.marmot_hip_backend_last_error.argtypes = [C.POINTER(C.c_char_p)]
     lib.marmot_hip_backend_residency_stats.restype = None
@@ -438,6 +457,15 @@ class HipContext:
         sig.weight_layout = WEIGHT_LAYOUT_SEPARATE
         return sig
 
+    def float_op_signature(self, op_id: int, dtype: int = DTYPE_F32) -> OpSignature:
+        """Normalization and elementwise operations: one dtype for input, weight, output (cpu/kernels/normalization.def,
+        elementwise.def)."""
+        sig = OpSignature()
+        sig.op_id = op_id
+        sig.input_dtype = sig.weight_dtype = sig.output_dtype = dtype
+        sig.accum_dtype = DTYPE_F32
+        return sig
+
     def query(self, sig: OpSignature, caps: Optional[DeviceCaps] = None) -> KernelSelection:
         caps = caps if caps is not None else self.lib.marmot_hip_detect_default_caps()
         return self.lib.marmot_hip_query_kernel(C.byref(sig), C.byref(caps))
@@ -534,6 +562,13 @@ class Program:
     def topk(self, op_index: int, x, values, indices, k: int, axis: int = 1):
         self.code += struct.pack("<HHHHII", op_index, self.reg(x), self.reg(values), self.reg(indices),
                                  axis & 0xFFFFFFFF, k)
+
+    def rms_norm(self, op_index: int, x, weight, residual, out, eps: float):
+        self.code += struct.pack("<HHHHHf", op_index, self.reg(x), self.reg(weight), self.reg(residual),
+                                 self.reg(out), eps)
+
+    def binary(self, op_index: int, a, b, out):
+        self.code += struct.pack("<HHHH", op_index, self.reg(a), self.reg(b), self.reg(out))
 
     def quantize(self, op_index: int, x, out):
         self.code += struct.pack("<HHIHII", op_index, self.reg(x), BC_INVALID_OFFSET, self.reg(out),

@@ -61,6 +61,8 @@ int main(void) {
     VAL(MARMOT_BC_SCHEMA_TOPK); VAL(MARMOT_BC_SCHEMA_MOE_EXPERTS); VAL(MARMOT_BC_SCHEMA_MATMUL);
     VAL(MARMOT_BC_SCHEMA_QUANTIZE); VAL(MARMOT_BC_SCHEMA_DEQUANTIZE);
     VAL(MARMOT_BC_REG_INVALID); VAL(MARMOT_BC_INVALID_OFFSET); VAL(MARMOT_BC_END);
+    VAL(MARMOT_OP_RMS_NORM); VAL(MARMOT_OP_RMS_NORM_GEMMA); VAL(MARMOT_OP_SWIGLU); VAL(MARMOT_OP_GEGLU); VAL(MARMOT_OP_ADD);
+    VAL(MARMOT_BC_SCHEMA_RMS_NORM); VAL(MARMOT_BC_SCHEMA_BINARY);
 
     SZ(marmot_shape_t); OFF(marmot_shape_t, ndim); OFF(marmot_shape_t, shape); OFF(marmot_shape_t, strides);
     SZ(marmot_quant_params_t);
@@ -100,6 +102,8 @@ int main(void) {
     OFF(marmot_embedding_gather_desc_t, prefer_gpu_private);
     OFF(marmot_embedding_gather_desc_t, allow_quant_decode_on_the_fly);
     SZ(marmot_topk_desc_t); OFF(marmot_topk_desc_t, axis); OFF(marmot_topk_desc_t, k);
+    SZ(marmot_rmsnorm_desc_t); OFF(marmot_rmsnorm_desc_t, residual); OFF(marmot_rmsnorm_desc_t, weight);
+    OFF(marmot_rmsnorm_desc_t, out); OFF(marmot_rmsnorm_desc_t, eps);
     SZ(marmot_moe_experts_desc_t); OFF(marmot_moe_experts_desc_t, out); OFF(marmot_moe_experts_desc_t, ffn_type);
     OFF(marmot_moe_experts_desc_t, weights_scale); OFF(marmot_moe_experts_desc_t, router_weight_policy);
     SZ(marmot_matmul_dims_t); SZ(marmot_quant_block_t); SZ(marmot_op_signature_dims_t);

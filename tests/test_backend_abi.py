@@ -57,6 +57,7 @@ def test_ctypes_structs_match_layout(golden_layout):
     pairs = {
         "marmot_shape_t": ta.Shape, "marmot_tensor_t": ta.Tensor, "marmot_matmul_epilogue_t": ta.Epilogue,
         "marmot_topk_desc_t": ta.TopkDesc, "marmot_moe_experts_desc_t": ta.MoeDesc,
+        "marmot_rmsnorm_desc_t": ta.RmsNormDesc,
         "marmot_op_signature_t": ta.OpSignature, "marmot_kernel_selection_t": ta.KernelSelection,
         "marmot_device_caps_t": ta.DeviceCaps, "marmot_device_ops_t": ta.DeviceOps,
         "marmot_bc_exec_ctx_t": ta.BcExecCtx, "marmot_bc_tables_t": ta.BcTables,
@@ -280,7 +281,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 48
+    assert t.op_count == 53
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -306,6 +307,12 @@ def test_bytecode_tables(lib, golden_layout):
         assert schema[base:base + 4] == [golden_layout[f"MARMOT_BC_SCHEMA_{n}"]
                                          for n in ("MATMUL", "MOE_EXPERTS", "QKV", "EMBEDDING")]
         assert sizes[base:base + 4] == [sizes[1], sizes[5], sizes[12], sizes[16]]
+    # the FLOAT32 ops between the linears: two normalizations, three binary ops
+    assert schema[48:50] == [golden_layout["MARMOT_BC_SCHEMA_RMS_NORM"]] * 2
+    assert schema[50:53] == [golden_layout["MARMOT_BC_SCHEMA_BINARY"]] * 3
+    assert sizes[48:50] == [struct.calcsize("<4Hf")] * 2 and sizes[50:53] == [struct.calcsize("<3H")] * 3
+    assert (ta.BC_OP_RMS_NORM_F32, ta.BC_OP_RMS_NORM_GEMMA_F32, ta.BC_OP_SWIGLU_F32, ta.BC_OP_GEGLU_F32,
+            ta.BC_OP_ADD_F32) == (48, 49, 50, 51, 52)
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -370,16 +377,19 @@ def test_kernel_def_files_name_exported_impls(lib):
     qkv = {f"{op}_quantized_hip_{dt}" for op in ("qkv_shared_input", "qkv_projection") for dt in ("f16", "f32")}
     assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_f32", "topk_hip",
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
-                             "embedding_quantized_hip"} | qkv
+                             "embedding_quantized_hip", "rms_norm_hip", "rms_norm_gemma_hip", "glu_hip",
+                             "add_hip"} | qkv
     for name in qkv:
         f = families[name]
         assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name
     for name, f in families.items():
         impl = f["IMPL_FUNCTION"].strip('"')
         schemes = re.findall(r"Q\d_[01K]", f.get("AXIS(scheme)", "")) or [""]
+        ops = re.findall(r"\w+", f.get("AXIS(op)", "")) or [""]
         for s in schemes:
-            sym = impl.replace("{scheme:lower}", s.lower())
-            assert hasattr(lib, sym), f"{name}: {sym} not exported"
+            for o in ops:
+                sym = impl.replace("{scheme:lower}", s.lower()).replace("{op}", o)
+                assert hasattr(lib, sym), f"{name}: {sym} not exported"
         assert f["PLATFORM"] == "HIP" and f["PROFILE"] == ("NONE" if f["OP"] == "embedding" else "ANY")
     mm = families["matmul_quantized_hip"]
     assert mm["OP"] == "matmul" and mm["MATMUL_LAYOUT"] == "NT" and mm["WEIGHT_LAYOUT"] == "SEPARATE"

@@ -520,3 +520,121 @@ def test_embedding_gather_errors(ctx):
     assert call(token_ids=tmp["no_ids"], o=tmp["no_out"]) == ta.SUCCESS
     for t in [tt, ids, out] + list(tmp.values()):
         ctx.host_freed(t)
+
+
+# ---------------------------------------------------------------- ops between the linears
+def test_impl_and_program_float_ops(ctx, oracle):
+    """hip_rmsnorm_impl / hip_rmsnorm_gemma_impl (rank 3, residual), hip_swiglu_f32 / hip_geglu_f32 (contiguous and
+    row-strided), hip_add_f32, their queries and bytecode ops, against the oracle."""
+    x = gaussian(980, (2, 5, 512))
+    r = gaussian(981, (2, 5, 512))
+    w = gaussian(982, (512,), 0.5) + np.float32(1.0)
+    xt, rt, wt = ta.HostTensor.dense(x), ta.HostTensor.dense(r), ta.HostTensor.dense(w)
+    ot = ta.HostTensor.empty((2, 5, 512), ta.DTYPE_F32)
+    for fn, off, op, bc in ((ctx.lib.hip_rmsnorm_impl, 0.0, ta.OP_RMS_NORM, ta.BC_OP_RMS_NORM_F32),
+                            (ctx.lib.hip_rmsnorm_gemma_impl, 1.0, ta.OP_RMS_NORM_GEMMA, ta.BC_OP_RMS_NORM_GEMMA_F32)):
+        desc = ta.RmsNormDesc(xt.ptr, rt.ptr, wt.ptr, ot.ptr, 1e-6)
+        assert fn(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
+        ref = oracle.rms_norm(x.reshape(10, 512), w, residual=r.reshape(10, 512), eps=1e-6, weight_offset=off)
+        assert np.allclose(ctx.to_host(ot).reshape(10, 512), ref, rtol=1e-5, atol=1e-8)
+        sel = ctx.query(ctx.float_op_signature(op))
+        assert sel.supported and sel.op_index == bc
+        assert not ctx.query(ctx.float_op_signature(op, ta.DTYPE_F16)).supported
+        prog = ta.Program()
+        prog.rms_norm(bc, xt, wt, None, ot, 1e-5)
+        assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+        ref = oracle.rms_norm(x.reshape(10, 512), w, eps=1e-5, weight_offset=off)
+        assert np.allclose(ctx.to_host(ot).reshape(10, 512), ref, rtol=1e-5, atol=1e-8)
+    bad = ta.HostTensor.dense(gaussian(983, (500,)))
+    desc = ta.RmsNormDesc(xt.ptr, None, bad.ptr, ot.ptr, 1e-6)
+    assert ctx.lib.hip_rmsnorm_impl(ctx.device_ctx, C.byref(desc)) == ta.DIMENSION_MISMATCH
+
+    g, u = gaussian(984, (6, 300), 2.0), gaussian(985, (6, 300))
+    gt, ut, yt = ta.HostTensor.dense(g), ta.HostTensor.dense(u), ta.HostTensor.empty((6, 300), ta.DTYPE_F32)
+    for fn, geglu, op, bc in ((ctx.lib.hip_swiglu_f32, False, ta.OP_SWIGLU, ta.BC_OP_SWIGLU_F32),
+                              (ctx.lib.hip_geglu_f32, True, ta.OP_GEGLU, ta.BC_OP_GEGLU_F32)):
+        assert fn(ctx.device_ctx, gt.ptr, ut.ptr, yt.ptr) == ta.SUCCESS, ctx.last_error()
+        assert np.allclose(ctx.to_host(yt), oracle.glu(g, u, geglu=geglu), rtol=1e-5, atol=1e-7)
+        sel = ctx.query(ctx.float_op_signature(op))
+        assert sel.supported and sel.op_index == bc
+        prog = ta.Program()
+        prog.binary(bc, ut, gt, yt)  # operands swapped: act(up) * gate
+        assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+        assert np.allclose(ctx.to_host(yt), oracle.glu(u, g, geglu=geglu), rtol=1e-5, atol=1e-7)
+    # row-strided: gate and up are the two halves of one [rows, 2 * cols] projection output
+    both = gaussian(986, (4, 512), 2.0)
+    whole = ta.HostTensor.dense(both)
+    halves = []
+    for h in range(2):
+        view = ta.HostTensor.dense(both)  # a fresh descriptor over the same memory, then narrowed to one half
+        view.array = whole.array
+        view.t.data = whole.t.data + h * 256 * 4
+        view.t.shape.shape[1] = 256
+        view.t.shape.strides[0] = 512
+        halves.append(view)
+    yo = ta.HostTensor.empty((4, 256), ta.DTYPE_F32)
+    assert ctx.lib.hip_swiglu_f32(ctx.device_ctx, halves[0].ptr, halves[1].ptr, yo.ptr) == ta.SUCCESS, ctx.last_error()
+    assert np.allclose(ctx.to_host(yo), oracle.glu(both[:, :256], both[:, 256:]), rtol=1e-5, atol=1e-7)
+
+    a, b_ = gaussian(987, (3, 7, 11)), gaussian(988, (3, 7, 11))
+    at, bt, st_ = ta.HostTensor.dense(a), ta.HostTensor.dense(b_), ta.HostTensor.empty((3, 7, 11), ta.DTYPE_F32)
+    assert ctx.lib.hip_add_f32(ctx.device_ctx, at.ptr, bt.ptr, st_.ptr) == ta.SUCCESS
+    assert np.array_equal(ctx.to_host(st_), a + b_)
+    sel = ctx.query(ctx.float_op_signature(ta.OP_ADD))
+    assert sel.supported and sel.op_index == ta.BC_OP_ADD_F32
+    for t in (xt, rt, wt, ot, bad, gt, ut, yt, whole, yo, at, bt, st_):
+        ctx.host_freed(t)
+
+
+def test_program_norm_feeds_linears_without_quantization_launches(ctx, oracle):
+    """A decoder layer's feed-forward half at 16 tokens as one bytecode program: rms_norm -> gate, up (Q4_K) -> swiglu
+    -> down (Q6_K) -> residual add. The normalization leaves its rows packed, gate and up both find them (no packing
+    launch of their own); the gated product is packed once by the down projection. Results against the oracle's
+    chain (bound against the output scale, as for every re-quantizing chain)."""
+    from tests.util import assert_moe_parity
+
+    T, H, F = 16, 1024, 2816
+    x = gaussian(990, (T, H))
+    w_norm = gaussian(991, (H,), 0.3) + np.float32(1.0)
+    gate = oracle.quantize(KIND_Q4_K, gaussian(992, (F, H), 0.03))
+    up = oracle.quantize(KIND_Q4_K, gaussian(993, (F, H), 0.03))
+    down = oracle.quantize(KIND_Q6_K, gaussian(994, (H, F), 0.03))
+    xt, wn = ta.HostTensor.dense(x), ta.HostTensor.dense(w_norm)
+    gw, uw = ta.HostTensor.quantized(gate, (F, H), KIND_Q4_K), ta.HostTensor.quantized(up, (F, H), KIND_Q4_K)
+    dw = ta.HostTensor.quantized(down, (H, F), KIND_Q6_K)
+    h, g, u, a = (ta.HostTensor.empty(s, ta.DTYPE_F32) for s in ((T, H), (T, F), (T, F), (T, F)))
+    d, y = ta.HostTensor.empty((T, H), ta.DTYPE_F32), ta.HostTensor.empty((T, H), ta.DTYPE_F32)
+    mm = {KIND_Q4_K: 3, KIND_Q6_K: 4}
+    prog = ta.Program()
+    prog.rms_norm(ta.BC_OP_RMS_NORM_F32, xt, wn, None, h, 1e-5)
+    prog.matmul(mm[KIND_Q4_K], h, gw, g)
+    prog.matmul(mm[KIND_Q4_K], h, uw, u)
+    prog.binary(ta.BC_OP_SWIGLU_F32, g, u, a)
+    prog.matmul(mm[KIND_Q6_K], a, dw, d)
+    prog.binary(ta.BC_OP_ADD_F32, xt, d, y)
+    ref_h = oracle.rms_norm(x, w_norm, eps=1e-5)
+    ref_a = oracle.glu(oracle.matmul(KIND_Q4_K, gate, ref_h, F, threads=8), oracle.matmul(KIND_Q4_K, up, ref_h, F, threads=8))
+    ref_d = oracle.matmul(KIND_Q6_K, down, ref_a, H, threads=8)
+    for run in range(2):
+        before = ctx.residency()
+        packs0, hits0 = before.activation_packs, before.activation_pack_hits
+        assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+        after = ctx.residency()
+        # two packed copies per run (the normalization's output, the gated product), three linears that found one
+        assert after.activation_packs - packs0 == 2, run
+        assert after.activation_pack_hits - hits0 == 2, run   # gate and up; down packed its own input
+        assert_moe_parity(ctx.to_host(d), ref_d, what=f"ffn chain run {run}")
+        assert np.allclose(ctx.to_host(y), x + ctx.to_host(d), rtol=0, atol=0)
+        assert np.allclose(ctx.to_host(h), ref_h, rtol=1e-5, atol=1e-8)
+    # writing the normalized tensor from the host ends its packed copy: the next linear packs the new contents
+    h.array[:] = gaussian(995, (T, H))
+    ctx.ops.memcpy_to_device(ctx.device_ctx, h.t.data, h.t.data, h.array.nbytes)
+    one = ta.Program()
+    one.matmul(mm[KIND_Q4_K], h, gw, g)
+    packs0 = ctx.residency().activation_packs
+    assert ctx.execute(one) == ta.SUCCESS, ctx.last_error()
+    assert ctx.residency().activation_packs - packs0 == 1
+    from tests.util import assert_matmul_parity
+    assert_matmul_parity(ctx.to_host(g), oracle.matmul(KIND_Q4_K, gate, h.array, F, threads=8), what="after host write")
+    for t in (xt, wn, gw, uw, dw, h, g, u, a, d, y):
+        ctx.host_freed(t)

@@ -756,6 +756,60 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
     }
 
     // epilogue: lane (j, kh) holds weight row m = wrow0 + j for tokens 32a + 8(r/4) + 4kh + r%4
+    if (KG > 1 && p.splits == 1 && wrow0 + G_WROWS_WAVE <= p.M && (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0) {
+        // Stores straight from this layout are 4 bytes per lane, 32 of them per lane (measured: 280 clocks per
+        // store instruction at issue, 9000 clocks for the tile). The wavefront's 32 rows x TOK tokens go through its
+        // own 8 KiB of LDS (the region its K partner just used for the reduction, read only by this wavefront) and
+        // leave as 16 bytes per lane: every instruction writes 8 tokens x 128 contiguous bytes.
+        static_assert(G_WROWS_WAVE == 32, "the transposed epilogue assumes 32 weight rows per wavefront");
+        float *tile = (float *)lds + (size_t)rgp * TA * 16 * 64;  // [token][32 rows]
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // the reduction's reads of this region are done
+#pragma unroll
+        for (int a = 0; a < TA; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * 32 + j] = total[a][r];
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        const int q4 = lane & 7, tl = lane >> 3;  // rows 4 q4 .. 4 q4 + 3 of token tl (+ 8 per step)
+        const size_t m4 = wrow0 + 4 * (size_t)q4;
+        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const bool has_bias = p.bias != nullptr;
+        if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < S::TOK / 8; ++it) {
+            const int t = it * 8 + tl;
+            const size_t n = tt * S::TOK + (size_t)t;
+            const float4 v = *(const float4 *)(tile + t * 32 + 4 * q4);
+            if (n >= p.N) {
+                continue;
+            }
+            float e4[4] = {v.x, v.y, v.z, v.w};
+            if (!p.out_is_f16) {
+                float4 o;  // bias4 is zero without a bias: the same addition as the per-element path
+                o.x = e4[0] + bias4[0], o.y = e4[1] + bias4[1], o.z = e4[2] + bias4[2], o.w = e4[3] + bias4[3];
+                *(float4 *)((float *)p.out + n * p.M + m4) = o;
+            } else {
+                uint16_t h[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
+                    if (has_bias) {
+                        h[e] = f2h(h2f(h[e]) + bias4[e]);
+                    }
+                }
+                *(uint2 *)((uint16_t *)p.out + n * p.M + m4) =
+                    make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            }
+        }
+        return;
+    }
     const size_t m = wrow0 + j;
     if (m >= p.M) {
         return;

@@ -542,10 +542,19 @@ static bool rows_plan(const marmot_hip_device *dev, size_t N, size_t K, size_t M
         return false;
     }
     pl.nslots = nslots;
-    // Segments a loader may have in flight: vmcnt counts 6 bits. Landed segments are published by polling the counter,
-    // so a deep window costs no latency.
+    // Segments a loader may have in flight: at most what the 6-bit load counter can count (landed segments are
+    // published by polling the counter) ...
     const uint32_t ipt = pl.slot_stride >> 10;
     pl.lag = 60u / ipt < 1u ? 1u : 60u / ipt;
+    // ... and about 48 KB per workgroup: with everything requested at once the memory system serves all of a
+    // workgroup's segments side by side, the first ones land as late as the last, and the consumers start when the
+    // stream is nearly over (measured at 4096 x 14336: segments in flight per loader unlimited / 4 / 3 / 2:
+    // 9.45 / 9.34 / 8.80 / 9.12 us).
+    {
+        uint32_t v = (48u * 1024u) / (loaders * task_bytes);
+        v = v < 2u ? 2u : v;
+        pl.lag = v < pl.lag ? v : pl.lag;
+    }
     // Segments requested before the workgroup barrier: no slot is reused there. Measured 0 / 2 / 4: 9.8 / 9.3 / 9.6 us.
     pl.pre = 2u;
     pl.pre = pl.pre > nslots / loaders ? nslots / loaders : pl.pre;

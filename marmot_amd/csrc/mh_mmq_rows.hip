@@ -622,7 +622,15 @@ static bool mmq_rows_plan(const marmot_hip_device *dev, size_t N, size_t K, size
         }
     }
     pl.nslots = nslots;
+    // tasks a loader keeps in flight: what the 6-bit load counter can count, and about 48 KB per workgroup (beyond
+    // that the first tasks land as late as the last, see the decode matvec)
     pl.lag = 60u / pl.ipt < 1u ? 1u : 60u / pl.ipt;
+    {
+        const uint32_t task_bytes = pl.R * pl.seg_blocks * Q4_K_BYTES;
+        uint32_t v = (48u * 1024u) / (loaders * task_bytes);
+        v = v < 2u ? 2u : v;
+        pl.lag = v < pl.lag ? v : pl.lag;
+    }
     pl.pre = 2u;
     pl.pre = pl.pre > nslots / loaders ? nslots / loaders : pl.pre;
     pl.pre = pl.pre > pl.lag ? pl.lag : pl.pre;

@@ -254,7 +254,8 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
  * (src/core/helpers/rope.c:61-127, 143-200) for marmot_rope_params_t fields (include/marmot/ops_types.h:98-112);
  * scaling_type as marmot_rope_scaling_type_t (include/marmot/types.h:254-261). head_dim is resolved against M as
  * cpu_matmul_qkv_resolve_head_dim does and returned in *head_dim_out. freqs_out: host array of at least M/2 floats.
- * The YaRN ramp (a non-zero extrapolation factor with a valid original context) returns NOT_IMPLEMENTED. */
+ * Includes the YaRN ramp (a non-zero extrapolation factor with a valid original context: correction range
+ * rope.c:38-59, ramp :28-36, attention scale :95-99). */
 int marmot_hip_rope_frequencies(int scaling_type, float theta, float freq_scale, float ext_factor,
                                 float attn_factor, float beta_fast, float beta_slow, uint32_t orig_ctx_len,
                                 uint32_t head_dim, size_t M, float *freqs_out, float *attn_scale_out,

@@ -788,7 +788,7 @@ marmot_error_t hip_matmul_quantized_q6_k(const void *device_ctx, const marmot_te
  * (cf. cpu_matmul_qkv_{q4_k,q6_k,q8_0}, src/backends/cpu/ops/matmul/qkv/matmul_qkv.c:1498-1532; validation as
  * cpu_matmul_qkv_validate_desc, :1230-1300), including the rotary epilogue (rope_params applied to q and/or k with
  * FLOAT32, INT32 or INT64 positions; frequencies as marmot_rope_freq_cache_ensure, src/core/helpers/rope.c). The fused
- * layout, dense weights and the YaRN frequency ramp return MARMOT_ERROR_NOT_IMPLEMENTED. */
+ * layout and dense weights return MARMOT_ERROR_NOT_IMPLEMENTED. */
 marmot_error_t hip_matmul_qkv_q4_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q8_0(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 marmot_error_t hip_matmul_qkv_q4_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);

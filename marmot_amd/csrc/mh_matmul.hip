@@ -562,13 +562,38 @@ int marmot_hip_rope_frequencies(int scaling_type, float theta, float freq_scale,
     if (!(ext_factor != 0.0f && orig_ctx_len > 0 && theta > 0.0f && beta_fast > 0.0f && beta_slow > 0.0f)) {
         ext_factor = 0.0f;
     }
+    // YaRN: correction range (rope_yarn_corr_dims, rope.c:38-59) and attention scale (rope.c:95-99)
+    float corr_low = 0.0f, corr_high = 0.0f;
+    float attn_scale = attn_factor;
     if (ext_factor != 0.0f) {
-        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "RoPE: the YaRN frequency ramp is not provided");
+        const float denom = 2.0f * logf(theta);
+        const float pi = 3.14159265358979323846f;
+        float low_raw = 0.0f, high_raw = 0.0f;
+        if (denom != 0.0f) {
+            low_raw = (float)(int)hd * logf((float)(int)orig_ctx_len / (beta_fast * 2.0f * pi)) / denom;
+            high_raw = (float)(int)hd * logf((float)(int)orig_ctx_len / (beta_slow * 2.0f * pi)) / denom;
+        }
+        corr_low = fmaxf(0.0f, floorf(low_raw));
+        corr_high = fminf((float)((int)hd - 1), ceilf(high_raw));
+        const float inv_scale = 1.0f / freq_scale;
+        attn_scale *= 1.0f + 0.1f * logf(inv_scale);
     }
-    *attn_scale_out = attn_factor;
+    *attn_scale_out = attn_scale;
     *head_dim_out = (uint32_t)hd;
     for (size_t i = 0; i < hd / 2; ++i) {  // compute_rope_frequencies (rope.c:112-127), host powf like the reference
-        freqs_out[i] = powf(theta, -((float)(2 * i) / (float)hd)) * freq_scale;
+        const float freq = powf(theta, -((float)(2 * i) / (float)hd));
+        float scale = freq_scale;
+        if (ext_factor != 0.0f) {  // rope_yarn_ramp (rope.c:28-36)
+            float d = corr_high - corr_low;
+            if (d < 0.001f) {
+                d = 0.001f;
+            }
+            const float y = ((float)i - corr_low) / d;
+            const float ramp = 1.0f - fminf(1.0f, fmaxf(0.0f, y));
+            const float mix = ramp * ext_factor;
+            scale = freq_scale + mix * (1.0f - freq_scale);
+        }
+        freqs_out[i] = freq * scale;
     }
     return MARMOT_HIP_SUCCESS;
 }

@@ -2371,14 +2371,39 @@ int mo_rope_frequencies(const mo_rope_params *p, size_t head_dim, float *freqs_o
           p->beta_slow > 0.0f)) {
         ext_factor = 0.0f; /* rope.c:85-93: without the correction range YaRN degenerates to linear scaling */
     }
-    if (ext_factor != 0.0f) {
-        return MO_ERR_NOT_IMPLEMENTED; /* YaRN ramp: not restated */
+    float corr_low = 0.0f, corr_high = 0.0f;
+    if (ext_factor != 0.0f) { /* rope_yarn_corr_dims (rope.c:46-59) with rope_yarn_corr_factor (:38-44) */
+        const float denom = 2.0f * logf(p->theta);
+        const float pi = 3.14159265358979323846f;
+        float low_raw = 0.0f, high_raw = 0.0f;
+        if (denom != 0.0f) {
+            low_raw = (float)(int)head_dim * logf((float)(int)p->orig_ctx_len / (p->beta_fast * 2.0f * pi)) / denom;
+            high_raw = (float)(int)head_dim * logf((float)(int)p->orig_ctx_len / (p->beta_slow * 2.0f * pi)) / denom;
+        }
+        corr_low = fmaxf(0.0f, floorf(low_raw));
+        corr_high = fminf((float)((int)head_dim - 1), ceilf(high_raw));
     }
-    *attn_scale_out = attn_factor; /* rope.c:95-99 with ext_factor == 0 */
+    float attn_scale = attn_factor; /* rope.c:95-99 */
+    if (ext_factor != 0.0f) {
+        const float inv_scale = 1.0f / freq_scale;
+        attn_scale *= 1.0f + 0.1f * logf(inv_scale);
+    }
+    *attn_scale_out = attn_scale;
     const size_t half = head_dim / 2;
-    for (size_t i = 0; i < half; ++i) { /* rope.c:114-126 */
+    for (size_t i = 0; i < half; ++i) { /* rope.c:112-127 */
         const float freq = powf(p->theta, -((float)(2 * i) / (float)head_dim));
-        freqs_out[i] = freq * freq_scale;
+        float scale = freq_scale;
+        if (ext_factor != 0.0f) { /* rope_yarn_ramp (rope.c:28-36) */
+            float d = corr_high - corr_low;
+            if (d < 0.001f) {
+                d = 0.001f;
+            }
+            const float y = ((float)i - corr_low) / d;
+            const float ramp = 1.0f - fminf(1.0f, fmaxf(0.0f, y));
+            const float mix = ramp * ext_factor;
+            scale = freq_scale + mix * (1.0f - freq_scale);
+        }
+        freqs_out[i] = freq * scale;
     }
     return MO_OK;
 }

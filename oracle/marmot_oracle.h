@@ -142,8 +142,8 @@ size_t mo_rope_resolve_head_dim(size_t dim, uint32_t head_dim);
 
 /*
  * marmot_rope_freq_cache_ensure without the cache (src/core/helpers/rope.c:61-127, 143-200): head_dim/2 angular
- * frequencies theta^(-2i/head_dim) * scale and the attention scale. The YaRN ramp (ext_factor != 0 after
- * rope_scaling_prepare) is not restated: returns MO_ERR_NOT_IMPLEMENTED.
+ * frequencies theta^(-2i/head_dim) * scale and the attention scale, including the YaRN ramp (ext_factor != 0 after
+ * rope_scaling_prepare: correction range rope.c:38-59, ramp :28-36, attention scale :95-99).
  */
 int mo_rope_frequencies(const mo_rope_params *p, size_t head_dim, float *freqs_out, float *attn_scale_out);
 

@@ -388,8 +388,8 @@ def test_impl_qkv_errors(ctx, oracle):
     rope.positions = pos2.ptr
     rope.scaling_type, rope.ext_factor, rope.freq_scale, rope.orig_ctx_len = 2, 1.0, 0.5, 4096
     rope.beta_fast, rope.beta_slow = 32.0, 1.0
-    d, keep = build(rope=rope)  # the YaRN ramp is declined
-    assert fn(ctx.device_ctx, C.byref(d)) == ta.NOT_IMPLEMENTED and "YaRN" in ctx.last_error()[1]
+    d, keep = build(rope=rope)  # the YaRN ramp is computed like any other scaling
+    assert fn(ctx.device_ctx, C.byref(d)) == ta.SUCCESS, ctx.last_error()
     rope.apply_to_q = False  # parameters present but applied to neither q nor k: plain projection (matmul_qkv.c:812-814)
     rope.positions = None
     d, keep = build(rope=rope)

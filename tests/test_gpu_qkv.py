@@ -163,10 +163,16 @@ def test_qkv_rope_errors(hip, oracle):
     ws = _weights(oracle, kind, M, K, 740)
     x = gaussian(741, (2, K))
     pos = np.array([1, 2], np.int32)
-    with pytest.raises(capi.MarmotHipError) as e:  # the YaRN ramp is declined, not approximated
-        hip.linear_qkv(x, *ws, kind, M, positions=pos,
-                       rope=dict(scaling_type=2, ext_factor=1.0, freq_scale=0.5, orig_ctx_len=4096))
-    assert e.value.code == -8
+    # the YaRN ramp: frequencies and attention scale are the oracle's bits (host code, the reference's formulas)
+    from oracle.pyoracle import RopeParams as RP
+    yarn = dict(scaling_type=2, ext_factor=1.0, freq_scale=0.5, orig_ctx_len=4096, beta_fast=32.0, beta_slow=1.0)
+    f_hip, a_hip, hd = hip.rope_frequencies(M, head_dim=64, theta=10000.0, **yarn)
+    f_ref, a_ref = oracle.rope_frequencies(RP.default(head_dim=64, theta=10000.0, **yarn), 64)
+    assert hd == 64 and a_hip == a_ref and np.array_equal(f_hip, f_ref) and a_ref > 1.0
+    q, k_, _ = hip.linear_qkv(x, *ws, kind, M, positions=pos, rope=dict(theta=10000.0, head_dim=64, **yarn))
+    rq, rk, _ = oracle.matmul_qkv(kind, *ws, x, M, positions=pos, rope=RP.default(theta=10000.0, head_dim=64, **yarn))
+    assert_matmul_parity(q, rq, what="yarn q")
+    assert_matmul_parity(k_, rk, what="yarn k")
     # YaRN parameters without an original context length degenerate to linear scaling (rope.c:85-93)
     q, _, _ = hip.linear_qkv(x, *ws, kind, M, positions=pos, rope=dict(scaling_type=2, ext_factor=1.0, freq_scale=0.5))
     from oracle.pyoracle import RopeParams

@@ -130,9 +130,30 @@ def test_rope_frequencies_and_rotation_closed_form(oracle):
         f3, a3 = oracle.rope_frequencies(
             RopeParams.default(theta=theta, freq_scale=0.25, attn_factor=1.5, scaling_type=ROPE_SCALING_LINEAR), head_dim)
         assert np.array_equal(f3, f * np.float32(0.25)) and a3 == 1.5
-    with pytest.raises(RuntimeError):  # the YaRN ramp is not restated
-        oracle.rope_frequencies(RopeParams.default(scaling_type=ROPE_SCALING_YARN, ext_factor=1.0, freq_scale=0.5,
-                                                   orig_ctx_len=4096), 64)
+    # YaRN (rope.c:28-59, 95-126). Known correction range for 128 dims, 4096 original context, base 10000,
+    # beta_fast 32, beta_slow 1: pairs 0..20 keep their frequency (ramp 1 up to floor(20.9)), pairs from 46 = ceil(45.04)
+    # on are interpolated by freq_scale (ramp 0), linear in between; attention scale attn_factor * (1 + 0.1 ln(1/s)).
+    yarn = RopeParams.default(theta=10000.0, scaling_type=ROPE_SCALING_YARN, ext_factor=1.0, freq_scale=0.25,
+                              attn_factor=1.0, orig_ctx_len=4096, beta_fast=32.0, beta_slow=1.0)
+    f, a = oracle.rope_frequencies(yarn, 128)
+    base = (10000.0 ** (-(2.0 * np.arange(64)) / 128)).astype(np.float64)
+    d, lo, hi = 128, 4096 / (32 * 2 * np.pi), 4096 / (1 * 2 * np.pi)
+    low = max(0.0, np.floor(d * np.log(lo) / (2 * np.log(10000.0))))
+    high = min(d - 1.0, np.ceil(d * np.log(hi) / (2 * np.log(10000.0))))
+    assert (low, high) == (20.0, 46.0)
+    ramp = 1.0 - np.clip((np.arange(64) - low) / (high - low), 0.0, 1.0)
+    want = base * (0.25 + ramp * (1.0 - 0.25))
+    assert np.allclose(f, want, rtol=3e-6, atol=0)
+    assert np.allclose(f[:21], base[:21], rtol=3e-6) and np.allclose(f[46:], base[46:] * 0.25, rtol=3e-6)
+    assert abs(a - (1.0 + 0.1 * np.log(4.0))) < 1e-6
+    # half the extrapolation factor mixes half-way; no original context length degenerates to linear scaling
+    half = RopeParams.default(theta=10000.0, scaling_type=ROPE_SCALING_YARN, ext_factor=0.5, freq_scale=0.25,
+                              orig_ctx_len=4096, beta_fast=32.0, beta_slow=1.0)
+    f_half, _ = oracle.rope_frequencies(half, 128)
+    assert np.allclose(f_half, base * (0.25 + 0.5 * ramp * 0.75), rtol=3e-6, atol=0)
+    lin = RopeParams.default(theta=10000.0, scaling_type=ROPE_SCALING_YARN, ext_factor=1.0, freq_scale=0.25)
+    f_lin, a_lin = oracle.rope_frequencies(lin, 128)
+    assert np.allclose(f_lin, base * 0.25, rtol=3e-6, atol=0) and a_lin == 1.0
     assert oracle.L.mo_rope_resolve_head_dim(512, 128) == 128
     for bad in (0, 1024, 96, 7):  # absent, larger than the row, not a divisor, odd
         assert oracle.L.mo_rope_resolve_head_dim(512, bad) == 512

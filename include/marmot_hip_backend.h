@@ -661,8 +661,7 @@ const marmot_device_ops_t *marmot_get_hip_ops(void);
  * Matching rules follow the generated queries (scripts/codegen/templates/backend_query.c.j2:60-104): profile is
  * a wildcard; matmul needs layout NT, input F32 or F16, output F32 (or F16 with F16 input), accumulation F32,
  * weight layout SEPARATE, contiguous strides, epilogue flags within {BIAS}, no variant flags, and a weight
- * scheme of Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K (Q2_K, Q3_K, Q5_K and Q6_K with F16 input
- * are declined: the caller falls back). */
+ * scheme of Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K. */
 marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *sig, const marmot_device_caps_t *caps);
 marmot_device_caps_t marmot_hip_detect_default_caps(void);
 bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_backend_preferences_t *prefs_out);

@@ -1968,15 +1968,6 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         if ((sig->epilogue_flags & ~(uint32_t)MARMOT_EPILOGUE_BIAS) != 0 || sig->variant_flags != 0) {
             return unsupported("HIP quantized matmul fuses only the bias epilogue");
         }
-        if (kind == MARMOT_HIP_KIND_Q6_K && in16) {
-            return unsupported("HIP Q6_K matmul takes FLOAT32 activations");
-        }
-        if (kind == MARMOT_HIP_KIND_Q5_K && in16) {
-            return unsupported("HIP Q5_K matmul takes FLOAT32 activations");
-        }
-        if ((kind == MARMOT_HIP_KIND_Q2_K || kind == MARMOT_HIP_KIND_Q3_K) && in16) {
-            return unsupported("HIP Q2_K / Q3_K matmul takes FLOAT32 activations");
-        }
         const size_t N = sig->dims.matmul.N, K = sig->dims.matmul.K, M = sig->dims.matmul.M;
         const double bytes =
             (double)M * (double)marmot_hip_row_bytes(kind, K) + (double)N * K * (in32 ? 4 : 2) + (double)N * M * 4;

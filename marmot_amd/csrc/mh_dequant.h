@@ -185,6 +185,77 @@ __device__ __forceinline__ float dequant_value(const uint8_t *blk, int v) {
     }
 }
 
+// ---- weights as the reference's fp16 direct dots see them
+// cpu_vec_dot_{q2_k,q3_k,q5_k,q6_k}_f16 (vec_dot_impl.h:866-971, 1025-1128) decode their blocks with index patterns
+// of their own, which differ from the dequantizers above; the reference's matmul golden for fp16 activations records
+// what they compute. A backend that replaces that path has to return the same numbers, so the direct fp16 route
+// mirrors the functions as written. Value v (0..255) of a block:
+//   Q2_K: one scale / min pair per 128 values (scales[v / 128]), 2-bit values in sequential order (bits 2 (v % 4) of
+//         qs[v / 4]);
+__device__ __forceinline__ float direct_f16_weight_q2_k(const uint8_t *blk, int v) {
+    const BlockQ2_K *b = (const BlockQ2_K *)blk;
+    const uint8_t sc = b->scales[v >> 7];
+    const float dl = h2f(b->d) * (float)(sc & 0xF);
+    const float ml = h2f(b->dmin) * (float)(sc >> 4);
+    const int q = (b->qs[v >> 2] >> ((v & 3) * 2)) & 3;
+    return dl * (float)q - ml;
+}
+//   Q3_K: the high-bit mask advances once per 128 values instead of once per 32;
+__device__ __forceinline__ float direct_f16_weight_q3_k(const uint8_t *blk, int v) {
+    const BlockQ3_K *b = (const BlockQ3_K *)blk;
+    const int c = v >> 7, j = (v >> 5) & 3, li = v & 31;  // li = l + 16 * half
+    const float dl = h2f(b->d) * (float)q3k_group_scale(b->scales, v >> 4);
+    const int q2 = (b->qs[32 * c + li] >> (2 * j)) & 3;
+    const int q = q2 - (((b->hmask[li] >> c) & 1) ? 0 : 4);
+    return dl * (float)q;
+}
+//   Q5_K: the fifth bit is bit 0 of byte 8 g + l (+ 32 for the high nibbles) counted from the start of qh, which for
+//         most values is a byte of another element or of qs;
+__device__ __forceinline__ float direct_f16_weight_q5_k(const uint8_t *blk, int v) {
+    const BlockQ5_K *b = (const BlockQ5_K *)blk;
+    const int j = v >> 5, l = v & 31, g = j >> 1;
+    uint8_t sc, m;
+    const uint8_t *s = b->scales;
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (uint8_t)((s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4));
+        m = (uint8_t)((s[j + 4] >> 4) | ((s[j] >> 6) << 4));
+    }
+    const float d1 = h2f(b->d) * (float)sc;
+    const float m1 = h2f(b->dmin) * (float)m;
+    const uint8_t byte = b->qs[32 * g + l];
+    const int h = b->qh[8 * g + l + ((j & 1) ? 32 : 0)] & 1;  // runs past qh[32] into qs: still inside the block
+    const int q = ((j & 1) ? (byte >> 4) : (byte & 0xF)) | (h << 4);
+    return d1 * (float)q - m1;
+}
+//   Q6_K: one scale per 128 values (scales[v / 128]), nibbles and high pairs in sequential order.
+__device__ __forceinline__ float direct_f16_weight_q6_k(const uint8_t *blk, int v) {
+    const BlockQ6_K *b = (const BlockQ6_K *)blk;
+    const float scale = h2f(b->d) * (float)b->scales[v >> 7];
+    const int nib = (v & 1) ? (b->ql[v >> 1] >> 4) : (b->ql[v >> 1] & 0xF);
+    const int hi2 = (b->qh[v >> 2] >> ((v & 3) * 2)) & 3;
+    const int q = (int)(int8_t)(nib | (hi2 << 4)) - 32;
+    return scale * (float)q;
+}
+
+// the weight the reference's fp16 direct dot multiplies with activation v of a block
+template <int KIND>
+__device__ __forceinline__ float direct_f16_weight(const uint8_t *blk, int v) {
+    if constexpr (KIND == MARMOT_HIP_KIND_Q2_K) {
+        return direct_f16_weight_q2_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q3_K) {
+        return direct_f16_weight_q3_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_K) {
+        return direct_f16_weight_q5_k(blk, v);
+    } else if constexpr (KIND == MARMOT_HIP_KIND_Q6_K) {
+        return direct_f16_weight_q6_k(blk, v);
+    } else {
+        return dequant_value<KIND>(blk, v);
+    }
+}
+
 template <int KIND>
 struct KindTraits {
     static constexpr int BV = (KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q8_0 ||

@@ -22,8 +22,8 @@ int static_scratch_init(marmot_hip_device *dev) {
 
 // ------------------------------------------------------------------------------------------------
 // Direct route: out[n, m] = sum_k dequant(W[m, k]) * (float)x_f16[n, k], fp32 accumulate.
-// Counterpart of cpu_vec_dot_{q4_0,q4_1,q5_0,q5_1,q8_0,q4_k}_f16 (vec_dot_impl.h:220-286, 351-450, 973-1023): the same
-// per-value fp32 weights, summed in a different order. One wavefront per weight row; a lane visits 8
+// Counterpart of cpu_vec_dot_{scheme}_f16 (vec_dot_impl.h:220-286, 351-450, 866-1128): the same per-value fp32 weights
+// (for Q2_K, Q3_K, Q5_K and Q6_K the ones those functions decode, see direct_f16_weight), summed in a different order. One wavefront per weight row; a lane visits 8
 // consecutive k at a time (one 16-byte load of fp16 activations per column).
 // ------------------------------------------------------------------------------------------------
 struct DirectParams {
@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void k_matvec_direct_f16(const DirectParams p)
         float wv[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            wv[i] = (k0 + i < p.K) ? dequant_value<KIND>(blk, v0 + i) : 0.0f;
+            wv[i] = (k0 + i < p.K) ? direct_f16_weight<KIND>(blk, v0 + i) : 0.0f;
         }
 #pragma unroll
         for (int n = 0; n < NC; ++n) {
@@ -166,10 +166,19 @@ int launch_matvec_f16(marmot_hip_device *dev, int kind, const void *d_w, const v
     case MARMOT_HIP_KIND_Q5_1:
         set_route("matvec_q5_1_f16_direct");
         return launch_direct_kind<MARMOT_HIP_KIND_Q5_1>(dev, p, N);
+    case MARMOT_HIP_KIND_Q2_K:
+        set_route("matvec_q2_k_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q2_K>(dev, p, N);
+    case MARMOT_HIP_KIND_Q3_K:
+        set_route("matvec_q3_k_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q3_K>(dev, p, N);
+    case MARMOT_HIP_KIND_Q5_K:
+        set_route("matvec_q5_k_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q5_K>(dev, p, N);
+    case MARMOT_HIP_KIND_Q6_K:
+        set_route("matvec_q6_k_f16_direct");
+        return launch_direct_kind<MARMOT_HIP_KIND_Q6_K>(dev, p, N);
     default:
-        // Q2_K, Q3_K, Q5_K and Q6_K: the reference's fp16 direct dots (vec_dot_impl.h:866-971, 1025-1128) decode blocks with
-        // index patterns that disagree with its own dequantizers; this backend declines the combination so that the
-        // caller falls back (NOT_IMPLEMENTED is the reference's fallback signal, dispatch_execute.c:214-233).
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED,
                          "quantized matmul: fp16 activations without packing are not offered for quant kind %d", kind);
     }

@@ -157,17 +157,15 @@ def test_query_kernel_matmul_rules(lib):
     assert _query(lib, _sig(inp=ta.DTYPE_F16, out=ta.DTYPE_F32)).supported
     assert _query(lib, _sig(inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).supported
     assert not _query(lib, _sig(inp=ta.DTYPE_F32, out=ta.DTYPE_F16)).supported
-    # Q6_K with fp16 activations is declined (caller falls back)
-    sel = _query(lib, _sig(kind=ta.KIND_Q6_K, inp=ta.DTYPE_F16))
-    assert not sel.supported and sel.op_index == 0xFFFF and b"Q6_K" in sel.fallback_reason
-    sel = _query(lib, _sig(kind=ta.KIND_Q5_K, inp=ta.DTYPE_F16))
-    assert not sel.supported and b"Q5_K" in sel.fallback_reason
+    # every weight scheme takes fp16 activations (the K-quants as the reference's fp16 direct dots compute them)
+    for kind in (ta.KIND_Q2_K, ta.KIND_Q3_K, ta.KIND_Q5_K, ta.KIND_Q6_K):
+        assert _query(lib, _sig(kind=kind, inp=ta.DTYPE_F16)).supported
+    sel = _query(lib, _sig(kind=ta.KIND_Q8_K))
+    assert not sel.supported and sel.op_index == 0xFFFF and sel.fallback_reason
     # unsupported scheme, layout, weight layout, stride mode, epilogue, variant
     assert not _query(lib, _sig(kind=ta.KIND_Q8_K)).supported
     s = _sig(); s.qscheme_id = 13  # beyond the enumeration
     assert not _query(lib, s).supported
-    for kind in (ta.KIND_Q2_K, ta.KIND_Q3_K):
-        assert not _query(lib, _sig(kind=kind, inp=ta.DTYPE_F16)).supported
     s = _sig(); s.matmul_layout = 1
     assert not _query(lib, s).supported
     s = _sig(); s.weight_layout = 2
@@ -375,7 +373,7 @@ def test_kernel_def_files_name_exported_impls(lib):
             fields = dict(re.findall(r"^\s*([A-Z_]+(?:\(\w+\))?):\s*(.+?),?\s*$", body, re.M))
             families[name] = fields
     qkv = {f"{op}_quantized_hip_{dt}" for op in ("qkv_shared_input", "qkv_projection") for dt in ("f16", "f32")}
-    assert set(families) == {"matmul_quantized_hip", "matmul_quantized_hip_f32", "topk_hip",
+    assert set(families) == {"matmul_quantized_hip", "topk_hip",
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
                              "embedding_quantized_hip", "rms_norm_hip", "rms_norm_gemma_hip", "glu_hip",
                              "add_hip"} | qkv
@@ -394,5 +392,5 @@ def test_kernel_def_files_name_exported_impls(lib):
     mm = families["matmul_quantized_hip"]
     assert mm["OP"] == "matmul" and mm["MATMUL_LAYOUT"] == "NT" and mm["WEIGHT_LAYOUT"] == "SEPARATE"
     assert mm["EPILOGUE"] == "[BIAS]" and mm["ACCUM_DTYPE"] == "FLOAT32" and mm["STRIDE_MODE"] == "CONTIGUOUS"
-    assert families["matmul_quantized_hip_f32"]["INPUT_DTYPE"] == "FLOAT32"
-    assert families["matmul_quantized_hip_f32"]["AXIS(scheme)"] == "[Q2_K, Q3_K, Q5_K, Q6_K]"
+    assert mm["AXIS(scheme)"] == "[Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K]"
+    assert mm["INPUT_DTYPE"] == "[FLOAT16, FLOAT32]"

@@ -74,14 +74,17 @@ def test_impl_matmul_fp16_and_errors(ctx, oracle):
     assert st == ta.UNSUPPORTED_DTYPE and "FLOAT32 input or FLOAT16" in ctx.last_error()[1]
     st, *_ = _linear(ctx, KIND_Q4_K, wq, M, K, gaussian(733, (N, K + 256)))
     assert st == ta.DIMENSION_MISMATCH and "mismatch on K" in ctx.last_error()[1]
-    # a Q6_K weight handed to the Q4_K entry, and Q6_K with fp16 activations: not implemented -> caller falls back
+    # a Q6_K weight handed to the Q4_K entry: not implemented -> caller falls back
     w6 = oracle.quantize(KIND_Q6_K, gaussian(734, (M, K), 0.02))
     xt = ta.HostTensor.dense(gaussian(735, (N, K)))
     wt = ta.HostTensor.quantized(w6, (M, K), KIND_Q6_K)
     yt = ta.HostTensor.empty((N, M), ta.DTYPE_F32)
     assert ctx.lib.hip_matmul_quantized_q4_k(ctx.device_ctx, xt.ptr, wt.ptr, None, yt.ptr) == ta.NOT_IMPLEMENTED
-    st, *_ = _linear(ctx, KIND_Q6_K, w6, M, K, x16)
-    assert st == ta.NOT_IMPLEMENTED
+    # Q6_K with fp16 activations takes the reference's direct fp16 dot, like every other format
+    st, _, _, y6 = _linear(ctx, KIND_Q6_K, w6, M, K, x16)
+    assert st == ta.SUCCESS, ctx.last_error()
+    assert_matmul_parity(y6.array.astype(np.float32), oracle.matmul(KIND_Q6_K, w6, x16, M).astype(np.float32),
+                         tol=2e-3, what="Q6_K f16 direct")
     # generic (non block-quantized) weight
     wt.t.quant_kind = ta.KIND_GENERIC
     assert ctx.lib.hip_matmul_quantized_q6_k(ctx.device_ctx, xt.ptr, wt.ptr, None, yt.ptr) == ta.UNSUPPORTED_DTYPE

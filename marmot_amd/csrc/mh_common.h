@@ -214,6 +214,7 @@ struct ActScratch {
 //   MARMOT_HIP_NO_LDS_RING     loader / consumer matvec (weights through an LDS ring) -> register-streaming matvec
 //   MARMOT_HIP_NO_FUSED_QUANT  activation quantization inside the matvec -> separate quantization launch
 //   MARMOT_HIP_NO_GEMM         fp16 prefill GEMM -> fp16 matvec
+//   MARMOT_HIP_NO_GEMM_LOADERS prefill GEMM tile fed by loader wavefronts -> the tile whose wavefronts load for themselves
 //   MARMOT_HIP_MOE_NO_VALIDATE skip the read-back of the expert-id error flag (no stream synchronization per call)
 struct marmot_hip_knobs {
     bool no_mmq = false;
@@ -221,6 +222,7 @@ struct marmot_hip_knobs {
     bool no_lds_ring = false;
     bool no_fused_quant = false;
     bool no_gemm = false;
+    bool no_gemm_loaders = false;
     bool moe_no_validate = false;
 };
 

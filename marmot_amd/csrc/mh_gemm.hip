@@ -25,6 +25,7 @@
 // K is split across workgroups only when there are too few tiles to fill the chip (short prompts); those partial sums
 // meet in a small second kernel in a fixed order.
 #include "mh_common.h"
+#include "mh_rows.h"
 
 #include <stdlib.h>
 
@@ -98,6 +99,9 @@ __device__ __forceinline__ void decode_header(const uint4 &hdr, Scales &s) {
     // vector form of get_scale_min_k4 (kquant_common.h:29-37; same packing as vec_dot_impl.h:541-556)
     s.d = h2f((uint16_t)(hdr.x & 0xffffu));
     s.dmin = h2f((uint16_t)(hdr.x >> 16));
+    // Keep the two conversions as instructions of their own: folded into the 32 multiply-adds per tile that use them
+    // they become mixed-precision multiply-adds, which issue at a fraction of the plain fp32 rate.
+    asm volatile("" : "+v"(s.d), "+v"(s.dmin));
     s.sc_lo = hdr.y & 0x3f3f3f3fu;
     s.mn_lo = hdr.z & 0x3f3f3f3fu;
     s.sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
@@ -862,6 +866,410 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
     }
 }
 
+// ------------------------------------------------------------------ 64 tokens x 128 weight rows, loader wavefronts
+// The same tile as the TA = 2, KG = 2 shape above with the memory work taken away from the wavefronts that drive the
+// matrix cores. A vector-memory instruction costs the wavefront that issues it the time the compute unit's one
+// address / tag pipeline needs for everything queued in front of it (measured on this kernel's predecessor: about
+// 230 clocks per instruction when eight wavefronts issue in the same K-step, 13 instructions per wavefront and block),
+// and a wavefront that waits at the memory issue stage issues no MFMA either. Here:
+//   * wavefronts 0..3 (one per SIMD) compute: wavefront c owns weight rows 64 (c % 2) .. + 63 (two B operands) x all 64
+//     tokens (two A operands), four MFMAs per K-step, and the K-steps 8 (c / 2) .. + 7 of every block. It issues no
+//     vector-memory instruction inside the K loop. Each A operand read from LDS feeds two MFMAs and each unpacked
+//     B operand feeds two: half the LDS reads per MFMA of a 32-row wavefront tile. (Eight compute wavefronts of
+//     32 rows x 64 tokens, two per SIMD, were measured slower: the SIMD serves the older wavefront first, the two
+//     finish a block 1100 clocks apart and the barrier waits for the second.)
+//   * wavefronts 4..7 (one per SIMD) load: per block they bring the activation tile (64 tokens x 512 bytes, two
+//     contiguous token rows per instruction) and the raw weight blocks (128 rows x 144 bytes, nine lanes per block,
+//     so an instruction touches about 14 cache lines instead of 32 to 64) into one of three LDS stages with
+//     direct-to-LDS loads, two blocks ahead, and compute the sub-block sums of the tokens they loaded themselves
+//     (no synchronization between loaders) into the stage's S area before the barrier that hands the stage over.
+// One barrier per block orders everything: behind barrier i the stage of block i is complete (tile, weights, sums) and
+// the stage of block i - 1 is free for block i + 2. The barrier is an LDS-count wait plus s_barrier written by hand:
+// the usual workgroup barrier also waits for the wavefront's outstanding global loads, which here are the two blocks
+// in flight.
+constexpr int L_TOK = 64;
+constexpr int L_WROWS = 128;
+constexpr int L_COMPUTE = 4;
+constexpr int L_LOADERS = 4;
+constexpr int L_THREADS = (L_COMPUTE + L_LOADERS) * 64;
+constexpr int L_STAGE_A = L_TOK * 512;              // 32,768
+constexpr int L_STAGE_W = L_WROWS * Q4_K_BYTES;     // 18,432
+constexpr int L_STAGE_S = 2 * 64 * 16;              // sub-block sums operand of the two token sub-tiles
+constexpr int L_STAGE = L_STAGE_A + L_STAGE_W + L_STAGE_S;
+constexpr int L_STAGES = 3;
+constexpr int L_LDS_BYTES = L_STAGES * L_STAGE;     // 159,744 of 163,840
+constexpr int L_OUT_PITCH = L_WROWS + 4;            // floats per token of the output tile in LDS
+static_assert(L_TOK * L_OUT_PITCH * 4 <= L_LDS_BYTES, "the output tile reuses the stages");
+
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__global__ __launch_bounds__(L_THREADS) void k_gemm_q4k_f16_ls(const GemmParams p) {
+    warm_kernel_arguments<sizeof(GemmParams)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * L_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = (int)(b1 - b0);
+
+    floatx16 total[2][2];  // [row tile][token tile], compute wavefronts only
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                total[t][a][r] = 0.0f;
+            }
+        }
+    }
+    const int kg = (wave >> 1) & 1, rg = wave & 1;
+    const int j = lane & 31, kh = lane >> 5;
+
+    if (wave >= L_COMPUTE) {
+        // ------------------------------------------------------------------------------------------------ loaders
+        const int L = wave - L_COMPUTE;
+        const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+        const uint8_t *tile_x = (const uint8_t *)(p.x + tt * L_TOK * p.K);
+        const uint32_t row_pitch = (uint32_t)(p.K * 2);
+        const uint32_t last_row = (uint32_t)(p.N - 1 - tt * L_TOK);  // token rows beyond it re-read it
+        // Activation tile: token t of the tile owns 512 bytes of the stage as 32 chunks of 16 bytes, chunk c stored in
+        // slot c ^ (t % 16) (the MFMA operand reads of 16 tokens x one chunk then fall into 16 different bank groups).
+        // Loader L brings tokens 16 L .. 16 L + 15, two per instruction.
+        uint32_t a_voff[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t t = (uint32_t)(16 * L + 2 * c + (lane >> 5));
+            const uint32_t slot = (uint32_t)(lane & 31);
+            const uint32_t trow = t < last_row ? t : last_row;
+            a_voff[c] = trow * row_pitch + 16u * (slot ^ (t & 15u));
+        }
+        // Weight blocks: piece q of the stage is 16 bytes q % 9 of tile row q / 9; loader L brings pieces
+        // 256 pass + 64 L + lane. Rows beyond M re-read row M - 1 (never stored).
+        const size_t row_bytes = p.nb * Q4_K_BYTES;
+        const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+        uint32_t w_voff[5];
+#pragma unroll
+        for (int pass = 0; pass < 5; ++pass) {
+            const uint32_t q = (uint32_t)(256 * pass + 64 * L + lane);
+            const uint32_t r = q / 9u, c9 = q - 9u * r;
+            const uint32_t rr = r < last_wrow ? r : last_wrow;
+            w_voff[pass] = rr * (uint32_t)row_bytes + 16u * c9;
+        }
+        const uint8_t *wbase = p.w + row0 * row_bytes;
+        const bool fifth = L < 2;  // pieces 1024 .. 1151
+        const int per_block = fifth ? 13 : 12;
+        auto issue = [&](size_t b, int stage) {
+            const uint32_t s0 = lds_base + (uint32_t)(stage * L_STAGE);
+            const uint8_t *xb = tile_x + b * 512;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                dma_set_lds_base(s0 + (uint32_t)(8192 * L + 1024 * c));
+                dma16_to_lds<0>(xb, a_voff[c]);
+            }
+            const uint8_t *wb = wbase + b * Q4_K_BYTES;
+#pragma unroll
+            for (int pass = 0; pass < 4; ++pass) {
+                dma_set_lds_base(s0 + (uint32_t)(L_STAGE_A + (256 * pass + 64 * L) * 16));
+                dma16_to_lds<0>(wb, w_voff[pass]);
+            }
+            if (fifth) {
+                dma_set_lds_base(s0 + (uint32_t)(L_STAGE_A + (1024 + 64 * L) * 16));
+                dma16_to_lds<0>(wb, w_voff[4]);
+            }
+        };
+        // Sub-block sums of this loader's 16 tokens: lane -> token 16 L + lane % 16, sub-blocks 2 (lane / 16) and + 1.
+        const int st = 16 * L + (lane & 15), pair = lane >> 4;
+        const uint32_t sum_dst = (uint32_t)(L_STAGE_A + L_STAGE_W + (st >> 5) * 1024 + (st & 31) * 16 + 4 * pair);
+        auto sums = [&](int stage) {
+            uint8_t *sa = lds + (size_t)stage * L_STAGE;
+            float s0 = 0.0f, s1 = 0.0f;
+            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint4 v = *(const uint4 *)(sa + st * 512 + 16 * ((8 * pair + c) ^ (st & 15)));
+                float acc = c < 4 ? s0 : s1;
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.x), ones, acc, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.y), ones, acc, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.z), ones, acc, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.w), ones, acc, false);
+                if (c < 4) {
+                    s0 = acc;
+                } else {
+                    s1 = acc;
+                }
+            }
+            s0 *= 0.03125f;  // exact; keeps the value within fp16 range whatever the activations are
+            s1 *= 0.03125f;
+            const uint16_t h0 = f2h(s0), h1 = f2h(s1);
+            const uint16_t l0 = f2h(s0 - h2f(h0)), l1 = f2h(s1 - h2f(h1));
+            // S operand of token sub-tile a: lane i holds the 8 hi parts of token 32 a + i, lane 32 + i the lo parts
+            *(uint32_t *)(sa + sum_dst) = (uint32_t)h0 | ((uint32_t)h1 << 16);
+            *(uint32_t *)(sa + sum_dst + 512) = (uint32_t)l0 | ((uint32_t)l1 << 16);
+        };
+
+        issue(b0, 0);
+        if (nblk > 1) {
+            issue(b0 + 1, 1);
+        }
+        wait_vmcnt_at_most(nblk > 1 ? per_block : 0);
+        compiler_memory_fence();
+        sums(0);
+        lds_barrier();
+        for (int i = 0; i < nblk; ++i) {
+            if (i + 2 < nblk) {
+                issue(b0 + (size_t)i + 2, (i + 2) % L_STAGES);
+            }
+            if (i + 1 < nblk) {
+                wait_vmcnt_at_most(i + 2 < nblk ? per_block : 0);
+                compiler_memory_fence();
+                sums((i + 1) % L_STAGES);
+            }
+            lds_barrier();
+        }
+    } else {
+        // ------------------------------------------------------------------------------------------------ compute
+        // MFMA A operand of K-step 8 kg + i, token sub-tile a, lane (j, kh): token 32 a + j, chunk
+        // 16 kg + 4 (i / 2) + 2 kh + i % 2 of the token's 32.
+        uint32_t a_off[4][2];
+#pragma unroll
+        for (int s3 = 0; s3 < 4; ++s3) {
+#pragma unroll
+            for (int tp = 0; tp < 2; ++tp) {
+                a_off[s3][tp] = (uint32_t)(j * 512 + 256 * kg + 16 * ((4 * s3 + 2 * kh + tp) ^ (j & 15)));
+            }
+        }
+        // this lane's two weight rows (row tiles 0 and 1) inside the stage, and the offset of its 16 bytes of 64-value
+        // group 2 kg inside a block (+ 32: group 2 kg + 1)
+        const uint32_t w_off0 = (uint32_t)(L_STAGE_A + (64 * rg + j) * Q4_K_BYTES);
+        const uint32_t q_off = (uint32_t)(16 + 64 * kg + 16 * kh);
+
+        lds_barrier();
+        for (int blk = 0; blk < nblk; ++blk) {
+            const uint8_t *stage = lds + (size_t)(blk % L_STAGES) * L_STAGE;
+            Scales sc[2];
+            uint4 wq[2][2];
+            uint32_t scw[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint8_t *wr = stage + w_off0 + t * 32 * Q4_K_BYTES;
+                const uint4 hdr = *(const uint4 *)wr;
+                wq[t][0] = *(const uint4 *)(wr + q_off);
+                wq[t][1] = *(const uint4 *)(wr + q_off + 32);
+                decode_header(hdr, sc[t]);
+                scw[t] = kg ? sc[t].sc_hi : sc[t].sc_lo;
+            }
+            __half2 scp[2], cp[2];
+            uint32_t m0[2] = {0, 0}, m1[2] = {0, 0};
+            // piece `piece` of B operand t for this wavefront's K-step i (sub-block 4 kg + i / 2, half i % 2)
+            auto b_piece = [&](int t, int i, int piece) -> uint32_t {
+                const int s_ = i >> 1, tp = i & 1, gi = i >> 2;
+                if (piece == 0) {
+                    if (tp == 0) {
+                        const uint32_t sel = s_ == 0 ? 0x04000400u : s_ == 1 ? 0x04010401u
+                                           : s_ == 2 ? 0x04020402u : 0x04030403u;
+                        scp[t] = __hsub2(as_h2(__builtin_amdgcn_perm(0x64646464u, scw[t], sel)), as_h2(0x64006400u));
+                        cp[t] = __hmul2(scp[t], as_h2(0xe400e400u));  // -1024 * sc, exact
+                    }
+                    const uint32_t q0 = tp ? wq[t][gi].z : wq[t][gi].x;
+                    const uint32_t q1 = tp ? wq[t][gi].w : wq[t][gi].y;
+                    m0[t] = ((s_ & 1) ? (q0 >> 4) : q0) & 0x0f0f0f0fu;
+                    m1[t] = ((s_ & 1) ? (q1 >> 4) : q1) & 0x0f0f0f0fu;
+                }
+                switch (piece) {
+                case 0: return dequant_pair<0>(m0[t], scp[t], cp[t]);
+                case 1: return dequant_pair<1>(m0[t], scp[t], cp[t]);
+                case 2: return dequant_pair<0>(m1[t], scp[t], cp[t]);
+                default: return dequant_pair<1>(m1[t], scp[t], cp[t]);
+                }
+            };
+            auto read_a = [&](int i, half8(&aop)[2]) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    aop[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + a_off[i >> 1][i & 1] + a * 16384));
+                }
+            };
+
+            floatx16 acc[2][2];
+            half8 aop[2][2];       // A operands of the K-step in flight and of the next one
+            uint32_t bop[2][2][4];  // B operands likewise
+            read_a(0, aop[0]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int piece = 0; piece < 4; ++piece) {
+                    bop[0][t][piece] = b_piece(t, 0, piece);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = i & 1, n = c ^ 1;
+                if (i < 7) {
+                    read_a(i + 1, aop[n]);  // lands while the MFMAs below run
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const half8 bcur =
+                        __builtin_bit_cast(half8, make_uint4(bop[c][t][0], bop[c][t][1], bop[c][t][2], bop[c][t][3]));
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+                        if (i == 0) {
+                            const floatx16 zero = {0};
+                            acc[t][a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, zero, 0, 0, 0);
+                        } else {
+                            acc[t][a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, acc[t][a], 0, 0, 0);
+                        }
+                        if (i < 7) {  // the next K-step's B operands, two pieces in the shadow of each MFMA
+                            bop[n][t][2 * a] = b_piece(t, i + 1, 2 * a);
+                            bop[n][t][2 * a + 1] = b_piece(t, i + 1, 2 * a + 1);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            // per-block scale of the P product
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        total[t][a][r] = __builtin_fmaf(sc[t].d, acc[t][a][r], total[t][a][r]);
+                    }
+                }
+            }
+            // Q product of the block, all eight sub-blocks: row tile kg by the wavefronts of K half kg
+            const uint8_t *stage_s = stage + L_STAGE_A + L_STAGE_W;
+            auto q_term = [&](floatx16(&tot)[2], const Scales &s) {
+                const half8 b2 = mins_operand(s.mn_lo, s.mn_hi);
+                const float ndmin = -s.dmin;
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const half8 a2 = __builtin_bit_cast(half8, *(const uint4 *)(stage_s + ((size_t)a * 64 + lane) * 16));
+                    const floatx16 zero = {0};
+                    const floatx16 mq = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        tot[a][r] = __builtin_fmaf(ndmin, mq[r], tot[a][r]);
+                    }
+                }
+            };
+            if (kg == 0) {
+                q_term(total[0], sc[0]);
+            } else {
+                q_term(total[1], sc[1]);
+            }
+            lds_barrier();
+        }
+    }
+
+    // ---- the two K halves meet in LDS as one [token][weight row] tile, then every thread stores 16 bytes per step.
+    // Lane (j, kh) of compute wavefront (kg, rg) holds weight row 64 rg + 32 t + j for tokens
+    // 32 a + 8 (r / 4) + 4 kh + r % 4.
+    float *tile = (float *)lds;
+    if (wave < L_COMPUTE && kg == 1) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * L_OUT_PITCH + 64 * rg + 32 * t + j] = total[t][a][r];
+                }
+            }
+        }
+    }
+    lds_barrier();
+    if (wave < L_COMPUTE && kg == 0) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * L_OUT_PITCH + 64 * rg + 32 * t + j;
+                    *e = total[t][a][r] + *e;
+                }
+            }
+        }
+    }
+    lds_barrier();
+
+    const bool partials = p.splits > 1;
+    const bool has_bias = !partials && p.bias != nullptr;
+    const bool out_f16 = !partials && p.out_is_f16;
+    float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
+    const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    for (int idx = tid; idx < L_TOK * L_WROWS / 4; idx += L_THREADS) {
+        const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
+        const size_t n = tt * L_TOK + (size_t)t;
+        const size_t m4 = row0 + 4 * (size_t)q4;
+        if (n >= p.N || m4 >= p.M) {
+            continue;
+        }
+        const float4 v = *(const float4 *)(tile + t * L_OUT_PITCH + 4 * q4);
+        const float e4[4] = {v.x, v.y, v.z, v.w};
+        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (m4 + e < p.M) {
+                    bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
+                }
+            }
+        }
+        if (!out_f16) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[e] = has_bias ? e4[e] + bias4[e] : e4[e];
+            }
+            float *dst = out32 + n * p.M + m4;
+            if (vec) {  // M % 4 == 0: the four rows exist
+                *(float4 *)dst = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = o[e];
+                    }
+                }
+            }
+        } else {
+            uint16_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
+                if (has_bias) {
+                    h[e] = f2h(h2f(h[e]) + bias4[e]);
+                }
+            }
+            uint16_t *dst = (uint16_t *)p.out + n * p.M + m4;
+            if (vec) {
+                *(uint2 *)dst = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = h[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
 // sums the K-split partials in split order, then bias / output cast like the single-pass epilogue
 template <int V>
 __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ partial, int splits, size_t N, size_t M,
@@ -985,6 +1393,40 @@ static int launch_gemm_shape(marmot_hip_device *dev, GemmParams p, size_t N, siz
     return MARMOT_HIP_SUCCESS;
 }
 
+static int launch_gemm_ls(marmot_hip_device *dev, GemmParams p, size_t N, size_t K, size_t M, const void *d_bias,
+                          int bias_dtype, void *d_out, int out_dtype) {
+    const size_t nb = K / QK_K;
+    const size_t tiles_n = (N + L_TOK - 1) / L_TOK;
+    const size_t tiles_m = (M + L_WROWS - 1) / L_WROWS;
+    const size_t tiles = tiles_n * tiles_m;
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    size_t splits = 1;
+    if (tiles * 2 <= cus) {  // fewer tiles than half the chip: split K across workgroups (short prompts)
+        splits = cus / tiles;
+        const size_t max_splits = nb / 2 > 0 ? nb / 2 : 1;  // at least two blocks per workgroup
+        splits = splits > max_splits ? max_splits : splits;
+    }
+    const size_t blocks_per_split = (nb + splits - 1) / splits;
+    splits = (nb + blocks_per_split - 1) / blocks_per_split;
+    float *partial = nullptr;
+    if (splits > 1) {
+        void *ws = nullptr;
+        MH_TRY(workspace_reserve(dev, splits * N * M * sizeof(float), &ws));
+        partial = (float *)ws;
+    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_f16_ls));
+    p.out = splits > 1 ? (void *)partial : d_out;
+    p.splits = (int)splits;
+    p.blocks_per_split = (int)blocks_per_split;
+    hipLaunchKernelGGL(k_gemm_q4k_f16_ls, dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits),
+                       dim3(L_THREADS), L_LDS_BYTES, dev->stream, p);
+    MH_HIP(hipGetLastError());
+    if (splits > 1) {
+        MH_TRY(launch_splitk_reduce(dev, partial, (int)splits, N, M, d_bias, bias_dtype, d_out, out_dtype));
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
 static int launch_gemm_big(marmot_hip_device *dev, GemmParams p, size_t N, size_t K, size_t M, const void *d_bias,
                            int bias_dtype, void *d_out, int out_dtype) {
     const size_t nb = K / QK_K;
@@ -1055,6 +1497,10 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     set_route("gemm_q4_k_f16_mfma");
     if (big) {
         return launch_gemm_big(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
+    }
+    // the loader-wavefront kernel moves 16-byte pieces of the weight blocks; K < 2^22 keeps its 32-bit offsets exact
+    if (!dev->knobs.no_gemm_loaders && (((uintptr_t)d_w) & 15) == 0 && K < ((size_t)1 << 22)) {
+        return launch_gemm_ls(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
     }
     return launch_gemm_shape<2, 2>(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
 }

@@ -102,3 +102,38 @@ def test_config3_prefill_gemm(hip, oracle, N):
     # rows outside the checked band: K-split and full tiles must agree with a float64 product everywhere
     full_exact = exact_f64(oracle, blocks, x[:8], M, K)
     assert parity_metrics(got[:8], full_exact)[2] <= 1e-5
+
+
+def test_gemm_loader_tile_and_self_loading_tile_agree(oracle, monkeypatch):
+    """The 64 x 128 tile exists twice: fed by loader wavefronts (default) and with wavefronts that load for
+    themselves (MARMOT_HIP_NO_GEMM_LOADERS, read when a device object is created). Both compute the same exact-operand
+    products and differ only in fp32 summation order: each must meet the oracle bound, and they must agree with one
+    another to the same bound, on ragged token / row counts, one block of K, K split across workgroups, bias and
+    fp16 output."""
+    from marmot_amd import HipBackend
+
+    loaders = HipBackend(0)
+    monkeypatch.setenv("MARMOT_HIP_NO_GEMM_LOADERS", "1")
+    plain = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_GEMM_LOADERS")
+    try:
+        cases = [(9, 256, 33), (70, 512, 129), (64, 4096, 128), (130, 1024, 300), (200, 768, 515), (512, 2048, 640)]
+        for n, (N, K, M) in enumerate(cases):
+            print(f"gemm tile pair N={N} K={K} M={M}", flush=True)
+            blocks = oracle.quantize(KIND_Q4_K, gaussian(560 + n, (M, K), 0.02))
+            x = gaussian(570 + n, (N, K)).astype(np.float16)
+            bias = gaussian(580 + n, (M,)) if n % 2 else None
+            a, ref = check_against_oracle(loaders, oracle, blocks, x, M, K, f"loader tile {N}x{K}x{M}", bias=bias)
+            b, _ = check_against_oracle(plain, oracle, blocks, x, M, K, f"self-loading tile {N}x{K}x{M}", bias=bias)
+            assert np.max(np.abs(a - b)) <= 1e-5 * np.max(np.abs(ref))
+        N, K, M = 96, 1024, 260
+        blocks = oracle.quantize(KIND_Q4_K, gaussian(590, (M, K), 0.02))
+        x = gaussian(591, (N, K)).astype(np.float16)
+        bias = gaussian(592, (M,)).astype(np.float16)
+        a, _ = check_against_oracle(loaders, oracle, blocks, x, M, K, "loader tile f16 out", bias=bias, out_dtype=np.float16)
+        b, _ = check_against_oracle(plain, oracle, blocks, x, M, K, "self-loading tile f16 out", bias=bias,
+                                    out_dtype=np.float16)
+        assert np.max(np.abs(a - b)) <= 2e-3 * np.max(np.abs(a))
+    finally:
+        loaders.close()
+        plain.close()

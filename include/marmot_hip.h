@@ -177,6 +177,17 @@ int marmot_hip_dequantize(marmot_hip_device_t *dev, int kind, const void *d_bloc
 int marmot_hip_quantize_activations(marmot_hip_device_t *dev, int act_kind, const void *d_x, int in_dtype,
                                     size_t rows, size_t k, void *d_blocks_out);
 
+/* ------------------------------------------------------------------ K-quant weight quantizers
+ * Replaces cpu_quantize_q4_k / cpu_quantize_q5_k / cpu_quantize_q6_k -> cpu_quantize_blockwise
+ * (src/backends/cpu/quantization/ops/quantize_core.c:199-265) with the per-block searches of
+ * src/backends/cpu/quantization/formats/q4k_gguf.c:35-131, q5k_gguf.c:35-160, q6k_gguf.c:35-61 and
+ * src/backends/cpu/quantization/common/kquant_common.h:39-130 (make_qkx2_quants), 150-236 (make_qx_quants),
+ * 310-369 (quantize_row_q6_k_ref_single). d_x: [rows, k] fp32, row-major; d_blocks_out: rows x ceil(k / 256) blocks of
+ * `kind` (Q4_K, Q5_K or Q6_K), a partial last block quantizes zeros beyond k and zeroes the bytes the reference zeroes.
+ * The blocks equal the reference's byte for byte (model preparation: not a per-token path). */
+int marmot_hip_quantize_weights(marmot_hip_device_t *dev, int kind, const float *d_x, size_t rows, size_t k,
+                                void *d_blocks_out);
+
 /* ------------------------------------------------------------------ quantized linear
  * Replaces cpu_matmul_quantized_{scheme} (every weight scheme of the reference) -> cpu_matmul_quantized_impl
  * (src/backends/cpu/ops/matmul/quantized/matmul_quant_dispatch.c:373-591, 905-929) incl. the bias epilogue

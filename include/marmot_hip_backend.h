@@ -821,7 +821,8 @@ marmot_error_t hip_geglu_f32(const void *device_ctx, const marmot_tensor_t *a, c
                              marmot_tensor_t *out);
 marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
                            marmot_tensor_t *out);
-/* output->quant_kind selects the activation block format: Q8_0 or Q8_K */
+/* output->quant_kind selects the block format: the activation formats Q8_0 and Q8_K (FLOAT32 or FLOAT16 input) or the
+ * weight formats Q4_K, Q5_K and Q6_K (FLOAT32 input; cf. cpu_quantize_q4_k / _q5_k / _q6_k, quantize_core.c:199-265) */
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output);
 /* input->quant_kind selects the weight block format: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K,
  * Q6_K or Q8_K */

@@ -231,6 +231,23 @@ class HipBackend:
         d_out.free()
         return out
 
+    def quantize_weights(self, kind: int, x: np.ndarray) -> np.ndarray:
+        """fp32 rows -> Q4_K / Q5_K / Q6_K blocks on the device (the reference's K-quant quantizers, byte for byte);
+        returns [rows, row_bytes] uint8."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if x.ndim == 1:
+            x = x[None, :]
+        rows, k = x.shape
+        d_x = self.to_device(x)
+        d_out = self.alloc(max(1, rows * row_bytes(kind, k)))
+        try:
+            check(self.lib.marmot_hip_quantize_weights(self.dev, kind, C.c_void_p(d_x.ptr), rows, k,
+                                                       C.c_void_p(d_out.ptr)))
+            return d_out.download(np.uint8, (rows, row_bytes(kind, k)))
+        finally:
+            d_x.free()
+            d_out.free()
+
     def linear(self, x: np.ndarray, weight: np.ndarray, kind: int, M: int, bias: np.ndarray | None = None,
                out_dtype=np.float32, force_pack: bool = False) -> np.ndarray:
         """marmot_linear(input[N,K], weight[M,K] as GGUF blocks) -> out[N,M]."""

@@ -96,6 +96,7 @@ SIGNATURES = {
     "marmot_hip_row_bytes": (_sz, [_i, _sz]),
     "marmot_hip_dequantize": (_i, [_vp, _i, _vp, _sz, _sz, _vp]),
     "marmot_hip_quantize_activations": (_i, [_vp, _i, _vp, _i, _sz, _sz, _vp]),
+    "marmot_hip_quantize_weights": (_i, [_vp, _i, _vp, _sz, _sz, _vp]),
     "marmot_hip_matmul_quantized": (_i, [_vp, _i, _vp, _vp, _i, _sz, _sz, _sz, _vp, _i, _vp, _i, _u32]),
     "marmot_hip_matmul_quantized_noalloc": (_i, [_vp, _i, _vp, _vp, _i, _sz, _sz, _sz, _vp, _i, _vp, _i, _u32]),
     "marmot_hip_matmul_quantized_dual": (_i, [_vp, _i, _vp, _vp, _vp, _i, _sz, _sz, _sz, _vp, _vp, _i, _u32]),

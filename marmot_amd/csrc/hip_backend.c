@@ -1226,9 +1226,14 @@ static marmot_error_t quantize_locked(hip_backend_t *b, const marmot_tensor_t *i
     if (st != MARMOT_SUCCESS) {
         return st;
     }
-    const int rc = marmot_hip_quantize_activations(
-        b->dev, kind, d_x, input->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, rows, k,
-        d_q);
+    int rc;
+    if (kind == MARMOT_QUANT_KIND_Q8_0 || kind == MARMOT_QUANT_KIND_Q8_K) {
+        rc = marmot_hip_quantize_activations(
+            b->dev, kind, d_x, input->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, rows,
+            k, d_q);
+    } else {
+        rc = marmot_hip_quantize_weights(b->dev, kind, (const float *)d_x, rows, k, d_q);
+    }
     if (rc != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(rc);
     }
@@ -1241,11 +1246,16 @@ static marmot_error_t quantize_block(const void *device_ctx, const marmot_tensor
     if (b == nullptr || input == nullptr || output == nullptr) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize: null argument");
     }
-    if (output->quant_kind != MARMOT_QUANT_KIND_Q8_0 && output->quant_kind != MARMOT_QUANT_KIND_Q8_K) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP quantize produces the activation formats Q8_0 and Q8_K");
+    const bool act_kind = output->quant_kind == MARMOT_QUANT_KIND_Q8_0 || output->quant_kind == MARMOT_QUANT_KIND_Q8_K;
+    const bool weight_kind = output->quant_kind == MARMOT_QUANT_KIND_Q4_K ||
+        output->quant_kind == MARMOT_QUANT_KIND_Q5_K || output->quant_kind == MARMOT_QUANT_KIND_Q6_K;
+    if (!act_kind && !weight_kind) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED,
+                    "HIP quantize produces the activation formats Q8_0 and Q8_K and the weight formats Q4_K, Q5_K and Q6_K");
     }
-    if (input->dtype != MARMOT_DTYPE_FLOAT32 && input->dtype != MARMOT_DTYPE_FLOAT16) {
-        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Quantize input must be FLOAT32 or FLOAT16");
+    if (input->dtype != MARMOT_DTYPE_FLOAT32 && !(act_kind && input->dtype == MARMOT_DTYPE_FLOAT16)) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE,
+                    "Quantize input must be FLOAT32 (or FLOAT16 for the activation formats)");
     }
     if (!rows_contiguous(input)) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Quantize expects a contiguous 2D input");
@@ -2067,12 +2077,15 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
             return unsupported("HIP TopK takes FLOAT32 values");
         }
         return selected(MARMOT_HIP_BC_OP_TOPK_F32, launch_us, 0.0);
-    case MARMOT_OP_QUANTIZE:
-        if (!(in32 || in16) ||
-            (sig->qscheme_id != MARMOT_QSCHEME_Q8_0 && sig->qscheme_id != MARMOT_QSCHEME_Q8_K)) {
-            return unsupported("HIP quantize produces Q8_0 and Q8_K from FLOAT32/FLOAT16");
+    case MARMOT_OP_QUANTIZE: {
+        const bool act = sig->qscheme_id == MARMOT_QSCHEME_Q8_0 || sig->qscheme_id == MARMOT_QSCHEME_Q8_K;
+        const bool wgt = sig->qscheme_id == MARMOT_QSCHEME_Q4_K || sig->qscheme_id == MARMOT_QSCHEME_Q5_K ||
+            sig->qscheme_id == MARMOT_QSCHEME_Q6_K;
+        if (!((act && (in32 || in16)) || (wgt && in32))) {
+            return unsupported("HIP quantize produces Q8_0 and Q8_K from FLOAT32/FLOAT16, Q4_K, Q5_K and Q6_K from FLOAT32");
         }
         return selected(MARMOT_HIP_BC_OP_QUANTIZE_BLOCK, launch_us, 0.0);
+    }
     case MARMOT_OP_DEQUANTIZE:
         if (kind_of_scheme(sig->qscheme_id) == 0 || !out32) {
             return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q8_K to FLOAT32");

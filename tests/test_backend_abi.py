@@ -206,7 +206,11 @@ def test_query_kernel_other_ops(lib):
     assert _query(lib, _sig(op=ta.OP_TOPK)).op_index == 9
     assert _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q8_K)).op_index == 10
     assert _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q8_0, inp=ta.DTYPE_F16)).op_index == 10
-    assert not _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_K)).supported
+    # weight formats with the K-quant searches on the device: FLOAT32 input only
+    assert _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_K)).op_index == 10
+    assert _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q6_K)).op_index == 10
+    assert not _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_K, inp=ta.DTYPE_F16)).supported
+    assert not _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_0)).supported
     assert _query(lib, _sig(op=ta.OP_DEQUANTIZE, kind=ta.KIND_Q6_K)).op_index == 11
     assert not _query(lib, _sig(op=12345)).supported
 

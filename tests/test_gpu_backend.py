@@ -152,7 +152,7 @@ def test_program_quantize_dequantize_topk(ctx, oracle):
     xt = ta.HostTensor.dense(x)
     p = ta.Program()
     outs = {}
-    for kind in (KIND_Q8_0, KIND_Q8_K):
+    for kind in (KIND_Q8_0, KIND_Q8_K, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K):
         qt = ta.HostTensor(np.zeros(rows * row_bytes(kind, k), np.uint8), (rows, k), ta.DTYPE_I8, kind)
         back = ta.HostTensor.empty((rows, k), ta.DTYPE_F32)
         sel = ctx.query(_sig_for(ta.OP_QUANTIZE, kind))
@@ -165,7 +165,10 @@ def test_program_quantize_dequantize_topk(ctx, oracle):
     p.topk(ctx.query(_sig_for(ta.OP_TOPK, 0)).op_index, logits, vals, idx, 6)
     assert ctx.execute(p) == ta.SUCCESS, ctx.last_error()
     for kind, (qt, back) in outs.items():
-        ref_q = np.stack([oracle.pack(kind, x[r]) for r in range(rows)])
+        if kind in (KIND_Q8_0, KIND_Q8_K):
+            ref_q = np.stack([oracle.pack(kind, x[r]) for r in range(rows)])
+        else:
+            ref_q = oracle.quantize(kind, x)  # the K-quant weight quantizers (cpu_quantize_q4_k / _q5_k / _q6_k)
         assert np.array_equal(ctx.to_host(qt).reshape(rows, -1), ref_q)
         assert np.array_equal(bits(ctx.to_host(back)), bits(oracle.dequantize(kind, ref_q, k)))
     ov, oi = oracle.topk(logits.array, 6)

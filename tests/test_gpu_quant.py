@@ -95,3 +95,69 @@ def test_activation_quantizer_rounding_ties(hip, oracle):
         got = hip.quantize_activations(act_kind, x)
         exp = oracle.pack(act_kind, x[0])[None, :]
         assert np.array_equal(got, exp)
+
+
+# ---------------------------------------------------------------- K-quant weight quantizers on the device
+WEIGHT_QUANT_KINDS = {"q4_k": KIND_Q4_K, "q5_k": KIND_Q5_K, "q6_k": KIND_Q6_K}
+
+
+@pytest.mark.parametrize("name", list(WEIGHT_QUANT_KINDS))
+def test_weight_quantizer_reference_golden_and_reference_build(hip, name):
+    """The reference's own golden blocks (its quantization test's 96-value pattern repeated to 256,
+    test_backend_quantization.c:209-215) and the blocks its compiled quantizers wrote for Gaussian rows (fixture made
+    by the reference build): the device writes the same bytes."""
+    kind = WEIGHT_QUANT_KINDS[name]
+    gold = np.load("tests/golden/reference_goldens.npz")
+    src = gold["g_llama_test_input"]
+    x = np.array([src[i % 96] for i in range(256)], dtype=np.float32)
+    assert np.array_equal(hip.quantize_weights(kind, x)[0], gold[f"g_llama_{name}"])
+    ref = np.load("tests/golden/ref_gaussian.npz")
+    got = hip.quantize_weights(kind, ref[f"{name}_w"])
+    assert np.array_equal(got, ref[f"{name}_blocks"]), f"{(got != ref[f'{name}_blocks']).sum()} bytes differ"
+
+
+@pytest.mark.parametrize("name", list(WEIGHT_QUANT_KINDS))
+def test_weight_quantizer_bit_exact(hip, oracle, name):
+    """Byte equality with the CPU oracle: Gaussian weights at model scale, wide dynamic range, rows that are constant,
+    all zero, all positive, all negative, tiny and huge, sub-blocks of zeros inside a live block, and a partial last
+    block (the bytes beyond it are zeroed like the reference's)."""
+    kind = WEIGHT_QUANT_KINDS[name]
+    rng = np.random.default_rng(900 + kind)
+    cases = [gaussian(901 + kind, (24, 1024), 0.02)]
+    wide = gaussian(902 + kind, (8, 768)) * np.exp(rng.uniform(-12.0, 6.0, size=(8, 768))).astype(np.float32)
+    cases.append(wide.astype(np.float32))
+    special = np.zeros((10, 512), dtype=np.float32)
+    special[0, :] = 0.37
+    special[1, :] = 0.0
+    special[2, :] = np.abs(gaussian(903, (512,)))
+    special[3, :] = -np.abs(gaussian(904, (512,)))
+    special[4, :] = gaussian(905, (512,)) * 1e-20
+    special[5, :] = gaussian(906, (512,)) * 1e20
+    special[6, :] = gaussian(907, (512,))
+    special[6, 32:96] = 0.0            # zero sub-blocks inside a live block
+    special[6, 256:272] = 0.0
+    special[7, ::2] = 1.0              # two levels only
+    special[8, 5] = 3.0                # one value, the rest zero
+    special[9, :] = np.linspace(-1.0, 1.0, 512, dtype=np.float32)
+    cases.append(special)
+    cases.append(gaussian(908 + kind, (5, 300), 0.5))    # partial last block of 44 values
+    cases.append(gaussian(909 + kind, (3, 70)))          # a single partial block
+    for n, x in enumerate(cases):
+        print(f"weight quantizer {name} case {n} shape {x.shape}", flush=True)
+        got = hip.quantize_weights(kind, x)
+        exp = oracle.quantize(kind, x)
+        assert got.shape == exp.shape
+        bad = np.argwhere(got != exp)
+        assert bad.size == 0, f"{name} case {n}: {len(bad)} bytes differ, first at row {bad[0][0]} byte {bad[0][1]}"
+
+
+def test_weight_quantizer_config_shapes(hip, oracle):
+    """The decode configuration's own weights: N(0, 0.02) rows of 4096 and 14336 values through the device quantizer
+    equal the oracle's blocks, and the quantized linear on them equals the one on the oracle's."""
+    for name, k, rows in (("q4_k", 4096, 96), ("q6_k", 14336, 40)):
+        kind = WEIGHT_QUANT_KINDS[name]
+        w = gaussian(920 + k, (rows, k), 0.02)
+        got = hip.quantize_weights(kind, w)
+        assert np.array_equal(got, oracle.quantize(kind, w))
+    with pytest.raises(Exception):
+        hip.quantize_weights(KIND_Q4_0, gaussian(930, (2, 64)))

@@ -417,6 +417,31 @@ int marmot_hip_gguf_tensor(const marmot_hip_gguf_t *g, size_t index, marmot_hip_
 int marmot_hip_gguf_find(const marmot_hip_gguf_t *g, const char *name, marmot_hip_gguf_tensor_t *out);
 int marmot_hip_gguf_upload(marmot_hip_device_t *dev, const marmot_hip_gguf_t *g, size_t index, void **d_out);
 
+/* Key/value metadata of the file (marmot_gguf_find_kv, include/marmot/graph/gguf_loader.h:165; the value kinds of
+ * marmot_gguf_value_type_t :72-86). Entries are views into the mapping, valid until marmot_hip_gguf_close:
+ *   type      GGUF value type (0 u8, 1 i8, 2 u16, 3 i16, 4 u32, 5 i32, 6 f32, 7 bool, 8 string, 9 array, 10 u64,
+ *             11 i64, 12 f64); elem_type: element type of an array, else 0
+ *   count     elements of an array, else 1
+ *   data      scalar: its little-endian bytes (unaligned); string: its characters (not NUL-terminated); array of
+ *             scalars: the elements; array of strings: the first length-prefixed string
+ *   nbytes    bytes of that payload
+ * The typed readers take an element index (0 for a scalar or a plain string): _int for the integer and bool types,
+ * _float for every numeric type, _string for a string or an element of a string array. */
+typedef struct {
+    const char *key;    /* NUL-terminated */
+    uint32_t type;
+    uint32_t elem_type;
+    uint64_t count;
+    const void *data;
+    size_t nbytes;
+} marmot_hip_gguf_kv_t;
+size_t marmot_hip_gguf_kv_count(const marmot_hip_gguf_t *g);
+int marmot_hip_gguf_kv(const marmot_hip_gguf_t *g, size_t index, marmot_hip_gguf_kv_t *out);
+int marmot_hip_gguf_find_kv(const marmot_hip_gguf_t *g, const char *key, marmot_hip_gguf_kv_t *out);
+int marmot_hip_gguf_kv_int(const marmot_hip_gguf_kv_t *kv, uint64_t index, int64_t *out);
+int marmot_hip_gguf_kv_float(const marmot_hip_gguf_kv_t *kv, uint64_t index, double *out);
+int marmot_hip_gguf_kv_string(const marmot_hip_gguf_kv_t *kv, uint64_t index, const char **chars, size_t *length);
+
 /* ------------------------------------------------------------------ introspection
  * Name of the kernel route the last marmot_hip_matmul_quantized call on this thread took
  * (counterpart of the reference's MARMOT_METAL_LOG_MATMUL_QUANT route log,

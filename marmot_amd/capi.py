@@ -50,6 +50,12 @@ class GgufTensor(C.Structure):
                 ("ndim", C.c_uint32), ("shape", C.c_uint64 * 4), ("data", C.c_void_p), ("nbytes", C.c_size_t)]
 
 
+class GgufKv(C.Structure):
+    """marmot_hip_gguf_kv_t"""
+    _fields_ = [("key", C.c_char_p), ("type", C.c_uint32), ("elem_type", C.c_uint32), ("count", C.c_uint64),
+                ("data", C.c_void_p), ("nbytes", C.c_size_t)]
+
+
 class MoeProbe(C.Structure):
     """marmot_hip_moe_probe_t"""
     _fields_ = [("d_sorted_tokens", C.c_void_p), ("d_route_pos", C.c_void_p), ("d_gate_out", C.c_void_p),
@@ -131,6 +137,12 @@ SIGNATURES = {
     "marmot_hip_gguf_tensor": (_i, [_vp, _sz, C.POINTER(GgufTensor)]),
     "marmot_hip_gguf_find": (_i, [_vp, C.c_char_p, C.POINTER(GgufTensor)]),
     "marmot_hip_gguf_upload": (_i, [_vp, _vp, _sz, C.POINTER(_vp)]),
+    "marmot_hip_gguf_kv_count": (_sz, [_vp]),
+    "marmot_hip_gguf_kv": (_i, [_vp, _sz, C.POINTER(GgufKv)]),
+    "marmot_hip_gguf_find_kv": (_i, [_vp, C.c_char_p, C.POINTER(GgufKv)]),
+    "marmot_hip_gguf_kv_int": (_i, [C.POINTER(GgufKv), C.c_uint64, C.POINTER(C.c_int64)]),
+    "marmot_hip_gguf_kv_float": (_i, [C.POINTER(GgufKv), C.c_uint64, C.POINTER(C.c_double)]),
+    "marmot_hip_gguf_kv_string": (_i, [C.POINTER(GgufKv), C.c_uint64, C.POINTER(C.c_char_p), C.POINTER(_sz)]),
 }
 
 _lib = None

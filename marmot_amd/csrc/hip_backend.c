@@ -459,13 +459,22 @@ static marmot_error_t host_is_newer_locked(hip_backend_t *b, const void *src, si
         b->upload_bytes += size;
         return MARMOT_SUCCESS;
     }
-    // not mirrored as a whole: the first kernel that reads the range uploads it; partial overlaps are refreshed
+    // not inside one mirror: partial overlaps are refreshed when a kernel next reads them
+    bool any = false;
     for (size_t i = 0; i < b->n_mirrors; ++i) {
         if (overlaps(&b->mirrors[i], p, size)) {
             b->mirrors[i].host_newer = true;
+            any = true;
         }
     }
-    return MARMOT_SUCCESS;
+    if (any) {
+        return MARMOT_SUCCESS;
+    }
+    // A range the backend has never seen: marmot_tensor_to_device on a fresh tensor, which is how an execution session
+    // puts a model's weights on the device before the first token (src/graph/execution_session.cpp:315-320). Mirror and
+    // upload it now, so that the first kernel that reads it finds it resident.
+    const void *d = nullptr;
+    return acquire_read(b, src, size, &d);
 }
 
 static marmot_error_t ops_memcpy_to_device(const void *device_ctx, void *dst, const void *src, size_t size) {

@@ -1,5 +1,6 @@
-// GGUF file reader for the weights of the path: maps a file read-only, parses the header, the key/value table (only
-// general.alignment is interpreted) and the tensor table, and exposes every tensor as a view into the mapping with the
+// GGUF file reader for the weights of the path: maps a file read-only, parses the header, the key/value table (kept as
+// views into the mapping for marmot_hip_gguf_find_kv; only general.alignment is interpreted here) and the tensor table,
+// and exposes every tensor as a view into the mapping with the
 // shape convention and the ggml-type -> quant-kind mapping of the reference's loader (src/graph/gguf/loader.cpp:
 // map_ggml_type :300-490, set_tensor_data_views :492-575, load_file :577-770). Host code only. Tensor views are host
 // pointers: the tensor-level backend mirrors them on first use; marmot_hip_gguf_upload copies one tensor to the device
@@ -10,6 +11,7 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <cstdint>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -33,6 +35,13 @@ struct marmot_hip_gguf {
         size_t nbytes = 0;
     };
     std::vector<Entry> tensors;
+    struct Kv {
+        std::string key;
+        uint32_t type = 0, elem_type = 0;
+        uint64_t count = 1;
+        size_t offset = 0, nbytes = 0;  // payload inside the mapping
+    };
+    std::vector<Kv> kv;
 };
 
 namespace {
@@ -94,9 +103,20 @@ size_t scalar_size(uint32_t type) {
     }
 }
 
-bool skip_value(Cursor &c, uint32_t type, uint32_t *u32_out) {
+// Steps over one value and records where its payload lies: a scalar's bytes, a string's characters, an array's
+// elements (for an array of strings the first length-prefixed string; nbytes covers all of them).
+bool skip_value(Cursor &c, uint32_t type, uint32_t *u32_out, marmot_hip_gguf::Kv *kv) {
+    kv->type = type;
+    kv->elem_type = 0;
+    kv->count = 1;
     if (type == 8) {
-        return c.read_string(nullptr);
+        uint64_t len = 0;
+        if (!c.read(len) || len > c.size - c.off) {
+            return false;
+        }
+        kv->offset = c.off;
+        kv->nbytes = (size_t)len;
+        return c.skip(len);
     }
     if (type == 9) {
         uint32_t elem = 0;
@@ -107,21 +127,31 @@ bool skip_value(Cursor &c, uint32_t type, uint32_t *u32_out) {
         if (elem == 9) {
             return false;  // nested arrays do not occur in GGUF files
         }
+        kv->elem_type = elem;
+        kv->count = count;
+        kv->offset = c.off;
         if (elem == 8) {
             for (uint64_t i = 0; i < count; ++i) {
                 if (!c.read_string(nullptr)) {
                     return false;
                 }
             }
+            kv->nbytes = c.off - kv->offset;
             return true;
         }
         const size_t es = scalar_size(elem);
-        return es != 0 && count <= (c.size - c.off) / es && c.skip(count * es);
+        if (es == 0 || count > (c.size - c.off) / es) {
+            return false;
+        }
+        kv->nbytes = (size_t)count * es;
+        return c.skip(count * es);
     }
     const size_t s = scalar_size(type);
     if (s == 0) {
         return false;
     }
+    kv->offset = c.off;
+    kv->nbytes = s;
     if (type == 4 && u32_out != nullptr) {
         return c.read(*u32_out);
     }
@@ -270,15 +300,19 @@ int marmot_hip_gguf_open(const char *path, marmot_hip_gguf_t **out) {
     if (n_tensors > g->size / 24 || n_kv > g->size / 12) {
         return fail(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF table sizes exceed the file");
     }
+    g->kv.reserve((size_t)n_kv);
     for (uint64_t i = 0; i < n_kv; ++i) {
         std::string key;
         uint32_t type = 0, u32 = 0;
         if (!c.read_string(&key) || key.empty() || !c.read(type)) {
             return fail(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Invalid GGUF key");
         }
-        if (!skip_value(c, type, &u32)) {
+        marmot_hip_gguf::Kv entry;
+        if (!skip_value(c, type, &u32, &entry)) {
             return fail(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Unable to parse GGUF value");
         }
+        entry.key = key;
+        g->kv.push_back(std::move(entry));
         if (key == "general.alignment" && type == 4 && u32 != 0) {
             g->alignment = u32;
         }
@@ -381,6 +415,118 @@ int marmot_hip_gguf_find(const marmot_hip_gguf_t *g, const char *name, marmot_hi
         }
     }
     return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF tensor '%s' not found", name);
+}
+
+// ---- key/value metadata (marmot_gguf_find_kv, include/marmot/graph/gguf_loader.h:165; values of
+// marmot_gguf_value_t :108-132 as views into the mapping)
+static void fill_kv(const marmot_hip_gguf_t *g, const marmot_hip_gguf::Kv &e, marmot_hip_gguf_kv_t *out) {
+    out->key = e.key.c_str();
+    out->type = e.type;
+    out->elem_type = e.elem_type;
+    out->count = e.count;
+    out->data = g->data + e.offset;
+    out->nbytes = e.nbytes;
+}
+
+size_t marmot_hip_gguf_kv_count(const marmot_hip_gguf_t *g) {
+    return g != nullptr ? g->kv.size() : 0;
+}
+
+int marmot_hip_gguf_kv(const marmot_hip_gguf_t *g, size_t index, marmot_hip_gguf_kv_t *out) {
+    if (g == nullptr || out == nullptr || index >= g->kv.size()) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF key/value index out of range");
+    }
+    fill_kv(g, g->kv[index], out);
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_gguf_find_kv(const marmot_hip_gguf_t *g, const char *key, marmot_hip_gguf_kv_t *out) {
+    if (g == nullptr || key == nullptr || out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF lookup: null argument");
+    }
+    for (const auto &e : g->kv) {
+        if (e.key == key) {
+            fill_kv(g, e, out);
+            return MARMOT_HIP_SUCCESS;
+        }
+    }
+    return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF key '%s' not found", key);
+}
+
+// one element of a scalar value (index 0) or of an array of scalars, widened
+static bool kv_scalar_at(const marmot_hip_gguf_kv_t *kv, uint64_t index, uint64_t *u, int64_t *i, double *f,
+                         int *cls /* 0 unsigned, 1 signed, 2 float */) {
+    const uint32_t t = kv->type == 9 ? kv->elem_type : kv->type;
+    const size_t es = scalar_size(t);
+    if (es == 0 || index >= kv->count || (index + 1) * es > kv->nbytes) {
+        return false;
+    }
+    const uint8_t *p = (const uint8_t *)kv->data + index * es;
+    switch (t) {
+    case 0: case 7: { uint8_t v; std::memcpy(&v, p, 1); *u = v; *cls = 0; return true; }
+    case 1: { int8_t v; std::memcpy(&v, p, 1); *i = v; *cls = 1; return true; }
+    case 2: { uint16_t v; std::memcpy(&v, p, 2); *u = v; *cls = 0; return true; }
+    case 3: { int16_t v; std::memcpy(&v, p, 2); *i = v; *cls = 1; return true; }
+    case 4: { uint32_t v; std::memcpy(&v, p, 4); *u = v; *cls = 0; return true; }
+    case 5: { int32_t v; std::memcpy(&v, p, 4); *i = v; *cls = 1; return true; }
+    case 6: { float v; std::memcpy(&v, p, 4); *f = v; *cls = 2; return true; }
+    case 10: { uint64_t v; std::memcpy(&v, p, 8); *u = v; *cls = 0; return true; }
+    case 11: { int64_t v; std::memcpy(&v, p, 8); *i = v; *cls = 1; return true; }
+    case 12: { double v; std::memcpy(&v, p, 8); *f = v; *cls = 2; return true; }
+    default: return false;
+    }
+}
+
+int marmot_hip_gguf_kv_int(const marmot_hip_gguf_kv_t *kv, uint64_t index, int64_t *out) {
+    uint64_t u = 0;
+    int64_t i = 0;
+    double f = 0;
+    int cls = 0;
+    if (kv == nullptr || out == nullptr || !kv_scalar_at(kv, index, &u, &i, &f, &cls) || cls == 2 ||
+        (cls == 0 && u > (uint64_t)INT64_MAX)) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF value is not an integer that fits int64");
+    }
+    *out = cls == 0 ? (int64_t)u : i;
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_gguf_kv_float(const marmot_hip_gguf_kv_t *kv, uint64_t index, double *out) {
+    uint64_t u = 0;
+    int64_t i = 0;
+    double f = 0;
+    int cls = 0;
+    if (kv == nullptr || out == nullptr || !kv_scalar_at(kv, index, &u, &i, &f, &cls)) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF value is not a number");
+    }
+    *out = cls == 2 ? f : (cls == 0 ? (double)u : (double)i);
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_gguf_kv_string(const marmot_hip_gguf_kv_t *kv, uint64_t index, const char **chars, size_t *length) {
+    if (kv == nullptr || chars == nullptr || length == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF string: null argument");
+    }
+    if (kv->type == 8 && index == 0) {
+        *chars = (const char *)kv->data;
+        *length = kv->nbytes;
+        return MARMOT_HIP_SUCCESS;
+    }
+    if (kv->type != 9 || kv->elem_type != 8 || index >= kv->count) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF value is not a string (or the index is out of range)");
+    }
+    Cursor c{(const uint8_t *)kv->data, kv->nbytes};  // lengths were validated when the file was opened
+    for (uint64_t i = 0; i < index; ++i) {
+        if (!c.read_string(nullptr)) {
+            return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF string array is malformed");
+        }
+    }
+    uint64_t len = 0;
+    if (!c.read(len) || len > c.size - c.off) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "GGUF string array is malformed");
+    }
+    *chars = (const char *)c.p + c.off;
+    *length = (size_t)len;
+    return MARMOT_HIP_SUCCESS;
 }
 
 int marmot_hip_gguf_upload(marmot_hip_device_t *dev, const marmot_hip_gguf_t *g, size_t index, void **d_out) {

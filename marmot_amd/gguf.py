@@ -43,6 +43,39 @@ class GgufFile:
         capi.check(self.lib.marmot_hip_gguf_find(self.handle, name.encode(), C.byref(t)))
         return self.by_name[t.name.decode()]
 
+    # ---- key/value metadata (marmot_gguf_find_kv)
+    def _value(self, kv):
+        """Python value of one entry: int / float / bool / str, or a list of them for arrays."""
+        def one(t, i):
+            if t == 8:
+                p, n = C.c_char_p(), C.c_size_t()
+                capi.check(self.lib.marmot_hip_gguf_kv_string(C.byref(kv), i, C.byref(p), C.byref(n)))
+                return C.string_at(p, n.value).decode()
+            if t in (6, 12):
+                v = C.c_double()
+                capi.check(self.lib.marmot_hip_gguf_kv_float(C.byref(kv), i, C.byref(v)))
+                return v.value
+            v = C.c_int64()
+            capi.check(self.lib.marmot_hip_gguf_kv_int(C.byref(kv), i, C.byref(v)))
+            return bool(v.value) if t == 7 else v.value
+        if kv.type == 9:
+            return [one(kv.elem_type, i) for i in range(kv.count)]
+        return one(kv.type, 0)
+
+    def metadata(self) -> Dict[str, object]:
+        """Every key of the file with its value, in file order."""
+        out = {}
+        for i in range(self.lib.marmot_hip_gguf_kv_count(self.handle)):
+            kv = capi.GgufKv()
+            capi.check(self.lib.marmot_hip_gguf_kv(self.handle, i, C.byref(kv)))
+            out[kv.key.decode()] = self._value(kv)
+        return out
+
+    def get(self, key: str):
+        kv = capi.GgufKv()
+        capi.check(self.lib.marmot_hip_gguf_find_kv(self.handle, key.encode(), C.byref(kv)))
+        return self._value(kv)
+
     def array(self, info: GgufTensorInfo) -> np.ndarray:
         """The tensor's bytes inside the mapping (no copy; valid until close): uint8 block bytes for quantized
         tensors, else the dense values in the file's dimension order."""

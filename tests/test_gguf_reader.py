@@ -46,6 +46,28 @@ def test_every_weight_format_round_trips(tmp_path, oracle):
         assert e.shape == (256, 8, 3) and e.nbytes == 3 * 8 * 144  # the file's order is kept for rank 3
         with pytest.raises(capi.MarmotHipError):
             g.find("missing")
+        # key/value metadata: every value kind the writer produces, typed readers, file order
+        md = g.metadata()
+        assert list(md)[:6] == ["general.architecture", "llama.block_count", "tokenizer.ggml.tokens",
+                                "llama.rope.freq_base", "some.flag", "some.ints"]
+        assert md["general.architecture"] == "llama" and md["llama.block_count"] == 1
+        assert md["tokenizer.ggml.tokens"] == ["a", "bc"] and md["llama.rope.freq_base"] == 10000.0
+        assert md["some.flag"] is True and md["some.ints"] == [1, 2, 3] and md["general.alignment"] == 32
+        assert g.get("llama.block_count") == 1
+        with pytest.raises(capi.MarmotHipError):
+            g.get("llama.missing")
+        import ctypes as C
+        kv = capi.GgufKv()
+        capi.check(g.lib.marmot_hip_gguf_find_kv(g.handle, b"tokenizer.ggml.tokens", C.byref(kv)))
+        assert (kv.type, kv.elem_type, kv.count) == (9, 8, 2) and kv.nbytes == 8 + 1 + 8 + 2
+        v, f = C.c_int64(), C.c_double()
+        assert g.lib.marmot_hip_gguf_kv_int(C.byref(kv), 0, C.byref(v)) != 0       # a string is no integer
+        p, n = C.c_char_p(), C.c_size_t()
+        assert g.lib.marmot_hip_gguf_kv_string(C.byref(kv), 2, C.byref(p), C.byref(n)) != 0   # past the end
+        capi.check(g.lib.marmot_hip_gguf_find_kv(g.handle, b"llama.rope.freq_base", C.byref(kv)))
+        assert g.lib.marmot_hip_gguf_kv_int(C.byref(kv), 0, C.byref(v)) != 0       # a float is no integer
+        capi.check(g.lib.marmot_hip_gguf_kv_float(C.byref(kv), 0, C.byref(f)))
+        assert f.value == 10000.0 and g.lib.marmot_hip_gguf_kv_float(C.byref(kv), 1, C.byref(f)) != 0
 
 
 def test_alignment_and_version(tmp_path):

@@ -80,3 +80,39 @@ def test_views_into_the_mapping_are_mirrored_once(model, oracle):
         for t in (wt, bt, xt, yt):
             ctx.host_freed(t)
         assert ctx.residency().mirrors == mirrors - 4
+
+
+def test_session_style_preload_then_linears_upload_nothing(model, oracle):
+    """What an execution session does with a model's weights (marmot_tensor_to_device on every tensor before the
+    first token, src/graph/execution_session.cpp:315-320): each announced view is mirrored and uploaded at once, the
+    architecture comes from the file's metadata, and the linears that follow upload only their activations."""
+    path, weights = model
+    with ta.HipContext() as ctx, GgufFile(path) as g:
+        assert g.get("general.architecture") == "test"
+        tensors = {}
+        base = ctx.residency()
+        total = 0
+        for n in NAMES:
+            info = g.find(f"blk.0.{n}.weight")
+            t = ta.HostTensor.quantized(g.array(info), info.shape, info.kind)
+            ctx.host_changed(t)  # marmot_tensor_to_device: dst == src == the host pointer
+            tensors[n] = (info, t)
+            total += info.nbytes
+        loaded = ctx.residency()
+        assert loaded.mirrors == base.mirrors + len(NAMES) and loaded.uploads == base.uploads + len(NAMES)
+        assert loaded.upload_bytes - base.upload_bytes == total
+        x = gaussian(1400, (2, K))
+        for n, (info, wt) in tensors.items():
+            xt = ta.HostTensor.dense(x)
+            yt = ta.HostTensor.empty((2, M), ta.DTYPE_F32)
+            before = ctx.residency()
+            prog = ta.Program()
+            prog.matmul(ctx.query(ctx.matmul_signature(xt, wt, yt)).op_index, xt, wt, yt)
+            assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+            after = ctx.residency()
+            assert after.upload_bytes - before.upload_bytes == x.nbytes, n   # the activations only
+            assert_matmul_parity(ctx.to_host(yt), oracle.matmul(info.kind, weights[n], x, M), what=f"preloaded {n}")
+            ctx.host_freed(xt)
+            ctx.host_freed(yt)
+        for _, t in tensors.values():
+            ctx.host_freed(t)

@@ -28,9 +28,10 @@ METRIC = "Q4_K matvec GB/s (% HBM peak) + prefill GEMM TOPS (% MFMA peak)"
 HBM_PEAK_GBPS = 8000.0
 MALL_BYTES = 256 << 20
 # HBM bytes per launch of the Q4_K 4096x14336 N=1 matvec kernels (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain
-# copy kernel, profiles/matvec_q4_k_4096x14336_n1.md): fused-quantization kernel and kernel on pre-packed activations
-TRAFFIC_FUSED = 33_670_000
-TRAFFIC_PREPACKED = 33_297_000
+# copy kernel, profiles/matvec_q4_k_4096x14336_n1.md): the row-owning kernel with the activation quantization inside
+# (k_matvec_rows_q4k) and the streaming kernel on pre-packed activations (k_matvec_ls)
+TRAFFIC_FUSED = 33_737_000
+TRAFFIC_PREPACKED = 33_288_000
 
 
 def algorithmic_bytes(kind_row_bytes: int, M: int, K: int, N: int) -> int:

@@ -881,10 +881,11 @@ __global__ __launch_bounds__(G_THREADS) void k_gemm_q4k_f16(const GemmParams p) 
 //   * wavefronts 4..7 (one per SIMD) load: per block they bring the activation tile (64 tokens x 512 bytes, two
 //     contiguous token rows per instruction) and the raw weight blocks (128 rows x 144 bytes, nine lanes per block,
 //     so an instruction touches about 14 cache lines instead of 32 to 64) into one of three LDS stages with
-//     direct-to-LDS loads, two blocks ahead, and compute the sub-block sums of the tokens they loaded themselves
-//     (no synchronization between loaders) into the stage's S area before the barrier that hands the stage over.
-// One barrier per block orders everything: behind barrier i the stage of block i is complete (tile, weights, sums) and
-// the stage of block i - 1 is free for block i + 2. The barrier is an LDS-count wait plus s_barrier written by hand:
+//     direct-to-LDS loads, two blocks ahead, and compute the sub-block sums of the block in work (16 tokens per
+//     loader) into the stage's S area while the next block is still landing.
+// One barrier per block orders everything: behind barrier i the tile and the weights of block i are complete, the
+// sums of block i - 1 too (its Q product runs one block late, like in the tile above), and the tile and weight areas of
+// block i - 1's stage are free for block i + 2. The barrier is an LDS-count wait plus s_barrier written by hand:
 // the usual workgroup barrier also waits for the wavefront's outstanding global loads, which here are the two blocks
 // in flight.
 constexpr int L_TOK = 64;
@@ -1022,17 +1023,18 @@ __global__ __launch_bounds__(L_THREADS) void k_gemm_q4k_f16_ls(const GemmParams 
             issue(b0 + 1, 1);
         }
         wait_vmcnt_at_most(nblk > 1 ? per_block : 0);
-        compiler_memory_fence();
-        sums(0);
         lds_barrier();
         for (int i = 0; i < nblk; ++i) {
             if (i + 2 < nblk) {
                 issue(b0 + (size_t)i + 2, (i + 2) % L_STAGES);
             }
+            // The sums of block i, whose tile is complete since the barrier that opened this round, while block i + 1
+            // is still landing; the compute wavefronts take them one block late (the Q product of block i runs behind
+            // the next barrier), so nobody waits for them inside the round.
+            compiler_memory_fence();
+            sums(i % L_STAGES);
             if (i + 1 < nblk) {
                 wait_vmcnt_at_most(i + 2 < nblk ? per_block : 0);
-                compiler_memory_fence();
-                sums((i + 1) % L_STAGES);
             }
             lds_barrier();
         }
@@ -1052,6 +1054,23 @@ __global__ __launch_bounds__(L_THREADS) void k_gemm_q4k_f16_ls(const GemmParams 
         // group 2 kg inside a block (+ 32: group 2 kg + 1)
         const uint32_t w_off0 = (uint32_t)(L_STAGE_A + (64 * rg + j) * Q4_K_BYTES);
         const uint32_t q_off = (uint32_t)(16 + 64 * kg + 16 * kh);
+
+        // Q product of a block, all eight sub-blocks: row tile kg by the wavefronts of K half kg, one block late
+        uint32_t prev_mn_lo = 0, prev_mn_hi = 0;
+        float prev_ndmin = 0.0f;
+        auto q_term = [&](const uint8_t *stage_s, floatx16(&tot)[2]) {
+            const half8 b2 = mins_operand(prev_mn_lo, prev_mn_hi);
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const half8 a2 = __builtin_bit_cast(half8, *(const uint4 *)(stage_s + ((size_t)a * 64 + lane) * 16));
+                const floatx16 zero = {0};
+                const floatx16 mq = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    tot[a][r] = __builtin_fmaf(prev_ndmin, mq[r], tot[a][r]);
+                }
+            }
+        };
 
         lds_barrier();
         for (int blk = 0; blk < nblk; ++blk) {
@@ -1149,28 +1168,28 @@ __global__ __launch_bounds__(L_THREADS) void k_gemm_q4k_f16_ls(const GemmParams 
                     }
                 }
             }
-            // Q product of the block, all eight sub-blocks: row tile kg by the wavefronts of K half kg
-            const uint8_t *stage_s = stage + L_STAGE_A + L_STAGE_W;
-            auto q_term = [&](floatx16(&tot)[2], const Scales &s) {
-                const half8 b2 = mins_operand(s.mn_lo, s.mn_hi);
-                const float ndmin = -s.dmin;
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    const half8 a2 = __builtin_bit_cast(half8, *(const uint4 *)(stage_s + ((size_t)a * 64 + lane) * 16));
-                    const floatx16 zero = {0};
-                    const floatx16 mq = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        tot[a][r] = __builtin_fmaf(ndmin, mq[r], tot[a][r]);
-                    }
+            // Q product of the previous block: its sums were written during the previous round and are complete since the
+            // barrier that opened this one; its stage's tile and weights are being refilled, its S area is not
+            if (blk > 0) {
+                const uint8_t *prev_s = lds + (size_t)((blk - 1) % L_STAGES) * L_STAGE + L_STAGE_A + L_STAGE_W;
+                if (kg == 0) {
+                    q_term(prev_s, total[0]);
+                } else {
+                    q_term(prev_s, total[1]);
                 }
-            };
-            if (kg == 0) {
-                q_term(total[0], sc[0]);
-            } else {
-                q_term(total[1], sc[1]);
             }
+            prev_mn_lo = kg ? sc[1].mn_lo : sc[0].mn_lo;
+            prev_mn_hi = kg ? sc[1].mn_hi : sc[0].mn_hi;
+            prev_ndmin = -(kg ? sc[1].dmin : sc[0].dmin);
             lds_barrier();
+        }
+        {   // the last block's Q product: its sums are complete since the loop's last barrier
+            const uint8_t *last_s = lds + (size_t)((nblk - 1) % L_STAGES) * L_STAGE + L_STAGE_A + L_STAGE_W;
+            if (kg == 0) {
+                q_term(last_s, total[0]);
+            } else {
+                q_term(last_s, total[1]);
+            }
         }
     }
 

@@ -198,8 +198,8 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
-    """Every benchmark configuration (C1..C5, QKV, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "OPS", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
+    """Every benchmark configuration (C1..C5, QKV, OPS, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -283,11 +283,79 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV
         sweep_moe(hip, rng, emit, steps)
     if "QKV" in only:
         sweep_qkv(hip, rng, emit, steps, warmup)
+    if "OPS" in only:
+        sweep_ops(hip, rng, emit, steps, warmup)
     if "LOGITS" in only:
         # the vocabulary-sized matvec at the end of a decode step (Llama-3 vocabulary, 128256 rows of 4096)
         for kind in (capi.KIND_Q6_K, capi.KIND_Q4_K):
             for N in (1, 4):
                 linear_case("LOGITS", kind, 128256, 4096, N)
+
+
+def sweep_ops(hip, rng, emit, steps: int, warmup: int):
+    """The operations between the linears at decode and prefill sizes of a Llama-3-8B layer: RMS normalization and
+    residual add over [T, 4096], SwiGLU over [T, 14336], rotary embedding of the q rows [T x 32, 128] (FLOAT32 and
+    FLOAT16). Inputs and outputs rotate over copies larger than twice the Infinity Cache, so every figure is an HBM
+    rate; inside a layer the producer's output is usually still cache-resident and the operations run faster."""
+    import ctypes as C
+
+    from marmot_amd import DT_F16, DT_F32, capi
+
+    lib, dev = hip.lib, hip.dev
+    vp = C.c_void_p
+
+    def rotating(nbytes, fill=None):
+        stride = (nbytes + 255) & ~255
+        copies = max(2, -(-2 * MALL_BYTES // stride) + 1)
+        buf = hip.alloc(stride * copies)
+        if fill is not None:
+            for c in range(copies):
+                buf.upload(fill, offset=c * stride)
+        return buf, stride, copies
+
+    def run(name, T, nbytes, step, copies):
+        ms = time_steps_graph(hip, step, steps, warmup)
+        emit({"config": "OPS", "workload": f"{name} T={T}", "us": round(ms * 1e3, 2),
+              "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+              "copies": copies})
+
+    for T in (16, 512):
+        H, F, heads, D = 4096, 14336, 32, 128
+        x = rng.standard_normal((T, H), dtype=np.float32)
+        d_x, sx, cx = rotating(x.nbytes, x)
+        d_r, _, _ = rotating(x.nbytes, x)
+        d_y, sy, cy = rotating(x.nbytes)
+        d_w = hip.to_device(np.ones(H, np.float32))
+        run("rms_norm [T,4096] fp32 with residual and weight", T, 3 * x.nbytes + H * 4,
+            lambda i: capi.check(lib.marmot_hip_rms_norm(dev, vp(d_x.ptr + (i % cx) * sx), vp(d_r.ptr + (i % cx) * sx),
+                                                         vp(d_w.ptr), 0.0, 1e-5, T, H, vp(d_y.ptr + (i % cy) * sy))), cx)
+        run("add [T,4096] fp32", T, 3 * x.nbytes,
+            lambda i: capi.check(lib.marmot_hip_add(dev, vp(d_x.ptr + (i % cx) * sx), vp(d_r.ptr + (i % cx) * sx),
+                                                    T * H, vp(d_y.ptr + (i % cy) * sy))), cx)
+        pos = np.repeat(np.arange(T, dtype=np.int32) + 1000, heads)
+        freqs, scale, hd = hip.rope_frequencies(D, head_dim=D, theta=500000.0)
+        d_p, d_f = hip.to_device(pos), hip.to_device(freqs)
+        arg = capi.Rope(d_p.ptr, capi.DT_I32, d_f.ptr, scale, hd, 0, 0, 0)
+        for rope_type in (0, 1):
+            arg.rope_type = rope_type
+            run(f"rope q rows [T x 32,128] fp32 {'neox' if rope_type else 'norm'}", T, 2 * x.nbytes + pos.nbytes,
+                lambda i: capi.check(lib.marmot_hip_rope(dev, vp(d_x.ptr + (i % cx) * sx), DT_F32, T * heads, D, D, D,
+                                                         C.byref(arg), vp(d_y.ptr + (i % cy) * sy))), cx)
+        arg.rope_type = 0
+        run("rope q rows [T x 32,128] fp16 norm", T, x.nbytes + pos.nbytes,
+            lambda i: capi.check(lib.marmot_hip_rope(dev, vp(d_x.ptr + (i % cx) * sx), DT_F16, T * heads, D, D, D,
+                                                     C.byref(arg), vp(d_y.ptr + (i % cy) * sy))), cx)
+        for b in (d_x, d_r, d_y, d_w, d_p, d_f):
+            b.free()
+        g = rng.standard_normal((T, F), dtype=np.float32)
+        d_g, sg, cg = rotating(g.nbytes, g)
+        d_u, _, _ = rotating(g.nbytes, g)
+        d_o, so, co = rotating(g.nbytes)
+        run("swiglu [T,14336] fp32", T, 3 * g.nbytes,
+            lambda i: capi.check(lib.marmot_hip_glu(dev, 0, vp(d_g.ptr + (i % cg) * sg), vp(d_u.ptr + (i % cg) * sg),
+                                                    T, F, F, F, F, vp(d_o.ptr + (i % co) * so))), cg)
+        for b in (d_g, d_u, d_o):
+            b.free()
 
 
 def sweep_qkv(hip, rng, emit, steps: int, warmup: int):

@@ -344,6 +344,16 @@ int marmot_hip_swiglu_pack(marmot_hip_device_t *dev, const float *d_gate, const 
                            int weight_kind, void *d_packed);
 /* Replaces cpu_add for contiguous fp32 tensors of equal shape (the residual add). */
 int marmot_hip_add(marmot_hip_device_t *dev, const float *d_a, const float *d_b, size_t n, float *d_out);
+/* Replaces cpu_rope (src/backends/cpu/ops/rope/rope_dispatch.c:145-372; validation :18-88) for FLOAT32 and FLOAT16
+ * rows: d_x and d_out hold `rows` rows of `dim` values at row strides (in elements) >= dim; row r is rotated by
+ * positions[r]: angle_i = (float)position * freq_i, cos and sin times attn_scale, pairs (2i, 2i+1) for rope_type 0
+ * and (i, i + dim/2) for 1; arithmetic in fp32, one rounding at a FLOAT16 store. rope->d_freqs holds the dim/2
+ * frequencies of marmot_hip_rope_frequencies for head_dim == dim (rope->head_dim must say so); the apply flags are
+ * not read. d_out == d_x rotates in place; other overlaps are not supported. Errors in the reference's order: odd dim
+ * DIMENSION_MISMATCH, empty input INVALID_ARGUMENT, positions type UNSUPPORTED_DTYPE, a stride below dim
+ * DIMENSION_MISMATCH. */
+int marmot_hip_rope(marmot_hip_device_t *dev, const void *d_x, int dtype, size_t rows, size_t dim,
+                    size_t x_row_stride, size_t out_row_stride, const marmot_hip_rope_t *rope, void *d_out);
 
 /* ------------------------------------------------------------------ MoE
  * Replaces cpu_topk_impl (src/backends/cpu/ops/moe/moe_ops.c:789-889): top-k over the last axis of

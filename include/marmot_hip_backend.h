@@ -366,6 +366,7 @@ typedef enum {
     MARMOT_OP_LINEAR = 708,
     MARMOT_OP_QKV_SHARED_INPUT = 771,
     MARMOT_OP_QKV_ROPE = 778,
+    MARMOT_OP_ROPE = 843,
     MARMOT_OP_EMBEDDING = 853,
     MARMOT_OP_ADD = 876,
     MARMOT_OP_TOPK = 901,
@@ -682,7 +683,9 @@ bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_bac
  *   QUANTIZE    u16 input; u32 quant-params const offset; u16 output; u32 kind; u32 layout   (:912-941)
  *   DEQUANTIZE  u16 input; u16 output; u32 kind; u32 layout            (bytecode_compile.c:942-962)
  *   RMS_NORM    u16 input, weight, residual (0xFFFF none), output; f32 eps      (bytecode_compile.c:530-552)
- *   BINARY      u16 input_a, input_b, output                            (bytecode_compile.c:357-375) */
+ *   BINARY      u16 input_a, input_b, output                            (bytecode_compile.c:357-375)
+ *   ROPE        u16 input, output, positions (0xFFFF: the parameters' own tensor); u32 rope-params const offset;
+ *               u32 n_past; u32 n_rot                                   (bytecode_compile.c:598-623) */
 enum {
     MARMOT_HIP_BC_OP_END = 0,
     MARMOT_HIP_BC_OP_MATMUL_Q4_0 = 1,
@@ -739,7 +742,9 @@ enum {
     MARMOT_HIP_BC_OP_SWIGLU_F32 = 50,
     MARMOT_HIP_BC_OP_GEGLU_F32 = 51,
     MARMOT_HIP_BC_OP_ADD_F32 = 52,
-    MARMOT_HIP_BC_OP_COUNT = 53,
+    /* rotary embedding of FLOAT32 or FLOAT16 rows */
+    MARMOT_HIP_BC_OP_ROPE = 53,
+    MARMOT_HIP_BC_OP_COUNT = 54,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -821,6 +826,13 @@ marmot_error_t hip_geglu_f32(const void *device_ctx, const marmot_tensor_t *a, c
                              marmot_tensor_t *out);
 marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
                            marmot_tensor_t *out);
+/* marmot_rope (cf. cpu_rope, src/backends/cpu/ops/rope/rope_dispatch.c:145-372): the last dimension of x, FLOAT32 or
+ * FLOAT16, is rotated into out (same shape and type; out == x rotates in place), one position per row from
+ * params->positions (FLOAT32, INT32 or INT64, as many values as x has rows); frequencies and attention scale as
+ * marmot_rope_freq_cache_ensure for the rotated dimension (src/core/helpers/rope.c:143-200), all scaling types.
+ * Contiguous tensors, or rows at one stride >= their length; FLOAT64 and BFLOAT16 are declined NOT_IMPLEMENTED. */
+marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
+                        marmot_tensor_t *out);
 /* output->quant_kind selects the block format: the activation formats Q8_0 and Q8_K (FLOAT32 or FLOAT16 input) or the
  * weight formats Q4_K, Q5_K and Q6_K (FLOAT32 input; cf. cpu_quantize_q4_k / _q5_k / _q6_k, quantize_core.c:199-265) */
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output);

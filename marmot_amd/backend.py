@@ -474,6 +474,39 @@ class HipBackend:
             for b_ in bufs:
                 b_.free()
 
+    def rope(self, x: np.ndarray, positions: np.ndarray, rope_type: int = 0, dim=None, x_row_stride=None,
+             out_row_stride=None, in_place: bool = False, **freq_kw) -> np.ndarray:
+        """marmot_rope (include/marmot/ops/rope.h; CPU implementation src/backends/cpu/ops/rope/rope_dispatch.c): the
+        last dimension of x (float32 or float16, rank >= 2) is rotated, one position (float32, int32 or int64) per row;
+        freq_kw are the keyword arguments of rope_frequencies (head_dim is the rotated dimension). With `dim` and row
+        strides (in elements), x is a flat buffer of positions.size rows of dim values at x_row_stride and the result
+        a flat buffer of rows at out_row_stride (its gaps keep the NaN they are filled with)."""
+        x = np.ascontiguousarray(x)
+        pos = np.ascontiguousarray(positions)
+        pos_dt = {np.dtype(np.float32): capi.DT_F32, np.dtype(np.int32): capi.DT_I32,
+                  np.dtype(np.int64): capi.DT_I64}[pos.dtype]
+        if dim is None:
+            dim = x.shape[-1]
+            rows = x.size // dim
+            xs = os_ = dim
+            out_shape, out_size = x.shape, x.size
+        else:
+            rows, xs, os_ = pos.size, x_row_stride, out_row_stride
+            out_size = (rows - 1) * os_ + dim
+            out_shape = (out_size,)
+        freq_kw.pop("head_dim", None)
+        freqs, scale, hd = self.rope_frequencies(dim, head_dim=dim, **freq_kw)
+        d_x, d_p, d_f = self.to_device(x), self.to_device(pos), self.to_device(freqs)
+        d_o = d_x if in_place else self.to_device(np.full(out_size, np.nan, dtype=x.dtype))
+        arg = capi.Rope(d_p.ptr, pos_dt, d_f.ptr, scale, hd, rope_type, 0, 0)
+        try:
+            check(self.lib.marmot_hip_rope(self.dev, C.c_void_p(d_x.ptr), _np_dtype_id(x.dtype), rows, dim, xs, os_,
+                                           C.byref(arg), C.c_void_p(d_o.ptr)))
+            return d_o.download(x.dtype, out_shape)
+        finally:
+            for b in {d_x, d_p, d_f, d_o}:
+                b.free()
+
     def packed_activation_layout(self, kind: int, N: int, K: int) -> "capi.PackedLayout":
         lay = capi.PackedLayout()
         check(self.lib.marmot_hip_packed_activation_layout(kind, N, K, C.byref(lay)))

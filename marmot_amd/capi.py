@@ -121,6 +121,7 @@ SIGNATURES = {
     "marmot_hip_glu": (_i, [_vp, _i, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
     "marmot_hip_swiglu_pack": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
     "marmot_hip_add": (_i, [_vp, _vp, _vp, _sz, _vp]),
+    "marmot_hip_rope": (_i, [_vp, _vp, _i, _sz, _sz, _sz, _sz, C.POINTER(Rope), _vp]),
     "marmot_hip_topk": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
     "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "marmot_hip_moe_experts": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i,

@@ -297,6 +297,20 @@ static marmot_error_t acquire_write(hip_backend_t *b, void *host, size_t n, void
     return MARMOT_SUCCESS;
 }
 
+// device address of a kernel output whose rows lie further apart than their length: the bytes between the rows are
+// not written by the kernel and must survive the next download of the range, so the host's bytes go up first
+// whenever the device does not hold them yet
+static marmot_error_t acquire_write_rows(hip_backend_t *b, void *host, size_t span, bool gaps, void **d_out) {
+    if (gaps) {
+        const void *unused = nullptr;
+        const marmot_error_t st = acquire_read(b, host, span, &unused);
+        if (st != MARMOT_SUCCESS) {
+            return st;
+        }
+    }
+    return acquire_write(b, host, span, d_out);
+}
+
 // ------------------------------------------------------------------ tensor helpers
 static size_t dtype_size(marmot_dtype_t t) {
     switch (t) {
@@ -1468,8 +1482,7 @@ static marmot_error_t binary_f32(const void *device_ctx, hip_binary_op_t op, con
         st = acquire_read(b, c->data, strided_span_bytes(c), &d_c);
     }
     if (st == MARMOT_SUCCESS) {
-        // a row-strided output keeps the bytes between its rows: acquire_write uploads them when only the host has them
-        st = acquire_write(b, out->data, strided_span_bytes(out), &d_y);
+        st = acquire_write_rows(b, out->data, strided_span_bytes(out), !dense_contiguous(out), &d_y);
     }
     if (st == MARMOT_SUCCESS) {
         int rc;
@@ -1487,6 +1500,135 @@ static marmot_error_t binary_f32(const void *device_ctx, hip_binary_op_t op, con
             rc = marmot_hip_glu(b->dev, op == HIP_BIN_GEGLU ? MARMOT_HIP_FFN_GEGLU : MARMOT_HIP_FFN_SWIGLU,
                                 (const float *)d_a, (const float *)d_c, rows, cols, sa, sc, so, (float *)d_y);
         }
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
+// marmot_rope (cpu_rope and cpu_rope_validate, src/backends/cpu/ops/rope/rope_dispatch.c:18-88, 145-196): the last
+// dimension of x is rotated, one position per row of it; checks in the reference's order. FLOAT32 and FLOAT16 rows.
+// The dimensions before the last must lie at one stride from row to row (contiguous tensors, and 2-D views whose
+// rows are further apart than their length), which is what the kernel walks.
+static bool rows_at_one_stride(const marmot_tensor_t *t, size_t *row_stride_out) {
+    const size_t nd = t->shape.ndim;
+    const size_t row_stride = t->shape.strides[nd - 2];
+    for (size_t i = nd - 2; i > 0; --i) {
+        if (t->shape.shape[i - 1] != 1 && t->shape.strides[i - 1] != t->shape.strides[i] * t->shape.shape[i]) {
+            return false;
+        }
+    }
+    *row_stride_out = row_stride;
+    return true;
+}
+
+static marmot_error_t rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
+                           marmot_tensor_t *out) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RoPE: null device context");
+    }
+    if (params == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RoPE parameters are null");
+    }
+    const marmot_tensor_t *positions = params->positions;
+    if (positions == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RoPE parameters require positions tensor");
+    }
+    if (x == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null pointer in RoPE");
+    }
+    const marmot_dtype_t dtype = x->dtype;
+    const bool reference_dtype = dtype == MARMOT_DTYPE_FLOAT32 || dtype == MARMOT_DTYPE_FLOAT64 ||
+        dtype == MARMOT_DTYPE_FLOAT16 || dtype == MARMOT_DTYPE_BFLOAT16;
+    if (!reference_dtype || out->dtype != dtype) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "RoPE dtype not supported");
+    }
+    if (x->shape.ndim < 2) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RoPE requires at least 2D tensor");
+    }
+    const size_t ndim = x->shape.ndim;
+    const size_t dim = x->shape.shape[ndim - 1];
+    if (dim % 2 != 0) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RoPE requires even dimension");
+    }
+    const size_t total = tensor_numel(x);
+    if (x->shape.shape[ndim - 2] == 0 || dim == 0 || total == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RoPE input tensor must be non-empty");
+    }
+    const size_t rows = total / dim;
+    if (tensor_numel(positions) != rows) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RoPE positions shape mismatch");
+    }
+    if (out->shape.ndim != ndim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RoPE output shape mismatch");
+    }
+    for (size_t i = 0; i < ndim; ++i) {
+        if (out->shape.shape[i] != x->shape.shape[i]) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RoPE output shape mismatch");
+        }
+    }
+    if (positions->dtype != MARMOT_DTYPE_FLOAT32 && positions->dtype != MARMOT_DTYPE_INT32 &&
+        positions->dtype != MARMOT_DTYPE_INT64) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "RoPE positions tensor must be FLOAT32, INT32, or INT64");
+    }
+    if (x->shape.strides[ndim - 1] != 1 || out->shape.strides[ndim - 1] != 1) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "RoPE requires contiguous inner dimension");
+    }
+    if (x->shape.strides[ndim - 2] < dim || out->shape.strides[ndim - 2] < dim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "RoPE requires row strides >= feature dimension");
+    }
+    if (dtype != MARMOT_DTYPE_FLOAT32 && dtype != MARMOT_DTYPE_FLOAT16) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP RoPE handles FLOAT32 and FLOAT16 tensors");
+    }
+    if (params->rope_type != MARMOT_ROPE_TYPE_NORM && params->rope_type != MARMOT_ROPE_TYPE_NEOX) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RoPE: unknown rope type");
+    }
+    size_t x_stride = 0, out_stride = 0;
+    if (!rows_at_one_stride(x, &x_stride) || !rows_at_one_stride(out, &out_stride) || !dense_contiguous(positions)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP RoPE needs rows at one stride and contiguous positions");
+    }
+    if (x->data == nullptr || out->data == nullptr || positions->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "RoPE: tensor without data");
+    }
+    const size_t elt = dtype_size(dtype);
+    const size_t x_span = ((rows - 1) * x_stride + dim) * elt, out_span = ((rows - 1) * out_stride + dim) * elt;
+    marmot_rope_params_t keyed = *params;  // the frequencies are those of the rotated dimension (rope.c:143-200)
+    keyed.head_dim = (uint32_t)dim;
+    pthread_mutex_lock(&b->mu);
+    hip_rope_entry_t *e = nullptr;
+    marmot_error_t st = rope_entry_locked(b, &keyed, dim, &e);
+    const void *d_x = nullptr, *d_pos = nullptr, *d_freqs = nullptr;
+    void *d_y = nullptr;
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, x->data, x_span, &d_x);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, positions->data, dense_bytes(positions), &d_pos);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, e->freqs, dim / 2 * sizeof(float), &d_freqs);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write_rows(b, out->data, out_span, out_stride != dim, &d_y);
+    }
+    if (st == MARMOT_SUCCESS) {
+        const marmot_hip_rope_t r = {
+            .d_positions = d_pos,
+            .positions_dtype = positions->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32
+                : positions->dtype == MARMOT_DTYPE_INT32               ? MARMOT_HIP_DTYPE_I32
+                                                                       : MARMOT_HIP_DTYPE_I64,
+            .d_freqs = d_freqs,
+            .attn_scale = e->attn_scale,
+            .head_dim = e->head_dim,
+            .rope_type = params->rope_type == MARMOT_ROPE_TYPE_NEOX ? 1 : 0,
+        };
+        const int rc = marmot_hip_rope(b->dev, d_x, dtype == MARMOT_DTYPE_FLOAT16 ? MARMOT_HIP_DTYPE_F16
+                                                                                   : MARMOT_HIP_DTYPE_F32,
+                                       rows, dim, x_stride, out_stride, &r, d_y);
         st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
     }
     pthread_mutex_unlock(&b->mu);
@@ -1794,6 +1936,37 @@ static marmot_error_t bc_exec_add(const void *exec_ctx, marmot_tensor_t **regs, 
     return bc_exec_binary(HIP_BIN_ADD, exec_ctx, regs, imm);
 }
 
+// ROPE: u16 input, output, positions (0xFFFF: the positions of the parameters); u32 rope-params const offset;
+// u32 n_past; u32 n_rot (bytecode_compile.c:598-623; bytecode_exec_cpu.gen.c:41088-41119). n_past and n_rot are
+// carried but not read by the operation (rope_dispatch.c:145-372).
+static marmot_error_t bc_exec_rope(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                   const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *x = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    const uint16_t positions_idx = rd_u16(&pc);
+    const uint32_t params_off = rd_u32(&pc);
+    marmot_rope_params_t params;
+    const marmot_rope_params_t *params_ptr = nullptr;
+    if (params_off != MARMOT_BC_INVALID_OFFSET) {
+        if (const_pool == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for rope params");
+        }
+        memcpy(&params, const_pool + params_off, sizeof(params));
+        params_ptr = &params;
+    }
+    if (positions_idx != MARMOT_BC_REG_INVALID) {
+        if (params_ptr == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Missing rope params");
+        }
+        params.positions = regs[positions_idx];
+    }
+    return rope(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, x, params_ptr, out);
+}
+
 static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     0,               // END
     12, 12, 12, 12,  // MATMUL: 3 x u16 + u32 + u16
@@ -1812,6 +1985,7 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     12, 26, 28, 21,  // Q8_1
     12, 12,          // RMS_NORM, RMS_NORM_GEMMA: 4 x u16 + f32
     6, 6, 6,         // SWIGLU, GEGLU, ADD (BINARY): 3 x u16
+    18,              // ROPE: 3 x u16 + 3 x u32
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1832,6 +2006,7 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_MATMUL,      MARMOT_BC_SCHEMA_MOE_EXPERTS, MARMOT_BC_SCHEMA_QKV, MARMOT_BC_SCHEMA_EMBEDDING,
     MARMOT_BC_SCHEMA_RMS_NORM,    MARMOT_BC_SCHEMA_RMS_NORM,
     MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,
+    MARMOT_BC_SCHEMA_ROPE,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -1850,6 +2025,7 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_matmul_q8_1, bc_exec_moe,         bc_exec_qkv_q8_1,    bc_exec_embedding,
     bc_exec_rms_norm,    bc_exec_rms_norm_gemma,
     bc_exec_swiglu,      bc_exec_geglu,       bc_exec_add,
+    bc_exec_rope,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -2081,6 +2257,12 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         return selected(sig->op_id == MARMOT_OP_SWIGLU  ? MARMOT_HIP_BC_OP_SWIGLU_F32
                         : sig->op_id == MARMOT_OP_GEGLU ? MARMOT_HIP_BC_OP_GEGLU_F32
                                                         : MARMOT_HIP_BC_OP_ADD_F32, launch_us, 0.0);
+    case MARMOT_OP_ROPE:
+        // rope_scalar (cpu/kernels/rope.def): rows and result of one type, FLOAT32 or FLOAT16
+        if (!((in32 && out32) || (in16 && out16))) {
+            return unsupported("HIP RoPE handles FLOAT32 and FLOAT16 tensors");
+        }
+        return selected(MARMOT_HIP_BC_OP_ROPE, launch_us, 0.0);
     case MARMOT_OP_TOPK:
         if (!in32 || !out32) {
             return unsupported("HIP TopK takes FLOAT32 values");
@@ -2286,6 +2468,10 @@ marmot_error_t hip_geglu_f32(const void *device_ctx, const marmot_tensor_t *a, c
 marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
                            marmot_tensor_t *out) {
     return binary_f32(device_ctx, HIP_BIN_ADD, a, b, out);
+}
+marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
+                        marmot_tensor_t *out) {
+    return rope(device_ctx, x, params, out);
 }
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
     return quantize_block(device_ctx, input, output);

@@ -40,9 +40,11 @@ BACKEND_HIP = 3
 OP_DEQUANTIZE, OP_MOE_EXPERTS, OP_MATMUL, OP_QUANTIZE, OP_LINEAR, OP_TOPK = 210, 263, 498, 524, 708, 901
 OP_QKV_PROJECTION, OP_QKV_SHARED_INPUT, OP_QKV_ROPE = 191, 771, 778
 OP_EMBEDDING = 853
+OP_ROPE = 843
 OP_SWIGLU, OP_GEGLU, OP_RMS_NORM_GEMMA, OP_ADD, OP_RMS_NORM = 331, 410, 447, 876, 929
 # this backend's bytecode ops for them (include/marmot_hip_backend.h)
 BC_OP_RMS_NORM_F32, BC_OP_RMS_NORM_GEMMA_F32, BC_OP_SWIGLU_F32, BC_OP_GEGLU_F32, BC_OP_ADD_F32 = 48, 49, 50, 51, 52
+BC_OP_ROPE = 53
 PREFERENCE_DEFAULT, PREFERENCE_ENABLE, PREFERENCE_DISABLE = 0, 1, 2
 QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q4_1: 2, KIND_Q5_0: 3, KIND_Q5_1: 4, KIND_Q8_0: 5, KIND_Q2_K: 6, KIND_Q3_K: 7, KIND_Q4_K: 8,
@@ -263,6 +265,7 @@ BACKEND_SYMBOLS = [
     "hip_matmul_qkv_q5_k", "hip_matmul_qkv_q6_k", "hip_embedding_gather", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
     "hip_rmsnorm_impl", "hip_rmsnorm_gemma_impl", "hip_swiglu_f32", "hip_geglu_f32", "hip_add_f32",
+    "hip_rope",
 ]
 
 
@@ -303,6 +306,8 @@ def bind(lib: C.CDLL) -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]
+    lib.hip_rope.restype = C.c_int
+    lib.hip_rope.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(RopeParams), C.POINTER(Tensor)]
     lib.marmot_hip_backend_last_error.restype = C.c_int
     lib.marmot_hip_backend_last_error.argtypes = [C.POINTER(C.c_char_p)]
     lib.marmot_hip_backend_residency_stats.restype = None
@@ -569,6 +574,17 @@ class Program:
 
     def binary(self, op_index: int, a, b, out):
         self.code += struct.pack("<HHHH", op_index, self.reg(a), self.reg(b), self.reg(out))
+
+    def rope(self, op_index: int, x, out, params: Optional[RopeParams], positions: Optional[HostTensor] = None,
+             n_past: int = 0, n_rot: int = 0):
+        """bytecode_compile.c:598-623: the parameters travel in the constant pool; a positions register replaces
+        the tensor they name."""
+        off = BC_INVALID_OFFSET
+        if params is not None:
+            self._keep.append(params)
+            off = self._const(bytes(params), 8)
+        self.code += struct.pack("<HHHHIII", op_index, self.reg(x), self.reg(out), self.reg(positions), off, n_past,
+                                 n_rot)
 
     def quantize(self, op_index: int, x, out):
         self.code += struct.pack("<HHIHII", op_index, self.reg(x), BC_INVALID_OFFSET, self.reg(out),

@@ -24,6 +24,7 @@
 #define MO_OK 0
 #define MO_ERR_INVALID_ARGUMENT (-1)
 #define MO_ERR_OUT_OF_MEMORY (-2)
+#define MO_ERR_DIMENSION_MISMATCH (-7)
 #define MO_ERR_INVALID_OPERATION (-5)
 #define MO_ERR_UNSUPPORTED_DTYPE (-6)
 #define MO_ERR_NOT_IMPLEMENTED (-8)
@@ -2443,6 +2444,83 @@ void mo_rope_rotate_row(float *row, size_t dim, size_t head_dim, float position,
     for (size_t h = 0; h < head_count; ++h) {
         rope_rotate_head(row + h * head_dim, head_dim, position, freqs, attn_scale, rope_type);
     }
+}
+
+/* cpu_rope, scalar path (src/backends/cpu/ops/rope/rope_dispatch.c:145-196, 287-372): rows of `dim` values, one
+ * position per row, values loaded as fp32, rotated in fp32 and rounded once by the store */
+int mo_rope(
+    const void *x, int dtype, size_t rows, size_t dim, size_t x_row_stride, size_t out_row_stride,
+    const mo_rope_params *rope, const void *positions, int pos_dtype, void *out
+) {
+    if (x == NULL || out == NULL || rope == NULL || positions == NULL) {
+        return MO_ERR_INVALID_ARGUMENT; /* :147-155, 22-25 */
+    }
+    if (dtype != MO_DTYPE_F32 && dtype != MO_DTYPE_F16) {
+        return MO_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (dim % 2 != 0) {
+        return MO_ERR_DIMENSION_MISMATCH; /* :45-49 */
+    }
+    if (rows == 0 || dim == 0) {
+        return MO_ERR_INVALID_ARGUMENT; /* :51-56 */
+    }
+    if (pos_dtype != MO_DTYPE_F32 && pos_dtype != MO_DTYPE_I32 && pos_dtype != MO_DTYPE_I64) {
+        return MO_ERR_UNSUPPORTED_DTYPE; /* :164-168 */
+    }
+    if (x_row_stride < dim || out_row_stride < dim) {
+        return MO_ERR_DIMENSION_MISMATCH; /* :183-186 */
+    }
+    const size_t half = dim / 2;
+    float *freqs = (float *)malloc(half * sizeof(float));
+    if (freqs == NULL) {
+        return MO_ERR_OUT_OF_MEMORY;
+    }
+    float attn_scale = 1.0f;
+    const int st = mo_rope_frequencies(rope, dim, freqs, &attn_scale); /* cpu_rope_prepare_freqs (:123-143) */
+    if (st != MO_OK) {
+        free(freqs);
+        return st;
+    }
+    const int is_neox = rope->rope_type == 1;
+    for (size_t token = 0; token < rows; ++token) {
+        float pos; /* cpu_rope_position_as_f32 (cpu_backend_internal.h:567-578) */
+        if (pos_dtype == MO_DTYPE_F32) {
+            pos = ((const float *)positions)[token];
+        } else if (pos_dtype == MO_DTYPE_I32) {
+            pos = (float)((const int32_t *)positions)[token];
+        } else {
+            pos = (float)((const int64_t *)positions)[token];
+        }
+        const size_t base_in = token * x_row_stride, base_out = token * out_row_stride;
+        for (size_t i = 0; i < half; ++i) { /* :343-367 */
+            const float angle = pos * freqs[i];
+            float sin_theta = sinf(angle);
+            float cos_theta = cosf(angle);
+            cos_theta *= attn_scale;
+            sin_theta *= attn_scale;
+            const size_t even_offset = is_neox ? i : 2 * i;
+            const size_t odd_offset = is_neox ? (i + half) : (2 * i + 1);
+            float x_even, x_odd;
+            if (dtype == MO_DTYPE_F16) {
+                x_even = mo_f16_to_f32(((const uint16_t *)x)[base_in + even_offset]);
+                x_odd = mo_f16_to_f32(((const uint16_t *)x)[base_in + odd_offset]);
+            } else {
+                x_even = ((const float *)x)[base_in + even_offset];
+                x_odd = ((const float *)x)[base_in + odd_offset];
+            }
+            const float rotated_even = x_even * cos_theta - x_odd * sin_theta;
+            const float rotated_odd = x_even * sin_theta + x_odd * cos_theta;
+            if (dtype == MO_DTYPE_F16) {
+                ((uint16_t *)out)[base_out + even_offset] = mo_f32_to_f16(rotated_even);
+                ((uint16_t *)out)[base_out + odd_offset] = mo_f32_to_f16(rotated_odd);
+            } else {
+                ((float *)out)[base_out + even_offset] = rotated_even;
+                ((float *)out)[base_out + odd_offset] = rotated_odd;
+            }
+        }
+    }
+    free(freqs);
+    return MO_OK;
 }
 
 /* matmul_qkv.c:749-947 (cpu_matmul_qkv_run_separate_quantized_impl), value load/store helpers :89-116 */

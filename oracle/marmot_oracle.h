@@ -152,6 +152,18 @@ void mo_rope_rotate_row(float *row, size_t dim, size_t head_dim, float position,
                         int rope_type);
 
 /*
+ * marmot_rope on rows (cpu_rope, src/backends/cpu/ops/rope/rope_dispatch.c:145-372, scalar path): x and out hold
+ * `rows` rows of `dim` values of dtype (MO_DTYPE_F32 or MO_DTYPE_F16) at the given row strides (in elements, >= dim);
+ * row r is rotated by positions[r] with the frequencies of mo_rope_frequencies(rope, dim); rope->head_dim and the
+ * apply flags play no part. x == out is allowed. Pinned by the closed form and the inputs of the reference's own test
+ * (tests/backend/test_rope.c:5-42, 44-118).
+ */
+int mo_rope(
+    const void *x, int dtype, size_t rows, size_t dim, size_t x_row_stride, size_t out_row_stride,
+    const mo_rope_params *rope, const void *positions, int pos_dtype, void *out
+);
+
+/*
  * mo_matmul_qkv_separate with the rotary epilogue (matmul_qkv.c:812-822, 829-831, 917-925, 700-747): q and/or k rows
  * are rotated in fp32 before the store. positions: N values of pos_dtype (MO_DTYPE_F32, MO_DTYPE_I32 or
  * MO_DTYPE_I64), converted to float as cpu_rope_position_as_f32 does (cpu_backend_internal.h:567-578).

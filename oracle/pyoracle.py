@@ -111,6 +111,9 @@ class Oracle:
         L.mo_rope_frequencies.argtypes = [C.POINTER(RopeParams), C.c_size_t, C.c_void_p, C.POINTER(C.c_float)]
         L.mo_rope_resolve_head_dim.restype = C.c_size_t
         L.mo_rope_resolve_head_dim.argtypes = [C.c_size_t, C.c_uint32]
+        L.mo_rope.restype = C.c_int
+        L.mo_rope.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t,
+                              C.POINTER(RopeParams), C.c_void_p, C.c_int, C.c_void_p]
         L.mo_rope_rotate_row.restype = None
         L.mo_rope_rotate_row.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, C.c_void_p, C.c_float, C.c_int]
         L.mo_embedding_gather_quantized.restype = C.c_int
@@ -248,6 +251,29 @@ class Oracle:
         freqs = np.ascontiguousarray(freqs, dtype=np.float32)
         self.L.mo_rope_rotate_row(_ptr(out), out.shape[0], head_dim, position, _ptr(freqs), attn_scale, rope_type)
         return out
+
+    def rope(self, x: np.ndarray, positions: np.ndarray, rope: "RopeParams", dim=None, x_row_stride=None,
+             out_row_stride=None):
+        """marmot_rope: the last dimension of x (float32 or float16, rank >= 2) is rotated, one position (float32,
+        int32 or int64) per row; `rope.head_dim` is not used. With `dim` and row strides (in elements), x is a flat
+        buffer holding positions.size rows of dim values at x_row_stride and the result a flat buffer of rows at
+        out_row_stride (the gaps hold NaN). Returns (status, out)."""
+        assert x.dtype in (np.float32, np.float16)
+        x = np.ascontiguousarray(x)
+        pos = np.ascontiguousarray(positions)
+        pos_dt = {np.dtype(np.float32): DT_F32, np.dtype(np.int32): DT_I32, np.dtype(np.int64): DT_I64}[pos.dtype]
+        dt = DT_F16 if x.dtype == np.float16 else DT_F32
+        if dim is None:
+            dim = x.shape[-1]
+            rows = x.size // dim if dim else 0
+            out = np.full(x.shape, np.nan, dtype=x.dtype)
+            xs = os_ = dim
+        else:
+            rows, xs, os_ = pos.size, x_row_stride, out_row_stride
+            assert x.ndim == 1 and (rows == 0 or x.size >= (rows - 1) * xs + dim)
+            out = np.full(max(rows - 1, 0) * os_ + dim, np.nan, dtype=x.dtype)
+        st = self.L.mo_rope(_ptr(x), dt, rows, dim, xs, os_, C.byref(rope), _ptr(pos), pos_dt, _ptr(out))
+        return st, out
 
     def matmul_qkv(self, kind: int, wq, wk, wv, x: np.ndarray, M: int, bq=None, bk=None, bv=None, rope=None,
                    positions=None):

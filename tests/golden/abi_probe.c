@@ -63,6 +63,7 @@ int main(void) {
     VAL(MARMOT_BC_REG_INVALID); VAL(MARMOT_BC_INVALID_OFFSET); VAL(MARMOT_BC_END);
     VAL(MARMOT_OP_RMS_NORM); VAL(MARMOT_OP_RMS_NORM_GEMMA); VAL(MARMOT_OP_SWIGLU); VAL(MARMOT_OP_GEGLU); VAL(MARMOT_OP_ADD);
     VAL(MARMOT_BC_SCHEMA_RMS_NORM); VAL(MARMOT_BC_SCHEMA_BINARY);
+    VAL(MARMOT_OP_ROPE); VAL(MARMOT_BC_SCHEMA_ROPE);
 
     SZ(marmot_shape_t); OFF(marmot_shape_t, ndim); OFF(marmot_shape_t, shape); OFF(marmot_shape_t, strides);
     SZ(marmot_quant_params_t);

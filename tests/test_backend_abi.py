@@ -212,6 +212,10 @@ def test_query_kernel_other_ops(lib):
     assert not _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_K, inp=ta.DTYPE_F16)).supported
     assert not _query(lib, _sig(op=ta.OP_QUANTIZE, kind=ta.KIND_Q4_0)).supported
     assert _query(lib, _sig(op=ta.OP_DEQUANTIZE, kind=ta.KIND_Q6_K)).op_index == 11
+    # rope: rows and result of one type, FLOAT32 or FLOAT16
+    assert _query(lib, _sig(op=ta.OP_ROPE, kind=ta.KIND_GENERIC)).op_index == ta.BC_OP_ROPE
+    assert _query(lib, _sig(op=ta.OP_ROPE, kind=ta.KIND_GENERIC, inp=ta.DTYPE_F16, out=ta.DTYPE_F16)).op_index == 53
+    assert not _query(lib, _sig(op=ta.OP_ROPE, kind=ta.KIND_GENERIC, inp=ta.DTYPE_F16, out=ta.DTYPE_F32)).supported
     assert not _query(lib, _sig(op=12345)).supported
 
 
@@ -283,7 +287,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 53
+    assert t.op_count == 54
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -315,6 +319,9 @@ def test_bytecode_tables(lib, golden_layout):
     assert sizes[48:50] == [struct.calcsize("<4Hf")] * 2 and sizes[50:53] == [struct.calcsize("<3H")] * 3
     assert (ta.BC_OP_RMS_NORM_F32, ta.BC_OP_RMS_NORM_GEMMA_F32, ta.BC_OP_SWIGLU_F32, ta.BC_OP_GEGLU_F32,
             ta.BC_OP_ADD_F32) == (48, 49, 50, 51, 52)
+    # the rotary embedding: input, output and positions registers, parameter offset, n_past, n_rot
+    assert schema[53] == golden_layout["MARMOT_BC_SCHEMA_ROPE"] and sizes[53] == struct.calcsize("<3H3I") == 18
+    assert ta.BC_OP_ROPE == 53 and ta.OP_ROPE == golden_layout["MARMOT_OP_ROPE"]
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -358,6 +365,12 @@ def test_program_encoding_matches_reference_immediates():
     rp.theta, rp.apply_to_q = 10000.0, True
     q.qkv(14, x, w, w, w, *outs, rope=rp)
     assert struct.unpack_from("<I", q.code, 30 + 2 + 14 + 4)[0] == 0 and len(q.const_pool) == C.sizeof(ta.RopeParams)
+    # ROPE: input, output, positions register (absent: the tensor the parameters name), offset, n_past, n_rot
+    r = ta.Program()
+    r.rope(53, x, y, rp)
+    assert bytes(r.code) == struct.pack("<HHHHIII", 53, 0, 1, 0xFFFF, 0, 0, 0)
+    r.rope(53, x, y, rp, positions=b, n_past=7, n_rot=64)
+    assert struct.unpack_from("<HHHHIII", r.code, 20) == (53, 0, 1, 2, C.sizeof(ta.RopeParams), 7, 64)
     # EMBEDDING: table, ids, out; output dtype, scale, padding id, three flag bytes
     e = ta.Program()
     ids = ta.HostTensor.dense(np.zeros((2, 3), np.int64))
@@ -380,7 +393,7 @@ def test_kernel_def_files_name_exported_impls(lib):
     assert set(families) == {"matmul_quantized_hip", "topk_hip",
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
                              "embedding_quantized_hip", "rms_norm_hip", "rms_norm_gemma_hip", "glu_hip",
-                             "add_hip"} | qkv
+                             "add_hip", "rope_hip"} | qkv
     for name in qkv:
         f = families[name]
         assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name

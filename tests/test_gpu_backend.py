@@ -592,6 +592,141 @@ def test_impl_and_program_float_ops(ctx, oracle):
         ctx.host_freed(t)
 
 
+def _rope_params(pos_t, **kw):
+    rp = ta.RopeParams()
+    rp.positions = pos_t.ptr if pos_t is not None else None
+    rp.scaling_type, rp.rope_type, rp.theta, rp.freq_scale, rp.ext_factor, rp.attn_factor = 0, 0, 10000.0, 1.0, 0.0, 1.0
+    rp.beta_fast, rp.beta_slow, rp.orig_ctx_len, rp.head_dim = 32.0, 1.0, 0, 0
+    for k, v in kw.items():
+        setattr(rp, k, v)
+    return rp
+
+
+def test_impl_and_program_rope(ctx, oracle):
+    """hip_rope (rank 3, FLOAT32 and FLOAT16, NORM and NEOX, the three position types, in place, row-strided views),
+    its query and bytecode op with and without a positions register, and cpu_rope's error order."""
+    from oracle.pyoracle import RopeParams as OracleRope
+    from tests.test_gpu_ops import rope_close
+
+    x = gaussian(1300, (2, 9, 128))
+    pos = (np.arange(18, dtype=np.int32).reshape(2, 9) * 113) % 4096
+    for np_dt, dt in ((np.float32, ta.DTYPE_F32), (np.float16, ta.DTYPE_F16)):
+        xv = x.astype(np_dt)
+        xt, ot = ta.HostTensor.dense(xv), ta.HostTensor.empty((2, 9, 128), dt)
+        for p in (pos, pos.astype(np.int64), pos.astype(np.float32) + np.float32(0.25)):
+            pt = ta.HostTensor.dense(p)
+            for rope_type in (0, 1):
+                rp = _rope_params(pt, rope_type=rope_type, theta=500000.0)
+                assert ctx.lib.hip_rope(ctx.device_ctx, xt.ptr, C.byref(rp), ot.ptr) == ta.SUCCESS, ctx.last_error()
+                st, ref = oracle.rope(xv, p, OracleRope.default(theta=500000.0, rope_type=rope_type))
+                rope_close(ctx.to_host(ot), ref, xv, f"hip_rope {np_dt.__name__} {p.dtype} type {rope_type}")
+            ctx.host_freed(pt)
+        sel = ctx.query(ctx.float_op_signature(ta.OP_ROPE, dt))
+        assert sel.supported and sel.op_index == ta.BC_OP_ROPE
+        # the program: parameters in the constant pool; a positions register replaces the tensor they name
+        pt, pt2 = ta.HostTensor.dense(pos), ta.HostTensor.dense(pos + 5)
+        rp = _rope_params(pt, theta=10000.0, scaling_type=1, freq_scale=0.5, attn_factor=1.25)
+        oracle_rp = OracleRope.default(theta=10000.0, scaling_type=1, freq_scale=0.5, attn_factor=1.25)
+        prog = ta.Program()
+        prog.rope(sel.op_index, xt, ot, rp)
+        assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+        rope_close(ctx.to_host(ot), oracle.rope(xv, pos, oracle_rp)[1], xv, "program rope")
+        prog = ta.Program()
+        prog.rope(sel.op_index, xt, ot, rp, positions=pt2, n_past=5, n_rot=128)
+        assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+        rope_close(ctx.to_host(ot), oracle.rope(xv, pos + 5, oracle_rp)[1], xv, "program rope, positions register")
+        prog = ta.Program()
+        prog.rope(sel.op_index, xt, ot, None, positions=pt2)
+        assert ctx.execute(prog) == ta.INVALID_ARGUMENT  # a positions register without parameters
+        # in place
+        it = ta.HostTensor.dense(xv.copy())
+        rp = _rope_params(pt)
+        assert ctx.lib.hip_rope(ctx.device_ctx, it.ptr, C.byref(rp), it.ptr) == ta.SUCCESS, ctx.last_error()
+        rope_close(ctx.to_host(it), oracle.rope(xv, pos, OracleRope.default())[1], xv, "in place")
+        for t in (xt, ot, pt, pt2, it):
+            ctx.host_freed(t)
+
+    # row-strided views: q is the first 128 columns of a [rows, 384] projection output, rotated into the first 128
+    # columns of another; the other columns of the output keep what the host wrote there
+    rows = 12
+    both, dst = gaussian(1301, (rows, 384)), gaussian(1302, (rows, 384))
+    whole_in, whole_out = ta.HostTensor.dense(both), ta.HostTensor.dense(dst)
+    views = []
+    for whole in (whole_in, whole_out):
+        v = ta.HostTensor.dense(both)
+        v.array = whole.array
+        v.t.data = whole.t.data
+        v.t.shape.shape[1] = 128
+        v.t.shape.strides[0] = 384
+        views.append(v)
+    p = np.arange(rows, dtype=np.int32) * 7
+    pt = ta.HostTensor.dense(p)
+    rp = _rope_params(pt, rope_type=1)
+    assert ctx.lib.hip_rope(ctx.device_ctx, views[0].ptr, C.byref(rp), views[1].ptr) == ta.SUCCESS, ctx.last_error()
+    got = ctx.to_host(views[1]).reshape(rows, 384)
+    rope_close(got[:, :128], oracle.rope(both[:, :128], p, OracleRope.default(rope_type=1))[1], both, "strided rope")
+    assert np.array_equal(got[:, 128:], dst[:, 128:])
+    # the same for a gated product written into a row-strided half
+    g, u = gaussian(1303, (rows, 128)), gaussian(1304, (rows, 128))
+    dst2 = gaussian(1305, (rows, 384))
+    whole2 = ta.HostTensor.dense(dst2)
+    v2 = ta.HostTensor.dense(dst2)
+    v2.array = whole2.array
+    v2.t.data = whole2.t.data
+    v2.t.shape.shape[1] = 128
+    v2.t.shape.strides[0] = 384
+    gt, ut = ta.HostTensor.dense(g), ta.HostTensor.dense(u)
+    # the gated products want all three operands row-strided or all contiguous: narrow views of wider buffers
+    gv, uv = [], []
+    for src, keep in ((g, gv), (u, uv)):
+        wide = ta.HostTensor.dense(np.concatenate([src, np.zeros((rows, 64), np.float32)], axis=1))
+        wide.t.shape.shape[1] = 128
+        keep.append(wide)
+    assert ctx.lib.hip_swiglu_f32(ctx.device_ctx, gv[0].ptr, uv[0].ptr, v2.ptr) == ta.SUCCESS, ctx.last_error()
+    got2 = ctx.to_host(v2).reshape(rows, 384)
+    assert np.allclose(got2[:, :128], oracle.glu(g, u), rtol=1e-5, atol=1e-7)
+    assert np.array_equal(got2[:, 128:], dst2[:, 128:])
+
+    # errors, in cpu_rope's order (rope_dispatch.c:18-88, 145-188)
+    xt, ot = ta.HostTensor.dense(x), ta.HostTensor.empty((2, 9, 128), ta.DTYPE_F32)
+    good = _rope_params(pt)
+    full = ta.HostTensor.dense(pos)
+    rp = _rope_params(full)
+    lib, dc = ctx.lib, ctx.device_ctx
+    assert lib.hip_rope(dc, xt.ptr, None, ot.ptr) == ta.INVALID_ARGUMENT
+    assert lib.hip_rope(dc, xt.ptr, C.byref(_rope_params(None)), ot.ptr) == ta.INVALID_ARGUMENT
+    assert lib.hip_rope(dc, None, C.byref(rp), ot.ptr) == ta.INVALID_ARGUMENT
+    o16 = ta.HostTensor.empty((2, 9, 128), ta.DTYPE_F16)
+    assert lib.hip_rope(dc, xt.ptr, C.byref(rp), o16.ptr) == ta.UNSUPPORTED_DTYPE       # types differ
+    i32 = ta.HostTensor.dense(np.zeros((2, 9, 128), np.int32))
+    assert lib.hip_rope(dc, i32.ptr, C.byref(rp), i32.ptr) == ta.UNSUPPORTED_DTYPE
+    v1 = ta.HostTensor.dense(np.zeros(128, np.float32))
+    assert lib.hip_rope(dc, v1.ptr, C.byref(rp), v1.ptr) == ta.DIMENSION_MISMATCH       # rank 1
+    odd = ta.HostTensor.dense(np.zeros((18, 7), np.float32))
+    assert lib.hip_rope(dc, odd.ptr, C.byref(rp), odd.ptr) == ta.DIMENSION_MISMATCH     # odd dimension
+    empty = ta.HostTensor.dense(np.zeros((0, 8), np.float32))
+    assert lib.hip_rope(dc, empty.ptr, C.byref(rp), empty.ptr) == ta.INVALID_ARGUMENT
+    assert lib.hip_rope(dc, xt.ptr, C.byref(good), ot.ptr) == ta.DIMENSION_MISMATCH     # 12 positions for 18 rows
+    o2 = ta.HostTensor.empty((2, 9, 64), ta.DTYPE_F32)
+    assert lib.hip_rope(dc, xt.ptr, C.byref(rp), o2.ptr) == ta.DIMENSION_MISMATCH       # output shape
+    p16 = ta.HostTensor.dense(pos.astype(np.float16))
+    assert lib.hip_rope(dc, xt.ptr, C.byref(_rope_params(p16)), ot.ptr) == ta.UNSUPPORTED_DTYPE
+    tr = ta.HostTensor.dense(x)
+    tr.t.shape.strides[2], tr.t.shape.strides[1] = 2, 256
+    assert lib.hip_rope(dc, tr.ptr, C.byref(rp), ot.ptr) == ta.NOT_IMPLEMENTED          # inner stride
+    short = ta.HostTensor.dense(x)
+    short.t.shape.strides[1] = 64
+    assert lib.hip_rope(dc, short.ptr, C.byref(rp), ot.ptr) == ta.DIMENSION_MISMATCH    # row stride < dim
+    f64 = ta.HostTensor.dense(np.zeros((2, 9, 128), np.float32))
+    f64.t.dtype = 10  # MARMOT_DTYPE_FLOAT64: the reference rotates it, this backend declines
+    assert lib.hip_rope(dc, f64.ptr, C.byref(rp), f64.ptr) == ta.NOT_IMPLEMENTED
+    assert not ctx.query(ctx.float_op_signature(ta.OP_ROPE, 10)).supported
+    assert lib.hip_rope(dc, xt.ptr, C.byref(rp), ot.ptr) == ta.SUCCESS
+    for t in (whole_in, whole_out, pt, whole2, gt, ut, gv[0], uv[0], xt, ot, full, o16, i32, v1, odd, empty, o2, p16,
+              f64):
+        ctx.host_freed(t)
+
+
 def test_program_norm_feeds_linears_without_quantization_launches(ctx, oracle):
     """A decoder layer's feed-forward half at 16 tokens as one bytecode program: rms_norm -> gate, up (Q4_K) -> swiglu
     -> down (Q6_K) -> residual add. The normalization leaves its rows packed, gate and up both find them (no packing

@@ -134,3 +134,108 @@ def test_ops_argument_errors(hip):
     assert lib.marmot_hip_glu(dev, 0, d.ptr, d.ptr, 2, 8, 4, 8, 8, d.ptr) != 0       # stride shorter than a row
     assert lib.marmot_hip_add(dev, d.ptr, None, 4, d.ptr) == -1
     d.free()
+
+
+# ---------------------------------------------------------------- stand-alone rotary embedding
+# The device's sincosf and the C library's sinf / cosf agree to a few units in the last place of sin and cos, which
+# reach a result as |x| * 2^-23 each; a FLOAT16 result can then round to the neighbouring half value.
+def rope_close(got, ref, x, what):
+    g, r = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    scale = np.abs(np.asarray(x, np.float64)).max()
+    tol = 2e-6 * scale if np.asarray(got).dtype == np.float32 else 1.1e-3 * np.maximum(np.abs(r), 1e-3)
+    assert np.all(np.isfinite(g)) and np.all(np.abs(g - r) <= tol), f"{what}: {np.abs(g - r).max():.3e}"
+
+
+def test_rope_reference_test_cases(hip, oracle):
+    """The cases of the reference's own test (tests/backend/test_rope.c) at its tolerances."""
+    from tests.test_oracle_ops import rope_closed_form, rope_test_inputs
+    x, pos = rope_test_inputs()
+    for dtype, tol in ((np.float32, 1e-5), (np.float16, 4e-3)):
+        for rope_type in (0, 1):
+            got = hip.rope(x.astype(dtype), pos, rope_type=rope_type, theta=10000.0)
+            want = rope_closed_form(x.astype(dtype), pos, 10000.0, rope_type)
+            assert got.dtype == dtype and np.max(np.abs(got.astype(np.float64) - want)) <= tol, (dtype, rope_type)
+    ipos = np.rint(pos).astype(np.int32)
+    for p in (ipos, ipos.astype(np.int64)):
+        assert np.max(np.abs(hip.rope(x, p, theta=10000.0) - rope_closed_form(x, p, 10000.0, 0))) <= 1e-5
+    y = np.cos(np.arange(32, dtype=np.float32) * np.float32(0.09), dtype=np.float32).reshape(1, 4, 8)
+    assert np.array_equal(hip.rope(y, np.zeros((1, 4), np.float32), theta=10000.0), y)  # zero positions: identity
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_rope_matches_oracle(hip, oracle, dtype):
+    from oracle.pyoracle import RopeParams
+    x = gaussian(1200, (4, 33, 128)).astype(dtype)
+    cases = [(dict(theta=500000.0), np.arange(132, dtype=np.int32).reshape(4, 33) * 61),
+             (dict(theta=10000.0, scaling_type=1, freq_scale=0.25, attn_factor=1.5),
+              (np.arange(132, dtype=np.int64).reshape(4, 33) * 997) % 8192),
+             (dict(theta=10000.0, scaling_type=2, ext_factor=1.0, freq_scale=0.5, orig_ctx_len=4096, beta_fast=32.0,
+                   beta_slow=1.0), gaussian(1201, (4, 33), 300.0))]
+    for kw, pos in cases:
+        for rope_type in (0, 1):
+            st, ref = oracle.rope(x, pos, RopeParams.default(rope_type=rope_type, **kw))
+            assert st == 0
+            rope_close(hip.rope(x, pos, rope_type=rope_type, **kw), ref, x, f"{dtype.__name__} {kw} type {rope_type}")
+    # in place, and an odd number of rows of a width that is not a multiple of the workgroup
+    x2 = gaussian(1202, (7, 6)).astype(dtype)
+    p2 = np.array([0, 1, 5, 17, 4096, 100000, 3], np.int32)
+    st, ref = oracle.rope(x2, p2, RopeParams.default())
+    rope_close(hip.rope(x2, p2, in_place=True), ref, x2, "in place")
+    # row strides: input rows 160 apart, output rows 144 apart (even: paired accesses) and 145 / 131 apart (odd:
+    # single-element accesses); the gaps of the output keep their contents
+    rows = 21
+    xr = gaussian(1203, (rows, 128)).astype(dtype)
+    pr = (np.arange(rows, dtype=np.int32) * 37)
+    for xs, os_ in ((160, 144), (145, 131)):
+        flat = np.full((rows - 1) * xs + 128, 7.0, dtype)
+        for r in range(rows):
+            flat[r * xs:r * xs + 128] = xr[r]
+        for rope_type in (0, 1):
+            rp = RopeParams.default(theta=500000.0, rope_type=rope_type)
+            st, ref = oracle.rope(flat, pr, rp, dim=128, x_row_stride=xs, out_row_stride=os_)
+            got = hip.rope(flat, pr, rope_type=rope_type, theta=500000.0, dim=128, x_row_stride=xs, out_row_stride=os_)
+            assert st == 0 and np.array_equal(np.isnan(got), np.isnan(ref))
+            live = ~np.isnan(ref)
+            rope_close(got[live], ref[live], xr, f"strides {xs}/{os_} type {rope_type}")
+
+
+def test_rope_prefill_shape_and_invariants(hip, oracle):
+    """512 tokens x 32 heads x 128: the q rows of a prefill step, rotated in one launch; against the oracle on a slice
+    and through what a rotation fixes on the whole (pair norms kept, the inverse rotation restores the rows)."""
+    from oracle.pyoracle import RopeParams
+    T, Hh, D = 512, 32, 128
+    x = gaussian(1210, (T, Hh, D))
+    pos = np.repeat(np.arange(T, dtype=np.int32)[:, None] + 1000, Hh, axis=1)
+    for rope_type in (0, 1):
+        y = hip.rope(x, pos, rope_type=rope_type, theta=500000.0)
+        st, ref = oracle.rope(x[:16], pos[:16], RopeParams.default(theta=500000.0, rope_type=rope_type))
+        rope_close(y[:16], ref, x, f"prefill type {rope_type}")
+        pairs = (lambda v: np.stack([v[..., :D // 2], v[..., D // 2:]], -1)) if rope_type == 1 else \
+            (lambda v: v.reshape(v.shape[:-1] + (D // 2, 2)))
+        nx = np.linalg.norm(pairs(x.astype(np.float64)), axis=-1)
+        ny = np.linalg.norm(pairs(y.astype(np.float64)), axis=-1)
+        assert np.allclose(nx, ny, rtol=1e-5, atol=1e-6)
+        back = hip.rope(y, -pos, rope_type=rope_type, theta=500000.0)
+        assert np.max(np.abs(back - x)) <= 1e-5
+
+
+def test_rope_argument_errors(hip):
+    d = hip.to_device(np.zeros(1024, np.float32))
+    lib, dev = hip.lib, hip.dev
+    r = capi.Rope(d.ptr, capi.DT_I32, d.ptr, 1.0, 8, 0, 0, 0)
+    import ctypes as C
+    call = lambda *a: lib.marmot_hip_rope(dev, *a)
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 8, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == 0
+    assert call(None, capi.DT_F32, 2, 8, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == -1
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 8, 8, 8, None, C.c_void_p(d.ptr)) == -1
+    assert call(C.c_void_p(d.ptr), capi.DT_I32, 2, 8, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == -6
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 7, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == -7   # odd dimension
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 0, 8, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == -1   # empty
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 8, 6, 8, C.byref(r), C.c_void_p(d.ptr)) == -7   # stride < row
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 16, 16, 16, C.byref(r), C.c_void_p(d.ptr)) == -1  # 4 freqs for dim 16
+    r.positions_dtype = capi.DT_F16
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 8, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == -6
+    r.positions_dtype, r.d_positions = capi.DT_I32, None
+    assert call(C.c_void_p(d.ptr), capi.DT_F32, 2, 8, 8, 8, C.byref(r), C.c_void_p(d.ptr)) == -1
+    hip.synchronize()
+    d.free()

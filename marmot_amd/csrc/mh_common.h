@@ -215,6 +215,7 @@ struct ActScratch {
 //   MARMOT_HIP_NO_FUSED_QUANT  activation quantization inside the matvec -> separate quantization launch
 //   MARMOT_HIP_NO_GEMM         fp16 prefill GEMM -> fp16 matvec
 //   MARMOT_HIP_NO_GEMM_LOADERS prefill GEMM tile fed by loader wavefronts -> the tile whose wavefronts load for themselves
+//   MARMOT_HIP_NO_GEMM_I8      tiled int8 GEMM on Q8_K activations (48 rows and more) -> 32-row passes of the small-batch kernel
 //   MARMOT_HIP_MOE_NO_VALIDATE skip the read-back of the expert-id error flag (no stream synchronization per call)
 struct marmot_hip_knobs {
     bool no_mmq = false;
@@ -223,6 +224,7 @@ struct marmot_hip_knobs {
     bool no_fused_quant = false;
     bool no_gemm = false;
     bool no_gemm_loaders = false;
+    bool no_gemm_i8 = false;
     bool moe_no_validate = false;
 };
 
@@ -367,6 +369,12 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);
+// Tiled int8 GEMM on Q8_K activations (mh_gemm_i8.hip): Q4_K weights, 48 activation rows and more
+bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
+                     const ActScratch &act);
+size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, int weights);
+int launch_gemm_i8(marmot_hip_device *dev, const WeightSet &ws, const ActScratch &act, size_t N, size_t K, size_t M,
+                   int out_dtype, void *scratch);
 int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                    size_t M, int out_dtype, void *scratch);
 bool mmq_grouped_supported(const marmot_hip_device *dev, int kind, size_t K);

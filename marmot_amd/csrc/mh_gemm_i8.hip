@@ -1,0 +1,444 @@
+// Prefill with fp32 activations: Q4_K weights x Q8_K activations as a tiled GEMM on the int8 matrix cores.
+//
+// Same integer arithmetic as cpu_vec_dot_q4_k_q8_k (src/backends/cpu/ops/matmul/quantized/vec_dot_impl.h:689-732):
+// per 256-value block
+//     isum = sum_j sc_j * (q_j . a_j),   msum = sum_j mn_j * (sum of a over sub-block j),
+//     y += a.d * (w.d * isum - w.dmin * msum)
+// A workgroup computes 128 weight rows x 64 tokens over a range of blocks. The 6-bit scale is folded into the
+// matrix-core operand, so that the eight sub-block products of a block chain through ONE accumulator and the fp32
+// work per output happens once per block instead of once per sub-block: sc = 8 * (sc >> 3) + (sc & 7), and both
+// q * (sc & 7) and q * (sc >> 3) are at most 15 * 7 = 105, i.e. int8. Per sub-block and 32 x 32 output tile that is
+//     X += A . (q * (sc & 7)),   Y += A . (q * (sc >> 3)),   T += A . mn        (v_mfma_i32_32x32x32_i8, exact)
+// and per block isum = X + 8 Y, msum = T. All integer results are exact (|isum| < 2^25); only the fp32 accumulation
+// over blocks is ordered differently from the CPU.
+//
+// Wavefronts are specialised like in the fp16 tile kernel: wavefronts 0..3 (one per SIMD) compute, wavefront c owns
+// weight rows 32 c .. 32 c + 31 of the tile and all 64 tokens (two 32 x 32 tiles) over all eight sub-blocks and issues
+// no vector-memory instruction inside the K loop; wavefronts 4..7 bring, per block, the int8 activation tile
+// (64 tokens x 256 bytes, chunks XOR-swizzled by token), the raw weight blocks (128 rows x 144 bytes) and the 64
+// activation scales into one of four LDS stages with direct-to-LDS loads, three blocks ahead. One barrier per block.
+#include "mh_rows.h"
+
+namespace mh {
+
+typedef int i8_intx4 __attribute__((ext_vector_type(4)));
+typedef int i8_intx16 __attribute__((ext_vector_type(16)));
+typedef unsigned short i8_u16x2 __attribute__((ext_vector_type(2)));
+
+struct GemmI8Params {
+    const uint8_t *w;   // Q4_K blocks, M rows of nb blocks
+    const int8_t *qs;   // quantized activations, rows of kp bytes
+    const float *ad;    // activation block scales [N][nb]
+    size_t kp;
+    size_t N, M, nb;
+    void *out;          // [N][M] of the output type, or fp32 partials [splits][N][M] when splits > 1
+    int splits;
+    int blocks_per_split;
+    const void *bias;
+    int bias_is_f16;
+    int bias_first;     // fp16 output: f16(dot + bias) instead of f16(f16(dot) + bias)
+    int out_is_f16;
+};
+
+constexpr int I8_TOK = 64;
+constexpr int I8_WROWS = 128;
+constexpr int I8_COMPUTE = 4;
+constexpr int I8_LOADERS = 4;
+constexpr int I8_THREADS = (I8_COMPUTE + I8_LOADERS) * 64;
+constexpr int I8_STAGE_A = I8_TOK * QK_K;             // 16,384
+constexpr int I8_STAGE_W = I8_WROWS * Q4_K_BYTES;     // 18,432
+constexpr int I8_STAGE_D = I8_TOK * 4;                // 256
+constexpr int I8_STAGE = I8_STAGE_A + I8_STAGE_W + I8_STAGE_D;
+constexpr int I8_STAGES = 4;
+constexpr int I8_AHEAD = I8_STAGES - 1;
+constexpr int I8_LDS_BYTES = I8_STAGES * I8_STAGE;    // 140,288
+constexpr int I8_OUT_PITCH = I8_WROWS + 4;            // floats per token of the output tile in LDS
+static_assert(I8_TOK * I8_OUT_PITCH * 4 <= I8_LDS_BYTES, "the output tile reuses the stages");
+static_assert(I8_STAGE % 16 == 0, "stages keep 16-byte alignment");
+
+__device__ __forceinline__ void i8_lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// One direct-to-LDS load of 64 x 4 bytes (see dma16_to_lds): lane l's dword lands at LDS address M0 + 4 l.
+__device__ __forceinline__ void dma4_to_lds(const uint8_t *base, uint32_t voff) {
+    asm volatile("global_load_lds_dword %0, %1" : : "v"(voff), "s"(base) : "memory");
+}
+
+// the four bytes of `nib` (each 0..15) times the scalar in both 16-bit halves of `s16` (0..7): no byte overflows
+__device__ __forceinline__ int i8_scale_bytes(uint32_t nib, uint32_t s16) {
+    const i8_u16x2 r = __builtin_bit_cast(i8_u16x2, nib) * __builtin_bit_cast(i8_u16x2, s16);
+    return __builtin_bit_cast(int, r);
+}
+
+__global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Params p) {
+    warm_kernel_arguments<sizeof(GemmI8Params)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * I8_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = (int)(b1 - b0);
+    const int j = lane & 31, kh = lane >> 5;
+
+    float total[2][16];  // [token tile][register], compute wavefronts only
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
+        }
+    }
+
+    if (wave >= I8_COMPUTE) {
+        // ------------------------------------------------------------------------------------------------ loaders
+        const int L = wave - I8_COMPUTE;
+        const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+        const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);  // token rows beyond it re-read it
+        const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
+        // Activation tile: token t owns 256 bytes of the stage as 16 chunks of 16 bytes, chunk c stored in slot
+        // c ^ (t % 16) (the MFMA operand reads of 32 tokens x one chunk then spread over the bank groups). One
+        // instruction moves four token rows; loader L brings tokens 16 L .. 16 L + 15.
+        uint32_t a_voff[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t t = (uint32_t)(16 * L + 4 * c + (lane >> 4));
+            const uint32_t slot = (uint32_t)(lane & 15);
+            const uint32_t trow = t < last_tok ? t : last_tok;
+            a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+        }
+        // Weight blocks: piece q of the stage is 16 bytes q % 9 of tile row q / 9; loader L brings pieces
+        // 256 pass + 64 L + lane. Rows beyond M re-read row M - 1 (never stored).
+        const size_t row_bytes = p.nb * Q4_K_BYTES;
+        const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+        uint32_t w_voff[5];
+#pragma unroll
+        for (int pass = 0; pass < 5; ++pass) {
+            const uint32_t q = (uint32_t)(256 * pass + 64 * L + lane);
+            const uint32_t r = q / 9u, c9 = q - 9u * r;
+            const uint32_t rr = r < last_wrow ? r : last_wrow;
+            w_voff[pass] = rr * (uint32_t)row_bytes + 16u * c9;
+        }
+        const uint8_t *wbase = p.w + row0 * row_bytes;
+        const bool fifth = L < 2;   // pieces 1024 .. 1151
+        const bool scales = L == 3;  // the 64 activation scales of the block
+        uint32_t d_voff;
+        {
+            const uint32_t t = (uint32_t)lane;
+            const uint32_t trow = t < last_tok ? t : last_tok;
+            d_voff = (uint32_t)((trow * p.nb) * 4);
+        }
+        const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
+        const int per_block = 8 + (fifth ? 1 : 0) + (scales ? 1 : 0);
+        auto issue = [&](size_t b, int stage) {
+            const uint32_t s0 = lds_base + (uint32_t)(stage * I8_STAGE);
+            const uint8_t *qb = tile_q + b * QK_K;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                dma_set_lds_base(s0 + (uint32_t)(4096 * L + 1024 * c));
+                dma16_to_lds<0>(qb, a_voff[c]);
+            }
+            const uint8_t *wb = wbase + b * Q4_K_BYTES;
+#pragma unroll
+            for (int pass = 0; pass < 4; ++pass) {
+                dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (256 * pass + 64 * L) * 16));
+                dma16_to_lds<0>(wb, w_voff[pass]);
+            }
+            if (fifth) {
+                dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (1024 + 64 * L) * 16));
+                dma16_to_lds<0>(wb, w_voff[4]);
+            }
+            if (scales) {
+                dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + I8_STAGE_W));
+                dma4_to_lds(tile_d + b * 4, d_voff);
+            }
+        };
+        // blocks issued but not needed yet when block `need` must have landed: need + 1 .. min(newest, nblk - 1)
+        auto newer_than = [&](int need, int newest) {
+            const int last = newest < nblk - 1 ? newest : nblk - 1;
+            return last > need ? last - need : 0;
+        };
+        for (int i = 0; i < I8_AHEAD; ++i) {
+            if (i < nblk) {
+                issue(b0 + (size_t)i, i);
+            }
+        }
+        wait_vmcnt_at_most(newer_than(0, I8_AHEAD - 1) * per_block);
+        i8_lds_barrier();
+        for (int i = 0; i < nblk; ++i) {
+            if (i + I8_AHEAD < nblk) {
+                issue(b0 + (size_t)(i + I8_AHEAD), (i + I8_AHEAD) % I8_STAGES);  // the stage block i - 1 has left
+            }
+            if (i + 1 < nblk) {
+                wait_vmcnt_at_most(newer_than(i + 1, i + I8_AHEAD) * per_block);
+            }
+            i8_lds_barrier();
+        }
+    } else {
+        // ------------------------------------------------------------------------------------------------ compute
+        const uint32_t w_off = (uint32_t)(I8_STAGE_A + (32 * wave + j) * Q4_K_BYTES);
+        // A operand of sub-block sb, token tile a, lane (j, kh): token 32 a + j, chunk 2 sb + kh at slot chunk ^ (j % 16)
+        uint32_t a_off[8];
+#pragma unroll
+        for (int sb = 0; sb < 8; ++sb) {
+            a_off[sb] = (uint32_t)(j * QK_K + 16 * ((2 * sb + kh) ^ (j & 15)));
+        }
+        const uint32_t d_off = (uint32_t)(I8_STAGE_A + I8_STAGE_W + 16 * kh);
+
+        i8_lds_barrier();
+        for (int blk = 0; blk < nblk; ++blk) {
+            const uint8_t *stage = lds + (size_t)(blk % I8_STAGES) * I8_STAGE;
+            const uint8_t *wr = stage + w_off;
+            const uint4 hdr = *(const uint4 *)wr;
+            uint4 wq[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                wq[g] = *(const uint4 *)(wr + 16 + 32 * g + 16 * kh);
+            }
+            // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
+            float d = h2f((uint16_t)(hdr.x & 0xffffu));
+            float dmin = h2f((uint16_t)(hdr.x >> 16));
+            asm volatile("" : "+v"(d), "+v"(dmin));  // plain fp32 values: no mixed-precision multiply-adds below
+            const uint32_t sc_lo = hdr.y & 0x3f3f3f3fu;
+            const uint32_t mn_lo = hdr.z & 0x3f3f3f3fu;
+            const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
+            const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+            const uint32_t s3_lo[2] = {sc_lo & 0x07070707u, sc_hi & 0x07070707u};          // sc & 7
+            const uint32_t s3_hi[2] = {(sc_lo >> 3) & 0x07070707u, (sc_hi >> 3) & 0x07070707u};  // sc >> 3
+
+            i8_intx16 X[2], Y[2], T[2];
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                const uint4 src = wq[sb >> 1];
+                uint32_t nib[4];
+                if (sb & 1) {
+                    nib[0] = (src.x >> 4) & 0x0f0f0f0fu;
+                    nib[1] = (src.y >> 4) & 0x0f0f0f0fu;
+                    nib[2] = (src.z >> 4) & 0x0f0f0f0fu;
+                    nib[3] = (src.w >> 4) & 0x0f0f0f0fu;
+                } else {
+                    nib[0] = src.x & 0x0f0f0f0fu;
+                    nib[1] = src.y & 0x0f0f0f0fu;
+                    nib[2] = src.z & 0x0f0f0f0fu;
+                    nib[3] = src.w & 0x0f0f0f0fu;
+                }
+                // byte sb % 4 of the packed 3-bit halves in both 16-bit lanes; of the packed mins in all four bytes
+                const uint32_t sel16 = 0x0c000c00u | (uint32_t)(sb & 3) | ((uint32_t)(sb & 3) << 16);
+                const uint32_t lo16 = __builtin_amdgcn_perm(0u, s3_lo[sb >> 2], sel16);
+                const uint32_t hi16 = __builtin_amdgcn_perm(0u, s3_hi[sb >> 2], sel16);
+                const int mn4 = (int)__builtin_amdgcn_perm(0u, sb < 4 ? mn_lo : mn_hi, 0x01010101u * (sb & 3));
+                const i8_intx4 bx = {i8_scale_bytes(nib[0], lo16), i8_scale_bytes(nib[1], lo16),
+                                     i8_scale_bytes(nib[2], lo16), i8_scale_bytes(nib[3], lo16)};
+                const i8_intx4 by = {i8_scale_bytes(nib[0], hi16), i8_scale_bytes(nib[1], hi16),
+                                     i8_scale_bytes(nib[2], hi16), i8_scale_bytes(nib[3], hi16)};
+                const i8_intx4 bt = {mn4, mn4, mn4, mn4};
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const uint4 av = *(const uint4 *)(stage + a_off[sb] + a * (32 * QK_K));
+                    const i8_intx4 aop = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                    if (sb == 0) {
+                        const i8_intx16 zero = {0};
+                        X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bx, zero, 0, 0, 0);
+                        Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, by, zero, 0, 0, 0);
+                        T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bt, zero, 0, 0, 0);
+                    } else {
+                        X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bx, X[a], 0, 0, 0);
+                        Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, by, Y[a], 0, 0, 0);
+                        T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bt, T[a], 0, 0, 0);
+                    }
+                }
+            }
+            // once per block and output: y += a.d * (w.d * isum - w.dmin * msum)
+            const float ndmin = -dmin;
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    // registers 4 g .. 4 g + 3 are tokens 32 a + 8 g + 4 kh .. + 3
+                    const float4 da4 = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * g));
+                    const float da[4] = {da4.x, da4.y, da4.z, da4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = 4 * g + e;
+                        const int isum = X[a][r] + (Y[a][r] << 3);
+                        const float v = __builtin_fmaf(ndmin, (float)T[a][r], d * (float)isum);
+                        total[a][r] = __builtin_fmaf(da[e], v, total[a][r]);
+                    }
+                }
+            }
+            i8_lds_barrier();
+        }
+    }
+
+    // ---- the output tile meets in LDS as [token][weight row], then every thread stores 16 bytes per step.
+    // Lane (j, kh) of compute wavefront c holds weight row 32 c + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4.
+    float *tile = (float *)lds;
+    if (wave < I8_COMPUTE) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * wave + j] = total[a][r];
+            }
+        }
+    }
+    i8_lds_barrier();
+
+    const bool partials = p.splits > 1;
+    const bool has_bias = !partials && p.bias != nullptr;
+    const bool out_f16 = !partials && p.out_is_f16;
+    float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
+    const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    for (int idx = tid; idx < I8_TOK * I8_WROWS / 4; idx += I8_THREADS) {
+        const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
+        const size_t n = tt * I8_TOK + (size_t)t;
+        const size_t m4 = row0 + 4 * (size_t)q4;
+        if (n >= p.N || m4 >= p.M) {
+            continue;
+        }
+        const float4 v = *(const float4 *)(tile + t * I8_OUT_PITCH + 4 * q4);
+        const float e4[4] = {v.x, v.y, v.z, v.w};
+        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (m4 + e < p.M) {
+                    bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
+                }
+            }
+        }
+        if (!out_f16) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[e] = has_bias ? e4[e] + bias4[e] : e4[e];
+            }
+            float *dst = out32 + n * p.M + m4;
+            if (vec) {  // M % 4 == 0: the four rows exist
+                *(float4 *)dst = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = o[e];
+                    }
+                }
+            }
+        } else {
+            uint16_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (p.bias_first) {
+                    h[e] = f2h(has_bias ? e4[e] + bias4[e] : e4[e]);
+                } else {
+                    h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
+                    if (has_bias) {
+                        h[e] = f2h(h2f(h[e]) + bias4[e]);
+                    }
+                }
+            }
+            uint16_t *dst = (uint16_t *)p.out + n * p.M + m4;
+            if (vec) {
+                *(uint2 *)dst = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = h[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host side
+// From this many activation rows on the tile kernel replaces the 32-row passes of the streaming small-batch kernel.
+constexpr size_t I8_MIN_ROWS = 48;
+
+static size_t gemm_i8_splits(const marmot_hip_device *dev, size_t N, size_t M, size_t nb, size_t *blocks_per_split) {
+    const size_t tiles = ((N + I8_TOK - 1) / I8_TOK) * ((M + I8_WROWS - 1) / I8_WROWS);
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    size_t splits = 1;
+    if (tiles * 2 <= cus) {  // fewer tiles than half the chip: split K across workgroups (short prompts)
+        splits = cus / tiles;
+        const size_t max_splits = nb / 2 > 0 ? nb / 2 : 1;  // at least two blocks per workgroup
+        splits = splits > max_splits ? max_splits : splits;
+    }
+    const size_t bps = (nb + splits - 1) / splits;
+    *blocks_per_split = bps;
+    return (nb + bps - 1) / bps;
+}
+
+bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
+                     const ActScratch &act) {
+    if (dev->knobs.no_gemm_i8 || kind != MARMOT_HIP_KIND_Q4_K || N < I8_MIN_ROWS || K % QK_K != 0) {
+        return false;
+    }
+    if ((((uintptr_t)act.qs) & 15) != 0 || act.kp % 16 != 0 || N * act.kp >= ((size_t)1 << 32) ||
+        N * (K / QK_K) * 4 >= ((size_t)1 << 32) || I8_WROWS * (K / QK_K) * Q4_K_BYTES >= ((size_t)1 << 32)) {
+        return false;  // 16-byte direct-to-LDS loads with 32-bit lane offsets
+    }
+    for (int i = 0; i < count; ++i) {
+        if ((((uintptr_t)weights[i]) & 15) != 0) {
+            return false;
+        }
+    }
+    return true;
+}
+
+size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, int weights) {
+    size_t bps = 0;
+    const size_t splits = gemm_i8_splits(dev, N, M, K / QK_K, &bps);
+    return splits > 1 ? splits * N * M * sizeof(float) * (size_t)weights : 0;
+}
+
+int launch_gemm_i8(marmot_hip_device *dev, const WeightSet &ws, const ActScratch &act, size_t N, size_t K, size_t M,
+                   int out_dtype, void *scratch) {
+    const size_t nb = K / QK_K;
+    size_t bps = 0;
+    const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
+    float *partial = (float *)scratch;
+    if (splits > 1 && partial == nullptr) {
+        void *wsp = nullptr;
+        MH_TRY(workspace_reserve(dev, gemm_i8_scratch_bytes(dev, N, K, M, ws.count), &wsp));
+        partial = (float *)wsp;
+    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_q8k_tile));
+    const dim3 grid((unsigned)((M + I8_WROWS - 1) / I8_WROWS), (unsigned)((N + I8_TOK - 1) / I8_TOK), (unsigned)splits);
+    for (int which = 0; which < ws.count; ++which) {
+        GemmI8Params p;
+        p.w = (const uint8_t *)ws.w[which];
+        p.qs = act.qs;
+        p.ad = act.d;
+        p.kp = act.kp;
+        p.N = N;
+        p.M = M;
+        p.nb = nb;
+        float *part = splits > 1 ? partial + (size_t)which * splits * N * M : nullptr;
+        p.out = splits > 1 ? (void *)part : ws.out[which];
+        p.splits = (int)splits;
+        p.blocks_per_split = (int)bps;
+        p.bias = ws.bias[which];
+        p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
+        p.bias_first = ws.bias_first ? 1 : 0;
+        p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+        hipLaunchKernelGGL(k_gemm_q4k_q8k_tile, grid, dim3(I8_THREADS), I8_LDS_BYTES, dev->stream, p);
+        MH_HIP(hipGetLastError());
+        if (splits > 1) {
+            MH_TRY(launch_splitk_reduce(dev, part, (int)splits, N, M, ws.bias[which], ws.bias_dtype, ws.out[which],
+                                        out_dtype, ws.bias_first));
+        }
+    }
+    set_route("mmq_q4_k_q8_k_mfma_tile");
+    return MARMOT_HIP_SUCCESS;
+}
+
+} // namespace mh

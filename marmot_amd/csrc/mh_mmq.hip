@@ -908,7 +908,10 @@ static MmqPlan mmq_plan(const marmot_hip_device *dev, int kind, size_t N, size_t
 // bytes of fp32 partials launch_mmq needs for this shape (0 when K is not split across workgroups)
 size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M, int weights) {
     const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K, weights);
-    return pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (size_t)weights : 0;
+    const size_t passes = pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (size_t)weights : 0;
+    // the tiled GEMM may take the call instead (decided at launch, when the operands' alignment is known)
+    const size_t tiled = (kind == MARMOT_HIP_KIND_Q4_K && !dev->knobs.no_gemm_i8) ? gemm_i8_scratch_bytes(dev, N, K, M, weights) : 0;
+    return passes > tiled ? passes : tiled;
 }
 
 static size_t mmq6_lds_bytes(int W) {
@@ -1035,6 +1038,9 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
                    size_t M, int out_dtype, void *scratch) {
     if (!mmq_supported(dev, kind, N, K, ws.count)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
+    }
+    if (gemm_i8_applies(dev, kind, N, K, ws.w, ws.count, act)) {
+        return launch_gemm_i8(dev, ws, act, N, K, M, out_dtype, scratch);
     }
     const size_t nb = K / QK_K;
     const MmqPlan pl = mmq_plan(dev, kind, N, M, nb, ws.count);

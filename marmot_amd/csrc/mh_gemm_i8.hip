@@ -42,7 +42,8 @@ struct GemmI8Params {
 
 constexpr int I8_TOK = 64;
 constexpr int I8_WROWS = 128;
-constexpr int I8_COMPUTE = 4;
+constexpr int I8_TA = 1;                              // 32-token tiles per compute wavefront
+constexpr int I8_COMPUTE = 4 * (2 / I8_TA);
 constexpr int I8_LOADERS = 4;
 constexpr int I8_THREADS = (I8_COMPUTE + I8_LOADERS) * 64;
 constexpr int I8_STAGE_A = I8_TOK * QK_K;             // 16,384
@@ -88,9 +89,9 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
     const int nblk = (int)(b1 - b0);
     const int j = lane & 31, kh = lane >> 5;
 
-    float total[2][16];  // [token tile][register], compute wavefronts only
+    float total[I8_TA][16];  // [token tile][register], compute wavefronts only
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < I8_TA; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             total[a][r] = 0.0f;
@@ -170,20 +171,24 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
                 issue(b0 + (size_t)i, i);
             }
         }
-        wait_vmcnt_at_most(newer_than(0, I8_AHEAD - 1) * per_block);
+        // Behind the barrier that opens round i (the compute wavefronts work on block i) blocks i AND i + 1 are
+        // complete: the compute wavefronts fetch the weights of block i + 1 while they finish block i.
+        wait_vmcnt_at_most(newer_than(1, I8_AHEAD - 1) * per_block);
         i8_lds_barrier();
         for (int i = 0; i < nblk; ++i) {
             if (i + I8_AHEAD < nblk) {
                 issue(b0 + (size_t)(i + I8_AHEAD), (i + I8_AHEAD) % I8_STAGES);  // the stage block i - 1 has left
             }
             if (i + 1 < nblk) {
-                wait_vmcnt_at_most(newer_than(i + 1, i + I8_AHEAD) * per_block);
+                wait_vmcnt_at_most(newer_than(i + 2, i + I8_AHEAD) * per_block);
             }
             i8_lds_barrier();
         }
     } else {
         // ------------------------------------------------------------------------------------------------ compute
-        const uint32_t w_off = (uint32_t)(I8_STAGE_A + (32 * wave + j) * Q4_K_BYTES);
+        const int rg = wave & 3;           // weight rows 32 rg .. + 31 of the tile
+        const int ta0 = (wave >> 2) * I8_TA;  // first 32-token tile of this wavefront
+        const uint32_t w_off = (uint32_t)(I8_STAGE_A + (32 * rg + j) * Q4_K_BYTES);
         // A operand of sub-block sb, token tile a, lane (j, kh): token 32 a + j, chunk 2 sb + kh at slot chunk ^ (j % 16)
         uint32_t a_off[8];
 #pragma unroll
@@ -193,15 +198,28 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
         const uint32_t d_off = (uint32_t)(I8_STAGE_A + I8_STAGE_W + 16 * kh);
 
         i8_lds_barrier();
-        for (int blk = 0; blk < nblk; ++blk) {
-            const uint8_t *stage = lds + (size_t)(blk % I8_STAGES) * I8_STAGE;
-            const uint8_t *wr = stage + w_off;
-            const uint4 hdr = *(const uint4 *)wr;
-            uint4 wq[4];
+        // this lane's weight row of block 0; the row of block blk + 1 is fetched while block blk is finished
+        uint4 hdr, wq[4];
+        auto read_weights = [&](int b) {
+            const uint8_t *wr = lds + (size_t)(b % I8_STAGES) * I8_STAGE + w_off;
+            hdr = *(const uint4 *)wr;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 wq[g] = *(const uint4 *)(wr + 16 + 32 * g + 16 * kh);
             }
+        };
+        read_weights(0);
+        for (int blk = 0; blk < nblk; ++blk) {
+            const uint8_t *stage = lds + (size_t)(blk % I8_STAGES) * I8_STAGE;
+            auto read_a = [&](int sb, i8_intx4(&aop)[I8_TA]) {
+#pragma unroll
+                for (int a = 0; a < I8_TA; ++a) {
+                    const uint4 av = *(const uint4 *)(stage + a_off[sb] + (ta0 + a) * (32 * QK_K));
+                    aop[a] = i8_intx4{(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                }
+            };
+            i8_intx4 aop[2][I8_TA];  // A operands of the sub-block in work and of the next one
+            read_a(0, aop[0]);
             // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
             float d = h2f((uint16_t)(hdr.x & 0xffffu));
             float dmin = h2f((uint16_t)(hdr.x >> 16));
@@ -210,60 +228,127 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
             const uint32_t mn_lo = hdr.z & 0x3f3f3f3fu;
             const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
             const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
-            const uint32_t s3_lo[2] = {sc_lo & 0x07070707u, sc_hi & 0x07070707u};          // sc & 7
+            const uint32_t s3_lo[2] = {sc_lo & 0x07070707u, sc_hi & 0x07070707u};                // sc & 7
             const uint32_t s3_hi[2] = {(sc_lo >> 3) & 0x07070707u, (sc_hi >> 3) & 0x07070707u};  // sc >> 3
+            uint4 wcur[4] = {wq[0], wq[1], wq[2], wq[3]};
 
-            i8_intx16 X[2], Y[2], T[2];
+            i8_intx16 X[I8_TA], Y[I8_TA], T[I8_TA];
+            float4 da4[I8_TA][4];
+            // B operands of sub-block sb: the nibbles times (sc & 7), times (sc >> 3), and the min in every byte. Built
+            // in six pieces, one behind each matrix-core instruction of the previous sub-block, so that the vector
+            // instructions issue while the matrix cores work instead of in front of them.
+            uint32_t nib[4], lo16 = 0, hi16 = 0;
+            i8_intx4 bx[2], by[2];
+            int bt[2];
+            auto prep = [&](int sb, int piece) {
+                const int n = sb & 1;
+                const uint4 src = wcur[sb >> 1];
+                switch (piece) {
+                case 0:
+                    if (sb & 1) {
+                        nib[0] = (src.x >> 4) & 0x0f0f0f0fu;
+                        nib[1] = (src.y >> 4) & 0x0f0f0f0fu;
+                    } else {
+                        nib[0] = src.x & 0x0f0f0f0fu;
+                        nib[1] = src.y & 0x0f0f0f0fu;
+                    }
+                    break;
+                case 1:
+                    if (sb & 1) {
+                        nib[2] = (src.z >> 4) & 0x0f0f0f0fu;
+                        nib[3] = (src.w >> 4) & 0x0f0f0f0fu;
+                    } else {
+                        nib[2] = src.z & 0x0f0f0f0fu;
+                        nib[3] = src.w & 0x0f0f0f0fu;
+                    }
+                    break;
+                case 2: {
+                    // byte sb % 4 of the packed 3-bit halves in both 16-bit lanes; of the packed mins in all four bytes
+                    const uint32_t sel16 = 0x0c000c00u | (uint32_t)(sb & 3) | ((uint32_t)(sb & 3) << 16);
+                    lo16 = __builtin_amdgcn_perm(0u, s3_lo[sb >> 2], sel16);
+                    hi16 = __builtin_amdgcn_perm(0u, s3_hi[sb >> 2], sel16);
+                    bt[n] = (int)__builtin_amdgcn_perm(0u, sb < 4 ? mn_lo : mn_hi, 0x01010101u * (sb & 3));
+                    break;
+                }
+                case 3:
+                    bx[n][0] = i8_scale_bytes(nib[0], lo16);
+                    bx[n][1] = i8_scale_bytes(nib[1], lo16);
+                    bx[n][2] = i8_scale_bytes(nib[2], lo16);
+                    break;
+                case 4:
+                    bx[n][3] = i8_scale_bytes(nib[3], lo16);
+                    by[n][0] = i8_scale_bytes(nib[0], hi16);
+                    by[n][1] = i8_scale_bytes(nib[1], hi16);
+                    break;
+                default:
+                    by[n][2] = i8_scale_bytes(nib[2], hi16);
+                    by[n][3] = i8_scale_bytes(nib[3], hi16);
+                    break;
+                }
+            };
+#pragma unroll
+            for (int piece = 0; piece < 6; ++piece) {
+                prep(0, piece);
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int sb = 0; sb < 8; ++sb) {
-                const uint4 src = wq[sb >> 1];
-                uint32_t nib[4];
-                if (sb & 1) {
-                    nib[0] = (src.x >> 4) & 0x0f0f0f0fu;
-                    nib[1] = (src.y >> 4) & 0x0f0f0f0fu;
-                    nib[2] = (src.z >> 4) & 0x0f0f0f0fu;
-                    nib[3] = (src.w >> 4) & 0x0f0f0f0fu;
-                } else {
-                    nib[0] = src.x & 0x0f0f0f0fu;
-                    nib[1] = src.y & 0x0f0f0f0fu;
-                    nib[2] = src.z & 0x0f0f0f0fu;
-                    nib[3] = src.w & 0x0f0f0f0fu;
+                const int c = sb & 1;
+                if (sb < 7) {
+                    read_a(sb + 1, aop[c ^ 1]);  // lands while the MFMAs below run
+                } else if (blk + 1 < nblk) {
+                    read_weights(blk + 1);  // complete since the barrier that opened this round
                 }
-                // byte sb % 4 of the packed 3-bit halves in both 16-bit lanes; of the packed mins in all four bytes
-                const uint32_t sel16 = 0x0c000c00u | (uint32_t)(sb & 3) | ((uint32_t)(sb & 3) << 16);
-                const uint32_t lo16 = __builtin_amdgcn_perm(0u, s3_lo[sb >> 2], sel16);
-                const uint32_t hi16 = __builtin_amdgcn_perm(0u, s3_hi[sb >> 2], sel16);
-                const int mn4 = (int)__builtin_amdgcn_perm(0u, sb < 4 ? mn_lo : mn_hi, 0x01010101u * (sb & 3));
-                const i8_intx4 bx = {i8_scale_bytes(nib[0], lo16), i8_scale_bytes(nib[1], lo16),
-                                     i8_scale_bytes(nib[2], lo16), i8_scale_bytes(nib[3], lo16)};
-                const i8_intx4 by = {i8_scale_bytes(nib[0], hi16), i8_scale_bytes(nib[1], hi16),
-                                     i8_scale_bytes(nib[2], hi16), i8_scale_bytes(nib[3], hi16)};
-                const i8_intx4 bt = {mn4, mn4, mn4, mn4};
+                if (sb == 6) {
+                    // activation scales: registers 4 g .. 4 g + 3 of token tile a are tokens 32 a + 8 g + 4 kh .. + 3
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    const uint4 av = *(const uint4 *)(stage + a_off[sb] + a * (32 * QK_K));
-                    const i8_intx4 aop = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
-                    if (sb == 0) {
-                        const i8_intx16 zero = {0};
-                        X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bx, zero, 0, 0, 0);
-                        Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, by, zero, 0, 0, 0);
-                        T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bt, zero, 0, 0, 0);
-                    } else {
-                        X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bx, X[a], 0, 0, 0);
-                        Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, by, Y[a], 0, 0, 0);
-                        T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bt, T[a], 0, 0, 0);
+                    for (int a = 0; a < I8_TA; ++a) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            da4[a][g] = *(const float4 *)(stage + d_off + 4 * (32 * (ta0 + a) + 8 * g));
+                        }
                     }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const i8_intx4 btv = {bt[c], bt[c], bt[c], bt[c]};
+#pragma unroll
+                for (int a = 0; a < I8_TA; ++a) {
+                    constexpr int PP = 2 / I8_TA;  // preparation pieces behind each matrix-core instruction
+                    const i8_intx4 av = aop[c][a];
+                    const i8_intx16 zero = {0};
+                    X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bx[c], sb == 0 ? zero : X[a], 0, 0, 0);
+                    if (sb < 7) {
+#pragma unroll
+                        for (int q = 0; q < PP; ++q) {
+                            prep(sb + 1, PP * (3 * a) + q);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, by[c], sb == 0 ? zero : Y[a], 0, 0, 0);
+                    if (sb < 7) {
+#pragma unroll
+                        for (int q = 0; q < PP; ++q) {
+                            prep(sb + 1, PP * (3 * a + 1) + q);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, btv, sb == 0 ? zero : T[a], 0, 0, 0);
+                    if (sb < 7) {
+#pragma unroll
+                        for (int q = 0; q < PP; ++q) {
+                            prep(sb + 1, PP * (3 * a + 2) + q);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
             // once per block and output: y += a.d * (w.d * isum - w.dmin * msum)
             const float ndmin = -dmin;
 #pragma unroll
-            for (int a = 0; a < 2; ++a) {
+            for (int a = 0; a < I8_TA; ++a) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    // registers 4 g .. 4 g + 3 are tokens 32 a + 8 g + 4 kh .. + 3
-                    const float4 da4 = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * g));
-                    const float da[4] = {da4.x, da4.y, da4.z, da4.w};
+                    const float da[4] = {da4[a][g].x, da4[a][g].y, da4[a][g].z, da4[a][g].w};
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int r = 4 * g + e;
@@ -278,14 +363,15 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
     }
 
     // ---- the output tile meets in LDS as [token][weight row], then every thread stores 16 bytes per step.
-    // Lane (j, kh) of compute wavefront c holds weight row 32 c + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4.
+    // Lane (j, kh) of a compute wavefront holds weight row 32 rg + j for tokens 32 (ta0 + a) + 8 (r / 4) + 4 kh + r % 4.
     float *tile = (float *)lds;
     if (wave < I8_COMPUTE) {
+        const int rg = wave & 3, ta0 = (wave >> 2) * I8_TA;
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < I8_TA; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * wave + j] = total[a][r];
+                tile[(32 * (ta0 + a) + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j] = total[a][r];
             }
         }
     }

@@ -12,11 +12,16 @@
 // and per block isum = X + 8 Y, msum = T. All integer results are exact (|isum| < 2^25); only the fp32 accumulation
 // over blocks is ordered differently from the CPU.
 //
-// Wavefronts are specialised like in the fp16 tile kernel: wavefronts 0..3 (one per SIMD) compute, wavefront c owns
-// weight rows 32 c .. 32 c + 31 of the tile and all 64 tokens (two 32 x 32 tiles) over all eight sub-blocks and issues
-// no vector-memory instruction inside the K loop; wavefronts 4..7 bring, per block, the int8 activation tile
-// (64 tokens x 256 bytes, chunks XOR-swizzled by token), the raw weight blocks (128 rows x 144 bytes) and the 64
-// activation scales into one of four LDS stages with direct-to-LDS loads, three blocks ahead. One barrier per block.
+// Eight wavefronts, two per SIMD: wavefront (rg, kg) owns weight rows 32 rg .. 32 rg + 31 of the tile and all 64 tokens
+// (two 32 x 32 tiles) and works on every second block of the workgroup's K range (K group kg), so a round consumes two
+// consecutive blocks; the two K groups' sums meet in LDS at the end. There are no loader wavefronts: at the start of a
+// round every wavefront issues its quarter of its K group's next block (int8 activation tile 64 tokens x 256 bytes
+// with the chunks XOR-swizzled by token, raw weight blocks 128 rows x 144 bytes, 64 activation scales) as
+// direct-to-LDS loads into the other round buffer, then computes, then waits for its own loads; one barrier per round.
+// On this chip a wavefront's instruction stream costs about 5.6 clocks per vector instruction and 16 per
+// matrix-core or LDS instruction whatever else the SIMD does, so the kernel is bound by its instruction count
+// (per block and wavefront: 378 vector, 48 matrix-core, 29 LDS); the operand preparation of sub-block s + 1 is placed
+// between the matrix-core instructions of sub-block s so that the matrix cores never wait for it.
 #include "mh_rows.h"
 
 namespace mh {
@@ -42,17 +47,14 @@ struct GemmI8Params {
 
 constexpr int I8_TOK = 64;
 constexpr int I8_WROWS = 128;
-constexpr int I8_TA = 1;                              // 32-token tiles per compute wavefront
-constexpr int I8_COMPUTE = 4 * (2 / I8_TA);
-constexpr int I8_LOADERS = 4;
-constexpr int I8_THREADS = (I8_COMPUTE + I8_LOADERS) * 64;
+constexpr int I8_WAVES = 8;
+constexpr int I8_THREADS = I8_WAVES * 64;
 constexpr int I8_STAGE_A = I8_TOK * QK_K;             // 16,384
 constexpr int I8_STAGE_W = I8_WROWS * Q4_K_BYTES;     // 18,432
 constexpr int I8_STAGE_D = I8_TOK * 4;                // 256
-constexpr int I8_STAGE = I8_STAGE_A + I8_STAGE_W + I8_STAGE_D;
-constexpr int I8_STAGES = 4;
-constexpr int I8_AHEAD = I8_STAGES - 1;
-constexpr int I8_LDS_BYTES = I8_STAGES * I8_STAGE;    // 140,288
+constexpr int I8_STAGE = I8_STAGE_A + I8_STAGE_W + I8_STAGE_D;   // one block of the tile: 35,072 bytes
+constexpr int I8_ROUND = 2 * I8_STAGE;                // a round is two consecutive blocks, one per K group
+constexpr int I8_LDS_BYTES = 2 * I8_ROUND;            // the round in work and the round in flight: 140,288
 constexpr int I8_OUT_PITCH = I8_WROWS + 4;            // floats per token of the output tile in LDS
 static_assert(I8_TOK * I8_OUT_PITCH * 4 <= I8_LDS_BYTES, "the output tile reuses the stages");
 static_assert(I8_STAGE % 16 == 0, "stages keep 16-byte alignment");
@@ -78,6 +80,8 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = wave & 3;   // weight rows 32 rg .. + 31 of the tile; also this wavefront's share of the loads
+    const int kg = wave >> 2;  // K group: blocks b0 + kg, b0 + kg + 2, ...
     const size_t tt = blockIdx.y;
     const size_t row0 = (size_t)blockIdx.x * I8_WROWS;
     const int split = blockIdx.z;
@@ -87,138 +91,121 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
         b1 = p.nb;
     }
     const int nblk = (int)(b1 - b0);
+    const int rounds = (nblk + 1) / 2;
     const int j = lane & 31, kh = lane >> 5;
 
-    float total[I8_TA][16];  // [token tile][register], compute wavefronts only
+    float total[2][16];  // [token tile][register]
 #pragma unroll
-    for (int a = 0; a < I8_TA; ++a) {
+    for (int a = 0; a < 2; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             total[a][r] = 0.0f;
         }
     }
 
-    if (wave >= I8_COMPUTE) {
-        // ------------------------------------------------------------------------------------------------ loaders
-        const int L = wave - I8_COMPUTE;
-        const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
-        const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);  // token rows beyond it re-read it
-        const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
-        // Activation tile: token t owns 256 bytes of the stage as 16 chunks of 16 bytes, chunk c stored in slot
-        // c ^ (t % 16) (the MFMA operand reads of 32 tokens x one chunk then spread over the bank groups). One
-        // instruction moves four token rows; loader L brings tokens 16 L .. 16 L + 15.
-        uint32_t a_voff[4];
+    // ---- loads: the four wavefronts of a K group bring that group's block of every round, a quarter each
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);  // token rows beyond it re-read it
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
+    // Activation tile: token t owns 256 bytes of the stage as 16 chunks of 16 bytes, chunk c stored in slot
+    // c ^ (t % 16) (the MFMA operand reads of 32 tokens x one chunk then spread over the bank groups). One
+    // instruction moves four token rows; wavefront rg brings tokens 16 rg .. 16 rg + 15.
+    uint32_t a_voff[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t t = (uint32_t)(16 * rg + 4 * c + (lane >> 4));
+        const uint32_t slot = (uint32_t)(lane & 15);
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+    }
+    // Weight blocks: piece q of the stage is 16 bytes q % 9 of tile row q / 9; wavefront rg brings pieces
+    // 256 pass + 64 rg + lane. Rows beyond M re-read row M - 1 (never stored).
+    const size_t row_bytes = p.nb * Q4_K_BYTES;
+    const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+    uint32_t w_voff[5];
+#pragma unroll
+    for (int pass = 0; pass < 5; ++pass) {
+        const uint32_t q = (uint32_t)(256 * pass + 64 * rg + lane);
+        const uint32_t r = q / 9u, c9 = q - 9u * r;
+        const uint32_t rr = r < last_wrow ? r : last_wrow;
+        w_voff[pass] = rr * (uint32_t)row_bytes + 16u * c9;
+    }
+    const uint8_t *wbase = p.w + row0 * row_bytes;
+    const bool fifth = rg < 2;    // pieces 1024 .. 1151
+    const bool scales = rg == 3;  // the 64 activation scales of the block
+    uint32_t d_voff;
+    {
+        const uint32_t t = (uint32_t)lane;
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        d_voff = (uint32_t)((trow * p.nb) * 4);
+    }
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
+    // block b0 + 2 round + kg into the K group's half of round buffer round % 2 (nothing when the block does not exist)
+    auto issue = [&](int round) {
+        const int bi = 2 * round + kg;
+        if (bi >= nblk) {
+            return;
+        }
+        const size_t b = b0 + (size_t)bi;
+        const uint32_t s0 = lds_base + (uint32_t)((round & 1) * I8_ROUND + kg * I8_STAGE);
+        const uint8_t *qb = tile_q + b * QK_K;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const uint32_t t = (uint32_t)(16 * L + 4 * c + (lane >> 4));
-            const uint32_t slot = (uint32_t)(lane & 15);
-            const uint32_t trow = t < last_tok ? t : last_tok;
-            a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+            dma_set_lds_base(s0 + (uint32_t)(4096 * rg + 1024 * c));
+            dma16_to_lds<0>(qb, a_voff[c]);
         }
-        // Weight blocks: piece q of the stage is 16 bytes q % 9 of tile row q / 9; loader L brings pieces
-        // 256 pass + 64 L + lane. Rows beyond M re-read row M - 1 (never stored).
-        const size_t row_bytes = p.nb * Q4_K_BYTES;
-        const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
-        uint32_t w_voff[5];
+        const uint8_t *wb = wbase + b * Q4_K_BYTES;
 #pragma unroll
-        for (int pass = 0; pass < 5; ++pass) {
-            const uint32_t q = (uint32_t)(256 * pass + 64 * L + lane);
-            const uint32_t r = q / 9u, c9 = q - 9u * r;
-            const uint32_t rr = r < last_wrow ? r : last_wrow;
-            w_voff[pass] = rr * (uint32_t)row_bytes + 16u * c9;
+        for (int pass = 0; pass < 4; ++pass) {
+            dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (256 * pass + 64 * rg) * 16));
+            dma16_to_lds<0>(wb, w_voff[pass]);
         }
-        const uint8_t *wbase = p.w + row0 * row_bytes;
-        const bool fifth = L < 2;   // pieces 1024 .. 1151
-        const bool scales = L == 3;  // the 64 activation scales of the block
-        uint32_t d_voff;
-        {
-            const uint32_t t = (uint32_t)lane;
-            const uint32_t trow = t < last_tok ? t : last_tok;
-            d_voff = (uint32_t)((trow * p.nb) * 4);
+        if (fifth) {
+            dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (1024 + 64 * rg) * 16));
+            dma16_to_lds<0>(wb, w_voff[4]);
         }
-        const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
-        const int per_block = 8 + (fifth ? 1 : 0) + (scales ? 1 : 0);
-        auto issue = [&](size_t b, int stage) {
-            const uint32_t s0 = lds_base + (uint32_t)(stage * I8_STAGE);
-            const uint8_t *qb = tile_q + b * QK_K;
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                dma_set_lds_base(s0 + (uint32_t)(4096 * L + 1024 * c));
-                dma16_to_lds<0>(qb, a_voff[c]);
-            }
-            const uint8_t *wb = wbase + b * Q4_K_BYTES;
-#pragma unroll
-            for (int pass = 0; pass < 4; ++pass) {
-                dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (256 * pass + 64 * L) * 16));
-                dma16_to_lds<0>(wb, w_voff[pass]);
-            }
-            if (fifth) {
-                dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (1024 + 64 * L) * 16));
-                dma16_to_lds<0>(wb, w_voff[4]);
-            }
-            if (scales) {
-                dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + I8_STAGE_W));
-                dma4_to_lds(tile_d + b * 4, d_voff);
-            }
-        };
-        // blocks issued but not needed yet when block `need` must have landed: need + 1 .. min(newest, nblk - 1)
-        auto newer_than = [&](int need, int newest) {
-            const int last = newest < nblk - 1 ? newest : nblk - 1;
-            return last > need ? last - need : 0;
-        };
-        for (int i = 0; i < I8_AHEAD; ++i) {
-            if (i < nblk) {
-                issue(b0 + (size_t)i, i);
-            }
+        if (scales) {
+            dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + I8_STAGE_W));
+            dma4_to_lds(tile_d + b * 4, d_voff);
         }
-        // Behind the barrier that opens round i (the compute wavefronts work on block i) blocks i AND i + 1 are
-        // complete: the compute wavefronts fetch the weights of block i + 1 while they finish block i.
-        wait_vmcnt_at_most(newer_than(1, I8_AHEAD - 1) * per_block);
-        i8_lds_barrier();
-        for (int i = 0; i < nblk; ++i) {
-            if (i + I8_AHEAD < nblk) {
-                issue(b0 + (size_t)(i + I8_AHEAD), (i + I8_AHEAD) % I8_STAGES);  // the stage block i - 1 has left
-            }
-            if (i + 1 < nblk) {
-                wait_vmcnt_at_most(newer_than(i + 2, i + I8_AHEAD) * per_block);
-            }
-            i8_lds_barrier();
-        }
-    } else {
-        // ------------------------------------------------------------------------------------------------ compute
-        const int rg = wave & 3;           // weight rows 32 rg .. + 31 of the tile
-        const int ta0 = (wave >> 2) * I8_TA;  // first 32-token tile of this wavefront
-        const uint32_t w_off = (uint32_t)(I8_STAGE_A + (32 * rg + j) * Q4_K_BYTES);
-        // A operand of sub-block sb, token tile a, lane (j, kh): token 32 a + j, chunk 2 sb + kh at slot chunk ^ (j % 16)
-        uint32_t a_off[8];
-#pragma unroll
-        for (int sb = 0; sb < 8; ++sb) {
-            a_off[sb] = (uint32_t)(j * QK_K + 16 * ((2 * sb + kh) ^ (j & 15)));
-        }
-        const uint32_t d_off = (uint32_t)(I8_STAGE_A + I8_STAGE_W + 16 * kh);
+    };
 
-        i8_lds_barrier();
-        // this lane's weight row of block 0; the row of block blk + 1 is fetched while block blk is finished
-        uint4 hdr, wq[4];
-        auto read_weights = [&](int b) {
-            const uint8_t *wr = lds + (size_t)(b % I8_STAGES) * I8_STAGE + w_off;
-            hdr = *(const uint4 *)wr;
+    // ---- compute: this wavefront's weight row 32 rg + j of its K group's block, all 64 tokens
+    const uint32_t w_off = (uint32_t)(kg * I8_STAGE + I8_STAGE_A + (32 * rg + j) * Q4_K_BYTES);
+    // A operand of sub-block sb, token tile a, lane (j, kh): token 32 a + j, chunk 2 sb + kh at slot chunk ^ (j % 16)
+    uint32_t a_off[8];
+#pragma unroll
+    for (int sb = 0; sb < 8; ++sb) {
+        a_off[sb] = (uint32_t)(kg * I8_STAGE + j * QK_K + 16 * ((2 * sb + kh) ^ (j & 15)));
+    }
+    const uint32_t d_off = (uint32_t)(kg * I8_STAGE + I8_STAGE_A + I8_STAGE_W + 16 * kh);
+
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    i8_lds_barrier();
+    for (int round = 0; round < rounds; ++round) {
+        // the next round's blocks land in the other buffer while this round computes: the barrier that closed the
+        // previous round guarantees that nobody reads that buffer any more
+        if (round + 1 < rounds) {
+            issue(round + 1);
+        }
+        if (2 * round + kg < nblk) {
+            const uint8_t *stage = lds + (size_t)(round & 1) * I8_ROUND;
+            const uint8_t *wr = stage + w_off;
+            const uint4 hdr = *(const uint4 *)wr;
+            uint4 wq[4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 wq[g] = *(const uint4 *)(wr + 16 + 32 * g + 16 * kh);
             }
-        };
-        read_weights(0);
-        for (int blk = 0; blk < nblk; ++blk) {
-            const uint8_t *stage = lds + (size_t)(blk % I8_STAGES) * I8_STAGE;
-            auto read_a = [&](int sb, i8_intx4(&aop)[I8_TA]) {
+            auto read_a = [&](int sb, i8_intx4(&aop)[2]) {
 #pragma unroll
-                for (int a = 0; a < I8_TA; ++a) {
-                    const uint4 av = *(const uint4 *)(stage + a_off[sb] + (ta0 + a) * (32 * QK_K));
+                for (int a = 0; a < 2; ++a) {
+                    const uint4 av = *(const uint4 *)(stage + a_off[sb] + a * (32 * QK_K));
                     aop[a] = i8_intx4{(int)av.x, (int)av.y, (int)av.z, (int)av.w};
                 }
             };
-            i8_intx4 aop[2][I8_TA];  // A operands of the sub-block in work and of the next one
+            i8_intx4 aop[2][2];  // A operands of the sub-block in work and of the next one
             read_a(0, aop[0]);
             // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
             float d = h2f((uint16_t)(hdr.x & 0xffffu));
@@ -230,19 +217,17 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
             const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
             const uint32_t s3_lo[2] = {sc_lo & 0x07070707u, sc_hi & 0x07070707u};                // sc & 7
             const uint32_t s3_hi[2] = {(sc_lo >> 3) & 0x07070707u, (sc_hi >> 3) & 0x07070707u};  // sc >> 3
-            uint4 wcur[4] = {wq[0], wq[1], wq[2], wq[3]};
 
-            i8_intx16 X[I8_TA], Y[I8_TA], T[I8_TA];
-            float4 da4[I8_TA][4];
+            i8_intx16 X[2], Y[2], T[2];
+            float4 da4[2][4];
             // B operands of sub-block sb: the nibbles times (sc & 7), times (sc >> 3), and the min in every byte. Built
-            // in six pieces, one behind each matrix-core instruction of the previous sub-block, so that the vector
-            // instructions issue while the matrix cores work instead of in front of them.
+            // in six pieces, one behind each matrix-core instruction of the previous sub-block.
             uint32_t nib[4], lo16 = 0, hi16 = 0;
             i8_intx4 bx[2], by[2];
             int bt[2];
             auto prep = [&](int sb, int piece) {
                 const int n = sb & 1;
-                const uint4 src = wcur[sb >> 1];
+                const uint4 src = wq[sb >> 1];
                 switch (piece) {
                 case 0:
                     if (sb & 1) {
@@ -296,48 +281,36 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
                 const int c = sb & 1;
                 if (sb < 7) {
                     read_a(sb + 1, aop[c ^ 1]);  // lands while the MFMAs below run
-                } else if (blk + 1 < nblk) {
-                    read_weights(blk + 1);  // complete since the barrier that opened this round
                 }
                 if (sb == 6) {
                     // activation scales: registers 4 g .. 4 g + 3 of token tile a are tokens 32 a + 8 g + 4 kh .. + 3
 #pragma unroll
-                    for (int a = 0; a < I8_TA; ++a) {
+                    for (int a = 0; a < 2; ++a) {
 #pragma unroll
                         for (int g = 0; g < 4; ++g) {
-                            da4[a][g] = *(const float4 *)(stage + d_off + 4 * (32 * (ta0 + a) + 8 * g));
+                            da4[a][g] = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * g));
                         }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 const i8_intx4 btv = {bt[c], bt[c], bt[c], bt[c]};
 #pragma unroll
-                for (int a = 0; a < I8_TA; ++a) {
-                    constexpr int PP = 2 / I8_TA;  // preparation pieces behind each matrix-core instruction
+                for (int a = 0; a < 2; ++a) {
                     const i8_intx4 av = aop[c][a];
                     const i8_intx16 zero = {0};
                     X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bx[c], sb == 0 ? zero : X[a], 0, 0, 0);
                     if (sb < 7) {
-#pragma unroll
-                        for (int q = 0; q < PP; ++q) {
-                            prep(sb + 1, PP * (3 * a) + q);
-                        }
+                        prep(sb + 1, 3 * a);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, by[c], sb == 0 ? zero : Y[a], 0, 0, 0);
                     if (sb < 7) {
-#pragma unroll
-                        for (int q = 0; q < PP; ++q) {
-                            prep(sb + 1, PP * (3 * a + 1) + q);
-                        }
+                        prep(sb + 1, 3 * a + 1);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, btv, sb == 0 ? zero : T[a], 0, 0, 0);
                     if (sb < 7) {
-#pragma unroll
-                        for (int q = 0; q < PP; ++q) {
-                            prep(sb + 1, PP * (3 * a + 2) + q);
-                        }
+                        prep(sb + 1, 3 * a + 2);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -345,7 +318,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
             // once per block and output: y += a.d * (w.d * isum - w.dmin * msum)
             const float ndmin = -dmin;
 #pragma unroll
-            for (int a = 0; a < I8_TA; ++a) {
+            for (int a = 0; a < 2; ++a) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const float da[4] = {da4[a][g].x, da4[a][g].y, da4[a][g].z, da4[a][g].w};
@@ -358,20 +331,31 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
                     }
                 }
             }
-            i8_lds_barrier();
         }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's share of the next round has landed
+        i8_lds_barrier();
     }
 
-    // ---- the output tile meets in LDS as [token][weight row], then every thread stores 16 bytes per step.
-    // Lane (j, kh) of a compute wavefront holds weight row 32 rg + j for tokens 32 (ta0 + a) + 8 (r / 4) + 4 kh + r % 4.
+    // ---- the two K groups meet in LDS as one [token][weight row] tile, then every thread stores 16 bytes per step.
+    // Lane (j, kh) of a wavefront holds weight row 32 rg + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4.
     float *tile = (float *)lds;
-    if (wave < I8_COMPUTE) {
-        const int rg = wave & 3, ta0 = (wave >> 2) * I8_TA;
+    if (kg == 1) {
 #pragma unroll
-        for (int a = 0; a < I8_TA; ++a) {
+        for (int a = 0; a < 2; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                tile[(32 * (ta0 + a) + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j] = total[a][r];
+                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j] = total[a][r];
+            }
+        }
+    }
+    i8_lds_barrier();
+    if (kg == 0) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j;
+                *e = total[a][r] + *e;
             }
         }
     }

@@ -26,17 +26,27 @@ __device__ __forceinline__ void q8k_block_store(const float (&v)[4], int lane, s
             best_idx = lane * 4 + i;
         }
     }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const float o_abs = __shfl_xor(best_abs, off);
-        const float o_val = __shfl_xor(best_val, off);
-        const int o_idx = __shfl_xor(best_idx, off);
-        if (o_abs > best_abs || (o_abs == best_abs && o_idx < best_idx)) {
-            best_abs = o_abs;
-            best_val = o_val;
-            best_idx = o_idx;
-        }
+    // Across the wavefront: the largest magnitude by data-parallel-primitive moves inside each row of 16 lanes (no LDS
+    // round trips) and a scalar maximum over the four rows; the first lane that holds it is the lowest index, since
+    // lanes hold consecutive values; its signed value comes over as a scalar.
+    float wmax = best_abs;
+    wmax = fmaxf(wmax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, wmax), 0xB1, 0xF, 0xF, true)));
+    wmax = fmaxf(wmax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, wmax), 0x4E, 0xF, 0xF, true)));
+    wmax = fmaxf(wmax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, wmax), 0x141, 0xF, 0xF, true)));
+    wmax = fmaxf(wmax, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, wmax), 0x140, 0xF, 0xF, true)));
+    {
+        const int wi = __builtin_bit_cast(int, wmax);
+        const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(wi, 0));
+        const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(wi, 16));
+        const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(wi, 32));
+        const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(wi, 48));
+        wmax = fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
     }
+    const unsigned long long holders = __ballot(best_abs == wmax);
+    const int first = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(holders | (1ull << 63)));
+    best_val = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, best_val), first));
+    best_abs = wmax;
+    (void)best_idx;
 
     int q[4] = {0, 0, 0, 0};
     float d = 0.0f;
@@ -50,8 +60,8 @@ __device__ __forceinline__ void q8k_block_store(const float (&v)[4], int lane, s
         d = 1.0f / iscale;
     }
     int s = q[0] + q[1] + q[2] + q[3];
-    s += __shfl_xor(s, 1);
-    s += __shfl_xor(s, 2); // lanes 4j..4j+3 hold the sum of values 16j..16j+15
+    s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xF, 0xF, true);  // lane ^ 1
+    s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xF, 0xF, true);  // lane ^ 2: lanes 4j..4j+3 hold the sum of values 16j..16j+15
     const uint32_t packed = (uint32_t)(uint8_t)(int8_t)q[0] | ((uint32_t)(uint8_t)(int8_t)q[1] << 8) |
         ((uint32_t)(uint8_t)(int8_t)q[2] << 16) | ((uint32_t)(uint8_t)(int8_t)q[3] << 24);
 

@@ -117,27 +117,53 @@ __device__ __forceinline__ float load_act_value(const void *x, const void *x2, s
 
 // Q8_K (matmul_quant_pack.c:106-142): one wavefront per 256-value block, 4 consecutive values per lane.
 // AOS = marmot_q8_k_block_t output; otherwise the library's structure-of-arrays scratch.
-template <int SRC, bool AOS>
+// PER_WAVE consecutive blocks per wavefront, all of them requested before the first is quantized.
+template <int SRC, bool AOS, int PER_WAVE>
 __global__ __launch_bounds__(256) void k_quantize_q8_k(const void *__restrict__ x, const void *__restrict__ x2,
                                                        size_t rows, size_t k, size_t nb,
                                                        uint8_t *__restrict__ blocks_out, ActScratch soa) {
     warm_kernel_arguments<6 * 8 + sizeof(ActScratch), 6 * 8 + sizeof(ActScratch)>();
     const int lane = threadIdx.x & 63;
-    const size_t wave = (size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (wave >= rows * nb) {
+    const size_t first = ((size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * PER_WAVE;
+    const size_t total = rows * nb;
+    if (first >= total) {
         return;
     }
-    const size_t row = wave / nb;
-    const size_t b = wave - row * nb;
-    const size_t col0 = b * QK_K + (size_t)lane * 4;
-
-    float v[4];
+    float v[PER_WAVE][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const size_t col = col0 + i;
-        v[i] = col < k ? load_act_value<SRC>(x, x2, row * k + col) : 0.0f;
+    for (int w = 0; w < PER_WAVE; ++w) {
+        const size_t id = first + w < total ? first + w : total - 1;  // beyond the end: re-read, never stored
+        const size_t row = id / nb;
+        const size_t b = id - row * nb;
+        const size_t col0 = b * QK_K + (size_t)lane * 4;
+        bool vec = false;
+        if constexpr (SRC == SRC_F32) {
+            // whole 16-byte groups inside the row: one load instead of four
+            vec = (k & 3) == 0 && ((((uintptr_t)x) & 15) == 0) && col0 + 3 < k;
+            if (vec) {
+                const float4 f = *(const float4 *)((const float *)x + row * k + col0);
+                v[w][0] = f.x;
+                v[w][1] = f.y;
+                v[w][2] = f.z;
+                v[w][3] = f.w;
+            }
+        }
+        if (!vec) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const size_t col = col0 + i;
+                v[w][i] = col < k ? load_act_value<SRC>(x, x2, row * k + col) : 0.0f;
+            }
+        }
     }
-    q8k_block_store<AOS>(v, lane, row, b, nb, blocks_out, soa);
+#pragma unroll
+    for (int w = 0; w < PER_WAVE; ++w) {
+        if (first + w < total) {  // uniform over the wavefront
+            const size_t id = first + w;
+            const size_t row = id / nb;
+            q8k_block_store<AOS>(v[w], lane, row, id - row * nb, nb, blocks_out, soa);
+        }
+    }
 }
 
 // Q8_0 (matmul_quant_pack.c:23-62, block.c:221-232 scalar): 32 lanes per block, one value per lane.
@@ -198,9 +224,11 @@ static int launch_quantize_src(marmot_hip_device *dev, int act_kind, const void 
                                size_t k, uint8_t *blocks_out, const ActScratch &soa) {
     if (act_kind == MARMOT_HIP_KIND_Q8_K) {
         const size_t nb = (k + QK_K - 1) / QK_K;
-        const size_t waves = rows * nb;
-        const dim3 grid((unsigned)((waves + 3) / 4));
-        hipLaunchKernelGGL((k_quantize_q8_k<SRC, AOS>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb,
+        const size_t blocks = rows * nb;
+        // one block per wavefront: the reductions inside a block are a chain of dependent steps, and many resident
+        // wavefronts hide it better than several blocks in one wavefront (measured at 512 x 4096: 7.0 us against 9.0)
+        const dim3 grid((unsigned)((blocks + 3) / 4));
+        hipLaunchKernelGGL((k_quantize_q8_k<SRC, AOS, 1>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb,
                            blocks_out, soa);
     } else {
         const size_t nb = (k + QK - 1) / QK;

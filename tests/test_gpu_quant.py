@@ -69,7 +69,9 @@ def test_dequantize_q8_k_and_golden_blocks(hip, oracle, ref_goldens):
 
 @pytest.mark.parametrize("act_kind", [KIND_Q8_0, KIND_Q8_K])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
-@pytest.mark.parametrize("rows,k", [(1, 2048), (5, 4096), (3, 300), (2, 70), (16, 14336)])
+# (300, 4000), (257, 4099) and (512, 4096): prompt-sized inputs, where a wavefront quantizes four blocks per launch slot
+@pytest.mark.parametrize("rows,k", [(1, 2048), (5, 4096), (3, 300), (2, 70), (16, 14336), (300, 4000), (257, 4099),
+                                    (512, 4096)])
 def test_activation_quantizer_bit_exact(hip, oracle, act_kind, dtype, rows, k):
     print(f"act quant kind={act_kind} {np.dtype(dtype).name} rows={rows} k={k}", flush=True)
     x = gaussian(300 + rows * 7 + k, (rows, k)).astype(dtype)

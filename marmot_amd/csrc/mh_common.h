@@ -215,7 +215,7 @@ struct ActScratch {
 //   MARMOT_HIP_NO_FUSED_QUANT  activation quantization inside the matvec -> separate quantization launch
 //   MARMOT_HIP_NO_GEMM         fp16 prefill GEMM -> fp16 matvec
 //   MARMOT_HIP_NO_GEMM_LOADERS prefill GEMM tile fed by loader wavefronts -> the tile whose wavefronts load for themselves
-//   MARMOT_HIP_NO_GEMM_I8      tiled int8 GEMM on Q8_K activations (48 rows and more) -> 32-row passes of the small-batch kernel
+//   MARMOT_HIP_NO_GEMM_I8      tiled int8 GEMM on Q8_K activations (33 rows and more) -> 32-row passes of the small-batch kernel
 //   MARMOT_HIP_MOE_NO_VALIDATE skip the read-back of the expert-id error flag (no stream synchronization per call)
 struct marmot_hip_knobs {
     bool no_mmq = false;
@@ -369,7 +369,7 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);
-// Tiled int8 GEMM on Q8_K activations (mh_gemm_i8.hip): Q4_K weights, 48 activation rows and more
+// Tiled int8 GEMM on Q8_K activations (mh_gemm_i8.hip): Q4_K weights, 33 activation rows and more
 bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                      const ActScratch &act);
 size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, int weights);

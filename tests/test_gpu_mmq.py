@@ -222,8 +222,8 @@ def test_row_owning_and_streaming_small_batch_kernels(hip, oracle, monkeypatch):
         streaming.close()
 
 
-# ---------------------------------------------------------------- tiled int8 GEMM (Q4_K, 48 activation rows and more)
-@pytest.mark.parametrize("N,M,K", [(48, 128, 256), (64, 100, 512), (100, 203, 2048), (130, 300, 1024), (64, 128, 4096),
+# ---------------------------------------------------------------- tiled int8 GEMM (Q4_K, 33 activation rows and more)
+@pytest.mark.parametrize("N,M,K", [(33, 96, 512), (40, 4096, 1024), (48, 128, 256), (64, 100, 512), (100, 203, 2048), (130, 300, 1024), (64, 128, 4096),
                                    (192, 64, 7168), (512, 512, 4096)])
 def test_tiled_int8_gemm_matches_oracle(hip, oracle, N, M, K):
     """Prefill with fp32 activations: 128 rows x 64 tokens per workgroup on the int8 matrix cores. Full and ragged

@@ -198,6 +198,37 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
+def prefill_int8(hip, tokens: int, steps: int, warmup: int):
+    """Q4_K prefill with fp32 activations (what marmot's own graph feeds): the reference's integer path, i.e. the
+    activations are quantized to Q8_K (one launch) and the tiled int8 GEMM follows; weight 4096 x 4096."""
+    from marmot_amd import DT_F32, capi
+
+    M = K = 4096
+    kind = capi.KIND_Q4_K
+    blocks = random_blocks(np.random.Generator(np.random.PCG64(32)), kind, M, K)
+    x = np.random.Generator(np.random.PCG64(33)).standard_normal((tokens, K), dtype=np.float32)
+    d_w, d_x = hip.to_device(blocks), hip.to_device(x)
+    d_out = hip.alloc(tokens * M * 4)
+    ms = time_steps_graph(hip, lambda i: hip.linear_d(kind, d_w, d_x, DT_F32, tokens, K, M, d_out, DT_F32), steps,
+                          warmup, chunk=20)
+    ops = 2.0 * tokens * M * K
+    out = {
+        "workload": f"Q4_K prefill, weight {M}x{K}, {tokens} tokens fp32 -> Q8_K on device, fp32 out (int8 MFMA, "
+                    f"exact integer block sums, fp32 accumulate over blocks)",
+        "route": hip.last_route(),
+        "ms_per_step": round(ms, 5),
+        "tops": round(ops / (ms * 1e-3) / 1e12, 2),
+        "peak_tops": 5000.0,
+        "frac_of_int8_mfma_peak": round(ops / (ms * 1e-3) / 1e12 / 5000.0, 4),
+        "tokens_per_s": round(tokens / (ms * 1e-3), 1),
+        "steps": steps,
+        "includes": "activation quantization launch and the GEMM kernel",
+    }
+    for b in (d_w, d_x, d_out):
+        b.free()
+    return out
+
+
 def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "OPS", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
     """Every benchmark configuration (C1..C5, QKV, OPS, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
@@ -662,6 +693,8 @@ def main():
     if (args.kind, args.shape, N) == ("q4_k", "4096x14336", 1) and not args.no_prefill:
         # as many steps as it takes for the clocks to settle under the matrix-core load (tens of milliseconds)
         result["prefill_gemm"] = prefill_gemm(hip, args.prefill_tokens, max(100, args.steps // 2),
+                                              max(20, args.steps // 20))
+        result["prefill_int8"] = prefill_int8(hip, args.prefill_tokens, max(100, args.steps // 2),
                                               max(20, args.steps // 20))
     if not args.no_cpu:
         cb, err = cpu_baseline(kind, blocks, x, M, K, nbytes, got, args.cpu_seconds)

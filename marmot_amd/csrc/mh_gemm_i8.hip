@@ -5,7 +5,7 @@
 //     isum = sum_j sc_j * (q_j . a_j),   msum = sum_j mn_j * (sum of a over sub-block j),
 //     y += a.d * (w.d * isum - w.dmin * msum)
 // A workgroup computes 128 weight rows x 64 tokens over a range of blocks. The 6-bit scale is folded into the
-// matrix-core operand, so that the eight sub-block products of a block chain through ONE accumulator and the fp32
+// matrix-core operand, so that the eight sub-block products of a block chain through the accumulators and the fp32
 // work per output happens once per block instead of once per sub-block: sc = 8 * (sc >> 3) + (sc & 7), and both
 // q * (sc & 7) and q * (sc >> 3) are at most 15 * 7 = 105, i.e. int8. Per sub-block and 32 x 32 output tile that is
 //     X += A . (q * (sc & 7)),   Y += A . (q * (sc >> 3)),   T += A . mn        (v_mfma_i32_32x32x32_i8, exact)

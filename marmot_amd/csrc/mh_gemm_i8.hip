@@ -74,6 +74,103 @@ __device__ __forceinline__ int i8_scale_bytes(uint32_t nib, uint32_t s16) {
     return __builtin_bit_cast(int, r);
 }
 
+// The two K groups of a workgroup meet in LDS as one [token][weight row] tile, then every thread stores 16 bytes per
+// step. Lane (j, kh) of wavefront (rg, kg) holds weight row 32 rg + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4. Every
+// wavefront of the workgroup calls this after its last read of the stages (the function contains barriers).
+__device__ __forceinline__ void i8_merge_and_store(const GemmI8Params &p, uint8_t *lds, const float (&total)[2][16],
+                                                   int tid, int rg, int kg, int j, int kh, size_t tt, size_t row0,
+                                                   int split) {
+    float *tile = (float *)lds;
+    if (kg == 1) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j] = total[a][r];
+            }
+        }
+    }
+    i8_lds_barrier();
+    if (kg == 0) {
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j;
+                *e = total[a][r] + *e;
+            }
+        }
+    }
+    i8_lds_barrier();
+
+    const bool partials = p.splits > 1;
+    const bool has_bias = !partials && p.bias != nullptr;
+    const bool out_f16 = !partials && p.out_is_f16;
+    float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
+    const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    for (int idx = tid; idx < I8_TOK * I8_WROWS / 4; idx += I8_THREADS) {
+        const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
+        const size_t n = tt * I8_TOK + (size_t)t;
+        const size_t m4 = row0 + 4 * (size_t)q4;
+        if (n >= p.N || m4 >= p.M) {
+            continue;
+        }
+        const float4 v = *(const float4 *)(tile + t * I8_OUT_PITCH + 4 * q4);
+        const float e4[4] = {v.x, v.y, v.z, v.w};
+        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (m4 + e < p.M) {
+                    bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
+                }
+            }
+        }
+        if (!out_f16) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[e] = has_bias ? e4[e] + bias4[e] : e4[e];
+            }
+            float *dst = out32 + n * p.M + m4;
+            if (vec) {  // M % 4 == 0: the four rows exist
+                *(float4 *)dst = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = o[e];
+                    }
+                }
+            }
+        } else {
+            uint16_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (p.bias_first) {
+                    h[e] = f2h(has_bias ? e4[e] + bias4[e] : e4[e]);
+                } else {
+                    h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
+                    if (has_bias) {
+                        h[e] = f2h(h2f(h[e]) + bias4[e]);
+                    }
+                }
+            }
+            uint16_t *dst = (uint16_t *)p.out + n * p.M + m4;
+            if (vec) {
+                *(uint2 *)dst = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = h[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
 __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Params p) {
     warm_kernel_arguments<sizeof(GemmI8Params)>();
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -336,97 +433,232 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
         i8_lds_barrier();
     }
 
-    // ---- the two K groups meet in LDS as one [token][weight row] tile, then every thread stores 16 bytes per step.
-    // Lane (j, kh) of a wavefront holds weight row 32 rg + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4.
-    float *tile = (float *)lds;
-    if (kg == 1) {
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j] = total[a][r];
-            }
-        }
-    }
-    i8_lds_barrier();
-    if (kg == 0) {
-#pragma unroll
-        for (int a = 0; a < 2; ++a) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j;
-                *e = total[a][r] + *e;
-            }
-        }
-    }
-    i8_lds_barrier();
+    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+}
 
-    const bool partials = p.splits > 1;
-    const bool has_bias = !partials && p.bias != nullptr;
-    const bool out_f16 = !partials && p.out_is_f16;
-    float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
-    const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
-    for (int idx = tid; idx < I8_TOK * I8_WROWS / 4; idx += I8_THREADS) {
-        const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
-        const size_t n = tt * I8_TOK + (size_t)t;
-        const size_t m4 = row0 + 4 * (size_t)q4;
-        if (n >= p.N || m4 >= p.M) {
-            continue;
-        }
-        const float4 v = *(const float4 *)(tile + t * I8_OUT_PITCH + 4 * q4);
-        const float e4[4] = {v.x, v.y, v.z, v.w};
-        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (has_bias) {
+// ------------------------------------------------------------------ Q6_K x Q8_K
+// cpu_vec_dot_q6_k_q8_k (vec_dot_impl.h:783-828): per block y += a.d * w.d * sum_g sc_g * ((u_g - 32) . a_g) over 16
+// groups of 16 values, u the unsigned 6-bit values, sc signed bytes. The scale cannot be folded into an int8 operand
+// here (63 * 127), so every group is one v_mfma_i32_32x32x16_i8 per 32 x 32 tile whose result takes the scale with
+// one integer multiply-add per output, and the offset is taken out as 32 * sum_g sc_g * (sum of a over group g): a
+// second MFMA per group with the scale byte broadcast as the column operand, chained over the groups (exact, like the
+// CPU's use of the stored sums). Same tile and wavefront roles as the Q4_K kernel, except that the two K groups share
+// every block: K group kg takes the block's half kg (128 values = groups 8 kg .. 8 kg + 7, which have their own
+// 64 + 32 bytes of low and high bits), so a round is one block and both groups apply the per-block scales to their
+// partial sums. Blocks are 210 bytes: rows must be a multiple of 8 blocks (16-byte aligned rows); the stage holds for
+// each of the 128 rows the 14 chunks of 16 bytes from the one that contains the block start, at a stride of 240 bytes
+// (the 15th chunk slot is not loaded), and the block is read at offset (210 b) % 16 inside the row slot.
+constexpr int I6_ROWB = 240;
+constexpr int I6_STAGE_W = I8_WROWS * I6_ROWB;                     // 30,720
+constexpr int I6_STAGE = I6_STAGE_W + I8_STAGE_A + I8_STAGE_D;     // 47,360
+constexpr int I6_LDS_BYTES = 2 * I6_STAGE;                         // 94,720
+static_assert(I8_TOK * I8_OUT_PITCH * 4 <= I6_LDS_BYTES, "the output tile reuses the stages");
+static_assert(I6_STAGE % 16 == 0, "stages keep 16-byte alignment");
+
+__global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Params p) {
+    warm_kernel_arguments<sizeof(GemmI8Params)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = wave & 3;   // weight rows 32 rg .. + 31 of the tile
+    const int kg = wave >> 2;  // half of every block
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * I8_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = (int)(b1 - b0);
+    const int j = lane & 31, kh = lane >> 5;
+
+    float total[2][16];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                if (m4 + e < p.M) {
-                    bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
-                }
-            }
-        }
-        if (!out_f16) {
-            float o[4];
+    for (int a = 0; a < 2; ++a) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                o[e] = has_bias ? e4[e] + bias4[e] : e4[e];
-            }
-            float *dst = out32 + n * p.M + m4;
-            if (vec) {  // M % 4 == 0: the four rows exist
-                *(float4 *)dst = make_float4(o[0], o[1], o[2], o[3]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (m4 + e < p.M) {
-                        dst[e] = o[e];
-                    }
-                }
-            }
-        } else {
-            uint16_t h[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                if (p.bias_first) {
-                    h[e] = f2h(has_bias ? e4[e] + bias4[e] : e4[e]);
-                } else {
-                    h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
-                    if (has_bias) {
-                        h[e] = f2h(h2f(h[e]) + bias4[e]);
-                    }
-                }
-            }
-            uint16_t *dst = (uint16_t *)p.out + n * p.M + m4;
-            if (vec) {
-                *(uint2 *)dst = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (m4 + e < p.M) {
-                        dst[e] = h[e];
-                    }
-                }
-            }
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
         }
     }
+
+    // ---- loads: 16 activation instructions (two per wavefront), 30 weight instructions of 64 chunk slots (128 rows x
+    // 15 slots; wavefront w takes instructions w, w + 8, w + 16, w + 24), the activation scales by wavefront 7
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
+    uint32_t a_voff[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const uint32_t t = (uint32_t)(8 * wave + 4 * c + (lane >> 4));
+        const uint32_t slot = (uint32_t)(lane & 15);
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+    }
+    const size_t row_bytes = p.nb * Q6_K_BYTES;
+    const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+    uint32_t w_voff[4];
+    bool w_on[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        const uint32_t q = (uint32_t)(64 * (wave + 8 * m) + lane);  // chunk slot: row q / 15, chunk q % 15
+        const uint32_t r = q / 15u, pc = q - 15u * r;
+        const uint32_t rr = r < last_wrow ? r : last_wrow;  // rows beyond M re-read row M - 1 (never stored)
+        w_voff[m] = rr * (uint32_t)row_bytes + 16u * pc;
+        w_on[m] = wave + 8 * m < 30 && r < (uint32_t)I8_WROWS && pc < 14u;
+    }
+    const uint8_t *wbase = p.w + row0 * row_bytes;
+    uint32_t d_voff;
+    {
+        const uint32_t t = (uint32_t)lane;
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        d_voff = (uint32_t)((trow * p.nb) * 4);
+    }
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
+    auto issue = [&](int bi) {
+        const size_t b = b0 + (size_t)bi;
+        const uint32_t s0 = lds_base + (uint32_t)((bi & 1) * I6_STAGE);
+        const uint8_t *qb = tile_q + b * QK_K;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            dma_set_lds_base(s0 + (uint32_t)(I6_STAGE_W + 2048 * wave + 1024 * c));
+            dma16_to_lds<0>(qb, a_voff[c]);
+        }
+        const uint8_t *wb = wbase + ((b * Q6_K_BYTES) & ~(size_t)15);  // the chunk that contains the block start
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            if (wave + 8 * m < 30) {  // uniform over the wavefront
+                dma_set_lds_base(s0 + (uint32_t)(1024 * (wave + 8 * m)));
+                if (w_on[m]) {
+                    dma16_to_lds<0>(wb, w_voff[m]);
+                }
+            }
+        }
+        if (wave == 7) {
+            dma_set_lds_base(s0 + (uint32_t)(I6_STAGE_W + I8_STAGE_A));
+            dma4_to_lds(tile_d + b * 4, d_voff);
+        }
+    };
+
+    // ---- compute: weight row 32 rg + j, half kg of the block, all 64 tokens
+    const uint32_t w_off = (uint32_t)((32 * rg + j) * I6_ROWB);
+    const uint32_t a_base = (uint32_t)(I6_STAGE_W + j * QK_K + 8 * kh);
+    const uint32_t d_off = (uint32_t)(I6_STAGE_W + I8_STAGE_A + 16 * kh);
+
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    i8_lds_barrier();
+    for (int blk = 0; blk < nblk; ++blk) {
+        if (blk + 1 < nblk) {
+            issue(blk + 1);  // into the other buffer, which the barrier that closed the previous block has released
+        }
+        {
+            const uint8_t *stage = lds + (size_t)(blk & 1) * I6_STAGE;
+            const int o = (int)(((b0 + (size_t)blk) * Q6_K_BYTES) & 15);
+            const uint8_t *wrow = stage + w_off + o;
+            uint2 scv;  // the eight scale bytes of this half
+            __builtin_memcpy(&scv, wrow + 192 + 8 * kg, 8);
+            uint16_t dh;
+            __builtin_memcpy(&dh, wrow + 208, 2);
+            float d = h2f(dh);
+            asm volatile("" : "+v"(d));
+            uint2 ql[2][2], qh[2];  // [second 32][second 16], [second 16]: this lane's 8 bytes each
+#pragma unroll
+            for (int s16 = 0; s16 < 2; ++s16) {
+                __builtin_memcpy(&qh[s16], wrow + 128 + 32 * kg + 16 * s16 + 8 * kh, 8);
+#pragma unroll
+                for (int h32 = 0; h32 < 2; ++h32) {
+                    __builtin_memcpy(&ql[h32][s16], wrow + 64 * kg + 32 * h32 + 16 * s16 + 8 * kh, 8);
+                }
+            }
+            const uint32_t scw[2] = {scv.x, scv.y};
+            // group g of this half (block group 8 kg + g): token tile a's 8 bytes of chunk 8 kg + g, swizzled by token
+            auto acts_of = [&](int g, int a) {
+                const uint2 v = *(const uint2 *)(stage + a_base + a * (32 * QK_K) + 16 * ((8 * kg + g) ^ (j & 15)));
+                return (long)(((unsigned long)v.y << 32) | v.x);
+            };
+            auto weights_of = [&](int g) {
+                const int q = (g >> 1) & 3, s16 = g & 1;
+                const uint2 l = ql[q & 1][s16], hh = qh[s16];
+                uint32_t x = (q >> 1) ? ((l.x >> 4) & 0x0f0f0f0fu) : (l.x & 0x0f0f0f0fu);
+                uint32_t y = (q >> 1) ? ((l.y >> 4) & 0x0f0f0f0fu) : (l.y & 0x0f0f0f0fu);
+                x |= ((hh.x >> (2 * q)) & 0x03030303u) << 4;
+                y |= ((hh.y >> (2 * q)) & 0x03030303u) << 4;
+                return (long)(((unsigned long)y << 32) | x);
+            };
+            int bsum[2][16];
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    bsum[a][r] = 0;
+                }
+            }
+            const i8_intx16 zero = {0};
+            i8_intx16 ds[2] = {zero, zero};
+            i8_intx16 dq[2][2];  // [token tile][group parity]
+            long av[2][2];
+            float4 da4[2][4];
+            long wv = weights_of(0);
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                av[a][0] = acts_of(0, a);
+                dq[a][0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[a][0], wv, zero, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                const int c = g & 1;
+                const uint32_t scb = (scw[g >> 2] >> (8 * (g & 3))) & 0xffu;
+                const int sc = (int)(int8_t)scb;
+                const uint32_t sc4 = __builtin_amdgcn_perm(0u, scw[g >> 2], 0x01010101u * (g & 3));  // byte broadcast
+                const long scl = (long)(((unsigned long)sc4 << 32) | sc4);
+                if (g < 7) {
+                    wv = weights_of(g + 1);
+                }
+                if (g == 5) {
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; ++q4) {
+                            da4[a][q4] = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * q4));
+                        }
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    ds[a] = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[a][c], scl, ds[a], 0, 0, 0);
+                    if (g < 7) {
+                        av[a][c ^ 1] = acts_of(g + 1, a);
+                        dq[a][c ^ 1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(av[a][c ^ 1], wv, zero, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        bsum[a][r] += __mul24(dq[a][c][r], sc);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // once per block, output and K group: y += (a.d * w.d) * (isum - 32 * ssum)
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const float da[4] = {da4[a][q4].x, da4[a][q4].y, da4[a][q4].z, da4[a][q4].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = 4 * q4 + e;
+                        const int isum = bsum[a][r] - (ds[a][r] << 5);
+                        total[a][r] = __builtin_fmaf(da[e] * d, (float)isum, total[a][r]);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's share of the next block has landed
+        i8_lds_barrier();
+    }
+    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
 // ------------------------------------------------------------------ host side
@@ -451,11 +683,20 @@ static size_t gemm_i8_splits(const marmot_hip_device *dev, size_t N, size_t M, s
 
 bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                      const ActScratch &act) {
-    if (dev->knobs.no_gemm_i8 || kind != MARMOT_HIP_KIND_Q4_K || N < I8_MIN_ROWS || K % QK_K != 0) {
+    if (dev->knobs.no_gemm_i8 || N < I8_MIN_ROWS || K % QK_K != 0) {
+        return false;
+    }
+    size_t block_bytes = Q4_K_BYTES;
+    if (kind == MARMOT_HIP_KIND_Q6_K) {
+        if ((K / QK_K) % 8 != 0) {
+            return false;  // rows of 210-byte blocks are 16-byte aligned only then
+        }
+        block_bytes = Q6_K_BYTES;
+    } else if (kind != MARMOT_HIP_KIND_Q4_K) {
         return false;
     }
     if ((((uintptr_t)act.qs) & 15) != 0 || act.kp % 16 != 0 || N * act.kp >= ((size_t)1 << 32) ||
-        N * (K / QK_K) * 4 >= ((size_t)1 << 32) || I8_WROWS * (K / QK_K) * Q4_K_BYTES >= ((size_t)1 << 32)) {
+        N * (K / QK_K) * 4 >= ((size_t)1 << 32) || I8_WROWS * (K / QK_K) * block_bytes >= ((size_t)1 << 32)) {
         return false;  // 16-byte direct-to-LDS loads with 32-bit lane offsets
     }
     for (int i = 0; i < count; ++i) {
@@ -472,8 +713,9 @@ size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, s
     return splits > 1 ? splits * N * M * sizeof(float) * (size_t)weights : 0;
 }
 
-int launch_gemm_i8(marmot_hip_device *dev, const WeightSet &ws, const ActScratch &act, size_t N, size_t K, size_t M,
-                   int out_dtype, void *scratch) {
+int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
+                   size_t M, int out_dtype, void *scratch) {
+    const bool q6 = kind == MARMOT_HIP_KIND_Q6_K;
     const size_t nb = K / QK_K;
     size_t bps = 0;
     const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
@@ -484,6 +726,7 @@ int launch_gemm_i8(marmot_hip_device *dev, const WeightSet &ws, const ActScratch
         partial = (float *)wsp;
     }
     MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_q8k_tile));
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q6k_q8k_tile));
     const dim3 grid((unsigned)((M + I8_WROWS - 1) / I8_WROWS), (unsigned)((N + I8_TOK - 1) / I8_TOK), (unsigned)splits);
     for (int which = 0; which < ws.count; ++which) {
         GemmI8Params p;
@@ -502,14 +745,18 @@ int launch_gemm_i8(marmot_hip_device *dev, const WeightSet &ws, const ActScratch
         p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
         p.bias_first = ws.bias_first ? 1 : 0;
         p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
-        hipLaunchKernelGGL(k_gemm_q4k_q8k_tile, grid, dim3(I8_THREADS), I8_LDS_BYTES, dev->stream, p);
+        if (q6) {
+            hipLaunchKernelGGL(k_gemm_q6k_q8k_tile, grid, dim3(I8_THREADS), I6_LDS_BYTES, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL(k_gemm_q4k_q8k_tile, grid, dim3(I8_THREADS), I8_LDS_BYTES, dev->stream, p);
+        }
         MH_HIP(hipGetLastError());
         if (splits > 1) {
             MH_TRY(launch_splitk_reduce(dev, part, (int)splits, N, M, ws.bias[which], ws.bias_dtype, ws.out[which],
                                         out_dtype, ws.bias_first));
         }
     }
-    set_route("mmq_q4_k_q8_k_mfma_tile");
+    set_route(q6 ? "mmq_q6_k_q8_k_mfma_tile" : "mmq_q4_k_q8_k_mfma_tile");
     return MARMOT_HIP_SUCCESS;
 }
 

@@ -910,7 +910,8 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_
     const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K, weights);
     const size_t passes = pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (size_t)weights : 0;
     // the tiled GEMM may take the call instead (decided at launch, when the operands' alignment is known)
-    const size_t tiled = (kind == MARMOT_HIP_KIND_Q4_K && !dev->knobs.no_gemm_i8) ? gemm_i8_scratch_bytes(dev, N, K, M, weights) : 0;
+    const size_t tiled = ((kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && !dev->knobs.no_gemm_i8)
+        ? gemm_i8_scratch_bytes(dev, N, K, M, weights) : 0;
     return passes > tiled ? passes : tiled;
 }
 
@@ -1042,7 +1043,7 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "small-batch MFMA matmul: unsupported kind or shape");
     }
     if (gemm_i8_applies(dev, kind, N, K, ws.w, ws.count, act)) {
-        return launch_gemm_i8(dev, ws, act, N, K, M, out_dtype, scratch);
+        return launch_gemm_i8(dev, kind, ws, act, N, K, M, out_dtype, scratch);
     }
     const size_t nb = K / QK_K;
     const MmqPlan pl = mmq_plan(dev, kind, N, M, nb, ws.count);

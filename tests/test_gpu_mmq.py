@@ -318,3 +318,93 @@ def test_tiled_int8_gemm_integers_are_exact(hip):
     for b_ in (d_w, d_p, d_out):
         b_.free()
     assert np.array_equal(bits(got), bits(want))
+
+
+@pytest.mark.parametrize("N,M,K", [(33, 96, 2048), (64, 128, 2048), (100, 203, 4096), (130, 300, 6144), (64, 128, 14336),
+                                   (512, 512, 4096)])
+def test_tiled_int8_gemm_q6k_matches_oracle(hip, oracle, N, M, K):
+    """The Q6_K form of the tile kernel (rows of a multiple of 8 blocks): blocks at every offset inside a 16-byte chunk,
+    ragged tiles, K split across workgroups, bias. Rows of another length keep the 32-row passes."""
+    kind = KIND_Q6_K
+    blocks = oracle.quantize(kind, gaussian(430 + N, (M, K), 0.02))
+    x = gaussian(431 + N, (N, K))
+    bias = gaussian(432, (M,))
+    got = hip.linear(x, blocks, kind, M, bias=bias)
+    assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"Q6_K tile {M}x{K} N={N}")
+    if K == 2048:
+        K2 = 1024 + 256  # five blocks per row: rows are not 16-byte aligned
+        b2 = oracle.quantize(kind, gaussian(433, (M, K2), 0.02))
+        x2 = gaussian(434, (N, K2))
+        got2 = hip.linear(x2, b2, kind, M)
+        assert hip.last_route() == "mmq_q6_k_q8_k_mfma"
+        assert_matmul_parity(got2, oracle.matmul(kind, b2, x2, M), what="Q6_K passes, unaligned rows")
+
+
+def test_tiled_int8_gemm_q6k_random_blocks_and_exact_integers(hip, oracle):
+    """Arbitrary Q6_K block bytes against the oracle; then packed activations and blocks whose scales are powers of two:
+    the output must equal, bit for bit, a.d * w.d * (sum_g sc_g * ((u_g - 32) . a_g)) formed in exact integer
+    arithmetic per half block and added the way the kernel adds (each half of a workgroup's blocks in block order, the
+    two halves, then the workgroups along K)."""
+    kind = KIND_Q6_K
+    N, M, K = 70, 200, 2048
+    nb = K // 256
+    rng = np.random.default_rng(440)
+    blocks = random_valid_blocks(rng, kind, M, K)
+    x = gaussian(441, (N, K))
+    got = hip.linear(x, blocks, kind, M)
+    assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what="Q6_K tile, random blocks")
+
+    blocks = blocks.reshape(M, nb, 210).copy()
+    d_exp = rng.integers(-14, -8, size=(M, nb))
+    blocks[:, :, 208:210] = np.ldexp(1.0, d_exp).astype(np.float16).view(np.uint8).reshape(M, nb, 2)
+    blocks[:, :, 192:208] = rng.integers(-31, 32, size=(M, nb, 16)).astype(np.int8).view(np.uint8)  # keeps sums < 2^24
+    q = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+    a_exp = rng.integers(-8, -2, size=(N, nb))
+    lay = hip.packed_activation_layout(kind, N, K)
+    image = np.zeros(lay.total_bytes, np.uint8)
+    vals = np.zeros((N, lay.values_per_row), np.int8)
+    vals[:, :K] = q
+    image[lay.values_offset:lay.values_offset + vals.size] = vals.view(np.uint8).reshape(-1)
+    ad = np.ldexp(1.0, a_exp).astype(np.float32)
+    image[lay.scales_offset:lay.scales_offset + ad.nbytes] = ad.view(np.uint8).reshape(-1)
+    sums = q.reshape(N, K // 16, 16).astype(np.int16).sum(axis=2, dtype=np.int16)
+    image[lay.sums_offset:lay.sums_offset + sums.nbytes] = sums.view(np.uint8).reshape(-1)
+    # the 6-bit values of a block (q6k_gguf.c:63-99): value 128 h + 32 q + l = (ql[64 h + 32 (q & 1) + l] nibble q >> 1)
+    # | ((qh[32 h + l] >> 2 q) & 3) << 4, minus 32; group 16 values
+    ql = blocks[:, :, 0:128].astype(np.int64).reshape(M, nb, 2, 2, 32)    # [h][q & 1][l]
+    qh = blocks[:, :, 128:192].astype(np.int64).reshape(M, nb, 2, 32)     # [h][l]
+    u = np.zeros((M, nb, 2, 4, 32), np.int64)
+    for qq in range(4):
+        nib = (ql[:, :, :, qq & 1, :] >> 4) if (qq >> 1) else (ql[:, :, :, qq & 1, :] & 15)
+        u[:, :, :, qq, :] = nib | (((qh >> (2 * qq)) & 3) << 4)
+    w = (u - 32).reshape(M, nb, 2, 8, 16)                                  # [half][group of the half][16]
+    sc = blocks[:, :, 192:208].view(np.int8).astype(np.int64).reshape(M, nb, 2, 8)
+    a = q.astype(np.int64).reshape(N, nb, 2, 8, 16)
+    # four tiles on a chip of `cus` compute units: K is split over workgroups (at least two blocks each), every
+    # workgroup adds its two halves, and the reduction adds the workgroups' partial sums in order, starting from zero
+    cus = hip.caps()["num_compute_units"]
+    tiles = -(-N // 64) * -(-M // 128)
+    splits = min(cus // tiles, nb // 2) if tiles * 2 <= cus else 1
+    per_split = -(-nb // max(splits, 1))
+    want = np.zeros((N, M), np.float32)
+    for b_lo in range(0, nb, per_split):
+        halves = [np.zeros((N, M), np.float32), np.zeros((N, M), np.float32)]
+        for b in range(b_lo, min(nb, b_lo + per_split)):
+            scale = (np.ldexp(1.0, a_exp[:, b, None]).astype(np.float32) *
+                     np.ldexp(1.0, d_exp[None, :, b]).astype(np.float32))
+            for h in range(2):
+                dots = np.einsum("ngk,mgk->nmg", a[:, b, h], w[:, b, h])      # [N, M, 8]
+                isum = (dots * sc[None, :, b, h, :]).sum(axis=2)
+                assert np.abs(isum).max() < 2 ** 24
+                halves[h] = (halves[h] + scale * isum.astype(np.float32)).astype(np.float32)
+        part = (halves[0] + halves[1]).astype(np.float32)
+        want = part if per_split >= nb else (want + part).astype(np.float32)
+    d_w, d_p, d_out = hip.to_device(blocks.reshape(M, nb * 210)), hip.to_device(image), hip.alloc(N * M * 4)
+    hip.linear_prepacked_d(kind, d_w, d_p, N, K, M, d_out)
+    assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
+    got = d_out.download(np.float32, (N, M))
+    for b_ in (d_w, d_p, d_out):
+        b_.free()
+    assert np.array_equal(bits(got), bits(want))

@@ -649,7 +649,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int r = 4 * q4 + e;
-                        const int isum = bsum[a][r] - (ds[a][r] << 5);
+                        const int isum = bsum[a][r] + __mul24(ds[a][r], -32);  // one multiply-add; |ds| < 2^22
                         total[a][r] = __builtin_fmaf(da[e] * d, (float)isum, total[a][r]);
                     }
                 }

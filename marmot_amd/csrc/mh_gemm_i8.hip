@@ -436,6 +436,334 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
     i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
+// ------------------------------------------------------------------ Q5_K x Q8_K
+// The Q4_K kernel with the fifth bit (cpu_vec_dot_q5_k_q8_k, vec_dot_impl.h:734-781): q5 = q4 + 16 bit, so
+// isum = sum_j sc_j * (q4_j . a_j) + 16 * sum_j sc_j * (bit_j . a_j); the second sum is one more scale plane,
+// bit * sc <= 63. Blocks are 176 bytes (11 chunks of 16 per row): two round buffers of 2 x 39,168 bytes.
+constexpr int I5_STAGE_W = I8_WROWS * Q5_K_BYTES;                  // 22,528
+constexpr int I5_STAGE = I8_STAGE_A + I5_STAGE_W + I8_STAGE_D;     // 39,168
+constexpr int I5_ROUND = 2 * I5_STAGE;
+constexpr int I5_LDS_BYTES = 2 * I5_ROUND;                         // 156,672 of 163,840
+static_assert(I5_STAGE % 16 == 0, "stages keep 16-byte alignment");
+
+__global__ __launch_bounds__(I8_THREADS) void k_gemm_q5k_q8k_tile(const GemmI8Params p) {
+    warm_kernel_arguments<sizeof(GemmI8Params)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = wave & 3;   // weight rows 32 rg .. + 31 of the tile; also this wavefront's share of the loads
+    const int kg = wave >> 2;  // K group: blocks b0 + kg, b0 + kg + 2, ...
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * I8_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = (int)(b1 - b0);
+    const int rounds = (nblk + 1) / 2;
+    const int j = lane & 31, kh = lane >> 5;
+
+    float total[2][16];  // [token tile][register]
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
+        }
+    }
+
+    // ---- loads: the four wavefronts of a K group bring that group's block of every round, a quarter each
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);  // token rows beyond it re-read it
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
+    // Activation tile: token t owns 256 bytes of the stage as 16 chunks of 16 bytes, chunk c stored in slot
+    // c ^ (t % 16) (the MFMA operand reads of 32 tokens x one chunk then spread over the bank groups). One
+    // instruction moves four token rows; wavefront rg brings tokens 16 rg .. 16 rg + 15.
+    uint32_t a_voff[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t t = (uint32_t)(16 * rg + 4 * c + (lane >> 4));
+        const uint32_t slot = (uint32_t)(lane & 15);
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+    }
+    // Weight blocks: piece q of the stage is 16 bytes q % 11 of tile row q / 11; wavefront rg brings pieces
+    // 256 pass + 64 rg + lane. Rows beyond M re-read row M - 1 (never stored).
+    const size_t row_bytes = p.nb * Q5_K_BYTES;
+    const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+    uint32_t w_voff[6];
+#pragma unroll
+    for (int pass = 0; pass < 6; ++pass) {
+        const uint32_t q = (uint32_t)(256 * pass + 64 * rg + lane);
+        const uint32_t r = q / 11u, c11 = q - 11u * r;
+        const uint32_t rr = r < last_wrow ? r : last_wrow;
+        w_voff[pass] = rr * (uint32_t)row_bytes + 16u * c11;
+    }
+    const uint8_t *wbase = p.w + row0 * row_bytes;
+    const bool sixth = rg < 2;    // pieces 1280 .. 1407
+    const bool scales = rg == 3;  // the 64 activation scales of the block
+    uint32_t d_voff;
+    {
+        const uint32_t t = (uint32_t)lane;
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        d_voff = (uint32_t)((trow * p.nb) * 4);
+    }
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
+    // block b0 + 2 round + kg into the K group's half of round buffer round % 2 (nothing when the block does not exist)
+    auto issue = [&](int round) {
+        const int bi = 2 * round + kg;
+        if (bi >= nblk) {
+            return;
+        }
+        const size_t b = b0 + (size_t)bi;
+        const uint32_t s0 = lds_base + (uint32_t)((round & 1) * I5_ROUND + kg * I5_STAGE);
+        const uint8_t *qb = tile_q + b * QK_K;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            dma_set_lds_base(s0 + (uint32_t)(4096 * rg + 1024 * c));
+            dma16_to_lds<0>(qb, a_voff[c]);
+        }
+        const uint8_t *wb = wbase + b * Q5_K_BYTES;
+#pragma unroll
+        for (int pass = 0; pass < 5; ++pass) {
+            dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (256 * pass + 64 * rg) * 16));
+            dma16_to_lds<0>(wb, w_voff[pass]);
+        }
+        if (sixth) {
+            dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + (1280 + 64 * rg) * 16));
+            dma16_to_lds<0>(wb, w_voff[5]);
+        }
+        if (scales) {
+            dma_set_lds_base(s0 + (uint32_t)(I8_STAGE_A + I5_STAGE_W));
+            dma4_to_lds(tile_d + b * 4, d_voff);
+        }
+    };
+
+    // ---- compute: this wavefront's weight row 32 rg + j of its K group's block, all 64 tokens
+    const uint32_t w_off = (uint32_t)(kg * I5_STAGE + I8_STAGE_A + (32 * rg + j) * Q5_K_BYTES);
+    // A operand of sub-block sb, token tile a, lane (j, kh): token 32 a + j, chunk 2 sb + kh at slot chunk ^ (j % 16)
+    uint32_t a_off[8];
+#pragma unroll
+    for (int sb = 0; sb < 8; ++sb) {
+        a_off[sb] = (uint32_t)(kg * I5_STAGE + j * QK_K + 16 * ((2 * sb + kh) ^ (j & 15)));
+    }
+    const uint32_t d_off = (uint32_t)(kg * I5_STAGE + I8_STAGE_A + I5_STAGE_W + 16 * kh);
+
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    i8_lds_barrier();
+    for (int round = 0; round < rounds; ++round) {
+        // the next round's blocks land in the other buffer while this round computes: the barrier that closed the
+        // previous round guarantees that nobody reads that buffer any more
+        if (round + 1 < rounds) {
+            issue(round + 1);
+        }
+        if (2 * round + kg < nblk) {
+            const uint8_t *stage = lds + (size_t)(round & 1) * I5_ROUND;
+            const uint8_t *wr = stage + w_off;
+            const uint4 hdr = *(const uint4 *)wr;
+            uint4 wq[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                wq[g] = *(const uint4 *)(wr + 48 + 32 * g + 16 * kh);
+            }
+            // fifth bits of this lane's 16 positions: bit sb of byte l belongs to sub-block sb (q5k_gguf.c:162-198)
+            const uint4 wqh = *(const uint4 *)(wr + 16 + 16 * kh);
+            auto read_a = [&](int sb, i8_intx4(&aop)[2]) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const uint4 av = *(const uint4 *)(stage + a_off[sb] + a * (32 * QK_K));
+                    aop[a] = i8_intx4{(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                }
+            };
+            i8_intx4 aop[2][2];  // A operands of the sub-block in work and of the next one
+            read_a(0, aop[0]);
+            // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
+            float d = h2f((uint16_t)(hdr.x & 0xffffu));
+            float dmin = h2f((uint16_t)(hdr.x >> 16));
+            asm volatile("" : "+v"(d), "+v"(dmin));  // plain fp32 values: no mixed-precision multiply-adds below
+            const uint32_t sc_lo = hdr.y & 0x3f3f3f3fu;
+            const uint32_t mn_lo = hdr.z & 0x3f3f3f3fu;
+            const uint32_t sc_hi = (hdr.w & 0x0f0f0f0fu) | (((hdr.y >> 6) & 0x03030303u) << 4);
+            const uint32_t mn_hi = ((hdr.w >> 4) & 0x0f0f0f0fu) | (((hdr.z >> 6) & 0x03030303u) << 4);
+            const uint32_t s3_lo[2] = {sc_lo & 0x07070707u, sc_hi & 0x07070707u};                // sc & 7
+            const uint32_t s3_hi[2] = {(sc_lo >> 3) & 0x07070707u, (sc_hi >> 3) & 0x07070707u};  // sc >> 3
+
+            // Two sweeps over the eight sub-blocks, so that three accumulator chains are never live together with the
+            // partial sums of the other two. First the Q4_K part, X += A . (q4 * (sc & 7)), Y += A . (q4 * (sc >> 3)),
+            // folded into P = X + 8 Y; then Z += A . (bit * sc) (the fifth bit times the whole 6-bit scale is at most
+            // 63) and T += A . mn, which read the activation operands a second time. isum = P + 16 Z, msum = T.
+            i8_intx16 X[2], Y[2];
+            float4 da4[2][4];
+            uint32_t nib[4], lo16 = 0, hi16 = 0;
+            i8_intx4 bx[2], by[2];
+            auto prep1 = [&](int sb, int piece) {
+                const int n = sb & 1;
+                const uint4 src = wq[sb >> 1];
+                switch (piece) {
+                case 0:
+                    if (sb & 1) {
+                        nib[0] = (src.x >> 4) & 0x0f0f0f0fu;
+                        nib[1] = (src.y >> 4) & 0x0f0f0f0fu;
+                        nib[2] = (src.z >> 4) & 0x0f0f0f0fu;
+                        nib[3] = (src.w >> 4) & 0x0f0f0f0fu;
+                    } else {
+                        nib[0] = src.x & 0x0f0f0f0fu;
+                        nib[1] = src.y & 0x0f0f0f0fu;
+                        nib[2] = src.z & 0x0f0f0f0fu;
+                        nib[3] = src.w & 0x0f0f0f0fu;
+                    }
+                    break;
+                case 1: {
+                    const uint32_t sel16 = 0x0c000c00u | (uint32_t)(sb & 3) | ((uint32_t)(sb & 3) << 16);
+                    lo16 = __builtin_amdgcn_perm(0u, s3_lo[sb >> 2], sel16);
+                    hi16 = __builtin_amdgcn_perm(0u, s3_hi[sb >> 2], sel16);
+                    bx[n][0] = i8_scale_bytes(nib[0], lo16);
+                    bx[n][1] = i8_scale_bytes(nib[1], lo16);
+                    break;
+                }
+                case 2:
+                    bx[n][2] = i8_scale_bytes(nib[2], lo16);
+                    bx[n][3] = i8_scale_bytes(nib[3], lo16);
+                    by[n][0] = i8_scale_bytes(nib[0], hi16);
+                    break;
+                default:
+                    by[n][1] = i8_scale_bytes(nib[1], hi16);
+                    by[n][2] = i8_scale_bytes(nib[2], hi16);
+                    by[n][3] = i8_scale_bytes(nib[3], hi16);
+                    break;
+                }
+            };
+#pragma unroll
+            for (int piece = 0; piece < 4; ++piece) {
+                prep1(0, piece);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                const int c = sb & 1;
+                read_a(sb < 7 ? sb + 1 : 0, aop[c ^ 1]);  // the next sub-block's operands; at the end, the second sweep's first
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const i8_intx4 av = aop[c][a];
+                    const i8_intx16 zero = {0};
+                    X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bx[c], sb == 0 ? zero : X[a], 0, 0, 0);
+                    if (sb < 7) {
+                        prep1(sb + 1, 2 * a);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    Y[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, by[c], sb == 0 ? zero : Y[a], 0, 0, 0);
+                    if (sb < 7) {
+                        prep1(sb + 1, 2 * a + 1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // second sweep: bz = fifth bits times the 6-bit scale, bt = the min in every byte
+            i8_intx4 bz[2];
+            int bt[2];
+            uint32_t bits[4], sc16 = 0;
+            auto prep2 = [&](int sb, int piece) {
+                const int n = sb & 1;
+                switch (piece) {
+                case 0:
+                    bits[0] = (wqh.x >> sb) & 0x01010101u;
+                    bits[1] = (wqh.y >> sb) & 0x01010101u;
+                    break;
+                case 1:
+                    bits[2] = (wqh.z >> sb) & 0x01010101u;
+                    bits[3] = (wqh.w >> sb) & 0x01010101u;
+                    break;
+                case 2: {
+                    const uint32_t sel16 = 0x0c000c00u | (uint32_t)(sb & 3) | ((uint32_t)(sb & 3) << 16);
+                    sc16 = __builtin_amdgcn_perm(0u, sb < 4 ? sc_lo : sc_hi, sel16);
+                    bt[n] = (int)__builtin_amdgcn_perm(0u, sb < 4 ? mn_lo : mn_hi, 0x01010101u * (sb & 3));
+                    bz[n][0] = i8_scale_bytes(bits[0], sc16);
+                    break;
+                }
+                default:
+                    bz[n][1] = i8_scale_bytes(bits[1], sc16);
+                    bz[n][2] = i8_scale_bytes(bits[2], sc16);
+                    bz[n][3] = i8_scale_bytes(bits[3], sc16);
+                    break;
+                }
+            };
+#pragma unroll
+            for (int piece = 0; piece < 4; ++piece) {
+                prep2(0, piece);
+            }
+            // P = X + 8 Y takes X's registers; Y's become free for the second sweep
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    X[a][r] = X[a][r] + (Y[a][r] << 3);
+                }
+            }
+            i8_intx16 Z[2], T[2];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                const int c = sb & 1;  // sweep 1 ended with sub-block 0's operands in aop[0]
+                if (sb < 7) {
+                    read_a(sb + 1, aop[c ^ 1]);
+                }
+                if (sb == 6) {
+                    // activation scales: registers 4 g .. 4 g + 3 of token tile a are tokens 32 a + 8 g + 4 kh .. + 3
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            da4[a][g] = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * g));
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const i8_intx4 btv = {bt[c], bt[c], bt[c], bt[c]};
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const i8_intx4 av = aop[c][a];
+                    const i8_intx16 zero = {0};
+                    Z[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bz[c], sb == 0 ? zero : Z[a], 0, 0, 0);
+                    if (sb < 7) {
+                        prep2(sb + 1, 2 * a);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    T[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, btv, sb == 0 ? zero : T[a], 0, 0, 0);
+                    if (sb < 7) {
+                        prep2(sb + 1, 2 * a + 1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            // once per block and output: y += a.d * (w.d * isum - w.dmin * msum)
+            const float ndmin = -dmin;
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float da[4] = {da4[a][g].x, da4[a][g].y, da4[a][g].z, da4[a][g].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = 4 * g + e;
+                        const int isum = X[a][r] + (Z[a][r] << 4);
+                        const float v = __builtin_fmaf(ndmin, (float)T[a][r], d * (float)isum);
+                        total[a][r] = __builtin_fmaf(da[e], v, total[a][r]);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's share of the next round has landed
+        i8_lds_barrier();
+    }
+
+    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+}
+
 // ------------------------------------------------------------------ Q6_K x Q8_K
 // cpu_vec_dot_q6_k_q8_k (vec_dot_impl.h:783-828): per block y += a.d * w.d * sum_g sc_g * ((u_g - 32) . a_g) over 16
 // groups of 16 values, u the unsigned 6-bit values, sc signed bytes. The scale cannot be folded into an int8 operand
@@ -687,7 +1015,9 @@ bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K,
         return false;
     }
     size_t block_bytes = Q4_K_BYTES;
-    if (kind == MARMOT_HIP_KIND_Q6_K) {
+    if (kind == MARMOT_HIP_KIND_Q5_K) {
+        block_bytes = Q5_K_BYTES;
+    } else if (kind == MARMOT_HIP_KIND_Q6_K) {
         if ((K / QK_K) % 8 != 0) {
             return false;  // rows of 210-byte blocks are 16-byte aligned only then
         }
@@ -715,7 +1045,7 @@ size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, s
 
 int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                    size_t M, int out_dtype, void *scratch) {
-    const bool q6 = kind == MARMOT_HIP_KIND_Q6_K;
+    const bool q6 = kind == MARMOT_HIP_KIND_Q6_K, q5 = kind == MARMOT_HIP_KIND_Q5_K;
     const size_t nb = K / QK_K;
     size_t bps = 0;
     const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
@@ -727,6 +1057,7 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
     }
     MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_q8k_tile));
     MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q6k_q8k_tile));
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q5k_q8k_tile));
     const dim3 grid((unsigned)((M + I8_WROWS - 1) / I8_WROWS), (unsigned)((N + I8_TOK - 1) / I8_TOK), (unsigned)splits);
     for (int which = 0; which < ws.count; ++which) {
         GemmI8Params p;
@@ -747,6 +1078,8 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
         p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
         if (q6) {
             hipLaunchKernelGGL(k_gemm_q6k_q8k_tile, grid, dim3(I8_THREADS), I6_LDS_BYTES, dev->stream, p);
+        } else if (q5) {
+            hipLaunchKernelGGL(k_gemm_q5k_q8k_tile, grid, dim3(I8_THREADS), I5_LDS_BYTES, dev->stream, p);
         } else {
             hipLaunchKernelGGL(k_gemm_q4k_q8k_tile, grid, dim3(I8_THREADS), I8_LDS_BYTES, dev->stream, p);
         }
@@ -756,7 +1089,7 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
                                         out_dtype, ws.bias_first));
         }
     }
-    set_route(q6 ? "mmq_q6_k_q8_k_mfma_tile" : "mmq_q4_k_q8_k_mfma_tile");
+    set_route(q6 ? "mmq_q6_k_q8_k_mfma_tile" : q5 ? "mmq_q5_k_q8_k_mfma_tile" : "mmq_q4_k_q8_k_mfma_tile");
     return MARMOT_HIP_SUCCESS;
 }
 

@@ -910,7 +910,7 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_
     const MmqPlan pl = mmq_plan(dev, kind, N, M, K / QK_K, weights);
     const size_t passes = pl.S > 1 ? (size_t)pl.S * N * M * sizeof(float) * (size_t)weights : 0;
     // the tiled GEMM may take the call instead (decided at launch, when the operands' alignment is known)
-    const size_t tiled = ((kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q6_K) && !dev->knobs.no_gemm_i8)
+    const size_t tiled = ((mmq_is_q4k_family(kind) || kind == MARMOT_HIP_KIND_Q6_K) && !dev->knobs.no_gemm_i8)
         ? gemm_i8_scratch_bytes(dev, N, K, M, weights) : 0;
     return passes > tiled ? passes : tiled;
 }

@@ -225,53 +225,58 @@ def test_row_owning_and_streaming_small_batch_kernels(hip, oracle, monkeypatch):
 # ---------------------------------------------------------------- tiled int8 GEMM (Q4_K, 33 activation rows and more)
 @pytest.mark.parametrize("N,M,K", [(33, 96, 512), (40, 4096, 1024), (48, 128, 256), (64, 100, 512), (100, 203, 2048), (130, 300, 1024), (64, 128, 4096),
                                    (192, 64, 7168), (512, 512, 4096)])
-def test_tiled_int8_gemm_matches_oracle(hip, oracle, N, M, K):
+@pytest.mark.parametrize("name", ["q4_k", "q5_k"])
+def test_tiled_int8_gemm_matches_oracle(hip, oracle, name, N, M, K):
     """Prefill with fp32 activations: 128 rows x 64 tokens per workgroup on the int8 matrix cores. Full and ragged
     tiles in both directions, one to 28 blocks per row, K split across workgroups when the tiles do not fill the chip
     (partials + ordered reduction), bias."""
-    kind = KIND_Q4_K
+    kind = KINDS[name]
     blocks = oracle.quantize(kind, gaussian(400 + N, (M, K), 0.02))
     x = gaussian(401 + N, (N, K))
     bias = gaussian(402, (M,))
     got = hip.linear(x, blocks, kind, M, bias=bias)
-    assert hip.last_route() == "mmq_q4_k_q8_k_mfma_tile"
-    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"tile {M}x{K} N={N}")
+    assert hip.last_route() == f"mmq_{name}_q8_k_mfma_tile"
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"{name} tile {M}x{K} N={N}")
 
 
-def test_tiled_int8_gemm_random_blocks_and_the_pass_kernel(hip, oracle, monkeypatch):
+@pytest.mark.parametrize("name", ["q4_k", "q5_k"])
+def test_tiled_int8_gemm_random_blocks_and_the_pass_kernel(hip, oracle, monkeypatch, name):
     """Arbitrary block bytes (every nibble, scale and min pattern) against the oracle; a device object created with
     MARMOT_HIP_NO_GEMM_I8 keeps the 32-row passes of the streaming kernel, and both kernels agree within the bound."""
     from marmot_amd import HipBackend
 
-    kind = KIND_Q4_K
+    kind = KINDS[name]
     N, M, K = 96, 160, 1536
     blocks = random_valid_blocks(np.random.default_rng(410), kind, M, K)
     x = gaussian(411, (N, K))
     ref = oracle.matmul(kind, blocks, x, M)
     tiled = hip.linear(x, blocks, kind, M)
-    assert hip.last_route() == "mmq_q4_k_q8_k_mfma_tile"
+    assert hip.last_route() == f"mmq_{name}_q8_k_mfma_tile"
     assert_matmul_parity(tiled, ref, what="tile, random blocks")
     monkeypatch.setenv("MARMOT_HIP_NO_GEMM_I8", "1")
     passes = HipBackend(0)
     monkeypatch.delenv("MARMOT_HIP_NO_GEMM_I8")
     try:
         got = passes.linear(x, blocks, kind, M)
-        assert passes.last_route() == "mmq_q4_k_q8_k_mfma"
+        assert passes.last_route() == f"mmq_{name}_q8_k_mfma"
         assert_matmul_parity(got, ref, what="passes, random blocks")
         assert_matmul_parity(tiled, got, what="tile against passes")
     finally:
         passes.close()
 
 
-def test_tiled_int8_gemm_integers_are_exact(hip):
+@pytest.mark.parametrize("name", ["q4_k", "q5_k"])
+def test_tiled_int8_gemm_integers_are_exact(hip, name):
     """Packed activations and weight blocks whose scales are powers of two: every fp32 operation of the kernel except
     the one addition per block is then exact, so the output must equal, bit for bit, the block sums
     a.d * (w.d * isum - w.dmin * msum) formed in exact integer arithmetic and added in block order."""
-    kind = KIND_Q4_K
+    kind = KINDS[name]
+    q5 = name == "q5_k"
+    bb, qs_off = (176, 48) if q5 else (144, 16)
     N, M, K = 70, 200, 512
     nb = K // 256
     rng = np.random.default_rng(420)
-    blocks = random_valid_blocks(rng, kind, M, K).reshape(M, nb, 144).copy()
+    blocks = random_valid_blocks(rng, kind, M, K).reshape(M, nb, bb).copy()
     d_exp = rng.integers(-12, -6, size=(M, nb))
     m_exp = rng.integers(-12, -6, size=(M, nb))
     blocks[:, :, 0:2] = np.ldexp(1.0, d_exp).astype(np.float16).view(np.uint8).reshape(M, nb, 2)
@@ -298,10 +303,14 @@ def test_tiled_int8_gemm_integers_are_exact(hip):
         else:
             sc[:, :, jj] = (s12[:, :, jj + 4] & 15) | ((s12[:, :, jj - 4] >> 6) << 4)
             mn[:, :, jj] = (s12[:, :, jj + 4] >> 4) | ((s12[:, :, jj] >> 6) << 4)
-    qs = blocks[:, :, 16:144].reshape(M, nb, 4, 32).astype(np.int64)
+    qs = blocks[:, :, qs_off:qs_off + 128].reshape(M, nb, 4, 32).astype(np.int64)
     wq = np.zeros((M, nb, 8, 32), np.int64)
     wq[:, :, 0::2, :] = qs & 15
     wq[:, :, 1::2, :] = qs >> 4
+    if q5:  # bit sb of qh[l] is the fifth bit of value l of sub-block sb (q5k_gguf.c:162-198)
+        qh = blocks[:, :, 16:48].astype(np.int64)
+        for sb_ in range(8):
+            wq[:, :, sb_, :] += ((qh >> sb_) & 1) << 4
     a = q.reshape(N, nb, 8, 32).astype(np.int64)
     want = np.zeros((N, M), np.float32)
     for b in range(nb):
@@ -311,9 +320,9 @@ def test_tiled_int8_gemm_integers_are_exact(hip):
         assert np.abs(isum).max() < 2 ** 24 and np.abs(msum).max() < 2 ** 24
         v = (np.ldexp(1.0, d_exp[None, :, b]) * isum - np.ldexp(1.0, m_exp[None, :, b]) * msum).astype(np.float32)
         want = (want + (np.ldexp(1.0, a_exp[:, b, None]).astype(np.float32) * v)).astype(np.float32)
-    d_w, d_p, d_out = hip.to_device(blocks.reshape(M, nb * 144)), hip.to_device(image), hip.alloc(N * M * 4)
+    d_w, d_p, d_out = hip.to_device(blocks.reshape(M, nb * bb)), hip.to_device(image), hip.alloc(N * M * 4)
     hip.linear_prepacked_d(kind, d_w, d_p, N, K, M, d_out)
-    assert hip.last_route() == "mmq_q4_k_q8_k_mfma_tile"
+    assert hip.last_route() == f"mmq_{name}_q8_k_mfma_tile"
     got = d_out.download(np.float32, (N, M))
     for b_ in (d_w, d_p, d_out):
         b_.free()

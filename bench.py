@@ -229,8 +229,8 @@ def prefill_int8(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV", "OPS", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
-    """Every benchmark configuration (C1..C5, QKV, OPS, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
+    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -310,6 +310,8 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C5", "QKV
                 linear_case("LEGACY", kind, 14336, 4096, N)
     if "C4" in only:
         sweep_layer_stack(hip, rng, emit, steps)
+    if "C4P" in only:
+        sweep_layer_stack(hip, rng, emit, steps, N=512, config="C4P")
     if "C5" in only:
         sweep_moe(hip, rng, emit, steps)
     if "QKV" in only:
@@ -432,11 +434,11 @@ def sweep_qkv(hip, rng, emit, steps: int, warmup: int):
             b.free()
 
 
-def sweep_layer_stack(hip, rng, emit, steps: int):
-    """C4: the seven linears of one layer at 16 tokens; 4 copies of the 139 MB of weights rotate."""
+def sweep_layer_stack(hip, rng, emit, steps: int, N: int = 16, config: str = "C4"):
+    """C4: the seven linears of one layer at 16 tokens; 4 copies of the 139 MB of weights rotate. C4P: the same layer
+    at 512 tokens of a prompt (fp32 activations: the tiled int8 GEMMs)."""
     from marmot_amd import DT_F32, capi, row_bytes
 
-    N = 16
     specs = [(capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 1024, 4096), (capi.KIND_Q6_K, 1024, 4096),
              (capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 14336, 4096), (capi.KIND_Q4_K, 14336, 4096),
              (capi.KIND_Q6_K, 4096, 14336)]
@@ -478,10 +480,11 @@ def sweep_layer_stack(hip, rng, emit, steps: int):
                                        weight_offset=(i % copies) * stride)
 
     ms_shared = time_steps_graph(hip, layer_step_shared, max(50, steps // 10), 10, chunk=50)
-    emit({"config": "C4", "workload": "7 linears of a Llama-3-8B layer (q,k,o,gate,up Q4_K; v,down Q6_K), N=16",
+    ops = sum(2.0 * N * M * K for _, M, K in specs)
+    emit({"config": config, "workload": f"7 linears of a Llama-3-8B layer (q,k,o,gate,up Q4_K; v,down Q6_K), N={N}",
           "us": round(ms * 1e3, 2), "GB/s": round(total / ms / 1e6, 1),
           "frac_of_hbm_peak": round(total / ms / 1e6 / HBM_PEAK_GBPS, 4), "tokens_per_s": round(N / ms * 1e3),
-          "algorithmic_bytes": total,
+          "TOP/s": round(ops / ms / 1e9, 1), "algorithmic_bytes": total,
           "us_shared_inputs": round(ms_shared * 1e3, 2),
           "shared_inputs": "q/k/v and gate/up take activations packed once per distinct input (4 packs, 7 linears)"})
     for b in packed.values():

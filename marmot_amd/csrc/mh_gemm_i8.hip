@@ -302,8 +302,9 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
                     aop[a] = i8_intx4{(int)av.x, (int)av.y, (int)av.z, (int)av.w};
                 }
             };
-            i8_intx4 aop[2][2];  // A operands of the sub-block in work and of the next one
+            i8_intx4 aop[3][2];  // A operands of the sub-block in work and of the next two
             read_a(0, aop[0]);
+            read_a(1, aop[1]);
             // 6-bit scales and mins as bytes (get_scale_min_k4, kquant_common.h:29-37)
             float d = h2f((uint16_t)(hdr.x & 0xffffu));
             float dmin = h2f((uint16_t)(hdr.x >> 16));
@@ -376,8 +377,8 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
 #pragma unroll
             for (int sb = 0; sb < 8; ++sb) {
                 const int c = sb & 1;
-                if (sb < 7) {
-                    read_a(sb + 1, aop[c ^ 1]);  // lands while the MFMAs below run
+                if (sb < 6) {
+                    read_a(sb + 2, aop[(sb + 2) % 3]);  // lands while the MFMAs of this and the next sub-block run
                 }
                 if (sb == 6) {
                     // activation scales: registers 4 g .. 4 g + 3 of token tile a are tokens 32 a + 8 g + 4 kh .. + 3
@@ -393,7 +394,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
                 const i8_intx4 btv = {bt[c], bt[c], bt[c], bt[c]};
 #pragma unroll
                 for (int a = 0; a < 2; ++a) {
-                    const i8_intx4 av = aop[c][a];
+                    const i8_intx4 av = aop[sb % 3][a];
                     const i8_intx16 zero = {0};
                     X[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bx[c], sb == 0 ? zero : X[a], 0, 0, 0);
                     if (sb < 7) {

@@ -61,6 +61,21 @@ def test_impl_matmul_matches_oracle(ctx, oracle, kind):
     assert_matmul_parity(yt.array, oracle.matmul(kind, wq, x, M, bias=bias), what=f"impl kind={kind}")
 
 
+@pytest.mark.parametrize("kind", [KIND_Q4_K, KIND_Q5_K, KIND_Q6_K])
+def test_impl_matmul_prompt_rows(ctx, oracle, kind):
+    """A prompt's worth of fp32 rows through the tensor-level entry (the tiled int8 GEMMs behind it): 100 rows, ragged
+    tiles, bias, host tensors mirrored by the residency layer."""
+    M, K, N = 200, 2048, 100
+    wq = oracle.quantize(kind, gaussian(740 + kind, (M, K), 0.02))
+    x = gaussian(741 + kind, (N, K))
+    bias = gaussian(742 + kind, (M,))
+    st, xt, wt, yt = _linear(ctx, kind, wq, M, K, x, bias=bias)
+    assert st == ta.SUCCESS, ctx.last_error()
+    assert_matmul_parity(yt.array, oracle.matmul(kind, wq, x, M, bias=bias), what=f"impl prompt rows kind={kind}")
+    for t in (xt, wt, yt):
+        ctx.host_freed(t)
+
+
 def test_impl_matmul_fp16_and_errors(ctx, oracle):
     M, K, N = 64, 512, 3
     wq = oracle.quantize(KIND_Q4_K, gaussian(730, (M, K), 0.02))

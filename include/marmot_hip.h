@@ -276,15 +276,14 @@ int marmot_hip_rope_frequencies(int scaling_type, float theta, float freq_scale,
  * Replaces cpu_embedding_gather_scalar for block-quantized tables (cpu_embedding_run_worker and
  * cpu_embedding_copy_row_quantized, src/backends/cpu/ops/embedding/scalar/embedding_scalar.c:241-303, 381-447;
  * descriptor marmot_embedding_gather_desc_t, include/marmot/ops_types.h:160-170).
- *   d_table : vocab rows of marmot_hip_row_bytes(kind, dim) bytes (any weight kind except Q4_1, whose tables the
- *             reference decodes in an order of its own without a golden vector: NOT_IMPLEMENTED)
+ *   d_table : vocab rows of marmot_hip_row_bytes(kind, dim) bytes (any weight kind)
  *   d_ids   : n token ids of ids_dtype (MARMOT_HIP_DTYPE_I32 or _I64)
  *   d_out   : [n, dim] of out_dtype (F32 or F16): decoded value * scale, one rounding for F16
  * A token equal to padding_id (when padding_id >= 0) gives a zero row. A token outside [0, vocab) gives a zero row,
  * or MARMOT_HIP_ERROR_INVALID_ARGUMENT when bounds_check is non-zero (the ids are then read back and checked on the
- * host before the launch; not possible, and skipped, while a graph is being captured). Q4_0 tables are decoded in the
- * embedding path's interleaved nibble order (value i = nibble i % 2 of byte i / 2, embedding_scalar.c:221-229), the
- * other kinds bit-exactly like marmot_hip_dequantize. */
+ * host before the launch; not possible, and skipped, while a graph is being captured). Q4_0 and Q4_1 tables are
+ * decoded in the embedding path's interleaved nibble order (value i = nibble i % 2 of byte i / 2,
+ * embedding_scalar.c:221-240), the other kinds bit-exactly like marmot_hip_dequantize. */
 int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, const void *d_table, size_t vocab,
                                           size_t dim, const void *d_ids, int ids_dtype, size_t n, void *d_out,
                                           int out_dtype, float scale, int32_t padding_id, int bounds_check);

@@ -806,8 +806,8 @@ marmot_error_t hip_matmul_qkv_q5_k(const void *device_ctx, const marmot_matmul_q
 marmot_error_t hip_matmul_qkv_q6_k(const void *device_ctx, const marmot_matmul_qkv_desc_t *desc);
 /* marmot_embedding_gather with a block-quantized table [vocab, dim] (cf. cpu_embedding_gather,
  * src/backends/cpu/ops/embedding/embedding_dispatch.c:4-16 -> embedding_scalar.c:460-591): token ids INT32 or INT64 of
- * any shape, output FLOAT32 or FLOAT16 viewed as [tokens, dim]; weights->quant_kind selects Q4_0, Q5_0, Q5_1,
- * Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K (Q4_1 tables are declined). */
+ * any shape, output FLOAT32 or FLOAT16 viewed as [tokens, dim]; weights->quant_kind selects Q4_0, Q4_1, Q5_0,
+ * Q5_1, Q8_0, Q8_1, Q2_K, Q3_K, Q4_K, Q5_K or Q6_K. */
 marmot_error_t hip_embedding_gather(const void *device_ctx, const marmot_embedding_gather_desc_t *desc);
 marmot_error_t hip_moe_experts_impl(const void *device_ctx, const marmot_moe_experts_desc_t *desc);
 marmot_error_t hip_topk_impl(const void *device_ctx, const marmot_topk_desc_t *desc);

@@ -1034,7 +1034,7 @@ static marmot_error_t embedding_gather(const void *device_ctx, const marmot_embe
     if (!kind_is_block(weights->quant_kind) || weights->quant_layout != MARMOT_QUANT_LAYOUT_GGUF) {
         return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Unsupported quantized embedding layout");
     }
-    if (!kind_supported_weight(weights->quant_kind) || weights->quant_kind == MARMOT_QUANT_KIND_Q4_1) {
+    if (!kind_supported_weight(weights->quant_kind)) {
         return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "Quantized embedding kind not supported on HIP");
     }
     const size_t vocab = weights->shape.shape[0], dim = weights->shape.shape[1];
@@ -2214,10 +2214,7 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         const int kind = kind_of_scheme(sig->qscheme_id);
         const uint16_t mm = matmul_op_of_kind(kind);
         if (mm == MARMOT_KERNEL_OP_INDEX_INVALID) {
-            return unsupported("HIP embedding gather handles Q4_0, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q6_K tables");
-        }
-        if (kind == MARMOT_HIP_KIND_Q4_1) {
-            return unsupported("HIP embedding gather does not offer Q4_1 tables");
+            return unsupported("HIP embedding gather handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q6_K tables");
         }
         if (sig->input_dtype != MARMOT_DTYPE_INT32 && sig->input_dtype != MARMOT_DTYPE_INT64) {
             return unsupported("HIP embedding gather takes INT32 or INT64 token ids");

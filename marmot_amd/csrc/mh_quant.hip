@@ -71,6 +71,11 @@ __global__ __launch_bounds__(256) void k_embedding_gather(const uint8_t *__restr
             const uint8_t packed = blk[2 + (v >> 1)];
             const int q = ((v & 1) ? (packed >> 4) : (packed & 0x0f)) - 8;
             y = h2f((uint16_t)(blk[0] | (blk[1] << 8))) * (float)q;
+        } else if constexpr (KIND == MARMOT_HIP_KIND_Q4_1) {
+            // the same interleaved order for Q4_1 tables (embedding_scalar.c:231-240): scale * q + min, two roundings
+            const uint8_t packed = blk[4 + (v >> 1)];
+            const int q = (v & 1) ? (packed >> 4) : (packed & 0x0f);
+            y = h2f((uint16_t)(blk[0] | (blk[1] << 8))) * (float)q + h2f((uint16_t)(blk[2] | (blk[3] << 8)));
         } else {
             y = dequant_value<KIND>(blk, v);
         }
@@ -405,11 +410,6 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
     if (!is_weight_kind(kind)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "embedding gather: unsupported quant kind %d", kind);
     }
-    if (kind == MARMOT_HIP_KIND_Q4_1) {
-        // the reference decodes Q4_1 tables in an interleaved nibble order of its own (embedding_scalar.c:231-240)
-        // and holds no golden vector for it: declined, the caller falls back
-        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "embedding gather: Q4_1 tables are not offered");
-    }
     if (ids_dtype != MARMOT_HIP_DTYPE_I32 && ids_dtype != MARMOT_HIP_DTYPE_I64) {
         return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "embedding gather: token ids must be INT32 or INT64");
     }
@@ -473,6 +473,10 @@ int marmot_hip_embedding_gather_quantized(marmot_hip_device_t *dev, int kind, co
         break;
     case MARMOT_HIP_KIND_Q5_1:
         hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q5_1>), grid, block, 0, dev->stream, table, vocab, dim,
+                           d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
+        break;
+    case MARMOT_HIP_KIND_Q4_1:
+        hipLaunchKernelGGL((k_embedding_gather<MARMOT_HIP_KIND_Q4_1>), grid, block, 0, dev->stream, table, vocab, dim,
                            d_ids, i64, d_out, f16, scale, (int)padding_id, flag);
         break;
     default:

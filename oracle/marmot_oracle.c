@@ -2710,8 +2710,20 @@ int mo_embedding_gather_quantized(
             case MO_KIND_Q8_0:
                 q8_0_dequantize_block((const blk_q8_0 *)blk, (uint32_t)count, decoded);
                 break;
-            /* Q4_1 tables are decoded in the interleaved order too (:231-240); the reference holds no golden for
-             * that case, so it is not restated: NOT_IMPLEMENTED below. Q5_0 / Q5_1 use their dequantizers. */
+            case MO_KIND_Q4_1: { /* cpu_embedding_decode_q4_1_interleaved, :231-240. The reference holds no golden for
+                                  * this case: the tests pin it as the Q4_1 dequantizer's values (golden) in the
+                                  * Q4_0 case's nibble order (golden). */
+                const blk_q4_1 *q = (const blk_q4_1 *)blk;
+                const float sc = mo_f16_to_f32(q->scale);
+                const float mn = mo_f16_to_f32(q->min);
+                for (size_t i = 0; i < count; ++i) {
+                    const uint8_t packed = q->qs[i >> 1];
+                    const uint8_t v = (uint8_t)((i & 1) ? ((packed >> 4) & 0x0f) : (packed & 0x0f));
+                    decoded[i] = sc * (float)v + mn;
+                }
+                break;
+            }
+            /* Q5_0 / Q5_1 use their dequantizers. */
             case MO_KIND_Q8_1:
                 q8_1_dequantize_block((const blk_q8_1 *)blk, (uint32_t)count, decoded);
                 break;

@@ -270,14 +270,13 @@ def test_query_kernel_embedding_rules(lib):
         s.weight_layout = ta.WEIGHT_LAYOUT_SEPARATE
         return s
     for kind, op in ((ta.KIND_Q4_0, 16), (ta.KIND_Q8_0, 17), (ta.KIND_Q4_K, 18), (ta.KIND_Q6_K, 19),
-                     (ta.KIND_Q5_K, 23), (ta.KIND_Q5_0, 31), (ta.KIND_Q5_1, 35), (ta.KIND_Q2_K, 39), (ta.KIND_Q3_K, 43),
+                     (ta.KIND_Q5_K, 23), (ta.KIND_Q4_1, 27), (ta.KIND_Q5_0, 31), (ta.KIND_Q5_1, 35), (ta.KIND_Q2_K, 39), (ta.KIND_Q3_K, 43),
                      (ta.KIND_Q8_1, 47)):
         for ids in (ta.DTYPE_I32, ta.DTYPE_I64):
             for out in (ta.DTYPE_F32, ta.DTYPE_F16):
                 sel = _query(lib, sig(kind, ids, out))
                 assert sel.supported and sel.op_index == op
     assert not _query(lib, sig(kind=ta.KIND_Q8_K)).supported
-    assert not _query(lib, sig(kind=ta.KIND_Q4_1)).supported  # interleaved table order without a golden: declined
     assert not _query(lib, sig(kind=ta.KIND_GENERIC)).supported
     assert not _query(lib, sig(ids=ta.DTYPE_F32)).supported
     assert not _query(lib, sig(out=ta.DTYPE_I32)).supported

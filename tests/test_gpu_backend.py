@@ -536,7 +536,9 @@ def test_embedding_gather_errors(ctx):
     assert call(o=tmp["int_out"]) == ta.UNSUPPORTED_DTYPE
     assert call(o=tmp["short_out"]) == ta.DIMENSION_MISMATCH
     assert call(weights=tmp["q8_k"]) == ta.NOT_IMPLEMENTED
-    assert call(weights=tmp["q4_1"]) == ta.NOT_IMPLEMENTED  # Q4_1 tables are declined
+    # Q4_1 tables are taken (the embedding path's interleaved nibble order): the Q4_K bytes read as Q4_1 blocks are a
+    # table of another width, so the shapes disagree here
+    assert call(weights=tmp["q4_1"]) in (ta.DIMENSION_MISMATCH, ta.INVALID_ARGUMENT)
     assert call(weights=tmp["flat"]) == ta.DIMENSION_MISMATCH
     assert call(token_ids=tmp["no_ids"], o=tmp["no_out"]) == ta.SUCCESS
     for t in [tt, ids, out] + list(tmp.values()):

@@ -191,7 +191,7 @@ def prefill_gemm(hip, tokens: int, steps: int, warmup: int):
         "frac_of_mfma_peak": round(flops / (ms * 1e-3) / 1e12 / 2500.0, 4),
         "tokens_per_s": round(tokens / (ms * 1e-3), 1),
         "steps": steps,
-        "includes": "sub-block sums, GEMM and K-split reduction kernels",
+        "includes": "every kernel of the op (512 tokens: one launch, sub-block sums computed inside; K-split partials and their reduction only below half a chip of tiles)",
     }
     for b in (d_w, d_x, d_out):
         b.free()

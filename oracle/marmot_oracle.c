@@ -3239,3 +3239,217 @@ done:
     free(up_buf);
     return status;
 }
+
+/* ======================= paged attention ======================= */
+
+/* marmot_f32_to_bf16_ref / marmot_bf16_to_f32_ref (src/utils/dtype_ref.c:86-104): round to nearest even on the bits */
+static uint16_t pa_f32_to_bf16(float value) {
+    uint32_t bits;
+    memcpy(&bits, &value, sizeof(bits));
+    const uint32_t bias = 0x7FFFu + ((bits >> 16) & 1u);
+    return (uint16_t)((bits + bias) >> 16);
+}
+
+static float pa_bf16_to_f32(uint16_t h) {
+    const uint32_t bits = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &bits, sizeof(f));
+    return f;
+}
+
+/* cpu_load_as_f32 / cpu_store_from_f32 (cpu_backend_internal.h:641-680) for the three float types */
+static float pa_load(int dtype, const void *data, size_t index) {
+    switch (dtype) {
+    case MO_DTYPE_F16:
+        return mo_f16_to_f32(((const uint16_t *)data)[index]);
+    case MO_DTYPE_BF16:
+        return pa_bf16_to_f32(((const uint16_t *)data)[index]);
+    default:
+        return ((const float *)data)[index];
+    }
+}
+
+static void pa_store(int dtype, void *data, size_t index, float value) {
+    switch (dtype) {
+    case MO_DTYPE_F16:
+        ((uint16_t *)data)[index] = mo_f32_to_f16(value);
+        break;
+    case MO_DTYPE_BF16:
+        ((uint16_t *)data)[index] = pa_f32_to_bf16(value);
+        break;
+    default:
+        ((float *)data)[index] = value;
+        break;
+    }
+}
+
+static int pa_float_dtype(int dtype) {
+    return dtype == MO_DTYPE_F32 || dtype == MO_DTYPE_F16 || dtype == MO_DTYPE_BF16;
+}
+
+/* cpu_paged_attention_choose_block_n, paged_attention_ref.c:31-50 */
+static size_t pa_block_n(size_t head_dim) {
+    size_t rows = (64u * 1024u) / (2 * head_dim * sizeof(float));
+    if (rows < 32) {
+        rows = 32;
+    }
+    if (rows > 256) {
+        rows = 256;
+    }
+    return rows;
+}
+
+int mo_paged_attention(const mo_paged_attention_args *a) {
+    if (a == NULL || a->token_meta == NULL || a->q == NULL || a->k_new == NULL || a->v_new == NULL || a->kv_k == NULL ||
+        a->kv_v == NULL || a->block_table == NULL || a->out == NULL) {
+        return MO_ERR_INVALID_ARGUMENT; /* :574-577, :799-803 */
+    }
+    if (a->token_count == 0) {
+        return 0;
+    }
+    if (a->num_q_heads == 0 || a->num_kv_heads == 0 || a->head_dim == 0 || a->block_size == 0 ||
+        (a->block_size & (a->block_size - 1u)) != 0 || a->num_q_heads % a->num_kv_heads != 0) {
+        return MO_ERR_INVALID_ARGUMENT; /* :581-596 */
+    }
+    if (!pa_float_dtype(a->act_dtype) || !pa_float_dtype(a->kv_dtype)) {
+        return MO_ERR_UNSUPPORTED_DTYPE; /* :622-630 */
+    }
+    if (a->kv_layers <= a->layer_idx) {
+        return MO_ERR_DIMENSION_MISMATCH; /* :673-676 */
+    }
+    uint32_t shift = 0;
+    while ((1u << shift) < a->block_size) {
+        ++shift;
+    }
+    const uint32_t mask = a->block_size - 1u;
+    const size_t hd = a->head_dim;
+    for (size_t t = 0; t < a->token_count; ++t) { /* :809-823 */
+        const uint32_t seq_slot = a->token_meta[t * a->meta_stride[0]];
+        const uint32_t kv_slot = a->token_meta[t * a->meta_stride[0] + 2 * a->meta_stride[1]];
+        if (seq_slot >= a->max_seqs || (kv_slot >> shift) >= a->kv_blocks) {
+            return MO_ERR_DIMENSION_MISMATCH;
+        }
+    }
+    /* the new rows go into the cache first (:346-373): same dtype = bit copy, otherwise through fp32 */
+    for (size_t t = 0; t < a->token_count; ++t) {
+        const uint32_t kv_slot = a->token_meta[t * a->meta_stride[0] + 2 * a->meta_stride[1]];
+        const size_t base = (size_t)(kv_slot >> shift) * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] +
+                            (size_t)(kv_slot & mask) * a->kv_stride[3];
+        for (size_t h = 0; h < a->num_kv_heads; ++h) {
+            for (size_t d = 0; d < hd; ++d) {
+                const size_t dst = base + h * a->kv_stride[2] + d * a->kv_stride[4];
+                const size_t ks = t * a->k_stride[0] + h * a->k_stride[1] + d * a->k_stride[2];
+                const size_t vs = t * a->v_stride[0] + h * a->v_stride[1] + d * a->v_stride[2];
+                if (a->act_dtype == a->kv_dtype && a->act_dtype != MO_DTYPE_F32) {
+                    ((uint16_t *)a->kv_k)[dst] = ((const uint16_t *)a->k_new)[ks];
+                    ((uint16_t *)a->kv_v)[dst] = ((const uint16_t *)a->v_new)[vs];
+                } else {
+                    pa_store(a->kv_dtype, a->kv_k, dst, pa_load(a->act_dtype, a->k_new, ks));
+                    pa_store(a->kv_dtype, a->kv_v, dst, pa_load(a->act_dtype, a->v_new, vs));
+                }
+            }
+        }
+    }
+    const size_t block_n = pa_block_n(hd);
+    float *q_vec = (float *)malloc(hd * sizeof(float));
+    float *out_vec = (float *)malloc(hd * sizeof(float));
+    float *k_block = (float *)malloc(block_n * hd * sizeof(float));
+    float *v_block = (float *)malloc(block_n * hd * sizeof(float));
+    float *scores = (float *)malloc(block_n * sizeof(float));
+    if (q_vec == NULL || out_vec == NULL || k_block == NULL || v_block == NULL || scores == NULL) {
+        free(q_vec), free(out_vec), free(k_block), free(v_block), free(scores);
+        return MO_ERR_INVALID_ARGUMENT;
+    }
+    const size_t group = a->num_q_heads / a->num_kv_heads;
+    for (size_t t = 0; t < a->token_count; ++t) { /* cpu_paged_attention_attention_range, :398-569 */
+        const uint32_t seq_slot = a->token_meta[t * a->meta_stride[0]];
+        const uint32_t pos = a->token_meta[t * a->meta_stride[0] + a->meta_stride[1]];
+        const uint32_t kv_len = pos + 1u;
+        for (size_t qh = 0; qh < a->num_q_heads; ++qh) {
+            const size_t kvh = qh / group;
+            const size_t q_base = t * a->q_stride[0] + qh * a->q_stride[1];
+            const size_t out_base = t * a->out_stride[0] + qh * a->out_stride[1];
+            for (size_t d = 0; d < hd; ++d) {
+                q_vec[d] = pa_load(a->act_dtype, a->q, q_base + d * a->q_stride[2]);
+            }
+            if (a->scale != 1.0f) {
+                for (size_t d = 0; d < hd; ++d) {
+                    q_vec[d] *= a->scale;
+                }
+            }
+            memset(out_vec, 0, hd * sizeof(float));
+            float max_score = -INFINITY, sum = 0.0f;
+            int has_any = 0;
+            for (uint32_t k_start = 0; k_start < kv_len; k_start += (uint32_t)block_n) {
+                uint32_t k_limit = k_start + (uint32_t)block_n;
+                if (k_limit > kv_len || k_limit < k_start) {
+                    k_limit = kv_len;
+                }
+                size_t k_count = 0;
+                for (uint32_t p = k_start; p < k_limit; ++p) {
+                    const uint32_t logical = p >> shift;
+                    if (logical >= a->max_blocks_per_seq) {
+                        break;
+                    }
+                    const uint32_t tb = a->block_table[(size_t)seq_slot * a->table_stride[0] +
+                                                       (size_t)logical * a->table_stride[1]];
+                    if (tb == 0xFFFFFFFFu) {
+                        continue;
+                    }
+                    const size_t base = (size_t)tb * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] +
+                                        kvh * a->kv_stride[2] + (size_t)(p & mask) * a->kv_stride[3];
+                    for (size_t d = 0; d < hd; ++d) {
+                        k_block[k_count * hd + d] = pa_load(a->kv_dtype, a->kv_k, base + d * a->kv_stride[4]);
+                        v_block[k_count * hd + d] = pa_load(a->kv_dtype, a->kv_v, base + d * a->kv_stride[4]);
+                    }
+                    ++k_count;
+                }
+                if (k_count == 0) {
+                    continue;
+                }
+                float row_max = -INFINITY;
+                for (size_t kj = 0; kj < k_count; ++kj) { /* cpu_paged_attention_dot_f32_scalar */
+                    float dot = 0.0f;
+                    for (size_t d = 0; d < hd; ++d) {
+                        dot += q_vec[d] * k_block[kj * hd + d];
+                    }
+                    scores[kj] = dot;
+                    if (dot > row_max) {
+                        row_max = dot;
+                    }
+                }
+                const float next_max = max_score > row_max ? max_score : row_max;
+                const float exp_prev = max_score == -INFINITY ? 0.0f : expf(max_score - next_max);
+                if (exp_prev != 1.0f) {
+                    for (size_t d = 0; d < hd; ++d) {
+                        out_vec[d] *= exp_prev;
+                    }
+                }
+                float block_sum = 0.0f; /* cpu_paged_attention_block_sum_f32_scalar */
+                for (size_t kj = 0; kj < k_count; ++kj) {
+                    const float weight = expf(scores[kj] - next_max);
+                    block_sum += weight;
+                    for (size_t d = 0; d < hd; ++d) {
+                        out_vec[d] += weight * v_block[kj * hd + d];
+                    }
+                }
+                sum = sum * exp_prev + block_sum;
+                max_score = next_max;
+                has_any = 1;
+            }
+            if (!has_any) {
+                for (size_t d = 0; d < hd; ++d) {
+                    pa_store(a->act_dtype, a->out, out_base + d * a->out_stride[2], 0.0f);
+                }
+                continue;
+            }
+            const float inv_sum = sum > 0.0f ? 1.0f / sum : 0.0f;
+            for (size_t d = 0; d < hd; ++d) {
+                pa_store(a->act_dtype, a->out, out_base + d * a->out_stride[2],
+                         inv_sum != 1.0f ? out_vec[d] * inv_sum : out_vec[d]);
+            }
+        }
+    }
+    free(q_vec), free(out_vec), free(k_block), free(v_block), free(scores);
+    return 0;
+}

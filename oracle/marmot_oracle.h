@@ -52,6 +52,7 @@ enum {
 enum {
     MO_DTYPE_F32 = 0,
     MO_DTYPE_F16 = 1,
+    MO_DTYPE_BF16 = 2,
     MO_DTYPE_I32 = 3,
     MO_DTYPE_I64 = 11,
 };
@@ -219,6 +220,36 @@ int mo_moe_experts(
 
 /* row grain used to split weight rows over threads (matmul_quant_compute.c:1222-1240) */
 size_t mo_row_grain(size_t row_count, size_t cols_in_tile, size_t thread_cap);
+
+/* ======================= paged attention ======================= */
+/* cpu_paged_attention_impl (src/backends/cpu/ops/paged_attention/paged_attention_ref.c:573-1082) for FLOAT32 / FLOAT16 /
+ * BFLOAT16 activations and KV caches (the FP8 cache of MARMOT_ENABLE_FP8 builds is not restated): first every token's
+ * k_new / v_new rows are written into the paged cache at the token's kv_slot (:346-373), then every token attends over
+ * positions 0 .. pos of its sequence through the block table with an online softmax in blocks of block_n positions
+ * (:398-569; scalar kernels paged_attention/scalar). All strides are in elements.
+ *   token_meta  [token_count, 4] uint32: seq_slot, pos, kv_slot, flags (flags are not read)
+ *   q, out      [tokens, num_q_heads, head_dim], k_new, v_new [tokens, num_kv_heads, head_dim] of act_dtype
+ *   kv_k, kv_v  [blocks, layers, num_kv_heads, block_size, head_dim] of kv_dtype (updated in place)
+ *   block_table [max_seqs, max_blocks_per_seq] uint32, 0xFFFFFFFF = no block */
+typedef struct {
+    uint32_t token_count, layer_idx, num_q_heads, num_kv_heads, head_dim, block_size;
+    float scale;
+    int act_dtype, kv_dtype;
+    const uint32_t *token_meta;
+    size_t meta_stride[2];
+    const void *q, *k_new, *v_new;
+    size_t q_stride[3], k_stride[3], v_stride[3];
+    void *kv_k, *kv_v;
+    size_t kv_stride[5];
+    size_t kv_blocks, kv_layers;
+    const uint32_t *block_table;
+    size_t table_stride[2];
+    size_t max_seqs, max_blocks_per_seq;
+    void *out;
+    size_t out_stride[3];
+} mo_paged_attention_args;
+
+int mo_paged_attention(const mo_paged_attention_args *a);
 
 #ifdef __cplusplus
 }

@@ -33,10 +33,65 @@ BLOCK_BYTES = {KIND_Q4_0: 18, KIND_Q8_0: 34, KIND_Q4_K: 144, KIND_Q5_K: 176, KIN
                KIND_Q4_1: 20, KIND_Q5_0: 22, KIND_Q5_1: 24, KIND_Q2_K: 84, KIND_Q3_K: 110,
                KIND_Q8_1: 36}
 DT_F32, DT_F16 = 0, 1
+DT_BF16 = 2
 DT_I32, DT_I64 = 3, 11  # marmot_dtype_t values of the position tensors the rotary epilogue accepts
 ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_YARN, ROPE_SCALING_LONGROPE = 0, 1, 2, 3
 ROPE_TYPE_NORM, ROPE_TYPE_NEOX = 0, 1
 
+
+
+class PagedAttentionArgs(C.Structure):
+    """mo_paged_attention_args: the tensors of marmot_paged_attention_desc_t as pointers and element strides."""
+    _fields_ = [("token_count", C.c_uint32), ("layer_idx", C.c_uint32), ("num_q_heads", C.c_uint32),
+                ("num_kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("block_size", C.c_uint32),
+                ("scale", C.c_float), ("act_dtype", C.c_int), ("kv_dtype", C.c_int),
+                ("token_meta", C.c_void_p), ("meta_stride", C.c_size_t * 2),
+                ("q", C.c_void_p), ("k_new", C.c_void_p), ("v_new", C.c_void_p),
+                ("q_stride", C.c_size_t * 3), ("k_stride", C.c_size_t * 3), ("v_stride", C.c_size_t * 3),
+                ("kv_k", C.c_void_p), ("kv_v", C.c_void_p), ("kv_stride", C.c_size_t * 5),
+                ("kv_blocks", C.c_size_t), ("kv_layers", C.c_size_t),
+                ("block_table", C.c_void_p), ("table_stride", C.c_size_t * 2),
+                ("max_seqs", C.c_size_t), ("max_blocks_per_seq", C.c_size_t),
+                ("out", C.c_void_p), ("out_stride", C.c_size_t * 3)]
+
+
+def float_dtype_code(a: np.ndarray, bf16: bool = False) -> int:
+    """marmot_dtype_t of a float tensor held in numpy: bfloat16 travels as uint16 bits."""
+    if bf16:
+        assert a.dtype == np.uint16
+        return DT_BF16
+    return {np.dtype(np.float32): DT_F32, np.dtype(np.float16): DT_F16}[a.dtype]
+
+
+def element_strides(a: np.ndarray):
+    assert all(s % a.itemsize == 0 for s in a.strides)
+    return [s // a.itemsize for s in a.strides]
+
+
+def paged_attention_args(token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx, scale, act_bf16=False,
+                         kv_bf16=False, token_count=None, ptr=None):
+    """(PagedAttentionArgs over the given numpy arrays, freshly allocated out array). `ptr` maps an array to the
+    address to put into the struct (default: the array's own memory)."""
+    ptr = ptr or (lambda a: a.ctypes.data)
+    assert token_meta.dtype == np.uint32 and block_table.dtype == np.uint32
+    out = np.zeros(q.shape, dtype=q.dtype)
+    a = PagedAttentionArgs()
+    a.token_count = q.shape[0] if token_count is None else token_count
+    a.layer_idx, a.scale = layer_idx, scale
+    a.num_q_heads, a.num_kv_heads, a.head_dim, a.block_size = q.shape[1], k_new.shape[1], q.shape[2], kv_k.shape[3]
+    a.act_dtype, a.kv_dtype = float_dtype_code(q, act_bf16), float_dtype_code(kv_k, kv_bf16)
+    a.token_meta, a.meta_stride = ptr(token_meta), (C.c_size_t * 2)(*element_strides(token_meta))
+    a.q, a.k_new, a.v_new = ptr(q), ptr(k_new), ptr(v_new)
+    a.q_stride = (C.c_size_t * 3)(*element_strides(q))
+    a.k_stride = (C.c_size_t * 3)(*element_strides(k_new))
+    a.v_stride = (C.c_size_t * 3)(*element_strides(v_new))
+    assert kv_k.shape == kv_v.shape and kv_k.strides == kv_v.strides
+    a.kv_k, a.kv_v, a.kv_stride = ptr(kv_k), ptr(kv_v), (C.c_size_t * 5)(*element_strides(kv_k))
+    a.kv_blocks, a.kv_layers = kv_k.shape[0], kv_k.shape[1]
+    a.block_table, a.table_stride = ptr(block_table), (C.c_size_t * 2)(*element_strides(block_table))
+    a.max_seqs, a.max_blocks_per_seq = block_table.shape
+    a.out, a.out_stride = ptr(out), (C.c_size_t * 3)(*element_strides(out))
+    return a, out
 
 class RopeParams(C.Structure):
     """mo_rope_params: marmot_rope_params_t without the positions tensor."""
@@ -136,6 +191,8 @@ class Oracle:
             C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_void_p,
             C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
         ]
+        L.mo_paged_attention.restype = C.c_int
+        L.mo_paged_attention.argtypes = [C.POINTER(PagedAttentionArgs)]
         L.mo_row_grain.restype = C.c_size_t
         L.mo_row_grain.argtypes = [C.c_size_t, C.c_size_t, C.c_size_t]
 
@@ -235,6 +292,16 @@ class Oracle:
         if st != 0:
             raise RuntimeError(f"mo_matmul_quantized -> {st}")
         return out
+
+    def paged_attention(self, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx: int, scale: float,
+                        act_bf16: bool = False, kv_bf16: bool = False, token_count=None):
+        """marmot_paged_attention: kv_k / kv_v ([blocks, layers, kv heads, block size, head dim]) are updated in place;
+        q / k_new / v_new are [tokens, heads, head dim] arrays (views with any strides) of float32, float16, or uint16
+        holding bfloat16 bits (act_bf16 / kv_bf16). Returns (status, out)."""
+        args, out = paged_attention_args(token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx, scale, act_bf16,
+                                         kv_bf16, token_count)
+        st = self.L.mo_paged_attention(C.byref(args))
+        return st, out
 
     def rope_frequencies(self, rope: "RopeParams", head_dim: int):
         """(angular frequencies [head_dim / 2], attention scale) of marmot_rope_freq_cache_ensure."""

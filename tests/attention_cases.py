@@ -1,0 +1,107 @@
+"""Synthetic paged-attention workloads shared by the CPU and GPU tests: a paged KV cache with history, new tokens of
+several sequences (prompt chunks and single decode tokens in one call, in any order), and the two independent
+statements of the expected result: the cache after the write (pure data movement and dtype conversion) and dense
+softmax attention in float64 over each token's history read back through the block table."""
+import numpy as np
+
+NO_BLOCK = 0xFFFFFFFF
+
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Round to nearest even on the float32 bits, as the reference's bfloat16 conversion does."""
+    b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def to_storage(x32: np.ndarray, name: str) -> np.ndarray:
+    """float32 values in the storage type `name` ('f32', 'f16', 'bf16': bfloat16 bits in uint16)."""
+    if name == "f32":
+        return np.ascontiguousarray(x32, dtype=np.float32)
+    if name == "f16":
+        return x32.astype(np.float16)
+    return f32_to_bf16_bits(x32)
+
+
+def to_f32(a: np.ndarray, name: str) -> np.ndarray:
+    return bf16_bits_to_f32(a).reshape(a.shape) if name == "bf16" else a.astype(np.float32)
+
+
+def make_case(seed, seqs, num_q_heads, num_kv_heads, head_dim, block_size, act="f32", kv="f32", layers=2, layer_idx=1,
+              spare_blocks=3, shuffle_tokens=True):
+    """seqs: list of (history_len, new_tokens). Physical blocks are a random permutation; sequence slots are a random
+    subset of the block table's rows; rows the call does not write hold finite garbage."""
+    rng = np.random.default_rng(seed)
+    max_seqs = len(seqs) + 2
+    need = [-(-(h + n) // block_size) for h, n in seqs]
+    max_blocks = max(need) + 1
+    blocks = sum(need) + spare_blocks
+    phys = rng.permutation(blocks)
+    slots = rng.permutation(max_seqs)[:len(seqs)]
+    table = np.full((max_seqs, max_blocks), NO_BLOCK, dtype=np.uint32)
+    shape = (blocks, layers, num_kv_heads, block_size, head_dim)
+    kv_k = to_storage(rng.standard_normal(shape, dtype=np.float32), kv)
+    kv_v = to_storage(rng.standard_normal(shape, dtype=np.float32), kv)
+    meta = []
+    nxt = 0
+    for s, (hist, new) in enumerate(seqs):
+        for b in range(need[s]):
+            table[slots[s], b] = phys[nxt]
+            nxt += 1
+        for p in range(hist, hist + new):
+            meta.append((slots[s], p, int(table[slots[s], p // block_size]) * block_size + p % block_size, 0))
+    meta = np.array(meta, dtype=np.uint32).reshape(-1, 4)
+    if shuffle_tokens:
+        meta = meta[rng.permutation(len(meta))]
+    T = len(meta)
+    q = to_storage(rng.standard_normal((T, num_q_heads, head_dim), dtype=np.float32), act)
+    k_new = to_storage(rng.standard_normal((T, num_kv_heads, head_dim), dtype=np.float32), act)
+    v_new = to_storage(rng.standard_normal((T, num_kv_heads, head_dim), dtype=np.float32), act)
+    return {"token_meta": np.ascontiguousarray(meta), "q": q, "k_new": k_new, "v_new": v_new, "kv_k": kv_k, "kv_v": kv_v,
+            "block_table": table, "layer_idx": layer_idx, "block_size": block_size, "act": act, "kv": kv,
+            "scale": float(1.0 / np.sqrt(head_dim))}
+
+
+def cache_after_write(case):
+    """The caches once every token's new rows are stored at its kv_slot: same storage type = the same bits,
+    otherwise through float32."""
+    act, kv, bs, layer = case["act"], case["kv"], case["block_size"], case["layer_idx"]
+    kv_k, kv_v = case["kv_k"].copy(), case["kv_v"].copy()
+    for t, (_, _, slot, _) in enumerate(case["token_meta"]):
+        b, off = int(slot) // bs, int(slot) % bs
+        for dst, src in ((kv_k, case["k_new"]), (kv_v, case["v_new"])):
+            dst[b, layer, :, off, :] = src[t] if act == kv else to_storage(to_f32(src[t], act), kv)
+    return kv_k, kv_v
+
+
+def dense_reference(case, kv_k, kv_v) -> np.ndarray:
+    """softmax(scale * q . K) V in float64 over positions 0 .. pos of each token's sequence, read from the given
+    caches through the block table (positions without a block are skipped)."""
+    bs, layer = case["block_size"], case["layer_idx"]
+    q = to_f32(case["q"], case["act"]).astype(np.float64)
+    k64 = to_f32(kv_k, case["kv"]).astype(np.float64)
+    v64 = to_f32(kv_v, case["kv"]).astype(np.float64)
+    T, hq, d = q.shape
+    group = hq // case["k_new"].shape[1]
+    table = case["block_table"]
+    out = np.zeros((T, hq, d))
+    for t, (seq, pos, _, _) in enumerate(case["token_meta"]):
+        rows = [(int(table[seq, p // bs]), p % bs) for p in range(int(pos) + 1)
+                if p // bs < table.shape[1] and table[seq, p // bs] != NO_BLOCK]
+        if not rows:
+            continue
+        bi = np.array([r[0] for r in rows])
+        oi = np.array([r[1] for r in rows])
+        for h in range(hq):
+            K = k64[bi, layer, h // group, oi, :]
+            V = v64[bi, layer, h // group, oi, :]
+            s = (K @ q[t, h]) * case["scale"]
+            w = np.exp(s - s.max())
+            out[t, h] = (w / w.sum()) @ V
+    return out
+
+
+TOLERANCE = {"f32": 2e-5, "f16": 1.5e-3, "bf16": 1.2e-2}  # of the largest |v|: fp32 accumulation, one output rounding

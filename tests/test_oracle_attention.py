@@ -1,0 +1,101 @@
+"""CPU: the oracle's restatement of marmot_paged_attention (src/backends/cpu/ops/paged_attention/paged_attention_ref.c),
+pinned by (1) the closed-form case of the reference's own test (tests/backend/test_backend_paged_attention.c:162-288:
+two tokens, identity keys and values, expected softmax weights and cache contents), (2) dense softmax attention in
+float64 over each token's history read back through the block table -- what paged attention reduces to -- on caches
+with history, shuffled physical blocks, grouped query heads, prompt chunks and decode tokens in one call, and (3) the
+cache write as pure data movement (same storage type: the same bits; otherwise one conversion through float32)."""
+import numpy as np
+import pytest
+
+from tests.attention_cases import NO_BLOCK, TOLERANCE, cache_after_write, dense_reference, make_case, to_f32
+
+MO_INVALID, MO_DTYPE, MO_DIMS = -1, -6, -7
+
+
+def run(oracle, case, **kw):
+    kv_k, kv_v = case["kv_k"].copy(), case["kv_v"].copy()
+    st, out = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], kv_k, kv_v,
+                                     case["block_table"], case["layer_idx"], case["scale"],
+                                     act_bf16=case["act"] == "bf16", kv_bf16=case["kv"] == "bf16", **kw)
+    return st, out, kv_k, kv_v
+
+
+def test_reference_closed_form_case(oracle):
+    """Two tokens of one sequence, one head of two values, block size 4, scale 1: q = k = v = identity rows."""
+    eye = np.array([[[1.0, 0.0]], [[0.0, 1.0]]], dtype=np.float32)
+    meta = np.array([[0, 0, 0, 2], [0, 1, 1, 1]], dtype=np.uint32)
+    kv_k = np.zeros((1, 1, 1, 4, 2), np.float32)
+    kv_v = np.zeros_like(kv_k)
+    table = np.zeros((1, 1), np.uint32)
+    st, out = oracle.paged_attention(meta, eye, eye.copy(), eye.copy(), kv_k, kv_v, table, 0, 1.0)
+    assert st == 0
+    e = np.exp(np.float32(1.0))
+    assert abs(out[0, 0, 0] - 1.0) < 1e-4 and abs(out[0, 0, 1]) < 1e-4
+    assert abs(out[1, 0, 0] - 1.0 / (1.0 + e)) < 1e-4 and abs(out[1, 0, 1] - e / (1.0 + e)) < 1e-4
+    for cache in (kv_k, kv_v):
+        assert np.array_equal(cache[0, 0, 0, :2], np.eye(2, dtype=np.float32)) and not cache[0, 0, 0, 2:].any()
+
+
+@pytest.mark.parametrize("act,kv", [("f32", "f32"), ("f16", "f16"), ("f32", "f16"), ("f16", "f32"), ("bf16", "bf16"),
+                                    ("f32", "bf16"), ("bf16", "f16")])
+def test_matches_dense_attention_in_float64(oracle, act, kv):
+    case = make_case(11, [(37, 1), (0, 19), (130, 5), (64, 1)], num_q_heads=8, num_kv_heads=2, head_dim=64, block_size=16,
+                     act=act, kv=kv)
+    st, out, kv_k, kv_v = run(oracle, case)
+    assert st == 0
+    want_k, want_v = cache_after_write(case)
+    assert np.array_equal(kv_k.view(np.uint8), want_k.view(np.uint8))
+    assert np.array_equal(kv_v.view(np.uint8), want_v.view(np.uint8))
+    ref = dense_reference(case, want_k, want_v)
+    err = np.max(np.abs(to_f32(out, act).astype(np.float64) - ref))
+    assert err <= TOLERANCE[act] * np.abs(to_f32(want_v, kv)).max(), err
+
+
+def test_long_history_spans_several_score_blocks(oracle):
+    """head_dim 128: the reference scores 64 positions per block; 700 positions are eleven blocks with a running
+    maximum that changes (keys scaled up so that late positions dominate)."""
+    case = make_case(12, [(699, 1), (300, 2)], num_q_heads=4, num_kv_heads=4, head_dim=128, block_size=32)
+    case["kv_k"][...] *= np.linspace(0.2, 3.0, case["kv_k"].shape[0], dtype=np.float32)[:, None, None, None, None]
+    st, out, kv_k, kv_v = run(oracle, case)
+    assert st == 0
+    ref = dense_reference(case, kv_k, kv_v)
+    assert np.max(np.abs(out - ref)) <= TOLERANCE["f32"] * np.abs(kv_v).max()
+
+
+def test_missing_blocks_strided_views_and_token_count(oracle):
+    case = make_case(13, [(40, 3), (5, 1)], num_q_heads=4, num_kv_heads=2, head_dim=32, block_size=8)
+    seq = case["token_meta"][0, 0]
+    case["block_table"][seq, 1] = NO_BLOCK  # a hole: positions 8..15 of that sequence are skipped
+    st, out, kv_k, kv_v = run(oracle, case)
+    assert st == 0
+    ref = dense_reference(case, kv_k, kv_v)
+    assert np.max(np.abs(out - ref)) <= TOLERANCE["f32"] * np.abs(kv_v).max()
+    # a sequence whose table row is empty attends over nothing: zeros
+    empty = dict(case, block_table=np.full_like(case["block_table"], NO_BLOCK))
+    st, out0, _, _ = run(oracle, empty)
+    assert st == 0 and not out0.any()
+    # q / k_new / v_new as strided views (a fused projection's output), and fewer tokens than rows
+    T = case["q"].shape[0]
+    fused = np.zeros((T, 4 + 2 + 2, 32), np.float32)
+    fused[:, :4], fused[:, 4:6], fused[:, 6:] = case["q"], case["k_new"], case["v_new"]
+    view = dict(case, q=fused[:, :4], k_new=fused[:, 4:6], v_new=fused[:, 6:])
+    st, out_v, kv_k2, kv_v2 = run(oracle, view)
+    assert st == 0 and np.array_equal(out_v, out) and np.array_equal(kv_k2, kv_k)
+    st, out_p, _, _ = run(oracle, case, token_count=2)
+    assert st == 0 and not out_p[2:].any() and out_p[:2].any()
+
+
+def test_argument_errors(oracle):
+    case = make_case(14, [(3, 2)], num_q_heads=2, num_kv_heads=2, head_dim=8, block_size=4)
+    assert run(oracle, dict(case, layer_idx=2))[0] == MO_DIMS
+    bad = dict(case, token_meta=case["token_meta"].copy())
+    bad["token_meta"][0, 0] = case["block_table"].shape[0]
+    assert run(oracle, bad)[0] == MO_DIMS  # seq_slot out of range (paged_attention_ref.c:815-818)
+    bad["token_meta"][0, 0] = 0
+    bad["token_meta"][0, 2] = case["kv_k"].shape[0] * 4
+    assert run(oracle, bad)[0] == MO_DIMS  # kv_slot block out of range (:819-822)
+    odd = dict(case, kv_k=np.zeros((4, 2, 2, 6, 8), np.float32), kv_v=np.zeros((4, 2, 2, 6, 8), np.float32))
+    assert run(oracle, odd)[0] == MO_INVALID  # block size not a power of two (:586-589)
+    three = dict(case, q=np.zeros((2, 3, 8), np.float32))
+    assert run(oracle, three)[0] == MO_INVALID  # 3 query heads over 2 kv heads (:590-595)
+    assert run(oracle, case, token_count=0)[0] == 0

@@ -61,6 +61,7 @@ enum {
 enum {
     MARMOT_HIP_DTYPE_F32 = 0,
     MARMOT_HIP_DTYPE_F16 = 1,
+    MARMOT_HIP_DTYPE_BF16 = 2, /* paged attention only: activations and KV cache */
     MARMOT_HIP_DTYPE_I32 = 3,  /* position tensors of the rotary epilogue only */
     MARMOT_HIP_DTYPE_U8 = 6,   /* storage type of block-quantized tensors (GGUF reader) */
     MARMOT_HIP_DTYPE_I64 = 11,
@@ -353,6 +354,41 @@ int marmot_hip_add(marmot_hip_device_t *dev, const float *d_a, const float *d_b,
  * DIMENSION_MISMATCH. */
 int marmot_hip_rope(marmot_hip_device_t *dev, const void *d_x, int dtype, size_t rows, size_t dim,
                     size_t x_row_stride, size_t out_row_stride, const marmot_hip_rope_t *rope, void *d_out);
+
+/* ------------------------------------------------------------------ paged attention
+ * Replaces cpu_paged_attention_impl (src/backends/cpu/ops/paged_attention/paged_attention_ref.c:573-1082; descriptor
+ * marmot_paged_attention_desc_t, include/marmot/ops/paged_attention.h:32-57) for FLOAT32 / FLOAT16 / BFLOAT16
+ * activations and KV caches (the FP8 cache of MARMOT_ENABLE_FP8 builds is not offered). The tensors of the descriptor
+ * arrive as device pointers with their strides in elements:
+ *   d_token_meta  [token_count, 4] uint32: seq_slot, pos, kv_slot, flags (flags are not read)
+ *   d_q, d_out    [tokens, num_q_heads, head_dim], d_k_new, d_v_new [tokens, num_kv_heads, head_dim] of act_dtype
+ *   d_kv_k, d_kv_v [kv_blocks, kv_layers, num_kv_heads, block_size, head_dim] of kv_dtype, updated in place
+ *   d_block_table [max_seqs, max_blocks_per_seq] uint32, 0xFFFFFFFF = no block
+ * First every token's new key / value rows are stored at its kv_slot (block = kv_slot / block_size, same storage
+ * type: the same bits, otherwise one conversion through FLOAT32), then out[t, h] = softmax(scale * q[t, h] . K) V over
+ * positions 0 .. pos of the token's sequence read through the block table (positions without a block are skipped, a
+ * token with no position gives zeros); FLOAT32 arithmetic, one rounding at the store. head_dim up to 256.
+ * validate_meta != 0: seq_slot and kv_slot ranges are checked on the device before anything is written and
+ * MARMOT_HIP_ERROR_DIMENSION_MISMATCH is returned (one stream synchronization; skipped while a graph is being
+ * captured). Without the check, tokens with an out-of-range slot are skipped. */
+typedef struct marmot_hip_paged_attention {
+    uint32_t token_count, layer_idx, num_q_heads, num_kv_heads, head_dim, block_size;
+    float scale;
+    int act_dtype, kv_dtype;
+    const uint32_t *d_token_meta;
+    size_t meta_stride[2];
+    const void *d_q, *d_k_new, *d_v_new;
+    size_t q_stride[3], k_stride[3], v_stride[3];
+    void *d_kv_k, *d_kv_v;
+    size_t kv_stride[5];
+    size_t kv_blocks, kv_layers;
+    const uint32_t *d_block_table;
+    size_t table_stride[2];
+    size_t max_seqs, max_blocks_per_seq;
+    void *d_out;
+    size_t out_stride[3];
+} marmot_hip_paged_attention_t;
+int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot_hip_paged_attention_t *args, int validate_meta);
 
 /* ------------------------------------------------------------------ MoE
  * Replaces cpu_topk_impl (src/backends/cpu/ops/moe/moe_ops.c:789-889): top-k over the last axis of

@@ -507,6 +507,75 @@ class HipBackend:
             for b in {d_x, d_p, d_f, d_o}:
                 b.free()
 
+    def paged_attention_args(self, dev_ptr, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out, layer_idx: int,
+                             scale: float, act_bf16: bool = False, kv_bf16: bool = False, token_count=None):
+        """marmot_hip_paged_attention_t over numpy arrays (shapes, dtypes and element strides) whose device addresses
+        dev_ptr(array) gives; bfloat16 tensors travel as uint16 bits."""
+        def code(a, bf16):
+            if bf16:
+                assert a.dtype == np.uint16
+                return capi.DT_BF16
+            return _np_dtype_id(a.dtype)
+
+        def strides(a):
+            return [st // a.itemsize for st in a.strides]
+
+        p = capi.PagedAttention()
+        p.token_count = q.shape[0] if token_count is None else token_count
+        p.layer_idx, p.scale = layer_idx, scale
+        p.num_q_heads, p.num_kv_heads, p.head_dim, p.block_size = q.shape[1], k_new.shape[1], q.shape[2], kv_k.shape[3]
+        p.act_dtype, p.kv_dtype = code(q, act_bf16), code(kv_k, kv_bf16)
+        p.d_token_meta, p.meta_stride = dev_ptr(token_meta), (C.c_size_t * 2)(*strides(token_meta))
+        p.d_q, p.d_k_new, p.d_v_new = dev_ptr(q), dev_ptr(k_new), dev_ptr(v_new)
+        p.q_stride = (C.c_size_t * 3)(*strides(q))
+        p.k_stride = (C.c_size_t * 3)(*strides(k_new))
+        p.v_stride = (C.c_size_t * 3)(*strides(v_new))
+        p.d_kv_k, p.d_kv_v, p.kv_stride = dev_ptr(kv_k), dev_ptr(kv_v), (C.c_size_t * 5)(*strides(kv_k))
+        p.kv_blocks, p.kv_layers = kv_k.shape[0], kv_k.shape[1]
+        p.d_block_table, p.table_stride = dev_ptr(block_table), (C.c_size_t * 2)(*strides(block_table))
+        p.max_seqs, p.max_blocks_per_seq = block_table.shape
+        p.d_out, p.out_stride = dev_ptr(out), (C.c_size_t * 3)(*strides(out))
+        return p
+
+    def paged_attention(self, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx: int, scale: float,
+                        act_bf16: bool = False, kv_bf16: bool = False, token_count=None, validate: bool = True):
+        """marmot_paged_attention (include/marmot/ops/paged_attention.h; CPU implementation
+        src/backends/cpu/ops/paged_attention/paged_attention_ref.c): token_meta [tokens, 4] uint32 (seq_slot, pos,
+        kv_slot, flags), q [tokens, q heads, head dim], k_new / v_new [tokens, kv heads, head dim] (float32, float16 or
+        uint16 holding bfloat16 bits; views with any strides), kv_k / kv_v [blocks, layers, kv heads, block size, head
+        dim] (updated in place), block_table [sequences, blocks per sequence] uint32. Returns out like q."""
+        out = np.zeros(q.shape, dtype=q.dtype)
+        arrays = [token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out]
+        roots = {}
+
+        def root_of(a):
+            while a.base is not None and isinstance(a.base, np.ndarray):
+                a = a.base
+            return a
+
+        for a in arrays:
+            r = root_of(a)
+            if id(r) not in roots:
+                assert r.flags.c_contiguous, "views must come from contiguous arrays"
+                roots[id(r)] = (r, self.to_device(r.reshape(-1).view(np.uint8)))
+
+        def dev_ptr(a):
+            r, d = roots[id(root_of(a))]
+            return d.ptr + (a.ctypes.data - r.ctypes.data)
+
+        p = self.paged_attention_args(dev_ptr, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out, layer_idx,
+                                      scale, act_bf16, kv_bf16, token_count)
+        try:
+            check(self.lib.marmot_hip_paged_attention(self.dev, C.byref(p), 1 if validate else 0))
+            for a in (kv_k, kv_v, out):
+                r, d = roots[id(root_of(a))]
+                flat = r.reshape(-1).view(np.uint8)
+                flat[...] = d.download(np.uint8, (flat.size,))
+            return out
+        finally:
+            for _, d in roots.values():
+                d.free()
+
     def packed_activation_layout(self, kind: int, N: int, K: int) -> "capi.PackedLayout":
         lay = capi.PackedLayout()
         check(self.lib.marmot_hip_packed_activation_layout(kind, N, K, C.byref(lay)))

@@ -11,6 +11,7 @@ KIND_Q4_1, KIND_Q5_0, KIND_Q5_1 = 2, 3, 4
 KIND_Q2_K, KIND_Q3_K = 7, 8
 KIND_Q8_1 = 6
 DT_F32, DT_F16 = 0, 1
+DT_BF16 = 2  # paged attention only
 DT_I32, DT_I64 = 3, 11  # position tensors of the rotary epilogue
 FLAG_FORCE_PACK = 1
 
@@ -42,6 +43,21 @@ class Rope(C.Structure):
     _fields_ = [("d_positions", C.c_void_p), ("positions_dtype", C.c_int), ("d_freqs", C.c_void_p),
                 ("attn_scale", C.c_float), ("head_dim", C.c_uint32), ("rope_type", C.c_int),
                 ("apply_to_q", C.c_int), ("apply_to_k", C.c_int)]
+
+
+class PagedAttention(C.Structure):
+    """marmot_hip_paged_attention_t: device pointers and element strides of the paged attention tensors"""
+    _fields_ = [("token_count", C.c_uint32), ("layer_idx", C.c_uint32), ("num_q_heads", C.c_uint32),
+                ("num_kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("block_size", C.c_uint32),
+                ("scale", C.c_float), ("act_dtype", C.c_int), ("kv_dtype", C.c_int),
+                ("d_token_meta", C.c_void_p), ("meta_stride", C.c_size_t * 2),
+                ("d_q", C.c_void_p), ("d_k_new", C.c_void_p), ("d_v_new", C.c_void_p),
+                ("q_stride", C.c_size_t * 3), ("k_stride", C.c_size_t * 3), ("v_stride", C.c_size_t * 3),
+                ("d_kv_k", C.c_void_p), ("d_kv_v", C.c_void_p), ("kv_stride", C.c_size_t * 5),
+                ("kv_blocks", C.c_size_t), ("kv_layers", C.c_size_t),
+                ("d_block_table", C.c_void_p), ("table_stride", C.c_size_t * 2),
+                ("max_seqs", C.c_size_t), ("max_blocks_per_seq", C.c_size_t),
+                ("d_out", C.c_void_p), ("out_stride", C.c_size_t * 3)]
 
 
 class GgufTensor(C.Structure):
@@ -122,6 +138,7 @@ SIGNATURES = {
     "marmot_hip_swiglu_pack": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
     "marmot_hip_add": (_i, [_vp, _vp, _vp, _sz, _vp]),
     "marmot_hip_rope": (_i, [_vp, _vp, _i, _sz, _sz, _sz, _sz, C.POINTER(Rope), _vp]),
+    "marmot_hip_paged_attention": (_i, [_vp, C.POINTER(PagedAttention), _i]),
     "marmot_hip_topk": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
     "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),
     "marmot_hip_moe_experts": (_i, [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp, _vp, _f, _i, _i,

@@ -1,0 +1,378 @@
+// Paged attention (marmot_paged_attention; CPU counterpart cpu_paged_attention_impl,
+// src/backends/cpu/ops/paged_attention/paged_attention_ref.c:573-1082): every token's new key / value rows are written
+// into the paged cache at the token's kv_slot, then every (token, query head) attends over positions 0 .. pos of its
+// sequence through the block table.
+//
+// Attention kernel: one workgroup of 256 threads per (token, query head), 16 groups of 16 lanes. A group walks the
+// positions g, g + 16, g + 32, ...: its 16 lanes split the head dimension (a lane holds EPL consecutive values of the
+// query, of the running output and of each key / value row, so a row is read as one contiguous run by the group), the
+// dot product is reduced inside the group with data-parallel-primitive moves, and the group keeps its own running
+// maximum, sum and output (online softmax). The 16 groups meet in LDS at the end. All arithmetic is fp32 like the
+// reference's; only the order of the sums differs (per group instead of per block of positions). Rows are read with
+// 16-byte loads when the head dimension is exactly 16 x EPL values with unit stride, element by element otherwise.
+// A token whose sequence slot or cache block is out of range is skipped (the host rejects such calls when it may read
+// the metadata, like the reference).
+#include "mh_common.h"
+
+#include <math.h>
+
+namespace mh {
+
+constexpr uint32_t PA_NO_BLOCK = 0xFFFFFFFFu;
+
+struct PaParams {
+    uint32_t token_count, layer_idx, num_q_heads, num_kv_heads, head_dim, block_size;
+    float scale;
+    int act_dtype, kv_dtype;
+    const uint32_t *meta;
+    size_t meta_stride[2];
+    const void *q, *k_new, *v_new;
+    size_t q_stride[3], k_stride[3], v_stride[3];
+    void *kv_k, *kv_v;
+    size_t kv_stride[5];
+    size_t kv_blocks, kv_layers;
+    const uint32_t *table;
+    size_t table_stride[2];
+    size_t max_seqs, max_blocks;
+    void *out;
+    size_t out_stride[3];
+    uint32_t shift, mask, group;
+    int q_vec, kv_vec;  // 16-byte loads of the query / of the cache rows
+    int *flag;          // metadata check: 1 + index of an offending token (maximum)
+};
+
+// marmot_f32_to_bf16_ref / marmot_bf16_to_f32_ref (src/utils/dtype_ref.c:86-104): round to nearest even on the bits
+__device__ __forceinline__ uint16_t pa_f2bf(float v) {
+    const uint32_t bits = __float_as_uint(v);
+    return (uint16_t)((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float pa_bf2f(uint16_t h) {
+    return __uint_as_float((uint32_t)h << 16);
+}
+
+__device__ __forceinline__ float pa_load(const void *data, int dtype, size_t i) {
+    if (dtype == MARMOT_HIP_DTYPE_F16) {
+        return h2f(((const uint16_t *)data)[i]);
+    }
+    if (dtype == MARMOT_HIP_DTYPE_BF16) {
+        return pa_bf2f(((const uint16_t *)data)[i]);
+    }
+    return ((const float *)data)[i];
+}
+
+__device__ __forceinline__ void pa_store(void *data, int dtype, size_t i, float v) {
+    if (dtype == MARMOT_HIP_DTYPE_F16) {
+        ((uint16_t *)data)[i] = f2h(v);
+    } else if (dtype == MARMOT_HIP_DTYPE_BF16) {
+        ((uint16_t *)data)[i] = pa_f2bf(v);
+    } else {
+        ((float *)data)[i] = v;
+    }
+}
+
+// EPL consecutive values starting at element `first` (unit stride, 16-byte aligned start for the storage type)
+template <int EPL>
+__device__ __forceinline__ void pa_load_run(const void *data, int dtype, size_t first, float (&v)[EPL]) {
+    if (dtype == MARMOT_HIP_DTYPE_F32) {
+#pragma unroll
+        for (int e = 0; e < EPL; e += 4) {
+            const float4 f = *(const float4 *)((const float *)data + first + e);
+            v[e] = f.x, v[e + 1] = f.y, v[e + 2] = f.z, v[e + 3] = f.w;
+        }
+    } else {
+        uint32_t w[EPL / 2];
+        if constexpr (EPL == 4) {
+            const uint2 u = *(const uint2 *)((const uint16_t *)data + first);
+            w[0] = u.x, w[1] = u.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL / 2; e += 4) {
+                const uint4 u = *(const uint4 *)((const uint16_t *)data + first + 2 * e);
+                w[e] = u.x, w[e + 1] = u.y, w[e + 2] = u.z, w[e + 3] = u.w;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < EPL / 2; ++e) {
+            if (dtype == MARMOT_HIP_DTYPE_F16) {
+                v[2 * e] = h2f((uint16_t)(w[e] & 0xffffu));
+                v[2 * e + 1] = h2f((uint16_t)(w[e] >> 16));
+            } else {
+                v[2 * e] = __uint_as_float(w[e] << 16);
+                v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+            }
+        }
+    }
+}
+
+// ---- metadata check (paged_attention_ref.c:809-823): sequence slots inside the block table, kv slots inside the cache
+__global__ __launch_bounds__(256) void k_pa_check(const PaParams p) {
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= p.token_count) {
+        return;
+    }
+    const uint32_t seq = p.meta[t * p.meta_stride[0]];
+    const uint32_t slot = p.meta[t * p.meta_stride[0] + 2 * p.meta_stride[1]];
+    if (seq >= p.max_seqs || (slot >> p.shift) >= p.kv_blocks) {
+        atomicMax(p.flag, (int)(p.token_count - t));  // the maximum names the first offender
+    }
+}
+
+// ---- cache write (cpu_paged_attention_kv_write_range, :346-373): one workgroup per (token, kv head)
+__global__ __launch_bounds__(128) void k_pa_write(const PaParams p) {
+    const uint32_t t = blockIdx.x, h = blockIdx.y;
+    const uint32_t slot = p.meta[t * p.meta_stride[0] + 2 * p.meta_stride[1]];
+    const uint32_t block = slot >> p.shift;
+    if (block >= p.kv_blocks) {
+        return;
+    }
+    const size_t dst0 = (size_t)block * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2] +
+                        (size_t)(slot & p.mask) * p.kv_stride[3];
+    const size_t k0 = (size_t)t * p.k_stride[0] + (size_t)h * p.k_stride[1];
+    const size_t v0 = (size_t)t * p.v_stride[0] + (size_t)h * p.v_stride[1];
+    const bool bits16 = p.act_dtype == p.kv_dtype && p.act_dtype != MARMOT_HIP_DTYPE_F32;
+    for (uint32_t d = threadIdx.x; d < p.head_dim; d += blockDim.x) {
+        const size_t dst = dst0 + d * p.kv_stride[4];
+        if (bits16) {  // same 16-bit storage type: the bits travel unchanged
+            ((uint16_t *)p.kv_k)[dst] = ((const uint16_t *)p.k_new)[k0 + d * p.k_stride[2]];
+            ((uint16_t *)p.kv_v)[dst] = ((const uint16_t *)p.v_new)[v0 + d * p.v_stride[2]];
+        } else {
+            pa_store(p.kv_k, p.kv_dtype, dst, pa_load(p.k_new, p.act_dtype, k0 + d * p.k_stride[2]));
+            pa_store(p.kv_v, p.kv_dtype, dst, pa_load(p.v_new, p.act_dtype, v0 + d * p.v_stride[2]));
+        }
+    }
+}
+
+// ---- attention (cpu_paged_attention_attention_range, :398-569)
+template <int EPL>
+__global__ __launch_bounds__(256) void k_pa_attend(const PaParams p) {
+    warm_kernel_arguments<sizeof(PaParams), sizeof(PaParams)>();
+    __shared__ float s_acc[16][16 * EPL];
+    __shared__ float s_m[16], s_l[16];
+    const uint32_t t = blockIdx.x, qh = blockIdx.y;
+    const int tid = threadIdx.x, g = tid >> 4, l = tid & 15;
+    const uint32_t seq = p.meta[t * p.meta_stride[0]];
+    const uint32_t pos = p.meta[t * p.meta_stride[0] + p.meta_stride[1]];
+    const uint32_t kv_len = seq < p.max_seqs ? pos + 1u : 0u;
+    const uint32_t kvh = qh / p.group;
+    const uint32_t d0 = (uint32_t)l * EPL;  // this lane's first value of the head dimension
+
+    float qv[EPL];
+    const size_t q_base = (size_t)t * p.q_stride[0] + (size_t)qh * p.q_stride[1];
+    if (p.q_vec) {
+        pa_load_run<EPL>(p.q, p.act_dtype, q_base + d0, qv);
+    } else {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            qv[e] = d0 + e < p.head_dim ? pa_load(p.q, p.act_dtype, q_base + (size_t)(d0 + e) * p.q_stride[2]) : 0.0f;
+        }
+    }
+    if (p.scale != 1.0f) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            qv[e] *= p.scale;
+        }
+    }
+
+    float m = -INFINITY, lsum = 0.0f;
+    float acc[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        acc[e] = 0.0f;
+    }
+    const size_t head_base = (size_t)p.layer_idx * p.kv_stride[1] + (size_t)kvh * p.kv_stride[2];
+    const uint32_t *table_row = p.table + (size_t)seq * p.table_stride[0];
+    for (uint32_t pp = (uint32_t)g; pp < kv_len; pp += 16u) {
+        const uint32_t logical = pp >> p.shift;
+        if (logical >= p.max_blocks) {
+            break;
+        }
+        const uint32_t tb = table_row[(size_t)logical * p.table_stride[1]];
+        if (tb == PA_NO_BLOCK || tb >= p.kv_blocks) {
+            continue;
+        }
+        const size_t base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(pp & p.mask) * p.kv_stride[3];
+        float kr[EPL], vr[EPL];
+        if (p.kv_vec) {
+            pa_load_run<EPL>(p.kv_k, p.kv_dtype, base + d0, kr);
+            pa_load_run<EPL>(p.kv_v, p.kv_dtype, base + d0, vr);
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const bool in = d0 + e < p.head_dim;
+                const size_t i = base + (size_t)(d0 + e) * p.kv_stride[4];
+                kr[e] = in ? pa_load(p.kv_k, p.kv_dtype, i) : 0.0f;
+                vr[e] = in ? pa_load(p.kv_v, p.kv_dtype, i) : 0.0f;
+            }
+        }
+        float dot = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            dot = __builtin_fmaf(qv[e], kr[e], dot);
+        }
+        dot = row16_sum(dot);
+        if (dot > m) {  // the same decision in all 16 lanes of the group
+            const float corr = m == -INFINITY ? 0.0f : expf(m - dot);
+            lsum *= corr;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                acc[e] *= corr;
+            }
+            m = dot;
+        }
+        const float w = expf(dot - m);
+        lsum += w;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            acc[e] = __builtin_fmaf(w, vr[e], acc[e]);
+        }
+    }
+
+    // the 16 groups meet: out = sum_g acc_g * exp(m_g - M) / sum_g l_g * exp(m_g - M)
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        s_acc[g][d0 + e] = acc[e];
+    }
+    if (l == 0) {
+        s_m[g] = m;
+        s_l[g] = lsum;
+    }
+    __syncthreads();
+    const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)qh * p.out_stride[1];
+    for (uint32_t d = (uint32_t)tid; d < p.head_dim; d += 256u) {
+        float big = -INFINITY;
+#pragma unroll
+        for (int gg = 0; gg < 16; ++gg) {
+            big = fmaxf(big, s_m[gg]);
+        }
+        float o = 0.0f;
+        if (big != -INFINITY) {  // has_any (:552-557)
+            float total = 0.0f;
+#pragma unroll
+            for (int gg = 0; gg < 16; ++gg) {
+                const float f = s_m[gg] == -INFINITY ? 0.0f : expf(s_m[gg] - big);
+                total = __builtin_fmaf(s_l[gg], f, total);
+                o = __builtin_fmaf(s_acc[gg][d], f, o);
+            }
+            o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        }
+        pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
+    }
+}
+
+static bool pa_float_dtype(int d) {
+    return d == MARMOT_HIP_DTYPE_F32 || d == MARMOT_HIP_DTYPE_F16 || d == MARMOT_HIP_DTYPE_BF16;
+}
+
+static size_t pa_elem_size(int d) {
+    return d == MARMOT_HIP_DTYPE_F32 ? 4 : 2;
+}
+
+} // namespace mh
+
+using namespace mh;
+
+extern "C" int marmot_hip_fill_bytes_internal(marmot_hip_device_t *dev, void *d_dst, int value, size_t size);
+
+extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot_hip_paged_attention_t *a,
+                                          int validate_meta) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
+    }
+    if (a == nullptr || a->d_token_meta == nullptr || a->d_q == nullptr || a->d_k_new == nullptr ||
+        a->d_v_new == nullptr || a->d_kv_k == nullptr || a->d_kv_v == nullptr || a->d_block_table == nullptr ||
+        a->d_out == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention descriptor invalid");
+    }
+    if (a->token_count == 0) {
+        return MARMOT_HIP_SUCCESS;
+    }
+    if (a->num_q_heads == 0 || a->num_kv_heads == 0 || a->head_dim == 0 || a->block_size == 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention requires non-zero dimensions");
+    }
+    if ((a->block_size & (a->block_size - 1u)) != 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention block_size must be power of two");
+    }
+    if (a->num_q_heads % a->num_kv_heads != 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention requires num_q_heads divisible by num_kv_heads");
+    }
+    if (!pa_float_dtype(a->act_dtype) || !pa_float_dtype(a->kv_dtype)) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "paged_attention dtype not supported");
+    }
+    if (a->kv_layers <= a->layer_idx) {
+        return set_error(MARMOT_HIP_ERROR_DIMENSION_MISMATCH, "paged_attention layer_idx out of range");
+    }
+    if (a->head_dim > 256) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "paged_attention: head_dim %u is more than 256", a->head_dim);
+    }
+    if (a->num_q_heads > 65535u || a->num_kv_heads > 65535u) {
+        return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "paged_attention: more than 65535 heads");
+    }
+    MH_HIP(hipSetDevice(dev->device_index));
+    PaParams p;
+    p.token_count = a->token_count, p.layer_idx = a->layer_idx, p.num_q_heads = a->num_q_heads;
+    p.num_kv_heads = a->num_kv_heads, p.head_dim = a->head_dim, p.block_size = a->block_size;
+    p.scale = a->scale, p.act_dtype = a->act_dtype, p.kv_dtype = a->kv_dtype;
+    p.meta = a->d_token_meta, p.q = a->d_q, p.k_new = a->d_k_new, p.v_new = a->d_v_new;
+    p.kv_k = a->d_kv_k, p.kv_v = a->d_kv_v, p.table = a->d_block_table, p.out = a->d_out;
+    for (int i = 0; i < 2; ++i) {
+        p.meta_stride[i] = a->meta_stride[i];
+        p.table_stride[i] = a->table_stride[i];
+    }
+    for (int i = 0; i < 3; ++i) {
+        p.q_stride[i] = a->q_stride[i], p.k_stride[i] = a->k_stride[i], p.v_stride[i] = a->v_stride[i];
+        p.out_stride[i] = a->out_stride[i];
+    }
+    for (int i = 0; i < 5; ++i) {
+        p.kv_stride[i] = a->kv_stride[i];
+    }
+    p.kv_blocks = a->kv_blocks, p.kv_layers = a->kv_layers, p.max_seqs = a->max_seqs, p.max_blocks = a->max_blocks_per_seq;
+    p.shift = 0;
+    while ((1u << p.shift) < a->block_size) {
+        ++p.shift;
+    }
+    p.mask = a->block_size - 1u;
+    p.group = a->num_q_heads / a->num_kv_heads;
+    const int epl = a->head_dim <= 64 ? 4 : (a->head_dim <= 128 ? 8 : 16);
+    // 16-byte runs: the head dimension is exactly 16 lanes x EPL values, unit stride, every row start 16-byte aligned
+    const size_t asz = pa_elem_size(a->act_dtype), ksz = pa_elem_size(a->kv_dtype);
+    const size_t run_a = (size_t)epl * asz < 16 ? (size_t)epl * asz : 16, run_k = (size_t)epl * ksz < 16 ? (size_t)epl * ksz : 16;
+    const bool exact = a->head_dim == (uint32_t)(16 * epl);
+    p.q_vec = exact && a->q_stride[2] == 1 && (((uintptr_t)a->d_q) % run_a) == 0 && (a->q_stride[0] * asz) % run_a == 0 &&
+              (a->q_stride[1] * asz) % run_a == 0;
+    p.kv_vec = exact && a->kv_stride[4] == 1 && (((uintptr_t)a->d_kv_k) % run_k) == 0 &&
+               (((uintptr_t)a->d_kv_v) % run_k) == 0;
+    for (int i = 0; i < 4 && p.kv_vec; ++i) {
+        p.kv_vec = (a->kv_stride[i] * ksz) % run_k == 0;
+    }
+    p.flag = nullptr;
+    if (validate_meta != 0 && !dev->capturing) {
+        void *ws = nullptr;
+        MH_TRY(workspace_reserve(dev, 256, &ws));
+        p.flag = (int *)ws;
+        MH_TRY(marmot_hip_fill_bytes_internal(dev, ws, 0, sizeof(int)));
+        hipLaunchKernelGGL(k_pa_check, dim3((a->token_count + 255) / 256), dim3(256), 0, dev->stream, p);
+        MH_HIP(hipGetLastError());
+        int host_flag = 0;
+        MH_HIP(hipMemcpyAsync(&host_flag, p.flag, sizeof(int), hipMemcpyDeviceToHost, dev->stream));
+        MH_HIP(hipStreamSynchronize(dev->stream));
+        if (host_flag != 0) {
+            return set_error(MARMOT_HIP_ERROR_DIMENSION_MISMATCH,
+                             "paged_attention seq_slot or kv_slot block out of range at token %u",
+                             a->token_count - (uint32_t)host_flag);
+        }
+    }
+    hipLaunchKernelGGL(k_pa_write, dim3(a->token_count, a->num_kv_heads), dim3(a->head_dim <= 64 ? 64 : 128), 0,
+                       dev->stream, p);
+    MH_HIP(hipGetLastError());
+    const dim3 grid(a->token_count, a->num_q_heads);
+    if (epl == 4) {
+        hipLaunchKernelGGL(k_pa_attend<4>, grid, dim3(256), 0, dev->stream, p);
+    } else if (epl == 8) {
+        hipLaunchKernelGGL(k_pa_attend<8>, grid, dim3(256), 0, dev->stream, p);
+    } else {
+        hipLaunchKernelGGL(k_pa_attend<16>, grid, dim3(256), 0, dev->stream, p);
+    }
+    MH_HIP(hipGetLastError());
+    set_route("paged_attention");
+    return MARMOT_HIP_SUCCESS;
+}

@@ -1,0 +1,134 @@
+"""GPU parity: paged attention through the C ABI against the CPU oracle and against dense float64 attention: the cache
+write is bit-exact (pure data movement and one dtype conversion), the attention output agrees within fp32 summation
+noise (both sides accumulate in fp32, in different orders) plus one rounding of the output type."""
+import numpy as np
+import pytest
+
+from marmot_amd import capi
+from tests.attention_cases import NO_BLOCK, TOLERANCE, cache_after_write, dense_reference, make_case, to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from marmot_amd import HipBackend
+
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def run_hip(hip, case, **kw):
+    kv_k, kv_v = case["kv_k"].copy(), case["kv_v"].copy()
+    out = hip.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], kv_k, kv_v,
+                              case["block_table"], case["layer_idx"], case["scale"], act_bf16=case["act"] == "bf16",
+                              kv_bf16=case["kv"] == "bf16", **kw)
+    return out, kv_k, kv_v
+
+
+def run_oracle(oracle, case, **kw):
+    kv_k, kv_v = case["kv_k"].copy(), case["kv_v"].copy()
+    st, out = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], kv_k, kv_v,
+                                     case["block_table"], case["layer_idx"], case["scale"],
+                                     act_bf16=case["act"] == "bf16", kv_bf16=case["kv"] == "bf16", **kw)
+    assert st == 0
+    return out, kv_k, kv_v
+
+
+def check(hip, oracle, case, what):
+    got, kv_k, kv_v = run_hip(hip, case)
+    assert hip.last_route() == "paged_attention"
+    ref, ref_k, ref_v = run_oracle(oracle, case)
+    assert np.array_equal(kv_k.view(np.uint8), ref_k.view(np.uint8)), f"{what}: key cache"
+    assert np.array_equal(kv_v.view(np.uint8), ref_v.view(np.uint8)), f"{what}: value cache"
+    act, kv = case["act"], case["kv"]
+    vmax = np.abs(to_f32(ref_v, kv)).max()
+    g32, r32 = to_f32(got, act).astype(np.float64), to_f32(ref, act).astype(np.float64)
+    assert np.max(np.abs(g32 - r32)) <= TOLERANCE[act] * vmax, f"{what}: against the oracle"
+    dense = dense_reference(case, ref_k, ref_v)
+    assert np.max(np.abs(g32 - dense)) <= TOLERANCE[act] * vmax, f"{what}: against dense float64 attention"
+
+
+def test_reference_closed_form_case(hip):
+    """tests/backend/test_backend_paged_attention.c:162-288"""
+    eye = np.array([[[1.0, 0.0]], [[0.0, 1.0]]], dtype=np.float32)
+    meta = np.array([[0, 0, 0, 2], [0, 1, 1, 1]], dtype=np.uint32)
+    kv_k = np.zeros((1, 1, 1, 4, 2), np.float32)
+    kv_v = np.zeros_like(kv_k)
+    out = hip.paged_attention(meta, eye, eye.copy(), eye.copy(), kv_k, kv_v, np.zeros((1, 1), np.uint32), 0, 1.0)
+    e = np.exp(np.float32(1.0))
+    assert abs(out[0, 0, 0] - 1.0) < 1e-4 and abs(out[0, 0, 1]) < 1e-4
+    assert abs(out[1, 0, 0] - 1.0 / (1.0 + e)) < 1e-4 and abs(out[1, 0, 1] - e / (1.0 + e)) < 1e-4
+    for cache in (kv_k, kv_v):
+        assert np.array_equal(cache[0, 0, 0, :2], np.eye(2, dtype=np.float32)) and not cache[0, 0, 0, 2:].any()
+
+
+@pytest.mark.parametrize("act,kv", [("f32", "f32"), ("f16", "f16"), ("f32", "f16"), ("f16", "f32"), ("bf16", "bf16"),
+                                    ("f32", "bf16"), ("bf16", "f16")])
+@pytest.mark.parametrize("head_dim", [64, 128, 256])
+def test_dtypes_and_head_dims(hip, oracle, act, kv, head_dim):
+    case = make_case(21 + head_dim, [(37, 1), (0, 19), (130, 5), (64, 1)], num_q_heads=8, num_kv_heads=2,
+                     head_dim=head_dim, block_size=16, act=act, kv=kv)
+    check(hip, oracle, case, f"{act}/{kv} head_dim={head_dim}")
+
+
+@pytest.mark.parametrize("head_dim,block_size,hq,hkv", [(2, 4, 1, 1), (40, 8, 6, 3), (80, 1, 4, 4), (96, 32, 2, 1),
+                                                        (200, 64, 3, 1), (128, 256, 4, 2)])
+def test_ragged_head_dims_and_block_sizes(hip, oracle, head_dim, block_size, hq, hkv):
+    """Head dimensions that are not 16 x 4 / 8 / 16 values take the element-wise loads; block sizes from 1 to 256."""
+    case = make_case(40 + head_dim, [(70, 3), (9, 1), (0, 2)], num_q_heads=hq, num_kv_heads=hkv, head_dim=head_dim,
+                     block_size=block_size, act="f32", kv="f16")
+    check(hip, oracle, case, f"head_dim={head_dim} block={block_size}")
+
+
+def test_long_context_decode_batch(hip, oracle):
+    """16 sequences with 1000 to 3000 positions of history, one token each, grouped query heads, fp16 cache."""
+    rng = np.random.default_rng(50)
+    seqs = [(int(h), 1) for h in rng.integers(1000, 3000, 16)]
+    case = make_case(51, seqs, num_q_heads=8, num_kv_heads=2, head_dim=128, block_size=16, act="f32", kv="f16",
+                     layers=1, layer_idx=0)
+    check(hip, oracle, case, "decode batch")
+
+
+def test_holes_strided_views_token_count_and_errors(hip, oracle):
+    case = make_case(13, [(40, 3), (5, 1)], num_q_heads=4, num_kv_heads=2, head_dim=32, block_size=8)
+    seq = case["token_meta"][0, 0]
+    case["block_table"][seq, 1] = NO_BLOCK
+    check(hip, oracle, case, "hole in the block table")
+    empty = dict(case, block_table=np.full_like(case["block_table"], NO_BLOCK))
+    out0, _, _ = run_hip(hip, empty)
+    assert not out0.any()
+    # q / k_new / v_new as views of one buffer (what a fused projection leaves), fewer tokens than rows
+    T = case["q"].shape[0]
+    fused = np.zeros((T, 8, 32), np.float32)
+    fused[:, :4], fused[:, 4:6], fused[:, 6:] = case["q"], case["k_new"], case["v_new"]
+    view = dict(case, q=fused[:, :4], k_new=fused[:, 4:6], v_new=fused[:, 6:])
+    plain, kv_k, _ = run_hip(hip, case)
+    out_v, kv_k2, _ = run_hip(hip, view)
+    assert np.array_equal(out_v, plain) and np.array_equal(kv_k2, kv_k)
+    out_p, kv_p, _ = run_hip(hip, case, token_count=2)  # only the first two tokens are stored and served
+    ref_p, ref_kp, _ = run_oracle(oracle, case, token_count=2)
+    assert not out_p[2:].any() and np.array_equal(kv_p, ref_kp)
+    assert np.max(np.abs(out_p - ref_p)) <= TOLERANCE["f32"] * np.abs(case["kv_v"]).max()
+    # errors, in the reference's order and with its codes
+    def code(c, **kw):
+        with pytest.raises(capi.MarmotHipError) as e:
+            run_hip(hip, c, **kw)
+        return e.value.code
+    assert code(dict(case, layer_idx=2)) == -7
+    bad = dict(case, token_meta=case["token_meta"].copy())
+    bad["token_meta"][1, 0] = case["block_table"].shape[0]
+    assert code(bad) == -7
+    bad["token_meta"][1, 0] = 0
+    bad["token_meta"][1, 2] = case["kv_k"].shape[0] * 8
+    assert code(bad) == -7
+    # without the check such a token is skipped: nothing outside the buffers is touched, the other tokens are served
+    out_s, _, _ = run_hip(hip, bad, validate=False)
+    keep = [t for t in range(T) if t != 1]
+    assert np.isfinite(out_s).all() and out_s[keep].any()
+    odd = dict(case, kv_k=np.zeros((4, 2, 2, 6, 32), np.float32), kv_v=np.zeros((4, 2, 2, 6, 32), np.float32))
+    assert code(odd) == -1
+    assert code(dict(case, q=np.zeros((T, 3, 32), np.float32))) == -1
+    big = make_case(14, [(3, 1)], num_q_heads=1, num_kv_heads=1, head_dim=320, block_size=4)
+    assert code(big) == -8  # head dimensions beyond 256 are left to the caller's fallback

@@ -352,6 +352,38 @@ struct marmot_embedding_gather_desc {
 };
 typedef struct marmot_embedding_gather_desc marmot_embedding_gather_desc_t;
 
+/* include/marmot/ops/paged_attention.h:14-19, 32-57 */
+#define MARMOT_PAGED_ATTENTION_DESC_VERSION 1
+#define MARMOT_PAGED_ATTENTION_KV_SCALE_EXT_VERSION 1
+typedef struct {
+    uint32_t struct_size;
+    uint32_t struct_version;
+    const marmot_tensor_t *kv_k_scale;
+    const marmot_tensor_t *kv_v_scale;
+} marmot_paged_attention_kv_scale_ext_t;
+typedef struct {
+    uint32_t struct_size;
+    uint32_t struct_version;
+    uint64_t flags;
+    uint32_t token_count;
+    uint32_t layer_idx;
+    uint32_t num_q_heads;
+    uint32_t num_kv_heads;
+    uint32_t head_dim;
+    uint32_t block_size;
+    float scale;
+    const marmot_tensor_t *token_meta;
+    const marmot_tensor_t *q;
+    const marmot_tensor_t *k_new;
+    const marmot_tensor_t *v_new;
+    const marmot_tensor_t *kv_k;
+    const marmot_tensor_t *kv_v;
+    const marmot_tensor_t *block_table;
+    marmot_tensor_t *out;
+    const void *pnext;
+    uint64_t reserved[4];
+} marmot_paged_attention_desc_t;
+
 /* include/marmot/traits_ids.gen.h:40-107 (the operations this backend answers for), :111-116, :120-133 */
 typedef enum {
     MARMOT_OP_INVALID = 0,
@@ -362,6 +394,7 @@ typedef enum {
     MARMOT_OP_GEGLU = 410,
     MARMOT_OP_RMS_NORM_GEMMA = 447,
     MARMOT_OP_MATMUL = 498,
+    MARMOT_OP_PAGED_ATTENTION = 503,
     MARMOT_OP_QUANTIZE = 524,
     MARMOT_OP_LINEAR = 708,
     MARMOT_OP_QKV_SHARED_INPUT = 771,
@@ -685,7 +718,10 @@ bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_bac
  *   RMS_NORM    u16 input, weight, residual (0xFFFF none), output; f32 eps      (bytecode_compile.c:530-552)
  *   BINARY      u16 input_a, input_b, output                            (bytecode_compile.c:357-375)
  *   ROPE        u16 input, output, positions (0xFFFF: the parameters' own tensor); u32 rope-params const offset;
- *               u32 n_past; u32 n_rot                                   (bytecode_compile.c:598-623) */
+ *               u32 n_past; u32 n_rot                                   (bytecode_compile.c:598-623)
+ *   PAGED_ATTENTION u16 token_meta, q, k_new, v_new, kv_k, kv_v, block_table, kv_k_scale, kv_v_scale (0xFFFF none),
+ *               out; u32 token_count, layer_idx, num_q_heads, num_kv_heads, head_dim, block_size; f32 scale
+ *                                                                       (bytecode_compile.c:553-597) */
 enum {
     MARMOT_HIP_BC_OP_END = 0,
     MARMOT_HIP_BC_OP_MATMUL_Q4_0 = 1,
@@ -744,7 +780,9 @@ enum {
     MARMOT_HIP_BC_OP_ADD_F32 = 52,
     /* rotary embedding of FLOAT32 or FLOAT16 rows */
     MARMOT_HIP_BC_OP_ROPE = 53,
-    MARMOT_HIP_BC_OP_COUNT = 54,
+    /* paged attention: cache write + attention through the block table */
+    MARMOT_HIP_BC_OP_PAGED_ATTENTION = 54,
+    MARMOT_HIP_BC_OP_COUNT = 55,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -831,6 +869,14 @@ marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, con
  * params->positions (FLOAT32, INT32 or INT64, as many values as x has rows); frequencies and attention scale as
  * marmot_rope_freq_cache_ensure for the rotated dimension (src/core/helpers/rope.c:143-200), all scaling types.
  * Contiguous tensors, or rows at one stride >= their length; FLOAT64 and BFLOAT16 are declined NOT_IMPLEMENTED. */
+/* marmot_paged_attention (cf. cpu_paged_attention_impl, src/backends/cpu/ops/paged_attention/paged_attention_ref.c:
+ * 573-1082): every token's k_new / v_new rows go into the paged cache at its kv_slot, then every token attends over
+ * positions 0 .. pos of its sequence through the block table. q / k_new / v_new / out of one type among FLOAT32,
+ * FLOAT16, BFLOAT16 and the cache of one of these types, any strides; validation, codes and messages in the
+ * reference's order. Declined with NOT_IMPLEMENTED: the FLOAT8_E4M3 cache (with its scale tensors in pnext) and head
+ * dimensions beyond 256. The cache tensors are read and written: their mirrors are brought up to date first and the
+ * device copy is the current one afterwards. */
+marmot_error_t hip_paged_attention_impl(const void *device_ctx, const marmot_paged_attention_desc_t *desc);
 marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
                         marmot_tensor_t *out);
 /* output->quant_kind selects the block format: the activation formats Q8_0 and Q8_K (FLOAT32 or FLOAT16 input) or the

@@ -1638,6 +1638,206 @@ static marmot_error_t rope(const void *device_ctx, const marmot_tensor_t *x, con
     return st;
 }
 
+// ------------------------------------------------------------------ paged attention
+static bool pa_float_dtype(marmot_dtype_t t) {
+    return t == MARMOT_DTYPE_FLOAT32 || t == MARMOT_DTYPE_FLOAT16 || t == MARMOT_DTYPE_BFLOAT16;
+}
+
+static int pa_lib_dtype(marmot_dtype_t t) {
+    return t == MARMOT_DTYPE_FLOAT16 ? MARMOT_HIP_DTYPE_F16
+        : t == MARMOT_DTYPE_BFLOAT16 ? MARMOT_HIP_DTYPE_BF16
+                                     : MARMOT_HIP_DTYPE_F32;
+}
+
+// bytes from the first to one past the last element of a tensor of any rank and strides
+static size_t strided_extent_bytes(const marmot_tensor_t *t) {
+    size_t last = 0;
+    for (size_t i = 0; i < t->shape.ndim; ++i) {
+        if (t->shape.shape[i] == 0) {
+            return 0;
+        }
+        last += (t->shape.shape[i] - 1) * t->shape.strides[i];
+    }
+    return (last + 1) * dtype_size(t->dtype);
+}
+
+// marmot_paged_attention: the checks of cpu_paged_attention_impl (paged_attention_ref.c:573-823) in its order, then
+// the library call on the mirrors. The token metadata is a host tensor here, so its ranges are checked on the host.
+static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged_attention_desc_t *desc) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention: null device context");
+    }
+    if (desc == nullptr || desc->struct_version != MARMOT_PAGED_ATTENTION_DESC_VERSION ||
+        desc->struct_size < sizeof(marmot_paged_attention_desc_t) || desc->token_meta == nullptr || desc->q == nullptr ||
+        desc->k_new == nullptr || desc->v_new == nullptr || desc->kv_k == nullptr || desc->kv_v == nullptr ||
+        desc->block_table == nullptr || desc->out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention descriptor invalid");
+    }
+    if (desc->token_count == 0) {
+        return MARMOT_SUCCESS;
+    }
+    if (desc->num_q_heads == 0 || desc->num_kv_heads == 0 || desc->head_dim == 0 || desc->block_size == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention requires non-zero dimensions");
+    }
+    if ((desc->block_size & (desc->block_size - 1u)) != 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention block_size must be power of two");
+    }
+    if (desc->num_q_heads % desc->num_kv_heads != 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention requires num_q_heads divisible by num_kv_heads");
+    }
+    const marmot_tensor_t *meta = desc->token_meta, *q = desc->q, *k_new = desc->k_new, *v_new = desc->v_new;
+    const marmot_tensor_t *kv_k = desc->kv_k, *kv_v = desc->kv_v, *table = desc->block_table;
+    marmot_tensor_t *out = desc->out;
+    const marmot_paged_attention_kv_scale_ext_t *ext = (const marmot_paged_attention_kv_scale_ext_t *)desc->pnext;
+    const bool has_scales = ext != nullptr && ext->struct_version == MARMOT_PAGED_ATTENTION_KV_SCALE_EXT_VERSION &&
+        ext->struct_size >= sizeof(*ext) && (ext->kv_k_scale != nullptr || ext->kv_v_scale != nullptr);
+    if (meta->dtype != MARMOT_DTYPE_UINT32 || table->dtype != MARMOT_DTYPE_UINT32) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "paged_attention requires uint32 metadata");
+    }
+    const bool kv_fp8 = kv_k->dtype == MARMOT_DTYPE_FLOAT8_E4M3 && kv_v->dtype == MARMOT_DTYPE_FLOAT8_E4M3;
+    if (!pa_float_dtype(q->dtype) || !pa_float_dtype(k_new->dtype) || !pa_float_dtype(v_new->dtype) ||
+        !pa_float_dtype(out->dtype) || (!kv_fp8 && (!pa_float_dtype(kv_k->dtype) || !pa_float_dtype(kv_v->dtype)))) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "paged_attention dtype not supported");
+    }
+    if (q->dtype != k_new->dtype || q->dtype != v_new->dtype || q->dtype != out->dtype) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "paged_attention requires matching q/k_new/v_new/out dtypes");
+    }
+    if (meta->shape.ndim != 2 || meta->shape.shape[1] != 4 || meta->shape.shape[0] != desc->token_count) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention token_meta shape invalid");
+    }
+    if (table->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention block_table must be 2D");
+    }
+    if (q->shape.ndim != 3 || k_new->shape.ndim != 3 || v_new->shape.ndim != 3 || out->shape.ndim != 3) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention expects 3D q/k_new/v_new/out tensors");
+    }
+    if (q->shape.shape[0] < desc->token_count || k_new->shape.shape[0] < desc->token_count ||
+        v_new->shape.shape[0] < desc->token_count || out->shape.shape[0] < desc->token_count) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention token_count exceeds tensor rows");
+    }
+    if (q->shape.shape[1] != desc->num_q_heads || out->shape.shape[1] != desc->num_q_heads) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention num_q_heads mismatch");
+    }
+    if (k_new->shape.shape[1] != desc->num_kv_heads || v_new->shape.shape[1] != desc->num_kv_heads) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention num_kv_heads mismatch");
+    }
+    if (q->shape.shape[2] != desc->head_dim || k_new->shape.shape[2] != desc->head_dim ||
+        v_new->shape.shape[2] != desc->head_dim || out->shape.shape[2] != desc->head_dim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention head_dim mismatch");
+    }
+    if (kv_k->shape.ndim != 5 || kv_v->shape.ndim != 5) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention kv cache must be 5D");
+    }
+    if (kv_k->shape.shape[1] <= desc->layer_idx) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention layer_idx out of range");
+    }
+    if (kv_k->shape.shape[2] != desc->num_kv_heads || kv_v->shape.shape[2] != desc->num_kv_heads) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention kv head mismatch");
+    }
+    if (kv_k->shape.shape[3] != desc->block_size || kv_v->shape.shape[3] != desc->block_size) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention block_size mismatch");
+    }
+    if (kv_k->shape.shape[4] != desc->head_dim || kv_v->shape.shape[4] != desc->head_dim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention kv head_dim mismatch");
+    }
+    if (kv_k->dtype != kv_v->dtype) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention kv dtype mismatch");
+    }
+    if (kv_fp8) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP paged_attention does not handle the FLOAT8_E4M3 cache");
+    }
+    if (has_scales) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention scale tensors require FP8 KV");
+    }
+    if (meta->data == nullptr || table->data == nullptr || q->data == nullptr || k_new->data == nullptr ||
+        v_new->data == nullptr || kv_k->data == nullptr || kv_v->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention requires non-null tensor data");
+    }
+    uint32_t shift = 0;
+    while ((1u << shift) < desc->block_size) {
+        ++shift;
+    }
+    const uint32_t *meta_host = (const uint32_t *)meta->data;
+    for (size_t t = 0; t < desc->token_count; ++t) {
+        const uint32_t seq_slot = meta_host[t * meta->shape.strides[0]];
+        const uint32_t kv_slot = meta_host[t * meta->shape.strides[0] + 2 * meta->shape.strides[1]];
+        if (seq_slot >= table->shape.shape[0]) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention seq_slot out of range");
+        }
+        if ((kv_slot >> shift) >= kv_k->shape.shape[0]) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention kv_slot block out of range");
+        }
+    }
+    if (desc->head_dim > 256) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP paged_attention handles head dimensions up to 256");
+    }
+    for (size_t i = 0; i < 5; ++i) {
+        if (kv_k->shape.strides[i] != kv_v->shape.strides[i]) {
+            return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP paged_attention needs key and value caches of one layout");
+        }
+    }
+    marmot_hip_paged_attention_t a = {
+        .token_count = desc->token_count, .layer_idx = desc->layer_idx, .num_q_heads = desc->num_q_heads,
+        .num_kv_heads = desc->num_kv_heads, .head_dim = desc->head_dim, .block_size = desc->block_size,
+        .scale = desc->scale, .act_dtype = pa_lib_dtype(q->dtype), .kv_dtype = pa_lib_dtype(kv_k->dtype),
+        .kv_blocks = kv_k->shape.shape[0], .kv_layers = kv_k->shape.shape[1],
+        .max_seqs = table->shape.shape[0], .max_blocks_per_seq = table->shape.shape[1],
+    };
+    for (size_t i = 0; i < 2; ++i) {
+        a.meta_stride[i] = meta->shape.strides[i];
+        a.table_stride[i] = table->shape.strides[i];
+    }
+    for (size_t i = 0; i < 3; ++i) {
+        a.q_stride[i] = q->shape.strides[i];
+        a.k_stride[i] = k_new->shape.strides[i];
+        a.v_stride[i] = v_new->shape.strides[i];
+        a.out_stride[i] = out->shape.strides[i];
+    }
+    for (size_t i = 0; i < 5; ++i) {
+        a.kv_stride[i] = kv_k->shape.strides[i];
+    }
+    pthread_mutex_lock(&b->mu);
+    const void *d_meta = nullptr, *d_q = nullptr, *d_k = nullptr, *d_v = nullptr, *d_table = nullptr;
+    void *d_kv_k = nullptr, *d_kv_v = nullptr, *d_out = nullptr;
+    marmot_error_t st = acquire_read(b, meta->data, strided_extent_bytes(meta), &d_meta);
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, table->data, strided_extent_bytes(table), &d_table);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, q->data, strided_extent_bytes(q), &d_q);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, k_new->data, strided_extent_bytes(k_new), &d_k);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_read(b, v_new->data, strided_extent_bytes(v_new), &d_v);
+    }
+    // the caches are read and written; the output may be a view with gaps: the host's bytes go up first
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write_rows(b, kv_k->data, strided_extent_bytes(kv_k), true, &d_kv_k);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write_rows(b, kv_v->data, strided_extent_bytes(kv_v), true, &d_kv_v);
+    }
+    if (st == MARMOT_SUCCESS) {
+        st = acquire_write_rows(b, out->data, strided_extent_bytes(out), true, &d_out);
+    }
+    if (st == MARMOT_SUCCESS) {
+        a.d_token_meta = (const uint32_t *)d_meta, a.d_block_table = (const uint32_t *)d_table;
+        a.d_q = d_q, a.d_k_new = d_k, a.d_v_new = d_v, a.d_kv_k = d_kv_k, a.d_kv_v = d_kv_v, a.d_out = d_out;
+        const int rc = marmot_hip_paged_attention(b->dev, &a, 0);
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+        mark_device_output((marmot_tensor_t *)kv_k);
+        mark_device_output((marmot_tensor_t *)kv_v);
+    }
+    return st;
+}
+
 static uint16_t rd_u16(const uint8_t **pc) {
     const uint16_t v = (uint16_t)((*pc)[0] | ((*pc)[1] << 8));
     *pc += 2;
@@ -1967,6 +2167,40 @@ static marmot_error_t bc_exec_rope(const void *exec_ctx, marmot_tensor_t **regs,
     return rope(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, x, params_ptr, out);
 }
 
+// PAGED_ATTENTION immediates (bytecode_compile.c:553-597) -> the descriptor the generated shim builds
+static marmot_error_t bc_exec_paged_attention(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                              const uint8_t *const_pool) {
+    (void)const_pool;
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    marmot_paged_attention_desc_t desc = {.struct_size = sizeof(desc), .struct_version = MARMOT_PAGED_ATTENTION_DESC_VERSION};
+    desc.token_meta = reg(regs, rd_u16(&pc));
+    desc.q = reg(regs, rd_u16(&pc));
+    desc.k_new = reg(regs, rd_u16(&pc));
+    desc.v_new = reg(regs, rd_u16(&pc));
+    desc.kv_k = reg(regs, rd_u16(&pc));
+    desc.kv_v = reg(regs, rd_u16(&pc));
+    desc.block_table = reg(regs, rd_u16(&pc));
+    marmot_paged_attention_kv_scale_ext_t ext = {.struct_size = sizeof(ext),
+                                                 .struct_version = MARMOT_PAGED_ATTENTION_KV_SCALE_EXT_VERSION};
+    ext.kv_k_scale = reg(regs, rd_u16(&pc));
+    ext.kv_v_scale = reg(regs, rd_u16(&pc));
+    desc.out = reg(regs, rd_u16(&pc));
+    desc.token_count = rd_u32(&pc);
+    desc.layer_idx = rd_u32(&pc);
+    desc.num_q_heads = rd_u32(&pc);
+    desc.num_kv_heads = rd_u32(&pc);
+    desc.head_dim = rd_u32(&pc);
+    desc.block_size = rd_u32(&pc);
+    desc.scale = rd_f32(&pc);
+    if (ext.kv_k_scale != nullptr || ext.kv_v_scale != nullptr) {
+        desc.pnext = &ext;
+    }
+    return paged_attention(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
+}
+
 static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     0,               // END
     12, 12, 12, 12,  // MATMUL: 3 x u16 + u32 + u16
@@ -1986,6 +2220,7 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     12, 12,          // RMS_NORM, RMS_NORM_GEMMA: 4 x u16 + f32
     6, 6, 6,         // SWIGLU, GEGLU, ADD (BINARY): 3 x u16
     18,              // ROPE: 3 x u16 + 3 x u32
+    48,              // PAGED_ATTENTION: 10 x u16 + 6 x u32 + f32
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -2007,6 +2242,7 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_RMS_NORM,    MARMOT_BC_SCHEMA_RMS_NORM,
     MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,
     MARMOT_BC_SCHEMA_ROPE,
+    MARMOT_BC_SCHEMA_PAGED_ATTENTION,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -2026,6 +2262,7 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_rms_norm,    bc_exec_rms_norm_gemma,
     bc_exec_swiglu,      bc_exec_geglu,       bc_exec_add,
     bc_exec_rope,
+    bc_exec_paged_attention,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -2260,6 +2497,15 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
             return unsupported("HIP RoPE handles FLOAT32 and FLOAT16 tensors");
         }
         return selected(MARMOT_HIP_BC_OP_ROPE, launch_us, 0.0);
+    case MARMOT_OP_PAGED_ATTENTION: {
+        // paged_attention_scalar (cpu/kernels/paged_attention.def): activations and result of one float type, the
+        // cache type as the weight type; the FLOAT8_E4M3 cache stays with the CPU
+        const bool act_ok = pa_float_dtype(sig->input_dtype) && sig->output_dtype == sig->input_dtype;
+        if (!act_ok || !pa_float_dtype(sig->weight_dtype)) {
+            return unsupported("HIP paged attention handles FLOAT32, FLOAT16 and BFLOAT16 activations and caches");
+        }
+        return selected(MARMOT_HIP_BC_OP_PAGED_ATTENTION, 2.0 * launch_us, 0.0);
+    }
     case MARMOT_OP_TOPK:
         if (!in32 || !out32) {
             return unsupported("HIP TopK takes FLOAT32 values");
@@ -2465,6 +2711,9 @@ marmot_error_t hip_geglu_f32(const void *device_ctx, const marmot_tensor_t *a, c
 marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, const marmot_tensor_t *b,
                            marmot_tensor_t *out) {
     return binary_f32(device_ctx, HIP_BIN_ADD, a, b, out);
+}
+marmot_error_t hip_paged_attention_impl(const void *device_ctx, const marmot_paged_attention_desc_t *desc) {
+    return paged_attention(device_ctx, desc);
 }
 marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
                         marmot_tensor_t *out) {

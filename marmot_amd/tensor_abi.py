@@ -28,6 +28,7 @@ SUCCESS, INVALID_ARGUMENT, OUT_OF_MEMORY, DEVICE_NOT_AVAILABLE, BACKEND_INIT_FAI
 INVALID_OPERATION, UNSUPPORTED_DTYPE, DIMENSION_MISMATCH, NOT_IMPLEMENTED = -5, -6, -7, -8
 # marmot_dtype_t
 DTYPE_F32, DTYPE_F16, DTYPE_I32, DTYPE_I8, DTYPE_U8, DTYPE_I64 = 0, 1, 3, 5, 6, 11
+DTYPE_BF16, DTYPE_U32, DTYPE_F8_E4M3 = 2, 8, 14
 # marmot_quant_kind_t / marmot_quant_layout_t / marmot_memory_location_t
 KIND_GENERIC, KIND_Q4_0, KIND_Q8_0, KIND_Q4_K, KIND_Q5_K, KIND_Q6_K, KIND_Q8_K = 0, 1, 5, 9, 10, 11, 12
 KIND_Q4_1, KIND_Q5_0, KIND_Q5_1 = 2, 3, 4
@@ -41,10 +42,12 @@ OP_DEQUANTIZE, OP_MOE_EXPERTS, OP_MATMUL, OP_QUANTIZE, OP_LINEAR, OP_TOPK = 210,
 OP_QKV_PROJECTION, OP_QKV_SHARED_INPUT, OP_QKV_ROPE = 191, 771, 778
 OP_EMBEDDING = 853
 OP_ROPE = 843
+OP_PAGED_ATTENTION = 503
 OP_SWIGLU, OP_GEGLU, OP_RMS_NORM_GEMMA, OP_ADD, OP_RMS_NORM = 331, 410, 447, 876, 929
 # this backend's bytecode ops for them (include/marmot_hip_backend.h)
 BC_OP_RMS_NORM_F32, BC_OP_RMS_NORM_GEMMA_F32, BC_OP_SWIGLU_F32, BC_OP_GEGLU_F32, BC_OP_ADD_F32 = 48, 49, 50, 51, 52
 BC_OP_ROPE = 53
+BC_OP_PAGED_ATTENTION = 54
 PREFERENCE_DEFAULT, PREFERENCE_ENABLE, PREFERENCE_DISABLE = 0, 1, 2
 QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q4_1: 2, KIND_Q5_0: 3, KIND_Q5_1: 4, KIND_Q8_0: 5, KIND_Q2_K: 6, KIND_Q3_K: 7, KIND_Q4_K: 8,
@@ -57,7 +60,7 @@ EPILOGUE_ROPE = 8
 BC_END, BC_REG_INVALID, BC_INVALID_OFFSET = 0, 0xFFFF, 0xFFFFFFFF
 
 _NP_OF_DTYPE = {DTYPE_F32: np.float32, DTYPE_F16: np.float16, DTYPE_I32: np.int32, DTYPE_I8: np.int8,
-                DTYPE_U8: np.uint8, DTYPE_I64: np.int64}
+                DTYPE_U8: np.uint8, DTYPE_I64: np.int64, DTYPE_U32: np.uint32}
 _DTYPE_OF_NP = {np.dtype(v): k for k, v in _NP_OF_DTYPE.items()}
 
 
@@ -121,6 +124,29 @@ class RmsNormDesc(C.Structure):
     """marmot_rmsnorm_desc_t"""
     _fields_ = [("x", C.POINTER(Tensor)), ("residual", C.POINTER(Tensor)), ("weight", C.POINTER(Tensor)),
                 ("out", C.POINTER(Tensor)), ("eps", C.c_float)]
+
+
+class PagedAttentionKvScaleExt(C.Structure):
+    """marmot_paged_attention_kv_scale_ext_t"""
+    _fields_ = [("struct_size", C.c_uint32), ("struct_version", C.c_uint32), ("kv_k_scale", C.POINTER(Tensor)),
+                ("kv_v_scale", C.POINTER(Tensor))]
+
+
+class PagedAttentionDesc(C.Structure):
+    """marmot_paged_attention_desc_t"""
+    _fields_ = [("struct_size", C.c_uint32), ("struct_version", C.c_uint32), ("flags", C.c_uint64),
+                ("token_count", C.c_uint32), ("layer_idx", C.c_uint32), ("num_q_heads", C.c_uint32),
+                ("num_kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("block_size", C.c_uint32),
+                ("scale", C.c_float)] + [(n, C.POINTER(Tensor)) for n in
+                                         ("token_meta", "q", "k_new", "v_new", "kv_k", "kv_v", "block_table", "out")] + [
+                    ("pnext", C.c_void_p), ("reserved", C.c_uint64 * 4)]
+
+    @classmethod
+    def default(cls) -> "PagedAttentionDesc":
+        """marmot_paged_attention_desc_default (include/marmot/ops/paged_attention.h:59-83)"""
+        d = cls()
+        d.struct_size, d.struct_version, d.scale = C.sizeof(cls), 1, 1.0
+        return d
 
 
 class MoeDesc(C.Structure):
@@ -265,7 +291,7 @@ BACKEND_SYMBOLS = [
     "hip_matmul_qkv_q5_k", "hip_matmul_qkv_q6_k", "hip_embedding_gather", "hip_moe_experts_impl", "hip_topk_impl", "hip_quantize_block",
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
     "hip_rmsnorm_impl", "hip_rmsnorm_gemma_impl", "hip_swiglu_f32", "hip_geglu_f32", "hip_add_f32",
-    "hip_rope",
+    "hip_rope", "hip_paged_attention_impl",
 ]
 
 
@@ -306,6 +332,8 @@ def bind(lib: C.CDLL) -> C.CDLL:
         fn = getattr(lib, name)
         fn.restype = C.c_int
         fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]
+    lib.hip_paged_attention_impl.restype = C.c_int
+    lib.hip_paged_attention_impl.argtypes = [C.c_void_p, C.POINTER(PagedAttentionDesc)]
     lib.hip_rope.restype = C.c_int
     lib.hip_rope.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(RopeParams), C.POINTER(Tensor)]
     lib.marmot_hip_backend_last_error.restype = C.c_int
@@ -358,6 +386,29 @@ class HostTensor:
         return cls(np.zeros(shape, dtype=_NP_OF_DTYPE[dtype]), shape, dtype)
 
     @classmethod
+    def strided(cls, view: np.ndarray, dtype: Optional[int] = None) -> "HostTensor":
+        """A tensor over a numpy array or view as it lies in memory (any strides; the view keeps its base alive).
+        `dtype` overrides the type the element size suggests (bfloat16 bits travel in uint16 arrays)."""
+        obj = cls.__new__(cls)
+        obj.array = view
+        obj.t = Tensor()
+        obj.t.shape.ndim = view.ndim
+        last = 0
+        for i in range(view.ndim):
+            assert view.strides[i] % view.itemsize == 0 and view.strides[i] >= 0
+            obj.t.shape.shape[i] = view.shape[i]
+            obj.t.shape.strides[i] = view.strides[i] // view.itemsize
+            last += (view.shape[i] - 1) * view.strides[i] if view.shape[i] else 0
+        obj.extent_bytes = last + view.itemsize if view.size else 0
+        obj.t.dtype = _DTYPE_OF_NP[view.dtype] if dtype is None else dtype
+        obj.t.data = view.ctypes.data
+        obj.t.capacity_bytes = obj.extent_bytes
+        obj.t.owns_data = False
+        obj.t.quant_kind, obj.t.quant_layout = KIND_GENERIC, LAYOUT_GENERIC
+        obj.t.backend, obj.t.memory_location, obj.t.needs_sync = BACKEND_HIP, MEMORY_HOST, False
+        return obj
+
+    @classmethod
     def quantized(cls, blocks: np.ndarray, shape: Sequence[int], kind: int) -> "HostTensor":
         """blocks: uint8 GGUF block bytes; shape: logical element shape as marmot stores it ([rows, cols] for a
         weight, [cols, rows, experts] for an expert stack)."""
@@ -407,7 +458,8 @@ class HipContext:
 
     def to_host(self, t: HostTensor) -> np.ndarray:
         if t.t.needs_sync:
-            self._check(self.ops.memcpy_from_device(self.device_ctx, t.t.data, t.t.data, t.array.nbytes))
+            nbytes = getattr(t, "extent_bytes", t.array.nbytes)  # a strided view: its whole extent in memory
+            self._check(self.ops.memcpy_from_device(self.device_ctx, t.t.data, t.t.data, nbytes))
             t.t.needs_sync = False
         return t.array
 
@@ -585,6 +637,16 @@ class Program:
             off = self._const(bytes(params), 8)
         self.code += struct.pack("<HHHHIII", op_index, self.reg(x), self.reg(out), self.reg(positions), off, n_past,
                                  n_rot)
+
+    def paged_attention(self, op_index: int, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out, token_count: int,
+                        layer_idx: int, num_q_heads: int, num_kv_heads: int, head_dim: int, block_size: int,
+                        scale: float, kv_k_scale=None, kv_v_scale=None):
+        """bytecode_compile.c:553-597: ten tensor registers (the two scale tensors of the FP8 cache may be absent), six
+        u32 and the scale."""
+        self.code += struct.pack("<H10H6If", op_index, self.reg(token_meta), self.reg(q), self.reg(k_new),
+                                 self.reg(v_new), self.reg(kv_k), self.reg(kv_v), self.reg(block_table),
+                                 self.reg(kv_k_scale), self.reg(kv_v_scale), self.reg(out), token_count, layer_idx,
+                                 num_q_heads, num_kv_heads, head_dim, block_size, scale)
 
     def quantize(self, op_index: int, x, out):
         self.code += struct.pack("<HHIHII", op_index, self.reg(x), BC_INVALID_OFFSET, self.reg(out),

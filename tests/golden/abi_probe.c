@@ -11,6 +11,7 @@
 #include "marmot/graph/op_signature.h"
 #include "marmot/ops_types.h"
 #include "marmot/ops/matmul.h"
+#include "marmot/ops/paged_attention.h"
 #include "core/bytecode/bytecode.h"
 #include "core/bytecode/bytecode_compile.h"
 #include "core/dispatch/kernel_query.h"
@@ -64,6 +65,9 @@ int main(void) {
     VAL(MARMOT_OP_RMS_NORM); VAL(MARMOT_OP_RMS_NORM_GEMMA); VAL(MARMOT_OP_SWIGLU); VAL(MARMOT_OP_GEGLU); VAL(MARMOT_OP_ADD);
     VAL(MARMOT_BC_SCHEMA_RMS_NORM); VAL(MARMOT_BC_SCHEMA_BINARY);
     VAL(MARMOT_OP_ROPE); VAL(MARMOT_BC_SCHEMA_ROPE);
+    VAL(MARMOT_OP_PAGED_ATTENTION); VAL(MARMOT_BC_SCHEMA_PAGED_ATTENTION); VAL(MARMOT_DTYPE_BFLOAT16);
+    VAL(MARMOT_DTYPE_UINT32); VAL(MARMOT_DTYPE_FLOAT8_E4M3); VAL(MARMOT_PAGED_ATTENTION_DESC_VERSION);
+    VAL(MARMOT_PAGED_ATTENTION_KV_SCALE_EXT_VERSION);
 
     SZ(marmot_shape_t); OFF(marmot_shape_t, ndim); OFF(marmot_shape_t, shape); OFF(marmot_shape_t, strides);
     SZ(marmot_quant_params_t);
@@ -102,6 +106,20 @@ int main(void) {
     OFF(marmot_embedding_gather_desc_t, padding_id); OFF(marmot_embedding_gather_desc_t, bounds_check);
     OFF(marmot_embedding_gather_desc_t, prefer_gpu_private);
     OFF(marmot_embedding_gather_desc_t, allow_quant_decode_on_the_fly);
+    SZ(marmot_paged_attention_desc_t); OFF(marmot_paged_attention_desc_t, struct_size);
+    OFF(marmot_paged_attention_desc_t, struct_version); OFF(marmot_paged_attention_desc_t, flags);
+    OFF(marmot_paged_attention_desc_t, token_count); OFF(marmot_paged_attention_desc_t, layer_idx);
+    OFF(marmot_paged_attention_desc_t, num_q_heads); OFF(marmot_paged_attention_desc_t, num_kv_heads);
+    OFF(marmot_paged_attention_desc_t, head_dim); OFF(marmot_paged_attention_desc_t, block_size);
+    OFF(marmot_paged_attention_desc_t, scale); OFF(marmot_paged_attention_desc_t, token_meta);
+    OFF(marmot_paged_attention_desc_t, q); OFF(marmot_paged_attention_desc_t, k_new);
+    OFF(marmot_paged_attention_desc_t, v_new); OFF(marmot_paged_attention_desc_t, kv_k);
+    OFF(marmot_paged_attention_desc_t, kv_v); OFF(marmot_paged_attention_desc_t, block_table);
+    OFF(marmot_paged_attention_desc_t, out); OFF(marmot_paged_attention_desc_t, pnext);
+    OFF(marmot_paged_attention_desc_t, reserved);
+    SZ(marmot_paged_attention_kv_scale_ext_t); OFF(marmot_paged_attention_kv_scale_ext_t, struct_size);
+    OFF(marmot_paged_attention_kv_scale_ext_t, struct_version); OFF(marmot_paged_attention_kv_scale_ext_t, kv_k_scale);
+    OFF(marmot_paged_attention_kv_scale_ext_t, kv_v_scale);
     SZ(marmot_topk_desc_t); OFF(marmot_topk_desc_t, axis); OFF(marmot_topk_desc_t, k);
     SZ(marmot_rmsnorm_desc_t); OFF(marmot_rmsnorm_desc_t, residual); OFF(marmot_rmsnorm_desc_t, weight);
     OFF(marmot_rmsnorm_desc_t, out); OFF(marmot_rmsnorm_desc_t, eps);

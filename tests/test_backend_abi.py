@@ -66,6 +66,8 @@ def test_ctypes_structs_match_layout(golden_layout):
         "marmot_quant_block_t": ta.QuantBlock, "marmot_rope_params_t": ta.RopeParams,
         "marmot_matmul_qkv_desc_t": ta.QkvDesc, "marmot_matmul_qkv_separate_t": ta.QkvSeparate,
         "marmot_embedding_gather_desc_t": ta.EmbeddingGatherDesc,
+        "marmot_paged_attention_desc_t": ta.PagedAttentionDesc,
+        "marmot_paged_attention_kv_scale_ext_t": ta.PagedAttentionKvScaleExt,
     }
     checked = 0
     for cname, cls in pairs.items():
@@ -75,7 +77,7 @@ def test_ctypes_structs_match_layout(golden_layout):
             if m:
                 assert getattr(cls, m.group(1)).offset == off, key
                 checked += 1
-    assert checked >= 90
+    assert checked >= 114
     assert ta.OP_MATMUL == golden_layout["MARMOT_OP_MATMUL"]
     assert ta.OP_MOE_EXPERTS == golden_layout["MARMOT_OP_MOE_EXPERTS"]
     assert ta.OP_TOPK == golden_layout["MARMOT_OP_TOPK"]
@@ -282,11 +284,29 @@ def test_query_kernel_embedding_rules(lib):
     assert not _query(lib, sig(out=ta.DTYPE_I32)).supported
 
 
+def test_query_kernel_paged_attention_rules(lib):
+    """cpu/kernels/paged_attention.def:6-22 without the FP8 cache: activations and result of one float type, the
+    cache type as the weight type."""
+    def sig(act=ta.DTYPE_F32, kv=ta.DTYPE_F16, out=None):
+        s = ta.OpSignature()
+        s.op_id, s.input_dtype, s.weight_dtype = ta.OP_PAGED_ATTENTION, act, kv
+        s.output_dtype = act if out is None else out
+        s.accum_dtype = ta.DTYPE_F32
+        return s
+    for act in (ta.DTYPE_F32, ta.DTYPE_F16, ta.DTYPE_BF16):
+        for kv in (ta.DTYPE_F32, ta.DTYPE_F16, ta.DTYPE_BF16):
+            sel = _query(lib, sig(act, kv))
+            assert sel.supported and sel.op_index == ta.BC_OP_PAGED_ATTENTION
+    assert not _query(lib, sig(kv=ta.DTYPE_F8_E4M3)).supported
+    assert not _query(lib, sig(act=ta.DTYPE_I32)).supported
+    assert not _query(lib, sig(out=ta.DTYPE_F16)).supported
+
+
 def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 54
+    assert t.op_count == 55
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -321,6 +341,13 @@ def test_bytecode_tables(lib, golden_layout):
     # the rotary embedding: input, output and positions registers, parameter offset, n_past, n_rot
     assert schema[53] == golden_layout["MARMOT_BC_SCHEMA_ROPE"] and sizes[53] == struct.calcsize("<3H3I") == 18
     assert ta.BC_OP_ROPE == 53 and ta.OP_ROPE == golden_layout["MARMOT_OP_ROPE"]
+    # paged attention: ten tensor registers, six u32 and the scale
+    assert schema[54] == golden_layout["MARMOT_BC_SCHEMA_PAGED_ATTENTION"]
+    assert sizes[54] == struct.calcsize("<10H6If") == 48
+    assert ta.BC_OP_PAGED_ATTENTION == 54 and ta.OP_PAGED_ATTENTION == golden_layout["MARMOT_OP_PAGED_ATTENTION"]
+    assert (ta.DTYPE_BF16, ta.DTYPE_U32, ta.DTYPE_F8_E4M3) == (
+        golden_layout["MARMOT_DTYPE_BFLOAT16"], golden_layout["MARMOT_DTYPE_UINT32"],
+        golden_layout["MARMOT_DTYPE_FLOAT8_E4M3"])
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 
@@ -340,6 +367,7 @@ def test_exec_entries_reject_null_arguments(lib):
     assert lib.hip_matmul_qkv_q4_k(None, None) == ta.INVALID_ARGUMENT
     assert lib.hip_topk_impl(None, None) == ta.INVALID_ARGUMENT
     assert lib.hip_embedding_gather(None, None) == ta.INVALID_ARGUMENT
+    assert lib.hip_paged_attention_impl(None, None) == ta.INVALID_ARGUMENT
 
 
 def test_program_encoding_matches_reference_immediates():
@@ -392,7 +420,7 @@ def test_kernel_def_files_name_exported_impls(lib):
     assert set(families) == {"matmul_quantized_hip", "topk_hip",
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
                              "embedding_quantized_hip", "rms_norm_hip", "rms_norm_gemma_hip", "glu_hip",
-                             "add_hip", "rope_hip"} | qkv
+                             "add_hip", "rope_hip", "paged_attention_hip"} | qkv
     for name in qkv:
         f = families[name]
         assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name

@@ -796,3 +796,150 @@ def test_program_norm_feeds_linears_without_quantization_launches(ctx, oracle):
     assert_matmul_parity(ctx.to_host(g), oracle.matmul(KIND_Q4_K, gate, h.array, F, threads=8), what="after host write")
     for t in (xt, wn, gw, uw, dw, h, g, u, a, d, y):
         ctx.host_freed(t)
+
+
+# ---------------------------------------------------------------- paged attention
+def _attention_tensors(case):
+    """Host tensors of a paged-attention case: q / k_new / v_new as views of one buffer (a fused projection's output),
+    bfloat16 as uint16 bits with the type said explicitly."""
+    from tests.attention_cases import to_storage
+
+    act_dt = {"f32": None, "f16": None, "bf16": ta.DTYPE_BF16}[case["act"]]
+    kv_dt = {"f32": None, "f16": None, "bf16": ta.DTYPE_BF16}[case["kv"]]
+    T, hq, d = case["q"].shape
+    hkv = case["k_new"].shape[1]
+    fused = np.zeros((T, hq + 2 * hkv, d), dtype=case["q"].dtype)
+    fused[:, :hq], fused[:, hq:hq + hkv], fused[:, hq + hkv:] = case["q"], case["k_new"], case["v_new"]
+    t = {
+        "fused": fused,
+        "token_meta": ta.HostTensor.dense(case["token_meta"]),
+        "q": ta.HostTensor.strided(fused[:, :hq], act_dt),
+        "k_new": ta.HostTensor.strided(fused[:, hq:hq + hkv], act_dt),
+        "v_new": ta.HostTensor.strided(fused[:, hq + hkv:], act_dt),
+        "kv_k": ta.HostTensor.strided(case["kv_k"].copy(), kv_dt),
+        "kv_v": ta.HostTensor.strided(case["kv_v"].copy(), kv_dt),
+        "block_table": ta.HostTensor.dense(case["block_table"]),
+        "out": ta.HostTensor.strided(np.zeros((T, hq, d), dtype=case["q"].dtype), act_dt),
+    }
+    desc = ta.PagedAttentionDesc.default()
+    desc.token_count, desc.layer_idx, desc.scale = T, case["layer_idx"], case["scale"]
+    desc.num_q_heads, desc.num_kv_heads, desc.head_dim, desc.block_size = hq, hkv, d, case["block_size"]
+    for name in ("token_meta", "q", "k_new", "v_new", "kv_k", "kv_v", "block_table", "out"):
+        setattr(desc, name, t[name].ptr)
+    return t, desc
+
+
+@pytest.mark.parametrize("act,kv", [("f32", "f16"), ("f16", "f16"), ("bf16", "bf16"), ("f32", "f32")])
+def test_impl_and_program_paged_attention(ctx, oracle, act, kv):
+    """hip_paged_attention_impl, its kernel query and its bytecode op against the oracle: caches bit for bit, output
+    within fp32 summation noise and one rounding of the output type; a second call (decode step) on the caches the
+    first one left on the device."""
+    from tests.attention_cases import TOLERANCE, make_case, to_f32
+
+    case = make_case(70, [(45, 1), (0, 12), (90, 3)], num_q_heads=8, num_kv_heads=2, head_dim=128, block_size=16,
+                     act=act, kv=kv)
+    ref_k, ref_v = case["kv_k"].copy(), case["kv_v"].copy()
+    st, ref = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], ref_k, ref_v,
+                                     case["block_table"], case["layer_idx"], case["scale"], act_bf16=act == "bf16",
+                                     kv_bf16=kv == "bf16")
+    assert st == 0
+    tol = TOLERANCE[act] * np.abs(to_f32(ref_v, kv)).max()
+
+    def close(got):
+        return np.max(np.abs(to_f32(got, act).astype(np.float64) - to_f32(ref, act).astype(np.float64))) <= tol
+
+    t, desc = _attention_tensors(case)
+    assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
+    assert close(ctx.to_host(t["out"]))
+    assert np.array_equal(ctx.to_host(t["kv_k"]).view(np.uint8), ref_k.view(np.uint8))
+    assert np.array_equal(ctx.to_host(t["kv_v"]).view(np.uint8), ref_v.view(np.uint8))
+    # the same call as a bytecode op on fresh tensors
+    sig = ta.OpSignature()
+    sig.op_id, sig.accum_dtype = ta.OP_PAGED_ATTENTION, ta.DTYPE_F32
+    sig.input_dtype = sig.output_dtype = t["q"].t.dtype
+    sig.weight_dtype = t["kv_k"].t.dtype
+    sel = ctx.query(sig)
+    assert sel.supported and sel.op_index == ta.BC_OP_PAGED_ATTENTION
+    t2, d2 = _attention_tensors(case)
+    p = ta.Program()
+    p.paged_attention(sel.op_index, t2["token_meta"], t2["q"], t2["k_new"], t2["v_new"], t2["kv_k"], t2["kv_v"],
+                      t2["block_table"], t2["out"], d2.token_count, d2.layer_idx, d2.num_q_heads, d2.num_kv_heads,
+                      d2.head_dim, d2.block_size, d2.scale)
+    assert ctx.execute(p) == ta.SUCCESS, ctx.last_error()
+    assert np.array_equal(ctx.to_host(t2["out"]).view(np.uint8), ctx.to_host(t["out"]).view(np.uint8))
+    assert np.array_equal(ctx.to_host(t2["kv_k"]).view(np.uint8), ref_k.view(np.uint8))
+    # a decode step on top: one more token per sequence, the caches stay on the device between the calls
+    step = make_case(71, [(46, 1), (12, 1), (93, 1)], num_q_heads=8, num_kv_heads=2, head_dim=128, block_size=16,
+                     act=act, kv=kv)
+    # same block table and cache as after the first call; only the new tokens' metadata and rows differ
+    bs = case["block_size"]
+    slots = sorted(set(int(s) for s in case["token_meta"][:, 0]))
+    last = {s: int(case["token_meta"][case["token_meta"][:, 0] == s, 1].max()) for s in slots}
+    meta = np.array([[s, last[s] + 1, int(case["block_table"][s, (last[s] + 1) // bs]) * bs + (last[s] + 1) % bs, 0]
+                     for s in slots], dtype=np.uint32)
+    nxt = dict(case, token_meta=meta, q=step["q"][:3], k_new=step["k_new"][:3], v_new=step["v_new"][:3], kv_k=ref_k,
+               kv_v=ref_v)
+    st, ref2 = oracle.paged_attention(meta, nxt["q"], nxt["k_new"], nxt["v_new"], ref_k, ref_v, case["block_table"],
+                                      case["layer_idx"], case["scale"], act_bf16=act == "bf16", kv_bf16=kv == "bf16")
+    assert st == 0
+    t3, d3 = _attention_tensors(nxt)
+    d3.kv_k, d3.kv_v = t["kv_k"].ptr, t["kv_v"].ptr  # the tensors the first call updated
+    assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(d3)) == ta.SUCCESS, ctx.last_error()
+    got2 = ctx.to_host(t3["out"])
+    assert np.max(np.abs(to_f32(got2, act).astype(np.float64) - to_f32(ref2, act).astype(np.float64))) <= tol
+    assert np.array_equal(ctx.to_host(t["kv_k"]).view(np.uint8), ref_k.view(np.uint8))
+    for group in (t, t2, t3):
+        for name, x in group.items():
+            if name != "fused":
+                ctx.host_freed(x)
+
+
+def test_impl_paged_attention_errors(ctx):
+    """The checks of cpu_paged_attention_impl in its order (paged_attention_ref.c:573-823), then what this backend
+    leaves to the fallback."""
+    from tests.attention_cases import make_case
+
+    case = make_case(72, [(5, 2)], num_q_heads=4, num_kv_heads=2, head_dim=64, block_size=8)
+    t, desc = _attention_tensors(case)
+
+    def call(**kw):
+        d = ta.PagedAttentionDesc.default()
+        C.memmove(C.byref(d), C.byref(desc), C.sizeof(d))
+        for k, v in kw.items():
+            setattr(d, k, v.ptr if isinstance(v, ta.HostTensor) else v)
+        return ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(d))
+
+    assert call() == ta.SUCCESS
+    assert call(struct_version=2) == ta.INVALID_ARGUMENT and "descriptor invalid" in ctx.last_error()[1]
+    assert call(token_count=0) == ta.SUCCESS
+    assert call(block_size=6) == ta.INVALID_ARGUMENT and "power of two" in ctx.last_error()[1]
+    assert call(num_kv_heads=3) == ta.INVALID_ARGUMENT
+    f32_meta = ta.HostTensor.dense(np.zeros((2, 4), np.float32))
+    assert call(token_meta=f32_meta) == ta.UNSUPPORTED_DTYPE and "uint32 metadata" in ctx.last_error()[1]
+    ints = ta.HostTensor.dense(np.zeros((2, 4, 64), np.int32))
+    assert call(q=ints) == ta.UNSUPPORTED_DTYPE
+    half_out = ta.HostTensor.dense(np.zeros((2, 4, 64), np.float16))
+    assert call(out=half_out) == ta.UNSUPPORTED_DTYPE and "matching" in ctx.last_error()[1]
+    assert call(token_count=1) == ta.DIMENSION_MISMATCH and "token_meta shape" in ctx.last_error()[1]
+    assert call(num_q_heads=8, num_kv_heads=2) == ta.DIMENSION_MISMATCH and "num_q_heads" in ctx.last_error()[1]
+    assert call(head_dim=32) == ta.DIMENSION_MISMATCH and "head_dim" in ctx.last_error()[1]
+    assert call(layer_idx=2) == ta.DIMENSION_MISMATCH and "layer_idx" in ctx.last_error()[1]
+    assert call(block_size=16) == ta.DIMENSION_MISMATCH and "block_size" in ctx.last_error()[1]
+    half_cache = ta.HostTensor.dense(case["kv_v"].astype(np.float16))
+    assert call(kv_v=half_cache) == ta.DIMENSION_MISMATCH and "kv dtype" in ctx.last_error()[1]
+    bad = case["token_meta"].copy()
+    bad[1, 0] = case["block_table"].shape[0]
+    assert call(token_meta=ta.HostTensor.dense(bad)) == ta.DIMENSION_MISMATCH and "seq_slot" in ctx.last_error()[1]
+    bad[1, 0], bad[1, 2] = 0, case["kv_k"].shape[0] * 8
+    assert call(token_meta=ta.HostTensor.dense(bad)) == ta.DIMENSION_MISMATCH and "kv_slot" in ctx.last_error()[1]
+    fp8 = [ta.HostTensor.strided(np.zeros(case["kv_k"].shape, np.uint8), ta.DTYPE_F8_E4M3) for _ in range(2)]
+    assert call(kv_k=fp8[0], kv_v=fp8[1]) == ta.NOT_IMPLEMENTED
+    ext = ta.PagedAttentionKvScaleExt(C.sizeof(ta.PagedAttentionKvScaleExt), 1, t["kv_k"].ptr, t["kv_v"].ptr)
+    assert call(pnext=C.addressof(ext)) == ta.INVALID_ARGUMENT and "require FP8" in ctx.last_error()[1]
+    wide = make_case(73, [(2, 1)], num_q_heads=1, num_kv_heads=1, head_dim=320, block_size=4)
+    tw, dw = _attention_tensors(wide)
+    assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(dw)) == ta.NOT_IMPLEMENTED
+    for group in (t, tw):
+        for name, x in group.items():
+            if name != "fused":
+                ctx.host_freed(x)

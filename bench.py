@@ -229,8 +229,8 @@ def prefill_int8(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
-    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "ATTN", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
+    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, ATTN, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -318,6 +318,8 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5
         sweep_qkv(hip, rng, emit, steps, warmup)
     if "OPS" in only:
         sweep_ops(hip, rng, emit, steps, warmup)
+    if "ATTN" in only:
+        sweep_attention(hip, rng, emit, steps)
     if "LOGITS" in only:
         # the vocabulary-sized matvec at the end of a decode step (Llama-3 vocabulary, 128256 rows of 4096)
         for kind in (capi.KIND_Q6_K, capi.KIND_Q4_K):
@@ -492,6 +494,61 @@ def sweep_layer_stack(hip, rng, emit, steps: int, N: int = 16, config: str = "C4
     for *_, d_w, d_x, d_out in layers:
         for b in (d_w, d_x, d_out):
             b.free()
+
+
+def sweep_attention(hip, rng, emit, steps: int):
+    """Paged attention of a Llama-3-8B layer (32 query heads over 8 key / value heads of 128, block size 16, fp16
+    cache, fp32 activations): a decode step of 16 sequences with 4096 positions of history each (one new token per
+    sequence), and a prompt of 512 tokens of one sequence. The figure is the cache bytes every (token, kv head) must
+    read, once per kv head, over the time of the whole op (cache write + attention)."""
+    import ctypes as C
+
+    hq, hkv, d, bs = 32, 8, 128, 16
+
+    def run(name, seqs):
+        need = [-(-(h + n) // bs) for h, n in seqs]
+        blocks = sum(need)
+        table = np.full((len(seqs), max(need)), 0xFFFFFFFF, dtype=np.uint32)
+        meta, nxt = [], 0
+        for s, (h, n) in enumerate(seqs):
+            table[s, :need[s]] = np.arange(nxt, nxt + need[s], dtype=np.uint32)
+            nxt += need[s]
+            meta += [(s, p, int(table[s, p // bs]) * bs + p % bs, 0) for p in range(h, h + n)]
+        meta = np.array(meta, dtype=np.uint32)
+        T = len(meta)
+        arrays = {
+            "token_meta": meta, "block_table": table,
+            "q": rng.standard_normal((T, hq, d), dtype=np.float32),
+            "k_new": rng.standard_normal((T, hkv, d), dtype=np.float32),
+            "v_new": rng.standard_normal((T, hkv, d), dtype=np.float32),
+            "kv_k": rng.standard_normal((blocks, 1, hkv, bs, d), dtype=np.float32).astype(np.float16),
+            "kv_v": rng.standard_normal((blocks, 1, hkv, bs, d), dtype=np.float32).astype(np.float16),
+            "out": np.zeros((T, hq, d), dtype=np.float32),
+        }
+        dev = {k: hip.to_device(v) for k, v in arrays.items()}
+        ptr_of = {id(v): dev[k].ptr for k, v in arrays.items()}
+        a = arrays
+        p = hip.paged_attention_args(lambda x: ptr_of[id(x)], a["token_meta"], a["q"], a["k_new"], a["v_new"], a["kv_k"],
+                                     a["kv_v"], a["block_table"], a["out"], 0, float(1.0 / np.sqrt(d)))
+
+        def step(i):
+            rc = hip.lib.marmot_hip_paged_attention(hip.dev, C.byref(p), 0)
+            if rc != 0:
+                raise RuntimeError(f"marmot_hip_paged_attention -> {rc}")
+
+        ms = time_steps_graph(hip, step, max(20, steps // 20), 5, chunk=20)
+        read = sum(int(pos) + 1 for _, pos, _, _ in meta) * hkv * d * 2 * 2  # K and V rows of fp16, once per kv head
+        total = read + T * (hq * 2 + hkv * 2) * d * 4 + T * hkv * d * 2 * 2
+        flops = 4.0 * sum(int(pos) + 1 for _, pos, _, _ in meta) * hq * d
+        emit({"config": "ATTN", "workload": name, "us": round(ms * 1e3, 2), "GB/s": round(total / ms / 1e6, 1),
+              "frac_of_hbm_peak": round(total / ms / 1e6 / HBM_PEAK_GBPS, 4), "TFLOP/s": round(flops / ms / 1e9, 2),
+              "tokens_per_s": round(T / ms * 1e3), "algorithmic_bytes": total})
+        for b in dev.values():
+            b.free()
+
+    run("paged attention, decode: 16 sequences x 4096 positions, 32/8 heads of 128, fp16 cache", [(4095, 1)] * 16)
+    run("paged attention, decode: 16 sequences x 512 positions", [(511, 1)] * 16)
+    run("paged attention, prompt: 512 tokens of one sequence", [(0, 512)])
 
 
 def sweep_moe(hip, rng, emit, steps: int):

@@ -311,6 +311,37 @@ static marmot_error_t acquire_write_rows(hip_backend_t *b, void *host, size_t sp
     return acquire_write(b, host, span, d_out);
 }
 
+// Several tensors of one call. Covering a host range that overlaps existing mirrors replaces them by one mirror over
+// the union (views of one buffer: gate / up halves, q / k / v slices), which frees their device memory: addresses
+// taken earlier in the same call would dangle. So every range is covered first, and the addresses are taken in a
+// second round, when every range lies inside a mirror and nothing is replaced any more.
+typedef enum { HIP_ACQ_READ, HIP_ACQ_WRITE, HIP_ACQ_UPDATE } hip_acq_mode_t;
+typedef struct {
+    void *host;
+    size_t bytes;
+    hip_acq_mode_t mode;  // UPDATE: read and written, or written with gaps whose bytes must survive
+    void *dev;
+} hip_acq_t;
+
+static marmot_error_t acquire_set(hip_backend_t *b, hip_acq_t *v, size_t n) {
+    for (int round = 0; round < 2; ++round) {
+        for (size_t i = 0; i < n; ++i) {
+            marmot_error_t st;
+            if (v[i].mode == HIP_ACQ_READ) {
+                const void *d = nullptr;
+                st = acquire_read(b, v[i].host, v[i].bytes, &d);
+                v[i].dev = (void *)d;
+            } else {
+                st = acquire_write_rows(b, v[i].host, v[i].bytes, v[i].mode == HIP_ACQ_UPDATE, &v[i].dev);
+            }
+            if (st != MARMOT_SUCCESS) {
+                return st;
+            }
+        }
+    }
+    return MARMOT_SUCCESS;
+}
+
 // ------------------------------------------------------------------ tensor helpers
 static size_t dtype_size(marmot_dtype_t t) {
     switch (t) {
@@ -1475,15 +1506,14 @@ static marmot_error_t binary_f32(const void *device_ctx, hip_binary_op_t op, con
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Binary operation: tensor without data");
     }
     pthread_mutex_lock(&b->mu);
-    const void *d_a = nullptr, *d_c = nullptr;
-    void *d_y = nullptr;
-    marmot_error_t st = acquire_read(b, a->data, strided_span_bytes(a), &d_a);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, c->data, strided_span_bytes(c), &d_c);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write_rows(b, out->data, strided_span_bytes(out), !dense_contiguous(out), &d_y);
-    }
+    hip_acq_t acq[3] = {
+        {a->data, strided_span_bytes(a), HIP_ACQ_READ, nullptr},
+        {c->data, strided_span_bytes(c), HIP_ACQ_READ, nullptr},
+        {out->data, strided_span_bytes(out), dense_contiguous(out) ? HIP_ACQ_WRITE : HIP_ACQ_UPDATE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 3);
+    const void *d_a = acq[0].dev, *d_c = acq[1].dev;
+    void *d_y = acq[2].dev;
     if (st == MARMOT_SUCCESS) {
         int rc;
         if (op == HIP_BIN_ADD) {
@@ -1604,16 +1634,14 @@ static marmot_error_t rope(const void *device_ctx, const marmot_tensor_t *x, con
     const void *d_x = nullptr, *d_pos = nullptr, *d_freqs = nullptr;
     void *d_y = nullptr;
     if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, x->data, x_span, &d_x);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, positions->data, dense_bytes(positions), &d_pos);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, e->freqs, dim / 2 * sizeof(float), &d_freqs);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write_rows(b, out->data, out_span, out_stride != dim, &d_y);
+        hip_acq_t acq[4] = {
+            {x->data, x_span, HIP_ACQ_READ, nullptr},
+            {positions->data, dense_bytes(positions), HIP_ACQ_READ, nullptr},
+            {e->freqs, dim / 2 * sizeof(float), HIP_ACQ_READ, nullptr},
+            {out->data, out_span, out_stride != dim ? HIP_ACQ_UPDATE : HIP_ACQ_WRITE, nullptr},
+        };
+        st = acquire_set(b, acq, 4);
+        d_x = acq[0].dev, d_pos = acq[1].dev, d_freqs = acq[2].dev, d_y = acq[3].dev;
     }
     if (st == MARMOT_SUCCESS) {
         const marmot_hip_rope_t r = {
@@ -1798,31 +1826,20 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
         a.kv_stride[i] = kv_k->shape.strides[i];
     }
     pthread_mutex_lock(&b->mu);
-    const void *d_meta = nullptr, *d_q = nullptr, *d_k = nullptr, *d_v = nullptr, *d_table = nullptr;
-    void *d_kv_k = nullptr, *d_kv_v = nullptr, *d_out = nullptr;
-    marmot_error_t st = acquire_read(b, meta->data, strided_extent_bytes(meta), &d_meta);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, table->data, strided_extent_bytes(table), &d_table);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, q->data, strided_extent_bytes(q), &d_q);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, k_new->data, strided_extent_bytes(k_new), &d_k);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, v_new->data, strided_extent_bytes(v_new), &d_v);
-    }
     // the caches are read and written; the output may be a view with gaps: the host's bytes go up first
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write_rows(b, kv_k->data, strided_extent_bytes(kv_k), true, &d_kv_k);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write_rows(b, kv_v->data, strided_extent_bytes(kv_v), true, &d_kv_v);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write_rows(b, out->data, strided_extent_bytes(out), true, &d_out);
-    }
+    hip_acq_t acq[8] = {
+        {meta->data, strided_extent_bytes(meta), HIP_ACQ_READ, nullptr},
+        {table->data, strided_extent_bytes(table), HIP_ACQ_READ, nullptr},
+        {q->data, strided_extent_bytes(q), HIP_ACQ_READ, nullptr},
+        {k_new->data, strided_extent_bytes(k_new), HIP_ACQ_READ, nullptr},
+        {v_new->data, strided_extent_bytes(v_new), HIP_ACQ_READ, nullptr},
+        {kv_k->data, strided_extent_bytes(kv_k), HIP_ACQ_UPDATE, nullptr},
+        {kv_v->data, strided_extent_bytes(kv_v), HIP_ACQ_UPDATE, nullptr},
+        {out->data, strided_extent_bytes(out), HIP_ACQ_UPDATE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 8);
+    const void *d_meta = acq[0].dev, *d_table = acq[1].dev, *d_q = acq[2].dev, *d_k = acq[3].dev, *d_v = acq[4].dev;
+    void *d_kv_k = acq[5].dev, *d_kv_v = acq[6].dev, *d_out = acq[7].dev;
     if (st == MARMOT_SUCCESS) {
         a.d_token_meta = (const uint32_t *)d_meta, a.d_block_table = (const uint32_t *)d_table;
         a.d_q = d_q, a.d_k_new = d_k, a.d_v_new = d_v, a.d_kv_k = d_kv_k, a.d_kv_v = d_kv_v, a.d_out = d_out;

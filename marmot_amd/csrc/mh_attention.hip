@@ -3,11 +3,11 @@
 // into the paged cache at the token's kv_slot, then every (token, query head) attends over positions 0 .. pos of its
 // sequence through the block table.
 //
-// Attention kernel: one workgroup of 256 threads per (token, query head), 16 groups of 16 lanes. A group walks the
-// positions g, g + 16, g + 32, ...: its 16 lanes split the head dimension (a lane holds EPL consecutive values of the
+// Attention kernel: one workgroup of 16 groups of 16 lanes per (token, up to four query heads of one key / value
+// head). A group walks the positions g, g + 16, g + 32, ...: its 16 lanes split the head dimension (a lane holds EPL consecutive values of the
 // query, of the running output and of each key / value row, so a row is read as one contiguous run by the group), the
 // dot product is reduced inside the group with data-parallel-primitive moves, and the group keeps its own running
-// maximum, sum and output (online softmax). The 16 groups meet in LDS at the end. All arithmetic is fp32 like the
+// maximum, sum and output (online softmax). The groups meet in LDS at the end. All arithmetic is fp32 like the
 // reference's; only the order of the sums differs (per group instead of per block of positions). Rows are read with
 // 16-byte loads when the head dimension is exactly 16 x EPL values with unit stride, element by element otherwise.
 // A token whose sequence slot or cache block is out of range is skipped (the host rejects such calls when it may read
@@ -39,6 +39,8 @@ struct PaParams {
     uint32_t shift, mask, group;
     int q_vec, kv_vec;  // 16-byte loads of the query / of the cache rows
     int *flag;          // metadata check: 1 + index of an offending token (maximum)
+    uint32_t splits;    // workgroups along the history of one (token, heads) pair
+    float *partial;     // splits > 1: [token][query head][split][2 + head_dim]: maximum, sum, unnormalized output
 };
 
 // marmot_f32_to_bf16_ref / marmot_bf16_to_f32_ref (src/utils/dtype_ref.c:86-104): round to nearest even on the bits
@@ -143,55 +145,74 @@ __global__ __launch_bounds__(128) void k_pa_write(const PaParams p) {
 }
 
 // ---- attention (cpu_paged_attention_attention_range, :398-569)
-template <int EPL>
-__global__ __launch_bounds__(256) void k_pa_attend(const PaParams p) {
+// One workgroup of 16 groups of 16 lanes per (token, QH query heads that share a key / value head): every key and
+// value row is fetched, converted and located once for the QH heads. A group takes two positions per step and
+// requests both before it works on either.
+constexpr int PA_GROUPS = 16;
+
+template <int EPL, int QH>
+__global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) {
     warm_kernel_arguments<sizeof(PaParams), sizeof(PaParams)>();
-    __shared__ float s_acc[16][16 * EPL];
-    __shared__ float s_m[16], s_l[16];
-    const uint32_t t = blockIdx.x, qh = blockIdx.y;
+    __shared__ float s_acc[PA_GROUPS][QH][16 * EPL];
+    __shared__ float s_m[PA_GROUPS][QH], s_l[PA_GROUPS][QH];
+    const uint32_t t = blockIdx.x;
+    const uint32_t qh0 = blockIdx.y * QH;  // first query head of this workgroup; QH divides the heads per kv head
     const int tid = threadIdx.x, g = tid >> 4, l = tid & 15;
     const uint32_t seq = p.meta[t * p.meta_stride[0]];
     const uint32_t pos = p.meta[t * p.meta_stride[0] + p.meta_stride[1]];
     const uint32_t kv_len = seq < p.max_seqs ? pos + 1u : 0u;
-    const uint32_t kvh = qh / p.group;
+    const uint32_t kvh = qh0 / p.group;
     const uint32_t d0 = (uint32_t)l * EPL;  // this lane's first value of the head dimension
 
-    float qv[EPL];
-    const size_t q_base = (size_t)t * p.q_stride[0] + (size_t)qh * p.q_stride[1];
-    if (p.q_vec) {
-        pa_load_run<EPL>(p.q, p.act_dtype, q_base + d0, qv);
-    } else {
+    float qv[QH][EPL];
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            qv[e] = d0 + e < p.head_dim ? pa_load(p.q, p.act_dtype, q_base + (size_t)(d0 + e) * p.q_stride[2]) : 0.0f;
+    for (int h = 0; h < QH; ++h) {
+        const size_t q_base = (size_t)t * p.q_stride[0] + (size_t)(qh0 + h) * p.q_stride[1];
+        if (p.q_vec) {
+            pa_load_run<EPL>(p.q, p.act_dtype, q_base + d0, qv[h]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                qv[h][e] = d0 + e < p.head_dim ? pa_load(p.q, p.act_dtype, q_base + (size_t)(d0 + e) * p.q_stride[2]) : 0.0f;
+            }
         }
-    }
-    if (p.scale != 1.0f) {
+        if (p.scale != 1.0f) {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            qv[e] *= p.scale;
+            for (int e = 0; e < EPL; ++e) {
+                qv[h][e] *= p.scale;
+            }
         }
     }
 
-    float m = -INFINITY, lsum = 0.0f;
-    float acc[EPL];
+    float m[QH], lsum[QH], acc[QH][EPL];
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-        acc[e] = 0.0f;
+    for (int h = 0; h < QH; ++h) {
+        m[h] = -INFINITY;
+        lsum[h] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            acc[h][e] = 0.0f;
+        }
     }
     const size_t head_base = (size_t)p.layer_idx * p.kv_stride[1] + (size_t)kvh * p.kv_stride[2];
     const uint32_t *table_row = p.table + (size_t)seq * p.table_stride[0];
-    for (uint32_t pp = (uint32_t)g; pp < kv_len; pp += 16u) {
+    // the cache row of position pp, or false when the position has no block (beyond the table, or a hole)
+    auto locate = [&](uint32_t pp, size_t &base) -> bool {
+        if (pp >= kv_len) {
+            return false;
+        }
         const uint32_t logical = pp >> p.shift;
         if (logical >= p.max_blocks) {
-            break;
+            return false;
         }
         const uint32_t tb = table_row[(size_t)logical * p.table_stride[1]];
         if (tb == PA_NO_BLOCK || tb >= p.kv_blocks) {
-            continue;
+            return false;
         }
-        const size_t base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(pp & p.mask) * p.kv_stride[3];
-        float kr[EPL], vr[EPL];
+        base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(pp & p.mask) * p.kv_stride[3];
+        return true;
+    };
+    auto fetch = [&](size_t base, float (&kr)[EPL], float (&vr)[EPL]) {
         if (p.kv_vec) {
             pa_load_run<EPL>(p.kv_k, p.kv_dtype, base + d0, kr);
             pa_load_run<EPL>(p.kv_v, p.kv_dtype, base + d0, vr);
@@ -204,59 +225,131 @@ __global__ __launch_bounds__(256) void k_pa_attend(const PaParams p) {
                 vr[e] = in ? pa_load(p.kv_v, p.kv_dtype, i) : 0.0f;
             }
         }
-        float dot = 0.0f;
+    };
+    auto absorb = [&](const float (&kr)[EPL], const float (&vr)[EPL]) {
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            dot = __builtin_fmaf(qv[e], kr[e], dot);
-        }
-        dot = row16_sum(dot);
-        if (dot > m) {  // the same decision in all 16 lanes of the group
-            const float corr = m == -INFINITY ? 0.0f : expf(m - dot);
-            lsum *= corr;
+        for (int h = 0; h < QH; ++h) {
+            float dot = 0.0f;
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
-                acc[e] *= corr;
+                dot = __builtin_fmaf(qv[h][e], kr[e], dot);
             }
-            m = dot;
-        }
-        const float w = expf(dot - m);
-        lsum += w;
+            dot = row16_sum(dot);
+            if (dot > m[h]) {  // the same decision in all 16 lanes of the group
+                const float corr = m[h] == -INFINITY ? 0.0f : expf(m[h] - dot);
+                lsum[h] *= corr;
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            acc[e] = __builtin_fmaf(w, vr[e], acc[e]);
+                for (int e = 0; e < EPL; ++e) {
+                    acc[h][e] *= corr;
+                }
+                m[h] = dot;
+            }
+            const float w = expf(dot - m[h]);
+            lsum[h] += w;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                acc[h][e] = __builtin_fmaf(w, vr[e], acc[h][e]);
+            }
+        }
+    };
+    // this workgroup's share of the history (the whole of it without a split)
+    const uint32_t chunk = (kv_len + p.splits - 1u) / p.splits;
+    const uint32_t first = blockIdx.z * chunk;
+    const uint32_t stop = first + chunk < kv_len ? first + chunk : kv_len;
+    for (uint32_t pp = first + (uint32_t)g; pp < stop; pp += 2u * PA_GROUPS) {
+        size_t base0 = 0, base1 = 0;
+        const bool have0 = locate(pp, base0), have1 = pp + PA_GROUPS < stop && locate(pp + PA_GROUPS, base1);
+        float k0[EPL], v0[EPL], k1[EPL], v1[EPL];
+        if (have0) {
+            fetch(base0, k0, v0);
+        }
+        if (have1) {
+            fetch(base1, k1, v1);
+        }
+        if (have0) {
+            absorb(k0, v0);
+        }
+        if (have1) {
+            absorb(k1, v1);
         }
     }
 
-    // the 16 groups meet: out = sum_g acc_g * exp(m_g - M) / sum_g l_g * exp(m_g - M)
+    // the groups meet: out = sum_g acc_g * exp(m_g - M) / sum_g l_g * exp(m_g - M)
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) {
-        s_acc[g][d0 + e] = acc[e];
-    }
-    if (l == 0) {
-        s_m[g] = m;
-        s_l[g] = lsum;
+    for (int h = 0; h < QH; ++h) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            s_acc[g][h][d0 + e] = acc[h][e];
+        }
+        if (l == 0) {
+            s_m[g][h] = m[h];
+            s_l[g][h] = lsum[h];
+        }
     }
     __syncthreads();
-    const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)qh * p.out_stride[1];
-    for (uint32_t d = (uint32_t)tid; d < p.head_dim; d += 256u) {
+    for (uint32_t idx = (uint32_t)tid; idx < (uint32_t)QH * p.head_dim; idx += 16u * PA_GROUPS) {
+        uint32_t h = 0, d = idx;  // idx = h * head_dim + d
+        while (d >= p.head_dim) {
+            d -= p.head_dim;
+            ++h;
+        }
         float big = -INFINITY;
 #pragma unroll
-        for (int gg = 0; gg < 16; ++gg) {
-            big = fmaxf(big, s_m[gg]);
+        for (int gg = 0; gg < PA_GROUPS; ++gg) {
+            big = fmaxf(big, s_m[gg][h]);
         }
-        float o = 0.0f;
+        float o = 0.0f, total = 0.0f;
         if (big != -INFINITY) {  // has_any (:552-557)
-            float total = 0.0f;
 #pragma unroll
-            for (int gg = 0; gg < 16; ++gg) {
-                const float f = s_m[gg] == -INFINITY ? 0.0f : expf(s_m[gg] - big);
-                total = __builtin_fmaf(s_l[gg], f, total);
-                o = __builtin_fmaf(s_acc[gg][d], f, o);
+            for (int gg = 0; gg < PA_GROUPS; ++gg) {
+                const float f = s_m[gg][h] == -INFINITY ? 0.0f : expf(s_m[gg][h] - big);
+                total = __builtin_fmaf(s_l[gg][h], f, total);
+                o = __builtin_fmaf(s_acc[gg][h][d], f, o);
             }
-            o = total > 0.0f ? o * (1.0f / total) : 0.0f;
         }
+        if (p.splits > 1u) {  // the shares of the history meet in k_pa_merge
+            float *part = p.partial + (((size_t)t * p.num_q_heads + qh0 + h) * p.splits + blockIdx.z) * (p.head_dim + 2u);
+            if (d == 0) {
+                part[0] = big;
+                part[1] = total;
+            }
+            part[2 + d] = o;
+            continue;
+        }
+        o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)(qh0 + h) * p.out_stride[1];
         pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
     }
+}
+
+// the shares of a (token, head) pair's history: out = sum_s o_s * exp(M_s - M) / sum_s l_s * exp(M_s - M)
+__global__ __launch_bounds__(256) void k_pa_merge(const PaParams p) {
+    const uint32_t t = blockIdx.x, qh = blockIdx.y;
+    const float *part = p.partial + ((size_t)t * p.num_q_heads + qh) * p.splits * (p.head_dim + 2u);
+    float big = -INFINITY;
+    for (uint32_t z = 0; z < p.splits; ++z) {
+        big = fmaxf(big, part[(size_t)z * (p.head_dim + 2u)]);
+    }
+    const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)qh * p.out_stride[1];
+    for (uint32_t d = threadIdx.x; d < p.head_dim; d += blockDim.x) {
+        float o = 0.0f, total = 0.0f;
+        if (big != -INFINITY) {
+            for (uint32_t z = 0; z < p.splits; ++z) {
+                const float *ps = part + (size_t)z * (p.head_dim + 2u);
+                const float f = ps[0] == -INFINITY ? 0.0f : expf(ps[0] - big);
+                total = __builtin_fmaf(ps[1], f, total);
+                o = __builtin_fmaf(ps[2 + d], f, o);
+            }
+        }
+        o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
+    }
+}
+
+template <int EPL, int QH>
+static void pa_launch(marmot_hip_device *dev, const PaParams &p) {
+    hipLaunchKernelGGL((k_pa_attend<EPL, QH>), dim3(p.token_count, p.num_q_heads / QH, p.splits),
+                       dim3(16 * PA_GROUPS), 0, dev->stream, p);
 }
 
 static bool pa_float_dtype(int d) {
@@ -364,15 +457,36 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     hipLaunchKernelGGL(k_pa_write, dim3(a->token_count, a->num_kv_heads), dim3(a->head_dim <= 64 ? 64 : 128), 0,
                        dev->stream, p);
     MH_HIP(hipGetLastError());
-    const dim3 grid(a->token_count, a->num_q_heads);
+    // query heads per workgroup: as many heads of one key / value head as the LDS tile of the final merge allows
+    const int qh_max = epl == 16 ? 2 : 4;
+    const int qh = (p.group % 4 == 0 && qh_max >= 4) ? 4 : (p.group % 2 == 0 ? 2 : 1);
+    // few (token, heads) pairs (a decode step): the history is split over workgroups until the chip is about eight
+    // workgroups per compute unit deep, and a second kernel joins the shares
+    const size_t pairs = (size_t)a->token_count * (a->num_q_heads / (uint32_t)qh);
+    const size_t want = 8u * (size_t)dev->props.multiProcessorCount;
+    p.splits = 1;
+    p.partial = nullptr;
+    if (pairs * 2 <= want) {
+        size_t sp = (want + pairs - 1) / pairs;
+        p.splits = (uint32_t)(sp > 64 ? 64 : sp);
+        void *ws = nullptr;
+        MH_TRY(workspace_reserve(dev, (size_t)a->token_count * a->num_q_heads * p.splits * (a->head_dim + 2u) * sizeof(float),
+                                 &ws));
+        p.partial = (float *)ws;
+    }
     if (epl == 4) {
-        hipLaunchKernelGGL(k_pa_attend<4>, grid, dim3(256), 0, dev->stream, p);
+        qh == 4 ? pa_launch<4, 4>(dev, p) : qh == 2 ? pa_launch<4, 2>(dev, p) : pa_launch<4, 1>(dev, p);
     } else if (epl == 8) {
-        hipLaunchKernelGGL(k_pa_attend<8>, grid, dim3(256), 0, dev->stream, p);
+        qh == 4 ? pa_launch<8, 4>(dev, p) : qh == 2 ? pa_launch<8, 2>(dev, p) : pa_launch<8, 1>(dev, p);
     } else {
-        hipLaunchKernelGGL(k_pa_attend<16>, grid, dim3(256), 0, dev->stream, p);
+        qh == 2 ? pa_launch<16, 2>(dev, p) : pa_launch<16, 1>(dev, p);
     }
     MH_HIP(hipGetLastError());
+    if (p.splits > 1u) {
+        hipLaunchKernelGGL(k_pa_merge, dim3(a->token_count, a->num_q_heads), dim3(a->head_dim <= 64 ? 64 : 128), 0,
+                           dev->stream, p);
+        MH_HIP(hipGetLastError());
+    }
     set_route("paged_attention");
     return MARMOT_HIP_SUCCESS;
 }

@@ -466,6 +466,11 @@ class HipContext:
     def host_freed(self, t: HostTensor):
         self.ops.on_host_ptr_freed(self.device_ctx, t.t.data)
 
+    def host_range_freed(self, t: HostTensor):
+        """on_host_range_freed over the tensor's whole extent: no mirror that touches it survives."""
+        nbytes = getattr(t, "extent_bytes", t.array.nbytes)
+        self.ops.on_host_range_freed(self.device_ctx, t.t.data, nbytes)
+
     def synchronize(self):
         self._check(self.ops.synchronize(self.device_ctx))
 

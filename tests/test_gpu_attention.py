@@ -91,6 +91,14 @@ def test_long_context_decode_batch(hip, oracle):
     check(hip, oracle, case, "decode batch")
 
 
+def test_prompt_of_many_tokens_takes_unsplit_histories(hip, oracle):
+    """A prompt chunk of 640 tokens on top of 100 positions of history, next to a short second sequence: enough
+    (token, heads) pairs that no history is split across workgroups (decode-sized calls above split it)."""
+    case = make_case(60, [(100, 640), (3, 8)], num_q_heads=4, num_kv_heads=2, head_dim=64, block_size=32, act="f16",
+                     kv="f16", layers=1, layer_idx=0)
+    check(hip, oracle, case, "prompt chunk")
+
+
 def test_holes_strided_views_token_count_and_errors(hip, oracle):
     case = make_case(13, [(40, 3), (5, 1)], num_q_heads=4, num_kv_heads=2, head_dim=32, block_size=8)
     seq = case["token_meta"][0, 0]

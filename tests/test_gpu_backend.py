@@ -799,9 +799,10 @@ def test_program_norm_feeds_linears_without_quantization_launches(ctx, oracle):
 
 
 # ---------------------------------------------------------------- paged attention
-def _attention_tensors(case):
+def _attention_tensors(ctx, case):
     """Host tensors of a paged-attention case: q / k_new / v_new as views of one buffer (a fused projection's output),
-    bfloat16 as uint16 bits with the type said explicitly."""
+    bfloat16 as uint16 bits with the type said explicitly. Like memory fresh from marmot's allocator, no mirror of a
+    previous owner of these addresses survives (the core notifies the backend when it frees host memory)."""
     from tests.attention_cases import to_storage
 
     act_dt = {"f32": None, "f16": None, "bf16": ta.DTYPE_BF16}[case["act"]]
@@ -821,6 +822,9 @@ def _attention_tensors(case):
         "block_table": ta.HostTensor.dense(case["block_table"]),
         "out": ta.HostTensor.strided(np.zeros((T, hq, d), dtype=case["q"].dtype), act_dt),
     }
+    for name, x in t.items():
+        if name != "fused":
+            ctx.host_range_freed(x)
     desc = ta.PagedAttentionDesc.default()
     desc.token_count, desc.layer_idx, desc.scale = T, case["layer_idx"], case["scale"]
     desc.num_q_heads, desc.num_kv_heads, desc.head_dim, desc.block_size = hq, hkv, d, case["block_size"]
@@ -848,7 +852,7 @@ def test_impl_and_program_paged_attention(ctx, oracle, act, kv):
     def close(got):
         return np.max(np.abs(to_f32(got, act).astype(np.float64) - to_f32(ref, act).astype(np.float64))) <= tol
 
-    t, desc = _attention_tensors(case)
+    t, desc = _attention_tensors(ctx, case)
     assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
     assert close(ctx.to_host(t["out"]))
     assert np.array_equal(ctx.to_host(t["kv_k"]).view(np.uint8), ref_k.view(np.uint8))
@@ -860,7 +864,7 @@ def test_impl_and_program_paged_attention(ctx, oracle, act, kv):
     sig.weight_dtype = t["kv_k"].t.dtype
     sel = ctx.query(sig)
     assert sel.supported and sel.op_index == ta.BC_OP_PAGED_ATTENTION
-    t2, d2 = _attention_tensors(case)
+    t2, d2 = _attention_tensors(ctx, case)
     p = ta.Program()
     p.paged_attention(sel.op_index, t2["token_meta"], t2["q"], t2["k_new"], t2["v_new"], t2["kv_k"], t2["kv_v"],
                       t2["block_table"], t2["out"], d2.token_count, d2.layer_idx, d2.num_q_heads, d2.num_kv_heads,
@@ -882,7 +886,7 @@ def test_impl_and_program_paged_attention(ctx, oracle, act, kv):
     st, ref2 = oracle.paged_attention(meta, nxt["q"], nxt["k_new"], nxt["v_new"], ref_k, ref_v, case["block_table"],
                                       case["layer_idx"], case["scale"], act_bf16=act == "bf16", kv_bf16=kv == "bf16")
     assert st == 0
-    t3, d3 = _attention_tensors(nxt)
+    t3, d3 = _attention_tensors(ctx, nxt)
     d3.kv_k, d3.kv_v = t["kv_k"].ptr, t["kv_v"].ptr  # the tensors the first call updated
     assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(d3)) == ta.SUCCESS, ctx.last_error()
     got2 = ctx.to_host(t3["out"])
@@ -900,7 +904,7 @@ def test_impl_paged_attention_errors(ctx):
     from tests.attention_cases import make_case
 
     case = make_case(72, [(5, 2)], num_q_heads=4, num_kv_heads=2, head_dim=64, block_size=8)
-    t, desc = _attention_tensors(case)
+    t, desc = _attention_tensors(ctx, case)
 
     def call(**kw):
         d = ta.PagedAttentionDesc.default()
@@ -937,7 +941,7 @@ def test_impl_paged_attention_errors(ctx):
     ext = ta.PagedAttentionKvScaleExt(C.sizeof(ta.PagedAttentionKvScaleExt), 1, t["kv_k"].ptr, t["kv_v"].ptr)
     assert call(pnext=C.addressof(ext)) == ta.INVALID_ARGUMENT and "require FP8" in ctx.last_error()[1]
     wide = make_case(73, [(2, 1)], num_q_heads=1, num_kv_heads=1, head_dim=320, block_size=4)
-    tw, dw = _attention_tensors(wide)
+    tw, dw = _attention_tensors(ctx, wide)
     assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(dw)) == ta.NOT_IMPLEMENTED
     for group in (t, tw):
         for name, x in group.items():

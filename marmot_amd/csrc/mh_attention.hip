@@ -72,6 +72,12 @@ __device__ __forceinline__ void pa_store(void *data, int dtype, size_t i, float 
     }
 }
 
+// exp(x) for x <= 0 (softmax weights and rescaling factors): the hardware's base-2 exponential, about 2 units in the
+// last place -- far inside the tolerance of the output, and a fraction of the library routine's instructions
+__device__ __forceinline__ float pa_exp(float x) {
+    return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
+}
+
 // EPL consecutive values starting at element `first` (unit stride, 16-byte aligned start for the storage type)
 template <int EPL>
 __device__ __forceinline__ void pa_load_run(const void *data, int dtype, size_t first, float (&v)[EPL]) {
@@ -236,7 +242,7 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
             }
             dot = row16_sum(dot);
             if (dot > m[h]) {  // the same decision in all 16 lanes of the group
-                const float corr = m[h] == -INFINITY ? 0.0f : expf(m[h] - dot);
+                const float corr = m[h] == -INFINITY ? 0.0f : pa_exp(m[h] - dot);
                 lsum[h] *= corr;
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) {
@@ -244,7 +250,7 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
                 }
                 m[h] = dot;
             }
-            const float w = expf(dot - m[h]);
+            const float w = pa_exp(dot - m[h]);
             lsum[h] += w;
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
@@ -302,7 +308,7 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
         if (big != -INFINITY) {  // has_any (:552-557)
 #pragma unroll
             for (int gg = 0; gg < PA_GROUPS; ++gg) {
-                const float f = s_m[gg][h] == -INFINITY ? 0.0f : expf(s_m[gg][h] - big);
+                const float f = s_m[gg][h] == -INFINITY ? 0.0f : pa_exp(s_m[gg][h] - big);
                 total = __builtin_fmaf(s_l[gg][h], f, total);
                 o = __builtin_fmaf(s_acc[gg][h][d], f, o);
             }
@@ -324,21 +330,26 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
 
 // the shares of a (token, head) pair's history: out = sum_s o_s * exp(M_s - M) / sum_s l_s * exp(M_s - M)
 __global__ __launch_bounds__(256) void k_pa_merge(const PaParams p) {
+    __shared__ float s_big[64], s_tot[64];  // splits <= 64
     const uint32_t t = blockIdx.x, qh = blockIdx.y;
     const float *part = p.partial + ((size_t)t * p.num_q_heads + qh) * p.splits * (p.head_dim + 2u);
+    if (threadIdx.x < p.splits) {
+        s_big[threadIdx.x] = part[(size_t)threadIdx.x * (p.head_dim + 2u)];
+        s_tot[threadIdx.x] = part[(size_t)threadIdx.x * (p.head_dim + 2u) + 1];
+    }
+    __syncthreads();
     float big = -INFINITY;
     for (uint32_t z = 0; z < p.splits; ++z) {
-        big = fmaxf(big, part[(size_t)z * (p.head_dim + 2u)]);
+        big = fmaxf(big, s_big[z]);
     }
     const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)qh * p.out_stride[1];
     for (uint32_t d = threadIdx.x; d < p.head_dim; d += blockDim.x) {
         float o = 0.0f, total = 0.0f;
         if (big != -INFINITY) {
             for (uint32_t z = 0; z < p.splits; ++z) {
-                const float *ps = part + (size_t)z * (p.head_dim + 2u);
-                const float f = ps[0] == -INFINITY ? 0.0f : expf(ps[0] - big);
-                total = __builtin_fmaf(ps[1], f, total);
-                o = __builtin_fmaf(ps[2 + d], f, o);
+                const float f = s_big[z] == -INFINITY ? 0.0f : pa_exp(s_big[z] - big);
+                total = __builtin_fmaf(s_tot[z], f, total);
+                o = __builtin_fmaf(part[(size_t)z * (p.head_dim + 2u) + 2 + d], f, o);
             }
         }
         o = total > 0.0f ? o * (1.0f / total) : 0.0f;

@@ -372,8 +372,10 @@ def test_impl_qkv_errors(ctx, oracle):
         if rope is not None:
             d.rope_params = C.pointer(rope)
         keep = (xt, wts, outs, bts, rope)
+        made.extend([xt] + list(wts) + list(outs) + [b for b in bts if b is not None])
         return d, keep
 
+    made = []  # every tensor a call may have mirrored: released at the end like the core does on tensor destruction
     d, keep = build()
     assert fn(ctx.device_ctx, C.byref(d)) == ta.SUCCESS
     assert fn(ctx.device_ctx, None) == ta.INVALID_ARGUMENT
@@ -415,6 +417,8 @@ def test_impl_qkv_errors(ctx, oracle):
     rope.positions = None
     d, keep = build(rope=rope)
     assert fn(ctx.device_ctx, C.byref(d)) == ta.SUCCESS
+    for t in made + [pos, pos1, pos2]:
+        ctx.host_freed(t)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])

@@ -1826,7 +1826,8 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
         a.kv_stride[i] = kv_k->shape.strides[i];
     }
     pthread_mutex_lock(&b->mu);
-    // the caches are read and written; the output may be a view with gaps: the host's bytes go up first
+    // the caches are read and written; an output that is a view with gaps, or has more rows than tokens, keeps its
+    // other bytes: the host's bytes go up first
     hip_acq_t acq[8] = {
         {meta->data, strided_extent_bytes(meta), HIP_ACQ_READ, nullptr},
         {table->data, strided_extent_bytes(table), HIP_ACQ_READ, nullptr},
@@ -1835,7 +1836,8 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
         {v_new->data, strided_extent_bytes(v_new), HIP_ACQ_READ, nullptr},
         {kv_k->data, strided_extent_bytes(kv_k), HIP_ACQ_UPDATE, nullptr},
         {kv_v->data, strided_extent_bytes(kv_v), HIP_ACQ_UPDATE, nullptr},
-        {out->data, strided_extent_bytes(out), HIP_ACQ_UPDATE, nullptr},
+        {out->data, strided_extent_bytes(out),
+         dense_contiguous(out) && out->shape.shape[0] == desc->token_count ? HIP_ACQ_WRITE : HIP_ACQ_UPDATE, nullptr},
     };
     marmot_error_t st = acquire_set(b, acq, 8);
     const void *d_meta = acq[0].dev, *d_table = acq[1].dev, *d_q = acq[2].dev, *d_k = acq[3].dev, *d_v = acq[4].dev;

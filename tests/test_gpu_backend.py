@@ -951,3 +951,142 @@ def test_impl_paged_attention_errors(ctx):
         for name, x in group.items():
             if name != "fused":
                 ctx.host_freed(x)
+
+
+def test_program_whole_decoder_layer(ctx, oracle):
+    """One decoder layer of a Llama-shaped model as ONE bytecode program on this backend, every node of the decode
+    graph between the embedding and the logits: rms_norm -> q, k, v projections (Q4_K, Q4_K, Q6_K) -> rotary embedding
+    of q and k -> paged attention (cache write + attention through the block table, fp16 cache) -> output projection
+    -> residual add -> rms_norm -> gate, up -> swiglu -> down -> residual add. 12 tokens: three sequences with history,
+    one of them a prompt chunk. Against the oracle's chain of the same operations."""
+    from oracle.pyoracle import RopeParams as OracleRope
+    from tests.attention_cases import make_case
+    from tests.util import assert_moe_parity
+
+    hq, hkv, hd, H, F, bs = 8, 2, 64, 512, 1024, 16
+    case = make_case(80, [(21, 1), (40, 1), (7, 10)], num_q_heads=hq, num_kv_heads=hkv, head_dim=hd, block_size=bs,
+                     act="f32", kv="f16", layers=1, layer_idx=0)
+    meta = case["token_meta"]
+    T = meta.shape[0]
+    x = gaussian(1400, (T, H))
+    w1 = gaussian(1401, (H,), 0.2) + np.float32(1.0)
+    w2 = gaussian(1402, (H,), 0.2) + np.float32(1.0)
+    wq = oracle.quantize(KIND_Q4_K, gaussian(1403, (hq * hd, H), 0.05))
+    wk = oracle.quantize(KIND_Q4_K, gaussian(1404, (hkv * hd, H), 0.05))
+    wv = oracle.quantize(KIND_Q6_K, gaussian(1405, (hkv * hd, H), 0.05))
+    wo = oracle.quantize(KIND_Q4_K, gaussian(1406, (H, hq * hd), 0.05))
+    wg = oracle.quantize(KIND_Q4_K, gaussian(1407, (F, H), 0.05))
+    wu = oracle.quantize(KIND_Q4_K, gaussian(1408, (F, H), 0.05))
+    wd = oracle.quantize(KIND_Q6_K, gaussian(1409, (H, F), 0.05))
+    pos = meta[:, 1].astype(np.int32)
+    pos_q, pos_k = np.repeat(pos, hq), np.repeat(pos, hkv)  # one position per (token, head) row
+    scale = float(1.0 / np.sqrt(hd))
+
+    # ---- the oracle's chain
+    r_h = oracle.rms_norm(x, w1, eps=1e-5)
+    r_q = oracle.matmul(KIND_Q4_K, wq, r_h, hq * hd, threads=8)
+    r_k = oracle.matmul(KIND_Q4_K, wk, r_h, hkv * hd, threads=8)
+    r_v = oracle.matmul(KIND_Q6_K, wv, r_h, hkv * hd, threads=8)
+    rp = OracleRope.default(rope_type=0)
+    st, r_qr = oracle.rope(r_q.reshape(T * hq, hd), pos_q, rp)
+    assert st == 0
+    st, r_kr = oracle.rope(r_k.reshape(T * hkv, hd), pos_k, rp)
+    assert st == 0
+    ref_k, ref_v = case["kv_k"].copy(), case["kv_v"].copy()
+    st, r_att = oracle.paged_attention(meta, r_qr.reshape(T, hq, hd), r_kr.reshape(T, hkv, hd), r_v.reshape(T, hkv, hd),
+                                       ref_k, ref_v, case["block_table"], 0, scale)
+    assert st == 0
+    r_o = oracle.matmul(KIND_Q4_K, wo, r_att.reshape(T, hq * hd), H, threads=8)
+    r_x1 = x + r_o
+    r_h2 = oracle.rms_norm(r_x1, w2, eps=1e-5)
+    r_a = oracle.glu(oracle.matmul(KIND_Q4_K, wg, r_h2, F, threads=8), oracle.matmul(KIND_Q4_K, wu, r_h2, F, threads=8))
+    r_y = r_x1 + oracle.matmul(KIND_Q6_K, wd, r_a, H, threads=8)
+
+    # ---- the same as one program; 2-D projection outputs are viewed as [tokens, heads, head_dim] / [rows, head_dim]
+    dense, empty, view = ta.HostTensor.dense, ta.HostTensor.empty, ta.HostTensor.strided
+    xt, w1t, w2t = dense(x), dense(w1), dense(w2)
+    wts = {n: ta.HostTensor.quantized(b, s, k) for n, (b, s, k) in {
+        "q": (wq, (hq * hd, H), KIND_Q4_K), "k": (wk, (hkv * hd, H), KIND_Q4_K), "v": (wv, (hkv * hd, H), KIND_Q6_K),
+        "o": (wo, (H, hq * hd), KIND_Q4_K), "g": (wg, (F, H), KIND_Q4_K), "u": (wu, (F, H), KIND_Q4_K),
+        "d": (wd, (H, F), KIND_Q6_K)}.items()}
+    h, q2, k2, v2 = empty((T, H), ta.DTYPE_F32), empty((T, hq * hd), ta.DTYPE_F32), empty((T, hkv * hd), ta.DTYPE_F32), \
+        empty((T, hkv * hd), ta.DTYPE_F32)
+    q_rows, k_rows = view(q2.array.reshape(T * hq, hd)), view(k2.array.reshape(T * hkv, hd))
+    q3, k3, v3 = view(q2.array.reshape(T, hq, hd)), view(k2.array.reshape(T, hkv, hd)), view(v2.array.reshape(T, hkv, hd))
+    att = empty((T, hq * hd), ta.DTYPE_F32)
+    att3 = view(att.array.reshape(T, hq, hd))
+    o, x1, h2, g, u, a, d, y = (empty(s, ta.DTYPE_F32) for s in
+                                ((T, H), (T, H), (T, H), (T, F), (T, F), (T, F), (T, H), (T, H)))
+    mt, tbl = dense(meta), dense(case["block_table"])
+    kvk, kvv = view(case["kv_k"].copy()), view(case["kv_v"].copy())
+    pq, pk = dense(pos_q), dense(pos_k)
+    rq, rk = _rope_params(pq, rope_type=0), _rope_params(pk, rope_type=0)
+    every = [xt, w1t, w2t, h, q2, k2, v2, att, o, x1, h2, g, u, a, d, y, mt, tbl, kvk, kvv, pq, pk] + list(wts.values())
+    for t in every:
+        ctx.host_range_freed(t)  # fresh memory: no mirror of a previous owner of these addresses
+    mm = {KIND_Q4_K: 3, KIND_Q6_K: 4}
+    p = ta.Program()
+    p.rms_norm(ta.BC_OP_RMS_NORM_F32, xt, w1t, None, h, 1e-5)
+    p.matmul(mm[KIND_Q4_K], h, wts["q"], q2)
+    p.matmul(mm[KIND_Q4_K], h, wts["k"], k2)
+    p.matmul(mm[KIND_Q6_K], h, wts["v"], v2)
+    p.rope(ta.BC_OP_ROPE, q_rows, q_rows, rq)
+    p.rope(ta.BC_OP_ROPE, k_rows, k_rows, rk)
+    p.paged_attention(ta.BC_OP_PAGED_ATTENTION, mt, q3, k3, v3, kvk, kvv, tbl, att3, T, 0, hq, hkv, hd, bs, scale)
+    p.matmul(mm[KIND_Q4_K], att, wts["o"], o)
+    p.binary(ta.BC_OP_ADD_F32, xt, o, x1)
+    p.rms_norm(ta.BC_OP_RMS_NORM_F32, x1, w2t, None, h2, 1e-5)
+    p.matmul(mm[KIND_Q4_K], h2, wts["g"], g)
+    p.matmul(mm[KIND_Q4_K], h2, wts["u"], u)
+    p.binary(ta.BC_OP_SWIGLU_F32, g, u, a)
+    p.matmul(mm[KIND_Q6_K], a, wts["d"], d)
+    p.binary(ta.BC_OP_ADD_F32, x1, d, y)
+    uploads0 = ctx.residency().uploads
+    assert ctx.execute(p) == ta.SUCCESS, ctx.last_error()
+    # intermediate tensors never travel: only the inputs (x, two norm weights), the seven weights, metadata and block
+    # table, the two caches, the two position tensors and the rotary frequency table were uploaded
+    assert ctx.residency().uploads - uploads0 == 3 + 7 + 2 + 2 + 2 + 1
+    # Stage by stage, every operation against the oracle ON THE DEVICE'S OWN INPUTS of that stage (each linear
+    # re-quantizes its input, so end-to-end differences grow with the chain; a stage's own error does not). Views are
+    # read through the tensor object that was written (the "device copy is newer" flag belongs to it).
+    from tests.attention_cases import TOLERANCE
+    from tests.util import assert_matmul_parity
+
+    g_h = ctx.to_host(h).copy()
+    assert np.allclose(g_h, r_h, rtol=1e-5, atol=1e-8)
+    g_q, g_k = ctx.to_host(q_rows).copy(), ctx.to_host(k_rows).copy()
+    g_v = ctx.to_host(v2).copy()
+    for got, w_, kind_, M_, pos_, heads in ((g_q, wq, KIND_Q4_K, hq * hd, pos_q, hq), (g_k, wk, KIND_Q4_K, hkv * hd, pos_k, hkv)):
+        st, want = oracle.rope(oracle.matmul(kind_, w_, g_h, M_, threads=8).reshape(T * heads, hd), pos_, rp)
+        assert st == 0
+        assert_matmul_parity(got, want, what="projection + rotary embedding")
+    assert_matmul_parity(g_v, oracle.matmul(KIND_Q6_K, wv, g_h, hkv * hd, threads=8), what="v projection")
+    s_k, s_v = case["kv_k"].copy(), case["kv_v"].copy()
+    st, want = oracle.paged_attention(meta, g_q.reshape(T, hq, hd), g_k.reshape(T, hkv, hd), g_v.reshape(T, hkv, hd),
+                                      s_k, s_v, case["block_table"], 0, scale)
+    assert st == 0
+    g_att = ctx.to_host(att3).reshape(T, hq * hd).copy()
+    assert np.max(np.abs(g_att - want.reshape(T, hq * hd))) <= TOLERANCE["f32"] * np.abs(s_v.astype(np.float32)).max()
+    assert np.array_equal(ctx.to_host(kvk).view(np.uint8), s_k.view(np.uint8))  # the cache after the device's own rows
+    assert np.array_equal(ctx.to_host(kvv).view(np.uint8), s_v.view(np.uint8))
+    g_o = ctx.to_host(o).copy()
+    assert_matmul_parity(g_o, oracle.matmul(KIND_Q4_K, wo, g_att, H, threads=8), what="output projection")
+    g_x1 = ctx.to_host(x1).copy()
+    assert np.array_equal(bits(g_x1), bits(x + g_o))
+    g_h2 = ctx.to_host(h2).copy()
+    assert np.allclose(g_h2, oracle.rms_norm(g_x1, w2, eps=1e-5), rtol=1e-5, atol=1e-8)
+    g_a = ctx.to_host(a).copy()
+    want_a = oracle.glu(oracle.matmul(KIND_Q4_K, wg, g_h2, F, threads=8), oracle.matmul(KIND_Q4_K, wu, g_h2, F, threads=8))
+    assert_moe_parity(g_a, want_a, what="gate, up and the gated product")
+    g_d = ctx.to_host(d).copy()
+    assert_matmul_parity(g_d, oracle.matmul(KIND_Q6_K, wd, g_a, H, threads=8), what="down projection")
+    assert np.array_equal(bits(ctx.to_host(y)), bits(g_x1 + g_d))
+    # end to end against the oracle's own chain: five re-quantization points in a row
+    assert_moe_parity(g_att, r_att.reshape(T, hq * hd), what="attention output inside the layer")
+    assert_moe_parity(ctx.to_host(y), r_y, tol=1e-2, what="decoder layer output, end to end")
+    # the cache rows the layer wrote: fp16 roundings of keys / values that differ from the oracle's by the linears'
+    # summation order, so the comparison is numerical, not bitwise
+    got_k = ctx.to_host(kvk).astype(np.float32)
+    assert np.max(np.abs(got_k - ref_k.astype(np.float32))) <= 2e-3 * np.abs(ref_k.astype(np.float32)).max()
+    for t in every:
+        ctx.host_freed(t)

@@ -229,8 +229,8 @@ def prefill_int8(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "ATTN", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
-    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, ATTN, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "ATTN", "LAYER", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
+    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, ATTN, LAYER, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -320,6 +320,8 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5
         sweep_ops(hip, rng, emit, steps, warmup)
     if "ATTN" in only:
         sweep_attention(hip, rng, emit, steps)
+    if "LAYER" in only:
+        sweep_whole_layer(hip, rng, emit, steps)
     if "LOGITS" in only:
         # the vocabulary-sized matvec at the end of a decode step (Llama-3 vocabulary, 128256 rows of 4096)
         for kind in (capi.KIND_Q6_K, capi.KIND_Q4_K):
@@ -549,6 +551,91 @@ def sweep_attention(hip, rng, emit, steps: int):
     run("paged attention, decode: 16 sequences x 4096 positions, 32/8 heads of 128, fp16 cache", [(4095, 1)] * 16)
     run("paged attention, decode: 16 sequences x 512 positions", [(511, 1)] * 16)
     run("paged attention, prompt: 512 tokens of one sequence", [(0, 512)])
+
+
+def sweep_whole_layer(hip, rng, emit, steps: int, T: int = 16, context: int = 4096):
+    """One decode step of a whole Llama-3-8B layer for 16 sequences with 4096 positions of history each, every op on
+    the device: rms_norm (leaves its rows packed) -> q, k (Q4_K), v (Q6_K) -> rotary embedding of q and k -> paged
+    attention (fp16 cache) -> pack -> o (Q4_K) -> add -> rms_norm (packed) -> gate, up (Q4_K) -> swiglu (packed) ->
+    down (Q6_K) -> add. Four copies of the 139 MB of weights rotate; the 268 MB cache is one copy."""
+    import ctypes as C
+
+    from marmot_amd import DT_F32, capi, row_bytes
+
+    lib, dev, vp, chk = hip.lib, hip.dev, C.c_void_p, capi.check
+    H, F, hq, hkv, hd, bs = 4096, 14336, 32, 8, 128, 16
+    Q4, Q6 = capi.KIND_Q4_K, capi.KIND_Q6_K
+    specs = {"q": (Q4, hq * hd, H), "k": (Q4, hkv * hd, H), "v": (Q6, hkv * hd, H), "o": (Q4, H, hq * hd),
+             "g": (Q4, F, H), "u": (Q4, F, H), "d": (Q6, H, F)}
+    copies, weights, wbytes = 4, {}, 0
+    for name, (kind, M, K) in specs.items():
+        stride = (M * row_bytes(kind, K) + 255) & ~255
+        blocks = random_blocks(rng, kind, M, K)
+        buf = hip.alloc(stride * copies)
+        for c in range(copies):
+            buf.upload(blocks, offset=c * stride)
+        weights[name] = (buf, stride)
+        wbytes += M * row_bytes(kind, K)
+    f32 = lambda *shape: hip.to_device(rng.standard_normal(shape, dtype=np.float32))
+    x, wn1, wn2 = f32(T, H), hip.to_device(np.ones(H, np.float32)), hip.to_device(np.ones(H, np.float32))
+    h, q, k, v, att, o, x1, h2, g, u, d, y = (hip.alloc(T * n * 4) for n in
+                                              (H, hq * hd, hkv * hd, hkv * hd, hq * hd, H, H, H, F, F, H, H))
+    packs = {n: hip.alloc(hip.packed_activation_bytes(Q4, T, K)) for n, K in (("h", H), ("att", hq * hd), ("h2", H), ("a", F))}
+    blocks_per_seq = -(-context // bs)
+    table = np.arange(T * blocks_per_seq, dtype=np.uint32).reshape(T, blocks_per_seq)
+    meta = np.array([[s_, context - 1, int(table[s_, (context - 1) // bs]) * bs + (context - 1) % bs, 0] for s_ in range(T)],
+                    dtype=np.uint32)
+    cache_shape = (T * blocks_per_seq, 1, hkv, bs, hd)
+    arrays = {"token_meta": meta, "block_table": table, "kv_k": np.zeros(cache_shape, np.float16),
+              "kv_v": np.zeros(cache_shape, np.float16)}
+    arrays["kv_k"][...] = rng.standard_normal(cache_shape, dtype=np.float32)
+    arrays["kv_v"][...] = rng.standard_normal(cache_shape, dtype=np.float32)
+    devs = {n: hip.to_device(a) for n, a in arrays.items()}
+    shaped = {"q": np.empty((T, hq, hd), np.float32), "k_new": np.empty((T, hkv, hd), np.float32),
+              "v_new": np.empty((T, hkv, hd), np.float32), "out": np.empty((T, hq, hd), np.float32)}
+    ptr_of = {id(arrays[n]): devs[n].ptr for n in arrays}
+    ptr_of.update({id(shaped["q"]): q.ptr, id(shaped["k_new"]): k.ptr, id(shaped["v_new"]): v.ptr, id(shaped["out"]): att.ptr})
+    pa = hip.paged_attention_args(lambda a: ptr_of[id(a)], meta, shaped["q"], shaped["k_new"], shaped["v_new"],
+                                  arrays["kv_k"], arrays["kv_v"], table, shaped["out"], 0, float(1.0 / np.sqrt(hd)))
+    freqs, scale, rhd = hip.rope_frequencies(hd, head_dim=hd, theta=500000.0)
+    d_f = hip.to_device(freqs)
+    pos_q = hip.to_device(np.repeat(meta[:, 1].astype(np.int32), hq))
+    pos_k = hip.to_device(np.repeat(meta[:, 1].astype(np.int32), hkv))
+    rope_q = capi.Rope(pos_q.ptr, capi.DT_I32, d_f.ptr, scale, rhd, 0, 0, 0)
+    rope_k = capi.Rope(pos_k.ptr, capi.DT_I32, d_f.ptr, scale, rhd, 0, 0, 0)
+
+    def linear(name, packed, out, i):
+        kind, M, K = specs[name]
+        buf, stride = weights[name]
+        chk(lib.marmot_hip_matmul_prepacked(dev, kind, vp(buf.ptr + (i % copies) * stride), vp(packed.ptr), T, K, M, None,
+                                            DT_F32, vp(out.ptr), DT_F32))
+
+    def step(i):
+        chk(lib.marmot_hip_rms_norm_pack(dev, vp(x.ptr), None, vp(wn1.ptr), 0.0, 1e-5, T, H, Q4, vp(h.ptr), vp(packs["h"].ptr)))
+        linear("q", packs["h"], q, i)
+        linear("k", packs["h"], k, i)
+        linear("v", packs["h"], v, i)
+        chk(lib.marmot_hip_rope(dev, vp(q.ptr), DT_F32, T * hq, hd, hd, hd, C.byref(rope_q), vp(q.ptr)))
+        chk(lib.marmot_hip_rope(dev, vp(k.ptr), DT_F32, T * hkv, hd, hd, hd, C.byref(rope_k), vp(k.ptr)))
+        chk(lib.marmot_hip_paged_attention(dev, C.byref(pa), 0))
+        chk(lib.marmot_hip_pack_activations(dev, Q4, vp(att.ptr), DT_F32, T, hq * hd, vp(packs["att"].ptr)))
+        linear("o", packs["att"], o, i)
+        chk(lib.marmot_hip_add(dev, vp(x.ptr), vp(o.ptr), T * H, vp(x1.ptr)))
+        chk(lib.marmot_hip_rms_norm_pack(dev, vp(x1.ptr), None, vp(wn2.ptr), 0.0, 1e-5, T, H, Q4, vp(h2.ptr), vp(packs["h2"].ptr)))
+        linear("g", packs["h2"], g, i)
+        linear("u", packs["h2"], u, i)
+        chk(lib.marmot_hip_swiglu_pack(dev, vp(g.ptr), vp(u.ptr), T, F, Q6, vp(packs["a"].ptr)))
+        linear("d", packs["a"], d, i)
+        chk(lib.marmot_hip_add(dev, vp(x1.ptr), vp(d.ptr), T * H, vp(y.ptr)))
+
+    ms = time_steps_graph(hip, step, max(20, steps // 20), 5, chunk=10)
+    cache_read = T * context * hkv * hd * 2 * 2
+    emit({"config": "LAYER", "workload": f"whole Llama-3-8B decoder layer, decode step of {T} sequences x {context} positions "
+          "(norms, q/k/v/o/gate/up/down linears, rotary embedding, paged attention with fp16 cache, SwiGLU, residual adds)",
+          "us": round(ms * 1e3, 2), "GB/s": round((wbytes + cache_read) / ms / 1e6, 1),
+          "frac_of_hbm_peak": round((wbytes + cache_read) / ms / 1e6 / HBM_PEAK_GBPS, 4),
+          "tokens_per_s_per_layer": round(T / ms * 1e3), "weight_bytes": wbytes, "cache_bytes_read": cache_read,
+          "launches_per_step": 16})
 
 
 def sweep_moe(hip, rng, emit, steps: int):

@@ -3257,6 +3257,70 @@ static float pa_bf16_to_f32(uint16_t h) {
     return f;
 }
 
+/* marmot_fp8_quantize with 4 exponent bits, 3 mantissa bits, bias 7, no infinity, max 240 (dtype_ref.c:118-176) */
+uint8_t mo_f32_to_fp8_e4m3(float value) {
+    if (isnan(value)) {
+        return 0x79; /* exponent field 15, payload 1, sign 0 */
+    }
+    const uint8_t sign = value < 0 ? 0x80 : 0;
+    const float mag = fabsf(value);
+    if (isinf(value) || mag > 240.0f) {
+        return (uint8_t)(sign | 0x77); /* largest finite: exponent field 14, mantissa 7 */
+    }
+    if (mag == 0.0f) {
+        return sign;
+    }
+    int e;
+    float m = frexpf(mag, &e); /* mag = m * 2^e, m in [0.5, 1) */
+    m *= 2.0f;
+    e -= 1;
+    int field = e + 7;
+    if (field > 0 && field < 15) {
+        int r = (int)lrintf((m - 1.0f) * 8.0f); /* nearest, ties to even */
+        if (r == 8) {
+            r = 0;
+            field += 1;
+            if (field >= 15) {
+                return (uint8_t)(sign | 0x77);
+            }
+        }
+        return (uint8_t)(sign | (field << 3) | (r & 7));
+    }
+    /* below the smallest normal 2^-6: multiples of 2^-9 */
+    int r = (int)lrintf(ldexpf(mag, 6 + 3));
+    if (r == 0) {
+        return sign;
+    }
+    if (r > 7) {
+        r = 7;
+    }
+    return (uint8_t)(sign | r);
+}
+
+/* marmot_fp8_dequantize, same format (dtype_ref.c:178-205) */
+float mo_fp8_e4m3_to_f32(uint8_t bits) {
+    const int field = (bits >> 3) & 15, mant = bits & 7;
+    const float s = (bits & 0x80) ? -1.0f : 1.0f;
+    if (field == 15) {
+        return nanf("");
+    }
+    if (field == 0) {
+        return mant == 0 ? ((bits & 0x80) ? -0.0f : 0.0f) : s * ldexpf((float)mant / 8.0f, -6);
+    }
+    return s * ldexpf(1.0f + (float)mant / 8.0f, field - 7);
+}
+
+/* cpu_paged_attention_fp8_quant / _dequant / _scale_from_max (paged_attention_ref.c:142-163) */
+static uint8_t pa_fp8_quant(float value, float scale) {
+    return scale > 0.0f ? mo_f32_to_fp8_e4m3(value / scale) : 0;
+}
+static float pa_fp8_dequant(uint8_t v, float scale) {
+    return scale > 0.0f ? mo_fp8_e4m3_to_f32(v) * scale : 0.0f;
+}
+static float pa_fp8_scale(float max_abs) {
+    return max_abs > 0.0f ? max_abs / 240.0f : 1.0f;
+}
+
 /* cpu_load_as_f32 / cpu_store_from_f32 (cpu_backend_internal.h:641-680) for the three float types */
 static float pa_load(int dtype, const void *data, size_t index) {
     switch (dtype) {
@@ -3311,8 +3375,12 @@ int mo_paged_attention(const mo_paged_attention_args *a) {
         (a->block_size & (a->block_size - 1u)) != 0 || a->num_q_heads % a->num_kv_heads != 0) {
         return MO_ERR_INVALID_ARGUMENT; /* :581-596 */
     }
-    if (!pa_float_dtype(a->act_dtype) || !pa_float_dtype(a->kv_dtype)) {
+    const int fp8 = a->kv_dtype == MO_DTYPE_F8_E4M3;
+    if (!pa_float_dtype(a->act_dtype) || (!fp8 && !pa_float_dtype(a->kv_dtype))) {
         return MO_ERR_UNSUPPORTED_DTYPE; /* :622-630 */
+    }
+    if (fp8 && (a->kv_k_scale == NULL || a->kv_v_scale == NULL)) {
+        return MO_ERR_INVALID_ARGUMENT; /* :695-698 */
     }
     if (a->kv_layers <= a->layer_idx) {
         return MO_ERR_DIMENSION_MISMATCH; /* :673-676 */
@@ -3330,8 +3398,100 @@ int mo_paged_attention(const mo_paged_attention_args *a) {
             return MO_ERR_DIMENSION_MISMATCH;
         }
     }
+    if (fp8) { /* :825-989 */
+        const size_t nb = a->kv_blocks, nh = a->num_kv_heads;
+        uint32_t *min_off = (uint32_t *)malloc(nb * sizeof(uint32_t));
+        float *new_k = (float *)calloc(nb * nh, sizeof(float)), *new_v = (float *)calloc(nb * nh, sizeof(float));
+        if (min_off == NULL || new_k == NULL || new_v == NULL) {
+            free(min_off), free(new_k), free(new_v);
+            return MO_ERR_INVALID_ARGUMENT;
+        }
+        for (size_t b = 0; b < nb; ++b) {
+            min_off[b] = a->block_size; /* "untouched" */
+        }
+        for (size_t t = 0; t < a->token_count; ++t) { /* largest magnitudes of the new rows, first offset written */
+            const uint32_t kv_slot = a->token_meta[t * a->meta_stride[0] + 2 * a->meta_stride[1]];
+            const uint32_t b = kv_slot >> shift, off = kv_slot & mask;
+            if (off < min_off[b]) {
+                min_off[b] = off;
+            }
+            for (size_t h = 0; h < nh; ++h) {
+                for (size_t d = 0; d < hd; ++d) {
+                    const float kx = fabsf(pa_load(a->act_dtype, a->k_new, t * a->k_stride[0] + h * a->k_stride[1] + d * a->k_stride[2]));
+                    const float vx = fabsf(pa_load(a->act_dtype, a->v_new, t * a->v_stride[0] + h * a->v_stride[1] + d * a->v_stride[2]));
+                    if (kx > new_k[b * nh + h]) {
+                        new_k[b * nh + h] = kx;
+                    }
+                    if (vx > new_v[b * nh + h]) {
+                        new_v[b * nh + h] = vx;
+                    }
+                }
+            }
+        }
+        uint8_t *caches[2] = {(uint8_t *)a->kv_k, (uint8_t *)a->kv_v};
+        float *scales[2] = {a->kv_k_scale, a->kv_v_scale};
+        float *news[2] = {new_k, new_v};
+        for (size_t b = 0; b < nb; ++b) {
+            if (min_off[b] == a->block_size) {
+                continue;
+            }
+            const uint32_t existing = min_off[b];
+            for (size_t h = 0; h < nh; ++h) {
+                const size_t si = b * a->scale_stride[0] + (size_t)a->layer_idx * a->scale_stride[1] + h * a->scale_stride[2];
+                for (int which = 0; which < 2; ++which) {
+                    const float old_scale = scales[which][si];
+                    float big = 0.0f;
+                    if (existing > 0 && old_scale > 0.0f) {
+                        for (uint32_t p = 0; p < existing; ++p) {
+                            const size_t base = b * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] +
+                                                h * a->kv_stride[2] + (size_t)p * a->kv_stride[3];
+                            for (size_t d = 0; d < hd; ++d) {
+                                const float x = fabsf(pa_fp8_dequant(caches[which][base + d * a->kv_stride[4]], old_scale));
+                                if (x > big) {
+                                    big = x;
+                                }
+                            }
+                        }
+                    }
+                    if (news[which][b * nh + h] > big) {
+                        big = news[which][b * nh + h];
+                    }
+                    const float new_scale = pa_fp8_scale(big);
+                    if (existing > 0 && new_scale != old_scale) { /* re-encode what the block already holds */
+                        for (uint32_t p = 0; p < existing; ++p) {
+                            const size_t base = b * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] +
+                                                h * a->kv_stride[2] + (size_t)p * a->kv_stride[3];
+                            for (size_t d = 0; d < hd; ++d) {
+                                uint8_t *c = &caches[which][base + d * a->kv_stride[4]];
+                                *c = pa_fp8_quant(pa_fp8_dequant(*c, old_scale), new_scale);
+                            }
+                        }
+                    }
+                    scales[which][si] = new_scale;
+                }
+            }
+        }
+        for (size_t t = 0; t < a->token_count; ++t) { /* the new rows, encoded with their block's scale */
+            const uint32_t kv_slot = a->token_meta[t * a->meta_stride[0] + 2 * a->meta_stride[1]];
+            const size_t b = kv_slot >> shift;
+            for (size_t h = 0; h < nh; ++h) {
+                const size_t si = b * a->scale_stride[0] + (size_t)a->layer_idx * a->scale_stride[1] + h * a->scale_stride[2];
+                const size_t base = b * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] + h * a->kv_stride[2] +
+                                    (size_t)(kv_slot & mask) * a->kv_stride[3];
+                for (size_t d = 0; d < hd; ++d) {
+                    ((uint8_t *)a->kv_k)[base + d * a->kv_stride[4]] = pa_fp8_quant(
+                        pa_load(a->act_dtype, a->k_new, t * a->k_stride[0] + h * a->k_stride[1] + d * a->k_stride[2]),
+                        a->kv_k_scale[si]);
+                    ((uint8_t *)a->kv_v)[base + d * a->kv_stride[4]] = pa_fp8_quant(
+                        pa_load(a->act_dtype, a->v_new, t * a->v_stride[0] + h * a->v_stride[1] + d * a->v_stride[2]),
+                        a->kv_v_scale[si]);
+                }
+            }
+        }
+        free(min_off), free(new_k), free(new_v);
+    }
     /* the new rows go into the cache first (:346-373): same dtype = bit copy, otherwise through fp32 */
-    for (size_t t = 0; t < a->token_count; ++t) {
+    for (size_t t = 0; !fp8 && t < a->token_count; ++t) {
         const uint32_t kv_slot = a->token_meta[t * a->meta_stride[0] + 2 * a->meta_stride[1]];
         const size_t base = (size_t)(kv_slot >> shift) * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] +
                             (size_t)(kv_slot & mask) * a->kv_stride[3];
@@ -3398,6 +3558,18 @@ int mo_paged_attention(const mo_paged_attention_args *a) {
                     }
                     const size_t base = (size_t)tb * a->kv_stride[0] + (size_t)a->layer_idx * a->kv_stride[1] +
                                         kvh * a->kv_stride[2] + (size_t)(p & mask) * a->kv_stride[3];
+                    if (fp8) { /* :474-498: the block's scales */
+                        const size_t si = (size_t)tb * a->scale_stride[0] + (size_t)a->layer_idx * a->scale_stride[1] +
+                                          kvh * a->scale_stride[2];
+                        for (size_t d = 0; d < hd; ++d) {
+                            k_block[k_count * hd + d] =
+                                pa_fp8_dequant(((const uint8_t *)a->kv_k)[base + d * a->kv_stride[4]], a->kv_k_scale[si]);
+                            v_block[k_count * hd + d] =
+                                pa_fp8_dequant(((const uint8_t *)a->kv_v)[base + d * a->kv_stride[4]], a->kv_v_scale[si]);
+                        }
+                        ++k_count;
+                        continue;
+                    }
                     for (size_t d = 0; d < hd; ++d) {
                         k_block[k_count * hd + d] = pa_load(a->kv_dtype, a->kv_k, base + d * a->kv_stride[4]);
                         v_block[k_count * hd + d] = pa_load(a->kv_dtype, a->kv_v, base + d * a->kv_stride[4]);

@@ -55,6 +55,7 @@ enum {
     MO_DTYPE_BF16 = 2,
     MO_DTYPE_I32 = 3,
     MO_DTYPE_I64 = 11,
+    MO_DTYPE_F8_E4M3 = 14,
 };
 
 enum {
@@ -247,9 +248,20 @@ typedef struct {
     size_t max_seqs, max_blocks_per_seq;
     void *out;
     size_t out_stride[3];
+    /* kv_dtype == MO_DTYPE_F8_E4M3 (paged_attention_ref.c:825-989): one fp32 scale per (block, layer, kv head) for keys
+     * and for values, [blocks, layers, kv heads] at scale_stride, read and updated: a block's scale is the largest
+     * magnitude among its rows below the first offset written by this call (decoded with the old scale) and the new
+     * rows, divided by 240; rows already in the block are re-encoded when the scale changes. */
+    float *kv_k_scale, *kv_v_scale;
+    size_t scale_stride[3];
 } mo_paged_attention_args;
 
 int mo_paged_attention(const mo_paged_attention_args *a);
+
+/* marmot_f32_to_fp8_e4m3_ref / marmot_fp8_e4m3_to_f32_ref (src/utils/dtype_ref.c:118-212): 1-4-3 bits, bias 7, exponent
+ * field 15 is NaN, largest finite value 240, round to nearest even, saturating. */
+uint8_t mo_f32_to_fp8_e4m3(float value);
+float mo_fp8_e4m3_to_f32(uint8_t bits);
 
 #ifdef __cplusplus
 }

@@ -34,6 +34,7 @@ BLOCK_BYTES = {KIND_Q4_0: 18, KIND_Q8_0: 34, KIND_Q4_K: 144, KIND_Q5_K: 176, KIN
                KIND_Q8_1: 36}
 DT_F32, DT_F16 = 0, 1
 DT_BF16 = 2
+DT_F8_E4M3 = 14
 DT_I32, DT_I64 = 3, 11  # marmot_dtype_t values of the position tensors the rotary epilogue accepts
 ROPE_SCALING_NONE, ROPE_SCALING_LINEAR, ROPE_SCALING_YARN, ROPE_SCALING_LONGROPE = 0, 1, 2, 3
 ROPE_TYPE_NORM, ROPE_TYPE_NEOX = 0, 1
@@ -52,7 +53,8 @@ class PagedAttentionArgs(C.Structure):
                 ("kv_blocks", C.c_size_t), ("kv_layers", C.c_size_t),
                 ("block_table", C.c_void_p), ("table_stride", C.c_size_t * 2),
                 ("max_seqs", C.c_size_t), ("max_blocks_per_seq", C.c_size_t),
-                ("out", C.c_void_p), ("out_stride", C.c_size_t * 3)]
+                ("out", C.c_void_p), ("out_stride", C.c_size_t * 3),
+                ("kv_k_scale", C.c_void_p), ("kv_v_scale", C.c_void_p), ("scale_stride", C.c_size_t * 3)]
 
 
 def float_dtype_code(a: np.ndarray, bf16: bool = False) -> int:
@@ -69,7 +71,7 @@ def element_strides(a: np.ndarray):
 
 
 def paged_attention_args(token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx, scale, act_bf16=False,
-                         kv_bf16=False, token_count=None, ptr=None):
+                         kv_bf16=False, token_count=None, ptr=None, kv_k_scale=None, kv_v_scale=None):
     """(PagedAttentionArgs over the given numpy arrays, freshly allocated out array). `ptr` maps an array to the
     address to put into the struct (default: the array's own memory)."""
     ptr = ptr or (lambda a: a.ctypes.data)
@@ -79,7 +81,15 @@ def paged_attention_args(token_meta, q, k_new, v_new, kv_k, kv_v, block_table, l
     a.token_count = q.shape[0] if token_count is None else token_count
     a.layer_idx, a.scale = layer_idx, scale
     a.num_q_heads, a.num_kv_heads, a.head_dim, a.block_size = q.shape[1], k_new.shape[1], q.shape[2], kv_k.shape[3]
-    a.act_dtype, a.kv_dtype = float_dtype_code(q, act_bf16), float_dtype_code(kv_k, kv_bf16)
+    a.act_dtype = float_dtype_code(q, act_bf16)
+    if kv_k.dtype == np.uint8:  # the FLOAT8_E4M3 cache with its per-block scales [blocks, layers, kv heads]
+        a.kv_dtype = DT_F8_E4M3
+        if kv_k_scale is not None:
+            assert kv_k_scale.dtype == np.float32 and kv_k_scale.strides == kv_v_scale.strides
+            a.kv_k_scale, a.kv_v_scale = ptr(kv_k_scale), ptr(kv_v_scale)
+            a.scale_stride = (C.c_size_t * 3)(*element_strides(kv_k_scale))
+    else:
+        a.kv_dtype = float_dtype_code(kv_k, kv_bf16)
     a.token_meta, a.meta_stride = ptr(token_meta), (C.c_size_t * 2)(*element_strides(token_meta))
     a.q, a.k_new, a.v_new = ptr(q), ptr(k_new), ptr(v_new)
     a.q_stride = (C.c_size_t * 3)(*element_strides(q))
@@ -191,6 +201,10 @@ class Oracle:
             C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_void_p,
             C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
         ]
+        L.mo_f32_to_fp8_e4m3.restype = C.c_uint8
+        L.mo_f32_to_fp8_e4m3.argtypes = [C.c_float]
+        L.mo_fp8_e4m3_to_f32.restype = C.c_float
+        L.mo_fp8_e4m3_to_f32.argtypes = [C.c_uint8]
         L.mo_paged_attention.restype = C.c_int
         L.mo_paged_attention.argtypes = [C.POINTER(PagedAttentionArgs)]
         L.mo_row_grain.restype = C.c_size_t
@@ -294,12 +308,14 @@ class Oracle:
         return out
 
     def paged_attention(self, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx: int, scale: float,
-                        act_bf16: bool = False, kv_bf16: bool = False, token_count=None):
+                        act_bf16: bool = False, kv_bf16: bool = False, token_count=None, kv_k_scale=None,
+                        kv_v_scale=None):
         """marmot_paged_attention: kv_k / kv_v ([blocks, layers, kv heads, block size, head dim]) are updated in place;
         q / k_new / v_new are [tokens, heads, head dim] arrays (views with any strides) of float32, float16, or uint16
-        holding bfloat16 bits (act_bf16 / kv_bf16). Returns (status, out)."""
+        holding bfloat16 bits (act_bf16 / kv_bf16); a uint8 cache is FLOAT8_E4M3 with its float32 scale tensors
+        [blocks, layers, kv heads], updated in place too. Returns (status, out)."""
         args, out = paged_attention_args(token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx, scale, act_bf16,
-                                         kv_bf16, token_count)
+                                         kv_bf16, token_count, kv_k_scale=kv_k_scale, kv_v_scale=kv_v_scale)
         st = self.L.mo_paged_attention(C.byref(args))
         return st, out
 

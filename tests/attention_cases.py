@@ -105,3 +105,60 @@ def dense_reference(case, kv_k, kv_v) -> np.ndarray:
 
 
 TOLERANCE = {"f32": 2e-5, "f16": 1.5e-3, "bf16": 1.2e-2}  # of the largest |v|: fp32 accumulation, one output rounding
+
+
+# ---------------------------------------------------------------- the FLOAT8_E4M3 cache
+def fp8_values() -> np.ndarray:
+    """The 256 codes of the reference's e4m3 (1-4-3 bits, bias 7, exponent field 15 = NaN, largest finite 240),
+    from the format's definition."""
+    code = np.arange(256)
+    field, mant = (code >> 3) & 15, code & 7
+    mag = np.where(field == 0, mant / 8.0 * 2.0 ** -6, (1 + mant / 8.0) * 2.0 ** (field.astype(np.float64) - 7))
+    val = np.where(code & 0x80, -mag, mag)
+    return np.where(field == 15, np.nan, val)
+
+
+def fp8_encode(x: np.ndarray) -> np.ndarray:
+    """Nearest representable value, ties to the even mantissa, saturating at 240 -- found by searching the table of
+    magnitudes (no exponent arithmetic), for float32 input; one quirk of the reference is kept (below)."""
+    x = np.asarray(x, dtype=np.float32)
+    table = fp8_values()[:0x78]  # non-negative finite codes 0 .. 0x77, ascending
+    mag = np.abs(x).astype(np.float64)
+    hi = np.clip(np.searchsorted(table, mag, side="left"), 0, 0x77)
+    lo = np.clip(hi - 1, 0, 0x77)
+    d_lo, d_hi = mag - table[lo], table[hi] - mag
+    pick = np.where(d_lo < d_hi, lo, np.where(d_hi < d_lo, hi, np.where(lo % 2 == 0, lo, hi)))
+    pick = np.where(mag >= 240.0, 0x77, pick)
+    # the reference never rounds a magnitude below the smallest normal 2^-6 up into the normal range: it clamps the
+    # subnormal mantissa to 7 (src/utils/dtype_ref.c:166-174)
+    pick = np.where(mag < 2.0 ** -6, np.minimum(pick, 7), pick)
+    return (pick | np.where(x < 0, 0x80, 0)).astype(np.uint8)  # the sign of a negative value; -0.0 encodes as +0
+
+
+def fp8_cache_update(case, kv, scales):
+    """What one call does to an fp8 cache and its scales [blocks, layers, kv heads], for keys or values alike
+    (`kv` = (cache, new rows as float32)): per touched block and head, scale = max(largest decoded magnitude among the
+    rows below the first offset written, largest new magnitude) / 240 (1 when that is 0); rows already there are
+    re-encoded when the scale changes; the new rows are encoded with it."""
+    cache, new = kv
+    cache, scales = cache.copy(), scales.copy()
+    bs, layer = case["block_size"], case["layer_idx"]
+    values = fp8_values().astype(np.float32)
+    slots = case["token_meta"][:, 2].astype(np.int64)
+    for b in np.unique(slots // bs):
+        toks = np.nonzero(slots // bs == b)[0]
+        existing = int((slots[toks] % bs).min())
+        for h in range(cache.shape[2]):
+            old = np.float32(scales[b, layer, h])
+            big = np.float32(0.0)
+            if existing > 0 and old > 0:
+                big = np.abs(values[cache[b, layer, h, :existing]] * old).max()
+            big = max(big, np.abs(new[toks, h]).max())
+            scale = np.float32(big) / np.float32(240.0) if big > 0 else np.float32(1.0)
+            if existing > 0 and scale != old:
+                dec = values[cache[b, layer, h, :existing]] * old if old > 0 else np.zeros((existing, cache.shape[4]), np.float32)
+                cache[b, layer, h, :existing] = fp8_encode(dec.astype(np.float32) / scale)
+            scales[b, layer, h] = scale
+            for t in toks:
+                cache[b, layer, h, slots[t] % bs] = fp8_encode(new[t, h].astype(np.float32) / scale)
+    return cache, scales

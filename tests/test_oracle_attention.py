@@ -99,3 +99,97 @@ def test_argument_errors(oracle):
     three = dict(case, q=np.zeros((2, 3, 8), np.float32))
     assert run(oracle, three)[0] == MO_INVALID  # 3 query heads over 2 kv heads (:590-595)
     assert run(oracle, case, token_count=0)[0] == 0
+
+
+# ---------------------------------------------------------------- the FLOAT8_E4M3 cache
+def test_fp8_e4m3_conversions(oracle):
+    """The reference's e4m3 (src/utils/dtype_ref.c:118-212) against the format's definition: every code decodes to the
+    value its fields say; encoding is the nearest code by table search with ties to the even mantissa, saturation at
+    240 and the reference's clamp below the smallest normal; encode(decode(code)) is the code."""
+    from tests.attention_cases import fp8_encode, fp8_values
+
+    vals = fp8_values()
+    dec = np.array([oracle.L.mo_fp8_e4m3_to_f32(c) for c in range(256)], dtype=np.float64)
+    assert np.array_equal(np.isnan(dec), np.isnan(vals)) and np.array_equal(dec[~np.isnan(dec)], vals[~np.isnan(vals)])
+    finite = [c for c in range(256) if not np.isnan(vals[c])]
+    # encode(decode(code)) == code, except that -0.0 encodes as +0 (the sign is taken from `value < 0`)
+    assert all(oracle.L.mo_f32_to_fp8_e4m3(float(vals[c])) == (0 if c == 0x80 else c) for c in finite)
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(4000).astype(np.float32) * np.float32(s) for s in (0.001, 0.02, 1, 30, 300)])
+    mids = ((vals[:0x77] + vals[1:0x78]) / 2).astype(np.float32)  # exact midpoints: ties
+    x = np.concatenate([x, mids, -mids, np.array([0.0, -0.0, 240, 241, 1e9, -1e9, 2.0 ** -6, 2.0 ** -10], np.float32)])
+    enc = np.array([oracle.L.mo_f32_to_fp8_e4m3(float(v)) for v in x], dtype=np.uint8)
+    assert np.array_equal(enc, fp8_encode(x))
+    assert oracle.L.mo_f32_to_fp8_e4m3(float("nan")) == 0x79 and oracle.L.mo_f32_to_fp8_e4m3(float("inf")) == 0x77
+
+
+def _fp8_case(seed, seqs, **kw):
+    """An empty fp8 cache (codes 0, scales 0) and a call that fills it."""
+    case = make_case(seed, seqs, act="f32", kv="f32", **kw)
+    shape = case["kv_k"].shape
+    case["kv_k"], case["kv_v"] = np.zeros(shape, np.uint8), np.zeros(shape, np.uint8)
+    case["k_scale"], case["v_scale"] = np.zeros(shape[:3], np.float32), np.zeros(shape[:3], np.float32)
+    case["kv"] = "fp8"
+    return case
+
+
+def run_fp8(oracle, case):
+    kv_k, kv_v, ks, vs = (case[n].copy() for n in ("kv_k", "kv_v", "k_scale", "v_scale"))
+    st, out = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], kv_k, kv_v,
+                                     case["block_table"], case["layer_idx"], case["scale"], kv_k_scale=ks, kv_v_scale=vs)
+    return st, out, kv_k, kv_v, ks, vs
+
+
+def fp8_dense(case, kv_k, kv_v, ks, vs):
+    """Dense float64 attention over the decoded cache (code value x block scale)."""
+    from tests.attention_cases import fp8_values
+
+    vals = fp8_values().astype(np.float32)
+    dk = vals[kv_k] * ks[:, :, :, None, None]
+    dv = vals[kv_v] * vs[:, :, :, None, None]
+    return dense_reference(dict(case, kv="f32"), dk.astype(np.float32), dv.astype(np.float32)), dv
+
+
+def test_fp8_cache_prefill_then_decode_with_growing_scales(oracle):
+    """Call 1 fills blocks from empty (scales 0 -> max / 240); call 2 appends one louder token per sequence into
+    partly filled blocks: the scale grows and the rows already there are re-encoded; a quieter token leaves scale and
+    bytes alone. Cache bytes and scales against the independent numpy statement, attention against dense float64
+    attention over the decoded cache."""
+    from tests.attention_cases import fp8_cache_update
+
+    case = _fp8_case(31, [(0, 21), (0, 9), (0, 40)], num_q_heads=4, num_kv_heads=2, head_dim=32, block_size=16, layers=2,
+                     layer_idx=1)
+    st, out, kv_k, kv_v, ks, vs = run_fp8(oracle, case)
+    assert st == 0
+    want_k, want_ks = fp8_cache_update(case, (case["kv_k"], case["k_new"]), case["k_scale"])
+    want_v, want_vs = fp8_cache_update(case, (case["kv_v"], case["v_new"]), case["v_scale"])
+    assert np.array_equal(kv_k, want_k) and np.array_equal(ks, want_ks)
+    assert np.array_equal(kv_v, want_v) and np.array_equal(vs, want_vs)
+    ref, dv = fp8_dense(case, kv_k, kv_v, ks, vs)
+    assert np.max(np.abs(out - ref)) <= TOLERANCE["f32"] * np.abs(dv).max()
+    # call 2: one token per sequence at the next position; sequence 0 louder (x4), sequence 1 quieter (x0.25)
+    bs = case["block_size"]
+    seqs = sorted(set(int(s) for s in case["token_meta"][:, 0]))
+    nxt = {s: int(case["token_meta"][case["token_meta"][:, 0] == s, 1].max()) + 1 for s in seqs}
+    meta = np.array([[s, nxt[s], int(case["block_table"][s, nxt[s] // bs]) * bs + nxt[s] % bs, 0] for s in seqs], np.uint32)
+    rng = np.random.default_rng(32)
+    gain = np.array([4.0, 0.25, 1.0], np.float32)[:, None, None]
+    step = dict(case, token_meta=meta, q=rng.standard_normal((3, 4, 32), dtype=np.float32),
+                k_new=rng.standard_normal((3, 2, 32), dtype=np.float32) * gain,
+                v_new=rng.standard_normal((3, 2, 32), dtype=np.float32) * gain,
+                kv_k=kv_k, kv_v=kv_v, k_scale=ks, v_scale=vs)
+    st, out2, k2, v2, ks2, vs2 = run_fp8(oracle, step)
+    assert st == 0
+    want_k2, want_ks2 = fp8_cache_update(step, (kv_k, step["k_new"]), ks)
+    want_v2, want_vs2 = fp8_cache_update(step, (kv_v, step["v_new"]), vs)
+    assert np.array_equal(k2, want_k2) and np.array_equal(ks2, want_ks2)
+    assert np.array_equal(v2, want_v2) and np.array_equal(vs2, want_vs2)
+    b_loud, b_quiet = int(meta[0, 2]) // bs, int(meta[1, 2]) // bs
+    assert (ks2[b_loud, 1] > ks[b_loud, 1]).all() and not np.array_equal(k2[b_loud, 1, :, :nxt[seqs[0]] % bs], kv_k[b_loud, 1, :, :nxt[seqs[0]] % bs])
+    assert np.array_equal(ks2[b_quiet, 1], ks[b_quiet, 1])
+    ref2, dv2 = fp8_dense(step, k2, v2, ks2, vs2)
+    assert np.max(np.abs(out2 - ref2)) <= TOLERANCE["f32"] * np.abs(dv2).max()
+    # the scale tensors are required with an fp8 cache (paged_attention_ref.c:695-698)
+    st, _ = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], case["kv_k"].copy(),
+                                   case["kv_v"].copy(), case["block_table"], 1, case["scale"])
+    assert st == MO_INVALID

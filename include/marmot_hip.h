@@ -65,6 +65,7 @@ enum {
     MARMOT_HIP_DTYPE_I32 = 3,  /* position tensors of the rotary epilogue only */
     MARMOT_HIP_DTYPE_U8 = 6,   /* storage type of block-quantized tensors (GGUF reader) */
     MARMOT_HIP_DTYPE_I64 = 11,
+    MARMOT_HIP_DTYPE_F8_E4M3 = 14, /* paged attention only: the KV cache with per-block scales */
 };
 
 /* marmot_router_weight_policy_t (include/marmot/types.h:283-288), marmot_ffn_type_t (:276-281) */
@@ -358,7 +359,7 @@ int marmot_hip_rope(marmot_hip_device_t *dev, const void *d_x, int dtype, size_t
 /* ------------------------------------------------------------------ paged attention
  * Replaces cpu_paged_attention_impl (src/backends/cpu/ops/paged_attention/paged_attention_ref.c:573-1082; descriptor
  * marmot_paged_attention_desc_t, include/marmot/ops/paged_attention.h:32-57) for FLOAT32 / FLOAT16 / BFLOAT16
- * activations and KV caches (the FP8 cache of MARMOT_ENABLE_FP8 builds is not offered). The tensors of the descriptor
+ * activations and FLOAT32 / FLOAT16 / BFLOAT16 / FLOAT8_E4M3 KV caches. The tensors of the descriptor
  * arrive as device pointers with their strides in elements:
  *   d_token_meta  [token_count, 4] uint32: seq_slot, pos, kv_slot, flags (flags are not read)
  *   d_q, d_out    [tokens, num_q_heads, head_dim], d_k_new, d_v_new [tokens, num_kv_heads, head_dim] of act_dtype
@@ -387,6 +388,13 @@ typedef struct marmot_hip_paged_attention {
     size_t max_seqs, max_blocks_per_seq;
     void *d_out;
     size_t out_stride[3];
+    /* kv_dtype == MARMOT_HIP_DTYPE_F8_E4M3 (paged_attention_ref.c:825-989): fp32 scales [kv_blocks, kv_layers,
+     * num_kv_heads] for keys and for values at scale_stride, read and updated. A block's scale becomes the largest
+     * magnitude among its rows below the first offset this call writes (decoded with the old scale) and the new rows,
+     * divided by 240; rows already in the block are re-encoded when the scale changes; bytes and scales equal the
+     * reference's bit for bit (its e4m3: bias 7, exponent field 15 = NaN, src/utils/dtype_ref.c:118-212). */
+    float *d_kv_k_scale, *d_kv_v_scale;
+    size_t scale_stride[3];
 } marmot_hip_paged_attention_t;
 int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot_hip_paged_attention_t *args, int validate_meta);
 

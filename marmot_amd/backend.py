@@ -508,7 +508,8 @@ class HipBackend:
                 b.free()
 
     def paged_attention_args(self, dev_ptr, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out, layer_idx: int,
-                             scale: float, act_bf16: bool = False, kv_bf16: bool = False, token_count=None):
+                             scale: float, act_bf16: bool = False, kv_bf16: bool = False, token_count=None,
+                             kv_k_scale=None, kv_v_scale=None):
         """marmot_hip_paged_attention_t over numpy arrays (shapes, dtypes and element strides) whose device addresses
         dev_ptr(array) gives; bfloat16 tensors travel as uint16 bits."""
         def code(a, bf16):
@@ -524,7 +525,15 @@ class HipBackend:
         p.token_count = q.shape[0] if token_count is None else token_count
         p.layer_idx, p.scale = layer_idx, scale
         p.num_q_heads, p.num_kv_heads, p.head_dim, p.block_size = q.shape[1], k_new.shape[1], q.shape[2], kv_k.shape[3]
-        p.act_dtype, p.kv_dtype = code(q, act_bf16), code(kv_k, kv_bf16)
+        p.act_dtype = code(q, act_bf16)
+        if kv_k.dtype == np.uint8:  # FLOAT8_E4M3 cache with float32 scales [blocks, layers, kv heads]
+            p.kv_dtype = capi.DT_F8_E4M3
+        else:
+            p.kv_dtype = code(kv_k, kv_bf16)
+        if kv_k_scale is not None:
+            assert kv_k_scale.dtype == np.float32 and kv_k_scale.strides == kv_v_scale.strides
+            p.d_kv_k_scale, p.d_kv_v_scale = dev_ptr(kv_k_scale), dev_ptr(kv_v_scale)
+            p.scale_stride = (C.c_size_t * 3)(*strides(kv_k_scale))
         p.d_token_meta, p.meta_stride = dev_ptr(token_meta), (C.c_size_t * 2)(*strides(token_meta))
         p.d_q, p.d_k_new, p.d_v_new = dev_ptr(q), dev_ptr(k_new), dev_ptr(v_new)
         p.q_stride = (C.c_size_t * 3)(*strides(q))
@@ -538,14 +547,19 @@ class HipBackend:
         return p
 
     def paged_attention(self, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, layer_idx: int, scale: float,
-                        act_bf16: bool = False, kv_bf16: bool = False, token_count=None, validate: bool = True):
+                        act_bf16: bool = False, kv_bf16: bool = False, token_count=None, validate: bool = True,
+                        kv_k_scale=None, kv_v_scale=None):
         """marmot_paged_attention (include/marmot/ops/paged_attention.h; CPU implementation
         src/backends/cpu/ops/paged_attention/paged_attention_ref.c): token_meta [tokens, 4] uint32 (seq_slot, pos,
         kv_slot, flags), q [tokens, q heads, head dim], k_new / v_new [tokens, kv heads, head dim] (float32, float16 or
         uint16 holding bfloat16 bits; views with any strides), kv_k / kv_v [blocks, layers, kv heads, block size, head
-        dim] (updated in place), block_table [sequences, blocks per sequence] uint32. Returns out like q."""
+        dim] (updated in place; uint8 = FLOAT8_E4M3 with the float32 scale tensors kv_k_scale / kv_v_scale [blocks,
+        layers, kv heads], updated in place too), block_table [sequences, blocks per sequence] uint32. Returns out
+        like q."""
         out = np.zeros(q.shape, dtype=q.dtype)
         arrays = [token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out]
+        scales = [a for a in (kv_k_scale, kv_v_scale) if a is not None]
+        arrays += scales
         roots = {}
 
         def root_of(a):
@@ -564,10 +578,10 @@ class HipBackend:
             return d.ptr + (a.ctypes.data - r.ctypes.data)
 
         p = self.paged_attention_args(dev_ptr, token_meta, q, k_new, v_new, kv_k, kv_v, block_table, out, layer_idx,
-                                      scale, act_bf16, kv_bf16, token_count)
+                                      scale, act_bf16, kv_bf16, token_count, kv_k_scale, kv_v_scale)
         try:
             check(self.lib.marmot_hip_paged_attention(self.dev, C.byref(p), 1 if validate else 0))
-            for a in (kv_k, kv_v, out):
+            for a in [kv_k, kv_v, out] + scales:
                 r, d = roots[id(root_of(a))]
                 flat = r.reshape(-1).view(np.uint8)
                 flat[...] = d.download(np.uint8, (flat.size,))

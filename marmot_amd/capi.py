@@ -12,6 +12,7 @@ KIND_Q2_K, KIND_Q3_K = 7, 8
 KIND_Q8_1 = 6
 DT_F32, DT_F16 = 0, 1
 DT_BF16 = 2  # paged attention only
+DT_F8_E4M3 = 14  # paged attention only: the KV cache
 DT_I32, DT_I64 = 3, 11  # position tensors of the rotary epilogue
 FLAG_FORCE_PACK = 1
 
@@ -57,7 +58,8 @@ class PagedAttention(C.Structure):
                 ("kv_blocks", C.c_size_t), ("kv_layers", C.c_size_t),
                 ("d_block_table", C.c_void_p), ("table_stride", C.c_size_t * 2),
                 ("max_seqs", C.c_size_t), ("max_blocks_per_seq", C.c_size_t),
-                ("d_out", C.c_void_p), ("out_stride", C.c_size_t * 3)]
+                ("d_out", C.c_void_p), ("out_stride", C.c_size_t * 3),
+                ("d_kv_k_scale", C.c_void_p), ("d_kv_v_scale", C.c_void_p), ("scale_stride", C.c_size_t * 3)]
 
 
 class GgufTensor(C.Structure):

@@ -39,6 +39,10 @@ struct PaParams {
     uint32_t shift, mask, group;
     int q_vec, kv_vec;  // 16-byte loads of the query / of the cache rows
     int *flag;          // metadata check: 1 + index of an offending token (maximum)
+    float *k_scale, *v_scale;  // FLOAT8_E4M3 cache: scales [blocks][layers][kv heads] at scale_stride
+    size_t scale_stride[3];
+    uint32_t *new_kmax, *new_vmax;  // scratch [blocks][kv heads]: largest new magnitudes as float bits
+    uint32_t *min_off;              // scratch [blocks]: first offset this call writes (block_size = untouched)
     uint32_t splits;    // workgroups along the history of one (token, heads) pair
     float *partial;     // splits > 1: [token][query head][split][2 + head_dim]: maximum, sum, unnormalized output
 };
@@ -52,7 +56,66 @@ __device__ __forceinline__ float pa_bf2f(uint16_t h) {
     return __uint_as_float((uint32_t)h << 16);
 }
 
+// The reference's e4m3 (marmot_fp8_dequantize / marmot_fp8_quantize with 4 exponent bits, 3 mantissa bits, bias 7,
+// no infinity, largest finite value 240: src/utils/dtype_ref.c:118-212).
+__device__ __forceinline__ float pa_fp8_to_f32(uint32_t c) {
+    const uint32_t field = (c >> 3) & 15u, mant = c & 7u, sign = (c & 0x80u) << 24;
+    if (field == 15u) {
+        return __uint_as_float(0x7fc00000u);
+    }
+    if (field == 0u) {
+        return __uint_as_float(__float_as_uint((float)mant * 0.001953125f) | sign);  // mant / 8 * 2^-6
+    }
+    return __uint_as_float(sign | ((field + 120u) << 23) | (mant << 20));  // (1 + mant / 8) * 2^(field - 7)
+}
+
+__device__ __forceinline__ uint32_t pa_f32_to_fp8(float value) {
+    if (value != value) {
+        return 0x79u;
+    }
+    const uint32_t sign = value < 0.0f ? 0x80u : 0u;
+    const float mag = fabsf(value);
+    if (mag > 240.0f) {  // infinity included
+        return sign | 0x77u;
+    }
+    if (mag == 0.0f) {
+        return sign;
+    }
+    int e;
+    float m = frexpf(mag, &e);  // mag = m * 2^e, m in [0.5, 1)
+    m *= 2.0f;
+    e -= 1;
+    int field = e + 7;
+    if (field > 0 && field < 15) {
+        int r = (int)rintf((m - 1.0f) * 8.0f);  // nearest, ties to even
+        if (r == 8) {
+            r = 0;
+            field += 1;
+            if (field >= 15) {
+                return sign | 0x77u;
+            }
+        }
+        return sign | ((uint32_t)field << 3) | (uint32_t)(r & 7);
+    }
+    int r = (int)rintf(ldexpf(mag, 9));  // below the smallest normal 2^-6: multiples of 2^-9, never rounded up into
+    if (r == 0) {                        // the normal range
+        return sign;
+    }
+    return sign | (uint32_t)(r > 7 ? 7 : r);
+}
+
+// cpu_paged_attention_fp8_quant / _dequant / _scale_from_max (paged_attention_ref.c:142-163)
+__device__ __forceinline__ uint32_t pa_fp8_quant(float value, float scale) {
+    return scale > 0.0f ? pa_f32_to_fp8(value / scale) : 0u;
+}
+__device__ __forceinline__ float pa_fp8_dequant(uint32_t c, float scale) {
+    return scale > 0.0f ? pa_fp8_to_f32(c) * scale : 0.0f;
+}
+
 __device__ __forceinline__ float pa_load(const void *data, int dtype, size_t i) {
+    if (dtype == MARMOT_HIP_DTYPE_F8_E4M3) {  // the code's value; the caller applies the block's scale
+        return pa_fp8_to_f32(((const uint8_t *)data)[i]);
+    }
     if (dtype == MARMOT_HIP_DTYPE_F16) {
         return h2f(((const uint16_t *)data)[i]);
     }
@@ -81,7 +144,22 @@ __device__ __forceinline__ float pa_exp(float x) {
 // EPL consecutive values starting at element `first` (unit stride, 16-byte aligned start for the storage type)
 template <int EPL>
 __device__ __forceinline__ void pa_load_run(const void *data, int dtype, size_t first, float (&v)[EPL]) {
-    if (dtype == MARMOT_HIP_DTYPE_F32) {
+    if (dtype == MARMOT_HIP_DTYPE_F8_E4M3) {
+        uint32_t w[EPL / 4];
+        if constexpr (EPL == 4) {
+            w[0] = *(const uint32_t *)((const uint8_t *)data + first);
+        } else if constexpr (EPL == 8) {
+            const uint2 u = *(const uint2 *)((const uint8_t *)data + first);
+            w[0] = u.x, w[1] = u.y;
+        } else {
+            const uint4 u = *(const uint4 *)((const uint8_t *)data + first);
+            w[0] = u.x, w[1] = u.y, w[2] = u.z, w[3] = u.w;
+        }
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            v[e] = pa_fp8_to_f32((w[e / 4] >> (8 * (e % 4))) & 0xffu);
+        }
+    } else if (dtype == MARMOT_HIP_DTYPE_F32) {
 #pragma unroll
         for (int e = 0; e < EPL; e += 4) {
             const float4 f = *(const float4 *)((const float *)data + first + e);
@@ -150,6 +228,124 @@ __global__ __launch_bounds__(128) void k_pa_write(const PaParams p) {
     }
 }
 
+// ---- the FLOAT8_E4M3 cache write (paged_attention_ref.c:825-989) in four launches
+// 1. scratch: no new magnitudes, no block touched
+__global__ __launch_bounds__(256) void k_pa_fp8_init(const PaParams p) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < p.kv_blocks * p.num_kv_heads) {
+        p.new_kmax[i] = 0u;
+        p.new_vmax[i] = 0u;
+    }
+    if (i < p.kv_blocks) {
+        p.min_off[i] = p.block_size;
+    }
+}
+
+__device__ __forceinline__ float pa_block_max(float v, float *red) {  // maximum over a workgroup of 128 threads
+    red[threadIdx.x] = v;
+    __syncthreads();
+    for (int s = 64; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) {
+            red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+        }
+        __syncthreads();
+    }
+    const float r = red[0];
+    __syncthreads();
+    return r;
+}
+
+// 2. per (token, kv head): the largest magnitudes of the new key and value rows into their block's entry (non-negative
+//    floats order like their bits), and the first offset written in the block
+__global__ __launch_bounds__(128) void k_pa_fp8_scan_new(const PaParams p) {
+    __shared__ float red[128];
+    const uint32_t t = blockIdx.x, h = blockIdx.y;
+    const uint32_t slot = p.meta[t * p.meta_stride[0] + 2 * p.meta_stride[1]];
+    const uint32_t block = slot >> p.shift;
+    if (block >= p.kv_blocks) {
+        return;
+    }
+    float km = 0.0f, vm = 0.0f;
+    for (uint32_t d = threadIdx.x; d < p.head_dim; d += 128u) {
+        km = fmaxf(km, fabsf(pa_load(p.k_new, p.act_dtype, (size_t)t * p.k_stride[0] + (size_t)h * p.k_stride[1] + d * p.k_stride[2])));
+        vm = fmaxf(vm, fabsf(pa_load(p.v_new, p.act_dtype, (size_t)t * p.v_stride[0] + (size_t)h * p.v_stride[1] + d * p.v_stride[2])));
+    }
+    km = pa_block_max(km, red);
+    vm = pa_block_max(vm, red);
+    if (threadIdx.x == 0) {
+        atomicMax(p.new_kmax + (size_t)block * p.num_kv_heads + h, __float_as_uint(km));
+        atomicMax(p.new_vmax + (size_t)block * p.num_kv_heads + h, __float_as_uint(vm));
+        if (h == 0) {
+            atomicMin(p.min_off + block, slot & p.mask);
+        }
+    }
+}
+
+// 3. per (touched block, kv head): the new scale; rows already in the block are re-encoded when it changes. The token
+//    that writes the block's first new row does the block's work, so the launch grows with the call, not the cache.
+__global__ __launch_bounds__(128) void k_pa_fp8_rescale(const PaParams p) {
+    __shared__ float red[128];
+    const uint32_t t = blockIdx.x, h = blockIdx.y;
+    const uint32_t slot = p.meta[t * p.meta_stride[0] + 2 * p.meta_stride[1]];
+    const uint32_t b = slot >> p.shift;
+    if (b >= p.kv_blocks) {
+        return;
+    }
+    const uint32_t existing = p.min_off[b];
+    if ((slot & p.mask) != existing) {
+        return;
+    }
+    const size_t si = (size_t)b * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] + (size_t)h * p.scale_stride[2];
+    const size_t base = (size_t)b * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2];
+    const uint32_t cells = existing * p.head_dim;
+    for (int which = 0; which < 2; ++which) {
+        uint8_t *cache = (uint8_t *)(which ? p.kv_v : p.kv_k);
+        float *scales = which ? p.v_scale : p.k_scale;
+        const float old_scale = scales[si];
+        float big = 0.0f;
+        if (existing > 0 && old_scale > 0.0f) {
+            for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
+                const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
+                big = fmaxf(big, fabsf(pa_fp8_dequant(cache[base + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4]], old_scale)));
+            }
+        }
+        big = pa_block_max(big, red);
+        big = fmaxf(big, __uint_as_float((which ? p.new_vmax : p.new_kmax)[(size_t)b * p.num_kv_heads + h]));
+        const float new_scale = big > 0.0f ? big / 240.0f : 1.0f;
+        if (existing > 0 && new_scale != old_scale) {
+            for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
+                const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
+                uint8_t *cell = cache + base + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
+                *cell = (uint8_t)pa_fp8_quant(pa_fp8_dequant(*cell, old_scale), new_scale);
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            scales[si] = new_scale;
+        }
+    }
+}
+
+// 4. per (token, kv head): the new rows, encoded with their block's scale
+__global__ __launch_bounds__(128) void k_pa_fp8_store(const PaParams p) {
+    const uint32_t t = blockIdx.x, h = blockIdx.y;
+    const uint32_t slot = p.meta[t * p.meta_stride[0] + 2 * p.meta_stride[1]];
+    const uint32_t block = slot >> p.shift;
+    if (block >= p.kv_blocks) {
+        return;
+    }
+    const size_t si = (size_t)block * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] + (size_t)h * p.scale_stride[2];
+    const float ks = p.k_scale[si], vs = p.v_scale[si];
+    const size_t dst0 = (size_t)block * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2] +
+                        (size_t)(slot & p.mask) * p.kv_stride[3];
+    for (uint32_t d = threadIdx.x; d < p.head_dim; d += 128u) {
+        const float kx = pa_load(p.k_new, p.act_dtype, (size_t)t * p.k_stride[0] + (size_t)h * p.k_stride[1] + d * p.k_stride[2]);
+        const float vx = pa_load(p.v_new, p.act_dtype, (size_t)t * p.v_stride[0] + (size_t)h * p.v_stride[1] + d * p.v_stride[2]);
+        ((uint8_t *)p.kv_k)[dst0 + d * p.kv_stride[4]] = (uint8_t)pa_fp8_quant(kx, ks);
+        ((uint8_t *)p.kv_v)[dst0 + d * p.kv_stride[4]] = (uint8_t)pa_fp8_quant(vx, vs);
+    }
+}
+
 // ---- attention (cpu_paged_attention_attention_range, :398-569)
 // One workgroup of 16 groups of 16 lanes per (token, QH query heads that share a key / value head): every key and
 // value row is fetched, converted and located once for the QH heads. A group takes two positions per step and
@@ -203,7 +399,8 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
     const size_t head_base = (size_t)p.layer_idx * p.kv_stride[1] + (size_t)kvh * p.kv_stride[2];
     const uint32_t *table_row = p.table + (size_t)seq * p.table_stride[0];
     // the cache row of position pp, or false when the position has no block (beyond the table, or a hole)
-    auto locate = [&](uint32_t pp, size_t &base) -> bool {
+    const bool fp8 = p.kv_dtype == MARMOT_HIP_DTYPE_F8_E4M3;
+    auto locate = [&](uint32_t pp, size_t &base, uint32_t &tb_out) -> bool {
         if (pp >= kv_len) {
             return false;
         }
@@ -216,9 +413,10 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
             return false;
         }
         base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(pp & p.mask) * p.kv_stride[3];
+        tb_out = tb;
         return true;
     };
-    auto fetch = [&](size_t base, float (&kr)[EPL], float (&vr)[EPL]) {
+    auto fetch = [&](size_t base, uint32_t tb, float (&kr)[EPL], float (&vr)[EPL]) {
         if (p.kv_vec) {
             pa_load_run<EPL>(p.kv_k, p.kv_dtype, base + d0, kr);
             pa_load_run<EPL>(p.kv_v, p.kv_dtype, base + d0, vr);
@@ -229,6 +427,16 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
                 const size_t i = base + (size_t)(d0 + e) * p.kv_stride[4];
                 kr[e] = in ? pa_load(p.kv_k, p.kv_dtype, i) : 0.0f;
                 vr[e] = in ? pa_load(p.kv_v, p.kv_dtype, i) : 0.0f;
+            }
+        }
+        if (fp8) {  // code value times the block's scale: the reference's decoded element (:474-498)
+            const size_t si = (size_t)tb * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] +
+                              (size_t)kvh * p.scale_stride[2];
+            const float ks = p.k_scale[si], vs = p.v_scale[si];
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                kr[e] = ks > 0.0f ? kr[e] * ks : 0.0f;
+                vr[e] = vs > 0.0f ? vr[e] * vs : 0.0f;
             }
         }
     };
@@ -264,13 +472,14 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
     const uint32_t stop = first + chunk < kv_len ? first + chunk : kv_len;
     for (uint32_t pp = first + (uint32_t)g; pp < stop; pp += 2u * PA_GROUPS) {
         size_t base0 = 0, base1 = 0;
-        const bool have0 = locate(pp, base0), have1 = pp + PA_GROUPS < stop && locate(pp + PA_GROUPS, base1);
+        uint32_t tb0 = 0, tb1 = 0;
+        const bool have0 = locate(pp, base0, tb0), have1 = pp + PA_GROUPS < stop && locate(pp + PA_GROUPS, base1, tb1);
         float k0[EPL], v0[EPL], k1[EPL], v1[EPL];
         if (have0) {
-            fetch(base0, k0, v0);
+            fetch(base0, tb0, k0, v0);
         }
         if (have1) {
-            fetch(base1, k1, v1);
+            fetch(base1, tb1, k1, v1);
         }
         if (have0) {
             absorb(k0, v0);
@@ -368,7 +577,7 @@ static bool pa_float_dtype(int d) {
 }
 
 static size_t pa_elem_size(int d) {
-    return d == MARMOT_HIP_DTYPE_F32 ? 4 : 2;
+    return d == MARMOT_HIP_DTYPE_F32 ? 4 : (d == MARMOT_HIP_DTYPE_F8_E4M3 ? 1 : 2);
 }
 
 } // namespace mh
@@ -399,8 +608,15 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     if (a->num_q_heads % a->num_kv_heads != 0) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention requires num_q_heads divisible by num_kv_heads");
     }
-    if (!pa_float_dtype(a->act_dtype) || !pa_float_dtype(a->kv_dtype)) {
+    const bool fp8 = a->kv_dtype == MARMOT_HIP_DTYPE_F8_E4M3;
+    if (!pa_float_dtype(a->act_dtype) || (!fp8 && !pa_float_dtype(a->kv_dtype))) {
         return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "paged_attention dtype not supported");
+    }
+    if (fp8 && (a->d_kv_k_scale == nullptr || a->d_kv_v_scale == nullptr)) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention FP8 KV requires scale tensors");
+    }
+    if (!fp8 && (a->d_kv_k_scale != nullptr || a->d_kv_v_scale != nullptr)) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "paged_attention scale tensors require FP8 KV");
     }
     if (a->kv_layers <= a->layer_idx) {
         return set_error(MARMOT_HIP_ERROR_DIMENSION_MISMATCH, "paged_attention layer_idx out of range");
@@ -448,6 +664,11 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     for (int i = 0; i < 4 && p.kv_vec; ++i) {
         p.kv_vec = (a->kv_stride[i] * ksz) % run_k == 0;
     }
+    p.k_scale = a->d_kv_k_scale, p.v_scale = a->d_kv_v_scale;
+    for (int i = 0; i < 3; ++i) {
+        p.scale_stride[i] = a->scale_stride[i];
+    }
+    p.new_kmax = p.new_vmax = p.min_off = nullptr;
     p.flag = nullptr;
     if (validate_meta != 0 && !dev->capturing) {
         void *ws = nullptr;
@@ -465,9 +686,9 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
                              a->token_count - (uint32_t)host_flag);
         }
     }
-    hipLaunchKernelGGL(k_pa_write, dim3(a->token_count, a->num_kv_heads), dim3(a->head_dim <= 64 ? 64 : 128), 0,
-                       dev->stream, p);
-    MH_HIP(hipGetLastError());
+    // workspace: [fp8 scratch][partial results of split histories]
+    const size_t fp8_words = fp8 ? 2 * a->kv_blocks * a->num_kv_heads + a->kv_blocks : 0;
+    const size_t fp8_bytes = (fp8_words * sizeof(uint32_t) + 255) & ~(size_t)255;
     // query heads per workgroup: as many heads of one key / value head as the LDS tile of the final merge allows
     const int qh_max = epl == 16 ? 2 : 4;
     const int qh = (p.group % 4 == 0 && qh_max >= 4) ? 4 : (p.group % 2 == 0 ? 2 : 1);
@@ -480,11 +701,33 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     if (pairs * 2 <= want) {
         size_t sp = (want + pairs - 1) / pairs;
         p.splits = (uint32_t)(sp > 64 ? 64 : sp);
-        void *ws = nullptr;
-        MH_TRY(workspace_reserve(dev, (size_t)a->token_count * a->num_q_heads * p.splits * (a->head_dim + 2u) * sizeof(float),
-                                 &ws));
-        p.partial = (float *)ws;
     }
+    const size_t partial_bytes =
+        p.splits > 1u ? (size_t)a->token_count * a->num_q_heads * p.splits * (a->head_dim + 2u) * sizeof(float) : 0;
+    if (fp8_bytes + partial_bytes != 0) {
+        void *ws = nullptr;
+        MH_TRY(workspace_reserve(dev, fp8_bytes + partial_bytes, &ws));
+        if (fp8) {
+            p.new_kmax = (uint32_t *)ws;
+            p.new_vmax = p.new_kmax + a->kv_blocks * a->num_kv_heads;
+            p.min_off = p.new_vmax + a->kv_blocks * a->num_kv_heads;
+        }
+        p.partial = p.splits > 1u ? (float *)((uint8_t *)ws + fp8_bytes) : nullptr;
+    }
+    const dim3 per_token(a->token_count, a->num_kv_heads);
+    if (fp8) {
+        const size_t cells = a->kv_blocks * a->num_kv_heads;
+        if (cells > ((size_t)1 << 32)) {
+            return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "paged_attention: FP8 cache of %zu blocks", a->kv_blocks);
+        }
+        hipLaunchKernelGGL(k_pa_fp8_init, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, dev->stream, p);
+        hipLaunchKernelGGL(k_pa_fp8_scan_new, per_token, dim3(128), 0, dev->stream, p);
+        hipLaunchKernelGGL(k_pa_fp8_rescale, per_token, dim3(128), 0, dev->stream, p);
+        hipLaunchKernelGGL(k_pa_fp8_store, per_token, dim3(128), 0, dev->stream, p);
+    } else {
+        hipLaunchKernelGGL(k_pa_write, per_token, dim3(a->head_dim <= 64 ? 64 : 128), 0, dev->stream, p);
+    }
+    MH_HIP(hipGetLastError());
     if (epl == 4) {
         qh == 4 ? pa_launch<4, 4>(dev, p) : qh == 2 ? pa_launch<4, 2>(dev, p) : pa_launch<4, 1>(dev, p);
     } else if (epl == 8) {

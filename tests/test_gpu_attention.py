@@ -140,3 +140,113 @@ def test_holes_strided_views_token_count_and_errors(hip, oracle):
     assert code(dict(case, q=np.zeros((T, 3, 32), np.float32))) == -1
     big = make_case(14, [(3, 1)], num_q_heads=1, num_kv_heads=1, head_dim=320, block_size=4)
     assert code(big) == -8  # head dimensions beyond 256 are left to the caller's fallback
+
+
+# ---------------------------------------------------------------- the FLOAT8_E4M3 cache
+def _fp8_case(seed, seqs, act="f32", room=0, **kw):
+    """An empty fp8 cache (codes 0, scales 0) and a call that fills it; `room` more positions per sequence have blocks
+    in the table for later decode steps."""
+    case = make_case(seed, [(h, n + room) for h, n in seqs], act=act, kv="f32", **kw)
+    meta = case["token_meta"]
+    last = {int(s): int(meta[meta[:, 0] == s, 1].max()) for s in set(meta[:, 0])}
+    keep = np.array([int(pos) <= last[int(s)] - room for s, pos, _, _ in meta])
+    case["token_meta"] = np.ascontiguousarray(meta[keep])
+    for n in ("q", "k_new", "v_new"):
+        case[n] = np.ascontiguousarray(case[n][keep])
+    shape = case["kv_k"].shape
+    case["kv_k"], case["kv_v"] = np.zeros(shape, np.uint8), np.zeros(shape, np.uint8)
+    case["k_scale"], case["v_scale"] = np.zeros(shape[:3], np.float32), np.zeros(shape[:3], np.float32)
+    return case
+
+
+def _fp8_both(hip, oracle, case, what):
+    """One call on both sides from the same cache state: cache bytes and scales bit-exact (the write path is integer
+    and exactly rounded float work: maxima, one division, the e4m3 encoder), attention within fp32 summation noise of
+    the oracle and of dense float64 attention over the decoded cache. Returns the state after the call."""
+    from tests.attention_cases import fp8_values
+
+    state = {n: case[n].copy() for n in ("kv_k", "kv_v", "k_scale", "v_scale")}
+    got = hip.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], state["kv_k"], state["kv_v"],
+                              case["block_table"], case["layer_idx"], case["scale"], act_bf16=case["act"] == "bf16",
+                              kv_k_scale=state["k_scale"], kv_v_scale=state["v_scale"])
+    assert hip.last_route() == "paged_attention"
+    ref_state = {n: case[n].copy() for n in ("kv_k", "kv_v", "k_scale", "v_scale")}
+    st, ref = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], ref_state["kv_k"],
+                                     ref_state["kv_v"], case["block_table"], case["layer_idx"], case["scale"],
+                                     act_bf16=case["act"] == "bf16", kv_k_scale=ref_state["k_scale"],
+                                     kv_v_scale=ref_state["v_scale"])
+    assert st == 0
+    for n in ("k_scale", "v_scale", "kv_k", "kv_v"):
+        assert np.array_equal(state[n].view(np.uint8), ref_state[n].view(np.uint8)), f"{what}: {n}"
+    vals = fp8_values().astype(np.float32)
+    dk = (vals[state["kv_k"]] * state["k_scale"][:, :, :, None, None]).astype(np.float32)
+    dv = (vals[state["kv_v"]] * state["v_scale"][:, :, :, None, None]).astype(np.float32)
+    act = case["act"]
+    vmax = np.abs(dv).max()
+    g32, r32 = to_f32(got, act).astype(np.float64), to_f32(ref, act).astype(np.float64)
+    assert np.max(np.abs(g32 - r32)) <= TOLERANCE[act] * vmax, f"{what}: against the oracle"
+    dense = dense_reference(dict(case, kv="f32"), dk, dv)
+    assert np.max(np.abs(g32 - dense)) <= TOLERANCE[act] * vmax, f"{what}: against dense float64 attention"
+    return state
+
+
+def _next_step(case, state, seed, gains, act="f32"):
+    """One more token per sequence at its next position, new rows scaled per sequence by `gains`."""
+    from tests.attention_cases import to_storage
+
+    bs = case["block_size"]
+    meta0 = case["token_meta"]
+    seqs = sorted(set(int(s) for s in meta0[:, 0]))
+    nxt = {s: int(meta0[meta0[:, 0] == s, 1].max()) + 1 for s in seqs}
+    meta = np.array([[s, nxt[s], int(case["block_table"][s, nxt[s] // bs]) * bs + nxt[s] % bs, 0] for s in seqs],
+                    np.uint32)
+    rng = np.random.default_rng(seed)
+    hq, hkv, d = case["q"].shape[1], case["k_new"].shape[1], case["q"].shape[2]
+    gain = np.asarray(gains, np.float32)[:len(seqs), None, None]
+    return dict(case, token_meta=meta, q=to_storage(rng.standard_normal((len(seqs), hq, d), dtype=np.float32), act),
+                k_new=to_storage(rng.standard_normal((len(seqs), hkv, d), dtype=np.float32) * gain, act),
+                v_new=to_storage(rng.standard_normal((len(seqs), hkv, d), dtype=np.float32) * gain, act),
+                kv_k=state["kv_k"], kv_v=state["kv_v"], k_scale=state["k_scale"], v_scale=state["v_scale"])
+
+
+@pytest.mark.parametrize("act,head_dim,block_size,hq,hkv", [("f32", 32, 16, 4, 2), ("f16", 64, 16, 8, 2),
+                                                            ("bf16", 128, 32, 8, 8), ("f32", 256, 16, 2, 1),
+                                                            ("f16", 40, 8, 6, 3)])
+def test_fp8_cache_prefill_then_decode(hip, oracle, act, head_dim, block_size, hq, hkv):
+    """Call 1 fills blocks from empty (scales 0 -> max / 240); then three decode steps append to partly filled
+    blocks: a louder token grows the block's scale and re-encodes the rows already there, a quieter one leaves scale
+    and bytes alone; a step that opens a new block finds scale 0."""
+    case = _fp8_case(300 + head_dim, [(0, 21), (0, 9), (0, 2 * block_size - 1)], act=act, room=3, num_q_heads=hq,
+                     num_kv_heads=hkv, head_dim=head_dim, block_size=block_size, layers=2, layer_idx=1)
+    state = _fp8_both(hip, oracle, case, "prefill")
+    assert (state["k_scale"][:, 0] == 0).all(), "other layers' scales are not touched"
+    for i, gains in enumerate(([4.0, 0.25, 1.0], [0.5, 8.0, 2.0], [1.0, 1.0, 16.0])):
+        before = state
+        case = _next_step(case, state, 400 + i, gains, act)
+        state = _fp8_both(hip, oracle, case, f"decode step {i}")
+        if i == 0:
+            b_loud, b_quiet = (int(case["token_meta"][r, 2]) // block_size for r in (0, 1))
+            assert (state["k_scale"][b_loud, 1] > before["k_scale"][b_loud, 1]).all()
+            assert np.array_equal(state["k_scale"][b_quiet, 1], before["k_scale"][b_quiet, 1])
+
+
+def test_fp8_cache_long_context_decode_batch(hip, oracle):
+    """A decode batch over long fp8 histories takes the split-history kernels and the 16-byte cache loads."""
+    case = _fp8_case(77, [(0, 700), (0, 333), (0, 1025), (0, 64)], room=1, num_q_heads=8, num_kv_heads=2, head_dim=128,
+                     block_size=16, layers=1, layer_idx=0)
+    state = _fp8_both(hip, oracle, case, "prompts")
+    step = _next_step(case, state, 78, [1.0, 3.0, 0.5, 1.0])
+    _fp8_both(hip, oracle, step, "decode over long histories")
+
+
+def test_fp8_cache_errors(hip):
+    case = _fp8_case(5, [(0, 3)], num_q_heads=2, num_kv_heads=1, head_dim=16, block_size=4)
+    args = (case["token_meta"], case["q"], case["k_new"], case["v_new"])
+    with pytest.raises(capi.MarmotHipError) as e:  # paged_attention_ref.c:695-698
+        hip.paged_attention(*args, case["kv_k"].copy(), case["kv_v"].copy(), case["block_table"], 1, case["scale"])
+    assert e.value.code == -1 and "requires scale tensors" in str(e.value)
+    f32 = make_case(5, [(0, 3)], num_q_heads=2, num_kv_heads=1, head_dim=16, block_size=4)
+    with pytest.raises(capi.MarmotHipError) as e:
+        hip.paged_attention(*args, f32["kv_k"].copy(), f32["kv_v"].copy(), f32["block_table"], 1, f32["scale"],
+                            kv_k_scale=case["k_scale"].copy(), kv_v_scale=case["v_scale"].copy())
+    assert e.value.code == -1

@@ -872,9 +872,10 @@ marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, con
 /* marmot_paged_attention (cf. cpu_paged_attention_impl, src/backends/cpu/ops/paged_attention/paged_attention_ref.c:
  * 573-1082): every token's k_new / v_new rows go into the paged cache at its kv_slot, then every token attends over
  * positions 0 .. pos of its sequence through the block table. q / k_new / v_new / out of one type among FLOAT32,
- * FLOAT16, BFLOAT16 and the cache of one of these types, any strides; validation, codes and messages in the
- * reference's order. Declined with NOT_IMPLEMENTED: the FLOAT8_E4M3 cache (with its scale tensors in pnext) and head
- * dimensions beyond 256. The cache tensors are read and written: their mirrors are brought up to date first and the
+ * FLOAT16, BFLOAT16 and the cache of one of these types or FLOAT8_E4M3 (then with FLOAT32 scale tensors [blocks,
+ * layers, kv heads] in pnext, read and written like the cache), any strides; validation, codes and messages in the
+ * reference's order. Declined with NOT_IMPLEMENTED: head dimensions beyond 256, key and value caches (or scales) of
+ * different strides. The cache tensors are read and written: their mirrors are brought up to date first and the
  * device copy is the current one afterwards. */
 marmot_error_t hip_paged_attention_impl(const void *device_ctx, const marmot_paged_attention_desc_t *desc);
 marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,

@@ -1672,9 +1672,10 @@ static bool pa_float_dtype(marmot_dtype_t t) {
 }
 
 static int pa_lib_dtype(marmot_dtype_t t) {
-    return t == MARMOT_DTYPE_FLOAT16 ? MARMOT_HIP_DTYPE_F16
-        : t == MARMOT_DTYPE_BFLOAT16 ? MARMOT_HIP_DTYPE_BF16
-                                     : MARMOT_HIP_DTYPE_F32;
+    return t == MARMOT_DTYPE_FLOAT16     ? MARMOT_HIP_DTYPE_F16
+        : t == MARMOT_DTYPE_BFLOAT16     ? MARMOT_HIP_DTYPE_BF16
+        : t == MARMOT_DTYPE_FLOAT8_E4M3 ? MARMOT_HIP_DTYPE_F8_E4M3
+                                         : MARMOT_HIP_DTYPE_F32;
 }
 
 // bytes from the first to one past the last element of a tensor of any rank and strides
@@ -1772,10 +1773,26 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
     if (kv_k->dtype != kv_v->dtype) {
         return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention kv dtype mismatch");
     }
-    if (kv_fp8) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP paged_attention does not handle the FLOAT8_E4M3 cache");
-    }
-    if (has_scales) {
+    const marmot_tensor_t *k_scale = has_scales ? ext->kv_k_scale : nullptr, *v_scale = has_scales ? ext->kv_v_scale : nullptr;
+    if (kv_fp8) {  // paged_attention_ref.c:694-722
+        if (k_scale == nullptr || v_scale == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention FP8 KV requires scale tensors");
+        }
+        if (k_scale->dtype != MARMOT_DTYPE_FLOAT32 || v_scale->dtype != MARMOT_DTYPE_FLOAT32) {
+            return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "paged_attention FP8 scale dtype must be float32");
+        }
+        if (k_scale->shape.ndim != 3 || v_scale->shape.ndim != 3) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention FP8 scale tensors must be 3D");
+        }
+        for (size_t i = 0; i < 3; ++i) {
+            if (k_scale->shape.shape[i] != kv_k->shape.shape[i] || v_scale->shape.shape[i] != kv_v->shape.shape[i]) {
+                return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "paged_attention FP8 scale tensor shape mismatch");
+            }
+        }
+        if (k_scale->data == nullptr || v_scale->data == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention FP8 scale tensors missing data");
+        }
+    } else if (has_scales) {
         return fail(MARMOT_ERROR_INVALID_ARGUMENT, "paged_attention scale tensors require FP8 KV");
     }
     if (meta->data == nullptr || table->data == nullptr || q->data == nullptr || k_new->data == nullptr ||
@@ -1805,6 +1822,11 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
             return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP paged_attention needs key and value caches of one layout");
         }
     }
+    for (size_t i = 0; kv_fp8 && i < 3; ++i) {
+        if (k_scale->shape.strides[i] != v_scale->shape.strides[i]) {
+            return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP paged_attention needs key and value scales of one layout");
+        }
+    }
     marmot_hip_paged_attention_t a = {
         .token_count = desc->token_count, .layer_idx = desc->layer_idx, .num_q_heads = desc->num_q_heads,
         .num_kv_heads = desc->num_kv_heads, .head_dim = desc->head_dim, .block_size = desc->block_size,
@@ -1825,10 +1847,13 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
     for (size_t i = 0; i < 5; ++i) {
         a.kv_stride[i] = kv_k->shape.strides[i];
     }
+    for (size_t i = 0; kv_fp8 && i < 3; ++i) {
+        a.scale_stride[i] = k_scale->shape.strides[i];
+    }
     pthread_mutex_lock(&b->mu);
     // the caches are read and written; an output that is a view with gaps, or has more rows than tokens, keeps its
     // other bytes: the host's bytes go up first
-    hip_acq_t acq[8] = {
+    hip_acq_t acq[10] = {
         {meta->data, strided_extent_bytes(meta), HIP_ACQ_READ, nullptr},
         {table->data, strided_extent_bytes(table), HIP_ACQ_READ, nullptr},
         {q->data, strided_extent_bytes(q), HIP_ACQ_READ, nullptr},
@@ -1839,12 +1864,19 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
         {out->data, strided_extent_bytes(out),
          dense_contiguous(out) && out->shape.shape[0] == desc->token_count ? HIP_ACQ_WRITE : HIP_ACQ_UPDATE, nullptr},
     };
-    marmot_error_t st = acquire_set(b, acq, 8);
+    if (kv_fp8) {
+        acq[8] = (hip_acq_t){k_scale->data, strided_extent_bytes(k_scale), HIP_ACQ_UPDATE, nullptr};
+        acq[9] = (hip_acq_t){v_scale->data, strided_extent_bytes(v_scale), HIP_ACQ_UPDATE, nullptr};
+    }
+    marmot_error_t st = acquire_set(b, acq, kv_fp8 ? 10 : 8);
     const void *d_meta = acq[0].dev, *d_table = acq[1].dev, *d_q = acq[2].dev, *d_k = acq[3].dev, *d_v = acq[4].dev;
     void *d_kv_k = acq[5].dev, *d_kv_v = acq[6].dev, *d_out = acq[7].dev;
     if (st == MARMOT_SUCCESS) {
         a.d_token_meta = (const uint32_t *)d_meta, a.d_block_table = (const uint32_t *)d_table;
         a.d_q = d_q, a.d_k_new = d_k, a.d_v_new = d_v, a.d_kv_k = d_kv_k, a.d_kv_v = d_kv_v, a.d_out = d_out;
+        if (kv_fp8) {
+            a.d_kv_k_scale = (float *)acq[8].dev, a.d_kv_v_scale = (float *)acq[9].dev;
+        }
         const int rc = marmot_hip_paged_attention(b->dev, &a, 0);
         st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
     }
@@ -1853,6 +1885,10 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
         mark_device_output(out);
         mark_device_output((marmot_tensor_t *)kv_k);
         mark_device_output((marmot_tensor_t *)kv_v);
+        if (kv_fp8) {
+            mark_device_output((marmot_tensor_t *)k_scale);
+            mark_device_output((marmot_tensor_t *)v_scale);
+        }
     }
     return st;
 }
@@ -2518,10 +2554,11 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         return selected(MARMOT_HIP_BC_OP_ROPE, launch_us, 0.0);
     case MARMOT_OP_PAGED_ATTENTION: {
         // paged_attention_scalar (cpu/kernels/paged_attention.def): activations and result of one float type, the
-        // cache type as the weight type; the FLOAT8_E4M3 cache stays with the CPU
+        // cache type as the weight type, FLOAT8_E4M3 included
         const bool act_ok = pa_float_dtype(sig->input_dtype) && sig->output_dtype == sig->input_dtype;
-        if (!act_ok || !pa_float_dtype(sig->weight_dtype)) {
-            return unsupported("HIP paged attention handles FLOAT32, FLOAT16 and BFLOAT16 activations and caches");
+        if (!act_ok || !(pa_float_dtype(sig->weight_dtype) || sig->weight_dtype == MARMOT_DTYPE_FLOAT8_E4M3)) {
+            return unsupported("HIP paged attention handles FLOAT32, FLOAT16 and BFLOAT16 activations and those or "
+                               "FLOAT8_E4M3 caches");
         }
         return selected(MARMOT_HIP_BC_OP_PAGED_ATTENTION, 2.0 * launch_us, 0.0);
     }

@@ -285,8 +285,8 @@ def test_query_kernel_embedding_rules(lib):
 
 
 def test_query_kernel_paged_attention_rules(lib):
-    """cpu/kernels/paged_attention.def:6-22 without the FP8 cache: activations and result of one float type, the
-    cache type as the weight type."""
+    """cpu/kernels/paged_attention.def:3-22: activations and result of one float type, the cache type (FLOAT8_E4M3
+    included) as the weight type."""
     def sig(act=ta.DTYPE_F32, kv=ta.DTYPE_F16, out=None):
         s = ta.OpSignature()
         s.op_id, s.input_dtype, s.weight_dtype = ta.OP_PAGED_ATTENTION, act, kv
@@ -297,7 +297,8 @@ def test_query_kernel_paged_attention_rules(lib):
         for kv in (ta.DTYPE_F32, ta.DTYPE_F16, ta.DTYPE_BF16):
             sel = _query(lib, sig(act, kv))
             assert sel.supported and sel.op_index == ta.BC_OP_PAGED_ATTENTION
-    assert not _query(lib, sig(kv=ta.DTYPE_F8_E4M3)).supported
+    assert _query(lib, sig(kv=ta.DTYPE_F8_E4M3)).supported
+    assert not _query(lib, sig(kv=ta.DTYPE_I32)).supported
     assert not _query(lib, sig(act=ta.DTYPE_I32)).supported
     assert not _query(lib, sig(out=ta.DTYPE_F16)).supported
 

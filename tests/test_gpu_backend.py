@@ -810,7 +810,7 @@ def _attention_tensors(ctx, case):
     from tests.attention_cases import to_storage
 
     act_dt = {"f32": None, "f16": None, "bf16": ta.DTYPE_BF16}[case["act"]]
-    kv_dt = {"f32": None, "f16": None, "bf16": ta.DTYPE_BF16}[case["kv"]]
+    kv_dt = {"f32": None, "f16": None, "bf16": ta.DTYPE_BF16, "fp8": ta.DTYPE_F8_E4M3}[case["kv"]]
     T, hq, d = case["q"].shape
     hkv = case["k_new"].shape[1]
     fused = np.zeros((T, hq + 2 * hkv, d), dtype=case["q"].dtype)
@@ -826,6 +826,9 @@ def _attention_tensors(ctx, case):
         "block_table": ta.HostTensor.dense(case["block_table"]),
         "out": ta.HostTensor.strided(np.zeros((T, hq, d), dtype=case["q"].dtype), act_dt),
     }
+    if case["kv"] == "fp8":  # FLOAT32 scales [blocks, layers, kv heads], handed over through the descriptor's pnext
+        t["k_scale"] = ta.HostTensor.dense(case["k_scale"].copy())
+        t["v_scale"] = ta.HostTensor.dense(case["v_scale"].copy())
     for name, x in t.items():
         if name != "fused":
             ctx.host_range_freed(x)
@@ -902,6 +905,68 @@ def test_impl_and_program_paged_attention(ctx, oracle, act, kv):
                 ctx.host_freed(x)
 
 
+def test_impl_and_program_paged_attention_fp8_cache(ctx, oracle):
+    """The FLOAT8_E4M3 cache through hip_paged_attention_impl (scale tensors in the descriptor's extension) and through
+    the bytecode op (scale tensors as registers): a prompt call that fills an empty cache, then a louder decode step on
+    the cache and scales the first call left on the device. Cache bytes and scales bit for bit against the oracle."""
+    from tests.attention_cases import TOLERANCE
+    from tests.test_gpu_attention import _fp8_case, _next_step
+
+    case = _fp8_case(90, [(0, 21), (0, 9), (0, 40)], room=1, num_q_heads=8, num_kv_heads=2, head_dim=64, block_size=16)
+    case["kv"] = "fp8"
+
+    def reference(c):
+        state = {n: c[n].copy() for n in ("kv_k", "kv_v", "k_scale", "v_scale")}
+        st, ref = oracle.paged_attention(c["token_meta"], c["q"], c["k_new"], c["v_new"], state["kv_k"], state["kv_v"],
+                                         c["block_table"], c["layer_idx"], c["scale"], kv_k_scale=state["k_scale"],
+                                         kv_v_scale=state["v_scale"])
+        assert st == 0
+        return ref, state
+
+    def same_state(t, state):
+        return all(np.array_equal(ctx.to_host(t[n]).view(np.uint8), state[n].view(np.uint8))
+                   for n in ("kv_k", "kv_v", "k_scale", "v_scale"))
+
+    ref, state = reference(case)
+    tol = TOLERANCE["f32"] * 240.0 * max(state["v_scale"].max(), 1e-30)
+    t, desc = _attention_tensors(ctx, case)
+    ext = ta.PagedAttentionKvScaleExt(C.sizeof(ta.PagedAttentionKvScaleExt), 1, t["k_scale"].ptr, t["v_scale"].ptr)
+    desc.pnext = C.addressof(ext)
+    assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
+    assert np.max(np.abs(ctx.to_host(t["out"]).astype(np.float64) - ref)) <= tol
+    assert same_state(t, state)
+    # the same call as a bytecode op on fresh tensors
+    sig = ta.OpSignature()
+    sig.op_id, sig.accum_dtype = ta.OP_PAGED_ATTENTION, ta.DTYPE_F32
+    sig.input_dtype = sig.output_dtype = ta.DTYPE_F32
+    sig.weight_dtype = ta.DTYPE_F8_E4M3
+    sel = ctx.query(sig)
+    assert sel.supported and sel.op_index == ta.BC_OP_PAGED_ATTENTION
+    t2, d2 = _attention_tensors(ctx, case)
+    p = ta.Program()
+    p.paged_attention(sel.op_index, t2["token_meta"], t2["q"], t2["k_new"], t2["v_new"], t2["kv_k"], t2["kv_v"],
+                      t2["block_table"], t2["out"], d2.token_count, d2.layer_idx, d2.num_q_heads, d2.num_kv_heads,
+                      d2.head_dim, d2.block_size, d2.scale, kv_k_scale=t2["k_scale"], kv_v_scale=t2["v_scale"])
+    assert ctx.execute(p) == ta.SUCCESS, ctx.last_error()
+    assert np.array_equal(ctx.to_host(t2["out"]).view(np.uint8), ctx.to_host(t["out"]).view(np.uint8))
+    assert same_state(t2, state)
+    # a decode step, sequence 0 four times louder: its block's scale grows and its rows are re-encoded on the device
+    step = _next_step(dict(case, **state), state, 91, [4.0, 0.25, 1.0])
+    ref2, state2 = reference(step)
+    assert not np.array_equal(state2["k_scale"], state["k_scale"])
+    t3, d3 = _attention_tensors(ctx, step)
+    d3.kv_k, d3.kv_v = t["kv_k"].ptr, t["kv_v"].ptr  # the tensors the first call updated
+    d3.pnext = C.addressof(ext)
+    assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(d3)) == ta.SUCCESS, ctx.last_error()
+    tol2 = TOLERANCE["f32"] * 240.0 * state2["v_scale"].max()
+    assert np.max(np.abs(ctx.to_host(t3["out"]).astype(np.float64) - ref2)) <= tol2
+    assert same_state(t, state2)
+    for group in (t, t2, t3):
+        for name, x in group.items():
+            if name != "fused":
+                ctx.host_freed(x)
+
+
 def test_impl_paged_attention_errors(ctx):
     """The checks of cpu_paged_attention_impl in its order (paged_attention_ref.c:573-823), then what this backend
     leaves to the fallback."""
@@ -941,9 +1006,18 @@ def test_impl_paged_attention_errors(ctx):
     bad[1, 0], bad[1, 2] = 0, case["kv_k"].shape[0] * 8
     assert call(token_meta=ta.HostTensor.dense(bad)) == ta.DIMENSION_MISMATCH and "kv_slot" in ctx.last_error()[1]
     fp8 = [ta.HostTensor.strided(np.zeros(case["kv_k"].shape, np.uint8), ta.DTYPE_F8_E4M3) for _ in range(2)]
-    assert call(kv_k=fp8[0], kv_v=fp8[1]) == ta.NOT_IMPLEMENTED
+    assert call(kv_k=fp8[0], kv_v=fp8[1]) == ta.INVALID_ARGUMENT and "requires scale tensors" in ctx.last_error()[1]
     ext = ta.PagedAttentionKvScaleExt(C.sizeof(ta.PagedAttentionKvScaleExt), 1, t["kv_k"].ptr, t["kv_v"].ptr)
     assert call(pnext=C.addressof(ext)) == ta.INVALID_ARGUMENT and "require FP8" in ctx.last_error()[1]
+    # the scale tensors of an FP8 cache: FLOAT32, [blocks, layers, kv heads] (paged_attention_ref.c:694-722)
+    shape3 = case["kv_k"].shape[:3]
+    for arr, code, text in ((np.zeros(shape3, np.float16), ta.UNSUPPORTED_DTYPE, "must be float32"),
+                            (np.zeros(shape3[:2], np.float32), ta.DIMENSION_MISMATCH, "must be 3D"),
+                            (np.zeros((shape3[0], shape3[1], shape3[2] + 1), np.float32), ta.DIMENSION_MISMATCH,
+                             "shape mismatch")):
+        sc = [ta.HostTensor.dense(arr.copy()) for _ in range(2)]
+        bad_ext = ta.PagedAttentionKvScaleExt(C.sizeof(ta.PagedAttentionKvScaleExt), 1, sc[0].ptr, sc[1].ptr)
+        assert call(kv_k=fp8[0], kv_v=fp8[1], pnext=C.addressof(bad_ext)) == code and text in ctx.last_error()[1]
     wide = make_case(73, [(2, 1)], num_q_heads=1, num_kv_heads=1, head_dim=320, block_size=4)
     tw, dw = _attention_tensors(ctx, wide)
     assert ctx.lib.hip_paged_attention_impl(ctx.device_ctx, C.byref(dw)) == ta.NOT_IMPLEMENTED

@@ -507,7 +507,7 @@ def sweep_attention(hip, rng, emit, steps: int):
 
     hq, hkv, d, bs = 32, 8, 128, 16
 
-    def run(name, seqs):
+    def run(name, seqs, fp8=False):
         need = [-(-(h + n) // bs) for h, n in seqs]
         blocks = sum(need)
         table = np.full((len(seqs), max(need)), 0xFFFFFFFF, dtype=np.uint32)
@@ -527,11 +527,18 @@ def sweep_attention(hip, rng, emit, steps: int):
             "kv_v": rng.standard_normal((blocks, 1, hkv, bs, d), dtype=np.float32).astype(np.float16),
             "out": np.zeros((T, hq, d), dtype=np.float32),
         }
+        if fp8:  # finite e4m3 codes of either sign; scales under which the new rows never raise a block's maximum,
+            # the steady state of a decode loop (no re-encoding of the rows already there)
+            for n in ("kv_k", "kv_v"):
+                arrays[n] = (rng.integers(0, 0x78, arrays[n].shape) | (rng.integers(0, 2, arrays[n].shape) << 7)).astype(np.uint8)
+            arrays["k_scale"] = np.full((blocks, 1, hkv), 0.05, dtype=np.float32)
+            arrays["v_scale"] = np.full((blocks, 1, hkv), 0.05, dtype=np.float32)
         dev = {k: hip.to_device(v) for k, v in arrays.items()}
         ptr_of = {id(v): dev[k].ptr for k, v in arrays.items()}
         a = arrays
         p = hip.paged_attention_args(lambda x: ptr_of[id(x)], a["token_meta"], a["q"], a["k_new"], a["v_new"], a["kv_k"],
-                                     a["kv_v"], a["block_table"], a["out"], 0, float(1.0 / np.sqrt(d)))
+                                     a["kv_v"], a["block_table"], a["out"], 0, float(1.0 / np.sqrt(d)),
+                                     kv_k_scale=a.get("k_scale"), kv_v_scale=a.get("v_scale"))
 
         def step(i):
             rc = hip.lib.marmot_hip_paged_attention(hip.dev, C.byref(p), 0)
@@ -539,8 +546,9 @@ def sweep_attention(hip, rng, emit, steps: int):
                 raise RuntimeError(f"marmot_hip_paged_attention -> {rc}")
 
         ms = time_steps_graph(hip, step, max(20, steps // 20), 5, chunk=20)
-        read = sum(int(pos) + 1 for _, pos, _, _ in meta) * hkv * d * 2 * 2  # K and V rows of fp16, once per kv head
-        total = read + T * (hq * 2 + hkv * 2) * d * 4 + T * hkv * d * 2 * 2
+        esz = 1 if fp8 else 2
+        read = sum(int(pos) + 1 for _, pos, _, _ in meta) * hkv * d * 2 * esz  # K and V rows, once per kv head
+        total = read + T * (hq * 2 + hkv * 2) * d * 4 + T * hkv * d * 2 * esz
         flops = 4.0 * sum(int(pos) + 1 for _, pos, _, _ in meta) * hq * d
         emit({"config": "ATTN", "workload": name, "us": round(ms * 1e3, 2), "GB/s": round(total / ms / 1e6, 1),
               "frac_of_hbm_peak": round(total / ms / 1e6 / HBM_PEAK_GBPS, 4), "TFLOP/s": round(flops / ms / 1e9, 2),
@@ -551,6 +559,7 @@ def sweep_attention(hip, rng, emit, steps: int):
     run("paged attention, decode: 16 sequences x 4096 positions, 32/8 heads of 128, fp16 cache", [(4095, 1)] * 16)
     run("paged attention, decode: 16 sequences x 512 positions", [(511, 1)] * 16)
     run("paged attention, prompt: 512 tokens of one sequence", [(0, 512)])
+    run("paged attention, decode: 16 sequences x 4096 positions, FLOAT8_E4M3 cache", [(4095, 1)] * 16, fp8=True)
 
 
 def sweep_whole_layer(hip, rng, emit, steps: int, T: int = 16, context: int = 4096):

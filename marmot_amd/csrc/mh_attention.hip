@@ -155,9 +155,22 @@ __device__ __forceinline__ void pa_load_run(const void *data, int dtype, size_t 
             const uint4 u = *(const uint4 *)((const uint8_t *)data + first);
             w[0] = u.x, w[1] = u.y, w[2] = u.z, w[3] = u.w;
         }
+        // Codes whose exponent field is below 15 mean the same in this format and in the hardware's e4m3 (bias 7,
+        // same subnormals), which converts two bytes per instruction; a word that holds a field of 15 (this format's
+        // NaN) takes the bit-level decoder.
+        typedef float pa_f2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-        for (int e = 0; e < EPL; ++e) {
-            v[e] = pa_fp8_to_f32((w[e / 4] >> (8 * (e % 4))) & 0xffu);
+        for (int i = 0; i < EPL / 4; ++i) {
+            if (((((w[i] & 0x78787878u) + 0x08080808u) & 0x80808080u)) == 0u) {
+                const pa_f2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);
+                const pa_f2 hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
+                v[4 * i] = lo.x, v[4 * i + 1] = lo.y, v[4 * i + 2] = hi.x, v[4 * i + 3] = hi.y;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[4 * i + e] = pa_fp8_to_f32((w[i] >> (8 * e)) & 0xffu);
+                }
+            }
         }
     } else if (dtype == MARMOT_HIP_DTYPE_F32) {
 #pragma unroll

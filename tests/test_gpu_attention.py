@@ -250,3 +250,53 @@ def test_fp8_cache_errors(hip):
         hip.paged_attention(*args, f32["kv_k"].copy(), f32["kv_v"].copy(), f32["block_table"], 1, f32["scale"],
                             kv_k_scale=case["k_scale"].copy(), kv_v_scale=case["v_scale"].copy())
     assert e.value.code == -1
+
+
+@pytest.mark.parametrize("head_dim", [64, 128, 256, 24])
+def test_fp8_cache_given_codes(hip, oracle, head_dim):
+    """Histories written as raw codes, one kind per sequence: only subnormal codes (magnitudes up to 7 x 2^-9, either
+    sign, -0 included), every finite code, and all 256 codes (exponent field 15 decodes to NaN: that sequence checks
+    the cache write next to NaN codes, bit for bit; its attention output is not compared: the reference's result is
+    NaN throughout once one score is NaN, the device's softmax gives a NaN score the weight 0, and the reference's
+    tests define nothing for NaN inputs). Each other sequence's output is judged against its own largest value."""
+    from tests.attention_cases import fp8_values
+
+    hist = 40
+    case = _fp8_case(500 + head_dim, [(hist, 1)] * 3, room=0, num_q_heads=4, num_kv_heads=2, head_dim=head_dim,
+                     block_size=16, layers=1, layer_idx=0)
+    rng = np.random.default_rng(head_dim)
+    shape = case["kv_k"].shape
+    kinds = [lambda n: (rng.integers(0, 8, n) | (rng.integers(0, 2, n) << 7)),
+             lambda n: (rng.integers(0, 0x78, n) | (rng.integers(0, 2, n) << 7)),
+             lambda n: rng.integers(0, 256, n)]
+    order = {int(s): i for i, s in enumerate(case["token_meta"][:, 0])}  # token row of each sequence slot
+    for slot, row in order.items():
+        blocks = case["block_table"][slot]
+        for b in blocks[blocks != NO_BLOCK]:
+            for cache in (case["kv_k"], case["kv_v"]):
+                cache[b] = kinds[row % 3](shape[1:]).astype(np.uint8)
+        if row % 3 == 0:  # quiet new rows beside the subnormal history
+            case["k_new"][row] *= 1e-3
+            case["v_new"][row] *= 1e-3
+    case["k_scale"][...] = 1.0
+    case["v_scale"][...] = 1.0
+    state = {n: case[n].copy() for n in ("kv_k", "kv_v", "k_scale", "v_scale")}
+    got = hip.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], state["kv_k"], state["kv_v"],
+                              case["block_table"], 0, case["scale"], kv_k_scale=state["k_scale"],
+                              kv_v_scale=state["v_scale"])
+    ref_state = {n: case[n].copy() for n in ("kv_k", "kv_v", "k_scale", "v_scale")}
+    st, ref = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], ref_state["kv_k"],
+                                     ref_state["kv_v"], case["block_table"], 0, case["scale"],
+                                     kv_k_scale=ref_state["k_scale"], kv_v_scale=ref_state["v_scale"])
+    assert st == 0
+    for n in ("k_scale", "v_scale", "kv_k", "kv_v"):
+        assert np.array_equal(state[n].view(np.uint8), ref_state[n].view(np.uint8)), n
+    vals = fp8_values()
+    for slot, row in order.items():
+        if row % 3 == 2:
+            assert np.isnan(ref[row]).any()
+            continue
+        blocks = case["block_table"][slot]
+        blocks = blocks[blocks != NO_BLOCK]
+        vmax = np.nanmax(np.abs(vals[state["kv_v"][blocks]] * state["v_scale"][blocks][:, :, :, None, None]))
+        assert vmax > 0 and np.max(np.abs(got[row].astype(np.float64) - ref[row])) <= TOLERANCE["f32"] * vmax, row

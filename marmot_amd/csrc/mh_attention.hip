@@ -311,28 +311,34 @@ __global__ __launch_bounds__(128) void k_pa_fp8_rescale(const PaParams p) {
     const size_t si = (size_t)b * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] + (size_t)h * p.scale_stride[2];
     const size_t base = (size_t)b * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2];
     const uint32_t cells = existing * p.head_dim;
+    uint8_t *const kc = (uint8_t *)p.kv_k + base, *const vc = (uint8_t *)p.kv_v + base;
+    // The largest decoded magnitude among the rows already there: a finite code's magnitude grows with its low seven
+    // bits, so the largest such field is found first and decoded once (NaN codes, field 15, never win a maximum).
+    uint32_t kbig = 0, vbig = 0;
+    for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
+        const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
+        const size_t at = (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
+        const uint32_t kb = kc[at] & 0x7fu, vb = vc[at] & 0x7fu;
+        kbig = kb < 0x78u && kb > kbig ? kb : kbig;
+        vbig = vb < 0x78u && vb > vbig ? vb : vbig;
+    }
+    const float old_k = p.k_scale[si], old_v = p.v_scale[si];  // read by every thread before the barriers below,
+    kbig = (uint32_t)pa_block_max((float)kbig, red);           // written by thread 0 after them
+    vbig = (uint32_t)pa_block_max((float)vbig, red);
     for (int which = 0; which < 2; ++which) {
-        uint8_t *cache = (uint8_t *)(which ? p.kv_v : p.kv_k);
+        uint8_t *cache = which ? vc : kc;
         float *scales = which ? p.v_scale : p.k_scale;
-        const float old_scale = scales[si];
-        float big = 0.0f;
-        if (existing > 0 && old_scale > 0.0f) {
-            for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
-                const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
-                big = fmaxf(big, fabsf(pa_fp8_dequant(cache[base + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4]], old_scale)));
-            }
-        }
-        big = pa_block_max(big, red);
+        const float old_scale = which ? old_v : old_k;
+        float big = pa_fp8_dequant(which ? vbig : kbig, old_scale);
         big = fmaxf(big, __uint_as_float((which ? p.new_vmax : p.new_kmax)[(size_t)b * p.num_kv_heads + h]));
         const float new_scale = big > 0.0f ? big / 240.0f : 1.0f;
         if (existing > 0 && new_scale != old_scale) {
             for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
                 const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
-                uint8_t *cell = cache + base + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
+                uint8_t *cell = cache + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
                 *cell = (uint8_t)pa_fp8_quant(pa_fp8_dequant(*cell, old_scale), new_scale);
             }
         }
-        __syncthreads();
         if (threadIdx.x == 0) {
             scales[si] = new_scale;
         }

@@ -257,8 +257,8 @@ def test_fp8_cache_given_codes(hip, oracle, head_dim):
     """Histories written as raw codes, one kind per sequence: only subnormal codes (magnitudes up to 7 x 2^-9, either
     sign, -0 included), every finite code, and all 256 codes (exponent field 15 decodes to NaN: that sequence checks
     the cache write next to NaN codes, bit for bit; its attention output is not compared: the reference's result is
-    NaN throughout once one score is NaN, the device's softmax gives a NaN score the weight 0, and the reference's
-    tests define nothing for NaN inputs). Each other sequence's output is judged against its own largest value."""
+    NaN throughout once one score is NaN, the device's stays finite where the values it weights are finite, and the
+    reference's tests define nothing for NaN inputs). Each other sequence's output is judged against its own largest value."""
     from tests.attention_cases import fp8_values
 
     hist = 40

@@ -149,6 +149,20 @@ size_t marmot_hip_graph_last_capture_nodes(marmot_hip_device_t *dev);
  * launch of the same size. size and d_src must be multiples of 16. */
 int marmot_hip_read_probe(marmot_hip_device_t *dev, const void *d_src, size_t size, void *d_sink);
 
+/* Measurement aid, no counterpart in the reference: a one-wavefront kernel on the device object's stream that stores the
+ * device's constant-rate counter (100 MHz, 10 ns per tick) into the 8 bytes at d_ticks. Unlike a HIP event it can be
+ * recorded into a captured graph, so a benchmark can bracket the steps of one graph replay without the submission of
+ * the graph in the figure (bench.py does). */
+int marmot_hip_timestamp(marmot_hip_device_t *dev, void *d_ticks);
+
+/* Diagnostic, no counterpart in the reference: in a library built with `make TIMELINE=1` (-DMH_TIMELINE; it is
+ * written to marmot_amd/lib/libmarmot_hip_timeline.so) the instrumented kernels (the row-owning Q4_K matvec, the read
+ * probe) store the device's 100 MHz constant-rate counter at marked points: one 8-byte word per wavefront and mark, at
+ * word (wavefront index in the launch) * 16 + mark of `d_marks` (device memory of the caller, `bytes` long; later
+ * launches overwrite earlier ones; NULL turns the marks off). The product build has no marks in its kernels and
+ * returns MARMOT_HIP_ERROR_NOT_IMPLEMENTED. */
+int marmot_hip_timeline_attach(marmot_hip_device_t *dev, void *d_marks, size_t bytes);
+
 /* Timing helpers (HIP events on the device object's stream). */
 int marmot_hip_event_create(marmot_hip_device_t *dev, void **out_event);
 void marmot_hip_event_destroy(marmot_hip_device_t *dev, void *event);

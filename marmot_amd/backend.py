@@ -151,6 +151,9 @@ class HipBackend:
         check(self.lib.marmot_hip_event_create(self.dev, C.byref(e)))
         return e
 
+    def event_destroy(self, e):
+        self.lib.marmot_hip_event_destroy(self.dev, e)
+
     def record(self, e):
         check(self.lib.marmot_hip_event_record(self.dev, e))
 

@@ -211,6 +211,7 @@ struct ActScratch {
 // creates another device object). Each one turns a route off and leaves the slower general one:
 //   MARMOT_HIP_NO_MMQ          small-batch kernels on the int8 matrix cores -> packed matvec
 //   MARMOT_HIP_NO_ROW_KERNELS  row-owning kernels (one workgroup per compute unit) -> the streaming kernels
+//   MARMOT_HIP_NO_RESIDENT_ROWS the resident-share Q4_K decode kernel (one activation row) -> the ring form of the row kernel
 //   MARMOT_HIP_NO_LDS_RING     loader / consumer matvec (weights through an LDS ring) -> register-streaming matvec
 //   MARMOT_HIP_NO_FUSED_QUANT  activation quantization inside the matvec -> separate quantization launch
 //   MARMOT_HIP_NO_GEMM         fp16 prefill GEMM -> fp16 matvec
@@ -220,6 +221,7 @@ struct ActScratch {
 struct marmot_hip_knobs {
     bool no_mmq = false;
     bool no_row_kernels = false;
+    bool no_resident_rows = false;
     bool no_lds_ring = false;
     bool no_fused_quant = false;
     bool no_gemm = false;
@@ -251,6 +253,10 @@ struct marmot_hip_device {
     size_t static_scratch_bytes = 0;
     bool use_static_scratch = false;
     std::unordered_set<const void *> large_lds_kernels;  // kernels whose dynamic-LDS limit has been raised (under mu)
+    // Timeline build only (-DMH_TIMELINE): device buffer of the caller that instrumented kernels write their marks to
+    // (marmot_hip_timeline_attach); nullptr = marks off.
+    unsigned long long *timeline = nullptr;
+    uint32_t timeline_words = 0;
     // allocation accounting
     std::mutex mu;
     std::unordered_map<void *, size_t> allocs;
@@ -284,6 +290,48 @@ __device__ __forceinline__ void warm_kernel_arguments() {
     }
     asm volatile("" ::"s"(touched));
 }
+
+// Timeline marks (diagnostic build, -DMH_TIMELINE; the product build compiles them to nothing). MH_MARK(p, slot) keeps
+// the wavefront's cycle counter (s_memtime, one scalar instruction, nobody waits for it) in registers; when the
+// wavefront leaves, MH_MARK_FLUSH(p) has lane 0 store the marks into words
+// (wavefront index in the launch) * MH_TIMELINE_SLOTS + slot of the attached buffer. Slots 0 .. 11 are the kernel's;
+// 12 / 13 hold the cycle counter and the 100 MHz constant-rate counter (common to the whole device) at the first
+// mark, 14 / 15 the same pair at the flush, which gives the cycle counter's rate and a common time base.
+#define MH_TIMELINE_SLOTS 16
+#if defined(MH_TIMELINE)
+struct TimelineArg {
+    unsigned long long *buf;
+    uint32_t words;
+};
+__device__ __forceinline__ void timeline_flush(const TimelineArg &t, unsigned long long (&tm)[MH_TIMELINE_SLOTS]) {
+    tm[14] = __builtin_readcyclecounter();
+    tm[15] = __builtin_amdgcn_s_memrealtime();
+    if (t.buf != nullptr && (threadIdx.x & 63u) == 0) {
+        const uint32_t wave = (blockIdx.y * gridDim.x + blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+        const uint32_t base = wave * MH_TIMELINE_SLOTS;
+        if (base + MH_TIMELINE_SLOTS <= t.words) {
+#pragma unroll
+            for (int i = 0; i < MH_TIMELINE_SLOTS; ++i) {
+                t.buf[base + i] = tm[i];
+            }
+        }
+    }
+}
+#define MH_TIMELINE_FIELD ::mh::TimelineArg timeline;
+#define MH_TIMELINE_SET(p, dev) ((p).timeline = ::mh::TimelineArg{(dev)->timeline, (dev)->timeline_words})
+#define MH_MARK_DECL                                                                                                   \
+    unsigned long long mh_tm[MH_TIMELINE_SLOTS] = {};                                                                  \
+    mh_tm[12] = __builtin_readcyclecounter();                                                                          \
+    mh_tm[13] = __builtin_amdgcn_s_memrealtime();
+#define MH_MARK(p, slot) (mh_tm[slot] = __builtin_readcyclecounter())
+#define MH_MARK_FLUSH(p) ::mh::timeline_flush((p).timeline, mh_tm)
+#else
+#define MH_TIMELINE_FIELD
+#define MH_TIMELINE_SET(p, dev) ((void)0)
+#define MH_MARK_DECL
+#define MH_MARK(p, slot) ((void)0)
+#define MH_MARK_FLUSH(p) ((void)0)
+#endif
 
 // s_waitcnt vmcnt(n) for a run-time n: the immediate must be a constant, and it must be the exact count (a smaller one
 // would also wait for loads of the newer steps, i.e. for a full memory latency)
@@ -348,6 +396,10 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
 // it does not cover.
 int launch_matvec_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, size_t N, size_t K,
                            size_t M, int out_dtype);
+// Resident-share form of the same for ONE weight and ONE activation row (mh_matvec_rows2.hip): the workgroup's rows are
+// copied into LDS once, the loaders also fetch the activation row. Same return convention.
+int launch_matvec_rows2_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, size_t N, size_t K,
+                            size_t M, int out_dtype);
 // Row-owning small-batch Q4_K matmul on the int8 matrix cores for 1..16 activation rows (mh_mmq_rows.hip): fp32 rows
 // are quantized inside the kernel (act == nullptr), packed rows are copied into LDS by the kernel's loaders; K is
 // split inside the workgroup. Returns

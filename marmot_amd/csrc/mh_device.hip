@@ -170,6 +170,7 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
     // route switches: read here, never on a launch path
     dev->knobs.no_mmq = getenv("MARMOT_HIP_NO_MMQ") != nullptr;
     dev->knobs.no_row_kernels = getenv("MARMOT_HIP_NO_ROW_KERNELS") != nullptr;
+    dev->knobs.no_resident_rows = getenv("MARMOT_HIP_NO_RESIDENT_ROWS") != nullptr;
     dev->knobs.no_lds_ring = getenv("MARMOT_HIP_NO_LDS_RING") != nullptr;
     dev->knobs.no_fused_quant = getenv("MARMOT_HIP_NO_FUSED_QUANT") != nullptr;
     dev->knobs.no_gemm = getenv("MARMOT_HIP_NO_GEMM") != nullptr;
@@ -358,6 +359,24 @@ int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev) {
     MH_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
     dev->capturing = true;
     return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_timeline_attach(marmot_hip_device_t *dev, void *d_marks, size_t bytes) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "timeline_attach: null device");
+    }
+#if defined(MH_TIMELINE)
+    if (d_marks != nullptr && ((((uintptr_t)d_marks) & 7) != 0 || bytes / 8 > 0xffffffffull)) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "timeline_attach: the buffer must be 8-byte aligned");
+    }
+    dev->timeline = (unsigned long long *)d_marks;
+    dev->timeline_words = d_marks != nullptr ? (uint32_t)(bytes / 8) : 0;
+    return MARMOT_HIP_SUCCESS;
+#else
+    (void)d_marks;
+    (void)bytes;
+    return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "timeline_attach: this library was built without -DMH_TIMELINE");
+#endif
 }
 
 size_t marmot_hip_graph_max_nodes(void) {

@@ -1369,6 +1369,13 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
     p.expert_stride = 0;
     const int nw = ws.count;
     const bool fused = act == nullptr;
+    if (kind == MARMOT_HIP_KIND_Q4_K && fused && N == 1 && nw == 1 && !dev->knobs.no_row_kernels &&
+        !dev->knobs.no_resident_rows) {
+        const int st = launch_matvec_rows2_q4k(dev, ws, d_x_f32, N, K, M, out_dtype);
+        if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {
+            return st;
+        }
+    }
     if (kind == MARMOT_HIP_KIND_Q4_K && fused && N <= 2 && !dev->knobs.no_row_kernels) {
         const int st = launch_matvec_rows_q4k(dev, ws, d_x_f32, N, K, M, out_dtype);
         if (st != MARMOT_HIP_ERROR_NOT_IMPLEMENTED) {

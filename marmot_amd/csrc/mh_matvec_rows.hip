@@ -50,6 +50,7 @@ struct RowsParams {
     int bias_is_f16;
     int bias_first;
     int out_is_f16;
+    MH_TIMELINE_FIELD
 };
 
 // LDS control words (uint32): [0] wavefronts that have stored their quantized activations; then per ring slot
@@ -86,6 +87,8 @@ __device__ __forceinline__ void store_result(const RowsParams &p, void *out, con
 template <int NC, int G>
 __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    MH_MARK_DECL
+    MH_MARK(p, 0);  // timeline: wavefront started
     warm_kernel_arguments<sizeof(RowsParams), sizeof(RowsParams)>();
     constexpr int SB = 16 * G;   // block positions per wavefront
     constexpr int NQ = 2 * G;    // 16-byte pieces of packed nibbles per lane and block
@@ -105,7 +108,7 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
     const uint32_t row0 = blockIdx.x * p.rows_per_wg;
     const uint32_t rows_here = p.M - row0 < p.rows_per_wg ? p.M - row0 : p.rows_per_wg;
     const uint32_t groups = (rows_here + p.rpt - 1) >> p.rpt_shift;
-    const uint8_t *__restrict__ wbase = p.w[blockIdx.y];
+    const uint8_t *__restrict__ wbase = uniform_pointer(p.w[blockIdx.y]);  // the loads take it in scalar registers
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
     // Segment order: index gi = round * C + consumer; consumer c works on K segment c % segs of row group
     // c / segs + round * wstep. Only the last round can be incomplete, and there the missing segments are the last
@@ -118,7 +121,6 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
         // loader count is a multiple of segs and divides the consumer count, which makes loader l's segments
         // l, l + L, l + 2 L, ... one K segment (l % segs) of row groups l / segs + j * (L / segs): constant strides.
         const uint32_t l = (uint32_t)wave - C;
-        const uint32_t ipt = p.slot_stride >> 10;  // load instructions per segment
         const uint32_t lane16 = (uint32_t)lane * 16u;
         uint32_t lseg = l, rg = 0;
         while (lseg >= segs) {
@@ -130,6 +132,10 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
         const uint32_t seg_nb = p.nb - seg_first < p.seg_blocks ? p.nb - seg_first : p.seg_blocks;
         const uint32_t task_bytes = segs == 1 ? p.rpt * p.row_bytes : seg_nb * (uint32_t)Q4_K_BYTES;
         const uint32_t full = task_bytes >> 10;  // whole KiBs of a segment
+        // Load instructions per segment of THIS loader (it always works on one K segment, and the last K segment of a
+        // row can be shorter than the others): the landed-segment arithmetic below divides the outstanding
+        // instructions by it, so it must be the number actually issued, not the slot size.
+        const uint32_t ipt = (task_bytes + 1023u) >> 10;
         // per-lane offset of the (possibly partial) last KiB: lanes beyond the segment re-read its last 16 bytes into
         // the padding of the slot, so every instruction is issued by all lanes and the count per segment is exact
         uint32_t tail_in = full * 1024u + lane16;
@@ -145,6 +151,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
         const uint32_t dst_step = L * p.slot_stride, dst_wrap = p.nslots * p.slot_stride;
         uint32_t issued = 0, published = 0;
         auto publish = [&]() {
+            if (published == 0) {
+                MH_MARK(p, 4);  // loader: its first segment has landed
+            }
             if (lane == 0) {
                 __atomic_store_n(landed + pub_slot, pub_gi + 1u, __ATOMIC_RELAXED);
             }
@@ -202,10 +211,13 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
         };
         // A first few segments are requested before the workgroup barrier (the consumers are still fetching their
         // kernel arguments and requesting the activations then); nothing is published before the control words are zero.
+        MH_MARK(p, 1);  // loader: about to issue its first request
         for (uint32_t i = 0; i < p.pre && rg < groups; ++i, rg += rg_step) {
             issue_segment();
         }
+        MH_MARK(p, 2);  // loader: first requests issued
         __builtin_amdgcn_s_barrier();
+        MH_MARK(p, 3);  // loader: workgroup barrier passed
         // publish what has landed without waiting for it: loads complete in issue order, so the segments behind the
         // `outstanding` youngest instructions are in LDS
         auto publish_landed = [&]() {
@@ -235,10 +247,13 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
                 publish();
             }
         }
+        MH_MARK(p, 5);  // loader: last request issued
         while (published < issued) {
             wait_vmcnt_at_most((int)((issued - published - 1u) * ipt));
             publish();
         }
+        MH_MARK(p, 6);  // loader: its last segment has landed
+        MH_MARK_FLUSH(p);
         return;
     }
     // -------------------------------------------------------------------- consumer
@@ -265,6 +280,7 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
             }
         }
     }
+    MH_MARK(p, 1);  // consumer: activation loads issued
     for (uint32_t i = threadIdx.x; i < ctrl_words(p.nslots, p.rows_per_wg >> p.rpt_shift); i += C * 64u) {
         ctrl[i] = 0;
     }
@@ -272,6 +288,7 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
     // requests in arrival order) and the control words are zero.
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_s_barrier();
+    MH_MARK(p, 2);  // consumer: workgroup barrier passed
     void *const out = p.out[blockIdx.y];
     const void *const bias = p.bias[blockIdx.y];
     {
@@ -321,7 +338,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
             if (lane == 0) {
                 __atomic_fetch_add(ctrl + CTRL_XQ, 1u, __ATOMIC_RELAXED);
             }
+            MH_MARK(p, 3);  // consumer: own part of the activations quantized (their loads have arrived)
             lds_wait_at_least(ctrl + CTRL_XQ, C);
+            MH_MARK(p, 4);  // consumer: every consumer's part is in LDS
 #pragma unroll
             for (int n = 0; n < NC; ++n) {
                 const uint8_t *xq = lds + p.xq_off + (size_t)n * p.xq_stride;
@@ -364,8 +383,15 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
         while (rslot >= p.nslots) {
             rslot -= p.nslots;
         }
+        MH_MARK(p, 5);  // consumer: ready for its first segment
         for (uint32_t rg = wq; rg < groups; rg += wstep) {
             lds_wait_at_least(landed + rslot, gi + 1u);
+            if (rg == wq) {
+                MH_MARK(p, 6);  // consumer: first segment there
+            }
+            if (rg + wstep >= groups) {
+                MH_MARK(p, 7);  // consumer: last segment there
+            }
             const uint8_t *blk = lds + p.ring_off + (size_t)rslot * p.slot_stride + blk_off;
             const uint4 hdr = *(const uint4 *)blk;
             uint4 q[NQ];
@@ -460,6 +486,8 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
                 }
             }
         }
+        MH_MARK(p, 8);  // consumer: done
+        MH_MARK_FLUSH(p);
     }
 }
 
@@ -619,6 +647,7 @@ int launch_matvec_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const fl
     p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
     p.bias_first = ws.bias_first ? 1 : 0;
     p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    MH_TIMELINE_SET(p, dev);
     set_route("matvec_rows_q4_k_q8_k_fused");
     const int nw = ws.count;
     if (N == 1) {

@@ -200,7 +200,18 @@ __global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, u
 // Read-only stream of 16-byte loads, 8 in flight per lane, each workgroup over one contiguous run of 32 KiB: what a
 // kernel that only has to fetch its operand can reach. The loaded words are folded and stored only if they match a
 // value the fold cannot produce from the all-ones test pattern, so nothing is written.
-__global__ __launch_bounds__(256) void k_read16(const uint4 *__restrict__ src, uint32_t *sink, size_t n16) {
+struct ReadProbeParams {
+    const uint4 *src;
+    uint32_t *sink;
+    size_t n16;
+    MH_TIMELINE_FIELD
+};
+__global__ __launch_bounds__(256) void k_read16(const ReadProbeParams p) {
+    MH_MARK_DECL
+    MH_MARK(p, 0);  // timeline: wavefront started
+    const uint4 *__restrict__ src = p.src;
+    uint32_t *sink = p.sink;
+    const size_t n16 = p.n16;
     const size_t base = (size_t)blockIdx.x * 256 * 8 + threadIdx.x;
     uint4 v[8];
 #pragma unroll
@@ -208,6 +219,7 @@ __global__ __launch_bounds__(256) void k_read16(const uint4 *__restrict__ src, u
         const size_t idx = base + (size_t)i * 256;
         v[i] = idx < n16 ? src[idx] : make_uint4(0, 0, 0, 0);
     }
+    MH_MARK(p, 1);  // loads issued
     uint32_t a = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -216,6 +228,11 @@ __global__ __launch_bounds__(256) void k_read16(const uint4 *__restrict__ src, u
     if (a == 0x12345678u) {
         sink[threadIdx.x] = a;
     }
+#if defined(MH_TIMELINE)
+    asm volatile("" ::"v"(a));  // the marks below must not move above the fold: it is what waits for the loads
+#endif
+    MH_MARK(p, 2);  // data arrived
+    MH_MARK_FLUSH(p);
 }
 
 __global__ void k_fill_bytes(uint8_t *dst, uint8_t value, size_t n) {
@@ -304,8 +321,28 @@ int marmot_hip_read_probe(marmot_hip_device_t *dev, const void *d_src, size_t si
     if (grid > 0x7fffffffu) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "read_probe: %zu bytes are more than one launch covers", size);
     }
-    hipLaunchKernelGGL(k_read16, dim3((unsigned)grid), dim3(256), 0, dev->stream, (const uint4 *)d_src,
-                       (uint32_t *)d_sink, n16);
+    ReadProbeParams p;
+    p.src = (const uint4 *)d_src;
+    p.sink = (uint32_t *)d_sink;
+    p.n16 = n16;
+    MH_TIMELINE_SET(p, dev);
+    hipLaunchKernelGGL(k_read16, dim3((unsigned)grid), dim3(256), 0, dev->stream, p);
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
+}
+
+// One wavefront that stores the device's constant-rate 100 MHz counter: a time stamp inside a stream or a captured graph
+__global__ void k_timestamp(unsigned long long *out) {
+    if (threadIdx.x == 0) {
+        *out = __builtin_amdgcn_s_memrealtime();
+    }
+}
+
+int marmot_hip_timestamp(marmot_hip_device_t *dev, void *d_ticks) {
+    if (dev == nullptr || d_ticks == nullptr || (((uintptr_t)d_ticks) & 7) != 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "timestamp: null or misaligned argument");
+    }
+    hipLaunchKernelGGL(k_timestamp, dim3(1), dim3(64), 0, dev->stream, (unsigned long long *)d_ticks);
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
 }

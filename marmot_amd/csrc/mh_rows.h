@@ -17,7 +17,7 @@ typedef const __attribute__((address_space(1))) uint8_t glb_u8_t;
 // The instruction's immediate offset is added to the global address AND to the LDS address, so the KIB-th KiB of a
 // contiguous copy needs neither a new M0 nor a new address register.
 __device__ __forceinline__ void dma_set_lds_base(uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(__builtin_amdgcn_readfirstlane(lds_addr)) : "memory");
 }
 template <int KIB>
 __device__ __forceinline__ void dma16_to_lds(const uint8_t *base, uint32_t voff) {
@@ -30,6 +30,14 @@ __device__ __forceinline__ uint32_t vmcnt_now() {
     uint32_t v;
     asm volatile("s_getreg_b32 %0, hwreg(HW_REG_IB_STS)" : "=s"(v) : : "memory");
     return (v & 15u) | (((v >> 22) & 3u) << 4);
+}
+// A pointer that is the same in every lane, said so to the compiler (scalar registers)
+template <class T>
+__device__ __forceinline__ T *uniform_pointer(T *ptr) {
+    const uint64_t v = (uint64_t)(uintptr_t)ptr;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (T *)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 __device__ __forceinline__ void compiler_memory_fence() {
     asm volatile("" ::: "memory");
@@ -71,7 +79,10 @@ __device__ __forceinline__ int dot16r(const uint4 &w, const uint4 &a, int acc) {
 // is the reference's magic-number add, whose low mantissa byte IS the int8 result when |iscale * x| <= 127 (always,
 // for finite input whose maximum does not overflow 127 / max). Blocks that hold NaN / Inf, tiny maxima, or a +/- tie
 // take the exact slow path (index tracking and the reference's clamps) for the whole wavefront.
-__device__ __forceinline__ void q8k_quantize16(const float (&v)[16], int lane_in_row, uint4 &q, int &bsum, float &d) {
+// rot: the lane holds its four 4-value groups in rotated order, v[4 k + e] is value 4 ((rot + k) % 4) + e of the lane's
+// 16 (the caller read them that way to avoid LDS bank conflicts and stores word k of q at word (rot + k) % 4).
+__device__ __forceinline__ void q8k_quantize16(const float (&v)[16], int lane_in_row, uint4 &q, int &bsum, float &d,
+                                               int rot = 0) {
     int pmax = (int)0x80000000;
     uint32_t nmax = 0;
 #pragma unroll
@@ -117,10 +128,11 @@ __device__ __forceinline__ void q8k_quantize16(const float (&v)[16], int lane_in
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const float ax = fabsf(v[i]);
-        const bool gt = ax > best_abs;
+        const int idx = 16 * lane_in_row + 4 * ((rot + (i >> 2)) & 3) + (i & 3);
+        const bool gt = ax > best_abs || (ax == best_abs && ax > 0.0f && idx < best_idx);
         best_abs = gt ? ax : best_abs;
         best_val = gt ? v[i] : best_val;
-        best_idx = gt ? 16 * lane_in_row + i : best_idx;
+        best_idx = gt ? idx : best_idx;
     }
 #pragma unroll
     for (int o = 1; o < 16; o <<= 1) {

@@ -239,3 +239,69 @@ def test_loader_consumer_matvec_equals_register_streaming_matvec(oracle, name, m
         ring.close()
         streaming.close()
 
+
+
+def _special_activations(K: int) -> np.ndarray:
+    """One activation row that drives the Q8_K packer through its exact path and its corner cases, block by block:
+    +max and -max of equal magnitude in every order and lane position (first occurrence decides the sign of every
+    code), an all-zero block, a block of tiny values, a block with one huge value, ordinary blocks in between."""
+    x = gaussian(7001, (1, K))
+    nb = K // 256
+    for b in range(nb):
+        blk = x[0, b * 256:(b + 1) * 256]
+        mode = b % 8
+        if mode == 1:  # tie: +m first, then -m, positions spread over the 16-value groups of different lanes
+            m = np.float32(np.abs(blk).max() * 1.5)
+            p, q = (17 * b) % 256, (17 * b + 101) % 256
+            lo, hi = min(p, q), max(p, q)
+            blk[lo], blk[hi] = m, -m
+        elif mode == 2:  # tie: -m first
+            m = np.float32(np.abs(blk).max() * 1.25)
+            p, q = (29 * b + 3) % 256, (29 * b + 64) % 256
+            lo, hi = min(p, q), max(p, q)
+            blk[lo], blk[hi] = -m, m
+        elif mode == 3:
+            blk[:] = 0.0
+        elif mode == 4:
+            blk *= np.float32(1e-36)  # below the packer's fast-path range
+        elif mode == 5:
+            blk[(13 * b) % 256] = np.float32(-3.0e4)
+        elif mode == 6:  # tie inside one lane's 16 values, in its rotated groups
+            m = np.float32(np.abs(blk).max() * 2.0)
+            base = 16 * ((5 * b) % 16)
+            blk[base + 13], blk[base + 2] = m, -m
+    return x
+
+
+@pytest.mark.parametrize("M,K", [(4096, 14336), (4100, 14336), (14336, 4096), (14337, 4096), (4096, 11008),
+                                 (8192, 8192), (28672, 2048)])
+def test_resident_share_decode_kernel(oracle, M, K, monkeypatch):
+    """The resident-share Q4_K decode kernel (one activation row, weights of 16 MB and more, rows of up to 64 blocks):
+    whole and ragged last workgroups, one and two K segments per row, odd block counts, the Q8_K packer's exact path
+    (ties, zero and tiny blocks); against the oracle and against the ring form of the row kernel, which it replaces
+    for these shapes and whose lane mapping and summation order it keeps (bit-equal results)."""
+    from marmot_amd import HipBackend
+
+    kind = KIND_Q4_K
+    resident = HipBackend(0)
+    monkeypatch.setenv("MARMOT_HIP_NO_RESIDENT_ROWS", "1")
+    ring = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_RESIDENT_ROWS")
+    try:
+        rng = np.random.Generator(np.random.PCG64(M + K))
+        blocks = random_valid_blocks(rng, kind, M, K)
+        bias = gaussian(M, (M,))
+        for x, with_bias in ((gaussian(K, (1, K)), False), (_special_activations(K), True)):
+            got = resident.linear(x, blocks, kind, M, bias=bias if with_bias else None)
+            assert resident.last_route() == "matvec_rows2_q4_k_q8_k_fused", resident.last_route()
+            other = ring.linear(x, blocks, kind, M, bias=bias if with_bias else None)
+            assert ring.last_route() != "matvec_rows2_q4_k_q8_k_fused"
+            ref = oracle.matmul(kind, blocks, x, M, threads=THREADS)
+            if with_bias:
+                ref = ref + bias[None, :]
+            assert_matmul_parity(got, ref, what=f"resident share {M}x{K} bias={with_bias}")
+            assert_matmul_parity(other, ref, what=f"ring {M}x{K} bias={with_bias}")
+            assert np.array_equal(bits(got), bits(other)), f"{M}x{K}: resident-share and ring kernels differ"
+    finally:
+        resident.close()
+        ring.close()

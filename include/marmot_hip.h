@@ -143,19 +143,19 @@ void marmot_hip_graph_destroy(marmot_hip_device_t *dev, void *graph_exec);
 size_t marmot_hip_graph_max_nodes(void);
 size_t marmot_hip_graph_last_capture_nodes(marmot_hip_device_t *dev);
 
-/* Measurement aid, no counterpart in the reference: one launch that only reads `size` bytes at d_src (16-byte loads,
+/* DIAGNOSTIC (measurement aid, not an operator), no counterpart in the reference: one launch that only reads `size` bytes at d_src (16-byte loads,
  * nothing is written; d_sink is 1 KiB of device memory the kernel may touch only for a pattern the test data cannot
  * produce). bench.py times it beside the matvec to report the read bandwidth this box delivers to one dependent
  * launch of the same size. size and d_src must be multiples of 16. */
 int marmot_hip_read_probe(marmot_hip_device_t *dev, const void *d_src, size_t size, void *d_sink);
 
-/* Measurement aid, no counterpart in the reference: a one-wavefront kernel on the device object's stream that stores the
+/* DIAGNOSTIC (measurement aid, not an operator), no counterpart in the reference: a one-wavefront kernel on the device object's stream that stores the
  * device's constant-rate counter (100 MHz, 10 ns per tick) into the 8 bytes at d_ticks. Unlike a HIP event it can be
  * recorded into a captured graph, so a benchmark can bracket the steps of one graph replay without the submission of
  * the graph in the figure (bench.py does). */
 int marmot_hip_timestamp(marmot_hip_device_t *dev, void *d_ticks);
 
-/* Diagnostic, no counterpart in the reference: in a library built with `make TIMELINE=1` (-DMH_TIMELINE; it is
+/* DIAGNOSTIC, no counterpart in the reference: in a library built with `make TIMELINE=1` (-DMH_TIMELINE; it is
  * written to marmot_amd/lib/libmarmot_hip_timeline.so) the instrumented kernels (the row-owning Q4_K matvec, the read
  * probe) store the device's 100 MHz constant-rate counter at marked points: one 8-byte word per wavefront and mark, at
  * word (wavefront index in the launch) * 16 + mark of `d_marks` (device memory of the caller, `bytes` long; later
@@ -431,7 +431,8 @@ int marmot_hip_moe_experts(marmot_hip_device_t *dev, const float *d_hidden, size
                            const void *d_down, const int32_t *d_topk_ids, const float *d_topk_weights,
                            float weights_scale, int router_weight_policy, int ffn_type, float *d_out);
 
-/* The same call with its stages observable, for parity tests that check each stage of cpu_moe_experts_impl
+/* DIAGNOSTIC (test hook, not an operator; no counterpart in the reference's backend interface). The same call with its
+ * stages observable, for parity tests that check each stage of cpu_moe_experts_impl
  * (moe_ops.c:951-1042: gate/up projections, the quantized GLU product, down projection + combine) against a CPU
  * restatement instead of only the final sum. Every pointer may be null. Outputs are in expert-sorted route order
  * (moe_ops.c:929-943); d_route_pos[t*k + j] is the sorted position of token t's j-th route, -1 if it was dropped.

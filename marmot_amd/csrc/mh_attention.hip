@@ -43,6 +43,7 @@ struct PaParams {
     size_t scale_stride[3];
     uint32_t *new_kmax, *new_vmax;  // scratch [blocks][kv heads]: largest new magnitudes as float bits
     uint32_t *min_off;              // scratch [blocks]: first offset this call writes (block_size = untouched)
+    uint32_t *claim;                // scratch [blocks][kv heads]: the token whose workgroup rescales the block (~0 = none yet)
     uint32_t splits;    // workgroups along the history of one (token, heads) pair
     float *partial;     // splits > 1: [token][query head][split][2 + head_dim]: maximum, sum, unnormalized output
 };
@@ -248,6 +249,7 @@ __global__ __launch_bounds__(256) void k_pa_fp8_init(const PaParams p) {
     if (i < p.kv_blocks * p.num_kv_heads) {
         p.new_kmax[i] = 0u;
         p.new_vmax[i] = 0u;
+        p.claim[i] = 0xffffffffu;
     }
     if (i < p.kv_blocks) {
         p.min_off[i] = p.block_size;
@@ -294,8 +296,11 @@ __global__ __launch_bounds__(128) void k_pa_fp8_scan_new(const PaParams p) {
     }
 }
 
-// 3. per (touched block, kv head): the new scale; rows already in the block are re-encoded when it changes. The token
-//    that writes the block's first new row does the block's work, so the launch grows with the call, not the cache.
+// 3. per (touched block, kv head): the new scale; rows already in the block are re-encoded when it changes. A token
+//    that writes the block's first new row does the block's work, so the launch grows with the call, not the cache;
+//    when several tokens of a call carry that offset (the same kv_slot twice), the first workgroup to claim the block
+//    does it alone: two of them would read each other's new scale as the old one and encode the rows twice. The
+//    reference touches each block once, whatever duplicates a call holds (paged_attention_ref.c:866-946).
 __global__ __launch_bounds__(128) void k_pa_fp8_rescale(const PaParams p) {
     __shared__ float red[128];
     const uint32_t t = blockIdx.x, h = blockIdx.y;
@@ -306,6 +311,15 @@ __global__ __launch_bounds__(128) void k_pa_fp8_rescale(const PaParams p) {
     }
     const uint32_t existing = p.min_off[b];
     if ((slot & p.mask) != existing) {
+        return;
+    }
+    if (threadIdx.x == 0) {
+        red[0] = __uint_as_float(atomicCAS(p.claim + (size_t)b * p.num_kv_heads + h, 0xffffffffu, t));
+    }
+    __syncthreads();
+    const bool mine = __float_as_uint(red[0]) == 0xffffffffu;
+    __syncthreads();
+    if (!mine) {
         return;
     }
     const size_t si = (size_t)b * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] + (size_t)h * p.scale_stride[2];
@@ -687,7 +701,7 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     for (int i = 0; i < 3; ++i) {
         p.scale_stride[i] = a->scale_stride[i];
     }
-    p.new_kmax = p.new_vmax = p.min_off = nullptr;
+    p.new_kmax = p.new_vmax = p.min_off = p.claim = nullptr;
     p.flag = nullptr;
     if (validate_meta != 0 && !dev->capturing) {
         void *ws = nullptr;
@@ -706,7 +720,7 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
         }
     }
     // workspace: [fp8 scratch][partial results of split histories]
-    const size_t fp8_words = fp8 ? 2 * a->kv_blocks * a->num_kv_heads + a->kv_blocks : 0;
+    const size_t fp8_words = fp8 ? 3 * a->kv_blocks * a->num_kv_heads + a->kv_blocks : 0;
     const size_t fp8_bytes = (fp8_words * sizeof(uint32_t) + 255) & ~(size_t)255;
     // query heads per workgroup: as many heads of one key / value head as the LDS tile of the final merge allows
     const int qh_max = epl == 16 ? 2 : 4;
@@ -730,6 +744,7 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
             p.new_kmax = (uint32_t *)ws;
             p.new_vmax = p.new_kmax + a->kv_blocks * a->num_kv_heads;
             p.min_off = p.new_vmax + a->kv_blocks * a->num_kv_heads;
+            p.claim = p.min_off + a->kv_blocks;
         }
         p.partial = p.splits > 1u ? (float *)((uint8_t *)ws + fp8_bytes) : nullptr;
     }

@@ -132,6 +132,7 @@ def fp8_encode(x: np.ndarray) -> np.ndarray:
     # the reference never rounds a magnitude below the smallest normal 2^-6 up into the normal range: it clamps the
     # subnormal mantissa to 7 (src/utils/dtype_ref.c:166-174)
     pick = np.where(mag < 2.0 ** -6, np.minimum(pick, 7), pick)
+    pick = np.where(np.isnan(x), 0x79, pick)  # the reference's NaN code (no sign: `value < 0` is false for NaN)
     return (pick | np.where(x < 0, 0x80, 0)).astype(np.uint8)  # the sign of a negative value; -0.0 encodes as +0
 
 
@@ -152,7 +153,8 @@ def fp8_cache_update(case, kv, scales):
             old = np.float32(scales[b, layer, h])
             big = np.float32(0.0)
             if existing > 0 and old > 0:
-                big = np.abs(values[cache[b, layer, h, :existing]] * old).max()
+                mags = np.abs(values[cache[b, layer, h, :existing]] * old)
+                big = np.float32(np.nanmax(mags)) if np.isfinite(mags).any() else np.float32(0.0)  # NaN codes never win
             big = max(big, np.abs(new[toks, h]).max())
             scale = np.float32(big) / np.float32(240.0) if big > 0 else np.float32(1.0)
             if existing > 0 and scale != old:
@@ -162,3 +164,44 @@ def fp8_cache_update(case, kv, scales):
             for t in toks:
                 cache[b, layer, h, slots[t] % bs] = fp8_encode(new[t, h].astype(np.float32) / scale)
     return cache, scales
+
+
+def fp8_hand_cases():
+    """Three consecutive calls on ONE block of four positions, one kv head of four values, whose cache bytes and scales
+    follow from the format by hand (no restatement of the update rule is involved): every quotient value / scale lands
+    on an e4m3 value with a wide margin to its neighbours, so the last bits of the float32 divisions do not matter.
+      call 1, position 0 into the empty block: the block's scale becomes max|row| / 240 bit for bit and the row's
+              largest element encodes to +-0x77 (240);
+      call 2, position 1 twice as loud: the scale doubles and the row already there is re-encoded with it (its codes
+              halve in value), the new row's largest element is +-0x77;
+      call 3, position 2 quieter: the scale and every byte already there stay as they are.
+    Returns a list of steps: (pos, k row, v row, expected k codes [4 positions x 4], expected k scale, v codes, v scale);
+    positions not written yet keep the cache's initial zero bytes."""
+    f = np.float32
+    steps = []
+    # e4m3 codes used: 240 = 0x77, 120 = 0x6f, 80 = 0x6a, 60 = 0x67, 40 = 0x62, 30 = 0x5f, 20 = 0x5a, 160 = 0x72, 0 = 0
+    k1, v1 = [1.0, -3.0, 0.5, 0.0], [-2.0, 0.5, 0.25, 2.0]
+    sk1, sv1 = f(3.0) / f(240.0), f(2.0) / f(240.0)
+    kc1 = [[0x6A, 0xF7, 0x62, 0x00], [0] * 4, [0] * 4, [0] * 4]
+    vc1 = [[0xF7, 0x67, 0x5F, 0x77], [0] * 4, [0] * 4, [0] * 4]
+    steps.append((0, k1, v1, kc1, sk1, vc1, sv1))
+    k2, v2 = [6.0, 0.0, 0.0, -1.5], [0.0, 1.0, -4.0, 0.0]
+    sk2, sv2 = f(6.0) / f(240.0), f(4.0) / f(240.0)
+    kc2 = [[0x62, 0xEF, 0x5A, 0x00], [0x77, 0x00, 0x00, 0xE7], [0] * 4, [0] * 4]
+    vc2 = [[0xEF, 0x5F, 0x57, 0x6F], [0x00, 0x67, 0xF7, 0x00], [0] * 4, [0] * 4]
+    steps.append((1, k2, v2, kc2, sk2, vc2, sv2))
+    k3, v3 = [3.0, -0.75, 0.0, 0.0], [4.0, 0.0, -2.0, 0.0]  # v3 as loud as the block already is: same scale
+    kc3 = [kc2[0], kc2[1], [0x6F, 0xDF, 0x00, 0x00], [0] * 4]
+    vc3 = [vc2[0], vc2[1], [0x77, 0x00, 0xEF, 0x00], [0] * 4]
+    steps.append((2, k3, v3, kc3, sk2, vc3, sv2))
+    return steps
+
+
+def fp8_hand_case_arrays(pos, k_row, v_row):
+    """The arrays of one call of fp8_hand_cases (one sequence in slot 0, block 0, one q head)."""
+    meta = np.array([[0, pos, pos, 0]], dtype=np.uint32)
+    q = np.array([[[0.5, -0.25, 1.0, 0.125]]], dtype=np.float32)
+    k_new = np.array([[k_row]], dtype=np.float32)
+    v_new = np.array([[v_row]], dtype=np.float32)
+    table = np.array([[0]], dtype=np.uint32)
+    return meta, q, k_new, v_new, table

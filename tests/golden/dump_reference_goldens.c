@@ -17,6 +17,9 @@
 
 #include "backend/matmul_quantized_golden_cases.h"
 #include "backend/golden_vec_dot_llama.h"
+/* the conversion goldens of tests/backend/test_backend_conversions.c: FLOAT8_E4M3 codes and round trips */
+#define MARMOT_ENABLE_FP8 1
+#include "backend/golden_data.h"
 
 static void emit(const char *name, const char *dtype, const void *data, size_t nbytes) {
     uint32_t nl = (uint32_t)strlen(name);
@@ -116,5 +119,13 @@ int main(void) {
         snprintf(name, sizeof(name), "matmul_%s_expected_f16", c->name);
         emit(name, "f4", c->expected_f16, c->N * c->M * 4);
     }
+    /* e4m3 conversion goldens (g_conv_fp8, g_conv_fp8_half_bridge, tests/backend/golden_data.h:1859-1893) */
+    emit("g_conv_fp8_src", "f4", g_conv_fp8.src, sizeof(g_conv_fp8.src));
+    emit("g_conv_fp8_e4m3_bits", "u1", g_conv_fp8.e4m3_bits, sizeof(g_conv_fp8.e4m3_bits));
+    emit("g_conv_fp8_e4m3_roundtrip", "f4", g_conv_fp8.e4m3_roundtrip, sizeof(g_conv_fp8.e4m3_roundtrip));
+    emit("g_conv_fp8_half_bridge_src", "f4", g_conv_fp8_half_bridge.src, sizeof(g_conv_fp8_half_bridge.src));
+    emit("g_conv_fp8_half_bridge_f16_bits", "u2", g_conv_fp8_half_bridge.f16_bits, sizeof(g_conv_fp8_half_bridge.f16_bits));
+    emit("g_conv_fp8_half_bridge_fp8_bits", "u1", g_conv_fp8_half_bridge.fp8_bits, sizeof(g_conv_fp8_half_bridge.fp8_bits));
+    emit("g_conv_fp8_half_bridge_roundtrip", "f4", g_conv_fp8_half_bridge.roundtrip, sizeof(g_conv_fp8_half_bridge.roundtrip));
     return 0;
 }

@@ -300,3 +300,37 @@ def test_fp8_cache_given_codes(hip, oracle, head_dim):
         blocks = blocks[blocks != NO_BLOCK]
         vmax = np.nanmax(np.abs(vals[state["kv_v"][blocks]] * state["v_scale"][blocks][:, :, :, None, None]))
         assert vmax > 0 and np.max(np.abs(got[row].astype(np.float64) - ref[row])) <= TOLERANCE["f32"] * vmax, row
+
+
+def test_fp8_cache_update_hand_computed(hip):
+    """The hand-computed fp8 cache scenario (tests/attention_cases.py::fp8_hand_cases: first row of a block, a louder
+    row, a row that is not louder) through the HIP entry point: bytes and scale bits as computed by hand."""
+    from tests.attention_cases import fp8_hand_case_arrays, fp8_hand_cases
+
+    kv_k, kv_v = np.zeros((1, 1, 1, 4, 4), np.uint8), np.zeros((1, 1, 1, 4, 4), np.uint8)
+    ks, vs = np.zeros((1, 1, 1), np.float32), np.zeros((1, 1, 1), np.float32)
+    for pos, k_row, v_row, k_codes, k_scale, v_codes, v_scale in fp8_hand_cases():
+        meta, q, k_new, v_new, table = fp8_hand_case_arrays(pos, k_row, v_row)
+        hip.paged_attention(meta, q, k_new, v_new, kv_k, kv_v, table, 0, 0.5, kv_k_scale=ks, kv_v_scale=vs)
+        assert kv_k[0, 0, 0].tolist() == k_codes, (pos, kv_k[0, 0, 0])
+        assert kv_v[0, 0, 0].tolist() == v_codes, (pos, kv_v[0, 0, 0])
+        assert ks.view(np.uint32)[0, 0, 0] == np.float32(k_scale).view(np.uint32), (pos, ks)
+        assert vs.view(np.uint32)[0, 0, 0] == np.float32(v_scale).view(np.uint32), (pos, vs)
+
+
+def test_fp8_cache_duplicate_slot_rescales_the_block_once(hip, oracle):
+    """Two tokens of one call carry the same kv_slot (the block's first offset written): the block must be rescaled
+    exactly once, like the reference does it; scales and the rows already there against the oracle. The duplicated
+    row itself is written twice with the same scale (whichever token's values end up there is not defined)."""
+    case = _fp8_case(901, [(0, 5)], room=1, num_q_heads=2, num_kv_heads=2, head_dim=32, block_size=8)
+    state = _fp8_both(hip, oracle, case, "prefill")
+    bs = case["block_size"]
+    seq = int(case["token_meta"][0, 0])
+    slot = int(case["block_table"][seq, 0]) * bs + 5
+    meta = np.array([[seq, 5, slot, 0], [seq, 5, slot, 0]], np.uint32)
+    rng = np.random.default_rng(902)
+    row_k = rng.standard_normal((1, 2, 32), dtype=np.float32) * np.float32(8.0)  # louder than the block: it is rescaled
+    row_v = rng.standard_normal((1, 2, 32), dtype=np.float32) * np.float32(8.0)
+    step = dict(case, token_meta=meta, q=rng.standard_normal((2, 2, 32), dtype=np.float32),
+                k_new=np.repeat(row_k, 2, axis=0), v_new=np.repeat(row_v, 2, axis=0), **state)
+    _fp8_both(hip, oracle, step, "duplicate slot")

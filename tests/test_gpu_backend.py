@@ -278,19 +278,22 @@ def test_config4_layer_stack_as_one_program(ctx, oracle):
     # second execution: weights stay resident, only nothing new is uploaded
     assert ctx.execute(p) == ta.SUCCESS
     assert ctx.residency().upload_bytes == after.upload_bytes
-    # bit-exact dequantization of each weight through the DEQUANTIZE schema (one at a time: 58M..235M floats)
+    # bit-exact dequantization of EVERY row of each weight through the DEQUANTIZE schema, in bands of 2048 rows (a band
+    # is a view into the resident weight: 29M floats at a time instead of 58M .. 235M)
     for name, kind, M, K, wq, wt, yt, src in layers:
-        rows = min(M, 2048)  # the first 2048 rows of each weight; full matrices are covered by the config-2 tests
-        sub = ta.HostTensor.quantized(wq.reshape(-1)[: rows * row_bytes(kind, K)], (rows, K), kind)
-        sub.t.data = wt.t.data  # a view of the resident weight
-        dq = ta.HostTensor.empty((rows, K), ta.DTYPE_F32)
-        pd = ta.Program()
-        pd.dequantize(ctx.query(_sig_for(ta.OP_DEQUANTIZE, kind)).op_index, sub, dq)
-        assert ctx.execute(pd) == ta.SUCCESS, ctx.last_error()
-        got = ctx.to_host(dq)
-        ref = oracle.dequantize(kind, wq[:rows], K)
-        assert np.array_equal(bits(got), bits(ref)), f"dequant {name}"
-        ctx.host_freed(dq)
+        rb = row_bytes(kind, K)
+        for r0 in range(0, M, 2048):
+            rows = min(2048, M - r0)
+            sub = ta.HostTensor.quantized(wq.reshape(-1)[r0 * rb: (r0 + rows) * rb], (rows, K), kind)
+            sub.t.data = wt.t.data + r0 * rb  # a view of the resident weight
+            dq = ta.HostTensor.empty((rows, K), ta.DTYPE_F32)
+            pd = ta.Program()
+            pd.dequantize(ctx.query(_sig_for(ta.OP_DEQUANTIZE, kind)).op_index, sub, dq)
+            assert ctx.execute(pd) == ta.SUCCESS, ctx.last_error()
+            got = ctx.to_host(dq)
+            ref = oracle.dequantize(kind, wq[r0:r0 + rows], K)
+            assert np.array_equal(bits(got), bits(ref)), f"dequant {name} rows {r0}.."
+            ctx.host_freed(dq)
     for t in p.regs:
         ctx.host_freed(t)
 

@@ -95,6 +95,13 @@ def test_config3_prefill_gemm(hip, oracle, N):
     print(f"C3 N={N}: hip vs cpu floored-rel {m_floor:.3e} sum-rel {m_sum:.3e} max-norm {m_max:.3e}; "
           f"vs float64: hip {e_gpu[0]:.3e}/{e_gpu[2]:.3e}, cpu {e_cpu[0]:.3e}/{e_cpu[2]:.3e}", flush=True)
     assert m_max <= 1e-5 and m_sum <= 1e-5
+    # The floored metric max |y - r| / max(|r|, 1e-3 rms(r)) <= 1e-3 cannot be met AGAINST THE CPU at this shape: the
+    # CPU route's own sequential fp32 sum over 4096 products is 2.5e-3 .. 3.3e-3 away from exact arithmetic on that
+    # metric (outputs near zero), the HIP result 0.6e-3 .. 1.1e-3. What is asserted: the HIP result is closer to
+    # exact arithmetic than the CPU is, on that very metric, and its distance from the CPU is what the two distances
+    # from exact arithmetic explain.
+    assert e_gpu[0] <= e_cpu[0] and e_gpu[0] <= 1.5e-3, (e_gpu, e_cpu)
+    assert m_floor <= e_gpu[0] + e_cpu[0] + 1e-6, (m_floor, e_gpu, e_cpu)
     scale = np.sqrt(np.mean(ref.astype(np.float64) ** 2, axis=1, keepdims=True))
     assert np.all(np.abs(g - ref) <= 2e-5 * scale + 5e-5 * np.abs(ref))
     # the HIP result is at least as close to exact arithmetic as the CPU reference's sequential fp32 sum

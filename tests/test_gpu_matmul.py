@@ -305,3 +305,30 @@ def test_resident_share_decode_kernel(oracle, M, K, monkeypatch):
     finally:
         resident.close()
         ring.close()
+
+
+@pytest.mark.parametrize("name", ["q4_k", "q6_k"])
+def test_logits_projection_at_vocabulary_size(hip, oracle, name):
+    """The logits projection of a Llama-3 model: 128256 rows of 4096 (295 MB of Q4_K, 431 MB of Q6_K: beyond the sizes at
+    which the row-owning kernels hand over to the streaming ones), one and four activation rows, on arbitrary valid
+    block bytes (no quantizer run)."""
+    kind = KINDS[name]
+    M, K = 128256, 4096
+    rng = np.random.Generator(np.random.PCG64(128256 + kind))
+    blocks = random_valid_blocks(rng, kind, M, K)
+    d_w = hip.to_device(blocks)
+    try:
+        for N in (1, 4):
+            print(f"logits {name} {M}x{K} N={N}", flush=True)
+            x = gaussian(9000 + N, (N, K))
+            d_x = hip.to_device(x)
+            d_o = hip.alloc(N * M * 4)
+            hip.linear_d(kind, d_w, d_x, 0, N, K, M, d_o, 0)
+            got = d_o.download(np.float32, (N, M))
+            d_x.free()
+            d_o.free()
+            ref = oracle.matmul(kind, blocks, x, M, threads=THREADS)
+            m = assert_matmul_parity(got, ref, what=f"logits {name} N={N}")
+            print("   route:", hip.last_route(), "metrics:", m, flush=True)
+    finally:
+        d_w.free()

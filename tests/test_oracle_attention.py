@@ -193,3 +193,66 @@ def test_fp8_cache_prefill_then_decode_with_growing_scales(oracle):
     st, _ = oracle.paged_attention(case["token_meta"], case["q"], case["k_new"], case["v_new"], case["kv_k"].copy(),
                                    case["kv_v"].copy(), case["block_table"], 1, case["scale"])
     assert st == MO_INVALID
+
+
+def test_fp8_e4m3_reference_goldens(oracle, ref_goldens):
+    """The e4m3 vectors of the reference's own conversion test (tests/backend/test_backend_conversions.c:78-97 over
+    g_conv_fp8 and g_conv_fp8_half_bridge, tests/backend/golden_data.h:1859-1893): codes and round trips."""
+    src = ref_goldens["g_conv_fp8_src"]
+    assert [oracle.L.mo_f32_to_fp8_e4m3(float(v)) for v in src] == ref_goldens["g_conv_fp8_e4m3_bits"].tolist()
+    back = np.array([oracle.L.mo_fp8_e4m3_to_f32(int(c)) for c in ref_goldens["g_conv_fp8_e4m3_bits"]], np.float32)
+    assert np.array_equal(back, ref_goldens["g_conv_fp8_e4m3_roundtrip"])
+    half = ref_goldens["g_conv_fp8_half_bridge_f16_bits"].view(np.float16).astype(np.float32)
+    assert np.array_equal(half, ref_goldens["g_conv_fp8_half_bridge_src"])  # the f16 leg is exact for these values
+    assert [oracle.L.mo_f32_to_fp8_e4m3(float(v)) for v in half] == ref_goldens["g_conv_fp8_half_bridge_fp8_bits"].tolist()
+    back = np.array([oracle.L.mo_fp8_e4m3_to_f32(int(c)) for c in ref_goldens["g_conv_fp8_half_bridge_fp8_bits"]], np.float32)
+    assert np.array_equal(back, ref_goldens["g_conv_fp8_half_bridge_roundtrip"])
+
+
+def test_fp8_cache_update_hand_computed(oracle):
+    """The per-block scale and re-encoding rule of the fp8 cache (paged_attention_ref.c:825-989) on cases whose bytes
+    follow from the format by hand: first row of a block (scale = max / 240 bit for bit, largest element = 0x77), a
+    louder row (scale doubles, the row already there is re-encoded), a row that is not louder (nothing already there
+    changes)."""
+    from tests.attention_cases import fp8_hand_case_arrays, fp8_hand_cases
+
+    kv_k, kv_v = np.zeros((1, 1, 1, 4, 4), np.uint8), np.zeros((1, 1, 1, 4, 4), np.uint8)
+    ks, vs = np.zeros((1, 1, 1), np.float32), np.zeros((1, 1, 1), np.float32)
+    for pos, k_row, v_row, k_codes, k_scale, v_codes, v_scale in fp8_hand_cases():
+        meta, q, k_new, v_new, table = fp8_hand_case_arrays(pos, k_row, v_row)
+        st, _ = oracle.paged_attention(meta, q, k_new, v_new, kv_k, kv_v, table, 0, 0.5, kv_k_scale=ks, kv_v_scale=vs)
+        assert st == 0
+        assert kv_k[0, 0, 0].tolist() == k_codes, (pos, kv_k[0, 0, 0])
+        assert kv_v[0, 0, 0].tolist() == v_codes, (pos, kv_v[0, 0, 0])
+        assert ks.view(np.uint32)[0, 0, 0] == np.float32(k_scale).view(np.uint32), (pos, ks)
+        assert vs.view(np.uint32)[0, 0, 0] == np.float32(v_scale).view(np.uint32), (pos, vs)
+
+
+def test_fp8_cache_update_ignores_nan_codes_in_the_block_maximum(oracle):
+    """Rows already in a block may hold NaN codes (exponent field 15): the reference's maximum over the block skips
+    them (a comparison with NaN is false, paged_attention_ref.c:866-905), so the new scale comes from the finite
+    codes and the new rows; a NaN code re-encodes to the NaN code."""
+    from tests.attention_cases import fp8_cache_update
+
+    case = _fp8_case(41, [(0, 6)], num_q_heads=2, num_kv_heads=2, head_dim=16, block_size=8, layers=1, layer_idx=0)
+    st, _, kv_k, kv_v, ks, vs = run_fp8(oracle, case)
+    assert st == 0
+    seq = int(case["token_meta"][0, 0])
+    b = int(case["block_table"][seq, 0])
+    kv_k[b, 0, 0, 2, 3] = 0x7F   # NaN codes among the rows already there
+    kv_k[b, 0, 1, 4, 0] = 0xFF
+    kv_v[b, 0, 0, 1, 5] = 0x7A
+    meta = np.array([[seq, 6, b * 8 + 6, 0]], np.uint32)
+    rng = np.random.default_rng(42)
+    step = dict(case, token_meta=meta, q=rng.standard_normal((1, 2, 16), dtype=np.float32),
+                k_new=rng.standard_normal((1, 2, 16), dtype=np.float32) * np.float32(5.0),
+                v_new=rng.standard_normal((1, 2, 16), dtype=np.float32) * np.float32(5.0),
+                kv_k=kv_k, kv_v=kv_v, k_scale=ks, v_scale=vs)
+    st, _, k2, v2, ks2, vs2 = run_fp8(oracle, step)
+    assert st == 0
+    want_k, want_ks = fp8_cache_update(step, (kv_k, step["k_new"]), ks)
+    want_v, want_vs = fp8_cache_update(step, (kv_v, step["v_new"]), vs)
+    assert np.isfinite(ks2).all() and np.isfinite(vs2).all() and (ks2[b, 0] > ks[b, 0]).all()
+    assert np.array_equal(ks2, want_ks) and np.array_equal(vs2, want_vs)
+    assert np.array_equal(k2, want_k) and np.array_equal(v2, want_v)
+    assert k2[b, 0, 0, 2, 3] & 0x7F >= 0x78 and v2[b, 0, 0, 1, 5] & 0x7F >= 0x78  # still NaN codes

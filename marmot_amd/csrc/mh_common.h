@@ -253,6 +253,10 @@ struct marmot_hip_device {
     size_t static_scratch_bytes = 0;
     bool use_static_scratch = false;
     std::unordered_set<const void *> large_lds_kernels;  // kernels whose dynamic-LDS limit has been raised (under mu)
+    // SpinGuard (mh_rows.h): the device word in which a row-owning kernel records that a wavefront gave up waiting, and
+    // the polls a wavefront may spend (MARMOT_HIP_SPIN_LIMIT, read at creation)
+    uint32_t *fault_word = nullptr;
+    uint32_t spin_limit = 1u << 26;
     // Timeline build only (-DMH_TIMELINE): device buffer of the caller that instrumented kernels write their marks to
     // (marmot_hip_timeline_attach); nullptr = marks off.
     unsigned long long *timeline = nullptr;

@@ -187,6 +187,16 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
         delete dev;
         return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
     }
+    if (const char *limit = getenv("MARMOT_HIP_SPIN_LIMIT")) {
+        const long long v = atoll(limit);
+        dev->spin_limit = v < 0 ? 0u : (v > 0xffffffffll ? 0xffffffffu : (uint32_t)v);
+    }
+    if (check_hip(hipMalloc((void **)&dev->fault_word, 256), "hipMalloc(fault word)") != 0 ||
+        check_hip(hipMemset(dev->fault_word, 0, 256), "hipMemset(fault word)") != 0) {
+        (void)hipStreamDestroy(dev->stream);
+        delete dev;
+        return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
+    }
     *out_dev = dev;
     return MARMOT_HIP_SUCCESS;
 }
@@ -205,6 +215,9 @@ void marmot_hip_device_destroy(marmot_hip_device_t *dev) {
     }
     for (auto &kv : dev->allocs) {
         (void)hipFree(kv.first);
+    }
+    if (dev->fault_word != nullptr) {
+        (void)hipFree(dev->fault_word);
     }
     (void)hipStreamDestroy(dev->stream);
     delete dev;
@@ -303,6 +316,15 @@ int marmot_hip_synchronize(marmot_hip_device_t *dev) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "synchronize: null device");
     }
     MH_HIP(hipStreamSynchronize(dev->stream));
+    // a row-owning kernel whose wavefronts gave up waiting for one another (SpinGuard, mh_rows.h) has left its mark
+    uint32_t fault = 0;
+    MH_HIP(hipMemcpy(&fault, dev->fault_word, sizeof(fault), hipMemcpyDeviceToHost));
+    if (fault != 0) {
+        MH_HIP(hipMemset(dev->fault_word, 0, sizeof(fault)));
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
+                         "a row-owning kernel gave up waiting inside a workgroup (spin limit %u): its outputs are not valid",
+                         dev->spin_limit);
+    }
     return MARMOT_HIP_SUCCESS;
 }
 

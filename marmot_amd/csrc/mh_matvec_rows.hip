@@ -50,6 +50,8 @@ struct RowsParams {
     int bias_is_f16;
     int bias_first;
     int out_is_f16;
+    uint32_t *fault;      // device word for SpinGuard, and the polls a wavefront may spend
+    uint32_t spin_limit;
     MH_TIMELINE_FIELD
 };
 
@@ -96,6 +98,7 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
     constexpr int NS = 2 * G;    // 32-value sub-blocks per lane and block
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // uniform: scalar registers and branches
+    SpinGuard guard{p.spin_limit, p.fault};
     uint32_t *const ctrl = (uint32_t *)lds;
     uint32_t *const landed = ctrl + CTRL_SLOTS;
     uint32_t *const consumed = ctrl + CTRL_SLOTS + p.nslots;
@@ -235,6 +238,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
                 // still published: the consumer that frees the slot may itself be waiting for a segment of another
                 // loader that waits for a consumer of one of those.
                 while (lds_peek(consumed + slot) < gi - p.nslots + 1u) {
+                    if (!guard.spend()) {
+                        return;
+                    }
                     publish_landed();
                     __builtin_amdgcn_s_sleep(1);
                 }
@@ -339,7 +345,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
                 __atomic_fetch_add(ctrl + CTRL_XQ, 1u, __ATOMIC_RELAXED);
             }
             MH_MARK(p, 3);  // consumer: own part of the activations quantized (their loads have arrived)
-            lds_wait_at_least(ctrl + CTRL_XQ, C);
+            if (!lds_wait_at_least(ctrl + CTRL_XQ, C, guard)) {
+                return;
+            }
             MH_MARK(p, 4);  // consumer: every consumer's part is in LDS
 #pragma unroll
             for (int n = 0; n < NC; ++n) {
@@ -385,7 +393,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows_q4k(const RowsParams p) {
         }
         MH_MARK(p, 5);  // consumer: ready for its first segment
         for (uint32_t rg = wq; rg < groups; rg += wstep) {
-            lds_wait_at_least(landed + rslot, gi + 1u);
+            if (!lds_wait_at_least(landed + rslot, gi + 1u, guard)) {
+                return;
+            }
             if (rg == wq) {
                 MH_MARK(p, 6);  // consumer: first segment there
             }
@@ -647,6 +657,8 @@ int launch_matvec_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const fl
     p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
     p.bias_first = ws.bias_first ? 1 : 0;
     p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+    p.fault = dev->fault_word;
+    p.spin_limit = dev->spin_limit;
     MH_TIMELINE_SET(p, dev);
     set_route("matvec_rows_q4_k_q8_k_fused");
     const int nw = ws.count;

@@ -83,7 +83,8 @@ __global__ __launch_bounds__(1024) void k_matvec_rows2_q4k(const uint8_t *__rest
                                                           void *__restrict__ out, uint32_t M, uint32_t nb,
                                                           uint32_t rows_per_wg, uint32_t w_off, uint32_t xs_off,
                                                           uint32_t c_wait, uint32_t shape, uint32_t flags,
-                                                          const void *__restrict__ bias, uint32_t xq_off R2_TIMELINE_PARAM) {
+                                                          const void *__restrict__ bias, uint32_t xq_off, uint32_t *fault,
+                                                          uint32_t spin_limit R2_TIMELINE_PARAM) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     R2_TIMELINE_LOCAL
     MH_MARK_DECL
@@ -102,6 +103,7 @@ __global__ __launch_bounds__(1024) void k_matvec_rows2_q4k(const uint8_t *__rest
     const uint32_t rows_here = M - row0 < rows_per_wg ? M - row0 : rows_per_wg;
     const uint32_t share = rows_here * row_bytes;  // bytes this workgroup owns: one contiguous run
     const uint32_t lane16 = (uint32_t)lane * 16u;
+    SpinGuard guard{spin_limit, fault};
 
     if (wave < LOADERS) {
         // ---------------------------------------------------------------- loader
@@ -163,6 +165,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows2_q4k(const uint8_t *__rest
             if (c >= c_wait && !staging_free) {
                 // this KiB overwrites staged activations: every consumer must have taken its part
                 while (lds_peek(ctrl + CTRL_X_TAKEN) < C) {
+                    if (!guard.spend()) {
+                        return;
+                    }
                     publish();
                 }
                 staging_free = true;
@@ -277,7 +282,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows2_q4k(const uint8_t *__rest
         __atomic_fetch_add(ctrl + CTRL_XQ_DONE, 1u, __ATOMIC_RELAXED);
     }
     MH_MARK(tl, 4);  // consumer: own part quantized
-    lds_wait_at_least(ctrl + CTRL_XQ_DONE, C);
+    if (!lds_wait_at_least(ctrl + CTRL_XQ_DONE, C, guard)) {
+        return;
+    }
     MH_MARK(tl, 5);  // consumer: all parts quantized
 
     // -- 2. this lane's slice: a lane owns half a block (sub-blocks 0..3 or 4..7) at block position b of its K segment
@@ -344,6 +351,9 @@ __global__ __launch_bounds__(1024) void k_matvec_rows2_q4k(const uint8_t *__rest
                 }
                 if (__builtin_amdgcn_readfirstlane((int)ok)) {
                     break;
+                }
+                if (!guard.spend()) {
+                    return;
                 }
             }
             compiler_memory_fence();
@@ -528,12 +538,12 @@ int launch_matvec_rows2_q4k(marmot_hip_device *dev, const WeightSet &ws, const f
         MH_TRY(allow_large_lds(dev, (const void *)k_matvec_rows2_q4k<1>));
         hipLaunchKernelGGL((k_matvec_rows2_q4k<1>), grid, block, pl.lds, dev->stream, (const uint8_t *)ws.w[0], d_x_f32,
                            ws.out[0], (uint32_t)M, (uint32_t)(K / QK_K), pl.rows_per_wg, pl.w_off, pl.xs_off, pl.c_wait,
-                           shape, flags, ws.bias[0], pl.xq_off R2_TIMELINE_VALUE);
+                           shape, flags, ws.bias[0], pl.xq_off, dev->fault_word, dev->spin_limit R2_TIMELINE_VALUE);
     } else {
         MH_TRY(allow_large_lds(dev, (const void *)k_matvec_rows2_q4k<2>));
         hipLaunchKernelGGL((k_matvec_rows2_q4k<2>), grid, block, pl.lds, dev->stream, (const uint8_t *)ws.w[0], d_x_f32,
                            ws.out[0], (uint32_t)M, (uint32_t)(K / QK_K), pl.rows_per_wg, pl.w_off, pl.xs_off, pl.c_wait,
-                           shape, flags, ws.bias[0], pl.xq_off R2_TIMELINE_VALUE);
+                           shape, flags, ws.bias[0], pl.xq_off, dev->fault_word, dev->spin_limit R2_TIMELINE_VALUE);
     }
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;

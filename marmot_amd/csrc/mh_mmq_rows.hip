@@ -55,6 +55,8 @@ struct MmqRowsParams {
     uint32_t xq_off, xd_off, partial_off, ring_off;
     uint64_t div_tab;  // 4 bits per consumer: consumer / ks
     int bias_is_f16, bias_first, out_is_f16;
+    uint32_t *fault;      // device word for SpinGuard, and the polls a wavefront may spend
+    uint32_t spin_limit;
 };
 
 // control words: [0] wavefronts that stored their quantized activations, then landed[nslots], consumed[nslots],
@@ -112,6 +114,7 @@ __global__ __launch_bounds__(1024) void k_mmq_rows_q4k(const MmqRowsParams p) {
     warm_kernel_arguments<sizeof(MmqRowsParams), sizeof(MmqRowsParams)>();
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    SpinGuard guard{p.spin_limit, p.fault};
     uint32_t *const ctrl = (uint32_t *)lds;
     uint32_t *const landed = ctrl + MR_CTRL_SLOTS;
     uint32_t *const consumed = ctrl + MR_CTRL_SLOTS + p.nslots;
@@ -286,6 +289,9 @@ __global__ __launch_bounds__(1024) void k_mmq_rows_q4k(const MmqRowsParams p) {
                 // published: the consumer that frees the slot may itself be waiting for a task of another loader
                 // that waits for a consumer of one of those.
                 while (lds_peek(consumed + slot) < gi - p.nslots + 1u) {
+                    if (!guard.spend()) {
+                        return;
+                    }
                     publish_landed();
                     __builtin_amdgcn_s_sleep(1);
                 }
@@ -328,7 +334,9 @@ __global__ __launch_bounds__(1024) void k_mmq_rows_q4k(const MmqRowsParams p) {
         if ((uint32_t)wave >= TC) {
             return;  // this wavefront takes no tasks
         }
-        lds_wait_at_least(ctrl + MR_CTRL_XQ, L);  // every loader's share of the activation copy has landed
+        if (!lds_wait_at_least(ctrl + MR_CTRL_XQ, L, guard)) {  // every loader's share of the activation copy has landed
+            return;
+        }
     } else {
         // 16 values per thread and pass, every pass requested before anything else happens in this workgroup (the
         // memory pipeline serves requests in arrival order: a load behind the weight requests waits for all of them)
@@ -383,7 +391,9 @@ __global__ __launch_bounds__(1024) void k_mmq_rows_q4k(const MmqRowsParams p) {
         if ((uint32_t)wave >= TC) {
             return;  // this wavefront takes no tasks
         }
-        lds_wait_at_least(ctrl + MR_CTRL_XQ, C);
+        if (!lds_wait_at_least(ctrl + MR_CTRL_XQ, C, guard)) {
+            return;
+        }
     }
 
     // -- 2. tasks, as they land
@@ -410,7 +420,9 @@ __global__ __launch_bounds__(1024) void k_mmq_rows_q4k(const MmqRowsParams p) {
         for (uint32_t s = 0; s < p.spk; ++s) {
             const uint32_t seg = kp * p.spk + s;
             const bool exists = rgi < groups && seg < p.segs;
-            lds_wait_at_least(landed + rslot, gi + 1u);
+            if (!lds_wait_at_least(landed + rslot, gi + 1u, guard)) {
+                return;
+            }
             if (exists) {
                 const uint32_t b_first = seg * p.seg_blocks;
                 const uint32_t seg_nb = p.nb - b_first < p.seg_blocks ? p.nb - b_first : p.seg_blocks;
@@ -672,6 +684,8 @@ int launch_mmq_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float
         }
     }
     MmqRowsParams p;
+    p.fault = dev->fault_word;
+    p.spin_limit = dev->spin_limit;
     for (int i = 0; i < 3; ++i) {
         const int src = i < ws.count ? i : 0;
         p.w[i] = (const uint8_t *)ws.w[src];

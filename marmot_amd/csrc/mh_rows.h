@@ -46,11 +46,36 @@ __device__ __forceinline__ void compiler_memory_fence() {
 __device__ __forceinline__ uint32_t lds_peek(const uint32_t *word) {
     return __builtin_amdgcn_readfirstlane(__atomic_load_n(word, __ATOMIC_RELAXED));
 }
-__device__ __forceinline__ void lds_wait_at_least(const uint32_t *word, uint32_t value) {
+// Bounded spinning. The wavefronts of a row-owning kernel wait for one another through LDS words (segments landed,
+// slots read, activations quantized). Every poll takes one from the wavefront's budget; a wavefront whose budget runs
+// out waits for its own outstanding loads (they may still be writing LDS), sets a bit in a device word that the host
+// reads at the next synchronize, and leaves the kernel; the wavefronts that wait for it run out in turn. A protocol
+// error therefore ends as MARMOT_HIP_ERROR_INVALID_OPERATION instead of a hang. The default budget (2^26 polls of
+// >= 100 clocks) is seconds; MARMOT_HIP_SPIN_LIMIT sets another one when a device object is created.
+struct SpinGuard {
+    uint32_t left;
+    uint32_t *fault;
+    __device__ __forceinline__ bool spend() {  // false: the budget is gone and the fault is recorded
+        if (left != 0) {
+            --left;
+            return true;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        if ((threadIdx.x & 63u) == 0 && fault != nullptr) {
+            atomicOr(fault, 1u);
+        }
+        return false;
+    }
+};
+__device__ __forceinline__ bool lds_wait_at_least(const uint32_t *word, uint32_t value, SpinGuard &guard) {
     while (lds_peek(word) < value) {
+        if (!guard.spend()) {
+            return false;
+        }
         __builtin_amdgcn_s_sleep(1);
     }
     compiler_memory_fence();
+    return true;
 }
 
 // ---- 16-lane (one DPP row) reductions

@@ -155,6 +155,17 @@ int marmot_hip_read_probe(marmot_hip_device_t *dev, const void *d_src, size_t si
  * the graph in the figure (bench.py does). */
 int marmot_hip_timestamp(marmot_hip_device_t *dev, void *d_ticks);
 
+/* DIAGNOSTIC, no counterpart in the reference, no device needed: the launch plan of a ring kernel for a shape as plain
+ * numbers, for the host-side model that checks the loader / consumer protocol over the plan space
+ * (tests/test_rows_protocol.py). kernel 0 = ring form of the Q4_K decode row kernel (13 values: G, wavefronts, rows per
+ * workgroup, K segments, blocks per segment, rows per task, lag, pre, consumers, slots, slot bytes, grid, LDS bytes);
+ * kernel 1 = row-owning small-batch kernel (20 values: token slots, wavefronts, rows per workgroup, rows per group,
+ * blocks per task, tasks along K, consumers per row group, tasks per K part, row groups per round, rounds, task
+ * consumers, consumers, slots, slot bytes, instructions per task, lag, pre, grid, prologue lag, LDS bytes).
+ * Returns MARMOT_HIP_ERROR_NOT_IMPLEMENTED (error text untouched) for shapes the kernel does not take. */
+int marmot_hip_rows_plan_probe(int kernel, uint32_t compute_units, size_t N, size_t K, size_t M, int weights, int packed,
+                               uint32_t *out, size_t n_out);
+
 /* DIAGNOSTIC, no counterpart in the reference: in a library built with `make TIMELINE=1` (-DMH_TIMELINE; it is
  * written to marmot_amd/lib/libmarmot_hip_timeline.so) the instrumented kernels (the row-owning Q4_K matvec, the read
  * probe) store the device's 100 MHz constant-rate counter at marked points: one 8-byte word per wavefront and mark, at

@@ -102,6 +102,7 @@ SIGNATURES = {
     "marmot_hip_synchronize": (_i, [_vp]),
     "marmot_hip_read_probe": (_i, [_vp, _vp, _sz, _vp]),
     "marmot_hip_timeline_attach": (_i, [_vp, _vp, _sz]),
+    "marmot_hip_rows_plan_probe": (_i, [_i, C.c_uint32, _sz, _sz, _sz, _i, _i, C.POINTER(C.c_uint32), _sz]),
     "marmot_hip_timestamp": (_i, [_vp, _vp]),
     "marmot_hip_allocator_usage": (_i, [_vp, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "marmot_hip_stream": (_vp, [_vp]),

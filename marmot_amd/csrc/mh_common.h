@@ -400,6 +400,9 @@ int launch_matvec_set(marmot_hip_device *dev, int kind, const WeightSet &ws, con
 // it does not cover.
 int launch_matvec_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, size_t N, size_t K,
                            size_t M, int out_dtype);
+// Launch plans of the two ring kernels as numbers (no device needed): diagnostics behind marmot_hip_rows_plan_probe
+bool rows_plan_probe(uint32_t cus, size_t N, size_t K, size_t M, int nw, uint32_t *out, size_t n_out);
+bool mmq_rows_plan_probe(uint32_t cus, size_t N, size_t K, size_t M, int nw, bool packed, uint32_t *out, size_t n_out);
 // Resident-share form of the same for ONE weight and ONE activation row (mh_matvec_rows2.hip): the workgroup's rows are
 // copied into LDS once, the loaders also fetch the activation row. Same return convention.
 int launch_matvec_rows2_q4k(marmot_hip_device *dev, const WeightSet &ws, const float *d_x_f32, size_t N, size_t K,

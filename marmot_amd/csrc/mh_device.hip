@@ -383,6 +383,17 @@ int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev) {
     return MARMOT_HIP_SUCCESS;
 }
 
+int marmot_hip_rows_plan_probe(int kernel, uint32_t compute_units, size_t N, size_t K, size_t M, int weights, int packed,
+                               uint32_t *out, size_t n_out) {
+    if (out == nullptr || compute_units == 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "rows_plan_probe: null output or no compute units");
+    }
+    const bool ok = kernel == 0   ? mh::rows_plan_probe(compute_units, N, K, M, weights, out, n_out)
+                    : kernel == 1 ? mh::mmq_rows_plan_probe(compute_units, N, K, M, weights, packed != 0, out, n_out)
+                                  : false;
+    return ok ? MARMOT_HIP_SUCCESS : MARMOT_HIP_ERROR_NOT_IMPLEMENTED;
+}
+
 int marmot_hip_timeline_attach(marmot_hip_device_t *dev, void *d_marks, size_t bytes) {
     if (dev == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "timeline_attach: null device");

@@ -601,6 +601,22 @@ static bool rows_plan(const marmot_hip_device *dev, size_t N, size_t K, size_t M
     return true;
 }
 
+// The launch plan as numbers, for the host-side model of the ring protocol (tests/test_rows_protocol.py)
+bool rows_plan_probe(uint32_t cus, size_t N, size_t K, size_t M, int nw, uint32_t *out, size_t n_out) {
+    marmot_hip_device fake;
+    fake.props.multiProcessorCount = (int)cus;
+    RowsPlan pl;
+    if (n_out < 13 || !rows_plan(&fake, N, K, M, nw, pl)) {
+        return false;
+    }
+    const uint32_t v[13] = {(uint32_t)pl.G, (uint32_t)pl.W, pl.rows_per_wg, pl.segs, pl.seg_blocks, pl.rpt, pl.lag,
+                            pl.pre, pl.consumers, pl.nslots, pl.slot_stride, pl.grid, (uint32_t)pl.lds};
+    for (int i = 0; i < 13; ++i) {
+        out[i] = v[i];
+    }
+    return true;
+}
+
 template <int NC, int G>
 static int launch_rows(marmot_hip_device *dev, const RowsParams &p, const RowsPlan &pl, int nw) {
     MH_TRY(allow_large_lds(dev, (const void *)k_matvec_rows_q4k<NC, G>));

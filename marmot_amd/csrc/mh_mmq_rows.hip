@@ -650,6 +650,23 @@ static bool mmq_rows_plan(const marmot_hip_device *dev, size_t N, size_t K, size
     return true;
 }
 
+// The launch plan as numbers, for the host-side model of the ring protocol (tests/test_rows_protocol.py)
+bool mmq_rows_plan_probe(uint32_t cus, size_t N, size_t K, size_t M, int nw, bool packed, uint32_t *out, size_t n_out) {
+    marmot_hip_device fake;
+    fake.props.multiProcessorCount = (int)cus;
+    MmqRowsPlan pl;
+    if (n_out < 20 || !mmq_rows_plan(&fake, N, K, M, nw, packed, pl)) {
+        return false;
+    }
+    const uint32_t v[20] = {(uint32_t)pl.NT, pl.W, pl.rows_per_wg, pl.R, pl.seg_blocks, pl.segs, pl.ks, pl.spk,
+                            pl.rgs_per_round, pl.rounds, pl.task_consumers, pl.consumers, pl.nslots, pl.slot_stride,
+                            pl.ipt, pl.lag, pl.pre, pl.grid, pl.lag < 2u ? pl.lag : 2u, (uint32_t)pl.lds};
+    for (int i = 0; i < 20; ++i) {
+        out[i] = v[i];
+    }
+    return true;
+}
+
 template <int NT, bool PACKED>
 static int launch_mmq_rows_nt(marmot_hip_device *dev, const MmqRowsParams &p, const MmqRowsPlan &pl, int nw) {
     MH_TRY(allow_large_lds(dev, (const void *)k_mmq_rows_q4k<NT, PACKED>));
@@ -717,7 +734,7 @@ int launch_mmq_rows_q4k(marmot_hip_device *dev, const WeightSet &ws, const float
     p.ipt = pl.ipt;
     p.lag = pl.lag;
     p.pre = pl.pre;
-    p.lag_prologue = pl.lag < 2u ? pl.lag : 2u;
+    p.lag_prologue = pl.lag < 2u ? pl.lag : 2u;  // (mmq_rows_plan_probe reports the same expression)
     p.magic_row = ((1u << 20) + 9u * pl.seg_blocks - 1u) / (9u * pl.seg_blocks);
     p.xq_off = pl.xq_off;
     p.xd_off = pl.xd_off;

@@ -61,9 +61,10 @@ enum {
 enum {
     MARMOT_HIP_DTYPE_F32 = 0,
     MARMOT_HIP_DTYPE_F16 = 1,
-    MARMOT_HIP_DTYPE_BF16 = 2, /* paged attention only: activations and KV cache */
+    MARMOT_HIP_DTYPE_BF16 = 2, /* paged attention (activations and KV cache) and marmot_hip_convert */
     MARMOT_HIP_DTYPE_I32 = 3,  /* position tensors of the rotary epilogue only */
     MARMOT_HIP_DTYPE_U8 = 6,   /* storage type of block-quantized tensors (GGUF reader) */
+    MARMOT_HIP_DTYPE_U32 = 8,  /* row indices of marmot_hip_gather_rows */
     MARMOT_HIP_DTYPE_I64 = 11,
     MARMOT_HIP_DTYPE_F8_E4M3 = 14, /* paged attention only: the KV cache with per-block scales */
 };
@@ -380,6 +381,43 @@ int marmot_hip_add(marmot_hip_device_t *dev, const float *d_a, const float *d_b,
  * DIMENSION_MISMATCH. */
 int marmot_hip_rope(marmot_hip_device_t *dev, const void *d_x, int dtype, size_t rows, size_t dim,
                     size_t x_row_stride, size_t out_row_stride, const marmot_hip_rope_t *rope, void *d_out);
+
+/* ------------------------------------------------------------------ tensor operations around the linears
+ * The nodes a GGUF model graph places between its quantized linears besides the ones above (graph_builder.cpp:555-1140),
+ * so that a graph's values can stay on the device from the embedding to the logits. */
+enum {
+    MARMOT_HIP_UNARY_GELU = 0,      /* x * 0.5 * (1 + erf(x / sqrt 2)) */
+    MARMOT_HIP_UNARY_GELU_TANH = 1, /* 0.5 * x * (1 + tanh(sqrt(2 / pi) * (x + 0.044715 x^3))) */
+    MARMOT_HIP_UNARY_SILU = 2,      /* x / (1 + exp(-x)) */
+};
+/* Replaces cpu_unary_gelu / _gelu_tanh / _silu for FLOAT32 and FLOAT16 values (gelu_scalar, gelu_tanh_scalar,
+ * silu_scalar_fn, src/backends/cpu/ops/unary/scalar/unary_scalar.c:201-218): n contiguous values of `dtype`, fp32
+ * arithmetic in the reference's expression order, FLOAT16 rounded once at the store. d_out may be d_x. */
+int marmot_hip_unary(marmot_hip_device_t *dev, int op, const void *d_x, int dtype, size_t n, void *d_out);
+/* Replaces cpu_softmax_impl for FLOAT32 (src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103 ->
+ * softmax_f32_scalar.c:30-83): a contiguous tensor seen as [outer, axis, inner], normalized along `axis`
+ * (marmot_softmax_prepare, src/core/helpers/norm.c:123-179, yields the three sizes): maximum, exp(x - max) with
+ * differences at or below -88 giving exactly 0, sum, one multiplication by 1 / sum. d_out may be d_x. */
+int marmot_hip_softmax(marmot_hip_device_t *dev, const float *d_x, size_t outer, size_t axis, size_t inner,
+                       float *d_out);
+/* Replaces cpu_convert_{f32,f16,bf16}_to_{f32,f16,bf16} (src/backends/cpu/ops/convert/dtype_convert.c:17-130 and the
+ * bridges through FLOAT32, src/utils/dtype_ref.c:106-114): n contiguous values; to FLOAT16 and to BFLOAT16 round to
+ * nearest even (the reference's vector body; its scalar tail of n % 8 values truncates FLOAT16, dtype_ref.c:14-50,
+ * which is not reproduced). Equal types copy. */
+int marmot_hip_convert(marmot_hip_device_t *dev, void *d_dst, int dst_dtype, const void *d_src, int src_dtype,
+                       size_t n);
+/* Replaces cpu_gather_rows (src/backends/cpu/ops/tensor_ops/tensor_ops.c:464-547): out row r = x row idx[r * idx_stride]
+ * for r < rows_out <= 65535; rows of row_bytes bytes at the given byte strides; indices MARMOT_HIP_DTYPE_I32 or _U32.
+ * An index outside [0, rows_in) returns MARMOT_HIP_ERROR_INVALID_ARGUMENT "gather_rows index out of range" (device
+ * flag read back: one stream synchronization, skipped while a graph is being captured, where such rows are zeroed). */
+int marmot_hip_gather_rows(marmot_hip_device_t *dev, const void *d_x, size_t rows_in, size_t row_bytes,
+                           size_t in_stride_bytes, const void *d_idx, int idx_dtype, size_t idx_stride, size_t rows_out,
+                           void *d_out, size_t out_stride_bytes);
+/* Replaces cpu_slice (tensor_ops.c:401-462): the box [starts, starts + sizes) of a contiguous tensor of shape
+ * in_shape (ndim <= 8 dimensions, elements of 1, 2, 4 or 8 bytes) copied into a contiguous tensor of shape sizes.
+ * The three arrays are host memory and are read before the call returns. */
+int marmot_hip_slice(marmot_hip_device_t *dev, const void *d_x, size_t elem_size, int ndim, const size_t *in_shape,
+                     const size_t *starts, const size_t *sizes, void *d_out);
 
 /* ------------------------------------------------------------------ paged attention
  * Replaces cpu_paged_attention_impl (src/backends/cpu/ops/paged_attention/paged_attention_ref.c:573-1082; descriptor

@@ -239,6 +239,24 @@ struct marmot_topk_desc {
 };
 typedef struct marmot_topk_desc marmot_topk_desc_t;
 
+/* include/marmot/ops_types.h:189-193 */
+struct marmot_softmax_desc {
+    const marmot_tensor_t *x;
+    marmot_tensor_t *out;
+    int32_t axis;
+};
+typedef struct marmot_softmax_desc marmot_softmax_desc_t;
+
+/* include/marmot/ops_types.h:90-96 */
+struct marmot_activation_params {
+    const marmot_tensor_t *parameter_tensor;
+    const marmot_tensor_t *bias;
+    float alpha;
+    float beta;
+    float gamma;
+};
+typedef struct marmot_activation_params marmot_activation_params_t;
+
 /* include/marmot/ops_types.h:181-187 */
 struct marmot_rmsnorm_desc {
     const marmot_tensor_t *x;
@@ -389,21 +407,30 @@ typedef enum {
     MARMOT_OP_INVALID = 0,
     MARMOT_OP_QKV_PROJECTION = 191,
     MARMOT_OP_DEQUANTIZE = 210,
+    MARMOT_OP_GATHER_ROWS = 244,
+    MARMOT_OP_RESHAPE = 258,
     MARMOT_OP_MOE_EXPERTS = 263,
     MARMOT_OP_SWIGLU = 331,
+    MARMOT_OP_SILU = 352,
     MARMOT_OP_GEGLU = 410,
     MARMOT_OP_RMS_NORM_GEMMA = 447,
     MARMOT_OP_MATMUL = 498,
+    MARMOT_OP_VIEW = 502,
     MARMOT_OP_PAGED_ATTENTION = 503,
     MARMOT_OP_QUANTIZE = 524,
+    MARMOT_OP_GELU = 621,
+    MARMOT_OP_GELU_TANH = 642,
     MARMOT_OP_LINEAR = 708,
     MARMOT_OP_QKV_SHARED_INPUT = 771,
     MARMOT_OP_QKV_ROPE = 778,
+    MARMOT_OP_SLICE = 809,
     MARMOT_OP_ROPE = 843,
     MARMOT_OP_EMBEDDING = 853,
     MARMOT_OP_ADD = 876,
     MARMOT_OP_TOPK = 901,
     MARMOT_OP_RMS_NORM = 929,
+    MARMOT_OP_CONVERT = 932,
+    MARMOT_OP_SOFTMAX = 994,
     MARMOT_OP_COUNT = 995,
 } marmot_op_id_t;
 
@@ -721,7 +748,16 @@ bool marmot_hip_default_preferences(const marmot_device_caps_t *caps, marmot_bac
  *               u32 n_past; u32 n_rot                                   (bytecode_compile.c:598-623)
  *   PAGED_ATTENTION u16 token_meta, q, k_new, v_new, kv_k, kv_v, block_table, kv_k_scale, kv_v_scale (0xFFFF none),
  *               out; u32 token_count, layer_idx, num_q_heads, num_kv_heads, head_dim, block_size; f32 scale
- *                                                                       (bytecode_compile.c:553-597) */
+ *                                                                       (bytecode_compile.c:553-597)
+ *   UNARY       u16 input, output; u32 activation-params const offset (0xFFFFFFFF none)  (bytecode_compile.c:331-356)
+ *   SOFTMAX     u16 input, output; u32 axis (two's complement)          (bytecode_compile.c:440-458)
+ *   RESHAPE     u16 input, output; u32 const offset of new_ndim size_t values; u64 new_ndim   (:718-745)
+ *   VIEW        u16 input, output; u64 byte offset                      (bytecode_compile.c:746-763)
+ *   SLICE       u16 input, output; u32 const offset of starts; u32 const offset of sizes (size_t per dimension of
+ *               the output)                                              (bytecode_compile.c:863-892)
+ *   GATHER_ROWS u16 input, indices, output                              (bytecode_compile.c:893-911)
+ *   CONVERT     u32 const offset of the destination pointer; u32 const offset of the source pointer (host addresses
+ *               stored in the const pool); u64 n; u32 dst dtype; u32 src dtype   (bytecode_compile.c:1020-1043) */
 enum {
     MARMOT_HIP_BC_OP_END = 0,
     MARMOT_HIP_BC_OP_MATMUL_Q4_0 = 1,
@@ -782,7 +818,17 @@ enum {
     MARMOT_HIP_BC_OP_ROPE = 53,
     /* paged attention: cache write + attention through the block table */
     MARMOT_HIP_BC_OP_PAGED_ATTENTION = 54,
-    MARMOT_HIP_BC_OP_COUNT = 55,
+    /* the remaining nodes of a GGUF model graph: activations, router softmax, conversions, row gather, views */
+    MARMOT_HIP_BC_OP_GELU = 55,
+    MARMOT_HIP_BC_OP_GELU_TANH = 56,
+    MARMOT_HIP_BC_OP_SILU = 57,
+    MARMOT_HIP_BC_OP_SOFTMAX_F32 = 58,
+    MARMOT_HIP_BC_OP_RESHAPE = 59,
+    MARMOT_HIP_BC_OP_VIEW = 60,
+    MARMOT_HIP_BC_OP_SLICE = 61,
+    MARMOT_HIP_BC_OP_GATHER_ROWS = 62,
+    MARMOT_HIP_BC_OP_CONVERT = 63,
+    MARMOT_HIP_BC_OP_COUNT = 64,
 };
 bool marmot_hip_bc_get_tables(marmot_bc_tables_t *out);
 
@@ -880,6 +926,35 @@ marmot_error_t hip_add_f32(const void *device_ctx, const marmot_tensor_t *a, con
 marmot_error_t hip_paged_attention_impl(const void *device_ctx, const marmot_paged_attention_desc_t *desc);
 marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
                         marmot_tensor_t *out);
+/* The remaining nodes of a GGUF model graph (src/graph/gguf/graph_builder.cpp:555-1140).
+ * hip_gelu / hip_gelu_tanh / hip_silu (cf. cpu_unary_gelu_f32 and friends, src/backends/cpu/ops/unary/scalar/
+ * unary_scalar.c:201-218, 387-396): contiguous FLOAT32 or FLOAT16 tensors of equal shape; activation parameters with a
+ * bias or a parameter tensor are declined NOT_IMPLEMENTED.
+ * hip_softmax_impl (cf. cpu_softmax_impl, src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103; validation as
+ * marmot_softmax_prepare, src/core/helpers/norm.c:123-179): contiguous FLOAT32 tensors, any axis.
+ * hip_reshape / hip_view (cf. cpu_reshape, cpu_view, src/backends/cpu/ops/tensor_ops/tensor_ops.c:29-158): metadata
+ * only, no device work: the output aliases the input's host range, which the residency table resolves to the same
+ * mirror; an output buffer the tensor owned is released (and its mirror dropped) as the reference does.
+ * hip_slice (cf. cpu_slice, tensor_ops.c:401-462): contiguous tensors of up to 8 dimensions.
+ * hip_gather_rows (cf. cpu_gather_rows, tensor_ops.c:464-547): 2-D tensors with unit column stride.
+ * hip_convert (cf. cpu_convert_dispatch, src/backends/cpu/ops/convert/): n values between FLOAT32, FLOAT16 and
+ * BFLOAT16 at host addresses known to (or made known to) the residency table. */
+marmot_error_t hip_gelu(const void *device_ctx, const marmot_tensor_t *x, const marmot_activation_params_t *params,
+                        marmot_tensor_t *out);
+marmot_error_t hip_gelu_tanh(const void *device_ctx, const marmot_tensor_t *x, const marmot_activation_params_t *params,
+                             marmot_tensor_t *out);
+marmot_error_t hip_silu(const void *device_ctx, const marmot_tensor_t *x, const marmot_activation_params_t *params,
+                        marmot_tensor_t *out);
+marmot_error_t hip_softmax_impl(const void *device_ctx, const marmot_softmax_desc_t *desc);
+marmot_error_t hip_reshape(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out,
+                           const size_t *new_shape, size_t new_ndim);
+marmot_error_t hip_view(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out, size_t byte_offset);
+marmot_error_t hip_slice(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out, const size_t *starts,
+                         const size_t *sizes);
+marmot_error_t hip_gather_rows(const void *device_ctx, const marmot_tensor_t *input, const marmot_tensor_t *indices,
+                               marmot_tensor_t *out);
+marmot_error_t hip_convert(const void *device_ctx, marmot_dtype_t dst_dtype, void *dst, marmot_dtype_t src_dtype,
+                           const void *src, size_t n);
 /* output->quant_kind selects the block format: the activation formats Q8_0 and Q8_K (FLOAT32 or FLOAT16 input) or the
  * weight formats Q4_K, Q5_K and Q6_K (FLOAT32 input; cf. cpu_quantize_q4_k / _q5_k / _q6_k, quantize_core.c:199-265) */
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output);

@@ -465,6 +465,106 @@ class HipBackend:
             for b in bufs:
                 b.free()
 
+    # ---- tensor operations around the linears
+    UNARY_GELU, UNARY_GELU_TANH, UNARY_SILU = 0, 1, 2
+
+    def unary(self, op: int, x: np.ndarray, in_place: bool = False) -> np.ndarray:
+        """GELU (erf form), GELU (tanh form) or SiLU of float32 / float16 values (cpu_unary_gelu / _gelu_tanh / _silu,
+        src/backends/cpu/ops/unary/scalar/unary_scalar.c:201-218)."""
+        x = np.ascontiguousarray(x)
+        dt = {np.dtype(np.float32): capi.DT_F32, np.dtype(np.float16): capi.DT_F16}[x.dtype]
+        d_x = self.to_device(x) if x.size else None
+        d_out = d_x if in_place or not x.size else self.alloc(x.nbytes)
+        try:
+            if x.size:
+                check(self.lib.marmot_hip_unary(self.dev, op, C.c_void_p(d_x.ptr), dt, x.size, C.c_void_p(d_out.ptr)))
+                return d_out.download(x.dtype, x.shape)
+            return x.copy()
+        finally:
+            for b_ in {id(d_x): d_x, id(d_out): d_out}.values():
+                if b_ is not None:
+                    b_.free()
+
+    def softmax(self, x: np.ndarray, axis: int = -1, in_place: bool = False) -> np.ndarray:
+        """marmot_softmax of a contiguous float32 tensor along one axis (cpu_softmax_impl,
+        src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        axis = axis % x.ndim
+        outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+        inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+        if x.size == 0:
+            return x.copy()
+        d_x = self.to_device(x)
+        d_out = d_x if in_place else self.alloc(x.nbytes)
+        try:
+            check(self.lib.marmot_hip_softmax(self.dev, C.c_void_p(d_x.ptr), outer, x.shape[axis], inner,
+                                              C.c_void_p(d_out.ptr)))
+            return d_out.download(np.float32, x.shape)
+        finally:
+            d_x.free()
+            if d_out is not d_x:
+                d_out.free()
+
+    def convert(self, src: np.ndarray, src_dtype: int, dst_dtype: int) -> np.ndarray:
+        """marmot_convert between FLOAT32 (float32 arrays), FLOAT16 and BFLOAT16 (uint16 bit patterns)
+        (src/backends/cpu/ops/convert/dtype_convert.c:17-130)."""
+        src = np.ascontiguousarray(src)
+        assert src.dtype == (np.float32 if src_dtype == capi.DT_F32 else np.uint16)
+        out_np = np.float32 if dst_dtype == capi.DT_F32 else np.uint16
+        if src.size == 0:
+            return np.zeros(src.shape, out_np)
+        d_src = self.to_device(src)
+        d_dst = self.alloc(src.size * np.dtype(out_np).itemsize)
+        try:
+            check(self.lib.marmot_hip_convert(self.dev, C.c_void_p(d_dst.ptr), dst_dtype, C.c_void_p(d_src.ptr),
+                                              src_dtype, src.size))
+            return d_dst.download(out_np, src.shape)
+        finally:
+            d_src.free()
+            d_dst.free()
+
+    def gather_rows(self, x: np.ndarray, idx: np.ndarray, out_stride: int | None = None) -> np.ndarray:
+        """marmot_gather_rows (cpu_gather_rows, src/backends/cpu/ops/tensor_ops/tensor_ops.c:464-547): x is a 2-D array
+        whose rows may be a strided view (unit column stride), idx int32 or uint32. With out_stride (elements) the
+        rows land that far apart in a buffer filled with 0xFF bytes, which is returned whole as [rows, out_stride]."""
+        assert x.ndim == 2 and idx.ndim == 1 and (x.shape[1] <= 1 or x.strides[1] == x.itemsize)
+        idx = np.ascontiguousarray(idx)
+        idt = {np.dtype(np.int32): capi.DT_I32, np.dtype(np.uint32): capi.DT_U32}[idx.dtype]
+        rows_in, cols = x.shape
+        in_stride = x.strides[0] // x.itemsize if rows_in > 1 else cols
+        span = ((rows_in - 1) * in_stride + cols) if rows_in else 0
+        flat = np.lib.stride_tricks.as_strided(x, shape=(span,), strides=(x.itemsize,)) if span else x.reshape(-1)
+        ostride = cols if out_stride is None else out_stride
+        n_out = idx.shape[0]
+        if n_out == 0 or cols == 0:
+            return np.zeros((n_out, ostride), x.dtype)
+        out_host = np.full((n_out, ostride), 0xFF, np.uint8).repeat(x.itemsize, axis=1).view(x.dtype)
+        bufs = [self.to_device(np.ascontiguousarray(flat)), self.to_device(idx), self.to_device(out_host)]
+        try:
+            check(self.lib.marmot_hip_gather_rows(self.dev, C.c_void_p(bufs[0].ptr), rows_in, cols * x.itemsize,
+                                                  in_stride * x.itemsize, C.c_void_p(bufs[1].ptr), idt, 1, n_out,
+                                                  C.c_void_p(bufs[2].ptr), ostride * x.itemsize))
+            return bufs[2].download(x.dtype, (n_out, ostride))
+        finally:
+            for b_ in bufs:
+                b_.free()
+
+    def slice(self, x: np.ndarray, starts, sizes) -> np.ndarray:
+        """marmot_slice (cpu_slice, tensor_ops.c:401-462): the box [starts, starts + sizes) of a contiguous array."""
+        x = np.ascontiguousarray(x)
+        n = x.ndim
+        out = np.zeros(tuple(int(v) for v in sizes), x.dtype)
+        arr = lambda v: (C.c_size_t * n)(*[int(i) for i in v])
+        d_x = self.to_device(x) if x.size else self.alloc(16)
+        d_out = self.alloc(max(out.nbytes, 16))
+        try:
+            check(self.lib.marmot_hip_slice(self.dev, C.c_void_p(d_x.ptr), x.itemsize, n, arr(x.shape), arr(starts),
+                                            arr(sizes), C.c_void_p(d_out.ptr)))
+            return d_out.download(x.dtype, out.shape) if out.size else out
+        finally:
+            d_x.free()
+            d_out.free()
+
     def add(self, a: np.ndarray, b: np.ndarray) -> np.ndarray:
         a = np.ascontiguousarray(a, dtype=np.float32)
         b = np.ascontiguousarray(b, dtype=np.float32)

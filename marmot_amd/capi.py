@@ -11,7 +11,8 @@ KIND_Q4_1, KIND_Q5_0, KIND_Q5_1 = 2, 3, 4
 KIND_Q2_K, KIND_Q3_K = 7, 8
 KIND_Q8_1 = 6
 DT_F32, DT_F16 = 0, 1
-DT_BF16 = 2  # paged attention only
+DT_BF16 = 2  # paged attention and conversions
+DT_U32 = 8  # row indices of gather_rows
 DT_F8_E4M3 = 14  # paged attention only: the KV cache
 DT_I32, DT_I64 = 3, 11  # position tensors of the rotary epilogue
 FLAG_FORCE_PACK = 1
@@ -143,6 +144,11 @@ SIGNATURES = {
     "marmot_hip_swiglu_pack": (_i, [_vp, _vp, _vp, _sz, _sz, _i, _vp]),
     "marmot_hip_add": (_i, [_vp, _vp, _vp, _sz, _vp]),
     "marmot_hip_rope": (_i, [_vp, _vp, _i, _sz, _sz, _sz, _sz, C.POINTER(Rope), _vp]),
+    "marmot_hip_unary": (_i, [_vp, _i, _vp, _i, _sz, _vp]),
+    "marmot_hip_softmax": (_i, [_vp, _vp, _sz, _sz, _sz, _vp]),
+    "marmot_hip_convert": (_i, [_vp, _vp, _i, _vp, _i, _sz]),
+    "marmot_hip_gather_rows": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _i, _sz, _sz, _vp, _sz]),
+    "marmot_hip_slice": (_i, [_vp, _vp, _sz, _i, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), _vp]),
     "marmot_hip_paged_attention": (_i, [_vp, C.POINTER(PagedAttention), _i]),
     "marmot_hip_topk": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _vp]),
     "marmot_hip_softmax_rows": (_i, [_vp, _vp, _sz, _sz, _vp]),

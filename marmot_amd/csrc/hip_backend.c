@@ -1893,6 +1893,442 @@ static marmot_error_t paged_attention(const void *device_ctx, const marmot_paged
     return st;
 }
 
+// ------------------------------------------------------------------ the remaining nodes of a model graph
+// bytes a tensor occupies (marmot_tensor_size_bytes, src/core/tensor/metadata.c:74-146): block-quantized tensors of
+// two or more dimensions by rows of blocks (for ranks other than two the first dimension is the row length)
+static size_t tensor_storage_bytes(const marmot_tensor_t *t) {
+    const size_t n = tensor_numel(t);
+    if (n == 0) {
+        return 0;
+    }
+    if (kind_is_block(t->quant_kind) && t->quant_layout == MARMOT_QUANT_LAYOUT_GGUF && t->shape.ndim >= 2) {
+        size_t rows, inner;
+        if (t->shape.ndim == 2) {
+            rows = t->shape.shape[0];
+            inner = t->shape.shape[1];
+        } else {
+            inner = t->shape.shape[0];
+            rows = n / inner;
+        }
+        return rows * marmot_hip_row_bytes((int)t->quant_kind, inner);
+    }
+    if (t->dtype == MARMOT_DTYPE_INT4 || t->dtype == MARMOT_DTYPE_UINT4) {
+        return (n + 1) / 2;
+    }
+    return n * dtype_size(t->dtype);
+}
+
+static bool same_shape(const marmot_tensor_t *a, const marmot_tensor_t *c) {
+    if (a->shape.ndim != c->shape.ndim) {
+        return false;
+    }
+    for (size_t i = 0; i < a->shape.ndim; ++i) {
+        if (a->shape.shape[i] != c->shape.shape[i]) {
+            return false;
+        }
+    }
+    return true;
+}
+
+static void ops_on_host_ptr_freed(void *device_ctx, const void *ptr);
+
+// the output takes over the input's storage: what the alias-making operations share (tensor_ops.c:74-89, 138-155)
+static void alias_storage(const marmot_tensor_t *x, marmot_tensor_t *out, size_t byte_offset) {
+    out->data = (uint8_t *)x->data + byte_offset;
+    out->capacity_bytes = x->capacity_bytes > byte_offset ? x->capacity_bytes - byte_offset : 0;
+    out->owns_data = false;
+    out->quant_params = x->quant_params;
+    out->quant_kind = x->quant_kind;
+    out->quant_layout = x->quant_layout;
+    out->backend = x->backend;
+    out->memory_location = x->memory_location;
+    out->needs_sync = x->needs_sync;
+    out->packed_data = nullptr;
+    out->packed_src_data = nullptr;
+    out->packed_bytes = 0;
+    out->packed_row_bytes = 0;
+    out->packed_rows = 0;
+}
+
+// marmot_reshape (cpu_reshape, src/backends/cpu/ops/tensor_ops/tensor_ops.c:29-91): metadata only. The output aliases
+// the input's host bytes; the residency table resolves both to one mirror, so nothing moves on the device either.
+static marmot_error_t reshape(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out,
+                              const size_t *new_shape, size_t new_ndim) {
+    if (x == nullptr || out == nullptr || new_shape == nullptr || new_ndim == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null pointer in reshape");
+    }
+    if (new_ndim > MARMOT_MAX_DIMS) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Reshape rank exceeds the tensor rank limit");
+    }
+    size_t new_elements = 1;
+    for (size_t i = 0; i < new_ndim; ++i) {
+        new_elements *= new_shape[i];
+    }
+    if (tensor_numel(x) != new_elements) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Reshape element count mismatch");
+    }
+    if (out->owns_data && out->data != nullptr && out->data != x->data) {
+        ops_on_host_ptr_freed((void *)device_ctx, out->data);
+        free(out->data);
+    }
+    out->shape.ndim = new_ndim;
+    for (size_t i = 0; i < new_ndim; ++i) {
+        out->shape.shape[i] = new_shape[i];
+    }
+    bool has_stride = false;
+    for (size_t i = 0; i < new_ndim; ++i) {
+        if (out->shape.strides[i] != 0) {
+            has_stride = true;
+            break;
+        }
+    }
+    if (!has_stride) {
+        out->shape.strides[new_ndim - 1] = 1;
+        for (size_t i = new_ndim - 1; i-- > 0;) {
+            out->shape.strides[i] = out->shape.strides[i + 1] * out->shape.shape[i + 1];
+        }
+    }
+    out->dtype = x->dtype;
+    alias_storage(x, out, 0);
+    out->capacity_bytes = x->capacity_bytes;
+    return MARMOT_SUCCESS;
+}
+
+// marmot_view (cpu_view, tensor_ops.c:93-158): metadata only, checks in the reference's order
+static marmot_error_t view(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out, size_t byte_offset) {
+    if (x == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null pointer in view");
+    }
+    if (x->dtype != out->dtype) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "View requires matching dtypes");
+    }
+    if (x->backend != out->backend) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "View requires matching backends");
+    }
+    const size_t elem_size = dtype_size(x->dtype);
+    if (elem_size != 0 && (byte_offset % elem_size) != 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "View byte offset must align to dtype size");
+    }
+    marmot_tensor_t probe = *out;
+    probe.quant_kind = x->quant_kind;
+    probe.quant_layout = x->quant_layout;
+    const size_t out_bytes = tensor_storage_bytes(&probe);
+    if (x->capacity_bytes < byte_offset) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "View byte offset exceeds input capacity");
+    }
+    if (out_bytes > x->capacity_bytes - byte_offset) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "View exceeds input capacity");
+    }
+    if (out_bytes != 0 && x->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "View requires non-null input data");
+    }
+    if (out->owns_data && out->data != nullptr) {
+        ops_on_host_ptr_freed((void *)device_ctx, out->data);
+        free(out->data);
+    }
+    if (out->packed_data != nullptr) {
+        free(out->packed_data);
+    }
+    if (out->quant_params != nullptr && out->quant_params != x->quant_params) {
+        free(out->quant_params);
+    }
+    alias_storage(x, out, byte_offset);
+    return MARMOT_SUCCESS;
+}
+
+// marmot_slice (cpu_slice, tensor_ops.c:401-462): the box [starts, starts + sizes) of a contiguous tensor. The
+// reference walks the shapes, not the strides, and does not check the box; here a box outside the input and an output
+// whose shape is not `sizes` are errors.
+static marmot_error_t slice(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out,
+                            const size_t *starts, const size_t *sizes) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || x == nullptr || out == nullptr || starts == nullptr || sizes == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null pointer in slice");
+    }
+    const size_t ndim = x->shape.ndim;
+    if (ndim == 0) {
+        return MARMOT_SUCCESS;
+    }
+    if (ndim > 8 || out->shape.ndim != ndim) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Slice input and output ranks must match (at most 8)");
+    }
+    if (x->dtype != out->dtype) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Slice requires matching input/output dtypes");
+    }
+    const size_t elem_size = dtype_size(x->dtype);
+    if (elem_size == 0 || kind_is_block(x->quant_kind)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP slice handles dense element types");
+    }
+    for (size_t d = 0; d < ndim; ++d) {
+        if (out->shape.shape[d] != sizes[d]) {
+            return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Slice output shape must equal the slice sizes");
+        }
+        if (starts[d] > x->shape.shape[d] || sizes[d] > x->shape.shape[d] - starts[d]) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Slice box lies outside the input");
+        }
+    }
+    if (!dense_contiguous(x) || !dense_contiguous(out)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP slice needs contiguous tensors");
+    }
+    if (tensor_numel(out) == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+    if (x->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Slice: tensor without data");
+    }
+    pthread_mutex_lock(&b->mu);
+    hip_acq_t acq[2] = {
+        {x->data, dense_bytes(x), HIP_ACQ_READ, nullptr},
+        {out->data, dense_bytes(out), HIP_ACQ_WRITE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 2);
+    if (st == MARMOT_SUCCESS) {
+        const int rc = marmot_hip_slice(b->dev, acq[0].dev, elem_size, (int)ndim, x->shape.shape, starts, sizes, acq[1].dev);
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
+// marmot_gather_rows (cpu_gather_rows, tensor_ops.c:464-547): checks in the reference's order; rows with unit column
+// stride (the reference also walks column strides)
+static marmot_error_t gather_rows(const void *device_ctx, const marmot_tensor_t *input, const marmot_tensor_t *indices,
+                                  marmot_tensor_t *out) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || input == nullptr || indices == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null pointer in gather_rows");
+    }
+    if (input->shape.ndim != 2 || out->shape.ndim != 2) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "gather_rows expects 2D input/output tensors");
+    }
+    if (indices->shape.ndim != 1) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "gather_rows indices must be 1D");
+    }
+    if (input->dtype != out->dtype) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "gather_rows requires matching input/output dtypes");
+    }
+    const size_t rows_in = input->shape.shape[0], cols = input->shape.shape[1], rows_out = out->shape.shape[0];
+    if (rows_out != indices->shape.shape[0] || cols != out->shape.shape[1]) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "gather_rows output shape mismatch");
+    }
+    if (rows_out == 0 || cols == 0) {
+        return MARMOT_SUCCESS;
+    }
+    const size_t elem_size = dtype_size(input->dtype);
+    if (elem_size == 0) {
+        return MARMOT_SUCCESS;
+    }
+    if (input->data == nullptr || out->data == nullptr || indices->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "gather_rows requires non-null tensor data");
+    }
+    if (indices->dtype != MARMOT_DTYPE_INT32 && indices->dtype != MARMOT_DTYPE_UINT32) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "gather_rows indices dtype unsupported");
+    }
+    if (kind_is_block(input->quant_kind)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP gather_rows handles dense element types");
+    }
+    const size_t in_s0 = input->shape.strides[0], out_s0 = out->shape.strides[0], idx_s0 = indices->shape.strides[0];
+    if ((cols != 1 && (input->shape.strides[1] != 1 || out->shape.strides[1] != 1)) || (rows_in > 1 && in_s0 < cols) ||
+        (rows_out > 1 && out_s0 < cols)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP gather_rows needs rows with unit column stride");
+    }
+    if (rows_in == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "gather_rows index out of range");
+    }
+    const size_t row_bytes = cols * elem_size;
+    const size_t in_span = ((rows_in - 1) * in_s0 + cols) * elem_size;
+    const size_t out_span = ((rows_out - 1) * out_s0 + cols) * elem_size;
+    const size_t idx_span = ((rows_out - 1) * idx_s0 + 1) * 4;
+    pthread_mutex_lock(&b->mu);
+    hip_acq_t acq[3] = {
+        {input->data, in_span, HIP_ACQ_READ, nullptr},
+        {indices->data, idx_span, HIP_ACQ_READ, nullptr},
+        {out->data, out_span, out_s0 == cols || rows_out == 1 ? HIP_ACQ_WRITE : HIP_ACQ_UPDATE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 3);
+    // the library takes at most 65535 rows per call
+    for (size_t r0 = 0; st == MARMOT_SUCCESS && r0 < rows_out; r0 += 65535) {
+        const size_t n = rows_out - r0 < 65535 ? rows_out - r0 : 65535;
+        const int rc = marmot_hip_gather_rows(
+            b->dev, acq[0].dev, rows_in, row_bytes, in_s0 * elem_size, (const uint8_t *)acq[1].dev + r0 * idx_s0 * 4,
+            indices->dtype == MARMOT_DTYPE_INT32 ? MARMOT_HIP_DTYPE_I32 : MARMOT_HIP_DTYPE_U32, idx_s0, n,
+            (uint8_t *)acq[2].dev + r0 * out_s0 * elem_size, out_s0 * elem_size);
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
+// marmot_softmax (cpu_softmax_impl, src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103; marmot_softmax_prepare,
+// src/core/helpers/norm.c:123-179, checks in its order): FLOAT32, contiguous, any axis
+static marmot_error_t softmax(const void *device_ctx, const marmot_softmax_desc_t *desc) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (desc == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax descriptor is null");
+    }
+    if (desc->x == nullptr || desc->out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax input or output is null");
+    }
+    if (b == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "HIP context is null for softmax");
+    }
+    const marmot_tensor_t *x = desc->x;
+    marmot_tensor_t *out = desc->out;
+    if (x->dtype != out->dtype) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Softmax input and output dtype mismatch");
+    }
+    if (!same_shape(x, out)) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Softmax input/output shape mismatch");
+    }
+    if (x->shape.ndim == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax requires at least 1D tensor");
+    }
+    int axis = desc->axis;
+    if (axis < 0) {
+        axis += (int)x->shape.ndim;
+    }
+    if (axis < 0 || axis >= (int)x->shape.ndim) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax axis out of range");
+    }
+    const size_t axis_size = x->shape.shape[axis];
+    if (axis_size == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax axis dimension must be non-zero");
+    }
+    size_t inner = 1;
+    for (size_t i = (size_t)axis + 1; i < x->shape.ndim; ++i) {
+        inner *= x->shape.shape[i];
+    }
+    if (axis_size * inner == 0) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax row extent is zero");
+    }
+    const size_t total = tensor_numel(x);
+    const size_t outer = total / (axis_size * inner);
+    if (x->dtype != MARMOT_DTYPE_FLOAT32) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP softmax handles FLOAT32 tensors");
+    }
+    if (!dense_contiguous(x) || !dense_contiguous(out)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP softmax needs contiguous tensors");
+    }
+    if (total == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+    if (x->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Softmax: tensor without data");
+    }
+    pthread_mutex_lock(&b->mu);
+    hip_acq_t acq[2] = {
+        {x->data, dense_bytes(x), HIP_ACQ_READ, nullptr},
+        {out->data, dense_bytes(out), HIP_ACQ_WRITE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 2);
+    if (st == MARMOT_SUCCESS) {
+        const int rc = marmot_hip_softmax(b->dev, (const float *)acq[0].dev, outer, axis_size, inner, (float *)acq[1].dev);
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
+// GELU (erf form), GELU (tanh form), SiLU of contiguous FLOAT32 / FLOAT16 tensors (cpu_unary_{gelu,gelu_tanh,silu}_*,
+// src/backends/cpu/ops/unary/scalar/unary_scalar.c:201-218, 387-396)
+static marmot_error_t unary(const void *device_ctx, int op, const marmot_tensor_t *x,
+                            const marmot_activation_params_t *params, marmot_tensor_t *out) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || x == nullptr || out == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Unary operation: null tensor");
+    }
+    if (params != nullptr && (params->bias != nullptr || params->parameter_tensor != nullptr)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP unary operations take no bias or parameter tensor");
+    }
+    if (x->dtype != out->dtype) {
+        return fail(MARMOT_ERROR_UNSUPPORTED_DTYPE, "Unary operation: input and output dtype mismatch");
+    }
+    if (!same_shape(x, out)) {
+        return fail(MARMOT_ERROR_DIMENSION_MISMATCH, "Unary operation: shapes do not match");
+    }
+    if (x->dtype != MARMOT_DTYPE_FLOAT32 && x->dtype != MARMOT_DTYPE_FLOAT16) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP unary operations handle FLOAT32 and FLOAT16 tensors");
+    }
+    if (!dense_contiguous(x) || !dense_contiguous(out)) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP unary operations need contiguous tensors");
+    }
+    const size_t n = tensor_numel(x);
+    if (n == 0) {
+        mark_device_output(out);
+        return MARMOT_SUCCESS;
+    }
+    if (x->data == nullptr || out->data == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Unary operation: tensor without data");
+    }
+    pthread_mutex_lock(&b->mu);
+    hip_acq_t acq[2] = {
+        {x->data, dense_bytes(x), HIP_ACQ_READ, nullptr},
+        {out->data, dense_bytes(out), HIP_ACQ_WRITE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 2);
+    if (st == MARMOT_SUCCESS) {
+        const int rc = marmot_hip_unary(b->dev, op, acq[0].dev,
+                                        x->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32 : MARMOT_HIP_DTYPE_F16, n,
+                                        acq[1].dev);
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    pthread_mutex_unlock(&b->mu);
+    if (st == MARMOT_SUCCESS) {
+        mark_device_output(out);
+    }
+    return st;
+}
+
+// marmot_convert between FLOAT32, FLOAT16 and BFLOAT16 (src/backends/cpu/ops/convert/dtype_convert.c). The operation
+// names host addresses, not tensors, so no tensor can be marked "device copy is newer": outside a graph batch the
+// destination's host bytes are brought up to date before the call returns; inside a batch (whose values are consumed by
+// later nodes on the device) the device copy stays the current one, like any node's output.
+static marmot_error_t convert(const void *device_ctx, marmot_dtype_t dst_dtype, void *dst, marmot_dtype_t src_dtype,
+                              const void *src, size_t n) {
+    hip_backend_t *b = backend_of(device_ctx);
+    if (b == nullptr || dst == nullptr || src == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Convert: null argument");
+    }
+    const bool src_ok = src_dtype == MARMOT_DTYPE_FLOAT32 || src_dtype == MARMOT_DTYPE_FLOAT16 ||
+        src_dtype == MARMOT_DTYPE_BFLOAT16;
+    const bool dst_ok = dst_dtype == MARMOT_DTYPE_FLOAT32 || dst_dtype == MARMOT_DTYPE_FLOAT16 ||
+        dst_dtype == MARMOT_DTYPE_BFLOAT16;
+    if (!src_ok || !dst_ok) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP convert handles FLOAT32, FLOAT16 and BFLOAT16");
+    }
+    if (n == 0) {
+        return MARMOT_SUCCESS;
+    }
+    const size_t src_bytes = n * dtype_size(src_dtype), dst_bytes = n * dtype_size(dst_dtype);
+    pthread_mutex_lock(&b->mu);
+    hip_acq_t acq[2] = {
+        {(void *)src, src_bytes, HIP_ACQ_READ, nullptr},
+        {dst, dst_bytes, HIP_ACQ_WRITE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 2);
+    if (st == MARMOT_SUCCESS) {
+        // marmot_dtype_t and the library's dtype codes agree for these three types
+        const int rc = marmot_hip_convert(b->dev, acq[1].dev, (int)dst_dtype, acq[0].dev, (int)src_dtype, n);
+        st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
+    }
+    if (st == MARMOT_SUCCESS && !b->batching) {
+        st = make_host_current_locked(b, dst, dst_bytes);
+    }
+    pthread_mutex_unlock(&b->mu);
+    return st;
+}
+
 static uint16_t rd_u16(const uint8_t **pc) {
     const uint16_t v = (uint16_t)((*pc)[0] | ((*pc)[1] << 8));
     *pc += 2;
@@ -2256,6 +2692,174 @@ static marmot_error_t bc_exec_paged_attention(const void *exec_ctx, marmot_tenso
     return paged_attention(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
 }
 
+static uint64_t rd_u64(const uint8_t **pc) {
+    const uint64_t lo = rd_u32(pc);
+    const uint64_t hi = rd_u32(pc);
+    return lo | (hi << 32);
+}
+
+// data of the const pool at an offset (marmot_bc_const_data, src/core/bytecode/bytecode.h): nullptr for "none"
+static const void *const_data(const uint8_t *const_pool, uint32_t off) {
+    return off == MARMOT_BC_INVALID_OFFSET || const_pool == nullptr ? nullptr : const_pool + off;
+}
+
+// UNARY: u16 input, output; u32 activation-params const offset (bytecode_compile.c:331-356)
+static marmot_error_t bc_exec_unary(int op, const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                    const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *x = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    const uint32_t params_off = rd_u32(&pc);
+    marmot_activation_params_t params;
+    const marmot_activation_params_t *params_ptr = nullptr;
+    if (params_off != MARMOT_BC_INVALID_OFFSET) {
+        if (const_pool == nullptr) {
+            return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for unary params");
+        }
+        memcpy(&params, const_pool + params_off, sizeof(params));
+        params_ptr = &params;
+    }
+    return unary(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, op, x, params_ptr, out);
+}
+
+static marmot_error_t bc_exec_gelu(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                   const uint8_t *const_pool) {
+    return bc_exec_unary(MARMOT_HIP_UNARY_GELU, exec_ctx, regs, imm, const_pool);
+}
+
+static marmot_error_t bc_exec_gelu_tanh(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                        const uint8_t *const_pool) {
+    return bc_exec_unary(MARMOT_HIP_UNARY_GELU_TANH, exec_ctx, regs, imm, const_pool);
+}
+
+static marmot_error_t bc_exec_silu(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                   const uint8_t *const_pool) {
+    return bc_exec_unary(MARMOT_HIP_UNARY_SILU, exec_ctx, regs, imm, const_pool);
+}
+
+// SOFTMAX: u16 input, output; u32 axis (bytecode_compile.c:440-458)
+static marmot_error_t bc_exec_softmax(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                      const uint8_t *const_pool) {
+    (void)const_pool;
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    marmot_softmax_desc_t desc = {0};
+    desc.x = reg(regs, rd_u16(&pc));
+    desc.out = reg(regs, rd_u16(&pc));
+    desc.axis = (int32_t)rd_u32(&pc);
+    return softmax(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, &desc);
+}
+
+// RESHAPE: u16 input, output; u32 const offset of the new shape; u64 new_ndim (bytecode_compile.c:718-745)
+static marmot_error_t bc_exec_reshape(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                      const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *x = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    const uint32_t shape_off = rd_u32(&pc);
+    const uint64_t ndim = rd_u64(&pc);
+    if (shape_off != MARMOT_BC_INVALID_OFFSET && const_pool == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for reshape shape");
+    }
+    if (ndim > MARMOT_MAX_DIMS) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Reshape rank exceeds the tensor rank limit");
+    }
+    size_t shape[MARMOT_MAX_DIMS] = {0};
+    const void *src = const_data(const_pool, shape_off);
+    if (src != nullptr) {
+        memcpy(shape, src, (size_t)ndim * sizeof(size_t));
+    }
+    return reshape(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, x, out, src != nullptr ? shape : nullptr,
+                   (size_t)ndim);
+}
+
+// VIEW: u16 input, output; u64 byte offset (bytecode_compile.c:746-763)
+static marmot_error_t bc_exec_view(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                   const uint8_t *const_pool) {
+    (void)const_pool;
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *x = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    const uint64_t byte_offset = rd_u64(&pc);
+    return view(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, x, out, (size_t)byte_offset);
+}
+
+// SLICE: u16 input, output; u32 const offsets of starts and sizes, one size_t per output dimension
+// (bytecode_compile.c:863-892)
+static marmot_error_t bc_exec_slice(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                    const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *x = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    const uint32_t starts_off = rd_u32(&pc);
+    const uint32_t sizes_off = rd_u32(&pc);
+    if ((starts_off != MARMOT_BC_INVALID_OFFSET || sizes_off != MARMOT_BC_INVALID_OFFSET) && const_pool == nullptr) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for slice starts");
+    }
+    size_t starts[MARMOT_MAX_DIMS] = {0}, sizes[MARMOT_MAX_DIMS] = {0};
+    const void *s0 = const_data(const_pool, starts_off), *s1 = const_data(const_pool, sizes_off);
+    const size_t ndim = out != nullptr && out->shape.ndim <= MARMOT_MAX_DIMS ? out->shape.ndim : 0;
+    if (s0 != nullptr) {
+        memcpy(starts, s0, ndim * sizeof(size_t));
+    }
+    if (s1 != nullptr) {
+        memcpy(sizes, s1, ndim * sizeof(size_t));
+    }
+    return slice(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, x, out, s0 != nullptr ? starts : nullptr,
+                 s1 != nullptr ? sizes : nullptr);
+}
+
+// GATHER_ROWS: u16 input, indices, output (bytecode_compile.c:893-911)
+static marmot_error_t bc_exec_gather_rows(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                          const uint8_t *const_pool) {
+    (void)const_pool;
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const marmot_tensor_t *x = reg(regs, rd_u16(&pc));
+    const marmot_tensor_t *idx = reg(regs, rd_u16(&pc));
+    marmot_tensor_t *out = reg(regs, rd_u16(&pc));
+    return gather_rows(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, x, idx, out);
+}
+
+// CONVERT: u32 const offsets of the destination and source host addresses; u64 n; u32 dst dtype; u32 src dtype
+// (bytecode_compile.c:1020-1043; the addresses are stored by value, marmot_bc_add_const_ptr_value :88)
+static marmot_error_t bc_exec_convert(const void *exec_ctx, marmot_tensor_t **regs, const uint8_t *imm,
+                                      const uint8_t *const_pool) {
+    if (!exec_args_ok(exec_ctx, regs, imm)) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null bytecode exec arguments");
+    }
+    const uint8_t *pc = imm;
+    const uint32_t dst_off = rd_u32(&pc);
+    const uint32_t src_off = rd_u32(&pc);
+    const uint64_t n = rd_u64(&pc);
+    const marmot_dtype_t dst_dtype = (marmot_dtype_t)rd_u32(&pc);
+    const marmot_dtype_t src_dtype = (marmot_dtype_t)rd_u32(&pc);
+    if (const_pool == nullptr || dst_off == MARMOT_BC_INVALID_OFFSET || src_off == MARMOT_BC_INVALID_OFFSET) {
+        return fail(MARMOT_ERROR_INVALID_ARGUMENT, "Null const pool for convert dst");
+    }
+    void *dst = nullptr;
+    const void *src = nullptr;
+    memcpy(&dst, const_pool + dst_off, sizeof(dst));
+    memcpy(&src, const_pool + src_off, sizeof(src));
+    return convert(((const marmot_bc_exec_ctx_t *)exec_ctx)->device_ctx, dst_dtype, dst, src_dtype, src, (size_t)n);
+}
+
 static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     0,               // END
     12, 12, 12, 12,  // MATMUL: 3 x u16 + u32 + u16
@@ -2276,6 +2880,13 @@ static const uint16_t k_imm_size[MARMOT_HIP_BC_OP_COUNT] = {
     6, 6, 6,         // SWIGLU, GEGLU, ADD (BINARY): 3 x u16
     18,              // ROPE: 3 x u16 + 3 x u32
     48,              // PAGED_ATTENTION: 10 x u16 + 6 x u32 + f32
+    8, 8, 8,         // GELU, GELU_TANH, SILU (UNARY): 2 x u16 + u32
+    8,               // SOFTMAX: 2 x u16 + u32
+    16,              // RESHAPE: 2 x u16 + u32 + u64
+    12,              // VIEW: 2 x u16 + u64
+    12,              // SLICE: 2 x u16 + 2 x u32
+    6,               // GATHER_ROWS: 3 x u16
+    24,              // CONVERT: 2 x u32 + u64 + 2 x u32
 };
 
 static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
@@ -2298,6 +2909,10 @@ static const marmot_bc_schema_id_t k_schema_id[MARMOT_HIP_BC_OP_COUNT] = {
     MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,      MARMOT_BC_SCHEMA_BINARY,
     MARMOT_BC_SCHEMA_ROPE,
     MARMOT_BC_SCHEMA_PAGED_ATTENTION,
+    MARMOT_BC_SCHEMA_UNARY,       MARMOT_BC_SCHEMA_UNARY,       MARMOT_BC_SCHEMA_UNARY,
+    MARMOT_BC_SCHEMA_SOFTMAX,
+    MARMOT_BC_SCHEMA_RESHAPE,     MARMOT_BC_SCHEMA_VIEW,        MARMOT_BC_SCHEMA_SLICE,
+    MARMOT_BC_SCHEMA_GATHER_ROWS, MARMOT_BC_SCHEMA_CONVERT,
 };
 
 static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
@@ -2318,6 +2933,10 @@ static const marmot_bc_exec_fn k_exec_table[MARMOT_HIP_BC_OP_COUNT] = {
     bc_exec_swiglu,      bc_exec_geglu,       bc_exec_add,
     bc_exec_rope,
     bc_exec_paged_attention,
+    bc_exec_gelu,        bc_exec_gelu_tanh,   bc_exec_silu,
+    bc_exec_softmax,
+    bc_exec_reshape,     bc_exec_view,        bc_exec_slice,
+    bc_exec_gather_rows, bc_exec_convert,
 };
 
 // ------------------------------------------------------------------ kernel query
@@ -2581,6 +3200,37 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
             return unsupported("HIP dequantize handles Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1 and Q2_K to Q8_K to FLOAT32");
         }
         return selected(MARMOT_HIP_BC_OP_DEQUANTIZE_BLOCK, launch_us, 0.0);
+    case MARMOT_OP_GELU:
+    case MARMOT_OP_GELU_TANH:
+    case MARMOT_OP_SILU:
+        // gelu / gelu_tanh / silu (cpu/kernels/unary.def): values and result of one type, FLOAT32 or FLOAT16
+        if (!((in32 && out32) || (in16 && out16))) {
+            return unsupported("HIP unary operations handle FLOAT32 and FLOAT16 tensors");
+        }
+        return selected(sig->op_id == MARMOT_OP_GELU        ? MARMOT_HIP_BC_OP_GELU
+                        : sig->op_id == MARMOT_OP_GELU_TANH ? MARMOT_HIP_BC_OP_GELU_TANH
+                                                            : MARMOT_HIP_BC_OP_SILU, launch_us, 0.0);
+    case MARMOT_OP_SOFTMAX:
+        if (!in32 || !out32) {
+            return unsupported("HIP softmax handles FLOAT32 tensors");
+        }
+        return selected(MARMOT_HIP_BC_OP_SOFTMAX_F32, launch_us, 0.0);
+    case MARMOT_OP_RESHAPE:
+        return selected(MARMOT_HIP_BC_OP_RESHAPE, 0.0, 0.0);  // metadata only
+    case MARMOT_OP_VIEW:
+        return selected(MARMOT_HIP_BC_OP_VIEW, 0.0, 0.0);  // metadata only
+    case MARMOT_OP_SLICE:
+        return selected(MARMOT_HIP_BC_OP_SLICE, launch_us, 0.0);
+    case MARMOT_OP_GATHER_ROWS:
+        return selected(MARMOT_HIP_BC_OP_GATHER_ROWS, launch_us, 0.0);
+    case MARMOT_OP_CONVERT: {
+        const bool src_ok = in32 || in16 || sig->input_dtype == MARMOT_DTYPE_BFLOAT16;
+        const bool dst_ok = out32 || out16 || sig->output_dtype == MARMOT_DTYPE_BFLOAT16;
+        if (!src_ok || !dst_ok) {
+            return unsupported("HIP convert handles FLOAT32, FLOAT16 and BFLOAT16");
+        }
+        return selected(MARMOT_HIP_BC_OP_CONVERT, launch_us, 0.0);
+    }
     default:
         return unsupported("Operation not provided by the HIP backend");
     }
@@ -2774,6 +3424,40 @@ marmot_error_t hip_paged_attention_impl(const void *device_ctx, const marmot_pag
 marmot_error_t hip_rope(const void *device_ctx, const marmot_tensor_t *x, const marmot_rope_params_t *params,
                         marmot_tensor_t *out) {
     return rope(device_ctx, x, params, out);
+}
+marmot_error_t hip_gelu(const void *device_ctx, const marmot_tensor_t *x, const marmot_activation_params_t *params,
+                        marmot_tensor_t *out) {
+    return unary(device_ctx, MARMOT_HIP_UNARY_GELU, x, params, out);
+}
+marmot_error_t hip_gelu_tanh(const void *device_ctx, const marmot_tensor_t *x, const marmot_activation_params_t *params,
+                             marmot_tensor_t *out) {
+    return unary(device_ctx, MARMOT_HIP_UNARY_GELU_TANH, x, params, out);
+}
+marmot_error_t hip_silu(const void *device_ctx, const marmot_tensor_t *x, const marmot_activation_params_t *params,
+                        marmot_tensor_t *out) {
+    return unary(device_ctx, MARMOT_HIP_UNARY_SILU, x, params, out);
+}
+marmot_error_t hip_softmax_impl(const void *device_ctx, const marmot_softmax_desc_t *desc) {
+    return softmax(device_ctx, desc);
+}
+marmot_error_t hip_reshape(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out,
+                           const size_t *new_shape, size_t new_ndim) {
+    return reshape(device_ctx, x, out, new_shape, new_ndim);
+}
+marmot_error_t hip_view(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out, size_t byte_offset) {
+    return view(device_ctx, x, out, byte_offset);
+}
+marmot_error_t hip_slice(const void *device_ctx, const marmot_tensor_t *x, marmot_tensor_t *out, const size_t *starts,
+                         const size_t *sizes) {
+    return slice(device_ctx, x, out, starts, sizes);
+}
+marmot_error_t hip_gather_rows(const void *device_ctx, const marmot_tensor_t *input, const marmot_tensor_t *indices,
+                               marmot_tensor_t *out) {
+    return gather_rows(device_ctx, input, indices, out);
+}
+marmot_error_t hip_convert(const void *device_ctx, marmot_dtype_t dst_dtype, void *dst, marmot_dtype_t src_dtype,
+                           const void *src, size_t n) {
+    return convert(device_ctx, dst_dtype, dst, src_dtype, src, n);
 }
 marmot_error_t hip_quantize_block(const void *device_ctx, const marmot_tensor_t *input, marmot_tensor_t *output) {
     return quantize_block(device_ctx, input, output);

@@ -44,10 +44,14 @@ OP_EMBEDDING = 853
 OP_ROPE = 843
 OP_PAGED_ATTENTION = 503
 OP_SWIGLU, OP_GEGLU, OP_RMS_NORM_GEMMA, OP_ADD, OP_RMS_NORM = 331, 410, 447, 876, 929
+OP_GATHER_ROWS, OP_RESHAPE, OP_SILU, OP_VIEW, OP_GELU, OP_GELU_TANH, OP_SLICE, OP_CONVERT, OP_SOFTMAX = (
+    244, 258, 352, 502, 621, 642, 809, 932, 994)
 # this backend's bytecode ops for them (include/marmot_hip_backend.h)
 BC_OP_RMS_NORM_F32, BC_OP_RMS_NORM_GEMMA_F32, BC_OP_SWIGLU_F32, BC_OP_GEGLU_F32, BC_OP_ADD_F32 = 48, 49, 50, 51, 52
 BC_OP_ROPE = 53
 BC_OP_PAGED_ATTENTION = 54
+BC_OP_GELU, BC_OP_GELU_TANH, BC_OP_SILU, BC_OP_SOFTMAX_F32 = 55, 56, 57, 58
+BC_OP_RESHAPE, BC_OP_VIEW, BC_OP_SLICE, BC_OP_GATHER_ROWS, BC_OP_CONVERT = 59, 60, 61, 62, 63
 PREFERENCE_DEFAULT, PREFERENCE_ENABLE, PREFERENCE_DISABLE = 0, 1, 2
 QKV_LAYOUT_FUSED, QKV_LAYOUT_SEPARATE = 1, 2
 QSCHEME_OF_KIND = {KIND_Q4_0: 1, KIND_Q4_1: 2, KIND_Q5_0: 3, KIND_Q5_1: 4, KIND_Q8_0: 5, KIND_Q2_K: 6, KIND_Q3_K: 7, KIND_Q4_K: 8,
@@ -59,8 +63,10 @@ EPILOGUE_BIAS = 1
 EPILOGUE_ROPE = 8
 BC_END, BC_REG_INVALID, BC_INVALID_OFFSET = 0, 0xFFFF, 0xFFFFFFFF
 
+DTYPE_F64, DTYPE_I16, DTYPE_U16, DTYPE_U64 = 10, 4, 7, 9
 _NP_OF_DTYPE = {DTYPE_F32: np.float32, DTYPE_F16: np.float16, DTYPE_I32: np.int32, DTYPE_I8: np.int8,
-                DTYPE_U8: np.uint8, DTYPE_I64: np.int64, DTYPE_U32: np.uint32}
+                DTYPE_U8: np.uint8, DTYPE_I64: np.int64, DTYPE_U32: np.uint32, DTYPE_F64: np.float64,
+                DTYPE_I16: np.int16, DTYPE_U16: np.uint16, DTYPE_U64: np.uint64}
 _DTYPE_OF_NP = {np.dtype(v): k for k, v in _NP_OF_DTYPE.items()}
 
 
@@ -118,6 +124,15 @@ class EmbeddingGatherDesc(C.Structure):
 class TopkDesc(C.Structure):
     _fields_ = [("x", C.POINTER(Tensor)), ("values_out", C.POINTER(Tensor)), ("indices_out", C.POINTER(Tensor)),
                 ("axis", C.c_int32), ("k", C.c_uint32)]
+
+
+class SoftmaxDesc(C.Structure):
+    _fields_ = [("x", C.POINTER(Tensor)), ("out", C.POINTER(Tensor)), ("axis", C.c_int32)]
+
+
+class ActivationParams(C.Structure):
+    _fields_ = [("parameter_tensor", C.POINTER(Tensor)), ("bias", C.POINTER(Tensor)), ("alpha", C.c_float),
+                ("beta", C.c_float), ("gamma", C.c_float)]
 
 
 class RmsNormDesc(C.Structure):
@@ -292,6 +307,8 @@ BACKEND_SYMBOLS = [
     "hip_dequantize_block", "marmot_hip_backend_last_error", "marmot_hip_backend_residency_stats",
     "hip_rmsnorm_impl", "hip_rmsnorm_gemma_impl", "hip_swiglu_f32", "hip_geglu_f32", "hip_add_f32",
     "hip_rope", "hip_paged_attention_impl",
+    "hip_gelu", "hip_gelu_tanh", "hip_silu", "hip_softmax_impl", "hip_reshape", "hip_view", "hip_slice",
+    "hip_gather_rows", "hip_convert",
 ]
 
 
@@ -336,6 +353,23 @@ def bind(lib: C.CDLL) -> C.CDLL:
     lib.hip_paged_attention_impl.argtypes = [C.c_void_p, C.POINTER(PagedAttentionDesc)]
     lib.hip_rope.restype = C.c_int
     lib.hip_rope.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(RopeParams), C.POINTER(Tensor)]
+    for name in ("hip_gelu", "hip_gelu_tanh", "hip_silu"):
+        fn = getattr(lib, name)
+        fn.restype = C.c_int
+        fn.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(ActivationParams), C.POINTER(Tensor)]
+    lib.hip_softmax_impl.restype = C.c_int
+    lib.hip_softmax_impl.argtypes = [C.c_void_p, C.POINTER(SoftmaxDesc)]
+    lib.hip_reshape.restype = C.c_int
+    lib.hip_reshape.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(C.c_size_t), C.c_size_t]
+    lib.hip_view.restype = C.c_int
+    lib.hip_view.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.c_size_t]
+    lib.hip_slice.restype = C.c_int
+    lib.hip_slice.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(C.c_size_t),
+                              C.POINTER(C.c_size_t)]
+    lib.hip_gather_rows.restype = C.c_int
+    lib.hip_gather_rows.argtypes = [C.c_void_p, C.POINTER(Tensor), C.POINTER(Tensor), C.POINTER(Tensor)]
+    lib.hip_convert.restype = C.c_int
+    lib.hip_convert.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_size_t]
     lib.marmot_hip_backend_last_error.restype = C.c_int
     lib.marmot_hip_backend_last_error.argtypes = [C.POINTER(C.c_char_p)]
     lib.marmot_hip_backend_residency_stats.restype = None
@@ -403,6 +437,24 @@ class HostTensor:
         obj.t.dtype = _DTYPE_OF_NP[view.dtype] if dtype is None else dtype
         obj.t.data = view.ctypes.data
         obj.t.capacity_bytes = obj.extent_bytes
+        obj.t.owns_data = False
+        obj.t.quant_kind, obj.t.quant_layout = KIND_GENERIC, LAYOUT_GENERIC
+        obj.t.backend, obj.t.memory_location, obj.t.needs_sync = BACKEND_HIP, MEMORY_HOST, False
+        return obj
+
+    @classmethod
+    def header(cls, shape: Sequence[int], dtype: int) -> "HostTensor":
+        """A tensor without storage: what a graph hands a reshape or view node as its output. Its strides are zero
+        (reshape fills them in when none is set), its data pointer null."""
+        obj = cls.__new__(cls)
+        obj.array = None
+        obj.t = Tensor()
+        obj.t.shape.ndim = len(shape)
+        for i, n in enumerate(shape):
+            obj.t.shape.shape[i] = n
+        obj.t.dtype = dtype
+        obj.t.data = None
+        obj.t.capacity_bytes = 0
         obj.t.owns_data = False
         obj.t.quant_kind, obj.t.quant_layout = KIND_GENERIC, LAYOUT_GENERIC
         obj.t.backend, obj.t.memory_location, obj.t.needs_sync = BACKEND_HIP, MEMORY_HOST, False
@@ -659,3 +711,41 @@ class Program:
 
     def dequantize(self, op_index: int, x, out):
         self.code += struct.pack("<HHHII", op_index, self.reg(x), self.reg(out), x.t.quant_kind, x.t.quant_layout)
+
+    def unary(self, op_index: int, x, out, params: Optional[ActivationParams] = None):
+        """bytecode_compile.c:331-356."""
+        off = BC_INVALID_OFFSET
+        if params is not None:
+            self._keep.append(params)
+            off = self._const(bytes(params), 8)
+        self.code += struct.pack("<HHHI", op_index, self.reg(x), self.reg(out), off)
+
+    def softmax(self, op_index: int, x, out, axis: int = -1):
+        """bytecode_compile.c:440-458."""
+        self.code += struct.pack("<HHHI", op_index, self.reg(x), self.reg(out), axis & 0xFFFFFFFF)
+
+    def reshape(self, op_index: int, x, out, new_shape: Sequence[int]):
+        """bytecode_compile.c:718-745: the shape travels in the constant pool as size_t values."""
+        off = self._const(struct.pack(f"<{len(new_shape)}Q", *new_shape), 8)
+        self.code += struct.pack("<HHHIQ", op_index, self.reg(x), self.reg(out), off, len(new_shape))
+
+    def view(self, op_index: int, x, out, byte_offset: int):
+        """bytecode_compile.c:746-763."""
+        self.code += struct.pack("<HHHQ", op_index, self.reg(x), self.reg(out), byte_offset)
+
+    def slice(self, op_index: int, x, out, starts: Sequence[int], sizes: Sequence[int]):
+        """bytecode_compile.c:863-892."""
+        s0 = self._const(struct.pack(f"<{len(starts)}Q", *starts), 8)
+        s1 = self._const(struct.pack(f"<{len(sizes)}Q", *sizes), 8)
+        self.code += struct.pack("<HHHII", op_index, self.reg(x), self.reg(out), s0, s1)
+
+    def gather_rows(self, op_index: int, x, indices, out):
+        """bytecode_compile.c:893-911."""
+        self.code += struct.pack("<HHHH", op_index, self.reg(x), self.reg(indices), self.reg(out))
+
+    def convert(self, op_index: int, dst: HostTensor, src: HostTensor, n: int):
+        """bytecode_compile.c:1020-1043: the two host addresses travel by value in the constant pool."""
+        self._keep += [dst, src]
+        d = self._const(struct.pack("<Q", dst.t.data), 8)
+        s_ = self._const(struct.pack("<Q", src.t.data), 8)
+        self.code += struct.pack("<HIIQII", op_index, d, s_, n, dst.t.dtype, src.t.dtype)

@@ -3625,3 +3625,187 @@ int mo_paged_attention(const mo_paged_attention_args *a) {
     free(q_vec), free(out_vec), free(k_block), free(v_block), free(scores);
     return 0;
 }
+
+/* ------------------------------------------------------------------ tensor operations around the linears */
+
+/* gelu_scalar, gelu_tanh_scalar, silu_scalar_fn (src/backends/cpu/ops/unary/scalar/unary_scalar.c:201-218); FLOAT16
+ * values are widened, computed in fp32 and rounded back (CPU_UNARY_DEFINE_FLOAT_ACTIVATION, unary_scalar.c:360-385) */
+static float unary_value(int op, float x) {
+    switch (op) {
+    case 0: {
+        const float inv_sqrt2 = 0.7071067811865475f;
+        return x * 0.5f * (1.0f + erff(x * inv_sqrt2));
+    }
+    case 1: {
+        const float sqrt_2_over_pi = 0.7978845608028654f;
+        const float coeff = 0.044715f;
+        const float inner = sqrt_2_over_pi * (x + coeff * x * x * x);
+        return 0.5f * x * (1.0f + tanhf(inner));
+    }
+    default:
+        return x / (1.0f + expf(-x));
+    }
+}
+
+int mo_unary(int op, const void *x, int dtype, size_t n, void *out) {
+    if (op < 0 || op > 2 || (dtype != MO_DTYPE_F32 && dtype != MO_DTYPE_F16)) {
+        return -1;
+    }
+    for (size_t i = 0; i < n; ++i) {
+        if (dtype == MO_DTYPE_F32) {
+            ((float *)out)[i] = unary_value(op, ((const float *)x)[i]);
+        } else {
+            ((uint16_t *)out)[i] = mo_f32_to_f16(unary_value(op, mo_f16_to_f32(((const uint16_t *)x)[i])));
+        }
+    }
+    return 0;
+}
+
+/* softmax_f32_scalar (src/backends/cpu/ops/softmax/scalar/softmax_f32_scalar.c:30-83) over a contiguous tensor seen as
+ * [outer, axis, inner] (marmot_softmax_prepare, src/core/helpers/norm.c:123-179); softmax_safe_expf flushes
+ * differences at or below -88 to zero (softmax_internal.h:14-26) */
+int mo_softmax(const float *x, size_t outer, size_t axis, size_t inner, float *out) {
+    if (axis == 0) {
+        return -1;
+    }
+    for (size_t row = 0; row < outer * inner; ++row) {
+        const size_t o = row / inner, j = row % inner;
+        const size_t base = o * axis * inner + j;
+        float max_val = inner == 1 ? x[base] : -FLT_MAX;
+        for (size_t a = 0; a < axis; ++a) {
+            const float v = x[base + a * inner];
+            if (v > max_val) {
+                max_val = v;
+            }
+        }
+        float sum = 0.0f;
+        for (size_t a = 0; a < axis; ++a) {
+            const float diff = x[base + a * inner] - max_val;
+            const float e = diff <= -88.0f ? 0.0f : expf(diff);
+            out[base + a * inner] = e;
+            sum += e;
+        }
+        const float inv_sum = 1.0f / sum;
+        for (size_t a = 0; a < axis; ++a) {
+            out[base + a * inner] *= inv_sum;
+        }
+    }
+    return 0;
+}
+
+/* cpu_convert_* between FLOAT32, FLOAT16 and BFLOAT16 (src/backends/cpu/ops/convert/dtype_convert.c:17-130): the vector
+ * body's rounding (to nearest even) for every element; the 16-bit types convert to each other through FLOAT32
+ * (src/utils/dtype_ref.c:86-114) */
+static float conv_load(int dtype, const void *p, size_t i) {
+    if (dtype == MO_DTYPE_F32) {
+        return ((const float *)p)[i];
+    }
+    if (dtype == MO_DTYPE_F16) {
+        return mo_f16_to_f32(((const uint16_t *)p)[i]);
+    }
+    uint32_t bits = (uint32_t)((const uint16_t *)p)[i] << 16;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+int mo_convert(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n) {
+    const int ok_s = src_dtype == MO_DTYPE_F32 || src_dtype == MO_DTYPE_F16 || src_dtype == MO_DTYPE_BF16;
+    const int ok_d = dst_dtype == MO_DTYPE_F32 || dst_dtype == MO_DTYPE_F16 || dst_dtype == MO_DTYPE_BF16;
+    if (!ok_s || !ok_d) {
+        return -1;
+    }
+    if (src_dtype == dst_dtype) { /* equal types: a copy */
+        memcpy(dst, src, n * (src_dtype == MO_DTYPE_F32 ? 4 : 2));
+        return 0;
+    }
+    for (size_t i = 0; i < n; ++i) {
+        const float v = conv_load(src_dtype, src, i);
+        if (dst_dtype == MO_DTYPE_F32) {
+            ((float *)dst)[i] = v;
+        } else if (dst_dtype == MO_DTYPE_F16) {
+            ((uint16_t *)dst)[i] = mo_f32_to_f16(v);
+        } else {
+            uint32_t bits;
+            memcpy(&bits, &v, 4);
+            const uint32_t rounding_bias = 0x7FFFu + ((bits >> 16) & 1u);
+            ((uint16_t *)dst)[i] = (uint16_t)((bits + rounding_bias) >> 16);
+        }
+    }
+    return 0;
+}
+
+/* cpu_gather_rows (src/backends/cpu/ops/tensor_ops/tensor_ops.c:464-547), rows with unit column stride: strides in
+ * elements; returns -1 and the offending output row for an index outside [0, rows_in) */
+int mo_gather_rows(const void *x, size_t rows_in, size_t cols, size_t elem_size, size_t in_stride0, const void *idx,
+                   int idx_is_signed, size_t idx_stride, size_t rows_out, void *out, size_t out_stride0,
+                   size_t *bad_row) {
+    for (size_t r = 0; r < rows_out; ++r) {
+        int64_t row_idx;
+        if (idx_is_signed) {
+            row_idx = ((const int32_t *)idx)[r * idx_stride];
+        } else {
+            row_idx = (int64_t)((const uint32_t *)idx)[r * idx_stride];
+        }
+        if (row_idx < 0 || (size_t)row_idx >= rows_in) {
+            if (bad_row != NULL) {
+                *bad_row = r;
+            }
+            return -1;
+        }
+        memcpy((uint8_t *)out + r * out_stride0 * elem_size, (const uint8_t *)x + (size_t)row_idx * in_stride0 * elem_size,
+               cols * elem_size);
+    }
+    return 0;
+}
+
+/* cpu_slice (tensor_ops.c:401-462): contiguous input of shape in_shape, contiguous output of shape out_shape, a run of
+ * sizes[ndim - 1] elements copied per position of the leading dimensions */
+int mo_slice(const void *x, void *out, size_t elem_size, size_t ndim, const size_t *in_shape, const size_t *out_shape,
+             const size_t *starts, const size_t *sizes) {
+    if (ndim == 0) {
+        return 0;
+    }
+    if (ndim > 8) {
+        return -1;
+    }
+    size_t src_strides[8], dst_strides[8], counters[8] = {0};
+    src_strides[ndim - 1] = 1;
+    dst_strides[ndim - 1] = 1;
+    for (int i = (int)ndim - 2; i >= 0; --i) {
+        src_strides[i] = src_strides[i + 1] * in_shape[i + 1];
+        dst_strides[i] = dst_strides[i + 1] * out_shape[i + 1];
+    }
+    const size_t copy_block = sizes[ndim - 1] * elem_size;
+    const size_t loops = ndim > 1 ? ndim - 1 : 0;
+    for (size_t d = 0; d < ndim; ++d) {
+        if (sizes[d] == 0) {
+            return 0;
+        }
+    }
+    for (;;) {
+        size_t src_index = starts[ndim - 1] * src_strides[ndim - 1];
+        size_t dst_index = 0;
+        for (size_t d = 0; d < loops; ++d) {
+            src_index += (starts[d] + counters[d]) * src_strides[d];
+            dst_index += counters[d] * dst_strides[d];
+        }
+        memcpy((uint8_t *)out + dst_index * elem_size, (const uint8_t *)x + src_index * elem_size, copy_block);
+        if (loops == 0) {
+            break;
+        }
+        int dim = (int)loops - 1;
+        while (dim >= 0) {
+            counters[dim]++;
+            if (counters[dim] < sizes[dim]) {
+                break;
+            }
+            counters[dim] = 0;
+            dim--;
+        }
+        if (dim < 0) {
+            break;
+        }
+    }
+    return 0;
+}

@@ -263,6 +263,22 @@ int mo_paged_attention(const mo_paged_attention_args *a);
 uint8_t mo_f32_to_fp8_e4m3(float value);
 float mo_fp8_e4m3_to_f32(uint8_t bits);
 
+/* ---- tensor operations around the linears ----
+ * Pinned by tests/test_oracle_tensor_ops.py: the reference's conversion goldens (g_conv_f16, g_conv_bf16,
+ * g_conv_f16_bf16_bridge, tests/backend/golden_data.h:1814-1858), numpy's IEEE conversions on every FLOAT16 bit pattern
+ * and on seeded values around the rounding ties, the identity gelu(x) - gelu(-x) = x and float64 erf / tanh / exp
+ * closed forms, softmax rows that sum to one, are shift invariant and flush at -88, and numpy indexing for the gather
+ * and the slice. */
+/* op: 0 GELU (erf), 1 GELU (tanh), 2 SiLU; dtype MO_DTYPE_F32 or MO_DTYPE_F16 */
+int mo_unary(int op, const void *x, int dtype, size_t n, void *out);
+int mo_softmax(const float *x, size_t outer, size_t axis, size_t inner, float *out);
+int mo_convert(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n);
+int mo_gather_rows(const void *x, size_t rows_in, size_t cols, size_t elem_size, size_t in_stride0, const void *idx,
+                   int idx_is_signed, size_t idx_stride, size_t rows_out, void *out, size_t out_stride0,
+                   size_t *bad_row);
+int mo_slice(const void *x, void *out, size_t elem_size, size_t ndim, const size_t *in_shape, const size_t *out_shape,
+             const size_t *starts, const size_t *sizes);
+
 #ifdef __cplusplus
 }
 #endif

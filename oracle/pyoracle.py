@@ -209,6 +209,18 @@ class Oracle:
         L.mo_paged_attention.argtypes = [C.POINTER(PagedAttentionArgs)]
         L.mo_row_grain.restype = C.c_size_t
         L.mo_row_grain.argtypes = [C.c_size_t, C.c_size_t, C.c_size_t]
+        L.mo_unary.restype = C.c_int
+        L.mo_unary.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
+        L.mo_softmax.restype = C.c_int
+        L.mo_softmax.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
+        L.mo_convert.restype = C.c_int
+        L.mo_convert.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_size_t]
+        L.mo_gather_rows.restype = C.c_int
+        L.mo_gather_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_int,
+                                     C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t)]
+        L.mo_slice.restype = C.c_int
+        L.mo_slice.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.POINTER(C.c_size_t),
+                               C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
 
     # ---- fp16
     def f16_to_f32(self, h: int) -> float:
@@ -424,6 +436,64 @@ class Oracle:
         x = np.ascontiguousarray(x, dtype=np.float32)
         out = np.zeros_like(x)
         self.L.mo_softmax_rows(_ptr(x), x.shape[0], x.shape[1], _ptr(out))
+        return out
+
+    # ---- tensor operations around the linears
+    UNARY_GELU, UNARY_GELU_TANH, UNARY_SILU = 0, 1, 2
+
+    def unary(self, op: int, x: np.ndarray) -> np.ndarray:
+        """x: float32 or float16 values of any shape."""
+        x = np.ascontiguousarray(x)
+        assert x.dtype in (np.float32, np.float16)
+        out = np.zeros_like(x)
+        st = self.L.mo_unary(op, _ptr(x), DT_F32 if x.dtype == np.float32 else DT_F16, x.size, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_unary -> {st}")
+        return out
+
+    def softmax(self, x: np.ndarray, axis: int = -1) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        axis = axis % x.ndim
+        outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+        inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+        out = np.zeros_like(x)
+        st = self.L.mo_softmax(_ptr(x), outer, x.shape[axis], inner, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_softmax -> {st}")
+        return out
+
+    def convert(self, src: np.ndarray, src_dtype: int, dst_dtype: int) -> np.ndarray:
+        """src: float32 values, or uint16 bit patterns for FLOAT16 (1) / BFLOAT16 (2) sources; the result likewise."""
+        src = np.ascontiguousarray(src)
+        assert src.dtype == (np.float32 if src_dtype == DT_F32 else np.uint16)
+        out = np.zeros(src.shape, dtype=np.float32 if dst_dtype == DT_F32 else np.uint16)
+        st = self.L.mo_convert(_ptr(out), dst_dtype, _ptr(src), src_dtype, src.size)
+        if st != 0:
+            raise RuntimeError(f"mo_convert -> {st}")
+        return out
+
+    def gather_rows(self, x: np.ndarray, idx: np.ndarray) -> np.ndarray:
+        """x: 2-D array whose rows may be strided (unit column stride); idx: int32 or uint32, 1-D."""
+        assert x.ndim == 2 and idx.ndim == 1 and (x.shape[1] <= 1 or x.strides[1] == x.itemsize)
+        idx = np.ascontiguousarray(idx)
+        assert idx.dtype in (np.int32, np.uint32)
+        out = np.zeros((idx.shape[0], x.shape[1]), dtype=x.dtype)
+        bad = C.c_size_t(0)
+        st = self.L.mo_gather_rows(x.ctypes.data, x.shape[0], x.shape[1], x.itemsize, x.strides[0] // x.itemsize,
+                                   _ptr(idx), 1 if idx.dtype == np.int32 else 0, 1, idx.shape[0], _ptr(out),
+                                   x.shape[1], C.byref(bad))
+        if st != 0:
+            raise IndexError(int(bad.value))
+        return out
+
+    def slice(self, x: np.ndarray, starts, sizes) -> np.ndarray:
+        x = np.ascontiguousarray(x)
+        out = np.zeros(tuple(sizes), dtype=x.dtype)
+        n = x.ndim
+        arr = lambda v: (C.c_size_t * n)(*[int(i) for i in v])
+        st = self.L.mo_slice(_ptr(x), _ptr(out), x.itemsize, n, arr(x.shape), arr(out.shape), arr(starts), arr(sizes))
+        if st != 0:
+            raise RuntimeError(f"mo_slice -> {st}")
         return out
 
     def rms_norm(self, x, weight=None, residual=None, eps: float = 1e-5, weight_offset: float = 0.0) -> np.ndarray:

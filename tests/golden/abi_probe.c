@@ -68,6 +68,10 @@ int main(void) {
     VAL(MARMOT_OP_PAGED_ATTENTION); VAL(MARMOT_BC_SCHEMA_PAGED_ATTENTION); VAL(MARMOT_DTYPE_BFLOAT16);
     VAL(MARMOT_DTYPE_UINT32); VAL(MARMOT_DTYPE_FLOAT8_E4M3); VAL(MARMOT_PAGED_ATTENTION_DESC_VERSION);
     VAL(MARMOT_PAGED_ATTENTION_KV_SCALE_EXT_VERSION);
+    VAL(MARMOT_OP_GELU); VAL(MARMOT_OP_GELU_TANH); VAL(MARMOT_OP_SILU); VAL(MARMOT_OP_SOFTMAX); VAL(MARMOT_OP_RESHAPE);
+    VAL(MARMOT_OP_VIEW); VAL(MARMOT_OP_SLICE); VAL(MARMOT_OP_GATHER_ROWS); VAL(MARMOT_OP_CONVERT);
+    VAL(MARMOT_BC_SCHEMA_UNARY); VAL(MARMOT_BC_SCHEMA_SOFTMAX); VAL(MARMOT_BC_SCHEMA_RESHAPE); VAL(MARMOT_BC_SCHEMA_VIEW);
+    VAL(MARMOT_BC_SCHEMA_SLICE); VAL(MARMOT_BC_SCHEMA_GATHER_ROWS); VAL(MARMOT_BC_SCHEMA_CONVERT);
 
     SZ(marmot_shape_t); OFF(marmot_shape_t, ndim); OFF(marmot_shape_t, shape); OFF(marmot_shape_t, strides);
     SZ(marmot_quant_params_t);
@@ -121,6 +125,9 @@ int main(void) {
     OFF(marmot_paged_attention_kv_scale_ext_t, struct_version); OFF(marmot_paged_attention_kv_scale_ext_t, kv_k_scale);
     OFF(marmot_paged_attention_kv_scale_ext_t, kv_v_scale);
     SZ(marmot_topk_desc_t); OFF(marmot_topk_desc_t, axis); OFF(marmot_topk_desc_t, k);
+    SZ(marmot_softmax_desc_t); OFF(marmot_softmax_desc_t, out); OFF(marmot_softmax_desc_t, axis);
+    SZ(marmot_activation_params_t); OFF(marmot_activation_params_t, bias); OFF(marmot_activation_params_t, alpha);
+    OFF(marmot_activation_params_t, gamma);
     SZ(marmot_rmsnorm_desc_t); OFF(marmot_rmsnorm_desc_t, residual); OFF(marmot_rmsnorm_desc_t, weight);
     OFF(marmot_rmsnorm_desc_t, out); OFF(marmot_rmsnorm_desc_t, eps);
     SZ(marmot_moe_experts_desc_t); OFF(marmot_moe_experts_desc_t, out); OFF(marmot_moe_experts_desc_t, ffn_type);

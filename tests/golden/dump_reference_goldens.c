@@ -127,5 +127,32 @@ int main(void) {
     emit("g_conv_fp8_half_bridge_f16_bits", "u2", g_conv_fp8_half_bridge.f16_bits, sizeof(g_conv_fp8_half_bridge.f16_bits));
     emit("g_conv_fp8_half_bridge_fp8_bits", "u1", g_conv_fp8_half_bridge.fp8_bits, sizeof(g_conv_fp8_half_bridge.fp8_bits));
     emit("g_conv_fp8_half_bridge_roundtrip", "f4", g_conv_fp8_half_bridge.roundtrip, sizeof(g_conv_fp8_half_bridge.roundtrip));
+    /* the goldens of the tensor operations around the linears (tests/backend/golden_data.h): activations :449-476,
+     * softmax :521-545, slice :998-1040, FLOAT16 / BFLOAT16 conversions :1811-1858 */
+#define EMIT_FIELD(obj, field, dtype) emit(#obj "_" #field, dtype, obj.field, sizeof(obj.field))
+    EMIT_FIELD(g_activation, input, "f4");
+    EMIT_FIELD(g_activation, gelu, "f4");
+    EMIT_FIELD(g_activation, silu, "f4");
+    EMIT_FIELD(g_activation, gelu_tanh, "f4");
+    EMIT_FIELD(g_softmax, shape, "u8");
+    EMIT_FIELD(g_softmax, input, "f4");
+    EMIT_FIELD(g_softmax, expected_axis_last, "f4");
+    EMIT_FIELD(g_softmax, expected_axis0, "f4");
+    EMIT_FIELD(g_tensor_slice3d, shape_src, "u8");
+    EMIT_FIELD(g_tensor_slice3d, starts, "u8");
+    EMIT_FIELD(g_tensor_slice3d, sizes, "u8");
+    EMIT_FIELD(g_tensor_slice3d, src, "f4");
+    EMIT_FIELD(g_tensor_slice3d, expected, "f4");
+    EMIT_FIELD(g_conv_f16, src, "f4");
+    EMIT_FIELD(g_conv_f16, f16_bits, "u2");
+    EMIT_FIELD(g_conv_f16, roundtrip, "f4");
+    EMIT_FIELD(g_conv_bf16, src, "f4");
+    EMIT_FIELD(g_conv_bf16, bf16_bits, "u2");
+    EMIT_FIELD(g_conv_bf16, roundtrip, "f4");
+    EMIT_FIELD(g_conv_f16_bf16_bridge, src, "f4");
+    EMIT_FIELD(g_conv_f16_bf16_bridge, f16_bits, "u2");
+    EMIT_FIELD(g_conv_f16_bf16_bridge, bf16_bits, "u2");
+    EMIT_FIELD(g_conv_f16_bf16_bridge, bf16_from_f16_bits, "u2");
+    EMIT_FIELD(g_conv_f16_bf16_bridge, f16_from_bf16_bits, "u2");
     return 0;
 }

@@ -57,7 +57,8 @@ def test_ctypes_structs_match_layout(golden_layout):
     pairs = {
         "marmot_shape_t": ta.Shape, "marmot_tensor_t": ta.Tensor, "marmot_matmul_epilogue_t": ta.Epilogue,
         "marmot_topk_desc_t": ta.TopkDesc, "marmot_moe_experts_desc_t": ta.MoeDesc,
-        "marmot_rmsnorm_desc_t": ta.RmsNormDesc,
+        "marmot_rmsnorm_desc_t": ta.RmsNormDesc, "marmot_softmax_desc_t": ta.SoftmaxDesc,
+        "marmot_activation_params_t": ta.ActivationParams,
         "marmot_op_signature_t": ta.OpSignature, "marmot_kernel_selection_t": ta.KernelSelection,
         "marmot_device_caps_t": ta.DeviceCaps, "marmot_device_ops_t": ta.DeviceOps,
         "marmot_bc_exec_ctx_t": ta.BcExecCtx, "marmot_bc_tables_t": ta.BcTables,
@@ -307,7 +308,7 @@ def test_bytecode_tables(lib, golden_layout):
     t = ta.BcTables()
     assert lib.marmot_hip_bc_get_tables(C.byref(t))
     assert not lib.marmot_hip_bc_get_tables(None)
-    assert t.op_count == 55
+    assert t.op_count == 64
     assert not t.exec_table[0] and t.imm_size[0] == 0  # opcode 0 is END
     schema = [t.schema_id[i] for i in range(t.op_count)]
     assert schema[1:5] == [golden_layout["MARMOT_BC_SCHEMA_MATMUL"]] * 4
@@ -349,6 +350,20 @@ def test_bytecode_tables(lib, golden_layout):
     assert (ta.DTYPE_BF16, ta.DTYPE_U32, ta.DTYPE_F8_E4M3) == (
         golden_layout["MARMOT_DTYPE_BFLOAT16"], golden_layout["MARMOT_DTYPE_UINT32"],
         golden_layout["MARMOT_DTYPE_FLOAT8_E4M3"])
+    # the remaining nodes of a model graph: three unary activations, softmax, reshape, view, slice, gather_rows, convert
+    assert schema[55:58] == [golden_layout["MARMOT_BC_SCHEMA_UNARY"]] * 3 and sizes[55:58] == [struct.calcsize("<2HI")] * 3
+    assert schema[58] == golden_layout["MARMOT_BC_SCHEMA_SOFTMAX"] and sizes[58] == struct.calcsize("<2HI")
+    assert schema[59] == golden_layout["MARMOT_BC_SCHEMA_RESHAPE"] and sizes[59] == struct.calcsize("<2HIQ") == 16
+    assert schema[60] == golden_layout["MARMOT_BC_SCHEMA_VIEW"] and sizes[60] == struct.calcsize("<2HQ") == 12
+    assert schema[61] == golden_layout["MARMOT_BC_SCHEMA_SLICE"] and sizes[61] == struct.calcsize("<2H2I") == 12
+    assert schema[62] == golden_layout["MARMOT_BC_SCHEMA_GATHER_ROWS"] and sizes[62] == struct.calcsize("<3H")
+    assert schema[63] == golden_layout["MARMOT_BC_SCHEMA_CONVERT"] and sizes[63] == struct.calcsize("<2IQ2I") == 24
+    assert (ta.BC_OP_GELU, ta.BC_OP_GELU_TANH, ta.BC_OP_SILU, ta.BC_OP_SOFTMAX_F32, ta.BC_OP_RESHAPE, ta.BC_OP_VIEW,
+            ta.BC_OP_SLICE, ta.BC_OP_GATHER_ROWS, ta.BC_OP_CONVERT) == tuple(range(55, 64))
+    assert (ta.OP_GELU, ta.OP_GELU_TANH, ta.OP_SILU, ta.OP_SOFTMAX, ta.OP_RESHAPE, ta.OP_VIEW, ta.OP_SLICE,
+            ta.OP_GATHER_ROWS, ta.OP_CONVERT) == tuple(
+        golden_layout["MARMOT_OP_" + n] for n in ("GELU", "GELU_TANH", "SILU", "SOFTMAX", "RESHAPE", "VIEW", "SLICE",
+                                                 "GATHER_ROWS", "CONVERT"))
     for i in range(1, t.op_count):
         assert t.exec_table[i], f"exec entry {i} missing"
 

@@ -1,0 +1,195 @@
+"""Pins the oracle's tensor operations around the linears (activations, softmax, conversions, gather, slice) against the
+reference's own golden vectors for them (tests/backend/golden_data.h: g_activation, g_softmax, g_tensor_slice3d,
+g_conv_f16, g_conv_bf16, g_conv_f16_bf16_bridge) and against what the mathematics fixes independently of the code:
+numpy's IEEE conversions, float64 closed forms, identities and numpy indexing."""
+import math
+
+import numpy as np
+import pytest
+from scipy import special
+
+from oracle.pyoracle import DT_BF16, DT_F16, DT_F32
+
+
+def bits16(a):
+    return np.ascontiguousarray(a).view(np.uint16)
+
+
+# ------------------------------------------------------------------ conversions
+def test_conversion_goldens_of_the_reference(oracle, ref_goldens):
+    g = ref_goldens
+    src = g["g_conv_f16_src"]
+    assert np.array_equal(oracle.convert(src, DT_F32, DT_F16), g["g_conv_f16_f16_bits"])
+    assert np.array_equal(oracle.convert(g["g_conv_f16_f16_bits"], DT_F16, DT_F32), g["g_conv_f16_roundtrip"])
+    src = g["g_conv_bf16_src"]
+    assert np.array_equal(oracle.convert(src, DT_F32, DT_BF16), g["g_conv_bf16_bf16_bits"])
+    assert np.array_equal(oracle.convert(g["g_conv_bf16_bf16_bits"], DT_BF16, DT_F32), g["g_conv_bf16_roundtrip"])
+    src = g["g_conv_f16_bf16_bridge_src"]
+    f16 = oracle.convert(src, DT_F32, DT_F16)
+    bf16 = oracle.convert(src, DT_F32, DT_BF16)
+    assert np.array_equal(f16, g["g_conv_f16_bf16_bridge_f16_bits"])
+    assert np.array_equal(bf16, g["g_conv_f16_bf16_bridge_bf16_bits"])
+    assert np.array_equal(oracle.convert(f16, DT_F16, DT_BF16), g["g_conv_f16_bf16_bridge_bf16_from_f16_bits"])
+    assert np.array_equal(oracle.convert(bf16, DT_BF16, DT_F16), g["g_conv_f16_bf16_bridge_f16_from_bf16_bits"])
+
+
+def _bf16_round_to_nearest_even(x32):
+    """Independent statement: of the two neighbouring bfloat16 values pick the nearer one in exact arithmetic, ties to
+    the even code (the golden values above fix that the reference rounds and does not truncate)."""
+    b = x32.view(np.uint32).astype(np.uint64)
+    lo = (b >> 16) << 16
+    hi = lo + (1 << 16)
+    d_lo, d_hi = b - lo, hi - b
+    up = (d_hi < d_lo) | ((d_hi == d_lo) & (((lo >> 16) & 1) == 1))
+    return (np.where(up, hi, lo) >> 16).astype(np.uint16)
+
+
+def test_conversions_against_ieee_rounding(oracle):
+    # every FLOAT16 bit pattern widens like numpy's (NaNs keep their payload position; compare as bits)
+    allh = np.arange(1 << 16, dtype=np.uint16)
+    wide = oracle.convert(allh, DT_F16, DT_F32)
+    expect = allh.view(np.float16).astype(np.float32)
+    assert np.array_equal(wide.view(np.uint32), expect.view(np.uint32))
+    # and narrows back to itself (NaNs: any quiet pattern with the sign kept)
+    back = oracle.convert(wide, DT_F32, DT_F16)
+    finite = ~np.isnan(expect)
+    assert np.array_equal(back[finite], allh[finite])
+    assert np.all(np.isnan(back[~finite].view(np.float16)))
+    # seeded values, plus exact ties and their neighbours at every FLOAT16 exponent including the subnormal range and the
+    # overflow threshold 65520: numpy's astype is IEEE round-to-nearest-even
+    rng = np.random.Generator(np.random.PCG64(41))
+    vals = [rng.standard_normal(20000).astype(np.float32) * np.float32(s) for s in (1e-7, 1e-4, 1.0, 300.0, 7e4)]
+    h = allh[(allh & 0x7c00) != 0x7c00].view(np.float16).astype(np.float64)
+    with np.errstate(over="ignore"):
+        nxt = np.nextafter(h.astype(np.float16), np.float16(np.inf)).astype(np.float64)
+    ties = ((h + nxt) / 2).astype(np.float32)
+    vals += [ties, np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+             np.array([65504.0, 65519.99, 65520.0, 65536.0, -65520.0, 2.0 ** -25, 2.0 ** -24, 1.5 * 2.0 ** -25,
+                       np.inf, -np.inf, 0.0, -0.0], dtype=np.float32)]
+    x = np.concatenate(vals)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(oracle.convert(x, DT_F32, DT_F16), bits16(x.astype(np.float16)))
+    fin = x[np.isfinite(x)]
+    assert np.array_equal(oracle.convert(fin, DT_F32, DT_BF16), _bf16_round_to_nearest_even(fin))
+    # bfloat16 widens by appending zero bits; the bridges go through FLOAT32
+    allb = np.arange(1 << 16, dtype=np.uint16)
+    assert np.array_equal(oracle.convert(allb, DT_BF16, DT_F32).view(np.uint32), allb.astype(np.uint32) << 16)
+    some = allb[(allb & 0x7f80) != 0x7f80][::7]
+    with np.errstate(over="ignore"):
+        assert np.array_equal(oracle.convert(some, DT_BF16, DT_F16),
+                              bits16((some.astype(np.uint32) << 16).view(np.float32).astype(np.float16)))
+    someh = allh[(allh & 0x7c00) != 0x7c00][::5]
+    assert np.array_equal(oracle.convert(someh, DT_F16, DT_BF16),
+                          _bf16_round_to_nearest_even(someh.view(np.float16).astype(np.float32)))
+    assert np.array_equal(oracle.convert(x, DT_F32, DT_F32).view(np.uint32), x.view(np.uint32))
+
+
+# ------------------------------------------------------------------ activations
+def test_activation_goldens_of_the_reference(oracle, ref_goldens):
+    x = ref_goldens["g_activation_input"]
+    for op, key in ((oracle.UNARY_GELU, "gelu"), (oracle.UNARY_GELU_TANH, "gelu_tanh"), (oracle.UNARY_SILU, "silu")):
+        want = ref_goldens["g_activation_" + key]
+        got = oracle.unary(op, x)
+        # the goldens are float64 results printed with ten digits: at x = -6 the fp32 expression 1 + erf(.) is exactly 0
+        # where the golden says -5.9e-9, an absolute difference of |x| * 2^-30
+        assert np.allclose(got, want, rtol=2e-6, atol=1e-8), (key, got, want)
+
+
+def test_activations_against_float64_closed_forms(oracle):
+    rng = np.random.Generator(np.random.PCG64(42))
+    x = np.concatenate([rng.standard_normal(50000).astype(np.float32) * np.float32(3.0),
+                        np.linspace(-12, 12, 4801, dtype=np.float32), np.array([0.0, -0.0], np.float32)])
+    x64 = x.astype(np.float64)
+    gelu = oracle.unary(oracle.UNARY_GELU, x)
+    gelu_t = oracle.unary(oracle.UNARY_GELU_TANH, x)
+    silu = oracle.unary(oracle.UNARY_SILU, x)
+    # x * Phi(x): for x << 0 the fp32 expression 1 + erf(.) cancels, so the error is absolute (|x| * 2^-24), not relative
+    assert np.max(np.abs(gelu - 0.5 * x64 * (1.0 + special.erf(x64 / math.sqrt(2.0)))) - 1e-6 * np.abs(x64)) <= 1e-7
+    inner = math.sqrt(2.0 / math.pi) * (x64 + 0.044715 * x64 ** 3)
+    assert np.max(np.abs(gelu_t - 0.5 * x64 * (1.0 + np.tanh(inner))) - 1e-6 * np.abs(x64)) <= 1e-7
+    assert np.allclose(silu, x64 / (1.0 + np.exp(-x64)), rtol=1e-6, atol=1e-30)
+    # erf and tanh are odd: f(x) - f(-x) = x for both GELU forms; a wrong sign, a dropped 0.5 or a missing "1 +" fails
+    for f in (gelu, gelu_t):
+        op = oracle.UNARY_GELU if f is gelu else oracle.UNARY_GELU_TANH
+        assert np.max(np.abs((f.astype(np.float64) - oracle.unary(op, -x)) - x64) - 1e-6 * np.abs(x64)) <= 1e-7
+    assert gelu[-2] == 0 and silu[-2] == 0 and gelu_t[-2] == 0
+    # the two forms differ visibly (1.6e-4 around |x| = 2): the golden test above tells them apart
+    assert np.max(np.abs(gelu - gelu_t)) > 1e-4
+    # FLOAT16 values: widened, the fp32 formula, one rounding
+    h = rng.standard_normal(4096).astype(np.float16)
+    for op in (oracle.UNARY_GELU, oracle.UNARY_GELU_TANH, oracle.UNARY_SILU):
+        assert np.array_equal(bits16(oracle.unary(op, h)), bits16(oracle.unary(op, h.astype(np.float32)).astype(np.float16)))
+
+
+# ------------------------------------------------------------------ softmax
+def test_softmax_goldens_of_the_reference(oracle, ref_goldens):
+    shape = tuple(int(v) for v in ref_goldens["g_softmax_shape"])
+    x = ref_goldens["g_softmax_input"].reshape(shape)
+    assert np.allclose(oracle.softmax(x, -1).ravel(), ref_goldens["g_softmax_expected_axis_last"], rtol=2e-6)
+    assert np.allclose(oracle.softmax(x, 0).ravel(), ref_goldens["g_softmax_expected_axis0"], rtol=2e-6)
+
+
+def test_softmax_properties(oracle):
+    rng = np.random.Generator(np.random.PCG64(43))
+    for shape, axis in (((5, 8), -1), ((3, 128), 1), ((4, 1000), -1), ((2, 6, 5), 1), ((3, 4, 7), 0), ((1, 32000), 1),
+                        ((7,), 0)):
+        x = (rng.standard_normal(shape) * 4).astype(np.float32)
+        got = oracle.softmax(x, axis)
+        # the row sum is added sequentially in fp32: its error grows with the row length
+        rtol = max(3e-6, x.shape[axis] * 2e-9)
+        assert np.allclose(got, special.softmax(x.astype(np.float64), axis=axis), rtol=rtol, atol=1e-12), shape
+        assert np.allclose(got.sum(axis=axis, dtype=np.float64), 1.0, atol=max(1e-5, 2 * rtol))
+        # adding a constant that is exact in fp32 changes nothing: x - max is the same number
+        assert np.array_equal(oracle.softmax(x.astype(np.float32) * np.float32(0.25) + np.float32(0),
+                                             axis), oracle.softmax(x * np.float32(0.25), axis))
+    x = np.array([[0.0, -87.5, -88.0, -89.0, -1000.0]], np.float32)
+    got = oracle.softmax(x)
+    assert got[0, 1] > 0 and got[0, 2] == 0 and got[0, 3] == 0 and got[0, 4] == 0  # flushed at or below -88
+    # without the flush exp(-88) = 6e-39 (a subnormal) would have survived
+    assert np.float32(math.exp(-88.0)) > 0
+    # one multiplication by 1 / sum, not a division: 1/3 as fp32 times 1 differs from 1 / 3 in the last bit for these
+    y = oracle.softmax(np.zeros((1, 3), np.float32))
+    assert np.array_equal(y, np.full((1, 3), np.float32(1.0) / np.float32(3.0), np.float32))
+    z = oracle.softmax(np.log(np.array([[1, 2, 4, 3]], np.float64)).astype(np.float32))
+    e = np.exp((np.log(np.array([1, 2, 4, 3], np.float64)).astype(np.float32) - np.float32(math.log(4.0))).astype(np.float32))
+    assert np.allclose(z, e / e.sum(), rtol=1e-6)
+
+
+# ------------------------------------------------------------------ gather and slice
+def test_slice_golden_of_the_reference_and_numpy_indexing(oracle, ref_goldens):
+    g = ref_goldens
+    shape = tuple(int(v) for v in g["g_tensor_slice3d_shape_src"])
+    src = g["g_tensor_slice3d_src"].reshape(shape)
+    got = oracle.slice(src, g["g_tensor_slice3d_starts"], [int(v) for v in g["g_tensor_slice3d_sizes"]])
+    assert np.array_equal(got.ravel(), g["g_tensor_slice3d_expected"])
+    rng = np.random.Generator(np.random.PCG64(44))
+    for shape, dtype in (((9,), np.float32), ((5, 7), np.float16), ((3, 4, 5), np.int32), ((2, 3, 4, 5), np.uint8),
+                         ((2, 2, 3, 2, 3), np.float64), ((2, 1, 2, 2, 1, 3, 2, 2), np.int16)):
+        x = rng.integers(0, 250, size=shape).astype(dtype)
+        for _ in range(6):
+            starts = [int(rng.integers(0, n)) for n in shape]
+            sizes = [int(rng.integers(1, n - s + 1)) for n, s in zip(shape, starts)]
+            want = x[tuple(slice(s, s + n) for s, n in zip(starts, sizes))]
+            assert np.array_equal(oracle.slice(x, starts, sizes), want), (shape, starts, sizes)
+        assert np.array_equal(oracle.slice(x, [0] * len(shape), list(shape)), x)
+        assert oracle.slice(x, [0] * len(shape), [0] + list(shape[1:])).size == 0
+
+
+def test_gather_rows_against_numpy_indexing(oracle):
+    rng = np.random.Generator(np.random.PCG64(45))
+    for rows, cols, dtype in ((7, 5, np.float32), (100, 64, np.float16), (3, 1, np.int32), (16, 4096, np.float32),
+                              (9, 3, np.uint8)):
+        x = rng.integers(0, 250, size=(rows, cols)).astype(dtype)
+        for idt in (np.int32, np.uint32):
+            idx = rng.integers(0, rows, size=11).astype(idt)
+            assert np.array_equal(oracle.gather_rows(x, idx), x[idx.astype(np.int64)])
+        wide = rng.integers(0, 250, size=(rows, cols + 3)).astype(dtype)
+        idx = rng.integers(0, rows, size=5).astype(np.int32)
+        assert np.array_equal(oracle.gather_rows(wide[:, :cols], idx), wide[idx, :cols])  # strided rows
+        assert oracle.gather_rows(x, np.zeros(0, np.int32)).shape == (0, cols)
+    x = np.arange(12, dtype=np.float32).reshape(4, 3)
+    for bad, where in ((np.array([0, 4], np.int32), 1), (np.array([-1, 0], np.int32), 0),
+                       (np.array([1, 2, 0xFFFFFFFF], np.uint32), 2)):
+        with pytest.raises(IndexError) as e:
+            oracle.gather_rows(x, bad)
+        assert e.value.args[0] == where

@@ -1,6 +1,7 @@
 """CPU: the library's GGUF reader (host code, no GPU call) against files written by tests/gguf_writer.py: header and
 key/value skipping, general.alignment, the loader's shape convention ([rows, cols] for matrices, file order for
-expert stacks), the ggml-type mapping of every weight format, views that alias the file's bytes, error paths."""
+expert stacks), the ggml-type mapping of every weight format, views that alias the file's bytes, error paths; and
+against a committed file laid out like the synthetic MoE model of the reference's own loader test."""
 import os
 import struct
 
@@ -125,3 +126,60 @@ def test_malformed_files_are_rejected(tmp_path):
     with pytest.raises(capi.MarmotHipError):
         GgufFile(str(tmp_path / "does_not_exist.gguf"))
     assert not os.path.exists(str(tmp_path / "does_not_exist.gguf"))
+
+
+def test_synthetic_moe_file_of_the_reference_loader_test():
+    """tests/golden/synthetic_qwen3moe.gguf follows write_synthetic_qwen3moe_gguf (the reference's
+    tests/graph/test_gguf_loader.c:171-256) field by field: 16 key/value pairs, 17 FLOAT32 tensors whose offsets
+    accumulate the sizes without per-tensor alignment, 32-byte alignment of the data section only. Expectations below
+    are written down from that test, not from the generator."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "synthetic_qwen3moe.gguf")
+    raw = open(path, "rb").read()
+    # the committed bytes are what the committed generator writes
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("make_synthetic_gguf", os.path.join(os.path.dirname(path),
+                                                                                      "make_synthetic_gguf.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert mod.build() == raw
+    assert struct.unpack_from("<IIQQ", raw, 0) == (0x46554747, 3, 17, 16)
+    expect_kv = [("general.architecture", "qwen3moe"), ("general.alignment", 32), ("qwen3moe.context_length", 32),
+                 ("qwen3moe.embedding_length", 8), ("qwen3moe.block_count", 1), ("qwen3moe.attention.head_count", 2),
+                 ("qwen3moe.attention.head_count_kv", 1), ("qwen3moe.feed_forward_length", 6),
+                 ("qwen3moe.rope.dimension_count", 4), ("qwen3moe.attention.key_length", 4),
+                 ("qwen3moe.attention.layer_norm_rms_epsilon", float(np.float32(1.0e-5))),
+                 ("qwen3moe.rope.freq_base", 10000.0), ("qwen3moe.expert_count", 2), ("qwen3moe.expert_used_count", 1),
+                 ("qwen3moe.expert_shared_count", 1), ("qwen3moe.expert_weights_scale", 1.25)]
+    # name, dimensions as the file lists them (innermost first)
+    expect_tensors = [("output_norm.weight", (8,)), ("output.weight", (8, 16)), ("blk.0.attn_norm.weight", (8,)),
+                      ("blk.0.attn_q.weight", (8, 8)), ("blk.0.attn_k.weight", (8, 4)), ("blk.0.attn_v.weight", (8, 4)),
+                      ("blk.0.attn_output.weight", (8, 8)), ("blk.0.attn_q_norm.weight", (4,)),
+                      ("blk.0.attn_k_norm.weight", (4,)), ("blk.0.ffn_norm.weight", (8,)),
+                      ("blk.0.ffn_gate_inp.weight", (8, 2)), ("blk.0.ffn_gate_exps.weight", (8, 6, 2)),
+                      ("blk.0.ffn_up_exps.weight", (8, 6, 2)), ("blk.0.ffn_down_exps.weight", (6, 8, 2)),
+                      ("blk.0.ffn_gate_shexp.weight", (8, 6)), ("blk.0.ffn_up_shexp.weight", (8, 6)),
+                      ("blk.0.ffn_down_shexp.weight", (6, 8))]
+    with GgufFile(path) as g:
+        assert g.alignment == 32
+        assert list(g.metadata().items()) == expect_kv  # file order, types resolved (uint32, float32, string)
+        assert g.get("qwen3moe.expert_weights_scale") == 1.25 and g.get("general.architecture") == "qwen3moe"
+        assert [t.name for t in g.tensors] == [n for n, _ in expect_tensors]
+        data_start = None
+        offset = 0
+        for t, (info, (name, dims)) in enumerate(zip(g.tensors, expect_tensors)):
+            n = int(np.prod(dims))
+            assert info.ggml_type == 0 and info.kind == 0 and info.dtype == capi.DT_F32 and info.nbytes == 4 * n
+            # matrices are [rows, cols] (the file's two dimensions reversed), vectors and expert stacks keep file order
+            assert info.shape == (tuple(reversed(dims)) if len(dims) == 2 else dims), name
+            data_start = info.address - offset if data_start is None else data_start
+            assert info.address == data_start + offset, name  # offsets accumulate sizes: no per-tensor alignment
+            offset += 4 * n
+            want = np.float32(t) + np.arange(n, dtype=np.float32) / np.float32(1024.0)
+            assert np.array_equal(g.array(info).ravel(), want), name
+            assert g.find(name) == info
+        # the norm weights of 16 bytes leave the tensors behind them 16 bytes off the 32-byte alignment
+        assert (g.find("blk.0.attn_k_norm.weight").address - data_start) % 32 == 16
+        assert data_start % 32 == g.tensors[0].address % 32
+        # the data section starts at the first multiple of 32 behind the tensor infos and runs to the end of the file
+        assert offset == 4 * sum(int(np.prod(d)) for _, d in expect_tensors) and len(raw) - offset == (len(raw) - offset) // 32 * 32

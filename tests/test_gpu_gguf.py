@@ -1,6 +1,8 @@
 """GPU: weights taken from a GGUF file through the library's reader: uploaded with marmot_hip_gguf_upload and used by
 the raw-pointer matmul, and used in place (views into the file mapping) by the tensor-level backend, whose residency
 table mirrors them once. Results against the CPU oracle on the weights that were written to the file."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -116,3 +118,50 @@ def test_session_style_preload_then_linears_upload_nothing(model, oracle):
             ctx.host_freed(yt)
         for _, t in tensors.values():
             ctx.host_freed(t)
+
+
+def test_synthetic_moe_file_of_the_reference_loader_test_on_the_device(oracle):
+    """The file laid out like the reference's synthetic MoE model (tests/graph/test_gguf_loader.c:171-256; tensors at
+    offsets that are 16 modulo 32): every tensor uploads to the bytes the file holds, and tensors used in place (views
+    into the mapping at those offsets) go through the residency table into device operations: the final
+    normalization's weight, the router projection's rows gathered by expert id, the softmax over the two experts."""
+    import os
+
+    from marmot_amd import HipBackend
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "synthetic_qwen3moe.gguf")
+    hip = HipBackend(0)
+    try:
+        with GgufFile(path) as g:
+            for t, info in enumerate(g.tensors):
+                print(f"synthetic gguf upload {info.name}", flush=True)
+                d = g.upload(hip, info)
+                n = info.nbytes // 4
+                want = np.float32(t) + np.arange(n, dtype=np.float32) / np.float32(1024.0)
+                assert np.array_equal(d.download(np.float32, (n,)), want), info.name
+                d.free()
+    finally:
+        hip.close()
+    with ta.HipContext() as ctx, GgufFile(path) as g:
+        norm = g.find("blk.0.attn_k_norm.weight")   # 16 bytes, at an offset that is 16 modulo 32
+        router = g.find("blk.0.ffn_gate_inp.weight")  # [experts = 2, hidden = 8]
+        assert (norm.address - g.tensors[0].address) % 32 == 16
+        wt = ta.HostTensor.strided(g.array(norm))
+        x = gaussian(1300, (3, 4))
+        xt, ot = ta.HostTensor.dense(x), ta.HostTensor.empty((3, 4), ta.DTYPE_F32)
+        desc = ta.RmsNormDesc(xt.ptr, None, wt.ptr, ot.ptr, g.get("qwen3moe.attention.layer_norm_rms_epsilon"))
+        assert ctx.lib.hip_rmsnorm_impl(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
+        ref = oracle.rms_norm(x, g.array(norm).copy(), eps=float(np.float32(1e-5)))
+        assert np.allclose(ctx.to_host(ot), ref, rtol=1e-5, atol=1e-8)
+        rt = ta.HostTensor.strided(g.array(router))
+        ids = ta.HostTensor.dense(np.array([1, 0, 1], np.int32))
+        rows = ta.HostTensor.empty((3, 8), ta.DTYPE_F32)
+        probs = ta.HostTensor.empty((3, 8), ta.DTYPE_F32)
+        prog = ta.Program()
+        prog.gather_rows(ta.BC_OP_GATHER_ROWS, rt, ids, rows)
+        prog.softmax(ta.BC_OP_SOFTMAX_F32, rows, probs, -1)
+        assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+        assert np.array_equal(ctx.to_host(rows), g.array(router)[[1, 0, 1]])
+        assert np.allclose(ctx.to_host(probs), oracle.softmax(g.array(router)[[1, 0, 1]].copy()), rtol=3e-6)
+        for t in (wt, xt, ot, rt, ids, rows, probs):
+            ctx.host_range_freed(t)

@@ -13,6 +13,7 @@ timed alone with HIP events on the library's stream), `cpu_baseline` is the CPU 
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -28,9 +29,9 @@ METRIC = "Q4_K matvec GB/s (% HBM peak) + prefill GEMM TOPS (% MFMA peak)"
 HBM_PEAK_GBPS = 8000.0
 MALL_BYTES = 256 << 20
 # HBM bytes per launch of the Q4_K 4096x14336 N=1 matvec kernels (rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a plain
-# copy kernel, profiles/matvec_q4_k_4096x14336_n1.md): the row-owning kernel with the activation quantization inside
-# (k_matvec_rows_q4k) and the streaming kernel on pre-packed activations (k_matvec_ls)
-TRAFFIC_FUSED = 33_737_000
+# copy kernel, profiles/matvec_q4_k_4096x14336_n1.md): the resident-share kernel with the activation quantization
+# inside (k_matvec_rows2_q4k) and the streaming kernel on pre-packed activations (k_matvec_ls)
+TRAFFIC_FUSED = 33_667_000
 TRAFFIC_PREPACKED = 33_288_000
 
 
@@ -77,6 +78,15 @@ def time_steps_graph(hip, fn, steps: int, warmup: int, chunk: int = 500, repeats
     probe = hip.graph_capture(lambda: fn(warmup))
     per_step = max(1, hip.graph_last_capture_nodes())
     hip.graph_destroy(probe)
+    # Under rocprofv3 (it exports ROCPROF_* / ROCP_* variables to the program it starts) the steps are replayed twice
+    # only (no settling, one timed repeat), from graphs of 100 steps that are synchronized one by one: the queue
+    # interception of its kernel trace ends in a segmentation fault inside hipGraphLaunch once about ten thousand
+    # kernels of one process have gone through graph launches (observed: after 96 replays of 100-step graphs; 2200
+    # such kernels per call of this function are fine). The profiler's own per-kernel durations are what such a run is
+    # for, not this function's figure.
+    profiled = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ)
+    if profiled:
+        chunk, repeats, settle_ms = min(chunk, 100), 1, 0.0
     chunk = max(1, min(chunk, (hip.graph_max_nodes() - 2) // per_step))
     stamps = hip.alloc(16)
     n_graphs = -(-steps // chunk)
@@ -97,20 +107,28 @@ def time_steps_graph(hip, fn, steps: int, warmup: int, chunk: int = 500, repeats
 
         graphs.append(hip.graph_capture(body))
         done += n
+        if os.environ.get("BENCH_DEBUG"):
+            print(f"captured graph {len(graphs)} ({n} steps, {hip.graph_last_capture_nodes()} nodes)", file=sys.stderr, flush=True)
 
     def replay_ms():
-        for g in graphs:
+        for gi, g in enumerate(graphs):
+            if os.environ.get("BENCH_DEBUG"):
+                print(f"launch graph {gi}", file=sys.stderr, flush=True)
             hip.graph_launch(g)
+            if profiled:
+                hip.synchronize()
         hip.synchronize()
         t = stamps.download(np.uint64, (2,))
         return float(int(t[1]) - int(t[0])) * 1e-5  # 10 ns ticks -> ms
 
     # ---- settle: untimed replays until settle_ms of GPU time have passed
     once_ms = max(replay_ms(), 1e-3)
-    settle_replays = min(20000, int(settle_ms / once_ms) + 1)
+    settle_replays = min(20000, int(settle_ms / once_ms) + 1) if settle_ms > 0 else 0
     for _ in range(settle_replays):
         for g in graphs:
             hip.graph_launch(g)
+            if profiled:
+                hip.synchronize()
     hip.synchronize()
     # ---- timed repeats
     per_repeat = sorted(replay_ms() / steps for _ in range(repeats))
@@ -718,6 +736,92 @@ def sweep_moe(hip, rng, emit, steps: int):
           "algorithmic_bytes": nbytes})
 
 
+# Marks of the resident-share decode kernel in the timeline build (make -C marmot_amd/csrc TIMELINE=1): slot -> meaning
+TIMELINE_LOADER = {0: "start", 2: "first window requested", 3: "barrier passed", 4: "first instruction landed",
+                   8: "a quarter landed", 9: "half landed", 10: "three quarters landed", 6: "all requested",
+                   7: "all landed"}
+TIMELINE_CONSUMER = {0: "start", 1: "barrier passed", 2: "own activations landed", 3: "own activations in registers",
+                     4: "own part quantized", 5: "all parts quantized", 6: "task loop starts",
+                     7: "first task's bytes there", 8: "first task's products done", 9: "last task's bytes there",
+                     10: "last task done", 11: "leaves"}
+
+
+def timeline_report(shape: str, steps: int, warmup: int):
+    """Cycle-counter timeline of the Q4_K decode kernel for one activation row. Needs the timeline build of the
+    library (make -C marmot_amd/csrc TIMELINE=1; MARMOT_HIP_LIBRARY=marmot_amd/lib/libmarmot_hip_timeline.so): every
+    wavefront keeps up to 12 cycle-counter marks in registers and writes them, with the 100 MHz device clock at its
+    first mark and at its exit, into the attached buffer when it leaves. Prints, per mark, the distribution over the
+    wavefronts of one launch (microseconds since the workgroup's first wavefront started)."""
+    from marmot_amd import DT_F32, HipBackend, capi, row_bytes
+    from marmot_amd.capi import check
+
+    M, K = (int(v) for v in shape.split("x"))
+    kind = capi.KIND_Q4_K
+    hip = HipBackend(0)
+    rb = row_bytes(kind, K)
+    stride = (M * rb + 255) & ~255
+    copies = max(2, -(-2 * MALL_BYTES // stride) + 1)
+    rng = np.random.Generator(np.random.PCG64(10))
+    blocks = random_blocks(rng, kind, M, K)
+    d_w = hip.alloc(stride * copies)
+    for c in range(copies):
+        d_w.upload(blocks, offset=c * stride)
+    d_x = hip.to_device(rng.standard_normal((1, K), dtype=np.float32))
+    d_out = hip.alloc(M * 4)
+    slots, waves_per_wg = 16, 16
+    words = hip.caps()["num_compute_units"] * waves_per_wg * slots
+    d_tl = hip.alloc(words * 8)
+
+    def step(i):
+        hip.linear_d(kind, d_w, d_x, DT_F32, 1, K, M, d_out, DT_F32, weight_offset=(i % copies) * stride)
+
+    check(hip.lib.marmot_hip_timeline_attach(hip.dev, None, 0))
+    ms = time_steps_graph(hip, step, steps, warmup)
+    route = hip.last_route()
+    print(f"{M}x{K}: {ms * 1e3:.3f} us per launch with the marks switched off (route {route})")
+    check(hip.lib.marmot_hip_timeline_attach(hip.dev, ctypes.c_void_p(d_tl.ptr), words * 8))
+    ms_on = time_steps_graph(hip, step, steps, warmup)
+    print(f"{M}x{K}: {ms_on * 1e3:.3f} us per launch with the marks written")
+
+    def stats(name, a):
+        a = np.asarray(a, dtype=np.float64)
+        a = a[~np.isnan(a)]
+        if a.size:
+            print(f"  {name:44s} min {a.min():6.2f} p10 {np.percentile(a, 10):6.2f} med {np.median(a):6.2f} "
+                  f"p90 {np.percentile(a, 90):6.2f} max {a.max():6.2f}")
+
+    for rep in range(2):
+        hip.lib.marmot_hip_memset(hip.dev, ctypes.c_void_p(d_tl.ptr), 0, words * 8)
+        g = hip.graph_capture(lambda: [step(7 + j) for j in range(200)])  # the buffer keeps the last launch
+        hip.graph_launch(g)
+        hip.synchronize()
+        hip.graph_destroy(g)
+        t = d_tl.download(np.uint64, (words // slots, slots)).astype(np.int64)
+        t = t[t[:, 12] != 0]
+        nw = t.shape[0]
+        # slots 12 / 14: cycle counter at the first mark / at the flush; 13 / 15: the 100 MHz clock at the same points
+        dc = (t[:, 14] - t[:, 12]).astype(np.float64)
+        dr = (t[:, 15] - t[:, 13]).astype(np.float64) * 10.0
+        rate = np.median(dc[dr > 0] / dr[dr > 0])  # cycle-counter ticks per nanosecond
+        print(f" launch {rep}: {nw} wavefronts; cycle counter at {rate * 1e3:.0f} MHz; first start to last exit "
+              f"{(t[:, 15].max() - t[:, 13].min()) * 0.01:.2f} us (100 MHz clock)")
+        wg = np.arange(nw) // waves_per_wg
+        wv = np.arange(nw) % waves_per_wg
+        nwg = int(wg.max()) + 1
+        base = np.array([t[wg == i, 12].min() for i in range(nwg)])[wg]
+        rel = (t - base[:, None]) / rate / 1e3
+        rel[t == 0] = np.nan
+        dev0 = t[:, 13].min()
+        stats("workgroup start after the first one", (np.array([t[wg == i, 13].min() for i in range(nwg)]) - dev0) * 0.01)
+        stats("workgroup end after the first start", (np.array([t[wg == i, 15].max() for i in range(nwg)]) - dev0) * 0.01)
+        loaders = wv < 4
+        for slot, label in TIMELINE_LOADER.items():
+            stats("loader: " + label, rel[loaders, slot])
+        for slot, label in TIMELINE_CONSUMER.items():
+            stats("consumer: " + label, rel[~loaders, slot])
+    hip.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -739,6 +843,9 @@ def main():
     ap.add_argument("--calibrate-read", type=int, default=0, metavar="MIB",
                     help="run only the read-only streaming kernel over this many MiB per launch, rotating over "
                          "copies beyond the Infinity Cache, and print its bandwidth")
+    ap.add_argument("--timeline", default="", metavar="MxK",
+                    help="print the cycle-counter timeline of the Q4_K decode kernel for this weight shape "
+                         "(needs the timeline build of the library)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists in the hot path)",
@@ -758,6 +865,10 @@ def main():
                           "launches": 23, "ms_per_launch": round(ms, 5),
                           "gbps_read_plus_write": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
         hip.close()
+        return
+
+    if args.timeline:
+        timeline_report(args.timeline, min(args.steps, 2000), min(args.warmup, 200))
         return
 
     if args.calibrate_read:

@@ -687,21 +687,18 @@ typedef struct {
 
 static marmot_error_t matmul_locked(hip_backend_t *b, const matmul_plan_t *p, const marmot_tensor_t *input,
                                     const marmot_tensor_t *weight, const marmot_tensor_t *bias, marmot_tensor_t *out) {
-    const void *d_w = nullptr, *d_x = nullptr, *d_b = nullptr;
-    void *d_y = nullptr;
-    marmot_error_t st = acquire_read(b, weight->data, p->M * marmot_hip_row_bytes(p->kind, p->K), &d_w);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, input->data, dense_bytes(input), &d_x);
-    }
-    if (st == MARMOT_SUCCESS && bias != nullptr) {
-        st = acquire_read(b, bias->data, dense_bytes(bias), &d_b);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, out->data, dense_bytes(out), &d_y);
-    }
+    hip_acq_t acq[4] = {
+        {weight->data, p->M * marmot_hip_row_bytes(p->kind, p->K), HIP_ACQ_READ, nullptr},
+        {input->data, dense_bytes(input), HIP_ACQ_READ, nullptr},
+        {out->data, dense_bytes(out), HIP_ACQ_WRITE, nullptr},
+        {bias != nullptr ? bias->data : nullptr, bias != nullptr ? dense_bytes(bias) : 0, HIP_ACQ_READ, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, bias != nullptr ? 4 : 3);
     if (st != MARMOT_SUCCESS) {
         return st;
     }
+    const void *d_w = acq[0].dev, *d_x = acq[1].dev, *d_b = bias != nullptr ? acq[3].dev : nullptr;
+    void *d_y = acq[2].dev;
     int rc;
     if (p->in_dtype == MARMOT_HIP_DTYPE_F32 && p->N >= HIP_PACK_MIN_ROWS) {
         // fp32 rows that a normalization already left packed, or that an earlier linear packed: no quantization
@@ -874,37 +871,55 @@ static marmot_error_t qkv_locked(hip_backend_t *b, const marmot_matmul_qkv_desc_
     const marmot_tensor_t *w[3] = {desc->separate.wq, desc->separate.wk, desc->separate.wv};
     const marmot_tensor_t *bias[3] = {desc->separate.bq, desc->separate.bk, desc->separate.bv};
     marmot_tensor_t *out[3] = {desc->out_q, desc->out_k, desc->out_v};
-    const void *d_w[3] = {nullptr, nullptr, nullptr}, *d_b[3] = {nullptr, nullptr, nullptr}, *d_x = nullptr;
-    void *d_o[3] = {nullptr, nullptr, nullptr};
-    marmot_error_t st = acquire_read(b, desc->input->data, dense_bytes(desc->input), &d_x);
-    for (int i = 0; i < 3 && st == MARMOT_SUCCESS; ++i) {
-        st = acquire_read(b, w[i]->data, M * marmot_hip_row_bytes(kind, K), &d_w[i]);
-        if (st == MARMOT_SUCCESS && bias[i] != nullptr) {
-            st = acquire_read(b, bias[i]->data, dense_bytes(bias[i]), &d_b[i]);
-        }
-    }
-    for (int i = 0; i < 3 && st == MARMOT_SUCCESS; ++i) {
-        st = acquire_write(b, out[i]->data, dense_bytes(out[i]), &d_o[i]);
-    }
-    if (st != MARMOT_SUCCESS) {
-        return st;
-    }
+    // every range of the call in one set: input, three weights, three outputs, then the optional ones
     const marmot_rope_params_t *r = desc->rope_params;
-    marmot_hip_rope_t rope;
-    const marmot_hip_rope_t *rope_ptr = nullptr;
-    if (r != nullptr && (r->apply_to_q || r->apply_to_k)) {
-        hip_rope_entry_t *e = nullptr;
+    const bool with_rope = r != nullptr && (r->apply_to_q || r->apply_to_k);
+    hip_rope_entry_t *e = nullptr;
+    marmot_error_t st = MARMOT_SUCCESS;
+    if (with_rope) {
         st = rope_entry_locked(b, r, M, &e);
-        const void *d_pos = nullptr, *d_freqs = nullptr;
-        if (st == MARMOT_SUCCESS) {
-            st = acquire_read(b, r->positions->data, dense_bytes(r->positions), &d_pos);
-        }
-        if (st == MARMOT_SUCCESS) {
-            st = acquire_read(b, e->freqs, (size_t)e->head_dim / 2 * sizeof(float), &d_freqs);
-        }
         if (st != MARMOT_SUCCESS) {
             return st;
         }
+    }
+    hip_acq_t acq[12];
+    size_t n_acq = 0;
+    acq[n_acq++] = (hip_acq_t){desc->input->data, dense_bytes(desc->input), HIP_ACQ_READ, nullptr};
+    for (int i = 0; i < 3; ++i) {
+        acq[n_acq++] = (hip_acq_t){w[i]->data, M * marmot_hip_row_bytes(kind, K), HIP_ACQ_READ, nullptr};
+    }
+    for (int i = 0; i < 3; ++i) {
+        acq[n_acq++] = (hip_acq_t){out[i]->data, dense_bytes(out[i]), HIP_ACQ_WRITE, nullptr};
+    }
+    int bias_at[3] = {-1, -1, -1}, pos_at = -1, freqs_at = -1;
+    for (int i = 0; i < 3; ++i) {
+        if (bias[i] != nullptr) {
+            bias_at[i] = (int)n_acq;
+            acq[n_acq++] = (hip_acq_t){bias[i]->data, dense_bytes(bias[i]), HIP_ACQ_READ, nullptr};
+        }
+    }
+    if (with_rope) {
+        pos_at = (int)n_acq;
+        acq[n_acq++] = (hip_acq_t){r->positions->data, dense_bytes(r->positions), HIP_ACQ_READ, nullptr};
+        freqs_at = (int)n_acq;
+        acq[n_acq++] = (hip_acq_t){e->freqs, (size_t)e->head_dim / 2 * sizeof(float), HIP_ACQ_READ, nullptr};
+    }
+    st = acquire_set(b, acq, n_acq);
+    if (st != MARMOT_SUCCESS) {
+        return st;
+    }
+    const void *d_x = acq[0].dev;
+    const void *d_w[3] = {acq[1].dev, acq[2].dev, acq[3].dev}, *d_b[3] = {nullptr, nullptr, nullptr};
+    void *d_o[3] = {acq[4].dev, acq[5].dev, acq[6].dev};
+    for (int i = 0; i < 3; ++i) {
+        if (bias_at[i] >= 0) {
+            d_b[i] = acq[bias_at[i]].dev;
+        }
+    }
+    marmot_hip_rope_t rope;
+    const marmot_hip_rope_t *rope_ptr = nullptr;
+    if (with_rope) {
+        const void *d_pos = acq[pos_at].dev, *d_freqs = acq[freqs_at].dev;
         rope = (marmot_hip_rope_t){
             .d_positions = d_pos,
             .positions_dtype = r->positions->dtype == MARMOT_DTYPE_FLOAT32 ? MARMOT_HIP_DTYPE_F32
@@ -1090,15 +1105,14 @@ static marmot_error_t embedding_gather(const void *device_ctx, const marmot_embe
         return MARMOT_SUCCESS;
     }
     pthread_mutex_lock(&b->mu);
-    const void *d_w = nullptr, *d_ids = nullptr;
-    void *d_out = nullptr;
-    marmot_error_t st = acquire_read(b, weights->data, vocab * marmot_hip_row_bytes((int)weights->quant_kind, dim), &d_w);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, ids->data, dense_bytes(ids), &d_ids);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, out->data, dense_bytes(out), &d_out);
-    }
+    hip_acq_t acq[3] = {
+        {weights->data, vocab * marmot_hip_row_bytes((int)weights->quant_kind, dim), HIP_ACQ_READ, nullptr},
+        {ids->data, dense_bytes(ids), HIP_ACQ_READ, nullptr},
+        {out->data, dense_bytes(out), HIP_ACQ_WRITE, nullptr},
+    };
+    marmot_error_t st = acquire_set(b, acq, 3);
+    const void *d_w = acq[0].dev, *d_ids = acq[1].dev;
+    void *d_out = acq[2].dev;
     // the library takes at most 65535 tokens per call
     const size_t id_size = dtype_size(ids->dtype), row_size = dim * dtype_size(out->dtype);
     for (size_t t0 = 0; st == MARMOT_SUCCESS && t0 < tokens; t0 += 65535) {
@@ -1132,30 +1146,22 @@ static marmot_error_t moe_locked(hip_backend_t *b, const marmot_moe_experts_desc
                                  size_t E, size_t k) {
     const marmot_tensor_t *h = desc->hidden_states, *g = desc->gate_exps, *u = desc->up_exps, *d = desc->down_exps;
     const int kgu = (int)g->quant_kind, kd = (int)d->quant_kind;
-    const void *d_h = nullptr, *d_g = nullptr, *d_u = nullptr, *d_d = nullptr, *d_ids = nullptr, *d_wts = nullptr;
-    void *d_out = nullptr;
-    marmot_error_t st = acquire_read(b, h->data, dense_bytes(h), &d_h);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, g->data, expert_tensor_bytes(kgu, F, H, E), &d_g);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, u->data, expert_tensor_bytes(kgu, F, H, E), &d_u);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, d->data, expert_tensor_bytes(kd, H, F, E), &d_d);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, desc->topk_ids->data, dense_bytes(desc->topk_ids), &d_ids);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_read(b, desc->topk_weights->data, dense_bytes(desc->topk_weights), &d_wts);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, desc->out->data, dense_bytes(desc->out), &d_out);
-    }
+    hip_acq_t acq[7] = {
+        {h->data, dense_bytes(h), HIP_ACQ_READ, nullptr},
+        {g->data, expert_tensor_bytes(kgu, F, H, E), HIP_ACQ_READ, nullptr},
+        {u->data, expert_tensor_bytes(kgu, F, H, E), HIP_ACQ_READ, nullptr},
+        {d->data, expert_tensor_bytes(kd, H, F, E), HIP_ACQ_READ, nullptr},
+        {desc->topk_ids->data, dense_bytes(desc->topk_ids), HIP_ACQ_READ, nullptr},
+        {desc->topk_weights->data, dense_bytes(desc->topk_weights), HIP_ACQ_READ, nullptr},
+        {desc->out->data, dense_bytes(desc->out), HIP_ACQ_WRITE, nullptr},
+    };
+    const marmot_error_t st = acquire_set(b, acq, 7);
     if (st != MARMOT_SUCCESS) {
         return st;
     }
+    const void *d_h = acq[0].dev, *d_g = acq[1].dev, *d_u = acq[2].dev, *d_d = acq[3].dev, *d_ids = acq[4].dev,
+               *d_wts = acq[5].dev;
+    void *d_out = acq[6].dev;
     const int rc = marmot_hip_moe_experts(b->dev, (const float *)d_h, T, H, F, E, k, kgu, kd, d_g, d_u, d_d,
                                           (const int32_t *)d_ids, (const float *)d_wts, desc->weights_scale,
                                           (int)desc->router_weight_policy, (int)desc->ffn_type, (float *)d_out);
@@ -1212,18 +1218,17 @@ static marmot_error_t moe_experts(const void *device_ctx, const marmot_moe_exper
 }
 
 static marmot_error_t topk_locked(hip_backend_t *b, const marmot_topk_desc_t *desc, size_t rows, size_t cols) {
-    const void *d_x = nullptr;
-    void *d_v = nullptr, *d_i = nullptr;
-    marmot_error_t st = acquire_read(b, desc->x->data, dense_bytes(desc->x), &d_x);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, desc->values_out->data, dense_bytes(desc->values_out), &d_v);
-    }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, desc->indices_out->data, dense_bytes(desc->indices_out), &d_i);
-    }
+    hip_acq_t acq[3] = {
+        {desc->x->data, dense_bytes(desc->x), HIP_ACQ_READ, nullptr},
+        {desc->values_out->data, dense_bytes(desc->values_out), HIP_ACQ_WRITE, nullptr},
+        {desc->indices_out->data, dense_bytes(desc->indices_out), HIP_ACQ_WRITE, nullptr},
+    };
+    const marmot_error_t st = acquire_set(b, acq, 3);
     if (st != MARMOT_SUCCESS) {
         return st;
     }
+    const void *d_x = acq[0].dev;
+    void *d_v = acq[1].dev, *d_i = acq[2].dev;
     const int rc = marmot_hip_topk(b->dev, (const float *)d_x, rows, cols, desc->k, (float *)d_v, (int32_t *)d_i);
     if (rc != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(rc);
@@ -1271,15 +1276,16 @@ static marmot_error_t topk(const void *device_ctx, const marmot_topk_desc_t *des
 static marmot_error_t quantize_locked(hip_backend_t *b, const marmot_tensor_t *input, marmot_tensor_t *output,
                                       size_t rows, size_t k) {
     const int kind = (int)output->quant_kind;
-    const void *d_x = nullptr;
-    void *d_q = nullptr;
-    marmot_error_t st = acquire_read(b, input->data, dense_bytes(input), &d_x);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, output->data, rows * marmot_hip_row_bytes(kind, k), &d_q);
-    }
+    hip_acq_t acq[2] = {
+        {input->data, dense_bytes(input), HIP_ACQ_READ, nullptr},
+        {output->data, rows * marmot_hip_row_bytes(kind, k), HIP_ACQ_WRITE, nullptr},
+    };
+    const marmot_error_t st = acquire_set(b, acq, 2);
     if (st != MARMOT_SUCCESS) {
         return st;
     }
+    const void *d_x = acq[0].dev;
+    void *d_q = acq[1].dev;
     int rc;
     if (kind == MARMOT_QUANT_KIND_Q8_0 || kind == MARMOT_QUANT_KIND_Q8_K) {
         rc = marmot_hip_quantize_activations(
@@ -1327,15 +1333,16 @@ static marmot_error_t quantize_block(const void *device_ctx, const marmot_tensor
 static marmot_error_t dequantize_locked(hip_backend_t *b, const marmot_tensor_t *input, marmot_tensor_t *output,
                                         size_t rows, size_t k) {
     const int kind = (int)input->quant_kind;
-    const void *d_q = nullptr;
-    void *d_y = nullptr;
-    marmot_error_t st = acquire_read(b, input->data, rows * marmot_hip_row_bytes(kind, k), &d_q);
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, output->data, dense_bytes(output), &d_y);
-    }
+    hip_acq_t acq[2] = {
+        {input->data, rows * marmot_hip_row_bytes(kind, k), HIP_ACQ_READ, nullptr},
+        {output->data, dense_bytes(output), HIP_ACQ_WRITE, nullptr},
+    };
+    const marmot_error_t st = acquire_set(b, acq, 2);
     if (st != MARMOT_SUCCESS) {
         return st;
     }
+    const void *d_q = acq[0].dev;
+    void *d_y = acq[1].dev;
     const int rc = marmot_hip_dequantize(b->dev, kind, d_q, rows, k, (float *)d_y);
     if (rc != MARMOT_HIP_SUCCESS) {
         return fail_from_lib(rc);
@@ -1417,18 +1424,22 @@ static marmot_error_t rmsnorm(const void *device_ctx, const marmot_rmsnorm_desc_
     }
     const size_t rows = n / cols;
     pthread_mutex_lock(&b->mu);
-    const void *d_x = nullptr, *d_r = nullptr, *d_w = nullptr;
-    void *d_y = nullptr;
-    marmot_error_t st = acquire_read(b, x->data, n * sizeof(float), &d_x);
-    if (st == MARMOT_SUCCESS && res != nullptr) {
-        st = acquire_read(b, res->data, n * sizeof(float), &d_r);
+    hip_acq_t acq[4];
+    size_t n_acq = 0;
+    int res_at = -1, w_at = -1;
+    acq[n_acq++] = (hip_acq_t){x->data, n * sizeof(float), HIP_ACQ_READ, nullptr};
+    acq[n_acq++] = (hip_acq_t){out->data, n * sizeof(float), HIP_ACQ_WRITE, nullptr};  // also ends any packed copy of the old contents
+    if (res != nullptr) {
+        res_at = (int)n_acq;
+        acq[n_acq++] = (hip_acq_t){res->data, n * sizeof(float), HIP_ACQ_READ, nullptr};
     }
-    if (st == MARMOT_SUCCESS && w != nullptr) {
-        st = acquire_read(b, w->data, cols * sizeof(float), &d_w);
+    if (w != nullptr) {
+        w_at = (int)n_acq;
+        acq[n_acq++] = (hip_acq_t){w->data, cols * sizeof(float), HIP_ACQ_READ, nullptr};
     }
-    if (st == MARMOT_SUCCESS) {
-        st = acquire_write(b, out->data, n * sizeof(float), &d_y);  // also ends any packed copy of the old contents
-    }
+    marmot_error_t st = acquire_set(b, acq, n_acq);
+    const void *d_x = acq[0].dev, *d_r = res_at >= 0 ? acq[res_at].dev : nullptr, *d_w = w_at >= 0 ? acq[w_at].dev : nullptr;
+    void *d_y = acq[1].dev;
     if (st == MARMOT_SUCCESS) {
         int rc;
         // Rows that the linears behind this normalization would quantize in a launch of their own are packed here,

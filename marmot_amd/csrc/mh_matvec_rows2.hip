@@ -1,10 +1,9 @@
 // Decode matvec for Q4_K weights and ONE fp32 activation row, "resident share" form: one workgroup per compute unit
 // owns a contiguous run of weight rows, and that run (up to ~140 KB) is copied into LDS exactly once, byte for byte as
 // it lies in memory (no ring, no slot reuse, LDS offset = offset in the share).
-//   * Four loader wavefronts (wavefronts 0..3, the first ones the dispatcher starts; their arguments arrive preloaded
-//     in scalar registers) request the share front to back with direct-to-LDS loads of 1 KiB per instruction, KiB c by
-//     loader c % 4, a bounded number of instructions in flight each. They publish "instructions completed" counters
-//     read from their own load counter without waiting.
+//   * Four loader wavefronts (wavefronts 0..3, the first ones the dispatcher starts) request the share front to back
+//     with direct-to-LDS loads of 1 KiB per instruction, KiB c by loader c % 4, a bounded number of instructions in
+//     flight each. They publish "instructions completed" counters read from their own load counter without waiting.
 //   * Twelve consumer wavefronts first request THEIR blocks of the activation row (four 256-value blocks each, the
 //     same 1 KiB instructions into a staging area that the LAST weight bytes reuse later), wait on their own load
 //     counter, quantize to Q8_K once per workgroup (bit-identical to cpu_matmul_quant_pack_q8_k_f32,
@@ -76,8 +75,9 @@ __device__ __forceinline__ void rows2_store(void *out, const void *bias, uint32_
     }
 }
 
-// shape: pad_shift | rpt_shift << 4 | seg_blocks << 8. The first fourteen argument words are preloaded into scalar
-// registers (compiler option for this file), the rest is fetched on first use.
+// shape: pad_shift | rpt_shift << 4 | seg_blocks << 8. Plain scalar arguments, ordered by first use. (Preloading the
+// first fourteen words into scalar registers, -mllvm -amdgpu-kernarg-preload-count=14, was measured at 0.03 us per
+// launch and is not used: rocprofv3's kernel trace crashes in hipGraphLaunch on graphs that hold such a kernel.)
 template <int SEGS>
 __global__ __launch_bounds__(1024) void k_matvec_rows2_q4k(const uint8_t *__restrict__ w, const float *__restrict__ x,
                                                           void *__restrict__ out, uint32_t M, uint32_t nb,

@@ -570,6 +570,266 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
     }
 }
 
+// ---- attention with the scores on the matrix cores (FLOAT16 cache rows of 128 values, blocks of 16 positions or more)
+// One workgroup of four wavefronts per (token, QH query heads of one key / value head, share of the history); a
+// wavefront takes tiles of 16 consecutive positions (one cache block, or a 16-aligned part of one).
+//   * Scores: S[position][head] = K[position][:] . q[head][:] as v_mfma_f32_16x16x16_f16 with the KEY ROWS as the row
+//     operand, read from the cache straight into operand registers (lane (r, j) = (lane % 16, lane / 16) reads the 64
+//     contiguous bytes of dimensions 32 j .. 32 j + 31 of position r: the k index of the c-th instruction stands for
+//     dimensions 32 j + 4 c .. + 3, the same in both operands, so no value moves between lanes and none is converted).
+//     The query is the column operand, scaled and split once into a FLOAT16 high part and a FLOAT16 remainder (two
+//     instructions per step: products of FLOAT16 values are exact in fp32, the split leaves 2^-22 of the query).
+//     Columns beyond QH are zero.
+//   * The result layout puts positions 4 j + i (i = 0..3) of head n in lane (n, j): the online softmax of a head runs in
+//     the four lanes n, n + 16, n + 32, n + 48 (two cross-lane exchanges per maximum and per sum).
+//   * Output: the 16 lanes of group j hold dimensions 8 n .. 8 n + 7 of the value rows of THEIR four positions; the
+//     weights of head h for these positions are fetched from lane (h, j) with ds_swizzle broadcasts; fp32
+//     multiply-adds as before. The running output is rescaled only when a maximum moved (wavefront-wide test).
+// The 16 partial outputs (4 wavefronts x 4 groups) meet in LDS like the 16 groups of k_pa_attend. fp32 accumulation
+// everywhere; only the order of the sums differs from the reference.
+typedef _Float16 pa_half4 __attribute__((ext_vector_type(4)));
+typedef float pa_float4 __attribute__((ext_vector_type(4)));
+
+template <int PATTERN>
+__device__ __forceinline__ float pa_swizzle(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), PATTERN));
+}
+// value of lane (h, j) in every lane of the 16-lane group j (bit-mask mode: lane' = (lane & 0x10) | h inside each half)
+template <int H>
+__device__ __forceinline__ float pa_group_bcast(float v) {
+    return pa_swizzle<0x10 | (H << 5)>(v);
+}
+// exchange with the lane 16 / 32 lanes away
+__device__ __forceinline__ float pa_xor16(float v) {
+    return pa_swizzle<0x1f | (0x10 << 10)>(v);
+}
+__device__ __forceinline__ float pa_xor32(float v) {
+    return __shfl_xor(v, 32);
+}
+
+template <int QH>
+__global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
+    constexpr int EPL = 8;  // head_dim == 128
+    __shared__ float s_acc[PA_GROUPS][QH][16 * EPL];
+    __shared__ float s_m[PA_GROUPS][QH], s_l[PA_GROUPS][QH];
+    const uint32_t t = blockIdx.x;
+    const uint32_t qh0 = blockIdx.y * QH;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, j = lane >> 4;
+    const uint32_t seq = p.meta[t * p.meta_stride[0]];
+    const uint32_t pos = p.meta[t * p.meta_stride[0] + p.meta_stride[1]];
+    const uint32_t kv_len = seq < p.max_seqs ? pos + 1u : 0u;
+    const uint32_t kvh = qh0 / p.group;
+
+    // the query: head n (zero beyond QH), dimensions 32 j .. 32 j + 31, scaled, as high part + remainder
+    pa_half4 qhi[8], qlo[8];
+    {
+        float qv[32];
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            qv[e] = 0.0f;
+        }
+        if (n < QH) {
+            const size_t q_base = (size_t)t * p.q_stride[0] + (size_t)(qh0 + n) * p.q_stride[1];
+            if (p.q_vec) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float part[8];
+                    pa_load_run<8>(p.q, p.act_dtype, q_base + 32u * j + 8u * c, part);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        qv[8 * c + e] = part[e];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 32; ++e) {
+                    qv[e] = pa_load(p.q, p.act_dtype, q_base + (size_t)(32 * j + e) * p.q_stride[2]);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float v = p.scale != 1.0f ? qv[4 * c + e] * p.scale : qv[4 * c + e];
+                const _Float16 hi = (_Float16)v;
+                qhi[c][e] = hi;
+                qlo[c][e] = (_Float16)(v - (float)hi);
+            }
+        }
+    }
+
+    float m = -INFINITY, lsum = 0.0f;  // of head n (replicated in the four lanes n + 16 j)
+    float acc[QH][EPL];
+#pragma unroll
+    for (int h = 0; h < QH; ++h) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            acc[h][e] = 0.0f;
+        }
+    }
+    const size_t head_base = (size_t)p.layer_idx * p.kv_stride[1] + (size_t)kvh * p.kv_stride[2];
+    const uint32_t *table_row = p.table + (size_t)seq * p.table_stride[0];
+    // this workgroup's share of the history, in whole tiles of 16 positions
+    const uint32_t tiles = (kv_len + 15u) >> 4;
+    const uint32_t tiles_per_split = (tiles + p.splits - 1u) / p.splits;
+    const uint32_t tile_first = blockIdx.z * tiles_per_split;
+    const uint32_t tile_stop = tile_first + tiles_per_split < tiles ? tile_first + tiles_per_split : tiles;
+    for (uint32_t tile = tile_first + (uint32_t)wave; tile < tile_stop; tile += 4u) {
+        const uint32_t p0 = tile << 4;  // first position of the tile
+        const uint32_t logical = p0 >> p.shift;
+        if (logical >= p.max_blocks) {
+            continue;
+        }
+        const uint32_t tb = table_row[(size_t)logical * p.table_stride[1]];
+        if (tb == PA_NO_BLOCK || tb >= p.kv_blocks) {
+            continue;  // a hole: none of the tile's positions has a block
+        }
+        const size_t tile_base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(p0 & p.mask) * p.kv_stride[3];
+        // key rows: position n of the tile, dimensions 32 j .. + 31; value rows: positions 4 j + i, dimensions 8 n .. + 7
+        const uint16_t *krow = (const uint16_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
+        uint4 kq[4], vq[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            kq[c] = *(const uint4 *)(krow + 8 * c);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            vq[i] = *(const uint4 *)((const uint16_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+        }
+        pa_float4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const pa_half4 k0 = __builtin_bit_cast(pa_half4, make_uint2(kq[c].x, kq[c].y));
+            const pa_half4 k1 = __builtin_bit_cast(pa_half4, make_uint2(kq[c].z, kq[c].w));
+            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qhi[2 * c], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qlo[2 * c], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qhi[2 * c + 1], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qlo[2 * c + 1], sc, 0, 0, 0);
+        }
+        // positions beyond the sequence (the last tile): no score, no value
+        const bool whole = p0 + 16u <= kv_len;
+        float s4[4] = {sc[0], sc[1], sc[2], sc[3]};
+        if (!whole) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (p0 + 4u * j + (uint32_t)i >= kv_len) {
+                    s4[i] = -INFINITY;
+                    vq[i] = make_uint4(0, 0, 0, 0);
+                }
+            }
+        }
+        // online softmax of head n over the tile's 16 positions (lanes n, n + 16, n + 32, n + 48)
+        float big = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+        big = fmaxf(big, pa_xor16(big));
+        big = fmaxf(big, pa_xor32(big));
+        const float m_new = fmaxf(m, big);
+        const float corr = m == -INFINITY ? 0.0f : pa_exp(m - m_new);
+        float w4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            w4[i] = pa_exp(s4[i] - m_new);
+        }
+        float tsum = (w4[0] + w4[1]) + (w4[2] + w4[3]);
+        tsum += pa_xor16(tsum);
+        tsum += pa_xor32(tsum);
+        lsum = lsum * corr + tsum;
+        const bool moved = m_new != m;
+        m = m_new;
+        // rescale the running output of the heads whose maximum moved
+        if (__builtin_amdgcn_ballot_w64(moved && n < QH) != 0) {
+            float f[QH];
+            f[0] = pa_group_bcast<0>(corr);
+            if constexpr (QH > 1) {
+                f[1] = pa_group_bcast<1>(corr);
+            }
+            if constexpr (QH > 2) {
+                f[2] = pa_group_bcast<2>(corr);
+                f[3] = pa_group_bcast<3>(corr);
+            }
+#pragma unroll
+            for (int h = 0; h < QH; ++h) {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    acc[h][e] *= f[h];
+                }
+            }
+        }
+        // values: this group's four positions, dimensions 8 n .. 8 n + 7
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float vr[EPL];
+            const uint32_t vw[4] = {vq[i].x, vq[i].y, vq[i].z, vq[i].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vr[2 * e] = h2f((uint16_t)(vw[e] & 0xffffu));
+                vr[2 * e + 1] = h2f((uint16_t)(vw[e] >> 16));
+            }
+            float wh[QH];
+            wh[0] = pa_group_bcast<0>(w4[i]);
+            if constexpr (QH > 1) {
+                wh[1] = pa_group_bcast<1>(w4[i]);
+            }
+            if constexpr (QH > 2) {
+                wh[2] = pa_group_bcast<2>(w4[i]);
+                wh[3] = pa_group_bcast<3>(w4[i]);
+            }
+#pragma unroll
+            for (int h = 0; h < QH; ++h) {
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    acc[h][e] = __builtin_fmaf(wh[h], vr[e], acc[h][e]);
+                }
+            }
+        }
+    }
+
+    // the 16 partial outputs meet: group g = 4 wave + j; a wavefront's sum of weights is counted once (its group 0)
+    const int g = 4 * wave + j;
+    const uint32_t d0 = (uint32_t)n * EPL;
+#pragma unroll
+    for (int h = 0; h < QH; ++h) {
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            s_acc[g][h][d0 + e] = acc[h][e];
+        }
+    }
+    if (n < QH) {
+        s_m[g][n] = m;
+        s_l[g][n] = j == 0 ? lsum : 0.0f;
+    }
+    __syncthreads();
+    for (uint32_t idx = (uint32_t)tid; idx < (uint32_t)QH * 128u; idx += 256u) {
+        const uint32_t h = idx >> 7, d = idx & 127u;
+        float top = -INFINITY;
+#pragma unroll
+        for (int gg = 0; gg < PA_GROUPS; ++gg) {
+            top = fmaxf(top, s_m[gg][h]);
+        }
+        float o = 0.0f, total = 0.0f;
+        if (top != -INFINITY) {
+#pragma unroll
+            for (int gg = 0; gg < PA_GROUPS; ++gg) {
+                const float f = s_m[gg][h] == -INFINITY ? 0.0f : pa_exp(s_m[gg][h] - top);
+                total = __builtin_fmaf(s_l[gg][h], f, total);
+                o = __builtin_fmaf(s_acc[gg][h][d], f, o);
+            }
+        }
+        if (p.splits > 1u) {
+            float *part = p.partial + (((size_t)t * p.num_q_heads + qh0 + h) * p.splits + blockIdx.z) * (p.head_dim + 2u);
+            if (d == 0) {
+                part[0] = top;
+                part[1] = total;
+            }
+            part[2 + d] = o;
+            continue;
+        }
+        o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)(qh0 + h) * p.out_stride[1];
+        pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
+    }
+}
+
 // the shares of a (token, head) pair's history: out = sum_s o_s * exp(M_s - M) / sum_s l_s * exp(M_s - M)
 __global__ __launch_bounds__(256) void k_pa_merge(const PaParams p) {
     __shared__ float s_big[64], s_tot[64];  // splits <= 64
@@ -762,7 +1022,19 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
         hipLaunchKernelGGL(k_pa_write, per_token, dim3(a->head_dim <= 64 ? 64 : 128), 0, dev->stream, p);
     }
     MH_HIP(hipGetLastError());
-    if (epl == 4) {
+    // FLOAT16 cache rows of 128 contiguous values in blocks of 16 positions or more: the scores on the matrix cores
+    const bool mfma_scores = a->kv_dtype == MARMOT_HIP_DTYPE_F16 && p.kv_vec && a->head_dim == 128 && a->block_size >= 16 &&
+                             !dev->knobs.no_attention_mfma;
+    if (mfma_scores) {
+        const dim3 grid(p.token_count, p.num_q_heads / (uint32_t)qh, p.splits), block(256);
+        if (qh == 4) {
+            hipLaunchKernelGGL((k_pa_attend_mfma<4>), grid, block, 0, dev->stream, p);
+        } else if (qh == 2) {
+            hipLaunchKernelGGL((k_pa_attend_mfma<2>), grid, block, 0, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL((k_pa_attend_mfma<1>), grid, block, 0, dev->stream, p);
+        }
+    } else if (epl == 4) {
         qh == 4 ? pa_launch<4, 4>(dev, p) : qh == 2 ? pa_launch<4, 2>(dev, p) : pa_launch<4, 1>(dev, p);
     } else if (epl == 8) {
         qh == 4 ? pa_launch<8, 4>(dev, p) : qh == 2 ? pa_launch<8, 2>(dev, p) : pa_launch<8, 1>(dev, p);
@@ -775,6 +1047,6 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
                            dev->stream, p);
         MH_HIP(hipGetLastError());
     }
-    set_route("paged_attention");
+    set_route(mfma_scores ? "paged_attention_mfma_scores" : "paged_attention");
     return MARMOT_HIP_SUCCESS;
 }

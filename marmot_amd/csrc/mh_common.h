@@ -222,6 +222,7 @@ struct marmot_hip_knobs {
     bool no_mmq = false;
     bool no_row_kernels = false;
     bool no_resident_rows = false;
+    bool no_attention_mfma = false;  // MARMOT_HIP_NO_ATTENTION_MFMA: paged attention scores on the vector units
     bool no_lds_ring = false;
     bool no_fused_quant = false;
     bool no_gemm = false;

@@ -570,7 +570,8 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
     }
 }
 
-// ---- attention with the scores on the matrix cores (FLOAT16 cache rows of 128 values, blocks of 16 positions or more)
+// ---- attention with the scores on the matrix cores (FLOAT16 or BFLOAT16 cache rows of 128 values, blocks of 16
+// positions or more)
 // One workgroup of four wavefronts per (token, QH query heads of one key / value head, share of the history); a
 // wavefront takes tiles of 16 consecutive positions (one cache block, or a 16-aligned part of one).
 //   * Scores: S[position][head] = K[position][:] . q[head][:] as v_mfma_f32_16x16x16_f16 with the KEY ROWS as the row
@@ -578,8 +579,8 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
 //     contiguous bytes of dimensions 32 j .. 32 j + 31 of position r: the k index of the c-th instruction stands for
 //     dimensions 32 j + 4 c .. + 3, the same in both operands, so no value moves between lanes and none is converted).
 //     The query is the column operand, scaled and split once into a FLOAT16 high part and a FLOAT16 remainder (two
-//     instructions per step: products of FLOAT16 values are exact in fp32, the split leaves 2^-22 of the query).
-//     Columns beyond QH are zero.
+//     instructions per step: products of FLOAT16 values are exact in fp32, the split leaves 2^-22 of the query); for
+//     a BFLOAT16 cache (v_mfma_f32_16x16x16_bf16) into three BFLOAT16 parts of 8 bits each. Columns beyond QH are zero.
 //   * The result layout puts positions 4 j + i (i = 0..3) of head n in lane (n, j): the online softmax of a head runs in
 //     the four lanes n, n + 16, n + 32, n + 48 (two cross-lane exchanges per maximum and per sum).
 //   * Output: the 16 lanes of group j hold dimensions 8 n .. 8 n + 7 of the value rows of THEIR four positions; the
@@ -588,6 +589,7 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
 // The 16 partial outputs (4 wavefronts x 4 groups) meet in LDS like the 16 groups of k_pa_attend. fp32 accumulation
 // everywhere; only the order of the sums differs from the reference.
 typedef _Float16 pa_half4 __attribute__((ext_vector_type(4)));
+typedef short pa_short4 __attribute__((ext_vector_type(4)));
 typedef float pa_float4 __attribute__((ext_vector_type(4)));
 
 template <int PATTERN>
@@ -607,7 +609,7 @@ __device__ __forceinline__ float pa_xor32(float v) {
     return __shfl_xor(v, 32);
 }
 
-template <int QH>
+template <int QH, bool BF16>
 __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
     constexpr int EPL = 8;  // head_dim == 128
     __shared__ float s_acc[PA_GROUPS][QH][16 * EPL];
@@ -620,8 +622,9 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
     const uint32_t kv_len = seq < p.max_seqs ? pos + 1u : 0u;
     const uint32_t kvh = qh0 / p.group;
 
-    // the query: head n (zero beyond QH), dimensions 32 j .. 32 j + 31, scaled, as high part + remainder
-    pa_half4 qhi[8], qlo[8];
+    // the query: head n (zero beyond QH), dimensions 32 j .. 32 j + 31, scaled, as high part + remainder(s)
+    constexpr int PARTS = BF16 ? 3 : 2;
+    uint2 qpart[PARTS][8];  // four 16-bit values of the storage type each
     {
         float qv[32];
 #pragma unroll
@@ -649,15 +652,37 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
         }
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
+            uint16_t bits[PARTS][4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float v = p.scale != 1.0f ? qv[4 * c + e] * p.scale : qv[4 * c + e];
-                const _Float16 hi = (_Float16)v;
-                qhi[c][e] = hi;
-                qlo[c][e] = (_Float16)(v - (float)hi);
+                float v = p.scale != 1.0f ? qv[4 * c + e] * p.scale : qv[4 * c + e];
+#pragma unroll
+                for (int part = 0; part < PARTS; ++part) {  // each remainder is exact in fp32
+                    if constexpr (BF16) {
+                        bits[part][e] = pa_f2bf(v);
+                        v -= pa_bf2f(bits[part][e]);
+                    } else {
+                        bits[part][e] = f2h(v);
+                        v -= h2f(bits[part][e]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int part = 0; part < PARTS; ++part) {
+                qpart[part][c] = make_uint2((uint32_t)bits[part][0] | ((uint32_t)bits[part][1] << 16),
+                                            (uint32_t)bits[part][2] | ((uint32_t)bits[part][3] << 16));
             }
         }
     }
+    auto mma = [&](const uint2 kbits, const uint2 qbits, const pa_float4 c_in) -> pa_float4 {
+        if constexpr (BF16) {
+            return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(pa_short4, kbits),
+                                                             __builtin_bit_cast(pa_short4, qbits), c_in, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(pa_half4, kbits),
+                                                         __builtin_bit_cast(pa_half4, qbits), c_in, 0, 0, 0);
+        }
+    };
 
     float m = -INFINITY, lsum = 0.0f;  // of head n (replicated in the four lanes n + 16 j)
     float acc[QH][EPL];
@@ -700,12 +725,15 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
         pa_float4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const pa_half4 k0 = __builtin_bit_cast(pa_half4, make_uint2(kq[c].x, kq[c].y));
-            const pa_half4 k1 = __builtin_bit_cast(pa_half4, make_uint2(kq[c].z, kq[c].w));
-            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qhi[2 * c], sc, 0, 0, 0);
-            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k0, qlo[2 * c], sc, 0, 0, 0);
-            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qhi[2 * c + 1], sc, 0, 0, 0);
-            sc = __builtin_amdgcn_mfma_f32_16x16x16f16(k1, qlo[2 * c + 1], sc, 0, 0, 0);
+            const uint2 k0 = make_uint2(kq[c].x, kq[c].y), k1 = make_uint2(kq[c].z, kq[c].w);
+#pragma unroll
+            for (int part = 0; part < PARTS; ++part) {
+                sc = mma(k0, qpart[part][2 * c], sc);
+            }
+#pragma unroll
+            for (int part = 0; part < PARTS; ++part) {
+                sc = mma(k1, qpart[part][2 * c + 1], sc);
+            }
         }
         // positions beyond the sequence (the last tile): no score, no value
         const bool whole = p0 + 16u <= kv_len;
@@ -762,8 +790,13 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
             const uint32_t vw[4] = {vq[i].x, vq[i].y, vq[i].z, vq[i].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                vr[2 * e] = h2f((uint16_t)(vw[e] & 0xffffu));
-                vr[2 * e + 1] = h2f((uint16_t)(vw[e] >> 16));
+                if constexpr (BF16) {
+                    vr[2 * e] = __uint_as_float(vw[e] << 16);
+                    vr[2 * e + 1] = __uint_as_float(vw[e] & 0xffff0000u);
+                } else {
+                    vr[2 * e] = h2f((uint16_t)(vw[e] & 0xffffu));
+                    vr[2 * e + 1] = h2f((uint16_t)(vw[e] >> 16));
+                }
             }
             float wh[QH];
             wh[0] = pa_group_bcast<0>(w4[i]);
@@ -986,9 +1019,15 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     const int qh_max = epl == 16 ? 2 : 4;
     const int qh = (p.group % 4 == 0 && qh_max >= 4) ? 4 : (p.group % 2 == 0 ? 2 : 1);
     // few (token, heads) pairs (a decode step): the history is split over workgroups until the chip is about eight
-    // workgroups per compute unit deep, and a second kernel joins the shares
+    // (three for the matrix-core kernel) workgroups per compute unit deep, and a second kernel joins the shares
     const size_t pairs = (size_t)a->token_count * (a->num_q_heads / (uint32_t)qh);
-    const size_t want = 8u * (size_t)dev->props.multiProcessorCount;
+    // FLOAT16 cache rows of 128 contiguous values in blocks of 16 positions or more: the scores on the matrix cores
+    const bool kv_bf16 = a->kv_dtype == MARMOT_HIP_DTYPE_BF16;
+    const bool mfma_scores = (a->kv_dtype == MARMOT_HIP_DTYPE_F16 || kv_bf16) && p.kv_vec && a->head_dim == 128 &&
+                             a->block_size >= 16 && !dev->knobs.no_attention_mfma;
+    // (measured, 16 sequences x 4096 / x 512 positions, 32 / 8 heads: the matrix-core kernel 57.6 / 22.1 us at eight
+    // workgroups per compute unit, 56.2 / 16.2 at four, 50.5 / 17.0 at three, 52.1 / 15.5 at two, 76.1 / 17.0 at one)
+    const size_t want = (mfma_scores ? 3u : 8u) * (size_t)dev->props.multiProcessorCount;
     p.splits = 1;
     p.partial = nullptr;
     if (pairs * 2 <= want) {
@@ -1022,17 +1061,22 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
         hipLaunchKernelGGL(k_pa_write, per_token, dim3(a->head_dim <= 64 ? 64 : 128), 0, dev->stream, p);
     }
     MH_HIP(hipGetLastError());
-    // FLOAT16 cache rows of 128 contiguous values in blocks of 16 positions or more: the scores on the matrix cores
-    const bool mfma_scores = a->kv_dtype == MARMOT_HIP_DTYPE_F16 && p.kv_vec && a->head_dim == 128 && a->block_size >= 16 &&
-                             !dev->knobs.no_attention_mfma;
     if (mfma_scores) {
         const dim3 grid(p.token_count, p.num_q_heads / (uint32_t)qh, p.splits), block(256);
-        if (qh == 4) {
-            hipLaunchKernelGGL((k_pa_attend_mfma<4>), grid, block, 0, dev->stream, p);
+        if (kv_bf16) {
+            if (qh == 4) {
+                hipLaunchKernelGGL((k_pa_attend_mfma<4, true>), grid, block, 0, dev->stream, p);
+            } else if (qh == 2) {
+                hipLaunchKernelGGL((k_pa_attend_mfma<2, true>), grid, block, 0, dev->stream, p);
+            } else {
+                hipLaunchKernelGGL((k_pa_attend_mfma<1, true>), grid, block, 0, dev->stream, p);
+            }
+        } else if (qh == 4) {
+            hipLaunchKernelGGL((k_pa_attend_mfma<4, false>), grid, block, 0, dev->stream, p);
         } else if (qh == 2) {
-            hipLaunchKernelGGL((k_pa_attend_mfma<2>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<2, false>), grid, block, 0, dev->stream, p);
         } else {
-            hipLaunchKernelGGL((k_pa_attend_mfma<1>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<1, false>), grid, block, 0, dev->stream, p);
         }
     } else if (epl == 4) {
         qh == 4 ? pa_launch<4, 4>(dev, p) : qh == 2 ? pa_launch<4, 2>(dev, p) : pa_launch<4, 1>(dev, p);

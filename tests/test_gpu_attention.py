@@ -39,14 +39,14 @@ def run_oracle(oracle, case, **kw):
 def check(hip, oracle, case, what):
     got, kv_k, kv_v = run_hip(hip, case)
     # FLOAT16 caches with rows of 128 values in blocks of 16 positions or more take the kernel whose scores run on the
-    # matrix cores; everything else the kernel that works on the vector units
-    mfma = case["kv"] == "f16" and case["q"].shape[-1] == 128 and case["block_size"] >= 16
+    # matrix cores (BFLOAT16 caches likewise); everything else the kernel that works on the vector units
+    mfma = case["kv"] in ("f16", "bf16") and case["q"].shape[-1] == 128 and case["block_size"] >= 16
     assert hip.last_route() == ("paged_attention_mfma_scores" if mfma else "paged_attention"), what
     ref, ref_k, ref_v = run_oracle(oracle, case)
     assert np.array_equal(kv_k.view(np.uint8), ref_k.view(np.uint8)), f"{what}: key cache"
     assert np.array_equal(kv_v.view(np.uint8), ref_v.view(np.uint8)), f"{what}: value cache"
     act, kv = case["act"], case["kv"]
-    vmax = np.abs(to_f32(ref_v, kv)).max()
+    vmax = np.nanmax(np.abs(to_f32(ref_v, kv)))  # (rows that no token reads may hold NaN)
     g32, r32 = to_f32(got, act).astype(np.float64), to_f32(ref, act).astype(np.float64)
     assert np.max(np.abs(g32 - r32)) <= TOLERANCE[act] * vmax, f"{what}: against the oracle"
     dense = dense_reference(case, ref_k, ref_v)
@@ -83,6 +83,47 @@ def test_ragged_head_dims_and_block_sizes(hip, oracle, head_dim, block_size, hq,
     case = make_case(40 + head_dim, [(70, 3), (9, 1), (0, 2)], num_q_heads=hq, num_kv_heads=hkv, head_dim=head_dim,
                      block_size=block_size, act="f32", kv="f16")
     check(hip, oracle, case, f"head_dim={head_dim} block={block_size}")
+
+
+@pytest.mark.parametrize("kv", ["f16", "bf16"])
+@pytest.mark.parametrize("hq,hkv,block_size", [(3, 3, 16), (6, 3, 32), (8, 2, 16), (16, 2, 64), (4, 1, 128)])
+def test_matrix_core_scores_path(hip, oracle, hq, hkv, block_size, kv):
+    """FLOAT16 caches with rows of 128 values: the scores run on the matrix cores (key rows as the row operand, the query
+    split into two FLOAT16 parts). Histories that end on, before and behind a 16-position tile edge; one, two, four and
+    eight query heads per key / value head; NaN in every cache row no token may read (rows behind a sequence's end and
+    blocks outside the table); a hole in the table; queries of very large and very small magnitude."""
+    hists = [0, 14, 15, 16, 31, 32, 33, 255, 256, 257, 700]
+    case = make_case(900 + hq + block_size, [(h, 1) for h in hists] + [(40, 5)], num_q_heads=hq, num_kv_heads=hkv,
+                     head_dim=128, block_size=block_size, act="f32", kv=kv)
+    # rows that no token attends to: behind the last position of every sequence, and every unreferenced block
+    bs, table = block_size, case["block_table"]
+    nan = np.nan if kv == "f16" else np.uint16(0x7fc0)  # BFLOAT16 rows travel as bit patterns
+    last = {}
+    for seq, pos, _, _ in case["token_meta"]:
+        last[int(seq)] = max(last.get(int(seq), -1), int(pos))
+    used = np.zeros(case["kv_k"].shape[0], bool)
+    for seq, end in last.items():
+        for b in range(table.shape[1]):
+            tb = int(table[seq, b])
+            if tb == int(NO_BLOCK):
+                continue
+            used[tb] = True
+            lo = max(0, end + 1 - b * bs)
+            if lo < bs:
+                case["kv_k"][tb, :, :, lo:, :] = nan
+                case["kv_v"][tb, :, :, lo:, :] = nan
+    case["kv_k"][~used] = nan
+    case["kv_v"][~used] = nan
+    check(hip, oracle, case, f"matrix-core scores {hq}/{hkv} block {block_size}")
+    # a hole in the middle of the longest history
+    longest = max(last, key=last.get)
+    holed = dict(case, block_table=table.copy())
+    holed["block_table"][longest, 1] = NO_BLOCK
+    check(hip, oracle, holed, "matrix-core scores, hole")
+    # magnitudes: scores of +-60 (one position takes all the weight) and of 1e-6 (uniform weights)
+    for factor in (40.0, 1e-4):
+        scaled = dict(case, q=(case["q"] * np.float32(factor)).astype(np.float32))
+        check(hip, oracle, scaled, f"matrix-core scores, query x {factor}")
 
 
 def test_long_context_decode_batch(hip, oracle):

@@ -107,13 +107,9 @@ def time_steps_graph(hip, fn, steps: int, warmup: int, chunk: int = 500, repeats
 
         graphs.append(hip.graph_capture(body))
         done += n
-        if os.environ.get("BENCH_DEBUG"):
-            print(f"captured graph {len(graphs)} ({n} steps, {hip.graph_last_capture_nodes()} nodes)", file=sys.stderr, flush=True)
 
     def replay_ms():
-        for gi, g in enumerate(graphs):
-            if os.environ.get("BENCH_DEBUG"):
-                print(f"launch graph {gi}", file=sys.stderr, flush=True)
+        for g in graphs:
             hip.graph_launch(g)
             if profiled:
                 hip.synchronize()

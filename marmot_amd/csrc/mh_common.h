@@ -227,6 +227,8 @@ struct marmot_hip_knobs {
     bool no_fused_quant = false;
     bool no_gemm = false;
     bool no_gemm_loaders = false;
+    bool gemm_wide = false;      // MARMOT_HIP_GEMM_WIDE: the 128 x 128 prefill tile at every token count
+    bool no_gemm_wide = false;   // MARMOT_HIP_NO_GEMM_WIDE: never
     bool no_gemm_i8 = false;
     bool moe_no_validate = false;
 };

@@ -176,6 +176,8 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
     dev->knobs.no_fused_quant = getenv("MARMOT_HIP_NO_FUSED_QUANT") != nullptr;
     dev->knobs.no_gemm = getenv("MARMOT_HIP_NO_GEMM") != nullptr;
     dev->knobs.no_gemm_loaders = getenv("MARMOT_HIP_NO_GEMM_LOADERS") != nullptr;
+    dev->knobs.gemm_wide = getenv("MARMOT_HIP_GEMM_WIDE") != nullptr;
+    dev->knobs.no_gemm_wide = getenv("MARMOT_HIP_NO_GEMM_WIDE") != nullptr;
     dev->knobs.no_gemm_i8 = getenv("MARMOT_HIP_NO_GEMM_I8") != nullptr;
     dev->knobs.moe_no_validate = getenv("MARMOT_HIP_MOE_NO_VALIDATE") != nullptr;
     // default priority, non-blocking with respect to the legacy default stream

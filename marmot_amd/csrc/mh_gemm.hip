@@ -1289,6 +1289,436 @@ __global__ __launch_bounds__(L_THREADS) void k_gemm_q4k_f16_ls(const GemmParams 
     }
 }
 
+// ------------------------------------------------------------------ 128 tokens x 128 weight rows, loader wavefronts
+// The tile above spends most of the SIMD's issue slots on vector instructions that do not depend on the number of
+// tokens (the nibble unpack: 200 of 400 per block and wavefront). Here one unpacked weight operand feeds FOUR matrix
+// instructions: a compute wavefront owns 64 weight rows x all 128 tokens (2 x 4 tiles) and one K quarter of every
+// half-block. 128 accumulator registers per wavefront leave no room for a second set, so the block scale d is not
+// applied to a per-block product afterwards; the running tile T is kept in units of the current block's d instead:
+//     T <- T * (d_prev / d_b)        once per block, then the block's matrix instructions accumulate sc*q . x onto T,
+// and the min term of block b - 1 enters as -(dmin_(b-1) / d_b) * Q. Blocks with d == 0 keep the unit and run with
+// zero scales. Against the tile above this costs two more roundings per block and element (the ratio and the rescale),
+// the same order as the fp32 accumulation itself.
+//   * A round is HALF a block (128 values of K): three LDS stages of 128 tokens x 256 bytes of activations and
+//     128 rows x 80 bytes of weights (the 16-byte header and the 64 bytes of quants of this half), two rounds ahead.
+//   * wavefronts 4..7 load (32 tokens and a share of the weight pieces each) and compute the sub-block sums of the
+//     round in work; the sums of a block sit in one of two 4 KiB areas and are used one block late.
+//   * wavefronts 0..3 compute: (rg = rows 64 rg .. + 63, kg = the 64-value group 2 h + kg of the block in round h).
+// 512 tokens x 4096 rows are 128 such tiles; K is then split over two workgroups per tile.
+constexpr int W_TOK = 128;
+constexpr int W_WROWS = 128;
+constexpr int W_THREADS = 512;
+constexpr int W_STAGE_A = W_TOK * 256;              // 32,768
+constexpr int W_ROW = 80;                           // header + the quants of one half
+constexpr int W_STAGE_W = W_WROWS * W_ROW;          // 10,240
+constexpr int W_STAGE = W_STAGE_A + W_STAGE_W;
+constexpr int W_STAGES = 3;
+constexpr int W_SUMS = 4 * 64 * 16;                 // sub-block sums operand of the four token sub-tiles of one block
+constexpr int W_LDS_BYTES = W_STAGES * W_STAGE + 2 * W_SUMS;   // 137,216
+constexpr int W_OUT_PITCH = W_WROWS + 4;
+static_assert(W_TOK * W_OUT_PITCH * 4 <= W_STAGES * W_STAGE, "the output tile reuses the stages");
+
+__global__ __launch_bounds__(W_THREADS) void k_gemm_q4k_f16_wide(const GemmParams p) {
+    warm_kernel_arguments<sizeof(GemmParams)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * W_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nblk = (int)(b1 - b0);
+    const int nr = 2 * nblk;
+
+    floatx16 T[2][4];  // [row tile][token tile], compute wavefronts only
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                T[t][a][r] = 0.0f;
+            }
+        }
+    }
+    const int kg = (wave >> 1) & 1, rg = wave & 1;
+    const int j = lane & 31, kh = lane >> 5;
+    uint8_t *const sums_area = lds + W_STAGES * W_STAGE;
+
+    if (wave >= 4) {
+        // ------------------------------------------------------------------------------------------------ loaders
+        const int L = wave - 4;
+        const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+        const uint8_t *tile_x = (const uint8_t *)(p.x + tt * W_TOK * p.K) + b0 * 512;
+        const uint32_t row_pitch = (uint32_t)(p.K * 2);
+        const uint32_t last_row = (uint32_t)(p.N - 1 - tt * W_TOK);  // token rows beyond it re-read it
+        // Activations: token t of the tile owns 256 bytes of the stage as 16 chunks of 16 bytes, chunk c stored in slot
+        // c ^ (t % 16). Loader L brings tokens 32 L .. 32 L + 31, four per instruction.
+        uint32_t a_voff[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const uint32_t t = (uint32_t)(32 * L + 4 * c + (lane >> 4));
+            const uint32_t slot = (uint32_t)(lane & 15);
+            const uint32_t trow = t < last_row ? t : last_row;
+            a_voff[c] = trow * row_pitch + 16u * (slot ^ (t & 15u));
+        }
+        // Weights: piece q of the stage is 16 bytes q % 5 of tile row q / 5 (0: header, 1..4: the quants of this half);
+        // loader L brings pieces 64 (L + 4 pass) + lane. Rows beyond M re-read row M - 1 (never stored).
+        const size_t row_bytes = p.nb * Q4_K_BYTES;
+        const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+        uint32_t w_voff[3], w_half[3];
+#pragma unroll
+        for (int pass = 0; pass < 3; ++pass) {
+            const uint32_t q = (uint32_t)(64 * (L + 4 * pass) + lane);
+            const uint32_t r = q / 5u, c5 = q - 5u * r;
+            const uint32_t rr = r < last_wrow ? r : last_wrow;
+            w_voff[pass] = rr * (uint32_t)row_bytes + (c5 == 0 ? 0u : 16u * c5);
+            w_half[pass] = c5 == 0 ? 0u : 64u;
+        }
+        const uint8_t *wbase = p.w + row0 * row_bytes + b0 * Q4_K_BYTES;
+        const bool third = L < 2;  // pieces 512 .. 639
+        const int per_round = third ? 11 : 10;
+        auto issue = [&](int round, int stage) {
+            const uint32_t s0 = lds_base + (uint32_t)(stage * W_STAGE);
+            const uint8_t *xb = tile_x + (size_t)round * 256;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                dma_set_lds_base(s0 + (uint32_t)(8192 * L + 1024 * c));
+                dma16_to_lds<0>(xb, a_voff[c]);
+            }
+            const uint8_t *wb = wbase + (size_t)(round >> 1) * Q4_K_BYTES;
+            const uint32_t hsel = (round & 1) ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+                dma_set_lds_base(s0 + (uint32_t)(W_STAGE_A + 1024 * (L + 4 * pass)));
+                dma16_to_lds<0>(wb, w_voff[pass] + (w_half[pass] & hsel));
+            }
+            if (third) {
+                dma_set_lds_base(s0 + (uint32_t)(W_STAGE_A + 1024 * (L + 8)));
+                dma16_to_lds<0>(wb, w_voff[2] + (w_half[2] & hsel));
+            }
+        };
+        // Sub-block sums of this loader's 32 tokens: lane -> token 32 L + lane % 32, sub-blocks 2 (lane / 32) and + 1 of
+        // the half in work.
+        const int st = 32 * L + (lane & 31), pair = lane >> 5;
+        const uint32_t sum_dst = (uint32_t)(L * 1024 + (lane & 31) * 16 + 4 * pair);
+        auto sums = [&](int round, int stage) {
+            const uint8_t *sa = lds + (size_t)stage * W_STAGE;
+            float s0 = 0.0f, s1 = 0.0f;
+            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint4 v = *(const uint4 *)(sa + st * 256 + 16 * ((8 * pair + c) ^ (st & 15)));
+                float acc = c < 4 ? s0 : s1;
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.x), ones, acc, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.y), ones, acc, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.z), ones, acc, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, v.w), ones, acc, false);
+                if (c < 4) {
+                    s0 = acc;
+                } else {
+                    s1 = acc;
+                }
+            }
+            s0 *= 0.03125f;  // exact; keeps the value within fp16 range whatever the activations are
+            s1 *= 0.03125f;
+            const uint16_t h0 = f2h(s0), h1 = f2h(s1);
+            const uint16_t l0 = f2h(s0 - h2f(h0)), l1 = f2h(s1 - h2f(h1));
+            // S operand of token sub-tile a = L: lane i holds the 8 hi parts of token 32 a + i, lane 32 + i the lo parts
+            uint8_t *dst = sums_area + ((round >> 1) & 1) * W_SUMS + sum_dst + 8 * (round & 1);
+            *(uint32_t *)dst = (uint32_t)h0 | ((uint32_t)h1 << 16);
+            *(uint32_t *)(dst + 512) = (uint32_t)l0 | ((uint32_t)l1 << 16);
+        };
+
+        issue(0, 0);
+        issue(1, 1);
+        wait_vmcnt_at_most(per_round);
+        lds_barrier();
+        for (int i = 0; i < nr; ++i) {
+            if (i + 2 < nr) {
+                issue(i + 2, (i + 2) % W_STAGES);
+            }
+            compiler_memory_fence();
+            sums(i, i % W_STAGES);
+            if (i + 1 < nr) {
+                wait_vmcnt_at_most(i + 2 < nr ? per_round : 0);
+            }
+            lds_barrier();
+        }
+    } else {
+        // ------------------------------------------------------------------------------------------------ compute
+        // MFMA A operand of K-step i4 = 2 s + tp of a round (s: low / high nibbles = sub-block 2 g / 2 g + 1 of the
+        // wavefront's 64-value group g), token sub-tile a, lane (j, kh): token 32 a + j, chunk
+        // 8 kg + 4 s + 2 kh + tp of the token's 16.
+        uint32_t a_off[4];
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+            a_off[i4] = (uint32_t)(j * 256 + 16 * ((8 * kg + 4 * (i4 >> 1) + 2 * kh + (i4 & 1)) ^ (j & 15)));
+        }
+        const uint32_t w_off0 = (uint32_t)(W_STAGE_A + (64 * rg + j) * W_ROW);
+        const uint32_t q_off = (uint32_t)(16 + 32 * kg + 16 * kh);
+
+        float d_eff[2] = {1.0f, 1.0f};  // the unit of T[t]
+        uint32_t prev_mn_lo = 0, prev_mn_hi = 0;
+        float prev_ndmin = 0.0f;
+        // Q product of a block, all eight sub-blocks: row tile kg by the wavefronts of K quarter kg, one block late
+        auto q_term = [&](const uint8_t *s_area, float coeff, floatx16(&tot)[4]) {
+            const half8 b2 = mins_operand(prev_mn_lo, prev_mn_hi);
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const half8 a2 = __builtin_bit_cast(half8, *(const uint4 *)(s_area + ((size_t)a * 64 + lane) * 16));
+                const floatx16 zero = {0};
+                const floatx16 mq = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2, zero, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    tot[a][r] = __builtin_fmaf(coeff, mq[r], tot[a][r]);
+                }
+            }
+        };
+
+        auto round_fn = [&](int bb, int h) {
+            const int round = 2 * bb + h;
+            const uint8_t *stage = lds + (size_t)(round % W_STAGES) * W_STAGE;
+            uint4 wq[2];
+            uint32_t scw[2];
+            uint32_t mn_lo_t[2], mn_hi_t[2];
+            float dmin_t[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint8_t *wr = stage + w_off0 + t * 32 * W_ROW;
+                const uint4 hdr = *(const uint4 *)wr;
+                wq[t] = *(const uint4 *)(wr + q_off);
+                Scales sc;
+                decode_header(hdr, sc);
+                const bool dead = sc.d == 0.0f;
+                if (h == 0) {
+                    const float dn = dead ? d_eff[t] : sc.d;
+                    const float ratio = d_eff[t] / dn;
+                    d_eff[t] = dn;
+                    if (bb > 0) {
+#pragma unroll
+                        for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                T[t][a][r] *= ratio;
+                            }
+                        }
+                    }
+                }
+                const uint32_t word = h ? sc.sc_hi : sc.sc_lo;
+                scw[t] = dead ? 0u : (kg ? word >> 16 : word);
+                mn_lo_t[t] = sc.mn_lo;
+                mn_hi_t[t] = sc.mn_hi;
+                dmin_t[t] = sc.dmin;
+            }
+            if (h == 0 && bb > 0) {
+                const uint8_t *prev_s = sums_area + ((bb - 1) & 1) * W_SUMS;
+                if (kg == 0) {
+                    q_term(prev_s, prev_ndmin / d_eff[0], T[0]);
+                } else {
+                    q_term(prev_s, prev_ndmin / d_eff[1], T[1]);
+                }
+            }
+            if (h == 1) {
+                prev_mn_lo = kg ? mn_lo_t[1] : mn_lo_t[0];
+                prev_mn_hi = kg ? mn_hi_t[1] : mn_hi_t[0];
+                prev_ndmin = -(kg ? dmin_t[1] : dmin_t[0]);
+            }
+
+            __half2 scp[2], cp[2];
+            uint32_t m0[2] = {0, 0}, m1[2] = {0, 0};
+            // piece `piece` of B operand t for K-step i4 (nibble half s = i4 / 2, byte half tp = i4 % 2)
+            auto b_piece = [&](int t, int i4, int piece) -> uint32_t {
+                const int s_ = i4 >> 1, tp = i4 & 1;
+                if (piece == 0) {
+                    if (tp == 0) {
+                        const uint32_t sel = s_ == 0 ? 0x04000400u : 0x04010401u;
+                        scp[t] = __hsub2(as_h2(__builtin_amdgcn_perm(0x64646464u, scw[t], sel)), as_h2(0x64006400u));
+                        cp[t] = __hmul2(scp[t], as_h2(0xe400e400u));  // -1024 * sc, exact
+                    }
+                    const uint32_t q0 = tp ? wq[t].z : wq[t].x;
+                    const uint32_t q1 = tp ? wq[t].w : wq[t].y;
+                    m0[t] = (s_ ? (q0 >> 4) : q0) & 0x0f0f0f0fu;
+                    m1[t] = (s_ ? (q1 >> 4) : q1) & 0x0f0f0f0fu;
+                }
+                switch (piece) {
+                case 0: return dequant_pair<0>(m0[t], scp[t], cp[t]);
+                case 1: return dequant_pair<1>(m0[t], scp[t], cp[t]);
+                case 2: return dequant_pair<0>(m1[t], scp[t], cp[t]);
+                default: return dequant_pair<1>(m1[t], scp[t], cp[t]);
+                }
+            };
+            auto read_a = [&](int i4, half8(&aop)[4]) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    aop[a] = __builtin_bit_cast(half8, *(const uint4 *)(stage + a_off[i4] + a * 8192));
+                }
+            };
+
+            half8 aop[2][4];
+            uint32_t bop[2][2][4];
+            read_a(0, aop[0]);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int piece = 0; piece < 4; ++piece) {
+                    bop[0][t][piece] = b_piece(t, 0, piece);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int c = i4 & 1, n = c ^ 1;
+                if (i4 < 3) {
+                    read_a(i4 + 1, aop[n]);  // lands while the MFMAs below run
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const half8 bcur =
+                        __builtin_bit_cast(half8, make_uint4(bop[c][t][0], bop[c][t][1], bop[c][t][2], bop[c][t][3]));
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) {
+                        T[t][a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[c][a], bcur, T[t][a], 0, 0, 0);
+                        if (i4 < 3) {  // the next K-step's B operands, one piece in the shadow of each MFMA
+                            bop[n][t][a] = b_piece(t, i4 + 1, a);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+        };
+
+        lds_barrier();
+        for (int bb = 0; bb < nblk; ++bb) {
+            round_fn(bb, 0);
+            lds_barrier();
+            round_fn(bb, 1);
+            lds_barrier();
+        }
+        // leave the unit: T[t] in plain numbers, then the last block's Q product (its sums are complete since the last
+        // barrier)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    T[t][a][r] *= d_eff[t];
+                }
+            }
+        }
+        {
+            const uint8_t *last_s = sums_area + ((nblk - 1) & 1) * W_SUMS;
+            if (kg == 0) {
+                q_term(last_s, prev_ndmin, T[0]);
+            } else {
+                q_term(last_s, prev_ndmin, T[1]);
+            }
+        }
+    }
+
+    // ---- the two K quarters meet in LDS as one [token][weight row] tile, then every thread stores 16 bytes per step.
+    // Lane (j, kh) of compute wavefront (kg, rg) holds weight row 64 rg + 32 t + j for tokens
+    // 32 a + 8 (r / 4) + 4 kh + r % 4.
+    float *tile = (float *)lds;
+    if (wave < 4 && kg == 1) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * W_OUT_PITCH + 64 * rg + 32 * t + j] = T[t][a][r];
+                }
+            }
+        }
+    }
+    lds_barrier();
+    if (wave < 4 && kg == 0) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * W_OUT_PITCH + 64 * rg + 32 * t + j;
+                    *e = T[t][a][r] + *e;
+                }
+            }
+        }
+    }
+    lds_barrier();
+
+    const bool partials = p.splits > 1;
+    const bool has_bias = !partials && p.bias != nullptr;
+    const bool out_f16 = !partials && p.out_is_f16;
+    float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
+    const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    for (int idx = tid; idx < W_TOK * W_WROWS / 4; idx += W_THREADS) {
+        const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
+        const size_t n = tt * W_TOK + (size_t)t;
+        const size_t m4 = row0 + 4 * (size_t)q4;
+        if (n >= p.N || m4 >= p.M) {
+            continue;
+        }
+        const float4 v = *(const float4 *)(tile + t * W_OUT_PITCH + 4 * q4);
+        const float e4[4] = {v.x, v.y, v.z, v.w};
+        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (m4 + e < p.M) {
+                    bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
+                }
+            }
+        }
+        if (!out_f16) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[e] = has_bias ? e4[e] + bias4[e] : e4[e];
+            }
+            float *dst = out32 + n * p.M + m4;
+            if (vec) {  // M % 4 == 0: the four rows exist
+                *(float4 *)dst = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = o[e];
+                    }
+                }
+            }
+        } else {
+            uint16_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
+                if (has_bias) {
+                    h[e] = f2h(h2f(h[e]) + bias4[e]);
+                }
+            }
+            uint16_t *dst = (uint16_t *)p.out + n * p.M + m4;
+            if (vec) {
+                *(uint2 *)dst = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = h[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
 // sums the K-split partials in split order, then bias / output cast like the single-pass epilogue
 template <int V>
 __global__ __launch_bounds__(256) void k_gemm_reduce(const float *__restrict__ partial, int splits, size_t N, size_t M,
@@ -1446,6 +1876,39 @@ static int launch_gemm_ls(marmot_hip_device *dev, GemmParams p, size_t N, size_t
     return MARMOT_HIP_SUCCESS;
 }
 
+static int launch_gemm_wide(marmot_hip_device *dev, GemmParams p, size_t N, size_t K, size_t M, const void *d_bias,
+                            int bias_dtype, void *d_out, int out_dtype) {
+    const size_t nb = K / QK_K;
+    const size_t tiles_n = (N + W_TOK - 1) / W_TOK;
+    const size_t tiles_m = (M + W_WROWS - 1) / W_WROWS;
+    const size_t tiles = tiles_n * tiles_m;
+    const size_t cus = (size_t)dev->props.multiProcessorCount;
+    size_t splits = 1;
+    if (tiles * 2 <= cus) {  // fewer tiles than half the chip: split K across workgroups
+        splits = cus / tiles;
+        splits = splits > nb ? nb : splits;
+    }
+    const size_t blocks_per_split = (nb + splits - 1) / splits;
+    splits = (nb + blocks_per_split - 1) / blocks_per_split;
+    float *partial = nullptr;
+    if (splits > 1) {
+        void *ws = nullptr;
+        MH_TRY(workspace_reserve(dev, splits * N * M * sizeof(float), &ws));
+        partial = (float *)ws;
+    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q4k_f16_wide));
+    p.out = splits > 1 ? (void *)partial : d_out;
+    p.splits = (int)splits;
+    p.blocks_per_split = (int)blocks_per_split;
+    hipLaunchKernelGGL(k_gemm_q4k_f16_wide, dim3((unsigned)tiles_m, (unsigned)tiles_n, (unsigned)splits),
+                       dim3(W_THREADS), W_LDS_BYTES, dev->stream, p);
+    MH_HIP(hipGetLastError());
+    if (splits > 1) {
+        MH_TRY(launch_splitk_reduce(dev, partial, (int)splits, N, M, d_bias, bias_dtype, d_out, out_dtype));
+    }
+    return MARMOT_HIP_SUCCESS;
+}
+
 static int launch_gemm_big(marmot_hip_device *dev, GemmParams p, size_t N, size_t K, size_t M, const void *d_bias,
                            int bias_dtype, void *d_out, int out_dtype) {
     const size_t nb = K / QK_K;
@@ -1519,6 +1982,15 @@ int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const voi
     }
     // the loader-wavefront kernel moves 16-byte pieces of the weight blocks; K < 2^22 keeps its 32-bit offsets exact
     if (!dev->knobs.no_gemm_loaders && (((uintptr_t)d_w) & 15) == 0 && K < ((size_t)1 << 22)) {
+        // 128 x 128 tiles when one round of them covers most of the chip with the whole K inside each workgroup
+        // (513 .. 1024 tokens at 4096 rows): one unpacked weight operand then feeds four matrix instructions
+        const size_t wide_tiles = ((N + W_TOK - 1) / W_TOK) * ((M + W_WROWS - 1) / W_WROWS);
+        const size_t ls_tiles = ((N + L_TOK - 1) / L_TOK) * ((M + L_WROWS - 1) / L_WROWS);
+        const bool wide = wide_tiles <= cus && 8 * wide_tiles >= 5 * cus && ls_tiles > cus;
+        if (dev->knobs.gemm_wide || (wide && !dev->knobs.no_gemm_wide)) {
+            set_route("gemm_q4_k_f16_mfma_wide");
+            return launch_gemm_wide(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
+        }
         return launch_gemm_ls(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);
     }
     return launch_gemm_shape<2, 2>(dev, p, N, K, M, d_bias, bias_dtype, d_out, out_dtype);

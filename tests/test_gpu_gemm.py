@@ -144,3 +144,64 @@ def test_gemm_loader_tile_and_self_loading_tile_agree(oracle, monkeypatch):
     finally:
         loaders.close()
         plain.close()
+
+
+def test_gemm_wide_tile(oracle, monkeypatch):
+    """The 128 x 128 tile keeps its running sums in units of the current block's super-block scale (one rescale per
+    block instead of a second accumulator set). Forced at every token count with MARMOT_HIP_GEMM_WIDE: ragged token /
+    row counts, one block of K, K split across workgroups, every scale / min / nibble pattern with super-block scales
+    of both signs down to fp16 denormals, blocks and whole rows whose scale is zero, bias and fp16 output; and the
+    default device must take the tile by itself where one round of such tiles covers most of the chip."""
+    from marmot_amd import HipBackend
+
+    monkeypatch.setenv("MARMOT_HIP_GEMM_WIDE", "1")
+    wide = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_GEMM_WIDE")
+    plain = HipBackend(0)
+    try:
+        cases = [(9, 256, 33), (130, 256, 128), (256, 512, 128), (300, 768, 515), (512, 1024, 300), (640, 2048, 640)]
+        for n, (N, K, M) in enumerate(cases):
+            print(f"wide tile N={N} K={K} M={M}", flush=True)
+            blocks = oracle.quantize(KIND_Q4_K, gaussian(660 + n, (M, K), 0.02))
+            x = gaussian(670 + n, (N, K)).astype(np.float16)
+            bias = gaussian(680 + n, (M,)) if n % 2 else None
+            a, ref = check_against_oracle(wide, oracle, blocks, x, M, K, f"wide tile {N}x{K}x{M}", bias=bias)
+            assert wide.last_route() == "gemm_q4_k_f16_mfma_wide"
+            b, _ = check_against_oracle(plain, oracle, blocks, x, M, K, f"default tile {N}x{K}x{M}", bias=bias)
+            assert np.max(np.abs(a - b)) <= 1e-5 * np.max(np.abs(ref))
+        rng = np.random.default_rng(690)
+        M, K, N = 256, 2048, 200
+        blocks = random_valid_blocks(rng, KIND_Q4_K, M, K)
+        x = (gaussian(691, (N, K)) * 300.0).astype(np.float16)
+        x[0, :] = 60000.0
+        x[1, :] = 0.0
+        check_against_oracle(wide, oracle, blocks, x, M, K, "wide tile random bytes")
+        dead = blocks.copy().reshape(M, K // 256, 144)
+        dead[::3, 1, 0:2] = 0   # a block in the middle of every third row
+        dead[5, :, 0:2] = 0     # a whole row (its min terms remain)
+        dead[7, 0, 0:2] = 0     # the first block of a row
+        dead[9, -1, 0:2] = 0    # the last one
+        dead[11, 2:5, 0:2] = 0  # a run
+        dead = dead.reshape(blocks.shape)
+        bias = gaussian(692, (M,)).astype(np.float16)
+        check_against_oracle(wide, oracle, dead, x, M, K, "wide tile zero scales")
+        soft = oracle.quantize(KIND_Q4_K, gaussian(694, (M, K), 0.02)).reshape(M, K // 256, 144).copy()
+        soft[::4, 3, 0:2] = 0
+        soft[6, :, 0:2] = 0
+        x16 = gaussian(695, (N, K)).astype(np.float16)
+        check_against_oracle(wide, oracle, soft.reshape(blocks.shape), x16, M, K, "wide tile f16 out", bias=bias,
+                             out_dtype=np.float16)
+        # the band the default route takes by itself: 6 x 32 tiles at 768 tokens x 4096 rows on 256 compute units
+        M = K = 4096
+        N = 768
+        blocks = quantize_weights(oracle, KIND_Q4_K, gaussian(30, (M, K), 0.02))
+        x = gaussian(693, (N, K)).astype(np.float16)
+        got = plain.linear(x, blocks, KIND_Q4_K, M)
+        units = plain.caps()["num_compute_units"]
+        if 192 <= units and 8 * 192 >= 5 * units:
+            assert plain.last_route() == "gemm_q4_k_f16_mfma_wide", plain.last_route()
+        exact = exact_f64(oracle, blocks[1000:1256], x, 256, K)
+        assert parity_metrics(got[:, 1000:1256], exact)[2] <= 2e-6
+    finally:
+        wide.close()
+        plain.close()

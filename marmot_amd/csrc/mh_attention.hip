@@ -547,6 +547,13 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
             big = fmaxf(big, s_m[gg][h]);
         }
         float o = 0.0f, total = 0.0f;
+        // a NaN score (NaN in the query or in a row of the history) leaves a NaN sum of weights in its group: the head's
+        // output is NaN then, as in the reference, whatever the maxima say (they skip NaN)
+        bool bad = false;
+#pragma unroll
+        for (int gg = 0; gg < PA_GROUPS; ++gg) {
+            bad = bad || s_l[gg][h] != s_l[gg][h];
+        }
         if (big != -INFINITY) {  // has_any (:552-557)
 #pragma unroll
             for (int gg = 0; gg < PA_GROUPS; ++gg) {
@@ -559,12 +566,12 @@ __global__ __launch_bounds__(16 * PA_GROUPS) void k_pa_attend(const PaParams p) 
             float *part = p.partial + (((size_t)t * p.num_q_heads + qh0 + h) * p.splits + blockIdx.z) * (p.head_dim + 2u);
             if (d == 0) {
                 part[0] = big;
-                part[1] = total;
+                part[1] = bad ? __uint_as_float(0x7fc00000u) : total;
             }
             part[2 + d] = o;
             continue;
         }
-        o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        o = bad ? __uint_as_float(0x7fc00000u) : (total > 0.0f ? o * (1.0f / total) : 0.0f);
         const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)(qh0 + h) * p.out_stride[1];
         pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
     }
@@ -609,8 +616,33 @@ __device__ __forceinline__ float pa_xor32(float v) {
     return __shfl_xor(v, 32);
 }
 
-template <int QH, bool BF16>
+// Four e4m3 codes of a word as two words of FLOAT16 pairs holding the codes' values times 2^-8: a code moved to the
+// high byte of a half and shifted right by one (arithmetic) has its sign in bit 15 and its exponent and mantissa where
+// FLOAT16 keeps them, with the exponent bias 8 too small; denormal codes stay exact (both formats are linear there).
+// Codes with all exponent bits set (NaN in the reference's e4m3) come out as finite values: pa_fp8_nan_bits finds them.
+typedef short pa_short2 __attribute__((ext_vector_type(2)));
+template <int HI>
+__device__ __forceinline__ uint32_t pa_fp8x2_to_f16(uint32_t w) {
+    const uint32_t x = __builtin_amdgcn_perm(w, w, HI ? 0x030c020cu : 0x010c000cu);
+    const pa_short2 sh = __builtin_bit_cast(pa_short2, x) >> (short)1;
+    return __builtin_bit_cast(uint32_t, sh) & 0xbf80bf80u;
+}
+// bit 7 of a byte is set iff that byte of w is a NaN code (exponent field 15)
+__device__ __forceinline__ uint32_t pa_fp8_nan_bits(uint32_t w) {
+    return (w & 0x78787878u) + 0x08080808u;
+}
+// the same two words through the reference's decoder (NaN codes become NaN)
+template <int HI>
+__device__ __forceinline__ uint32_t pa_fp8x2_to_f16_slow(uint32_t w) {
+    const uint32_t c0 = (w >> (HI ? 16 : 0)) & 0xffu, c1 = (w >> (HI ? 24 : 8)) & 0xffu;
+    return (uint32_t)f2h(pa_fp8_to_f32(c0) * 0.00390625f) | ((uint32_t)f2h(pa_fp8_to_f32(c1) * 0.00390625f) << 16);
+}
+
+constexpr int PA_KV_F16 = 0, PA_KV_BF16 = 1, PA_KV_FP8 = 2;
+
+template <int QH, int KVT>
 __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
+    constexpr bool BF16 = KVT == PA_KV_BF16, FP8 = KVT == PA_KV_FP8;
     constexpr int EPL = 8;  // head_dim == 128
     __shared__ float s_acc[PA_GROUPS][QH][16 * EPL];
     __shared__ float s_m[PA_GROUPS][QH], s_l[PA_GROUPS][QH];
@@ -712,15 +744,81 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
         }
         const size_t tile_base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(p0 & p.mask) * p.kv_stride[3];
         // key rows: position n of the tile, dimensions 32 j .. + 31; value rows: positions 4 j + i, dimensions 8 n .. + 7
-        const uint16_t *krow = (const uint16_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
         uint4 kq[4], vq[4];
+        float k_unit = 1.0f, v_unit = 1.0f;  // FLOAT8_E4M3: what one unit of the FLOAT16 operands stands for
+        if constexpr (FP8) {
+            // codes -> FLOAT16 operands in registers (exact); the block's scale and the 2^8 of the conversion are applied
+            // to the scores and to the softmax weights. A scale that is not positive decodes to zeros (the reference's
+            // cpu_paged_attention_fp8_dequant); a tile that holds a NaN code takes the reference's decoder.
+            const size_t si = (size_t)tb * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] +
+                              (size_t)kvh * p.scale_stride[2];
+            const float ks = p.k_scale[si], vs = p.v_scale[si];
+            const uint8_t *krow = (const uint8_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
+            const uint4 kr0 = *(const uint4 *)krow, kr1 = *(const uint4 *)(krow + 16);
+            uint2 vr[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            kq[c] = *(const uint4 *)(krow + 8 * c);
-        }
+            for (int i = 0; i < 4; ++i) {
+                vr[i] = *(const uint2 *)((const uint8_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+            }
+            const uint32_t kw[8] = {kr0.x, kr0.y, kr0.z, kr0.w, kr1.x, kr1.y, kr1.z, kr1.w};
+            uint32_t nan_k = 0, nan_v = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            vq[i] = *(const uint4 *)((const uint16_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+            for (int c = 0; c < 8; ++c) {
+                nan_k |= pa_fp8_nan_bits(kw[c]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                nan_v |= pa_fp8_nan_bits(vr[i].x) | pa_fp8_nan_bits(vr[i].y);
+            }
+            const bool k_live = ks > 0.0f, v_live = vs > 0.0f;
+            const bool slow = ((nan_k & 0x80808080u) != 0 && k_live) || ((nan_v & 0x80808080u) != 0 && v_live);
+            if (__builtin_amdgcn_ballot_w64(slow) == 0) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    kq[c] = make_uint4(pa_fp8x2_to_f16<0>(kw[2 * c]), pa_fp8x2_to_f16<1>(kw[2 * c]),
+                                       pa_fp8x2_to_f16<0>(kw[2 * c + 1]), pa_fp8x2_to_f16<1>(kw[2 * c + 1]));
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    vq[i] = make_uint4(pa_fp8x2_to_f16<0>(vr[i].x), pa_fp8x2_to_f16<1>(vr[i].x),
+                                       pa_fp8x2_to_f16<0>(vr[i].y), pa_fp8x2_to_f16<1>(vr[i].y));
+                }
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    kq[c] = make_uint4(pa_fp8x2_to_f16_slow<0>(kw[2 * c]), pa_fp8x2_to_f16_slow<1>(kw[2 * c]),
+                                       pa_fp8x2_to_f16_slow<0>(kw[2 * c + 1]), pa_fp8x2_to_f16_slow<1>(kw[2 * c + 1]));
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    vq[i] = make_uint4(pa_fp8x2_to_f16_slow<0>(vr[i].x), pa_fp8x2_to_f16_slow<1>(vr[i].x),
+                                       pa_fp8x2_to_f16_slow<0>(vr[i].y), pa_fp8x2_to_f16_slow<1>(vr[i].y));
+                }
+            }
+            if (!k_live) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    kq[c] = make_uint4(0, 0, 0, 0);
+                }
+            }
+            if (!v_live) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    vq[i] = make_uint4(0, 0, 0, 0);
+                }
+            }
+            k_unit = k_live ? ks * 256.0f : 0.0f;
+            v_unit = v_live ? vs * 256.0f : 0.0f;
+        } else {
+            const uint16_t *krow = (const uint16_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                kq[c] = *(const uint4 *)(krow + 8 * c);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                vq[i] = *(const uint4 *)((const uint16_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+            }
         }
         pa_float4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -738,6 +836,12 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
         // positions beyond the sequence (the last tile): no score, no value
         const bool whole = p0 + 16u <= kv_len;
         float s4[4] = {sc[0], sc[1], sc[2], sc[3]};
+        if constexpr (FP8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s4[i] *= k_unit;
+            }
+        }
         if (!whole) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -799,13 +903,14 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
                 }
             }
             float wh[QH];
-            wh[0] = pa_group_bcast<0>(w4[i]);
+            const float wi = FP8 ? w4[i] * v_unit : w4[i];  // the value rows' unit goes with the weight
+            wh[0] = pa_group_bcast<0>(wi);
             if constexpr (QH > 1) {
-                wh[1] = pa_group_bcast<1>(w4[i]);
+                wh[1] = pa_group_bcast<1>(wi);
             }
             if constexpr (QH > 2) {
-                wh[2] = pa_group_bcast<2>(w4[i]);
-                wh[3] = pa_group_bcast<3>(w4[i]);
+                wh[2] = pa_group_bcast<2>(wi);
+                wh[3] = pa_group_bcast<3>(wi);
             }
 #pragma unroll
             for (int h = 0; h < QH; ++h) {
@@ -840,6 +945,13 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
             top = fmaxf(top, s_m[gg][h]);
         }
         float o = 0.0f, total = 0.0f;
+        // a NaN score (NaN in the query or in a row of the history) leaves a NaN sum of weights in its group: the head's
+        // output is NaN then, as in the reference, whatever the maxima say (they skip NaN)
+        bool bad = false;
+#pragma unroll
+        for (int gg = 0; gg < PA_GROUPS; ++gg) {
+            bad = bad || s_l[gg][h] != s_l[gg][h];
+        }
         if (top != -INFINITY) {
 #pragma unroll
             for (int gg = 0; gg < PA_GROUPS; ++gg) {
@@ -852,12 +964,12 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
             float *part = p.partial + (((size_t)t * p.num_q_heads + qh0 + h) * p.splits + blockIdx.z) * (p.head_dim + 2u);
             if (d == 0) {
                 part[0] = top;
-                part[1] = total;
+                part[1] = bad ? __uint_as_float(0x7fc00000u) : total;
             }
             part[2 + d] = o;
             continue;
         }
-        o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        o = bad ? __uint_as_float(0x7fc00000u) : (total > 0.0f ? o * (1.0f / total) : 0.0f);
         const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)(qh0 + h) * p.out_stride[1];
         pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
     }
@@ -880,6 +992,10 @@ __global__ __launch_bounds__(256) void k_pa_merge(const PaParams p) {
     const size_t out_base = (size_t)t * p.out_stride[0] + (size_t)qh * p.out_stride[1];
     for (uint32_t d = threadIdx.x; d < p.head_dim; d += blockDim.x) {
         float o = 0.0f, total = 0.0f;
+        bool bad = false;  // a share saw a NaN score
+        for (uint32_t z = 0; z < p.splits; ++z) {
+            bad = bad || s_tot[z] != s_tot[z];
+        }
         if (big != -INFINITY) {
             for (uint32_t z = 0; z < p.splits; ++z) {
                 const float f = s_big[z] == -INFINITY ? 0.0f : pa_exp(s_big[z] - big);
@@ -887,7 +1003,7 @@ __global__ __launch_bounds__(256) void k_pa_merge(const PaParams p) {
                 o = __builtin_fmaf(part[(size_t)z * (p.head_dim + 2u) + 2 + d], f, o);
             }
         }
-        o = total > 0.0f ? o * (1.0f / total) : 0.0f;
+        o = bad ? __uint_as_float(0x7fc00000u) : (total > 0.0f ? o * (1.0f / total) : 0.0f);
         pa_store(p.out, p.act_dtype, out_base + (size_t)d * p.out_stride[2], o);
     }
 }
@@ -1023,8 +1139,12 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     const size_t pairs = (size_t)a->token_count * (a->num_q_heads / (uint32_t)qh);
     // FLOAT16 cache rows of 128 contiguous values in blocks of 16 positions or more: the scores on the matrix cores
     const bool kv_bf16 = a->kv_dtype == MARMOT_HIP_DTYPE_BF16;
-    const bool mfma_scores = (a->kv_dtype == MARMOT_HIP_DTYPE_F16 || kv_bf16) && p.kv_vec && a->head_dim == 128 &&
-                             a->block_size >= 16 && !dev->knobs.no_attention_mfma;
+    bool rows16 = (((uintptr_t)a->d_kv_k) & 15) == 0;  // FLOAT8_E4M3: 16 codes per load of a key row
+    for (int i = 0; i < 4; ++i) {
+        rows16 = rows16 && (a->kv_stride[i] * ksz) % 16 == 0;
+    }
+    const bool mfma_scores = (a->kv_dtype == MARMOT_HIP_DTYPE_F16 || kv_bf16 || (fp8 && rows16)) && p.kv_vec &&
+                             a->head_dim == 128 && a->block_size >= 16 && !dev->knobs.no_attention_mfma;
     // (measured, 16 sequences x 4096 / x 512 positions, 32 / 8 heads: the matrix-core kernel 57.6 / 22.1 us at eight
     // workgroups per compute unit, 56.2 / 16.2 at four, 50.5 / 17.0 at three, 52.1 / 15.5 at two, 76.1 / 17.0 at one)
     const size_t want = (mfma_scores ? 3u : 8u) * (size_t)dev->props.multiProcessorCount;
@@ -1063,20 +1183,28 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     MH_HIP(hipGetLastError());
     if (mfma_scores) {
         const dim3 grid(p.token_count, p.num_q_heads / (uint32_t)qh, p.splits), block(256);
-        if (kv_bf16) {
+        if (fp8) {
             if (qh == 4) {
-                hipLaunchKernelGGL((k_pa_attend_mfma<4, true>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_FP8>), grid, block, 0, dev->stream, p);
             } else if (qh == 2) {
-                hipLaunchKernelGGL((k_pa_attend_mfma<2, true>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_FP8>), grid, block, 0, dev->stream, p);
             } else {
-                hipLaunchKernelGGL((k_pa_attend_mfma<1, true>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_FP8>), grid, block, 0, dev->stream, p);
+            }
+        } else if (kv_bf16) {
+            if (qh == 4) {
+                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_BF16>), grid, block, 0, dev->stream, p);
+            } else if (qh == 2) {
+                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_BF16>), grid, block, 0, dev->stream, p);
+            } else {
+                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_BF16>), grid, block, 0, dev->stream, p);
             }
         } else if (qh == 4) {
-            hipLaunchKernelGGL((k_pa_attend_mfma<4, false>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_F16>), grid, block, 0, dev->stream, p);
         } else if (qh == 2) {
-            hipLaunchKernelGGL((k_pa_attend_mfma<2, false>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_F16>), grid, block, 0, dev->stream, p);
         } else {
-            hipLaunchKernelGGL((k_pa_attend_mfma<1, false>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_F16>), grid, block, 0, dev->stream, p);
         }
     } else if (epl == 4) {
         qh == 4 ? pa_launch<4, 4>(dev, p) : qh == 2 ? pa_launch<4, 2>(dev, p) : pa_launch<4, 1>(dev, p);

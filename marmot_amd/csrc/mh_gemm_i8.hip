@@ -990,6 +990,184 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
     i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
+// ------------------------------------------------------------------ Q8_0 / Q4_0 x Q8_0
+// cpu_vec_dot_q8_0_q8_0 / cpu_vec_dot_q4_0_q8_0 (vec_dot_impl.h:452-479 and its Q4_0 sibling): per 32-value block
+//     y += (float)(q . a) * (w.d * a.d),
+// integer dot exact, one fp32 multiply-add per block in block order. Here a block of 32 weight rows x 32 tokens is one
+// v_mfma_i32_32x32x32_i8, and every output takes its block's product of the two scales with three vector
+// instructions (convert, scale product, multiply-add): the formats have one scale per 32 values and nothing to fold,
+// so the kernel is bound by these, at about an eighth of the int8 peak.
+// Same tile and wavefront roles as the Q6_K kernel: a round is 256 values of K (eight blocks), K group kg takes blocks
+// 4 kg .. 4 kg + 3 of every round. Weight rows must be a multiple of eight blocks (K % 256 == 0: rows and rounds start
+// on 16-byte boundaries); the stage holds each row's 272 (Q8_0) / 144 (Q4_0) bytes of the round at a pitch of 304 / 144
+// bytes (lanes 0..15 of a read then fall into different banks), the activation tile as in the kernels above, and the
+// 8 x 64 activation scales of the round as [block][token] (one dword gather per block and round).
+template <int KIND>
+struct Q80Tile {
+    static constexpr int BLK = KIND == MARMOT_HIP_KIND_Q8_0 ? 34 : 18;
+    static constexpr int CHUNK = 8 * BLK;
+    static constexpr int PIECES = CHUNK / 16;
+    static constexpr int PITCH_P = KIND == MARMOT_HIP_KIND_Q8_0 ? 19 : 9;
+    static constexpr int ROWB = PITCH_P * 16;
+    static constexpr int STAGE_W = I8_WROWS * ROWB;
+    static constexpr int STAGE_D = 8 * I8_TOK * 4;
+    static constexpr int STAGE = STAGE_W + I8_STAGE_A + STAGE_D;
+    static constexpr int LDS_BYTES = 2 * STAGE;
+    static constexpr int W_INSTR = (I8_WROWS * PITCH_P + 63) / 64;
+    static constexpr int W_PER_WAVE = (W_INSTR + I8_WAVES - 1) / I8_WAVES;
+    static_assert(CHUNK % 16 == 0 && STAGE % 16 == 0, "16-byte pieces");
+    static_assert(I8_TOK * I8_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
+};
+
+// p.nb counts rounds (K / 256); p.ad holds 8 p.nb scales per token
+template <int KIND>
+__global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params p) {
+    using T = Q80Tile<KIND>;
+    warm_kernel_arguments<sizeof(GemmI8Params)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = wave & 3;   // weight rows 32 rg .. + 31 of the tile
+    const int kg = wave >> 2;  // blocks 4 kg .. 4 kg + 3 of every round
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * I8_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nrounds = (int)(b1 - b0);
+    const int j = lane & 31, kh = lane >> 5;
+
+    float total[2][16];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
+        }
+    }
+
+    // ---- loads per round: 16 activation instructions (two per wavefront), W_INSTR weight instructions of 64 piece
+    // slots (wavefront w takes instructions w, w + 8, ...), one gather of 64 activation scales per wavefront
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
+    uint32_t a_voff[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const uint32_t t = (uint32_t)(8 * wave + 4 * c + (lane >> 4));
+        const uint32_t slot = (uint32_t)(lane & 15);
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+    }
+    const size_t row_bytes = p.nb * T::CHUNK;
+    const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
+    uint32_t w_voff[T::W_PER_WAVE];
+    bool w_on[T::W_PER_WAVE];
+#pragma unroll
+    for (int m = 0; m < T::W_PER_WAVE; ++m) {
+        const uint32_t q = (uint32_t)(64 * (wave + 8 * m) + lane);  // piece slot: row q / PITCH_P, piece q % PITCH_P
+        const uint32_t r = q / (uint32_t)T::PITCH_P, pc = q - (uint32_t)T::PITCH_P * r;
+        const uint32_t rr = r < last_wrow ? r : last_wrow;  // rows beyond M re-read row M - 1 (never stored)
+        w_voff[m] = rr * (uint32_t)row_bytes + 16u * pc;
+        w_on[m] = wave + 8 * m < T::W_INSTR && r < (uint32_t)I8_WROWS && pc < (uint32_t)T::PIECES;
+    }
+    const uint8_t *wbase = p.w + row0 * row_bytes;
+    uint32_t d_voff;
+    {
+        const uint32_t t = (uint32_t)lane;
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        d_voff = (uint32_t)((trow * 8u * p.nb + (uint32_t)wave) * 4u);  // block `wave` of the round, token `lane`
+    }
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * 8u * p.nb);
+    auto issue = [&](int ri) {
+        const size_t b = b0 + (size_t)ri;
+        const uint32_t s0 = lds_base + (uint32_t)((ri & 1) * T::STAGE);
+        const uint8_t *qb = tile_q + b * QK_K;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            dma_set_lds_base(s0 + (uint32_t)(T::STAGE_W + 2048 * wave + 1024 * c));
+            dma16_to_lds<0>(qb, a_voff[c]);
+        }
+        const uint8_t *wb = wbase + b * T::CHUNK;
+#pragma unroll
+        for (int m = 0; m < T::W_PER_WAVE; ++m) {
+            if (wave + 8 * m < T::W_INSTR) {  // uniform over the wavefront
+                dma_set_lds_base(s0 + (uint32_t)(1024 * (wave + 8 * m)));
+                if (w_on[m]) {
+                    dma16_to_lds<0>(wb, w_voff[m]);
+                }
+            }
+        }
+        dma_set_lds_base(s0 + (uint32_t)(T::STAGE_W + I8_STAGE_A + 256 * wave));
+        dma4_to_lds(tile_d + b * 32, d_voff);
+    };
+
+    // ---- compute: weight row 32 rg + j, the lane's 16 values (16 kh .. + 15) of each of its four blocks, all 64 tokens
+    const uint32_t w_off = (uint32_t)((32 * rg + j) * T::ROWB);
+    const uint32_t a_base = (uint32_t)(T::STAGE_W + j * QK_K);
+    const uint32_t d_off = (uint32_t)(T::STAGE_W + I8_STAGE_A + 16 * kh);
+
+    issue(0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    i8_lds_barrier();
+    for (int ri = 0; ri < nrounds; ++ri) {
+        if (ri + 1 < nrounds) {
+            issue(ri + 1);  // into the other buffer, which the barrier that closed the previous round has released
+        }
+        {
+            const uint8_t *stage = lds + (size_t)(ri & 1) * T::STAGE;
+            const uint8_t *wrow = stage + w_off;
+            const i8_intx16 zero = {0};
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi) {
+                const int blk = 4 * kg + bi;
+                uint16_t dh;
+                __builtin_memcpy(&dh, wrow + T::BLK * blk, 2);
+                float dw = h2f(dh);
+                asm volatile("" : "+v"(dw));  // a conversion of its own (not folded into mixed-precision multiplies)
+                i8_intx4 wv;
+                if constexpr (KIND == MARMOT_HIP_KIND_Q8_0) {
+                    __builtin_memcpy(&wv, wrow + T::BLK * blk + 2 + 16 * kh, 16);
+                } else {
+                    // byte i of the block: value i in the low nibble, value 16 + i in the high nibble, both minus 8:
+                    // (n + 0x78) ^ 0x80 is n - 8 as a signed byte, without carries between bytes
+                    uint4 raw;
+                    __builtin_memcpy(&raw, wrow + T::BLK * blk + 2, 16);
+                    const uint32_t rw[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t nib = (kh ? (rw[e] >> 4) : rw[e]) & 0x0f0f0f0fu;
+                        wv[e] = (int)((nib + 0x78787878u) ^ 0x80808080u);
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const i8_intx4 av = *(const i8_intx4 *)(stage + a_base + a * (32 * QK_K) +
+                                                           16 * ((2 * blk + kh) ^ (j & 15)));
+                    const i8_intx16 dq = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, wv, zero, 0, 0, 0);
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const float4 d4 = *(const float4 *)(stage + d_off + 256 * blk + 4 * (32 * a + 8 * q4));
+                        const float da[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int r = 4 * q4 + e;
+                            total[a][r] = __builtin_fmaf((float)dq[r], dw * da[e], total[a][r]);
+                        }
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's share of the next round has landed
+        i8_lds_barrier();
+    }
+    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+}
+
 // ------------------------------------------------------------------ host side
 // From this many activation rows on (more than one 32-row pass of the streaming small-batch kernel) the tile kernel
 // is the faster one on every shape measured (4096 x 4096, 14336 x 4096, 4096 x 14336; e.g. 4096 x 14336 at 48 rows
@@ -1091,6 +1269,73 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
         }
     }
     set_route(q6 ? "mmq_q6_k_q8_k_mfma_tile" : q5 ? "mmq_q5_k_q8_k_mfma_tile" : "mmq_q4_k_q8_k_mfma_tile");
+    return MARMOT_HIP_SUCCESS;
+}
+
+// Q8_0 / Q4_0 weights on Q8_0 activations: rows of whole rounds (K % 256 == 0), 33 activation rows and more
+bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
+                      const ActScratch &act) {
+    if (dev->knobs.no_gemm_i8 || N < I8_MIN_ROWS || K % QK_K != 0 ||
+        (kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_0)) {
+        return false;
+    }
+    const size_t chunk = kind == MARMOT_HIP_KIND_Q8_0 ? 272 : 144;
+    if ((((uintptr_t)act.qs) & 15) != 0 || act.kp % 16 != 0 || N * act.kp >= ((size_t)1 << 32) ||
+        N * (K / 32) * 4 >= ((size_t)1 << 32) || I8_WROWS * (K / QK_K) * chunk >= ((size_t)1 << 32)) {
+        return false;  // 16-byte direct-to-LDS loads with 32-bit lane offsets
+    }
+    for (int i = 0; i < count; ++i) {
+        if ((((uintptr_t)weights[i]) & 15) != 0) {
+            return false;
+        }
+    }
+    return true;
+}
+
+int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
+                    size_t M, int out_dtype, void *scratch) {
+    const bool q8 = kind == MARMOT_HIP_KIND_Q8_0;
+    const size_t nb = K / QK_K;
+    size_t bps = 0;
+    const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
+    float *partial = (float *)scratch;
+    if (splits > 1 && partial == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "tiled Q8_0 GEMM: no room for the K-split partial sums");
+    }
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<MARMOT_HIP_KIND_Q8_0>));
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<MARMOT_HIP_KIND_Q4_0>));
+    const dim3 grid((unsigned)((M + I8_WROWS - 1) / I8_WROWS), (unsigned)((N + I8_TOK - 1) / I8_TOK), (unsigned)splits);
+    for (int which = 0; which < ws.count; ++which) {
+        GemmI8Params p;
+        p.w = (const uint8_t *)ws.w[which];
+        p.qs = act.qs;
+        p.ad = act.d;
+        p.kp = act.kp;
+        p.N = N;
+        p.M = M;
+        p.nb = nb;
+        float *part = splits > 1 ? partial + (size_t)which * splits * N * M : nullptr;
+        p.out = splits > 1 ? (void *)part : ws.out[which];
+        p.splits = (int)splits;
+        p.blocks_per_split = (int)bps;
+        p.bias = ws.bias[which];
+        p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
+        p.bias_first = ws.bias_first ? 1 : 0;
+        p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+        if (q8) {
+            hipLaunchKernelGGL((k_gemm_q80_tile<MARMOT_HIP_KIND_Q8_0>), grid, dim3(I8_THREADS),
+                               Q80Tile<MARMOT_HIP_KIND_Q8_0>::LDS_BYTES, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL((k_gemm_q80_tile<MARMOT_HIP_KIND_Q4_0>), grid, dim3(I8_THREADS),
+                               Q80Tile<MARMOT_HIP_KIND_Q4_0>::LDS_BYTES, dev->stream, p);
+        }
+        MH_HIP(hipGetLastError());
+        if (splits > 1) {
+            MH_TRY(launch_splitk_reduce(dev, part, (int)splits, N, M, ws.bias[which], ws.bias_dtype, ws.out[which],
+                                        out_dtype, ws.bias_first));
+        }
+    }
+    set_route(q8 ? "gemm_q8_0_q8_0_mfma_tile" : "gemm_q4_0_q8_0_mfma_tile");
     return MARMOT_HIP_SUCCESS;
 }
 

@@ -266,7 +266,10 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
-    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr ? 2 : 1) : 0);
+    // Q8_0 / Q4_0 weights from 33 rows on: the tiled int8 GEMM (its K-split partial sums behind the activations)
+    const bool q80_kind = (kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0) && N >= 33 && K % QK_K == 0;
+    const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr ? 2 : 1) : 0) +
+                        (q80_kind ? gemm_i8_scratch_bytes(dev, N, K, M, d_w1 != nullptr ? 2 : 1) : 0);
     void *ws = nullptr;
     int st = workspace_reserve(dev, need, &ws);
     if (st != MARMOT_HIP_SUCCESS) {
@@ -277,6 +280,9 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     st = launch_quantize_act_soa(dev, act_kind, d_input, in_dtype, N, K, act);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
+    }
+    if (q80_kind && gemm_q80_applies(dev, kind, N, K, rows_ws.w, rows_ws.count, act)) {
+        return launch_gemm_q80(dev, kind, rows_ws, act, N, K, M, out_dtype, (uint8_t *)ws + act_bytes);
     }
     if (rows_kernel) {
         st = launch_mmq_rows_q4k(dev, rows_ws, nullptr, &act, N, K, M, out_dtype);
@@ -513,6 +519,22 @@ int marmot_hip_matmul_prepacked(marmot_hip_device_t *dev, int kind, const void *
         }
         return launch_mmq(dev, kind, d_weight, nullptr, act, N, K, M, d_bias, bias_dtype, d_out, nullptr, out_dtype,
                           nullptr);
+    }
+    {
+        WeightSet ws;
+        ws.w[0] = d_weight;
+        ws.out[0] = d_out;
+        ws.bias[0] = d_bias;
+        ws.bias_dtype = bias_dtype;
+        if (gemm_q80_applies(dev, kind, N, K, ws.w, 1, act)) {
+            MH_HIP(hipSetDevice(dev->device_index));
+            const size_t partial_bytes = gemm_i8_scratch_bytes(dev, N, K, M, 1);
+            void *scratch = nullptr;
+            if (partial_bytes != 0) {
+                MH_TRY(workspace_reserve(dev, partial_bytes, &scratch));
+            }
+            return launch_gemm_q80(dev, kind, ws, act, N, K, M, out_dtype, scratch);
+        }
     }
     return launch_matvec_packed(dev, kind, d_weight, nullptr, &act, nullptr, N, K, M, d_bias, bias_dtype, d_out,
                                 nullptr, out_dtype);

@@ -417,3 +417,119 @@ def test_tiled_int8_gemm_q6k_random_blocks_and_exact_integers(hip, oracle):
     for b_ in (d_w, d_p, d_out):
         b_.free()
     assert np.array_equal(bits(got), bits(want))
+
+
+# ---------------------------------------------------------------- tiled int8 GEMM for the 32-value formats (Q8_0, Q4_0)
+Q80_KINDS = {"q8_0": 5, "q4_0": 1}
+
+
+@pytest.mark.parametrize("N,M,K", [(33, 96, 512), (40, 4096, 1024), (48, 128, 256), (64, 100, 512), (100, 203, 2048),
+                                   (130, 300, 1024), (64, 128, 4096), (192, 64, 7168), (512, 512, 4096)])
+@pytest.mark.parametrize("name", ["q8_0", "q4_0"])
+def test_tiled_int8_gemm_32_value_formats_match_oracle(hip, oracle, name, N, M, K):
+    """Prefill with fp32 activations for Q8_0 / Q4_0 weights (activations packed to Q8_0): one int8 matrix instruction
+    per 32-value block and 32 x 32 outputs, the two block scales applied per output and block as in
+    cpu_vec_dot_q8_0_q8_0 (vec_dot_impl.h:452-479). Full and ragged tiles, one to 28 rounds of 256 values, K split
+    across workgroups when the tiles do not fill the chip, bias."""
+    kind = Q80_KINDS[name]
+    blocks = oracle.quantize(kind, gaussian(430 + N, (M, K), 0.02))
+    x = gaussian(431 + N, (N, K))
+    bias = gaussian(432, (M,))
+    got = hip.linear(x, blocks, kind, M, bias=bias)
+    assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"{name} tile {M}x{K} N={N}")
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_0"])
+def test_tiled_int8_gemm_32_value_formats_random_blocks_routes_and_epilogues(hip, oracle, monkeypatch, name):
+    """Arbitrary block bytes (every code, scales of both signs down to fp16 denormals) against the oracle and against
+    the packed matvec that a device object created with MARMOT_HIP_NO_GEMM_I8 keeps; shapes the tile does not cover
+    (K not a multiple of 256, fewer than 33 rows) stay on the matvec; fp16 output with an fp16 bias; the dual call
+    equals two single calls bit for bit."""
+    from marmot_amd import HipBackend
+
+    kind = Q80_KINDS[name]
+    N, M, K = 96, 160, 1536
+    blocks = random_valid_blocks(np.random.default_rng(440), kind, M, K)
+    x = gaussian(441, (N, K))
+    ref = oracle.matmul(kind, blocks, x, M)
+    tiled = hip.linear(x, blocks, kind, M)
+    assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
+    assert_matmul_parity(tiled, ref, what="tile, random blocks")
+    monkeypatch.setenv("MARMOT_HIP_NO_GEMM_I8", "1")
+    plain = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_GEMM_I8")
+    try:
+        got = plain.linear(x, blocks, kind, M)
+        assert plain.last_route() == f"matvec_{name}_q8_0"
+        assert_matmul_parity(got, ref, what="matvec, random blocks")
+        assert_matmul_parity(tiled, got, what="tile against matvec")
+    finally:
+        plain.close()
+    for n2, k2 in ((32, 1536), (96, 1536 + 32)):
+        b2 = oracle.quantize(kind, gaussian(442, (M, k2), 0.02))
+        x2 = gaussian(443, (n2, k2))
+        got = hip.linear(x2, b2, kind, M)
+        assert hip.last_route() == f"matvec_{name}_q8_0", (n2, k2, hip.last_route())
+        assert_matmul_parity(got, oracle.matmul(kind, b2, x2, M), what=f"{name} N={n2} K={k2}")
+    soft = oracle.quantize(kind, gaussian(444, (M, K), 0.02))
+    bias16 = gaussian(445, (M,)).astype(np.float16)
+    x16 = x.astype(np.float16)  # fp16 activations forced through the packed path, fp16 output
+    got16 = hip.linear(x16, soft, kind, M, bias=bias16, out_dtype=np.float16, force_pack=True)
+    assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
+    ref16 = oracle.matmul(kind, soft, x16, M, bias=bias16, out_dtype=np.float16, force_pack=True)
+    assert np.max(np.abs(got16.astype(np.float32) - ref16.astype(np.float32))) <= 2e-3 * np.max(np.abs(ref16.astype(np.float32)))
+    other = oracle.quantize(kind, gaussian(446, (M, K), 0.02))
+    a, b = hip.linear_dual(x, soft, other, kind, M)
+    assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
+    assert np.array_equal(bits(a), bits(hip.linear(x, soft, kind, M)))
+    assert np.array_equal(bits(b), bits(hip.linear(x, other, kind, M)))
+
+
+@pytest.mark.parametrize("name", ["q8_0", "q4_0"])
+def test_tiled_int8_gemm_32_value_formats_integers_are_exact(hip, name):
+    """Packed activations and weight blocks whose scales are powers of two: the integer dot, its conversion and the
+    product of the two scales are then exact, and what is left is one rounding per block in the multiply-add that
+    accumulates it. The output must equal, bit for bit, that chain formed from exact integer dots: blocks 0..3 and
+    4..7 of the one round of 256 values are accumulated separately, each in block order, and the two sums are added."""
+    kind = Q80_KINDS[name]
+    q8 = name == "q8_0"
+    bb = 34 if q8 else 18
+    N, M, K = 70, 200, 256
+    nb = K // 32
+    rng = np.random.default_rng(450)
+    blocks = random_valid_blocks(rng, kind, M, K).reshape(M, nb, bb).copy()
+    d_exp = rng.integers(-12, -6, size=(M, nb))
+    blocks[:, :, 0:2] = np.ldexp(1.0, d_exp).astype(np.float16).view(np.uint8).reshape(M, nb, 2)
+    q = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+    a_exp = rng.integers(-8, -2, size=(N, nb))
+    lay = hip.packed_activation_layout(kind, N, K)
+    image = np.zeros(lay.total_bytes, np.uint8)
+    vals = np.zeros((N, lay.values_per_row), np.int8)
+    vals[:, :K] = q
+    image[lay.values_offset:lay.values_offset + vals.size] = vals.view(np.uint8).reshape(-1)
+    ad = np.ldexp(1.0, a_exp).astype(np.float32)
+    image[lay.scales_offset:lay.scales_offset + ad.nbytes] = ad.view(np.uint8).reshape(-1)
+    if q8:
+        wq = blocks[:, :, 2:].view(np.int8).astype(np.int64)                       # [M, nb, 32]
+    else:  # byte i: value i in the low nibble, value 16 + i in the high nibble, both minus 8
+        qs = blocks[:, :, 2:].astype(np.int64)
+        wq = np.concatenate([(qs & 15) - 8, (qs >> 4) - 8], axis=2)
+    a = q.reshape(N, nb, 32).astype(np.int64)
+    dots = np.einsum("nbk,mbk->nmb", a, wq)                                        # [N, M, nb]
+    scale = np.ldexp(1.0, a_exp[:, None, :] + d_exp[None, :, :])
+    terms = dots * scale                                                           # exact in float64
+    halves = []
+    for first in (0, 4):
+        acc = np.zeros((N, M), np.float32)
+        for b in range(first, first + 4):  # fp32 fused multiply-add: one rounding of the exact sum
+            acc = (acc.astype(np.float64) + terms[:, :, b]).astype(np.float32)
+        halves.append(acc)
+    want = halves[0] + halves[1]
+    d_w, d_p, d_out = hip.to_device(blocks.reshape(M, nb * bb)), hip.to_device(image), hip.alloc(N * M * 4)
+    hip.linear_prepacked_d(kind, d_w, d_p, N, K, M, d_out)
+    assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
+    got = d_out.download(np.float32, (N, M))
+    for b_ in (d_w, d_p, d_out):
+        b_.free()
+    assert np.array_equal(bits(got), bits(want))

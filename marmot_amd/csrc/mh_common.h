@@ -438,7 +438,7 @@ bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K,
 size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, int weights);
 int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                    size_t M, int out_dtype, void *scratch);
-// Tiled int8 GEMM on Q8_0 activations (mh_gemm_i8.hip): Q8_0 and Q4_0 weights, K a multiple of 256, 33 rows and more;
+// Tiled int8 GEMM on Q8_0 activations (mh_gemm_i8.hip): Q8_0 and Q4_0 weights, K a multiple of 256, nine rows and more;
 // `scratch` holds gemm_i8_scratch_bytes for the K-split partial sums
 bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                       const ActScratch &act);

@@ -268,8 +268,8 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
-    // Q8_0 / Q4_0 weights from 33 rows on: the tiled int8 GEMM (its K-split partial sums behind the activations)
-    const bool q80_kind = (kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0) && N >= 33 && K % QK_K == 0;
+    // Q8_0 / Q4_0 weights from nine rows on: the tiled int8 GEMM (its K-split partial sums behind the activations)
+    const bool q80_kind = (kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0) && N >= 9 && K % QK_K == 0;
     const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr ? 2 : 1) : 0) +
                         (q80_kind ? gemm_i8_scratch_bytes(dev, N, K, M, d_w1 != nullptr ? 2 : 1) : 0);
     void *ws = nullptr;

@@ -281,8 +281,8 @@ def prefill_int8(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "ATTN", "LAYER", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32")):
-    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, ATTN, LAYER, LOGITS, Q5K, LEGACY, Q23K, PREFILL32) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "ATTN", "LAYER", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32", "PREFILLFMT")):
+    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, ATTN, LAYER, LOGITS, Q5K, LEGACY, Q23K, PREFILL32, PREFILLFMT) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -346,6 +346,26 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5
                 else:
                     ms = time_steps_graph(hip, step, max(40, steps // 20), 10, chunk=20)
                 emit({"config": "PREFILL32", "workload": f"{names[kind]} {M}x{K} N={N} fp32 activations",
+                      "route": hip.last_route(), "us": round(ms * 1e3, 1),
+                      "TOP/s": round(2.0 * N * M * K / ms / 1e9, 1), "tokens_per_s": round(N / ms * 1e3)})
+                for b in (d_w, d_x, d_out):
+                    b.free()
+    if "PREFILLFMT" in only:
+        # prefill for the other formats the hot path names: Q8_0 / Q4_0 with fp32 activations (Q8_0 integer path, tiled
+        # int8 GEMM) and Q8_0 / Q4_0 / Q6_K with fp16 activations (direct route: decoded weights on the fp16 matrix cores)
+        from marmot_amd import DT_F16
+        for kind, dt in ((capi.KIND_Q8_0, DT_F32), (capi.KIND_Q4_0, DT_F32), (capi.KIND_Q8_0, DT_F16),
+                         (capi.KIND_Q4_0, DT_F16), (capi.KIND_Q6_K, DT_F16)):
+            for N in (16, 128, 512):
+                M = K = 4096
+                d_w = hip.to_device(random_blocks(rng, kind, M, K))
+                x = rng.standard_normal((N, K), dtype=np.float32)
+                d_x = hip.to_device(x if dt == DT_F32 else x.astype(np.float16))
+                d_out = hip.alloc(N * M * 4)
+                step = lambda i: hip.linear_d(kind, d_w, d_x, dt, N, K, M, d_out, DT_F32)
+                ms = time_steps_graph(hip, step, max(40, steps // 20), 10, chunk=20)
+                emit({"config": "PREFILLFMT",
+                      "workload": f"{names[kind]} {M}x{K} N={N} {'fp32' if dt == DT_F32 else 'fp16'} activations",
                       "route": hip.last_route(), "us": round(ms * 1e3, 1),
                       "TOP/s": round(2.0 * N * M * K / ms / 1e9, 1), "tokens_per_s": round(N / ms * 1e3)})
                 for b in (d_w, d_x, d_out):

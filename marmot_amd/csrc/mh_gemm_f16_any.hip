@@ -11,8 +11,8 @@
 //
 // Tiling. A workgroup of four wavefronts owns 128 weight rows x 64 tokens and walks K in rounds of 32 values (one block
 // of the 32-value formats, an eighth of a K-quant block). Per round every thread decodes 16 weights of one row (the
-// same 16-value half of the round for all rows), splits them and stores them into one of two LDS stages in MFMA operand
-// order; wavefront c then multiplies its 32 rows with the 64 tokens: two K-steps x two parts x two token tiles = eight
+// same 16-value half of the round for all rows; for Q8_0, Q4_0 and Q6_K the bytes are requested a round earlier),
+// splits them and stores them into one of two LDS stages in MFMA operand order; wavefront c then multiplies its 32 rows with the 64 tokens: two K-steps x two parts x two token tiles = eight
 // matrix instructions, activations straight from memory (16 bytes per lane, K-step and token tile). One barrier per
 // round. K is split across workgroups when the tiles do not fill the chip; the partial sums meet in k_gemm_reduce.
 #include "mh_common.h"
@@ -43,6 +43,88 @@ struct GemmAnyParams {
     int rounds_per_split;
 };
 
+// The 16 weights a thread decodes per round, in two steps so that the bytes can be requested a round before they are
+// needed: fetch() issues the loads, decode() turns them into the fp32 weights of direct_f16_weight<KIND> (same
+// expressions, same bits). Formats without a form of their own keep the pointer and load inside decode().
+template <int KIND>
+struct AnyRaw {
+    const uint8_t *blk;
+    int v0;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        blk = b;
+        v0 = v;
+    }
+    __device__ __forceinline__ void decode(float (&w)[16]) const {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            w[i] = direct_f16_weight<KIND>(blk, v0 + i);
+        }
+    }
+};
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q8_0> {
+    uint4 q;
+    uint16_t s;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        __builtin_memcpy(&s, b, 2);
+        __builtin_memcpy(&q, b + 2 + v, 16);
+    }
+    __device__ __forceinline__ void decode(float (&w)[16]) const {
+        const float d = h2f(s);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            w[i] = (float)(int8_t)(qw[i >> 2] >> (8 * (i & 3))) * d;  // dequant_value_q8_0
+        }
+    }
+};
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q4_0> {
+    uint4 q;
+    uint16_t s;
+    int high;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        __builtin_memcpy(&s, b, 2);
+        __builtin_memcpy(&q, b + 2, 16);
+        high = v >= 16;
+    }
+    __device__ __forceinline__ void decode(float (&w)[16]) const {
+        const float d = h2f(s);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t byte = (qw[i >> 2] >> (8 * (i & 3))) & 0xffu;
+            const int nib = (int)(high ? byte >> 4 : byte & 0xfu);
+            w[i] = (float)(nib - 8) * d;  // dequant_value_q4_0
+        }
+    }
+};
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q6_K> {
+    uint2 ql;
+    uint32_t qh;
+    int8_t sc;
+    uint16_t d;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {  // v: a multiple of 16
+        __builtin_memcpy(&ql, b + (v >> 1), 8);
+        __builtin_memcpy(&qh, b + 128 + (v >> 2), 4);
+        sc = (int8_t)b[192 + (v >> 7)];
+        __builtin_memcpy(&d, b + 208, 2);
+    }
+    __device__ __forceinline__ void decode(float (&w)[16]) const {  // direct_f16_weight_q6_k for v .. v + 15
+        const float scale = h2f(d) * (float)sc;
+        const uint32_t lw[2] = {ql.x, ql.y};
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t byte = (lw[i >> 3] >> (8 * ((i >> 1) & 3))) & 0xffu;
+            const uint32_t nib = (i & 1) ? byte >> 4 : byte & 0xfu;
+            const uint32_t hi2 = (qh >> (8 * (i >> 2) + 2 * (i & 3))) & 3u;
+            const int qv = (int)(int8_t)(nib | (hi2 << 4)) - 32;
+            w[i] = scale * (float)qv;
+        }
+    }
+};
+
 template <int KIND>
 __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams p) {
     using KT = KindTraits<KIND>;
@@ -70,20 +152,22 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
     auto slot = [](int ks, int part, int c, int half, int row) -> uint32_t {
         return (uint32_t)(((((ks * 2 + part) * 4 + c) * 2 + half) * 32 + row) * 16);
     };
-    auto decode = [&](size_t round, int stage) {
+    auto fetch = [&](size_t round, AnyRaw<KIND> &raw) {
         const size_t k0 = round * FA_ROUND + (size_t)(16 * dks);
         const size_t b = k0 / KT::BV;
-        const int v0 = (int)(k0 - b * KT::BV);
-        const uint8_t *blk = wrow + b * KT::BB;
+        raw.fetch(wrow + b * KT::BB, (int)(k0 - b * KT::BV));
+    };
+    auto decode = [&](const AnyRaw<KIND> &raw, int stage) {
+        float w[16];
+        raw.decode(w);
         uint32_t hi[8], lo[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             uint16_t h[2], l[2];
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                const float w = direct_f16_weight<KIND>(blk, v0 + 2 * i + e);
-                h[e] = f2h(w);
-                l[e] = f2h(w - h2f(h[e]));
+                h[e] = f2h(w[2 * i + e]);
+                l[e] = f2h(w[2 * i + e] - h2f(h[e]));
             }
             hi[i] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
             lo[i] = (uint32_t)l[0] | ((uint32_t)l[1] << 16);
@@ -114,13 +198,9 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
         }
     }
 
-    if (r0 < r1) {
-        decode(r0, 0);
-    }
-    __syncthreads();
-    for (size_t round = r0; round < r1; ++round) {
-        const int stage = (int)((round - r0) & 1);
-        uint4 xa[2][2];  // [K-step][token tile]
+    // rounds in flight: the weights of round + 2 and the activations of round + 1 are requested while round is
+    // multiplied and round + 1 is decoded
+    auto load_x = [&](size_t round, uint4 (&xa)[2][2]) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
@@ -128,8 +208,28 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
                 xa[ks][a] = *(const uint4 *)(xrow[a] + round * FA_ROUND + (size_t)(16 * ks));
             }
         }
+    };
+    AnyRaw<KIND> raw;
+    uint4 xa[2][2];  // [K-step][token tile]
+    if (r0 < r1) {
+        fetch(r0, raw);
+        load_x(r0, xa);
+        decode(raw, 0);
+        if (r0 + 1 < r1) {
+            fetch(r0 + 1, raw);
+        }
+    }
+    __syncthreads();
+    for (size_t round = r0; round < r1; ++round) {
+        const int stage = (int)((round - r0) & 1);
+        AnyRaw<KIND> raw_next = raw;
+        uint4 xa_next[2][2];
+        if (round + 2 < r1) {
+            fetch(round + 2, raw_next);
+        }
         if (round + 1 < r1) {
-            decode(round + 1, stage ^ 1);  // the other stage: the barrier that closed the previous round released it
+            load_x(round + 1, xa_next);
+            decode(raw, stage ^ 1);  // the other stage: the barrier that closed the previous round released it
         }
         const uint8_t *st = lds + (size_t)stage * FA_STAGE;
 #pragma unroll
@@ -141,6 +241,16 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
                 for (int a = 0; a < 2; ++a) {
                     acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(fa_half8, xa[ks][a]), wb, acc[a],
                                                                     0, 0, 0);
+                }
+            }
+        }
+        raw = raw_next;
+        if (round + 1 < r1) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    xa[ks][a] = xa_next[ks][a];
                 }
             }
         }

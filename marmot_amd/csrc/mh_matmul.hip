@@ -723,7 +723,12 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes =
         fuse_quant ? 0 : ((act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255);
-    const size_t mmq_bytes = mmq ? ((mmq_scratch_bytes(dev, kind, N, K, M, 3) + 255) & ~(size_t)255) : 0;
+    // Q8_0 / Q4_0 weights from nine rows on: the tiled int8 GEMM, its K-split partial sums where the mmq scratch would be
+    const bool q80_kind = !fuse_quant && (kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0) && N >= 9 &&
+                          K % QK_K == 0;
+    const size_t mmq_bytes = mmq ? ((mmq_scratch_bytes(dev, kind, N, K, M, 3) + 255) & ~(size_t)255)
+        : q80_kind               ? ((gemm_i8_scratch_bytes(dev, N, K, M, 3) + 255) & ~(size_t)255)
+                                 : 0;
     void *wsp = nullptr;
     int st = MARMOT_HIP_SUCCESS;
     if (act_bytes + mmq_bytes + stage_bytes != 0) {
@@ -755,6 +760,8 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
             // the row-owning kernel took it
         } else if (mmq) {
             st = launch_mmq_set(dev, kind, ws, act, N, K, M, mm_out_dtype, (uint8_t *)wsp + act_bytes);
+        } else if (q80_kind && gemm_q80_applies(dev, kind, N, K, ws.w, ws.count, act)) {
+            st = launch_gemm_q80(dev, kind, ws, act, N, K, M, mm_out_dtype, (uint8_t *)wsp + act_bytes);
         } else {
             st = launch_matvec_set(dev, kind, ws, &act, nullptr, N, K, M, mm_out_dtype);
         }

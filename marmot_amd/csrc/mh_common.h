@@ -456,7 +456,7 @@ int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int split
 bool gemm_f16_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M);
 int launch_gemm_f16(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K, size_t M,
                     const void *d_bias, int bias_dtype, void *d_out, int out_dtype);
-// fp16 activations and every other weight format (mh_gemm_f16_any.hip): 9 rows and more, K a multiple of 32
+// fp16 activations and every other weight format (mh_gemm_f16_any.hip): 9 rows and more, K a multiple of 128
 bool gemm_f16_any_supported(const marmot_hip_device *dev, int kind, size_t N, size_t K, size_t M);
 int launch_gemm_f16_any(marmot_hip_device *dev, int kind, const void *d_w, const void *d_x, size_t N, size_t K,
                         size_t M, const void *d_bias, int bias_dtype, void *d_out, int out_dtype);

@@ -8,13 +8,17 @@
 // numbers, w = hi + lo with |w - hi - lo| <= 2^-22 |w|; hi * x and lo * x are exact in fp32, so the result differs from
 // exact arithmetic by 2^-22 per weight and by the fp32 accumulation, less than the reference's own sequential sum.
 // Weights must be below the fp16 maximum in magnitude (65504; any trained model's are below 100).
+// Q8_0, Q4_0 and Q6_K weights are an integer times a scale that is constant over a round of 32 values (Q6_K, as the
+// reference's fp16 dot decodes it: over 128): for them the INTEGER is the fp16 operand (exact, one part instead of two)
+// and the scale is applied to the round's (four rounds') product in fp32, as d is in the Q4_K kernels.
 //
 // Tiling. A workgroup of four wavefronts owns 128 weight rows x 64 tokens and walks K in rounds of 32 values (one block
 // of the 32-value formats, an eighth of a K-quant block). Per round every thread decodes 16 weights of one row (the
 // same 16-value half of the round for all rows; for Q8_0, Q4_0 and Q6_K the bytes are requested a round earlier),
 // splits them and stores them into one of two LDS stages in MFMA operand order; wavefront c then multiplies its 32 rows with the 64 tokens: two K-steps x two parts x two token tiles = eight
-// matrix instructions, activations straight from memory (16 bytes per lane, K-step and token tile). One barrier per
-// round. K is split across workgroups when the tiles do not fill the chip; the partial sums meet in k_gemm_reduce.
+// matrix instructions; the activations come through LDS in stages of four rounds (whole 256-byte runs of a token's row
+// per 16 lanes: a lane-per-token gather of 16 bytes costs the compute unit's address unit 32 cache lines per
+// instruction and was the bound of the first form, 102 us whatever the format). One barrier per round. K is split across workgroups when the tiles do not fill the chip; the partial sums meet in k_gemm_reduce.
 #include "mh_common.h"
 #include "mh_dequant.h"
 
@@ -27,7 +31,9 @@ constexpr int FA_TOK = 64;
 constexpr int FA_WROWS = 128;
 constexpr int FA_THREADS = 256;
 constexpr int FA_ROUND = 32;                          // values of K per round
-constexpr int FA_STAGE = 2 * 2 * 4 * 2 * 32 * 16;     // K-step x part x wavefront x k half x row x 16 bytes = 16,384
+constexpr int FA_XROUNDS = 4;                         // rounds per activation stage (128 values of K)
+constexpr int FA_XSTAGE = FA_TOK * FA_XROUNDS * FA_ROUND * 2;   // 16,384
+constexpr int FA_OUT_PITCH = FA_WROWS + 4;             // floats per token of the output tile in LDS
 constexpr int FA_MIN_TOKENS = 9;
 
 struct GemmAnyParams {
@@ -41,6 +47,30 @@ struct GemmAnyParams {
     size_t row_bytes;
     int splits;
     int rounds_per_split;
+};
+
+// Four bytes (each below 256 - the fp16 integers 1024 .. 1279 are exact) as two words of fp16 pairs holding byte - OFF
+// + 1024: (0x64, byte) as fp16 bits is 1024 + byte.
+template <int OFF>
+__device__ __forceinline__ void any_bytes_to_f16(uint32_t bytes, uint32_t &lo, uint32_t &hi) {
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    const h2_t off = {(_Float16)(-(float)OFF), (_Float16)(-(float)OFF)};
+    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, bytes, 0x04010400u);
+    const uint32_t b = __builtin_amdgcn_perm(0x64646464u, bytes, 0x04030402u);
+    lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, a) + off);
+    hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, b) + off);
+}
+
+// formats whose weights are an integer times one scale per round (or per four rounds): the integer is the exact fp16
+// operand and the scale goes onto the round's product, like d in the Q4_K kernels
+template <int KIND>
+struct AnyInt {
+    static constexpr bool ON = KIND == MARMOT_HIP_KIND_Q8_0 || KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q6_K;
+    static constexpr int SCALE_ROUNDS = KIND == MARMOT_HIP_KIND_Q6_K ? 4 : 1;  // rounds that share a scale
+    // bytes of one weight stage: K-step x part x wavefront x k half x row x 16 bytes (+ 128 scales)
+    static constexpr int WSTAGE = ON ? 2 * 4 * 2 * 32 * 16 + 512 : 2 * 2 * 4 * 2 * 32 * 16;
+    static constexpr int LDS_BYTES = 2 * WSTAGE + 2 * FA_XSTAGE;
+    static_assert(FA_TOK * FA_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
 };
 
 // The 16 weights a thread decodes per round, in two steps so that the bytes can be requested a round before they are
@@ -77,6 +107,15 @@ struct AnyRaw<MARMOT_HIP_KIND_Q8_0> {
             w[i] = (float)(int8_t)(qw[i >> 2] >> (8 * (i & 3))) * d;  // dequant_value_q8_0
         }
     }
+    // the 16 integers as exact fp16 values (two per word, in order) and the scale they share
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale) const {
+        scale = h2f(s);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            any_bytes_to_f16<1152>(qw[e] ^ 0x80808080u, h[2 * e], h[2 * e + 1]);  // byte + 128, then - 128
+        }
+    }
 };
 template <>
 struct AnyRaw<MARMOT_HIP_KIND_Q4_0> {
@@ -96,6 +135,15 @@ struct AnyRaw<MARMOT_HIP_KIND_Q4_0> {
             const uint32_t byte = (qw[i >> 2] >> (8 * (i & 3))) & 0xffu;
             const int nib = (int)(high ? byte >> 4 : byte & 0xfu);
             w[i] = (float)(nib - 8) * d;  // dequant_value_q4_0
+        }
+    }
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale) const {
+        scale = h2f(s);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t nib = (high ? qw[e] >> 4 : qw[e]) & 0x0f0f0f0fu;
+            any_bytes_to_f16<1032>(nib, h[2 * e], h[2 * e + 1]);  // nibble - 8
         }
     }
 };
@@ -123,12 +171,39 @@ struct AnyRaw<MARMOT_HIP_KIND_Q6_K> {
             w[i] = scale * (float)qv;
         }
     }
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale) const {
+        scale = h2f(d) * (float)sc;
+        // value i: nibble i % 2 of byte i / 2 of ql, bits 2 (i % 4) .. + 1 of byte i / 4 of qh as bits 4..5
+        const uint32_t lw[2] = {ql.x, ql.y};
+        // the high pairs of values 4 b + t, already at bits 4..5, in byte b of plane t
+        const uint32_t pl[4] = {(qh << 4) & 0x30303030u, (qh << 2) & 0x30303030u, qh & 0x30303030u,
+                                (qh >> 2) & 0x30303030u};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {  // values 4 k .. 4 k + 3: bytes 2 (k % 2), 2 (k % 2) + 1 of word k / 2 of ql
+            const uint32_t even = lw[k >> 1] & 0x0f0f0f0fu, odd = (lw[k >> 1] >> 4) & 0x0f0f0f0fu;
+            // [even byte 2 (k % 2), odd same, even next, odd next]; perm selectors 0..3 = second operand, 4..7 = first
+            const uint32_t nibs = __builtin_amdgcn_perm(odd, even, (k & 1) ? 0x07030602u : 0x05010400u);
+            // [plane 0 byte k, plane 1 byte k, plane 2 byte k, plane 3 byte k]
+            const uint32_t sel = 0x04000400u + 0x01010101u * (uint32_t)k;
+            const uint32_t p01 = __builtin_amdgcn_perm(pl[1], pl[0], sel);  // bytes (p0[k], p1[k], p0[k], p1[k])
+            const uint32_t p23 = __builtin_amdgcn_perm(pl[3], pl[2], sel);
+            const uint32_t his = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+            any_bytes_to_f16<1056>(nibs | his, h[2 * k], h[2 * k + 1]);  // 6-bit value - 32
+        }
+    }
 };
 
+// Workgroup barrier that waits for this wavefront's LDS traffic only: __syncthreads() also waits for its outstanding
+// global loads, which here are the weights and activations requested rounds ahead (measured: the kernel ran at the
+// latency of one such request per round, 79 us at 512 tokens whatever the format).
+__device__ __forceinline__ void fa_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int KIND>
-__global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams p) {
+__global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyParams p) {
     using KT = KindTraits<KIND>;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * FA_STAGE];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // 2 weight stages + 2 activation stages (any_lds_bytes)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -149,8 +224,12 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
     wr = wr < p.M ? wr : p.M - 1;  // rows beyond M re-read the last row (never stored)
     const uint8_t *const wrow = p.w + wr * p.row_bytes;
     // LDS slot of (K-step ks, part, wavefront c, k half, row j): 16 bytes
+    constexpr bool INTW = AnyInt<KIND>::ON;
+    constexpr int PARTS = INTW ? 1 : 2;
+    constexpr int SCALE_OFF = 2 * PARTS * 4 * 2 * 32 * 16;  // INTW: 128 floats behind the operands of a stage
+    constexpr int WSTAGE = AnyInt<KIND>::WSTAGE;
     auto slot = [](int ks, int part, int c, int half, int row) -> uint32_t {
-        return (uint32_t)(((((ks * 2 + part) * 4 + c) * 2 + half) * 32 + row) * 16);
+        return (uint32_t)(((((ks * PARTS + part) * 4 + c) * 2 + half) * 32 + row) * 16);
     };
     auto fetch = [&](size_t round, AnyRaw<KIND> &raw) {
         const size_t k0 = round * FA_ROUND + (size_t)(16 * dks);
@@ -158,6 +237,19 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
         raw.fetch(wrow + b * KT::BB, (int)(k0 - b * KT::BV));
     };
     auto decode = [&](const AnyRaw<KIND> &raw, int stage) {
+        if constexpr (INTW) {
+            uint32_t h[8];
+            float scale;
+            raw.ints(h, scale);
+            uint8_t *st = lds + (size_t)stage * WSTAGE;
+            const int c = drow >> 5, row = drow & 31;
+            *(uint4 *)(st + slot(dks, 0, c, 0, row)) = make_uint4(h[0], h[1], h[2], h[3]);
+            *(uint4 *)(st + slot(dks, 0, c, 1, row)) = make_uint4(h[4], h[5], h[6], h[7]);
+            if (dks == 0) {
+                *(float *)(st + SCALE_OFF + 4 * drow) = scale;
+            }
+            return;
+        }
         float w[16];
         raw.decode(w);
         uint32_t hi[8], lo[8];
@@ -172,7 +264,7 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
             hi[i] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
             lo[i] = (uint32_t)l[0] | ((uint32_t)l[1] << 16);
         }
-        uint8_t *st = lds + (size_t)stage * FA_STAGE;
+        uint8_t *st = lds + (size_t)stage * WSTAGE;
         const int c = drow >> 5, row = drow & 31;
         *(uint4 *)(st + slot(dks, 0, c, 0, row)) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
         *(uint4 *)(st + slot(dks, 0, c, 1, row)) = make_uint4(hi[4], hi[5], hi[6], hi[7]);
@@ -180,113 +272,223 @@ __global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams
         *(uint4 *)(st + slot(dks, 1, c, 1, row)) = make_uint4(lo[4], lo[5], lo[6], lo[7]);
     };
 
-    // activations: token tile a, lane (j, kh) -> token 32 a + j (tokens beyond N re-read the last one), 8 values
-    const uint16_t *xrow[2];
+    // Activations go through LDS in stages of four rounds (128 values of K): 64 tokens x 256 bytes, token t's 16-byte
+    // chunk c in slot c ^ (t % 16) (the operand reads of 16 tokens x one chunk then fall into different banks). Every
+    // thread brings four chunks per stage, consecutive lanes consecutive chunks of a token's row (16 lanes per token:
+    // whole 256-byte runs), a stage ahead, and stores them before the barrier that ends the stage in work.
+    uint8_t *const xlds = lds + 2 * WSTAGE;
+    const uint16_t *xsrc[4];
+    uint32_t xdst[4];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
-        size_t t = tok0 + (size_t)(32 * a + j);
-        t = t < p.N ? t : p.N - 1;
-        xrow[a] = p.x + t * p.K + (size_t)(8 * kh);
+    for (int i = 0; i < 4; ++i) {
+        const int piece = i * FA_THREADS + tid;
+        const int t = piece >> 4, c = piece & 15;
+        size_t tok = tok0 + (size_t)t;
+        tok = tok < p.N ? tok : p.N - 1;  // tokens beyond N re-read the last one (never stored)
+        xsrc[i] = p.x + tok * p.K + (size_t)(8 * c);
+        xdst[i] = (uint32_t)(t * 256 + 16 * (c ^ (t & 15)));
     }
+    auto x_request = [&](size_t round, uint4 (&xg)[4]) {  // round: the first of a stage
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            xg[i] = *(const uint4 *)(xsrc[i] + round * FA_ROUND);
+        }
+    };
+    auto x_store = [&](int xstage, const uint4 (&xg)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *(uint4 *)(xlds + (size_t)xstage * FA_XSTAGE + xdst[i]) = xg[i];
+        }
+    };
 
     fa_floatx16 acc[2];
+    fa_floatx16 grp[2];  // INTW: the products of the rounds that share a scale
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             acc[a][r] = 0.0f;
+            grp[a][r] = 0.0f;
         }
     }
 
-    // rounds in flight: the weights of round + 2 and the activations of round + 1 are requested while round is
-    // multiplied and round + 1 is decoded
-    auto load_x = [&](size_t round, uint4 (&xa)[2][2]) {
+    AnyRaw<KIND> raw[2];
+    auto multiply = [&](size_t round, int stage) {
+        const uint8_t *st = lds + (size_t)stage * WSTAGE;
+        // this round's activations: stage (round / 4) % 2, token 32 a + j, chunk 4 (round % 4) + 2 ks + kh
+        const size_t rel = round - r0;
+        const uint8_t *xs = xlds + (size_t)((rel / FA_XROUNDS) & 1) * FA_XSTAGE;
+        const int q = (int)(rel % FA_XROUNDS);
+        fa_half8 x[2][2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
-                xa[ks][a] = *(const uint4 *)(xrow[a] + round * FA_ROUND + (size_t)(16 * ks));
+                x[ks][a] = __builtin_bit_cast(
+                    fa_half8, *(const uint4 *)(xs + (32 * a + j) * 256 + 16 * ((4 * q + 2 * ks + kh) ^ (j & 15))));
             }
         }
-    };
-    AnyRaw<KIND> raw;
-    uint4 xa[2][2];  // [K-step][token tile]
-    if (r0 < r1) {
-        fetch(r0, raw);
-        load_x(r0, xa);
-        decode(raw, 0);
-        if (r0 + 1 < r1) {
-            fetch(r0 + 1, raw);
-        }
-    }
-    __syncthreads();
-    for (size_t round = r0; round < r1; ++round) {
-        const int stage = (int)((round - r0) & 1);
-        AnyRaw<KIND> raw_next = raw;
-        uint4 xa_next[2][2];
-        if (round + 2 < r1) {
-            fetch(round + 2, raw_next);
-        }
-        if (round + 1 < r1) {
-            load_x(round + 1, xa_next);
-            decode(raw, stage ^ 1);  // the other stage: the barrier that closed the previous round released it
-        }
-        const uint8_t *st = lds + (size_t)stage * FA_STAGE;
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int part = 0; part < 2; ++part) {
-                const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, part, wave, kh, j)));
+        if constexpr (INTW) {
+            constexpr int SR = AnyInt<KIND>::SCALE_ROUNDS;
+            const bool opens = SR == 1 || (round % SR) == 0, closes = SR == 1 || (round % SR) == SR - 1;
+            if (opens) {
 #pragma unroll
                 for (int a = 0; a < 2; ++a) {
-                    acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(fa_half8, xa[ks][a]), wb, acc[a],
-                                                                    0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        grp[a][r] = 0.0f;
+                    }
                 }
             }
-        }
-        raw = raw_next;
-        if (round + 1 < r1) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, 0, wave, kh, j)));
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    grp[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], wb, grp[a], 0, 0, 0);
+                }
+            }
+            if (closes) {
+                const float scale = *(const float *)(st + SCALE_OFF + 4 * (32 * wave + j));
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        float t = __builtin_fmaf(scale, grp[a][r], acc[a][r]);
+                        // keeps the scaling inside its round (an empty statement the optimizer cannot move across the
+                        // barrier): sunk behind the later rounds, every round holds its own 32 product registers
+                        // until the end of the stage, and the four sets spill
+                        asm volatile("" : "+v"(t));
+                        acc[a][r] = t;
+                    }
+                }
+            }
+        } else {
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    xa[ks][a] = xa_next[ks][a];
+                for (int part = 0; part < 2; ++part) {
+                    const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, part, wave, kh, j)));
+#pragma unroll
+                    for (int a = 0; a < 2; ++a) {
+                        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], wb, acc[a], 0, 0, 0);
+                    }
                 }
             }
         }
-        __syncthreads();
+    };
+    // One round: the operands of `round` are in LDS stage `stage`; the weights of round + 1 wait in raw_ready. Requests
+    // round + 2's weights into raw_free (free since the previous round decoded it), decodes round + 1 into the other
+    // stage, multiplies. (Requests three rounds ahead, with four sets of registers, measured the same and spilled.)
+    auto step = [&](size_t round, int stage, AnyRaw<KIND> &raw_free, const AnyRaw<KIND> &raw_ready) {
+        if (round + 2 < r1) {
+            fetch(round + 2, raw_free);
+        }
+        if (round + 1 < r1) {
+            decode(raw_ready, stage ^ 1);  // the other stage: the barrier that closed the previous round released it
+        }
+        multiply(round, stage);
+    };
+    uint4 xg[4];
+    if (r0 < r1) {  // (at least four rounds)
+        fetch(r0, raw[0]);
+        x_request(r0, xg);
+        fetch(r0 + 1, raw[1]);
+        decode(raw[0], 0);
+        x_store(0, xg);
+    }
+    fa_barrier();
+    // r0 and the number of rounds are multiples of four (the launcher sees to it): stages of four rounds, two sets of
+    // weight registers that take turns (nothing in flight is ever copied: a copy would wait for the loads it copies)
+    for (size_t round = r0; round < r1; round += FA_XROUNDS) {
+        const bool more = round + FA_XROUNDS < r1;
+        if (more) {
+            x_request(round + FA_XROUNDS, xg);
+        }
+        step(round, 0, raw[0], raw[1]);
+        fa_barrier();
+        step(round + 1, 1, raw[1], raw[0]);
+        fa_barrier();
+        step(round + 2, 0, raw[0], raw[1]);
+        fa_barrier();
+        step(round + 3, 1, raw[1], raw[0]);
+        if (more) {
+            x_store((int)((((round - r0) / FA_XROUNDS) + 1) & 1), xg);
+        }
+        fa_barrier();
     }
 
-    // lane (j, kh) of wavefront c holds weight row 32 c + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4
-    const size_t m = row0 + (size_t)(32 * wave + j);
-    if (m >= p.M) {
-        return;
-    }
-    const bool partials = p.splits > 1;
-    float bias = 0.0f;
-    const bool has_bias = !partials && p.bias != nullptr;
-    if (has_bias) {
-        bias = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m]) : ((const float *)p.bias)[m];
-    }
+    // Lane (j, kh) of wavefront c holds weight row 32 c + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4: the tile goes
+    // through LDS as [token][weight row] (the stages are free behind the loop's last barrier) and every thread stores 16
+    // bytes per step (stores of one float per lane cost the address unit as much as these and move a quarter).
+    float *tile = (float *)lds;
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const size_t n = tok0 + (size_t)(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3));
-            if (n >= p.N) {
-                continue;
-            }
-            const float v = acc[a][r];
-            if (partials) {
-                ((float *)p.out)[((size_t)split * p.N + n) * p.M + m] = v;
-            } else if (!p.out_is_f16) {
-                ((float *)p.out)[n * p.M + m] = has_bias ? v + bias : v;
-            } else {
-                uint16_t h = f2h(v);  // round to the output type first, then add the bias in it
-                if (has_bias) {
-                    h = f2h(h2f(h) + bias);
+            tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * FA_OUT_PITCH + 32 * wave + j] = acc[a][r];
+        }
+    }
+    fa_barrier();
+    const bool partials = p.splits > 1;
+    const bool has_bias = !partials && p.bias != nullptr;
+    const bool out_f16 = !partials && p.out_is_f16;
+    float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
+    const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    for (int idx = tid; idx < FA_TOK * FA_WROWS / 4; idx += FA_THREADS) {
+        const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
+        const size_t n = tok0 + (size_t)t;
+        const size_t m4 = row0 + 4 * (size_t)q4;
+        if (n >= p.N || m4 >= p.M) {
+            continue;
+        }
+        const float4 v = *(const float4 *)(tile + t * FA_OUT_PITCH + 4 * q4);
+        const float e4[4] = {v.x, v.y, v.z, v.w};
+        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (m4 + e < p.M) {
+                    bias4[e] = p.bias_is_f16 ? h2f(((const uint16_t *)p.bias)[m4 + e]) : ((const float *)p.bias)[m4 + e];
                 }
-                ((uint16_t *)p.out)[n * p.M + m] = h;
+            }
+        }
+        if (!out_f16) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[e] = has_bias ? e4[e] + bias4[e] : e4[e];
+            }
+            float *dst = out32 + n * p.M + m4;
+            if (vec) {  // M % 4 == 0: the four rows exist
+                *(float4 *)dst = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = o[e];
+                    }
+                }
+            }
+        } else {
+            uint16_t h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                h[e] = f2h(e4[e]);  // round to the output type first, then add the bias in it
+                if (has_bias) {
+                    h[e] = f2h(h2f(h[e]) + bias4[e]);
+                }
+            }
+            uint16_t *dst = (uint16_t *)p.out + n * p.M + m4;
+            if (vec) {
+                *(uint2 *)dst = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (m4 + e < p.M) {
+                        dst[e] = h[e];
+                    }
+                }
             }
         }
     }
@@ -296,12 +498,13 @@ bool gemm_f16_any_supported(const marmot_hip_device *dev, int kind, size_t N, si
     if (dev->knobs.no_gemm || kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q8_K) {
         return false;
     }
-    return N >= FA_MIN_TOKENS && K % FA_ROUND == 0 && K % block_values(kind) == 0 && M >= 1;
+    return N >= FA_MIN_TOKENS && K % (FA_XROUNDS * FA_ROUND) == 0 && K % block_values(kind) == 0 && M >= 1;
 }
 
 template <int KIND>
 static int launch_any_kind(marmot_hip_device *dev, GemmAnyParams p, const dim3 grid) {
-    hipLaunchKernelGGL((k_gemm_any_f16<KIND>), grid, dim3(FA_THREADS), 0, dev->stream, p);
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_any_f16<KIND>));
+    hipLaunchKernelGGL((k_gemm_any_f16<KIND>), grid, dim3(FA_THREADS), AnyInt<KIND>::LDS_BYTES, dev->stream, p);
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;
 }
@@ -318,16 +521,22 @@ int launch_gemm_f16_any(marmot_hip_device *dev, int kind, const void *d_w, const
     const size_t tiles_n = (N + FA_TOK - 1) / FA_TOK, tiles_m = (M + FA_WROWS - 1) / FA_WROWS;
     const size_t tiles = tiles_n * tiles_m;
     const size_t cus = (size_t)dev->props.multiProcessorCount;
-    // two workgroups per compute unit overlap each other's barriers; fewer tiles than that: split K (at least 16 rounds
-    // per workgroup)
+    // A workgroup's round is a chain of dependent steps (decode, LDS, barrier, LDS, matrix instructions) with one
+    // wavefront per SIMD: three workgroups per compute unit overlap each other's chains (measured at 512 tokens x 4096
+    // rows, Q8_0: one workgroup per compute unit without a K split 134 us, two 93, three 84, four 96). Fewer tiles than
+    // that: split K (at least 16 rounds per workgroup).
     size_t splits = 1;
-    if (tiles < 2 * cus) {
-        splits = (2 * cus) / tiles;
+    const size_t want = 3;
+    if (tiles < want * cus) {
+        splits = (want * cus) / tiles;
         const size_t max_splits = rounds / 16 > 0 ? rounds / 16 : 1;
         splits = splits > max_splits ? max_splits : splits;
         splits = splits > 16 ? 16 : splits;
     }
-    const size_t rps = (rounds + splits - 1) / splits;
+    size_t rps = (rounds + splits - 1) / splits;
+    // whole activation stages per workgroup; whole K-quant blocks (the rounds that share a scale stay together)
+    const size_t grain = block_values(kind) == QK_K ? 8 : FA_XROUNDS;
+    rps = (rps + grain - 1) / grain * grain;
     splits = (rounds + rps - 1) / rps;
     float *partial = nullptr;
     if (splits > 1) {

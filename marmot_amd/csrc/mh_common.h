@@ -431,8 +431,7 @@ size_t mmq_scratch_bytes(const marmot_hip_device *dev, int kind, size_t N, size_
 int launch_mmq(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, const ActScratch &act, size_t N,
                size_t K, size_t M, const void *d_bias, int bias_dtype, void *d_out0, void *d_out1, int out_dtype,
                void *scratch);
-// Tiled int8 GEMM on Q8_K activations (mh_gemm_i8.hip): Q4_K and Q5_K weights, and Q6_K weights whose rows are a
-// multiple of 8 blocks; 33 activation rows and more
+// Tiled int8 GEMM on Q8_K activations (mh_gemm_i8.hip): Q4_K, Q5_K and Q6_K weights; 33 activation rows and more
 bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                      const ActScratch &act);
 size_t gemm_i8_scratch_bytes(const marmot_hip_device *dev, size_t N, size_t K, size_t M, int weights);

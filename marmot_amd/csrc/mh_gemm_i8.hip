@@ -774,9 +774,10 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q5k_q8k_tile(const GemmI8Pa
 // CPU's use of the stored sums). Same tile and wavefront roles as the Q4_K kernel, except that the two K groups share
 // every block: K group kg takes the block's half kg (128 values = groups 8 kg .. 8 kg + 7, which have their own
 // 64 + 32 bytes of low and high bits), so a round is one block and both groups apply the per-block scales to their
-// partial sums. Blocks are 210 bytes: rows must be a multiple of 8 blocks (16-byte aligned rows); the stage holds for
-// each of the 128 rows the 14 chunks of 16 bytes from the one that contains the block start, at a stride of 240 bytes
-// (the 15th chunk slot is not loaded), and the block is read at offset (210 b) % 16 inside the row slot.
+// partial sums. Blocks are 210 bytes, so a block (and, unless a row is a multiple of 8 blocks, a row) starts at any even
+// address: the stage holds for each of the 128 rows the 14 chunks of 16 bytes from the one that contains the block start,
+// at a stride of 240 bytes (the 15th chunk slot is not loaded), and a lane reads its row's block at that row's own offset
+// (row start + 210 b) % 16 inside the row slot.
 constexpr int I6_ROWB = 240;
 constexpr int I6_STAGE_W = I8_WROWS * I6_ROWB;                     // 30,720
 constexpr int I6_STAGE = I6_STAGE_W + I8_STAGE_A + I8_STAGE_D;     // 47,360
@@ -827,17 +828,22 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
     }
     const size_t row_bytes = p.nb * Q6_K_BYTES;
     const uint32_t last_wrow = (uint32_t)(p.M - 1 - row0);
-    uint32_t w_voff[4];
+    // Rows need not start on a 16-byte boundary (210-byte blocks: they do only when a row is a multiple of 8 blocks):
+    // every row's 14 chunks start at ITS OWN boundary below the block start, w_row[m] + 210 b rounded down; the tile's
+    // first row is addressed from the 16-byte boundary below it (`lead` bytes before it).
+    const uint32_t lead = (uint32_t)((row0 * row_bytes) & 15);
+    uint32_t w_row[4], w_pc[4];
     bool w_on[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
         const uint32_t q = (uint32_t)(64 * (wave + 8 * m) + lane);  // chunk slot: row q / 15, chunk q % 15
         const uint32_t r = q / 15u, pc = q - 15u * r;
         const uint32_t rr = r < last_wrow ? r : last_wrow;  // rows beyond M re-read row M - 1 (never stored)
-        w_voff[m] = rr * (uint32_t)row_bytes + 16u * pc;
+        w_row[m] = lead + rr * (uint32_t)row_bytes;
+        w_pc[m] = 16u * pc;
         w_on[m] = wave + 8 * m < 30 && r < (uint32_t)I8_WROWS && pc < 14u;
     }
-    const uint8_t *wbase = p.w + row0 * row_bytes;
+    const uint8_t *wbase = p.w + ((row0 * row_bytes) & ~(size_t)15);
     uint32_t d_voff;
     {
         const uint32_t t = (uint32_t)lane;
@@ -854,13 +860,13 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
             dma_set_lds_base(s0 + (uint32_t)(I6_STAGE_W + 2048 * wave + 1024 * c));
             dma16_to_lds<0>(qb, a_voff[c]);
         }
-        const uint8_t *wb = wbase + ((b * Q6_K_BYTES) & ~(size_t)15);  // the chunk that contains the block start
+        const uint32_t boff = (uint32_t)(b * Q6_K_BYTES);
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
             if (wave + 8 * m < 30) {  // uniform over the wavefront
                 dma_set_lds_base(s0 + (uint32_t)(1024 * (wave + 8 * m)));
                 if (w_on[m]) {
-                    dma16_to_lds<0>(wb, w_voff[m]);
+                    dma16_to_lds<0>(wbase, ((w_row[m] + boff) & ~15u) + w_pc[m]);  // from the chunk that holds the block start
                 }
             }
         }
@@ -872,6 +878,11 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
 
     // ---- compute: weight row 32 rg + j, half kg of the block, all 64 tokens
     const uint32_t w_off = (uint32_t)((32 * rg + j) * I6_ROWB);
+    uint32_t w_own;  // byte offset of this lane's weight row from wbase (the clamped row, like the loads)
+    {
+        const uint32_t r = (uint32_t)(32 * rg + j);
+        w_own = lead + (r < last_wrow ? r : last_wrow) * (uint32_t)row_bytes;
+    }
     const uint32_t a_base = (uint32_t)(I6_STAGE_W + j * QK_K + 8 * kh);
     const uint32_t d_off = (uint32_t)(I6_STAGE_W + I8_STAGE_A + 16 * kh);
 
@@ -884,7 +895,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
         }
         {
             const uint8_t *stage = lds + (size_t)(blk & 1) * I6_STAGE;
-            const int o = (int)(((b0 + (size_t)blk) * Q6_K_BYTES) & 15);
+            const uint32_t o = (w_own + (uint32_t)((b0 + (size_t)blk) * Q6_K_BYTES)) & 15u;  // this lane's row
             const uint8_t *wrow = stage + w_off + o;
             uint2 scv;  // the eight scale bytes of this half
             __builtin_memcpy(&scv, wrow + 192 + 8 * kg, 8);
@@ -1197,10 +1208,7 @@ bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K,
     if (kind == MARMOT_HIP_KIND_Q5_K) {
         block_bytes = Q5_K_BYTES;
     } else if (kind == MARMOT_HIP_KIND_Q6_K) {
-        if ((K / QK_K) % 8 != 0) {
-            return false;  // rows of 210-byte blocks are 16-byte aligned only then
-        }
-        block_bytes = Q6_K_BYTES;
+        block_bytes = Q6_K_BYTES;  // (rows of 210-byte blocks need not be 16-byte aligned: the kernel rounds down per row)
     } else if (kind != MARMOT_HIP_KIND_Q4_K) {
         return false;
     }

@@ -342,12 +342,14 @@ def test_tiled_int8_gemm_q6k_matches_oracle(hip, oracle, N, M, K):
     assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
     assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"Q6_K tile {M}x{K} N={N}")
     if K == 2048:
-        K2 = 1024 + 256  # five blocks per row: rows are not 16-byte aligned
-        b2 = oracle.quantize(kind, gaussian(433, (M, K2), 0.02))
-        x2 = gaussian(434, (N, K2))
-        got2 = hip.linear(x2, b2, kind, M)
-        assert hip.last_route() == "mmq_q6_k_q8_k_mfma"
-        assert_matmul_parity(got2, oracle.matmul(kind, b2, x2, M), what="Q6_K passes, unaligned rows")
+        # rows that are not a multiple of 8 blocks start at any even address (rows of 5, 14 and 43 blocks: the last two
+        # are the hidden size of Qwen2-7B and the FFN size of Llama-2-7B): the tile rounds down per row
+        for K2 in (1024 + 256, 3584, 11008):
+            b2 = oracle.quantize(kind, gaussian(433, (M, K2), 0.02))
+            x2 = gaussian(434, (N, K2))
+            got2 = hip.linear(x2, b2, kind, M)
+            assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
+            assert_matmul_parity(got2, oracle.matmul(kind, b2, x2, M), what=f"Q6_K tile, unaligned rows K={K2}")
 
 
 def test_tiled_int8_gemm_q6k_random_blocks_and_exact_integers(hip, oracle):
@@ -356,14 +358,16 @@ def test_tiled_int8_gemm_q6k_random_blocks_and_exact_integers(hip, oracle):
     arithmetic per half block and added the way the kernel adds (each half of a workgroup's blocks in block order, the
     two halves, then the workgroups along K)."""
     kind = KIND_Q6_K
-    N, M, K = 70, 200, 2048
-    nb = K // 256
     rng = np.random.default_rng(440)
+    for N, M, K in ((70, 200, 2048), (70, 200, 1792), (100, 131, 3328)):  # rows of 8, 7 and 13 blocks
+        blocks = random_valid_blocks(rng, kind, M, K)
+        x = gaussian(441, (N, K))
+        got = hip.linear(x, blocks, kind, M)
+        assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
+        assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what=f"Q6_K tile, random blocks K={K}")
+    N, M, K = 70, 200, 1792  # the exact-integer part on rows of 7 blocks: every row starts at another offset mod 16
+    nb = K // 256
     blocks = random_valid_blocks(rng, kind, M, K)
-    x = gaussian(441, (N, K))
-    got = hip.linear(x, blocks, kind, M)
-    assert hip.last_route() == "mmq_q6_k_q8_k_mfma_tile"
-    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what="Q6_K tile, random blocks")
 
     blocks = blocks.reshape(M, nb, 210).copy()
     d_exp = rng.integers(-14, -8, size=(M, nb))

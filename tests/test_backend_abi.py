@@ -436,7 +436,8 @@ def test_kernel_def_files_name_exported_impls(lib):
     assert set(families) == {"matmul_quantized_hip", "topk_hip",
                              "moe_experts_quantized_hip", "quantize_block_hip", "dequantize_block_hip",
                              "embedding_quantized_hip", "rms_norm_hip", "rms_norm_gemma_hip", "glu_hip",
-                             "add_hip", "rope_hip", "paged_attention_hip"} | qkv
+                             "add_hip", "rope_hip", "paged_attention_hip", "unary_hip", "softmax_hip",
+                             "tensor_ops_hip", "convert_hip"} | qkv
     for name in qkv:
         f = families[name]
         assert f["INPUT_DTYPE"] == f["OUTPUT_DTYPE"] and f["EPILOGUE"] == "[BIAS, ROPE]" and f["OP"] in name

@@ -189,6 +189,65 @@ __global__ __launch_bounds__(256) void k_quantize_q8_0(const void *__restrict__ 
     q8_0_block_store<AOS>(v, col < k, lane32, row, b, nb, blocks_out, soa);
 }
 
+// The same blocks into the structure-of-arrays scratch with eight lanes per block and four consecutive values per lane
+// (one 16-byte load, one dword store) for rows of whole blocks: the maximum and the sum of 32 values do not depend on the
+// order in which they are combined, and every value sees the expressions of q8_0_block_store, so the codes, scales and
+// sums are the same bits. (One value per lane stores single bytes: 10.8 us for 512 x 4096 values against 4 us here.)
+template <int SRC>
+__global__ __launch_bounds__(256) void k_quantize_q8_0_x4(const void *__restrict__ x, const void *__restrict__ x2,
+                                                          size_t rows, size_t k, size_t nb, ActScratch soa) {
+    const int lane8 = threadIdx.x & 7;
+    const size_t blk_id = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 3;
+    if (blk_id >= rows * nb) {
+        return;
+    }
+    const size_t row = blk_id / nb;
+    const size_t b = blk_id - row * nb;
+    const size_t i0 = row * k + b * QK + (size_t)(4 * lane8);
+    float v[4];
+    if constexpr (SRC == SRC_F32) {
+        const float4 f = *(const float4 *)((const float *)x + i0);
+        v[0] = f.x, v[1] = f.y, v[2] = f.z, v[3] = f.w;
+    } else if constexpr (SRC == SRC_F16) {
+        const uint2 h = *(const uint2 *)((const uint16_t *)x + i0);
+        v[0] = h2f((uint16_t)(h.x & 0xffffu)), v[1] = h2f((uint16_t)(h.x >> 16));
+        v[2] = h2f((uint16_t)(h.y & 0xffffu)), v[3] = h2f((uint16_t)(h.y >> 16));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = load_act_value<SRC>(x, x2, i0 + i);
+        }
+    }
+    float max_abs = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) {
+        max_abs = fmaxf(max_abs, __shfl_xor(max_abs, off));
+    }
+    float scale = max_abs / 127.0f;
+    if (scale < FLT_MIN) {
+        scale = 1.0f;
+    }
+    const float inv_scale = 1.0f / scale;
+    int s = 0;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int q = (int)roundf(v[i] * inv_scale);
+        q = q < -127 ? -127 : (q > 127 ? 127 : q);
+        s += q;
+        packed |= ((uint32_t)q & 0xffu) << (8 * i);
+    }
+#pragma unroll
+    for (int off = 1; off < 8; off <<= 1) {
+        s += __shfl_xor(s, off);
+    }
+    *(uint32_t *)(soa.qs + row * soa.kp + b * QK + (size_t)(4 * lane8)) = packed;
+    if (lane8 == 0) {
+        soa.d[row * nb + b] = h2f(f2h(scale));
+        soa.sums[row * nb + b] = (int16_t)s;
+    }
+}
+
 // Plain 16-byte copy: device-to-device copies of the library, and the known-traffic kernel that profiler
 // counters (FETCH_SIZE / WRITE_SIZE) are calibrated against.
 __global__ __launch_bounds__(256) void k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
@@ -255,9 +314,16 @@ static int launch_quantize_src(marmot_hip_device *dev, int act_kind, const void 
     } else {
         const size_t nb = (k + QK - 1) / QK;
         const size_t blocks = rows * nb;
-        const dim3 grid((unsigned)((blocks + 7) / 8));
-        hipLaunchKernelGGL((k_quantize_q8_0<SRC, AOS>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb,
-                           blocks_out, soa);
+        const size_t elem = SRC == SRC_F16 ? 2 : 4;
+        const bool aligned = (((uintptr_t)d_x) % (4 * elem)) == 0 && (d_x2 == nullptr || (((uintptr_t)d_x2) & 15) == 0);
+        if (!AOS && k % QK == 0 && aligned && (((uintptr_t)soa.qs) & 3) == 0 && soa.kp % 4 == 0) {
+            const dim3 grid((unsigned)((blocks + 31) / 32));
+            hipLaunchKernelGGL((k_quantize_q8_0_x4<SRC>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb, soa);
+        } else {
+            const dim3 grid((unsigned)((blocks + 7) / 8));
+            hipLaunchKernelGGL((k_quantize_q8_0<SRC, AOS>), grid, dim3(256), 0, dev->stream, d_x, d_x2, rows, k, nb,
+                               blocks_out, soa);
+        }
     }
     MH_HIP(hipGetLastError());
     return MARMOT_HIP_SUCCESS;

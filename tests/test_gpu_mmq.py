@@ -489,6 +489,23 @@ def test_tiled_int8_gemm_32_value_formats_random_blocks_routes_and_epilogues(hip
     assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
     assert np.array_equal(bits(a), bits(hip.linear(x, soft, kind, M)))
     assert np.array_equal(bits(b), bits(hip.linear(x, other, kind, M)))
+    # activations packed once by the caller, K split across workgroups (one tile: four splits), with a bias: the same
+    # bits as the call that packs for itself
+    from marmot_amd import DT_F32
+    n3, m3, k3 = 40, 128, 2048
+    w3 = oracle.quantize(kind, gaussian(447, (m3, k3), 0.02))
+    x3 = gaussian(448, (n3, k3))
+    b3 = gaussian(449, (m3,))
+    d_w, d_x, d_b = hip.to_device(w3), hip.to_device(x3), hip.to_device(b3)
+    d_p, d_out = hip.alloc(hip.packed_activation_bytes(kind, n3, k3)), hip.alloc(n3 * m3 * 4)
+    hip.pack_activations_d(kind, d_x, DT_F32, n3, k3, d_p)
+    hip.linear_prepacked_d(kind, d_w, d_p, n3, k3, m3, d_out, d_bias=d_b)
+    assert hip.last_route() == f"gemm_{name}_q8_0_mfma_tile"
+    pre = d_out.download(np.float32, (n3, m3))
+    for b_ in (d_w, d_x, d_b, d_p, d_out):
+        b_.free()
+    assert np.array_equal(bits(pre), bits(hip.linear(x3, w3, kind, m3, bias=b3)))
+    assert_matmul_parity(pre, oracle.matmul(kind, w3, x3, m3, bias=b3), what=f"{name} prepacked, K split")
 
 
 @pytest.mark.parametrize("name", ["q8_0", "q4_0"])

@@ -844,6 +844,8 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
         w_on[m] = wave + 8 * m < 30 && r < (uint32_t)I8_WROWS && pc < 14u;
     }
     const uint8_t *wbase = p.w + ((row0 * row_bytes) & ~(size_t)15);
+    const size_t w_end64 = (size_t)lead + (p.M - row0) * row_bytes;  // the tensor's end, from wbase
+    const uint32_t w_end = w_end64 > 0xffffffffull ? 0xffffffffu : (uint32_t)w_end64;
     uint32_t d_voff;
     {
         const uint32_t t = (uint32_t)lane;
@@ -865,8 +867,20 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
         for (int m = 0; m < 4; ++m) {
             if (wave + 8 * m < 30) {  // uniform over the wavefront
                 dma_set_lds_base(s0 + (uint32_t)(1024 * (wave + 8 * m)));
-                if (w_on[m]) {
-                    dma16_to_lds<0>(wbase, ((w_row[m] + boff) & ~15u) + w_pc[m]);  // from the chunk that holds the block start
+                const uint32_t voff = ((w_row[m] + boff) & ~15u) + w_pc[m];  // from the chunk that holds the block start
+                // The last chunk of the tensor's last block ends up to 14 bytes behind the tensor when its size is not
+                // a multiple of 16: those bytes may not exist. Such a chunk (rows beyond M repeat it) is brought two
+                // bytes at a time, only the bytes that exist, by plain loads and LDS stores; the barrier that ends
+                // the round waits for both.
+                const bool past = voff + 16u > w_end;
+                if (w_on[m] && !past) {
+                    dma16_to_lds<0>(wbase, voff);
+                }
+                if (w_on[m] && past) {
+                    const uint32_t slot = (uint32_t)((bi & 1) * I6_STAGE + 1024 * (wave + 8 * m) + 16 * lane);
+                    for (uint32_t e = 0; e < 16u && voff + e < w_end; e += 2u) {
+                        *(uint16_t *)(lds + slot + e) = *(const uint16_t *)(wbase + voff + e);
+                    }
                 }
             }
         }

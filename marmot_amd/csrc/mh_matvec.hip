@@ -944,7 +944,7 @@ __global__ __launch_bounds__((matvec_max_threads<Fmt, NC, C, R, FUSED>())) void 
     }
 }
 
-// ------------------------------------------------------------------ loader / consumer variant (16-byte aligned rows)
+// ------------------------------------------------------------------ loader / consumer variant (rows of an even number of bytes)
 // Same arithmetic, lane mapping and reduction order as k_matvec, but the weights take the way global -> LDS ->
 // registers and the wavefronts are specialised: W consumers quantize the activations, read weight rows from an LDS
 // ring and compute; one loader copies the workgroup's rows (contiguous in memory) into the ring with direct-to-LDS
@@ -986,24 +986,42 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
     float *partial = (float *)lds_raw;
     const int pstride = 4 * W;
     const uint32_t stage_bytes = (uint32_t)(R * p.row_bytes);
-    const uint32_t stage_stride = (stage_bytes + 1023u) & ~1023u;
+    // Rows need not be multiples of 16 bytes: a step is copied from the 16-byte boundary below its first row (`lead`
+    // bytes early, rows of a workgroup are contiguous in memory) and read `lead` bytes into its stage.
+    const uint32_t stage_stride = (stage_bytes + 15u + 1023u) & ~1023u;
     uint8_t *ring = lds_raw + (((size_t)rows * NC * pstride * sizeof(float) + 15) & ~(size_t)15);
 
     if (loader) {
         const int chunks = (int)(stage_stride >> 10);  // direct-to-LDS instructions per step (1 KiB each)
-        const bool ragged = row0 + rows > p.M;         // some step is cut short: its instruction count is unknown
+        // Some step is cut short (rows beyond M), or the tensor ends inside this workgroup off a 16-byte boundary (its
+        // last chunk then comes through registers): the loads in flight are not whole steps of `chunks` instructions.
+        const bool ragged = row0 + rows > p.M || (row0 + rows == p.M && ((p.M * p.row_bytes) & 15) != 0);
+        int step_loads[MV_LS_STAGES];  // direct-to-LDS instructions of the step in each stage
         auto issue_step = [&](int t) {
             const size_t r = row0 + (size_t)t * R;
             uint32_t valid = stage_bytes;  // bytes of this step that exist (rows beyond M are not read)
             if (r + R > p.M) {
                 valid = r < p.M ? (uint32_t)((p.M - r) * p.row_bytes) : 0u;
             }
-            const uint8_t *src = wbase + r * p.row_bytes;
+            const size_t first = r * p.row_bytes;
+            const uint32_t lead = (uint32_t)(first & 15);
+            const uint8_t *src = wbase + (first - lead);
+            valid = valid != 0 ? valid + lead : 0u;
+            // bytes of the tensor from src on: a chunk that would end behind the tensor (its size need not be a multiple
+            // of 16) is brought two bytes at a time, only the bytes that exist
+            const size_t left = p.M * p.row_bytes - (first - lead);
             uint8_t *dst = ring + (size_t)(t % MV_LS_STAGES) * stage_stride;
+            step_loads[t % MV_LS_STAGES] = (int)((valid + 1023u) >> 10);  // chunks that hold a byte of the step
             for (int c = 0; c < chunks; ++c) {
                 const uint32_t off = (uint32_t)c * 1024u + (uint32_t)lane * 16u;
                 if (off < valid) {
-                    __builtin_amdgcn_global_load_lds((glb_u8 *)(src + off), (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+                    if ((size_t)off + 16 <= left) {
+                        __builtin_amdgcn_global_load_lds((glb_u8 *)(src + off), (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+                    } else {
+                        for (uint32_t e = 0; e < 16u && (size_t)off + e < left; e += 2u) {
+                            *(uint16_t *)(dst + off + e) = *(const uint16_t *)(src + off + e);
+                        }
+                    }
                 }
             }
         };
@@ -1022,7 +1040,11 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
             if (newer > load_steps - 1 - b) {
                 newer = load_steps - 1 - b;
             }
-            wait_vmcnt_at_most(ragged ? 0 : newer * chunks);
+            int in_flight = 0;  // instructions of the steps issued after step b
+            for (int k2 = 1; k2 <= newer; ++k2) {
+                in_flight += step_loads[(b + k2) % MV_LS_STAGES];
+            }
+            wait_vmcnt_at_most(ragged ? 0 : in_flight);
             __builtin_amdgcn_s_barrier();  // barrier b: step b may be read; the consumers are done with step b - 1
             if (b >= 1 && b + MV_LS_STAGES - 1 < load_steps) {
                 issue_step(b + MV_LS_STAGES - 1);  // into the stage of step b - 1
@@ -1065,7 +1087,8 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
         for (int b = 0; b < load_steps; ++b) {
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the previous stage has been read before it is reused
             __builtin_amdgcn_s_barrier();        // barrier b
-            const uint8_t *stage = ring + (size_t)(b % MV_LS_STAGES) * stage_stride;
+            const uint8_t *stage = ring + (size_t)(b % MV_LS_STAGES) * stage_stride +
+                                   (((row0 + (size_t)b * R) * p.row_bytes) & 15);  // the step's first row
             typename Fmt::Wt wt[R][C];
 #pragma unroll
             for (int rr = 0; rr < R; ++rr) {
@@ -1123,12 +1146,12 @@ __global__ __launch_bounds__((matvec_ls_max_consumers<Fmt>() + 1) * 64) void k_m
     }
 }
 
-// rows whose bytes can be copied as 16-byte chunks: row pitch and base address multiples of 16, at most 8 K slices
+// rows whose bytes can be copied as 16-byte chunks: base address a multiple of 16, even row pitch, at most 8 K slices
 template <class Fmt>
 static bool matvec_ls_usable(const marmot_hip_device *dev, const MatvecParams &p, size_t K, int C) {
     const size_t nb = (K + Fmt::BV - 1) / Fmt::BV;
     const size_t wave_loads = (nb + Fmt::BPW - 1) / Fmt::BPW;
-    return p.items == nullptr && K % Fmt::BV == 0 && p.row_bytes % 16 == 0 && (((uintptr_t)p.w[0]) & 15) == 0 &&
+    return p.items == nullptr && K % Fmt::BV == 0 && p.row_bytes % 2 == 0 && (((uintptr_t)p.w[0]) & 15) == 0 &&
            (((uintptr_t)p.w[1]) & 15) == 0 && (((uintptr_t)p.w[2]) & 15) == 0 && wave_loads <= (size_t)(matvec_ls_max_consumers<Fmt>() * C) &&
            !dev->knobs.no_lds_ring;
 }
@@ -1137,7 +1160,7 @@ template <class Fmt, int NC, int C, int R, bool FUSED>
 static int launch_ls(marmot_hip_device *dev, MatvecParams p, int W, size_t M, int nw) {
     const dim3 grid((unsigned)((M + p.rows_per_wg - 1) / p.rows_per_wg), nw, 1);
     const size_t part = (((size_t)p.rows_per_wg * NC * 4 * W * sizeof(float)) + 15) & ~(size_t)15;
-    const size_t stage_stride = ((size_t)R * p.row_bytes + 1023) & ~(size_t)1023;
+    const size_t stage_stride = ((size_t)R * p.row_bytes + 15 + 1023) & ~(size_t)1023;
     const size_t lds = part + MV_LS_STAGES * stage_stride;
     MH_TRY(allow_large_lds(dev, (const void *)k_matvec_ls<Fmt, NC, C, R, FUSED>));
     hipLaunchKernelGGL((k_matvec_ls<Fmt, NC, C, R, FUSED>), grid, dim3((W + 1) * 64), lds, dev->stream, p);

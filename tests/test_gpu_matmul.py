@@ -122,6 +122,22 @@ def test_linear_k_sweep(hip, oracle, name, K):
         assert_matmul_parity(got, ref, what=f"{name} K={K} N={N}")
 
 
+@pytest.mark.parametrize("name,K", [("q6_k", 3584), ("q6_k", 256 * 13), ("q8_0", 32 * 113), ("q2_k", 256 * 7),
+                                    ("q3_k", 256 * 5), ("q4_0", 32 * 99)])
+def test_linear_rows_off_16_byte_boundaries(hip, oracle, name, K):
+    """Rows whose byte length is not a multiple of 16 (3584 = the hidden size of Qwen2-7B in Q6_K: 14 blocks of 210
+    bytes) at decode sizes: the loader of the LDS ring copies every step from the 16-byte boundary below its first row,
+    and the tensor's last bytes come two at a time when the tensor does not end on such a boundary. Row counts that end
+    inside a step, on a step and on a workgroup."""
+    kind = KINDS[name]
+    for M in (3584, 1031, 64):
+        blocks = oracle.quantize(kind, gaussian(75, (M, K), 0.02))
+        for N in (1, 2, 4):
+            x = gaussian(76 + N, (N, K))
+            got = hip.linear(x, blocks, kind, M)
+            assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, threads=8), what=f"{name} {M}x{K} N={N}")
+
+
 @pytest.mark.parametrize("name", ["q4_0", "q4_1", "q5_0", "q5_1", "q8_0", "q8_1", "q2_k", "q3_k", "q4_k", "q5_k", "q6_k"])
 def test_linear_ragged_k(hip, oracle, name):
     """K not a multiple of the block: weight and activation tails are zero-padded blocks."""

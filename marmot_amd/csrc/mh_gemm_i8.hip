@@ -1215,7 +1215,10 @@ static size_t gemm_i8_splits(const marmot_hip_device *dev, size_t N, size_t M, s
 
 bool gemm_i8_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                      const ActScratch &act) {
-    if (dev->knobs.no_gemm_i8 || N < I8_MIN_ROWS || K % QK_K != 0) {
+    // Q6_K: the small-batch kernel holds 16 rows per pass, and from the second pass on the tile is faster (14336 x 4096
+    // at 17 .. 32 rows: 48 us in two passes, the tile 41 us at 33 rows; 18944 x 3584: 87 - 94 against 63 us)
+    const size_t min_rows = kind == MARMOT_HIP_KIND_Q6_K ? 17 : I8_MIN_ROWS;
+    if (dev->knobs.no_gemm_i8 || N < min_rows || K % QK_K != 0) {
         return false;
     }
     size_t block_bytes = Q4_K_BYTES;

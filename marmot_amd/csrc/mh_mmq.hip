@@ -668,9 +668,13 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
         tok[r] = 8 * (r >> 2) + 4 * kh + (r & 3);
     }
 
+    const size_t row_bytes = p.nb * Q6_K_BYTES;
+    const uint32_t lead = (uint32_t)((row0 * row_bytes) & 15);
     if (loader) {
-        const size_t row_bytes = p.nb * Q6_K_BYTES;
-        uint32_t w_off[W_LOADS];
+        // Rows need not start on 16-byte boundaries (they do only when a row is a multiple of 8 blocks): every row's 14
+        // chunks start at ITS OWN boundary below the block start; the group's first row is addressed from the boundary
+        // below it (`lead` bytes before it).
+        uint32_t w_row[W_LOADS], w_pc[W_LOADS];
         bool w_on[W_LOADS];
 #pragma unroll
         for (int c = 0; c < W_LOADS; ++c) {
@@ -680,10 +684,16 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
             if (m >= p.M) {
                 m = p.M - 1;  // harmless re-read; never stored
             }
-            w_off[c] = (uint32_t)((m - row0) * row_bytes + 16 * pc);
+            w_row[c] = lead + (uint32_t)((m - row0) * row_bytes);
+            w_pc[c] = (uint32_t)(16 * pc);
             w_on[c] = row < 32 && pc < 14;
         }
-        const uint8_t *wgroup = wbase + row0 * row_bytes;
+        const uint8_t *wgroup = wbase + ((row0 * row_bytes) & ~(size_t)15);
+        // the tensor's end from wgroup: a chunk that would end behind it (the tensor's size need not be a multiple of
+        // 16) comes two bytes at a time through registers, and the loads in flight are then not whole steps
+        const size_t w_end64 = (size_t)lead + (p.M - row0) * row_bytes;
+        const uint32_t w_end = w_end64 > 0xffffffffull ? 0xffffffffu : (uint32_t)w_end64;
+        const bool ragged_end = row0 + 32 >= p.M && (w_end & 15u) != 0;
         uint32_t a_off[A_LOADS];
 #pragma unroll
         for (int c = 0; c < A_LOADS; ++c) {
@@ -708,13 +718,20 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
                     if (b >= p.nb) {
                         b = p.nb - 1;
                     }
-                    const size_t blk_lo = (b * Q6_K_BYTES) & ~(size_t)15;  // chunk that contains the block start
+                    const uint32_t boff = (uint32_t)(b * Q6_K_BYTES);
                     uint8_t *dst = lds + ((size_t)w * STAGES + (t % STAGES)) * STAGE;
 #pragma unroll
                     for (int c = 0; c < W_LOADS; ++c) {
-                        if (w_on[c]) {
-                            __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + w_off[c] + blk_lo),
-                                                             (lds_u8 *)(dst + c * 1024), 16, 0, 0);
+                        const uint32_t voff = ((w_row[c] + boff) & ~15u) + w_pc[c];  // from the chunk with the block start
+                        const bool past = voff + 16u > w_end;
+                        if (w_on[c] && !past) {
+                            __builtin_amdgcn_global_load_lds((glb_u8 *)(wgroup + voff), (lds_u8 *)(dst + c * 1024), 16, 0,
+                                                             0);
+                        }
+                        if (w_on[c] && past) {
+                            for (uint32_t e = 0; e < 16u && voff + e < w_end; e += 2u) {
+                                *(uint16_t *)(dst + c * 1024 + 16 * lane + e) = *(const uint16_t *)(wgroup + voff + e);
+                            }
                         }
                     }
 #pragma unroll
@@ -729,7 +746,8 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
                 }
             }
             const int newer = t < p.bpw ? (AHEAD - 1) : (AHEAD - 1) - (t - p.bpw + 1);
-            wait_vmcnt_at_most(newer > 0 ? newer * W * LOADS : 0);
+            wait_vmcnt_at_most(newer > 0 && !ragged_end ? newer * W * LOADS : 0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // the LDS stores of a tensor-end chunk
             __builtin_amdgcn_s_barrier();
         }
     } else {
@@ -737,11 +755,19 @@ __global__ __launch_bounds__(320) void k_mmq_q6k_ls(const MmqParams p) {
         const size_t b_first = first_block(wave);
         const uint8_t *ring = lds + (size_t)wave * STAGES * STAGE;
         const int ti = j & (TOK - 1);
+        uint32_t w_own;  // byte offset of this lane's weight row from the group's 16-byte boundary (the clamped row)
+        {
+            size_t m = row0 + (size_t)j;
+            if (m >= p.M) {
+                m = p.M - 1;
+            }
+            w_own = lead + (uint32_t)((m - row0) * row_bytes);
+        }
         for (int t = 0; t < steps; ++t) {
             const int blk = t - AHEAD;
             if (blk >= 0 && blk < nblk) {
                 const uint8_t *stage = ring + (blk % STAGES) * STAGE;
-                const int o = (int)(((b_first + blk) * Q6_K_BYTES) & 15);
+                const uint32_t o = (w_own + (uint32_t)((b_first + blk) * Q6_K_BYTES)) & 15u;  // this lane's row
                 const uint8_t *wrow = stage + j * MMQ6_ROWB + o;
                 const uint8_t *a_blk = stage + A_OFF + ti * QK_K + 8 * kh;
                 const float *ad_blk = (const float *)(stage + D_OFF);
@@ -853,9 +879,9 @@ struct MmqPlan {
     int W, S, bpw;
 };
 
-// rows of a multiple of 8 blocks are 16-byte aligned: the loader/consumer kernel applies
+// the loader / consumer kernel takes rows of any number of blocks (it rounds the 16-byte loads down per row)
 static bool mmq6_uses_loader(size_t nb) {
-    return nb % 8 == 0;
+    return nb != 0;
 }
 
 // W (consumer) wavefronts per workgroup and S workgroups split K.

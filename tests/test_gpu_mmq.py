@@ -82,6 +82,22 @@ def test_k_split_over_wavefronts_and_workgroups(hip, oracle, name, M, K):
         assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M), what=f"{name} {M}x{K} N={N}")
 
 
+@pytest.mark.parametrize("K", [1280, 3584, 11008])
+def test_q6k_rows_off_16_byte_boundaries(hip, oracle, K):
+    """Q6_K rows of 5, 14 and 43 blocks (210-byte blocks: such rows start at any even address) through the loader /
+    consumer kernel, which rounds its 16-byte loads down per row; row counts that end inside a group of 32, tensors
+    that do not end on a 16-byte boundary (the last chunk then comes two bytes at a time), K split over wavefronts and
+    workgroups."""
+    kind = KIND_Q6_K
+    for M in (70, 1031, 4096):
+        blocks = oracle.quantize(kind, gaussian(345, (M, K), 0.02))
+        for N in (5, 8, 16):
+            x = gaussian(346 + N, (N, K))
+            got = hip.linear(x, blocks, kind, M)
+            assert hip.last_route() == "mmq_q6_k_q8_k_mfma"
+            assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, threads=8), what=f"Q6_K {M}x{K} N={N}")
+
+
 @pytest.mark.parametrize("name", ["q4_k", "q6_k"])
 @pytest.mark.parametrize("M,K", [(96, 1024), (64, 14336)])
 def test_bias_and_fp16_epilogues(hip, oracle, name, M, K):

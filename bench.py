@@ -351,11 +351,13 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5
                 for b in (d_w, d_x, d_out):
                     b.free()
     if "PREFILLFMT" in only:
-        # prefill for the other formats the hot path names: Q8_0 / Q4_0 with fp32 activations (Q8_0 integer path, tiled
-        # int8 GEMM) and Q8_0 / Q4_0 / Q6_K with fp16 activations (direct route: decoded weights on the fp16 matrix cores)
+        # prefill for the other formats: the 32-value formats and Q2_K / Q3_K with fp32 activations (integer path) and
+        # fp16 activations (direct route: decoded weights on the fp16 matrix cores)
         from marmot_amd import DT_F16
-        for kind, dt in ((capi.KIND_Q8_0, DT_F32), (capi.KIND_Q4_0, DT_F32), (capi.KIND_Q8_0, DT_F16),
-                         (capi.KIND_Q4_0, DT_F16), (capi.KIND_Q6_K, DT_F16)):
+        for kind, dt in ((capi.KIND_Q8_0, DT_F32), (capi.KIND_Q4_0, DT_F32), (capi.KIND_Q4_1, DT_F32),
+                         (capi.KIND_Q5_0, DT_F32), (capi.KIND_Q5_1, DT_F32), (capi.KIND_Q2_K, DT_F32),
+                         (capi.KIND_Q3_K, DT_F32), (capi.KIND_Q8_0, DT_F16), (capi.KIND_Q4_0, DT_F16),
+                         (capi.KIND_Q6_K, DT_F16), (capi.KIND_Q5_K, DT_F16), (capi.KIND_Q4_1, DT_F16)):
             for N in (16, 128, 512):
                 M = K = 4096
                 d_w = hip.to_device(random_blocks(rng, kind, M, K))

@@ -296,6 +296,143 @@ __global__ __launch_bounds__(128) void k_pa_fp8_scan_new(const PaParams p) {
     }
 }
 
+// Maxima of four values over a workgroup of 128 threads (two wavefronts): lanes first, then the two wavefronts
+// through LDS. `red` holds 8 floats and is free again on return.
+__device__ __forceinline__ void pa_block_max4(float (&v)[4], float *red) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = fmaxf(v[i], __shfl_xor(v[i], s));
+        }
+    }
+    if ((threadIdx.x & 63u) == 0u) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            red[(threadIdx.x >> 6) * 4 + i] = v[i];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[i] = fmaxf(red[i], red[4 + i]);
+    }
+    __syncthreads();
+}
+
+// The rows already in one (block, kv head): the first `existing` positions. `vec`: rows of a multiple of 16 codes at
+// 16-byte aligned addresses, taken 16 codes at a time.
+struct PaFp8Rows {
+    uint8_t *kc, *vc;
+    size_t si;
+    uint32_t existing;
+    bool vec;
+};
+
+__device__ __forceinline__ PaFp8Rows pa_fp8_rows(const PaParams &p, uint32_t b, uint32_t h, uint32_t existing) {
+    PaFp8Rows r;
+    const size_t base = (size_t)b * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2];
+    r.kc = (uint8_t *)p.kv_k + base, r.vc = (uint8_t *)p.kv_v + base;
+    r.si = (size_t)b * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] + (size_t)h * p.scale_stride[2];
+    r.existing = existing;
+    r.vec = p.kv_stride[4] == 1 && (p.head_dim & 15u) == 0u && (p.kv_stride[3] & 15u) == 0u &&
+            (((uintptr_t)r.kc | (uintptr_t)r.vc) & 15u) == 0u;
+    return r;
+}
+
+__device__ __forceinline__ uint32_t pa_fp8_big_field(uint32_t big, uint32_t word) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t c = (word >> (8 * e)) & 0x7fu;
+        big = c < 0x78u && c > big ? c : big;
+    }
+    return big;
+}
+
+// This thread's share of the largest finite magnitude fields (low seven bits) among the rows already there: a finite
+// code's magnitude grows with that field, so the largest one is found first and decoded once (NaN codes, field 15
+// of the exponent, never win a maximum).
+__device__ __forceinline__ void pa_fp8_scan_rows(const PaParams &p, const PaFp8Rows &r, uint32_t &kbig, uint32_t &vbig) {
+    kbig = vbig = 0u;
+    if (r.vec) {
+        const uint32_t per_row = p.head_dim >> 4, chunks = r.existing * per_row;
+        for (uint32_t c = threadIdx.x; c < chunks; c += 128u) {
+            const uint32_t pos = c / per_row;
+            const size_t at = (size_t)pos * p.kv_stride[3] + (size_t)(c - pos * per_row) * 16u;
+            const uint4 k = *(const uint4 *)(r.kc + at), v = *(const uint4 *)(r.vc + at);
+            kbig = pa_fp8_big_field(pa_fp8_big_field(pa_fp8_big_field(pa_fp8_big_field(kbig, k.x), k.y), k.z), k.w);
+            vbig = pa_fp8_big_field(pa_fp8_big_field(pa_fp8_big_field(pa_fp8_big_field(vbig, v.x), v.y), v.z), v.w);
+        }
+        return;
+    }
+    const uint32_t cells = r.existing * p.head_dim;
+    for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
+        const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
+        const size_t at = (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
+        const uint32_t kb = r.kc[at] & 0x7fu, vb = r.vc[at] & 0x7fu;
+        kbig = kb < 0x78u && kb > kbig ? kb : kbig;
+        vbig = vb < 0x78u && vb > vbig ? vb : vbig;
+    }
+}
+
+__device__ __forceinline__ uint32_t pa_fp8_recode4(uint32_t word, float old_scale, float new_scale) {
+    uint32_t out = 0u;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        out |= pa_fp8_quant(pa_fp8_dequant((word >> (8 * e)) & 0xffu, old_scale), new_scale) << (8 * e);
+    }
+    return out;
+}
+
+// The new scale of one cache tensor of the block from the largest magnitude field found in it and the largest new
+// magnitude; the rows already there are re-encoded when the scale changes. `old_scale` was read before any thread
+// could have written the new one (a barrier lies between).
+__device__ __forceinline__ float pa_fp8_rescale_rows(const PaParams &p, const PaFp8Rows &r, int which, uint32_t big_field,
+                                                     float new_max, float old_scale) {
+    uint8_t *cache = which ? r.vc : r.kc;
+    const float big = fmaxf(pa_fp8_dequant(big_field, old_scale), new_max);
+    const float new_scale = big > 0.0f ? big / 240.0f : 1.0f;
+    if (r.existing > 0 && new_scale != old_scale) {
+        if (r.vec) {
+            const uint32_t per_row = p.head_dim >> 4, chunks = r.existing * per_row;
+            for (uint32_t c = threadIdx.x; c < chunks; c += 128u) {
+                const uint32_t pos = c / per_row;
+                uint4 *cell = (uint4 *)(cache + (size_t)pos * p.kv_stride[3] + (size_t)(c - pos * per_row) * 16u);
+                uint4 w = *cell;
+                w.x = pa_fp8_recode4(w.x, old_scale, new_scale), w.y = pa_fp8_recode4(w.y, old_scale, new_scale);
+                w.z = pa_fp8_recode4(w.z, old_scale, new_scale), w.w = pa_fp8_recode4(w.w, old_scale, new_scale);
+                *cell = w;
+            }
+        } else {
+            const uint32_t cells = r.existing * p.head_dim;
+            for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
+                const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
+                uint8_t *cell = cache + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
+                *cell = (uint8_t)pa_fp8_quant(pa_fp8_dequant(*cell, old_scale), new_scale);
+            }
+        }
+    }
+    if (threadIdx.x == 0) {
+        (which ? p.v_scale : p.k_scale)[r.si] = new_scale;
+    }
+    return new_scale;
+}
+
+// The work on one (block, kv head): the new scales from the rows already there (the first `existing` positions) and
+// this thread's share of the largest new magnitudes; the rows already there are re-encoded where a scale changes.
+// Whole workgroup of 128.
+__device__ __forceinline__ void pa_fp8_rescale_block(const PaParams &p, uint32_t b, uint32_t h, uint32_t existing,
+                                                     float new_km, float new_vm, float *red, float *new_scales) {
+    const PaFp8Rows r = pa_fp8_rows(p, b, h, existing);
+    const float old_k = p.k_scale[r.si], old_v = p.v_scale[r.si];
+    uint32_t kbig, vbig;
+    pa_fp8_scan_rows(p, r, kbig, vbig);
+    float m[4] = {new_km, new_vm, (float)kbig, (float)vbig};
+    pa_block_max4(m, red);
+    new_scales[0] = pa_fp8_rescale_rows(p, r, 0, (uint32_t)m[2], m[0], old_k);
+    new_scales[1] = pa_fp8_rescale_rows(p, r, 1, (uint32_t)m[3], m[1], old_v);
+}
+
 // 3. per (touched block, kv head): the new scale; rows already in the block are re-encoded when it changes. A token
 //    that writes the block's first new row does the block's work, so the launch grows with the call, not the cache;
 //    when several tokens of a call carry that offset (the same kv_slot twice), the first workgroup to claim the block
@@ -322,41 +459,9 @@ __global__ __launch_bounds__(128) void k_pa_fp8_rescale(const PaParams p) {
     if (!mine) {
         return;
     }
-    const size_t si = (size_t)b * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] + (size_t)h * p.scale_stride[2];
-    const size_t base = (size_t)b * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2];
-    const uint32_t cells = existing * p.head_dim;
-    uint8_t *const kc = (uint8_t *)p.kv_k + base, *const vc = (uint8_t *)p.kv_v + base;
-    // The largest decoded magnitude among the rows already there: a finite code's magnitude grows with its low seven
-    // bits, so the largest such field is found first and decoded once (NaN codes, field 15, never win a maximum).
-    uint32_t kbig = 0, vbig = 0;
-    for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
-        const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
-        const size_t at = (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
-        const uint32_t kb = kc[at] & 0x7fu, vb = vc[at] & 0x7fu;
-        kbig = kb < 0x78u && kb > kbig ? kb : kbig;
-        vbig = vb < 0x78u && vb > vbig ? vb : vbig;
-    }
-    const float old_k = p.k_scale[si], old_v = p.v_scale[si];  // read by every thread before the barriers below,
-    kbig = (uint32_t)pa_block_max((float)kbig, red);           // written by thread 0 after them
-    vbig = (uint32_t)pa_block_max((float)vbig, red);
-    for (int which = 0; which < 2; ++which) {
-        uint8_t *cache = which ? vc : kc;
-        float *scales = which ? p.v_scale : p.k_scale;
-        const float old_scale = which ? old_v : old_k;
-        float big = pa_fp8_dequant(which ? vbig : kbig, old_scale);
-        big = fmaxf(big, __uint_as_float((which ? p.new_vmax : p.new_kmax)[(size_t)b * p.num_kv_heads + h]));
-        const float new_scale = big > 0.0f ? big / 240.0f : 1.0f;
-        if (existing > 0 && new_scale != old_scale) {
-            for (uint32_t c = threadIdx.x; c < cells; c += 128u) {
-                const uint32_t pos = c / p.head_dim, d = c - pos * p.head_dim;
-                uint8_t *cell = cache + (size_t)pos * p.kv_stride[3] + (size_t)d * p.kv_stride[4];
-                *cell = (uint8_t)pa_fp8_quant(pa_fp8_dequant(*cell, old_scale), new_scale);
-            }
-        }
-        if (threadIdx.x == 0) {
-            scales[si] = new_scale;
-        }
-    }
+    float scales[2];
+    pa_fp8_rescale_block(p, b, h, existing, __uint_as_float(p.new_kmax[(size_t)b * p.num_kv_heads + h]),
+                         __uint_as_float(p.new_vmax[(size_t)b * p.num_kv_heads + h]), red, scales);
 }
 
 // 4. per (token, kv head): the new rows, encoded with their block's scale
@@ -376,6 +481,72 @@ __global__ __launch_bounds__(128) void k_pa_fp8_store(const PaParams p) {
         const float vx = pa_load(p.v_new, p.act_dtype, (size_t)t * p.v_stride[0] + (size_t)h * p.v_stride[1] + d * p.v_stride[2]);
         ((uint8_t *)p.kv_k)[dst0 + d * p.kv_stride[4]] = (uint8_t)pa_fp8_quant(kx, ks);
         ((uint8_t *)p.kv_v)[dst0 + d * p.kv_stride[4]] = (uint8_t)pa_fp8_quant(vx, vs);
+    }
+}
+
+// The same update in one launch, for calls of at most PA_FP8_ONE_TOKENS tokens. Every (token, kv head) workgroup finds
+// the tokens of the call that write its block; the workgroup of the first of them does the block's work alone (largest
+// new magnitudes, new scales, re-encoding, then the new rows in token order, so of two tokens with one kv_slot the
+// later one stays, as in the reference's token loop) and the others leave. No scratch memory, no order between
+// workgroups: each (block, kv head) is touched by exactly one.
+constexpr uint32_t PA_FP8_ONE_TOKENS = 1024;
+__global__ __launch_bounds__(128) void k_pa_fp8_update(const PaParams p) {
+    __shared__ float red[128];
+    __shared__ uint32_t members[PA_FP8_ONE_TOKENS / 32];
+    __shared__ uint32_t first_off;
+    const uint32_t t = blockIdx.x, h = blockIdx.y;
+    const uint32_t b = p.meta[t * p.meta_stride[0] + 2 * p.meta_stride[1]] >> p.shift;
+    if (b >= p.kv_blocks) {
+        return;
+    }
+    if (threadIdx.x < PA_FP8_ONE_TOKENS / 32) {
+        members[threadIdx.x] = 0u;
+    }
+    if (threadIdx.x == 0) {
+        first_off = p.block_size;
+    }
+    __syncthreads();
+    for (uint32_t u = threadIdx.x; u < p.token_count; u += 128u) {
+        const uint32_t slot = p.meta[u * p.meta_stride[0] + 2 * p.meta_stride[1]];
+        if ((slot >> p.shift) == b) {
+            atomicOr(members + (u >> 5), 1u << (u & 31u));
+            atomicMin(&first_off, slot & p.mask);
+        }
+    }
+    __syncthreads();
+    bool first = (members[t >> 5] & ((1u << (t & 31u)) - 1u)) == 0u;
+    for (uint32_t w = 0; w < (t >> 5); ++w) {
+        first = first && members[w] == 0u;
+    }
+    if (!first) {
+        return;
+    }
+    const uint32_t words = (p.token_count + 31u) >> 5;
+    float km = 0.0f, vm = 0.0f;
+    for (uint32_t w = t >> 5; w < words; ++w) {
+        for (uint32_t bits = members[w]; bits != 0u; bits &= bits - 1u) {
+            const uint32_t u = w * 32u + (uint32_t)__ffs(bits) - 1u;
+            for (uint32_t d = threadIdx.x; d < p.head_dim; d += 128u) {
+                km = fmaxf(km, fabsf(pa_load(p.k_new, p.act_dtype, (size_t)u * p.k_stride[0] + (size_t)h * p.k_stride[1] + d * p.k_stride[2])));
+                vm = fmaxf(vm, fabsf(pa_load(p.v_new, p.act_dtype, (size_t)u * p.v_stride[0] + (size_t)h * p.v_stride[1] + d * p.v_stride[2])));
+            }
+        }
+    }
+    float scales[2];
+    pa_fp8_rescale_block(p, b, h, first_off, km, vm, red, scales);
+    const size_t dst0 = (size_t)b * p.kv_stride[0] + (size_t)p.layer_idx * p.kv_stride[1] + (size_t)h * p.kv_stride[2];
+    for (uint32_t w = t >> 5; w < words; ++w) {
+        for (uint32_t bits = members[w]; bits != 0u; bits &= bits - 1u) {
+            const uint32_t u = w * 32u + (uint32_t)__ffs(bits) - 1u;
+            const uint32_t slot = p.meta[u * p.meta_stride[0] + 2 * p.meta_stride[1]];
+            const size_t dst = dst0 + (size_t)(slot & p.mask) * p.kv_stride[3];
+            for (uint32_t d = threadIdx.x; d < p.head_dim; d += 128u) {
+                const float kx = pa_load(p.k_new, p.act_dtype, (size_t)u * p.k_stride[0] + (size_t)h * p.k_stride[1] + d * p.k_stride[2]);
+                const float vx = pa_load(p.v_new, p.act_dtype, (size_t)u * p.v_stride[0] + (size_t)h * p.v_stride[1] + d * p.v_stride[2]);
+                ((uint8_t *)p.kv_k)[dst + d * p.kv_stride[4]] = (uint8_t)pa_fp8_quant(kx, scales[0]);
+                ((uint8_t *)p.kv_v)[dst + d * p.kv_stride[4]] = (uint8_t)pa_fp8_quant(vx, scales[1]);
+            }
+        }
     }
 }
 
@@ -1173,10 +1344,14 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
         if (cells > ((size_t)1 << 32)) {
             return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "paged_attention: FP8 cache of %zu blocks", a->kv_blocks);
         }
-        hipLaunchKernelGGL(k_pa_fp8_init, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, dev->stream, p);
-        hipLaunchKernelGGL(k_pa_fp8_scan_new, per_token, dim3(128), 0, dev->stream, p);
-        hipLaunchKernelGGL(k_pa_fp8_rescale, per_token, dim3(128), 0, dev->stream, p);
-        hipLaunchKernelGGL(k_pa_fp8_store, per_token, dim3(128), 0, dev->stream, p);
+        if (a->token_count <= PA_FP8_ONE_TOKENS && !dev->knobs.no_fp8_update_fused) {
+            hipLaunchKernelGGL(k_pa_fp8_update, per_token, dim3(128), 0, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL(k_pa_fp8_init, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, dev->stream, p);
+            hipLaunchKernelGGL(k_pa_fp8_scan_new, per_token, dim3(128), 0, dev->stream, p);
+            hipLaunchKernelGGL(k_pa_fp8_rescale, per_token, dim3(128), 0, dev->stream, p);
+            hipLaunchKernelGGL(k_pa_fp8_store, per_token, dim3(128), 0, dev->stream, p);
+        }
     } else {
         hipLaunchKernelGGL(k_pa_write, per_token, dim3(a->head_dim <= 64 ? 64 : 128), 0, dev->stream, p);
     }

@@ -223,6 +223,7 @@ struct marmot_hip_knobs {
     bool no_row_kernels = false;
     bool no_resident_rows = false;
     bool no_attention_mfma = false;  // MARMOT_HIP_NO_ATTENTION_MFMA: paged attention scores on the vector units
+    bool no_fp8_update_fused = false;  // MARMOT_HIP_NO_FP8_UPDATE_FUSED: FLOAT8_E4M3 cache update in four launches
     bool no_lds_ring = false;
     bool no_fused_quant = false;
     bool no_gemm = false;
@@ -439,6 +440,7 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
                    size_t M, int out_dtype, void *scratch);
 // Tiled int8 GEMM on Q8_0 activations (mh_gemm_i8.hip): Q8_0 and Q4_0 weights, K a multiple of 256, nine rows and more;
 // `scratch` holds gemm_i8_scratch_bytes for the K-split partial sums
+bool gemm_q80_kind(int kind);  // Q8_0, Q4_0, Q4_1, Q5_0, Q5_1: the 32-value formats of the tiled int8 GEMM
 bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                       const ActScratch &act);
 int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,

@@ -172,6 +172,7 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
     dev->knobs.no_row_kernels = getenv("MARMOT_HIP_NO_ROW_KERNELS") != nullptr;
     dev->knobs.no_resident_rows = getenv("MARMOT_HIP_NO_RESIDENT_ROWS") != nullptr;
     dev->knobs.no_attention_mfma = getenv("MARMOT_HIP_NO_ATTENTION_MFMA") != nullptr;
+    dev->knobs.no_fp8_update_fused = getenv("MARMOT_HIP_NO_FP8_UPDATE_FUSED") != nullptr;
     dev->knobs.no_lds_ring = getenv("MARMOT_HIP_NO_LDS_RING") != nullptr;
     dev->knobs.no_fused_quant = getenv("MARMOT_HIP_NO_FUSED_QUANT") != nullptr;
     dev->knobs.no_gemm = getenv("MARMOT_HIP_NO_GEMM") != nullptr;

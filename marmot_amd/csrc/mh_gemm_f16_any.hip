@@ -2,23 +2,24 @@
 // v_mfma_f32_32x32x16_f16 with fp32 accumulation.
 //
 // Arithmetic. The reference's direct fp16 dots (cpu_vec_dot_*_f16, vec_dot_impl.h:240-450 for the 32-value formats,
-// :866-1128 for the K-quants) decode a weight to fp32 and add w * (float)x in fp32, element by element. Here a weight is
-// decoded by the same function as in the fp16 matvec (direct_f16_weight<KIND>, mh_dequant.h: the reference's own index
-// patterns, which for Q2_K / Q3_K / Q5_K / Q6_K differ from its dequantizers), then written as the sum of two fp16
-// numbers, w = hi + lo with |w - hi - lo| <= 2^-22 |w|; hi * x and lo * x are exact in fp32, so the result differs from
-// exact arithmetic by 2^-22 per weight and by the fp32 accumulation, less than the reference's own sequential sum.
-// Weights must be below the fp16 maximum in magnitude (65504; any trained model's are below 100).
-// Q8_0, Q4_0 and Q6_K weights are an integer times a scale that is constant over a round of 32 values (Q6_K, as the
-// reference's fp16 dot decodes it: over 128): for them the INTEGER is the fp16 operand (exact, one part instead of two)
-// and the scale is applied to the round's (four rounds') product in fp32, as d is in the Q4_K kernels.
+// :866-1128 for the K-quants) decode a weight to fp32 and add w * (float)x in fp32, element by element. The weight they
+// see (direct_f16_weight<KIND>, mh_dequant.h: the reference's own index patterns, which for Q2_K / Q3_K / Q5_K / Q6_K
+// differ from its dequantizers) is, in every format, scale * integer + offset with a scale and an offset that are
+// constant over a round of 32 values or more (Q6_K and Q2_K, as those dots decode them: over 128; Q3_K's group scales
+// go into the integer). Here the INTEGER is the fp16 operand (exact; its products with fp16 activations are exact in
+// fp32), the scale is applied to the span's product in fp32 as d is in the Q4_K kernels, and the offset to the span's
+// sum of activations, which one more matrix instruction against ones delivers. The result differs from exact
+// arithmetic by the fp32 accumulation and two roundings per span, less than the reference's own sequential sum.
 //
 // Tiling. A workgroup of four wavefronts owns 128 weight rows x 64 tokens and walks K in rounds of 32 values (one block
-// of the 32-value formats, an eighth of a K-quant block). Per round every thread decodes 16 weights of one row (the
-// same 16-value half of the round for all rows; for Q8_0, Q4_0 and Q6_K the bytes are requested a round earlier),
-// splits them and stores them into one of two LDS stages in MFMA operand order; wavefront c then multiplies its 32 rows with the 64 tokens: two K-steps x two parts x two token tiles = eight
-// matrix instructions; the activations come through LDS in stages of four rounds (whole 256-byte runs of a token's row
-// per 16 lanes: a lane-per-token gather of 16 bytes costs the compute unit's address unit 32 cache lines per
-// instruction and was the bound of the first form, 102 us whatever the format). One barrier per round. K is split across workgroups when the tiles do not fill the chip; the partial sums meet in k_gemm_reduce.
+// of the 32-value formats, an eighth of a K-quant block). Per round every thread turns 16 weights of one row (the same
+// 16-value half of the round for all rows; the bytes are requested a round earlier) into fp16 integers and stores them
+// into one of two LDS stages in MFMA operand order; wavefront c then multiplies its 32 rows with the 64 tokens: two
+// K-steps x two token tiles = four matrix instructions (eight with an offset); the activations come through LDS in
+// stages of four rounds (whole 256-byte runs of a token's row per 16 lanes: a lane-per-token gather of 16 bytes costs
+// the compute unit's address unit 32 cache lines per instruction and was the bound of the first form, 102 us whatever
+// the format). One barrier per round. K is split across workgroups when the tiles do not fill the chip; the partial
+// sums meet in k_gemm_reduce.
 #include "mh_common.h"
 #include "mh_dequant.h"
 
@@ -61,36 +62,33 @@ __device__ __forceinline__ void any_bytes_to_f16(uint32_t bytes, uint32_t &lo, u
     hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, b) + off);
 }
 
-// formats whose weights are an integer times one scale per round (or per four rounds): the integer is the exact fp16
-// operand and the scale goes onto the round's product, like d in the Q4_K kernels
+// Every format's weight is an integer times a scale that is constant over a round of 32 values or more, plus (Q4_1,
+// Q5_1, Q5_K, Q2_K) an offset that is constant over the same span: the integer is the exact fp16 operand, the scale goes
+// onto the span's product like d in the Q4_K kernels, and the offset multiplies the span's sum of activations, which a
+// matrix instruction against a row of ones delivers in the layout of the products.
 template <int KIND>
 struct AnyInt {
-    static constexpr bool ON = KIND == MARMOT_HIP_KIND_Q8_0 || KIND == MARMOT_HIP_KIND_Q4_0 || KIND == MARMOT_HIP_KIND_Q6_K;
-    static constexpr int SCALE_ROUNDS = KIND == MARMOT_HIP_KIND_Q6_K ? 4 : 1;  // rounds that share a scale
-    // bytes of one weight stage: K-step x part x wavefront x k half x row x 16 bytes (+ 128 scales)
-    static constexpr int WSTAGE = ON ? 2 * 4 * 2 * 32 * 16 + 512 : 2 * 2 * 4 * 2 * 32 * 16;
+    static constexpr bool HAS_MIN = KIND == MARMOT_HIP_KIND_Q4_1 || KIND == MARMOT_HIP_KIND_Q5_1 ||
+                                    KIND == MARMOT_HIP_KIND_Q5_K || KIND == MARMOT_HIP_KIND_Q2_K;
+    // rounds that share a scale (and an offset): Q6_K and Q2_K as the reference's fp16 dots decode them, 128 values;
+    // Q3_K's six-bit group scales (per 16 values) are multiplied into the integer operand, which leaves d per block
+    static constexpr int SCALE_ROUNDS = (KIND == MARMOT_HIP_KIND_Q6_K || KIND == MARMOT_HIP_KIND_Q2_K) ? 4
+        : KIND == MARMOT_HIP_KIND_Q3_K                                                                 ? 8
+                                                                                                       : 1;
+    // bytes of one weight stage: K-step x wavefront x k half x row x 16 bytes + 128 scales (+ 128 offsets)
+    static constexpr int SCALE_OFF = 2 * 4 * 2 * 32 * 16;
+    static constexpr int WSTAGE = SCALE_OFF + 512 + (HAS_MIN ? 512 : 0);
     static constexpr int LDS_BYTES = 2 * WSTAGE + 2 * FA_XSTAGE;
     static_assert(FA_TOK * FA_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
 };
 
-// The 16 weights a thread decodes per round, in two steps so that the bytes can be requested a round before they are
-// needed: fetch() issues the loads, decode() turns them into the fp32 weights of direct_f16_weight<KIND> (same
-// expressions, same bits). Formats without a form of their own keep the pointer and load inside decode().
+// The 16 weights a thread handles per round, in two steps so that the bytes can be requested a round before they are
+// needed: fetch(block, v) issues the loads for values v .. v + 15 of the block (v a multiple of 16), ints() turns them
+// into the 16 integers as exact fp16 values (two per word, in order), the scale they share and their offset. The
+// weight of direct_f16_weight<KIND> (mh_dequant.h) is scale * integer + offset, up to that function's own roundings.
 template <int KIND>
-struct AnyRaw {
-    const uint8_t *blk;
-    int v0;
-    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
-        blk = b;
-        v0 = v;
-    }
-    __device__ __forceinline__ void decode(float (&w)[16]) const {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            w[i] = direct_f16_weight<KIND>(blk, v0 + i);
-        }
-    }
-};
+struct AnyRaw;
+
 template <>
 struct AnyRaw<MARMOT_HIP_KIND_Q8_0> {
     uint4 q;
@@ -99,17 +97,9 @@ struct AnyRaw<MARMOT_HIP_KIND_Q8_0> {
         __builtin_memcpy(&s, b, 2);
         __builtin_memcpy(&q, b + 2 + v, 16);
     }
-    __device__ __forceinline__ void decode(float (&w)[16]) const {
-        const float d = h2f(s);
-        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            w[i] = (float)(int8_t)(qw[i >> 2] >> (8 * (i & 3))) * d;  // dequant_value_q8_0
-        }
-    }
-    // the 16 integers as exact fp16 values (two per word, in order) and the scale they share
-    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale) const {
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         scale = h2f(s);
+        offset = 0.0f;
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -118,61 +108,82 @@ struct AnyRaw<MARMOT_HIP_KIND_Q8_0> {
     }
 };
 template <>
-struct AnyRaw<MARMOT_HIP_KIND_Q4_0> {
+struct AnyRaw<MARMOT_HIP_KIND_Q8_1> {  // scale, the carried sum (unused), 32 codes
     uint4 q;
     uint16_t s;
-    int high;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
         __builtin_memcpy(&s, b, 2);
-        __builtin_memcpy(&q, b + 2, 16);
-        high = v >= 16;
+        __builtin_memcpy(&q, b + 4 + v, 16);
     }
-    __device__ __forceinline__ void decode(float (&w)[16]) const {
-        const float d = h2f(s);
-        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t byte = (qw[i >> 2] >> (8 * (i & 3))) & 0xffu;
-            const int nib = (int)(high ? byte >> 4 : byte & 0xfu);
-            w[i] = (float)(nib - 8) * d;  // dequant_value_q4_0
-        }
-    }
-    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale) const {
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         scale = h2f(s);
+        offset = 0.0f;
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const uint32_t nib = (high ? qw[e] >> 4 : qw[e]) & 0x0f0f0f0fu;
-            any_bytes_to_f16<1032>(nib, h[2 * e], h[2 * e + 1]);  // nibble - 8
+            any_bytes_to_f16<1152>(qw[e] ^ 0x80808080u, h[2 * e], h[2 * e + 1]);
         }
     }
 };
+
+// The 32-value formats with nibbles: byte i of qs holds value i (low nibble) and value 16 + i (high nibble); Q5_0 / Q5_1
+// keep the fifth bit of value i in bit i of a 32-bit word before qs. HDR: bytes before that word / before qs.
+template <int HDR, bool FIFTH, bool MIN, int CENTRE>
+struct AnyRawNibbles {
+    uint4 q;
+    uint32_t qh;
+    uint16_t s, m;
+    int high;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        __builtin_memcpy(&s, b, 2);
+        if constexpr (MIN) {
+            __builtin_memcpy(&m, b + 2, 2);
+        }
+        if constexpr (FIFTH) {
+            __builtin_memcpy(&qh, b + HDR, 4);
+        }
+        __builtin_memcpy(&q, b + HDR + (FIFTH ? 4 : 0), 16);
+        high = v >= 16;
+    }
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
+        scale = h2f(s);
+        offset = MIN ? h2f(m) : 0.0f;
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+        const uint32_t hbits = FIFTH ? (high ? qh >> 16 : qh) : 0u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            uint32_t val = (high ? qw[e] >> 4 : qw[e]) & 0x0f0f0f0fu;
+            if constexpr (FIFTH) {  // bits 4 e .. 4 e + 3 to bit 4 of bytes 0 .. 3
+                val |= ((((hbits >> (4 * e)) & 0xfu) * 0x00204081u) & 0x01010101u) << 4;
+            }
+            any_bytes_to_f16<1024 + CENTRE>(val, h[2 * e], h[2 * e + 1]);
+        }
+    }
+};
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q4_0> : AnyRawNibbles<2, false, false, 8> {};   // (nibble - 8) * d
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q4_1> : AnyRawNibbles<4, false, true, 0> {};    // nibble * d + m
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q5_0> : AnyRawNibbles<2, true, false, 16> {};   // (value - 16) * d
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q5_1> : AnyRawNibbles<4, true, true, 0> {};     // value * d + m
+
 template <>
 struct AnyRaw<MARMOT_HIP_KIND_Q6_K> {
     uint2 ql;
     uint32_t qh;
     int8_t sc;
     uint16_t d;
-    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {  // v: a multiple of 16
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
         __builtin_memcpy(&ql, b + (v >> 1), 8);
         __builtin_memcpy(&qh, b + 128 + (v >> 2), 4);
         sc = (int8_t)b[192 + (v >> 7)];
         __builtin_memcpy(&d, b + 208, 2);
     }
-    __device__ __forceinline__ void decode(float (&w)[16]) const {  // direct_f16_weight_q6_k for v .. v + 15
-        const float scale = h2f(d) * (float)sc;
-        const uint32_t lw[2] = {ql.x, ql.y};
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t byte = (lw[i >> 3] >> (8 * ((i >> 1) & 3))) & 0xffu;
-            const uint32_t nib = (i & 1) ? byte >> 4 : byte & 0xfu;
-            const uint32_t hi2 = (qh >> (8 * (i >> 2) + 2 * (i & 3))) & 3u;
-            const int qv = (int)(int8_t)(nib | (hi2 << 4)) - 32;
-            w[i] = scale * (float)qv;
-        }
-    }
-    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale) const {
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         scale = h2f(d) * (float)sc;
+        offset = 0.0f;
         // value i: nibble i % 2 of byte i / 2 of ql, bits 2 (i % 4) .. + 1 of byte i / 4 of qh as bits 4..5
         const uint32_t lw[2] = {ql.x, ql.y};
         // the high pairs of values 4 b + t, already at bits 4..5, in byte b of plane t
@@ -189,6 +200,108 @@ struct AnyRaw<MARMOT_HIP_KIND_Q6_K> {
             const uint32_t p23 = __builtin_amdgcn_perm(pl[3], pl[2], sel);
             const uint32_t his = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
             any_bytes_to_f16<1056>(nibs | his, h[2 * k], h[2 * k + 1]);  // 6-bit value - 32
+        }
+    }
+};
+
+// Q5_K as cpu_vec_dot_q5_k_f16 reads it (direct_f16_weight_q5_k): sub-block j = v / 32 has the Q4_K scale / min pair
+// j; value l of it is nibble j % 2 of qs[32 (j / 2) + l] plus 16 x bit 0 of the byte 8 (j / 2) + l + 32 (j % 2) behind
+// the start of qh (block bytes 16 ..; for most values a byte of qs).
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q5_K> {
+    uint4 q, hb;
+    uint32_t s0, s1, s2, dd;
+    int j;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        j = v >> 5;
+        const int l0 = v & 31, g = j >> 1;
+        __builtin_memcpy(&dd, b, 4);
+        __builtin_memcpy(&s0, b + 4, 4);
+        __builtin_memcpy(&s1, b + 8, 4);
+        __builtin_memcpy(&s2, b + 12, 4);
+        __builtin_memcpy(&hb, b + 16 + 8 * g + l0 + 32 * (j & 1), 16);
+        __builtin_memcpy(&q, b + 48 + 32 * g + l0, 16);
+    }
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
+        // scales[j], scales[j + 4] (j < 4) or scales[j + 4], scales[j - 4], scales[j] (j >= 4): byte j % 4 of a word
+        const int sh = 8 * (j & 3);
+        const uint32_t a = (s0 >> sh) & 0xffu, b = (s1 >> sh) & 0xffu, c = (s2 >> sh) & 0xffu;
+        const uint32_t sc = j < 4 ? (a & 63u) : ((c & 0xfu) | ((a >> 6) << 4));
+        const uint32_t mn = j < 4 ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
+        scale = h2f((uint16_t)(dd & 0xffffu)) * (float)sc;
+        offset = -(h2f((uint16_t)(dd >> 16)) * (float)mn);
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w}, hw[4] = {hb.x, hb.y, hb.z, hb.w};
+        const int shift = (j & 1) ? 4 : 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t val = ((qw[e] >> shift) & 0x0f0f0f0fu) | ((hw[e] & 0x01010101u) << 4);
+            any_bytes_to_f16<1024>(val, h[2 * e], h[2 * e + 1]);
+        }
+    }
+};
+
+// Q2_K as cpu_vec_dot_q2_k_f16 reads it (direct_f16_weight_q2_k): one scale / min pair per 128 values (scales[v / 128]),
+// value v in bits 2 (v % 4) .. + 1 of qs[v / 4].
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q2_K> {
+    uint32_t q, dd;
+    uint8_t sc;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        sc = b[v >> 7];
+        __builtin_memcpy(&q, b + 16 + (v >> 2), 4);
+        __builtin_memcpy(&dd, b + 80, 4);
+    }
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
+        scale = h2f((uint16_t)(dd & 0xffffu)) * (float)(sc & 0xFu);
+        offset = -(h2f((uint16_t)(dd >> 16)) * (float)(sc >> 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t b = (q >> (8 * e)) & 0xffu;  // pair k of the byte to byte k: b << 6 k puts bit 2 k at 8 k
+            const uint32_t val = (b | (b << 6) | (b << 12) | (b << 18)) & 0x03030303u;
+            any_bytes_to_f16<1024>(val, h[2 * e], h[2 * e + 1]);
+        }
+    }
+};
+
+// Q3_K as cpu_vec_dot_q3_k_f16 reads it (direct_f16_weight_q3_k): value v = 128 c + 32 j + li is bits 2 j .. + 1 of
+// qs[32 c + li], minus 4 unless bit c of hmask[li] is set, times the six-bit scale of group v / 16 (minus 32), times d.
+// The integer operand is value x group scale (at most 128 in magnitude, exact in fp16); d is the block's scale.
+template <>
+struct AnyRaw<MARMOT_HIP_KIND_Q3_K> {
+    uint4 q, hm;
+    uint32_t t0, t1, t2;
+    uint16_t d;
+    int v0;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        v0 = v;
+        const int c = v >> 7, li = v & 31;
+        __builtin_memcpy(&hm, b + li, 16);
+        __builtin_memcpy(&q, b + 32 + 32 * c + li, 16);
+        __builtin_memcpy(&t0, b + 96, 4);
+        __builtin_memcpy(&t1, b + 100, 4);
+        __builtin_memcpy(&t2, b + 104, 4);
+        __builtin_memcpy(&d, b + 108, 2);
+    }
+    __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
+        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+        scale = h2f(d);
+        offset = 0.0f;
+        const int c = v0 >> 7, j = (v0 >> 5) & 3, is = v0 >> 4;
+        // q3k_group_scale(scales, is): low nibble from scales[is] (is < 8) or the high nibble of scales[is - 8], two
+        // more bits from scales[8 + is % 4]
+        const uint64_t low8 = (uint64_t)t0 | ((uint64_t)t1 << 32);
+        const uint32_t low = (uint32_t)(low8 >> (8 * (is & 7) + (is < 8 ? 0 : 4))) & 0xfu;
+        const uint32_t high = (t2 >> (8 * (is & 3) + 2 * (is >> 2))) & 3u;
+        const _Float16 gs = (_Float16)(float)((int)(low | (high << 4)) - 32);
+        const h2_t gs2 = {gs, gs};
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w}, hw[4] = {hm.x, hm.y, hm.z, hm.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t val = ((qw[e] >> (2 * j)) & 0x03030303u) | (((hw[e] >> c) & 0x01010101u) << 2);  // 0 .. 7
+            uint32_t lo, hi;
+            any_bytes_to_f16<1028>(val, lo, hi);  // value - 4
+            h[2 * e] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, lo) * gs2);
+            h[2 * e + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2_t, hi) * gs2);
         }
     }
 };
@@ -223,13 +336,12 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
     size_t wr = row0 + (size_t)drow;
     wr = wr < p.M ? wr : p.M - 1;  // rows beyond M re-read the last row (never stored)
     const uint8_t *const wrow = p.w + wr * p.row_bytes;
-    // LDS slot of (K-step ks, part, wavefront c, k half, row j): 16 bytes
-    constexpr bool INTW = AnyInt<KIND>::ON;
-    constexpr int PARTS = INTW ? 1 : 2;
-    constexpr int SCALE_OFF = 2 * PARTS * 4 * 2 * 32 * 16;  // INTW: 128 floats behind the operands of a stage
+    // LDS slot of (K-step ks, wavefront c, k half, row j): 16 bytes
+    constexpr bool HAS_MIN = AnyInt<KIND>::HAS_MIN;
+    constexpr int SCALE_OFF = AnyInt<KIND>::SCALE_OFF;  // 128 scales (and 128 offsets) behind the operands of a stage
     constexpr int WSTAGE = AnyInt<KIND>::WSTAGE;
-    auto slot = [](int ks, int part, int c, int half, int row) -> uint32_t {
-        return (uint32_t)(((((ks * PARTS + part) * 4 + c) * 2 + half) * 32 + row) * 16);
+    auto slot = [](int ks, int c, int half, int row) -> uint32_t {
+        return (uint32_t)((((ks * 4 + c) * 2 + half) * 32 + row) * 16);
     };
     auto fetch = [&](size_t round, AnyRaw<KIND> &raw) {
         const size_t k0 = round * FA_ROUND + (size_t)(16 * dks);
@@ -237,39 +349,19 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
         raw.fetch(wrow + b * KT::BB, (int)(k0 - b * KT::BV));
     };
     auto decode = [&](const AnyRaw<KIND> &raw, int stage) {
-        if constexpr (INTW) {
-            uint32_t h[8];
-            float scale;
-            raw.ints(h, scale);
-            uint8_t *st = lds + (size_t)stage * WSTAGE;
-            const int c = drow >> 5, row = drow & 31;
-            *(uint4 *)(st + slot(dks, 0, c, 0, row)) = make_uint4(h[0], h[1], h[2], h[3]);
-            *(uint4 *)(st + slot(dks, 0, c, 1, row)) = make_uint4(h[4], h[5], h[6], h[7]);
-            if (dks == 0) {
-                *(float *)(st + SCALE_OFF + 4 * drow) = scale;
-            }
-            return;
-        }
-        float w[16];
-        raw.decode(w);
-        uint32_t hi[8], lo[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            uint16_t h[2], l[2];
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                h[e] = f2h(w[2 * i + e]);
-                l[e] = f2h(w[2 * i + e] - h2f(h[e]));
-            }
-            hi[i] = (uint32_t)h[0] | ((uint32_t)h[1] << 16);
-            lo[i] = (uint32_t)l[0] | ((uint32_t)l[1] << 16);
-        }
+        uint32_t h[8];
+        float scale, offset;
+        raw.ints(h, scale, offset);
         uint8_t *st = lds + (size_t)stage * WSTAGE;
         const int c = drow >> 5, row = drow & 31;
-        *(uint4 *)(st + slot(dks, 0, c, 0, row)) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        *(uint4 *)(st + slot(dks, 0, c, 1, row)) = make_uint4(hi[4], hi[5], hi[6], hi[7]);
-        *(uint4 *)(st + slot(dks, 1, c, 0, row)) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        *(uint4 *)(st + slot(dks, 1, c, 1, row)) = make_uint4(lo[4], lo[5], lo[6], lo[7]);
+        *(uint4 *)(st + slot(dks, c, 0, row)) = make_uint4(h[0], h[1], h[2], h[3]);
+        *(uint4 *)(st + slot(dks, c, 1, row)) = make_uint4(h[4], h[5], h[6], h[7]);
+        if (dks == 0) {
+            *(float *)(st + SCALE_OFF + 4 * drow) = scale;
+            if constexpr (HAS_MIN) {
+                *(float *)(st + SCALE_OFF + 512 + 4 * drow) = offset;
+            }
+        }
     };
 
     // Activations go through LDS in stages of four rounds (128 values of K): 64 tokens x 256 bytes, token t's 16-byte
@@ -302,15 +394,19 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
     };
 
     fa_floatx16 acc[2];
-    fa_floatx16 grp[2];  // INTW: the products of the rounds that share a scale
+    fa_floatx16 grp[2];                      // the products of the rounds that share a scale
+    fa_floatx16 xsum[HAS_MIN ? 2 : 1];       // the sums of their activations (every lane: its 16 tokens' sums)
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             acc[a][r] = 0.0f;
             grp[a][r] = 0.0f;
+            xsum[HAS_MIN ? a : 0][r] = 0.0f;
         }
     }
+    const fa_half8 ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f,
+                           (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
 
     AnyRaw<KIND> raw[2];
     auto multiply = [&](size_t round, int stage) {
@@ -328,51 +424,48 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
                     fa_half8, *(const uint4 *)(xs + (32 * a + j) * 256 + 16 * ((4 * q + 2 * ks + kh) ^ (j & 15))));
             }
         }
-        if constexpr (INTW) {
-            constexpr int SR = AnyInt<KIND>::SCALE_ROUNDS;
-            const bool opens = SR == 1 || (round % SR) == 0, closes = SR == 1 || (round % SR) == SR - 1;
-            if (opens) {
+        constexpr int SR = AnyInt<KIND>::SCALE_ROUNDS;
+        const bool opens = SR == 1 || (round % SR) == 0, closes = SR == 1 || (round % SR) == SR - 1;
+        if (opens) {
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
+            for (int a = 0; a < 2; ++a) {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        grp[a][r] = 0.0f;
-                    }
+                for (int r = 0; r < 16; ++r) {
+                    grp[a][r] = 0.0f;
+                    xsum[HAS_MIN ? a : 0][r] = 0.0f;
                 }
             }
+        }
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, 0, wave, kh, j)));
+        for (int ks = 0; ks < 2; ++ks) {
+            const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, wave, kh, j)));
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
-                    grp[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], wb, grp[a], 0, 0, 0);
+            for (int a = 0; a < 2; ++a) {
+                grp[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], wb, grp[a], 0, 0, 0);
+                if constexpr (HAS_MIN) {
+                    xsum[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], ones, xsum[a], 0, 0, 0);
                 }
             }
-            if (closes) {
-                const float scale = *(const float *)(st + SCALE_OFF + 4 * (32 * wave + j));
-#pragma unroll
-                for (int a = 0; a < 2; ++a) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        float t = __builtin_fmaf(scale, grp[a][r], acc[a][r]);
-                        // keeps the scaling inside its round (an empty statement the optimizer cannot move across the
-                        // barrier): sunk behind the later rounds, every round holds its own 32 product registers
-                        // until the end of the stage, and the four sets spill
-                        asm volatile("" : "+v"(t));
-                        acc[a][r] = t;
-                    }
-                }
+        }
+        if (closes) {
+            const float scale = *(const float *)(st + SCALE_OFF + 4 * (32 * wave + j));
+            float offset = 0.0f;
+            if constexpr (HAS_MIN) {
+                offset = *(const float *)(st + SCALE_OFF + 512 + 4 * (32 * wave + j));
             }
-        } else {
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
+            for (int a = 0; a < 2; ++a) {
 #pragma unroll
-                for (int part = 0; part < 2; ++part) {
-                    const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, part, wave, kh, j)));
-#pragma unroll
-                    for (int a = 0; a < 2; ++a) {
-                        acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], wb, acc[a], 0, 0, 0);
+                for (int r = 0; r < 16; ++r) {
+                    float t = __builtin_fmaf(scale, grp[a][r], acc[a][r]);
+                    if constexpr (HAS_MIN) {
+                        t = __builtin_fmaf(offset, xsum[a][r], t);
                     }
+                    // keeps the scaling inside its round (an empty statement the optimizer cannot move across the
+                    // barrier): sunk behind the later rounds, every round holds its own 32 product registers
+                    // until the end of the stage, and the four sets spill
+                    asm volatile("" : "+v"(t));
+                    acc[a][r] = t;
                 }
             }
         }

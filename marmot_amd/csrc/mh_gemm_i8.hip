@@ -34,6 +34,7 @@ struct GemmI8Params {
     const uint8_t *w;   // Q4_K blocks, M rows of nb blocks
     const int8_t *qs;   // quantized activations, rows of kp bytes
     const float *ad;    // activation block scales [N][nb]
+    const int16_t *sums = nullptr;  // Q8_0 activations: sum of a block's codes [N][8 nb] (formats with a minimum)
     size_t kp;
     size_t N, M, nb;
     void *out;          // [N][M] of the output type, or fp32 partials [splits][N][M] when splits > 1
@@ -1015,9 +1016,12 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
     i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
-// ------------------------------------------------------------------ Q8_0 / Q4_0 x Q8_0
+// ------------------------------------------------------------------ the 32-value formats x Q8_0
 // cpu_vec_dot_q8_0_q8_0 / cpu_vec_dot_q4_0_q8_0 (vec_dot_impl.h:452-479 and its Q4_0 sibling): per 32-value block
 //     y += (float)(q . a) * (w.d * a.d),
+// Q5_0 likewise with q = (nibble | fifth bit << 4) - 16; Q4_1 and Q5_1 (vec_dot_impl.h:186-217, 288-349) keep q
+// unsigned and add w.min * a.d * sum(a) per block: a.d * sum(a) depends on the token alone and is formed once per
+// round and token into LDS ([block][token], beside the scales), so the term costs one more multiply-add per output.
 // integer dot exact, one fp32 multiply-add per block in block order. Here a block of 32 weight rows x 32 tokens is one
 // v_mfma_i32_32x32x32_i8, and every output takes its block's product of the two scales with three vector
 // instructions (convert, scale product, multiply-add): the formats have one scale per 32 values and nothing to fold,
@@ -1029,18 +1033,26 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
 // 8 x 64 activation scales of the round as [block][token] (one dword gather per block and round).
 template <int KIND>
 struct Q80Tile {
-    static constexpr int BLK = KIND == MARMOT_HIP_KIND_Q8_0 ? 34 : 18;
+    static constexpr bool HAS_MIN = KIND == MARMOT_HIP_KIND_Q4_1 || KIND == MARMOT_HIP_KIND_Q5_1;
+    static constexpr bool FIFTH = KIND == MARMOT_HIP_KIND_Q5_0 || KIND == MARMOT_HIP_KIND_Q5_1;
+    static constexpr int BLK = KIND == MARMOT_HIP_KIND_Q8_0 ? 34 : 18 + (HAS_MIN ? 2 : 0) + (FIFTH ? 4 : 0);
+    static constexpr int QS_AT = BLK - (KIND == MARMOT_HIP_KIND_Q8_0 ? 32 : 16);  // the values behind the header
     static constexpr int CHUNK = 8 * BLK;
     static constexpr int PIECES = CHUNK / 16;
-    static constexpr int PITCH_P = KIND == MARMOT_HIP_KIND_Q8_0 ? 19 : 9;
+    // an odd number of 16-byte pieces: 16 rows start in 16 different bank groups (Q8_0: 19, so that the second group a
+    // read at byte 2 of a block touches is not another row's first)
+    static constexpr int PITCH_P = KIND == MARMOT_HIP_KIND_Q8_0 ? 19 : (PIECES | 1);
     static constexpr int ROWB = PITCH_P * 16;
     static constexpr int STAGE_W = I8_WROWS * ROWB;
     static constexpr int STAGE_D = 8 * I8_TOK * 4;
-    static constexpr int STAGE = STAGE_W + I8_STAGE_A + STAGE_D;
+    static constexpr int STAGE_S = HAS_MIN ? I8_TOK * 16 : 0;       // the round's 8 code sums of every token
+    static constexpr int STAGE_M = HAS_MIN ? 8 * I8_TOK * 4 : 0;    // scale x sum as [block][token]
+    static constexpr int STAGE = STAGE_W + I8_STAGE_A + STAGE_D + STAGE_S + STAGE_M;
     static constexpr int LDS_BYTES = 2 * STAGE;
     static constexpr int W_INSTR = (I8_WROWS * PITCH_P + 63) / 64;
     static constexpr int W_PER_WAVE = (W_INSTR + I8_WAVES - 1) / I8_WAVES;
     static_assert(CHUNK % 16 == 0 && STAGE % 16 == 0, "16-byte pieces");
+    static_assert(PITCH_P >= PIECES, "a row's pieces fit its pitch");
     static_assert(I8_TOK * I8_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
 };
 
@@ -1108,6 +1120,8 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
         d_voff = (uint32_t)((trow * 8u * p.nb + (uint32_t)wave) * 4u);  // block `wave` of the round, token `lane`
     }
     const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * 8u * p.nb);
+    const uint8_t *tile_s = (const uint8_t *)(p.sums + tt * I8_TOK * 8u * p.nb);
+    const uint32_t s_voff = (uint32_t)(((uint32_t)lane < last_tok ? (uint32_t)lane : last_tok) * 16u * p.nb);
     auto issue = [&](int ri) {
         const size_t b = b0 + (size_t)ri;
         const uint32_t s0 = lds_base + (uint32_t)((ri & 1) * T::STAGE);
@@ -1129,6 +1143,23 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
         }
         dma_set_lds_base(s0 + (uint32_t)(T::STAGE_W + I8_STAGE_A + 256 * wave));
         dma4_to_lds(tile_d + b * 32, d_voff);
+        if constexpr (T::HAS_MIN) {
+            if (wave == 7) {  // 16 bytes per token: the round's eight sums
+                dma_set_lds_base(s0 + (uint32_t)(T::STAGE_W + I8_STAGE_A + T::STAGE_D));
+                dma16_to_lds<0>(tile_s + b * 16, s_voff);
+            }
+        }
+    };
+    // scale x sum of a landed round, one (block, token) per thread
+    auto fold_sums = [&](int ri) {
+        if constexpr (T::HAS_MIN) {
+            uint8_t *stage = lds + (size_t)(ri & 1) * T::STAGE;
+            const int blk = tid >> 6, tok = tid & 63;
+            const float da = *(const float *)(stage + T::STAGE_W + I8_STAGE_A + 4 * tid);
+            const int16_t sum = *(const int16_t *)(stage + T::STAGE_W + I8_STAGE_A + T::STAGE_D + 16 * tok + 2 * blk);
+            *(float *)(stage + T::STAGE_W + I8_STAGE_A + T::STAGE_D + T::STAGE_S + 4 * tid) = da * (float)sum;
+            i8_lds_barrier();
+        }
     };
 
     // ---- compute: weight row 32 rg + j, the lane's 16 values (16 kh .. + 15) of each of its four blocks, all 64 tokens
@@ -1139,6 +1170,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
     issue(0);
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
     i8_lds_barrier();
+    fold_sums(0);
     for (int ri = 0; ri < nrounds; ++ri) {
         if (ri + 1 < nrounds) {
             issue(ri + 1);  // into the other buffer, which the barrier that closed the previous round has released
@@ -1154,19 +1186,40 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
                 __builtin_memcpy(&dh, wrow + T::BLK * blk, 2);
                 float dw = h2f(dh);
                 asm volatile("" : "+v"(dw));  // a conversion of its own (not folded into mixed-precision multiplies)
+                float mw = 0.0f;
+                if constexpr (T::HAS_MIN) {
+                    uint16_t mh;
+                    __builtin_memcpy(&mh, wrow + T::BLK * blk + 2, 2);
+                    mw = h2f(mh);
+                    asm volatile("" : "+v"(mw));
+                }
                 i8_intx4 wv;
                 if constexpr (KIND == MARMOT_HIP_KIND_Q8_0) {
                     __builtin_memcpy(&wv, wrow + T::BLK * blk + 2 + 16 * kh, 16);
                 } else {
-                    // byte i of the block: value i in the low nibble, value 16 + i in the high nibble, both minus 8:
-                    // (n + 0x78) ^ 0x80 is n - 8 as a signed byte, without carries between bytes
+                    // byte i of the block: value i in the low nibble, value 16 + i in the high nibble; Q5_0 / Q5_1: bit
+                    // i (16 + i) of the 32-bit word before them is the value's fifth bit. Q4_0: (n + 0x78) ^ 0x80 is
+                    // n - 8 as a signed byte, Q5_0: (v + 0x70) ^ 0x80 is v - 16, both without carries between bytes.
                     uint4 raw;
-                    __builtin_memcpy(&raw, wrow + T::BLK * blk + 2, 16);
+                    __builtin_memcpy(&raw, wrow + T::BLK * blk + T::QS_AT, 16);
                     const uint32_t rw[4] = {raw.x, raw.y, raw.z, raw.w};
+                    uint32_t qh = 0u;
+                    if constexpr (T::FIFTH) {
+                        __builtin_memcpy(&qh, wrow + T::BLK * blk + T::QS_AT - 4, 4);
+                        qh = kh ? qh >> 16 : qh;
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const uint32_t nib = (kh ? (rw[e] >> 4) : rw[e]) & 0x0f0f0f0fu;
-                        wv[e] = (int)((nib + 0x78787878u) ^ 0x80808080u);
+                        uint32_t v = (kh ? (rw[e] >> 4) : rw[e]) & 0x0f0f0f0fu;
+                        if constexpr (T::FIFTH) {  // bits 4 e .. 4 e + 3 to bit 4 of bytes 0 .. 3
+                            v |= ((((qh >> (4 * e)) & 0xfu) * 0x00204081u) & 0x01010101u) << 4;
+                        }
+                        if constexpr (KIND == MARMOT_HIP_KIND_Q4_0) {
+                            v = (v + 0x78787878u) ^ 0x80808080u;
+                        } else if constexpr (KIND == MARMOT_HIP_KIND_Q5_0) {
+                            v = (v + 0x70707070u) ^ 0x80808080u;
+                        }
+                        wv[e] = (int)v;
                     }
                 }
 #pragma unroll
@@ -1183,12 +1236,33 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
                             const int r = 4 * q4 + e;
                             total[a][r] = __builtin_fmaf((float)dq[r], dw * da[e], total[a][r]);
                         }
+                        if constexpr (T::HAS_MIN) {
+                            const float4 m4 = *(const float4 *)(stage + d_off + T::STAGE_D + T::STAGE_S + 256 * blk +
+                                                                4 * (32 * a + 8 * q4));
+                            const float ms[4] = {m4.x, m4.y, m4.z, m4.w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const int r = 4 * q4 + e;
+                                total[a][r] = __builtin_fmaf(mw, ms[e], total[a][r]);
+                            }
+                        }
+                    }
+                    if constexpr (T::HAS_MIN) {
+                        // one matrix product and its 16 outputs at a time (left alone, the compiler forms all eight
+                        // products of the round first and spills their 128 results)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            asm volatile("" : "+v"(total[a][r]));
+                        }
                     }
                 }
             }
         }
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's share of the next round has landed
         i8_lds_barrier();
+        if (ri + 1 < nrounds) {
+            fold_sums(ri + 1);
+        }
     }
     i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
@@ -1301,15 +1375,20 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
 // eight the packed matvec streams the weights once; measured at 4096 x 4096 / 14336 x 4096: the matvec takes 16.6 /
 // 33 us at 9 rows and 34 / 74 us at 32, this kernel 16 / 30 us at 33)
 constexpr size_t Q80_MIN_ROWS = 9;
+bool gemm_q80_kind(int kind) {
+    return kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q4_1 ||
+           kind == MARMOT_HIP_KIND_Q5_0 || kind == MARMOT_HIP_KIND_Q5_1;
+}
+
 bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                       const ActScratch &act) {
-    if (dev->knobs.no_gemm_i8 || N < Q80_MIN_ROWS || K % QK_K != 0 ||
-        (kind != MARMOT_HIP_KIND_Q8_0 && kind != MARMOT_HIP_KIND_Q4_0)) {
+    if (dev->knobs.no_gemm_i8 || N < Q80_MIN_ROWS || K % QK_K != 0 || !gemm_q80_kind(kind)) {
         return false;
     }
-    const size_t chunk = kind == MARMOT_HIP_KIND_Q8_0 ? 272 : 144;
+    const size_t chunk = 8 * block_bytes(kind);
     if ((((uintptr_t)act.qs) & 15) != 0 || act.kp % 16 != 0 || N * act.kp >= ((size_t)1 << 32) ||
-        N * (K / 32) * 4 >= ((size_t)1 << 32) || I8_WROWS * (K / QK_K) * chunk >= ((size_t)1 << 32)) {
+        N * (K / 32) * 4 >= ((size_t)1 << 32) || I8_WROWS * (K / QK_K) * chunk >= ((size_t)1 << 32) ||
+        (((uintptr_t)act.sums) & 15) != 0) {
         return false;  // 16-byte direct-to-LDS loads with 32-bit lane offsets
     }
     for (int i = 0; i < count; ++i) {
@@ -1320,9 +1399,15 @@ bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K
     return true;
 }
 
+template <int KIND>
+static int launch_gemm_q80_kind(marmot_hip_device *dev, const GemmI8Params &p, dim3 grid) {
+    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<KIND>));
+    hipLaunchKernelGGL((k_gemm_q80_tile<KIND>), grid, dim3(I8_THREADS), Q80Tile<KIND>::LDS_BYTES, dev->stream, p);
+    return MARMOT_HIP_SUCCESS;
+}
+
 int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                     size_t M, int out_dtype, void *scratch) {
-    const bool q8 = kind == MARMOT_HIP_KIND_Q8_0;
     const size_t nb = K / QK_K;
     size_t bps = 0;
     const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
@@ -1330,14 +1415,13 @@ int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const
     if (splits > 1 && partial == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "tiled Q8_0 GEMM: no room for the K-split partial sums");
     }
-    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<MARMOT_HIP_KIND_Q8_0>));
-    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<MARMOT_HIP_KIND_Q4_0>));
     const dim3 grid((unsigned)((M + I8_WROWS - 1) / I8_WROWS), (unsigned)((N + I8_TOK - 1) / I8_TOK), (unsigned)splits);
     for (int which = 0; which < ws.count; ++which) {
         GemmI8Params p;
         p.w = (const uint8_t *)ws.w[which];
         p.qs = act.qs;
         p.ad = act.d;
+        p.sums = act.sums;
         p.kp = act.kp;
         p.N = N;
         p.M = M;
@@ -1350,12 +1434,22 @@ int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const
         p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
         p.bias_first = ws.bias_first ? 1 : 0;
         p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
-        if (q8) {
-            hipLaunchKernelGGL((k_gemm_q80_tile<MARMOT_HIP_KIND_Q8_0>), grid, dim3(I8_THREADS),
-                               Q80Tile<MARMOT_HIP_KIND_Q8_0>::LDS_BYTES, dev->stream, p);
-        } else {
-            hipLaunchKernelGGL((k_gemm_q80_tile<MARMOT_HIP_KIND_Q4_0>), grid, dim3(I8_THREADS),
-                               Q80Tile<MARMOT_HIP_KIND_Q4_0>::LDS_BYTES, dev->stream, p);
+        switch (kind) {
+        case MARMOT_HIP_KIND_Q8_0:
+            MH_TRY(launch_gemm_q80_kind<MARMOT_HIP_KIND_Q8_0>(dev, p, grid));
+            break;
+        case MARMOT_HIP_KIND_Q4_0:
+            MH_TRY(launch_gemm_q80_kind<MARMOT_HIP_KIND_Q4_0>(dev, p, grid));
+            break;
+        case MARMOT_HIP_KIND_Q4_1:
+            MH_TRY(launch_gemm_q80_kind<MARMOT_HIP_KIND_Q4_1>(dev, p, grid));
+            break;
+        case MARMOT_HIP_KIND_Q5_0:
+            MH_TRY(launch_gemm_q80_kind<MARMOT_HIP_KIND_Q5_0>(dev, p, grid));
+            break;
+        default:
+            MH_TRY(launch_gemm_q80_kind<MARMOT_HIP_KIND_Q5_1>(dev, p, grid));
+            break;
         }
         MH_HIP(hipGetLastError());
         if (splits > 1) {
@@ -1363,7 +1457,13 @@ int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const
                                         out_dtype, ws.bias_first));
         }
     }
-    set_route(q8 ? "gemm_q8_0_q8_0_mfma_tile" : "gemm_q4_0_q8_0_mfma_tile");
+    static const char *const routes[] = {"gemm_q8_0_q8_0_mfma_tile", "gemm_q4_0_q8_0_mfma_tile", "gemm_q4_1_q8_0_mfma_tile",
+                                         "gemm_q5_0_q8_0_mfma_tile", "gemm_q5_1_q8_0_mfma_tile"};
+    set_route(routes[kind == MARMOT_HIP_KIND_Q8_0   ? 0
+                     : kind == MARMOT_HIP_KIND_Q4_0 ? 1
+                     : kind == MARMOT_HIP_KIND_Q4_1 ? 2
+                     : kind == MARMOT_HIP_KIND_Q5_0 ? 3
+                                                    : 4]);
     return MARMOT_HIP_SUCCESS;
 }
 

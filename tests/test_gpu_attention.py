@@ -382,3 +382,36 @@ def test_fp8_cache_duplicate_slot_rescales_the_block_once(hip, oracle):
     step = dict(case, token_meta=meta, q=rng.standard_normal((2, 2, 32), dtype=np.float32),
                 k_new=np.repeat(row_k, 2, axis=0), v_new=np.repeat(row_v, 2, axis=0), **state)
     _fp8_both(hip, oracle, step, "duplicate slot")
+
+
+def test_fp8_cache_duplicate_slot_with_different_rows_keeps_the_later_one(hip, oracle):
+    """Calls of up to 1024 tokens update the cache in one launch in which one workgroup writes all new rows of a block
+    in token order: two tokens with one kv_slot and different rows leave the later token's row, as the reference's
+    token loop does, and both rows count for the block's scale."""
+    case = _fp8_case(911, [(0, 11)], room=1, num_q_heads=2, num_kv_heads=2, head_dim=32, block_size=8)
+    state = _fp8_both(hip, oracle, case, "prefill")
+    seq = int(case["token_meta"][0, 0])
+    slot = int(case["block_table"][seq, 1]) * 8 + 3
+    meta = np.array([[seq, 11, slot, 0]] * 3, np.uint32)
+    rng = np.random.default_rng(912)
+    gain = np.array([1.0, 9.0, 2.0], np.float32)[:, None, None]  # the loudest row is not the one that stays
+    step = dict(case, token_meta=meta, q=rng.standard_normal((3, 2, 32), dtype=np.float32),
+                k_new=rng.standard_normal((3, 2, 32), dtype=np.float32) * gain,
+                v_new=rng.standard_normal((3, 2, 32), dtype=np.float32) * gain, **state)
+    _fp8_both(hip, oracle, step, "duplicate slot, different rows")
+
+
+def test_fp8_cache_update_in_four_launches(oracle, monkeypatch):
+    """Calls of more than 1024 tokens (and every call under MARMOT_HIP_NO_FP8_UPDATE_FUSED, read when a device object
+    is created) update the cache in four launches with scratch memory between them: the same bytes and scales."""
+    from marmot_amd import HipBackend
+
+    monkeypatch.setenv("MARMOT_HIP_NO_FP8_UPDATE_FUSED", "1")
+    plain = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_FP8_UPDATE_FUSED")
+    case = _fp8_case(921, [(0, 21), (0, 9), (0, 31)], room=3, num_q_heads=4, num_kv_heads=2, head_dim=64,
+                     block_size=16)
+    state = _fp8_both(plain, oracle, case, "prefill, four launches")
+    for i, gains in enumerate([(1.0, 6.0, 0.2), (30.0, 1.0, 1.0), (0.0, 1.0, 50.0)]):
+        case = _next_step(case, state, 930 + i, gains)
+        state = _fp8_both(plain, oracle, case, f"decode step {i}, four launches")

@@ -441,18 +441,19 @@ def test_tiled_int8_gemm_q6k_random_blocks_and_exact_integers(hip, oracle):
 
 
 # ---------------------------------------------------------------- tiled int8 GEMM for the 32-value formats (Q8_0, Q4_0)
-Q80_KINDS = {"q8_0": 5, "q4_0": 1}
+Q80_KINDS = {"q8_0": 5, "q4_0": 1, "q4_1": 2, "q5_0": 3, "q5_1": 4}
 
 
 @pytest.mark.parametrize("N,M,K", [(9, 70, 256), (33, 96, 512), (40, 4096, 1024), (48, 128, 256), (64, 100, 512),
                                    (100, 203, 2048), (130, 300, 1024), (64, 128, 4096), (192, 64, 7168),
                                    (512, 512, 4096)])
-@pytest.mark.parametrize("name", ["q8_0", "q4_0"])
+@pytest.mark.parametrize("name", ["q8_0", "q4_0", "q4_1", "q5_0", "q5_1"])
 def test_tiled_int8_gemm_32_value_formats_match_oracle(hip, oracle, name, N, M, K):
-    """Prefill with fp32 activations for Q8_0 / Q4_0 weights (activations packed to Q8_0): one int8 matrix instruction
-    per 32-value block and 32 x 32 outputs, the two block scales applied per output and block as in
-    cpu_vec_dot_q8_0_q8_0 (vec_dot_impl.h:452-479). Full and ragged tiles, one to 28 rounds of 256 values, K split
-    across workgroups when the tiles do not fill the chip, bias."""
+    """Prefill with fp32 activations for Q8_0 / Q4_0 / Q4_1 / Q5_0 / Q5_1 weights (activations packed to Q8_0): one
+    int8 matrix instruction per 32-value block and 32 x 32 outputs, the two block scales applied per output and block
+    as in cpu_vec_dot_q8_0_q8_0 (vec_dot_impl.h:452-479), the minimum of Q4_1 / Q5_1 times the token's scaled code sum
+    added per block (:186-217, :288-349). Full and ragged tiles, one to 28 rounds of 256 values, K split across
+    workgroups when the tiles do not fill the chip, bias."""
     kind = Q80_KINDS[name]
     blocks = oracle.quantize(kind, gaussian(430 + N, (M, K), 0.02))
     x = gaussian(431 + N, (N, K))
@@ -462,7 +463,7 @@ def test_tiled_int8_gemm_32_value_formats_match_oracle(hip, oracle, name, N, M, 
     assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"{name} tile {M}x{K} N={N}")
 
 
-@pytest.mark.parametrize("name", ["q8_0", "q4_0"])
+@pytest.mark.parametrize("name", ["q8_0", "q4_0", "q4_1", "q5_0", "q5_1"])
 def test_tiled_int8_gemm_32_value_formats_random_blocks_routes_and_epilogues(hip, oracle, monkeypatch, name):
     """Arbitrary block bytes (every code, scales of both signs down to fp16 denormals) against the oracle and against
     the packed matvec that a device object created with MARMOT_HIP_NO_GEMM_I8 keeps; shapes the tile does not cover
@@ -525,7 +526,7 @@ def test_tiled_int8_gemm_32_value_formats_random_blocks_routes_and_epilogues(hip
     assert_matmul_parity(pre, oracle.matmul(kind, w3, x3, m3, bias=b3), what=f"{name} prepacked, K split")
 
 
-@pytest.mark.parametrize("name", ["q8_0", "q4_0"])
+@pytest.mark.parametrize("name", ["q8_0", "q4_0", "q5_0"])
 def test_tiled_int8_gemm_32_value_formats_integers_are_exact(hip, name):
     """Packed activations and weight blocks whose scales are powers of two: the integer dot, its conversion and the
     product of the two scales are then exact, and what is left is one rounding per block in the multiply-add that
@@ -533,7 +534,7 @@ def test_tiled_int8_gemm_32_value_formats_integers_are_exact(hip, name):
     4..7 of the one round of 256 values are accumulated separately, each in block order, and the two sums are added."""
     kind = Q80_KINDS[name]
     q8 = name == "q8_0"
-    bb = 34 if q8 else 18
+    bb = {"q8_0": 34, "q4_0": 18, "q5_0": 22}[name]
     N, M, K = 70, 200, 256
     nb = K // 32
     rng = np.random.default_rng(450)
@@ -551,9 +552,14 @@ def test_tiled_int8_gemm_32_value_formats_integers_are_exact(hip, name):
     image[lay.scales_offset:lay.scales_offset + ad.nbytes] = ad.view(np.uint8).reshape(-1)
     if q8:
         wq = blocks[:, :, 2:].view(np.int8).astype(np.int64)                       # [M, nb, 32]
-    else:  # byte i: value i in the low nibble, value 16 + i in the high nibble, both minus 8
+    elif name == "q4_0":  # byte i: value i in the low nibble, value 16 + i in the high nibble, both minus 8
         qs = blocks[:, :, 2:].astype(np.int64)
         wq = np.concatenate([(qs & 15) - 8, (qs >> 4) - 8], axis=2)
+    else:  # Q5_0: bit i of the 32-bit word at byte 2 is value i's fifth bit; the values minus 16
+        qs = blocks[:, :, 6:].astype(np.int64)
+        qh = blocks[:, :, 2:6].copy().view(np.uint32).astype(np.int64)          # [M, nb, 1]
+        fifth = (qh >> np.arange(32)) & 1                                          # [M, nb, 32]
+        wq = np.concatenate([qs & 15, qs >> 4], axis=2) + 16 * fifth - 16
     a = q.reshape(N, nb, 32).astype(np.int64)
     dots = np.einsum("nbk,mbk->nmb", a, wq)                                        # [N, M, nb]
     scale = np.ldexp(1.0, a_exp[:, None, :] + d_exp[None, :, :])

@@ -440,7 +440,11 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
                    size_t M, int out_dtype, void *scratch);
 // Tiled int8 GEMM on Q8_0 activations (mh_gemm_i8.hip): Q8_0 and Q4_0 weights, K a multiple of 256, nine rows and more;
 // `scratch` holds gemm_i8_scratch_bytes for the K-split partial sums
-bool gemm_q80_kind(int kind);  // Q8_0, Q4_0, Q4_1, Q5_0, Q5_1: the 32-value formats of the tiled int8 GEMM
+bool gemm_q23k_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
+                       const ActScratch &act);
+int launch_gemm_q23k(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
+                     size_t M, int out_dtype, void *scratch);
+bool gemm_q80_kind(int kind);  // Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K: formats of the tiled int8 GEMMs from nine rows on
 bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                       const ActScratch &act);
 int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,

@@ -1267,6 +1267,218 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
     i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
+// ------------------------------------------------------------------ Q2_K / Q3_K x Q8_K
+// cpu_vec_dot_q2_k_q8_k (vec_dot_impl.h:560-618): per block y += (a.d * w.d) * isum - (a.d * w.dmin) * summs with
+//     isum = sum over the 16 groups of 16 values of (group scale) * (q2 . a),   summs = sum (group min) * (sum of a),
+// cpu_vec_dot_q3_k_q8_k (:620-687): y += (a.d * w.d) * sum over groups of (six-bit scale - 32) * (q3 . a), q3 the
+// two-bit value minus 4 unless its mask bit is set. Groups of 16 values carry their own scale, and a matrix instruction
+// spans two of them, so the scale is multiplied into the int8 operand (both kh halves of a product then differ only in
+// the operand bytes), and what would not fit a signed byte goes into a second chain of products:
+//   Q2_K: chain 1 = q2 * scale (0 .. 45), chain 2 = the group's min in every byte (its product is min * sum of a);
+//   Q3_K: q3 = 2 vh + vb with vh in -2 .. 1 and vb in 0 .. 1: chain 1 = vh * scale (-64 .. 64), chain 2 = vb * scale,
+//         isum = 2 * chain 1 + chain 2 (q3 * scale itself reaches +128).
+// Four packed bytes are multiplied by one small factor in a single 32-bit multiply where no byte's product reaches 256.
+// Same tile and wavefront roles as the kernels above (a round is one block; K group kg takes its steps 4 kg .. + 3), but
+// the weights do not pass through LDS: lane (j, kh) is the only reader of its row's bytes for its half of every step
+// (16 + 8 + 4 bytes per block for Q2_K, 16 + 16 + 12 + 2 for Q3_K), requested a round ahead into registers; rows of
+// 84 / 110 bytes need only 4- / 2-byte alignment.
+constexpr int I23_STAGE = I8_STAGE_A + I8_STAGE_D;  // 64 tokens x 256 codes + 64 block scales: 16,640 bytes
+constexpr int I23_LDS_BYTES = (I8_TOK * I8_OUT_PITCH * 4 > 2 * I23_STAGE) ? I8_TOK * I8_OUT_PITCH * 4 : 2 * I23_STAGE;
+
+template <int KIND>
+struct Q23Raw;
+template <>
+struct Q23Raw<MARMOT_HIP_KIND_Q2_K> {
+    uint4 q;        // qs[32 kg + 16 kh ..]: the lane's 16 values of steps 4 kg .. 4 kg + 3, two bits per step
+    uint2 sc;       // scales[8 kg ..]: group 8 kg + 2 bi + kh belongs to step bi
+    uint32_t dd;    // d, dmin
+    __device__ __forceinline__ void fetch(const uint8_t *b, int kg, int kh) {
+        __builtin_memcpy(&sc, b + 8 * kg, 8);
+        __builtin_memcpy(&q, b + 16 + 32 * kg + 16 * kh, 16);
+        __builtin_memcpy(&dd, b + 80, 4);
+    }
+};
+template <>
+struct Q23Raw<MARMOT_HIP_KIND_Q3_K> {
+    uint4 q, hm;    // qs[32 kg + 16 kh ..], hmask[16 kh ..] (bit s of a mask byte belongs to step s)
+    uint32_t t0, t1, t2;
+    uint16_t d;
+    __device__ __forceinline__ void fetch(const uint8_t *b, int kg, int kh) {
+        __builtin_memcpy(&hm, b + 16 * kh, 16);
+        __builtin_memcpy(&q, b + 32 + 32 * kg + 16 * kh, 16);
+        __builtin_memcpy(&t0, b + 96, 4);
+        __builtin_memcpy(&t1, b + 100, 4);
+        __builtin_memcpy(&t2, b + 104, 4);
+        __builtin_memcpy(&d, b + 108, 2);
+    }
+};
+
+template <int KIND>
+__global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Params p) {
+    constexpr bool Q2 = KIND == MARMOT_HIP_KIND_Q2_K;
+    constexpr int BB = Q2 ? Q2_K_BYTES : Q3_K_BYTES;
+    warm_kernel_arguments<sizeof(GemmI8Params)>();
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = wave & 3;   // weight rows 32 rg .. + 31 of the tile
+    const int kg = wave >> 2;  // steps 4 kg .. 4 kg + 3 of every block
+    const size_t tt = blockIdx.y;
+    const size_t row0 = (size_t)blockIdx.x * I8_WROWS;
+    const int split = blockIdx.z;
+    const size_t b0 = (size_t)split * p.blocks_per_split;
+    size_t b1 = b0 + p.blocks_per_split;
+    if (b1 > p.nb) {
+        b1 = p.nb;
+    }
+    const int nrounds = (int)(b1 - b0);
+    const int j = lane & 31, kh = lane >> 5;
+
+    float total[2][16];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            total[a][r] = 0.0f;
+        }
+    }
+
+    // ---- loads per round: 16 activation instructions (two per wavefront), one gather of the 64 block scales
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
+    uint32_t a_voff[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const uint32_t t = (uint32_t)(8 * wave + 4 * c + (lane >> 4));
+        const uint32_t slot = (uint32_t)(lane & 15);
+        const uint32_t trow = t < last_tok ? t : last_tok;
+        a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
+    }
+    const uint32_t d_voff = (uint32_t)(((uint32_t)lane < last_tok ? (uint32_t)lane : last_tok) * 4u * p.nb);
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
+    size_t wr = row0 + (size_t)(32 * rg + j);
+    wr = wr < p.M ? wr : p.M - 1;  // rows beyond M re-read row M - 1 (never stored)
+    const uint8_t *wrow = p.w + wr * (p.nb * BB) + b0 * BB;
+    auto issue = [&](int ri, Q23Raw<KIND> &raw) {
+        const size_t b = b0 + (size_t)ri;
+        const uint32_t s0 = lds_base + (uint32_t)((ri & 1) * I23_STAGE);
+        const uint8_t *qb = tile_q + b * QK_K;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            dma_set_lds_base(s0 + (uint32_t)(2048 * wave + 1024 * c));
+            dma16_to_lds<0>(qb, a_voff[c]);
+        }
+        if (wave == 0) {
+            dma_set_lds_base(s0 + (uint32_t)I8_STAGE_A);
+            dma4_to_lds(tile_d + b * 4, d_voff);
+        }
+        raw.fetch(wrow + (size_t)ri * BB, kg, kh);
+    };
+
+    const uint32_t a_base = (uint32_t)(j * QK_K);
+    const uint32_t d_off = (uint32_t)(I8_STAGE_A + 16 * kh);
+    Q23Raw<KIND> cur, nxt;
+    issue(0, cur);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    i8_lds_barrier();
+    for (int ri = 0; ri < nrounds; ++ri) {
+        if (ri + 1 < nrounds) {
+            issue(ri + 1, nxt);  // into the other buffer, which the barrier that closed the previous round has released
+        }
+        {
+            const uint8_t *stage = lds + (size_t)(ri & 1) * I23_STAGE;
+            i8_intx16 c1[2], c2[2];
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    c1[a][r] = 0;
+                    c2[a][r] = 0;
+                }
+            }
+            const uint32_t qw[4] = {cur.q.x, cur.q.y, cur.q.z, cur.q.w};
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi) {
+                const int step = 4 * kg + bi;
+                i8_intx4 w1, w2;
+                if constexpr (Q2) {
+                    const uint32_t scb = ((bi < 2 ? cur.sc.x : cur.sc.y) >> (8 * (2 * (bi & 1) + kh))) & 0xffu;
+                    const uint32_t dsc = scb & 0xfu, mn = scb >> 4;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        w1[e] = (int)(((qw[e] >> (2 * bi)) & 0x03030303u) * dsc);
+                        w2[e] = (int)(mn * 0x01010101u);
+                    }
+                } else {
+                    // q3k_group_scale(scales, is) for group is = 2 step + kh, plus 32: low nibble from scales[is]
+                    // (is < 8) or the high nibble of scales[is - 8], two more bits from scales[8 + is % 4]
+                    const int is = 2 * step + kh;
+                    const uint64_t low8 = (uint64_t)cur.t0 | ((uint64_t)cur.t1 << 32);
+                    const uint32_t low = (uint32_t)(low8 >> (8 * (is & 7) + (is < 8 ? 0 : 4))) & 0xfu;
+                    const uint32_t high = (cur.t2 >> (8 * (is & 3) + 2 * (is >> 2))) & 3u;
+                    const uint32_t sp = low | (high << 4);              // scale + 32: 0 .. 63
+                    const uint32_t sbyte = (sp - 32u) & 0xffu;          // the scale as a signed byte
+                    const uint32_t bias = (uint32_t)((96 - 2 * (int)sp) * 0x01010101);
+                    const uint32_t hw[4] = {cur.hm.x, cur.hm.y, cur.hm.z, cur.hm.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t q2 = (qw[e] >> (2 * bi)) & 0x03030303u;
+                        const uint32_t hb = (hw[e] >> step) & 0x01010101u;
+                        const uint32_t uh = ((q2 >> 1) & 0x01010101u) | (hb << 1);  // (q3 + 4) / 2: 0 .. 3
+                        // vh * s + 128 = uh * sp + 32 (3 - uh) + 96 - 2 sp with vh = uh - 2, s = sp - 32: every partial
+                        // sum stays inside 0 .. 255 in every byte
+                        const uint32_t biased = uh * sp + ((uh ^ 0x03030303u) << 5) + bias;
+                        w1[e] = (int)(biased ^ 0x80808080u);
+                        w2[e] = (int)((q2 & 0x01010101u) * sbyte);
+                    }
+                }
+#pragma unroll
+                for (int a = 0; a < 2; ++a) {
+                    const i8_intx4 av = *(const i8_intx4 *)(stage + a_base + a * (32 * QK_K) +
+                                                           16 * ((2 * step + kh) ^ (j & 15)));
+                    c1[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, w1, c1[a], 0, 0, 0);
+                    c2[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, w2, c2[a], 0, 0, 0);
+                }
+            }
+            float dw, dmw = 0.0f;
+            if constexpr (Q2) {
+                dw = h2f((uint16_t)(cur.dd & 0xffffu));
+                dmw = h2f((uint16_t)(cur.dd >> 16));
+                asm volatile("" : "+v"(dmw));
+            } else {
+                dw = h2f(cur.d);
+            }
+            asm volatile("" : "+v"(dw));  // conversions of their own (not folded into mixed-precision multiplies)
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const float4 d4 = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * q4));
+                    const float da[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = 4 * q4 + e;
+                        if constexpr (Q2) {
+                            float t = __builtin_fmaf(da[e] * dw, (float)c1[a][r], total[a][r]);
+                            total[a][r] = __builtin_fmaf(-(da[e] * dmw), (float)c2[a][r], t);
+                        } else {
+                            total[a][r] = __builtin_fmaf(da[e] * dw, (float)(2 * c1[a][r] + c2[a][r]), total[a][r]);
+                        }
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the next round's activations and this lane's weights are here
+        i8_lds_barrier();
+        if (ri + 1 < nrounds) {
+            cur = nxt;
+        }
+    }
+    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+}
+
 // ------------------------------------------------------------------ host side
 // From this many activation rows on (more than one 32-row pass of the streaming small-batch kernel) the tile kernel
 // is the faster one on every shape measured (4096 x 4096, 14336 x 4096, 4096 x 14336; e.g. 4096 x 14336 at 48 rows
@@ -1375,14 +1587,23 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
 // eight the packed matvec streams the weights once; measured at 4096 x 4096 / 14336 x 4096: the matvec takes 16.6 /
 // 33 us at 9 rows and 34 / 74 us at 32, this kernel 16 / 30 us at 33)
 constexpr size_t Q80_MIN_ROWS = 9;
-bool gemm_q80_kind(int kind) {
+static bool q80_format(int kind) {
     return kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q4_1 ||
            kind == MARMOT_HIP_KIND_Q5_0 || kind == MARMOT_HIP_KIND_Q5_1;
+}
+static bool q23k_format(int kind) {
+    return kind == MARMOT_HIP_KIND_Q2_K || kind == MARMOT_HIP_KIND_Q3_K;
+}
+bool gemm_q80_kind(int kind) {
+    return q80_format(kind) || q23k_format(kind);
 }
 
 bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                       const ActScratch &act) {
-    if (dev->knobs.no_gemm_i8 || N < Q80_MIN_ROWS || K % QK_K != 0 || !gemm_q80_kind(kind)) {
+    if (q23k_format(kind)) {
+        return gemm_q23k_applies(dev, kind, N, K, weights, count, act);
+    }
+    if (dev->knobs.no_gemm_i8 || N < Q80_MIN_ROWS || K % QK_K != 0 || !q80_format(kind)) {
         return false;
     }
     const size_t chunk = 8 * block_bytes(kind);
@@ -1408,6 +1629,9 @@ static int launch_gemm_q80_kind(marmot_hip_device *dev, const GemmI8Params &p, d
 
 int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                     size_t M, int out_dtype, void *scratch) {
+    if (q23k_format(kind)) {
+        return launch_gemm_q23k(dev, kind, ws, act, N, K, M, out_dtype, scratch);
+    }
     const size_t nb = K / QK_K;
     size_t bps = 0;
     const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
@@ -1464,6 +1688,69 @@ int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const
                      : kind == MARMOT_HIP_KIND_Q4_1 ? 2
                      : kind == MARMOT_HIP_KIND_Q5_0 ? 3
                                                     : 4]);
+    return MARMOT_HIP_SUCCESS;
+}
+
+// Q2_K / Q3_K weights on Q8_K activations, nine activation rows and more (up to eight the packed matvec streams the
+// weights once)
+bool gemm_q23k_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
+                       const ActScratch &act) {
+    if (dev->knobs.no_gemm_i8 || N < Q80_MIN_ROWS || K % QK_K != 0 ||
+        (kind != MARMOT_HIP_KIND_Q2_K && kind != MARMOT_HIP_KIND_Q3_K)) {
+        return false;
+    }
+    if ((((uintptr_t)act.qs) & 15) != 0 || act.kp % 16 != 0 || N * act.kp >= ((size_t)1 << 32) ||
+        N * (K / QK_K) * 4 >= ((size_t)1 << 32)) {
+        return false;  // 16-byte direct-to-LDS loads with 32-bit lane offsets
+    }
+    for (int i = 0; i < count; ++i) {
+        if ((((uintptr_t)weights[i]) & 3) != 0) {
+            return false;
+        }
+    }
+    return true;
+}
+
+int launch_gemm_q23k(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
+                     size_t M, int out_dtype, void *scratch) {
+    const bool q2 = kind == MARMOT_HIP_KIND_Q2_K;
+    const size_t nb = K / QK_K;
+    size_t bps = 0;
+    const size_t splits = gemm_i8_splits(dev, N, M, nb, &bps);
+    float *partial = (float *)scratch;
+    if (splits > 1 && partial == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "tiled Q2_K / Q3_K GEMM: no room for the K-split partial sums");
+    }
+    const dim3 grid((unsigned)((M + I8_WROWS - 1) / I8_WROWS), (unsigned)((N + I8_TOK - 1) / I8_TOK), (unsigned)splits);
+    for (int which = 0; which < ws.count; ++which) {
+        GemmI8Params p;
+        p.w = (const uint8_t *)ws.w[which];
+        p.qs = act.qs;
+        p.ad = act.d;
+        p.kp = act.kp;
+        p.N = N;
+        p.M = M;
+        p.nb = nb;
+        float *part = splits > 1 ? partial + (size_t)which * splits * N * M : nullptr;
+        p.out = splits > 1 ? (void *)part : ws.out[which];
+        p.splits = (int)splits;
+        p.blocks_per_split = (int)bps;
+        p.bias = ws.bias[which];
+        p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
+        p.bias_first = ws.bias_first ? 1 : 0;
+        p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
+        if (q2) {
+            hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q2_K>), grid, dim3(I8_THREADS), I23_LDS_BYTES, dev->stream, p);
+        } else {
+            hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q3_K>), grid, dim3(I8_THREADS), I23_LDS_BYTES, dev->stream, p);
+        }
+        MH_HIP(hipGetLastError());
+        if (splits > 1) {
+            MH_TRY(launch_splitk_reduce(dev, part, (int)splits, N, M, ws.bias[which], ws.bias_dtype, ws.out[which],
+                                        out_dtype, ws.bias_first));
+        }
+    }
+    set_route(q2 ? "gemm_q2_k_q8_k_mfma_tile" : "gemm_q3_k_q8_k_mfma_tile");
     return MARMOT_HIP_SUCCESS;
 }
 

@@ -526,6 +526,63 @@ def test_tiled_int8_gemm_32_value_formats_random_blocks_routes_and_epilogues(hip
     assert_matmul_parity(pre, oracle.matmul(kind, w3, x3, m3, bias=b3), what=f"{name} prepacked, K split")
 
 
+Q23K_KINDS = {"q2_k": 7, "q3_k": 8}
+
+
+@pytest.mark.parametrize("N,M,K", [(9, 70, 256), (33, 96, 512), (40, 4096, 1024), (64, 100, 512), (100, 203, 2048),
+                                   (130, 300, 1024), (64, 128, 4096), (192, 64, 7168), (512, 512, 4096)])
+@pytest.mark.parametrize("name", ["q2_k", "q3_k"])
+def test_tiled_int8_gemm_q2k_q3k_match_oracle(hip, oracle, name, N, M, K):
+    """Prefill with fp32 activations for Q2_K / Q3_K weights (activations packed to Q8_K): group scales multiplied into
+    the int8 operands, two chains of matrix instructions per block (Q2_K: scaled values and group minima; Q3_K: the
+    value split into a signed high part and a low bit), cpu_vec_dot_q2_k_q8_k / cpu_vec_dot_q3_k_q8_k
+    (vec_dot_impl.h:560-687). Full and ragged tiles, one to 28 blocks, K split across workgroups, bias."""
+    kind = Q23K_KINDS[name]
+    blocks = oracle.quantize(kind, gaussian(460 + N, (M, K), 0.02))
+    x = gaussian(461 + N, (N, K))
+    bias = gaussian(462, (M,))
+    got = hip.linear(x, blocks, kind, M, bias=bias)
+    assert hip.last_route() == f"gemm_{name}_q8_k_mfma_tile"
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x, M, bias=bias), what=f"{name} tile {M}x{K} N={N}")
+
+
+@pytest.mark.parametrize("name", ["q2_k", "q3_k"])
+def test_tiled_int8_gemm_q2k_q3k_random_blocks_and_routes(hip, oracle, monkeypatch, name):
+    """Arbitrary block bytes (every two-bit value, mask bit, group scale and minimum, Q3_K's scale -32 with value -4
+    included: their product, +128, does not fit a signed byte) against the oracle and against the packed matvec of a
+    device object created with MARMOT_HIP_NO_GEMM_I8; fewer than nine rows stay on the matvec; the dual call equals two
+    single calls bit for bit."""
+    from marmot_amd import HipBackend
+
+    kind = Q23K_KINDS[name]
+    N, M, K = 96, 160, 1536
+    blocks = random_valid_blocks(np.random.default_rng(470), kind, M, K)
+    x = gaussian(471, (N, K))
+    ref = oracle.matmul(kind, blocks, x, M)
+    tiled = hip.linear(x, blocks, kind, M)
+    assert hip.last_route() == f"gemm_{name}_q8_k_mfma_tile"
+    assert_matmul_parity(tiled, ref, what="tile, random blocks")
+    monkeypatch.setenv("MARMOT_HIP_NO_GEMM_I8", "1")
+    plain = HipBackend(0)
+    monkeypatch.delenv("MARMOT_HIP_NO_GEMM_I8")
+    try:
+        got = plain.linear(x, blocks, kind, M)
+        assert plain.last_route() == f"matvec_{name}_q8_k"
+        assert_matmul_parity(got, ref, what="matvec, random blocks")
+        assert_matmul_parity(tiled, got, what="tile against matvec")
+    finally:
+        plain.close()
+    x8 = gaussian(472, (8, K))
+    got = hip.linear(x8, blocks, kind, M)
+    assert hip.last_route() == f"matvec_{name}_q8_k", hip.last_route()
+    assert_matmul_parity(got, oracle.matmul(kind, blocks, x8, M), what=f"{name} N=8")
+    other = random_valid_blocks(np.random.default_rng(473), kind, M, K)
+    a, b = hip.linear_dual(x, blocks, other, kind, M)
+    assert hip.last_route() == f"gemm_{name}_q8_k_mfma_tile"
+    assert np.array_equal(bits(a), bits(tiled))
+    assert np.array_equal(bits(b), bits(hip.linear(x, other, kind, M)))
+
+
 @pytest.mark.parametrize("name", ["q8_0", "q4_0", "q5_0"])
 def test_tiled_int8_gemm_32_value_formats_integers_are_exact(hip, name):
     """Packed activations and weight blocks whose scales are powers of two: the integer dot, its conversion and the

@@ -57,7 +57,8 @@ constexpr int I8_STAGE = I8_STAGE_A + I8_STAGE_W + I8_STAGE_D;   // one block of
 constexpr int I8_ROUND = 2 * I8_STAGE;                // a round is two consecutive blocks, one per K group
 constexpr int I8_LDS_BYTES = 2 * I8_ROUND;            // the round in work and the round in flight: 140,288
 constexpr int I8_OUT_PITCH = I8_WROWS + 4;            // floats per token of the output tile in LDS
-static_assert(I8_TOK * I8_OUT_PITCH * 4 <= I8_LDS_BYTES, "the output tile reuses the stages");
+constexpr int I8_OUT_TILE_BYTES = I8_TOK * I8_OUT_PITCH * 4;   // the output tile, which reuses the stages
+static_assert(I8_OUT_TILE_BYTES <= I8_LDS_BYTES, "the output tile reuses the stages");
 static_assert(I8_STAGE % 16 == 0, "stages keep 16-byte alignment");
 
 __device__ __forceinline__ void i8_lds_barrier() {
@@ -78,13 +79,15 @@ __device__ __forceinline__ int i8_scale_bytes(uint32_t nib, uint32_t s16) {
 // The two K groups of a workgroup meet in LDS as one [token][weight row] tile, then every thread stores 16 bytes per
 // step. Lane (j, kh) of wavefront (rg, kg) holds weight row 32 rg + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4. Every
 // wavefront of the workgroup calls this after its last read of the stages (the function contains barriers).
-__device__ __forceinline__ void i8_merge_and_store(const GemmI8Params &p, uint8_t *lds, const float (&total)[2][16],
+// NA: token tiles of 32 per workgroup (2, or 1 in the kernels that have a form for at most 32 activation rows).
+template <int NA>
+__device__ __forceinline__ void i8_merge_and_store(const GemmI8Params &p, uint8_t *lds, const float (&total)[NA][16],
                                                    int tid, int rg, int kg, int j, int kh, size_t tt, size_t row0,
                                                    int split) {
     float *tile = (float *)lds;
     if (kg == 1) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < NA; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j] = total[a][r];
@@ -94,7 +97,7 @@ __device__ __forceinline__ void i8_merge_and_store(const GemmI8Params &p, uint8_
     i8_lds_barrier();
     if (kg == 0) {
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < NA; ++a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * I8_OUT_PITCH + 32 * rg + j;
@@ -109,9 +112,9 @@ __device__ __forceinline__ void i8_merge_and_store(const GemmI8Params &p, uint8_
     const bool out_f16 = !partials && p.out_is_f16;
     float *const out32 = (float *)p.out + (partials ? (size_t)split * p.N * p.M : 0);
     const bool vec = (p.M & 3) == 0 && (((uintptr_t)p.out) & 15) == 0;
-    for (int idx = tid; idx < I8_TOK * I8_WROWS / 4; idx += I8_THREADS) {
+    for (int idx = tid; idx < 32 * NA * I8_WROWS / 4; idx += I8_THREADS) {
         const int t = idx >> 5, q4 = idx & 31;  // rows 4 q4 .. 4 q4 + 3 of token t
-        const size_t n = tt * I8_TOK + (size_t)t;
+        const size_t n = tt * (32 * NA) + (size_t)t;
         const size_t m4 = row0 + 4 * (size_t)q4;
         if (n >= p.N || m4 >= p.M) {
             continue;
@@ -435,7 +438,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q4k_q8k_tile(const GemmI8Pa
         i8_lds_barrier();
     }
 
-    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+    i8_merge_and_store<2>(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
 // ------------------------------------------------------------------ Q5_K x Q8_K
@@ -763,7 +766,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q5k_q8k_tile(const GemmI8Pa
         i8_lds_barrier();
     }
 
-    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+    i8_merge_and_store<2>(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
 // ------------------------------------------------------------------ Q6_K x Q8_K
@@ -783,7 +786,7 @@ constexpr int I6_ROWB = 240;
 constexpr int I6_STAGE_W = I8_WROWS * I6_ROWB;                     // 30,720
 constexpr int I6_STAGE = I6_STAGE_W + I8_STAGE_A + I8_STAGE_D;     // 47,360
 constexpr int I6_LDS_BYTES = 2 * I6_STAGE;                         // 94,720
-static_assert(I8_TOK * I8_OUT_PITCH * 4 <= I6_LDS_BYTES, "the output tile reuses the stages");
+static_assert(I8_OUT_TILE_BYTES <= I6_LDS_BYTES, "the output tile reuses the stages");
 static_assert(I6_STAGE % 16 == 0, "stages keep 16-byte alignment");
 
 __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Params p) {
@@ -1013,7 +1016,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q6k_q8k_tile(const GemmI8Pa
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's share of the next block has landed
         i8_lds_barrier();
     }
-    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+    i8_merge_and_store<2>(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
 // ------------------------------------------------------------------ the 32-value formats x Q8_0
@@ -1053,13 +1056,14 @@ struct Q80Tile {
     static constexpr int W_PER_WAVE = (W_INSTR + I8_WAVES - 1) / I8_WAVES;
     static_assert(CHUNK % 16 == 0 && STAGE % 16 == 0, "16-byte pieces");
     static_assert(PITCH_P >= PIECES, "a row's pieces fit its pitch");
-    static_assert(I8_TOK * I8_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
+    static_assert(I8_OUT_TILE_BYTES <= LDS_BYTES, "the output tile reuses the stages");
 };
 
 // p.nb counts rounds (K / 256); p.ad holds 8 p.nb scales per token
-template <int KIND>
+template <int KIND, int NA>
 __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params p) {
     using T = Q80Tile<KIND>;
+    constexpr int TOK = 32 * NA;  // tokens per workgroup: 64, or 32 for at most 32 activation rows
     warm_kernel_arguments<sizeof(GemmI8Params)>();
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
@@ -1078,9 +1082,9 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
     const int nrounds = (int)(b1 - b0);
     const int j = lane & 31, kh = lane >> 5;
 
-    float total[2][16];
+    float total[NA][16];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < NA; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             total[a][r] = 0.0f;
@@ -1090,12 +1094,12 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
     // ---- loads per round: 16 activation instructions (two per wavefront), W_INSTR weight instructions of 64 piece
     // slots (wavefront w takes instructions w, w + 8, ...), one gather of 64 activation scales per wavefront
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
-    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);
-    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
-    uint32_t a_voff[2];
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * TOK);
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * TOK * p.kp;
+    uint32_t a_voff[NA];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const uint32_t t = (uint32_t)(8 * wave + 4 * c + (lane >> 4));
+    for (int c = 0; c < NA; ++c) {
+        const uint32_t t = (uint32_t)(4 * NA * wave + 4 * c + (lane >> 4));
         const uint32_t slot = (uint32_t)(lane & 15);
         const uint32_t trow = t < last_tok ? t : last_tok;
         a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
@@ -1119,16 +1123,16 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
         const uint32_t trow = t < last_tok ? t : last_tok;
         d_voff = (uint32_t)((trow * 8u * p.nb + (uint32_t)wave) * 4u);  // block `wave` of the round, token `lane`
     }
-    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * 8u * p.nb);
-    const uint8_t *tile_s = (const uint8_t *)(p.sums + tt * I8_TOK * 8u * p.nb);
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * TOK * 8u * p.nb);
+    const uint8_t *tile_s = (const uint8_t *)(p.sums + tt * TOK * 8u * p.nb);
     const uint32_t s_voff = (uint32_t)(((uint32_t)lane < last_tok ? (uint32_t)lane : last_tok) * 16u * p.nb);
     auto issue = [&](int ri) {
         const size_t b = b0 + (size_t)ri;
         const uint32_t s0 = lds_base + (uint32_t)((ri & 1) * T::STAGE);
         const uint8_t *qb = tile_q + b * QK_K;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            dma_set_lds_base(s0 + (uint32_t)(T::STAGE_W + 2048 * wave + 1024 * c));
+        for (int c = 0; c < NA; ++c) {
+            dma_set_lds_base(s0 + (uint32_t)(T::STAGE_W + 1024 * NA * wave + 1024 * c));
             dma16_to_lds<0>(qb, a_voff[c]);
         }
         const uint8_t *wb = wbase + b * T::CHUNK;
@@ -1223,7 +1227,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
                     }
                 }
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
+                for (int a = 0; a < NA; ++a) {
                     const i8_intx4 av = *(const i8_intx4 *)(stage + a_base + a * (32 * QK_K) +
                                                            16 * ((2 * blk + kh) ^ (j & 15)));
                     const i8_intx16 dq = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, wv, zero, 0, 0, 0);
@@ -1264,7 +1268,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
             fold_sums(ri + 1);
         }
     }
-    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+    i8_merge_and_store<NA>(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
 // ------------------------------------------------------------------ Q2_K / Q3_K x Q8_K
@@ -1283,7 +1287,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q80_tile(const GemmI8Params
 // (16 + 8 + 4 bytes per block for Q2_K, 16 + 16 + 12 + 2 for Q3_K), requested a round ahead into registers; rows of
 // 84 / 110 bytes need only 4- / 2-byte alignment.
 constexpr int I23_STAGE = I8_STAGE_A + I8_STAGE_D;  // 64 tokens x 256 codes + 64 block scales: 16,640 bytes
-constexpr int I23_LDS_BYTES = (I8_TOK * I8_OUT_PITCH * 4 > 2 * I23_STAGE) ? I8_TOK * I8_OUT_PITCH * 4 : 2 * I23_STAGE;
+constexpr int I23_LDS_BYTES = (I8_OUT_TILE_BYTES > 2 * I23_STAGE) ? I8_OUT_TILE_BYTES : 2 * I23_STAGE;
 
 template <int KIND>
 struct Q23Raw;
@@ -1313,8 +1317,9 @@ struct Q23Raw<MARMOT_HIP_KIND_Q3_K> {
     }
 };
 
-template <int KIND>
+template <int KIND, int NA>
 __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Params p) {
+    constexpr int TOK = 32 * NA;  // tokens per workgroup: 64, or 32 for at most 32 activation rows
     constexpr bool Q2 = KIND == MARMOT_HIP_KIND_Q2_K;
     constexpr int BB = Q2 ? Q2_K_BYTES : Q3_K_BYTES;
     warm_kernel_arguments<sizeof(GemmI8Params)>();
@@ -1335,9 +1340,9 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
     const int nrounds = (int)(b1 - b0);
     const int j = lane & 31, kh = lane >> 5;
 
-    float total[2][16];
+    float total[NA][16];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < NA; ++a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             total[a][r] = 0.0f;
@@ -1346,18 +1351,18 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
 
     // ---- loads per round: 16 activation instructions (two per wavefront), one gather of the 64 block scales
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_u8_t *)lds;
-    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * I8_TOK);
-    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * I8_TOK * p.kp;
-    uint32_t a_voff[2];
+    const uint32_t last_tok = (uint32_t)(p.N - 1 - tt * TOK);
+    const uint8_t *tile_q = (const uint8_t *)p.qs + tt * TOK * p.kp;
+    uint32_t a_voff[NA];
 #pragma unroll
-    for (int c = 0; c < 2; ++c) {
-        const uint32_t t = (uint32_t)(8 * wave + 4 * c + (lane >> 4));
+    for (int c = 0; c < NA; ++c) {
+        const uint32_t t = (uint32_t)(4 * NA * wave + 4 * c + (lane >> 4));
         const uint32_t slot = (uint32_t)(lane & 15);
         const uint32_t trow = t < last_tok ? t : last_tok;
         a_voff[c] = trow * (uint32_t)p.kp + 16u * (slot ^ (t & 15u));
     }
     const uint32_t d_voff = (uint32_t)(((uint32_t)lane < last_tok ? (uint32_t)lane : last_tok) * 4u * p.nb);
-    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * I8_TOK * p.nb);
+    const uint8_t *tile_d = (const uint8_t *)(p.ad + tt * TOK * p.nb);
     size_t wr = row0 + (size_t)(32 * rg + j);
     wr = wr < p.M ? wr : p.M - 1;  // rows beyond M re-read row M - 1 (never stored)
     const uint8_t *wrow = p.w + wr * (p.nb * BB) + b0 * BB;
@@ -1366,8 +1371,8 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
         const uint32_t s0 = lds_base + (uint32_t)((ri & 1) * I23_STAGE);
         const uint8_t *qb = tile_q + b * QK_K;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            dma_set_lds_base(s0 + (uint32_t)(2048 * wave + 1024 * c));
+        for (int c = 0; c < NA; ++c) {
+            dma_set_lds_base(s0 + (uint32_t)(1024 * NA * wave + 1024 * c));
             dma16_to_lds<0>(qb, a_voff[c]);
         }
         if (wave == 0) {
@@ -1389,9 +1394,9 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
         }
         {
             const uint8_t *stage = lds + (size_t)(ri & 1) * I23_STAGE;
-            i8_intx16 c1[2], c2[2];
+            i8_intx16 c1[NA], c2[NA];
 #pragma unroll
-            for (int a = 0; a < 2; ++a) {
+            for (int a = 0; a < NA; ++a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     c1[a][r] = 0;
@@ -1435,7 +1440,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
                     }
                 }
 #pragma unroll
-                for (int a = 0; a < 2; ++a) {
+                for (int a = 0; a < NA; ++a) {
                     const i8_intx4 av = *(const i8_intx4 *)(stage + a_base + a * (32 * QK_K) +
                                                            16 * ((2 * step + kh) ^ (j & 15)));
                     c1[a] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, w1, c1[a], 0, 0, 0);
@@ -1452,7 +1457,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
             }
             asm volatile("" : "+v"(dw));  // conversions of their own (not folded into mixed-precision multiplies)
 #pragma unroll
-            for (int a = 0; a < 2; ++a) {
+            for (int a = 0; a < NA; ++a) {
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
                     const float4 d4 = *(const float4 *)(stage + d_off + 4 * (32 * a + 8 * q4));
@@ -1476,7 +1481,7 @@ __global__ __launch_bounds__(I8_THREADS) void k_gemm_q23k_tile(const GemmI8Param
             cur = nxt;
         }
     }
-    i8_merge_and_store(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
+    i8_merge_and_store<NA>(p, lds, total, tid, rg, kg, j, kh, tt, row0, split);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1620,10 +1625,17 @@ bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K
     return true;
 }
 
+// at most 32 activation rows: the form with one token tile of 32 per workgroup (half the matrix instructions and
+// epilogue of the 64-token form, whose second tile would hold no token)
 template <int KIND>
 static int launch_gemm_q80_kind(marmot_hip_device *dev, const GemmI8Params &p, dim3 grid) {
-    MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<KIND>));
-    hipLaunchKernelGGL((k_gemm_q80_tile<KIND>), grid, dim3(I8_THREADS), Q80Tile<KIND>::LDS_BYTES, dev->stream, p);
+    if (p.N <= 32) {
+        MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<KIND, 1>));
+        hipLaunchKernelGGL((k_gemm_q80_tile<KIND, 1>), grid, dim3(I8_THREADS), Q80Tile<KIND>::LDS_BYTES, dev->stream, p);
+    } else {
+        MH_TRY(allow_large_lds(dev, (const void *)k_gemm_q80_tile<KIND, 2>));
+        hipLaunchKernelGGL((k_gemm_q80_tile<KIND, 2>), grid, dim3(I8_THREADS), Q80Tile<KIND>::LDS_BYTES, dev->stream, p);
+    }
     return MARMOT_HIP_SUCCESS;
 }
 
@@ -1739,10 +1751,20 @@ int launch_gemm_q23k(marmot_hip_device *dev, int kind, const WeightSet &ws, cons
         p.bias_is_f16 = ws.bias_dtype == MARMOT_HIP_DTYPE_F16;
         p.bias_first = ws.bias_first ? 1 : 0;
         p.out_is_f16 = out_dtype == MARMOT_HIP_DTYPE_F16;
-        if (q2) {
-            hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q2_K>), grid, dim3(I8_THREADS), I23_LDS_BYTES, dev->stream, p);
+        if (N <= 32) {  // one token tile of 32 per workgroup
+            if (q2) {
+                hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q2_K, 1>), grid, dim3(I8_THREADS), I23_LDS_BYTES,
+                                   dev->stream, p);
+            } else {
+                hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q3_K, 1>), grid, dim3(I8_THREADS), I23_LDS_BYTES,
+                                   dev->stream, p);
+            }
+        } else if (q2) {
+            hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q2_K, 2>), grid, dim3(I8_THREADS), I23_LDS_BYTES,
+                               dev->stream, p);
         } else {
-            hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q3_K>), grid, dim3(I8_THREADS), I23_LDS_BYTES, dev->stream, p);
+            hipLaunchKernelGGL((k_gemm_q23k_tile<MARMOT_HIP_KIND_Q3_K, 2>), grid, dim3(I8_THREADS), I23_LDS_BYTES,
+                               dev->stream, p);
         }
         MH_HIP(hipGetLastError());
         if (splits > 1) {

@@ -444,7 +444,8 @@ def test_tiled_int8_gemm_q6k_random_blocks_and_exact_integers(hip, oracle):
 Q80_KINDS = {"q8_0": 5, "q4_0": 1, "q4_1": 2, "q5_0": 3, "q5_1": 4}
 
 
-@pytest.mark.parametrize("N,M,K", [(9, 70, 256), (33, 96, 512), (40, 4096, 1024), (48, 128, 256), (64, 100, 512),
+@pytest.mark.parametrize("N,M,K", [(9, 70, 256), (20, 300, 512), (32, 128, 1024), (33, 96, 512), (40, 4096, 1024),
+                                   (48, 128, 256), (64, 100, 512),
                                    (100, 203, 2048), (130, 300, 1024), (64, 128, 4096), (192, 64, 7168),
                                    (512, 512, 4096)])
 @pytest.mark.parametrize("name", ["q8_0", "q4_0", "q4_1", "q5_0", "q5_1"])
@@ -529,7 +530,8 @@ def test_tiled_int8_gemm_32_value_formats_random_blocks_routes_and_epilogues(hip
 Q23K_KINDS = {"q2_k": 7, "q3_k": 8}
 
 
-@pytest.mark.parametrize("N,M,K", [(9, 70, 256), (33, 96, 512), (40, 4096, 1024), (64, 100, 512), (100, 203, 2048),
+@pytest.mark.parametrize("N,M,K", [(9, 70, 256), (20, 300, 512), (32, 128, 1024), (33, 96, 512), (40, 4096, 1024),
+                                   (64, 100, 512), (100, 203, 2048),
                                    (130, 300, 1024), (64, 128, 4096), (192, 64, 7168), (512, 512, 4096)])
 @pytest.mark.parametrize("name", ["q2_k", "q3_k"])
 def test_tiled_int8_gemm_q2k_q3k_match_oracle(hip, oracle, name, N, M, K):

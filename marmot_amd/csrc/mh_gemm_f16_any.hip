@@ -20,6 +20,8 @@
 // the compute unit's address unit 32 cache lines per instruction and was the bound of the first form, 102 us whatever
 // the format). One barrier per round. K is split across workgroups when the tiles do not fill the chip; the partial
 // sums meet in k_gemm_reduce.
+#include <type_traits>
+
 #include "mh_common.h"
 #include "mh_dequant.h"
 
@@ -75,11 +77,8 @@ struct AnyInt {
     static constexpr int SCALE_ROUNDS = (KIND == MARMOT_HIP_KIND_Q6_K || KIND == MARMOT_HIP_KIND_Q2_K) ? 4
         : KIND == MARMOT_HIP_KIND_Q3_K                                                                 ? 8
                                                                                                        : 1;
-    // bytes of one weight stage: K-step x wavefront x k half x row x 16 bytes + 128 scales (+ 128 offsets)
-    static constexpr int SCALE_OFF = 2 * 4 * 2 * 32 * 16;
-    static constexpr int WSTAGE = SCALE_OFF + 512 + (HAS_MIN ? 512 : 0);
-    static constexpr int LDS_BYTES = 2 * WSTAGE + 2 * FA_XSTAGE;
-    static_assert(FA_TOK * FA_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
+    // LDS: two activation stages; the output tile reuses them
+    static constexpr int LDS_BYTES = 2 * FA_XSTAGE > FA_TOK * FA_OUT_PITCH * 4 ? 2 * FA_XSTAGE : FA_TOK * FA_OUT_PITCH * 4;
 };
 
 // The 16 weights a thread handles per round, in two steps so that the bytes can be requested a round before they are
@@ -314,9 +313,9 @@ __device__ __forceinline__ void fa_barrier() {
 }
 
 template <int KIND>
-__global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyParams p) {
+__global__ __launch_bounds__(FA_THREADS, 2) void k_gemm_any_f16(const GemmAnyParams p) {
     using KT = KindTraits<KIND>;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // 2 weight stages + 2 activation stages (any_lds_bytes)
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // two activation stages; later the output tile
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -331,44 +330,25 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
         r1 = rounds;
     }
 
-    // decode role: row tid / 2 of the tile, values 16 (tid % 2) .. + 15 of the round = K-step tid % 2
-    const int drow = tid >> 1, dks = tid & 1;
-    size_t wr = row0 + (size_t)drow;
+    // Lane (j, kh) of wavefront c owns weight row 32 c + j and, of every round, its values 16 kh .. 16 kh + 15: the
+    // first eight are its share of K-step 0, the other eight of K-step 1 (the activations are read to match). No other
+    // lane needs these bytes, so they come from memory straight into this lane's registers, four rounds ahead, and
+    // the products of row 32 c + j land in this lane's accumulators, where its scale and offset already are.
+    constexpr bool HAS_MIN = AnyInt<KIND>::HAS_MIN;
+    size_t wr = row0 + (size_t)(32 * wave + j);
     wr = wr < p.M ? wr : p.M - 1;  // rows beyond M re-read the last row (never stored)
     const uint8_t *const wrow = p.w + wr * p.row_bytes;
-    // LDS slot of (K-step ks, wavefront c, k half, row j): 16 bytes
-    constexpr bool HAS_MIN = AnyInt<KIND>::HAS_MIN;
-    constexpr int SCALE_OFF = AnyInt<KIND>::SCALE_OFF;  // 128 scales (and 128 offsets) behind the operands of a stage
-    constexpr int WSTAGE = AnyInt<KIND>::WSTAGE;
-    auto slot = [](int ks, int c, int half, int row) -> uint32_t {
-        return (uint32_t)((((ks * 4 + c) * 2 + half) * 32 + row) * 16);
-    };
     auto fetch = [&](size_t round, AnyRaw<KIND> &raw) {
-        const size_t k0 = round * FA_ROUND + (size_t)(16 * dks);
+        const size_t k0 = round * FA_ROUND + (size_t)(16 * kh);
         const size_t b = k0 / KT::BV;
         raw.fetch(wrow + b * KT::BB, (int)(k0 - b * KT::BV));
-    };
-    auto decode = [&](const AnyRaw<KIND> &raw, int stage) {
-        uint32_t h[8];
-        float scale, offset;
-        raw.ints(h, scale, offset);
-        uint8_t *st = lds + (size_t)stage * WSTAGE;
-        const int c = drow >> 5, row = drow & 31;
-        *(uint4 *)(st + slot(dks, c, 0, row)) = make_uint4(h[0], h[1], h[2], h[3]);
-        *(uint4 *)(st + slot(dks, c, 1, row)) = make_uint4(h[4], h[5], h[6], h[7]);
-        if (dks == 0) {
-            *(float *)(st + SCALE_OFF + 4 * drow) = scale;
-            if constexpr (HAS_MIN) {
-                *(float *)(st + SCALE_OFF + 512 + 4 * drow) = offset;
-            }
-        }
     };
 
     // Activations go through LDS in stages of four rounds (128 values of K): 64 tokens x 256 bytes, token t's 16-byte
     // chunk c in slot c ^ (t % 16) (the operand reads of 16 tokens x one chunk then fall into different banks). Every
     // thread brings four chunks per stage, consecutive lanes consecutive chunks of a token's row (16 lanes per token:
     // whole 256-byte runs), a stage ahead, and stores them before the barrier that ends the stage in work.
-    uint8_t *const xlds = lds + 2 * WSTAGE;
+    uint8_t *const xlds = lds;
     const uint16_t *xsrc[4];
     uint32_t xdst[4];
 #pragma unroll
@@ -380,18 +360,24 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
         xsrc[i] = p.x + tok * p.K + (size_t)(8 * c);
         xdst[i] = (uint32_t)(t * 256 + 16 * (c ^ (t & 15)));
     }
-    auto x_request = [&](size_t round, uint4 (&xg)[4]) {  // round: the first of a stage
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            xg[i] = *(const uint4 *)(xsrc[i] + round * FA_ROUND);
-        }
-    };
-    auto x_store = [&](int xstage, const uint4 (&xg)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *(uint4 *)(xlds + (size_t)xstage * FA_XSTAGE + xdst[i]) = xg[i];
-        }
-    };
+    // (macros over four named registers, not lambdas over an array or a struct: handed over by reference, the values
+    // stayed in private memory, and every stage waited for its loads at once to store them there)
+    uint4 xg0, xg1, xg2, xg3;
+#define FA_X_REQUEST(round_)                                         \
+    do {                                                             \
+        xg0 = *(const uint4 *)(xsrc[0] + (round_) * FA_ROUND);       \
+        xg1 = *(const uint4 *)(xsrc[1] + (round_) * FA_ROUND);       \
+        xg2 = *(const uint4 *)(xsrc[2] + (round_) * FA_ROUND);       \
+        xg3 = *(const uint4 *)(xsrc[3] + (round_) * FA_ROUND);       \
+    } while (0)
+#define FA_X_STORE(xstage_)                                          \
+    do {                                                             \
+        uint8_t *st_ = xlds + (size_t)(xstage_) * FA_XSTAGE;         \
+        *(uint4 *)(st_ + xdst[0]) = xg0;                             \
+        *(uint4 *)(st_ + xdst[1]) = xg1;                             \
+        *(uint4 *)(st_ + xdst[2]) = xg2;                             \
+        *(uint4 *)(st_ + xdst[3]) = xg3;                             \
+    } while (0)
 
     fa_floatx16 acc[2];
     fa_floatx16 grp[2];                      // the products of the rounds that share a scale
@@ -408,22 +394,20 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
     const fa_half8 ones = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f,
                            (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
 
-    AnyRaw<KIND> raw[2];
-    auto multiply = [&](size_t round, int stage) {
-        const uint8_t *st = lds + (size_t)stage * WSTAGE;
-        // this round's activations: stage (round / 4) % 2, token 32 a + j, chunk 4 (round % 4) + 2 ks + kh
+    // One round: the lane's 16 integers of the round as the operands of the two K-steps, then (in program order behind
+    // the decode, so the registers are free) the request for the round four later into the same registers, then the
+    // products with the 64 tokens.
+    auto step = [&](size_t round, AnyRaw<KIND> &raw, auto refill) {
+        uint32_t h[8];
+        float scale, offset;
+        raw.ints(h, scale, offset);
+        if constexpr (decltype(refill)::value) {
+            fetch(round + FA_XROUNDS, raw);
+        }
+        // this round's activations: stage (round / 4) % 2, token 32 a + j, chunk 4 (round % 4) + 2 kh + ks
         const size_t rel = round - r0;
         const uint8_t *xs = xlds + (size_t)((rel / FA_XROUNDS) & 1) * FA_XSTAGE;
         const int q = (int)(rel % FA_XROUNDS);
-        fa_half8 x[2][2];
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int a = 0; a < 2; ++a) {
-                x[ks][a] = __builtin_bit_cast(
-                    fa_half8, *(const uint4 *)(xs + (32 * a + j) * 256 + 16 * ((4 * q + 2 * ks + kh) ^ (j & 15))));
-            }
-        }
         constexpr int SR = AnyInt<KIND>::SCALE_ROUNDS;
         const bool opens = SR == 1 || (round % SR) == 0, closes = SR == 1 || (round % SR) == SR - 1;
         if (opens) {
@@ -438,21 +422,18 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
         }
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const fa_half8 wb = __builtin_bit_cast(fa_half8, *(const uint4 *)(st + slot(ks, wave, kh, j)));
+            const fa_half8 wb = __builtin_bit_cast(fa_half8, make_uint4(h[4 * ks], h[4 * ks + 1], h[4 * ks + 2], h[4 * ks + 3]));
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
-                grp[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], wb, grp[a], 0, 0, 0);
+                const fa_half8 x = __builtin_bit_cast(
+                    fa_half8, *(const uint4 *)(xs + (32 * a + j) * 256 + 16 * ((4 * q + 2 * kh + ks) ^ (j & 15))));
+                grp[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, wb, grp[a], 0, 0, 0);
                 if constexpr (HAS_MIN) {
-                    xsum[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks][a], ones, xsum[a], 0, 0, 0);
+                    xsum[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x, ones, xsum[a], 0, 0, 0);
                 }
             }
         }
         if (closes) {
-            const float scale = *(const float *)(st + SCALE_OFF + 4 * (32 * wave + j));
-            float offset = 0.0f;
-            if constexpr (HAS_MIN) {
-                offset = *(const float *)(st + SCALE_OFF + 512 + 4 * (32 * wave + j));
-            }
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
 #pragma unroll
@@ -461,56 +442,46 @@ __global__ __launch_bounds__(FA_THREADS, 3) void k_gemm_any_f16(const GemmAnyPar
                     if constexpr (HAS_MIN) {
                         t = __builtin_fmaf(offset, xsum[a][r], t);
                     }
-                    // keeps the scaling inside its round (an empty statement the optimizer cannot move across the
-                    // barrier): sunk behind the later rounds, every round holds its own 32 product registers
-                    // until the end of the stage, and the four sets spill
+                    // keeps the scaling inside its round (an empty statement the optimizer cannot move): sunk behind
+                    // the later rounds, every round would hold its own 32 product registers until the end of the stage
                     asm volatile("" : "+v"(t));
                     acc[a][r] = t;
                 }
             }
         }
     };
-    // One round: the operands of `round` are in LDS stage `stage`; the weights of round + 1 wait in raw_ready. Requests
-    // round + 2's weights into raw_free (free since the previous round decoded it), decodes round + 1 into the other
-    // stage, multiplies. (Requests three rounds ahead, with four sets of registers, measured the same and spilled.)
-    auto step = [&](size_t round, int stage, AnyRaw<KIND> &raw_free, const AnyRaw<KIND> &raw_ready) {
-        if (round + 2 < r1) {
-            fetch(round + 2, raw_free);
+    AnyRaw<KIND> raw[FA_XROUNDS];
+    if (r0 < r1) {  // (r0 and the number of rounds are multiples of four: the launcher sees to it)
+        FA_X_REQUEST(r0);
+#pragma unroll
+        for (int q = 0; q < FA_XROUNDS; ++q) {
+            fetch(r0 + (size_t)q, raw[q]);
         }
-        if (round + 1 < r1) {
-            decode(raw_ready, stage ^ 1);  // the other stage: the barrier that closed the previous round released it
-        }
-        multiply(round, stage);
-    };
-    uint4 xg[4];
-    if (r0 < r1) {  // (at least four rounds)
-        fetch(r0, raw[0]);
-        x_request(r0, xg);
-        fetch(r0 + 1, raw[1]);
-        decode(raw[0], 0);
-        x_store(0, xg);
+        FA_X_STORE(0);
     }
     fa_barrier();
-    // r0 and the number of rounds are multiples of four (the launcher sees to it): stages of four rounds, two sets of
-    // weight registers that take turns (nothing in flight is ever copied: a copy would wait for the loads it copies)
-    for (size_t round = r0; round < r1; round += FA_XROUNDS) {
-        const bool more = round + FA_XROUNDS < r1;
-        if (more) {
-            x_request(round + FA_XROUNDS, xg);
+    // Every stage but the last requests the next one; the last is peeled off so that the loop body has no branch (a
+    // load behind a branch makes the compiler wait for every load in flight at the next use of any of them).
+    size_t round = r0;
+    for (; round + FA_XROUNDS < r1; round += FA_XROUNDS) {
+        FA_X_REQUEST(round + FA_XROUNDS);
+#pragma unroll
+        for (int q = 0; q < FA_XROUNDS; ++q) {
+            step(round + (size_t)q, raw[q], std::true_type{});
         }
-        step(round, 0, raw[0], raw[1]);
-        fa_barrier();
-        step(round + 1, 1, raw[1], raw[0]);
-        fa_barrier();
-        step(round + 2, 0, raw[0], raw[1]);
-        fa_barrier();
-        step(round + 3, 1, raw[1], raw[0]);
-        if (more) {
-            x_store((int)((((round - r0) / FA_XROUNDS) + 1) & 1), xg);
+        FA_X_STORE((int)((((round - r0) / FA_XROUNDS) + 1) & 1));
+        fa_barrier();  // the stage just read is free for the stage after next; the next stage is complete
+    }
+    if (round < r1) {
+#pragma unroll
+        for (int q = 0; q < FA_XROUNDS; ++q) {
+            step(round + (size_t)q, raw[q], std::false_type{});
         }
         fa_barrier();
     }
 
+#undef FA_X_REQUEST
+#undef FA_X_STORE
     // Lane (j, kh) of wavefront c holds weight row 32 c + j for tokens 32 a + 8 (r / 4) + 4 kh + r % 4: the tile goes
     // through LDS as [token][weight row] (the stages are free behind the loop's last barrier) and every thread stores 16
     // bytes per step (stores of one float per lane cost the address unit as much as these and move a quarter).
@@ -614,12 +585,11 @@ int launch_gemm_f16_any(marmot_hip_device *dev, int kind, const void *d_w, const
     const size_t tiles_n = (N + FA_TOK - 1) / FA_TOK, tiles_m = (M + FA_WROWS - 1) / FA_WROWS;
     const size_t tiles = tiles_n * tiles_m;
     const size_t cus = (size_t)dev->props.multiProcessorCount;
-    // A workgroup's round is a chain of dependent steps (decode, LDS, barrier, LDS, matrix instructions) with one
-    // wavefront per SIMD: three workgroups per compute unit overlap each other's chains (measured at 512 tokens x 4096
-    // rows, Q8_0: one workgroup per compute unit without a K split 134 us, two 93, three 84, four 96). Fewer tiles than
-    // that: split K (at least 16 rounds per workgroup).
+    // Fewer tiles than compute units: split K until the chip is full once (at least 16 rounds per workgroup). More
+    // workgroups per compute unit did not pay (512 tokens x 4096 rows, Q8_0: 58 us without a K split, 67 us with two
+    // resident workgroups per compute unit and the reduction launch they need).
     size_t splits = 1;
-    const size_t want = 3;
+    const size_t want = 1;
     if (tiles < want * cus) {
         splits = (want * cus) / tiles;
         const size_t max_splits = rounds / 16 > 0 ? rounds / 16 : 1;

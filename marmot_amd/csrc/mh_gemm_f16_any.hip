@@ -32,12 +32,14 @@ typedef float fa_floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int FA_TOK = 64;
 constexpr int FA_WROWS = 128;
-constexpr int FA_THREADS = 256;
+constexpr int FA_GROUP = 256;                          // threads of one K group: four wavefronts x 32 rows
+constexpr int FA_THREADS = 2 * FA_GROUP;               // two K groups take alternate stages of the workgroup's rounds
 constexpr int FA_ROUND = 32;                          // values of K per round
 constexpr int FA_XROUNDS = 4;                         // rounds per activation stage (128 values of K)
 constexpr int FA_XSTAGE = FA_TOK * FA_XROUNDS * FA_ROUND * 2;   // 16,384
 constexpr int FA_OUT_PITCH = FA_WROWS + 4;             // floats per token of the output tile in LDS
 constexpr int FA_MIN_TOKENS = 9;
+static_assert(FA_XROUNDS == 4, "the stage loops are written out for four rounds");
 
 struct GemmAnyParams {
     const uint8_t *w;
@@ -73,12 +75,14 @@ struct AnyInt {
     static constexpr bool HAS_MIN = KIND == MARMOT_HIP_KIND_Q4_1 || KIND == MARMOT_HIP_KIND_Q5_1 ||
                                     KIND == MARMOT_HIP_KIND_Q5_K || KIND == MARMOT_HIP_KIND_Q2_K;
     // rounds that share a scale (and an offset): Q6_K and Q2_K as the reference's fp16 dots decode them, 128 values;
-    // Q3_K's six-bit group scales (per 16 values) are multiplied into the integer operand, which leaves d per block
-    static constexpr int SCALE_ROUNDS = (KIND == MARMOT_HIP_KIND_Q6_K || KIND == MARMOT_HIP_KIND_Q2_K) ? 4
-        : KIND == MARMOT_HIP_KIND_Q3_K                                                                 ? 8
-                                                                                                       : 1;
+    // Q3_K's six-bit group scales (per 16 values) are multiplied into the integer operand, which leaves d per block,
+    // applied per stage of four rounds (a K group sees every other stage)
+    static constexpr int SCALE_ROUNDS =
+        (KIND == MARMOT_HIP_KIND_Q6_K || KIND == MARMOT_HIP_KIND_Q2_K || KIND == MARMOT_HIP_KIND_Q3_K) ? 4 : 1;
+    static_assert(SCALE_ROUNDS == 1 || SCALE_ROUNDS == FA_XROUNDS, "a span of rounds is a stage");
     // LDS: two activation stages; the output tile reuses them
-    static constexpr int LDS_BYTES = 2 * FA_XSTAGE > FA_TOK * FA_OUT_PITCH * 4 ? 2 * FA_XSTAGE : FA_TOK * FA_OUT_PITCH * 4;
+    static constexpr int LDS_BYTES = 4 * FA_XSTAGE;  // two activation stages per K group; the output tile reuses them
+    static_assert(FA_TOK * FA_OUT_PITCH * 4 <= LDS_BYTES, "the output tile reuses the stages");
 };
 
 // The 16 weights a thread handles per round, in two steps so that the bytes can be requested a round before they are
@@ -88,17 +92,43 @@ struct AnyInt {
 template <int KIND>
 struct AnyRaw;
 
+// Blocks of 18, 22, 34, 110 and 210 bytes put their fields at addresses that are multiples of 2, not of 4, in every
+// other block, and a vector load from such an address is slow (512 tokens x 4096 x 4096: Q4_0, whose nibbles start 2
+// bytes into an 18-byte block, 57.7 us; Q4_1, whose nibbles start 4 bytes into a 20-byte block, 43.5 us with twice
+// the matrix instructions). Any16 fetches 16 bytes from the multiple of 4 below and brings the last two bytes
+// separately; the bytes are put together when they are used. No byte outside [p - 2, p + 16) is read. (For the 8- and
+// 4-byte fields of Q6_K the second instruction cost more than the misalignment: 59.7 -> 70.5 us.)
+typedef uint32_t any_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+struct Any16 {  // 16 bytes at an even address
+    any_u32x4_a4 d;
+    uint16_t t;
+    uint16_t mis;
+    __device__ __forceinline__ void fetch(const uint8_t *p) {
+        mis = (uint16_t)((uintptr_t)p & 2u);
+        const uint8_t *base = p - mis;
+        d = *(const any_u32x4_a4 *)base;
+        t = *(const uint16_t *)(base + (mis ? 16 : 14));
+    }
+    __device__ __forceinline__ uint4 get() const {
+        const uint32_t sh = 8u * mis;  // 0 or 16
+        return make_uint4(__builtin_amdgcn_alignbit(d.y, d.x, sh), __builtin_amdgcn_alignbit(d.z, d.y, sh),
+                          __builtin_amdgcn_alignbit(d.w, d.z, sh), mis ? (d.w >> 16) | ((uint32_t)t << 16) : d.w);
+    }
+};
 template <>
 struct AnyRaw<MARMOT_HIP_KIND_Q8_0> {
-    uint4 q;
+    Any16 q16;
     uint16_t s;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
+        q16.fetch(b + 2 + v);
+    }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *b, int) {
         __builtin_memcpy(&s, b, 2);
-        __builtin_memcpy(&q, b + 2 + v, 16);
     }
     __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         scale = h2f(s);
         offset = 0.0f;
+        const uint4 q = q16.get();
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -111,8 +141,10 @@ struct AnyRaw<MARMOT_HIP_KIND_Q8_1> {  // scale, the carried sum (unused), 32 co
     uint4 q;
     uint16_t s;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
-        __builtin_memcpy(&s, b, 2);
         __builtin_memcpy(&q, b + 4 + v, 16);
+    }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *b, int) {
+        __builtin_memcpy(&s, b, 2);
     }
     __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         scale = h2f(s);
@@ -129,24 +161,37 @@ struct AnyRaw<MARMOT_HIP_KIND_Q8_1> {  // scale, the carried sum (unused), 32 co
 // keep the fifth bit of value i in bit i of a 32-bit word before qs. HDR: bytes before that word / before qs.
 template <int HDR, bool FIFTH, bool MIN, int CENTRE>
 struct AnyRawNibbles {
-    uint4 q;
-    uint32_t qh;
-    uint16_t s, m;
+    // MIN formats have blocks of 20 / 24 bytes: every field on a multiple of 4, plain vector loads. The others (18 /
+    // 22 bytes) take the nibbles through Any16.
+    Any16 q16;
+    any_u32x4_a4 qa;
+    uint32_t qh, sm;
     int high;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
-        __builtin_memcpy(&s, b, 2);
         if constexpr (MIN) {
-            __builtin_memcpy(&m, b + 2, 2);
+            sm = *(const uint32_t *)b;  // scale, min
+            qa = *(const any_u32x4_a4 *)(b + HDR + (FIFTH ? 4 : 0));
+        } else {
+            uint16_t s;
+            __builtin_memcpy(&s, b, 2);
+            sm = s;
+            q16.fetch(b + HDR + (FIFTH ? 4 : 0));
         }
         if constexpr (FIFTH) {
             __builtin_memcpy(&qh, b + HDR, 4);
         }
-        __builtin_memcpy(&q, b + HDR + (FIFTH ? 4 : 0), 16);
         high = v >= 16;
     }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *, int) {}
     __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
-        scale = h2f(s);
-        offset = MIN ? h2f(m) : 0.0f;
+        scale = h2f((uint16_t)(sm & 0xffffu));
+        offset = MIN ? h2f((uint16_t)(sm >> 16)) : 0.0f;
+        uint4 q;
+        if constexpr (MIN) {
+            q = make_uint4(qa.x, qa.y, qa.z, qa.w);
+        } else {
+            q = q16.get();
+        }
         const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
         const uint32_t hbits = FIFTH ? (high ? qh >> 16 : qh) : 0u;
 #pragma unroll
@@ -170,13 +215,15 @@ struct AnyRaw<MARMOT_HIP_KIND_Q5_1> : AnyRawNibbles<4, true, true, 0> {};     //
 
 template <>
 struct AnyRaw<MARMOT_HIP_KIND_Q6_K> {
-    uint2 ql;
+    uint2 ql;  // (8 and 4 bytes at even addresses: plain loads; one more instruction each cost more than it saved)
     uint32_t qh;
     int8_t sc;
     uint16_t d;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
         __builtin_memcpy(&ql, b + (v >> 1), 8);
         __builtin_memcpy(&qh, b + 128 + (v >> 2), 4);
+    }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *b, int v) {  // one scale per 128 values
         sc = (int8_t)b[192 + (v >> 7)];
         __builtin_memcpy(&d, b + 208, 2);
     }
@@ -221,6 +268,7 @@ struct AnyRaw<MARMOT_HIP_KIND_Q5_K> {
         __builtin_memcpy(&hb, b + 16 + 8 * g + l0 + 32 * (j & 1), 16);
         __builtin_memcpy(&q, b + 48 + 32 * g + l0, 16);
     }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *, int) {}
     __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         // scales[j], scales[j + 4] (j < 4) or scales[j + 4], scales[j - 4], scales[j] (j >= 4): byte j % 4 of a word
         const int sh = 8 * (j & 3);
@@ -246,8 +294,10 @@ struct AnyRaw<MARMOT_HIP_KIND_Q2_K> {
     uint32_t q, dd;
     uint8_t sc;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
-        sc = b[v >> 7];
         __builtin_memcpy(&q, b + 16 + (v >> 2), 4);
+    }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *b, int v) {  // one scale / min pair per 128 values
+        sc = b[v >> 7];
         __builtin_memcpy(&dd, b + 80, 4);
     }
     __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
@@ -267,23 +317,22 @@ struct AnyRaw<MARMOT_HIP_KIND_Q2_K> {
 // The integer operand is value x group scale (at most 128 in magnitude, exact in fp16); d is the block's scale.
 template <>
 struct AnyRaw<MARMOT_HIP_KIND_Q3_K> {
-    uint4 q, hm;
-    uint32_t t0, t1, t2;
-    uint16_t d;
+    Any16 q16, hm16, tail16;  // tail16: the block's last 16 bytes = two bytes of qs, the 12 scale bytes, d
     int v0;
     __device__ __forceinline__ void fetch(const uint8_t *b, int v) {
         v0 = v;
         const int c = v >> 7, li = v & 31;
-        __builtin_memcpy(&hm, b + li, 16);
-        __builtin_memcpy(&q, b + 32 + 32 * c + li, 16);
-        __builtin_memcpy(&t0, b + 96, 4);
-        __builtin_memcpy(&t1, b + 100, 4);
-        __builtin_memcpy(&t2, b + 104, 4);
-        __builtin_memcpy(&d, b + 108, 2);
+        hm16.fetch(b + li);
+        q16.fetch(b + 32 + 32 * c + li);
+        tail16.fetch(b + 94);
     }
+    __device__ __forceinline__ void fetch_scale(const uint8_t *, int) {}
     __device__ __forceinline__ void ints(uint32_t (&h)[8], float &scale, float &offset) const {
         typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-        scale = h2f(d);
+        const uint4 q = q16.get(), hm = hm16.get(), tail = tail16.get();
+        const uint32_t t0 = __builtin_amdgcn_alignbit(tail.y, tail.x, 16), t1 = __builtin_amdgcn_alignbit(tail.z, tail.y, 16),
+                       t2 = __builtin_amdgcn_alignbit(tail.w, tail.z, 16);
+        scale = h2f((uint16_t)(tail.w >> 16));
         offset = 0.0f;
         const int c = v0 >> 7, j = (v0 >> 5) & 3, is = v0 >> 4;
         // q3k_group_scale(scales, is): low nibble from scales[is] (is < 8) or the high nibble of scales[is - 8], two
@@ -313,12 +362,14 @@ __device__ __forceinline__ void fa_barrier() {
 }
 
 template <int KIND>
-__global__ __launch_bounds__(FA_THREADS, 2) void k_gemm_any_f16(const GemmAnyParams p) {
+__global__ __launch_bounds__(FA_THREADS) void k_gemm_any_f16(const GemmAnyParams p) {
     using KT = KindTraits<KIND>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // two activation stages; later the output tile
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane((tid >> 6) & 3);  // rows 32 wave .. + 31 of the tile
+    const int kg = __builtin_amdgcn_readfirstlane(tid >> 8);          // K group: stages kg, kg + 2, ... of the rounds
+    const int gtid = tid & (FA_GROUP - 1);
     const int j = lane & 31, kh = lane >> 5;
     const size_t row0 = (size_t)blockIdx.x * FA_WROWS;
     const size_t tok0 = (size_t)blockIdx.y * FA_TOK;
@@ -338,22 +389,27 @@ __global__ __launch_bounds__(FA_THREADS, 2) void k_gemm_any_f16(const GemmAnyPar
     size_t wr = row0 + (size_t)(32 * wave + j);
     wr = wr < p.M ? wr : p.M - 1;  // rows beyond M re-read the last row (never stored)
     const uint8_t *const wrow = p.w + wr * p.row_bytes;
-    auto fetch = [&](size_t round, AnyRaw<KIND> &raw) {
+    // closes: the round ends a span of rounds that share a scale (the formats with such spans fetch the scale fields
+    // only then; known at compile time: a stage is a span, its last round closes it)
+    auto fetch = [&](size_t round, AnyRaw<KIND> &raw, auto closes) {
         const size_t k0 = round * FA_ROUND + (size_t)(16 * kh);
         const size_t b = k0 / KT::BV;
         raw.fetch(wrow + b * KT::BB, (int)(k0 - b * KT::BV));
+        if constexpr (AnyInt<KIND>::SCALE_ROUNDS == 1 || decltype(closes)::value) {
+            raw.fetch_scale(wrow + b * KT::BB, (int)(k0 - b * KT::BV));
+        }
     };
 
     // Activations go through LDS in stages of four rounds (128 values of K): 64 tokens x 256 bytes, token t's 16-byte
     // chunk c in slot c ^ (t % 16) (the operand reads of 16 tokens x one chunk then fall into different banks). Every
     // thread brings four chunks per stage, consecutive lanes consecutive chunks of a token's row (16 lanes per token:
     // whole 256-byte runs), a stage ahead, and stores them before the barrier that ends the stage in work.
-    uint8_t *const xlds = lds;
+    uint8_t *const xlds = lds + (size_t)kg * 2 * FA_XSTAGE;  // this K group's two stages
     const uint16_t *xsrc[4];
     uint32_t xdst[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int piece = i * FA_THREADS + tid;
+        const int piece = i * FA_GROUP + gtid;
         const int t = piece >> 4, c = piece & 15;
         size_t tok = tok0 + (size_t)t;
         tok = tok < p.N ? tok : p.N - 1;  // tokens beyond N re-read the last one (never stored)
@@ -397,16 +453,16 @@ __global__ __launch_bounds__(FA_THREADS, 2) void k_gemm_any_f16(const GemmAnyPar
     // One round: the lane's 16 integers of the round as the operands of the two K-steps, then (in program order behind
     // the decode, so the registers are free) the request for the round four later into the same registers, then the
     // products with the 64 tokens.
-    auto step = [&](size_t round, AnyRaw<KIND> &raw, auto refill) {
+    auto step = [&](size_t round, AnyRaw<KIND> &raw, auto refill, auto last_of_stage) {
         uint32_t h[8];
         float scale, offset;
         raw.ints(h, scale, offset);
         if constexpr (decltype(refill)::value) {
-            fetch(round + FA_XROUNDS, raw);
+            fetch(round + 2 * FA_XROUNDS, raw, last_of_stage);  // this K group's next stage
         }
-        // this round's activations: stage (round / 4) % 2, token 32 a + j, chunk 4 (round % 4) + 2 kh + ks
+        // this round's activations: the group's stage (round / 8) % 2, token 32 a + j, chunk 4 (round % 4) + 2 kh + ks
         const size_t rel = round - r0;
-        const uint8_t *xs = xlds + (size_t)((rel / FA_XROUNDS) & 1) * FA_XSTAGE;
+        const uint8_t *xs = xlds + (size_t)((rel / (2 * FA_XROUNDS)) & 1) * FA_XSTAGE;
         const int q = (int)(rel % FA_XROUNDS);
         constexpr int SR = AnyInt<KIND>::SCALE_ROUNDS;
         const bool opens = SR == 1 || (round % SR) == 0, closes = SR == 1 || (round % SR) == SR - 1;
@@ -450,34 +506,44 @@ __global__ __launch_bounds__(FA_THREADS, 2) void k_gemm_any_f16(const GemmAnyPar
             }
         }
     };
+    // The workgroup's rounds in stages of four; K group kg takes stages kg, kg + 2, ... (`mine` of them) in its own
+    // pair of LDS stages. Both groups pass the same number of barriers (`iters` after the first one). Every stage of a
+    // group but its last requests the next one; the last is peeled off so that the loop body has no branch (a load
+    // behind a branch makes the compiler wait for every load in flight at the next use of any of them).
+    const size_t nst = (r1 - r0) / FA_XROUNDS;  // (r0 and the number of rounds are multiples of four: the launcher)
+    const size_t mine = (nst + 1 - (size_t)kg) / 2;
+    const size_t iters = (nst + 1) / 2;
     AnyRaw<KIND> raw[FA_XROUNDS];
-    if (r0 < r1) {  // (r0 and the number of rounds are multiples of four: the launcher sees to it)
-        FA_X_REQUEST(r0);
-#pragma unroll
-        for (int q = 0; q < FA_XROUNDS; ++q) {
-            fetch(r0 + (size_t)q, raw[q]);
-        }
+    size_t round = r0 + (size_t)(FA_XROUNDS * kg);
+    if (mine > 0) {
+        FA_X_REQUEST(round);
+        fetch(round, raw[0], std::false_type{});
+        fetch(round + 1, raw[1], std::false_type{});
+        fetch(round + 2, raw[2], std::false_type{});
+        fetch(round + 3, raw[3], std::true_type{});
         FA_X_STORE(0);
     }
     fa_barrier();
-    // Every stage but the last requests the next one; the last is peeled off so that the loop body has no branch (a
-    // load behind a branch makes the compiler wait for every load in flight at the next use of any of them).
-    size_t round = r0;
-    for (; round + FA_XROUNDS < r1; round += FA_XROUNDS) {
-        FA_X_REQUEST(round + FA_XROUNDS);
-#pragma unroll
-        for (int q = 0; q < FA_XROUNDS; ++q) {
-            step(round + (size_t)q, raw[q], std::true_type{});
-        }
-        FA_X_STORE((int)((((round - r0) / FA_XROUNDS) + 1) & 1));
+    size_t it = 0;
+    for (; it + 1 < mine; ++it, round += 2 * FA_XROUNDS) {
+        FA_X_REQUEST(round + 2 * FA_XROUNDS);
+        step(round, raw[0], std::true_type{}, std::false_type{});
+        step(round + 1, raw[1], std::true_type{}, std::false_type{});
+        step(round + 2, raw[2], std::true_type{}, std::false_type{});
+        step(round + 3, raw[3], std::true_type{}, std::true_type{});
+        FA_X_STORE((int)((it + 1) & 1));
         fa_barrier();  // the stage just read is free for the stage after next; the next stage is complete
     }
-    if (round < r1) {
-#pragma unroll
-        for (int q = 0; q < FA_XROUNDS; ++q) {
-            step(round + (size_t)q, raw[q], std::false_type{});
-        }
+    if (it < mine) {
+        step(round, raw[0], std::false_type{}, std::false_type{});
+        step(round + 1, raw[1], std::false_type{}, std::false_type{});
+        step(round + 2, raw[2], std::false_type{}, std::false_type{});
+        step(round + 3, raw[3], std::false_type{}, std::true_type{});
         fa_barrier();
+        ++it;
+    }
+    for (; it < iters; ++it) {
+        fa_barrier();  // the group with one stage fewer
     }
 
 #undef FA_X_REQUEST
@@ -486,11 +552,24 @@ __global__ __launch_bounds__(FA_THREADS, 2) void k_gemm_any_f16(const GemmAnyPar
     // through LDS as [token][weight row] (the stages are free behind the loop's last barrier) and every thread stores 16
     // bytes per step (stores of one float per lane cost the address unit as much as these and move a quarter).
     float *tile = (float *)lds;
+    if (kg == 1) {
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+        for (int a = 0; a < 2; ++a) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * FA_OUT_PITCH + 32 * wave + j] = acc[a][r];
+            for (int r = 0; r < 16; ++r) {
+                tile[(32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * FA_OUT_PITCH + 32 * wave + j] = acc[a][r];
+            }
+        }
+    }
+    fa_barrier();
+    if (kg == 0) {  // the two K groups' sums meet: group 0's plus group 1's
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float *e = tile + (32 * a + 8 * (r >> 2) + 4 * kh + (r & 3)) * FA_OUT_PITCH + 32 * wave + j;
+                *e = acc[a][r] + *e;
+            }
         }
     }
     fa_barrier();

@@ -657,8 +657,9 @@ int launch_gemm_f16_any(marmot_hip_device *dev, int kind, const void *d_w, const
     if (!gemm_f16_any_supported(dev, kind, N, K, M)) {
         return set_error(MARMOT_HIP_ERROR_NOT_IMPLEMENTED, "fp16 GEMM: unsupported kind or shape");
     }
-    if ((((uintptr_t)d_x) & 15) != 0) {
-        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "fp16 GEMM: activations must be 16-byte aligned");
+    if ((((uintptr_t)d_x) & 15) != 0 || (((uintptr_t)d_w) & 3) != 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT,
+                         "fp16 GEMM: activations must be 16-byte aligned, weights 4-byte aligned");
     }
     const size_t rounds = K / FA_ROUND;
     const size_t tiles_n = (N + FA_TOK - 1) / FA_TOK, tiles_m = (M + FA_WROWS - 1) / FA_WROWS;

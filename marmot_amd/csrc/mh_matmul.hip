@@ -231,7 +231,8 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
             int st;
             if (gemm_f16_supported(dev, kind, N, K, M)) {
                 st = launch_gemm_f16(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);
-            } else if (gemm_f16_any_supported(dev, kind, N, K, M) && (((uintptr_t)d_input) & 15) == 0) {
+            } else if (gemm_f16_any_supported(dev, kind, N, K, M) && (((uintptr_t)d_input) & 15) == 0 &&
+                       (((uintptr_t)w) & 3) == 0) {  // (the kernel loads weight words from multiples of 4)
                 st = launch_gemm_f16_any(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);
             } else {
                 st = launch_matvec_f16(dev, kind, w, d_input, N, K, M, d_bias, bias_dtype, o, out_dtype);

@@ -444,6 +444,7 @@ bool gemm_q23k_applies(const marmot_hip_device *dev, int kind, size_t N, size_t 
                        const ActScratch &act);
 int launch_gemm_q23k(marmot_hip_device *dev, int kind, const WeightSet &ws, const ActScratch &act, size_t N, size_t K,
                      size_t M, int out_dtype, void *scratch);
+size_t gemm_q80_min_rows(int kind);  // activation rows from which the tiled kernel of the format takes over
 bool gemm_q80_kind(int kind);  // Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K: formats of the tiled int8 GEMMs from nine rows on
 bool gemm_q80_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                       const ActScratch &act);

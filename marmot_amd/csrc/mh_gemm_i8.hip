@@ -1592,6 +1592,12 @@ int launch_gemm_i8(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
 // eight the packed matvec streams the weights once; measured at 4096 x 4096 / 14336 x 4096: the matvec takes 16.6 /
 // 33 us at 9 rows and 34 / 74 us at 32, this kernel 16 / 30 us at 33)
 constexpr size_t Q80_MIN_ROWS = 9;
+// Q2_K / Q3_K: the packed matvec is bound by the unpacking of its many values per byte and pays it once per activation
+// row (14336 x 4096: 10 / 20 / 23 us (Q2_K), 13 / 23 / 34 us (Q3_K) at 1 / 4 / 8 rows; the tile 20 / 24 us at 16 rows)
+constexpr size_t Q23K_MIN_ROWS = 5;
+size_t gemm_q80_min_rows(int kind) {
+    return (kind == MARMOT_HIP_KIND_Q2_K || kind == MARMOT_HIP_KIND_Q3_K) ? Q23K_MIN_ROWS : Q80_MIN_ROWS;
+}
 static bool q80_format(int kind) {
     return kind == MARMOT_HIP_KIND_Q8_0 || kind == MARMOT_HIP_KIND_Q4_0 || kind == MARMOT_HIP_KIND_Q4_1 ||
            kind == MARMOT_HIP_KIND_Q5_0 || kind == MARMOT_HIP_KIND_Q5_1;
@@ -1707,7 +1713,7 @@ int launch_gemm_q80(marmot_hip_device *dev, int kind, const WeightSet &ws, const
 // weights once)
 bool gemm_q23k_applies(const marmot_hip_device *dev, int kind, size_t N, size_t K, const void *const *weights, int count,
                        const ActScratch &act) {
-    if (dev->knobs.no_gemm_i8 || N < Q80_MIN_ROWS || K % QK_K != 0 ||
+    if (dev->knobs.no_gemm_i8 || N < Q23K_MIN_ROWS || K % QK_K != 0 ||
         (kind != MARMOT_HIP_KIND_Q2_K && kind != MARMOT_HIP_KIND_Q3_K)) {
         return false;
     }

@@ -269,9 +269,9 @@ static int matmul_impl(marmot_hip_device *dev, int kind, const void *d_w0, const
     }
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes = (act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255;
-    // Q2_K, Q3_K and the 32-value formats (but Q8_1) from nine rows on: the tiled int8 GEMMs (their K-split partial
+    // Q2_K, Q3_K (from five rows on) and the 32-value formats but Q8_1 (from nine): the tiled int8 GEMMs (their K-split partial
     // sums behind the activations)
-    const bool q80_kind = gemm_q80_kind(kind) && N >= 9 && K % QK_K == 0;
+    const bool q80_kind = gemm_q80_kind(kind) && N >= gemm_q80_min_rows(kind) && K % QK_K == 0;
     const size_t need = act_bytes + (mmq ? mmq_scratch_bytes(dev, kind, N, K, M, d_w1 != nullptr ? 2 : 1) : 0) +
                         (q80_kind ? gemm_i8_scratch_bytes(dev, N, K, M, d_w1 != nullptr ? 2 : 1) : 0);
     void *ws = nullptr;
@@ -725,9 +725,9 @@ int marmot_hip_matmul_qkv_rope_quantized(marmot_hip_device_t *dev, int kind, con
     const int act_kind = is_k_quant(kind) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const size_t act_bytes =
         fuse_quant ? 0 : ((act_scratch_layout(act_kind, N, K, nullptr, nullptr) + 255) & ~(size_t)255);
-    // Q2_K, Q3_K and the 32-value formats (but Q8_1) from nine rows on: the tiled int8 GEMMs, their K-split partial
+    // Q2_K, Q3_K (from five rows on) and the 32-value formats but Q8_1 (from nine): the tiled int8 GEMMs, their K-split partial
     // sums where the mmq scratch would be
-    const bool q80_kind = !fuse_quant && gemm_q80_kind(kind) && N >= 9 && K % QK_K == 0;
+    const bool q80_kind = !fuse_quant && gemm_q80_kind(kind) && N >= gemm_q80_min_rows(kind) && K % QK_K == 0;
     const size_t mmq_bytes = mmq ? ((mmq_scratch_bytes(dev, kind, N, K, M, 3) + 255) & ~(size_t)255)
         : q80_kind               ? ((gemm_i8_scratch_bytes(dev, N, K, M, 3) + 255) & ~(size_t)255)
                                  : 0;

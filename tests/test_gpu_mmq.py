@@ -552,7 +552,7 @@ def test_tiled_int8_gemm_q2k_q3k_match_oracle(hip, oracle, name, N, M, K):
 def test_tiled_int8_gemm_q2k_q3k_random_blocks_and_routes(hip, oracle, monkeypatch, name):
     """Arbitrary block bytes (every two-bit value, mask bit, group scale and minimum, Q3_K's scale -32 with value -4
     included: their product, +128, does not fit a signed byte) against the oracle and against the packed matvec of a
-    device object created with MARMOT_HIP_NO_GEMM_I8; fewer than nine rows stay on the matvec; the dual call equals two
+    device object created with MARMOT_HIP_NO_GEMM_I8; fewer than five rows stay on the matvec; the dual call equals two
     single calls bit for bit."""
     from marmot_amd import HipBackend
 
@@ -574,10 +574,12 @@ def test_tiled_int8_gemm_q2k_q3k_random_blocks_and_routes(hip, oracle, monkeypat
         assert_matmul_parity(tiled, got, what="tile against matvec")
     finally:
         plain.close()
-    x8 = gaussian(472, (8, K))
-    got = hip.linear(x8, blocks, kind, M)
-    assert hip.last_route() == f"matvec_{name}_q8_k", hip.last_route()
-    assert_matmul_parity(got, oracle.matmul(kind, blocks, x8, M), what=f"{name} N=8")
+    for n_small, route in ((4, f"matvec_{name}_q8_k_fused"), (5, f"gemm_{name}_q8_k_mfma_tile"),
+                           (8, f"gemm_{name}_q8_k_mfma_tile")):
+        xs = gaussian(472 + n_small, (n_small, K))
+        got = hip.linear(xs, blocks, kind, M)
+        assert hip.last_route() == route, (n_small, hip.last_route())
+        assert_matmul_parity(got, oracle.matmul(kind, blocks, xs, M), what=f"{name} N={n_small}")
     other = random_valid_blocks(np.random.default_rng(473), kind, M, K)
     a, b = hip.linear_dual(x, blocks, other, kind, M)
     assert hip.last_route() == f"gemm_{name}_q8_k_mfma_tile"

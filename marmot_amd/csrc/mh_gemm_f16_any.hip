@@ -38,7 +38,9 @@ constexpr int FA_ROUND = 32;                          // values of K per round
 constexpr int FA_XROUNDS = 4;                         // rounds per activation stage (128 values of K)
 constexpr int FA_XSTAGE = FA_TOK * FA_XROUNDS * FA_ROUND * 2;   // 16,384
 constexpr int FA_OUT_PITCH = FA_WROWS + 4;             // floats per token of the output tile in LDS
-constexpr int FA_MIN_TOKENS = 9;
+// every token count (14336 x 4096 at 1 / 8 rows: Q8_0 30.4 / 30.6 us, Q6_K 28.2 / 28.4 us; the fp16 matvec, four rows
+// at a time, 40.3 / 117 us and 49.2 / 133 us; only 4096 x 4096 at one row is 1.5 us behind it)
+constexpr int FA_MIN_TOKENS = 1;
 static_assert(FA_XROUNDS == 4, "the stage loops are written out for four rounds");
 
 struct GemmAnyParams {

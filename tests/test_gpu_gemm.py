@@ -46,9 +46,10 @@ def check_against_oracle(hip, oracle, blocks, x, M, K, what, bias=None, out_dtyp
     return got32, ref32
 
 
-@pytest.mark.parametrize("N", [9, 64, 128, 130, 512])
+@pytest.mark.parametrize("N", [1, 2, 5, 8, 9, 64, 128, 130, 512])
 def test_gemm_small_shapes(hip, oracle, N):
-    """Token counts around the 128-token tile, M not a multiple of the 256-row tile, K-split and single pass."""
+    """Token counts from a decode step (one token: the fp16 route has no other kernel) to around the 128-token tile, M
+    not a multiple of the 256-row tile, K-split and single pass."""
     M, K = 300, 1024
     blocks = oracle.quantize(KIND_Q4_K, gaussian(500, (M, K), 0.02))
     x = gaussian(501 + N, (N, K)).astype(np.float16)

@@ -76,7 +76,7 @@ def test_gemm_every_format_matches_oracle(hip, oracle, name):
 def test_gemm_every_format_random_blocks_matvec_and_fp16_output(hip, matvec, oracle, name):
     """Arbitrary block bytes (every code, scale and min pattern; scales of both signs) and activations far from unit
     scale against the oracle; the fp16 matvec of a device object created with MARMOT_HIP_NO_GEMM decodes the same
-    weights and must agree; fp16 output with an fp16 bias; fewer than nine rows stay on the matvec."""
+    weights and must agree; fp16 output with an fp16 bias; one, three and eight rows."""
     kind = KINDS[name]
     rng = np.random.default_rng(730)
     M, K, N = 160, 1536, 96
@@ -92,8 +92,11 @@ def test_gemm_every_format_random_blocks_matvec_and_fp16_output(hip, matvec, ora
     x16 = gaussian(733, (N, K)).astype(np.float16)
     bias16 = gaussian(734, (M,)).astype(np.float16)
     check(hip, oracle, name, soft, x16, M, f"{name} f16 out", bias=bias16, out_dtype=np.float16)
-    hip.linear(x16[:8], soft, kind, M)
-    assert "direct" in hip.last_route()
+    for n in (1, 3, 8):  # decode steps and small batches take the same kernel (one tile of 64 tokens, few of them real)
+        few = check(hip, oracle, name, soft, x16[:n], M, f"{name} {n} tokens")
+        mv = matvec.linear(x16[:n], soft, kind, M)
+        assert "direct" in matvec.last_route()
+        assert np.max(np.abs(few - mv)) <= 1e-5 * np.max(np.abs(mv))
 
 
 def test_gemm_q6_k_layer_shape(hip, oracle):

@@ -787,16 +787,15 @@ __device__ __forceinline__ float pa_xor32(float v) {
     return __shfl_xor(v, 32);
 }
 
-// Four e4m3 codes of a word as two words of FLOAT16 pairs holding the codes' values times 2^-8: a code moved to the
-// high byte of a half and shifted right by one (arithmetic) has its sign in bit 15 and its exponent and mantissa where
-// FLOAT16 keeps them, with the exponent bias 8 too small; denormal codes stay exact (both formats are linear there).
-// Codes with all exponent bits set (NaN in the reference's e4m3) come out as finite values: pa_fp8_nan_bits finds them.
-typedef short pa_short2 __attribute__((ext_vector_type(2)));
+// Two e4m3 codes of a word (bytes 0, 1 or 2, 3) as a pair of FLOAT16 values in one instruction (gfx950's conversion
+// with a power-of-two scale, here 1): exact, denormal codes included (both formats are linear there). Codes with all
+// exponent bits set (NaN in the reference's e4m3, finite or NaN in the hardware's) are found by pa_fp8_nan_bits and
+// take the reference's decoder.
+typedef _Float16 pa_half2 __attribute__((ext_vector_type(2)));
 template <int HI>
 __device__ __forceinline__ uint32_t pa_fp8x2_to_f16(uint32_t w) {
-    const uint32_t x = __builtin_amdgcn_perm(w, w, HI ? 0x030c020cu : 0x010c000cu);
-    const pa_short2 sh = __builtin_bit_cast(pa_short2, x) >> (short)1;
-    return __builtin_bit_cast(uint32_t, sh) & 0xbf80bf80u;
+    const pa_half2 v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, HI != 0);
+    return __builtin_bit_cast(uint32_t, v);
 }
 // bit 7 of a byte is set iff that byte of w is a NaN code (exponent field 15)
 __device__ __forceinline__ uint32_t pa_fp8_nan_bits(uint32_t w) {
@@ -806,7 +805,7 @@ __device__ __forceinline__ uint32_t pa_fp8_nan_bits(uint32_t w) {
 template <int HI>
 __device__ __forceinline__ uint32_t pa_fp8x2_to_f16_slow(uint32_t w) {
     const uint32_t c0 = (w >> (HI ? 16 : 0)) & 0xffu, c1 = (w >> (HI ? 24 : 8)) & 0xffu;
-    return (uint32_t)f2h(pa_fp8_to_f32(c0) * 0.00390625f) | ((uint32_t)f2h(pa_fp8_to_f32(c1) * 0.00390625f) << 16);
+    return (uint32_t)f2h(pa_fp8_to_f32(c0)) | ((uint32_t)f2h(pa_fp8_to_f32(c1)) << 16);
 }
 
 constexpr int PA_KV_F16 = 0, PA_KV_BF16 = 1, PA_KV_FP8 = 2;
@@ -918,8 +917,8 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
         uint4 kq[4], vq[4];
         float k_unit = 1.0f, v_unit = 1.0f;  // FLOAT8_E4M3: what one unit of the FLOAT16 operands stands for
         if constexpr (FP8) {
-            // codes -> FLOAT16 operands in registers (exact); the block's scale and the 2^8 of the conversion are applied
-            // to the scores and to the softmax weights. A scale that is not positive decodes to zeros (the reference's
+            // codes -> FLOAT16 operands in registers (exact); the block's scale is applied to the scores and to the
+            // softmax weights. A scale that is not positive decodes to zeros (the reference's
             // cpu_paged_attention_fp8_dequant); a tile that holds a NaN code takes the reference's decoder.
             const size_t si = (size_t)tb * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] +
                               (size_t)kvh * p.scale_stride[2];
@@ -978,8 +977,8 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
                     vq[i] = make_uint4(0, 0, 0, 0);
                 }
             }
-            k_unit = k_live ? ks * 256.0f : 0.0f;
-            v_unit = v_live ? vs * 256.0f : 0.0f;
+            k_unit = k_live ? ks : 0.0f;
+            v_unit = v_live ? vs : 0.0f;
         } else {
             const uint16_t *krow = (const uint16_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
 #pragma unroll

@@ -809,8 +809,9 @@ __device__ __forceinline__ uint32_t pa_fp8x2_to_f16_slow(uint32_t w) {
 }
 
 constexpr int PA_KV_F16 = 0, PA_KV_BF16 = 1, PA_KV_FP8 = 2;
+constexpr uint32_t PA_PIPELINE_TILES = 24;  // tiles per workgroup (six per wavefront) from which the tile loop is pipelined
 
-template <int QH, int KVT>
+template <int QH, int KVT, bool PIPE>
 __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
     constexpr bool BF16 = KVT == PA_KV_BF16, FP8 = KVT == PA_KV_FP8;
     constexpr int EPL = 8;  // head_dim == 128
@@ -902,192 +903,252 @@ __global__ __launch_bounds__(256) void k_pa_attend_mfma(const PaParams p) {
     const uint32_t tiles_per_split = (tiles + p.splits - 1u) / p.splits;
     const uint32_t tile_first = blockIdx.z * tiles_per_split;
     const uint32_t tile_stop = tile_first + tiles_per_split < tiles ? tile_first + tiles_per_split : tiles;
-    for (uint32_t tile = tile_first + (uint32_t)wave; tile < tile_stop; tile += 4u) {
-        const uint32_t p0 = tile << 4;  // first position of the tile
-        const uint32_t logical = p0 >> p.shift;
-        if (logical >= p.max_blocks) {
-            continue;
-        }
-        const uint32_t tb = table_row[(size_t)logical * p.table_stride[1]];
-        if (tb == PA_NO_BLOCK || tb >= p.kv_blocks) {
-            continue;  // a hole: none of the tile's positions has a block
-        }
-        const size_t tile_base = (size_t)tb * p.kv_stride[0] + head_base + (size_t)(p0 & p.mask) * p.kv_stride[3];
+    // Tiles of this wavefront: tile_first + wave, + 4, ... Two memory latencies lie in front of a tile's arithmetic, the
+    // block table entry and then the rows it points to; with a handful of tiles per wavefront they were most of the
+    // kernel's time. So the loop of the PIPE form runs a pipeline: while tile k is worked on, the rows of tile k + 1 and the table entry
+    // of tile k + 2 are in flight. All of these loads are unconditional (a tile that does not exist or has no block
+    // reads block 0 and is marked): a load behind a branch would make the compiler wait for everything in flight.
+    struct TileRaw {
+        uint4 k[4], v[4];  // FLOAT8_E4M3: k[0..1] = the 32 key codes, v[0..1] = 4 x 8 value codes
+        float ks, vs;
+        uint32_t p0;
+        bool ok;
+    };
+    const uint32_t table_last = p.max_blocks > 0u ? p.max_blocks - 1u : 0u;
+    auto table_entry = [&](uint32_t tile) -> uint32_t {
+        const uint32_t logical = (tile << 4) >> p.shift;
+        return table_row[(size_t)(logical < table_last ? logical : table_last) * p.table_stride[1]];
+    };
+    auto request = [&](TileRaw &r, uint32_t tile, uint32_t tb) {
+        const uint32_t logical = (tile << 4) >> p.shift;
+        r.ok = tile < tile_stop && logical < p.max_blocks && tb != PA_NO_BLOCK && tb < p.kv_blocks;  // else: a hole
+        r.p0 = r.ok ? tile << 4 : 0u;
+        const uint32_t tbs = r.ok ? tb : 0u;
+        const size_t tile_base = (size_t)tbs * p.kv_stride[0] + head_base + (size_t)(r.p0 & p.mask) * p.kv_stride[3];
         // key rows: position n of the tile, dimensions 32 j .. + 31; value rows: positions 4 j + i, dimensions 8 n .. + 7
+        if constexpr (FP8) {
+            const size_t si = (size_t)tbs * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] +
+                              (size_t)kvh * p.scale_stride[2];
+            r.ks = p.k_scale[si];
+            r.vs = p.v_scale[si];
+            const uint8_t *krow = (const uint8_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
+            r.k[0] = *(const uint4 *)krow;
+            r.k[1] = *(const uint4 *)(krow + 16);
+            uint2 vr[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                vr[i] = *(const uint2 *)((const uint8_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+            }
+            r.v[0] = make_uint4(vr[0].x, vr[0].y, vr[1].x, vr[1].y);
+            r.v[1] = make_uint4(vr[2].x, vr[2].y, vr[3].x, vr[3].y);
+        } else {
+            const uint16_t *krow = (const uint16_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                r.k[c] = *(const uint4 *)(krow + 8 * c);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                r.v[i] = *(const uint4 *)((const uint16_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+            }
+        }
+    };
+    auto consume = [&](const TileRaw &r) {
+        if (!r.ok) {
+            return;
+        }
+        const uint32_t p0 = r.p0;  // first position of the tile
         uint4 kq[4], vq[4];
         float k_unit = 1.0f, v_unit = 1.0f;  // FLOAT8_E4M3: what one unit of the FLOAT16 operands stands for
         if constexpr (FP8) {
             // codes -> FLOAT16 operands in registers (exact); the block's scale is applied to the scores and to the
             // softmax weights. A scale that is not positive decodes to zeros (the reference's
             // cpu_paged_attention_fp8_dequant); a tile that holds a NaN code takes the reference's decoder.
-            const size_t si = (size_t)tb * p.scale_stride[0] + (size_t)p.layer_idx * p.scale_stride[1] +
-                              (size_t)kvh * p.scale_stride[2];
-            const float ks = p.k_scale[si], vs = p.v_scale[si];
-            const uint8_t *krow = (const uint8_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
-            const uint4 kr0 = *(const uint4 *)krow, kr1 = *(const uint4 *)(krow + 16);
-            uint2 vr[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                vr[i] = *(const uint2 *)((const uint8_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
-            }
-            const uint32_t kw[8] = {kr0.x, kr0.y, kr0.z, kr0.w, kr1.x, kr1.y, kr1.z, kr1.w};
-            uint32_t nan_k = 0, nan_v = 0;
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                nan_k |= pa_fp8_nan_bits(kw[c]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                nan_v |= pa_fp8_nan_bits(vr[i].x) | pa_fp8_nan_bits(vr[i].y);
-            }
-            const bool k_live = ks > 0.0f, v_live = vs > 0.0f;
-            const bool slow = ((nan_k & 0x80808080u) != 0 && k_live) || ((nan_v & 0x80808080u) != 0 && v_live);
-            if (__builtin_amdgcn_ballot_w64(slow) == 0) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    kq[c] = make_uint4(pa_fp8x2_to_f16<0>(kw[2 * c]), pa_fp8x2_to_f16<1>(kw[2 * c]),
-                                       pa_fp8x2_to_f16<0>(kw[2 * c + 1]), pa_fp8x2_to_f16<1>(kw[2 * c + 1]));
+            const float ks = r.ks, vs = r.vs;
+            const uint32_t kw[8] = {r.k[0].x, r.k[0].y, r.k[0].z, r.k[0].w, r.k[1].x, r.k[1].y, r.k[1].z, r.k[1].w};
+            const uint2 vr[4] = {make_uint2(r.v[0].x, r.v[0].y), make_uint2(r.v[0].z, r.v[0].w),
+                                 make_uint2(r.v[1].x, r.v[1].y), make_uint2(r.v[1].z, r.v[1].w)};
+                uint32_t nan_k = 0, nan_v = 0;
+    #pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    nan_k |= pa_fp8_nan_bits(kw[c]);
                 }
-#pragma unroll
+    #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    vq[i] = make_uint4(pa_fp8x2_to_f16<0>(vr[i].x), pa_fp8x2_to_f16<1>(vr[i].x),
-                                       pa_fp8x2_to_f16<0>(vr[i].y), pa_fp8x2_to_f16<1>(vr[i].y));
+                    nan_v |= pa_fp8_nan_bits(vr[i].x) | pa_fp8_nan_bits(vr[i].y);
                 }
-            } else {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    kq[c] = make_uint4(pa_fp8x2_to_f16_slow<0>(kw[2 * c]), pa_fp8x2_to_f16_slow<1>(kw[2 * c]),
-                                       pa_fp8x2_to_f16_slow<0>(kw[2 * c + 1]), pa_fp8x2_to_f16_slow<1>(kw[2 * c + 1]));
+                const bool k_live = ks > 0.0f, v_live = vs > 0.0f;
+                const bool slow = ((nan_k & 0x80808080u) != 0 && k_live) || ((nan_v & 0x80808080u) != 0 && v_live);
+                if (__builtin_amdgcn_ballot_w64(slow) == 0) {
+    #pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        kq[c] = make_uint4(pa_fp8x2_to_f16<0>(kw[2 * c]), pa_fp8x2_to_f16<1>(kw[2 * c]),
+                                           pa_fp8x2_to_f16<0>(kw[2 * c + 1]), pa_fp8x2_to_f16<1>(kw[2 * c + 1]));
+                    }
+    #pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        vq[i] = make_uint4(pa_fp8x2_to_f16<0>(vr[i].x), pa_fp8x2_to_f16<1>(vr[i].x),
+                                           pa_fp8x2_to_f16<0>(vr[i].y), pa_fp8x2_to_f16<1>(vr[i].y));
+                    }
+                } else {
+    #pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        kq[c] = make_uint4(pa_fp8x2_to_f16_slow<0>(kw[2 * c]), pa_fp8x2_to_f16_slow<1>(kw[2 * c]),
+                                           pa_fp8x2_to_f16_slow<0>(kw[2 * c + 1]), pa_fp8x2_to_f16_slow<1>(kw[2 * c + 1]));
+                    }
+    #pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        vq[i] = make_uint4(pa_fp8x2_to_f16_slow<0>(vr[i].x), pa_fp8x2_to_f16_slow<1>(vr[i].x),
+                                           pa_fp8x2_to_f16_slow<0>(vr[i].y), pa_fp8x2_to_f16_slow<1>(vr[i].y));
+                    }
                 }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    vq[i] = make_uint4(pa_fp8x2_to_f16_slow<0>(vr[i].x), pa_fp8x2_to_f16_slow<1>(vr[i].x),
-                                       pa_fp8x2_to_f16_slow<0>(vr[i].y), pa_fp8x2_to_f16_slow<1>(vr[i].y));
+                if (!k_live) {
+    #pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        kq[c] = make_uint4(0, 0, 0, 0);
+                    }
                 }
-            }
-            if (!k_live) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    kq[c] = make_uint4(0, 0, 0, 0);
+                if (!v_live) {
+    #pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        vq[i] = make_uint4(0, 0, 0, 0);
+                    }
                 }
-            }
-            if (!v_live) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    vq[i] = make_uint4(0, 0, 0, 0);
-                }
-            }
-            k_unit = k_live ? ks : 0.0f;
-            v_unit = v_live ? vs : 0.0f;
+                k_unit = k_live ? ks : 0.0f;
+                v_unit = v_live ? vs : 0.0f;
         } else {
-            const uint16_t *krow = (const uint16_t *)p.kv_k + tile_base + (size_t)n * p.kv_stride[3] + 32u * j;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                kq[c] = *(const uint4 *)(krow + 8 * c);
+                kq[c] = r.k[c];
+                vq[c] = r.v[c];
             }
-#pragma unroll
+        }
+            pa_float4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
+    #pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint2 k0 = make_uint2(kq[c].x, kq[c].y), k1 = make_uint2(kq[c].z, kq[c].w);
+    #pragma unroll
+                for (int part = 0; part < PARTS; ++part) {
+                    sc = mma(k0, qpart[part][2 * c], sc);
+                }
+    #pragma unroll
+                for (int part = 0; part < PARTS; ++part) {
+                    sc = mma(k1, qpart[part][2 * c + 1], sc);
+                }
+            }
+            // positions beyond the sequence (the last tile): no score, no value
+            const bool whole = p0 + 16u <= kv_len;
+            float s4[4] = {sc[0], sc[1], sc[2], sc[3]};
+            if constexpr (FP8) {
+    #pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s4[i] *= k_unit;
+                }
+            }
+            if (!whole) {
+    #pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (p0 + 4u * j + (uint32_t)i >= kv_len) {
+                        s4[i] = -INFINITY;
+                        vq[i] = make_uint4(0, 0, 0, 0);
+                    }
+                }
+            }
+            // online softmax of head n over the tile's 16 positions (lanes n, n + 16, n + 32, n + 48)
+            float big = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+            big = fmaxf(big, pa_xor16(big));
+            big = fmaxf(big, pa_xor32(big));
+            const float m_new = fmaxf(m, big);
+            const float corr = m == -INFINITY ? 0.0f : pa_exp(m - m_new);
+            float w4[4];
+    #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                vq[i] = *(const uint4 *)((const uint16_t *)p.kv_v + tile_base + (size_t)(4 * j + i) * p.kv_stride[3] + 8u * n);
+                w4[i] = pa_exp(s4[i] - m_new);
             }
-        }
-        pa_float4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint2 k0 = make_uint2(kq[c].x, kq[c].y), k1 = make_uint2(kq[c].z, kq[c].w);
-#pragma unroll
-            for (int part = 0; part < PARTS; ++part) {
-                sc = mma(k0, qpart[part][2 * c], sc);
+            float tsum = (w4[0] + w4[1]) + (w4[2] + w4[3]);
+            tsum += pa_xor16(tsum);
+            tsum += pa_xor32(tsum);
+            lsum = lsum * corr + tsum;
+            const bool moved = m_new != m;
+            m = m_new;
+            // rescale the running output of the heads whose maximum moved
+            if (__builtin_amdgcn_ballot_w64(moved && n < QH) != 0) {
+                float f[QH];
+                f[0] = pa_group_bcast<0>(corr);
+                if constexpr (QH > 1) {
+                    f[1] = pa_group_bcast<1>(corr);
+                }
+                if constexpr (QH > 2) {
+                    f[2] = pa_group_bcast<2>(corr);
+                    f[3] = pa_group_bcast<3>(corr);
+                }
+    #pragma unroll
+                for (int h = 0; h < QH; ++h) {
+    #pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        acc[h][e] *= f[h];
+                    }
+                }
             }
-#pragma unroll
-            for (int part = 0; part < PARTS; ++part) {
-                sc = mma(k1, qpart[part][2 * c + 1], sc);
-            }
-        }
-        // positions beyond the sequence (the last tile): no score, no value
-        const bool whole = p0 + 16u <= kv_len;
-        float s4[4] = {sc[0], sc[1], sc[2], sc[3]};
-        if constexpr (FP8) {
-#pragma unroll
+            // values: this group's four positions, dimensions 8 n .. 8 n + 7
+    #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                s4[i] *= k_unit;
-            }
-        }
-        if (!whole) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (p0 + 4u * j + (uint32_t)i >= kv_len) {
-                    s4[i] = -INFINITY;
-                    vq[i] = make_uint4(0, 0, 0, 0);
+                float vr[EPL];
+                const uint32_t vw[4] = {vq[i].x, vq[i].y, vq[i].z, vq[i].w};
+    #pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if constexpr (BF16) {
+                        vr[2 * e] = __uint_as_float(vw[e] << 16);
+                        vr[2 * e + 1] = __uint_as_float(vw[e] & 0xffff0000u);
+                    } else {
+                        vr[2 * e] = h2f((uint16_t)(vw[e] & 0xffffu));
+                        vr[2 * e + 1] = h2f((uint16_t)(vw[e] >> 16));
+                    }
+                }
+                float wh[QH];
+                const float wi = FP8 ? w4[i] * v_unit : w4[i];  // the value rows' unit goes with the weight
+                wh[0] = pa_group_bcast<0>(wi);
+                if constexpr (QH > 1) {
+                    wh[1] = pa_group_bcast<1>(wi);
+                }
+                if constexpr (QH > 2) {
+                    wh[2] = pa_group_bcast<2>(wi);
+                    wh[3] = pa_group_bcast<3>(wi);
+                }
+    #pragma unroll
+                for (int h = 0; h < QH; ++h) {
+    #pragma unroll
+                    for (int e = 0; e < EPL; ++e) {
+                        acc[h][e] = __builtin_fmaf(wh[h], vr[e], acc[h][e]);
+                    }
                 }
             }
+    };
+    const bool any_tile = p.kv_blocks > 0u && p.max_blocks > 0u && tile_first + (uint32_t)wave < tile_stop;
+    // Few tiles per wavefront (short histories, the tokens of a prompt): one after the other; the pipeline's extra
+    // requests (a tile and two table entries beyond the end) cost more than they hide there (16 x 512 positions
+    // 18.7 -> 22.9 us, a prompt of 512 tokens 76 -> 101 us with the pipeline everywhere).
+    if (any_tile && (!PIPE || tile_stop - tile_first < PA_PIPELINE_TILES)) {
+        TileRaw r;
+        for (uint32_t tile = tile_first + (uint32_t)wave; tile < tile_stop; tile += 4u) {
+            request(r, tile, table_entry(tile));
+            consume(r);
         }
-        // online softmax of head n over the tile's 16 positions (lanes n, n + 16, n + 32, n + 48)
-        float big = fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-        big = fmaxf(big, pa_xor16(big));
-        big = fmaxf(big, pa_xor32(big));
-        const float m_new = fmaxf(m, big);
-        const float corr = m == -INFINITY ? 0.0f : pa_exp(m - m_new);
-        float w4[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            w4[i] = pa_exp(s4[i] - m_new);
-        }
-        float tsum = (w4[0] + w4[1]) + (w4[2] + w4[3]);
-        tsum += pa_xor16(tsum);
-        tsum += pa_xor32(tsum);
-        lsum = lsum * corr + tsum;
-        const bool moved = m_new != m;
-        m = m_new;
-        // rescale the running output of the heads whose maximum moved
-        if (__builtin_amdgcn_ballot_w64(moved && n < QH) != 0) {
-            float f[QH];
-            f[0] = pa_group_bcast<0>(corr);
-            if constexpr (QH > 1) {
-                f[1] = pa_group_bcast<1>(corr);
-            }
-            if constexpr (QH > 2) {
-                f[2] = pa_group_bcast<2>(corr);
-                f[3] = pa_group_bcast<3>(corr);
-            }
-#pragma unroll
-            for (int h = 0; h < QH; ++h) {
-#pragma unroll
-                for (int e = 0; e < EPL; ++e) {
-                    acc[h][e] *= f[h];
-                }
-            }
-        }
-        // values: this group's four positions, dimensions 8 n .. 8 n + 7
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float vr[EPL];
-            const uint32_t vw[4] = {vq[i].x, vq[i].y, vq[i].z, vq[i].w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                if constexpr (BF16) {
-                    vr[2 * e] = __uint_as_float(vw[e] << 16);
-                    vr[2 * e + 1] = __uint_as_float(vw[e] & 0xffff0000u);
-                } else {
-                    vr[2 * e] = h2f((uint16_t)(vw[e] & 0xffffu));
-                    vr[2 * e + 1] = h2f((uint16_t)(vw[e] >> 16));
-                }
-            }
-            float wh[QH];
-            const float wi = FP8 ? w4[i] * v_unit : w4[i];  // the value rows' unit goes with the weight
-            wh[0] = pa_group_bcast<0>(wi);
-            if constexpr (QH > 1) {
-                wh[1] = pa_group_bcast<1>(wi);
-            }
-            if constexpr (QH > 2) {
-                wh[2] = pa_group_bcast<2>(wi);
-                wh[3] = pa_group_bcast<3>(wi);
-            }
-#pragma unroll
-            for (int h = 0; h < QH; ++h) {
-#pragma unroll
-                for (int e = 0; e < EPL; ++e) {
-                    acc[h][e] = __builtin_fmaf(wh[h], vr[e], acc[h][e]);
-                }
+    } else if (any_tile) {
+        if constexpr (PIPE) {
+            uint32_t tile = tile_first + (uint32_t)wave;
+            TileRaw ra, rb;
+            uint32_t e1 = table_entry(tile + 4u), e2 = table_entry(tile + 8u);
+            request(ra, tile, table_entry(tile));
+            for (; tile < tile_stop; tile += 8u) {
+                request(rb, tile + 4u, e1);
+                const uint32_t e3 = table_entry(tile + 12u);
+                consume(ra);
+                request(ra, tile + 8u, e2);
+                const uint32_t e4 = table_entry(tile + 16u);
+                consume(rb);
+                e1 = e3;
+                e2 = e4;
             }
         }
     }
@@ -1357,28 +1418,42 @@ extern "C" int marmot_hip_paged_attention(marmot_hip_device_t *dev, const marmot
     MH_HIP(hipGetLastError());
     if (mfma_scores) {
         const dim3 grid(p.token_count, p.num_q_heads / (uint32_t)qh, p.splits), block(256);
-        if (fp8) {
+        // FLOAT8_E4M3 decode steps over long contexts (few tokens, a block table of 2048 positions or more): the form
+        // whose tile loop is pipelined (16 x 4096 positions 60.7 -> 48.7 us). It needs the registers of a third
+        // resident wavefront per SIMD, which short histories and prompts miss more than they gain (FLOAT16, pipeline
+        // compiled in: 16 x 512 positions 18.7 -> 23.9 us, a prompt of 512 tokens 76 -> 105 us), and a FLOAT16 cache at
+        // 4096 positions runs at the memory's rate either way (53.0 / 53.0 us).
+        const bool pipe = fp8 && p.splits > 1u && (size_t)p.max_blocks * a->block_size >= 2048u;
+        if (fp8 && pipe) {
             if (qh == 4) {
-                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_FP8>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_FP8, true>), grid, block, 0, dev->stream, p);
             } else if (qh == 2) {
-                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_FP8>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_FP8, true>), grid, block, 0, dev->stream, p);
             } else {
-                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_FP8>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_FP8, true>), grid, block, 0, dev->stream, p);
+            }
+        } else if (fp8) {
+            if (qh == 4) {
+                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_FP8, false>), grid, block, 0, dev->stream, p);
+            } else if (qh == 2) {
+                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_FP8, false>), grid, block, 0, dev->stream, p);
+            } else {
+                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_FP8, false>), grid, block, 0, dev->stream, p);
             }
         } else if (kv_bf16) {
             if (qh == 4) {
-                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_BF16>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_BF16, false>), grid, block, 0, dev->stream, p);
             } else if (qh == 2) {
-                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_BF16>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_BF16, false>), grid, block, 0, dev->stream, p);
             } else {
-                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_BF16>), grid, block, 0, dev->stream, p);
+                hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_BF16, false>), grid, block, 0, dev->stream, p);
             }
         } else if (qh == 4) {
-            hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_F16>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<4, PA_KV_F16, false>), grid, block, 0, dev->stream, p);
         } else if (qh == 2) {
-            hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_F16>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<2, PA_KV_F16, false>), grid, block, 0, dev->stream, p);
         } else {
-            hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_F16>), grid, block, 0, dev->stream, p);
+            hipLaunchKernelGGL((k_pa_attend_mfma<1, PA_KV_F16, false>), grid, block, 0, dev->stream, p);
         }
     } else if (epl == 4) {
         qh == 4 ? pa_launch<4, 4>(dev, p) : qh == 2 ? pa_launch<4, 2>(dev, p) : pa_launch<4, 1>(dev, p);

@@ -286,6 +286,21 @@ def test_fp8_cache_long_context_decode_batch(hip, oracle):
     _fp8_both(hip, oracle, step, "decode over long histories")
 
 
+def test_fp8_cache_decode_over_a_wide_block_table(hip, oracle):
+    """Decode steps on an fp8 cache whose block table spans 2048 positions or more take the form of the kernel whose
+    tile loop is pipelined (rows of the next tile and the table entry of the one after in flight); sequences with few
+    tiles take its plain loop. A history of 2100 positions next to ones of 40 and 500, two decode steps, and a
+    sequence whose last tile is partial."""
+    case = _fp8_case(87, [(0, 2100), (0, 40), (0, 500)], room=2, num_q_heads=4, num_kv_heads=1, head_dim=128,
+                     block_size=16, layers=1, layer_idx=0)
+    assert case["block_table"].shape[1] * 16 >= 2048
+    state = _fp8_both(hip, oracle, case, "prompts")
+    step = _next_step(case, state, 88, [1.0, 2.0, 0.5])
+    state = _fp8_both(hip, oracle, step, "decode, wide table")
+    step = _next_step(step, state, 89, [4.0, 1.0, 1.0])
+    _fp8_both(hip, oracle, step, "second decode step")
+
+
 def test_fp8_cache_errors(hip):
     case = _fp8_case(5, [(0, 3)], num_q_heads=2, num_kv_heads=1, head_dim=16, block_size=4)
     args = (case["token_meta"], case["q"], case["k_new"], case["v_new"])

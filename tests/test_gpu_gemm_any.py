@@ -72,6 +72,17 @@ def test_gemm_every_format_matches_oracle(hip, oracle, name):
         check(hip, oracle, name, blocks, x, M, f"{name} {N}x{K}x{M}", bias=bias)
 
 
+@pytest.mark.parametrize("name", [n for n in NAMES if not n.endswith("_k")])
+def test_gemm_32_value_formats_odd_stage_counts(hip, oracle, name):
+    """A workgroup's two K groups take alternate stages of 128 values: one stage (the second group has none), three
+    and five stages, 29 stages split across workgroups."""
+    kind = KINDS[name]
+    for n, (N, K, M) in enumerate([(5, 128, 40), (70, 384, 129), (33, 640, 300), (12, 3712, 64)]):
+        blocks = oracle.quantize(kind, gaussian(750 + n, (M, K), 0.02))
+        x = gaussian(760 + n, (N, K)).astype(np.float16)
+        check(hip, oracle, name, blocks, x, M, f"{name} {N}x{K}x{M}")
+
+
 @pytest.mark.parametrize("name", NAMES)
 def test_gemm_every_format_random_blocks_matvec_and_fp16_output(hip, matvec, oracle, name):
     """Arbitrary block bytes (every code, scale and min pattern; scales of both signs) and activations far from unit

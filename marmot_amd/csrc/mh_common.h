@@ -455,7 +455,7 @@ int launch_mmq_set(marmot_hip_device *dev, int kind, const WeightSet &ws, const 
 bool mmq_grouped_supported(const marmot_hip_device *dev, int kind, size_t K);
 int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
                        const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
-                       size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1);
+                       size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1, int item_cols);
 // sums fp32 partials [splits][N][M] in split order, then bias and output cast (mh_gemm.hip)
 int launch_splitk_reduce(marmot_hip_device *dev, const float *partial, int splits, size_t N, size_t M,
                          const void *d_bias, int bias_dtype, void *d_out, int out_dtype, bool bias_first = false);

@@ -1154,7 +1154,7 @@ bool mmq_grouped_supported(const marmot_hip_device *dev, int kind, size_t K) {
 
 int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const void *d_w1, size_t expert_stride,
                        const ActScratch &act, const uint32_t *d_act_index, const int4 *d_items, const int *d_n_items,
-                       size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1) {
+                       size_t max_items, size_t K, size_t M, void *d_out0, void *d_out1, int item_cols) {
     if (max_items == 0 || M == 0 || K == 0) {
         return MARMOT_HIP_SUCCESS;
     }
@@ -1198,7 +1198,10 @@ int launch_mmq_grouped(marmot_hip_device *dev, int kind, const void *d_w0, const
     p.n_items = d_n_items;
     p.act_index = d_act_index;
     p.expert_stride = expert_stride;
-    const int st = mmq_launch<4>(dev, kind, p, pl, M, (unsigned)max_items);
+    // work items of up to 8, 16 or 32 routes (the caller cut them to match)
+    const int st = item_cols <= 8    ? mmq_launch<4>(dev, kind, p, pl, M, (unsigned)max_items)
+                   : item_cols <= 16 ? mmq_launch<8>(dev, kind, p, pl, M, (unsigned)max_items)
+                                     : mmq_launch<16>(dev, kind, p, pl, M, (unsigned)max_items);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }

@@ -9,7 +9,7 @@
 
 namespace mh {
 
-constexpr int MOE_ITEM_COLS = 8;   // routes per grouped-matvec work item
+constexpr int MOE_ITEM_COLS = 8;   // routes per grouped work item (16 or 32 when experts see many routes, see moe_item_cols)
 constexpr int MOE_MAX_EXPERTS = 1024;
 constexpr int MOE_MAX_TOPK = 64;
 
@@ -107,6 +107,7 @@ struct RouteArgs {
     float weights_scale;
     int renormalize;
     int decode_order;
+    int item_cols;                // routes per work item: 8, 16 or 32
 };
 
 constexpr int MOE_ROUTE_LDS = 4096;    // routes whose ids and positions are kept in LDS
@@ -186,12 +187,12 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * 64) void k_moe_route(const RouteA
         const bool first = id >= 0 && rank == 0;
         int total, n_items;
         const int seg = wave_excl_scan(first ? cnt : 0, lane, &total);
-        const int item0 = wave_excl_scan(first ? (cnt + MOE_ITEM_COLS - 1) / MOE_ITEM_COLS : 0, lane, &n_items);
+        const int item0 = wave_excl_scan(first ? (cnt + a.item_cols - 1) / a.item_cols : 0, lane, &n_items);
         if (first) {
             counts[id] = seg;
             int n = item0;
-            for (int j = 0; j < cnt; j += MOE_ITEM_COLS) {
-                a.items[n++] = make_int4(id, seg + j, (cnt - j) < MOE_ITEM_COLS ? (cnt - j) : MOE_ITEM_COLS, 0);
+            for (int j = 0; j < cnt; j += a.item_cols) {
+                a.items[n++] = make_int4(id, seg + j, (cnt - j) < a.item_cols ? (cnt - j) : a.item_cols, 0);
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the segment starts are in LDS (same wavefront)
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * 64) void k_moe_route(const RouteA
         for (int e = e0; e < e1; ++e) {
             const int c = counts[e];
             c_sum += c;
-            i_sum += (c + MOE_ITEM_COLS - 1) / MOE_ITEM_COLS;
+            i_sum += (c + a.item_cols - 1) / a.item_cols;
         }
         int total, n_items;
         int prefix = wave_excl_scan(c_sum, lane, &total);
@@ -260,8 +261,8 @@ __global__ __launch_bounds__(MOE_ROUTE_WAVES * 64) void k_moe_route(const RouteA
         for (int e = e0; e < e1; ++e) {
             const int c = counts[e];
             counts[e] = prefix;  // from here on: start of the expert's segment
-            for (int j = 0; j < c; j += MOE_ITEM_COLS) {
-                a.items[n++] = make_int4(e, prefix + j, (c - j) < MOE_ITEM_COLS ? (c - j) : MOE_ITEM_COLS, 0);
+            for (int j = 0; j < c; j += a.item_cols) {
+                a.items[n++] = make_int4(e, prefix + j, (c - j) < a.item_cols ? (c - j) : a.item_cols, 0);
             }
             prefix += c;
         }
@@ -446,7 +447,16 @@ static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, siz
     MH_HIP(hipSetDevice(dev->device_index));
 
     const size_t routes = T * k_per_token;
-    const size_t max_items = routes < E + routes / MOE_ITEM_COLS ? routes : E + routes / MOE_ITEM_COLS;
+    // Routes per work item. A work item streams its expert's rows once for its routes, so prompts, where an expert
+    // sees dozens of routes, take wider items (the small-batch kernels on the int8 matrix cores hold 16 or 32 activation
+    // rows per pass; the dot-product kernel of the 32-value formats holds 8): E = 128, top 8, 512 tokens: 325 us with 8.
+    const bool mmq_gu = mmq_grouped_supported(dev, kind_gate_up, H), mmq_dn = mmq_grouped_supported(dev, kind_down, F);
+    const auto q45 = [](int kind) { return kind == MARMOT_HIP_KIND_Q4_K || kind == MARMOT_HIP_KIND_Q5_K; };
+    size_t item_cols = MOE_ITEM_COLS;
+    if (mmq_gu && mmq_dn && routes >= 12 * E) {
+        item_cols = (routes >= 24 * E && q45(kind_gate_up) && q45(kind_down)) ? 32 : 16;
+    }
+    const size_t max_items = routes < E + routes / item_cols ? routes : E + routes / item_cols;
     const int act_gu = is_k_quant(kind_gate_up) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
     const int act_dn = is_k_quant(kind_down) ? MARMOT_HIP_KIND_Q8_K : MARMOT_HIP_KIND_Q8_0;
 
@@ -501,6 +511,7 @@ static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, siz
     ra.renormalize = router_weight_policy == MARMOT_HIP_ROUTER_RENORMALIZE_SELECTED;
     // cpu_moe_should_use_decode_path (moe_ops.c:417-424)
     ra.decode_order = (T <= 4 && routes <= 64) ? 1 : 0;
+    ra.item_cols = (int)item_cols;
     hipLaunchKernelGGL(k_moe_route, dim3(1), dim3(MOE_ROUTE_WAVES * 64), 0, dev->stream, ra);
     MH_HIP(hipGetLastError());
 
@@ -512,10 +523,10 @@ static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, siz
     const size_t gu_stride = F * ((H + bv_gu - 1) / bv_gu) * block_bytes(kind_gate_up);
     const size_t dn_stride = H * ((F + bv_dn - 1) / bv_dn) * block_bytes(kind_down);
     // Q4_K / Q6_K experts run on the int8 matrix cores, the 32-value formats on the dot-product matvec
-    const auto grouped_gu = mmq_grouped_supported(dev, kind_gate_up, H) ? launch_mmq_grouped : launch_matvec_grouped;
-    const auto grouped_dn = mmq_grouped_supported(dev, kind_down, F) ? launch_mmq_grouped : launch_matvec_grouped;
-    st = grouped_gu(dev, kind_gate_up, d_gate, d_up, gu_stride, hidden_q, sorted_tokens, items, flags, max_items, H, F,
-                    gate_out, up_out);
+    st = mmq_gu ? launch_mmq_grouped(dev, kind_gate_up, d_gate, d_up, gu_stride, hidden_q, sorted_tokens, items, flags,
+                                     max_items, H, F, gate_out, up_out, (int)item_cols)
+                : launch_matvec_grouped(dev, kind_gate_up, d_gate, d_up, gu_stride, hidden_q, sorted_tokens, items, flags,
+                                        max_items, H, F, gate_out, up_out);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
@@ -546,8 +557,10 @@ static int moe_experts_impl(marmot_hip_device_t *dev, const float *d_hidden, siz
                                   dev->stream));
         }
     }
-    st = grouped_dn(dev, kind_down, d_down, nullptr, dn_stride, fused_q, nullptr, items, flags, max_items, F, H,
-                    route_down, nullptr);
+    st = mmq_dn ? launch_mmq_grouped(dev, kind_down, d_down, nullptr, dn_stride, fused_q, nullptr, items, flags, max_items,
+                                     F, H, route_down, nullptr, (int)item_cols)
+                : launch_matvec_grouped(dev, kind_down, d_down, nullptr, dn_stride, fused_q, nullptr, items, flags,
+                                        max_items, F, H, route_down, nullptr);
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }

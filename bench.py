@@ -558,12 +558,33 @@ def sweep_layer_stack(hip, rng, emit, steps: int, N: int = 16, config: str = "C4
                                        weight_offset=(i % copies) * stride)
 
     ms_shared = time_steps_graph(hip, layer_step_shared, max(50, steps // 10), 10, chunk=50)
+
+    # The same again with the linears that share an input as the branches of one section (q | k | v, gate | up): they
+    # do not depend on each other, so the tail of one, the launch gap and the start-up of the next overlap.
+    def layer_step_branches(i):
+        for src, members in groups:
+            kind, M, K = specs[src]
+            hip.pack_activations_d(kind, layers[src][5], DT_F32, N, K, packed[src])
+
+            def one(m):
+                kind_m, M_m, K_m, stride, d_w, _, d_out = layers[m]
+                return lambda: hip.linear_prepacked_d(kind_m, d_w, packed[src], N, K_m, M_m, d_out,
+                                                      weight_offset=(i % copies) * stride)
+
+            if len(members) > 1:
+                hip.branches(*[one(m) for m in members])
+            else:
+                one(members[0])()
+
+    ms_branches = time_steps_graph(hip, layer_step_branches, max(50, steps // 10), 10, chunk=50)
     ops = sum(2.0 * N * M * K for _, M, K in specs)
     emit({"config": config, "workload": f"7 linears of a Llama-3-8B layer (q,k,o,gate,up Q4_K; v,down Q6_K), N={N}",
           "us": round(ms * 1e3, 2), "GB/s": round(total / ms / 1e6, 1),
           "frac_of_hbm_peak": round(total / ms / 1e6 / HBM_PEAK_GBPS, 4), "tokens_per_s": round(N / ms * 1e3),
           "TOP/s": round(ops / ms / 1e9, 1), "algorithmic_bytes": total,
           "us_shared_inputs": round(ms_shared * 1e3, 2),
+          "us_shared_inputs_branches": round(ms_branches * 1e3, 2),
+          "branches": "as shared_inputs, with q | k | v and gate | up as branches of one section (separate streams)",
           "shared_inputs": "q/k/v and gate/up take activations packed once per distinct input (4 packs, 7 linears)"})
     for b in packed.values():
         b.free()

@@ -144,6 +144,28 @@ void marmot_hip_graph_destroy(marmot_hip_device_t *dev, void *graph_exec);
 size_t marmot_hip_graph_max_nodes(void);
 size_t marmot_hip_graph_last_capture_nodes(marmot_hip_device_t *dev);
 
+/* Branches: calls that do not depend on each other may overlap on the device. No counterpart in the reference, whose
+ * interpreter runs the instructions of a bytecode program one after the other (marmot_bc_execute_with_hooks,
+ * src/core/bytecode/bytecode.c:196-286, called from src/graph/graph_executor.cpp:895);
+ * it is for an executor that knows which consecutive instructions are independent (the q, k and v projections of one
+ * normalized row; gate and up), because on this device the tail of one linear, the gap to the next launch and the
+ * next one's start-up cost 2 - 3 us per linear that nothing else hides.
+ *   branch_begin : opens a section; the calls that follow form its first branch
+ *   branch_next  : the calls that follow form the next branch; it starts after everything enqueued BEFORE
+ *                  branch_begin, and is unordered with respect to the other branches of the section
+ *   branch_join  : closes the section; whatever is enqueued afterwards starts after every branch has finished
+ * Works the same inside a batched submission (the branches become parallel paths of the HIP graph) and outside one
+ * (streams and events). A section holds at most MARMOT_HIP_MAX_BRANCHES branches; sections do not nest; a section
+ * opened inside a batched submission must be joined before graph_end_capture, and graph_begin_capture inside a
+ * section is refused (all INVALID_OPERATION / INVALID_ARGUMENT). Every branch has a workspace of its own, so calls of
+ * different branches share no scratch memory; the caller guarantees that no branch reads or writes what another
+ * branch of the same section writes. marmot_hip_synchronize inside a section waits for all its branches. The entry
+ * point that does not allocate may only be called in a section's first branch (its scratch array exists once). */
+#define MARMOT_HIP_MAX_BRANCHES 4
+int marmot_hip_branch_begin(marmot_hip_device_t *dev);
+int marmot_hip_branch_next(marmot_hip_device_t *dev);
+int marmot_hip_branch_join(marmot_hip_device_t *dev);
+
 /* DIAGNOSTIC (measurement aid, not an operator), no counterpart in the reference: one launch that only reads `size` bytes at d_src (16-byte loads,
  * nothing is written; d_sink is 1 KiB of device memory the kernel may touch only for a pattern the test data cannot
  * produce). bench.py times it beside the matvec to report the read bandwidth this box delivers to one dependent

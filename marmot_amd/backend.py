@@ -133,6 +133,20 @@ class HipBackend:
         check(st)
         return g
 
+    def branches(self, *fns):
+        """Runs fns[0](), fns[1](), ... as the branches of one section: what they enqueue may overlap on the device, and
+        whatever is enqueued afterwards starts after all of them (marmot_hip_branch_begin / _next / _join). The caller
+        guarantees that no branch touches what another one writes. At most MARMOT_HIP_MAX_BRANCHES functions."""
+        check(self.lib.marmot_hip_branch_begin(self.dev))
+        try:
+            for i, fn in enumerate(fns):
+                if i > 0:
+                    check(self.lib.marmot_hip_branch_next(self.dev))
+                fn()
+        finally:
+            st = self.lib.marmot_hip_branch_join(self.dev)
+        check(st)
+
     def graph_max_nodes(self) -> int:
         """Most nodes one captured graph may hold (graph_capture raises beyond it)."""
         return int(self.lib.marmot_hip_graph_max_nodes())

@@ -109,6 +109,9 @@ SIGNATURES = {
     "marmot_hip_stream": (_vp, [_vp]),
     "marmot_hip_last_error": (C.c_char_p, []),
     "marmot_hip_get_caps": (_i, [_vp, C.POINTER(Caps)]),
+    "marmot_hip_branch_begin": (_i, [_vp]),
+    "marmot_hip_branch_next": (_i, [_vp]),
+    "marmot_hip_branch_join": (_i, [_vp]),
     "marmot_hip_graph_begin_capture": (_i, [_vp]),
     "marmot_hip_graph_end_capture": (_i, [_vp, C.POINTER(_vp)]),
     "marmot_hip_graph_launch": (_i, [_vp, _vp]),

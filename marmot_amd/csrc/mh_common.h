@@ -245,6 +245,22 @@ struct marmot_hip_device {
     void *workspace = nullptr;
     size_t workspace_bytes = 0;
     bool capturing = false;  // between graph_begin_capture and graph_end_capture
+    // Branches (marmot_hip_branch_begin / _next / _join): calls that do not depend on each other go to different
+    // streams and may overlap on the device. `stream` above is the stream of the branch that is open (the main stream
+    // outside a section and in a section's first branch); a branch other than the first has a workspace of its own,
+    // parked in branch_workspace while another branch is open (the fields `workspace` / `workspace_bytes` always belong
+    // to the open branch), so calls of different branches never share scratch memory.
+    static constexpr int MAX_BRANCHES = MARMOT_HIP_MAX_BRANCHES;
+    hipStream_t main_stream = nullptr;
+    hipStream_t side_streams[MAX_BRANCHES - 1] = {};
+    hipEvent_t fork_event = nullptr;
+    hipEvent_t side_done[MAX_BRANCHES - 1] = {};
+    struct ParkedWorkspace {
+        void *ptr = nullptr;
+        size_t bytes = 0;
+    } branch_workspace[MAX_BRANCHES];
+    int branch = -1;        // -1: no section is open; 0: first branch (main stream); i > 0: side stream i - 1
+    int branches_used = 0;  // branches opened in the section so far
     // Executable graphs made by graph_end_capture and not destroyed yet: their kernel arguments hold workspace
     // addresses, so a workspace that is outgrown while any of them lives is retired, not freed.
     size_t live_graphs = 0;

@@ -138,6 +138,49 @@ size_t marmot_hip_row_bytes(int kind, size_t k) {
     return bv == 0 ? 0 : ((k + bv - 1) / bv) * block_bytes(kind);
 }
 
+// Streams and events of the branch sections (marmot_hip_branch_*), made once per device object: creating them inside
+// a section could fall into a stream capture. Default priority, like the main stream.
+static int branches_init(marmot_hip_device *dev) {
+    for (int i = 0; i < marmot_hip_device::MAX_BRANCHES - 1; ++i) {
+        if (check_hip(hipStreamCreateWithFlags(&dev->side_streams[i], hipStreamNonBlocking), "hipStreamCreateWithFlags") != 0 ||
+            check_hip(hipEventCreateWithFlags(&dev->side_done[i], hipEventDisableTiming), "hipEventCreateWithFlags") != 0) {
+            return -1;
+        }
+    }
+    return check_hip(hipEventCreateWithFlags(&dev->fork_event, hipEventDisableTiming), "hipEventCreateWithFlags");
+}
+
+static void branches_destroy(marmot_hip_device *dev) {
+    for (int i = 0; i < marmot_hip_device::MAX_BRANCHES - 1; ++i) {
+        if (dev->side_streams[i] != nullptr) {
+            (void)hipStreamDestroy(dev->side_streams[i]);
+        }
+        if (dev->side_done[i] != nullptr) {
+            (void)hipEventDestroy(dev->side_done[i]);
+        }
+    }
+    if (dev->fork_event != nullptr) {
+        (void)hipEventDestroy(dev->fork_event);
+    }
+}
+
+// Waits for everything this device object has enqueued: the open stream and, inside a branch section, the main stream
+// and the side streams of the branches opened so far.
+static hipError_t streams_synchronize(marmot_hip_device *dev) {
+    hipError_t e = hipStreamSynchronize(dev->stream);
+    if (dev->branch >= 0) {
+        if (e == hipSuccess && dev->stream != dev->main_stream) {
+            e = hipStreamSynchronize(dev->main_stream);
+        }
+        for (int i = 1; i < dev->branches_used && e == hipSuccess; ++i) {
+            if (dev->side_streams[i - 1] != dev->stream) {
+                e = hipStreamSynchronize(dev->side_streams[i - 1]);
+            }
+        }
+    }
+    return e;
+}
+
 int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
     if (out_dev == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "out_dev is null");
@@ -186,7 +229,15 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
         delete dev;
         return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
     }
+    dev->main_stream = dev->stream;
+    if (branches_init(dev) != 0) {
+        branches_destroy(dev);
+        (void)hipStreamDestroy(dev->main_stream);
+        delete dev;
+        return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
+    }
     if (static_scratch_init(dev) != 0) {
+        branches_destroy(dev);
         (void)hipStreamDestroy(dev->stream);
         delete dev;
         return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
@@ -197,6 +248,7 @@ int marmot_hip_device_create(int device_index, marmot_hip_device_t **out_dev) {
     }
     if (check_hip(hipMalloc((void **)&dev->fault_word, 256), "hipMalloc(fault word)") != 0 ||
         check_hip(hipMemset(dev->fault_word, 0, 256), "hipMemset(fault word)") != 0) {
+        branches_destroy(dev);
         (void)hipStreamDestroy(dev->stream);
         delete dev;
         return MARMOT_HIP_ERROR_BACKEND_INIT_FAILED;
@@ -210,9 +262,14 @@ void marmot_hip_device_destroy(marmot_hip_device_t *dev) {
         return;
     }
     (void)hipSetDevice(dev->device_index);
-    (void)hipStreamSynchronize(dev->stream);
+    (void)streams_synchronize(dev);
     if (dev->workspace != nullptr) {
         (void)hipFree(dev->workspace);
+    }
+    for (auto &parked : dev->branch_workspace) {
+        if (parked.ptr != nullptr) {
+            (void)hipFree(parked.ptr);
+        }
     }
     for (void *w : dev->retired_workspaces) {
         (void)hipFree(w);
@@ -223,7 +280,8 @@ void marmot_hip_device_destroy(marmot_hip_device_t *dev) {
     if (dev->fault_word != nullptr) {
         (void)hipFree(dev->fault_word);
     }
-    (void)hipStreamDestroy(dev->stream);
+    branches_destroy(dev);
+    (void)hipStreamDestroy(dev->main_stream);
     delete dev;
 }
 
@@ -262,7 +320,7 @@ void marmot_hip_free(marmot_hip_device_t *dev, void *dptr) {
         dev->current_bytes -= it->second;
         dev->allocs.erase(it);
     }
-    (void)hipStreamSynchronize(dev->stream);
+    (void)streams_synchronize(dev);
     (void)hipFree(dptr);
 }
 
@@ -319,7 +377,7 @@ int marmot_hip_synchronize(marmot_hip_device_t *dev) {
     if (dev == nullptr) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "synchronize: null device");
     }
-    MH_HIP(hipStreamSynchronize(dev->stream));
+    MH_HIP(streams_synchronize(dev));
     // a row-owning kernel whose wavefronts gave up waiting for one another (SpinGuard, mh_rows.h) has left its mark
     uint32_t fault = 0;
     MH_HIP(hipMemcpy(&fault, dev->fault_word, sizeof(fault), hipMemcpyDeviceToHost));
@@ -382,8 +440,74 @@ int marmot_hip_graph_begin_capture(marmot_hip_device_t *dev) {
     if (dev->capturing) {
         return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "graph_begin_capture: a capture is already active");
     }
+    if (dev->branch >= 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
+                         "graph_begin_capture: a branch section is open; join it first");
+    }
     MH_HIP(hipStreamBeginCapture(dev->stream, hipStreamCaptureModeThreadLocal));
     dev->capturing = true;
+    return MARMOT_HIP_SUCCESS;
+}
+
+// Parks the open branch's workspace and makes branch `to` the open one (its stream, its workspace).
+static void branch_switch(marmot_hip_device *dev, int to) {
+    dev->branch_workspace[dev->branch].ptr = dev->workspace;
+    dev->branch_workspace[dev->branch].bytes = dev->workspace_bytes;
+    dev->workspace = dev->branch_workspace[to].ptr;
+    dev->workspace_bytes = dev->branch_workspace[to].bytes;
+    dev->branch_workspace[to].ptr = nullptr;
+    dev->branch_workspace[to].bytes = 0;
+    dev->branch = to;
+    dev->stream = to == 0 ? dev->main_stream : dev->side_streams[to - 1];
+}
+
+int marmot_hip_branch_begin(marmot_hip_device_t *dev) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "branch_begin: null device");
+    }
+    if (dev->branch >= 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "branch_begin: a branch section is already open");
+    }
+    MH_HIP(hipEventRecord(dev->fork_event, dev->main_stream));
+    dev->branch = 0;
+    dev->branches_used = 1;
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_branch_next(marmot_hip_device_t *dev) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "branch_next: null device");
+    }
+    if (dev->branch < 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "branch_next: no branch section is open");
+    }
+    if (dev->branch + 1 >= marmot_hip_device::MAX_BRANCHES) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "branch_next: a section holds at most %d branches",
+                         marmot_hip_device::MAX_BRANCHES);
+    }
+    const int to = dev->branch + 1;
+    // the new branch starts behind everything that was enqueued before the section
+    MH_HIP(hipStreamWaitEvent(dev->side_streams[to - 1], dev->fork_event, 0));
+    branch_switch(dev, to);
+    dev->branches_used = to + 1;
+    return MARMOT_HIP_SUCCESS;
+}
+
+int marmot_hip_branch_join(marmot_hip_device_t *dev) {
+    if (dev == nullptr) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "branch_join: null device");
+    }
+    if (dev->branch < 0) {
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "branch_join: no branch section is open");
+    }
+    const int used = dev->branches_used;
+    branch_switch(dev, 0);
+    dev->branch = -1;
+    dev->branches_used = 0;
+    for (int i = 1; i < used; ++i) {
+        MH_HIP(hipEventRecord(dev->side_done[i - 1], dev->side_streams[i - 1]));
+        MH_HIP(hipStreamWaitEvent(dev->main_stream, dev->side_done[i - 1], 0));
+    }
     return MARMOT_HIP_SUCCESS;
 }
 
@@ -427,6 +551,11 @@ int marmot_hip_graph_end_capture(marmot_hip_device_t *dev, void **out_graph_exec
     *out_graph_exec = nullptr;
     if (!dev->capturing) {
         return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION, "graph_end_capture: no capture is active");
+    }
+    if (dev->branch >= 0) {
+        // the side streams have not joined the main stream yet: ending the capture now would fail inside the runtime
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
+                         "graph_end_capture: a branch section is open; call marmot_hip_branch_join first");
     }
     dev->capturing = false;
     hipGraph_t graph = nullptr;

@@ -431,6 +431,11 @@ int marmot_hip_matmul_quantized_noalloc(marmot_hip_device_t *dev, int kind, cons
     if (st != MARMOT_HIP_SUCCESS) {
         return st;
     }
+    if (dev->branch > 0) {
+        // the array exists once per device: a call in another branch of the same section could use it at the same time
+        return set_error(MARMOT_HIP_ERROR_INVALID_OPERATION,
+                         "matmul_quantized_noalloc: only in the first branch of a branch section");
+    }
     // same routes and kernels as marmot_hip_matmul_quantized; every scratch request of the call is served from this
     // device's copy of the static array (or refused when it is larger)
     dev->use_static_scratch = true;

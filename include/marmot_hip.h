@@ -100,7 +100,8 @@ int marmot_hip_synchronize(marmot_hip_device_t *dev);
 /* bytes currently held through marmot_hip_alloc, and the high-water mark
  * (marmot_device_ops_t.allocator_usage, include/marmot/allocator.h:27-36) */
 int marmot_hip_allocator_usage(marmot_hip_device_t *dev, size_t *current_bytes, size_t *peak_bytes, size_t *n_allocs);
-/* The hipStream_t all work of this device object is enqueued on (as void*). */
+/* The hipStream_t the work of this device object is enqueued on (as void*): the main stream, or inside a branch
+ * section (marmot_hip_branch_begin) the stream of the branch that is open. */
 void *marmot_hip_stream(marmot_hip_device_t *dev);
 const char *marmot_hip_last_error(void);
 

@@ -423,6 +423,12 @@ int marmot_hip_unary(marmot_hip_device_t *dev, int op, const void *d_x, int dtyp
  * differences at or below -88 giving exactly 0, sum, one multiplication by 1 / sum. d_out may be d_x. */
 int marmot_hip_softmax(marmot_hip_device_t *dev, const float *d_x, size_t outer, size_t axis, size_t inner,
                        float *d_out);
+/* The same for a tensor of `dtype` FLOAT32, FLOAT16 or BFLOAT16 (input and output of one type). The 16-bit types follow
+ * softmax_f16_scalar / softmax_bf16_scalar (src/backends/cpu/ops/softmax/scalar/softmax_misc_scalar.c:4-62, 64-122):
+ * maximum and sum in FLOAT32, each exponential rounded to the type when stored (the sum takes the unrounded value),
+ * and the stored value times 1 / sum rounded again. d_out may be d_x. */
+int marmot_hip_softmax_typed(marmot_hip_device_t *dev, int dtype, const void *d_x, size_t outer, size_t axis,
+                             size_t inner, void *d_out);
 /* Replaces cpu_convert_{f32,f16,bf16}_to_{f32,f16,bf16} (src/backends/cpu/ops/convert/dtype_convert.c:17-130 and the
  * bridges through FLOAT32, src/utils/dtype_ref.c:106-114): n contiguous values; to FLOAT16 and to BFLOAT16 round to
  * nearest even (the reference's vector body; its scalar tail of n % 8 values truncates FLOAT16, dtype_ref.c:14-50,

@@ -499,10 +499,13 @@ class HipBackend:
                 if b_ is not None:
                     b_.free()
 
-    def softmax(self, x: np.ndarray, axis: int = -1, in_place: bool = False) -> np.ndarray:
-        """marmot_softmax of a contiguous float32 tensor along one axis (cpu_softmax_impl,
-        src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103)."""
-        x = np.ascontiguousarray(x, dtype=np.float32)
+    def softmax(self, x: np.ndarray, axis: int = -1, in_place: bool = False, dtype: int = DT_F32) -> np.ndarray:
+        """marmot_softmax of a contiguous tensor along one axis (cpu_softmax_impl,
+        src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103). dtype FLOAT32: float32 values; FLOAT16 (1) /
+        BFLOAT16 (2): uint16 bit patterns in, uint16 bit patterns out."""
+        np_type = np.float32 if dtype == DT_F32 else np.uint16
+        x = np.ascontiguousarray(x, dtype=np_type) if dtype == DT_F32 else np.ascontiguousarray(x)
+        assert x.dtype == np_type
         axis = axis % x.ndim
         outer = int(np.prod(x.shape[:axis], dtype=np.int64))
         inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
@@ -511,9 +514,9 @@ class HipBackend:
         d_x = self.to_device(x)
         d_out = d_x if in_place else self.alloc(x.nbytes)
         try:
-            check(self.lib.marmot_hip_softmax(self.dev, C.c_void_p(d_x.ptr), outer, x.shape[axis], inner,
-                                              C.c_void_p(d_out.ptr)))
-            return d_out.download(np.float32, x.shape)
+            check(self.lib.marmot_hip_softmax_typed(self.dev, dtype, C.c_void_p(d_x.ptr), outer, x.shape[axis], inner,
+                                                    C.c_void_p(d_out.ptr)))
+            return d_out.download(np_type, x.shape)
         finally:
             d_x.free()
             if d_out is not d_x:

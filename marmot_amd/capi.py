@@ -149,6 +149,7 @@ SIGNATURES = {
     "marmot_hip_rope": (_i, [_vp, _vp, _i, _sz, _sz, _sz, _sz, C.POINTER(Rope), _vp]),
     "marmot_hip_unary": (_i, [_vp, _i, _vp, _i, _sz, _vp]),
     "marmot_hip_softmax": (_i, [_vp, _vp, _sz, _sz, _sz, _vp]),
+    "marmot_hip_softmax_typed": (_i, [_vp, _i, _vp, _sz, _sz, _sz, _vp]),
     "marmot_hip_convert": (_i, [_vp, _vp, _i, _vp, _i, _sz]),
     "marmot_hip_gather_rows": (_i, [_vp, _vp, _sz, _sz, _sz, _vp, _i, _sz, _sz, _vp, _sz]),
     "marmot_hip_slice": (_i, [_vp, _vp, _sz, _i, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), _vp]),

@@ -2178,7 +2178,7 @@ static marmot_error_t gather_rows(const void *device_ctx, const marmot_tensor_t 
 }
 
 // marmot_softmax (cpu_softmax_impl, src/backends/cpu/ops/softmax/softmax_dispatch.c:67-103; marmot_softmax_prepare,
-// src/core/helpers/norm.c:123-179, checks in its order): FLOAT32, contiguous, any axis
+// src/core/helpers/norm.c:123-179, checks in its order): FLOAT32, FLOAT16 or BFLOAT16, contiguous, any axis
 static marmot_error_t softmax(const void *device_ctx, const marmot_softmax_desc_t *desc) {
     hip_backend_t *b = backend_of(device_ctx);
     if (desc == nullptr) {
@@ -2221,8 +2221,8 @@ static marmot_error_t softmax(const void *device_ctx, const marmot_softmax_desc_
     }
     const size_t total = tensor_numel(x);
     const size_t outer = total / (axis_size * inner);
-    if (x->dtype != MARMOT_DTYPE_FLOAT32) {
-        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP softmax handles FLOAT32 tensors");
+    if (x->dtype != MARMOT_DTYPE_FLOAT32 && x->dtype != MARMOT_DTYPE_FLOAT16 && x->dtype != MARMOT_DTYPE_BFLOAT16) {
+        return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP softmax handles FLOAT32, FLOAT16 and BFLOAT16 tensors");
     }
     if (!dense_contiguous(x) || !dense_contiguous(out)) {
         return fail(MARMOT_ERROR_NOT_IMPLEMENTED, "HIP softmax needs contiguous tensors");
@@ -2241,7 +2241,8 @@ static marmot_error_t softmax(const void *device_ctx, const marmot_softmax_desc_
     };
     marmot_error_t st = acquire_set(b, acq, 2);
     if (st == MARMOT_SUCCESS) {
-        const int rc = marmot_hip_softmax(b->dev, (const float *)acq[0].dev, outer, axis_size, inner, (float *)acq[1].dev);
+        const int rc = marmot_hip_softmax_typed(b->dev, pa_lib_dtype(x->dtype), acq[0].dev, outer, axis_size, inner,
+                                                acq[1].dev);
         st = rc == MARMOT_HIP_SUCCESS ? MARMOT_SUCCESS : fail_from_lib(rc);
     }
     pthread_mutex_unlock(&b->mu);
@@ -3221,11 +3222,14 @@ marmot_kernel_selection_t marmot_hip_query_kernel(const marmot_op_signature_t *s
         return selected(sig->op_id == MARMOT_OP_GELU        ? MARMOT_HIP_BC_OP_GELU
                         : sig->op_id == MARMOT_OP_GELU_TANH ? MARMOT_HIP_BC_OP_GELU_TANH
                                                             : MARMOT_HIP_BC_OP_SILU, launch_us, 0.0);
-    case MARMOT_OP_SOFTMAX:
-        if (!in32 || !out32) {
-            return unsupported("HIP softmax handles FLOAT32 tensors");
+    case MARMOT_OP_SOFTMAX: {
+        // one executor for the three types: it reads the type from the tensors
+        const bool bf = sig->input_dtype == MARMOT_DTYPE_BFLOAT16 && sig->output_dtype == MARMOT_DTYPE_BFLOAT16;
+        if (!((in32 && out32) || (in16 && out16) || bf)) {
+            return unsupported("HIP softmax handles FLOAT32, FLOAT16 and BFLOAT16 tensors");
         }
         return selected(MARMOT_HIP_BC_OP_SOFTMAX_F32, launch_us, 0.0);
+    }
     case MARMOT_OP_RESHAPE:
         return selected(MARMOT_HIP_BC_OP_RESHAPE, 0.0, 0.0);  // metadata only
     case MARMOT_OP_VIEW:

@@ -95,57 +95,75 @@ __device__ __forceinline__ float block_reduce(float v, float *red, bool is_max) 
     return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-__global__ __launch_bounds__(256) void k_softmax(const float *x, float *out, size_t axis,
-                                                 size_t inner) {
+// FLOAT16 / BFLOAT16 rows follow softmax_f16_scalar / softmax_bf16_scalar (scalar/softmax_misc_scalar.c:4-122): maximum
+// and sum in FLOAT32, every exponential rounded to the tensor's type when it is stored (the sum takes the unrounded
+// one), and the stored value, widened again, times 1 / sum rounded a second time.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void k_softmax(const void *x, void *out, size_t axis, size_t inner) {
     __shared__ float red[4];
     const size_t row = blockIdx.x;
     const size_t o = row / inner, j = row - o * inner;
     const size_t base = o * axis * inner + j;
     float m = -INFINITY;
     for (size_t a = threadIdx.x; a < axis; a += 256) {
-        m = fmaxf(m, x[base + a * inner]);
+        m = fmaxf(m, load_as_f32<DTYPE>(x, base + a * inner));
     }
     m = block_reduce(m, red, true);
     float sum = 0.0f;
     for (size_t a = threadIdx.x; a < axis; a += 256) {
-        const float diff = x[base + a * inner] - m;
+        const float diff = load_as_f32<DTYPE>(x, base + a * inner) - m;
         const float e = diff <= -88.0f ? 0.0f : expf(diff);  // softmax_safe_expf, softmax_internal.h:14-26
-        out[base + a * inner] = e;
+        store_from_f32<DTYPE>(out, base + a * inner, e);
         sum += e;
     }
     sum = block_reduce(sum, red, false);
     const float inv = 1.0f / sum;
     for (size_t a = threadIdx.x; a < axis; a += 256) {
-        out[base + a * inner] *= inv;  // written by this thread above
+        // written by this thread above
+        store_from_f32<DTYPE>(out, base + a * inner, load_as_f32<DTYPE>(out, base + a * inner) * inv);
     }
 }
 
 // Short rows that lie contiguously (inner == 1, at most SOFTMAX_SMALL values, e.g. router logits over the experts): one
 // thread per row, everything in index order like the scalar CPU loop.
 constexpr size_t SOFTMAX_SMALL = 128;
-__global__ __launch_bounds__(64) void k_softmax_small(const float *x, float *out, size_t rows,
-                                                      size_t axis) {
+template <int DTYPE>
+__global__ __launch_bounds__(64) void k_softmax_small(const void *x, void *out, size_t rows, size_t axis) {
     const size_t row = (size_t)blockIdx.x * 64 + threadIdx.x;
     if (row >= rows) {
         return;
     }
-    const float *in = x + row * axis;
-    float *o = out + row * axis;
-    float m = in[0];
-    for (size_t i = 1; i < axis; ++i) {
-        m = in[i] > m ? in[i] : m;
+    const size_t base = row * axis;
+    // FLOAT32 rows start from their first value, the 16-bit rows from -FLT_MAX (softmax_find_max_f16,
+    // softmax_internal.h:119-150): the same maximum unless a row holds nothing above -FLT_MAX
+    float m = DTYPE == MARMOT_HIP_DTYPE_F32 ? load_as_f32<DTYPE>(x, base) : -3.402823466e+38f;
+    for (size_t i = DTYPE == MARMOT_HIP_DTYPE_F32 ? 1 : 0; i < axis; ++i) {
+        const float v = load_as_f32<DTYPE>(x, base + i);
+        m = v > m ? v : m;
     }
     float sum = 0.0f;
     for (size_t i = 0; i < axis; ++i) {
-        const float diff = in[i] - m;
+        const float diff = load_as_f32<DTYPE>(x, base + i) - m;
         const float e = diff <= -88.0f ? 0.0f : expf(diff);
-        o[i] = e;
+        store_from_f32<DTYPE>(out, base + i, e);
         sum += e;
     }
     const float inv = 1.0f / sum;
     for (size_t i = 0; i < axis; ++i) {
-        o[i] *= inv;
+        store_from_f32<DTYPE>(out, base + i, load_as_f32<DTYPE>(out, base + i) * inv);
     }
+}
+
+template <int DTYPE>
+static int launch_softmax(marmot_hip_device *dev, const void *d_x, size_t rows, size_t axis, size_t inner, void *d_out) {
+    if (inner == 1 && axis <= SOFTMAX_SMALL) {
+        hipLaunchKernelGGL(k_softmax_small<DTYPE>, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, dev->stream, d_x,
+                           d_out, rows, axis);
+    } else {
+        hipLaunchKernelGGL(k_softmax<DTYPE>, dim3((unsigned)rows), dim3(256), 0, dev->stream, d_x, d_out, axis, inner);
+    }
+    MH_HIP(hipGetLastError());
+    return MARMOT_HIP_SUCCESS;
 }
 
 // ------------------------------------------------------------------ conversion
@@ -289,8 +307,8 @@ int marmot_hip_unary(marmot_hip_device_t *dev, int op, const void *d_x, int dtyp
     return MARMOT_HIP_SUCCESS;
 }
 
-int marmot_hip_softmax(marmot_hip_device_t *dev, const float *d_x, size_t outer, size_t axis, size_t inner,
-                       float *d_out) {
+int marmot_hip_softmax_typed(marmot_hip_device_t *dev, int dtype, const void *d_x, size_t outer, size_t axis,
+                             size_t inner, void *d_out) {
     if (dev == nullptr) {
         return set_error(MARMOT_HIP_ERROR_DEVICE_NOT_AVAILABLE, "HIP device is not initialised");
     }
@@ -300,6 +318,9 @@ int marmot_hip_softmax(marmot_hip_device_t *dev, const float *d_x, size_t outer,
     if (axis == 0) {
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "Softmax axis dimension must be non-zero");
     }
+    if (dtype != MARMOT_HIP_DTYPE_F32 && dtype != MARMOT_HIP_DTYPE_F16 && dtype != MARMOT_HIP_DTYPE_BF16) {
+        return set_error(MARMOT_HIP_ERROR_UNSUPPORTED_DTYPE, "softmax: unsupported dtype %d", dtype);
+    }
     const size_t rows = outer * inner;
     if (rows == 0) {
         return MARMOT_HIP_SUCCESS;
@@ -308,15 +329,18 @@ int marmot_hip_softmax(marmot_hip_device_t *dev, const float *d_x, size_t outer,
         return set_error(MARMOT_HIP_ERROR_INVALID_ARGUMENT, "softmax: more than 2^31 - 1 rows");
     }
     MH_HIP(hipSetDevice(dev->device_index));
-    if (inner == 1 && axis <= SOFTMAX_SMALL) {
-        hipLaunchKernelGGL(k_softmax_small, dim3((unsigned)((rows + 63) / 64)), dim3(64), 0, dev->stream, d_x, d_out,
-                           rows, axis);
-        MH_HIP(hipGetLastError());
-        return MARMOT_HIP_SUCCESS;
+    if (dtype == MARMOT_HIP_DTYPE_F16) {
+        return launch_softmax<MARMOT_HIP_DTYPE_F16>(dev, d_x, rows, axis, inner, d_out);
     }
-    hipLaunchKernelGGL(k_softmax, dim3((unsigned)rows), dim3(256), 0, dev->stream, d_x, d_out, axis, inner);
-    MH_HIP(hipGetLastError());
-    return MARMOT_HIP_SUCCESS;
+    if (dtype == MARMOT_HIP_DTYPE_BF16) {
+        return launch_softmax<MARMOT_HIP_DTYPE_BF16>(dev, d_x, rows, axis, inner, d_out);
+    }
+    return launch_softmax<MARMOT_HIP_DTYPE_F32>(dev, d_x, rows, axis, inner, d_out);
+}
+
+int marmot_hip_softmax(marmot_hip_device_t *dev, const float *d_x, size_t outer, size_t axis, size_t inner,
+                       float *d_out) {
+    return marmot_hip_softmax_typed(dev, MARMOT_HIP_DTYPE_F32, d_x, outer, axis, inner, d_out);
 }
 
 int marmot_hip_convert(marmot_hip_device_t *dev, void *d_dst, int dst_dtype, const void *d_src, int src_dtype,

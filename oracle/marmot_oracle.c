@@ -3709,6 +3709,56 @@ static float conv_load(int dtype, const void *p, size_t i) {
     return f;
 }
 
+static void conv_store(int dtype, void *p, size_t i, float v) {
+    if (dtype == MO_DTYPE_F32) {
+        ((float *)p)[i] = v;
+    } else if (dtype == MO_DTYPE_F16) {
+        ((uint16_t *)p)[i] = mo_f32_to_f16(v);
+    } else {
+        uint32_t bits;
+        memcpy(&bits, &v, 4);
+        const uint32_t rounding_bias = 0x7FFFu + ((bits >> 16) & 1u);
+        ((uint16_t *)p)[i] = (uint16_t)((bits + rounding_bias) >> 16);
+    }
+}
+
+/* softmax_f16_scalar / softmax_bf16_scalar (src/backends/cpu/ops/softmax/scalar/softmax_misc_scalar.c:4-62, 64-122;
+ * softmax_find_max_f16 and softmax_scale_f16, softmax_internal.h:119-215) over [outer, axis, inner] of a 16-bit type:
+ * the maximum (from -FLT_MAX) and the sum of the exponentials are FLOAT32; every exponential is rounded to the tensor's
+ * type when it is stored, and the stored value, widened again, is multiplied by 1 / sum and rounded a second time.
+ * dtype FLOAT32 is mo_softmax. */
+int mo_softmax_typed(int dtype, const void *x, size_t outer, size_t axis, size_t inner, void *out) {
+    if (dtype == MO_DTYPE_F32) {
+        return mo_softmax((const float *)x, outer, axis, inner, (float *)out);
+    }
+    if ((dtype != MO_DTYPE_F16 && dtype != MO_DTYPE_BF16) || axis == 0) {
+        return -1;
+    }
+    for (size_t row = 0; row < outer * inner; ++row) {
+        const size_t o = row / inner, j = row % inner;
+        const size_t base = o * axis * inner + j;
+        float max_val = -FLT_MAX;
+        for (size_t a = 0; a < axis; ++a) {
+            const float v = conv_load(dtype, x, base + a * inner);
+            if (v > max_val) {
+                max_val = v;
+            }
+        }
+        float sum = 0.0f;
+        for (size_t a = 0; a < axis; ++a) {
+            const float diff = conv_load(dtype, x, base + a * inner) - max_val;
+            const float e = diff <= -88.0f ? 0.0f : expf(diff);
+            sum += e;
+            conv_store(dtype, out, base + a * inner, e);
+        }
+        const float inv_sum = 1.0f / sum;
+        for (size_t a = 0; a < axis; ++a) {
+            conv_store(dtype, out, base + a * inner, conv_load(dtype, out, base + a * inner) * inv_sum);
+        }
+    }
+    return 0;
+}
+
 int mo_convert(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n) {
     const int ok_s = src_dtype == MO_DTYPE_F32 || src_dtype == MO_DTYPE_F16 || src_dtype == MO_DTYPE_BF16;
     const int ok_d = dst_dtype == MO_DTYPE_F32 || dst_dtype == MO_DTYPE_F16 || dst_dtype == MO_DTYPE_BF16;
@@ -3720,17 +3770,7 @@ int mo_convert(void *dst, int dst_dtype, const void *src, int src_dtype, size_t 
         return 0;
     }
     for (size_t i = 0; i < n; ++i) {
-        const float v = conv_load(src_dtype, src, i);
-        if (dst_dtype == MO_DTYPE_F32) {
-            ((float *)dst)[i] = v;
-        } else if (dst_dtype == MO_DTYPE_F16) {
-            ((uint16_t *)dst)[i] = mo_f32_to_f16(v);
-        } else {
-            uint32_t bits;
-            memcpy(&bits, &v, 4);
-            const uint32_t rounding_bias = 0x7FFFu + ((bits >> 16) & 1u);
-            ((uint16_t *)dst)[i] = (uint16_t)((bits + rounding_bias) >> 16);
-        }
+        conv_store(dst_dtype, dst, i, conv_load(src_dtype, src, i));
     }
     return 0;
 }

@@ -272,6 +272,11 @@ float mo_fp8_e4m3_to_f32(uint8_t bits);
 /* op: 0 GELU (erf), 1 GELU (tanh), 2 SiLU; dtype MO_DTYPE_F32 or MO_DTYPE_F16 */
 int mo_unary(int op, const void *x, int dtype, size_t n, void *out);
 int mo_softmax(const float *x, size_t outer, size_t axis, size_t inner, float *out);
+/* the same for FLOAT16 / BFLOAT16 tensors (bit patterns in uint16): exponentials rounded to the type when stored,
+ * scaled from the stored value and rounded again (softmax_misc_scalar.c:4-122); pinned by the reference's g_softmax
+ * vector at the reference's own tolerances for these types (tests/backend/test_backend_softmax.c:53-54) and by a numpy
+ * model of the two roundings */
+int mo_softmax_typed(int dtype, const void *x, size_t outer, size_t axis, size_t inner, void *out);
 int mo_convert(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n);
 int mo_gather_rows(const void *x, size_t rows_in, size_t cols, size_t elem_size, size_t in_stride0, const void *idx,
                    int idx_is_signed, size_t idx_stride, size_t rows_out, void *out, size_t out_stride0,

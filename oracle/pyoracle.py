@@ -213,6 +213,8 @@ class Oracle:
         L.mo_unary.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
         L.mo_softmax.restype = C.c_int
         L.mo_softmax.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
+        L.mo_softmax_typed.restype = C.c_int
+        L.mo_softmax_typed.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
         L.mo_convert.restype = C.c_int
         L.mo_convert.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_size_t]
         L.mo_gather_rows.restype = C.c_int
@@ -460,6 +462,19 @@ class Oracle:
         st = self.L.mo_softmax(_ptr(x), outer, x.shape[axis], inner, _ptr(out))
         if st != 0:
             raise RuntimeError(f"mo_softmax -> {st}")
+        return out
+
+    def softmax_typed(self, x: np.ndarray, dtype: int, axis: int = -1) -> np.ndarray:
+        """x: float32 values (dtype FLOAT32) or uint16 bit patterns of FLOAT16 (1) / BFLOAT16 (2); the result likewise."""
+        x = np.ascontiguousarray(x)
+        assert x.dtype == (np.float32 if dtype == DT_F32 else np.uint16)
+        axis = axis % x.ndim
+        outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+        inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+        out = np.zeros_like(x)
+        st = self.L.mo_softmax_typed(dtype, _ptr(x), outer, x.shape[axis], inner, _ptr(out))
+        if st != 0:
+            raise RuntimeError(f"mo_softmax_typed -> {st}")
         return out
 
     def convert(self, src: np.ndarray, src_dtype: int, dst_dtype: int) -> np.ndarray:

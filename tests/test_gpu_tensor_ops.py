@@ -98,6 +98,36 @@ def test_softmax_matches_oracle_and_reference_goldens(hip, oracle, ref_goldens):
     assert hip.lib.marmot_hip_softmax(hip.dev, C.c_void_p(8), 1, 0, 1, C.c_void_p(8)) == -1
 
 
+def ulps16(a_bits: np.ndarray, b_bits: np.ndarray) -> np.ndarray:
+    """Distance in units of the last place between two arrays of non-negative 16-bit float patterns."""
+    return np.abs(a_bits.astype(np.int32) - b_bits.astype(np.int32))
+
+
+@pytest.mark.parametrize("dtype_name", ["f16", "bf16"])
+def test_softmax_16_bit_types_match_oracle_and_reference_goldens(hip, oracle, ref_goldens, dtype_name):
+    """FLOAT16 / BFLOAT16 softmax: the reference's check for these types (g_softmax at 5e-3 / 1.2e-2, twice that along
+    axis 0, tests/backend/test_backend_softmax.c:6-45, 53-54), then the oracle's two roundings: the device's expf and
+    the tree sum of long rows move a value across a rounding boundary now and then, by one unit of the last place at
+    most."""
+    dtype = capi.DT_F16 if dtype_name == "f16" else capi.DT_BF16
+    tol = 5e-3 if dtype_name == "f16" else 1.2e-2
+    shape = tuple(int(v) for v in ref_goldens["g_softmax_shape"])
+    xb = oracle.convert(ref_goldens["g_softmax_input"].reshape(shape).astype(np.float32), capi.DT_F32, dtype)
+    for axis, key, factor in ((-1, "g_softmax_expected_axis_last", 1.0), (0, "g_softmax_expected_axis0", 2.0)):
+        got = oracle.convert(hip.softmax(xb, axis, dtype=dtype), dtype, capi.DT_F32)
+        assert np.max(np.abs(got.ravel().astype(np.float64) - ref_goldens[key].astype(np.float64))) <= tol * factor
+    for shape, axis in (((5, 8), -1), ((300, 128), 1), ((4, 1000), -1), ((2, 6, 5), 1), ((3, 4, 7), 0), ((2, 32000), 1),
+                        ((7,), 0), ((1, 129), 1), ((64, 60), -1)):
+        print(f"softmax {dtype_name} {shape} axis {axis}", flush=True)
+        xb = oracle.convert(gaussian(1400 + len(shape) + shape[-1], shape, 3.0), capi.DT_F32, dtype)
+        got, ref = hip.softmax(xb, axis, dtype=dtype), oracle.softmax_typed(xb, dtype, axis)
+        d = ulps16(got, ref)
+        assert d.max() <= 1 and np.mean(d == 0) >= 0.99, (shape, int(d.max()), float(np.mean(d == 0)))
+        assert np.array_equal(hip.softmax(xb, axis, in_place=True, dtype=dtype), got)
+    assert hip.lib.marmot_hip_softmax_typed(hip.dev, capi.DT_I32, C.c_void_p(8), 1, 4, 1, C.c_void_p(8)) == -6
+    assert hip.lib.marmot_hip_softmax_typed(hip.dev, dtype, C.c_void_p(8), 1, 0, 1, C.c_void_p(8)) == -1
+
+
 def test_convert_is_bit_exact(hip, oracle, ref_goldens):
     g = ref_goldens
     assert np.array_equal(hip.convert(g["g_conv_f16_src"], DT_F32, DT_F16), g["g_conv_f16_f16_bits"])
@@ -194,8 +224,11 @@ def test_queries_for_the_graph_nodes(ctx):
             sel = ctx.query(_sig(ctx, op, dt))
             assert sel.supported and sel.op_index == bc
         assert not ctx.query(_sig(ctx, op, ta.DTYPE_BF16)).supported
-    assert ctx.query(_sig(ctx, ta.OP_SOFTMAX)).op_index == ta.BC_OP_SOFTMAX_F32
-    assert not ctx.query(_sig(ctx, ta.OP_SOFTMAX, ta.DTYPE_F16)).supported
+    for dt in (ta.DTYPE_F32, ta.DTYPE_F16, ta.DTYPE_BF16):  # one executor, the type is read from the tensors
+        sel = ctx.query(_sig(ctx, ta.OP_SOFTMAX, dt))
+        assert sel.supported and sel.op_index == ta.BC_OP_SOFTMAX_F32
+    assert not ctx.query(_sig(ctx, ta.OP_SOFTMAX, ta.DTYPE_F16, ta.DTYPE_F32)).supported
+    assert not ctx.query(_sig(ctx, ta.OP_SOFTMAX, ta.DTYPE_I32)).supported
     for op, bc in ((ta.OP_RESHAPE, ta.BC_OP_RESHAPE), (ta.OP_VIEW, ta.BC_OP_VIEW), (ta.OP_SLICE, ta.BC_OP_SLICE),
                    (ta.OP_GATHER_ROWS, ta.BC_OP_GATHER_ROWS)):
         sel = ctx.query(_sig(ctx, op, ta.DTYPE_F16))
@@ -251,6 +284,25 @@ def test_impl_unary_and_softmax(ctx, oracle):
         assert np.allclose(ctx.to_host(st), oracle.softmax(x, axis), rtol=3e-6, atol=1e-30)
         for t in (st, so):
             ctx.host_freed(t)
+    # FLOAT16 and BFLOAT16 tensors (bfloat16 bits travel in uint16 arrays): the implementation and the program
+    for dtype, ta_dtype in ((capi.DT_F16, ta.DTYPE_F16), (capi.DT_BF16, ta.DTYPE_BF16)):
+        for shape, axis in (((4, 8), -1), ((2, 6, 5), 1), ((5, 300), 1)):
+            xb = oracle.convert(gaussian(1730 + shape[-1], shape, 3.0), capi.DT_F32, dtype)
+            want = oracle.softmax_typed(xb, dtype, axis)
+            view = xb.view(np.float16) if dtype == capi.DT_F16 else xb
+            st = ta.HostTensor.strided(view.copy(), ta_dtype)
+            so = ta.HostTensor.strided(np.zeros_like(view), ta_dtype)
+            desc = ta.SoftmaxDesc(st.ptr, so.ptr, axis)
+            assert ctx.lib.hip_softmax_impl(ctx.device_ctx, C.byref(desc)) == ta.SUCCESS, ctx.last_error()
+            d = np.abs(ctx.to_host(so).view(np.uint16).astype(np.int32) - want.astype(np.int32))
+            assert d.max() <= 1 and np.mean(d == 0) >= 0.98, (dtype, shape, int(d.max()))
+            prog = ta.Program()
+            prog.softmax(ta.BC_OP_SOFTMAX_F32, st, st, axis)  # in place
+            assert ctx.execute(prog) == ta.SUCCESS, ctx.last_error()
+            d = np.abs(ctx.to_host(st).view(np.uint16).astype(np.int32) - want.astype(np.int32))
+            assert d.max() <= 1, (dtype, shape, int(d.max()))
+            for t in (st, so):
+                ctx.host_freed(t)
     st, so = ta.HostTensor.dense(gaussian(1720, (4, 8))), ta.HostTensor.empty((4, 8), ta.DTYPE_F32)
     for axis, code in ((2, ta.INVALID_ARGUMENT), (-3, ta.INVALID_ARGUMENT)):
         desc = ta.SoftmaxDesc(st.ptr, so.ptr, axis)

@@ -281,8 +281,8 @@ def prefill_int8(hip, tokens: int, steps: int, warmup: int):
     return out
 
 
-def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5", "QKV", "OPS", "ATTN", "LAYER", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32", "PREFILLFMT")):
-    """Every benchmark configuration (C1..C5, C4P, QKV, OPS, ATTN, LAYER, LOGITS, Q5K, LEGACY, Q23K, PREFILL32, PREFILLFMT) on the device, one JSON line each (documentation runs, not the
+def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "BRANCH", "C5", "QKV", "OPS", "ATTN", "LAYER", "LOGITS", "Q5K", "LEGACY", "Q23K", "PREFILL32", "PREFILLFMT")):
+    """Every benchmark configuration (C1..C5, C4P, BRANCH, QKV, OPS, ATTN, LAYER, LOGITS, Q5K, LEGACY, Q23K, PREFILL32, PREFILLFMT) on the device, one JSON line each (documentation runs, not the
     driver's line): weights rotate over copies larger than twice the Infinity Cache; times are HIP-graph replays."""
     from marmot_amd import DT_F16, DT_F32, capi, row_bytes
 
@@ -386,6 +386,8 @@ def sweep(hip, steps: int, warmup: int, only=("C1", "C2", "C3", "C4", "C4P", "C5
         sweep_layer_stack(hip, rng, emit, steps)
     if "C4P" in only:
         sweep_layer_stack(hip, rng, emit, steps, N=512, config="C4P")
+    if "BRANCH" in only:
+        sweep_branches(hip, rng, emit, steps)
     if "C5" in only:
         sweep_moe(hip, rng, emit, steps)
     if "QKV" in only:
@@ -591,6 +593,73 @@ def sweep_layer_stack(hip, rng, emit, steps: int, N: int = 16, config: str = "C4
     for *_, d_w, d_x, d_out in layers:
         for b in (d_w, d_x, d_out):
             b.free()
+
+
+def sweep_branches(hip, rng, emit, steps: int, N: int = 16):
+    """Independent linears of one layer (q | k | v and gate | up at 16 tokens, activations packed beforehand) four ways:
+    one after the other on one stream, as the branches of one section (fork + join per step), both eagerly (HIP events
+    around `steps` steps), and as an upper bound every linear on a device object of its own with nothing between them
+    (one graph of 200 steps each, launched together, host clock). The weights stay warm (one copy each): the figures
+    are for comparing the four, not against the rotating-weight rows of the other configurations."""
+    from marmot_amd import DT_F32, HipBackend, capi
+
+    groups = {
+        "q | k | v": [(capi.KIND_Q4_K, 4096, 4096), (capi.KIND_Q4_K, 1024, 4096), (capi.KIND_Q6_K, 1024, 4096)],
+        "gate | up": [(capi.KIND_Q4_K, 14336, 4096), (capi.KIND_Q4_K, 14336, 4096)],
+    }
+
+    def linear_on(backend, kind, M, K):
+        bufs = [backend.to_device(random_blocks(rng, kind, M, K)),
+                backend.to_device(rng.standard_normal((N, K), dtype=np.float32)),
+                backend.alloc(backend.packed_activation_bytes(kind, N, K)), backend.alloc(N * M * 4)]
+        backend.pack_activations_d(kind, bufs[1], DT_F32, N, K, bufs[2])
+        return (lambda: backend.linear_prepacked_d(kind, bufs[0], bufs[2], N, K, M, bufs[3])), bufs
+
+    for name, specs in groups.items():
+        made = [linear_on(hip, *spec) for spec in specs]
+        fns = [fn for fn, _ in made]
+        row_ms, _ = time_steps(hip, lambda i: [fn() for fn in fns], steps, 50)
+        section_ms, _ = time_steps(hip, lambda i: hip.branches(*fns), steps, 50)
+        graph_row = time_steps_graph(hip, lambda i: [fn() for fn in fns], steps, 10, chunk=50)
+        graph_section = time_steps_graph(hip, lambda i: hip.branches(*fns), steps, 10, chunk=50)
+        for _, bufs in made:
+            for b in bufs:
+                b.free()
+        # upper bound: no dependencies at all between the linears
+        others = []
+        for spec in specs:
+            backend = HipBackend(0)
+            fn, bufs = linear_on(backend, *spec)
+            fn()
+            backend.synchronize()
+            others.append((backend, backend.graph_capture(lambda fn=fn: [fn() for _ in range(200)]), bufs))
+
+        def together(reps):
+            for backend, g, _ in others:
+                backend.graph_launch(g)
+            for backend, _, _ in others:
+                backend.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                for backend, g, _ in others:
+                    backend.graph_launch(g)
+            for backend, _, _ in others:
+                backend.synchronize()
+            return (time.perf_counter() - t0) / reps / 200 * 1e3
+
+        together(5)
+        free_ms = together(20)
+        for backend, g, bufs in others:
+            backend.graph_destroy(g)
+            for b in bufs:
+                b.free()
+            backend.close()
+        emit({"config": "BRANCH", "workload": f"{name} of a Llama-3-8B layer, N={N}, packed activations, warm weights",
+              "us_in_a_row_eager": round(row_ms * 1e3, 2), "us_branch_section_eager": round(section_ms * 1e3, 2),
+              "us_in_a_row_graph": round(graph_row * 1e3, 2), "us_branch_section_graph": round(graph_section * 1e3, 2),
+              "us_unsynchronized_streams": round(free_ms * 1e3, 2),
+              "note": "unsynchronized streams: one device object and one 200-step graph per linear, launched together "
+                      "(an upper bound: nothing orders the linears)"})
 
 
 def sweep_attention(hip, rng, emit, steps: int):

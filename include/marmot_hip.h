@@ -160,7 +160,9 @@ size_t marmot_hip_graph_last_capture_nodes(marmot_hip_device_t *dev);
  * opened inside a batched submission must be joined before graph_end_capture, and graph_begin_capture inside a
  * section is refused (all INVALID_OPERATION / INVALID_ARGUMENT). Every branch has a workspace of its own, so calls of
  * different branches share no scratch memory; the caller guarantees that no branch reads or writes what another
- * branch of the same section writes. marmot_hip_synchronize inside a section waits for all its branches. The entry
+ * branch of the same section writes. The first section of a device object makes its side streams and cannot be
+ * recorded: run one section outside a batched submission first (INVALID_OPERATION otherwise), as for a workspace
+ * that has to grow. marmot_hip_synchronize inside a section waits for all its branches. The entry
  * point that does not allocate may only be called in a section's first branch (its scratch array exists once). */
 #define MARMOT_HIP_MAX_BRANCHES 4
 int marmot_hip_branch_begin(marmot_hip_device_t *dev);

@@ -155,9 +155,10 @@ def test_a_capture_cannot_grow_a_branch_workspace(hip, oracle):
         b.run()
         hip.synchronize()
         want = b.result()
+        hip.branches(lambda: None, lambda: None)  # the first section of a device object makes the side streams
         with pytest.raises(capi.MarmotHipError) as err:
             hip.graph_capture(lambda: hip.branches(a.run, b.run))
-        assert err.value.code == -5 and "eagerly" in err.value.detail
+        assert err.value.code == -5 and "workspace" in err.value.detail and "eagerly" in err.value.detail
         hip.branches(a.run, b.run)  # sizes the second branch's workspace
         g = hip.graph_capture(lambda: hip.branches(a.run, b.run))
         b.poison()
@@ -176,6 +177,18 @@ def last_error(lib) -> str:
 
 def test_misuse_is_refused(hip):
     lib, dev = hip.lib, hip.dev
+    import ctypes as C
+
+    # a device object's first section makes its side streams: not inside a capture
+    g = C.c_void_p()
+    buf = hip.alloc(64)
+    assert lib.marmot_hip_graph_begin_capture(dev) == 0
+    assert lib.marmot_hip_memset(dev, C.c_void_p(buf.ptr), 0, 64) == 0
+    assert lib.marmot_hip_branch_begin(dev) == -5
+    assert "side streams" in last_error(lib)
+    assert lib.marmot_hip_graph_end_capture(dev, C.byref(g)) == 0
+    hip.graph_destroy(g)
+    buf.free()
     assert lib.marmot_hip_branch_next(dev) == -5  # no section
     assert lib.marmot_hip_branch_join(dev) == -5
     assert lib.marmot_hip_branch_begin(dev) == 0
@@ -188,8 +201,6 @@ def test_misuse_is_refused(hip):
     assert lib.marmot_hip_branch_join(dev) == 0
     assert lib.marmot_hip_branch_join(dev) == -5
     # a section opened inside a capture must be joined before the capture ends
-    import ctypes as C
-
     assert lib.marmot_hip_graph_begin_capture(dev) == 0
     assert lib.marmot_hip_branch_begin(dev) == 0
     assert lib.marmot_hip_branch_next(dev) == 0
